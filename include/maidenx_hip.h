@@ -1,0 +1,185 @@
+/* maidenx_hip — C ABI of the MI355X (gfx950) compute backend for MaidenX.
+ *
+ * Every entry point is what maidenx_core::be::* would bind for a `Device::HIP` arm: the symbol
+ * family `hip_<op>_<dtype>` mirrors `cuda_<op>_<dtype>` of crates/maidenx_cuda (same argument
+ * order and meaning), with the numerical semantics of crates/maidenx_cpu.
+ *
+ * Conventions
+ *  - Data pointers are device pointers obtained from hip_malloc.  `metadata` pointers are HOST
+ *    pointers (as on the reference's CPU arm, crates/maidenx_core/src/be/ops/binary.rs:113-116);
+ *    their contents are consumed before the call returns.
+ *  - dtype suffixes: f32 = float, bf16 = the upper 16 bits of an IEEE binary32 (uint16_t storage),
+ *    bool = one byte holding 0 or 1.
+ *  - Kernels are queued on one in-order stream (hip_set_stream, default: the device's default
+ *    stream) and return without waiting.  hip_memcpy_d2h / hip_memcpy_h2d wait for completion.
+ *  - Kernel wrappers return void like the reference's; the first error since the last query is
+ *    kept and read with hip_get_last_status() / hip_status_string().
+ *  - Outputs are fully overwritten; no entry point relies on the incoming contents of an output.
+ *  - Strided operands must have fewer than 2^31 logical elements (contiguous ones have no limit).
+ */
+#ifndef MAIDENX_HIP_H
+#define MAIDENX_HIP_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t mx_bf16;   /* bf16 bit pattern */
+typedef uint8_t mx_bool;    /* 0 or 1 */
+
+/* ---- status ------------------------------------------------------------------------------------ */
+#define MX_HIP_OK 0
+#define MX_HIP_ERR_INVALID 1
+#define MX_HIP_ERR_OOM 2          /* crates/maidenx_core/src/error.rs:144-150 maps code 2 to OutOfMemory */
+#define MX_HIP_ERR_TOO_LARGE 3
+#define MX_HIP_ERR_LAUNCH 4
+#define MX_HIP_ERR_UNSUPPORTED 5
+int hip_get_last_status(void);          /* first error since the previous call; clears it */
+const char* hip_status_string(void);    /* text for the status last returned */
+
+/* ---- device / memory / stream: replaces crates/maidenx_cuda/src/lib.rs:39-152 --------------------
+ * (cuda_malloc, cuda_free, cuda_memcpy_h2d/d2h/d2d, cuda_set_device, cuda_get_device,
+ *  cuda_stream_create/destroy/synchronize).  Return 0 on success; hip_malloc returns 2 when the
+ *  device is out of memory. */
+int hip_set_device(int device_id);
+int hip_get_device(int* device_id);
+int hip_device_count(int* count);
+int hip_malloc(void** ptr, size_t size);
+int hip_free(void* ptr);
+int hip_memcpy_h2d(void* dst, const void* src, size_t size);
+int hip_memcpy_d2h(void* dst, const void* src, size_t size);
+int hip_memcpy_d2d(void* dst, const void* src, size_t size);
+int hip_stream_create(void** stream);
+int hip_stream_destroy(void* stream);
+int hip_stream_synchronize(void* stream);
+int hip_set_stream(void* stream);       /* stream used by every later kernel/copy (NULL = default) */
+void* hip_get_stream(void);
+int hip_synchronize(void);              /* wait for everything queued on the backend's stream */
+
+/* ---- binary: replaces crates/maidenx_cuda/src/ops/binary.rs:12-161 --------------------------------
+ * metadata = dims[n] | lhs_strides[n] | rhs_strides[n] | lhs_offset | rhs_offset   (NULL: contiguous)
+ * Semantics: crates/maidenx_cpu/src/ops/binary.rs:13-124 (out-of-place, contiguous output),
+ * :126-248 (in place, written through the lhs strides), :250-368 (logical).
+ * div: b == 0 gives (a == 0 ? 0 : +INF). */
+#define MX_DECL_BINARY(T, S)                                                                              \
+    void hip_add_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, T* out);     \
+    void hip_sub_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, T* out);     \
+    void hip_mul_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, T* out);     \
+    void hip_div_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, T* out);     \
+    void hip_maximum_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, T* out); \
+    void hip_minimum_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, T* out); \
+    void hip_logical_and_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_logical_or_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out);  \
+    void hip_logical_xor_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_eq_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_ne_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_lt_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_le_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_gt_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_ge_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* lhs, const T* rhs, mx_bool* out); \
+    void hip_add_inplace_##S(size_t num_els, size_t num_dims, const size_t* metadata, T* lhs, const T* rhs); \
+    void hip_sub_inplace_##S(size_t num_els, size_t num_dims, const size_t* metadata, T* lhs, const T* rhs); \
+    void hip_mul_inplace_##S(size_t num_els, size_t num_dims, const size_t* metadata, T* lhs, const T* rhs); \
+    void hip_div_inplace_##S(size_t num_els, size_t num_dims, const size_t* metadata, T* lhs, const T* rhs);
+MX_DECL_BINARY(float, f32)
+MX_DECL_BINARY(mx_bf16, bf16)
+
+/* ---- unary: replaces crates/maidenx_cuda/src/ops/unary.rs:21-77 ------------------------------------
+ * metadata = dims[n] | strides[n] | offset   (NULL: contiguous).  input == NULL means "in place on
+ * output" (crates/maidenx_cuda/kernels/ops/unary.cu:20).  Semantics:
+ * crates/maidenx_cpu/src/ops/unary.rs:14-122; the constant has the input dtype. */
+#define MX_DECL_UNARY1(NAME, T, S, O) \
+    void hip_##NAME##_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* input, O* output);
+#define MX_DECL_UNARYC(NAME, T, S, O) \
+    void hip_##NAME##_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* input, T constant, O* output);
+#define MX_DECL_UNARY(T, S)                                                                                 \
+    MX_DECL_UNARY1(neg, T, S, T) MX_DECL_UNARY1(abs, T, S, T) MX_DECL_UNARY1(sign, T, S, T)                 \
+    MX_DECL_UNARY1(square, T, S, T) MX_DECL_UNARY1(sqrt, T, S, T) MX_DECL_UNARY1(relu, T, S, T)             \
+    MX_DECL_UNARY1(sigmoid, T, S, T) MX_DECL_UNARY1(tanh, T, S, T) MX_DECL_UNARY1(gelu, T, S, T)            \
+    MX_DECL_UNARY1(sin, T, S, T) MX_DECL_UNARY1(cos, T, S, T) MX_DECL_UNARY1(tan, T, S, T)                  \
+    MX_DECL_UNARY1(ln, T, S, T) MX_DECL_UNARY1(log10, T, S, T) MX_DECL_UNARY1(log2, T, S, T)                \
+    MX_DECL_UNARY1(exp, T, S, T) MX_DECL_UNARY1(exp10, T, S, T) MX_DECL_UNARY1(exp2, T, S, T)               \
+    MX_DECL_UNARY1(softplus, T, S, T) MX_DECL_UNARY1(recip, T, S, T) MX_DECL_UNARY1(logical_not, T, S, mx_bool) \
+    MX_DECL_UNARYC(add_scalar, T, S, T) MX_DECL_UNARYC(sub_scalar, T, S, T) MX_DECL_UNARYC(mul_scalar, T, S, T) \
+    MX_DECL_UNARYC(div_scalar, T, S, T) MX_DECL_UNARYC(maximum_scalar, T, S, T)                             \
+    MX_DECL_UNARYC(minimum_scalar, T, S, T) MX_DECL_UNARYC(pow, T, S, T) MX_DECL_UNARYC(leaky_relu, T, S, T) \
+    MX_DECL_UNARYC(elu, T, S, T) MX_DECL_UNARYC(eq_scalar, T, S, mx_bool) MX_DECL_UNARYC(ne_scalar, T, S, mx_bool) \
+    MX_DECL_UNARYC(lt_scalar, T, S, mx_bool) MX_DECL_UNARYC(le_scalar, T, S, mx_bool)                       \
+    MX_DECL_UNARYC(gt_scalar, T, S, mx_bool) MX_DECL_UNARYC(ge_scalar, T, S, mx_bool)
+MX_DECL_UNARY(float, f32)
+MX_DECL_UNARY(mx_bf16, bf16)
+
+/* ---- reduction: replaces crates/maidenx_cuda/src/ops/reduction.rs:19-35 ---------------------------
+ * sum/mean/max/min metadata = dims[n] | strides[n] | red_len[r] | red_stride[r] | offset, r = 1
+ * (the only value the tensor layer produces, crates/maidenx_tensor/src/ops/reduction.rs:38).
+ * sum_to_shape metadata = in_dims[n] | in_strides[n] | out_dims[n] | offset; every output dim is 1
+ * or the input dim.  Semantics: crates/maidenx_cpu/src/ops/reduction.rs:6-183, 185-272, 383-553
+ * (mean divides once at the end; max starts from f32::MIN, min from f32::MAX; NaNs never win).
+ * Accumulation is f32 in a fixed order; bf16 results are rounded once. */
+#define MX_DECL_REDUCE(T, S)                                                                                \
+    void hip_sum_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out);  \
+    void hip_mean_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out); \
+    void hip_max_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out);  \
+    void hip_min_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out);  \
+    void hip_sum_to_shape_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* inp, T* out);
+MX_DECL_REDUCE(float, f32)
+MX_DECL_REDUCE(mx_bf16, bf16)
+
+/* ---- matmul: replaces crates/maidenx_cuda/src/ops/matmul.rs:12-29 ---------------------------------
+ * metadata = out_ndim, a_ndim, b_ndim | out_shape | a_shape | b_shape | a_strides | b_strides | a_off | b_off
+ * Semantics: crates/maidenx_cpu/src/ops/matmul.rs:5-122 (forward; strided operands use strides[0]
+ * as the batch stride) and :124-268 (backward; contiguous indexing, either gradient may be NULL).
+ * f32 accumulate; bf16 results are rounded once. */
+#define MX_DECL_MATMUL(T, S)                                                                                \
+    void hip_matmul_##S(size_t num_els, const size_t* metadata, const T* a, const T* b, T* c);              \
+    void hip_matmul_backward_##S(size_t num_els_a, size_t num_els_b, const size_t* metadata, const T* grad_output, \
+                                 const T* a, const T* b, T* grad_a, T* grad_b);
+MX_DECL_MATMUL(float, f32)
+MX_DECL_MATMUL(mx_bf16, bf16)
+
+/* ---- padding: replaces crates/maidenx_cuda/src/ops/padding.rs:13-71 (constant mode) ---------------
+ * metadata = in_dims[n] | in_strides[n] | in_offset | out_dims[n] | (pad_before, pad_after)[n]
+ * Semantics: crates/maidenx_cpu/src/ops/padding.rs:7-113 and :327-436.  Bit-exact. */
+#define MX_DECL_PAD(T, S)                                                                                   \
+    void hip_pad_with_constant_##S(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, \
+                                   const T* inp, T* out, T pad_value);                                      \
+    void hip_pad_with_constant_backward_##S(size_t num_els_in, size_t num_els_out, size_t num_dims,         \
+                                            const size_t* metadata, const T* grad_out, T* grad_in);
+MX_DECL_PAD(float, f32)
+MX_DECL_PAD(mx_bf16, bf16)
+
+/* ---- conv: replaces crates/maidenx_cuda/src/nn/conv.rs:12-24 --------------------------------------
+ * metadata = 12 slots B, C, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w as the kernel
+ * reads them (crates/maidenx_cpu/src/nn/conv.rs:20-34).  im2col writes [B][C*kh*kw][oh*ow];
+ * col2im sums in the reference's order and skips column indices >= num_els (:135).  Bit-exact. */
+#define MX_DECL_CONV(T, S)                                                                                  \
+    void hip_conv2d_im2col_##S(size_t num_els, const size_t* metadata, const T* input, T* col);             \
+    void hip_conv2d_col2im_##S(size_t num_els, const size_t* metadata, const T* col, T* output);
+MX_DECL_CONV(float, f32)
+MX_DECL_CONV(mx_bf16, bf16)
+
+/* ---- device-side fill / convert / strided copy --------------------------------------------------
+ * No backend symbol exists for these in the reference: it builds host vectors
+ * (crates/maidenx_tensor/src/creation.rs:144-164), converts dtypes on the host
+ * (crates/maidenx_core/src/buffer/mod.rs:155-196) and makes views contiguous element by element
+ * (crates/maidenx_tensor/src/f.rs:19-30).  hip_copy_strided takes the unary metadata layout. */
+void hip_fill_f32(size_t num_els, float* out, float value);
+void hip_fill_bf16(size_t num_els, mx_bf16* out, mx_bf16 value);
+void hip_fill_bool(size_t num_els, mx_bool* out, mx_bool value);
+void hip_copy_strided_f32(size_t num_els, size_t num_dims, const size_t* metadata, const float* input, float* output);
+void hip_copy_strided_bf16(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bf16* input, mx_bf16* output);
+void hip_cast_bool_f32(size_t num_els, const mx_bool* input, float* output);
+void hip_cast_bool_bf16(size_t num_els, const mx_bool* input, mx_bf16* output);
+void hip_cast_f32_bf16(size_t num_els, const float* input, mx_bf16* output);
+void hip_cast_bf16_f32(size_t num_els, const mx_bf16* input, float* output);
+void hip_cast_f32_bool(size_t num_els, const float* input, mx_bool* output);
+void hip_cast_bf16_bool(size_t num_els, const mx_bf16* input, mx_bool* output);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAIDENX_HIP_H */

@@ -1,0 +1,57 @@
+"""ctypes signatures of the `<prefix><op>_<dtype>` symbol families declared in include/maidenx_hip.h.
+
+The same table describes the reference's CPU symbols (crates/maidenx_cpu/src/ops/*.rs), which have
+identical argument lists, so a CPU restatement built with another prefix can be bound with it too.
+"""
+import ctypes as C
+
+SZ, P = C.c_size_t, C.c_void_p
+CONST = {"f32": C.c_float, "f64": C.c_double, "bf16": C.c_uint16, "bool": C.c_uint8}
+
+BINARY = ["add", "sub", "mul", "div", "maximum", "minimum", "logical_and", "logical_or", "logical_xor",
+          "eq", "ne", "lt", "le", "gt", "ge"]
+INPLACE = ["add_inplace", "sub_inplace", "mul_inplace", "div_inplace"]
+UNARY = ["neg", "abs", "sign", "square", "sqrt", "relu", "sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln",
+         "log10", "log2", "exp", "exp10", "exp2", "softplus", "recip", "logical_not"]
+UNARY_CONST = ["add_scalar", "sub_scalar", "mul_scalar", "div_scalar", "maximum_scalar", "minimum_scalar", "pow",
+               "leaky_relu", "elu", "eq_scalar", "ne_scalar", "lt_scalar", "le_scalar", "gt_scalar", "ge_scalar"]
+REDUCE = ["sum", "mean", "max", "min"]
+BOOL_OUT = {"logical_and", "logical_or", "logical_xor", "eq", "ne", "lt", "le", "gt", "ge", "logical_not",
+            "eq_scalar", "ne_scalar", "lt_scalar", "le_scalar", "gt_scalar", "ge_scalar"}
+
+
+def signatures(dtypes=("f32", "bf16")):
+    """name (without prefix) -> argtypes list."""
+    sig = {}
+    for dt in dtypes:
+        c = CONST[dt]
+        for op in BINARY:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, P, P]
+        for op in INPLACE:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, P]
+        for op in UNARY:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, P]
+        for op in UNARY_CONST:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, c, P]
+        for op in REDUCE:
+            sig[f"{op}_{dt}"] = [SZ, SZ, SZ, P, P, P]
+        sig[f"sum_to_shape_{dt}"] = [SZ, SZ, P, P, P]
+        sig[f"matmul_{dt}"] = [SZ, P, P, P, P]
+        sig[f"matmul_backward_{dt}"] = [SZ, SZ, P, P, P, P, P, P]
+        sig[f"pad_with_constant_{dt}"] = [SZ, SZ, SZ, P, P, P, c]
+        sig[f"pad_with_constant_backward_{dt}"] = [SZ, SZ, SZ, P, P, P]
+        sig[f"conv2d_im2col_{dt}"] = [SZ, P, P, P]
+        sig[f"conv2d_col2im_{dt}"] = [SZ, P, P, P]
+    return sig
+
+
+def extension_signatures():
+    """Entry points of the HIP library that have no counterpart symbol in the reference."""
+    sig = {}
+    for dt in ("f32", "bf16", "bool"):
+        sig[f"fill_{dt}"] = [SZ, P, CONST[dt]]
+    for dt in ("f32", "bf16"):
+        sig[f"copy_strided_{dt}"] = [SZ, SZ, P, P, P]
+    for a, b in (("bool", "f32"), ("bool", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "bool"), ("bf16", "bool")):
+        sig[f"cast_{a}_{b}"] = [SZ, P, P]
+    return sig

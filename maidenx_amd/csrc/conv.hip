@@ -1,0 +1,138 @@
+// im2col / col2im.  Replace cuda_conv2d_im2col_<T> / cuda_conv2d_col2im_<T> of
+// crates/maidenx_cuda/src/nn/conv.rs:12-24 with the CPU semantics of
+// crates/maidenx_cpu/src/nn/conv.rs:13-149.
+// Metadata (12 slots, as the kernel reads them): B, C, H, W, kh, kw, oh, ow, pad_h, pad_w,
+// stride_h, stride_w.
+//   im2col : col[b][(c*kh+i)*kw+j][ho*ow+wo] = in[b,c,ho*sh-ph+i, wo*sw-pw+j] or 0.  Write-bound:
+//            each lane produces 4 consecutive wo of one column row and stores them as one
+//            128-bit vector (when ow % 4 == 0 and the buffer is aligned), the shifted input
+//            reads come from cache.
+//   col2im : gather form with the reference's fixed summation order (ho then wo ascending, at
+//            most kh*kw terms), so the result is bit-exact and deterministic; column indices at
+//            or beyond num_els are skipped exactly as the reference does.
+#include "mxh.hpp"
+
+namespace mxh {
+
+struct ConvMeta {
+    uint32_t B, C, H, W, kh, kw, oh, ow, ph, pw, sh, sw;
+    FastDiv d_owv, d_oh, d_kw, d_kh, d_C;      // im2col index walk
+    FastDiv d_W, d_H, d_Cc;                    // col2im index walk
+};
+
+constexpr int CB = 256;
+
+template <class T, int VEC>
+struct alignas(sizeof(T) * VEC) CVec { T v[VEC]; };
+
+template <class T, int VEC>
+__global__ __launch_bounds__(CB) void im2col_kernel(ConvMeta m, const T* __restrict__ in, T* __restrict__ col, size_t nvec,
+                                                    size_t num_els) {
+    size_t v = (size_t)blockIdx.x * CB + threadIdx.x;
+    if (v >= nvec) return;
+    uint32_t r = (uint32_t)v, wov, ho, j, i, c, b;
+    fd_divmod(r, m.d_owv, r, wov);
+    fd_divmod(r, m.d_oh, r, ho);
+    fd_divmod(r, m.d_kw, r, j);
+    fd_divmod(r, m.d_kh, r, i);
+    fd_divmod(r, m.d_C, b, c);
+    int hi = (int)(ho * m.sh) - (int)m.ph + (int)i;
+    const T* src = in + ((size_t)(b * m.C + c) * m.H + (hi >= 0 ? hi : 0)) * m.W;
+    bool hok = hi >= 0 && hi < (int)m.H;
+    CVec<T, VEC> o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        int wi = (int)((wov * VEC + e) * m.sw) - (int)m.pw + (int)j;
+        bool ok = hok && wi >= 0 && wi < (int)m.W;
+        o.v[e] = ok ? src[wi] : T{};
+    }
+    size_t base = v * VEC;
+    if (base + VEC <= num_els) *(CVec<T, VEC>*)(col + base) = o;
+    else
+        for (int e = 0; e < VEC; ++e) if (base + e < num_els) col[base + e] = o.v[e];
+}
+
+template <class T> __device__ inline T acc_add(T a, T b);
+template <> __device__ inline float acc_add<float>(float a, float b) { return a + b; }
+template <> __device__ inline bf16_t acc_add<bf16_t>(bf16_t a, bf16_t b) { return f2bf(bf2f(a) + bf2f(b)); }   // rounds per add
+
+template <class T>
+__global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restrict__ col, T* __restrict__ out, size_t n_out,
+                                                    size_t num_els) {
+    size_t idx = (size_t)blockIdx.x * CB + threadIdx.x;
+    if (idx >= n_out) return;
+    uint32_t r = (uint32_t)idx, w, h, c, b;
+    fd_divmod(r, m.d_W, r, w);
+    fd_divmod(r, m.d_H, r, h);
+    fd_divmod(r, m.d_Cc, b, c);
+    uint32_t h_pad = h + m.ph, w_pad = w + m.pw;
+    uint32_t hs = h_pad > m.kh - 1 ? h_pad - (m.kh - 1) : 0, ws = w_pad > m.kw - 1 ? w_pad - (m.kw - 1) : 0;
+    uint32_t h_start = (hs + m.sh - 1) / m.sh, w_start = (ws + m.sw - 1) / m.sw;
+    uint32_t h_end = min(h_pad / m.sh + 1, m.oh), w_end = min(w_pad / m.sw + 1, m.ow);
+    T sum = T{};
+    for (uint32_t ho = h_start; ho < h_end; ++ho)
+        for (uint32_t wo = w_start; wo < w_end; ++wo) {
+            uint32_t i = h_pad - ho * m.sh, j = w_pad - wo * m.sw;
+            if (i < m.kh && j < m.kw) {
+                size_t ci = ((((size_t)(b * m.C + c) * m.kh * m.kw + i * m.kw + j) * m.oh + ho) * m.ow) + wo;
+                if (ci < num_els) sum = acc_add<T>(sum, col[ci]);
+            }
+        }
+    out[idx] = sum;
+}
+
+static bool parse_conv(const size_t* md, ConvMeta& m) {
+    for (int k = 0; k < 12; ++k) if (md[k] >= (1ull << 31)) return false;
+    m.B = (uint32_t)md[0]; m.C = (uint32_t)md[1]; m.H = (uint32_t)md[2]; m.W = (uint32_t)md[3];
+    m.kh = (uint32_t)md[4]; m.kw = (uint32_t)md[5]; m.oh = (uint32_t)md[6]; m.ow = (uint32_t)md[7];
+    m.ph = (uint32_t)md[8]; m.pw = (uint32_t)md[9]; m.sh = (uint32_t)md[10]; m.sw = (uint32_t)md[11];
+    return m.sh != 0 && m.sw != 0 && m.kh != 0 && m.kw != 0;
+}
+
+template <class T>
+void im2col(size_t num_els, const size_t* md, const T* in, T* col) {
+    if (!md || !in || !col) return;    // the reference returns silently
+    ConvMeta m;
+    if (!parse_conv(md, m)) { set_status(ERR_INVALID, "im2col: bad metadata"); return; }
+    size_t full = (size_t)m.B * m.C * m.kh * m.kw * m.oh * m.ow;
+    if (full == 0 || num_els == 0) return;
+    if (full >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "im2col: 2^32 or more column elements"); return; }
+    size_t n = num_els < full ? num_els : full;
+    constexpr int VEC = 16 / sizeof(T);
+    bool vec = m.ow % VEC == 0 && ((uintptr_t)col % 16) == 0;
+    uint32_t owv = vec ? m.ow / VEC : m.ow;
+    m.d_owv = make_fastdiv(owv); m.d_oh = make_fastdiv(m.oh); m.d_kw = make_fastdiv(m.kw);
+    m.d_kh = make_fastdiv(m.kh); m.d_C = make_fastdiv(m.C);
+    size_t nvec = vec ? (n + VEC - 1) / VEC : n;
+    if (vec) hipLaunchKernelGGL((im2col_kernel<T, VEC>), dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, in, col, nvec, n);
+    else hipLaunchKernelGGL((im2col_kernel<T, 1>), dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, in, col, nvec, n);
+    MXH_LAUNCH_CHECK("im2col");
+}
+
+template <class T>
+void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
+    if (!md || !col || !out) return;
+    ConvMeta m;
+    if (!parse_conv(md, m)) { set_status(ERR_INVALID, "col2im: bad metadata"); return; }
+    size_t n_out = (size_t)m.B * m.C * m.H * m.W;
+    if (n_out == 0) return;
+    if (n_out >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "col2im: 2^32 or more output elements"); return; }
+    m.d_W = make_fastdiv(m.W); m.d_H = make_fastdiv(m.H); m.d_Cc = make_fastdiv(m.C);
+    hipLaunchKernelGGL(col2im_kernel<T>, dim3(cdiv(n_out, CB)), dim3(CB), 0, stream(), m, col, out, n_out, num_els);
+    MXH_LAUNCH_CHECK("col2im");
+}
+
+}  // namespace mxh
+
+using namespace mxh;
+
+#define MXH_CONV_FOR(T, SUF)                                                                               \
+    extern "C" void hip_conv2d_im2col_##SUF(size_t num_els, const size_t* md, const T* in, T* col) {       \
+        im2col<T>(num_els, md, in, col);                                                                   \
+    }                                                                                                      \
+    extern "C" void hip_conv2d_col2im_##SUF(size_t num_els, const size_t* md, const T* col, T* out) {      \
+        col2im<T>(num_els, md, col, out);                                                                  \
+    }
+
+MXH_CONV_FOR(float, f32)
+MXH_CONV_FOR(bf16_t, bf16)

@@ -1,0 +1,317 @@
+// Strided / broadcast elementwise engine: kernels and the host-side path selection.
+//
+// Every out-of-place op of the reference writes a contiguous output and reads its operands
+// through (dims, strides, offset) metadata; the in-place ops write through the lhs strides.
+// The host collapses the iteration space, then picks one of two kernels:
+//   ew_nd : each lane owns VEC consecutive elements of the innermost collapsed dim.  The
+//           logical→memory index walk (a few multiply-high divisions) is done once per
+//           lane-vector, operands with inner stride 1 move as one 128-bit access, operands
+//           with inner stride 0 as one scalar load.
+//   ew_tr : an operand whose unit stride sits on a non-innermost dim (a transposed view) is
+//           read along that dim in 64x64 tiles, turned through LDS, and consumed along the
+//           output's innermost dim, so both the read and the write stay coalesced.
+#pragma once
+#include "mxh.hpp"
+
+namespace mxh {
+
+template <class T, int N>
+struct alignas(sizeof(T) * N) AVec {
+    T v[N];
+};
+
+template <int NIN>
+struct EwPtrs {
+    void* out;
+    const void* in[NIN];
+};
+
+constexpr int EW_BLOCK = 256;
+constexpr int EW_UNR = 4;
+
+// ---- ew_nd -------------------------------------------------------------------------------
+template <class Op, int VEC>
+__global__ __launch_bounds__(EW_BLOCK) void ew_nd_kernel(NdSpace<Op::NIN + 1> sp, EwPtrs<Op::NIN> p, size_t nvec,
+                                                         Op op) {
+    using In = typename Op::In;
+    using Out = typename Op::Out;
+    constexpr int NIN = Op::NIN;
+    const int last = sp.ndims - 1;
+    size_t v0 = (size_t)blockIdx.x * (EW_BLOCK * EW_UNR) + threadIdx.x;
+
+    In vals[EW_UNR][NIN][VEC];
+    int64_t ooff[EW_UNR];
+#pragma unroll
+    for (int u = 0; u < EW_UNR; ++u) {
+        size_t v = v0 + (size_t)u * EW_BLOCK;
+        if (v >= nvec) break;
+        int64_t off[NIN + 1];
+        if (sp.ndims == 1) {
+            size_t i = v * VEC;
+#pragma unroll
+            for (int k = 0; k <= NIN; ++k) off[k] = (int64_t)i * sp.strides[k][0];
+        } else {
+            uint32_t r = (uint32_t)v * VEC;
+#pragma unroll
+            for (int k = 0; k <= NIN; ++k) off[k] = 0;
+            for (int d = last; d > 0; --d) {
+                uint32_t q, c;
+                fd_divmod(r, sp.div[d], q, c);
+#pragma unroll
+                for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)c * sp.strides[k][d];
+                r = q;
+            }
+#pragma unroll
+            for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * sp.strides[k][0];
+        }
+        ooff[u] = off[0];
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) {
+            const In* src = (const In*)p.in[k] + off[k + 1];
+            if constexpr (VEC == 1) {
+                vals[u][k][0] = src[0];
+            } else {
+                const int64_t s = sp.strides[k + 1][last];
+                if (s == 1) {
+                    AVec<In, VEC> t = *(const AVec<In, VEC>*)src;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) vals[u][k][e] = t.v[e];
+                } else if (s == 0) {
+                    In t = src[0];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) vals[u][k][e] = t;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) vals[u][k][e] = src[(int64_t)e * s];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < EW_UNR; ++u) {
+        size_t v = v0 + (size_t)u * EW_BLOCK;
+        if (v >= nvec) break;
+        AVec<Out, VEC> r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            if constexpr (NIN == 1) r.v[e] = op(vals[u][0][e]);
+            else r.v[e] = op(vals[u][0][e], vals[u][1][e]);
+        }
+        Out* dst = (Out*)p.out + ooff[u];
+        if constexpr (VEC == 1) {
+            dst[0] = r.v[0];
+        } else {
+            *(AVec<Out, VEC>*)dst = r;
+        }
+    }
+}
+
+// ---- ew_tr -------------------------------------------------------------------------------
+constexpr int TR_TILE = 64;
+
+template <int NIN>
+struct TrPlan {
+    int pdim;              // the dim on which the staged operands have stride 1
+    uint32_t staged;       // bit k set: input k goes through LDS
+    uint32_t tiles_p, tiles_l;
+    FastDiv div_tiles_l, div_tiles_p;
+};
+
+template <class Op>
+__global__ __launch_bounds__(EW_BLOCK) void ew_tr_kernel(NdSpace<Op::NIN + 1> sp, EwPtrs<Op::NIN> p, TrPlan<Op::NIN> pl,
+                                                         Op op) {
+    using In = typename Op::In;
+    using Out = typename Op::Out;
+    constexpr int NIN = Op::NIN;
+    __shared__ In tile[NIN][TR_TILE][TR_TILE + 1];
+
+    const int last = sp.ndims - 1;
+    const int pd = pl.pdim;
+    // blockIdx.x → (outer, tile_p, tile_l), tile_l fastest
+    uint32_t b = blockIdx.x, tl, tp, outer;
+    fd_divmod(b, pl.div_tiles_l, b, tl);
+    fd_divmod(b, pl.div_tiles_p, outer, tp);
+    int64_t base[NIN + 1];
+#pragma unroll
+    for (int k = 0; k <= NIN; ++k) base[k] = 0;
+    {
+        uint32_t r = outer;
+        for (int d = last - 1; d >= 0; --d) {
+            if (d == pd) continue;
+            uint32_t q, c;
+            fd_divmod(r, sp.div[d], q, c);
+#pragma unroll
+            for (int k = 0; k <= NIN; ++k) base[k] += (int64_t)c * sp.strides[k][d];
+            r = q;
+        }
+    }
+    const uint32_t i0 = tp * TR_TILE, j0 = tl * TR_TILE;   // i along pdim, j along the innermost dim
+    const uint32_t np = sp.dims[pd], nl = sp.dims[last];
+    const uint32_t tx = threadIdx.x % TR_TILE, ty = threadIdx.x / TR_TILE;
+    constexpr int ROWS = EW_BLOCK / TR_TILE;
+
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) {
+        if (!((pl.staged >> k) & 1u)) continue;
+        const In* src = (const In*)p.in[k] + base[k + 1];
+        const int64_t sl = sp.strides[k + 1][last];
+        for (uint32_t r = ty; r < TR_TILE; r += ROWS) {
+            uint32_t i = i0 + tx, j = j0 + r;
+            if (i < np && j < nl) tile[k][r][tx] = src[(int64_t)i + (int64_t)j * sl];
+        }
+    }
+    __syncthreads();
+    for (uint32_t r = ty; r < TR_TILE; r += ROWS) {
+        uint32_t i = i0 + r, j = j0 + tx;
+        if (i >= np || j >= nl) continue;
+        In x[NIN];
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) {
+            if ((pl.staged >> k) & 1u) x[k] = tile[k][tx][r];
+            else
+                x[k] = ((const In*)p.in[k])[base[k + 1] + (int64_t)i * sp.strides[k + 1][pd] +
+                                            (int64_t)j * sp.strides[k + 1][last]];
+        }
+        Out o;
+        if constexpr (NIN == 1) o = op(x[0]);
+        else o = op(x[0], x[1]);
+        ((Out*)p.out)[base[0] + (int64_t)i * sp.strides[0][pd] + (int64_t)j * sp.strides[0][last]] = o;
+    }
+}
+
+// ---- host-side selection -------------------------------------------------------------------
+// in_strides[k] / out_strides are in elements, pointers already include the operand offsets.
+template <class Op>
+void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t* out_strides,
+               const size_t* const* in_strides, void* out, const void* const* in, Op op) {
+    using In = typename Op::In;
+    using Out = typename Op::Out;
+    constexpr int NIN = Op::NIN;
+    if (num_els == 0) return;
+    NdSpace<NIN + 1> sp;
+    const size_t* strides[NIN + 1];
+    strides[0] = out_strides;
+    for (int k = 0; k < NIN; ++k) strides[k + 1] = in_strides[k];
+    if (!collapse<NIN + 1>(num_dims, dims, strides, sp)) {
+        set_status(ERR_UNSUPPORTED, "elementwise: collapsed rank above 8");
+        return;
+    }
+    if (sp.ndims > 1 && num_els >= (1ull << 31)) {
+        set_status(ERR_TOO_LARGE, "elementwise: strided op with 2^31 or more elements");
+        return;
+    }
+    EwPtrs<NIN> p;
+    p.out = out;
+    for (int k = 0; k < NIN; ++k) p.in[k] = in[k];
+    const int last = sp.ndims - 1;
+
+    // transposed-view path?
+    if (sp.ndims >= 2 && sp.strides[0][last] == 1 && sp.dims[last] >= 32) {
+        int pd = -1;
+        uint32_t staged = 0;
+        for (int k = 0; k < NIN; ++k) {
+            int64_t sl = sp.strides[k + 1][last];
+            if (sl == 0 || sl == 1) continue;
+            for (int d = 0; d < last; ++d)
+                if (sp.strides[k + 1][d] == 1 && sp.dims[d] >= 32 && (pd < 0 || pd == d)) {
+                    pd = d;
+                    staged |= 1u << k;
+                    break;
+                }
+        }
+        if (pd >= 0) {
+            TrPlan<NIN> pl;
+            pl.pdim = pd;
+            pl.staged = staged;
+            pl.tiles_p = cdiv(sp.dims[pd], TR_TILE);
+            pl.tiles_l = cdiv(sp.dims[last], TR_TILE);
+            pl.div_tiles_l = make_fastdiv(pl.tiles_l);
+            pl.div_tiles_p = make_fastdiv(pl.tiles_p);
+            size_t outer = 1;
+            for (int d = 0; d < last; ++d)
+                if (d != pd) outer *= sp.dims[d];
+            size_t blocks = outer * pl.tiles_p * pl.tiles_l;
+            hipLaunchKernelGGL(ew_tr_kernel<Op>, dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream(), sp, p, pl, op);
+            MXH_LAUNCH_CHECK("ew_tr");
+            return;
+        }
+    }
+
+    // vector width: 16 bytes of the wider of In/Out
+    constexpr int VEC = 16 / (sizeof(In) > sizeof(Out) ? sizeof(In) : sizeof(Out));
+    bool vec_ok = sp.strides[0][last] == 1 && sp.dims[last] % VEC == 0;
+    auto aligned = [&](const void* ptr, size_t esz, int k) {
+        if (((uintptr_t)ptr) % (esz * VEC) != 0) return false;
+        for (int d = 0; d < last; ++d)
+            if (sp.strides[k][d] % VEC != 0) return false;
+        return true;
+    };
+    if (vec_ok) vec_ok = aligned(out, sizeof(Out), 0);
+    for (int k = 0; k < NIN && vec_ok; ++k)
+        if (sp.strides[k + 1][last] == 1) vec_ok = aligned(in[k], sizeof(In), k + 1);
+    if (vec_ok) {
+        size_t nvec = num_els / VEC;
+        unsigned blocks = cdiv(nvec, EW_BLOCK * EW_UNR);
+        hipLaunchKernelGGL((ew_nd_kernel<Op, VEC>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, nvec, op);
+    } else {
+        unsigned blocks = cdiv(num_els, EW_BLOCK * EW_UNR);
+        hipLaunchKernelGGL((ew_nd_kernel<Op, 1>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, num_els, op);
+    }
+    MXH_LAUNCH_CHECK("ew_nd");
+}
+
+// ---- metadata adapters (layouts of the reference's tensor layer) ---------------------------
+// binary / in-place: dims[n] | lhs_strides[n] | rhs_strides[n] | lhs_offset | rhs_offset
+template <class Op>
+void ew_binary(size_t num_els, size_t num_dims, const size_t* md, const void* lhs, const void* rhs, void* out, Op op,
+               bool inplace) {
+    using In = typename Op::In;
+    if (num_els == 0) return;
+    if ((!inplace && !out) || !lhs || !rhs) { set_status(ERR_INVALID, "binary: null buffer"); return; }
+    size_t one = num_els, unit = 1;
+    const size_t *dims, *ls, *rs;
+    size_t lo = 0, ro = 0;
+    size_t cont[64];
+    if (md == nullptr) { dims = &one; ls = rs = &unit; num_dims = 1; }
+    else {
+        if (num_dims > 64) { set_status(ERR_INVALID, "binary: rank above 64"); return; }
+        dims = md; ls = md + num_dims; rs = md + 2 * num_dims;
+        lo = md[3 * num_dims]; ro = md[3 * num_dims + 1];
+    }
+    const In* l = (const In*)lhs + lo;
+    const In* r = (const In*)rhs + ro;
+    const size_t* ins[2] = {ls, rs};
+    const void* inp[2] = {l, r};
+    if (inplace) {
+        ew_launch<Op>(num_els, num_dims, dims, ls, ins, (void*)l, inp, op);
+    } else {
+        contiguous_strides(num_dims, dims, cont);
+        ew_launch<Op>(num_els, num_dims, dims, cont, ins, out, inp, op);
+    }
+}
+
+// unary (+constant): dims[n] | strides[n] | offset ; a null input means "in place on out".
+template <class Op>
+void ew_unary(size_t num_els, size_t num_dims, const size_t* md, const void* input, void* out, Op op) {
+    using In = typename Op::In;
+    if (num_els == 0) return;
+    if (!out) { set_status(ERR_INVALID, "unary: null output"); return; }
+    size_t one = num_els, unit = 1;
+    const size_t *dims, *st;
+    size_t off = 0;
+    size_t cont[64];
+    if (md == nullptr) { dims = &one; st = &unit; num_dims = 1; }
+    else {
+        if (num_dims > 64) { set_status(ERR_INVALID, "unary: rank above 64"); return; }
+        dims = md; st = md + num_dims; off = md[2 * num_dims];
+    }
+    contiguous_strides(num_dims, dims, cont);
+    const void* src;
+    const size_t* ins[1];
+    if (input == nullptr) { src = out; ins[0] = cont; }
+    else { src = (const In*)input + off; ins[0] = st; }
+    const void* inp[1] = {src};
+    ew_launch<Op>(num_els, num_dims, dims, cont, ins, out, inp, op);
+}
+
+}  // namespace mxh

@@ -1,0 +1,40 @@
+// extern "C" entry points of the unary families (plain, with a by-value constant, and the
+// bool-producing forms).  Each replaces the `cuda_<op>_<dtype>` symbol of
+// crates/maidenx_cuda/src/ops/unary.rs:21-77; a null input means "in place on the output"
+// (crates/maidenx_cuda/kernels/ops/unary.cu:20).
+#include "elementwise.hpp"
+#include "ops.hpp"
+
+using namespace mxh;
+
+#define MXH_UNARY(NAME, OP, T, SUF, O)                                                                        \
+    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, O* out) { \
+        ew_unary(num_els, num_dims, md, in, out, OP<T>{});                                                    \
+    }
+#define MXH_UNARY_C(NAME, OP, T, SUF, O)                                                                      \
+    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, T c,   \
+                                       O* out) {                                                              \
+        ew_unary(num_els, num_dims, md, in, out, OP<T>{c});                                                   \
+    }
+
+#define MXH_ALL_FOR(T, SUF)                                                                                   \
+    MXH_UNARY(neg, OpNeg, T, SUF, T) MXH_UNARY(abs, OpAbs, T, SUF, T) MXH_UNARY(sign, OpSign, T, SUF, T)      \
+    MXH_UNARY(square, OpSquare, T, SUF, T) MXH_UNARY(sqrt, OpSqrt, T, SUF, T)                                 \
+    MXH_UNARY(relu, OpRelu, T, SUF, T) MXH_UNARY(sigmoid, OpSigmoid, T, SUF, T)                               \
+    MXH_UNARY(tanh, OpTanh, T, SUF, T) MXH_UNARY(gelu, OpGelu, T, SUF, T)                                     \
+    MXH_UNARY(sin, OpSin, T, SUF, T) MXH_UNARY(cos, OpCos, T, SUF, T) MXH_UNARY(tan, OpTan, T, SUF, T)        \
+    MXH_UNARY(ln, OpLn, T, SUF, T) MXH_UNARY(log10, OpLog10, T, SUF, T) MXH_UNARY(log2, OpLog2, T, SUF, T)    \
+    MXH_UNARY(exp, OpExp, T, SUF, T) MXH_UNARY(exp10, OpExp10, T, SUF, T) MXH_UNARY(exp2, OpExp2, T, SUF, T)  \
+    MXH_UNARY(softplus, OpSoftplus, T, SUF, T) MXH_UNARY(recip, OpRecip, T, SUF, T)                           \
+    MXH_UNARY(logical_not, OpLogicalNot, T, SUF, bool_t)                                                      \
+    MXH_UNARY_C(add_scalar, OpAddScalar, T, SUF, T) MXH_UNARY_C(sub_scalar, OpSubScalar, T, SUF, T)           \
+    MXH_UNARY_C(mul_scalar, OpMulScalar, T, SUF, T) MXH_UNARY_C(div_scalar, OpDivScalar, T, SUF, T)           \
+    MXH_UNARY_C(maximum_scalar, OpMaximumScalar, T, SUF, T) MXH_UNARY_C(minimum_scalar, OpMinimumScalar, T, SUF, T) \
+    MXH_UNARY_C(pow, OpPow, T, SUF, T) MXH_UNARY_C(leaky_relu, OpLeakyRelu, T, SUF, T)                        \
+    MXH_UNARY_C(elu, OpElu, T, SUF, T)                                                                        \
+    MXH_UNARY_C(eq_scalar, OpEqScalar, T, SUF, bool_t) MXH_UNARY_C(ne_scalar, OpNeScalar, T, SUF, bool_t)     \
+    MXH_UNARY_C(lt_scalar, OpLtScalar, T, SUF, bool_t) MXH_UNARY_C(le_scalar, OpLeScalar, T, SUF, bool_t)     \
+    MXH_UNARY_C(gt_scalar, OpGtScalar, T, SUF, bool_t) MXH_UNARY_C(ge_scalar, OpGeScalar, T, SUF, bool_t)
+
+MXH_ALL_FOR(float, f32)
+MXH_ALL_FOR(bf16_t, bf16)

@@ -1,0 +1,137 @@
+// Element functions of the backend, written against the reference's CPU semantics
+// (crates/maidenx_cpu/src/ops/{binary,unary}.rs).  f32 evaluates every step in f32 with no
+// fused multiply-add (the translation unit is built with -ffp-contract=off); bf16 follows the
+// `half` crate: arithmetic forms round after every operation, transcendental forms upcast,
+// evaluate in f32 and round once.
+#pragma once
+#include "mathfn.hpp"
+#include "mxh.hpp"
+
+namespace mxh {
+
+using bool_t = uint8_t;   // the reference's `bool` output buffers: one byte, 0 or 1
+
+template <class T> struct Ar;
+template <> struct Ar<float> {
+    using T = float;
+    static __device__ T zero() { return 0.0f; }
+    static __device__ T inf() { return INFINITY; }
+    static __device__ T from_f32(float v) { return v; }
+    static __device__ float to_f32(T v) { return v; }
+    static __device__ T add(T a, T b) { return a + b; }
+    static __device__ T sub(T a, T b) { return a - b; }
+    static __device__ T mul(T a, T b) { return a * b; }
+    static __device__ T div(T a, T b) { return a / b; }
+    static __device__ T neg(T a) { return -a; }
+    static __device__ T max_(T a, T b) { return fmaxf(a, b); }   // f32::max — a NaN operand is ignored
+    static __device__ T min_(T a, T b) { return fminf(a, b); }
+};
+template <> struct Ar<bf16_t> {
+    using T = bf16_t;
+    static __device__ T zero() { return T{0}; }
+    static __device__ T inf() { return T{0x7F80}; }
+    static __device__ T from_f32(float v) { return f2bf(v); }
+    static __device__ float to_f32(T v) { return bf2f(v); }
+    static __device__ T add(T a, T b) { return f2bf(bf2f(a) + bf2f(b)); }
+    static __device__ T sub(T a, T b) { return f2bf(bf2f(a) - bf2f(b)); }
+    static __device__ T mul(T a, T b) { return f2bf(bf2f(a) * bf2f(b)); }
+    static __device__ T div(T a, T b) { return f2bf(bf2f(a) / bf2f(b)); }
+    static __device__ T neg(T a) { return T{(uint16_t)(a.bits ^ 0x8000u)}; }
+    static __device__ T max_(T a, T b) { return bf2f(a) > bf2f(b) ? a : b; }   // `if a > b { a } else { b }`
+    static __device__ T min_(T a, T b) { return bf2f(a) < bf2f(b) ? a : b; }
+};
+template <class T> __device__ inline float F(T v) { return Ar<T>::to_f32(v); }
+template <class T> __device__ inline bool is_zero(T v) { return F(v) == 0.0f; }
+
+// ---- binary --------------------------------------------------------------------------------
+#define MXH_BIN(NAME, OUT, EXPR)                                          \
+    template <class T> struct NAME {                                      \
+        using In = T; using Out = OUT; static constexpr int NIN = 2;      \
+        __device__ Out operator()(T a, T b) const { using A = Ar<T>; (void)sizeof(A); return EXPR; } \
+    };
+MXH_BIN(OpAdd, T, A::add(a, b))
+MXH_BIN(OpSub, T, A::sub(a, b))
+MXH_BIN(OpMul, T, A::mul(a, b))
+// b == 0 ⇒ (a == 0 ? 0 : +INF) — the sign of a is ignored and a NaN a gives +INF
+MXH_BIN(OpDiv, T, is_zero(b) ? (is_zero(a) ? A::zero() : A::inf()) : A::div(a, b))
+MXH_BIN(OpMaximum, T, A::max_(a, b))
+MXH_BIN(OpMinimum, T, A::min_(a, b))
+MXH_BIN(OpLogicalAnd, bool_t, (bool_t)(!is_zero(a) && !is_zero(b)))
+MXH_BIN(OpLogicalOr, bool_t, (bool_t)(!is_zero(a) || !is_zero(b)))
+MXH_BIN(OpLogicalXor, bool_t, (bool_t)(!is_zero(a) != !is_zero(b)))
+MXH_BIN(OpEq, bool_t, (bool_t)(F(a) == F(b)))
+MXH_BIN(OpNe, bool_t, (bool_t)(F(a) != F(b)))
+MXH_BIN(OpLt, bool_t, (bool_t)(F(a) < F(b)))
+MXH_BIN(OpLe, bool_t, (bool_t)(F(a) <= F(b)))
+MXH_BIN(OpGt, bool_t, (bool_t)(F(a) > F(b)))
+MXH_BIN(OpGe, bool_t, (bool_t)(F(a) >= F(b)))
+
+// ---- unary ---------------------------------------------------------------------------------
+// EXPR_F sees `x` as f32 and yields f32 (rounded once for bf16); EXPR_T, when given, works on
+// the storage type with per-operation rounding.
+#define MXH_UN_F(NAME, EXPR_F)                                            \
+    template <class T> struct NAME {                                      \
+        using In = T; using Out = T; static constexpr int NIN = 1;        \
+        __device__ T operator()(T v) const { float x = F(v); return Ar<T>::from_f32(EXPR_F); } \
+    };
+#define MXH_UN_T(NAME, EXPR_T)                                            \
+    template <class T> struct NAME {                                      \
+        using In = T; using Out = T; static constexpr int NIN = 1;        \
+        __device__ T operator()(T x) const { using A = Ar<T>; (void)sizeof(A); return EXPR_T; } \
+    };
+
+__device__ inline float gelu_f32(float x) {
+    const float sqrt_2_over_pi = 0.7978845608028654f, coeff = 0.044715f;
+    float tanh_arg = sqrt_2_over_pi * (x + coeff * x * x * x);
+    return 0.5f * x * (1.0f + m_tanh(tanh_arg));
+}
+
+MXH_UN_T(OpNeg, A::neg(x))
+MXH_UN_F(OpAbs, fabsf(x))
+MXH_UN_F(OpSign, x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : 0.0f))
+MXH_UN_T(OpSquare, A::mul(x, x))
+MXH_UN_F(OpSqrt, sqrtf(x))
+MXH_UN_T(OpRelu, F(x) > 0.0f ? x : A::zero())          // NaN → 0, −0 → +0
+MXH_UN_F(OpSigmoid, 1.0f / (1.0f + m_exp(-x)))
+MXH_UN_F(OpTanh, m_tanh(x))
+MXH_UN_F(OpGelu, gelu_f32(x))
+MXH_UN_F(OpSin, m_sin(x))
+MXH_UN_F(OpCos, m_cos(x))
+MXH_UN_F(OpTan, m_tan(x))
+MXH_UN_F(OpLn, m_ln(x))
+MXH_UN_F(OpLog10, m_log10(x))
+MXH_UN_F(OpLog2, m_log2(x))
+MXH_UN_F(OpExp, m_exp(x))
+MXH_UN_F(OpExp10, m_pow(10.0f, x))
+MXH_UN_F(OpExp2, m_exp2(x))
+MXH_UN_F(OpSoftplus, m_ln(1.0f + m_exp(x)))
+MXH_UN_F(OpRecip, 1.0f / x)
+template <class T> struct OpLogicalNot {
+    using In = T; using Out = bool_t; static constexpr int NIN = 1;
+    __device__ bool_t operator()(T x) const { return (bool_t)is_zero(x); }
+};
+
+// ---- unary with a constant of the input dtype --------------------------------------------------
+#define MXH_UNC(NAME, OUT, EXPR)                                          \
+    template <class T> struct NAME {                                      \
+        using In = T; using Out = OUT; static constexpr int NIN = 1;      \
+        T c;                                                              \
+        __device__ Out operator()(T x) const { using A = Ar<T>; (void)sizeof(A); return EXPR; } \
+    };
+MXH_UNC(OpAddScalar, T, A::add(x, c))
+MXH_UNC(OpSubScalar, T, A::sub(x, c))
+MXH_UNC(OpMulScalar, T, A::mul(x, c))
+MXH_UNC(OpDivScalar, T, is_zero(c) ? (is_zero(x) ? A::zero() : A::inf()) : A::div(x, c))
+MXH_UNC(OpMaximumScalar, T, A::max_(x, c))
+MXH_UNC(OpMinimumScalar, T, A::min_(x, c))
+MXH_UNC(OpPow, T, A::from_f32(m_pow(F(x), F(c))))                      // powf even for c = 2
+MXH_UNC(OpLeakyRelu, T, F(x) > 0.0f ? x : A::mul(c, x))
+MXH_UNC(OpElu, T, F(x) > 0.0f ? x : A::from_f32(F(c) * (m_exp(F(x)) - 1.0f)))
+MXH_UNC(OpEqScalar, bool_t, (bool_t)(F(x) == F(c)))
+MXH_UNC(OpNeScalar, bool_t, (bool_t)(F(x) != F(c)))
+MXH_UNC(OpLtScalar, bool_t, (bool_t)(F(x) < F(c)))
+MXH_UNC(OpLeScalar, bool_t, (bool_t)(F(x) <= F(c)))
+MXH_UNC(OpGtScalar, bool_t, (bool_t)(F(x) > F(c)))
+MXH_UNC(OpGeScalar, bool_t, (bool_t)(F(x) >= F(c)))
+
+}  // namespace mxh

@@ -1,0 +1,142 @@
+// Constant padding, forward and backward.  Replaces cuda_pad_with_constant_<T> and
+// cuda_pad_with_constant_backward_<T> of crates/maidenx_cuda/src/ops/padding.rs:13-71 with the
+// CPU semantics of crates/maidenx_cpu/src/ops/padding.rs:7-113 and :327-436.
+// Metadata: in_dims[n] | in_strides[n] | in_offset | out_dims[n] | (pad_before, pad_after)[n]
+// Pure data movement, bit-exact.  One lane per output element; the coordinate walk uses
+// multiply-high division on the collapsed shape (dims without padding whose input strides chain
+// are merged, so [B,C,H,W] padded on H,W walks two divisions, not four).
+#include "mxh.hpp"
+
+namespace mxh {
+
+struct PadSpace {
+    int ndims;
+    uint32_t out_dims[MAXD];
+    uint32_t in_dims[MAXD];
+    uint32_t before[MAXD];
+    FastDiv div[MAXD];
+    int64_t in_strides[MAXD];
+};
+
+constexpr int PB = 256;
+
+// forward: out[i] = inside ? in[idx] : pad_value
+// backward (GATHER = false): grad_in[idx] = 0 + grad_out[i] for every inside i
+template <class T, bool FWD>
+__global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __restrict__ src, T* __restrict__ dst,
+                                                       size_t n_out, T pad_value) {
+    size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
+    if (i >= n_out) return;
+    uint32_t r = (uint32_t)i;
+    int64_t idx = 0;
+    bool inside = true;
+    for (int d = sp.ndims - 1; d >= 0; --d) {
+        uint32_t q, c;
+        if (d > 0) fd_divmod(r, sp.div[d], q, c);
+        else { q = 0; c = r; }
+        uint32_t ic = c - sp.before[d];               // wraps when c < before → fails the test below
+        inside = inside && ic < sp.in_dims[d];
+        idx += (int64_t)ic * sp.in_strides[d];
+        r = q;
+    }
+    if constexpr (FWD) {
+        dst[i] = inside ? src[idx] : pad_value;
+    } else {
+        if (inside) {
+            T g = src[i];
+            if constexpr (sizeof(T) == 4) dst[idx] = 0.0f + g;            // −0 → +0 like the reference's sums from zero
+            else dst[idx] = f2bf(0.0f + bf2f(g));
+        }
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(PB) void zero_kernel(T* p, size_t n) {
+    size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
+    if (i < n) p[i] = T{};
+}
+
+static bool build_space(size_t nd, const size_t* md, PadSpace& sp, size_t* in_off, bool* cont, bool* exact) {
+    const size_t* in_dims = md;
+    const size_t* in_strides = md + nd;
+    *in_off = md[2 * nd];
+    const size_t* out_dims = md + 2 * nd + 1;
+    const size_t* pads = md + 3 * nd + 1;
+    *cont = ref_is_contiguous(nd, in_dims, in_strides);
+    size_t cs[64];
+    if (nd > 64) return false;
+    contiguous_strides(nd, in_dims, cs);
+    const size_t* st = *cont ? cs : in_strides;     // padding.rs:76-93: contiguous inputs are indexed row-major
+    *exact = true;
+    int n = 0;
+    uint64_t od[64], id[64], bf[64];
+    int64_t is[64];
+    for (size_t d = 0; d < nd; ++d) {
+        if (out_dims[d] != in_dims[d] + pads[2 * d] + pads[2 * d + 1]) *exact = false;
+        bool plain = pads[2 * d] == 0 && out_dims[d] == in_dims[d];
+        if (plain && in_dims[d] == 1) continue;
+        // merge a pad-free dim into its (pad-free) outer neighbour when the input strides chain
+        if (n > 0 && plain && bf[n - 1] == 0 && od[n - 1] == id[n - 1] && (uint64_t)is[n - 1] == st[d] * in_dims[d]) {
+            od[n - 1] *= out_dims[d]; id[n - 1] *= in_dims[d]; is[n - 1] = (int64_t)st[d];
+        } else {
+            od[n] = out_dims[d]; id[n] = in_dims[d]; bf[n] = pads[2 * d]; is[n] = (int64_t)st[d]; ++n;
+        }
+    }
+    if (n == 0) { od[0] = id[0] = 1; bf[0] = 0; is[0] = 1; n = 1; }
+    if (n > MAXD) return false;
+    sp.ndims = n;
+    for (int d = 0; d < MAXD; ++d) {
+        sp.out_dims[d] = d < n ? (uint32_t)od[d] : 1;
+        sp.in_dims[d] = d < n ? (uint32_t)id[d] : 1;
+        sp.before[d] = d < n ? (uint32_t)bf[d] : 0;
+        sp.in_strides[d] = d < n ? is[d] : 0;
+        sp.div[d] = make_fastdiv(sp.out_dims[d]);
+    }
+    return true;
+}
+
+template <class T>
+void pad_forward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const T* in, T* out, T pad_value) {
+    (void)n_in;
+    if (!md || !in || !out) { set_status(ERR_INVALID, "pad: null argument"); return; }
+    if (n_out == 0) return;
+    if (n_out >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad: output of 2^31 or more elements"); return; }
+    PadSpace sp; size_t off; bool cont, exact;
+    if (!build_space(nd, md, sp, &off, &cont, &exact)) { set_status(ERR_UNSUPPORTED, "pad: rank above 8 after collapse"); return; }
+    hipLaunchKernelGGL((pad_const_kernel<T, true>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
+    MXH_LAUNCH_CHECK("pad_const");
+}
+
+template <class T>
+void pad_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const T* go, T* gi) {
+    if (!md || !go || !gi) { set_status(ERR_INVALID, "pad_backward: null argument"); return; }
+    if (n_out >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad_backward: 2^31 or more elements"); return; }
+    PadSpace sp; size_t off; bool cont, exact;
+    if (!build_space(nd, md, sp, &off, &cont, &exact)) { set_status(ERR_UNSUPPORTED, "pad_backward: rank above 8 after collapse"); return; }
+    // The reference writes num_els_in contiguous elements at grad_in + offset; positions no
+    // output element maps to hold 0.  With a contiguous input and out = in + pads every position is hit.
+    if (!(cont && exact) && n_in) {
+        hipLaunchKernelGGL(zero_kernel<T>, dim3(cdiv(n_in, PB)), dim3(PB), 0, stream(), gi + off, n_in);
+        MXH_LAUNCH_CHECK("pad_zero");
+    }
+    if (n_out == 0) return;
+    hipLaunchKernelGGL((pad_const_kernel<T, false>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
+    MXH_LAUNCH_CHECK("pad_const_backward");
+}
+
+}  // namespace mxh
+
+using namespace mxh;
+
+#define MXH_PAD_FOR(T, SUF)                                                                                  \
+    extern "C" void hip_pad_with_constant_##SUF(size_t n_in, size_t n_out, size_t nd, const size_t* md,      \
+                                                const T* in, T* out, T pad_value) {                          \
+        pad_forward<T>(n_in, n_out, nd, md, in, out, pad_value);                                             \
+    }                                                                                                        \
+    extern "C" void hip_pad_with_constant_backward_##SUF(size_t n_in, size_t n_out, size_t nd,               \
+                                                         const size_t* md, const T* go, T* gi) {             \
+        pad_backward<T>(n_in, n_out, nd, md, go, gi);                                                        \
+    }
+
+MXH_PAD_FOR(float, f32)
+MXH_PAD_FOR(bf16_t, bf16)

@@ -1,0 +1,463 @@
+// Reductions: sum / mean / max / min along one axis and sum_to_shape.  They replace the
+// `cuda_<op>_<dtype>` symbols of crates/maidenx_cuda/src/ops/reduction.rs:19-35 and follow the
+// CPU semantics of crates/maidenx_cpu/src/ops/reduction.rs.
+//
+// A contiguous input reduced along one axis is the 3-d problem [outer, L, S] → [outer, S]:
+//   S == 1 : "row" reduce.  One thread, one wave or one block per row (by row length); lanes
+//            read 128-bit vectors, partial sums meet in a wave64 DPP butterfly and then in LDS.
+//   S  > 1 : "column" reduce.  Lanes run along S (coalesced, 128-bit where alignment allows)
+//            and walk L; when outer*S alone cannot fill the chip, L is cut into chunks whose
+//            partial results go to library scratch and are folded by a second launch.
+// Accumulation is f32 in a fixed order (deterministic from run to run); bf16 is rounded once.
+// No atomics anywhere.
+#include <cfloat>
+
+#include "elementwise.hpp"
+#include "mxh.hpp"
+
+namespace mxh {
+
+// ---- reducers -------------------------------------------------------------------------------
+struct RSum {
+    static __device__ float init(bool) { return 0.0f; }
+    static __device__ float op(float a, float b) { return a + b; }
+};
+// `if val > out { val } else { out }` from f32::MIN: NaNs never win, −inf does not beat the seed.
+struct RMax {
+    static __device__ float init(bool is_bf16) { return is_bf16 ? -INFINITY : -FLT_MAX; }   // bf16(f32::MIN) is −inf
+    static __device__ float op(float a, float b) { return b > a ? b : a; }
+};
+struct RMin {
+    static __device__ float init(bool is_bf16) { return is_bf16 ? INFINITY : FLT_MAX; }
+    static __device__ float op(float a, float b) { return b < a ? b : a; }
+};
+
+template <class T> struct IO;
+template <> struct IO<float> {
+    static constexpr bool is_bf16 = false;
+    static __device__ float ld(float v) { return v; }
+    // div != 0: the mean's single division at the end (reduction.rs:264-268)
+    static __device__ float fin(float acc, float div) { return div != 0.0f ? acc / div : acc; }
+};
+template <> struct IO<bf16_t> {
+    static constexpr bool is_bf16 = true;
+    static __device__ float ld(bf16_t v) { return bf2f(v); }
+    static __device__ bf16_t fin(float acc, float div) {
+        bf16_t s = f2bf(acc);
+        return div != 0.0f ? f2bf(bf2f(s) / bf2f(f2bf(div))) : s;
+    }
+};
+
+// ---- wave64 butterfly on DPP ------------------------------------------------------------------
+template <class R, int CTRL>
+__device__ inline float dpp_combine(float v) {
+    int iv = __builtin_bit_cast(int, v);
+    int ov = __builtin_amdgcn_update_dpp(iv, iv, CTRL, 0xF, 0xF, false);
+    return R::op(v, __builtin_bit_cast(float, ov));
+}
+// After this every lane of a 16-lane row holds the row's result; the four rows are then
+// combined in a fixed order through readlane.
+template <class R>
+__device__ inline float wave_reduce(float v) {
+    v = dpp_combine<R, 0xB1>(v);    // quad_perm [1,0,3,2]
+    v = dpp_combine<R, 0x4E>(v);    // quad_perm [2,3,0,1]
+    v = dpp_combine<R, 0x141>(v);   // row_half_mirror
+    v = dpp_combine<R, 0x140>(v);   // row_mirror
+    int iv = __builtin_bit_cast(int, v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+    return R::op(R::op(r0, r1), R::op(r2, r3));
+}
+
+constexpr int RB = 256;
+
+// ---- row reduce: [rows, L] → [rows, chunks] ---------------------------------------------------
+// TPR threads cooperate on one (row, chunk).  VEC > 1 requires L % VEC == 0, chunk_len % VEC == 0
+// and a 16-byte aligned base.
+template <class TIn, class TOut, class R, int TPR, int VEC>
+__global__ __launch_bounds__(RB) void row_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t rows,
+                                                        size_t L, unsigned chunks, size_t chunk_len, float div,
+                                                        bool src_bf16) {
+    constexpr int RPB = RB / TPR;
+    size_t unit = (size_t)blockIdx.x * RPB + threadIdx.x / TPR;   // (row, chunk) pair
+    const unsigned t = threadIdx.x % TPR;
+    size_t total = rows * chunks;
+    float acc = R::init(src_bf16);
+    if (unit < total) {
+        size_t row = unit / chunks, chunk = unit % chunks;
+        size_t beg = chunk * chunk_len, end = beg + chunk_len < L ? beg + chunk_len : L;
+        const TIn* src = in + row * L;
+        if constexpr (VEC > 1) {
+            float a[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) a[e] = R::init(src_bf16);
+            for (size_t i = beg + (size_t)t * VEC; i < end; i += (size_t)TPR * VEC) {
+                AVec<TIn, VEC> v = *(const AVec<TIn, VEC>*)(src + i);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v.v[e]));
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc = R::op(acc, a[e]);
+        } else {
+            for (size_t i = beg + t; i < end; i += TPR) acc = R::op(acc, IO<TIn>::ld(src[i]));
+        }
+    }
+    if constexpr (TPR >= WAVE) acc = wave_reduce<R>(acc);
+    if constexpr (TPR > WAVE) {
+        __shared__ float part[RB / WAVE];
+        if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = acc;
+        __syncthreads();
+        acc = part[0];
+#pragma unroll
+        for (int w = 1; w < RB / WAVE; ++w) acc = R::op(acc, part[w]);
+    }
+    if (t == 0 && unit < total) out[unit] = IO<TOut>::fin(acc, div);
+}
+
+// ---- column reduce: [outer, L, S] → [outer, chunks, S] ------------------------------------------
+template <class TIn, class TOut, class R, int VEC>
+__global__ __launch_bounds__(RB) void col_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t outer,
+                                                        size_t L, size_t S, unsigned chunks, size_t chunk_len,
+                                                        FastDiv div_sv, FastDiv div_chunks, size_t total, float div,
+                                                        bool src_bf16) {
+    size_t tid = (size_t)blockIdx.x * RB + threadIdx.x;
+    if (tid >= total) return;
+    // tid → (o, chunk, jv), jv fastest.  total < 2^32 is checked by the host.
+    uint32_t rest, jv, o, chunk;
+    fd_divmod((uint32_t)tid, div_sv, rest, jv);
+    fd_divmod(rest, div_chunks, o, chunk);
+    size_t beg = (size_t)chunk * chunk_len, end = beg + chunk_len < L ? beg + chunk_len : L;
+    const TIn* src = in + ((size_t)o * L + beg) * S + (size_t)jv * VEC;
+    float a[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) a[e] = R::init(src_bf16);
+#pragma unroll 8
+    for (size_t l = beg; l < end; ++l, src += S) {
+        AVec<TIn, VEC> v = *(const AVec<TIn, VEC>*)src;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v.v[e]));
+    }
+    AVec<TOut, VEC> r;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) r.v[e] = IO<TOut>::fin(a[e], div);
+    *(AVec<TOut, VEC>*)(out + ((size_t)o * chunks + chunk) * S + (size_t)jv * VEC) = r;
+}
+
+// ---- generic single-axis reduce over a strided input (the reference's non-contiguous branch) ----
+// One thread per output element d; its inputs are the logical indices ((d/s)*L + l)*s + d%s
+// (s = the metadata's reduced stride, or d*L + l when that stride is 0), each mapped through the
+// strides the way get_strided_index does.
+template <class T, class R>
+__global__ __launch_bounds__(RB) void reduce_generic_kernel(NdSpace<1> sp, const T* __restrict__ in, T* __restrict__ out,
+                                                            size_t num_els, size_t out_size, size_t L, size_t s,
+                                                            float div) {
+    size_t d = (size_t)blockIdx.x * RB + threadIdx.x;
+    if (d >= out_size) return;
+    float acc = R::init(IO<T>::is_bf16);
+    for (size_t l = 0; l < L; ++l) {
+        size_t i = s != 0 ? ((d / s) * L + l) * s + d % s : d * L + l;
+        if (i >= num_els) continue;
+        uint32_t r = (uint32_t)i;
+        int64_t off = 0;
+        for (int k = sp.ndims - 1; k > 0; --k) {
+            uint32_t q, c;
+            fd_divmod(r, sp.div[k], q, c);
+            off += (int64_t)c * sp.strides[0][k];
+            r = q;
+        }
+        off += (int64_t)r * sp.strides[0][0];
+        acc = R::op(acc, IO<T>::ld(in[off]));
+    }
+    out[d] = IO<T>::fin(acc, div);
+}
+
+// ---- host drivers ---------------------------------------------------------------------------------
+constexpr size_t TARGET_BLOCKS = 2048;   // 256 CUs x 8 resident blocks
+
+template <class T> inline bool aligned16(const T* p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <class TIn, class TOut, class R, int TPR>
+void launch_row(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks, size_t chunk_len, float div,
+                bool src_bf16) {
+    constexpr int VEC = 16 / sizeof(TIn);
+    constexpr int RPB = RB / TPR;
+    unsigned blocks = cdiv(rows * chunks, RPB);
+    bool vec = aligned16(in) && L % VEC == 0 && chunk_len % VEC == 0;
+    if (vec)
+        hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, TPR, VEC>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows,
+                           L, chunks, chunk_len, div, src_bf16);
+    else
+        hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, TPR, 1>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows,
+                           L, chunks, chunk_len, div, src_bf16);
+    MXH_LAUNCH_CHECK("row_reduce");
+}
+
+template <class TIn, class TOut, class R>
+void row_stage(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks, size_t chunk_len, float div,
+               bool src_bf16) {
+    size_t len = chunks > 1 ? chunk_len : L;
+    if (len <= 32) launch_row<TIn, TOut, R, 1>(in, out, rows, L, chunks, chunk_len, div, src_bf16);
+    else if (len <= 2048) launch_row<TIn, TOut, R, WAVE>(in, out, rows, L, chunks, chunk_len, div, src_bf16);
+    else launch_row<TIn, TOut, R, RB>(in, out, rows, L, chunks, chunk_len, div, src_bf16);
+}
+
+// rows of length L (contiguous) → out[rows]
+template <class TIn, class TOut, class R>
+void row_reduce(const TIn* in, TOut* out, size_t rows, size_t L, float div, bool src_bf16) {
+    unsigned chunks = 1;
+    size_t chunk_len = L;
+    if (rows < TARGET_BLOCKS / 4 && L >= 16384) {
+        size_t want = TARGET_BLOCKS / rows;
+        size_t max_chunks = L / 4096;              // keep at least 4096 elements per chunk
+        chunks = (unsigned)(want < max_chunks ? want : max_chunks);
+        if (chunks < 1) chunks = 1;
+        chunk_len = ((L + chunks - 1) / chunks + 63) / 64 * 64;
+        chunks = (unsigned)((L + chunk_len - 1) / chunk_len);
+    }
+    if (chunks == 1) { row_stage<TIn, TOut, R>(in, out, rows, L, 1, L, div, src_bf16); return; }
+    float* part = (float*)scratch(rows * chunks * sizeof(float) + 256);
+    if (!part) return;
+    row_stage<TIn, float, R>(in, part, rows, L, chunks, chunk_len, 0.0f, src_bf16);
+    row_stage<float, TOut, R>(part, out, rows, chunks, 1, chunks, div, src_bf16);
+}
+
+template <class TIn, class TOut, class R>
+void col_stage(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, unsigned chunks, size_t chunk_len, float div,
+               bool src_bf16) {
+    constexpr int VI = 16 / sizeof(TIn), VO = 16 / sizeof(TOut);
+    constexpr int VEC = VI < VO ? VI : VO;
+    bool vec = S % VEC == 0 && ((uintptr_t)in % (VEC * sizeof(TIn))) == 0 && ((uintptr_t)out % (VEC * sizeof(TOut))) == 0;
+    size_t sv = vec ? S / VEC : S;
+    size_t total = outer * chunks * sv;
+    if (total >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "column reduce: more than 2^32 work items"); return; }
+    unsigned blocks = cdiv(total, RB);
+    FastDiv dsv = make_fastdiv((uint32_t)sv), dch = make_fastdiv(chunks);
+    if (vec)
+        hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, R, VEC>), dim3(blocks), dim3(RB), 0, stream(), in, out, outer, L, S,
+                           chunks, chunk_len, dsv, dch, total, div, src_bf16);
+    else
+        hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, R, 1>), dim3(blocks), dim3(RB), 0, stream(), in, out, outer, L, S,
+                           chunks, chunk_len, dsv, dch, total, div, src_bf16);
+    MXH_LAUNCH_CHECK("col_reduce");
+}
+
+// [outer, L, S] (contiguous) → out[outer, S]
+template <class TIn, class TOut, class R>
+void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, float div, bool src_bf16) {
+    size_t base_blocks = (outer * (S / 4 + 1) + RB - 1) / RB;
+    unsigned chunks = 1;
+    size_t chunk_len = L;
+    if (base_blocks < TARGET_BLOCKS && L >= 64) {
+        size_t want = (TARGET_BLOCKS + base_blocks - 1) / base_blocks;
+        size_t max_chunks = L / 32;                // at least 32 rows per chunk
+        chunks = (unsigned)(want < max_chunks ? want : max_chunks);
+        if (chunks < 1) chunks = 1;
+        chunk_len = (L + chunks - 1) / chunks;
+        chunks = (unsigned)((L + chunk_len - 1) / chunk_len);
+    }
+    if (chunks == 1) { col_stage<TIn, TOut, R>(in, out, outer, L, S, 1, L, div, src_bf16); return; }
+    float* part = (float*)scratch(outer * chunks * S * sizeof(float) + 256);
+    if (!part) return;
+    col_stage<TIn, float, R>(in, part, outer, L, S, chunks, chunk_len, 0.0f, src_bf16);
+    col_stage<float, TOut, R>(part, out, outer, chunks, S, 1, chunks, div, src_bf16);
+}
+
+// sum/mean/max/min metadata: dims[n] | strides[n] | red_len[r] | red_stride[r] | offset
+template <class T, class R>
+void reduce_axis(size_t num_els, size_t num_dims, size_t nred, const size_t* md, const T* in, T* out, bool mean) {
+    if (!md || !in || !out) { set_status(ERR_INVALID, "reduce: null argument"); return; }
+    if (nred != 1) { set_status(ERR_UNSUPPORTED, "reduce: exactly one reduced dim is supported"); return; }
+    if (num_els == 0) return;
+    const size_t* dims = md;
+    const size_t* strides = md + num_dims;
+    size_t L = md[2 * num_dims], s = md[2 * num_dims + 1], offset = md[2 * num_dims + 2];
+    if (L == 0) { set_status(ERR_INVALID, "reduce: zero-length axis"); return; }
+    float div = mean ? (float)L : 0.0f;
+    const T* src = in + offset;
+    size_t out_size = num_els / L;
+    if (out_size == 0) return;
+    if (ref_is_contiguous(num_dims, dims, strides) && s != 0 && num_els % (L * s) == 0) {
+        size_t outer = num_els / (L * s);
+        if (s == 1) row_reduce<T, T, R>(src, out, outer, L, div, IO<T>::is_bf16);
+        else col_reduce<T, T, R>(src, out, outer, L, s, div, IO<T>::is_bf16);
+        return;
+    }
+    if (num_els >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "reduce: strided input with 2^31 or more elements"); return; }
+    NdSpace<1> sp;
+    // not collapsed on purpose: the walk must visit dims exactly as get_strided_index does
+    if (num_dims > (size_t)MAXD) { set_status(ERR_UNSUPPORTED, "reduce: strided input of rank above 8"); return; }
+    sp.ndims = (int)(num_dims ? num_dims : 1);
+    for (int d = 0; d < MAXD; ++d) {
+        sp.dims[d] = d < (int)num_dims ? (uint32_t)dims[d] : 1;
+        sp.div[d] = make_fastdiv(sp.dims[d]);
+        sp.strides[0][d] = d < (int)num_dims ? (int64_t)strides[d] : 0;
+    }
+    hipLaunchKernelGGL((reduce_generic_kernel<T, R>), dim3(cdiv(out_size, RB)), dim3(RB), 0, stream(), sp, src, out, num_els,
+                       out_size, L, s, div);
+    MXH_LAUNCH_CHECK("reduce_generic");
+}
+
+// ---- sum_to_shape -----------------------------------------------------------------------------------
+// `0 + x` per element: what an all-kept sum_to_shape does through its zero-initialised cells (−0 → +0).
+template <class T> struct OpZeroPlus {
+    using In = T; using Out = T; static constexpr int NIN = 1;
+    __device__ T operator()(T x) const { return IO<T>::fin(0.0f + IO<T>::ld(x), 0.0f); }
+};
+template <> struct OpZeroPlus<float> {
+    using In = float; using Out = float; static constexpr int NIN = 1;
+    __device__ float operator()(float x) const { return 0.0f + x; }
+};
+
+// Non-contiguous input: gather into a contiguous copy with the reference's index rule
+// (reduction.rs:162-167): element (Σ coords·strides + offset) mod num_els of the already-offset slice.
+template <class T>
+__global__ __launch_bounds__(RB) void sts_gather_kernel(NdSpace<1> sp, const T* __restrict__ in, T* __restrict__ out,
+                                                        size_t num_els, size_t offset) {
+    size_t i = (size_t)blockIdx.x * RB + threadIdx.x;
+    if (i >= num_els) return;
+    uint32_t r = (uint32_t)i;
+    uint64_t off = 0;
+    for (int k = sp.ndims - 1; k > 0; --k) {
+        uint32_t q, c;
+        fd_divmod(r, sp.div[k], q, c);
+        off += (uint64_t)c * (uint64_t)sp.strides[0][k];
+        r = q;
+    }
+    off += (uint64_t)r * (uint64_t)sp.strides[0][0];
+    out[i] = in[(off + offset) % num_els];
+}
+
+// sum_to_shape metadata: in_dims[n] | in_strides[n] | out_dims[n] | offset
+template <class T>
+void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in, T* out) {
+    if (!md || !in || !out) { set_status(ERR_INVALID, "sum_to_shape: null argument"); return; }
+    if (num_els == 0) return;
+    if (num_dims > 64) { set_status(ERR_INVALID, "sum_to_shape: rank above 64"); return; }
+    const size_t* in_dims = md;
+    const size_t* in_strides = md + num_dims;
+    const size_t* out_dims = md + 2 * num_dims;
+    size_t offset = md[3 * num_dims];
+    const T* src = in + offset;
+
+    // groups of kept (factor 1) and reduced (factor = whole dim) dims; size-1 dims vanish
+    size_t g_len[64];
+    bool g_red[64];
+    int ng = 0;
+    for (size_t d = 0; d < num_dims; ++d) {
+        if (out_dims[d] == 0 || in_dims[d] % out_dims[d] != 0 || (out_dims[d] != 1 && out_dims[d] != in_dims[d])) {
+            set_status(ERR_UNSUPPORTED, "sum_to_shape: output dim must be 1 or the input dim");
+            return;
+        }
+        if (in_dims[d] == 1) continue;
+        bool red = out_dims[d] == 1;
+        if (ng > 0 && g_red[ng - 1] == red) g_len[ng - 1] *= in_dims[d];
+        else { g_len[ng] = in_dims[d]; g_red[ng] = red; ++ng; }
+    }
+
+    bool cont = ref_is_contiguous(num_dims, in_dims, in_strides);
+    bool any_red = false;
+    int nred_groups = 0;
+    for (int g = 0; g < ng; ++g) { any_red |= g_red[g]; nred_groups += g_red[g]; }
+    // Temporaries (slot 1 of the library scratch; the stage drivers' partials use slot 0):
+    // [gathered contiguous copy | ping | pong]
+    T* gathered = nullptr;
+    float *ping = nullptr, *pong = nullptr;
+    size_t gathered_bytes = cont ? 0 : (num_els * sizeof(T) + 255) / 256 * 256;
+    size_t stage_bytes = 0;
+    if (nred_groups > 1) {
+        size_t smallest = (size_t)-1;
+        for (int g = 0; g < ng; ++g) if (g_red[g] && g_len[g] < smallest) smallest = g_len[g];
+        stage_bytes = ((num_els / smallest) * sizeof(float) + 255) / 256 * 256;
+    }
+    if (gathered_bytes + 2 * stage_bytes) {
+        char* p = (char*)scratch(gathered_bytes + 2 * stage_bytes, 1);
+        if (!p) return;
+        if (!cont) { gathered = (T*)p; p += gathered_bytes; }
+        if (stage_bytes) { ping = (float*)p; pong = (float*)(p + stage_bytes); }
+    }
+    if (!cont) {
+        if (num_els >= (1ull << 31) || num_dims > (size_t)MAXD) {
+            set_status(ERR_UNSUPPORTED, "sum_to_shape: strided input too large or rank above 8");
+            return;
+        }
+        NdSpace<1> sp;
+        sp.ndims = (int)(num_dims ? num_dims : 1);
+        for (int d = 0; d < MAXD; ++d) {
+            sp.dims[d] = d < (int)num_dims ? (uint32_t)in_dims[d] : 1;
+            sp.div[d] = make_fastdiv(sp.dims[d]);
+            sp.strides[0][d] = d < (int)num_dims ? (int64_t)in_strides[d] : 0;
+        }
+        hipLaunchKernelGGL((sts_gather_kernel<T>), dim3(cdiv(num_els, RB)), dim3(RB), 0, stream(), sp, src, gathered, num_els,
+                           offset);
+        MXH_LAUNCH_CHECK("sts_gather");
+        src = gathered;
+    }
+
+    if (!any_red) {   // identity: out = 0 + in
+        size_t dims1 = num_els, st1 = 1;
+        const size_t* ins[1] = {&st1};
+        const void* inp[1] = {src};
+        ew_launch<OpZeroPlus<T>>(num_els, 1, &dims1, &st1, ins, out, inp, OpZeroPlus<T>{});
+    } else {
+        // fold reduced groups one at a time, innermost first
+        const void* cur = src;
+        bool cur_is_T = true;
+        while (true) {
+            int g = ng - 1;
+            while (!g_red[g]) --g;
+            size_t outer = 1, inner = 1;
+            for (int k = 0; k < g; ++k) outer *= g_len[k];
+            for (int k = g + 1; k < ng; ++k) inner *= g_len[k];
+            size_t L = g_len[g];
+            int remaining = 0;
+            for (int k = 0; k < ng; ++k) remaining += (k != g && g_red[k]);
+            bool last = remaining == 0;
+            float* tmp = (cur == (const void*)ping) ? pong : ping;
+            bool bf = IO<T>::is_bf16;
+            if (inner == 1) {
+                if (cur_is_T) { if (last) row_reduce<T, T, RSum>((const T*)cur, out, outer, L, 0.0f, bf); else row_reduce<T, float, RSum>((const T*)cur, tmp, outer, L, 0.0f, bf); }
+                else { if (last) row_reduce<float, T, RSum>((const float*)cur, out, outer, L, 0.0f, bf); else row_reduce<float, float, RSum>((const float*)cur, tmp, outer, L, 0.0f, bf); }
+            } else {
+                if (cur_is_T) { if (last) col_reduce<T, T, RSum>((const T*)cur, out, outer, L, inner, 0.0f, bf); else col_reduce<T, float, RSum>((const T*)cur, tmp, outer, L, inner, 0.0f, bf); }
+                else { if (last) col_reduce<float, T, RSum>((const float*)cur, out, outer, L, inner, 0.0f, bf); else col_reduce<float, float, RSum>((const float*)cur, tmp, outer, L, inner, 0.0f, bf); }
+            }
+            if (last) break;
+            cur = tmp;
+            cur_is_T = false;
+            // drop group g and merge its neighbours (both kept) if both exist
+            for (int k = g; k + 1 < ng; ++k) { g_len[k] = g_len[k + 1]; g_red[k] = g_red[k + 1]; }
+            --ng;
+            if (g > 0 && g < ng && g_red[g - 1] == g_red[g]) {
+                g_len[g - 1] *= g_len[g];
+                for (int k = g; k + 1 < ng; ++k) { g_len[k] = g_len[k + 1]; g_red[k] = g_red[k + 1]; }
+                --ng;
+            }
+        }
+    }
+}
+
+}  // namespace mxh
+
+using namespace mxh;
+
+#define MXH_REDUCE_FOR(T, SUF)                                                                                  \
+    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+        reduce_axis<T, RSum>(n, nd, nr, md, in, out, false);                                                    \
+    }                                                                                                           \
+    extern "C" void hip_mean_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {     \
+        reduce_axis<T, RSum>(n, nd, nr, md, in, out, true);                                                     \
+    }                                                                                                           \
+    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+        reduce_axis<T, RMax>(n, nd, nr, md, in, out, false);                                                    \
+    }                                                                                                           \
+    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+        reduce_axis<T, RMin>(n, nd, nr, md, in, out, false);                                                    \
+    }                                                                                                           \
+    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {        \
+        sum_to_shape<T>(n, nd, md, in, out);                                                                    \
+    }
+
+MXH_REDUCE_FOR(float, f32)
+MXH_REDUCE_FOR(bf16_t, bf16)

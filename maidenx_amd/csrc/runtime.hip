@@ -1,0 +1,115 @@
+// Device, memory, stream and status entry points of the backend.  They replace the
+// cuda_malloc / cuda_free / cuda_memcpy_* / cuda_set_device / cuda_get_device family of
+// crates/maidenx_cuda/src/lib.rs:39-117.
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "mxh.hpp"
+
+namespace mxh {
+
+static std::mutex g_mu;
+static std::mutex g_scratch_mu;
+static int g_status = OK;
+static int g_hip_err = 0;
+static char g_what[256] = "ok";
+static hipStream_t g_stream = nullptr;      // null = the device's default stream
+static void* g_scratch[16][2] = {{nullptr}};
+static size_t g_scratch_bytes[16][2] = {{0}};
+
+void set_status(int code, const char* what, int hip_err) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_status != OK) return;   // keep the first error
+    g_status = code;
+    g_hip_err = hip_err;
+    if (hip_err != 0)
+        snprintf(g_what, sizeof(g_what), "%s: %s", what, hipGetErrorString((hipError_t)hip_err));
+    else
+        snprintf(g_what, sizeof(g_what), "%s", what);
+}
+
+hipStream_t stream() { return g_stream; }
+
+void* scratch(size_t bytes, int slot) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16 || slot < 0 || slot > 1) {
+        set_status(ERR_INVALID, "scratch: bad device or slot");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_bytes[dev][slot] >= bytes) return g_scratch[dev][slot];
+    // grow: work already queued on the stream may still use the old block, so drain first
+    if (g_scratch[dev][slot]) {
+        (void)hipStreamSynchronize(g_stream);
+        (void)hipFree(g_scratch[dev][slot]);
+        g_scratch[dev][slot] = nullptr;
+        g_scratch_bytes[dev][slot] = 0;
+    }
+    size_t want = bytes < (32u << 20) ? (32u << 20) : bytes;
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, want);
+    if (e != hipSuccess) { set_status(ERR_OOM, "scratch: hipMalloc", (int)e); return nullptr; }
+    g_scratch[dev][slot] = p;
+    g_scratch_bytes[dev][slot] = want;
+    return p;
+}
+
+}  // namespace mxh
+
+using namespace mxh;
+
+extern "C" {
+
+int hip_set_device(int id) { return (int)hipSetDevice(id); }
+int hip_get_device(int* id) { return (int)hipGetDevice(id); }
+int hip_device_count(int* n) { return (int)hipGetDeviceCount(n); }
+
+int hip_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return (int)hipErrorInvalidValue;
+    if (bytes == 0) bytes = 1;
+    hipError_t e = hipMalloc(ptr, bytes);
+    return e == hipSuccess ? 0 : (e == hipErrorOutOfMemory ? ERR_OOM : (int)e);
+}
+int hip_free(void* ptr) { return (int)hipFree(ptr); }
+
+// The copies are ordered after everything queued on the backend's stream and return when done.
+int hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream());
+    if (e == hipSuccess) e = hipStreamSynchronize(stream());
+    return (int)e;
+}
+int hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream());
+    if (e == hipSuccess) e = hipStreamSynchronize(stream());
+    return (int)e;
+}
+int hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream());
+}
+
+int hip_stream_create(void** s) { return (int)hipStreamCreateWithFlags((hipStream_t*)s, hipStreamNonBlocking); }
+int hip_stream_destroy(void* s) { return (int)hipStreamDestroy((hipStream_t)s); }
+int hip_stream_synchronize(void* s) { return (int)hipStreamSynchronize((hipStream_t)s); }
+// Stream every later kernel and copy of the backend is queued on (null = default stream).
+int hip_set_stream(void* s) { g_stream = (hipStream_t)s; return 0; }
+void* hip_get_stream(void) { return (void*)g_stream; }
+int hip_synchronize(void) { return (int)hipStreamSynchronize(stream()); }
+
+// First error recorded since the last call (0 = none); reading it clears it.
+int hip_get_last_status(void) {
+    hipError_t e = hipGetLastError();
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_status == OK && e != hipSuccess) {
+        g_status = ERR_LAUNCH;
+        g_hip_err = (int)e;
+        snprintf(g_what, sizeof(g_what), "hip: %s", hipGetErrorString(e));
+    }
+    int s = g_status;
+    g_status = OK;
+    return s;
+}
+// Text of the error last returned by hip_get_last_status().
+const char* hip_status_string(void) { return g_what; }
+
+}  // extern "C"

@@ -1,0 +1,478 @@
+"""GPU parity: the HIP backend, called through its C ABI, against the CPU oracle on the same seeded
+inputs.  Bars: bit-exact for data movement, comparisons and single IEEE operations; <= 1 ulp for
+f32 transcendentals (tanh-based ones are reported, see test); reductions and matmuls against an
+f64 evaluation of the same inputs, f32 <= 1e-5 and bf16 <= 1e-2 of the sum of magnitudes."""
+import numpy as np
+import pytest
+
+import layouts as LY
+from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
+                     meta_matmul, meta_pad, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
+                     ulp_diff_f32)
+
+pytestmark = pytest.mark.gpu
+
+DTS = ["f32", "bf16"]
+
+
+def both(oracle, hip, name, *args_builder):
+    """Run the same call on both backends; args_builder() must build fresh argument objects."""
+    (build,) = args_builder
+    return oracle.call(name, *build()), hip.call(name, *build())
+
+
+def same_bits(a, b):
+    return np.array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(b).view(np.uint8))
+
+
+# ---------------------------------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------------------------------
+BIN_LAYOUTS = {
+    "contig": lambda: (LY.contiguous([37, 64]), LY.contiguous([37, 64])),
+    "contig_big": lambda: (LY.contiguous([1 << 18]), LY.contiguous([1 << 18])),
+    "offset_misaligned": lambda: (LY.contiguous([33, 20], off=1), LY.contiguous([33, 20], off=3)),
+    "rhs_row_bcast": lambda: (LY.contiguous([96, 256]), LY.broadcast([96, 256], [1, 256])),
+    "rhs_row_bcast_odd": lambda: (LY.contiguous([17, 30], off=1), LY.broadcast([17, 30], [1, 30])),
+    "lhs_col_bcast": lambda: (LY.broadcast([64, 48], [64, 1]), LY.contiguous([64, 48])),
+    "lhs_transposed": lambda: (LY.permuted([192, 160], [1, 0]), LY.contiguous([192, 160])),
+    "lhs_transposed_ragged": lambda: (LY.permuted([70, 45], [1, 0], off=1), LY.contiguous([70, 45])),
+    "both_transposed": lambda: (LY.permuted([100, 130], [1, 0]), LY.permuted([100, 130], [1, 0], off=2)),
+    "nhwc_view_plus_bias": lambda: (LY.permuted([2, 64, 12, 12], [0, 3, 1, 2]), LY.broadcast([2, 64, 12, 12], [1, 64, 1, 1])),
+    "scalar_bcast": lambda: (LY.contiguous([1000]), LY.broadcast([1000], [1])),
+    "batched_transpose3d": lambda: (LY.permuted([3, 40, 50], [0, 2, 1]), LY.contiguous([3, 40, 50])),
+    "rank5": lambda: (LY.permuted([2, 3, 4, 5, 6], [4, 2, 0, 3, 1]), LY.broadcast([2, 3, 4, 5, 6], [2, 1, 4, 1, 6])),
+    "one_element": lambda: (LY.contiguous([1]), LY.contiguous([1])),
+}
+
+
+def special_values(r, n, dt):
+    x = r.standard_normal(n).astype(np.float32)
+    k = min(n, 8)
+    x[:k] = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 3e38], dtype=np.float32)[:k]
+    return to_storage(x, dt)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("lname", list(BIN_LAYOUTS))
+def test_binary_ops_bit_exact(oracle, hip, lname, dt):
+    ll, rl = BIN_LAYOUTS[lname]()
+    r = rng(hash(lname) % 1000)
+    ls, rs = special_values(r, ll["size"], dt), special_values(r, rl["size"], dt)
+    # make zeros meet zeros / non-zeros for the division rule
+    n = int(np.prod(ll["dims"]))
+    md = meta_binary(ll["dims"], ll["strides"], rl["strides"], ll["off"], rl["off"])
+    for op in ["add", "sub", "mul", "div", "maximum", "minimum"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(ll["dims"]), md, In(ls), In(rs), Out(n, dt)))
+        if op in ("maximum", "minimum") and dt == "f32":
+            # f32::max may return either zero for (+0, -0): compare values, NaN-aware
+            assert np.array_equal(o, h, equal_nan=True), op
+        else:
+            fo, fh = to_float(o, dt), to_float(h, dt)
+            assert np.array_equal(np.isnan(fo), np.isnan(fh)), op
+            assert same_bits(np.where(np.isnan(fo), 0, fo), np.where(np.isnan(fh), 0, fh)), op
+    for op in ["eq", "ne", "lt", "le", "gt", "ge", "logical_and", "logical_or", "logical_xor"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(ll["dims"]), md, In(ls), In(rs), Out(n, "bool")))
+        assert np.array_equal(o, h), op
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("lname", ["contig", "offset_misaligned", "rhs_row_bcast", "scalar_bcast", "nhwc_view_plus_bias"])
+def test_inplace_ops_bit_exact(oracle, hip, lname, dt):
+    ll, rl = BIN_LAYOUTS[lname]()
+    lc = LY.contiguous(ll["dims"], off=ll["off"])       # accumulators are contiguous tensors
+    r = rng(5)
+    ls = to_storage(r.standard_normal(lc["size"]).astype(np.float32), dt)
+    rs = to_storage(r.standard_normal(rl["size"]).astype(np.float32), dt)
+    n = int(np.prod(lc["dims"]))
+    md = meta_binary(lc["dims"], lc["strides"], rl["strides"], lc["off"], rl["off"])
+    for op in ["add_inplace", "sub_inplace", "mul_inplace", "div_inplace"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lc["dims"]), md, InOut(ls.copy()), In(rs)))
+        assert same_bits(o, h), op
+
+
+def test_inplace_with_transposed_rhs(oracle, hip):
+    # accumulate_grad of a transposed operand: lhs contiguous, rhs a transposed view
+    lc, rl = LY.contiguous([130, 70]), LY.permuted([130, 70], [1, 0])
+    r = rng(6)
+    ls = r.standard_normal(lc["size"]).astype(np.float32)
+    rs = r.standard_normal(rl["size"]).astype(np.float32)
+    md = meta_binary(lc["dims"], lc["strides"], rl["strides"], 0, 0)
+    (o,), (h,) = both(oracle, hip, "add_inplace_f32", lambda: (130 * 70, 2, md, InOut(ls.copy()), In(rs)))
+    assert same_bits(o, h)
+
+
+UN_LAYOUTS = {
+    "contig": lambda: LY.contiguous([5000]),
+    "offset": lambda: LY.contiguous([77, 13], off=1),
+    "transposed": lambda: LY.permuted([150, 200], [1, 0]),
+    "bcast": lambda: LY.broadcast([40, 50], [1, 50]),
+    "perm4d": lambda: LY.permuted([2, 5, 6, 7], [3, 1, 0, 2]),
+}
+EXACT_UNARY = ["neg", "abs", "sign", "square", "sqrt", "relu", "recip"]
+ULP1_UNARY = ["exp", "sigmoid", "sin", "cos", "ln", "log2", "exp2", "softplus", "exp10", "log10", "tan"]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("lname", list(UN_LAYOUTS))
+def test_unary_exact_ops(oracle, hip, lname, dt):
+    lay = UN_LAYOUTS[lname]()
+    r = rng(3)
+    st = special_values(r, lay["size"], dt)
+    n = int(np.prod(lay["dims"]))
+    md = meta_unary(lay["dims"], lay["strides"], lay["off"])
+    for op in EXACT_UNARY:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lay["dims"]), md, In(st), Out(n, dt)))
+        fo, fh = to_float(o, dt), to_float(h, dt)
+        assert np.array_equal(np.isnan(fo), np.isnan(fh)), op
+        assert same_bits(np.where(np.isnan(fo), 0, fo), np.where(np.isnan(fh), 0, fh)), op
+    (o,), (h,) = both(oracle, hip, f"logical_not_{dt}", lambda: (n, len(lay["dims"]), md, In(st), Out(n, "bool")))
+    assert np.array_equal(o, h)
+    for op, c in [("add_scalar", 0.75), ("sub_scalar", 0.3), ("mul_scalar", 0.01), ("div_scalar", 3.0), ("div_scalar", 0.0),
+                  ("maximum_scalar", 0.1), ("minimum_scalar", -0.2), ("leaky_relu", 0.1)]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lay["dims"]), md, In(st), const_arg(c, dt), Out(n, dt)))
+        fo, fh = to_float(o, dt), to_float(h, dt)
+        assert np.array_equal(np.isnan(fo), np.isnan(fh)), op
+        assert np.array_equal(np.where(np.isnan(fo), 0, fo), np.where(np.isnan(fh), 0, fh)), (op, c)
+    for op in ["eq_scalar", "ne_scalar", "lt_scalar", "le_scalar", "gt_scalar", "ge_scalar"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lay["dims"]), md, In(st), const_arg(0.0, dt), Out(n, "bool")))
+        assert np.array_equal(o, h), op
+
+
+def test_unary_in_place_when_input_is_null(hip, oracle):
+    r = rng(8)
+    x = r.standard_normal(1000).astype(np.float32)
+    (want,) = oracle.call("square_f32", 1000, 1, meta_unary([1000], [1]), In(x), Out(1000, "f32"))
+    (got,) = hip.call("square_f32", 1000, 1, meta_unary([1000], [1]), None, InOut(x.copy()))
+    assert same_bits(want, got)
+
+
+@pytest.mark.parametrize("op", ULP1_UNARY + ["tanh", "gelu"])
+def test_unary_transcendental_f32_ulp(oracle, hip, op):
+    r = rng(17)
+    n = 1 << 16
+    x = np.concatenate([r.standard_normal(n // 2) * 1.0, r.uniform(-20, 20, n // 4), r.uniform(-90, 90, n // 4)]).astype(np.float32)
+    if op in ("ln", "log2", "log10"):
+        x = np.abs(x) + 1e-3
+    md = meta_unary([n], [1])
+    (o,), (h,) = both(oracle, hip, f"{op}_f32", lambda: (n, 1, md, In(x), Out(n, "f32")))
+    d = ulp_diff_f32(o, h)
+    x64 = x.astype(np.float64)
+    if op == "tanh":
+        # glibc tanhf is itself up to ~2 ulp from the true value, so the distance to it can exceed 1 ulp;
+        # the bar here is 1 ulp against the exact result and <= 2 ulp against the oracle.
+        exact = np.tanh(x64).astype(np.float32)
+        assert np.max(ulp_diff_f32(h, exact)) <= 1
+        assert np.max(d) <= 2
+    elif op == "gelu":
+        # (1 + tanh) cancels for negative x, so 1 ulp of tanh becomes many ulps of the result;
+        # bound the absolute distance instead (the reference's own test uses 1e-3).
+        assert np.max(np.abs(o.astype(np.float64) - h.astype(np.float64))) <= 4e-7 * np.maximum(1.0, np.max(np.abs(x64)))
+        exact = 0.5 * x64 * (1 + np.tanh(np.float32(0.7978845608028654) * (x64 + np.float32(0.044715) * x64 ** 3)))
+        assert np.max(np.abs(h - exact)) <= 4e-7 * np.maximum(1.0, np.max(np.abs(x64)))
+    elif op in ("tan", "log10", "softplus"):
+        # glibc's tanf / log10f are not correctly rounded (documented 1-2 ulp); softplus chains two roundings
+        assert np.max(d) <= 2, (op, int(np.max(d)))
+    else:
+        assert np.max(d) <= 1, (op, int(np.max(d)), x[np.argmax(d)])
+
+
+def test_pow_f32_ulp(oracle, hip):
+    r = rng(19)
+    n = 1 << 15
+    x = r.standard_normal(n).astype(np.float32)
+    md = meta_unary([n], [1])
+    for c in (2.0, 1.0, 3.0, 0.5, -1.0):
+        (o,), (h,) = both(oracle, hip, "pow_f32", lambda: (n, 1, md, In(x), const_arg(c, "f32"), Out(n, "f32")))
+        assert np.max(ulp_diff_f32(o, h)) <= 1, c
+
+
+@pytest.mark.parametrize("op", ["exp", "tanh", "gelu", "sigmoid"])
+def test_unary_transcendental_bf16(oracle, hip, op):
+    # all 2^16 bf16 inputs; f32 evaluation then one rounding: equal except where the f32 values
+    # straddle a bf16 rounding boundary (at most one bf16 step)
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    md = meta_unary([bits.size], [1])
+    (o,), (h,) = both(oracle, hip, f"{op}_bf16", lambda: (bits.size, 1, md, In(bits), Out(bits.size, "bf16")))
+    fo, fh = bf16_to_f32(o), bf16_to_f32(h)
+    assert np.array_equal(np.isnan(fo), np.isnan(fh))
+    ok = ~np.isnan(fo)
+    step = np.abs(o[ok].astype(np.int32) - h[ok].astype(np.int32))
+    assert np.max(step) <= 1
+    assert np.mean(step == 0) > 0.995
+
+
+# ---------------------------------------------------------------------------------------------------
+# reductions
+# ---------------------------------------------------------------------------------------------------
+RED_CASES = [([64, 96], 0), ([64, 96], 1), ([257, 130], 0), ([257, 130], 1), ([8, 16, 32], 0), ([8, 16, 32], 1), ([8, 16, 32], 2),
+             ([5000], 0), ([3, 70000], 1), ([70000, 3], 0), ([1, 40000], 0), ([10000, 1], 1), ([2, 3, 5, 7], 2), ([40000], 0),
+             ([300, 2048], 1), ([4, 300000], 1)]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,dim", RED_CASES)
+def test_reductions(oracle, hip, shape, dim, dt):
+    r = rng(23)
+    n = int(np.prod(shape))
+    x = r.uniform(-1, 1, n).astype(np.float32)
+    off = 1 if n % 2 else 0
+    st = to_storage(np.concatenate([np.full(off, 5.0, np.float32), x]), dt)
+    xs = to_float(st, dt)[off:].reshape(shape).astype(np.float64)
+    md = meta_reduce(shape, contiguous_strides(shape), dim, off)
+    tol = 1e-5 if dt == "f32" else 1e-2
+    for op in ["sum", "mean", "max", "min"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(shape), 1, md, In(st), Out(n // shape[dim], dt)))
+        fh = to_float(h, dt).astype(np.float64)
+        if op in ("max", "min"):
+            assert np.array_equal(to_float(o, dt), to_float(h, dt)), op
+            continue
+        truth = xs.sum(dim) if op == "sum" else xs.mean(dim)
+        scale = np.abs(xs).sum(dim) if op == "sum" else np.abs(xs).mean(dim)
+        err = np.abs(fh - truth.ravel()) / np.maximum(scale.ravel(), 1e-30)
+        assert np.max(err) <= tol, (op, float(np.max(err)))
+        if dt == "f32":   # the oracle (sequential f32) obeys the same bound, so the two agree to twice it
+            assert np.max(np.abs(fh - o.astype(np.float64)) / np.maximum(scale.ravel(), 1e-30)) <= 2 * tol
+
+
+def test_reduction_is_deterministic(hip):
+    r = rng(29)
+    x = r.uniform(-1, 1, 512 * 4096).astype(np.float32)
+    md = meta_reduce([512, 4096], [4096, 1], 0)
+    outs = [hip.call("sum_f32", x.size, 2, 1, md, In(x), Out(4096, "f32"))[0].copy() for _ in range(3)]
+    assert same_bits(outs[0], outs[1]) and same_bits(outs[0], outs[2])
+
+
+def test_max_seed_and_nan_rule(oracle, hip):
+    for data in ([-np.inf, np.nan, -np.inf, np.nan], [np.nan, 2.0, np.nan, -1.0]):
+        x = np.array(data, dtype=np.float32)
+        (o,), (h,) = both(oracle, hip, "max_f32", lambda: (4, 1, 1, meta_reduce([4], [1], 0), In(x), Out(1, "f32")))
+        assert same_bits(o, h)
+
+
+def test_reduce_strided_input_follows_reference_quirk(oracle, hip):
+    # non-contiguous input: the metadata carries the memory stride of the reduced dim as the logical
+    # one (tensor/ops/reduction.rs:728-729); the backend must reproduce what the CPU kernel does then
+    lay = LY.permuted([6, 8], [1, 0])
+    r = rng(31)
+    st = r.uniform(-1, 1, lay["size"]).astype(np.float32)
+    for dim in (0, 1):
+        md = meta_reduce(lay["dims"], lay["strides"], dim, 0)
+        (o,), (h,) = both(oracle, hip, "sum_f32", lambda: (48, 2, 1, md, In(st), Out(48 // lay["dims"][dim], "f32")))
+        assert np.allclose(o, h, atol=1e-6)
+
+
+STS_CASES = [([64, 96], [64, 96]), ([64, 96], [1, 96]), ([64, 96], [64, 1]), ([8, 64, 128], [1, 64, 1]), ([8, 64, 128], [8, 1, 128]),
+             ([2, 3, 4, 5], [1, 3, 1, 5]), ([2, 3, 4, 5], [2, 1, 4, 1]), ([10000, 1], [10000, 1]), ([10000, 1], [1, 1]), ([5], [1]),
+             ([300, 700], [1, 1]), ([2, 3, 4, 5, 6], [1, 3, 1, 5, 1])]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,out_shape", STS_CASES)
+def test_sum_to_shape(oracle, hip, shape, out_shape, dt):
+    r = rng(37)
+    n = int(np.prod(shape))
+    st = to_storage(r.uniform(-1, 1, n).astype(np.float32), dt)
+    md = meta_sum_to_shape(shape, contiguous_strides(shape), out_shape, 0)
+    n_out = int(np.prod(out_shape))
+    (o,), (h,) = both(oracle, hip, f"sum_to_shape_{dt}", lambda: (n, len(shape), md, In(st), Out(n_out, dt)))
+    xs = to_float(st, dt).reshape(shape).astype(np.float64)
+    axes = tuple(i for i, (a, b) in enumerate(zip(shape, out_shape)) if a != b)
+    if not axes:
+        assert same_bits(o, h)      # identity: 0 + x
+        return
+    truth = xs.sum(axis=axes).ravel()
+    scale = np.abs(xs).sum(axis=axes).ravel()
+    tol = 1e-5 if dt == "f32" else 1e-2
+    assert np.max(np.abs(to_float(h, dt) - truth) / np.maximum(scale, 1e-30)) <= tol
+
+
+def test_sum_to_shape_identity_negative_zero(oracle, hip):
+    x = np.array([-0.0, 1.0, -2.0, -0.0], dtype=np.float32)
+    (o,), (h,) = both(oracle, hip, "sum_to_shape_f32", lambda: (4, 1, meta_sum_to_shape([4], [1], [4]), In(x), Out(4, "f32")))
+    assert same_bits(o, h)
+
+
+def test_sum_to_shape_strided_input(oracle, hip):
+    # a stride-0 (broadcast) gradient view, offset 0 — the shape sum(0)'s backward hands over
+    lay = LY.broadcast([50, 30], [1, 30])
+    r = rng(41)
+    st = r.uniform(-1, 1, lay["size"]).astype(np.float32)
+    st = np.concatenate([st, np.zeros(50 * 30 - st.size, np.float32)])     # keep the reference's modulo index in bounds
+    for out_shape in ([1, 30], [50, 30], [50, 1]):
+        md = meta_sum_to_shape(lay["dims"], lay["strides"], out_shape, 0)
+        n_out = int(np.prod(out_shape))
+        (o,), (h,) = both(oracle, hip, "sum_to_shape_f32", lambda: (1500, 2, md, In(st), Out(n_out, "f32")))
+        assert np.allclose(o, h, rtol=1e-5, atol=1e-5), out_shape
+
+
+# ---------------------------------------------------------------------------------------------------
+# matmul
+# ---------------------------------------------------------------------------------------------------
+def matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt, b_bcast=False):
+    a = r.standard_normal((batch, m, k)).astype(np.float32)
+    b = (r.standard_normal((1 if b_bcast else batch, k, n)) * 0.02).astype(np.float32)
+    a_shape, b_shape = [batch, m, k], [batch, k, n]
+    a_st, b_st = contiguous_strides(a_shape), contiguous_strides(b_shape)
+    a_store, b_store = a, b
+    if a_perm:
+        a_store, a_st = np.ascontiguousarray(a.transpose(0, 2, 1)), [m * k, 1, m]
+    if b_perm:
+        b_store, b_st = np.ascontiguousarray(b.transpose(0, 2, 1)), [k * n, 1, k]
+    if b_bcast:
+        b_st[0] = 0
+    md = meta_matmul([batch, m, n], a_shape, b_shape, a_st, b_st)
+    sa, sb = to_storage(a_store.ravel(), dt), to_storage(b_store.ravel(), dt)
+    # values as the kernels see them (bf16-rounded)
+    av = to_float(to_storage(a.ravel(), dt), dt).reshape(a.shape).astype(np.float64)
+    bv = to_float(to_storage(b.ravel(), dt), dt).reshape(b.shape).astype(np.float64)
+    return sa, sb, md, av, np.broadcast_to(bv, (batch, k, n))
+
+
+MM_SHAPES = [(1, 128, 128, 128), (1, 256, 192, 320), (2, 130, 70, 97), (3, 64, 600, 64), (1, 1000, 3, 1), (1, 3, 1000, 1),
+             (1, 10000, 3, 1), (1, 1, 257, 1), (2, 37, 19, 53), (1, 512, 64, 64), (1, 100, 576, 64), (4, 16, 16, 16)]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", MM_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_forward(oracle, hip, shape, a_perm, b_perm, dt):
+    batch, m, k, n = shape
+    r = rng(43)
+    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt)
+    (h,) = hip.call(f"matmul_{dt}", batch * m * n, md, In(sa), In(sb), Out(batch * m * n, dt))
+    truth = np.einsum("bmk,bkn->bmn", av, bv)
+    scale = np.einsum("bmk,bkn->bmn", np.abs(av), np.abs(bv))
+    tol = 1e-5 if dt == "f32" else 1e-2
+    err = np.abs(to_float(h, dt).reshape(truth.shape) - truth) / np.maximum(scale, 1e-30)
+    assert np.max(err) <= tol, float(np.max(err))
+    if dt == "f32" and batch * m * n * k <= 5_000_000:
+        (o,) = oracle.call("matmul_f32", batch * m * n, md, In(sa), In(sb), Out(batch * m * n, "f32"))
+        assert np.max(np.abs(o - h).reshape(truth.shape) / np.maximum(scale, 1e-30)) <= 2e-5
+        if k <= 16:   # thread-per-output kernel keeps the reference's order: identical bits
+            assert same_bits(o, h)
+
+
+def test_matmul_broadcast_batch_uses_stride0(oracle, hip):
+    r = rng(47)
+    sa, sb, md, av, bv = matmul_inputs(r, 3, 40, 50, 60, False, False, "f32", b_bcast=True)
+    (o,), (h,) = both(oracle, hip, "matmul_f32", lambda: (3 * 40 * 60, md, In(sa), In(sb), Out(3 * 40 * 60, "f32")))
+    assert np.allclose(o, h, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape", [(1, 128, 128, 128), (2, 130, 70, 97), (1, 10000, 3, 1), (1, 300, 576, 64), (3, 33, 65, 17)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_matmul_backward(oracle, hip, shape, dt):
+    batch, m, k, n = shape
+    r = rng(53)
+    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, False, False, dt)
+    go = r.standard_normal((batch, m, n)).astype(np.float32)
+    sg = to_storage(go.ravel(), dt)
+    gv = to_float(sg, dt).reshape(go.shape).astype(np.float64)
+    ga, gb = hip.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), Out(batch * m * k, dt),
+                      Out(batch * k * n, dt))
+    tol = 1e-5 if dt == "f32" else 1e-2
+    ta = np.einsum("bmn,bkn->bmk", gv, bv)
+    tb = np.einsum("bmk,bmn->bkn", av, gv)
+    sa_ = np.einsum("bmn,bkn->bmk", np.abs(gv), np.abs(bv))
+    sb_ = np.einsum("bmk,bmn->bkn", np.abs(av), np.abs(gv))
+    assert np.max(np.abs(to_float(ga, dt).reshape(ta.shape) - ta) / np.maximum(sa_, 1e-30)) <= tol
+    assert np.max(np.abs(to_float(gb, dt).reshape(tb.shape) - tb) / np.maximum(sb_, 1e-30)) <= tol
+    # either gradient may be absent
+    (ga2,) = hip.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), Out(batch * m * k, dt), None)
+    (gb2,) = hip.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), None, Out(batch * k * n, dt))
+    assert same_bits(ga, ga2) and same_bits(gb, gb2)
+
+
+# ---------------------------------------------------------------------------------------------------
+# padding, im2col, col2im: bit-exact
+# ---------------------------------------------------------------------------------------------------
+PAD_CASES = [([2, 3, 8, 8], [(0, 0), (0, 0), (1, 1), (1, 1)]), ([7], [(3, 0)]), ([5, 6], [(1, 2), (0, 3)]), ([2, 3, 4], [(1, 0), (0, 2), (2, 1)]),
+             ([4, 16, 14, 14], [(0, 0), (0, 0), (1, 1), (1, 1)]), ([3, 5], [(0, 0), (0, 0)])]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,pads", PAD_CASES)
+def test_pad_constant_forward_backward(oracle, hip, shape, pads, dt):
+    r = rng(59)
+    out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+    n_in, n_out = int(np.prod(shape)), int(np.prod(out_shape))
+    st = to_storage(np.concatenate([[9.0], r.standard_normal(n_in)]).astype(np.float32), dt)
+    md = meta_pad(shape, contiguous_strides(shape), 1, out_shape, pads)
+    (o,), (h,) = both(oracle, hip, f"pad_with_constant_{dt}",
+                      lambda: (n_in, n_out, len(shape), md, In(st), Out(n_out, dt), const_arg(-1.5, dt)))
+    assert same_bits(o, h)
+    go = to_storage(r.standard_normal(n_out).astype(np.float32), dt)
+    go[:1] = to_storage(np.array([-0.0], np.float32), dt)
+    (o,), (h,) = both(oracle, hip, f"pad_with_constant_backward_{dt}",
+                      lambda: (n_in, n_out, len(shape), md, In(go), InOut(to_storage(np.full(n_in + 2, 7.0, np.float32), dt))))
+    assert same_bits(o, h)
+
+
+def test_pad_transposed_input(oracle, hip):
+    lay = LY.permuted([6, 9], [1, 0])
+    r = rng(61)
+    st = r.standard_normal(lay["size"]).astype(np.float32)
+    pads = [(1, 1), (2, 0)]
+    out_shape = [8, 11]
+    md = meta_pad(lay["dims"], lay["strides"], 0, out_shape, pads)
+    (o,), (h,) = both(oracle, hip, "pad_with_constant_f32", lambda: (54, 88, 2, md, In(st), Out(88, "f32"), 0.0))
+    assert same_bits(o, h)
+    assert np.array_equal(o.reshape(out_shape), np.pad(LY.gather(st, lay), pads))
+
+
+CONV_CASES = [(2, 3, 8, 8, 3, 3, 1, 1), (1, 4, 12, 12, 3, 3, 1, 1), (2, 2, 9, 7, 2, 3, 1, 2), (1, 1, 5, 5, 1, 1, 0, 1), (2, 3, 10, 10, 5, 5, 2, 2),
+             (3, 8, 14, 14, 3, 3, 1, 1), (1, 2, 6, 6, 3, 3, 0, 1)]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "_".join(map(str, c)))
+def test_im2col_col2im_bit_exact(oracle, hip, case, dt):
+    B, Cc, H, W, kh, kw, p, s = case
+    oh, ow = (H + 2 * p - kh) // s + 1, (W + 2 * p - kw) // s + 1
+    r = rng(67)
+    x = to_storage(r.standard_normal(B * Cc * H * W).astype(np.float32), dt)
+    n_col = B * Cc * kh * kw * oh * ow
+    md = meta_conv(B, Cc, H, W, kh, kw, oh, ow, p, p, s, s)
+    (o,), (h,) = both(oracle, hip, f"conv2d_im2col_{dt}", lambda: (n_col, md, In(x), Out(n_col, dt)))
+    assert same_bits(o, h)
+    y = to_storage(r.standard_normal(n_col).astype(np.float32), dt)
+    for num_els in (n_col, B * Cc * H * W):      # full, and the truncation the reference's Conv2d passes
+        (o,), (h,) = both(oracle, hip, f"conv2d_col2im_{dt}", lambda: (num_els, md, In(y), Out(B * Cc * H * W, dt)))
+        assert same_bits(o, h), num_els
+
+
+# ---------------------------------------------------------------------------------------------------
+# fill / cast / strided copy (device-side helpers without a reference symbol)
+# ---------------------------------------------------------------------------------------------------
+def test_fill_cast_copy(hip):
+    (f,) = hip.call("fill_f32", 1001, Out(1001, "f32"), 2.5)
+    assert np.all(f == 2.5)
+    (f,) = hip.call("fill_bf16", 77, Out(77, "bf16"), const_arg(1.0, "bf16"))
+    assert np.all(f == 0x3F80)
+    r = rng(71)
+    x = r.standard_normal(5000).astype(np.float32)
+    (b,) = hip.call("cast_f32_bf16", 5000, In(x), Out(5000, "bf16"))
+    assert np.array_equal(b, f32_to_bf16(x))
+    (back,) = hip.call("cast_bf16_f32", 5000, In(b), Out(5000, "f32"))
+    assert np.array_equal(back, bf16_to_f32(b))
+    m = (x > 0).astype(np.uint8)
+    (mf,) = hip.call("cast_bool_f32", 5000, In(m), Out(5000, "f32"))
+    assert np.array_equal(mf, m.astype(np.float32))
+    lay = LY.permuted([70, 90], [1, 0], off=1)
+    st = r.standard_normal(lay["size"]).astype(np.float32)
+    (c,) = hip.call("copy_strided_f32", 6300, 2, meta_unary(lay["dims"], lay["strides"], 1), In(st), Out(6300, "f32"))
+    assert np.array_equal(c.reshape(70, 90), LY.gather(st, lay))
+
+
+def test_error_reporting(hip):
+    import maidenx_amd.lib as L
+    x = np.zeros(16, np.float32)
+    md2 = np.array([4, 4, 4, 1, 4, 4, 4, 1, 0], dtype=np.uint64)     # dims | strides | red_len[2] | red_stride[2] | offset
+    buf = L.DeviceBuffer.from_numpy(x)
+    out = L.DeviceBuffer(64)
+    L.call("sum_f32", 16, 2, 2, md2, buf, out)          # two reduced dims: not supported, must say so
+    with pytest.raises(L.HipError):
+        L.check()
+    L.check()                                            # reading the status cleared it

@@ -1,0 +1,261 @@
+"""CPU: pin the parts of the oracle the reference's own vectors leave open, with checks a
+plausible mistake (wrong stride, dropped offset, transposed operand, wrong rounding) would fail:
+numpy N-d indexing for the strided walks, closed forms in f64, the bf16 rounding rule over all
+2^16 bit patterns, textbook matmul, adjoint identities for pad and im2col/col2im."""
+import numpy as np
+import pytest
+
+import layouts as LY
+from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
+                     meta_matmul, meta_pad, meta_reduce, meta_sum_to_shape, meta_unary, rng, ulp_diff_f32)
+
+
+def test_bf16_rounding_rule_exhaustive():
+    # every bf16 bit pattern survives f32 -> bf16 unchanged (NaNs stay NaN, quiet bit forced)
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    f = bf16_to_f32(bits)
+    back = f32_to_bf16(f)
+    nan = np.isnan(f)
+    assert np.array_equal(back[~nan], bits[~nan])
+    assert np.all(np.isnan(bf16_to_f32(back[nan])))
+    # ties go to even, everything else to nearest: check around every representable value
+    lo = (bits[:-1].astype(np.uint32) << 16)
+    finite = np.isfinite(f[:-1]) & np.isfinite(f[1:]) & (bits[:-1] & 0x7FFF != 0x7F7F)
+    mid = (lo + 0x8000).view(np.float32)          # exactly half way to the next bf16
+    up = (lo + 0x8001).view(np.float32)
+    down = (lo + 0x7FFF).view(np.float32)
+    even = np.where(bits[:-1] & 1 == 0, bits[:-1], bits[:-1] + 1)
+    assert np.array_equal(f32_to_bf16(mid)[finite], even[finite])
+    assert np.array_equal(f32_to_bf16(up)[finite], (bits[:-1] + 1)[finite])
+    assert np.array_equal(f32_to_bf16(down)[finite], bits[:-1][finite])
+
+
+def test_oracle_bf16_add_matches_host_rounding(oracle):
+    r = rng(1)
+    a = f32_to_bf16(r.standard_normal(4096).astype(np.float32))
+    b = f32_to_bf16(r.standard_normal(4096).astype(np.float32))
+    (out,) = oracle.call("add_bf16", 4096, 1, meta_binary([4096], [1], [1]), In(a), In(b), Out(4096, "bf16"))
+    assert np.array_equal(out, f32_to_bf16(bf16_to_f32(a) + bf16_to_f32(b)))
+
+
+LAYOUT_CASES = [
+    ("contig", lambda: (LY.contiguous([5, 7]), LY.contiguous([5, 7]))),
+    ("offset", lambda: (LY.contiguous([5, 7], off=1), LY.contiguous([5, 7], off=3))),
+    ("rhs_row_bcast", lambda: (LY.contiguous([5, 7]), LY.broadcast([5, 7], [1, 7]))),
+    ("lhs_col_bcast", lambda: (LY.broadcast([5, 7], [5, 1]), LY.contiguous([5, 7]))),
+    ("lhs_transposed", lambda: (LY.permuted([5, 7], [1, 0]), LY.contiguous([5, 7]))),
+    ("both_transposed", lambda: (LY.permuted([5, 7], [1, 0], off=2), LY.permuted([5, 7], [1, 0]))),
+    ("nchw_view_plus_bias", lambda: (LY.permuted([2, 3, 4, 5], [0, 3, 1, 2]), LY.broadcast([2, 3, 4, 5], [1, 3, 1, 1]))),
+    ("scalar_bcast", lambda: (LY.contiguous([6]), LY.broadcast([6], [1]))),
+]
+
+
+@pytest.mark.parametrize("name,mk", LAYOUT_CASES, ids=[c[0] for c in LAYOUT_CASES])
+def test_oracle_binary_index_math_vs_numpy(oracle, name, mk):
+    ll, rl = mk()
+    r = rng(7)
+    ls = r.standard_normal(ll["size"]).astype(np.float32)
+    rs = r.standard_normal(rl["size"]).astype(np.float32)
+    n = int(np.prod(ll["dims"]))
+    md = meta_binary(ll["dims"], ll["strides"], rl["strides"], ll["off"], rl["off"])
+    (out,) = oracle.call("sub_f32", n, len(ll["dims"]), md, In(ls), In(rs), Out(n, "f32"))
+    assert np.array_equal(out.reshape(ll["dims"]), LY.gather(ls, ll) - LY.gather(rs, rl))
+    # in place on a contiguous lhs with the same rhs view
+    lc = LY.contiguous(ll["dims"], off=1)
+    acc = r.standard_normal(lc["size"]).astype(np.float32)
+    want = acc.copy()
+    want[1:1 + n] = (LY.gather(acc, lc) + LY.gather(rs, rl)).ravel()
+    md = meta_binary(lc["dims"], lc["strides"], rl["strides"], 1, rl["off"])
+    (got,) = oracle.call("add_inplace_f32", n, len(lc["dims"]), md, InOut(acc), In(rs))
+    assert np.array_equal(got, want)
+
+
+def test_oracle_div_by_zero_rule(oracle):
+    a = np.array([0.0, 1.0, -1.0, np.nan, -0.0, 5.0], dtype=np.float32)
+    b = np.array([0.0, 0.0, 0.0, 0.0, -0.0, -0.0], dtype=np.float32)
+    (out,) = oracle.call("div_f32", 6, 1, meta_binary([6], [1], [1]), In(a), In(b), Out(6, "f32"))
+    assert np.array_equal(out, np.array([0.0, np.inf, np.inf, np.inf, 0.0, np.inf], dtype=np.float32))
+
+
+def test_oracle_unary_closed_forms(oracle):
+    r = rng(3)
+    x = (r.standard_normal(20000) * 3).astype(np.float32)
+    md = meta_unary([x.size], [1], 0)
+    x64 = x.astype(np.float64)
+    truth = {
+        "exp": np.exp(x64), "tanh": np.tanh(x64), "sigmoid": 1 / (1 + np.exp(-x64)),
+        "gelu": 0.5 * x64 * (1 + np.tanh(0.7978845608028654 * (x64 + 0.044715 * x64 ** 3))),
+        "softplus": np.log1p(np.exp(x64)), "square": x64 * x64, "neg": -x64, "relu": np.maximum(x64, 0),
+    }
+    for op, t in truth.items():
+        (out,) = oracle.call(f"{op}_f32", x.size, 1, md, In(x), Out(x.size, "f32"))
+        err = np.abs(out.astype(np.float64) - t)
+        scale = np.maximum(np.abs(t), 1e-30)
+        # gelu/softplus lose relative accuracy where 1+tanh / 1+exp cancel; bound them absolutely
+        if op in ("gelu", "softplus"):
+            assert np.max(err) < 2e-6, op
+        else:
+            assert np.max(err / scale) < 3e-7, op
+    (out,) = oracle.call("pow_f32", x.size, 1, md, In(x), 2.0, Out(x.size, "f32"))
+    assert np.max(ulp_diff_f32(out, (x64 * x64).astype(np.float32))) <= 1
+
+
+@pytest.mark.parametrize("shape,dim", [([6, 5], 0), ([6, 5], 1), ([3, 4, 5], 0), ([3, 4, 5], 1), ([3, 4, 5], 2), ([7], 0)])
+def test_oracle_reductions_vs_numpy(oracle, shape, dim):
+    r = rng(11)
+    x = r.uniform(-1, 1, int(np.prod(shape))).astype(np.float32)
+    st = np.concatenate([[9.0], x]).astype(np.float32)      # offset 1
+    md = meta_reduce(shape, contiguous_strides(shape), dim, 1)
+    xs = x.reshape(shape).astype(np.float64)
+    n = x.size
+    for op, ref in (("sum", xs.sum(dim)), ("mean", xs.mean(dim)), ("max", xs.max(dim)), ("min", xs.min(dim))):
+        (out,) = oracle.call(f"{op}_f32", n, len(shape), 1, md, In(st), Out(n // shape[dim], "f32"))
+        if op in ("max", "min"):
+            assert np.array_equal(out, ref.ravel().astype(np.float32))
+        else:
+            assert np.allclose(out, ref.ravel(), rtol=0, atol=1e-5)
+
+
+def test_oracle_max_seed_and_nan_rule(oracle):
+    # every element below the seed f32::MIN or NaN: the seed survives (reduction.rs:433,603)
+    x = np.array([-np.inf, np.nan, -np.inf, np.nan], dtype=np.float32)
+    (out,) = oracle.call("max_f32", 4, 1, 1, meta_reduce([4], [1], 0), In(x), Out(1, "f32"))
+    assert out[0] == np.finfo(np.float32).min
+    x = np.array([np.nan, 2.0, np.nan, -1.0], dtype=np.float32)
+    (out,) = oracle.call("max_f32", 4, 1, 1, meta_reduce([4], [1], 0), In(x), Out(1, "f32"))
+    assert out[0] == 2.0
+
+
+@pytest.mark.parametrize("shape,out_shape", [([4, 6], [4, 6]), ([4, 6], [1, 6]), ([4, 6], [4, 1]), ([3, 4, 5], [1, 4, 1]),
+                                             ([3, 4, 5], [3, 1, 5]), ([2, 3, 4, 5], [1, 3, 1, 5]), ([5], [1])])
+def test_oracle_sum_to_shape_vs_numpy(oracle, shape, out_shape):
+    r = rng(5)
+    x = r.uniform(-1, 1, int(np.prod(shape))).astype(np.float32)
+    md = meta_sum_to_shape(shape, contiguous_strides(shape), out_shape, 0)
+    (out,) = oracle.call("sum_to_shape_f32", x.size, len(shape), md, In(x), Out(int(np.prod(out_shape)), "f32"))
+    axes = tuple(i for i, (a, b) in enumerate(zip(shape, out_shape)) if a != b)
+    ref = x.reshape(shape).astype(np.float64).sum(axis=axes, keepdims=True)
+    assert np.allclose(out.reshape(out_shape), ref, atol=1e-5)
+
+
+def test_oracle_sum_to_shape_identity_turns_negative_zero_positive(oracle):
+    x = np.array([-0.0, 1.0, -2.0], dtype=np.float32)
+    (out,) = oracle.call("sum_to_shape_f32", 3, 1, meta_sum_to_shape([3], [1], [3]), In(x), Out(3, "f32"))
+    assert np.array_equal(out, x) and not np.signbit(out[0])
+
+
+def matmul_case(r, batch, m, k, n, a_perm=False, b_perm=False):
+    a = r.standard_normal((batch, m, k)).astype(np.float32)
+    b = (r.standard_normal((batch, k, n)) * 0.02).astype(np.float32)
+    a_shape, b_shape = [batch, m, k], [batch, k, n]
+    a_st, b_st = contiguous_strides(a_shape), contiguous_strides(b_shape)
+    a_store, b_store = a, b
+    if a_perm:      # a is a transposed view of storage [batch, k, m]
+        a_store = np.ascontiguousarray(a.transpose(0, 2, 1))
+        a_st = [m * k, 1, m]
+    if b_perm:
+        b_store = np.ascontiguousarray(b.transpose(0, 2, 1))
+        b_st = [k * n, 1, k]
+    md = meta_matmul([batch, m, n], a_shape, b_shape, a_st, b_st)
+    return a, b, a_store.ravel(), b_store.ravel(), md
+
+
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True), (True, True)])
+def test_oracle_matmul_vs_textbook(oracle, a_perm, b_perm):
+    r = rng(2)
+    batch, m, k, n = 3, 5, 7, 4
+    a, b, a_st, b_st, md = matmul_case(r, batch, m, k, n, a_perm, b_perm)
+    (c,) = oracle.call("matmul_f32", batch * m * n, md, In(a_st), In(b_st), Out(batch * m * n, "f32"))
+    ref = np.einsum("bmk,bkn->bmn", a.astype(np.float64), b.astype(np.float64))
+    assert np.allclose(c.reshape(batch, m, n), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_oracle_matmul_backward_vs_textbook(oracle):
+    r = rng(4)
+    batch, m, k, n = 2, 5, 6, 3
+    a, b, a_st, b_st, md = matmul_case(r, batch, m, k, n)
+    go = r.standard_normal((batch, m, n)).astype(np.float32)
+    ga, gb = oracle.call("matmul_backward_f32", a.size, b.size, md, In(go.ravel()), In(a_st), In(b_st), Out(a.size, "f32"),
+                         Out(b.size, "f32"))
+    ref_a = np.einsum("bmn,bkn->bmk", go.astype(np.float64), b.astype(np.float64))
+    ref_b = np.einsum("bmk,bmn->bkn", a.astype(np.float64), go.astype(np.float64))
+    assert np.allclose(ga.reshape(a.shape), ref_a, rtol=1e-5, atol=1e-6)
+    assert np.allclose(gb.reshape(b.shape), ref_b, rtol=1e-5, atol=1e-6)
+
+
+def test_oracle_bf16_matmul_rounds_every_step(oracle):
+    # 1 + 2^-9 * 256 terms: an f32 accumulator reaches 1.5, a bf16 accumulator stays at 1
+    k = 257
+    a = f32_to_bf16(np.ones(k, dtype=np.float32))
+    b = f32_to_bf16(np.concatenate([[1.0], np.full(k - 1, 2.0 ** -9)]).astype(np.float32))
+    md = meta_matmul([1, 1], [1, k], [k, 1], [k, 1], [1, 1])
+    (c,) = oracle.call("matmul_bf16", 1, md, In(a), In(b), Out(1, "bf16"))
+    assert bf16_to_f32(c)[0] == 1.0
+
+
+def test_oracle_pad_is_adjoint_of_its_backward(oracle):
+    r = rng(9)
+    shape, pads = [2, 3, 4], [(1, 0), (0, 2), (2, 1)]
+    out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+    n_in, n_out = int(np.prod(shape)), int(np.prod(out_shape))
+    md = meta_pad(shape, contiguous_strides(shape), 0, out_shape, pads)
+    x = r.standard_normal(n_in).astype(np.float32)
+    y = r.standard_normal(n_out).astype(np.float32)
+    (px,) = oracle.call("pad_with_constant_f32", n_in, n_out, 3, md, In(x), Out(n_out, "f32"), 0.0)
+    (by,) = oracle.call("pad_with_constant_backward_f32", n_in, n_out, 3, md, In(y), InOut(np.zeros(n_in, np.float32)))
+    ref = np.pad(x.reshape(shape), pads)
+    assert np.array_equal(px.reshape(out_shape), ref)
+    assert np.isclose(np.dot(px.astype(np.float64), y), np.dot(x.astype(np.float64), by))
+
+
+def im2col_numpy(x, kh, kw, ph, pw, sh, sw):
+    B, Cc, H, W = x.shape
+    oh, ow = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    xp = np.pad(x, [(0, 0), (0, 0), (ph, ph), (pw, pw)])
+    col = np.zeros((B, Cc * kh * kw, oh * ow), dtype=x.dtype)
+    for c in range(Cc):
+        for i in range(kh):
+            for j in range(kw):
+                patch = xp[:, c, i:i + sh * oh:sh, j:j + sw * ow:sw]
+                col[:, (c * kh + i) * kw + j, :] = patch.reshape(B, -1)
+    return col, oh, ow
+
+
+@pytest.mark.parametrize("kh,kw,p,s", [(3, 3, 1, 1), (3, 3, 0, 1), (2, 3, 1, 2), (1, 1, 0, 1), (5, 5, 2, 2)])
+def test_oracle_im2col_col2im_vs_bruteforce_and_adjoint(oracle, kh, kw, p, s):
+    r = rng(13)
+    B, Cc, H, W = 2, 3, 7, 8
+    x = r.standard_normal((B, Cc, H, W)).astype(np.float32)
+    col_ref, oh, ow = im2col_numpy(x, kh, kw, p, p, s, s)
+    md = meta_conv(B, Cc, H, W, kh, kw, oh, ow, p, p, s, s)
+    (col,) = oracle.call("conv2d_im2col_f32", col_ref.size, md, In(x.ravel()), Out(col_ref.size, "f32"))
+    assert np.array_equal(col.reshape(col_ref.shape), col_ref)
+    # adjoint identity <im2col(x), y> == <x, col2im(y)> when no column index is cut off
+    y = r.standard_normal(col_ref.size).astype(np.float32)
+    (back,) = oracle.call("conv2d_col2im_f32", y.size, md, In(y), Out(x.size, "f32"))
+    lhs = np.dot(col_ref.ravel().astype(np.float64), y.astype(np.float64))
+    rhs = np.dot(x.ravel().astype(np.float64), back.astype(np.float64))
+    assert np.isclose(lhs, rhs, rtol=1e-5)
+    # the reference's caller passes num_els = B*C*H*W: column indices at or beyond it contribute nothing
+    cut = x.size
+    y_cut = y.copy()
+    y_cut[cut:] = 0
+    (a,) = oracle.call("conv2d_col2im_f32", cut, md, In(y), Out(x.size, "f32"))
+    (b,) = oracle.call("conv2d_col2im_f32", y.size, md, In(y_cut), Out(x.size, "f32"))
+    assert np.array_equal(a, b)
+
+
+def test_oracle_threaded_mode_agrees_with_sequential(oracle):
+    r = rng(21)
+    x = r.uniform(-1, 1, 64 * 33).astype(np.float32)
+    md = meta_reduce([64, 33], [33, 1], 0)
+    (seq,) = oracle.call("max_f32", x.size, 2, 1, md, In(x), Out(33, "f32"))
+    (s1,) = oracle.call("sum_f32", x.size, 2, 1, md, In(x), Out(33, "f32"))
+    oracle.set_threads(4)
+    try:
+        (par,) = oracle.call("max_f32", x.size, 2, 1, md, In(x), Out(33, "f32"))
+        (s4,) = oracle.call("sum_f32", x.size, 2, 1, md, In(x), Out(33, "f32"))
+    finally:
+        oracle.set_threads(1)
+    assert np.array_equal(seq, par)
+    assert np.allclose(s1, s4, atol=1e-5)
