@@ -1,14 +1,22 @@
 // f32 math used by the elementwise kernels.
 //
-// The reference's CPU backend calls the platform libm (glibc expf/tanhf/powf...) through
-// Rust's f32 methods.  These kernels are HBM-bound, so the transcendental functions are
-// evaluated in f64 and rounded once: the result is the correctly rounded f32 value except
-// for inputs whose exact result lies within ~1e-12 (relative) of a rounding boundary, which
-// keeps it within 1 ulp of any libm whose own error is below 1 ulp.
-// Everything here compiles for host and device so it can be checked on the CPU.
+// The reference's CPU backend reaches the platform libm (glibc 2.35 here) through Rust's
+// f32::exp / f32::tanh / f32::powf.  Composite ops amplify a last-bit difference of the inner
+// function (1 + tanh(..) in gelu, 1 + exp(x) in softplus and sigmoid), so exp and tanh are not
+// merely accurate: they restate the algorithms that libm uses, operation for operation, and
+// return the same bits.
+//   expf   : the table-driven double-precision scheme of glibc >= 2.27 (from ARM's optimized
+//            routines): x*N/ln2 = k + r, 2^(k/N) from a 32-entry table, cubic in r, with the
+//            multiply-adds fused the way the FMA build of the library fuses them.
+//   tanhf, expm1f : the FDLIBM single-precision routines (Sun Microsystems, 1993).
+// Both were compared with the library over all 2^32 inputs on the CPU and agree on every one
+// (tests/test_mathfn.py samples this).  The remaining functions are evaluated in f64 and
+// rounded once, which keeps them within 1 ulp of any libm whose own error is below 1 ulp.
+// Everything here compiles for host and device.
 #pragma once
 #include <cmath>
 #include <cstdint>
+#include <cstring>
 
 #if defined(__HIPCC__)
 #define MXH_HD __host__ __device__ inline
@@ -18,60 +26,142 @@
 
 namespace mxh {
 
-MXH_HD double bits2d(uint64_t b) {
-    union { uint64_t u; double d; } c;
-    c.u = b;
-    return c.d;
-}
+MXH_HD uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+MXH_HD float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+MXH_HD uint64_t d2u(double f) { uint64_t u; memcpy(&u, &f, 8); return u; }
+MXH_HD double u2d(uint64_t u) { double f; memcpy(&f, &u, 8); return f; }
 
-// exp(r) for |r| <= 0.35 : Taylor to degree 11 (truncation below 1e-14 relative)
-MXH_HD double exp_poly(double r) {
-    double p = 1.0 / 39916800.0;
-    p = fma(p, r, 1.0 / 3628800.0);
-    p = fma(p, r, 1.0 / 362880.0);
-    p = fma(p, r, 1.0 / 40320.0);
-    p = fma(p, r, 1.0 / 5040.0);
-    p = fma(p, r, 1.0 / 720.0);
-    p = fma(p, r, 1.0 / 120.0);
-    p = fma(p, r, 1.0 / 24.0);
-    p = fma(p, r, 1.0 / 6.0);
-    p = fma(p, r, 0.5);
-    p = fma(p, r, 1.0);
-    p = fma(p, r, 1.0);
-    return p;
-}
-
-// e^x as a double, for |x| < 700
-MXH_HD double exp_d(double x) {
-    double n = rint(x * 1.4426950408889634);
-    double r = fma(-n, 0.6931471803691238, x);      // ln2 high part (its low 21 bits are zero)
-    r = fma(-n, 1.9082149292705877e-10, r);         // ln2 low part
-    double s = bits2d((uint64_t)(1023 + (int64_t)n) << 52);
-    return exp_poly(r) * s;
-}
+// bits(2^(i/32)) - (i << 47), i = 0..31 (each 2^(i/32) correctly rounded to double)
+#if defined(__HIP_DEVICE_COMPILE__)
+static __device__ __constant__
+#else
+static
+#endif
+const uint64_t EXP2F_TAB[32] = {
+    0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
+    0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
+    0x3fef06fe0a31b715ULL, 0x3feef1a7373aa9cbULL, 0x3feedea64c123422ULL, 0x3feece086061892dULL,
+    0x3feebfdad5362a27ULL, 0x3feeb42b569d4f82ULL, 0x3feeab07dd485429ULL, 0x3feea47eb03a5585ULL,
+    0x3feea09e667f3bcdULL, 0x3fee9f75e8ec5f74ULL, 0x3feea11473eb0187ULL, 0x3feea589994cce13ULL,
+    0x3feeace5422aa0dbULL, 0x3feeb737b0cdc5e5ULL, 0x3feec49182a3f090ULL, 0x3feed503b23e255dULL,
+    0x3feee89f995ad3adULL, 0x3feeff76f2fb5e47ULL, 0x3fef199bdd85529cULL, 0x3fef3720dcef9069ULL,
+    0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL
+};
 
 MXH_HD float m_exp(float x) {
-    if (!(x == x)) return x + x;
-    if (x > 89.0f) return INFINITY;
-    if (x < -104.0f) return 0.0f;
-    return (float)exp_d((double)x);
+    const double InvLn2N = 0x1.71547652b82fep+0 * 32, Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32, C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    uint32_t abstop = (f2u(x) >> 20) & 0x7ff;
+    if (abstop >= (f2u(88.0f) >> 20)) {
+        if (f2u(x) == f2u(-INFINITY)) return 0.0f;
+        if (abstop >= (f2u(INFINITY) >> 20)) return x + x;
+        if (x > 0x1.62e42ep6f) return INFINITY;      // overflow
+        if (x < -0x1.9fe368p6f) return 0.0f;         // underflow to zero
+    }
+    double xd = (double)x;
+    double kd = fma(InvLn2N, xd, Shift);
+    uint64_t ki = d2u(kd);
+    kd -= Shift;
+    double r = fma(InvLn2N, xd, -kd);
+    uint64_t t = EXP2F_TAB[ki % 32] + (ki << 47);
+    double s = u2d(t);
+    double z = fma(C0, r, C1);
+    double r2 = r * r;
+    double y = fma(C2, r, 1.0);
+    y = fma(z, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
+MXH_HD float m_expm1(float x) {
+    const float one = 1.0f, huge = 1.0e+30f, tiny = 1.0e-30f, o_threshold = 8.8721679688e+01f,
+                ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f,
+                Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f,
+                Q5 = -2.0109921195e-07f;
+    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
+    int32_t k;
+    uint32_t hx = f2u(x);
+    const uint32_t xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+    if (hx >= 0x4195b844u) {                 // |x| >= 27 ln2
+        if (hx >= 0x42b17218u) {             // |x| >= 88.72
+            if (hx > 0x7f800000u) return x + x;
+            if (hx == 0x7f800000u) return xsb == 0 ? x : -1.0f;
+            if (x > o_threshold) return huge * huge;
+        }
+        if (xsb != 0) {
+            if (x + tiny < 0.0f) return tiny - one;
+        }
+    }
+    if (hx > 0x3eb17218u) {                  // |x| > 0.5 ln2
+        if (hx < 0x3F851592u) {              // |x| < 1.5 ln2
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int32_t)(invln2 * x + (xsb == 0 ? 0.5f : -0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {           // |x| < 2^-25
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+        return y - one;
+    }
+    if (k < 23) {
+        t = u2f(0x3f800000u - (0x1000000u >> k));   // 1 - 2^-k
+        y = t - (e - x);
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+    } else {
+        t = u2f((uint32_t)(0x7f - k) << 23);        // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+    }
+    return y;
 }
 
 MXH_HD float m_tanh(float x) {
-    if (!(x == x)) return x + x;
-    double a = fabs((double)x);
-    double t;
-    if (a < 0.02) {
-        double a2 = a * a;   // odd Taylor series, truncation below 1e-15 relative here
-        t = a * fma(a2, fma(a2, fma(a2, fma(a2, 62.0 / 2835.0, -17.0 / 315.0), 2.0 / 15.0), -1.0 / 3.0), 1.0);
-    } else if (a < 20.0) {
-        double e = exp_d(2.0 * a);
-        t = 1.0 - 2.0 / (e + 1.0);
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    float t, z;
+    const int32_t jx = (int32_t)f2u(x);
+    const int32_t ix = jx & 0x7fffffff;
+    if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;   // inf, NaN
+    if (ix < 0x41b00000) {                    // |x| < 22
+        if (ix == 0) return x;                // +-0
+        if (ix < 0x24000000) return x * (one + x);   // |x| < 2^-55
+        if (ix >= 0x3f800000) {               // |x| >= 1
+            t = m_expm1(two * fabsf(x));
+            z = one - two / (t + two);
+        } else {
+            t = m_expm1(-two * fabsf(x));
+            z = -t / (t + two);
+        }
     } else {
-        t = 1.0;
+        z = one - tiny;
     }
-    float r = (float)t;
-    return x < 0.0f ? -r : r;
+    return jx >= 0 ? z : -z;
 }
 
 MXH_HD float m_pow(float x, float c) { return (float)pow((double)x, (double)c); }
