@@ -1,0 +1,382 @@
+#!/usr/bin/env python3
+"""Benchmark of the maidenx_hip backend on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul]
+
+The default workload is BASELINE.json's configs[1]: elementwise forward + backward of add, mul, div,
+exp, relu, gelu on [8192,8192] tensors, f32 and bf16, for contiguous operands, a [1,8192] broadcast
+rhs and a transposed lhs view, with the gradients taken through sum_to_shape and accumulated in
+place.  One "step" issues, through the C ABI, the chain of backend kernels the reference's tensor
+layer issues for all of these (crates/maidenx_tensor/src/ops/{binary,unary}.rs backward closures).
+Inputs are resident in HBM before the timed region starts.  One JSON line is printed.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+ESZ = {"f32": 4, "bf16": 2, "bool": 1}
+
+
+def u64(*parts):
+    out = []
+    for p in parts:
+        out.extend([int(p)] if np.isscalar(p) else [int(v) for v in p])
+    return np.array(out, dtype=np.uint64)
+
+
+def f32_to_bf16(a):
+    x = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((x + 0x7FFF + ((x >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def const(v, dt):
+    return float(v) if dt == "f32" else int(f32_to_bf16(np.array([v], np.float32))[0])
+
+
+class Call:
+    """One backend call with its C arguments ready, plus the bytes it must move at the least."""
+    __slots__ = ("fn", "args", "bytes", "tag", "keep")
+
+    def __init__(self, fn, args, nbytes, tag, keep):
+        self.fn, self.args, self.bytes, self.tag, self.keep = fn, args, nbytes, tag, keep
+
+
+class ChainBuilder:
+    """Builds the elementwise fwd+bwd kernel chains for one dtype on a backend.
+
+    alloc(count, dtag, init) -> (pointer, keepalive).  Buffers: x, y [R,C]; xT storage [C,R] for the
+    transposed view; row [C]; temporaries; gradient accumulators."""
+
+    def __init__(self, lib, prefix, alloc, dt, R, Cc, seed):
+        self.lib, self.prefix, self.dt, self.R, self.C = lib, prefix, dt, R, Cc
+        self.N = R * Cc
+        rng = np.random.default_rng(seed)
+        self.keep = []
+
+        def new(count, dtag=dt, init=None):
+            p, k = alloc(count, dtag, init)
+            self.keep.append(k)
+            return p
+        normal = lambda n: rng.standard_normal(n, dtype=np.float32)
+        self.x, self.y, self.xT = new(self.N, init=normal(self.N)), new(self.N, init=normal(self.N)), new(self.N, init=normal(self.N))
+        self.row = new(Cc, init=normal(Cc))
+        self.go = new(self.N, init=np.ones(self.N, np.float32))
+        self.z = new(self.N)
+        self.t = [new(self.N) for _ in range(8)]
+        self.mask = new(self.N, "bool")
+        self.gx, self.gy, self.gbase, self.gxv = (new(self.N, init=np.zeros(self.N, np.float32)) for _ in range(4))
+        self.grow = new(Cc, init=np.zeros(Cc, np.float32))
+        self.trow = new(Cc)
+        cs = [Cc, 1]
+        self.lay = {                                   # (strides, footprint in elements)
+            "contig": (cs, self.N), "row": ([0, 1], Cc), "transposed": ([1, R], self.N),
+        }
+        self.calls = []
+
+    # -- emitters ----------------------------------------------------------------------------------
+    def _fn(self, name):
+        return getattr(self.lib, self.prefix + name)
+
+    def binary(self, op, a, la, b, lb, out, tag=None, out_dt=None):
+        dt, e = self.dt, ESZ[self.dt]
+        md = u64([self.R, self.C], self.lay[la][0], self.lay[lb][0], 0, 0)
+        nb = (self.lay[la][1] + self.lay[lb][1]) * e + self.N * ESZ[out_dt or dt]
+        self.calls.append(Call(self._fn(f"{op}_{dt}"), (self.N, 2, md.ctypes.data, a, b, out), nb, tag or f"{op}_{dt}/{la}+{lb}", md))
+
+    def inplace(self, op, acc, b, lb, dims=None):
+        dims = dims or [self.R, self.C]
+        n = dims[0] * dims[1]
+        strides = {"contig": [dims[1], 1], "transposed_back": [1, dims[0]]}[lb]
+        md = u64(dims, [dims[1], 1], strides, 0, 0)
+        self.calls.append(Call(self._fn(f"{op}_inplace_{self.dt}"), (n, 2, md.ctypes.data, acc, b), 3 * n * ESZ[self.dt],
+                               f"{op}_inplace_{self.dt}/{lb}", md))
+
+    def inplace_row(self, acc, b):
+        md = u64([1, self.C], [self.C, 1], [self.C, 1], 0, 0)
+        self.calls.append(Call(self._fn(f"add_inplace_{self.dt}"), (self.C, 2, md.ctypes.data, acc, b), 3 * self.C * ESZ[self.dt],
+                               f"add_inplace_{self.dt}/row", md))
+
+    def unary(self, op, a, la, out, c=None, out_dt=None):
+        dt = self.dt
+        md = u64([self.R, self.C], self.lay[la][0], 0)
+        nb = self.lay[la][1] * ESZ[dt] + self.N * ESZ[out_dt or dt]
+        args = (self.N, 2, md.ctypes.data, a, out) if c is None else (self.N, 2, md.ctypes.data, a, const(c, dt), out)
+        self.calls.append(Call(self._fn(f"{op}_{dt}"), args, nb, f"{op}_{dt}/{la}", md))
+
+    def cast_bool(self, a, out):
+        self.calls.append(Call(self._fn(f"cast_bool_{self.dt}"), (self.N, a, out), self.N * (1 + ESZ[self.dt]), f"cast_bool_{self.dt}", None))
+
+    def sts(self, a, out, to_row):
+        out_dims = [1, self.C] if to_row else [self.R, self.C]
+        md = u64([self.R, self.C], [self.C, 1], out_dims, 0)
+        nb = (self.N + (self.C if to_row else self.N)) * ESZ[self.dt]
+        self.calls.append(Call(self._fn(f"sum_to_shape_{self.dt}"), (self.N, 2, md.ctypes.data, a, out), nb,
+                               f"sum_to_shape_{self.dt}/{'to_row' if to_row else 'identity'}", md))
+
+    # -- accumulate_grad of the lhs (and, for a transposed view, of the tensor it views) ---------------
+    def acc_lhs(self, g, case):
+        if case == "transposed":
+            self.inplace("add", self.gxv, g, "contig")                                  # the view's own grad
+            self.inplace("add", self.gbase, g, "transposed_back", dims=[self.C, self.R])  # transpose backward
+        else:
+            self.inplace("add", self.gx, g, "contig")
+
+    def acc_rhs(self, g, case):
+        if case == "bcast":
+            self.inplace_row(self.grow, g)
+        else:
+            self.inplace("add", self.gy, g, "contig")
+
+    def operands(self, case):
+        x, lx = (self.xT, "transposed") if case == "transposed" else (self.x, "contig")
+        y, ly = (self.row, "row") if case == "bcast" else (self.y, "contig")
+        return x, lx, y, ly
+
+    # -- the chains (crates/maidenx_tensor/src/ops/binary.rs:48-53,152-157,207-215; unary.rs:214-216,325-345,611-613)
+    def add(self, case):
+        x, lx, y, ly = self.operands(case)
+        t = self.t
+        self.binary("add", x, lx, y, ly, self.z)
+        self.sts(self.go, t[0], False)
+        gr = self.trow if case == "bcast" else t[1]
+        self.sts(self.go, gr, case == "bcast")
+        self.acc_lhs(t[0], case)
+        self.acc_rhs(gr, case)
+
+    def mul(self, case):
+        x, lx, y, ly = self.operands(case)
+        t = self.t
+        self.binary("mul", x, lx, y, ly, self.z)
+        self.binary("mul", self.go, "contig", y, ly, t[0])
+        self.sts(t[0], t[1], False)
+        self.binary("mul", self.go, "contig", x, lx, t[2])
+        gr = self.trow if case == "bcast" else t[3]
+        self.sts(t[2], gr, case == "bcast")
+        self.acc_lhs(t[1], case)
+        self.acc_rhs(gr, case)
+
+    def div(self, case):
+        x, lx, y, ly = self.operands(case)
+        t = self.t
+        self.binary("div", x, lx, y, ly, self.z)
+        self.binary("div", self.go, "contig", y, ly, t[0])
+        self.sts(t[0], t[1], False)
+        self.binary("mul", self.go, "contig", x, lx, t[2])
+        self.unary("square", y, ly, t[3])
+        self.binary("div", t[2], "contig", t[3], "contig", t[4])
+        self.unary("neg", t[4], "contig", t[5])
+        gr = self.trow if case == "bcast" else t[6]
+        self.sts(t[5], gr, case == "bcast")
+        self.acc_lhs(t[1], case)
+        self.acc_rhs(gr, case)
+
+    def exp(self, case):
+        x, lx, _, _ = self.operands(case)
+        self.unary("exp", x, lx, self.z)
+        self.binary("mul", self.go, "contig", self.z, "contig", self.t[0])
+        self.acc_lhs(self.t[0], case)
+
+    def relu(self, case):
+        x, lx, _, _ = self.operands(case)
+        self.unary("relu", x, lx, self.z)
+        self.unary("gt_scalar", x, lx, self.mask, c=0.0, out_dt="bool")
+        self.cast_bool(self.mask, self.t[0])
+        self.binary("mul", self.go, "contig", self.t[0], "contig", self.t[1])
+        self.acc_lhs(self.t[1], case)
+
+    def gelu(self, case):
+        x, lx, _, _ = self.operands(case)
+        t = self.t
+        c0, coeff = 0.7978845608028654, 0.044715
+        self.unary("gelu", x, lx, self.z)
+        self.binary("mul", x, lx, x, lx, t[0])                      # x_squared
+        self.binary("mul", t[0], "contig", x, lx, t[1])             # x_cubed
+        self.unary("mul_scalar", t[1], "contig", t[2], c=coeff)
+        self.binary("add", x, lx, t[2], "contig", t[1])
+        self.unary("mul_scalar", t[1], "contig", t[2], c=c0)        # tanh_arg
+        self.unary("tanh", t[2], "contig", t[1])                    # tanh_val
+        self.binary("mul", t[1], "contig", t[1], "contig", t[2])
+        self.unary("mul_scalar", t[2], "contig", t[3], c=-1.0)
+        self.unary("add_scalar", t[3], "contig", t[2], c=1.0)       # sech_squared
+        self.unary("mul_scalar", t[0], "contig", t[3], c=3.0 * coeff)
+        self.unary("add_scalar", t[3], "contig", t[4], c=1.0)
+        self.unary("mul_scalar", t[4], "contig", t[3], c=c0)        # inner_derivative
+        self.unary("add_scalar", t[1], "contig", t[4], c=1.0)
+        self.unary("mul_scalar", t[4], "contig", t[5], c=0.5)       # term1
+        self.binary("mul", x, lx, t[2], "contig", t[4])
+        self.binary("mul", t[4], "contig", t[3], "contig", t[6])
+        self.unary("mul_scalar", t[6], "contig", t[4], c=0.5)       # term2
+        self.binary("add", t[5], "contig", t[4], "contig", t[6])
+        self.binary("mul", self.go, "contig", t[6], "contig", t[7])
+        self.acc_lhs(t[7], case)
+
+    def build(self):
+        for case in ("contig", "bcast", "transposed"):
+            for op in (self.add, self.mul, self.div):
+                op(case)
+        for case in ("contig", "transposed"):
+            for op in (self.exp, self.relu, self.gelu):
+                op(case)
+        return self.calls
+
+
+def hip_backend():
+    import maidenx_amd.lib as L
+    lib = L.load()
+    if L.device_count() < 1:
+        sys.exit("bench.py needs one MI355X: no HIP device is visible")
+    assert lib.hip_set_device(0) == 0
+
+    def alloc(count, dtag, init):
+        if init is None:
+            buf = L.DeviceBuffer(count * ESZ[dtag])
+        else:
+            arr = f32_to_bf16(init) if dtag == "bf16" else np.ascontiguousarray(init, dtype={"f32": np.float32, "bool": np.uint8}[dtag])
+            buf = L.DeviceBuffer.from_numpy(arr)
+        return buf.ptr, buf
+    return L, lib, alloc
+
+
+def bind(lib, prefix):
+    import maidenx_amd._signatures as S
+    sig = dict(S.signatures())
+    if prefix == "hip_":
+        sig.update(S.extension_signatures())
+    for name, args in sig.items():
+        fn = getattr(lib, prefix + name, None)
+        if fn is not None:
+            fn.argtypes, fn.restype = args, None
+
+
+def run_elementwise(args):
+    L, lib, alloc = hip_backend()
+    R = Cc = 8192
+    chains, builders = [], []          # the builders own the device buffers: keep them alive
+    for i, dt in enumerate(("f32", "bf16")):
+        builders.append(ChainBuilder(lib, "hip_", alloc, dt, R, Cc, seed=0x5EED0002 + i))
+        chains += builders[-1].build()
+    step_bytes = sum(c.bytes for c in chains)
+    probe_tag = "mul_f32/contig+contig"           # the most frequent kernel of the chain
+    ev = [(C.c_void_p(), C.c_void_p()) for _ in range(4096)]
+    for a, b in ev:
+        lib.hip_event_create(C.byref(a)); lib.hip_event_create(C.byref(b))
+
+    def step(timed_events=None):
+        for c in chains:
+            if timed_events is not None and c.tag == probe_tag and timed_events[0] < len(ev):
+                a, b = ev[timed_events[0]]
+                lib.hip_event_record(a)
+                c.fn(*c.args)
+                lib.hip_event_record(b)
+                timed_events[0] += 1
+            else:
+                c.fn(*c.args)
+
+    for _ in range(args.warmup):
+        step()
+    L.synchronize()
+    used = [0]
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(used)
+    L.synchronize()
+    dt_s = time.perf_counter() - t0
+    ms = C.c_float()
+    durs = []
+    for a, b in ev[:used[0]]:
+        lib.hip_event_elapsed_ms(a, b, C.byref(ms))
+        durs.append(ms.value)
+    probe_bytes = next(c.bytes for c in chains if c.tag == probe_tag)
+    avg_ms = float(np.mean(durs))
+    achieved = probe_bytes / (avg_ms * 1e-3) / 1e9
+    value = step_bytes * args.steps / dt_s / 1e9
+    per_tag = {}
+    for c in chains:
+        per_tag[c.tag] = per_tag.get(c.tag, 0) + 1
+    result = {
+        "metric": "train steps/s; HBM GB/s elemwise/reduce; matmul TFLOP/s on 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt_s / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32+bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: elementwise fwd+bwd (add,mul,div,exp,relu,gelu) on [8192,8192], f32+bf16, "
+                               "contiguous / rhs [1,8192] broadcast / transposed lhs", "kernel_launches_per_step": len(chains),
+                   "algorithmic_GB_per_step": round(step_bytes / 1e9, 3)},
+        "roofline": {"bound": "hbm", "kernel": "ew_nd_kernel<OpMul<float>,4> (hip_mul_f32, contiguous [8192,8192])",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "avg_launch_us": round(avg_ms * 1e3, 2), "launches_timed": len(durs), "traffic": None},
+    }
+    L.synchronize()
+    del chains, builders
+    result["cpu_baseline"] = cpu_baseline_elementwise(args)
+    return result
+
+
+def cpu_baseline_elementwise(args):
+    """The same chain on the CPU oracle (a restatement of maidenx_cpu, threaded like its rayon loops),
+    on a bounded sample: [256,8192] instead of [8192,8192] (1/32 of the rows)."""
+    from tests.helpers import ensure_oracle_built
+    lib = C.CDLL(ensure_oracle_built())
+    bind(lib, "oracle_")
+    lib.oracle_set_num_threads.restype = C.c_int
+    cores = lib.oracle_set_num_threads(0)
+    R, Cc = 256, 8192
+
+    def alloc(count, dtag, init):
+        if init is None:
+            arr = np.zeros(count, dtype={"f32": np.float32, "bf16": np.uint16, "bool": np.uint8}[dtag])
+        else:
+            arr = f32_to_bf16(init) if dtag == "bf16" else np.ascontiguousarray(init, dtype={"f32": np.float32, "bool": np.uint8}[dtag])
+        return arr.ctypes.data, arr
+    chains, builders = [], []          # the builders own the host arrays: keep them alive
+    for i, dt in enumerate(("f32", "bf16")):
+        b = ChainBuilder(lib, "oracle_", alloc, dt, R, Cc, seed=0x5EED0002 + i)
+        builders.append(b)
+        # the oracle has no device-side cast: the reference converts bool -> float on the host
+        b.cast_bool = lambda a, out, b=b: b.calls.append(Call(lambda *x: None, (), 0, "host_cast", None))
+        chains += b.build()
+    nbytes = sum(c.bytes for c in chains)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        for c in chains:
+            c.fn(*c.args)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 20:
+            break
+    el = time.perf_counter() - t0
+    return {"value": round(nbytes * reps / el / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"same kernel chain on [{R},{Cc}] tensors (1/32 of the rows), {reps} passes, {el:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="elementwise")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X; nothing in this backend uses a second GPU (--gpus must be 1)")
+    if args.no_cpu_baseline:
+        global cpu_baseline_elementwise
+        cpu_baseline_elementwise = lambda a: None
+    if args.workload == "elementwise":
+        res = run_elementwise(args)
+    else:
+        sys.exit(f"unknown workload {args.workload}")
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

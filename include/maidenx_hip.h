@@ -59,6 +59,12 @@ int hip_stream_synchronize(void* stream);
 int hip_set_stream(void* stream);       /* stream used by every later kernel/copy (NULL = default) */
 void* hip_get_stream(void);
 int hip_synchronize(void);              /* wait for everything queued on the backend's stream */
+/* events recorded on the backend's stream (no counterpart in the reference; used for timing) */
+int hip_event_create(void** event);
+int hip_event_destroy(void* event);
+int hip_event_record(void* event);
+int hip_event_synchronize(void* event);
+int hip_event_elapsed_ms(void* start, void* stop, float* ms);
 
 /* ---- binary: replaces crates/maidenx_cuda/src/ops/binary.rs:12-161 --------------------------------
  * metadata = dims[n] | lhs_strides[n] | rhs_strides[n] | lhs_offset | rhs_offset   (NULL: contiguous)

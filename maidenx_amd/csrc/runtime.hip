@@ -96,6 +96,13 @@ int hip_set_stream(void* s) { g_stream = (hipStream_t)s; return 0; }
 void* hip_get_stream(void) { return (void*)g_stream; }
 int hip_synchronize(void) { return (int)hipStreamSynchronize(stream()); }
 
+// Events on the backend's stream, for timing kernels where they run.
+int hip_event_create(void** ev) { return (int)hipEventCreate((hipEvent_t*)ev); }
+int hip_event_destroy(void* ev) { return (int)hipEventDestroy((hipEvent_t)ev); }
+int hip_event_record(void* ev) { return (int)hipEventRecord((hipEvent_t)ev, stream()); }
+int hip_event_synchronize(void* ev) { return (int)hipEventSynchronize((hipEvent_t)ev); }
+int hip_event_elapsed_ms(void* start, void* stop, float* ms) { return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop); }
+
 // First error recorded since the last call (0 = none); reading it clears it.
 int hip_get_last_status(void) {
     hipError_t e = hipGetLastError();

@@ -42,6 +42,9 @@ def load():
         ("hip_stream_create", [C.POINTER(C.c_void_p)], C.c_int), ("hip_stream_destroy", [C.c_void_p], C.c_int),
         ("hip_stream_synchronize", [C.c_void_p], C.c_int), ("hip_set_stream", [C.c_void_p], C.c_int),
         ("hip_get_stream", [], C.c_void_p), ("hip_synchronize", [], C.c_int),
+        ("hip_event_create", [C.POINTER(C.c_void_p)], C.c_int), ("hip_event_destroy", [C.c_void_p], C.c_int),
+        ("hip_event_record", [C.c_void_p], C.c_int), ("hip_event_synchronize", [C.c_void_p], C.c_int),
+        ("hip_event_elapsed_ms", [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)], C.c_int),
     ]:
         fn = getattr(lib, name)
         fn.argtypes = args
