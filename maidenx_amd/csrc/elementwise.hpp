@@ -27,7 +27,10 @@ struct EwPtrs {
 };
 
 constexpr int EW_BLOCK = 256;
-constexpr int EW_UNR = 4;
+#ifndef MXH_EW_UNR
+#define MXH_EW_UNR 4
+#endif
+constexpr int EW_UNR = MXH_EW_UNR;
 
 // ---- ew_nd -------------------------------------------------------------------------------
 template <class Op, int VEC>
@@ -115,6 +118,7 @@ struct TrPlan {
     uint32_t staged;       // bit k set: input k goes through LDS
     uint32_t tiles_p, tiles_l;
     FastDiv div_tiles_l, div_tiles_p;
+    uint32_t super;        // 8x8 super-tile block order (both tile counts are multiples of 8)
 };
 
 template <class Op>
@@ -179,6 +183,133 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_tr_kernel(NdSpace<Op::NIN + 1> sp
     }
 }
 
+// ---- ew_trv: vectorised form of ew_tr ------------------------------------------------------------------
+// Tile: TP = 256 bytes of the unit-stride dim p by 64 of the innermost dim.  Phase 1 reads the staged
+// operands with 128-bit loads along p (each 16-lane group covers one 256-byte row segment) and
+// writes them to LDS as tile[l][p]; phase 2 lets every lane gather VEC values down a column of that
+// tile (pitch chosen so that the 64 lanes hit distinct banks), combine them with 128-bit loads of
+// the other operands along the innermost dim, and store 128 bits.  Needs every dim and stride
+// involved to be a multiple of VEC and 16-byte aligned bases (checked by the host).
+template <class T> struct TrvCfg {
+    static constexpr int VEC = 16 / sizeof(T);
+    static constexpr int TP = 256 / sizeof(T);          // tile extent along p
+    static constexpr int TL = 64;                       // tile extent along the innermost dim
+    static constexpr int PITCH = sizeof(T) == 4 ? TP + 1 : TP + 2;
+};
+
+template <class Op>
+__global__ __launch_bounds__(EW_BLOCK) void ew_trv_kernel(NdSpace<Op::NIN + 1> sp, EwPtrs<Op::NIN> p, TrPlan<Op::NIN> pl,
+                                                          Op op) {
+    using In = typename Op::In;
+    using Out = typename Op::Out;
+    using Cfg = TrvCfg<In>;
+    constexpr int NIN = Op::NIN, VEC = Cfg::VEC, TP = Cfg::TP, TL = Cfg::TL, PITCH = Cfg::PITCH;
+    __shared__ __attribute__((aligned(16))) In tile[NIN][TL * PITCH];
+
+    const int last = sp.ndims - 1;
+    const int pd = pl.pdim;
+    uint32_t b = blockIdx.x, tl, tp, outer;
+    fd_divmod(b, pl.div_tiles_l, b, tl);
+    fd_divmod(b, pl.div_tiles_p, outer, tp);
+    if (pl.super) {
+        // Blocks that run at the same time form 8x8 groups of tiles: the reads (rows of the staged
+        // operand, one row pitch apart) and the writes (rows of the output, also a pitch apart) then
+        // both spread over the memory channels instead of one of them hammering a few.
+        constexpr uint32_t S = 8;
+        uint32_t lin = tp * pl.tiles_l + tl;
+        uint32_t per_row = pl.tiles_l / S;
+        uint32_t st = lin / (S * S), in = lin % (S * S);
+        tp = (st / per_row) * S + in / S;
+        tl = (st % per_row) * S + in % S;
+    }
+    int64_t base[NIN + 1];
+#pragma unroll
+    for (int k = 0; k <= NIN; ++k) base[k] = 0;
+    {
+        uint32_t r = outer;
+        for (int d = last - 1; d >= 0; --d) {
+            if (d == pd) continue;
+            uint32_t q, c;
+            fd_divmod(r, sp.div[d], q, c);
+#pragma unroll
+            for (int k = 0; k <= NIN; ++k) base[k] += (int64_t)c * sp.strides[k][d];
+            r = q;
+        }
+    }
+    const uint32_t i0 = tp * TP, j0 = tl * TL;
+    const uint32_t np = sp.dims[pd], nl = sp.dims[last];
+    const int t = threadIdx.x;
+
+    // phase 1: (TP/VEC) vectors per row of the tile, TL rows
+    constexpr int VPR = TP / VEC;                       // 16
+    constexpr int N1 = TL * VPR / EW_BLOCK;             // 4 vectors per thread
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) {
+        if (!((pl.staged >> k) & 1u)) continue;
+        const In* src = (const In*)p.in[k] + base[k + 1];
+        const int64_t sl = sp.strides[k + 1][last];
+        AVec<In, VEC> v[N1];
+#pragma unroll
+        for (int u = 0; u < N1; ++u) {
+            int id = t + u * EW_BLOCK;
+            uint32_t j = j0 + id / VPR, i = i0 + (id % VPR) * VEC;
+            if (i < np && j < nl) v[u] = *(const AVec<In, VEC>*)(src + (int64_t)i + (int64_t)j * sl);
+        }
+#pragma unroll
+        for (int u = 0; u < N1; ++u) {
+            int id = t + u * EW_BLOCK;
+            int jl = id / VPR, il = (id % VPR) * VEC;
+            // 32-bit LDS writes: the row pitch is not a multiple of 16 bytes
+            const uint32_t* w = (const uint32_t*)&v[u];
+            uint32_t* dst = (uint32_t*)(&tile[k][jl * PITCH + il]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = w[e];
+        }
+    }
+    __syncthreads();
+
+    // phase 2: rows along p, (TL/VEC) vectors per row
+    constexpr int VPL = TL / VEC;
+    constexpr int N2 = TP * VPL / EW_BLOCK;             // 4 vectors per thread
+#pragma unroll
+    for (int u = 0; u < N2; ++u) {
+        int id = t + u * EW_BLOCK;
+        int il = id / VPL, jl = (id % VPL) * VEC;
+        uint32_t i = i0 + il, j = j0 + jl;
+        if (i >= np || j >= nl) continue;
+        In x[NIN][VEC];
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) {
+            if ((pl.staged >> k) & 1u) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) x[k][e] = tile[k][(jl + e) * PITCH + il];
+            } else {
+                const In* src = (const In*)p.in[k] + base[k + 1] + (int64_t)i * sp.strides[k + 1][pd] + (int64_t)j * sp.strides[k + 1][last];
+                const int64_t s = sp.strides[k + 1][last];
+                if (s == 1) {
+                    AVec<In, VEC> tv = *(const AVec<In, VEC>*)src;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) x[k][e] = tv.v[e];
+                } else if (s == 0) {
+                    In tv = src[0];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) x[k][e] = tv;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) x[k][e] = src[(int64_t)e * s];
+                }
+            }
+        }
+        AVec<Out, VEC> o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            if constexpr (NIN == 1) o.v[e] = op(x[0][e]);
+            else o.v[e] = op(x[0][e], x[1][e]);
+        }
+        *(AVec<Out, VEC>*)((Out*)p.out + base[0] + (int64_t)i * sp.strides[0][pd] + (int64_t)j) = o;
+    }
+}
+
 // ---- host-side selection -------------------------------------------------------------------
 // in_strides[k] / out_strides are in elements, pointers already include the operand offsets.
 template <class Op>
@@ -223,6 +354,37 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
             TrPlan<NIN> pl;
             pl.pdim = pd;
             pl.staged = staged;
+            // vector form: every access of 16 bytes must be aligned and never straddle a tile edge
+            constexpr int TV = TrvCfg<In>::VEC;
+            bool trv = sizeof(Out) == sizeof(In) && sp.dims[pd] % TV == 0 && sp.dims[last] % TV == 0 &&
+                       (uintptr_t)out % 16 == 0;
+            for (int d = 0; d < last && trv; ++d) trv = sp.strides[0][d] % TV == 0;
+            for (int k = 0; k < NIN && trv; ++k) {
+                bool st = (staged >> k) & 1u;
+                int64_t sl = sp.strides[k + 1][last];
+                if (!st && sl != 1) continue;                      // scalar reads: no constraint
+                trv = (uintptr_t)in[k] % 16 == 0;
+                for (int d = 0; d <= last && trv; ++d) {
+                    if (st && d == pd) continue;
+                    if (!st && d == last) continue;
+                    trv = sp.strides[k + 1][d] % TV == 0;
+                }
+            }
+            pl.super = 0;
+            if (trv) {
+                pl.tiles_p = cdiv(sp.dims[pd], TrvCfg<In>::TP);
+                pl.tiles_l = cdiv(sp.dims[last], TrvCfg<In>::TL);
+                pl.super = (pl.tiles_p % 8 == 0 && pl.tiles_l % 8 == 0) ? 1u : 0u;
+                pl.div_tiles_l = make_fastdiv(pl.tiles_l);
+                pl.div_tiles_p = make_fastdiv(pl.tiles_p);
+                size_t outer = 1;
+                for (int d = 0; d < last; ++d)
+                    if (d != pd) outer *= sp.dims[d];
+                size_t blocks = outer * pl.tiles_p * pl.tiles_l;
+                hipLaunchKernelGGL(ew_trv_kernel<Op>, dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream(), sp, p, pl, op);
+                MXH_LAUNCH_CHECK("ew_trv");
+                return;
+            }
             pl.tiles_p = cdiv(sp.dims[pd], TR_TILE);
             pl.tiles_l = cdiv(sp.dims[last], TR_TILE);
             pl.div_tiles_l = make_fastdiv(pl.tiles_l);

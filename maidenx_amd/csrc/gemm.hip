@@ -49,26 +49,43 @@ template <> struct Elem<bf16_t> {
     static __device__ bf16_t zero() { return bf16_t{0}; }
 };
 
-constexpr int GB = 256;          // threads per block
-constexpr int TM = 128, TN = 128;
+constexpr int GB = 256;          // threads per block: 2 x 2 waves
 constexpr int TK_BYTES = 128;    // reduction extent of one staged tile, in bytes per row
 
 template <class T, int N> struct alignas(sizeof(T) * N) GVec { T v[N]; };
+// 16 bytes as a native vector: staged tiles and fragments stay in registers as whole dwordx4 values
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <class T> __device__ inline uint32_t elem_bits(T v);
+template <> __device__ inline uint32_t elem_bits<float>(float v) { return __builtin_bit_cast(uint32_t, v); }
+template <> __device__ inline uint32_t elem_bits<bf16_t>(bf16_t v) { return v.bits; }
+// pack VEC elements (given one by one) into 16 bytes
+template <class T> struct Pack16;
+template <> struct Pack16<float> {
+    u32x4 r;
+    __device__ void set(int e, float v) { uint32_t b = __builtin_bit_cast(uint32_t, v); r[e] = b; }
+};
+template <> struct Pack16<bf16_t> {
+    u32x4 r = {0u, 0u, 0u, 0u};
+    __device__ void set(int e, bf16_t v) { r[e / 2] |= (uint32_t)v.bits << (16 * (e & 1)); }
+};
 
-// ---- staging one 128 x TK operand tile into LDS as [row][TK + PAD] ---------------------------------
-// `rows` is the operand's output index (i for X, j for Y).  RCONT: the reduction index has
-// stride 1 in memory (natural); otherwise the row index has stride 1 and the tile is turned here.
-template <class T, bool RCONT>
+// ---- staging one ROWS x TK operand tile into LDS as [row][TK + PAD] ---------------------------------
+// `row` is the operand's output index (i for X, j for Y).  RCONT: the reduction index has stride 1
+// in memory (natural); otherwise the row index has stride 1 and the tile is turned on the way in.
+template <class T, bool RCONT, int ROWS>
 struct Stager {
     static constexpr int VEC = Elem<T>::VEC;
     static constexpr int TK = TK_BYTES / sizeof(T);
-    static constexpr int PITCH = TK + VEC;                 // keeps 16-byte alignment, skews banks
-    static constexpr int NV = TM * TK / VEC / GB;          // 16-byte units per thread (4)
-    GVec<T, VEC> reg[NV];
+    static constexpr int PITCH = TK + VEC;                 // +16 bytes: keeps alignment, spreads banks
+    static constexpr int NV = ROWS * TK / VEC / GB;        // 16-byte units per thread
+    static constexpr bool PAIRS = !RCONT && sizeof(T) == 2;
+    u32x4 reg[NV];
 
-    // natural: unit u → (row, kv);  turned: unit u → (r-group of VEC, row)
+    // FAST: the tile lies fully inside the operand and wide accesses are aligned (no checks at all)
+    template <bool FAST>
     __device__ void load(const T* __restrict__ base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0,
-                         uint32_t nrows, uint32_t nred, bool fast) {
+                         uint32_t nrows, uint32_t nred) {
+        constexpr bool fast = FAST;
         const int t = threadIdx.x;
         if constexpr (RCONT) {
             constexpr int KV = TK / VEC;   // vectors per row
@@ -77,27 +94,59 @@ struct Stager {
                 int id = t + u * GB;
                 uint32_t row = row0 + id / KV, red = red0 + (id % KV) * VEC;
                 const T* p = base + (int64_t)row * s_row + red;
-                if (fast) {
-                    reg[u] = *(const GVec<T, VEC>*)p;
+                if constexpr (fast) {
+                    reg[u] = *(const u32x4*)p;
                 } else {
+                    Pack16<T> pk;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e)
-                        reg[u].v[e] = (row < nrows && red + e < nred) ? p[e] : Elem<T>::zero();
+                    for (int e = 0; e < VEC; ++e) pk.set(e, (row < nrows && red + e < nred) ? p[e] : Elem<T>::zero());
+                    reg[u] = pk.r;
                 }
             }
+        } else if constexpr (PAIRS) {
+            // 16-bit elements: lanes run along pairs of rows (one dword = rows 2q, 2q+1 at one reduction
+            // step, 256 contiguous bytes per wave); 8 steps are gathered and re-packed into the two
+            // [row][k..k+8) vectors.  Units: (ROWS/2 pairs) x (TK/8 groups); NV counts 16-byte outputs.
+            constexpr int NP = ROWS / 2;
+#pragma unroll
+            for (int u = 0; u < NV / 2; ++u) {
+                int id = t + u * GB;
+                uint32_t row = row0 + (id % NP) * 2, red = red0 + (id / NP) * VEC;
+                const T* p = base + (int64_t)row + (int64_t)red * s_red;
+                uint32_t d[VEC];
+                if constexpr (fast) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) d[e] = *(const uint32_t*)(p + (int64_t)e * s_red);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        uint32_t lo = (row < nrows && red + e < nred) ? p[(int64_t)e * s_red].bits : 0u;
+                        uint32_t hi = (row + 1 < nrows && red + e < nred) ? p[(int64_t)e * s_red + 1].bits : 0u;
+                        d[e] = lo | (hi << 16);
+                    }
+                }
+                u32x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < VEC / 2; ++e) {
+                    lo[e] = (d[2 * e] & 0xffffu) | (d[2 * e + 1] << 16);
+                    hi[e] = (d[2 * e] >> 16) | (d[2 * e + 1] & 0xffff0000u);
+                }
+                reg[2 * u] = lo;
+                reg[2 * u + 1] = hi;
+            }
         } else {
-            // lanes run along the row index (stride 1 in memory); each unit gathers VEC reduction
-            // steps of one row so that the LDS write is again one 16-byte [row][k..k+VEC) vector.
-            constexpr int RG = TK / VEC;   // reduction groups per tile
+            // 32-bit elements: lanes run along the row index (stride 1 in memory); each unit gathers VEC
+            // reduction steps of one row so that the LDS write is again one [row][k..k+VEC) vector.
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
                 int id = t + u * GB;
-                uint32_t row = row0 + id % TM, red = red0 + (id / TM) * VEC;
+                uint32_t row = row0 + id % ROWS, red = red0 + (id / ROWS) * VEC;
                 const T* p = base + (int64_t)row + (int64_t)red * s_red;
-                (void)RG;
+                Pack16<T> pk;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e)
-                    reg[u].v[e] = (fast || (row < nrows && red + e < nred)) ? p[(int64_t)e * s_red] : Elem<T>::zero();
+                    pk.set(e, (fast || (row < nrows && red + e < nred)) ? p[(int64_t)e * s_red] : Elem<T>::zero());
+                reg[u] = pk.r;
             }
         }
     }
@@ -105,39 +154,48 @@ struct Stager {
         const int t = threadIdx.x;
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
-            int id = t + u * GB;
             int row, kk;
-            if constexpr (RCONT) { constexpr int KV = TK / VEC; row = id / KV; kk = (id % KV) * VEC; }
-            else { row = id % TM; kk = (id / TM) * VEC; }
-            *(GVec<T, VEC>*)(lds + row * PITCH + kk) = reg[u];
+            if constexpr (RCONT) { int id = t + u * GB; constexpr int KV = TK / VEC; row = id / KV; kk = (id % KV) * VEC; }
+            else if constexpr (PAIRS) { int id = t + (u / 2) * GB; constexpr int NP = ROWS / 2; row = (id % NP) * 2 + (u & 1); kk = (id / NP) * VEC; }
+            else { int id = t + u * GB; row = id % ROWS; kk = (id / ROWS) * VEC; }
+            *(u32x4*)(lds + row * PITCH + kk) = reg[u];
         }
     }
 };
 
 template <class T> struct Mma;
 template <> struct Mma<bf16_t> {
-    static __device__ void run(const GVec<bf16_t, 8>& a, const GVec<bf16_t, 8>& b, f32x16& c) {
+    static __device__ void run(const u32x4& a, const u32x4& b, f32x16& c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
 };
 template <> struct Mma<float> {
     // one 16-byte fragment feeds four 32x32x2 steps; lane (row, h) holds k = 4h .. 4h+3 of an
     // 8-wide slice, and step e pairs element e of both operands — any fixed pairing of k is valid.
-    static __device__ void run(const GVec<float, 4>& a, const GVec<float, 4>& b, f32x16& c) {
+    static __device__ void run(const u32x4& a, const u32x4& b, f32x16& c) {
+        // (whole-vector casts: a bit cast applied to a single vector element reads element 0)
+        const f32x4 af = __builtin_bit_cast(f32x4, a), bf = __builtin_bit_cast(f32x4, b);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[e], b.v[e], c, 0, 0, 0);
+        for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(af[e], bf[e], c, 0, 0, 0);
     }
 };
 
-template <class T, bool XR, bool YR>
+// MT x MT MFMA tiles (32x32) per wave: block tile = (64*MT) x (64*MT).  MT = 4 (256x256, one block
+// per CU, two LDS buffers) is the large-problem configuration; MT = 2 (128x128) serves small ones.
+// The MFMA is issued with the operands swapped (Y fragment as "A"), so the accumulator of a lane
+// holds 4 consecutive output columns of one output row and leaves as one packed store.
+template <class T, bool XR, bool YR, int MT, bool FAST>
 __global__ __launch_bounds__(GB) void gemm_mfma_kernel(GemmArgs g) {
-    using SX = Stager<T, XR>;
-    using SY = Stager<T, YR>;
+    constexpr int TM = 64 * MT, TN = 64 * MT;
+    using SX = Stager<T, XR, TM>;
+    using SY = Stager<T, YR, TN>;
     constexpr int VEC = Elem<T>::VEC;
     constexpr int TK = SX::TK;
     constexpr int PITCH = SX::PITCH;
-    __shared__ __attribute__((aligned(16))) T lds_x[TM * PITCH];
-    __shared__ __attribute__((aligned(16))) T lds_y[TN * PITCH];
+    constexpr int NBUF = MT == 4 ? 2 : 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    T* lds_x = (T*)smem;                                  // [NBUF][TM*PITCH]
+    T* lds_y = lds_x + NBUF * TM * PITCH;                 // [NBUF][TN*PITCH]
 
     // block → (batch, tile_i, tile_j); neighbouring blocks share the X panel (tile_j fastest)
     uint32_t bid = blockIdx.x;
@@ -153,70 +211,124 @@ __global__ __launch_bounds__(GB) void gemm_mfma_kernel(GemmArgs g) {
     const int wm = wave / 2, wn = wave % 2;
     const int lrow = lane % 32, lk = (lane / 32) * VEC;
 
-    f32x16 acc[2][2];
+    f32x16 acc[MT][MT];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < MT; ++a)
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < MT; ++c)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][c][e] = 0.0f;
-
-    // fast path: tile fully inside and every 16-byte access aligned
-    auto vec_ok = [&](const T* p, int64_t s_row, bool rcont) {
-        if (!rcont) return true;   // turned loads are scalar
-        return ((uintptr_t)p % 16 == 0) && (s_row % VEC == 0);
-    };
-    const bool x_full = i0 + TM <= g.I, y_full = j0 + TN <= g.J;
-    const bool x_al = vec_ok(X, g.xi, XR), y_al = vec_ok(Y, g.yj, YR);
 
     SX sx;
     SY sy;
     const uint32_t nk = (g.R + TK - 1) / TK;
-    {
-        bool kfull = TK <= g.R;
-        sx.load(X, g.xi, g.xr, i0, 0, g.I, g.R, x_full && kfull && x_al);
-        sy.load(Y, g.yj, g.yr, j0, 0, g.J, g.R, y_full && kfull && y_al);
-    }
-    for (uint32_t kt = 0; kt < nk; ++kt) {
+    sx.template load<FAST>(X, g.xi, g.xr, i0, 0, g.I, g.R);
+    sy.template load<FAST>(Y, g.yj, g.yr, j0, 0, g.J, g.R);
+    if constexpr (NBUF == 2) {
         sx.store(lds_x);
         sy.store(lds_y);
         __syncthreads();
+    }
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+        const int cur = NBUF == 2 ? (kt & 1) : 0;
+        if constexpr (NBUF == 1) {
+            sx.store(lds_x);
+            sy.store(lds_y);
+            __syncthreads();
+        }
         if (kt + 1 < nk) {
             uint32_t r0 = (kt + 1) * TK;
-            bool kfull = r0 + TK <= g.R;
-            sx.load(X, g.xi, g.xr, i0, r0, g.I, g.R, x_full && kfull && x_al);
-            sy.load(Y, g.yj, g.yr, j0, r0, g.J, g.R, y_full && kfull && y_al);
+            sx.template load<FAST>(X, g.xi, g.xr, i0, r0, g.I, g.R);
+            sy.template load<FAST>(Y, g.yj, g.yr, j0, r0, g.J, g.R);
         }
+        const T* cx = lds_x + cur * TM * PITCH;
+        const T* cy = lds_y + cur * TN * PITCH;
 #pragma unroll
         for (int s = 0; s < TK / (2 * VEC); ++s) {
-            GVec<T, VEC> fa[2], fb[2];
+            u32x4 fa[MT], fb[MT];
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
-                fa[a] = *(const GVec<T, VEC>*)(lds_x + (wm * 64 + a * 32 + lrow) * PITCH + s * 2 * VEC + lk);
+            for (int a = 0; a < MT; ++a)
+                fa[a] = *(const u32x4*)(cx + (wm * 32 * MT + a * 32 + lrow) * PITCH + s * 2 * VEC + lk);
 #pragma unroll
-            for (int c = 0; c < 2; ++c)
-                fb[c] = *(const GVec<T, VEC>*)(lds_y + (wn * 64 + c * 32 + lrow) * PITCH + s * 2 * VEC + lk);
+            for (int c = 0; c < MT; ++c)
+                fb[c] = *(const u32x4*)(cy + (wn * 32 * MT + c * 32 + lrow) * PITCH + s * 2 * VEC + lk);
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < MT; ++a)
 #pragma unroll
-                for (int c = 0; c < 2; ++c) Mma<T>::run(fa[a], fb[c], acc[a][c]);
+                for (int c = 0; c < MT; ++c) Mma<T>::run(fb[c], fa[a], acc[a][c]);
+        }
+        if constexpr (NBUF == 2) {
+            if (kt + 1 < nk) {
+                sx.store(lds_x + (cur ^ 1) * TM * PITCH);
+                sy.store(lds_y + (cur ^ 1) * TN * PITCH);
+            }
         }
         __syncthreads();
     }
 
-    // accumulator element e of a 32x32 tile: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32
+    // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
+    // column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
     T* out = (T*)g.out + (int64_t)b * g.I * g.J;
+    const bool vec_store = FAST || ((g.J % 4 == 0) && ((uintptr_t)out % (4 * sizeof(T)) == 0));
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < MT; ++a) {
+        uint32_t row = i0 + wm * 32 * MT + a * 32 + lrow;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            uint32_t col = j0 + wn * 64 + c * 32 + lrow;
+        for (int c = 0; c < MT; ++c) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                uint32_t row = i0 + wm * 64 + a * 32 + 8 * (e / 4) + 4 * (lane / 32) + (e % 4);
-                if (row < g.I && col < g.J) out[(int64_t)row * g.J + col] = Elem<T>::st(acc[a][c][e]);
+            for (int q = 0; q < 4; ++q) {
+                uint32_t col = j0 + wn * 32 * MT + c * 32 + 8 * q + 4 * (lane / 32);
+                if (!FAST && (row >= g.I || col >= g.J)) continue;
+                T* dst = out + (int64_t)row * g.J + col;
+                if (vec_store && (FAST || col + 4 <= g.J)) {
+                    GVec<T, 4> v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v.v[e] = Elem<T>::st(acc[a][c][4 * q + e]);
+                    *(GVec<T, 4>*)dst = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < g.J) dst[e] = Elem<T>::st(acc[a][c][4 * q + e]);
+                }
             }
         }
+    }
+}
+
+template <class T, bool XR, bool YR, int MT, bool FAST>
+void launch_mfma_impl(GemmArgs g) {
+    constexpr int TM = 64 * MT;
+    using SX = Stager<T, XR, TM>;
+    constexpr int NBUF = MT == 4 ? 2 : 1;
+    constexpr size_t lds_bytes = (size_t)2 * NBUF * TM * SX::PITCH * sizeof(T);
+    g.tiles_i = cdiv(g.I, TM);
+    g.tiles_j = cdiv(g.J, TM);
+    size_t blocks = (size_t)g.tiles_i * g.tiles_j * g.batch;
+    if (blocks >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "matmul: too many tiles"); return; }
+    auto kern = gemm_mfma_kernel<T, XR, YR, MT, FAST>;
+    static bool attr_done = false;     // per instantiation
+    if (!attr_done) {
+        MXH_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(GB), lds_bytes, stream(), g);
+    MXH_LAUNCH_CHECK("gemm_mfma");
+}
+
+// The unchecked kernel needs whole tiles in all three extents, 16-byte aligned rows for naturally laid
+// out operands (4-byte aligned row pairs for turned 16-bit ones) and an output it can store 4 wide.
+template <class T, bool XR, bool YR, int MT>
+void launch_mfma(GemmArgs g) {
+    constexpr int TM = 64 * MT, VEC = Elem<T>::VEC, TK = TK_BYTES / sizeof(T);
+    auto op_ok = [&](const void* p, int64_t s_batch, int64_t s_row, int64_t s_red, bool rcont) {
+        if (rcont) return (uintptr_t)p % 16 == 0 && s_row % VEC == 0 && s_batch % VEC == 0;
+        if (sizeof(T) == 2) return (uintptr_t)p % 4 == 0 && s_red % 2 == 0 && s_batch % 2 == 0;
+        return true;
+    };
+    bool fast = g.I % TM == 0 && g.J % TM == 0 && g.R % TK == 0 && op_ok(g.X, g.xb, g.xi, g.xr, XR) &&
+                op_ok(g.Y, g.yb, g.yj, g.yr, YR) && (uintptr_t)g.out % 16 == 0;
+    if (fast) launch_mfma_impl<T, XR, YR, MT, true>(g);
+    else launch_mfma_impl<T, XR, YR, MT, false>(g);
 }
 
 // ---- small shapes -----------------------------------------------------------------------------------
@@ -282,22 +394,22 @@ void gemm_dispatch(GemmArgs g) {
         MXH_LAUNCH_CHECK("gemm_wavedot");
         return;
     }
-    g.tiles_i = cdiv(g.I, TM);
-    g.tiles_j = cdiv(g.J, TN);
-    size_t blocks = (size_t)g.tiles_i * g.tiles_j * g.batch;
-    if (blocks >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "matmul: too many tiles"); return; }
     bool xr = g.xr == 1, yr = g.yr == 1;
     bool xi = g.xi == 1, yj = g.yj == 1;
-    dim3 grid((unsigned)blocks), blk(GB);
-    if (xr && yr) hipLaunchKernelGGL((gemm_mfma_kernel<T, true, true>), grid, blk, 0, stream(), g);
-    else if (xr && yj) hipLaunchKernelGGL((gemm_mfma_kernel<T, true, false>), grid, blk, 0, stream(), g);
-    else if (xi && yr) hipLaunchKernelGGL((gemm_mfma_kernel<T, false, true>), grid, blk, 0, stream(), g);
-    else if (xi && yj) hipLaunchKernelGGL((gemm_mfma_kernel<T, false, false>), grid, blk, 0, stream(), g);
+    // 256x256 tiles when they fill the chip about as well as 128x128 ones would
+    size_t big_blocks = (size_t)cdiv(g.I, 256) * cdiv(g.J, 256) * g.batch;
+    bool big = g.I >= 256 && g.J >= 256 && big_blocks >= 192;
+#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, 4>(g) : launch_mfma<T, XR, YR, 2>(g))
+    if (xr && yr) MXH_GEMM_CASE(true, true);
+    else if (xr && yj) MXH_GEMM_CASE(true, false);
+    else if (xi && yr) MXH_GEMM_CASE(false, true);
+    else if (xi && yj) MXH_GEMM_CASE(false, false);
     else {
         // no unit stride on one operand: correct but slow
         hipLaunchKernelGGL(gemm_thread_kernel<T>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
+        MXH_LAUNCH_CHECK("gemm_thread");
     }
-    MXH_LAUNCH_CHECK("gemm_mfma");
+#undef MXH_GEMM_CASE
 }
 
 struct MMeta {

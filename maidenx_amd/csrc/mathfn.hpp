@@ -144,24 +144,22 @@ MXH_HD float m_expm1(float x) {
 
 MXH_HD float m_tanh(float x) {
     const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
-    float t, z;
     const int32_t jx = (int32_t)f2u(x);
     const int32_t ix = jx & 0x7fffffff;
     if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;   // inf, NaN
-    if (ix < 0x41b00000) {                    // |x| < 22
-        if (ix == 0) return x;                // +-0
-        if (ix < 0x24000000) return x * (one + x);   // |x| < 2^-55
-        if (ix >= 0x3f800000) {               // |x| >= 1
-            t = m_expm1(two * fabsf(x));
-            z = one - two / (t + two);
-        } else {
-            t = m_expm1(-two * fabsf(x));
-            z = -t / (t + two);
-        }
-    } else {
-        z = one - tiny;
-    }
-    return jx >= 0 ? z : -z;
+    // FDLIBM evaluates  1 - 2/(expm1(2|x|) + 2)  for |x| >= 1  and  -t/(t + 2), t = expm1(-2|x|)  below;
+    // both are one expm1 and one division, so each lane runs the same instructions with its own
+    // operands selected (the values, and therefore the bits, are those of the branchy original).
+    const bool big = ix >= 0x3f800000;
+    const float a2 = two * fabsf(x);
+    const float t = m_expm1(big ? a2 : -a2);
+    const float q = (big ? two : -t) / (t + two);
+    float z = big ? one - q : q;
+    if (ix >= 0x41b00000) z = one - tiny;         // |x| >= 22
+    float r = jx >= 0 ? z : -z;
+    if (ix < 0x24000000) r = x * (one + x);       // |x| < 2^-55
+    if (ix == 0) r = x;                           // +-0
+    return r;
 }
 
 MXH_HD float m_pow(float x, float c) { return (float)pow((double)x, (double)c); }

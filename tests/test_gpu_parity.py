@@ -36,6 +36,7 @@ BIN_LAYOUTS = {
     "rhs_row_bcast_odd": lambda: (LY.contiguous([17, 30], off=1), LY.broadcast([17, 30], [1, 30])),
     "lhs_col_bcast": lambda: (LY.broadcast([64, 48], [64, 1]), LY.contiguous([64, 48])),
     "lhs_transposed": lambda: (LY.permuted([192, 160], [1, 0]), LY.contiguous([192, 160])),
+    "lhs_transposed_supertiles": lambda: (LY.permuted([1024, 1024], [1, 0]), LY.contiguous([1024, 1024])),
     "lhs_transposed_ragged": lambda: (LY.permuted([70, 45], [1, 0], off=1), LY.contiguous([70, 45])),
     "both_transposed": lambda: (LY.permuted([100, 130], [1, 0]), LY.permuted([100, 130], [1, 0], off=2)),
     "nhwc_view_plus_bias": lambda: (LY.permuted([2, 64, 12, 12], [0, 3, 1, 2]), LY.broadcast([2, 64, 12, 12], [1, 64, 1, 1])),
