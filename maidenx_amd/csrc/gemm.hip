@@ -17,6 +17,8 @@
 // Small or skinny products (the MLP's [10000,3]x[3,1] and its [3,10000]x[10000,1] gradient) use
 // a thread-per-output kernel (bit-exact with the reference: k ascending, unfused f32) or a
 // wave-per-output dot kernel.
+#include <cstdlib>
+
 #include "mxh.hpp"
 
 namespace mxh {
@@ -49,7 +51,7 @@ template <> struct Elem<bf16_t> {
     static __device__ bf16_t zero() { return bf16_t{0}; }
 };
 
-constexpr int GB = 256;          // threads per block: 2 x 2 waves
+constexpr int GB = 256;          // threads per block of the small-shape kernels
 constexpr int TK_BYTES = 128;    // reduction extent of one staged tile, in bytes per row
 
 template <class T, int N> struct alignas(sizeof(T) * N) GVec { T v[N]; };
@@ -72,16 +74,26 @@ template <> struct Pack16<bf16_t> {
 // ---- staging one ROWS x TK operand tile into LDS as [row][TK + PAD] ---------------------------------
 // `row` is the operand's output index (i for X, j for Y).  RCONT: the reduction index has stride 1
 // in memory (natural); otherwise the row index has stride 1 and the tile is turned on the way in.
-template <class T, bool RCONT, int ROWS>
+// load() only issues global loads into registers; store() does any re-packing and writes LDS, so the
+// loads stay in flight across a whole k-tile of MFMAs.  NT = threads per block.
+template <class T, bool RCONT, int ROWS, int NT>
 struct Stager {
     static constexpr int VEC = Elem<T>::VEC;
     static constexpr int TK = TK_BYTES / sizeof(T);
     static constexpr int PITCH = TK + VEC;                 // +16 bytes: keeps alignment, spreads banks
-    static constexpr int NV = ROWS * TK / VEC / GB;        // 16-byte units per thread
+    static constexpr int NV = ROWS * TK / VEC / NT;        // 16-byte units per thread
     static constexpr bool PAIRS = !RCONT && sizeof(T) == 2;
-    u32x4 reg[NV];
+    static_assert(NV >= 1 && (!PAIRS || NV % 2 == 0), "tile too small for this block size");
+    u32x4 reg[NV];     // natural / 32-bit turned: final vectors.  16-bit turned: raw dwords (row pairs)
 
-    // FAST: the tile lies fully inside the operand and wide accesses are aligned (no checks at all)
+    // Buffer descriptor of one tile: the (uniform) tile origin is the base, so every lane addresses with
+    // one loop-invariant 32-bit offset plus a scalar offset per load instead of a 64-bit pointer each.
+    static __device__ __amdgpu_buffer_rsrc_t tile_rsrc(const T* base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0) {
+        const T* origin = base + (int64_t)row0 * s_row + (int64_t)red0 * s_red;
+        return __builtin_amdgcn_make_buffer_rsrc((void*)origin, 0, 0x7fffffff, 0x00020000);
+    }
+    // FAST: the tile lies fully inside the operand, wide accesses are aligned and offsets inside a tile
+    // fit 31 bits (no checks at all)
     template <bool FAST>
     __device__ void load(const T* __restrict__ base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0,
                          uint32_t nrows, uint32_t nred) {
@@ -91,11 +103,13 @@ struct Stager {
             constexpr int KV = TK / VEC;   // vectors per row
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
-                int id = t + u * GB;
+                int id = t + u * NT;
                 uint32_t row = row0 + id / KV, red = red0 + (id % KV) * VEC;
                 const T* p = base + (int64_t)row * s_row + red;
                 if constexpr (fast) {
-                    reg[u] = *(const u32x4*)p;
+                    uint32_t voff = (uint32_t)(((t / KV) * s_row + (t % KV) * VEC) * (int64_t)sizeof(T));
+                    uint32_t soff = (uint32_t)((int64_t)u * (NT / KV) * s_row * (int64_t)sizeof(T));
+                    reg[u] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base, s_row, s_red, row0, red0), voff, soff, 0);
                 } else {
                     Pack16<T> pk;
 #pragma unroll
@@ -105,60 +119,78 @@ struct Stager {
             }
         } else if constexpr (PAIRS) {
             // 16-bit elements: lanes run along pairs of rows (one dword = rows 2q, 2q+1 at one reduction
-            // step, 256 contiguous bytes per wave); 8 steps are gathered and re-packed into the two
-            // [row][k..k+8) vectors.  Units: (ROWS/2 pairs) x (TK/8 groups); NV counts 16-byte outputs.
+            // step, 256 contiguous bytes per wave).  A unit gathers 8 steps = 8 dwords = reg[2u], reg[2u+1].
             constexpr int NP = ROWS / 2;
 #pragma unroll
             for (int u = 0; u < NV / 2; ++u) {
-                int id = t + u * GB;
+                int id = t + u * NT;
                 uint32_t row = row0 + (id % NP) * 2, red = red0 + (id / NP) * VEC;
                 const T* p = base + (int64_t)row + (int64_t)red * s_red;
-                uint32_t d[VEC];
-                if constexpr (fast) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) d[e] = *(const uint32_t*)(p + (int64_t)e * s_red);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
+                for (int e = 0; e < VEC; ++e) {
+                    uint32_t d;
+                    if constexpr (fast) {
+                        uint32_t voff = (uint32_t)(((t % NP) * 2 + (t / NP) * VEC * s_red) * (int64_t)sizeof(T));
+                        uint32_t soff = (uint32_t)(((int64_t)u * (NT / NP) * VEC + e) * s_red * (int64_t)sizeof(T));
+                        d = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0), voff, soff, 0);
+                    } else {
                         uint32_t lo = (row < nrows && red + e < nred) ? p[(int64_t)e * s_red].bits : 0u;
                         uint32_t hi = (row + 1 < nrows && red + e < nred) ? p[(int64_t)e * s_red + 1].bits : 0u;
-                        d[e] = lo | (hi << 16);
+                        d = lo | (hi << 16);
                     }
+                    reg[2 * u + e / 4][e % 4] = d;
                 }
-                u32x4 lo, hi;
-#pragma unroll
-                for (int e = 0; e < VEC / 2; ++e) {
-                    lo[e] = (d[2 * e] & 0xffffu) | (d[2 * e + 1] << 16);
-                    hi[e] = (d[2 * e] >> 16) | (d[2 * e + 1] & 0xffff0000u);
-                }
-                reg[2 * u] = lo;
-                reg[2 * u + 1] = hi;
             }
         } else {
             // 32-bit elements: lanes run along the row index (stride 1 in memory); each unit gathers VEC
             // reduction steps of one row so that the LDS write is again one [row][k..k+VEC) vector.
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
-                int id = t + u * GB;
+                int id = t + u * NT;
                 uint32_t row = row0 + id % ROWS, red = red0 + (id / ROWS) * VEC;
                 const T* p = base + (int64_t)row + (int64_t)red * s_red;
                 Pack16<T> pk;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    pk.set(e, (fast || (row < nrows && red + e < nred)) ? p[(int64_t)e * s_red] : Elem<T>::zero());
+                for (int e = 0; e < VEC; ++e) {
+                    if constexpr (fast) {
+                        uint32_t voff = (uint32_t)(((t % ROWS) + (t / ROWS) * VEC * s_red) * (int64_t)sizeof(T));
+                        uint32_t soff = (uint32_t)(((int64_t)u * (NT / ROWS) * VEC + e) * s_red * (int64_t)sizeof(T));
+                        pk.r[e] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0), voff, soff, 0);
+                    } else {
+                        pk.set(e, (row < nrows && red + e < nred) ? p[(int64_t)e * s_red] : Elem<T>::zero());
+                    }
+                }
                 reg[u] = pk.r;
             }
         }
     }
     __device__ void store(T* lds) const {
         const int t = threadIdx.x;
+        if constexpr (PAIRS) {
+            constexpr int NP = ROWS / 2;
 #pragma unroll
-        for (int u = 0; u < NV; ++u) {
-            int row, kk;
-            if constexpr (RCONT) { int id = t + u * GB; constexpr int KV = TK / VEC; row = id / KV; kk = (id % KV) * VEC; }
-            else if constexpr (PAIRS) { int id = t + (u / 2) * GB; constexpr int NP = ROWS / 2; row = (id % NP) * 2 + (u & 1); kk = (id / NP) * VEC; }
-            else { int id = t + u * GB; row = id % ROWS; kk = (id / ROWS) * VEC; }
-            *(u32x4*)(lds + row * PITCH + kk) = reg[u];
+            for (int u = 0; u < NV / 2; ++u) {
+                int id = t + u * NT;
+                int row = (id % NP) * 2, kk = (id / NP) * VEC;
+                // d[e] = (row, k+e) | (row+1, k+e) << 16  →  [row][k..k+8) and [row+1][k..k+8)
+                u32x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    uint32_t d0 = reg[2 * u + (2 * e) / 4][(2 * e) % 4], d1 = reg[2 * u + (2 * e + 1) / 4][(2 * e + 1) % 4];
+                    lo[e] = (d0 & 0xffffu) | (d1 << 16);
+                    hi[e] = (d0 >> 16) | (d1 & 0xffff0000u);
+                }
+                *(u32x4*)(lds + row * PITCH + kk) = lo;
+                *(u32x4*)(lds + (row + 1) * PITCH + kk) = hi;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                int id = t + u * NT, row, kk;
+                if constexpr (RCONT) { constexpr int KV = TK / VEC; row = id / KV; kk = (id % KV) * VEC; }
+                else { row = id % ROWS; kk = (id / ROWS) * VEC; }
+                *(u32x4*)(lds + row * PITCH + kk) = reg[u];
+            }
         }
     }
 };
@@ -180,22 +212,32 @@ template <> struct Mma<float> {
     }
 };
 
-// MT x MT MFMA tiles (32x32) per wave: block tile = (64*MT) x (64*MT).  MT = 4 (256x256, one block
-// per CU, two LDS buffers) is the large-problem configuration; MT = 2 (128x128) serves small ones.
+// Block = WM x WN waves, each wave MI x MJ MFMA tiles of 32x32: block tile (32*MI*WM) x (32*MJ*WN).
+//   Big  : 4 x 2 waves of 2 x 4 tiles = 256 x 256, 512 threads.  One wave alone can issue a 32x32x16
+//          MFMA only every other slot of the matrix pipe, so the pipe needs two waves per SIMD: 8 waves
+//          per CU with 128 accumulator registers each (measured: 1.29 vs 1.81 PFLOP/s for an
+//          MFMA-only loop with one vs two waves per SIMD).
+//   Small: 2 x 2 waves of 2 x 2 tiles = 128 x 128, 256 threads, for problems with few tiles.
 // The MFMA is issued with the operands swapped (Y fragment as "A"), so the accumulator of a lane
 // holds 4 consecutive output columns of one output row and leaves as one packed store.
-template <class T, bool XR, bool YR, int MT, bool FAST>
-__global__ __launch_bounds__(GB) void gemm_mfma_kernel(GemmArgs g) {
-    constexpr int TM = 64 * MT, TN = 64 * MT;
-    using SX = Stager<T, XR, TM>;
-    using SY = Stager<T, YR, TN>;
+template <int WM_, int WN_, int MI_, int MJ_> struct GemmCfg {
+    static constexpr int WM = WM_, WN = WN_, MI = MI_, MJ = MJ_;
+    static constexpr int NT = WAVE * WM * WN, TM = 32 * MI * WM, TN = 32 * MJ * WN;
+};
+using CfgBig = GemmCfg<4, 2, 2, 4>;
+using CfgSmall = GemmCfg<2, 2, 2, 2>;
+
+template <class T, bool XR, bool YR, class Cfg, bool FAST>
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
+    using SX = Stager<T, XR, TM, NT>;
+    using SY = Stager<T, YR, TN, NT>;
     constexpr int VEC = Elem<T>::VEC;
     constexpr int TK = SX::TK;
     constexpr int PITCH = SX::PITCH;
-    constexpr int NBUF = MT == 4 ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    T* lds_x = (T*)smem;                                  // [NBUF][TM*PITCH]
-    T* lds_y = lds_x + NBUF * TM * PITCH;                 // [NBUF][TN*PITCH]
+    T* lds_x = (T*)smem;                                  // [2][TM*PITCH]
+    T* lds_y = lds_x + 2 * TM * PITCH;                    // [2][TN*PITCH]
 
     // block → (batch, tile_i, tile_j); neighbouring blocks share the X panel (tile_j fastest)
     uint32_t bid = blockIdx.x;
@@ -208,62 +250,78 @@ __global__ __launch_bounds__(GB) void gemm_mfma_kernel(GemmArgs g) {
     const T* Y = (const T*)g.Y + (int64_t)b * g.yb;
 
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-    const int wm = wave / 2, wn = wave % 2;
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
     const int lrow = lane % 32, lk = (lane / 32) * VEC;
 
-    f32x16 acc[MT][MT];
+    f32x16 acc[MI][MJ];
 #pragma unroll
-    for (int a = 0; a < MT; ++a)
+    for (int a = 0; a < MI; ++a)
 #pragma unroll
-        for (int c = 0; c < MT; ++c)
+        for (int c = 0; c < MJ; ++c)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][c][e] = 0.0f;
 
+    // Software pipeline (all indices compile-time after unrolling, one barrier per k-tile):
+    //   registers : tile kt+1 (global loads issued one whole tile earlier)
+    //   LDS[cur]  : tile kt, read as fragments one k-step ahead of the MFMAs that consume them
+    //   last step : registers -> LDS[cur^1], then the global loads of tile kt+2 are issued
+    // Loads past the last tile are redirected to it (harmless re-reads) so the loop body has no branches.
+    constexpr int S = TK / (2 * VEC);                       // k-steps per tile (4)
     SX sx;
     SY sy;
     const uint32_t nk = (g.R + TK - 1) / TK;
     sx.template load<FAST>(X, g.xi, g.xr, i0, 0, g.I, g.R);
     sy.template load<FAST>(Y, g.yj, g.yr, j0, 0, g.J, g.R);
-    if constexpr (NBUF == 2) {
-        sx.store(lds_x);
-        sy.store(lds_y);
-        __syncthreads();
+    sx.store(lds_x);
+    sy.store(lds_y);
+    {
+        uint32_t r1 = (nk > 1 ? 1u : 0u) * TK;
+        sx.template load<FAST>(X, g.xi, g.xr, i0, r1, g.I, g.R);
+        sy.template load<FAST>(Y, g.yj, g.yr, j0, r1, g.J, g.R);
     }
+    __syncthreads();
+
+    const int frag_x = (wm * 32 * MI + lrow) * PITCH + lk;   // + a*32*PITCH + s*2*VEC
+    const int frag_y = (wn * 32 * MJ + lrow) * PITCH + lk;
+    u32x4 fa[2][MI], fb[2][MJ];
+#pragma unroll
+    for (int a = 0; a < MI; ++a) fa[0][a] = *(const u32x4*)(lds_x + frag_x + a * 32 * PITCH);
+#pragma unroll
+    for (int c = 0; c < MJ; ++c) fb[0][c] = *(const u32x4*)(lds_y + frag_y + c * 32 * PITCH);
+
     for (uint32_t kt = 0; kt < nk; ++kt) {
-        const int cur = NBUF == 2 ? (kt & 1) : 0;
-        if constexpr (NBUF == 1) {
-            sx.store(lds_x);
-            sy.store(lds_y);
-            __syncthreads();
-        }
-        if (kt + 1 < nk) {
-            uint32_t r0 = (kt + 1) * TK;
-            sx.template load<FAST>(X, g.xi, g.xr, i0, r0, g.I, g.R);
-            sy.template load<FAST>(Y, g.yj, g.yr, j0, r0, g.J, g.R);
-        }
+        const int cur = kt & 1;
         const T* cx = lds_x + cur * TM * PITCH;
         const T* cy = lds_y + cur * TN * PITCH;
 #pragma unroll
-        for (int s = 0; s < TK / (2 * VEC); ++s) {
-            u32x4 fa[MT], fb[MT];
+        for (int s = 0; s < S; ++s) {
+            if (s + 1 < S) {
 #pragma unroll
-            for (int a = 0; a < MT; ++a)
-                fa[a] = *(const u32x4*)(cx + (wm * 32 * MT + a * 32 + lrow) * PITCH + s * 2 * VEC + lk);
+                for (int a = 0; a < MI; ++a) fa[(s + 1) & 1][a] = *(const u32x4*)(cx + frag_x + a * 32 * PITCH + (s + 1) * 2 * VEC);
 #pragma unroll
-            for (int c = 0; c < MT; ++c)
-                fb[c] = *(const u32x4*)(cy + (wn * 32 * MT + c * 32 + lrow) * PITCH + s * 2 * VEC + lk);
-#pragma unroll
-            for (int a = 0; a < MT; ++a)
-#pragma unroll
-                for (int c = 0; c < MT; ++c) Mma<T>::run(fb[c], fa[a], acc[a][c]);
-        }
-        if constexpr (NBUF == 2) {
-            if (kt + 1 < nk) {
+                for (int c = 0; c < MJ; ++c) fb[(s + 1) & 1][c] = *(const u32x4*)(cy + frag_y + c * 32 * PITCH + (s + 1) * 2 * VEC);
+            } else {
                 sx.store(lds_x + (cur ^ 1) * TM * PITCH);
                 sy.store(lds_y + (cur ^ 1) * TN * PITCH);
+                uint32_t nt = kt + 2 < nk ? kt + 2 : nk - 1;
+                sx.template load<FAST>(X, g.xi, g.xr, i0, nt * TK, g.I, g.R);
+                sy.template load<FAST>(Y, g.yj, g.yr, j0, nt * TK, g.J, g.R);
             }
+            // keep the memory operations of the next stage ahead of this step's MFMAs: the matrix
+            // pipe then works through them while LDS and the vector memory unit serve the next step
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int a = 0; a < MI; ++a)
+#pragma unroll
+                for (int c = 0; c < MJ; ++c) Mma<T>::run(fb[s & 1][c], fa[s & 1][a], acc[a][c]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
+        // first fragments of the next tile (the barrier above made LDS[cur^1] visible)
+#pragma unroll
+        for (int a = 0; a < MI; ++a) fa[0][a] = *(const u32x4*)(lds_x + (cur ^ 1) * TM * PITCH + frag_x + a * 32 * PITCH);
+#pragma unroll
+        for (int c = 0; c < MJ; ++c) fb[0][c] = *(const u32x4*)(lds_y + (cur ^ 1) * TN * PITCH + frag_y + c * 32 * PITCH);
     }
 
     // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
@@ -271,13 +329,13 @@ __global__ __launch_bounds__(GB) void gemm_mfma_kernel(GemmArgs g) {
     T* out = (T*)g.out + (int64_t)b * g.I * g.J;
     const bool vec_store = FAST || ((g.J % 4 == 0) && ((uintptr_t)out % (4 * sizeof(T)) == 0));
 #pragma unroll
-    for (int a = 0; a < MT; ++a) {
-        uint32_t row = i0 + wm * 32 * MT + a * 32 + lrow;
+    for (int a = 0; a < MI; ++a) {
+        uint32_t row = i0 + wm * 32 * MI + a * 32 + lrow;
 #pragma unroll
-        for (int c = 0; c < MT; ++c) {
+        for (int c = 0; c < MJ; ++c) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                uint32_t col = j0 + wn * 32 * MT + c * 32 + 8 * q + 4 * (lane / 32);
+                uint32_t col = j0 + wn * 32 * MJ + c * 32 + 8 * q + 4 * (lane / 32);
                 if (!FAST && (row >= g.I || col >= g.J)) continue;
                 T* dst = out + (int64_t)row * g.J + col;
                 if (vec_store && (FAST || col + 4 <= g.J)) {
@@ -295,40 +353,43 @@ __global__ __launch_bounds__(GB) void gemm_mfma_kernel(GemmArgs g) {
     }
 }
 
-template <class T, bool XR, bool YR, int MT, bool FAST>
+template <class T, bool XR, bool YR, class Cfg, bool FAST>
 void launch_mfma_impl(GemmArgs g) {
-    constexpr int TM = 64 * MT;
-    using SX = Stager<T, XR, TM>;
-    constexpr int NBUF = MT == 4 ? 2 : 1;
-    constexpr size_t lds_bytes = (size_t)2 * NBUF * TM * SX::PITCH * sizeof(T);
-    g.tiles_i = cdiv(g.I, TM);
-    g.tiles_j = cdiv(g.J, TM);
+    using SX = Stager<T, XR, Cfg::TM, Cfg::NT>;
+    constexpr size_t lds_bytes = (size_t)2 * (Cfg::TM + Cfg::TN) * SX::PITCH * sizeof(T);
+    g.tiles_i = cdiv(g.I, Cfg::TM);
+    g.tiles_j = cdiv(g.J, Cfg::TN);
     size_t blocks = (size_t)g.tiles_i * g.tiles_j * g.batch;
     if (blocks >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "matmul: too many tiles"); return; }
-    auto kern = gemm_mfma_kernel<T, XR, YR, MT, FAST>;
+    auto kern = gemm_mfma_kernel<T, XR, YR, Cfg, FAST>;
     static bool attr_done = false;     // per instantiation
     if (!attr_done) {
         MXH_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(GB), lds_bytes, stream(), g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), lds_bytes, stream(), g);
     MXH_LAUNCH_CHECK("gemm_mfma");
 }
 
 // The unchecked kernel needs whole tiles in all three extents, 16-byte aligned rows for naturally laid
 // out operands (4-byte aligned row pairs for turned 16-bit ones) and an output it can store 4 wide.
-template <class T, bool XR, bool YR, int MT>
+template <class T, bool XR, bool YR, class Cfg>
 void launch_mfma(GemmArgs g) {
-    constexpr int TM = 64 * MT, VEC = Elem<T>::VEC, TK = TK_BYTES / sizeof(T);
+    constexpr int VEC = Elem<T>::VEC, TK = TK_BYTES / sizeof(T);
     auto op_ok = [&](const void* p, int64_t s_batch, int64_t s_row, int64_t s_red, bool rcont) {
         if (rcont) return (uintptr_t)p % 16 == 0 && s_row % VEC == 0 && s_batch % VEC == 0;
         if (sizeof(T) == 2) return (uintptr_t)p % 4 == 0 && s_red % 2 == 0 && s_batch % 2 == 0;
         return true;
     };
-    bool fast = g.I % TM == 0 && g.J % TM == 0 && g.R % TK == 0 && op_ok(g.X, g.xb, g.xi, g.xr, XR) &&
+    // per-thread offsets inside one tile are 32-bit
+    auto span_ok = [&](int64_t s_row, int64_t s_red, int rows) {
+        return s_row >= 0 && s_red >= 0 && ((int64_t)rows * s_row + (int64_t)TK * s_red) * (int64_t)sizeof(T) < (1ll << 31);
+    };
+    bool fast = span_ok(g.xi, g.xr, Cfg::TM) && span_ok(g.yj, g.yr, Cfg::TN) &&
+                g.I % Cfg::TM == 0 && g.J % Cfg::TN == 0 && g.R % TK == 0 && op_ok(g.X, g.xb, g.xi, g.xr, XR) &&
                 op_ok(g.Y, g.yb, g.yj, g.yr, YR) && (uintptr_t)g.out % 16 == 0;
-    if (fast) launch_mfma_impl<T, XR, YR, MT, true>(g);
-    else launch_mfma_impl<T, XR, YR, MT, false>(g);
+    if (fast) launch_mfma_impl<T, XR, YR, Cfg, true>(g);
+    else launch_mfma_impl<T, XR, YR, Cfg, false>(g);
 }
 
 // ---- small shapes -----------------------------------------------------------------------------------
@@ -399,7 +460,8 @@ void gemm_dispatch(GemmArgs g) {
     // 256x256 tiles when they fill the chip about as well as 128x128 ones would
     size_t big_blocks = (size_t)cdiv(g.I, 256) * cdiv(g.J, 256) * g.batch;
     bool big = g.I >= 256 && g.J >= 256 && big_blocks >= 192;
-#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, 4>(g) : launch_mfma<T, XR, YR, 2>(g))
+    if (getenv("MXH_FORCE_MT2")) big = false;
+#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, CfgBig>(g) : launch_mfma<T, XR, YR, CfgSmall>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
     else if (xr && yj) MXH_GEMM_CASE(true, false);
     else if (xi && yr) MXH_GEMM_CASE(false, true);
