@@ -94,15 +94,19 @@ struct Stager {
     }
     // FAST: the tile lies fully inside the operand, wide accesses are aligned and offsets inside a tile
     // fit 31 bits (no checks at all)
+    // A "unit" is what one pass of all threads loads: NU of them make the tile.  load()/store() take a
+    // unit range so that a tile's traffic can be spread over the k-steps of the previous tile.
+    static constexpr int NU = PAIRS ? NV / 2 : NV;
     template <bool FAST>
     __device__ void load(const T* __restrict__ base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0,
-                         uint32_t nrows, uint32_t nred) {
+                         uint32_t nrows, uint32_t nred, int u0 = 0, int u1 = NU) {
         constexpr bool fast = FAST;
         const int t = threadIdx.x;
         if constexpr (RCONT) {
             constexpr int KV = TK / VEC;   // vectors per row
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
+                if (u < u0 || u >= u1) continue;
                 int id = t + u * NT;
                 uint32_t row = row0 + id / KV, red = red0 + (id % KV) * VEC;
                 const T* p = base + (int64_t)row * s_row + red;
@@ -123,6 +127,7 @@ struct Stager {
             constexpr int NP = ROWS / 2;
 #pragma unroll
             for (int u = 0; u < NV / 2; ++u) {
+                if (u < u0 || u >= u1) continue;
                 int id = t + u * NT;
                 uint32_t row = row0 + (id % NP) * 2, red = red0 + (id / NP) * VEC;
                 const T* p = base + (int64_t)row + (int64_t)red * s_red;
@@ -146,6 +151,7 @@ struct Stager {
             // reduction steps of one row so that the LDS write is again one [row][k..k+VEC) vector.
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
+                if (u < u0 || u >= u1) continue;
                 int id = t + u * NT;
                 uint32_t row = row0 + id % ROWS, red = red0 + (id / ROWS) * VEC;
                 const T* p = base + (int64_t)row + (int64_t)red * s_red;
@@ -164,12 +170,13 @@ struct Stager {
             }
         }
     }
-    __device__ void store(T* lds) const {
+    __device__ void store(T* lds, int u0 = 0, int u1 = NU) const {
         const int t = threadIdx.x;
         if constexpr (PAIRS) {
             constexpr int NP = ROWS / 2;
 #pragma unroll
             for (int u = 0; u < NV / 2; ++u) {
+                if (u < u0 || u >= u1) continue;
                 int id = t + u * NT;
                 int row = (id % NP) * 2, kk = (id / NP) * VEC;
                 // d[e] = (row, k+e) | (row+1, k+e) << 16  →  [row][k..k+8) and [row+1][k..k+8)
@@ -186,6 +193,7 @@ struct Stager {
         } else {
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
+                if (u < u0 || u >= u1) continue;
                 int id = t + u * NT, row, kk;
                 if constexpr (RCONT) { constexpr int KV = TK / VEC; row = id / KV; kk = (id % KV) * VEC; }
                 else { row = id % ROWS; kk = (id / ROWS) * VEC; }
@@ -261,12 +269,16 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][c][e] = 0.0f;
 
-    // Software pipeline (all indices compile-time after unrolling, one barrier per k-tile):
-    //   registers : tile kt+1 (global loads issued one whole tile earlier)
-    //   LDS[cur]  : tile kt, read as fragments one k-step ahead of the MFMAs that consume them
-    //   last step : registers -> LDS[cur^1], then the global loads of tile kt+2 are issued
-    // Loads past the last tile are redirected to it (harmless re-reads) so the loop body has no branches.
+    // Software pipeline (all indices compile-time after unrolling, one barrier per k-tile).  While the
+    // MFMAs work through LDS[cur] (tile kt), step s < S-1 of the tile
+    //   * moves a share of the registers (tile kt+1, loaded one tile ago) into LDS[cur^1] and refills
+    //     them with the same share of tile kt+2, so LDS writes and global loads trickle instead of burst,
+    //   * reads the fragments of step s+1;
+    // the last step starts with the barrier (LDS[cur^1] complete, LDS[cur] no longer read by anyone
+    // once the fragments of step S-1 are in registers) and reads step 0 of the next tile under the cover
+    // of its own MFMAs.  Loads past the last tile are redirected to it (harmless re-reads).
     constexpr int S = TK / (2 * VEC);                       // k-steps per tile (4)
+    static_assert(S >= 2 && S % 2 == 0, "fragment double buffer assumes an even number of steps");
     SX sx;
     SY sy;
     const uint32_t nk = (g.R + TK - 1) / TK;
@@ -293,19 +305,28 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         const int cur = kt & 1;
         const T* cx = lds_x + cur * TM * PITCH;
         const T* cy = lds_y + cur * TN * PITCH;
+        T* nx = lds_x + (cur ^ 1) * TM * PITCH;
+        T* ny = lds_y + (cur ^ 1) * TN * PITCH;
+        const uint32_t nt = (kt + 2 < nk ? kt + 2 : nk - 1) * TK;
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             if (s + 1 < S) {
+                const int x0 = SX::NU * s / (S - 1), x1 = SX::NU * (s + 1) / (S - 1);
+                const int y0 = SY::NU * s / (S - 1), y1 = SY::NU * (s + 1) / (S - 1);
+                sx.store(nx, x0, x1);
+                sy.store(ny, y0, y1);
+                sx.template load<FAST>(X, g.xi, g.xr, i0, nt, g.I, g.R, x0, x1);
+                sy.template load<FAST>(Y, g.yj, g.yr, j0, nt, g.J, g.R, y0, y1);
 #pragma unroll
                 for (int a = 0; a < MI; ++a) fa[(s + 1) & 1][a] = *(const u32x4*)(cx + frag_x + a * 32 * PITCH + (s + 1) * 2 * VEC);
 #pragma unroll
                 for (int c = 0; c < MJ; ++c) fb[(s + 1) & 1][c] = *(const u32x4*)(cy + frag_y + c * 32 * PITCH + (s + 1) * 2 * VEC);
             } else {
-                sx.store(lds_x + (cur ^ 1) * TM * PITCH);
-                sy.store(lds_y + (cur ^ 1) * TN * PITCH);
-                uint32_t nt = kt + 2 < nk ? kt + 2 : nk - 1;
-                sx.template load<FAST>(X, g.xi, g.xr, i0, nt * TK, g.I, g.R);
-                sy.template load<FAST>(Y, g.yj, g.yr, j0, nt * TK, g.J, g.R);
+                __syncthreads();
+#pragma unroll
+                for (int a = 0; a < MI; ++a) fa[0][a] = *(const u32x4*)(nx + frag_x + a * 32 * PITCH);
+#pragma unroll
+                for (int c = 0; c < MJ; ++c) fb[0][c] = *(const u32x4*)(ny + frag_y + c * 32 * PITCH);
             }
             // keep the memory operations of the next stage ahead of this step's MFMAs: the matrix
             // pipe then works through them while LDS and the vector memory unit serve the next step
@@ -316,12 +337,6 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                 for (int c = 0; c < MJ; ++c) Mma<T>::run(fb[s & 1][c], fa[s & 1][a], acc[a][c]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
-        // first fragments of the next tile (the barrier above made LDS[cur^1] visible)
-#pragma unroll
-        for (int a = 0; a < MI; ++a) fa[0][a] = *(const u32x4*)(lds_x + (cur ^ 1) * TM * PITCH + frag_x + a * 32 * PITCH);
-#pragma unroll
-        for (int c = 0; c < MJ; ++c) fb[0][c] = *(const u32x4*)(lds_y + (cur ^ 1) * TN * PITCH + frag_y + c * 32 * PITCH);
     }
 
     // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
