@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the maidenx_hip backend on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul|copy]
 
 The default workload is BASELINE.json's configs[1]: elementwise forward + backward of add, mul, div,
 exp, relu, gelu on [8192,8192] tensors, f32 and bf16, for contiguous operands, a [1,8192] broadcast
@@ -258,6 +258,58 @@ def bind(lib, prefix):
             fn.argtypes, fn.restype = args, None
 
 
+def timed_run(L, lib, chains, args, probe_tag):
+    """W untimed passes, then K timed passes of `chains`; every launch tagged `probe_tag` in the timed
+    passes is bracketed by events on the backend's stream.  Returns (seconds, [ms per probed launch])."""
+    n_probe = sum(1 for c in chains if c.tag == probe_tag) * args.steps
+    ev = [(C.c_void_p(), C.c_void_p()) for _ in range(min(n_probe, 4096))]
+    for a, b in ev:
+        lib.hip_event_create(C.byref(a)); lib.hip_event_create(C.byref(b))
+    used = 0
+    for _ in range(args.warmup):
+        for c in chains:
+            c.fn(*c.args)
+    L.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        for c in chains:
+            if c.tag == probe_tag and used < len(ev):
+                a, b = ev[used]
+                lib.hip_event_record(a)
+                c.fn(*c.args)
+                lib.hip_event_record(b)
+                used += 1
+            else:
+                c.fn(*c.args)
+    L.synchronize()
+    dt_s = time.perf_counter() - t0
+    L.check()
+    ms = C.c_float()
+    durs = []
+    for a, b in ev[:used]:
+        lib.hip_event_elapsed_ms(a, b, C.byref(ms))
+        durs.append(ms.value)
+        lib.hip_event_destroy(a); lib.hip_event_destroy(b)
+    return dt_s, durs
+
+
+def base_result(args, value, unit, dt_s, dtype, workload, extra_cfg):
+    cfg = {"workload": workload}
+    cfg.update(extra_cfg)
+    return {"metric": "train steps/s; HBM GB/s elemwise/reduce; matmul TFLOP/s on 1 MI355X",
+            "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(dt_s / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": cfg}
+
+
+def hbm_roofline(kernel, nbytes, durs):
+    avg_ms = float(np.mean(durs))
+    achieved = nbytes / (avg_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(avg_ms * 1e3, 2), "launches_timed": len(durs),
+            "traffic": None}
+
+
 def run_elementwise(args):
     L, lib, alloc = hip_backend()
     R = Cc = 8192
@@ -267,58 +319,208 @@ def run_elementwise(args):
         chains += builders[-1].build()
     step_bytes = sum(c.bytes for c in chains)
     probe_tag = "mul_f32/contig+contig"           # the most frequent kernel of the chain
-    ev = [(C.c_void_p(), C.c_void_p()) for _ in range(4096)]
-    for a, b in ev:
-        lib.hip_event_create(C.byref(a)); lib.hip_event_create(C.byref(b))
-
-    def step(timed_events=None):
-        for c in chains:
-            if timed_events is not None and c.tag == probe_tag and timed_events[0] < len(ev):
-                a, b = ev[timed_events[0]]
-                lib.hip_event_record(a)
-                c.fn(*c.args)
-                lib.hip_event_record(b)
-                timed_events[0] += 1
-            else:
-                c.fn(*c.args)
-
-    for _ in range(args.warmup):
-        step()
-    L.synchronize()
-    used = [0]
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(used)
-    L.synchronize()
-    dt_s = time.perf_counter() - t0
-    ms = C.c_float()
-    durs = []
-    for a, b in ev[:used[0]]:
-        lib.hip_event_elapsed_ms(a, b, C.byref(ms))
-        durs.append(ms.value)
+    dt_s, durs = timed_run(L, lib, chains, args, probe_tag)
     probe_bytes = next(c.bytes for c in chains if c.tag == probe_tag)
-    avg_ms = float(np.mean(durs))
-    achieved = probe_bytes / (avg_ms * 1e-3) / 1e9
     value = step_bytes * args.steps / dt_s / 1e9
-    per_tag = {}
-    for c in chains:
-        per_tag[c.tag] = per_tag.get(c.tag, 0) + 1
-    result = {
-        "metric": "train steps/s; HBM GB/s elemwise/reduce; matmul TFLOP/s on 1 MI355X",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(dt_s / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32+bf16", "data": "synthetic",
-        "config": {"workload": "configs[1]: elementwise fwd+bwd (add,mul,div,exp,relu,gelu) on [8192,8192], f32+bf16, "
-                               "contiguous / rhs [1,8192] broadcast / transposed lhs", "kernel_launches_per_step": len(chains),
-                   "algorithmic_GB_per_step": round(step_bytes / 1e9, 3)},
-        "roofline": {"bound": "hbm", "kernel": "ew_nd_kernel<OpMul<float>,4> (hip_mul_f32, contiguous [8192,8192])",
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "avg_launch_us": round(avg_ms * 1e3, 2), "launches_timed": len(durs), "traffic": None},
-    }
+    result = base_result(args, round(value, 1), "GB/s", dt_s, "f32+bf16",
+                         "configs[1]: elementwise fwd+bwd (add,mul,div,exp,relu,gelu) on [8192,8192], f32+bf16, "
+                         "contiguous / rhs [1,8192] broadcast / transposed lhs",
+                         {"kernel_launches_per_step": len(chains), "algorithmic_GB_per_step": round(step_bytes / 1e9, 3)})
+    result["roofline"] = hbm_roofline("ew_nd_kernel<OpMul<float>,4> (hip_mul_f32, contiguous [8192,8192])", probe_bytes, durs)
     L.synchronize()
     del chains, builders
-    result["cpu_baseline"] = cpu_baseline_elementwise(args)
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_elementwise(args)
     return result
+
+
+def run_copy(args):
+    """Counter calibration: nothing but contiguous copies of a [8192,8192] f32 tensor (268.4 MB read +
+    268.4 MB written per launch), so that HBM byte counters can be scaled by a kernel of known traffic."""
+    L, lib, alloc = hip_backend()
+    N = 8192 * 8192
+    src, dst = L.DeviceBuffer(N * 4), L.DeviceBuffer(N * 4)
+    lib.hip_fill_f32(N, src.ptr, 1.0)
+    md = u64([8192, 8192], [8192, 1], 0)
+    chains = [Call(lib.hip_copy_strided_f32, (N, 2, md.ctypes.data, src.ptr, dst.ptr), 2 * N * 4, "copy_f32", md) for _ in range(8)]
+    dt_s, durs = timed_run(L, lib, chains, args, "copy_f32")
+    value = sum(c.bytes for c in chains) * args.steps / dt_s / 1e9
+    result = base_result(args, round(value, 1), "GB/s", dt_s, "f32", "calibration: 8 contiguous copies of [8192,8192] f32 per step", {})
+    result["roofline"] = hbm_roofline("ew_nd_kernel<OpCopy> (hip_copy_strided_f32, contiguous [8192,8192])", 2 * N * 4, durs)
+    result["cpu_baseline"] = None
+    return result
+
+
+def reduce_calls(lib, prefix, ptr_in, ptr_out, ptr_tmp, shape, dt="f32"):
+    """configs[2] on one input: sum/mean/max along every single axis and over all axes (the tensor layer
+    chains single-axis calls from the last axis to the first, crates/maidenx_tensor/src/ops/reduction.rs:9-21)."""
+    e = ESZ[dt]
+    calls = []
+    n = int(np.prod(shape))
+
+    def one(op, dims, axis, src, dst):
+        strides = [int(np.prod(dims[i + 1:])) for i in range(len(dims))]
+        md = u64(dims, strides, dims[axis], strides[axis], 0)
+        cnt = int(np.prod(dims))
+        calls.append(Call(getattr(lib, f"{prefix}{op}_{dt}"), (cnt, len(dims), 1, md.ctypes.data, src, dst),
+                          (cnt + cnt // dims[axis]) * e, f"{op}_{dt}/{'x'.join(map(str, dims))}/dim{axis}", md))
+    for op in ("sum", "mean", "max"):
+        for axis in range(len(shape)):
+            one(op, list(shape), axis, ptr_in, ptr_out)
+        dims, src, k = list(shape), ptr_in, 0          # all axes: last to first, ping-pong temporaries
+        while dims:
+            dst = (ptr_out, ptr_tmp)[k % 2]
+            one(op, dims, len(dims) - 1, src, dst)
+            dims, src, k = dims[:-1], dst, k + 1
+    return calls
+
+
+def run_reduce(args):
+    L, lib, alloc = hip_backend()
+    rng = np.random.default_rng(0x5EED0003)
+    chains, keep = [], []
+    for shape in ((8192, 8192), (64, 512, 1024)):
+        n = int(np.prod(shape))
+        x = L.DeviceBuffer.from_numpy(rng.uniform(-1, 1, n).astype(np.float32))
+        out, tmp = L.DeviceBuffer(n * 4), L.DeviceBuffer(n * 4)
+        keep += [x, out, tmp]
+        chains += reduce_calls(lib, "hip_", x.ptr, out.ptr, tmp.ptr, shape)
+        if len(shape) == 3:
+            md = u64(shape, [shape[1] * shape[2], shape[2], 1], [1, shape[1], 1], 0)
+            chains.append(Call(lib.hip_sum_to_shape_f32, (n, 3, md.ctypes.data, x.ptr, out.ptr), (n + shape[1]) * 4,
+                               "sum_to_shape_f32/64x512x1024->1x512x1", md))
+    step_bytes = sum(c.bytes for c in chains)
+    probe_tag = "sum_f32/8192x8192/dim0"
+    dt_s, durs = timed_run(L, lib, chains, args, probe_tag)
+    value = step_bytes * args.steps / dt_s / 1e9
+    result = base_result(args, round(value, 1), "GB/s", dt_s, "f32",
+                         "configs[2]: sum/mean/max along dim 0, dim 1, all dims of [8192,8192] and [64,512,1024] f32, "
+                         "plus sum_to_shape [64,512,1024]->[1,512,1]",
+                         {"kernel_calls_per_step": len(chains), "algorithmic_GB_per_step": round(step_bytes / 1e9, 3)})
+    result["roofline"] = hbm_roofline("col_reduce_kernel<float,RSum> (hip_sum_f32, [8192,8192] along dim 0)",
+                                      next(c.bytes for c in chains if c.tag == probe_tag), durs)
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_reduce(args)
+    return result
+
+
+def cpu_baseline_reduce(args):
+    """configs[2] on the CPU oracle, threaded, on a bounded sample: [512,8192] and [4,512,1024]."""
+    from tests.helpers import ensure_oracle_built
+    lib = C.CDLL(ensure_oracle_built())
+    bind(lib, "oracle_")
+    lib.oracle_set_num_threads.restype = C.c_int
+    cores = lib.oracle_set_num_threads(0)
+    rng = np.random.default_rng(0x5EED0003)
+    chains, keep = [], []
+    for shape in ((512, 8192), (4, 512, 1024)):
+        n = int(np.prod(shape))
+        x = rng.uniform(-1, 1, n).astype(np.float32)
+        out, tmp = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        keep += [x, out, tmp]
+        chains += reduce_calls(lib, "oracle_", x.ctypes.data, out.ctypes.data, tmp.ctypes.data, shape)
+    nbytes = sum(c.bytes for c in chains)
+    t0, reps = time.perf_counter(), 0
+    while True:
+        for c in chains:
+            c.fn(*c.args)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 200:
+            break
+    el = time.perf_counter() - t0
+    return {"value": round(nbytes * reps / el / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"same calls on [512,8192] and [4,512,1024] (1/16 of the rows / batches), {reps} passes, {el:.1f} s"}
+
+
+def matmul_meta(batch, M, K, N):
+    if batch:
+        return u64(3, 3, 3, [batch, M, N], [batch, M, K], [batch, K, N], [M * K, K, 1], [K * N, N, 1], 0, 0)
+    return u64(2, 2, 2, [M, N], [M, K], [K, N], [K, 1], [N, 1], 0, 0)
+
+
+def matmul_calls(lib, prefix, new, dt, shapes, rng):
+    """configs[3]: C = A.B, then matmul_backward giving dA = dC.B^T and dB = A^T.dC in one call."""
+    calls, keep = [], []
+    for batch, M, K, N in shapes:
+        b = max(batch, 1)
+        A = new(rng.standard_normal(b * M * K, dtype=np.float32), dt)
+        B = new(rng.standard_normal(b * K * N, dtype=np.float32) * np.float32(0.02), dt)
+        dC = new(rng.standard_normal(b * M * N, dtype=np.float32), dt)
+        Cc, dA, dB = new(np.zeros(b * M * N, np.float32), dt), new(np.zeros(b * M * K, np.float32), dt), new(np.zeros(b * K * N, np.float32), dt)
+        keep += [A, B, dC, Cc, dA, dB]
+        md = matmul_meta(batch, M, K, N)
+        flop = 2.0 * b * M * N * K
+        name = f"{dt}/{'%dx' % batch if batch else ''}{M}x{K}x{N}"
+        calls.append(Call(getattr(lib, f"{prefix}matmul_{dt}"), (b * M * N, md.ctypes.data, A[0], B[0], Cc[0]), flop, f"matmul_{name}", md))
+        calls.append(Call(getattr(lib, f"{prefix}matmul_backward_{dt}"), (b * M * K, b * K * N, md.ctypes.data, dC[0], A[0], B[0], dA[0], dB[0]),
+                          2 * flop, f"matmul_backward_{name}", md))
+    return calls, keep
+
+
+def run_matmul(args):
+    L, lib, alloc = hip_backend()
+    rng = np.random.default_rng(0x5EED0004)
+
+    def new(arr, dt):
+        buf = L.DeviceBuffer.from_numpy(f32_to_bf16(arr) if dt == "bf16" else arr)
+        return buf.ptr, buf
+    shapes = ((0, 4096, 4096, 4096), (32, 512, 1024, 1024))
+    chains, keep = [], []
+    for dt in ("bf16", "f32"):
+        c, k = matmul_calls(lib, "hip_", new, dt, shapes, rng)
+        chains += c; keep += k
+    # the headline figure is the bf16 4096^3 forward + backward; f32 and the batched shape are reported beside it
+    def rate(tags):
+        sel = [c for c in chains if c.tag in tags]
+        a = argparse.Namespace(steps=args.steps, warmup=args.warmup)
+        dt_s, _ = timed_run(L, lib, sel, a, None)
+        return sum(c.bytes for c in sel) * args.steps / dt_s / 1e12, dt_s
+    head = ("matmul_bf16/4096x4096x4096", "matmul_backward_bf16/4096x4096x4096")
+    sel = [c for c in chains if c.tag in head]
+    dt_s, durs = timed_run(L, lib, sel, args, head[0])
+    value = sum(c.bytes for c in sel) * args.steps / dt_s / 1e12
+    others = {}
+    for dt in ("bf16", "f32"):
+        for shp in ("4096x4096x4096", "32x512x1024x1024"):
+            tags = (f"matmul_{dt}/{shp}", f"matmul_backward_{dt}/{shp}")
+            others[f"{dt} {shp} fwd+bwd TFLOP/s"] = round(rate(tags)[0], 1)
+    result = base_result(args, round(value, 1), "TFLOP/s", dt_s, "bf16",
+                         "configs[3]: matmul forward + backward (dA = dC.B^T, dB = A^T.dC), [4096,4096]x[4096,4096] bf16; "
+                         "f32 and the batched [32,512,1024]x[32,1024,1024] shape reported in `all`", {"all": others})
+    fwd_flop = 2.0 * 4096 ** 3
+    avg_ms = float(np.mean(durs))
+    ach = fwd_flop / (avg_ms * 1e-3) / 1e12
+    result["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<bf16, 256x256x64> (hip_matmul_bf16 4096^3 forward)",
+                          "achieved": round(ach, 1), "peak": MFMA_PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                          "frac": round(ach / MFMA_PEAK_TFLOPS["bf16"], 4), "avg_launch_us": round(avg_ms * 1e3, 2),
+                          "launches_timed": len(durs), "traffic": None}
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_matmul(args)
+    return result
+
+
+def cpu_baseline_matmul(args):
+    """The CPU oracle's matmul forward + backward, threaded, bf16, on a bounded sample: 512^3 (1/512 of the
+    flops of 4096^3; the triple loop has no blocking, so its rate per flop does not improve with size)."""
+    from tests.helpers import ensure_oracle_built
+    lib = C.CDLL(ensure_oracle_built())
+    bind(lib, "oracle_")
+    lib.oracle_set_num_threads.restype = C.c_int
+    cores = lib.oracle_set_num_threads(0)
+    rng = np.random.default_rng(0x5EED0004)
+
+    def new(arr, dt):
+        a = f32_to_bf16(arr) if dt == "bf16" else np.ascontiguousarray(arr)
+        return a.ctypes.data, a
+    chains, keep = matmul_calls(lib, "oracle_", new, "bf16", ((0, 512, 512, 512),), rng)
+    flop = sum(c.bytes for c in chains)
+    t0, reps = time.perf_counter(), 0
+    while True:
+        for c in chains:
+            c.fn(*c.args)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 50:
+            break
+    el = time.perf_counter() - t0
+    return {"value": round(flop * reps / el / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"bf16 [512,512]x[512,512] forward + backward, {reps} passes, {el:.1f} s"}
 
 
 def cpu_baseline_elementwise(args):
@@ -368,13 +570,10 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X; nothing in this backend uses a second GPU (--gpus must be 1)")
-    if args.no_cpu_baseline:
-        global cpu_baseline_elementwise
-        cpu_baseline_elementwise = lambda a: None
-    if args.workload == "elementwise":
-        res = run_elementwise(args)
-    else:
-        sys.exit(f"unknown workload {args.workload}")
+    runners = {"elementwise": run_elementwise, "reduce": run_reduce, "matmul": run_matmul, "copy": run_copy}
+    if args.workload not in runners:
+        sys.exit(f"unknown workload {args.workload}: choose from {sorted(runners)}")
+    res = runners[args.workload](args)
     print(json.dumps(res))
 
 

@@ -17,7 +17,6 @@
 // Small or skinny products (the MLP's [10000,3]x[3,1] and its [3,10000]x[10000,1] gradient) use
 // a thread-per-output kernel (bit-exact with the reference: k ascending, unfused f32) or a
 // wave-per-output dot kernel.
-#include <cstdlib>
 
 #include "mxh.hpp"
 
@@ -475,7 +474,6 @@ void gemm_dispatch(GemmArgs g) {
     // 256x256 tiles when they fill the chip about as well as 128x128 ones would
     size_t big_blocks = (size_t)cdiv(g.I, 256) * cdiv(g.J, 256) * g.batch;
     bool big = g.I >= 256 && g.J >= 256 && big_blocks >= 192;
-    if (getenv("MXH_FORCE_MT2")) big = false;
 #define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, CfgBig>(g) : launch_mfma<T, XR, YR, CfgSmall>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
     else if (xr && yj) MXH_GEMM_CASE(true, false);
