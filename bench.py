@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the maidenx_hip backend on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul|mlp|conv|copy]
 
 The default workload is BASELINE.json's configs[1]: elementwise forward + backward of add, mul, div,
 exp, relu, gelu on [8192,8192] tensors, f32 and bf16, for contiguous operands, a [1,8192] broadcast
@@ -560,6 +560,133 @@ def cpu_baseline_elementwise(args):
             "sample": f"same kernel chain on [{R},{Cc}] tensors (1/32 of the rows), {reps} passes, {el:.1f} s"}
 
 
+def _mlp_setup(mx):
+    i = np.arange(10000)
+    x = np.stack([(i % 100) / 100.0, (i % 100 + 1) / 100.0, (i % 100 + 2) / 100.0], 1).astype(np.float32)
+    y = ((i % 100) * 10 / 1000.0).astype(np.float32).reshape(-1, 1)
+    lin = mx.Linear(in_features=3, out_features=1, with_bias=True, seed=0x5EED0000)
+    return lin, mx.tensor(x).with_grad(), mx.tensor(y)
+
+
+def run_mlp(args):
+    """configs[0]: the loop of examples/device/cpu.rs (Linear(3->1) + MSELoss + SGD(0.01), 10000x3 input, full batch)
+    through the host layer; a step is one epoch (forward, loss, backward, SGD step, zero_grad)."""
+    hip_backend()
+    from maidenx_amd.tensor import host
+    mx = host()
+    lin, x, y = _mlp_setup(mx)
+    steps = max(args.steps, 200)
+    mx.train(lin, x, y, 0.01, max(args.warmup, 20))
+    mx.synchronize()
+    mx.reset_backend_calls()
+    t0 = time.perf_counter()
+    mx.train(lin, x, y, 0.01, steps)
+    mx.synchronize()
+    dt_s = time.perf_counter() - t0
+    calls = mx.backend_calls() / steps
+    a = argparse.Namespace(steps=steps, warmup=max(args.warmup, 20))
+    result = base_result(a, round(steps / dt_s, 1), "steps/s", dt_s, "f32",
+                         "configs[0]: README Linear(3->1, bias) + MSE + SGD(lr=0.01), f32, full batch 10000x3",
+                         {"backend_kernels_per_step": calls, "us_per_step": round(dt_s / steps * 1e6, 1)})
+    result["roofline"] = None
+    result["note"] = "launch-latency bound (about 200 KB touched per step): no roofline fraction applies"
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_mlp(args)
+    return result
+
+
+def _oracle_host(threads):
+    from tests.helpers import ensure_oracle_built, oracle_host
+    lib = C.CDLL(ensure_oracle_built(), mode=C.RTLD_GLOBAL)
+    lib.oracle_set_num_threads.restype = C.c_int
+    cores = lib.oracle_set_num_threads(threads)
+    return oracle_host(), cores
+
+
+def cpu_baseline_mlp(args):
+    """The same loop with the host layer instantiated over the CPU oracle; the faster of the oracle's two modes
+    (sequential, or threaded over all cores like the reference's rayon loops) is reported."""
+    best = None
+    for threads in (1, 0):
+        mo, cores = _oracle_host(threads)
+        lin, x, y = _mlp_setup(mo)
+        mo.train(lin, x, y, 0.01, 5)
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < 5.0:
+            mo.train(lin, x, y, 0.01, 50)
+            n += 50
+        rate = n / (time.perf_counter() - t0)
+        if best is None or rate > best[0]:
+            best = (rate, cores, n)
+    return {"value": round(best[0], 1), "unit": "steps/s", "cores": best[1], "kind": "port",
+            "sample": f"same loop, {best[2]} steps on {best[1]} thread(s) (best of sequential and all-core modes)"}
+
+
+def _conv_setup(mx, B, seed=0x5EED0004):
+    rng = np.random.default_rng(seed)
+    Cin = Cout = 64
+    H = W = 56
+    bound = 1.0 / np.sqrt(Cin * 9)
+    x = mx.tensor(rng.standard_normal((B, Cin, H, W), dtype=np.float32)).with_grad()
+    w = mx.tensor(rng.uniform(-bound, bound, (Cout, Cin, 3, 3)).astype(np.float32))
+    b = mx.tensor(rng.uniform(-bound, bound, (Cout,)).astype(np.float32))
+    target = mx.tensor(rng.standard_normal((B, Cout, H, W), dtype=np.float32))
+    return mx.Conv2d(w, b, stride=(1, 1), padding=(1, 1)), x, target
+
+
+def _conv_step(mx, conv, x, target):
+    loss = mx.mse_loss(conv.forward(x), target)
+    loss.backward()
+    conv.zero_grad()
+    return loss
+
+
+def run_conv(args):
+    """configs[4]: Conv2d(64->64, 3x3, stride 1, pad 1, bias) forward + MSE + backward on [32,64,56,56] f32 through
+    the host layer (im2col -> GEMM -> bias add; backward: strided copy, GEMM, col2im, GEMM, bias sums)."""
+    L, lib, alloc = hip_backend()
+    from maidenx_amd.tensor import host
+    mx = host()
+    conv, x, target = _conv_setup(mx, 32)
+    for _ in range(max(args.warmup, 2)):
+        _conv_step(mx, conv, x, target)
+    mx.synchronize()
+    mx.reset_backend_calls()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        _conv_step(mx, conv, x, target)
+    mx.synchronize()
+    dt_s = time.perf_counter() - t0
+    result = base_result(args, round(args.steps / dt_s, 2), "steps/s", dt_s, "f32",
+                         "configs[4]: Conv2d 64->64 3x3 s1 p1 + bias, MSE loss, forward + backward, input [32,64,56,56] f32",
+                         {"backend_kernels_per_step": mx.backend_calls() / args.steps})
+    # dominant HBM kernel: im2col at this shape, timed on its own through the C ABI
+    Bn, Cc, H, W = 32, 64, 56, 56
+    n_in, n_col = Bn * Cc * H * W, Bn * H * W * Cc * 9
+    src, col = L.DeviceBuffer(n_in * 4), L.DeviceBuffer(n_col * 4)
+    lib.hip_fill_f32(n_in, src.ptr, 1.0)
+    md = u64(Bn, Cc, H, W, 3, 3, H, W, 1, 1, 1, 1)
+    calls = [Call(lib.hip_conv2d_im2col_f32, (n_col, md.ctypes.data, src.ptr, col.ptr), (n_in + n_col) * 4, "im2col", md) for _ in range(4)]
+    _, durs = timed_run(L, lib, calls, argparse.Namespace(steps=5, warmup=1), "im2col")
+    result["roofline"] = hbm_roofline("im2col_kernel<float,4> (hip_conv2d_im2col_f32, [32,64,56,56] 3x3)", (n_in + n_col) * 4, durs)
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_conv(args)
+    return result
+
+
+def cpu_baseline_conv(args):
+    """The same step on the CPU oracle, threaded, on a bounded sample: batch 2 instead of 32 (the step is linear in
+    the batch), scaled to full-size steps per second."""
+    mo, cores = _oracle_host(0)
+    conv, x, target = _conv_setup(mo, 2)
+    _conv_step(mo, conv, x, target)
+    t0, n = time.perf_counter(), 0
+    while time.perf_counter() - t0 < 10.0:
+        _conv_step(mo, conv, x, target)
+        n += 1
+    el = time.perf_counter() - t0
+    return {"value": round(n / el / 16.0, 4), "unit": "steps/s", "cores": cores, "kind": "port",
+            "sample": f"{n} steps at batch 2 in {el:.1f} s, divided by 16 for batch 32"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -570,7 +697,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X; nothing in this backend uses a second GPU (--gpus must be 1)")
-    runners = {"elementwise": run_elementwise, "reduce": run_reduce, "matmul": run_matmul, "copy": run_copy}
+    runners = {"elementwise": run_elementwise, "reduce": run_reduce, "matmul": run_matmul, "copy": run_copy, "mlp": run_mlp, "conv": run_conv}
     if args.workload not in runners:
         sys.exit(f"unknown workload {args.workload}: choose from {sorted(runners)}")
     res = runners[args.workload](args)

@@ -1,0 +1,103 @@
+/* maidenx_host.h — C ABI of the host layer (libmaidenx_host.so).
+ *
+ * The host layer replays MaidenX's tensor / autograd / nn calls above the backend kernels of
+ * maidenx_hip.h: each function below names the reference function whose backend-call sequence it issues.
+ * Tensors are opaque handles; a handle is released with mxt_release.  f32 only.
+ *
+ * Functions that return a handle return NULL on error, functions that return int return non-zero;
+ * mxt_last_error() then gives the error kind (the variant of crates/maidenx_core/src/error.rs that the
+ * reference would return) and its text.
+ */
+#ifndef MAIDENX_HOST_H
+#define MAIDENX_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mxt_tensor;
+typedef void* mxt_module;
+
+/* error kinds */
+#define MXT_OK 0
+#define MXT_ERR_INVALID_SHAPE 1
+#define MXT_ERR_SHAPE_MISMATCH 2
+#define MXT_ERR_DIM_OUT_OF_BOUNDS 3
+#define MXT_ERR_INCOMPATIBLE_SHAPE 4
+#define MXT_ERR_INVALID_OPERATION 5
+#define MXT_ERR_INVALID_ARGUMENT 6
+#define MXT_ERR_UNSUPPORTED_DTYPE 7
+#define MXT_ERR_OUT_OF_MEMORY 8
+#define MXT_ERR_BACKEND 9
+int mxt_last_error(char* text, size_t cap);      /* kind of the last failure on this thread; copies its text */
+const char* mxt_backend_name(void);
+
+/* creation: crates/maidenx_tensor/src/creation.rs:25-84 (new), :253-305 (fill); randn is seeded here */
+mxt_tensor mxt_new(const float* data, const size_t* shape, size_t ndim);
+mxt_tensor mxt_fill(const size_t* shape, size_t ndim, float value);
+mxt_tensor mxt_randn(const size_t* shape, size_t ndim, uint64_t seed);
+void mxt_release(mxt_tensor t);
+
+/* metadata */
+size_t mxt_ndim(mxt_tensor t);
+size_t mxt_size(mxt_tensor t);
+size_t mxt_offset(mxt_tensor t);
+void mxt_shape(mxt_tensor t, size_t* out);
+void mxt_strides(mxt_tensor t, size_t* out);
+int mxt_requires_grad(mxt_tensor t);
+int mxt_is_contiguous(mxt_tensor t);
+int mxt_to_host(mxt_tensor t, float* out);       /* logical (row-major) order; bool tensors as 0/1 */
+
+/* autograd: crates/maidenx_tensor/src/wt.rs:92-104, src/lib.rs:213-323 */
+int mxt_with_grad(mxt_tensor t);
+mxt_tensor mxt_grad(mxt_tensor t);               /* NULL without error text if the tensor has no grad */
+int mxt_backward(mxt_tensor t);
+int mxt_zero_grad(mxt_tensor t);
+mxt_tensor mxt_detach(mxt_tensor t);
+
+/* ops: crates/maidenx_tensor/src/ops/{binary,unary,reduction,matmul,transform}.rs
+ *   binary         : add sub mul div matmul
+ *   binary_inplace : add_ sub_
+ *   unary          : neg square relu tanh gelu exp sum_all mean_all contiguous squeeze_all
+ *   unary_scalar   : add_scalar mul_scalar div_scalar pow gt_scalar
+ *   reduce         : sum mean                      (dim may be negative)
+ *   shape_op       : view reshape (-1 allowed) broadcast sum_to_shape transpose (2 args) squeeze unsqueeze (1 arg) */
+mxt_tensor mxt_binary(const char* op, mxt_tensor a, mxt_tensor b);
+int mxt_binary_inplace(const char* op, mxt_tensor a, mxt_tensor b);
+mxt_tensor mxt_unary(const char* op, mxt_tensor a);
+mxt_tensor mxt_unary_scalar(const char* op, mxt_tensor a, float c);
+mxt_tensor mxt_reduce(const char* op, mxt_tensor a, int dim, int keep_dim);
+mxt_tensor mxt_shape_op(const char* op, mxt_tensor a, const int64_t* args, size_t nargs);
+
+/* nn: crates/maidenx_nn/src/layers/linear.rs:20-98, layers/conv.rs:100-322, losses/mse.rs:21-29,
+ * optimizers/sgd.rs:17-33.  Modules take their parameters as tensors (bias may be NULL). */
+mxt_module mxt_linear_new(mxt_tensor weight, mxt_tensor bias);
+mxt_module mxt_linear_new_seeded(size_t in_features, size_t out_features, int with_bias, uint64_t seed);
+mxt_module mxt_conv2d_new(mxt_tensor weight, mxt_tensor bias, size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                          size_t pad_h, size_t pad_w);
+mxt_tensor mxt_module_forward(mxt_module m, mxt_tensor input);
+mxt_tensor mxt_module_weight(mxt_module m);
+mxt_tensor mxt_module_bias(mxt_module m);        /* NULL if the module has none */
+void mxt_module_release(mxt_module m);
+mxt_tensor mxt_mse_loss(mxt_tensor pred, mxt_tensor target);
+int mxt_sgd_step(mxt_module m, float lr);
+int mxt_sgd_zero_grad(mxt_module m);
+
+/* The loop of examples/device/cpu.rs:32-38 (forward, MSE, backward, SGD step, zero_grad), `epochs` times,
+ * without leaving native code.  losses (may be NULL) receives the loss of every epoch; reading it costs one
+ * device-to-host copy per epoch, so pass NULL when timing. */
+int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_t epochs, float* losses);
+
+/* bookkeeping */
+size_t mxt_backend_calls(void);                  /* kernels dispatched since the last reset */
+void mxt_reset_backend_calls(void);
+size_t mxt_device_allocations(void);             /* allocations that reached the backend (pool misses) */
+int mxt_synchronize(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

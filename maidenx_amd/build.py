@@ -60,7 +60,25 @@ def build(force=False, verbose=False):
         p = subprocess.run(cmd, capture_output=True, text=True)
         if p.returncode != 0:
             raise RuntimeError("link failed:\n" + p.stdout + p.stderr)
+    build_host(force)
     return LIB
+
+
+HOST_LIB = os.path.join(HERE, "libmaidenx_host.so")
+
+
+def build_host(force=False):
+    """libmaidenx_host.so: the C++ host layer (tensor / autograd / nn) above the C ABI.  Plain host code."""
+    hdir = os.path.join(HERE, "host")
+    srcs = [os.path.join(hdir, f) for f in os.listdir(hdir)] + [os.path.join(HERE, "..", "include", "maidenx_host.h"), LIB]
+    if not force and os.path.exists(HOST_LIB) and os.path.getmtime(HOST_LIB) > max(os.path.getmtime(f) for f in srcs):
+        return HOST_LIB
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", os.path.join(hdir, "host_hip.cpp"), "-o", HOST_LIB,
+           "-L" + HERE, "-lmaidenx_hip", "-Wl,-rpath,$ORIGIN"]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("host layer build failed:\n" + p.stdout + p.stderr)
+    return HOST_LIB
 
 
 if __name__ == "__main__":

@@ -81,19 +81,20 @@ __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restr
     out[idx] = sum;
 }
 
-static bool parse_conv(const size_t* md, ConvMeta& m) {
+// need_stride: col2im divides by the stride slots (the reference panics on 0); im2col only multiplies by them
+static bool parse_conv(const size_t* md, ConvMeta& m, bool need_stride) {
     for (int k = 0; k < 12; ++k) if (md[k] >= (1ull << 31)) return false;
     m.B = (uint32_t)md[0]; m.C = (uint32_t)md[1]; m.H = (uint32_t)md[2]; m.W = (uint32_t)md[3];
     m.kh = (uint32_t)md[4]; m.kw = (uint32_t)md[5]; m.oh = (uint32_t)md[6]; m.ow = (uint32_t)md[7];
     m.ph = (uint32_t)md[8]; m.pw = (uint32_t)md[9]; m.sh = (uint32_t)md[10]; m.sw = (uint32_t)md[11];
-    return m.sh != 0 && m.sw != 0 && m.kh != 0 && m.kw != 0;
+    return (!need_stride || (m.sh != 0 && m.sw != 0)) && m.kh != 0 && m.kw != 0;
 }
 
 template <class T>
 void im2col(size_t num_els, const size_t* md, const T* in, T* col) {
     if (!md || !in || !col) return;    // the reference returns silently
     ConvMeta m;
-    if (!parse_conv(md, m)) { set_status(ERR_INVALID, "im2col: bad metadata"); return; }
+    if (!parse_conv(md, m, false)) { set_status(ERR_INVALID, "im2col: bad metadata"); return; }
     size_t full = (size_t)m.B * m.C * m.kh * m.kw * m.oh * m.ow;
     if (full == 0 || num_els == 0) return;
     if (full >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "im2col: 2^32 or more column elements"); return; }
@@ -113,7 +114,7 @@ template <class T>
 void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
     if (!md || !col || !out) return;
     ConvMeta m;
-    if (!parse_conv(md, m)) { set_status(ERR_INVALID, "col2im: bad metadata"); return; }
+    if (!parse_conv(md, m, true)) { set_status(ERR_INVALID, "col2im: bad metadata (stride slot is 0)"); return; }
     size_t n_out = (size_t)m.B * m.C * m.H * m.W;
     if (n_out == 0) return;
     if (n_out >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "col2im: 2^32 or more output elements"); return; }

@@ -34,6 +34,10 @@ struct GemmArgs {
     int64_t yb, yr, yj;   // element strides of Y: batch, reduction, output column
     uint32_t I, J, R, batch;
     uint32_t tiles_i, tiles_j;
+    // split-K: the reduction is cut into `splits` chunks of r_chunk (a multiple of the k-tile); with splits > 1
+    // every block writes its f32 partial tile to part[split][batch*I*J] and a second kernel folds them
+    uint32_t splits, r_chunk;
+    float* part;
 };
 
 template <class T> struct Elem;
@@ -233,6 +237,50 @@ template <int WM_, int WN_, int MI_, int MJ_> struct GemmCfg {
 };
 using CfgBig = GemmCfg<4, 2, 2, 4>;
 using CfgSmall = GemmCfg<2, 2, 2, 2>;
+using CfgTall = GemmCfg<4, 1, 2, 2>;     // 256 x 64: few output columns (the convolution GEMM has 64)
+
+// swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
+// column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
+template <class O, class Cfg, bool FAST>
+__device__ __forceinline__ void store_tile(O* out, const f32x16 (&acc)[Cfg::MI][Cfg::MJ], const GemmArgs& g, uint32_t i0, uint32_t j0,
+                                           int wm, int wn, int lane) {
+    constexpr int MI = Cfg::MI, MJ = Cfg::MJ;
+    const int lrow = lane % 32;
+    const bool vec_store = FAST || ((g.J % 4 == 0) && ((uintptr_t)out % (4 * sizeof(O)) == 0));
+#pragma unroll
+    for (int a = 0; a < MI; ++a) {
+        uint32_t row = i0 + wm * 32 * MI + a * 32 + lrow;
+#pragma unroll
+        for (int c = 0; c < MJ; ++c) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t col = j0 + wn * 32 * MJ + c * 32 + 8 * q + 4 * (lane / 32);
+                if (!FAST && (row >= g.I || col >= g.J)) continue;
+                O* dst = out + (int64_t)row * g.J + col;
+                if (vec_store && (FAST || col + 4 <= g.J)) {
+                    GVec<O, 4> v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v.v[e] = Elem<O>::st(acc[a][c][4 * q + e]);
+                    *(GVec<O, 4>*)dst = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < g.J) dst[e] = Elem<O>::st(acc[a][c][4 * q + e]);
+                }
+            }
+        }
+    }
+}
+
+// Folds the split-K partials in split order (deterministic) and rounds once.
+template <class T>
+__global__ __launch_bounds__(256) void gemm_fold_kernel(const float* __restrict__ part, T* __restrict__ out, size_t n, uint32_t splits) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float acc = part[i];
+    for (uint32_t s = 1; s < splits; ++s) acc += part[(size_t)s * n + i];
+    out[i] = Elem<T>::st(acc);
+}
 
 template <class T, bool XR, bool YR, class Cfg, bool FAST>
 __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
@@ -251,7 +299,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     uint32_t tj = bid % g.tiles_j;
     uint32_t rest = bid / g.tiles_j;
     uint32_t ti = rest % g.tiles_i;
-    uint32_t b = rest / g.tiles_i;
+    rest /= g.tiles_i;
+    uint32_t b = rest % g.batch;
+    const uint32_t split = rest / g.batch;
+    const uint32_t rb = split * g.r_chunk;                                  // this block reduces over [rb, re)
+    const uint32_t re = g.R - rb < g.r_chunk ? g.R : rb + g.r_chunk;
     const uint32_t i0 = ti * TM, j0 = tj * TN;
     const T* X = (const T*)g.X + (int64_t)b * g.xb;
     const T* Y = (const T*)g.Y + (int64_t)b * g.yb;
@@ -280,15 +332,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     static_assert(S >= 2 && S % 2 == 0, "fragment double buffer assumes an even number of steps");
     SX sx;
     SY sy;
-    const uint32_t nk = (g.R + TK - 1) / TK;
-    sx.template load<FAST>(X, g.xi, g.xr, i0, 0, g.I, g.R);
-    sy.template load<FAST>(Y, g.yj, g.yr, j0, 0, g.J, g.R);
+    const uint32_t nk = (re - rb + TK - 1) / TK;
+    sx.template load<FAST>(X, g.xi, g.xr, i0, rb, g.I, re);
+    sy.template load<FAST>(Y, g.yj, g.yr, j0, rb, g.J, re);
     sx.store(lds_x);
     sy.store(lds_y);
     {
-        uint32_t r1 = (nk > 1 ? 1u : 0u) * TK;
-        sx.template load<FAST>(X, g.xi, g.xr, i0, r1, g.I, g.R);
-        sy.template load<FAST>(Y, g.yj, g.yr, j0, r1, g.J, g.R);
+        uint32_t r1 = rb + (nk > 1 ? 1u : 0u) * TK;
+        sx.template load<FAST>(X, g.xi, g.xr, i0, r1, g.I, re);
+        sy.template load<FAST>(Y, g.yj, g.yr, j0, r1, g.J, re);
     }
     __syncthreads();
 
@@ -306,7 +358,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         const T* cy = lds_y + cur * TN * PITCH;
         T* nx = lds_x + (cur ^ 1) * TM * PITCH;
         T* ny = lds_y + (cur ^ 1) * TN * PITCH;
-        const uint32_t nt = (kt + 2 < nk ? kt + 2 : nk - 1) * TK;
+        const uint32_t nt = rb + (kt + 2 < nk ? kt + 2 : nk - 1) * TK;
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             if (s + 1 < S) {
@@ -314,8 +366,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                 const int y0 = SY::NU * s / (S - 1), y1 = SY::NU * (s + 1) / (S - 1);
                 sx.store(nx, x0, x1);
                 sy.store(ny, y0, y1);
-                sx.template load<FAST>(X, g.xi, g.xr, i0, nt, g.I, g.R, x0, x1);
-                sy.template load<FAST>(Y, g.yj, g.yr, j0, nt, g.J, g.R, y0, y1);
+                sx.template load<FAST>(X, g.xi, g.xr, i0, nt, g.I, re, x0, x1);
+                sy.template load<FAST>(Y, g.yj, g.yr, j0, nt, g.J, re, y0, y1);
 #pragma unroll
                 for (int a = 0; a < MI; ++a) fa[(s + 1) & 1][a] = *(const u32x4*)(cx + frag_x + a * 32 * PITCH + (s + 1) * 2 * VEC);
 #pragma unroll
@@ -338,32 +390,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         }
     }
 
-    // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
-    // column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
-    T* out = (T*)g.out + (int64_t)b * g.I * g.J;
-    const bool vec_store = FAST || ((g.J % 4 == 0) && ((uintptr_t)out % (4 * sizeof(T)) == 0));
-#pragma unroll
-    for (int a = 0; a < MI; ++a) {
-        uint32_t row = i0 + wm * 32 * MI + a * 32 + lrow;
-#pragma unroll
-        for (int c = 0; c < MJ; ++c) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t col = j0 + wn * 32 * MJ + c * 32 + 8 * q + 4 * (lane / 32);
-                if (!FAST && (row >= g.I || col >= g.J)) continue;
-                T* dst = out + (int64_t)row * g.J + col;
-                if (vec_store && (FAST || col + 4 <= g.J)) {
-                    GVec<T, 4> v;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v.v[e] = Elem<T>::st(acc[a][c][4 * q + e]);
-                    *(GVec<T, 4>*)dst = v;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (col + e < g.J) dst[e] = Elem<T>::st(acc[a][c][4 * q + e]);
-                }
-            }
-        }
+    if (g.splits > 1) {
+        float* part = g.part + ((int64_t)split * g.batch + b) * g.I * g.J;
+        store_tile<float, Cfg, FAST>(part, acc, g, i0, j0, wm, wn, lane);
+    } else {
+        store_tile<T, Cfg, FAST>((T*)g.out + (int64_t)b * g.I * g.J, acc, g, i0, j0, wm, wn, lane);
     }
 }
 
@@ -371,10 +402,31 @@ template <class T, bool XR, bool YR, class Cfg, bool FAST>
 void launch_mfma_impl(GemmArgs g) {
     using SX = Stager<T, XR, Cfg::TM, Cfg::NT>;
     constexpr size_t lds_bytes = (size_t)2 * (Cfg::TM + Cfg::TN) * SX::PITCH * sizeof(T);
+    constexpr uint32_t TK = TK_BYTES / sizeof(T);
     g.tiles_i = cdiv(g.I, Cfg::TM);
     g.tiles_j = cdiv(g.J, Cfg::TN);
-    size_t blocks = (size_t)g.tiles_i * g.tiles_j * g.batch;
+    size_t tiles = (size_t)g.tiles_i * g.tiles_j * g.batch;
+    // Few output tiles and a long reduction (dB of a wide batch, the weight gradient of a convolution):
+    // when the tiles cover less than half of the CUs, cut the reduction so that every CU has work,
+    // each block keeping at least 8 k-tiles.
+    g.splits = 1;
+    g.r_chunk = g.R;
+    g.part = nullptr;
+    const size_t want_blocks = Cfg::NT >= 512 ? 256 : 512;       // one or two resident blocks per CU
+    if (tiles <= 128 && g.R >= 16 * TK) {
+        uint32_t want = (uint32_t)std::min<size_t>(cdiv(want_blocks, tiles), g.R / (8 * TK));
+        if (want > 1) {
+            g.r_chunk = (uint32_t)(cdiv(cdiv(g.R, want), TK) * TK);
+            g.splits = (uint32_t)cdiv(g.R, g.r_chunk);
+        }
+    }
+    size_t blocks = tiles * g.splits;
     if (blocks >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "matmul: too many tiles"); return; }
+    const size_t n_out = (size_t)g.batch * g.I * g.J;
+    if (g.splits > 1) {
+        g.part = (float*)scratch(n_out * g.splits * sizeof(float));
+        if (!g.part) return;
+    }
     auto kern = gemm_mfma_kernel<T, XR, YR, Cfg, FAST>;
     static bool attr_done = false;     // per instantiation
     if (!attr_done) {
@@ -383,6 +435,10 @@ void launch_mfma_impl(GemmArgs g) {
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), lds_bytes, stream(), g);
     MXH_LAUNCH_CHECK("gemm_mfma");
+    if (g.splits > 1) {
+        hipLaunchKernelGGL(gemm_fold_kernel<T>, dim3((unsigned)cdiv(n_out, 256)), dim3(256), 0, stream(), g.part, (T*)g.out, n_out, g.splits);
+        MXH_LAUNCH_CHECK("gemm_fold");
+    }
 }
 
 // The unchecked kernel needs whole tiles in all three extents, 16-byte aligned rows for naturally laid
@@ -474,7 +530,8 @@ void gemm_dispatch(GemmArgs g) {
     // 256x256 tiles when they fill the chip about as well as 128x128 ones would
     size_t big_blocks = (size_t)cdiv(g.I, 256) * cdiv(g.J, 256) * g.batch;
     bool big = g.I >= 256 && g.J >= 256 && big_blocks >= 192;
-#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, CfgBig>(g) : launch_mfma<T, XR, YR, CfgSmall>(g))
+    const bool tall = !big && g.J <= 64 && g.I >= 1024;
+#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, CfgBig>(g) : tall ? launch_mfma<T, XR, YR, CfgTall>(g) : launch_mfma<T, XR, YR, CfgSmall>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
     else if (xr && yj) MXH_GEMM_CASE(true, false);
     else if (xi && yr) MXH_GEMM_CASE(false, true);

@@ -1,0 +1,1044 @@
+// Host layer above the backend C ABI: the tensor, autograd and nn calls of MaidenX, restated in C++ so
+// that whole training steps (Linear + MSELoss + SGD, Conv2d) can be driven through the backend kernels
+// exactly as the reference's tensor layer drives `maidenx_core::be::*`.
+//
+// Every operation builds the same metadata array and issues the same backend calls, in the same order,
+// as the reference function it names:
+//   crates/maidenx_tensor/src/lib.rs            Tensor, TensorNode, backward, accumulate_grad, zero_grad
+//   crates/maidenx_tensor/src/ops/binary.rs     add sub mul div add_ sub_
+//   crates/maidenx_tensor/src/ops/unary.rs      neg square relu tanh gelu exp *_scalar pow gt_scalar
+//   crates/maidenx_tensor/src/ops/reduction.rs  sum sum_all sum_to_shape mean mean_all
+//   crates/maidenx_tensor/src/ops/matmul.rs     matmul and its backward
+//   crates/maidenx_tensor/src/ops/transform.rs  view squeeze unsqueeze transpose broadcast reshape
+//   crates/maidenx_core/src/layout.rs           Layout
+//   crates/maidenx_nn/src/{layers/linear.rs,layers/conv.rs,losses/mse.rs,optimizers/sgd.rs}
+//
+// The code is a template over a Backend: a struct of static functions (memory, the f32 kernels, and the
+// few helpers the reference runs on the host: fill, strided copy, bool -> f32 cast, scalar broadcast).
+// Only f32 tensors (and bool results of comparisons) exist here; that is what the MLP and conv workloads use.
+//
+// Deliberate differences from the reference, none visible in results:
+//   * buffers come from a size-bucketed pool instead of one device allocation per tensor;
+//   * `with_buffer_mut`'s copy-on-write of a shared buffer (lib.rs:166-180) is not reproduced: in-place
+//     ops write the buffer they are given;
+//   * contiguous(), zeros/ones, bool -> f32 and the broadcast of a 0-d tensor run on the device when the
+//     backend offers a kernel for them (the reference goes through host memory).
+#pragma once
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <functional>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_set>
+#include <vector>
+
+namespace mxt {
+
+// ---- errors: the variants of crates/maidenx_core/src/error.rs this layer can raise -------------------
+enum class ErrKind { None = 0, InvalidShape, ShapeMismatch, DimensionOutOfBounds, IncompatibleShape, InvalidOperation,
+                     InvalidArgument, UnsupportedDType, OutOfMemory, Backend };
+struct Error : std::runtime_error {
+    ErrKind kind;
+    Error(ErrKind k, const std::string& m) : std::runtime_error(m), kind(k) {}
+};
+
+using Shape = std::vector<size_t>;
+inline size_t shape_size(const Shape& s) { size_t n = 1; for (size_t d : s) n *= d; return n; }
+inline std::string shape_str(const Shape& s) {
+    std::string r = "[";
+    for (size_t i = 0; i < s.size(); ++i) r += (i ? ", " : "") + std::to_string(s[i]);
+    return r + "]";
+}
+
+// ---- crates/maidenx_core/src/layout.rs ------------------------------------------------------------
+struct Layout {
+    Shape shape, strides;
+    size_t offset = 0;
+    static Shape compute_strides(const Shape& shape) {               // layout.rs:337-349
+        Shape st(shape.size(), 1);
+        for (size_t i = shape.size(); i-- > 1;) st[i - 1] = st[i] * shape[i];
+        return st;
+    }
+    static Layout from_shape(const Shape& s) { return Layout{s, compute_strides(s), 0}; }
+    size_t ndim() const { return shape.size(); }
+    size_t size() const { return shape_size(shape); }
+    bool is_contiguous() const {                                      // layout.rs:60-74 (size-1 dims count)
+        size_t expected = 1;
+        for (size_t i = ndim(); i-- > 0;) {
+            if (strides[i] != expected) return false;
+            expected *= shape[i];
+        }
+        return true;
+    }
+    void view(const Shape& ns) {                                      // layout.rs:76-97
+        if (size() != shape_size(ns))
+            throw Error(ErrKind::IncompatibleShape, "Cannot reshape layout of size " + std::to_string(size()) + " to size " +
+                                                        std::to_string(shape_size(ns)));
+        if (!is_contiguous())
+            throw Error(ErrKind::InvalidOperation, "Cannot view a non-contiguous tensor. Use .contiguous() before .view()");
+        shape = ns;
+        strides = compute_strides(ns);
+    }
+    void transpose(size_t d0, size_t d1) {                            // layout.rs:99-113
+        if (d0 >= ndim() || d1 >= ndim()) throw Error(ErrKind::DimensionOutOfBounds, "transpose: dimension out of bounds");
+        std::swap(shape[d0], shape[d1]);
+        std::swap(strides[d0], strides[d1]);
+    }
+    Layout broadcast_to(const Shape& target) const {                  // layout.rs:252-296
+        if (shape.size() > target.size())
+            throw Error(ErrKind::InvalidArgument, "Cannot broadcast tensor of rank " + std::to_string(shape.size()) + " to rank " +
+                                                      std::to_string(target.size()));
+        size_t diff = target.size() - shape.size();
+        Layout r{target, Shape(target.size(), 0), offset};
+        for (size_t i = 0; i < target.size(); ++i) {
+            size_t src = i < diff ? 1 : shape[i - diff];
+            if (src == target[i]) r.strides[i] = i < diff ? 0 : strides[i - diff];
+            else if (src == 1) r.strides[i] = 0;
+            else throw Error(ErrKind::InvalidShape, "Cannot broadcast shape " + shape_str(shape) + " to shape " + shape_str(target) +
+                                                        " at dimension " + std::to_string(i));
+        }
+        return r;
+    }
+};
+
+enum class DType { F32, BOOL };
+inline size_t dtype_size(DType d) { return d == DType::F32 ? 4 : 1; }
+
+// ---- buffers: pooled backend memory ------------------------------------------------------------------
+// All kernels of a backend run in call order on one stream, so a block handed back to the pool can be
+// given to the next tensor at once: whatever still reads it was queued earlier.
+template <class B>
+struct Pool {
+    std::map<size_t, std::vector<void*>> free_blocks;
+    size_t cached = 0, live = 0, device_allocs = 0;
+    static constexpr size_t kMaxCached = size_t(64) << 30;
+    static size_t bucket(size_t bytes) {
+        if (bytes <= 256) return 256;
+        if (bytes <= (size_t(1) << 20)) { size_t b = 256; while (b < bytes) b <<= 1; return b; }
+        const size_t g = size_t(2) << 20;
+        return (bytes + g - 1) / g * g;
+    }
+    void* get(size_t bytes, size_t& cap) {
+        cap = bucket(bytes);
+        auto it = free_blocks.find(cap);
+        if (it != free_blocks.end() && !it->second.empty()) {
+            void* p = it->second.back();
+            it->second.pop_back();
+            cached -= cap;
+            live += cap;
+            return p;
+        }
+        void* p = B::alloc(cap);
+        if (!p) {                       // give cached blocks back and try once more
+            trim();
+            p = B::alloc(cap);
+            if (!p) throw Error(ErrKind::OutOfMemory, "out of memory");
+        }
+        ++device_allocs;
+        live += cap;
+        return p;
+    }
+    void put(void* p, size_t cap) {
+        live -= cap;
+        if (cached + cap > kMaxCached) { B::sync(); B::free(p); return; }
+        free_blocks[cap].push_back(p);
+        cached += cap;
+    }
+    void trim() {
+        B::sync();
+        for (auto& kv : free_blocks)
+            for (void* p : kv.second) B::free(p);
+        free_blocks.clear();
+        cached = 0;
+    }
+    static Pool& instance() { static Pool* p = new Pool(); return *p; }   // never destroyed: outlives every tensor
+};
+
+template <class B>
+struct Storage {
+    void* ptr = nullptr;
+    size_t cap = 0, len = 0;        // len in elements
+    explicit Storage(size_t elems, DType dt) : len(elems) { ptr = Pool<B>::instance().get(std::max<size_t>(1, elems) * dtype_size(dt), cap); }
+    ~Storage() { Pool<B>::instance().put(ptr, cap); }
+    Storage(const Storage&) = delete;
+    Storage& operator=(const Storage&) = delete;
+};
+
+template <class B> struct Node;
+template <class B> struct Tensor;
+template <class B> struct GradCell { std::shared_ptr<Tensor<B>> g; };
+
+// Count of backend kernel calls (what `be::*` would dispatch), for reporting.
+inline size_t& backend_calls() { static size_t n = 0; return n; }
+
+// ---- Tensor (crates/maidenx_tensor/src/lib.rs:21-58): shared data, own metadata, optional node ------
+template <class B>
+struct Tensor {
+    std::shared_ptr<Storage<B>> buf;
+    std::shared_ptr<GradCell<B>> grad_cell;      // shared by clones, like Arc<Mutex<Tensor>>
+    Layout layout;
+    DType dtype = DType::F32;
+    bool requires_grad = false;
+    std::shared_ptr<Node<B>> node;
+
+    using T = Tensor<B>;
+    using BackwardFn = std::function<std::vector<T>(const std::vector<T>&, const T&)>;
+
+    // -- accessors --
+    const Shape& shape() const { return layout.shape; }
+    const Shape& strides() const { return layout.strides; }
+    size_t offset() const { return layout.offset; }
+    size_t size() const { return layout.size(); }
+    size_t ndim() const { return layout.ndim(); }
+    bool is_contiguous() const { return layout.is_contiguous(); }
+    const float* f32() const { return (const float*)buf->ptr; }
+    float* f32() { return (float*)buf->ptr; }
+
+    // -- creation (creation.rs) --
+    static T empty(const Shape& shape, DType dt = DType::F32) {                     // creation.rs:115-131
+        T t;
+        t.layout = Layout::from_shape(shape);
+        t.dtype = dt;
+        t.buf = std::make_shared<Storage<B>>(t.layout.size(), dt);
+        return t;
+    }
+    static T fill(const Shape& shape, float v) {                                    // creation.rs:253-305
+        T t = empty(shape);
+        B::fill_f32(t.size(), t.f32(), v);
+        return t;
+    }
+    static T zeros(const Shape& shape) { return fill(shape, 0.0f); }                // creation.rs:144-176
+    static T ones(const Shape& shape) { return fill(shape, 1.0f); }
+    static T zeros_like(const T& s) { return zeros(s.shape()); }
+    static T ones_like(const T& s) { return ones(s.shape()); }
+    static T from_host(const float* data, const Shape& shape) {                     // creation.rs:25-84
+        T t = empty(shape);
+        if (t.size()) B::h2d(t.buf->ptr, data, t.size() * sizeof(float));
+        return t;
+    }
+    static T share_buffer(const T& s) {                                             // creation.rs:86-102
+        T t;
+        t.buf = s.buf;
+        t.layout = s.layout;
+        t.dtype = s.dtype;
+        return t;
+    }
+
+    // -- reading back --
+    std::vector<float> to_vec() const {                                            // logical order
+        T c = contiguous();
+        std::vector<float> out(c.size());
+        if (c.dtype == DType::F32) {
+            if (c.size()) B::d2h(out.data(), (const char*)c.buf->ptr + c.offset() * 4, c.size() * 4);
+        } else {
+            std::vector<uint8_t> raw(c.size());
+            if (c.size()) B::d2h(raw.data(), (const char*)c.buf->ptr + c.offset(), c.size());
+            for (size_t i = 0; i < raw.size(); ++i) out[i] = raw[i] ? 1.0f : 0.0f;
+        }
+        return out;
+    }
+    float item() const {                                                            // buffer/mod.rs:596-614
+        if (size() != 1) throw Error(ErrKind::InvalidShape, "item() needs a tensor with one element");
+        float v;
+        B::d2h(&v, (const char*)buf->ptr + offset() * 4, 4);
+        return v;
+    }
+
+    // -- grad plumbing (wt.rs:92-104, lib.rs:213-285) --
+    void with_grad() {
+        if (dtype != DType::F32) throw Error(ErrKind::UnsupportedDType, "with_grad needs a float tensor");
+        requires_grad = true;
+        if (!grad_cell) {
+            grad_cell = std::make_shared<GradCell<B>>();
+            grad_cell->g = std::make_shared<T>(zeros_like(*this));
+        }
+    }
+    bool has_grad() const { return grad_cell && grad_cell->g; }
+    T grad() const {
+        if (!has_grad()) throw Error(ErrKind::InvalidOperation, "tensor has no grad");
+        return *grad_cell->g;
+    }
+    void accumulate_grad(const T& g) const {                                        // lib.rs:221-241
+        if (has_grad()) grad_cell->g->add_(g);
+    }
+    T detach() const {                                                              // f.rs:67-73
+        T r = *this;
+        r.requires_grad = false;
+        r.node.reset();
+        return r;
+    }
+    void zero_grad() const {                                                        // lib.rs:243-285
+        std::unordered_set<const void*> visited;
+        zero_grad_impl(visited);
+    }
+    void zero_grad_impl(std::unordered_set<const void*>& visited) const {
+        if (!visited.insert(buf.get()).second) return;
+        if (has_grad()) *grad_cell->g = zeros_like(*grad_cell->g);
+        if (node)
+            for (const T& in : node->inputs)
+                if (in.requires_grad) in.zero_grad_impl(visited);
+    }
+    void backward() const {                                                         // lib.rs:293-301
+        if (!requires_grad) return;
+        T go = ones_like(*this);
+        std::unordered_set<const void*> visited;
+        backward_tracking(go, visited);
+    }
+    // The walk keys "visited" on the buffer, so views of one buffer count as one tensor (lib.rs:308-323).
+    void backward_tracking(const T& go, std::unordered_set<const void*>& visited) const {
+        if (!visited.insert(buf.get()).second) return;
+        if (!node || !node->backward) return;
+        std::vector<T> grads = node->backward(node->inputs, go);                    // lib.rs:93-111
+        for (size_t i = 0; i < node->inputs.size(); ++i) {
+            const T& in = node->inputs[i];
+            if (in.requires_grad && i < grads.size()) {
+                in.accumulate_grad(grads[i]);
+                in.backward_tracking(grads[i], visited);
+            }
+        }
+    }
+    void set_node(const char* op, std::vector<T> inputs, BackwardFn fn) {
+        node = std::make_shared<Node<B>>();
+        node->op = op;
+        node->inputs = std::move(inputs);
+        node->backward = std::move(fn);
+    }
+
+    // -- metadata builders --
+    static std::vector<size_t> meta_binary(const T& l, const T& r) {                // ops/binary.rs:754-769
+        std::vector<size_t> m(l.shape());
+        m.insert(m.end(), l.strides().begin(), l.strides().end());
+        m.insert(m.end(), r.strides().begin(), r.strides().end());
+        m.push_back(l.offset());
+        m.push_back(r.offset());
+        return m;
+    }
+    static std::vector<size_t> meta_unary(const T& t) {                             // ops/unary.rs:1309-1320
+        std::vector<size_t> m(t.shape());
+        m.insert(m.end(), t.strides().begin(), t.strides().end());
+        m.push_back(t.offset());
+        return m;
+    }
+    static std::vector<size_t> meta_reduce(const T& t, size_t dim) {                // ops/reduction.rs:722-732
+        std::vector<size_t> m(t.shape());
+        m.insert(m.end(), t.strides().begin(), t.strides().end());
+        m.push_back(t.shape()[dim]);
+        m.push_back(t.strides()[dim]);
+        m.push_back(t.offset());
+        return m;
+    }
+    static std::vector<size_t> meta_to_shape(const T& t, const Shape& target) {     // ops/reduction.rs:734-743
+        std::vector<size_t> m(t.shape());
+        m.insert(m.end(), t.strides().begin(), t.strides().end());
+        m.insert(m.end(), target.begin(), target.end());
+        m.push_back(t.offset());
+        return m;
+    }
+
+    void need_f32(const char* what) const {
+        if (dtype != DType::F32) throw Error(ErrKind::UnsupportedDType, std::string(what) + ": only f32 tensors are supported");
+    }
+
+    // -- binary ops (ops/binary.rs:11-215) --
+    using BinFn = void (*)(size_t, size_t, const size_t*, const float*, const float*, float*);
+    static std::pair<T, T> broadcast_tensors(const T& a, const T& b) {              // utils/broadcast.rs:4-31
+        size_t an = a.ndim(), bn = b.ndim(), on = std::max(an, bn);
+        Shape out(on);
+        for (size_t i = 0; i < on; ++i) {
+            size_t ad = i < an ? a.shape()[an - 1 - i] : 1, bd = i < bn ? b.shape()[bn - 1 - i] : 1;
+            if (ad == 1 || bd == 1 || ad == bd) out[on - 1 - i] = std::max(ad, bd);
+            else throw Error(ErrKind::InvalidShape, "Cannot broadcast shapes " + shape_str(a.shape()) + " and " + shape_str(b.shape()));
+        }
+        return {a.broadcast(out), b.broadcast(out)};
+    }
+    T binary_forward(const T& rhs_in, BinFn fn, T& lhs_b, T& rhs_b) const {
+        need_f32("binary op");
+        rhs_in.need_f32("binary op");
+        auto pr = broadcast_tensors(*this, rhs_in);
+        lhs_b = pr.first;
+        rhs_b = pr.second;
+        T result = empty(lhs_b.shape());
+        auto md = meta_binary(lhs_b, rhs_b);
+        fn(lhs_b.size(), lhs_b.ndim(), md.data(), lhs_b.f32(), rhs_b.f32(), result.f32());
+        ++backend_calls();
+        B::check();
+        return result;
+    }
+    T add(const T& rhs) const {                                                     // ops/binary.rs:11-60
+        T l, r;
+        T result = binary_forward(rhs, B::add, l, r);
+        if (requires_grad || r.requires_grad) {
+            result.with_grad();
+            Shape ls = shape(), rs = rhs.shape();
+            result.set_node("add", {*this, rhs}, [ls, rs](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.sum_to_shape(ls), go.sum_to_shape(rs)};
+            });
+        }
+        return result;
+    }
+    T sub(const T& rhs) const {                                                     // ops/binary.rs:62-111
+        T l, r;
+        T result = binary_forward(rhs, B::sub, l, r);
+        if (requires_grad || r.requires_grad) {
+            result.with_grad();
+            Shape ls = shape(), rs = rhs.shape();
+            result.set_node("sub", {*this, rhs}, [ls, rs](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.sum_to_shape(ls), go.neg().sum_to_shape(rs)};
+            });
+        }
+        return result;
+    }
+    T mul(const T& rhs) const {                                                     // ops/binary.rs:113-164
+        T l, r;
+        T result = binary_forward(rhs, B::mul, l, r);
+        if (requires_grad || r.requires_grad) {
+            result.with_grad();
+            Shape ls = shape(), rs = rhs.shape();
+            result.set_node("mul", {*this, rhs}, [ls, rs, l, r](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.mul(r).sum_to_shape(ls), go.mul(l).sum_to_shape(rs)};
+            });
+        }
+        return result;
+    }
+    T div(const T& rhs) const {                                                     // ops/binary.rs:166-222
+        T l, r;
+        T result = binary_forward(rhs, B::div, l, r);
+        if (requires_grad || r.requires_grad) {
+            result.with_grad();
+            Shape ls = shape(), rs = rhs.shape();
+            result.set_node("div", {*this, rhs}, [ls, rs, l, r](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.div(r).sum_to_shape(ls), go.mul(l).div(r.square()).neg().sum_to_shape(rs)};
+            });
+        }
+        return result;
+    }
+    using InplaceFn = void (*)(size_t, size_t, const size_t*, float*, const float*);
+    void inplace(const T& rhs_in, InplaceFn fn) {                                   // ops/binary.rs:653-700
+        need_f32("in-place op");
+        T rhs = shape() == rhs_in.shape() ? rhs_in : rhs_in.broadcast(shape());
+        auto md = meta_binary(*this, rhs);
+        fn(size(), ndim(), md.data(), f32(), rhs.f32());
+        ++backend_calls();
+        B::check();
+    }
+    void add_(const T& rhs) { inplace(rhs, B::add_inplace); }
+    void sub_(const T& rhs) { inplace(rhs, B::sub_inplace); }
+
+    // -- unary ops (ops/unary.rs) --
+    using UnFn = void (*)(size_t, size_t, const size_t*, const float*, float*);
+    using UnCFn = void (*)(size_t, size_t, const size_t*, const float*, float, float*);
+    T unary_forward(UnFn fn) const {
+        need_f32("unary op");
+        T result = empty(shape());
+        auto md = meta_unary(*this);
+        fn(size(), ndim(), md.data(), f32(), result.f32());
+        ++backend_calls();
+        B::check();
+        return result;
+    }
+    T unary_c_forward(UnCFn fn, float c) const {
+        need_f32("unary op");
+        T result = empty(shape());
+        auto md = meta_unary(*this);
+        fn(size(), ndim(), md.data(), f32(), c, result.f32());
+        ++backend_calls();
+        B::check();
+        return result;
+    }
+    T neg() const {                                                                 // ops/unary.rs:8-43
+        T result = unary_forward(B::neg);
+        if (requires_grad) {
+            result.with_grad();
+            result.set_node("neg", {*this}, [](const std::vector<T>&, const T& go) { return std::vector<T>{go.neg()}; });
+        }
+        return result;
+    }
+    T square() const {                                                              // ops/unary.rs:112-147
+        T result = unary_forward(B::square);
+        if (requires_grad) {
+            result.with_grad();
+            T input = *this;
+            result.set_node("square", {*this}, [input](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.mul_scalar(2.0f).mul(input)};
+            });
+        }
+        return result;
+    }
+    T relu() const {                                                                // ops/unary.rs:186-222
+        T result = unary_forward(B::relu);
+        if (requires_grad) {
+            result.with_grad();
+            T input = *this;
+            result.set_node("relu", {*this}, [input](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.mul(input.gt_scalar(0.0f).to_f32())};
+            });
+        }
+        return result;
+    }
+    T tanh() const {                                                                // ops/unary.rs:261-296
+        T result = unary_forward(B::tanh);
+        if (requires_grad) {
+            result.with_grad();
+            T output = result;
+            result.set_node("tanh", {*this}, [output](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.mul(output.pow(2.0f).neg().add_scalar(1.0f))};
+            });
+        }
+        return result;
+    }
+    T gelu() const {                                                                // ops/unary.rs:298-351
+        T result = unary_forward(B::gelu);
+        if (requires_grad) {
+            result.with_grad();
+            T input = *this;
+            result.set_node("gelu", {*this}, [input](const std::vector<T>&, const T& go) {
+                const float c0 = 0.7978845608028654f, coeff = 0.044715f;
+                T x2 = input.mul(input);
+                T x3 = x2.mul(input);
+                T tanh_arg = input.add(x3.mul_scalar(coeff)).mul_scalar(c0);
+                T tanh_val = tanh_arg.tanh();
+                T sech2 = tanh_val.mul(tanh_val).mul_scalar(-1.0f).add_scalar(1.0f);
+                T inner = x2.mul_scalar(3.0f * coeff).add_scalar(1.0f).mul_scalar(c0);
+                T term1 = tanh_val.add_scalar(1.0f).mul_scalar(0.5f);
+                T term2 = input.mul(sech2).mul(inner).mul_scalar(0.5f);
+                return std::vector<T>{go.mul(term1.add(term2))};
+            });
+        }
+        return result;
+    }
+    T exp() const {                                                                 // ops/unary.rs:583-618
+        T result = unary_forward(B::exp);
+        if (requires_grad) {
+            result.with_grad();
+            T output = result;
+            result.set_node("exp", {*this}, [output](const std::vector<T>&, const T& go) { return std::vector<T>{go.mul(output)}; });
+        }
+        return result;
+    }
+    T add_scalar(float c) const {                                                   // ops/unary.rs:794-830
+        T result = unary_c_forward(B::add_scalar, c);
+        if (requires_grad) {
+            result.with_grad();
+            result.set_node("add_scalar", {*this}, [](const std::vector<T>&, const T& go) { return std::vector<T>{go}; });
+        }
+        return result;
+    }
+    T mul_scalar(float c) const {                                                   // ops/unary.rs:870-907
+        T result = unary_c_forward(B::mul_scalar, c);
+        if (requires_grad) {
+            result.with_grad();
+            result.set_node("mul_scalar", {*this}, [c](const std::vector<T>&, const T& go) { return std::vector<T>{go.mul_scalar(c)}; });
+        }
+        return result;
+    }
+    T div_scalar(float c) const {                                                   // ops/unary.rs:909-946
+        T result = unary_c_forward(B::div_scalar, c);
+        if (requires_grad) {
+            result.with_grad();
+            result.set_node("div_scalar", {*this}, [c](const std::vector<T>&, const T& go) { return std::vector<T>{go.div_scalar(c)}; });
+        }
+        return result;
+    }
+    T pow(float e) const {                                                          // ops/unary.rs:1042-1082
+        T result = unary_c_forward(B::pow, e);
+        if (requires_grad) {
+            result.with_grad();
+            T input = *this;
+            result.set_node("pow", {*this}, [input, e](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.mul_scalar(e).mul(input.pow(e - 1.0f))};
+            });
+        }
+        return result;
+    }
+    T gt_scalar(float c) const {                                                    // ops/unary.rs:1264-1284 (bool result, no grad)
+        need_f32("gt_scalar");
+        T result = empty(shape(), DType::BOOL);
+        auto md = meta_unary(*this);
+        B::gt_scalar(size(), ndim(), md.data(), f32(), c, (uint8_t*)result.buf->ptr);
+        ++backend_calls();
+        B::check();
+        return result;
+    }
+    T to_f32() const {                                                              // wt.rs:65-90 (bool -> f32 keeps the layout)
+        if (dtype == DType::F32) return *this;
+        T r;
+        r.layout = layout;
+        r.dtype = DType::F32;
+        r.buf = std::make_shared<Storage<B>>(buf->len, DType::F32);
+        B::cast_bool_f32(buf->len, (const uint8_t*)buf->ptr, r.f32());
+        return r;
+    }
+
+    // -- reductions (ops/reduction.rs) --
+    using RedFn = void (*)(size_t, size_t, size_t, const size_t*, const float*, float*);
+    size_t norm_dim(int dim, size_t nd, bool allow_end = false) const {
+        long d = dim < 0 ? (long)nd + dim : dim;
+        if (d < 0 || (size_t)d >= nd + (allow_end ? 1 : 0))
+            throw Error(ErrKind::DimensionOutOfBounds, "dimension " + std::to_string(dim) + " out of bounds for " + std::to_string(nd) + " dims");
+        return (size_t)d;
+    }
+    T reduce_forward(RedFn fn, size_t dim, bool keep_dim) const {
+        need_f32("reduction");
+        Shape out = shape();
+        out.erase(out.begin() + dim);
+        T result = zeros(out);                                   // the reference zero-fills reduction outputs
+        auto md = meta_reduce(*this, dim);
+        fn(size(), ndim(), 1, md.data(), f32(), result.f32());
+        ++backend_calls();
+        B::check();
+        if (keep_dim) {
+            Shape ks = shape();
+            ks[dim] = 1;
+            result = result.view(ks);
+        }
+        return result;
+    }
+    T sum(int dim_in, bool keep_dim) const {                                        // ops/reduction.rs:9-74
+        size_t dim = norm_dim(dim_in, ndim());
+        T result = reduce_forward(B::sum, dim, keep_dim);
+        if (requires_grad) {
+            result.with_grad();
+            Shape in_shape = shape();
+            result.set_node("sum", {*this}, [in_shape, dim, keep_dim](const std::vector<T>&, const T& go) {
+                if (keep_dim) return std::vector<T>{go.broadcast(in_shape)};
+                Shape gs = in_shape;
+                gs[dim] = 1;
+                return std::vector<T>{go.reshape(gs).broadcast(in_shape)};
+            });
+        }
+        return result;
+    }
+    T sum_all() const {                                                             // ops/reduction.rs:76-83
+        T result = *this;
+        for (size_t d = ndim(); d-- > 0;) result = result.sum((int)d, false);
+        return result;
+    }
+    T sum_to_shape(const Shape& target) const {                                     // ops/reduction.rs:85-143
+        if (target.size() != ndim()) {
+            if (ndim() > target.size()) {
+                T result = *this;
+                while (result.ndim() > target.size()) result = result.sum(0, false);
+                return result.sum_to_shape(target);
+            }
+            throw Error(ErrKind::ShapeMismatch, "Target shape has more dimensions than input");
+        }
+        for (size_t i = 0; i < target.size(); ++i)
+            if (target[i] == 0 || shape()[i] % target[i] != 0)
+                throw Error(ErrKind::ShapeMismatch, "Dimension " + std::to_string(i) + " is not divisible: " + std::to_string(shape()[i]) +
+                                                        " -> " + std::to_string(target[i]));
+        need_f32("sum_to_shape");
+        T result = zeros(target);
+        auto md = meta_to_shape(*this, target);
+        B::sum_to_shape(size(), ndim(), md.data(), f32(), result.f32());
+        ++backend_calls();
+        B::check();
+        if (requires_grad) {
+            result.with_grad();
+            Shape in_shape = shape();
+            result.set_node("sum_to_shape", {*this}, [in_shape](const std::vector<T>&, const T& go) { return std::vector<T>{go.broadcast(in_shape)}; });
+        }
+        return result;
+    }
+    T mean(int dim_in, bool keep_dim) const {                                       // ops/reduction.rs:145-216
+        size_t dim = norm_dim(dim_in, ndim());
+        T result = reduce_forward(B::mean, dim, keep_dim);
+        if (requires_grad) {
+            result.with_grad();
+            Shape in_shape = shape();
+            size_t dim_size = shape()[dim];
+            result.set_node("sum", {*this}, [in_shape, dim, keep_dim, dim_size](const std::vector<T>&, const T& go_in) {
+                T go = go_in;
+                if (!keep_dim) {
+                    Shape gs = in_shape;
+                    gs[dim] = 1;
+                    go = go.view(gs);
+                }
+                return std::vector<T>{go.broadcast(in_shape).div_scalar((float)dim_size)};
+            });
+        }
+        return result;
+    }
+    T mean_all() const {                                                            // ops/reduction.rs:218-225
+        T result = *this;
+        for (size_t d = ndim(); d-- > 0;) result = result.mean((int)d, false);
+        return result;
+    }
+
+    // -- views and layout ops (ops/transform.rs) --
+    T view_like(const char* op, const Shape& ns) const {
+        T result = share_buffer(*this);
+        result.layout.view(ns);
+        if (requires_grad) {
+            result.with_grad();
+            Shape orig = shape();
+            result.set_node(op, {*this}, [orig](const std::vector<T>&, const T& go) { return std::vector<T>{go.reshape(orig)}; });
+        }
+        return result;
+    }
+    Shape shape_with_auto(const std::vector<long>& req) const {                     // ops/transform.rs:381-440
+        long product = 1;
+        int auto_idx = -1;
+        for (size_t i = 0; i < req.size(); ++i) {
+            if (req[i] == -1) {
+                if (auto_idx >= 0) throw Error(ErrKind::InvalidShape, "Only one dimension can be -1");
+                auto_idx = (int)i;
+            } else if (req[i] <= 0) {
+                throw Error(ErrKind::InvalidShape, "Invalid dimension size: " + std::to_string(req[i]));
+            } else {
+                product *= req[i];
+            }
+        }
+        Shape out(req.size());
+        long total = (long)size();
+        if (auto_idx >= 0) {
+            if (product == 0) throw Error(ErrKind::InvalidShape, "Cannot infer size for dimension -1");
+            long a = total / product;
+            if (a * product != total) throw Error(ErrKind::InvalidShape, "Cannot reshape tensor: incompatible dimensions");
+            for (size_t i = 0; i < req.size(); ++i) out[i] = (size_t)((int)i == auto_idx ? a : req[i]);
+        } else {
+            if (product != total) throw Error(ErrKind::InvalidShape, "Total size of new shape must be equal to old size");
+            for (size_t i = 0; i < req.size(); ++i) out[i] = (size_t)req[i];
+        }
+        return out;
+    }
+    static std::vector<long> as_long(const Shape& s) { return std::vector<long>(s.begin(), s.end()); }
+    T view(const Shape& ns) const { return view_like("view", shape_with_auto(as_long(ns))); }   // ops/transform.rs:10-28
+    T view(const std::vector<long>& ns) const { return view_like("view", shape_with_auto(ns)); }
+    T squeeze(int dim_in) const {                                                   // ops/transform.rs:30-71
+        size_t dim = norm_dim(dim_in, ndim());
+        if (shape()[dim] != 1) return *this;
+        Shape ns = shape();
+        ns.erase(ns.begin() + dim);
+        if (ns.empty()) ns.push_back(1);          // a squeezed [1] stays [1] (transform.rs:50-52)
+        return view_like("squeeze", ns);
+    }
+    T squeeze_all() const {                                                         // ops/transform.rs:73-92
+        Shape ns;
+        for (size_t d : shape())
+            if (d != 1) ns.push_back(d);
+        return view_like("squeeze_all", ns);
+    }
+    T unsqueeze(int dim_in) const {                                                 // ops/transform.rs:94-128
+        size_t dim = norm_dim(dim_in, ndim(), true);
+        Shape ns = shape();
+        ns.insert(ns.begin() + dim, 1);
+        return view_like("unsqueeze", ns);
+    }
+    T transpose(int d0_in, int d1_in) const {                                       // ops/transform.rs:132-162
+        long d0 = d0_in < 0 ? (long)ndim() + d0_in : d0_in, d1 = d1_in < 0 ? (long)ndim() + d1_in : d1_in;
+        if (d0 < 0 || d1 < 0) throw Error(ErrKind::DimensionOutOfBounds, "transpose: dimension out of bounds");
+        T result = share_buffer(*this);
+        result.layout.transpose((size_t)d0, (size_t)d1);
+        if (requires_grad) {
+            result.with_grad();
+            result.set_node("transpose", {*this}, [d0, d1](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.transpose((int)d0, (int)d1)};
+            });
+        }
+        return result;
+    }
+    T broadcast(const Shape& target) const {                                        // ops/transform.rs:278-316
+        if (shape() == target) return *this;
+        if (shape().empty()) return broadcast_scalar_to(target);
+        if (target.empty()) throw Error(ErrKind::InvalidShape, "Cannot broadcast non-scalar shape " + shape_str(shape()) + " to scalar ()");
+        T result = share_buffer(*this);
+        result.layout = layout.broadcast_to(target);
+        if (requires_grad) {
+            result.with_grad();
+            Shape orig = shape();
+            result.set_node("broadcast", {*this}, [orig](const std::vector<T>&, const T& go) { return std::vector<T>{go.sum_to_shape(orig)}; });
+        }
+        return result;
+    }
+    T broadcast_left(const Shape& batch) const {                                    // ops/transform.rs:322-326
+        Shape ns = batch;
+        ns.insert(ns.end(), shape().begin(), shape().end());
+        return broadcast(ns);
+    }
+    T broadcast_scalar_to(const Shape& target) const {                              // ops/transform.rs:328-349
+        need_f32("broadcast");
+        T result = empty(target);
+        B::broadcast_scalar_f32(result.size(), f32() + offset(), result.f32());     // the reference: item() + host fill
+        if (requires_grad) {
+            result.with_grad();
+            result.set_node("broadcast_scalar", {*this}, [](const std::vector<T>&, const T& go) { return std::vector<T>{go.sum_all()}; });
+        }
+        return result;
+    }
+    T contiguous() const {                                                          // f.rs:11-41
+        if (is_contiguous()) return *this;
+        T result = empty(shape(), dtype);
+        if (dtype == DType::F32) {
+            auto md = meta_unary(*this);
+            B::copy_strided_f32(size(), ndim(), md.data(), f32(), result.f32());
+        } else {
+            // bool tensors only come out of comparisons and are contiguous there
+            throw Error(ErrKind::UnsupportedDType, "contiguous() of a strided bool tensor");
+        }
+        return result;
+    }
+    T reshape(const std::vector<long>& req) const {                                 // ops/transform.rs:353-388
+        Shape ns = shape_with_auto(req);
+        if (is_contiguous()) return view_like("reshape", ns);
+        T result = contiguous();
+        result.layout.view(ns);
+        if (requires_grad) {           // node without with_grad, as the reference has it: gradients stop here
+            Shape orig = shape();
+            result.set_node("reshape", {*this}, [orig](const std::vector<T>&, const T& go) { return std::vector<T>{go.reshape(orig)}; });
+        }
+        return result;
+    }
+    T reshape(const Shape& ns) const { return reshape(as_long(ns)); }
+
+    // -- matmul (ops/matmul.rs:11-157) --
+    static std::pair<std::vector<size_t>, Shape> meta_matmul(const T& a, const T& b) {   // ops/matmul.rs:227-264
+        Shape as = a.shape(), bs = b.shape(), ast = a.strides(), bst = b.strides();
+        if (as.size() == 1) {
+            as.insert(as.begin(), 1);
+            ast.insert(ast.begin(), ast[0] * as[1]);
+        }
+        if (bs.size() == 1) {
+            bs.push_back(1);
+            bst.push_back(1);
+        }
+        size_t on = as.size();
+        Shape out(as.begin(), as.end() - 2);
+        out.push_back(as[on - 2]);
+        out.push_back(bs[on - 1]);
+        std::vector<size_t> m{on, as.size(), bs.size()};
+        m.insert(m.end(), out.begin(), out.end());
+        m.insert(m.end(), as.begin(), as.end());
+        m.insert(m.end(), bs.begin(), bs.end());
+        m.insert(m.end(), ast.begin(), ast.end());
+        m.insert(m.end(), bst.begin(), bst.end());
+        m.push_back(a.offset());
+        m.push_back(b.offset());
+        return {m, out};
+    }
+    static std::pair<T, T> unify_matmul_shapes(const T& a, const T& b) {            // ops/matmul.rs:161-194
+        T ae = a.ndim() == 1 ? a.unsqueeze(0) : a;
+        T be = b.ndim() == 1 ? b.unsqueeze((int)b.ndim()) : b;
+        size_t an = ae.ndim(), bn = be.ndim();
+        if (an < 2 || bn < 2) throw Error(ErrKind::InvalidShape, "matmul: both inputs must have at least 2D after expand");
+        size_t M = ae.shape()[an - 2], Ka = ae.shape()[an - 1], Kb = be.shape()[bn - 2], N = be.shape()[bn - 1];
+        if (Ka != Kb) throw Error(ErrKind::InvalidShape, "Incompatible shapes for matmul (K mismatch): " + std::to_string(Ka) + " vs " + std::to_string(Kb));
+        size_t al = an - 2, bl = bn - 2, ml = std::max(al, bl);
+        Shape lead(ml);
+        for (size_t i = 0; i < ml; ++i) {                                            // ops/matmul.rs:196-218
+            size_t ad = i < al ? ae.shape()[al - 1 - i] : 1, bd = i < bl ? be.shape()[bl - 1 - i] : 1;
+            if (ad != bd && ad != 1 && bd != 1)
+                throw Error(ErrKind::InvalidShape, "Cannot broadcast leading dims: mismatch " + std::to_string(ad) + " vs " + std::to_string(bd));
+            lead[ml - 1 - i] = std::max(ad, bd);
+        }
+        Shape as = lead, bs = lead;
+        as.push_back(M); as.push_back(Ka);
+        bs.push_back(Kb); bs.push_back(N);
+        return {ae.broadcast(as), be.broadcast(bs)};
+    }
+    T matmul(const T& rhs_in) const {
+        need_f32("matmul");
+        rhs_in.need_f32("matmul");
+        size_t ln = ndim(), rn = rhs_in.ndim();
+        auto pr = unify_matmul_shapes(*this, rhs_in);
+        const T &lhs = pr.first, &rhs = pr.second;
+        auto mm = meta_matmul(lhs, rhs);
+        T result = empty(mm.second);
+        B::matmul(result.size(), mm.first.data(), lhs.f32(), rhs.f32(), result.f32());
+        ++backend_calls();
+        B::check();
+        if (ln == 1 && rn == 1) result = result.squeeze_all();
+        else if (ln == 1 && rn >= 2) { int d = (int)result.ndim() - 2; if (result.shape()[d] == 1) result = result.squeeze(d); }
+        else if (ln >= 2 && rn == 1) { int d = (int)result.ndim() - 1; if (result.shape()[d] == 1) result = result.squeeze(d); }
+        if (requires_grad || rhs.requires_grad) {
+            result.with_grad();
+            result.set_node("matmul", {*this, rhs_in}, [](const std::vector<T>& in, const T& go) {     // ops/matmul.rs:63-146
+                const T &l = in[0], &r = in[1];
+                auto mm = meta_matmul(l, r);
+                T gl = zeros_like(l), gr = zeros_like(r);
+                B::matmul_backward(gl.size(), gr.size(), mm.first.data(), go.f32(), l.f32(), r.f32(), gl.f32(), gr.f32());
+                ++backend_calls();
+                B::check();
+                return std::vector<T>{gl, gr};      // zeros_like already has the inputs' shapes: no reshape branch is reached
+            });
+        }
+        return result;
+    }
+};
+
+template <class B>
+struct Node {
+    std::string op;
+    std::vector<Tensor<B>> inputs;
+    typename Tensor<B>::BackwardFn backward;
+};
+
+// ---- seeded normal values (the reference's randn draws from an unseeded thread_rng, creation.rs:318-331) ----
+struct SplitMix64 {
+    uint64_t s;
+    explicit SplitMix64(uint64_t seed) : s(seed) {}
+    uint64_t next() {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    double uniform() { return ((next() >> 11) + 0.5) * (1.0 / 9007199254740992.0); }   // (0, 1)
+    float normal() {                                                                    // Box-Muller, one value per pair
+        double u1 = uniform(), u2 = uniform();
+        return (float)(std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586 * u2));
+    }
+};
+template <class B>
+Tensor<B> randn(const Shape& shape, uint64_t seed) {
+    SplitMix64 g(seed);
+    std::vector<float> v(shape_size(shape));
+    for (float& x : v) x = g.normal();
+    return Tensor<B>::from_host(v.data(), shape);
+}
+
+// ---- nn ---------------------------------------------------------------------------------------------
+template <class B>
+struct Linear {                                                                     // nn/layers/linear.rs:11-98
+    using T = Tensor<B>;
+    T weight;                 // [out_features, in_features]
+    bool has_bias = false;
+    T bias;                   // 0-d tensor, as the reference creates it (linear.rs:44)
+    // The reference scales neither tensor: the result of mul_scalar(k) is dropped (linear.rs:40,46).
+    Linear(size_t in_f, size_t out_f, bool with_bias, uint64_t seed) {
+        weight = randn<B>({out_f, in_f}, seed);
+        weight.with_grad();
+        if (with_bias) {
+            bias = randn<B>({}, seed + 1);
+            bias.with_grad();
+            has_bias = true;
+        }
+    }
+    Linear(const T& w, const T* b) : weight(w) {
+        weight.with_grad();
+        if (b) { bias = *b; bias.with_grad(); has_bias = true; }
+    }
+    T forward(const T& input) const {                                               // linear.rs:60-81
+        Shape batch;
+        if (input.ndim() >= 2) batch.assign(input.shape().begin(), input.shape().end() - 2);
+        T w = batch.empty() ? weight : weight.broadcast_left(batch);
+        T out = input.matmul(w.transpose(-1, -2));
+        return has_bias ? out.add(bias) : out;
+    }
+    std::vector<T*> parameters() {
+        std::vector<T*> p{&weight};
+        if (has_bias) p.push_back(&bias);
+        return p;
+    }
+};
+
+template <class B>
+struct Conv2d {                                                                     // nn/layers/conv.rs:100-322
+    using T = Tensor<B>;
+    T weight;                 // [Cout, Cin, kh, kw]
+    bool has_bias = false;
+    T bias;                   // [Cout]
+    size_t kh, kw, sh, sw, ph, pw;
+    Conv2d(const T& w, const T* b, size_t kh_, size_t kw_, size_t sh_, size_t sw_, size_t ph_, size_t pw_)
+        : weight(w), kh(kh_), kw(kw_), sh(sh_), sw(sw_), ph(ph_), pw(pw_) {
+        weight.with_grad();
+        if (b) { bias = *b; bias.with_grad(); has_bias = true; }
+    }
+    // The caller writes stride then padding into slots 8..11 (conv.rs:352-365); the kernel reads them as
+    // padding then stride (crates/maidenx_cpu/src/nn/conv.rs:31-34).  Kept as is.
+    static std::vector<size_t> conv_meta(size_t Bn, size_t C, size_t H, size_t W, size_t kh, size_t kw, size_t oh, size_t ow,
+                                         size_t sh, size_t sw, size_t ph, size_t pw) {
+        return {Bn, C, H, W, kh, kw, oh, ow, sh, sw, ph, pw};
+    }
+    T forward(const T& input) const {                                               // conv.rs:185-310
+        if (input.ndim() != 4) throw Error(ErrKind::InvalidShape, "Expected 4D input (batch_size, channels, height, width)");
+        input.need_f32("conv2d");
+        const size_t Bn = input.shape()[0], C = input.shape()[1], H = input.shape()[2], W = input.shape()[3];
+        const size_t oh = (H + 2 * ph - kh) / sh + 1, ow = (W + 2 * pw - kw) / sw + 1;
+        const size_t kh_ = kh, kw_ = kw, sh_ = sh, sw_ = sw, ph_ = ph, pw_ = pw;
+        // im2col (conv.rs:333-376); the input buffer is passed from its start, as the reference passes it
+        T cols = T::empty({Bn * oh * ow, C * kh * kw});
+        {
+            auto md = conv_meta(Bn, C, H, W, kh, kw, oh, ow, sh, sw, ph, pw);
+            B::im2col(cols.size(), md.data(), input.f32(), cols.f32());
+            ++backend_calls();
+            B::check();
+        }
+        const Shape& ws = weight.shape();
+        T wm = weight.reshape(Shape{ws[0], ws[1] * ws[2] * ws[3]});
+        T out = cols.matmul(wm.transpose(-1, -2));
+        out = out.reshape(std::vector<long>{(long)Bn, (long)oh, (long)ow, -1});
+        out = out.transpose(1, 3).transpose(2, 3);
+        if (has_bias) out = out.add(bias.reshape(Shape{1, bias.shape()[0], 1, 1}));
+        if (input.requires_grad) {
+            std::vector<T> inputs{input, weight};
+            if (has_bias) inputs.push_back(bias);
+            out.set_node("conv2d", inputs, [=](const std::vector<T>& in, const T& go) {              // conv.rs:236-306
+                const T &x = in[0], &w = in[1];
+                std::vector<T> grads;
+                auto flat_grad = [&]() {
+                    T gr = go.transpose(2, 3).transpose(1, 3);
+                    return gr.reshape(Shape{go.shape()[0] * oh * ow, go.shape()[1]});
+                };
+                if (x.requires_grad) {
+                    const Shape& ws = w.shape();
+                    T wm = w.reshape(Shape{ws[0], ws[1] * ws[2] * ws[3]});
+                    T grad_cols = flat_grad().matmul(wm);
+                    // col2im divides by what it reads as the stride, i.e. by the padding the caller stored in
+                    // slots 10, 11: with padding 0 the reference panics (division by zero)
+                    if (ph_ == 0 || pw_ == 0)
+                        throw Error(ErrKind::InvalidOperation, "col2im: division by zero (padding 0 is read as stride 0)");
+                    T gi = T::empty({Bn, C, H, W});                                                  // col2im, conv.rs:378-418
+                    auto md = conv_meta(Bn, C, H, W, kh_, kw_, oh, ow, sh_, sw_, ph_, pw_);
+                    B::col2im(gi.size(), md.data(), grad_cols.f32(), gi.f32());
+                    ++backend_calls();
+                    B::check();
+                    grads.push_back(gi);
+                } else {
+                    grads.push_back(T::zeros_like(x));
+                }
+                if (w.requires_grad) {
+                    T gw = cols.transpose(-1, -2).matmul(flat_grad());
+                    grads.push_back(gw.reshape(Shape{w.shape()[0], w.shape()[1], kh_, kw_}));
+                } else {
+                    grads.push_back(T::zeros_like(w));
+                }
+                if (in.size() > 2) {
+                    const T& b = in[2];
+                    if (b.requires_grad) grads.push_back(go.sum(3, false).sum(2, false).sum(0, false));
+                    else grads.push_back(T::zeros_like(b));
+                }
+                return grads;
+            });
+        }
+        return out;
+    }
+    std::vector<T*> parameters() {
+        std::vector<T*> p{&weight};
+        if (has_bias) p.push_back(&bias);
+        return p;
+    }
+};
+
+template <class B>
+Tensor<B> mse_loss(const Tensor<B>& pred, const Tensor<B>& target) {                // nn/losses/mse.rs:21-29
+    Tensor<B> squared = pred.sub(target).pow(2.0f);
+    return squared.sum_all().div_scalar((float)squared.size());
+}
+
+template <class B>
+struct SGD {                                                                        // nn/optimizers/sgd.rs:6-37
+    float lr;
+    explicit SGD(float lr_) : lr(lr_) {}
+    void step(const std::vector<Tensor<B>*>& params) const {
+        for (Tensor<B>* p : params)
+            if (p->has_grad()) p->sub_(p->grad().mul_scalar(lr));
+    }
+    void zero_grad(const std::vector<Tensor<B>*>& params) const {
+        for (Tensor<B>* p : params) p->zero_grad();
+    }
+};
+
+}  // namespace mxt

@@ -49,6 +49,7 @@ template <typename T>
 void col2im(size_t num_els, const size_t* md, const T* col, T* output) {
     if (!md || !col || !output) return;
     CV p = parse(md);
+    if (p.sh == 0 || p.sw == 0) return;      // the reference panics here (usize division by zero, conv.rs:121-124)
     size_t chunk = p.C * p.H * p.W;
     ORC_PAR_FOR
     for (size_t b = 0; b < p.B; ++b) {

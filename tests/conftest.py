@@ -26,3 +26,18 @@ def hip():
     if L.device_count() < 1:
         pytest.fail("no HIP device visible: GPU tests must run on the MI355X box")
     return Runner("hip")
+
+
+@pytest.fixture(scope="session")
+def mx_oracle():
+    from helpers import oracle_host
+    return oracle_host()
+
+
+@pytest.fixture(scope="session")
+def mx_hip():
+    import maidenx_amd.lib as L
+    from maidenx_amd.tensor import host
+    if L.device_count() < 1:
+        pytest.fail("no HIP device visible: GPU tests must run on the MI355X box")
+    return host()

@@ -130,10 +130,20 @@ class Null:
     pass
 
 
+ORACLE_HOST_LIB = os.path.join(ORACLE_DIR, "liboracle_host.so")
+
+
 def ensure_oracle_built():
-    if not os.path.exists(ORACLE_LIB):
-        subprocess.run(["make", "-C", ORACLE_DIR, "-j8"], check=True, capture_output=True)
+    if not os.path.exists(ORACLE_LIB) or not os.path.exists(ORACLE_HOST_LIB):
+        subprocess.run(["make", "-C", ORACLE_DIR, "-j8", "all"], check=True, capture_output=True)
     return ORACLE_LIB
+
+
+def oracle_host():
+    """The product's host layer (tensor / autograd / nn) instantiated over the CPU oracle."""
+    from maidenx_amd.tensor import Host
+    ensure_oracle_built()
+    return Host(ORACLE_HOST_LIB)
 
 
 class Runner:

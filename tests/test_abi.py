@@ -35,3 +35,27 @@ def test_python_binding_covers_the_header():
                "hip_stream_synchronize", "hip_set_stream", "hip_get_stream", "hip_synchronize", "hip_event_create",
                "hip_event_destroy", "hip_event_record", "hip_event_synchronize", "hip_event_elapsed_ms"}
     assert set(declared_symbols()) == bound | runtime
+
+
+def host_symbols():
+    out = subprocess.run(["gcc", "-E", "-P", os.path.join(ROOT, "include", "maidenx_host.h")], check=True, capture_output=True, text=True).stdout
+    return sorted(set(re.findall(r"\b(mxt_[a-z0-9_]+)\s*\(", out)))
+
+
+def test_host_header_is_valid_c_and_cxx():
+    hdr = os.path.join(ROOT, "include", "maidenx_host.h")
+    for comp, lang in (("gcc", "c"), ("g++", "c++")):
+        subprocess.run([comp, "-x", lang, "-fsyntax-only", "-Wall", "-Werror", hdr], check=True)
+
+
+def test_host_library_exports_every_declared_symbol():
+    # loads without a GPU (no HIP call happens at load time); the oracle-backed build exports the same ABI
+    from helpers import ORACLE_HOST_LIB, ensure_oracle_built
+    from maidenx_amd.tensor import HOST_LIB_PATH
+    ensure_oracle_built()
+    names = host_symbols()
+    assert len(names) >= 40
+    for path in (HOST_LIB_PATH, ORACLE_HOST_LIB):
+        lib = ctypes.CDLL(path)
+        missing = [n for n in names if not hasattr(lib, n)]
+        assert not missing, (path, missing)

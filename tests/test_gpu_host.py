@@ -1,0 +1,96 @@
+"""The host layer on the HIP backend (libmaidenx_host.so -> libmaidenx_hip.so) against the same programs on the
+CPU oracle and against the reference's own expectations."""
+import numpy as np
+import pytest
+
+from host_programs import TKAT, check_case, conv_inputs, conv_numpy, conv_step, mlp_numpy, mlp_run, run_case
+from maidenx_amd.tensor import MxError
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])
+def test_reference_tensor_cases(mx_hip, case):
+    check_case(run_case(mx_hip, case), case)
+
+
+def test_backend_is_hip(mx_hip):
+    assert mx_hip.name == "hip"
+
+
+def test_errors_match(mx_hip):
+    mx = mx_hip
+    with pytest.raises(MxError) as e:
+        mx.tensor([1.0, 2.0, 3.0]).add(mx.tensor([1.0, 2.0]))
+    assert e.value.kind == "InvalidShape"
+    with pytest.raises(MxError) as e:
+        mx.tensor(np.ones((2, 3), np.float32)).transpose(0, 1).view((6,))
+    assert e.value.kind == "InvalidOperation"
+    x, w, b = conv_inputs(1, 2, 5, 5, 2, 3, seed=3)
+    with pytest.raises(MxError) as e:
+        conv_step(mx, x, w, b, 1, 0, np.zeros((1, 2, 3, 3), np.float32))
+    assert e.value.kind == "InvalidOperation"
+
+
+def composite(mx, a, b, c):
+    x, y, z = mx.tensor(a).with_grad(), mx.tensor(b).with_grad(), mx.tensor(c).with_grad()
+    h = x.matmul(y).add(z).gelu()                      # [M,K]x[K,N] + [N] broadcast
+    t = h.transpose(0, 1).mul(h.transpose(0, 1)).relu().tanh()
+    r = t.div(t.exp().add_scalar(1.5)).sum(0).mean(0).mul_scalar(3.0)
+    r.backward()
+    return {"r": r.numpy(), "gx": x.grad().numpy(), "gy": y.grad().numpy(), "gz": z.grad().numpy(), "h": h.numpy()}
+
+
+def test_composite_graph_matches_oracle(mx_hip, mx_oracle):
+    rng = np.random.default_rng(11)
+    a, b, c = (rng.standard_normal(s).astype(np.float32) for s in ((37, 19), (19, 23), (23,)))
+    got, ref = composite(mx_hip, a, b, c), composite(mx_oracle, a, b, c)
+    for k in ref:
+        scale = np.abs(ref[k]).max() + 1e-30
+        assert np.abs(got[k] - ref[k]).max() <= 2e-5 * scale, k       # f32 sums in a different order
+
+
+def test_scalar_operand_and_views(mx_hip, mx_oracle):
+    def prog(mx):
+        x = mx.tensor(np.linspace(-2, 2, 24, dtype=np.float32).reshape(2, 3, 4)).with_grad()
+        s = mx.tensor(np.array(0.75, np.float32), shape=()).with_grad()
+        y = x.transpose(0, 2).reshape((-1, 2)).mul(s).pow(2.0).sum_to_shape((1, 2)).sum_all()
+        y.backward()
+        return {"y": y.numpy(), "gs": s.grad().numpy(), "gx": x.grad().numpy()}
+    got, ref = prog(mx_hip), prog(mx_oracle)
+    for k in ref:
+        np.testing.assert_allclose(got[k], ref[k], rtol=1e-5, atol=1e-6, err_msg=k)
+
+
+def test_mlp_training(mx_hip, mx_oracle):
+    got = mlp_run(mx_hip, 60)
+    ref = mlp_run(mx_oracle, 60)
+    np.testing.assert_allclose(got["losses"], ref["losses"], rtol=1e-4)
+    np.testing.assert_allclose(got["weight"], ref["weight"], rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(got["bias"], ref["bias"], rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(got["input_grad"], ref["input_grad"], rtol=1e-3, atol=1e-7)
+    losses, w, b = mlp_numpy(60)
+    np.testing.assert_allclose(got["losses"], losses, rtol=2e-4)
+    np.testing.assert_allclose(got["weight"], w, rtol=1e-4, atol=1e-6)
+
+
+def test_mlp_steps_do_not_allocate_after_warmup(mx_hip):
+    mlp_run(mx_hip, 3)
+    before = mx_hip.device_allocations()
+    mlp_run(mx_hip, 20)
+    assert mx_hip.device_allocations() == before          # every buffer of a step comes from the pool
+
+
+@pytest.mark.parametrize("B,Cin,H,W,Cout,k,stride,pad", [(2, 3, 6, 5, 4, 3, 1, 1), (1, 2, 7, 7, 3, 3, 2, 2), (3, 4, 5, 5, 2, 1, 1, 1),
+                                                         (4, 16, 14, 14, 32, 3, 1, 1)])
+def test_conv2d_forward_backward(mx_hip, mx_oracle, B, Cin, H, W, Cout, k, stride, pad):
+    x, w, b = conv_inputs(B, Cin, H, W, Cout, k, seed=B * 100 + H)
+    oh, ow = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    target = np.random.default_rng(5).standard_normal((B, Cout, oh, ow)).astype(np.float32)
+    got = conv_step(mx_hip, x, w, b, stride, pad, target)
+    ref = conv_step(mx_oracle, x, w, b, stride, pad, target)
+    num = conv_numpy(x, w, b, stride, pad, target)
+    for key in ("out", "loss", "grad_b", "grad_w", "grad_x"):
+        scale = np.abs(ref[key]).max() + 1e-30
+        assert np.abs(got[key] - ref[key]).max() <= 2e-5 * scale, key
+        assert np.abs(got[key] - num[key]).max() <= 1e-4 * scale, key

@@ -342,7 +342,9 @@ def matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt, b_bcast=False):
 
 
 MM_SHAPES = [(1, 128, 128, 128), (1, 256, 192, 320), (2, 130, 70, 97), (3, 64, 600, 64), (1, 1000, 3, 1), (1, 3, 1000, 1),
-             (1, 10000, 3, 1), (1, 1, 257, 1), (2, 37, 19, 53), (1, 512, 64, 64), (1, 100, 576, 64), (4, 16, 16, 16)]
+             (1, 10000, 3, 1), (1, 1, 257, 1), (2, 37, 19, 53), (1, 512, 64, 64), (1, 100, 576, 64), (4, 16, 16, 16),
+             # long reductions with few output tiles (split over the reduction), tall outputs with few columns
+             (1, 96, 5000, 64), (1, 130, 4100, 70), (2, 64, 2048, 64), (1, 2048, 576, 64), (1, 1100, 100, 33)]
 
 
 @pytest.mark.parametrize("dt", DTS)
@@ -373,7 +375,8 @@ def test_matmul_broadcast_batch_uses_stride0(oracle, hip):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("shape", [(1, 128, 128, 128), (2, 130, 70, 97), (1, 10000, 3, 1), (1, 300, 576, 64), (3, 33, 65, 17)],
+@pytest.mark.parametrize("shape", [(1, 128, 128, 128), (2, 130, 70, 97), (1, 10000, 3, 1), (1, 300, 576, 64), (3, 33, 65, 17), (1, 3000, 96, 64),
+                          (1, 4096, 64, 576)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_matmul_backward(oracle, hip, shape, dt):
     batch, m, k, n = shape
