@@ -17,7 +17,7 @@ namespace mxh {
 struct ConvMeta {
     uint32_t B, C, H, W, kh, kw, oh, ow, ph, pw, sh, sw;
     FastDiv d_owv, d_oh, d_kw, d_kh, d_C;      // im2col index walk
-    FastDiv d_W, d_H, d_Cc;                    // col2im index walk
+    FastDiv d_W, d_H, d_Cc, d_sh, d_sw;        // col2im index walk
 };
 
 constexpr int CB = 256;
@@ -67,8 +67,12 @@ __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restr
     fd_divmod(r, m.d_Cc, b, c);
     uint32_t h_pad = h + m.ph, w_pad = w + m.pw;
     uint32_t hs = h_pad > m.kh - 1 ? h_pad - (m.kh - 1) : 0, ws = w_pad > m.kw - 1 ? w_pad - (m.kw - 1) : 0;
-    uint32_t h_start = (hs + m.sh - 1) / m.sh, w_start = (ws + m.sw - 1) / m.sw;
-    uint32_t h_end = min(h_pad / m.sh + 1, m.oh), w_end = min(w_pad / m.sw + 1, m.ow);
+    uint32_t h_start, w_start, h_last, w_last, rem;
+    fd_divmod(hs + m.sh - 1, m.d_sh, h_start, rem);
+    fd_divmod(ws + m.sw - 1, m.d_sw, w_start, rem);
+    fd_divmod(h_pad, m.d_sh, h_last, rem);
+    fd_divmod(w_pad, m.d_sw, w_last, rem);
+    uint32_t h_end = min(h_last + 1, m.oh), w_end = min(w_last + 1, m.ow);
     T sum = T{};
     for (uint32_t ho = h_start; ho < h_end; ++ho)
         for (uint32_t wo = w_start; wo < w_end; ++wo) {
@@ -119,6 +123,7 @@ void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
     if (n_out == 0) return;
     if (n_out >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "col2im: 2^32 or more output elements"); return; }
     m.d_W = make_fastdiv(m.W); m.d_H = make_fastdiv(m.H); m.d_Cc = make_fastdiv(m.C);
+    m.d_sh = make_fastdiv(m.sh); m.d_sw = make_fastdiv(m.sw);
     hipLaunchKernelGGL(col2im_kernel<T>, dim3(cdiv(n_out, CB)), dim3(CB), 0, stream(), m, col, out, n_out, num_els);
     MXH_LAUNCH_CHECK("col2im");
 }

@@ -2,10 +2,10 @@
 // cuda_pad_with_constant_backward_<T> of crates/maidenx_cuda/src/ops/padding.rs:13-71 with the
 // CPU semantics of crates/maidenx_cpu/src/ops/padding.rs:7-113 and :327-436.
 // Metadata: in_dims[n] | in_strides[n] | in_offset | out_dims[n] | (pad_before, pad_after)[n]
-// Pure data movement, bit-exact.  One lane per output element; the coordinate walk uses
+// Pure data movement, bit-exact.  One lane per 16 bytes of output; the coordinate walk uses
 // multiply-high division on the collapsed shape (dims without padding whose input strides chain
 // are merged, so [B,C,H,W] padded on H,W walks two divisions, not four).
-#include "mxh.hpp"
+#include "elementwise.hpp"
 
 namespace mxh {
 
@@ -21,32 +21,71 @@ struct PadSpace {
 constexpr int PB = 256;
 
 // forward: out[i] = inside ? in[idx] : pad_value
-// backward (GATHER = false): grad_in[idx] = 0 + grad_out[i] for every inside i
-template <class T, bool FWD>
+// backward (FWD = false): grad_in[idx] = 0 + grad_out[i] for every inside i
+// A thread owns Q consecutive output elements: one coordinate decomposition (multiply-high divisions), then
+// carries; the contiguous side (out for forward, grad_out for backward) moves as one Q-element vector.
+template <class T, bool FWD, int Q>
 __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __restrict__ src, T* __restrict__ dst,
                                                        size_t n_out, T pad_value) {
-    size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
-    if (i >= n_out) return;
-    uint32_t r = (uint32_t)i;
-    int64_t idx = 0;
-    bool inside = true;
-    for (int d = sp.ndims - 1; d >= 0; --d) {
-        uint32_t q, c;
-        if (d > 0) fd_divmod(r, sp.div[d], q, c);
-        else { q = 0; c = r; }
-        uint32_t ic = c - sp.before[d];               // wraps when c < before → fails the test below
-        inside = inside && ic < sp.in_dims[d];
-        idx += (int64_t)ic * sp.in_strides[d];
-        r = q;
+    size_t i0 = ((size_t)blockIdx.x * PB + threadIdx.x) * Q;
+    if (i0 >= n_out) return;
+    uint32_t c[MAXD];
+    {
+        uint32_t r = (uint32_t)i0;
+#pragma unroll
+        for (int d = MAXD - 1; d >= 0; --d) {
+            if (d >= sp.ndims) { c[d] = 0; continue; }
+            uint32_t q, m;
+            if (d > 0) fd_divmod(r, sp.div[d], q, m);
+            else { q = 0; m = r; }
+            c[d] = m;
+            r = q;
+        }
+    }
+    const bool full = i0 + Q <= n_out;
+    AVec<T, Q> v;
+    if constexpr (!FWD) {
+        if (full) v = *(const AVec<T, Q>*)(src + i0);
+        else
+            for (int e = 0; e < Q; ++e) v.v[e] = i0 + e < n_out ? src[i0 + e] : T{};
+    }
+#pragma unroll
+    for (int e = 0; e < Q; ++e) {
+        int64_t idx = 0;
+        bool inside = true;
+#pragma unroll
+        for (int d = 0; d < MAXD; ++d) {
+            if (d >= sp.ndims) break;
+            uint32_t ic = c[d] - sp.before[d];           // wraps when c < before → fails the test below
+            inside = inside && ic < sp.in_dims[d];
+            idx += (int64_t)ic * sp.in_strides[d];
+        }
+        if constexpr (FWD) {
+            v.v[e] = inside && (full || i0 + e < n_out) ? src[idx] : pad_value;
+        } else {
+            if (inside && (full || i0 + e < n_out)) {
+                T g = v.v[e];
+                if constexpr (sizeof(T) == 4) dst[idx] = 0.0f + g;        // −0 → +0 like the reference's sums from zero
+                else dst[idx] = f2bf(0.0f + bf2f(g));
+            }
+        }
+        // next output element: add one with carries
+        bool carry = true;
+#pragma unroll
+        for (int d = MAXD - 1; d >= 0; --d) {
+            if (d >= sp.ndims) continue;
+            if (carry) {
+                c[d] += 1;
+                carry = c[d] == sp.out_dims[d];
+                if (carry) c[d] = 0;
+            }
+        }
     }
     if constexpr (FWD) {
-        dst[i] = inside ? src[idx] : pad_value;
-    } else {
-        if (inside) {
-            T g = src[i];
-            if constexpr (sizeof(T) == 4) dst[idx] = 0.0f + g;            // −0 → +0 like the reference's sums from zero
-            else dst[idx] = f2bf(0.0f + bf2f(g));
-        }
+        if (full) *(AVec<T, Q>*)(dst + i0) = v;
+        else
+            for (int e = 0; e < Q; ++e)
+                if (i0 + e < n_out) dst[i0 + e] = v.v[e];
     }
 }
 
@@ -103,7 +142,11 @@ void pad_forward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const T
     if (n_out >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad: output of 2^31 or more elements"); return; }
     PadSpace sp; size_t off; bool cont, exact;
     if (!build_space(nd, md, sp, &off, &cont, &exact)) { set_status(ERR_UNSUPPORTED, "pad: rank above 8 after collapse"); return; }
-    hipLaunchKernelGGL((pad_const_kernel<T, true>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
+    constexpr int Q = 16 / sizeof(T);
+    if ((uintptr_t)out % 16 == 0)
+        hipLaunchKernelGGL((pad_const_kernel<T, true, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
+    else
+        hipLaunchKernelGGL((pad_const_kernel<T, true, 1>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
     MXH_LAUNCH_CHECK("pad_const");
 }
 
@@ -120,7 +163,11 @@ void pad_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const 
         MXH_LAUNCH_CHECK("pad_zero");
     }
     if (n_out == 0) return;
-    hipLaunchKernelGGL((pad_const_kernel<T, false>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
+    constexpr int Q = 16 / sizeof(T);
+    if ((uintptr_t)go % 16 == 0)
+        hipLaunchKernelGGL((pad_const_kernel<T, false, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
+    else
+        hipLaunchKernelGGL((pad_const_kernel<T, false, 1>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
     MXH_LAUNCH_CHECK("pad_const_backward");
 }
 

@@ -175,6 +175,10 @@ __global__ __launch_bounds__(RB) void reduce_generic_kernel(NdSpace<1> sp, const
 
 // ---- host drivers ---------------------------------------------------------------------------------
 constexpr size_t TARGET_BLOCKS = 2048;   // 256 CUs x 8 resident blocks
+// Column reductions keep 8 independent 16-byte loads in flight per thread, so two blocks per CU already cover the
+// memory latency; longer chunks mean fewer partials to write and fold (measured best on [8192,8192] and [64,512,1024]).
+constexpr size_t COL_TARGET_BLOCKS = 512;
+constexpr size_t COL_MIN_ROWS = 128;
 
 template <class T> inline bool aligned16(const T* p) { return ((uintptr_t)p & 15u) == 0; }
 
@@ -243,25 +247,42 @@ void col_stage(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, unsig
     MXH_LAUNCH_CHECK("col_reduce");
 }
 
+// Folds [outer, chunks, S] f32 partials.  Many chunks go through a second round of partials (the other half of the
+// scratch slot) so that the fold itself has enough threads.
+template <class TOut, class R>
+void fold_partials(const float* part, TOut* out, size_t outer, unsigned chunks, size_t S, float div, bool src_bf16) {
+    size_t base_blocks = (outer * (S / 4 + 1) + RB - 1) / RB;
+    if (chunks >= 64 && base_blocks < 64) {
+        unsigned c2 = 8;
+        size_t len2 = (chunks + c2 - 1) / c2;
+        c2 = (unsigned)((chunks + len2 - 1) / len2);
+        float* part2 = (float*)part + outer * (size_t)chunks * S + 64;
+        col_stage<float, float, R>(part, part2, outer, chunks, S, c2, len2, 0.0f, src_bf16);
+        col_stage<float, TOut, R>(part2, out, outer, c2, S, 1, c2, div, src_bf16);
+        return;
+    }
+    col_stage<float, TOut, R>(part, out, outer, chunks, S, 1, chunks, div, src_bf16);
+}
+
 // [outer, L, S] (contiguous) → out[outer, S]
 template <class TIn, class TOut, class R>
 void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, float div, bool src_bf16) {
     size_t base_blocks = (outer * (S / 4 + 1) + RB - 1) / RB;
     unsigned chunks = 1;
     size_t chunk_len = L;
-    if (base_blocks < TARGET_BLOCKS && L >= 64) {
-        size_t want = (TARGET_BLOCKS + base_blocks - 1) / base_blocks;
-        size_t max_chunks = L / 32;                // at least 32 rows per chunk
+    if (base_blocks < COL_TARGET_BLOCKS && L >= 2 * COL_MIN_ROWS) {
+        size_t want = (COL_TARGET_BLOCKS + base_blocks - 1) / base_blocks;
+        size_t max_chunks = L / COL_MIN_ROWS;   // at least this many rows per chunk
         chunks = (unsigned)(want < max_chunks ? want : max_chunks);
         if (chunks < 1) chunks = 1;
         chunk_len = (L + chunks - 1) / chunks;
         chunks = (unsigned)((L + chunk_len - 1) / chunk_len);
     }
     if (chunks == 1) { col_stage<TIn, TOut, R>(in, out, outer, L, S, 1, L, div, src_bf16); return; }
-    float* part = (float*)scratch(outer * chunks * S * sizeof(float) + 256);
+    float* part = (float*)scratch((outer * chunks * S + outer * 8 * S) * sizeof(float) + 1024);
     if (!part) return;
     col_stage<TIn, float, R>(in, part, outer, L, S, chunks, chunk_len, 0.0f, src_bf16);
-    col_stage<float, TOut, R>(part, out, outer, chunks, S, 1, chunks, div, src_bf16);
+    fold_partials<TOut, R>(part, out, outer, chunks, S, div, src_bf16);
 }
 
 // sum/mean/max/min metadata: dims[n] | strides[n] | red_len[r] | red_stride[r] | offset
