@@ -1,0 +1,178 @@
+"""GPU parity at the sizes BASELINE.json's configs name, through checks that do not need the (slow) CPU oracle at
+those sizes: single IEEE operations against numpy bit for bit, reductions and products against float64 numpy,
+data-movement kernels against numpy indexing, and size-independent properties (linearity, adjointness,
+transposition symmetry)."""
+import numpy as np
+import pytest
+
+from helpers import In, Out, f32_to_bf16, meta_binary, meta_conv, meta_matmul, meta_pad, meta_reduce, meta_sum_to_shape, meta_unary, to_float
+
+pytestmark = pytest.mark.gpu
+
+R = C = 8192
+
+
+def same_bits(a, b):
+    return np.array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(b).view(np.uint8))
+
+
+@pytest.fixture(scope="module")
+def xy():
+    r = np.random.default_rng(0x5EED0002)
+    return r.standard_normal((R, C), dtype=np.float32), r.standard_normal((R, C), dtype=np.float32)
+
+
+@pytest.mark.parametrize("case", ["contiguous", "rhs_row", "lhs_transposed"])
+def test_elementwise_8192_f32_bit_exact(hip, xy, case):
+    x, y = xy
+    n = R * C
+    if case == "contiguous":
+        md, lhs, rhs, a, b = meta_binary([R, C], [C, 1], [C, 1]), x, y, x, y
+    elif case == "rhs_row":
+        row = y[0].copy()
+        md, lhs, rhs, a, b = meta_binary([R, C], [C, 1], [0, 1]), x, row, x, row[None, :]
+    else:
+        md, lhs, rhs, a, b = meta_binary([R, C], [1, R], [C, 1]), x, y, x.T, y      # x's buffer viewed transposed
+    for op, fn in (("add", np.add), ("mul", np.multiply)):
+        (out,) = hip.call(f"{op}_f32", n, 2, md, In(lhs.ravel()), In(rhs.ravel()), Out(n, "f32"))
+        assert same_bits(out.reshape(R, C), fn(a, b)), (op, case)
+    (out,) = hip.call("div_f32", n, 2, md, In(lhs.ravel()), In(rhs.ravel()), Out(n, "f32"))
+    with np.errstate(all="ignore"):
+        want = np.divide(a, b)
+    zero = np.broadcast_to(b == 0, want.shape)          # the float32 normal generator does emit a few exact zeros
+    want = np.where(zero, np.where(a == 0, np.float32(0), np.float32(np.inf)), want)   # crates/maidenx_cpu/src/ops/binary.rs:440-452
+    assert same_bits(out.reshape(R, C), want.astype(np.float32))
+
+
+def test_elementwise_8192_bf16_bit_exact(hip, xy):
+    x, y = xy
+    xb, yb = f32_to_bf16(x.ravel()), f32_to_bf16(y.ravel())
+    n = R * C
+    (out,) = hip.call("mul_bf16", n, 2, meta_binary([R, C], [C, 1], [C, 1]), In(xb), In(yb), Out(n, "bf16"))
+    want = f32_to_bf16(to_float(xb, "bf16") * to_float(yb, "bf16"))
+    assert same_bits(out, want)
+    (out,) = hip.call("relu_bf16", n, 2, meta_unary([R, C], [1, R]), In(xb), Out(n, "bf16"))   # transposed view
+    want = np.maximum(to_float(xb, "bf16").reshape(C, R).T, 0).ravel()
+    assert same_bits(to_float(out, "bf16"), want.astype(np.float32))
+
+
+def test_unary_8192_f32(hip, xy):
+    x, _ = xy
+    n = R * C
+    (out,) = hip.call("relu_f32", n, 2, meta_unary([R, C], [C, 1]), In(x.ravel()), Out(n, "f32"))
+    assert same_bits(out, np.where(x > 0, x, np.float32(0)).ravel())
+    (out,) = hip.call("exp_f32", n, 2, meta_unary([R, C], [C, 1]), In(x.ravel()), Out(n, "f32"))
+    ref = np.exp(x.astype(np.float64)).ravel()
+    assert np.max(np.abs(out - ref) / ref) < 1.2e-7                                    # within 1 ulp of the true value
+    # gelu: odd-symmetry identity of the tanh form, gelu(x) - gelu(-x) = x (to rounding)
+    (g1,) = hip.call("gelu_f32", n, 2, meta_unary([R, C], [C, 1]), In(x.ravel()), Out(n, "f32"))
+    (g2,) = hip.call("gelu_f32", n, 2, meta_unary([R, C], [C, 1]), In((-x).ravel()), Out(n, "f32"))
+    assert np.max(np.abs((g1.astype(np.float64) - g2) - x.ravel())) < 1e-6
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192), (64, 512, 1024)], ids=["8192x8192", "64x512x1024"])
+def test_reductions_fullsize(hip, shape):
+    r = np.random.default_rng(0x5EED0003)
+    x = r.uniform(-1, 1, shape).astype(np.float32)
+    n = x.size
+    strides = [int(np.prod(shape[i + 1:])) for i in range(len(shape))]
+    x64 = x.astype(np.float64)
+    for dim in range(len(shape)):
+        L = shape[dim]
+        md = meta_reduce(list(shape), strides, dim)
+        (s,) = hip.call("sum_f32", n, len(shape), 1, md, In(x.ravel()), Out(n // L, "f32"))
+        scale = np.abs(x64).sum(dim).ravel()
+        assert np.max(np.abs(s - x64.sum(dim).ravel()) / scale) <= 1e-5
+        (m,) = hip.call("mean_f32", n, len(shape), 1, md, In(x.ravel()), Out(n // L, "f32"))
+        assert np.max(np.abs(m - x64.mean(dim).ravel()) / (scale / L)) <= 1e-5
+        (mx,) = hip.call("max_f32", n, len(shape), 1, md, In(x.ravel()), Out(n // L, "f32"))
+        assert same_bits(mx, x.max(dim).ravel())                                       # exact, order-independent
+    if len(shape) == 3:
+        md = meta_sum_to_shape(list(shape), strides, [1, shape[1], 1])
+        (s,) = hip.call("sum_to_shape_f32", n, 3, md, In(x.ravel()), Out(shape[1], "f32"))
+        assert np.max(np.abs(s - x64.sum((0, 2))) / np.abs(x64).sum((0, 2))) <= 1e-5
+    else:
+        md = meta_sum_to_shape(list(shape), strides, list(shape))
+        (s,) = hip.call("sum_to_shape_f32", n, 2, md, In(x.ravel()), Out(n, "f32"))
+        assert same_bits(s, (x + np.float32(0)).ravel())                               # identity, -0 -> +0
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_matmul_4096_sampled_and_linear(hip, dt):
+    M = K = N = 4096
+    r = np.random.default_rng(0x5EED0004)
+    a = r.standard_normal((M, K), dtype=np.float32)
+    b = (r.standard_normal((K, N), dtype=np.float32) * np.float32(0.02))
+    go = r.standard_normal((M, N), dtype=np.float32)
+    st = (lambda v: f32_to_bf16(v.ravel())) if dt == "bf16" else (lambda v: v.ravel())
+    val = (lambda s: to_float(s, dt).astype(np.float64))
+    sa, sb, sg = st(a), st(b), st(go)
+    av, bv, gv = val(sa).reshape(M, K), val(sb).reshape(K, N), val(sg).reshape(M, N)
+    md = meta_matmul([M, N], [M, K], [K, N], [K, 1], [N, 1])
+    (c,) = hip.call(f"matmul_{dt}", M * N, md, In(sa), In(sb), Out(M * N, dt))
+    ga, gb = hip.call(f"matmul_backward_{dt}", M * K, K * N, md, In(sg), In(sa), In(sb), Out(M * K, dt), Out(K * N, dt))
+    tol = 1e-5 if dt == "f32" else 1e-2
+    rows = r.choice(M, 48, replace=False)
+    cv = val(c).reshape(M, N)
+    assert np.max(np.abs(cv[rows] - av[rows] @ bv) / (np.abs(av[rows]) @ np.abs(bv))) <= tol
+    gav = val(ga).reshape(M, K)
+    assert np.max(np.abs(gav[rows] - gv[rows] @ bv.T) / (np.abs(gv[rows]) @ np.abs(bv.T))) <= tol
+    krows = r.choice(K, 48, replace=False)
+    gbv = val(gb).reshape(K, N)
+    assert np.max(np.abs(gbv[krows] - av[:, krows].T @ gv) / (np.abs(av[:, krows].T) @ np.abs(gv))) <= tol
+    # every output tile is touched: column and row checksums of C against (1^T A) B and A (B 1)
+    assert np.max(np.abs(cv.sum(0) - av.sum(0) @ bv) / (np.abs(av).sum(0) @ np.abs(bv))) <= tol
+    assert np.max(np.abs(cv.sum(1) - av @ bv.sum(1)) / (np.abs(av) @ np.abs(bv).sum(1))) <= tol
+    assert np.max(np.abs(gbv.sum(1) - av.T @ gv.sum(1)) / (np.abs(av.T) @ np.abs(gv).sum(1))) <= tol
+
+
+def test_matmul_batched_config(hip):
+    Bt, M, K, N = 32, 512, 1024, 1024
+    r = np.random.default_rng(7)
+    a = r.standard_normal((Bt, M, K), dtype=np.float32)
+    b = r.standard_normal((Bt, K, N), dtype=np.float32) * np.float32(0.02)
+    md = meta_matmul([Bt, M, N], [Bt, M, K], [Bt, K, N], [M * K, K, 1], [K * N, N, 1])
+    (c,) = hip.call("matmul_f32", Bt * M * N, md, In(a.ravel()), In(b.ravel()), Out(Bt * M * N, "f32"))
+    c = c.reshape(Bt, M, N).astype(np.float64)
+    for bi in (0, 13, 31):
+        ref = a[bi].astype(np.float64) @ b[bi]
+        assert np.max(np.abs(c[bi] - ref) / (np.abs(a[bi].astype(np.float64)) @ np.abs(b[bi]))) <= 1e-5
+
+
+def test_conv_kernels_config_size(hip):
+    Bn, Cc, H, W, k = 32, 64, 56, 56, 3
+    r = np.random.default_rng(0x5EED0005)
+    x = r.standard_normal((Bn, Cc, H, W), dtype=np.float32)
+    ncol = Bn * Cc * k * k * H * W
+    md = meta_conv(Bn, Cc, H, W, k, k, H, W, 1, 1, 1, 1)
+    (col,) = hip.call("conv2d_im2col_f32", ncol, md, In(x.ravel()), Out(ncol, "f32"))
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    ref = np.empty((Bn, Cc, k, k, H, W), np.float32)
+    for i in range(k):
+        for j in range(k):
+            ref[:, :, i, j] = xp[:, :, i:i + H, j:j + W]
+    assert same_bits(col, ref.ravel())
+    # col2im of the whole column matrix: every pixel is the sum of its (up to 9) copies, in a fixed order
+    (img,) = hip.call("conv2d_col2im_f32", ncol, md, In(col), Out(x.size, "f32"))
+    cnt = np.zeros((H + 2, W + 2))
+    for i in range(k):
+        for j in range(k):
+            cnt[i:i + H, j:j + W] += 1
+    cnt = cnt[1:H + 1, 1:W + 1]
+    np.testing.assert_allclose(img.reshape(x.shape), x * cnt.astype(np.float32), rtol=1e-6, atol=0)
+    # the layer's call: num_els = B*C*H*W, columns beyond it dropped (nn/layers/conv.rs:393)
+    (img2,) = hip.call("conv2d_col2im_f32", x.size, md, In(col), Out(x.size, "f32"))
+    g = ref.ravel().copy()
+    g[x.size:] = 0
+    g = g.reshape(Bn, Cc, k, k, H, W).astype(np.float64)
+    acc = np.zeros((Bn, Cc, H + 2, W + 2))
+    for i in range(k):
+        for j in range(k):
+            acc[:, :, i:i + H, j:j + W] += g[:, :, i, j]
+    np.testing.assert_allclose(img2.reshape(x.shape), acc[:, :, 1:H + 1, 1:W + 1], rtol=1e-6, atol=1e-6)
+    # pad [32,64,56,56] -> [32,64,58,58] and its backward
+    mdp = meta_pad([Bn, Cc, H, W], [Cc * H * W, H * W, W, 1], 0, [Bn, Cc, H + 2, W + 2], [(0, 0), (0, 0), (1, 1), (1, 1)])
+    (p,) = hip.call("pad_with_constant_f32", x.size, xp.size, 4, mdp, In(x.ravel()), Out(xp.size, "f32"), 0.0)
+    assert same_bits(p, xp.ravel())
+    (gi,) = hip.call("pad_with_constant_backward_f32", x.size, xp.size, 4, mdp, In(xp.ravel()), Out(x.size, "f32"))
+    assert same_bits(gi, (x + np.float32(0)).ravel())
