@@ -65,6 +65,16 @@ int hip_event_destroy(void* event);
 int hip_event_record(void* event);
 int hip_event_synchronize(void* event);
 int hip_event_elapsed_ms(void* start, void* stop, float* ms);
+/* Graph capture of a launch-bound call sequence (no counterpart in the reference).  begin_capture drains the
+ * device and routes every later kernel of this library to a capture stream; end_capture returns an executable
+ * graph and restores the previous stream; graph_launch replays it in stream order.  While capturing, the caller
+ * must issue nothing that allocates, copies to the host or synchronises: warm the same sequence up eagerly first,
+ * so that the library's scratch has its final size (a call that would have to grow it fails with
+ * MX_HIP_ERR_INVALID instead).  Fill with hip_fill_*, not memset. */
+int hip_graph_begin_capture(void);
+int hip_graph_end_capture(void** graph_exec);
+int hip_graph_launch(void* graph_exec);
+int hip_graph_destroy(void* graph_exec);
 
 /* ---- binary: replaces crates/maidenx_cuda/src/ops/binary.rs:12-161 --------------------------------
  * metadata = dims[n] | lhs_strides[n] | rhs_strides[n] | lhs_offset | rhs_offset   (NULL: contiguous)

@@ -15,6 +15,9 @@ static int g_status = OK;
 static int g_hip_err = 0;
 static char g_what[256] = "ok";
 static hipStream_t g_stream = nullptr;      // null = the device's default stream
+static hipStream_t g_capture_stream = nullptr;   // created on first use, default priority
+static hipStream_t g_saved_stream = nullptr;
+static bool g_capturing = false;
 static void* g_scratch[16][2] = {{nullptr}};
 static size_t g_scratch_bytes[16][2] = {{0}};
 
@@ -39,6 +42,10 @@ void* scratch(size_t bytes, int slot) {
     }
     std::lock_guard<std::mutex> lk(g_scratch_mu);
     if (g_scratch_bytes[dev][slot] >= bytes) return g_scratch[dev][slot];
+    if (g_capturing) {      // growing means a synchronise and a free, neither of which a capture allows
+        set_status(ERR_INVALID, "scratch would have to grow during graph capture: run the sequence eagerly once first");
+        return nullptr;
+    }
     // grow: work already queued on the stream may still use the old block, so drain first
     if (g_scratch[dev][slot]) {
         (void)hipStreamSynchronize(g_stream);
@@ -94,7 +101,11 @@ int hip_stream_synchronize(void* s) { return (int)hipStreamSynchronize((hipStrea
 // Stream every later kernel and copy of the backend is queued on (null = default stream).
 int hip_set_stream(void* s) { g_stream = (hipStream_t)s; return 0; }
 void* hip_get_stream(void) { return (void*)g_stream; }
-int hip_synchronize(void) { return (int)hipStreamSynchronize(stream()); }
+int hip_synchronize(void) {
+    hipError_t e = hipStreamSynchronize(stream());
+    if (e == hipSuccess && g_capture_stream && !g_capturing) e = hipStreamSynchronize(g_capture_stream);   // graph replays
+    return (int)e;
+}
 
 // Events on the backend's stream, for timing kernels where they run.
 int hip_event_create(void** ev) { return (int)hipEventCreate((hipEvent_t*)ev); }
@@ -118,5 +129,46 @@ int hip_get_last_status(void) {
 }
 // Text of the error last returned by hip_get_last_status().
 const char* hip_status_string(void) { return g_what; }
+
+
+int hip_graph_begin_capture(void) {
+    if (g_capturing) return (int)hipErrorInvalidValue;
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return (int)e;
+    if (!g_capture_stream) {
+        e = hipStreamCreate(&g_capture_stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    e = hipStreamBeginCapture(g_capture_stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return (int)e;
+    g_saved_stream = g_stream;
+    g_stream = g_capture_stream;
+    g_capturing = true;
+    return 0;
+}
+int hip_graph_end_capture(void** graph_exec) {
+    if (!g_capturing || !graph_exec) return (int)hipErrorInvalidValue;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(g_capture_stream, &graph);
+    g_stream = g_saved_stream;
+    g_capturing = false;
+    if (e != hipSuccess) return (int)e;
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return (int)e;
+    *graph_exec = (void*)exec;
+    return 0;
+}
+// Replays run on the capture stream, a blocking stream: work on the default stream orders with it.
+int hip_graph_launch(void* graph_exec) {
+    if (!graph_exec || !g_capture_stream || g_capturing) return (int)hipErrorInvalidValue;
+    return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, g_capture_stream);
+}
+int hip_graph_destroy(void* graph_exec) {
+    if (!graph_exec) return 0;
+    (void)hipStreamSynchronize(g_capture_stream);
+    return (int)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+}
 
 }  // extern "C"

@@ -19,6 +19,11 @@ struct HipBackend {
         if (st != MX_HIP_OK) throw mxt::Error(st == MX_HIP_ERR_OOM ? mxt::ErrKind::OutOfMemory : mxt::ErrKind::Backend,
                                               std::string("HIP backend: ") + hip_status_string());
     }
+    static constexpr bool has_graphs = true;
+    static void graph_begin() { if (hip_graph_begin_capture() != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_begin_capture failed"); }
+    static void graph_end(void** exec) { if (hip_graph_end_capture(exec) != 0) { *exec = nullptr; throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_end_capture failed"); } }
+    static void graph_launch(void* exec) { if (hip_graph_launch(exec) != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_launch failed"); }
+    static void graph_destroy(void* exec) { hip_graph_destroy(exec); }
     // host-side steps of the reference, done on the device
     static void fill_f32(size_t n, float* p, float v) { if (n) hip_fill_f32(n, p, v); }
     static void cast_bool_f32(size_t n, const uint8_t* in, float* out) { if (n) hip_cast_bool_f32(n, in, out); }

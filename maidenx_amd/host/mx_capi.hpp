@@ -15,9 +15,11 @@ struct Module {
     std::unique_ptr<mxt::Linear<B>> linear;
     std::unique_ptr<mxt::Conv2d<B>> conv;
     std::vector<T*> parameters() { return kind == 0 ? linear->parameters() : conv->parameters(); }
-    T forward(const T& x) { return kind == 0 ? linear->forward(x) : conv->forward(x); }
+    T forward(const T& x) const { return kind == 0 ? linear->forward(x) : conv->forward(x); }
 };
 
+inline bool g_graphs = true;
+inline size_t g_replayed = 0;
 inline thread_local int g_kind = 0;
 inline thread_local std::string g_text;
 inline void set_error(int k, const std::string& t) { g_kind = k; g_text = t; }
@@ -227,20 +229,10 @@ int mxt_sgd_step(mxt_module m, float lr) { return guard_i([&] { mxt::SGD<B>(lr).
 int mxt_sgd_zero_grad(mxt_module m) { return guard_i([&] { mxt::SGD<B>(0.0f).zero_grad(((Module*)m)->parameters()); }); }
 
 int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_t epochs, float* losses) {
-    return guard_i([&] {
-        Module* mod = (Module*)m;
-        T &x = ref(input), &y = ref(target);
-        mxt::SGD<B> opt(lr);
-        for (size_t e = 0; e < epochs; ++e) {
-            T pred = mod->forward(x);
-            T loss = mxt::mse_loss<B>(pred, y);
-            loss.backward();
-            opt.step(mod->parameters());
-            opt.zero_grad(mod->parameters());
-            if (losses) losses[e] = loss.item();
-        }
-    });
+    return guard_i([&] { g_replayed = mxt::train_loop<B>(*(Module*)m, ref(input), ref(target), lr, epochs, losses, g_graphs); });
 }
+void mxt_set_graph_replay(int enabled) { g_graphs = enabled != 0; }
+size_t mxt_last_train_replayed(void) { return g_replayed; }
 
 size_t mxt_backend_calls(void) { return mxt::backend_calls(); }
 void mxt_reset_backend_calls(void) { mxt::backend_calls() = 0; }

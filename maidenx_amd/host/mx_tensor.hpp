@@ -30,6 +30,7 @@
 #include <functional>
 #include <map>
 #include <memory>
+#include <set>
 #include <stdexcept>
 #include <string>
 #include <unordered_set>
@@ -112,8 +113,11 @@ inline size_t dtype_size(DType d) { return d == DType::F32 ? 4 : 1; }
 // given to the next tensor at once: whatever still reads it was queued earlier.
 template <class B>
 struct Pool {
-    std::map<size_t, std::vector<void*>> free_blocks;
+    // Free blocks per bucket, lowest address first: which block a request gets then depends only on the set of
+    // free blocks, not on the order they came back in, so a repeated call sequence settles into repeating addresses.
+    std::map<size_t, std::set<void*>> free_blocks;
     size_t cached = 0, live = 0, device_allocs = 0;
+    std::vector<void*>* trace = nullptr;        // when set, every block handed out is appended (see train loop)
     static constexpr size_t kMaxCached = size_t(64) << 30;
     static size_t bucket(size_t bytes) {
         if (bytes <= 256) return 256;
@@ -125,10 +129,11 @@ struct Pool {
         cap = bucket(bytes);
         auto it = free_blocks.find(cap);
         if (it != free_blocks.end() && !it->second.empty()) {
-            void* p = it->second.back();
-            it->second.pop_back();
+            void* p = *it->second.begin();
+            it->second.erase(it->second.begin());
             cached -= cap;
             live += cap;
+            if (trace) trace->push_back(p);
             return p;
         }
         void* p = B::alloc(cap);
@@ -139,12 +144,13 @@ struct Pool {
         }
         ++device_allocs;
         live += cap;
+        if (trace) trace->push_back(p);
         return p;
     }
     void put(void* p, size_t cap) {
         live -= cap;
         if (cached + cap > kMaxCached) { B::sync(); B::free(p); return; }
-        free_blocks[cap].push_back(p);
+        free_blocks[cap].insert(p);
         cached += cap;
     }
     void trim() {
@@ -169,7 +175,15 @@ struct Storage {
 
 template <class B> struct Node;
 template <class B> struct Tensor;
-template <class B> struct GradCell { std::shared_ptr<Tensor<B>> g; };
+// The gradient of a tensor.  The reference allocates and zero-fills it in with_grad() and zero_grad()
+// (wt.rs:100, lib.rs:262) and the first accumulate_grad adds into those zeros.  Here the zeros stay virtual until
+// someone needs them: the first accumulation of a contiguous gradient of the same shape writes 0 + g straight into
+// a fresh buffer (the identity sum_to_shape kernel, the same bits as zeros then add_inplace), anything else
+// materialises the zeros first.
+template <class B> struct GradCell {
+    std::shared_ptr<Tensor<B>> g;      // null while the gradient is still all zeros
+    Shape shape;
+};
 
 // Count of backend kernel calls (what `be::*` would dispatch), for reporting.
 inline size_t& backend_calls() { static size_t n = 0; return n; }
@@ -253,16 +267,28 @@ struct Tensor {
         requires_grad = true;
         if (!grad_cell) {
             grad_cell = std::make_shared<GradCell<B>>();
-            grad_cell->g = std::make_shared<T>(zeros_like(*this));
+            grad_cell->shape = shape();
         }
     }
-    bool has_grad() const { return grad_cell && grad_cell->g; }
+    bool has_grad() const { return (bool)grad_cell; }
     T grad() const {
         if (!has_grad()) throw Error(ErrKind::InvalidOperation, "tensor has no grad");
+        if (!grad_cell->g) grad_cell->g = std::make_shared<T>(zeros(grad_cell->shape));
         return *grad_cell->g;
     }
     void accumulate_grad(const T& g) const {                                        // lib.rs:221-241
-        if (has_grad()) grad_cell->g->add_(g);
+        if (!has_grad()) return;
+        if (!grad_cell->g && g.dtype == DType::F32 && g.is_contiguous() && g.shape() == grad_cell->shape) {
+            T fresh = empty(grad_cell->shape);
+            auto md = meta_to_shape(g, g.shape());
+            B::sum_to_shape(g.size(), g.ndim(), md.data(), g.f32(), fresh.f32());      // fresh = 0 + g
+            ++backend_calls();
+            B::check();
+            grad_cell->g = std::make_shared<T>(fresh);
+            return;
+        }
+        if (!grad_cell->g) grad_cell->g = std::make_shared<T>(zeros(grad_cell->shape));
+        grad_cell->g->add_(g);
     }
     T detach() const {                                                              // f.rs:67-73
         T r = *this;
@@ -276,7 +302,7 @@ struct Tensor {
     }
     void zero_grad_impl(std::unordered_set<const void*>& visited) const {
         if (!visited.insert(buf.get()).second) return;
-        if (has_grad()) *grad_cell->g = zeros_like(*grad_cell->g);
+        if (has_grad()) grad_cell->g.reset();                       // all zeros again
         if (node)
             for (const T& in : node->inputs)
                 if (in.requires_grad) in.zero_grad_impl(visited);
@@ -1040,5 +1066,74 @@ struct SGD {                                                                    
         for (Tensor<B>* p : params) p->zero_grad();
     }
 };
+
+// ---- the training loop of examples/device/cpu.rs:32-38 -----------------------------------------------
+// forward, loss, backward, optimizer step, zero_grad.  `losses` (may be null) receives every epoch's loss, which
+// costs a device-to-host copy per epoch.
+//
+// When the backend can record graphs and no loss is read back, the loop is launch-bound (tens of small kernels per
+// step), so it is recorded once and replayed: the pool hands out the same blocks in the same order every `period`
+// steps once it is warm (a step's allocations and releases are a fixed sequence), which makes the recorded pointers
+// valid for every replay and leaves the host-side tensors pointing at the right blocks afterwards.  The period is
+// measured, not assumed; without one the loop stays eager.
+template <class B, class Model>
+size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr, size_t epochs, float* losses, bool allow_graph) {
+    SGD<B> opt(lr);
+    auto step = [&](size_t e) {
+        Tensor<B> pred = model.forward(x);
+        Tensor<B> loss = mse_loss<B>(pred, y);
+        loss.backward();
+        opt.step(model.parameters());
+        opt.zero_grad(model.parameters());
+        if (losses) losses[e] = loss.item();
+    };
+    size_t done = 0, replayed = 0;
+    if constexpr (B::has_graphs) {
+        constexpr size_t kWarm = 16, kMaxPeriod = 4;      // the README loop settles into period 3 after 5 steps
+        if (allow_graph && !losses && epochs >= 2 * kWarm) {
+            Pool<B>& pool = Pool<B>::instance();
+            std::vector<std::vector<void*>> traces;
+            for (; done < kWarm; ++done) {
+                traces.emplace_back();
+                pool.trace = &traces.back();
+                step(done);
+                pool.trace = nullptr;
+            }
+            size_t period = 0;
+            for (size_t p = 1; p <= kMaxPeriod && !period; ++p) {
+                bool same = true;
+                for (size_t k = 0; k < 2 * p && same; ++k) same = traces[kWarm - 1 - k] == traces[kWarm - 1 - k - p];
+                if (same) period = p;
+            }
+            if (period) {
+                void* exec = nullptr;
+                const size_t allocs_before = pool.device_allocs, calls_before = backend_calls();
+                B::graph_begin();
+                try {
+                    for (size_t k = 0; k < period; ++k) step(done + k);
+                } catch (...) {
+                    try { B::graph_end(&exec); } catch (...) { exec = nullptr; }
+                    if (exec) B::graph_destroy(exec);
+                    throw;
+                }
+                B::graph_end(&exec);
+                if (pool.device_allocs != allocs_before) {
+                    B::graph_destroy(exec);
+                    throw Error(ErrKind::Backend, "training loop allocated device memory while it was being recorded");
+                }
+                // the recorded steps did not run yet: replay them, then as many more whole periods as fit
+                const size_t calls_per_period = backend_calls() - calls_before;
+                size_t periods = (epochs - done) / period;
+                for (size_t r = 0; r < periods; ++r) B::graph_launch(exec);
+                backend_calls() += calls_per_period * (periods - 1);
+                done += periods * period;
+                replayed = periods * period;
+                B::graph_destroy(exec);
+            }
+        }
+    }
+    for (; done < epochs; ++done) step(done);
+    return replayed;
+}
 
 }  // namespace mxt

@@ -40,7 +40,8 @@ def _bind(lib):
         "mxt_linear_new": ([P, P], P), "mxt_linear_new_seeded": ([SZ, SZ, I, C.c_uint64], P),
         "mxt_conv2d_new": ([P, P, SZ, SZ, SZ, SZ, SZ, SZ], P), "mxt_module_forward": ([P, P], P), "mxt_module_weight": ([P], P),
         "mxt_module_bias": ([P], P), "mxt_module_release": ([P], None), "mxt_mse_loss": ([P, P], P), "mxt_sgd_step": ([P, F], I),
-        "mxt_sgd_zero_grad": ([P], I), "mxt_train": ([P, P, P, F, SZ, P], I),
+        "mxt_sgd_zero_grad": ([P], I), "mxt_train": ([P, P, P, F, SZ, P], I), "mxt_set_graph_replay": ([I], None),
+        "mxt_last_train_replayed": ([], SZ),
         "mxt_backend_calls": ([], SZ), "mxt_reset_backend_calls": ([], None), "mxt_device_allocations": ([], SZ), "mxt_synchronize": ([], I),
     }
     for name, (args, res) in sig.items():
@@ -119,6 +120,12 @@ class Host:
         losses = np.zeros(epochs, np.float32) if record_losses else None
         self._rc(self.lib.mxt_train(module.h, x.h, y.h, lr, epochs, losses.ctypes.data if record_losses else None))
         return losses
+
+    def set_graph_replay(self, enabled):
+        self.lib.mxt_set_graph_replay(int(enabled))
+
+    def last_train_replayed(self):
+        return self.lib.mxt_last_train_replayed()
 
     def backend_calls(self):
         return self.lib.mxt_backend_calls()

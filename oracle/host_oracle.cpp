@@ -33,6 +33,7 @@ struct OracleBackend {
     static void h2d(void* d, const void* s, size_t n) { std::memcpy(d, s, n); }
     static void d2h(void* d, const void* s, size_t n) { std::memcpy(d, s, n); }
     static void check() {}
+    static constexpr bool has_graphs = false;
     // The reference does these on the host as well.
     static void fill_f32(size_t n, float* p, float v) { for (size_t i = 0; i < n; ++i) p[i] = v; }              // creation.rs:144-164, 253-305
     static void cast_bool_f32(size_t n, const uint8_t* in, float* out) { for (size_t i = 0; i < n; ++i) out[i] = in[i] ? 1.0f : 0.0f; }

@@ -94,3 +94,33 @@ def test_conv2d_forward_backward(mx_hip, mx_oracle, B, Cin, H, W, Cout, k, strid
         scale = np.abs(ref[key]).max() + 1e-30
         assert np.abs(got[key] - ref[key]).max() <= 2e-5 * scale, key
         assert np.abs(got[key] - num[key]).max() <= 1e-4 * scale, key
+
+
+def test_graph_replayed_training_equals_eager(mx_hip):
+    """mxt_train records the step as a HIP graph and replays it; every run is compared with the eager loop, with
+    eager work and synchronisations in between (the same graph machinery is set up and torn down each time)."""
+    from host_programs import mlp_data
+    mx = mx_hip
+    x, y = mlp_data()
+
+    def run(epochs, graphs):
+        mx.set_graph_replay(graphs)
+        lin = mx.Linear(mx.tensor(np.array([[0.3, -0.2, 0.5]], np.float32)), mx.tensor(np.array(0.1, np.float32), shape=()))
+        xin = mx.tensor(x).with_grad()
+        mx.train(lin, xin, mx.tensor(y), 0.01, epochs)
+        mx.synchronize()
+        replayed = mx.last_train_replayed()
+        return lin.weight.numpy(), lin.bias.numpy(), xin.grad().numpy(), replayed
+    try:
+        for epochs in (40, 41, 100, 75):       # 16 eager epochs, then whole periods of the recorded steps, then the rest eager
+            w0, b0, g0, r0 = run(epochs, False)
+            assert r0 == 0
+            w1, b1, g1, r1 = run(epochs, True)
+            assert r1 >= epochs - 16 - 3, "the loop fell back to eager launches"
+            assert np.array_equal(w0, w1) and np.array_equal(b0, b1) and np.array_equal(g0, g1), epochs
+            # eager work between the runs
+            t = mx.tensor(np.arange(12, dtype=np.float32).reshape(3, 4)).with_grad()
+            t.mul(t).sum_all().backward()
+            np.testing.assert_array_equal(t.grad().numpy(), 2 * np.arange(12, dtype=np.float32).reshape(3, 4))
+    finally:
+        mx.set_graph_replay(True)
