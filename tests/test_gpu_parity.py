@@ -367,6 +367,24 @@ def test_matmul_forward(oracle, hip, shape, a_perm, b_perm, dt):
             assert same_bits(o, h)
 
 
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", [(1, 4096, 64, 3072), (1, 4096, 128, 3072), (1, 3072, 320, 4096), (3, 2048, 192, 2048)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_matmul_whole_256_tiles(hip, shape, a_perm, b_perm, dt):
+    """At least 192 whole 256x256 output tiles: the unchecked 8-wave configuration (1, 2, 5 and 3 k-tiles for bf16),
+    for every operand layout."""
+    batch, m, k, n = shape
+    r = rng(59)
+    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt)
+    (h,) = hip.call(f"matmul_{dt}", batch * m * n, md, In(sa), In(sb), Out(batch * m * n, dt))
+    truth = np.einsum("bmk,bkn->bmn", av, bv)
+    scale = np.einsum("bmk,bkn->bmn", np.abs(av), np.abs(bv))
+    tol = 1e-5 if dt == "f32" else 1e-2
+    err = np.abs(to_float(h, dt).reshape(truth.shape) - truth) / np.maximum(scale, 1e-30)
+    assert np.max(err) <= tol, float(np.max(err))
+
+
 def test_matmul_broadcast_batch_uses_stride0(oracle, hip):
     r = rng(47)
     sa, sb, md, av, bv = matmul_inputs(r, 3, 40, 50, 60, False, False, "f32", b_bcast=True)
