@@ -22,7 +22,10 @@
 //   * `with_buffer_mut`'s copy-on-write of a shared buffer (lib.rs:166-180) is not reproduced: in-place
 //     ops write the buffer they are given;
 //   * contiguous(), zeros/ones, bool -> f32 and the broadcast of a 0-d tensor run on the device when the
-//     backend offers a kernel for them (the reference goes through host memory).
+//     backend offers a kernel for them (the reference goes through host memory);
+//   * the reference zero-fills the outputs of sum, sum_to_shape and matmul_backward from the host before the
+//     kernel overwrites them, and zero-fills every gradient when it is created: the first is skipped (the kernels
+//     write every output element), the second is deferred until the zeros are needed (see GradCell).
 #pragma once
 #include <cmath>
 #include <cstdint>
@@ -610,7 +613,7 @@ struct Tensor {
         need_f32("reduction");
         Shape out = shape();
         out.erase(out.begin() + dim);
-        T result = zeros(out);                                   // the reference zero-fills reduction outputs
+        T result = empty(out);       // the reference zero-fills first (reduction.rs:28); the kernels write every output
         auto md = meta_reduce(*this, dim);
         fn(size(), ndim(), 1, md.data(), f32(), result.f32());
         ++backend_calls();
@@ -656,7 +659,7 @@ struct Tensor {
                 throw Error(ErrKind::ShapeMismatch, "Dimension " + std::to_string(i) + " is not divisible: " + std::to_string(shape()[i]) +
                                                         " -> " + std::to_string(target[i]));
         need_f32("sum_to_shape");
-        T result = zeros(target);
+        T result = empty(target);    // zero-filled in the reference (reduction.rs:112); fully written by the kernel
         auto md = meta_to_shape(*this, target);
         B::sum_to_shape(size(), ndim(), md.data(), f32(), result.f32());
         ++backend_calls();
@@ -883,7 +886,7 @@ struct Tensor {
             result.set_node("matmul", {*this, rhs_in}, [](const std::vector<T>& in, const T& go) {     // ops/matmul.rs:63-146
                 const T &l = in[0], &r = in[1];
                 auto mm = meta_matmul(l, r);
-                T gl = zeros_like(l), gr = zeros_like(r);
+                T gl = empty(l.shape()), gr = empty(r.shape());     // zeros_like in the reference; both are fully written
                 B::matmul_backward(gl.size(), gr.size(), mm.first.data(), go.f32(), l.f32(), r.f32(), gl.f32(), gr.f32());
                 ++backend_calls();
                 B::check();
