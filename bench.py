@@ -327,6 +327,10 @@ def run_elementwise(args):
                          "contiguous / rhs [1,8192] broadcast / transposed lhs",
                          {"kernel_launches_per_step": len(chains), "algorithmic_GB_per_step": round(step_bytes / 1e9, 3)})
     result["roofline"] = hbm_roofline("ew_nd_kernel<OpMul<float>,4> (hip_mul_f32, contiguous [8192,8192])", probe_bytes, durs)
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size: a
+    # recorded measurement (counters cannot be collected from inside this process)
+    result["roofline"]["traffic"] = 805.3e6
+    result["roofline"]["traffic_source"] = "profiles/elementwise_8192x8192_hbm_traffic.txt"
     L.synchronize()
     del chains, builders
     result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_elementwise(args)
