@@ -1,9 +1,8 @@
-#!/usr/bin/env python3
 """Benchmark of the maidenx_hip backend on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul|mlp|conv|copy]
 
-The default workload is BASELINE.json's configs[1]: elementwise forward + backward of add, mul, div,
+The default workload is the elementwise configuration (configs[1]): forward + backward of add, mul, div,
 exp, relu, gelu on [8192,8192] tensors, f32 and bf16, for contiguous operands, a [1,8192] broadcast
 rhs and a transposed lhs view, with the gradients taken through sum_to_shape and accumulated in
 place.  One "step" issues, through the C ABI, the chain of backend kernels the reference's tensor

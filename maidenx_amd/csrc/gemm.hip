@@ -10,10 +10,12 @@
 // so the two transposed backward products need no materialised transpose: the operand whose
 // reduction index is strided is turned while it is staged into LDS.
 //
-// Large products run on MFMA (v_mfma_f32_32x32x16_bf16 / v_mfma_f32_32x32x2_f32): 128x128 output
-// tile per 256-thread block, 2x2 waves, each wave a 64x64 patch = 2x2 MFMA tiles, f32 accumulate,
-// one rounding at the end for bf16.  Operands sit in LDS as [row][k] with the reduction index
-// contiguous, so a lane fetches its whole fragment with one 128-bit ds_read.
+// Large products run on MFMA (v_mfma_f32_32x32x16_bf16 / v_mfma_f32_32x32x2_f32), f32 accumulate, one
+// rounding at the end for bf16: 256x256 output tiles on 8-wave blocks (two waves per SIMD keep the matrix
+// pipe fed), 128x128 on 4-wave blocks for problems with few tiles, 256x64 for narrow outputs; products
+// with few tiles and a long reduction are split over the reduction and folded in a fixed order.
+// Operands sit in LDS as [row][k] with the reduction index contiguous, so a lane fetches its whole
+// fragment with one 128-bit ds_read.
 // Small or skinny products (the MLP's [10000,3]x[3,1] and its [3,10000]x[10000,1] gradient) use
 // a thread-per-output kernel (bit-exact with the reference: k ascending, unfused f32) or a
 // wave-per-output dot kernel.

@@ -1,4 +1,4 @@
-"""GPU parity at the sizes BASELINE.json's configs name, through checks that do not need the (slow) CPU oracle at
+"""GPU parity at the full sizes of the benchmark configurations, through checks that do not need the (slow) CPU oracle at
 those sizes: single IEEE operations against numpy bit for bit, reductions and products against float64 numpy,
 data-movement kernels against numpy indexing, and size-independent properties (linearity, adjointness,
 transposition symmetry)."""
