@@ -90,8 +90,9 @@ int mxt_sgd_zero_grad(mxt_module m);
  * without leaving native code.  losses (may be NULL) receives the loss of every epoch; reading it costs one
  * device-to-host copy per epoch, so pass NULL when timing. */
 int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_t epochs, float* losses);
-/* With losses == NULL and at least 32 epochs the HIP build records the step as a graph after 16 eager epochs and
- * replays it (the loop is launch-bound); results are those of the eager loop.  mxt_set_graph_replay(0) keeps every
+/* With losses == NULL and at least 32 epochs the HIP build runs eagerly until the buffer addresses of a step repeat
+ * (8 to 64 epochs), then records that many steps as a graph and replays it (the loop is launch-bound); results are
+ * those of the eager loop.  mxt_set_graph_replay(0) keeps every
  * epoch eager; mxt_last_train_replayed() tells how many epochs of the last mxt_train call were replays. */
 void mxt_set_graph_replay(int enabled);
 size_t mxt_last_train_replayed(void);

@@ -1092,21 +1092,26 @@ size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr
     };
     size_t done = 0, replayed = 0;
     if constexpr (B::has_graphs) {
-        constexpr size_t kWarm = 16, kMaxPeriod = 4;      // the README loop settles into period 3 after 5 steps
-        if (allow_graph && !losses && epochs >= 2 * kWarm) {
+        constexpr size_t kMinWarm = 8, kMaxWarm = 64, kMaxPeriod = 4;   // the README loop settles into period 3 after 5 steps
+        if (allow_graph && !losses && epochs >= 4 * kMinWarm) {
             Pool<B>& pool = Pool<B>::instance();
             std::vector<std::vector<void*>> traces;
-            for (; done < kWarm; ++done) {
+            size_t period = 0;
+            const size_t warm_limit = std::min<size_t>(kMaxWarm, epochs / 2);
+            while (done < warm_limit && !period) {
                 traces.emplace_back();
                 pool.trace = &traces.back();
                 step(done);
                 pool.trace = nullptr;
-            }
-            size_t period = 0;
-            for (size_t p = 1; p <= kMaxPeriod && !period; ++p) {
-                bool same = true;
-                for (size_t k = 0; k < 2 * p && same; ++k) same = traces[kWarm - 1 - k] == traces[kWarm - 1 - k - p];
-                if (same) period = p;
+                ++done;
+                const size_t n = traces.size();
+                if (n < kMinWarm) continue;
+                // a period p is accepted when the last 2p steps repeat the p steps before them
+                for (size_t p = 1; p <= kMaxPeriod && !period && 3 * p <= n; ++p) {
+                    bool same = true;
+                    for (size_t k = 0; k < 2 * p && same; ++k) same = traces[n - 1 - k] == traces[n - 1 - k - p];
+                    if (same) period = p;
+                }
             }
             if (period) {
                 void* exec = nullptr;

@@ -113,3 +113,35 @@ def test_conv2d_backward_with_zero_padding_is_an_error(mx_oracle):
     with pytest.raises(MxError) as e:
         conv_step(mx_oracle, x, w, b, 1, 0, target)
     assert e.value.kind == "InvalidOperation"
+
+
+@pytest.mark.parametrize("op", ["add", "mul", "div", "exp", "relu", "gelu"])
+@pytest.mark.parametrize("case", ["contig", "bcast", "transposed"])
+def test_bench_chain_is_the_host_layers_call_sequence(mx_oracle, op, case):
+    """bench.py's ChainBuilder spells out, call by call, what forward + backward of each op dispatches to the
+    backend.  The host layer derives the same thing from the reference's backward closures; the number of backend
+    calls must agree (device-side casts are not backend calls in the reference and are not counted)."""
+    import bench
+    if op in ("exp", "relu", "gelu") and case == "bcast":
+        pytest.skip("unary ops have no broadcast case")
+    mx = mx_oracle
+    R, C = 6, 8
+
+    class FakeLib:
+        def __getattr__(self, name):
+            return lambda *a: None
+    b = bench.ChainBuilder(FakeLib(), "x_", lambda count, dtag, init: (0, None), "f32", R, C, seed=1)
+    getattr(b, op)(case)
+    want = sum(1 for c in b.calls if not c.tag.startswith("cast_bool"))
+
+    rng = np.random.default_rng(3)
+    if case == "transposed":
+        base = mx.tensor(rng.standard_normal((C, R)).astype(np.float32)).with_grad()
+        x = base.transpose(0, 1)
+    else:
+        x = mx.tensor(rng.standard_normal((R, C)).astype(np.float32)).with_grad()
+    y = mx.tensor(rng.standard_normal((1, C) if case == "bcast" else (R, C)).astype(np.float32) + 3.0).with_grad()
+    mx.reset_backend_calls()
+    z = getattr(x, op)(y) if op in ("add", "mul", "div") else getattr(x, op)()
+    z.backward()
+    assert mx.backend_calls() == want, (op, case, mx.backend_calls(), want)
