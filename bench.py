@@ -72,6 +72,7 @@ class ChainBuilder:
         self.go = new(self.N, init=np.ones(self.N, np.float32))
         self.z = new(self.N)
         self.t = [new(self.N) for _ in range(8)]
+        self.tf = [new(self.N, "f32") for _ in range(8)] if dt == "bf16" else []      # promoted intermediates (gelu backward)
         self.mask = new(self.N, "bool")
         self.gx, self.gy, self.gbase, self.gxv = (new(self.N, init=np.zeros(self.N, np.float32)) for _ in range(4))
         self.grow = new(Cc, init=np.zeros(Cc, np.float32))
@@ -86,8 +87,9 @@ class ChainBuilder:
     def _fn(self, name):
         return getattr(self.lib, self.prefix + name)
 
-    def binary(self, op, a, la, b, lb, out, tag=None, out_dt=None):
-        dt, e = self.dt, ESZ[self.dt]
+    def binary(self, op, a, la, b, lb, out, tag=None, out_dt=None, dt=None):
+        dt = dt or self.dt
+        e = ESZ[dt]
         md = u64([self.R, self.C], self.lay[la][0], self.lay[lb][0], 0, 0)
         nb = (self.lay[la][1] + self.lay[lb][1]) * e + self.N * ESZ[out_dt or dt]
         self.calls.append(Call(self._fn(f"{op}_{dt}"), (self.N, 2, md.ctypes.data, a, b, out), nb, tag or f"{op}_{dt}/{la}+{lb}", md))
@@ -105,12 +107,16 @@ class ChainBuilder:
         self.calls.append(Call(self._fn(f"add_inplace_{self.dt}"), (self.C, 2, md.ctypes.data, acc, b), 3 * self.C * ESZ[self.dt],
                                f"add_inplace_{self.dt}/row", md))
 
-    def unary(self, op, a, la, out, c=None, out_dt=None):
-        dt = self.dt
+    def unary(self, op, a, la, out, c=None, out_dt=None, dt=None):
+        dt = dt or self.dt
         md = u64([self.R, self.C], self.lay[la][0], 0)
         nb = self.lay[la][1] * ESZ[dt] + self.N * ESZ[out_dt or dt]
         args = (self.N, 2, md.ctypes.data, a, out) if c is None else (self.N, 2, md.ctypes.data, a, const(c, dt), out)
         self.calls.append(Call(self._fn(f"{op}_{dt}"), args, nb, f"{op}_{dt}/{la}", md))
+
+    def cast(self, src, dst, a, out):
+        """with_dtype of a whole buffer (crates/maidenx_tensor/src/wt.rs:65-84): a host loop in the reference, a device kernel here."""
+        self.calls.append(Call(self._fn(f"cast_{src}_{dst}"), (self.N, a, out), self.N * (ESZ[src] + ESZ[dst]), f"cast_{src}_{dst}", None))
 
     def cast_bool(self, a, out):
         self.calls.append(Call(self._fn(f"cast_bool_{self.dt}"), (self.N, a, out), self.N * (1 + ESZ[self.dt]), f"cast_bool_{self.dt}", None))
@@ -194,6 +200,8 @@ class ChainBuilder:
         self.acc_lhs(self.t[1], case)
 
     def gelu(self, case):
+        if self.dt == "bf16":
+            return self.gelu_bf16(case)
         x, lx, _, _ = self.operands(case)
         t = self.t
         c0, coeff = 0.7978845608028654, 0.044715
@@ -218,6 +226,49 @@ class ChainBuilder:
         self.binary("add", t[5], "contig", t[4], "contig", t[6])
         self.binary("mul", self.go, "contig", t[6], "contig", t[7])
         self.acc_lhs(t[7], case)
+
+    def gelu_bf16(self, case):
+        """The same closure on bf16 tensors.  A scalar that is not integer-valued promotes its tensor to f32
+        (ops/unary.rs:870-878), and a bf16 x f32 binary op promotes to f32 (utils/promotion.rs:16-33), so from the first
+        `mul_scalar(0.044715)` on the chain runs in f32 and the gradient is cast back when it is accumulated
+        (ops/binary.rs:660-662).  Every promotion is a with_dtype of a whole buffer."""
+        x, lx, _, _ = self.operands(case)
+        t, f = self.t, self.tf
+        c0, coeff = 0.7978845608028654, 0.044715
+        F = dict(dt="f32")
+        self.unary("gelu", x, lx, self.z)
+        self.binary("mul", x, lx, x, lx, t[0])                      # x_squared (bf16)
+        self.binary("mul", t[0], "contig", x, lx, t[1])             # x_cubed (bf16)
+        self.cast("bf16", "f32", t[1], f[0])
+        self.unary("mul_scalar", f[0], "contig", f[1], c=coeff, **F)
+        self.cast("bf16", "f32", x, f[0])                           # input promoted for the add (keeps its layout)
+        self.binary("add", f[0], lx, f[1], "contig", f[2], **F)
+        self.unary("mul_scalar", f[2], "contig", f[1], c=c0, **F)   # tanh_arg
+        self.unary("tanh", f[1], "contig", f[2], **F)               # tanh_val
+        self.binary("mul", f[2], "contig", f[2], "contig", f[1], **F)
+        self.unary("mul_scalar", f[1], "contig", f[3], c=-1.0, **F)
+        self.unary("add_scalar", f[3], "contig", f[1], c=1.0, **F)  # sech_squared
+        self.cast("bf16", "f32", t[0], f[3])                        # x_squared promoted
+        self.unary("mul_scalar", f[3], "contig", f[4], c=3.0 * coeff, **F)
+        self.unary("add_scalar", f[4], "contig", f[3], c=1.0, **F)
+        self.unary("mul_scalar", f[3], "contig", f[4], c=c0, **F)   # inner_derivative
+        self.unary("add_scalar", f[2], "contig", f[3], c=1.0, **F)
+        self.unary("mul_scalar", f[3], "contig", f[5], c=0.5, **F)  # term1
+        self.cast("bf16", "f32", x, f[0])                           # input promoted again for input * sech_squared
+        self.binary("mul", f[0], lx, f[1], "contig", f[3], **F)
+        self.binary("mul", f[3], "contig", f[4], "contig", f[6], **F)
+        self.unary("mul_scalar", f[6], "contig", f[3], c=0.5, **F)  # term2
+        self.binary("add", f[5], "contig", f[3], "contig", f[6], **F)
+        self.cast("bf16", "f32", self.go, f[0])                     # grad_out promoted
+        self.binary("mul", f[0], "contig", f[6], "contig", f[7], **F)
+        # accumulate_grad casts the f32 gradient to the parameter's dtype, once per add_
+        self.cast("f32", "bf16", f[7], t[7])
+        if case == "transposed":
+            self.inplace("add", self.gxv, t[7], "contig")
+            self.cast("f32", "bf16", f[7], t[6])
+            self.inplace("add", self.gbase, t[6], "transposed_back", dims=[self.C, self.R])
+        else:
+            self.inplace("add", self.gx, t[7], "contig")
 
     def build(self):
         for case in ("contig", "bcast", "transposed"):
@@ -548,6 +599,7 @@ def cpu_baseline_elementwise(args):
         builders.append(b)
         # the oracle has no device-side cast: the reference converts bool -> float on the host
         b.cast_bool = lambda a, out, b=b: b.calls.append(Call(lambda *x: None, (), 0, "host_cast", None))
+        b.cast = lambda src, dst, a, out, b=b: b.calls.append(Call(lambda *x: None, (), 0, "host_cast", None))
         chains += b.build()
     nbytes = sum(c.bytes for c in chains)
     t0 = time.perf_counter()
@@ -560,7 +612,8 @@ def cpu_baseline_elementwise(args):
             break
     el = time.perf_counter() - t0
     return {"value": round(nbytes * reps / el / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"same kernel chain on [{R},{Cc}] tensors (1/32 of the rows), {reps} passes, {el:.1f} s"}
+            "sample": f"same kernel chain on [{R},{Cc}] tensors (1/32 of the rows; the host-side dtype casts of the reference "
+                      f"are left out, in the CPU's favour), {reps} passes, {el:.1f} s"}
 
 
 def _mlp_setup(mx):
