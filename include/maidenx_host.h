@@ -2,7 +2,9 @@
  *
  * The host layer replays MaidenX's tensor / autograd / nn calls above the backend kernels of
  * maidenx_hip.h: each function below names the reference function whose backend-call sequence it issues.
- * Tensors are opaque handles; a handle is released with mxt_release.  f32 only.
+ * Tensors are opaque handles; a handle is released with mxt_release.  Float tensors are f32 or bf16 (comparisons
+ * give bool); mixed operands and non-integer scalars promote as the reference does (utils/promotion.rs:16-33,
+ * ops/unary.rs:872-876).  Conv2d is f32 only.
  *
  * Functions that return a handle return NULL on error, functions that return int return non-zero;
  * mxt_last_error() then gives the error kind (the variant of crates/maidenx_core/src/error.rs that the
@@ -35,9 +37,17 @@ typedef void* mxt_module;
 int mxt_last_error(char* text, size_t cap);      /* kind of the last failure on this thread; copies its text */
 const char* mxt_backend_name(void);
 
-/* creation: crates/maidenx_tensor/src/creation.rs:25-84 (new), :253-305 (fill); randn is seeded here */
+/* dtypes */
+#define MXT_F32 0
+#define MXT_BF16 1
+#define MXT_BOOL 2
+
+/* creation: crates/maidenx_tensor/src/creation.rs:25-84 (new), :253-305 (fill); randn is seeded here.  The _dtype
+ * forms take f32 values and store them in the given float dtype; the plain forms are f32. */
 mxt_tensor mxt_new(const float* data, const size_t* shape, size_t ndim);
 mxt_tensor mxt_fill(const size_t* shape, size_t ndim, float value);
+mxt_tensor mxt_new_dtype(const float* data, const size_t* shape, size_t ndim, int dtype);
+mxt_tensor mxt_fill_dtype(const size_t* shape, size_t ndim, float value, int dtype);
 mxt_tensor mxt_randn(const size_t* shape, size_t ndim, uint64_t seed);
 void mxt_release(mxt_tensor t);
 
@@ -47,6 +57,8 @@ size_t mxt_size(mxt_tensor t);
 size_t mxt_offset(mxt_tensor t);
 void mxt_shape(mxt_tensor t, size_t* out);
 void mxt_strides(mxt_tensor t, size_t* out);
+int mxt_dtype(mxt_tensor t);
+mxt_tensor mxt_to_dtype(mxt_tensor t, int dtype);   /* wt.rs:86-90: converts the whole buffer, keeps the layout */
 int mxt_requires_grad(mxt_tensor t);
 int mxt_is_contiguous(mxt_tensor t);
 int mxt_to_host(mxt_tensor t, float* out);       /* logical (row-major) order; bool tensors as 0/1 */
@@ -100,6 +112,7 @@ size_t mxt_last_train_replayed(void);
 /* bookkeeping */
 size_t mxt_backend_calls(void);                  /* kernels dispatched since the last reset */
 void mxt_reset_backend_calls(void);
+size_t mxt_cast_calls(void);                     /* whole-buffer dtype conversions since the last reset */
 size_t mxt_device_allocations(void);             /* allocations that reached the backend (pool misses) */
 int mxt_synchronize(void);
 

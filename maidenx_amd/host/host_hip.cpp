@@ -24,38 +24,40 @@ struct HipBackend {
     static void graph_end(void** exec) { if (hip_graph_end_capture(exec) != 0) { *exec = nullptr; throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_end_capture failed"); } }
     static void graph_launch(void* exec) { if (hip_graph_launch(exec) != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_launch failed"); }
     static void graph_destroy(void* exec) { hip_graph_destroy(exec); }
-    // host-side steps of the reference, done on the device
-    static void fill_f32(size_t n, float* p, float v) { if (n) hip_fill_f32(n, p, v); }
-    static void cast_bool_f32(size_t n, const uint8_t* in, float* out) { if (n) hip_cast_bool_f32(n, in, out); }
-    static void copy_strided_f32(size_t n, size_t nd, const size_t* md, const float* in, float* out) { hip_copy_strided_f32(n, nd, md, in, out); }
-    static void broadcast_scalar_f32(size_t n, const float* src, float* dst) {
-        const size_t md[3] = {n, 0, 0};                    // dims [n], strides [0], offset 0
-        hip_copy_strided_f32(n, 1, md, src, dst);
-    }
-    static constexpr auto add = &hip_add_f32;
-    static constexpr auto sub = &hip_sub_f32;
-    static constexpr auto mul = &hip_mul_f32;
-    static constexpr auto div = &hip_div_f32;
-    static constexpr auto add_inplace = &hip_add_inplace_f32;
-    static constexpr auto sub_inplace = &hip_sub_inplace_f32;
-    static constexpr auto neg = &hip_neg_f32;
-    static constexpr auto square = &hip_square_f32;
-    static constexpr auto relu = &hip_relu_f32;
-    static constexpr auto tanh = &hip_tanh_f32;
-    static constexpr auto gelu = &hip_gelu_f32;
-    static constexpr auto exp = &hip_exp_f32;
-    static constexpr auto add_scalar = &hip_add_scalar_f32;
-    static constexpr auto mul_scalar = &hip_mul_scalar_f32;
-    static constexpr auto div_scalar = &hip_div_scalar_f32;
-    static constexpr auto pow = &hip_pow_f32;
-    static constexpr auto gt_scalar = &hip_gt_scalar_f32;
-    static constexpr auto sum = &hip_sum_f32;
-    static constexpr auto mean = &hip_mean_f32;
-    static constexpr auto sum_to_shape = &hip_sum_to_shape_f32;
-    static constexpr auto matmul = &hip_matmul_f32;
-    static constexpr auto matmul_backward = &hip_matmul_backward_f32;
+    // f32-only kernels (conv) and the float <-> float conversions
     static constexpr auto im2col = &hip_conv2d_im2col_f32;
     static constexpr auto col2im = &hip_conv2d_col2im_f32;
+    static void cast_bf16_f32(size_t n, const uint16_t* in, float* out) { if (n) hip_cast_bf16_f32(n, in, out); }
+    static void cast_f32_bf16(size_t n, const float* in, uint16_t* out) { if (n) hip_cast_f32_bf16(n, in, out); }
+    // kernels per element type: float, and uint16_t holding bf16 bits
+    template <class E> struct K;
 };
+#define MXT_HIP_KERNELS(E, S)                                                                                          \
+    template <> struct HipBackend::K<E> {                                                                                \
+        using Bin = void (*)(size_t, size_t, const size_t*, const E*, const E*, E*);                                     \
+        using Inp = void (*)(size_t, size_t, const size_t*, E*, const E*);                                               \
+        using Un = void (*)(size_t, size_t, const size_t*, const E*, E*);                                                \
+        using Unc = void (*)(size_t, size_t, const size_t*, const E*, E, E*);                                            \
+        using Red = void (*)(size_t, size_t, size_t, const size_t*, const E*, E*);                                       \
+        static constexpr Bin bin[4] = {&hip_add_##S, &hip_sub_##S, &hip_mul_##S, &hip_div_##S};                          \
+        static constexpr Inp inplace[2] = {&hip_add_inplace_##S, &hip_sub_inplace_##S};                                  \
+        static constexpr Un un[6] = {&hip_neg_##S, &hip_square_##S, &hip_relu_##S, &hip_tanh_##S, &hip_gelu_##S, &hip_exp_##S}; \
+        static constexpr Unc unc[4] = {&hip_add_scalar_##S, &hip_mul_scalar_##S, &hip_div_scalar_##S, &hip_pow_##S};      \
+        static constexpr Red red[2] = {&hip_sum_##S, &hip_mean_##S};                                                     \
+        static constexpr auto gt_scalar = &hip_gt_scalar_##S;                                                            \
+        static constexpr auto sum_to_shape = &hip_sum_to_shape_##S;                                                      \
+        static constexpr auto matmul = &hip_matmul_##S;                                                                  \
+        static constexpr auto matmul_backward = &hip_matmul_backward_##S;                                                \
+        /* host-side steps of the reference, done on the device */                                                       \
+        static void fill(size_t n, E* p, E v) { if (n) hip_fill_##S(n, p, v); }                                          \
+        static void cast_from_bool(size_t n, const uint8_t* in, E* out) { if (n) hip_cast_bool_##S(n, in, out); }        \
+        static void copy_strided(size_t n, size_t nd, const size_t* md, const E* in, E* out) { hip_copy_strided_##S(n, nd, md, in, out); } \
+        static void broadcast_scalar(size_t n, const E* src, E* dst) {                                                   \
+            const size_t md[3] = {n, 0, 0}; /* dims [n], strides [0], offset 0 */                                        \
+            hip_copy_strided_##S(n, 1, md, src, dst);                                                                    \
+        }                                                                                                                \
+    };
+MXT_HIP_KERNELS(float, f32)
+MXT_HIP_KERNELS(uint16_t, bf16)
 using MxtBackend = HipBackend;
 #include "mx_capi.hpp"

@@ -74,6 +74,18 @@ mxt_tensor mxt_new(const float* data, const size_t* shape, size_t ndim) {
 mxt_tensor mxt_fill(const size_t* shape, size_t ndim, float value) {
     return guard_t([&] { return T::fill(to_shape(shape, ndim), value); });
 }
+static mxt::DType dtype_of(int code) {
+    if (code == MXT_F32) return mxt::DType::F32;
+    if (code == MXT_BF16) return mxt::DType::BF16;
+    if (code == MXT_BOOL) return mxt::DType::BOOL;
+    throw mxt::Error(mxt::ErrKind::InvalidArgument, "unknown dtype code");
+}
+mxt_tensor mxt_new_dtype(const float* data, const size_t* shape, size_t ndim, int dtype) {
+    return guard_t([&] { return T::from_host(data, to_shape(shape, ndim), dtype_of(dtype)); });
+}
+mxt_tensor mxt_fill_dtype(const size_t* shape, size_t ndim, float value, int dtype) {
+    return guard_t([&] { return T::fill(to_shape(shape, ndim), value, dtype_of(dtype)); });
+}
 mxt_tensor mxt_randn(const size_t* shape, size_t ndim, uint64_t seed) {
     return guard_t([&] { return mxt::randn<B>(to_shape(shape, ndim), seed); });
 }
@@ -84,6 +96,11 @@ size_t mxt_size(mxt_tensor t) { return ((T*)t)->size(); }
 size_t mxt_offset(mxt_tensor t) { return ((T*)t)->offset(); }
 void mxt_shape(mxt_tensor t, size_t* out) { for (size_t i = 0; i < ((T*)t)->ndim(); ++i) out[i] = ((T*)t)->shape()[i]; }
 void mxt_strides(mxt_tensor t, size_t* out) { for (size_t i = 0; i < ((T*)t)->ndim(); ++i) out[i] = ((T*)t)->strides()[i]; }
+int mxt_dtype(mxt_tensor t) {
+    mxt::DType d = ((T*)t)->dtype;
+    return d == mxt::DType::F32 ? MXT_F32 : d == mxt::DType::BF16 ? MXT_BF16 : MXT_BOOL;
+}
+mxt_tensor mxt_to_dtype(mxt_tensor t, int dtype) { return guard_t([&] { return ref(t).to_dtype(dtype_of(dtype)); }); }
 int mxt_requires_grad(mxt_tensor t) { return ((T*)t)->requires_grad ? 1 : 0; }
 int mxt_is_contiguous(mxt_tensor t) { return ((T*)t)->is_contiguous() ? 1 : 0; }
 int mxt_to_host(mxt_tensor t, float* out) {
@@ -235,7 +252,8 @@ void mxt_set_graph_replay(int enabled) { g_graphs = enabled != 0; }
 size_t mxt_last_train_replayed(void) { return g_replayed; }
 
 size_t mxt_backend_calls(void) { return mxt::backend_calls(); }
-void mxt_reset_backend_calls(void) { mxt::backend_calls() = 0; }
+void mxt_reset_backend_calls(void) { mxt::backend_calls() = 0; mxt::cast_calls() = 0; }
+size_t mxt_cast_calls(void) { return mxt::cast_calls(); }
 size_t mxt_device_allocations(void) { return mxt::Pool<B>::instance().device_allocs; }
 int mxt_synchronize(void) { return guard_i([&] { B::sync(); B::check(); }); }
 }  // extern "C"

@@ -15,7 +15,7 @@
 //
 // The code is a template over a Backend: a struct of static functions (memory, the f32 kernels, and the
 // few helpers the reference runs on the host: fill, strided copy, bool -> f32 cast, scalar broadcast).
-// Only f32 tensors (and bool results of comparisons) exist here; that is what the MLP and conv workloads use.
+// Float tensors are f32 or bf16 (bool results of comparisons); Conv2d is f32 only.
 //
 // Deliberate differences from the reference, none visible in results:
 //   * buffers come from a size-bucketed pool instead of one device allocation per tensor;
@@ -108,8 +108,45 @@ struct Layout {
     }
 };
 
-enum class DType { F32, BOOL };
-inline size_t dtype_size(DType d) { return d == DType::F32 ? 4 : 1; }
+enum class DType { F32, BF16, BOOL };
+inline size_t dtype_size(DType d) { return d == DType::F32 ? 4 : d == DType::BF16 ? 2 : 1; }
+inline bool is_float(DType d) { return d != DType::BOOL; }
+// crates/maidenx_tensor/src/utils/promotion.rs:16-33, for the dtypes that exist here
+inline DType promoted(DType a, DType b) { return a == b ? a : (a == DType::F32 || b == DType::F32) ? DType::F32 : DType::BF16; }
+
+// bf16 as the `half` crate stores it: the high half of an f32, round to nearest even, NaN kept quiet
+inline uint16_t f32_to_bf16(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    return (uint16_t)((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+inline float bf16_to_f32(uint16_t b) {
+    uint32_t x = (uint32_t)b << 16;
+    float f;
+    std::memcpy(&f, &x, 4);
+    return f;
+}
+template <class E> inline E scalar_as(float c);
+template <> inline float scalar_as<float>(float c) { return c; }
+template <> inline uint16_t scalar_as<uint16_t>(float c) { return f32_to_bf16(c); }     // be/ops/unary.rs:312: constant.as_<dtype>()
+
+// element type tags for the two float dtypes: float, and uint16_t holding bf16 bits
+template <class E> struct Tag { using type = E; };
+template <class F>
+void by_dtype(DType dt, const char* what, F&& f) {
+    if (dt == DType::F32) f(Tag<float>{});
+    else if (dt == DType::BF16) f(Tag<uint16_t>{});
+    else throw Error(ErrKind::UnsupportedDType, std::string(what) + ": needs a float tensor");
+}
+enum BinOp { ADD, SUB, MUL, DIV };
+enum InplaceOp { ADD_INPLACE, SUB_INPLACE };
+enum UnOp { NEG, SQUARE, RELU, TANH, GELU, EXP };
+enum UncOp { ADD_SCALAR, MUL_SCALAR, DIV_SCALAR, POW };
+enum RedOp { SUM, MEAN };
+// a float scalar with an integer value keeps the tensor's dtype, any other promotes it to f32
+// (ops/unary.rs:796-800, 872-876; crates/maidenx_core/src/scalar.rs:115-133)
+inline bool integer_valued(float c) { return c == std::trunc(c); }
 
 // ---- buffers: pooled backend memory ------------------------------------------------------------------
 // All kernels of a backend run in call order on one stream, so a block handed back to the pool can be
@@ -186,10 +223,13 @@ template <class B> struct Tensor;
 template <class B> struct GradCell {
     std::shared_ptr<Tensor<B>> g;      // null while the gradient is still all zeros
     Shape shape;
+    DType dtype = DType::F32;
 };
 
 // Count of backend kernel calls (what `be::*` would dispatch), for reporting.
 inline size_t& backend_calls() { static size_t n = 0; return n; }
+// Count of whole-buffer dtype conversions (with_dtype: a host loop in the reference, a kernel here).
+inline size_t& cast_calls() { static size_t n = 0; return n; }
 
 // ---- Tensor (crates/maidenx_tensor/src/lib.rs:21-58): shared data, own metadata, optional node ------
 template <class B>
@@ -213,6 +253,8 @@ struct Tensor {
     bool is_contiguous() const { return layout.is_contiguous(); }
     const float* f32() const { return (const float*)buf->ptr; }
     float* f32() { return (float*)buf->ptr; }
+    template <class E> E* p() const { return (E*)buf->ptr; }
+    template <class E> using K = typename B::template K<E>;
 
     // -- creation (creation.rs) --
     static T empty(const Shape& shape, DType dt = DType::F32) {                     // creation.rs:115-131
@@ -222,18 +264,30 @@ struct Tensor {
         t.buf = std::make_shared<Storage<B>>(t.layout.size(), dt);
         return t;
     }
-    static T fill(const Shape& shape, float v) {                                    // creation.rs:253-305
-        T t = empty(shape);
-        B::fill_f32(t.size(), t.f32(), v);
+    static T fill(const Shape& shape, float v, DType dt = DType::F32) {             // creation.rs:253-305
+        T t = empty(shape, dt);
+        by_dtype(dt, "fill", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::fill(t.size(), t.template p<E>(), scalar_as<E>(v));
+        });
         return t;
     }
-    static T zeros(const Shape& shape) { return fill(shape, 0.0f); }                // creation.rs:144-176
-    static T ones(const Shape& shape) { return fill(shape, 1.0f); }
-    static T zeros_like(const T& s) { return zeros(s.shape()); }
-    static T ones_like(const T& s) { return ones(s.shape()); }
-    static T from_host(const float* data, const Shape& shape) {                     // creation.rs:25-84
-        T t = empty(shape);
-        if (t.size()) B::h2d(t.buf->ptr, data, t.size() * sizeof(float));
+    static T zeros(const Shape& shape, DType dt = DType::F32) { return fill(shape, 0.0f, dt); }   // creation.rs:144-176
+    static T ones(const Shape& shape, DType dt = DType::F32) { return fill(shape, 1.0f, dt); }
+    static T zeros_like(const T& s) { return zeros(s.shape(), s.dtype); }
+    static T ones_like(const T& s) { return ones(s.shape(), s.dtype); }
+    static T from_host(const float* data, const Shape& shape, DType dt = DType::F32) {   // creation.rs:25-84
+        T t = empty(shape, dt);
+        if (!t.size()) return t;
+        if (dt == DType::F32) {
+            B::h2d(t.buf->ptr, data, t.size() * sizeof(float));
+        } else if (dt == DType::BF16) {
+            std::vector<uint16_t> v(t.size());
+            for (size_t i = 0; i < v.size(); ++i) v[i] = f32_to_bf16(data[i]);
+            B::h2d(t.buf->ptr, v.data(), v.size() * 2);
+        } else {
+            throw Error(ErrKind::UnsupportedDType, "from_host: needs a float dtype");
+        }
         return t;
     }
     static T share_buffer(const T& s) {                                             // creation.rs:86-102
@@ -248,49 +302,68 @@ struct Tensor {
     std::vector<float> to_vec() const {                                            // logical order
         T c = contiguous();
         std::vector<float> out(c.size());
+        if (!c.size()) return out;
+        const size_t esz = dtype_size(c.dtype);
+        const char* src = (const char*)c.buf->ptr + c.offset() * esz;
         if (c.dtype == DType::F32) {
-            if (c.size()) B::d2h(out.data(), (const char*)c.buf->ptr + c.offset() * 4, c.size() * 4);
+            B::d2h(out.data(), src, c.size() * 4);
+        } else if (c.dtype == DType::BF16) {
+            std::vector<uint16_t> raw(c.size());
+            B::d2h(raw.data(), src, c.size() * 2);
+            for (size_t i = 0; i < raw.size(); ++i) out[i] = bf16_to_f32(raw[i]);
         } else {
             std::vector<uint8_t> raw(c.size());
-            if (c.size()) B::d2h(raw.data(), (const char*)c.buf->ptr + c.offset(), c.size());
+            B::d2h(raw.data(), src, c.size());
             for (size_t i = 0; i < raw.size(); ++i) out[i] = raw[i] ? 1.0f : 0.0f;
         }
         return out;
     }
     float item() const {                                                            // buffer/mod.rs:596-614
         if (size() != 1) throw Error(ErrKind::InvalidShape, "item() needs a tensor with one element");
-        float v;
-        B::d2h(&v, (const char*)buf->ptr + offset() * 4, 4);
-        return v;
+        if (dtype == DType::F32) {
+            float v;
+            B::d2h(&v, (const char*)buf->ptr + offset() * 4, 4);
+            return v;
+        }
+        if (dtype == DType::BF16) {
+            uint16_t v;
+            B::d2h(&v, (const char*)buf->ptr + offset() * 2, 2);
+            return bf16_to_f32(v);
+        }
+        throw Error(ErrKind::UnsupportedDType, "item() of a bool tensor");
     }
 
     // -- grad plumbing (wt.rs:92-104, lib.rs:213-285) --
     void with_grad() {
-        if (dtype != DType::F32) throw Error(ErrKind::UnsupportedDType, "with_grad needs a float tensor");
+        if (!is_float(dtype)) throw Error(ErrKind::UnsupportedDType, "with_grad needs a float tensor");
         requires_grad = true;
         if (!grad_cell) {
             grad_cell = std::make_shared<GradCell<B>>();
             grad_cell->shape = shape();
+            grad_cell->dtype = dtype;
         }
     }
     bool has_grad() const { return (bool)grad_cell; }
     T grad() const {
         if (!has_grad()) throw Error(ErrKind::InvalidOperation, "tensor has no grad");
-        if (!grad_cell->g) grad_cell->g = std::make_shared<T>(zeros(grad_cell->shape));
+        if (!grad_cell->g) grad_cell->g = std::make_shared<T>(zeros(grad_cell->shape, grad_cell->dtype));
         return *grad_cell->g;
     }
     void accumulate_grad(const T& g) const {                                        // lib.rs:221-241
         if (!has_grad()) return;
-        if (!grad_cell->g && g.dtype == DType::F32 && g.is_contiguous() && g.shape() == grad_cell->shape) {
-            T fresh = empty(grad_cell->shape);
+        if (!grad_cell->g && g.dtype == grad_cell->dtype && g.is_contiguous() && g.shape() == grad_cell->shape) {
+            T fresh = empty(grad_cell->shape, g.dtype);
             auto md = meta_to_shape(g, g.shape());
-            B::sum_to_shape(g.size(), g.ndim(), md.data(), g.f32(), fresh.f32());      // fresh = 0 + g
+            by_dtype(g.dtype, "accumulate_grad", [&](auto tag) {
+                using E = typename decltype(tag)::type;
+                K<E>::sum_to_shape(g.size(), g.ndim(), md.data(), g.template p<E>(), fresh.template p<E>());      // fresh = 0 + g
+            });
             ++backend_calls();
             B::check();
             grad_cell->g = std::make_shared<T>(fresh);
             return;
         }
-        if (!grad_cell->g) grad_cell->g = std::make_shared<T>(zeros(grad_cell->shape));
+        if (!grad_cell->g) grad_cell->g = std::make_shared<T>(zeros(grad_cell->shape, grad_cell->dtype));
         grad_cell->g->add_(g);
     }
     T detach() const {                                                              // f.rs:67-73
@@ -372,7 +445,6 @@ struct Tensor {
     }
 
     // -- binary ops (ops/binary.rs:11-215) --
-    using BinFn = void (*)(size_t, size_t, const size_t*, const float*, const float*, float*);
     static std::pair<T, T> broadcast_tensors(const T& a, const T& b) {              // utils/broadcast.rs:4-31
         size_t an = a.ndim(), bn = b.ndim(), on = std::max(an, bn);
         Shape out(on);
@@ -383,22 +455,26 @@ struct Tensor {
         }
         return {a.broadcast(out), b.broadcast(out)};
     }
-    T binary_forward(const T& rhs_in, BinFn fn, T& lhs_b, T& rhs_b) const {
-        need_f32("binary op");
-        rhs_in.need_f32("binary op");
-        auto pr = broadcast_tensors(*this, rhs_in);
+    // promote both sides to the common dtype, broadcast, run the kernel (ops/binary.rs:17-44)
+    T binary_forward(const T& rhs_in, BinOp op, T& lhs_b, T& rhs_b) const {
+        if (!is_float(dtype) || !is_float(rhs_in.dtype)) throw Error(ErrKind::UnsupportedDType, "binary op: needs float tensors");
+        const DType dt = promoted(dtype, rhs_in.dtype);
+        auto pr = broadcast_tensors(to_dtype(dt), rhs_in.to_dtype(dt));
         lhs_b = pr.first;
         rhs_b = pr.second;
-        T result = empty(lhs_b.shape());
+        T result = empty(lhs_b.shape(), dt);
         auto md = meta_binary(lhs_b, rhs_b);
-        fn(lhs_b.size(), lhs_b.ndim(), md.data(), lhs_b.f32(), rhs_b.f32(), result.f32());
+        by_dtype(dt, "binary op", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::bin[op](lhs_b.size(), lhs_b.ndim(), md.data(), lhs_b.template p<E>(), rhs_b.template p<E>(), result.template p<E>());
+        });
         ++backend_calls();
         B::check();
         return result;
     }
     T add(const T& rhs) const {                                                     // ops/binary.rs:11-60
         T l, r;
-        T result = binary_forward(rhs, B::add, l, r);
+        T result = binary_forward(rhs, ADD, l, r);
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
@@ -410,7 +486,7 @@ struct Tensor {
     }
     T sub(const T& rhs) const {                                                     // ops/binary.rs:62-111
         T l, r;
-        T result = binary_forward(rhs, B::sub, l, r);
+        T result = binary_forward(rhs, SUB, l, r);
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
@@ -422,7 +498,7 @@ struct Tensor {
     }
     T mul(const T& rhs) const {                                                     // ops/binary.rs:113-164
         T l, r;
-        T result = binary_forward(rhs, B::mul, l, r);
+        T result = binary_forward(rhs, MUL, l, r);
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
@@ -434,7 +510,7 @@ struct Tensor {
     }
     T div(const T& rhs) const {                                                     // ops/binary.rs:166-222
         T l, r;
-        T result = binary_forward(rhs, B::div, l, r);
+        T result = binary_forward(rhs, DIV, l, r);
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
@@ -444,41 +520,49 @@ struct Tensor {
         }
         return result;
     }
-    using InplaceFn = void (*)(size_t, size_t, const size_t*, float*, const float*);
-    void inplace(const T& rhs_in, InplaceFn fn) {                                   // ops/binary.rs:653-700
-        need_f32("in-place op");
+    void inplace(const T& rhs_in, InplaceOp op) {                                   // ops/binary.rs:653-700
         T rhs = shape() == rhs_in.shape() ? rhs_in : rhs_in.broadcast(shape());
+        if (rhs.dtype != dtype) rhs = rhs.to_dtype(dtype);                          // binary.rs:660-662
         auto md = meta_binary(*this, rhs);
-        fn(size(), ndim(), md.data(), f32(), rhs.f32());
+        by_dtype(dtype, "in-place op", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::inplace[op](size(), ndim(), md.data(), this->template p<E>(), rhs.template p<E>());
+        });
         ++backend_calls();
         B::check();
     }
-    void add_(const T& rhs) { inplace(rhs, B::add_inplace); }
-    void sub_(const T& rhs) { inplace(rhs, B::sub_inplace); }
+    void add_(const T& rhs) { inplace(rhs, ADD_INPLACE); }
+    void sub_(const T& rhs) { inplace(rhs, SUB_INPLACE); }
 
     // -- unary ops (ops/unary.rs) --
-    using UnFn = void (*)(size_t, size_t, const size_t*, const float*, float*);
-    using UnCFn = void (*)(size_t, size_t, const size_t*, const float*, float, float*);
-    T unary_forward(UnFn fn) const {
-        need_f32("unary op");
-        T result = empty(shape());
+    T unary_forward(UnOp op) const {
+        T result = empty(shape(), dtype);
         auto md = meta_unary(*this);
-        fn(size(), ndim(), md.data(), f32(), result.f32());
+        by_dtype(dtype, "unary op", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::un[op](size(), ndim(), md.data(), this->template p<E>(), result.template p<E>());
+        });
         ++backend_calls();
         B::check();
         return result;
     }
-    T unary_c_forward(UnCFn fn, float c) const {
-        need_f32("unary op");
-        T result = empty(shape());
-        auto md = meta_unary(*this);
-        fn(size(), ndim(), md.data(), f32(), c, result.f32());
+    // `target` is the dtype the reference promotes the tensor to before the kernel runs
+    T unary_c_forward(UncOp op, float c, DType target) const {
+        if (!is_float(dtype)) throw Error(ErrKind::UnsupportedDType, "scalar op: needs a float tensor");
+        T input = to_dtype(target);
+        T result = empty(shape(), target);
+        auto md = meta_unary(input);
+        by_dtype(target, "scalar op", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::unc[op](input.size(), input.ndim(), md.data(), input.template p<E>(), scalar_as<E>(c), result.template p<E>());
+        });
         ++backend_calls();
         B::check();
         return result;
     }
+    DType scalar_target(float c) const { return integer_valued(c) ? dtype : DType::F32; }
     T neg() const {                                                                 // ops/unary.rs:8-43
-        T result = unary_forward(B::neg);
+        T result = unary_forward(NEG);
         if (requires_grad) {
             result.with_grad();
             result.set_node("neg", {*this}, [](const std::vector<T>&, const T& go) { return std::vector<T>{go.neg()}; });
@@ -486,7 +570,7 @@ struct Tensor {
         return result;
     }
     T square() const {                                                              // ops/unary.rs:112-147
-        T result = unary_forward(B::square);
+        T result = unary_forward(SQUARE);
         if (requires_grad) {
             result.with_grad();
             T input = *this;
@@ -497,18 +581,18 @@ struct Tensor {
         return result;
     }
     T relu() const {                                                                // ops/unary.rs:186-222
-        T result = unary_forward(B::relu);
+        T result = unary_forward(RELU);
         if (requires_grad) {
             result.with_grad();
             T input = *this;
             result.set_node("relu", {*this}, [input](const std::vector<T>&, const T& go) {
-                return std::vector<T>{go.mul(input.gt_scalar(0.0f).to_f32())};
+                return std::vector<T>{go.mul(input.gt_scalar(0.0f).to_dtype(input.dtype))};
             });
         }
         return result;
     }
     T tanh() const {                                                                // ops/unary.rs:261-296
-        T result = unary_forward(B::tanh);
+        T result = unary_forward(TANH);
         if (requires_grad) {
             result.with_grad();
             T output = result;
@@ -519,7 +603,7 @@ struct Tensor {
         return result;
     }
     T gelu() const {                                                                // ops/unary.rs:298-351
-        T result = unary_forward(B::gelu);
+        T result = unary_forward(GELU);
         if (requires_grad) {
             result.with_grad();
             T input = *this;
@@ -539,7 +623,7 @@ struct Tensor {
         return result;
     }
     T exp() const {                                                                 // ops/unary.rs:583-618
-        T result = unary_forward(B::exp);
+        T result = unary_forward(EXP);
         if (requires_grad) {
             result.with_grad();
             T output = result;
@@ -548,7 +632,7 @@ struct Tensor {
         return result;
     }
     T add_scalar(float c) const {                                                   // ops/unary.rs:794-830
-        T result = unary_c_forward(B::add_scalar, c);
+        T result = unary_c_forward(ADD_SCALAR, c, scalar_target(c));
         if (requires_grad) {
             result.with_grad();
             result.set_node("add_scalar", {*this}, [](const std::vector<T>&, const T& go) { return std::vector<T>{go}; });
@@ -556,7 +640,7 @@ struct Tensor {
         return result;
     }
     T mul_scalar(float c) const {                                                   // ops/unary.rs:870-907
-        T result = unary_c_forward(B::mul_scalar, c);
+        T result = unary_c_forward(MUL_SCALAR, c, scalar_target(c));
         if (requires_grad) {
             result.with_grad();
             result.set_node("mul_scalar", {*this}, [c](const std::vector<T>&, const T& go) { return std::vector<T>{go.mul_scalar(c)}; });
@@ -564,7 +648,7 @@ struct Tensor {
         return result;
     }
     T div_scalar(float c) const {                                                   // ops/unary.rs:909-946
-        T result = unary_c_forward(B::div_scalar, c);
+        T result = unary_c_forward(DIV_SCALAR, c, dtype);
         if (requires_grad) {
             result.with_grad();
             result.set_node("div_scalar", {*this}, [c](const std::vector<T>&, const T& go) { return std::vector<T>{go.div_scalar(c)}; });
@@ -572,7 +656,7 @@ struct Tensor {
         return result;
     }
     T pow(float e) const {                                                          // ops/unary.rs:1042-1082
-        T result = unary_c_forward(B::pow, e);
+        T result = unary_c_forward(POW, e, scalar_target(e));
         if (requires_grad) {
             result.with_grad();
             T input = *this;
@@ -583,39 +667,50 @@ struct Tensor {
         return result;
     }
     T gt_scalar(float c) const {                                                    // ops/unary.rs:1264-1284 (bool result, no grad)
-        need_f32("gt_scalar");
         T result = empty(shape(), DType::BOOL);
         auto md = meta_unary(*this);
-        B::gt_scalar(size(), ndim(), md.data(), f32(), c, (uint8_t*)result.buf->ptr);
+        by_dtype(dtype, "gt_scalar", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::gt_scalar(size(), ndim(), md.data(), this->template p<E>(), scalar_as<E>(c), (uint8_t*)result.buf->ptr);
+        });
         ++backend_calls();
         B::check();
         return result;
     }
-    T to_f32() const {                                                              // wt.rs:65-90 (bool -> f32 keeps the layout)
-        if (dtype == DType::F32) return *this;
-        T r;
-        r.layout = layout;
-        r.dtype = DType::F32;
-        r.buf = std::make_shared<Storage<B>>(buf->len, DType::F32);
-        B::cast_bool_f32(buf->len, (const uint8_t*)buf->ptr, r.f32());
+    // with_dtype (wt.rs:65-84): the whole buffer is converted, the layout stays; a clone of the tensor otherwise
+    // (promote_tensor, utils/promotion.rs:62-73), so requires_grad, the gradient and the node travel with it
+    T to_dtype(DType target) const {
+        if (dtype == target) return *this;
+        T r = *this;
+        r.dtype = target;
+        r.buf = std::make_shared<Storage<B>>(buf->len, target);
+        const size_t n = buf->len;
+        if (dtype == DType::BOOL && target == DType::F32) K<float>::cast_from_bool(n, (const uint8_t*)buf->ptr, r.template p<float>());
+        else if (dtype == DType::BOOL && target == DType::BF16) K<uint16_t>::cast_from_bool(n, (const uint8_t*)buf->ptr, r.template p<uint16_t>());
+        else if (dtype == DType::BF16 && target == DType::F32) B::cast_bf16_f32(n, p<uint16_t>(), r.template p<float>());
+        else if (dtype == DType::F32 && target == DType::BF16) B::cast_f32_bf16(n, p<float>(), r.template p<uint16_t>());
+        else throw Error(ErrKind::UnsupportedDType, "to_dtype: unsupported conversion");
+        ++cast_calls();
+        B::check();
         return r;
     }
 
     // -- reductions (ops/reduction.rs) --
-    using RedFn = void (*)(size_t, size_t, size_t, const size_t*, const float*, float*);
     size_t norm_dim(int dim, size_t nd, bool allow_end = false) const {
         long d = dim < 0 ? (long)nd + dim : dim;
         if (d < 0 || (size_t)d >= nd + (allow_end ? 1 : 0))
             throw Error(ErrKind::DimensionOutOfBounds, "dimension " + std::to_string(dim) + " out of bounds for " + std::to_string(nd) + " dims");
         return (size_t)d;
     }
-    T reduce_forward(RedFn fn, size_t dim, bool keep_dim) const {
-        need_f32("reduction");
+    T reduce_forward(RedOp op, size_t dim, bool keep_dim) const {
         Shape out = shape();
         out.erase(out.begin() + dim);
-        T result = empty(out);       // the reference zero-fills first (reduction.rs:28); the kernels write every output
+        T result = empty(out, dtype);       // the reference zero-fills first (reduction.rs:28); the kernels write every output
         auto md = meta_reduce(*this, dim);
-        fn(size(), ndim(), 1, md.data(), f32(), result.f32());
+        by_dtype(dtype, "reduction", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::red[op](size(), ndim(), 1, md.data(), this->template p<E>(), result.template p<E>());
+        });
         ++backend_calls();
         B::check();
         if (keep_dim) {
@@ -627,7 +722,7 @@ struct Tensor {
     }
     T sum(int dim_in, bool keep_dim) const {                                        // ops/reduction.rs:9-74
         size_t dim = norm_dim(dim_in, ndim());
-        T result = reduce_forward(B::sum, dim, keep_dim);
+        T result = reduce_forward(SUM, dim, keep_dim);
         if (requires_grad) {
             result.with_grad();
             Shape in_shape = shape();
@@ -658,10 +753,12 @@ struct Tensor {
             if (target[i] == 0 || shape()[i] % target[i] != 0)
                 throw Error(ErrKind::ShapeMismatch, "Dimension " + std::to_string(i) + " is not divisible: " + std::to_string(shape()[i]) +
                                                         " -> " + std::to_string(target[i]));
-        need_f32("sum_to_shape");
-        T result = empty(target);    // zero-filled in the reference (reduction.rs:112); fully written by the kernel
+        T result = empty(target, dtype);    // zero-filled in the reference (reduction.rs:112); fully written by the kernel
         auto md = meta_to_shape(*this, target);
-        B::sum_to_shape(size(), ndim(), md.data(), f32(), result.f32());
+        by_dtype(dtype, "sum_to_shape", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::sum_to_shape(size(), ndim(), md.data(), this->template p<E>(), result.template p<E>());
+        });
         ++backend_calls();
         B::check();
         if (requires_grad) {
@@ -673,7 +770,7 @@ struct Tensor {
     }
     T mean(int dim_in, bool keep_dim) const {                                       // ops/reduction.rs:145-216
         size_t dim = norm_dim(dim_in, ndim());
-        T result = reduce_forward(B::mean, dim, keep_dim);
+        T result = reduce_forward(MEAN, dim, keep_dim);
         if (requires_grad) {
             result.with_grad();
             Shape in_shape = shape();
@@ -788,9 +885,11 @@ struct Tensor {
         return broadcast(ns);
     }
     T broadcast_scalar_to(const Shape& target) const {                              // ops/transform.rs:328-349
-        need_f32("broadcast");
-        T result = empty(target);
-        B::broadcast_scalar_f32(result.size(), f32() + offset(), result.f32());     // the reference: item() + host fill
+        T result = empty(target, dtype);
+        by_dtype(dtype, "broadcast", [&](auto tag) {                                // the reference: item() + host fill
+            using E = typename decltype(tag)::type;
+            K<E>::broadcast_scalar(result.size(), this->template p<E>() + offset(), result.template p<E>());
+        });
         if (requires_grad) {
             result.with_grad();
             result.set_node("broadcast_scalar", {*this}, [](const std::vector<T>&, const T& go) { return std::vector<T>{go.sum_all()}; });
@@ -800,13 +899,12 @@ struct Tensor {
     T contiguous() const {                                                          // f.rs:11-41
         if (is_contiguous()) return *this;
         T result = empty(shape(), dtype);
-        if (dtype == DType::F32) {
-            auto md = meta_unary(*this);
-            B::copy_strided_f32(size(), ndim(), md.data(), f32(), result.f32());
-        } else {
-            // bool tensors only come out of comparisons and are contiguous there
-            throw Error(ErrKind::UnsupportedDType, "contiguous() of a strided bool tensor");
-        }
+        auto md = meta_unary(*this);
+        // bool tensors only come out of comparisons and are contiguous there
+        by_dtype(dtype, "contiguous", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::copy_strided(size(), ndim(), md.data(), this->template p<E>(), result.template p<E>());
+        });
         return result;
     }
     T reshape(const std::vector<long>& req) const {                                 // ops/transform.rs:353-388
@@ -868,14 +966,17 @@ struct Tensor {
         return {ae.broadcast(as), be.broadcast(bs)};
     }
     T matmul(const T& rhs_in) const {
-        need_f32("matmul");
-        rhs_in.need_f32("matmul");
+        if (!is_float(dtype) || !is_float(rhs_in.dtype)) throw Error(ErrKind::UnsupportedDType, "matmul: needs float tensors");
+        const DType dt = promoted(dtype, rhs_in.dtype);                              // ops/matmul.rs:18-30
         size_t ln = ndim(), rn = rhs_in.ndim();
-        auto pr = unify_matmul_shapes(*this, rhs_in);
+        auto pr = unify_matmul_shapes(to_dtype(dt), rhs_in.to_dtype(dt));
         const T &lhs = pr.first, &rhs = pr.second;
         auto mm = meta_matmul(lhs, rhs);
-        T result = empty(mm.second);
-        B::matmul(result.size(), mm.first.data(), lhs.f32(), rhs.f32(), result.f32());
+        T result = empty(mm.second, dt);
+        by_dtype(dt, "matmul", [&](auto tag) {
+            using E = typename decltype(tag)::type;
+            K<E>::matmul(result.size(), mm.first.data(), lhs.template p<E>(), rhs.template p<E>(), result.template p<E>());
+        });
         ++backend_calls();
         B::check();
         if (ln == 1 && rn == 1) result = result.squeeze_all();
@@ -883,14 +984,20 @@ struct Tensor {
         else if (ln >= 2 && rn == 1) { int d = (int)result.ndim() - 1; if (result.shape()[d] == 1) result = result.squeeze(d); }
         if (requires_grad || rhs.requires_grad) {
             result.with_grad();
-            result.set_node("matmul", {*this, rhs_in}, [](const std::vector<T>& in, const T& go) {     // ops/matmul.rs:63-146
-                const T &l = in[0], &r = in[1];
+            result.set_node("matmul", {*this, rhs_in}, [](const std::vector<T>& in, const T& go_in) {     // ops/matmul.rs:63-146
+                const DType dt = promoted(promoted(in[0].dtype, in[1].dtype), go_in.dtype);
+                const T l = in[0].to_dtype(dt), r = in[1].to_dtype(dt), go = go_in.to_dtype(dt);
                 auto mm = meta_matmul(l, r);
-                T gl = empty(l.shape()), gr = empty(r.shape());     // zeros_like in the reference; both are fully written
-                B::matmul_backward(gl.size(), gr.size(), mm.first.data(), go.f32(), l.f32(), r.f32(), gl.f32(), gr.f32());
+                T gl = empty(l.shape(), dt), gr = empty(r.shape(), dt);     // zeros_like in the reference; both are fully written
+                by_dtype(dt, "matmul backward", [&](auto tag) {
+                    using E = typename decltype(tag)::type;
+                    K<E>::matmul_backward(gl.size(), gr.size(), mm.first.data(), go.template p<E>(), l.template p<E>(), r.template p<E>(),
+                                          gl.template p<E>(), gr.template p<E>());
+                });
                 ++backend_calls();
                 B::check();
-                return std::vector<T>{gl, gr};      // zeros_like already has the inputs' shapes: no reshape branch is reached
+                // the gradients go back in the inputs' own dtypes (matmul.rs:137-143)
+                return std::vector<T>{gl.to_dtype(in[0].dtype), gr.to_dtype(in[1].dtype)};
             });
         }
         return result;

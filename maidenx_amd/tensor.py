@@ -17,6 +17,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 HOST_LIB_PATH = os.path.join(_HERE, "libmaidenx_host.so")
 
+DTYPES = ["f32", "bf16", "bool"]
 _KINDS = ["None", "InvalidShape", "ShapeMismatch", "DimensionOutOfBounds", "IncompatibleShape", "InvalidOperation",
           "InvalidArgument", "UnsupportedDType", "OutOfMemory", "Backend"]
 
@@ -31,7 +32,8 @@ def _bind(lib):
     P, SZ, I, F = C.c_void_p, C.c_size_t, C.c_int, C.c_float
     sig = {
         "mxt_last_error": ([C.c_char_p, SZ], I), "mxt_backend_name": ([], C.c_char_p),
-        "mxt_new": ([P, P, SZ], P), "mxt_fill": ([P, SZ, F], P), "mxt_randn": ([P, SZ, C.c_uint64], P), "mxt_release": ([P], None),
+        "mxt_new": ([P, P, SZ], P), "mxt_fill": ([P, SZ, F], P), "mxt_new_dtype": ([P, P, SZ, I], P), "mxt_fill_dtype": ([P, SZ, F, I], P),
+        "mxt_dtype": ([P], I), "mxt_to_dtype": ([P, I], P), "mxt_cast_calls": ([], SZ), "mxt_randn": ([P, SZ, C.c_uint64], P), "mxt_release": ([P], None),
         "mxt_ndim": ([P], SZ), "mxt_size": ([P], SZ), "mxt_offset": ([P], SZ), "mxt_shape": ([P, P], None), "mxt_strides": ([P, P], None),
         "mxt_requires_grad": ([P], I), "mxt_is_contiguous": ([P], I), "mxt_to_host": ([P, P], I),
         "mxt_with_grad": ([P], I), "mxt_grad": ([P], P), "mxt_backward": ([P], I), "mxt_zero_grad": ([P], I), "mxt_detach": ([P], P),
@@ -75,21 +77,22 @@ class Host:
             self._raise()
 
     # -- creation --
-    def tensor(self, data, shape=None):
+    def tensor(self, data, shape=None, dtype="f32"):
+        """f32 values stored as `dtype` ("f32" or "bf16", rounded to nearest even)."""
         a = np.ascontiguousarray(data, dtype=np.float32)
         shp = tuple(a.shape if shape is None else shape)
         s = (C.c_size_t * max(1, len(shp)))(*shp)
-        return self._t(self.lib.mxt_new(a.ctypes.data, s, len(shp)))
+        return self._t(self.lib.mxt_new_dtype(a.ctypes.data, s, len(shp), DTYPES.index(dtype)))
 
-    def fill(self, shape, value):
+    def fill(self, shape, value, dtype="f32"):
         s = (C.c_size_t * max(1, len(shape)))(*shape)
-        return self._t(self.lib.mxt_fill(s, len(shape), float(value)))
+        return self._t(self.lib.mxt_fill_dtype(s, len(shape), float(value), DTYPES.index(dtype)))
 
-    def zeros(self, shape):
-        return self.fill(shape, 0.0)
+    def zeros(self, shape, dtype="f32"):
+        return self.fill(shape, 0.0, dtype)
 
-    def ones(self, shape):
-        return self.fill(shape, 1.0)
+    def ones(self, shape, dtype="f32"):
+        return self.fill(shape, 1.0, dtype)
 
     def randn(self, shape, seed):
         s = (C.c_size_t * max(1, len(shape)))(*shape)
@@ -130,6 +133,9 @@ class Host:
     def backend_calls(self):
         return self.lib.mxt_backend_calls()
 
+    def cast_calls(self):
+        return self.lib.mxt_cast_calls()
+
     def reset_backend_calls(self):
         self.lib.mxt_reset_backend_calls()
 
@@ -164,6 +170,13 @@ class Tensor:
         out = (C.c_size_t * max(1, n))()
         self.m.lib.mxt_strides(self.h, out)
         return tuple(out[:n])
+
+    @property
+    def dtype(self):
+        return DTYPES[self.m.lib.mxt_dtype(self.h)]
+
+    def to_dtype(self, dtype):
+        return self.m._t(self.m.lib.mxt_to_dtype(self.h, DTYPES.index(dtype)))
 
     @property
     def offset(self):

@@ -7,20 +7,31 @@
 #include "../maidenx_amd/host/mx_tensor.hpp"
 
 extern "C" {
-#define ORC_BIN(N) void oracle_##N##_f32(size_t, size_t, const size_t*, const float*, const float*, float*);
-ORC_BIN(add) ORC_BIN(sub) ORC_BIN(mul) ORC_BIN(div)
-void oracle_add_inplace_f32(size_t, size_t, const size_t*, float*, const float*);
-void oracle_sub_inplace_f32(size_t, size_t, const size_t*, float*, const float*);
-#define ORC_UN(N) void oracle_##N##_f32(size_t, size_t, const size_t*, const float*, float*);
-ORC_UN(neg) ORC_UN(square) ORC_UN(relu) ORC_UN(tanh) ORC_UN(gelu) ORC_UN(exp)
-#define ORC_UNC(N) void oracle_##N##_f32(size_t, size_t, const size_t*, const float*, float, float*);
-ORC_UNC(add_scalar) ORC_UNC(mul_scalar) ORC_UNC(div_scalar) ORC_UNC(pow)
-void oracle_gt_scalar_f32(size_t, size_t, const size_t*, const float*, float, uint8_t*);
-void oracle_sum_f32(size_t, size_t, size_t, const size_t*, const float*, float*);
-void oracle_mean_f32(size_t, size_t, size_t, const size_t*, const float*, float*);
-void oracle_sum_to_shape_f32(size_t, size_t, const size_t*, const float*, float*);
-void oracle_matmul_f32(size_t, const size_t*, const float*, const float*, float*);
-void oracle_matmul_backward_f32(size_t, size_t, const size_t*, const float*, const float*, const float*, float*, float*);
+#define ORC_DECL(E, S)                                                                                             \
+    void oracle_add_##S(size_t, size_t, const size_t*, const E*, const E*, E*);                                     \
+    void oracle_sub_##S(size_t, size_t, const size_t*, const E*, const E*, E*);                                     \
+    void oracle_mul_##S(size_t, size_t, const size_t*, const E*, const E*, E*);                                     \
+    void oracle_div_##S(size_t, size_t, const size_t*, const E*, const E*, E*);                                     \
+    void oracle_add_inplace_##S(size_t, size_t, const size_t*, E*, const E*);                                       \
+    void oracle_sub_inplace_##S(size_t, size_t, const size_t*, E*, const E*);                                       \
+    void oracle_neg_##S(size_t, size_t, const size_t*, const E*, E*);                                               \
+    void oracle_square_##S(size_t, size_t, const size_t*, const E*, E*);                                            \
+    void oracle_relu_##S(size_t, size_t, const size_t*, const E*, E*);                                              \
+    void oracle_tanh_##S(size_t, size_t, const size_t*, const E*, E*);                                              \
+    void oracle_gelu_##S(size_t, size_t, const size_t*, const E*, E*);                                              \
+    void oracle_exp_##S(size_t, size_t, const size_t*, const E*, E*);                                               \
+    void oracle_add_scalar_##S(size_t, size_t, const size_t*, const E*, E, E*);                                     \
+    void oracle_mul_scalar_##S(size_t, size_t, const size_t*, const E*, E, E*);                                     \
+    void oracle_div_scalar_##S(size_t, size_t, const size_t*, const E*, E, E*);                                     \
+    void oracle_pow_##S(size_t, size_t, const size_t*, const E*, E, E*);                                            \
+    void oracle_gt_scalar_##S(size_t, size_t, const size_t*, const E*, E, uint8_t*);                                \
+    void oracle_sum_##S(size_t, size_t, size_t, const size_t*, const E*, E*);                                       \
+    void oracle_mean_##S(size_t, size_t, size_t, const size_t*, const E*, E*);                                      \
+    void oracle_sum_to_shape_##S(size_t, size_t, const size_t*, const E*, E*);                                      \
+    void oracle_matmul_##S(size_t, const size_t*, const E*, const E*, E*);                                          \
+    void oracle_matmul_backward_##S(size_t, size_t, const size_t*, const E*, const E*, const E*, E*, E*);
+ORC_DECL(float, f32)
+ORC_DECL(uint16_t, bf16)     // the oracle's bf16 is a struct of one uint16_t: the same bits at this boundary
 void oracle_conv2d_im2col_f32(size_t, const size_t*, const float*, float*);
 void oracle_conv2d_col2im_f32(size_t, const size_t*, const float*, float*);
 }
@@ -34,47 +45,51 @@ struct OracleBackend {
     static void d2h(void* d, const void* s, size_t n) { std::memcpy(d, s, n); }
     static void check() {}
     static constexpr bool has_graphs = false;
-    // The reference does these on the host as well.
-    static void fill_f32(size_t n, float* p, float v) { for (size_t i = 0; i < n; ++i) p[i] = v; }              // creation.rs:144-164, 253-305
-    static void cast_bool_f32(size_t n, const uint8_t* in, float* out) { for (size_t i = 0; i < n; ++i) out[i] = in[i] ? 1.0f : 0.0f; }
-    // crates/maidenx_tensor/src/f.rs:19-24: element by element through the logical index
-    static void copy_strided_f32(size_t n, size_t nd, const size_t* md, const float* in, float* out) {
-        const size_t *dims = md, *strides = md + nd;
-        const size_t off = md[2 * nd];
-        for (size_t i = 0; i < n; ++i) {
-            size_t rem = i, src = off;
-            for (size_t d = nd; d-- > 0;) {
-                src += (rem % dims[d]) * strides[d];
-                rem /= dims[d];
-            }
-            out[i] = in[src];
-        }
-    }
-    static void broadcast_scalar_f32(size_t n, const float* src, float* dst) { fill_f32(n, dst, *src); }        // transform.rs:328-331
-    static constexpr auto add = &oracle_add_f32;
-    static constexpr auto sub = &oracle_sub_f32;
-    static constexpr auto mul = &oracle_mul_f32;
-    static constexpr auto div = &oracle_div_f32;
-    static constexpr auto add_inplace = &oracle_add_inplace_f32;
-    static constexpr auto sub_inplace = &oracle_sub_inplace_f32;
-    static constexpr auto neg = &oracle_neg_f32;
-    static constexpr auto square = &oracle_square_f32;
-    static constexpr auto relu = &oracle_relu_f32;
-    static constexpr auto tanh = &oracle_tanh_f32;
-    static constexpr auto gelu = &oracle_gelu_f32;
-    static constexpr auto exp = &oracle_exp_f32;
-    static constexpr auto add_scalar = &oracle_add_scalar_f32;
-    static constexpr auto mul_scalar = &oracle_mul_scalar_f32;
-    static constexpr auto div_scalar = &oracle_div_scalar_f32;
-    static constexpr auto pow = &oracle_pow_f32;
-    static constexpr auto gt_scalar = &oracle_gt_scalar_f32;
-    static constexpr auto sum = &oracle_sum_f32;
-    static constexpr auto mean = &oracle_mean_f32;
-    static constexpr auto sum_to_shape = &oracle_sum_to_shape_f32;
-    static constexpr auto matmul = &oracle_matmul_f32;
-    static constexpr auto matmul_backward = &oracle_matmul_backward_f32;
     static constexpr auto im2col = &oracle_conv2d_im2col_f32;
     static constexpr auto col2im = &oracle_conv2d_col2im_f32;
+    // with_dtype on the host, element by element, as the reference does (crates/maidenx_core/src/buffer/mod.rs:155-196)
+    static void cast_bf16_f32(size_t n, const uint16_t* in, float* out) { for (size_t i = 0; i < n; ++i) out[i] = mxt::bf16_to_f32(in[i]); }
+    static void cast_f32_bf16(size_t n, const float* in, uint16_t* out) { for (size_t i = 0; i < n; ++i) out[i] = mxt::f32_to_bf16(in[i]); }
+    template <class E> struct K;
 };
+template <class E> inline E orc_one();
+template <> inline float orc_one<float>() { return 1.0f; }
+template <> inline uint16_t orc_one<uint16_t>() { return 0x3F80; }
+#define MXT_ORC_KERNELS(E, S)                                                                                          \
+    template <> struct OracleBackend::K<E> {                                                                             \
+        using Bin = void (*)(size_t, size_t, const size_t*, const E*, const E*, E*);                                     \
+        using Inp = void (*)(size_t, size_t, const size_t*, E*, const E*);                                               \
+        using Un = void (*)(size_t, size_t, const size_t*, const E*, E*);                                                \
+        using Unc = void (*)(size_t, size_t, const size_t*, const E*, E, E*);                                            \
+        using Red = void (*)(size_t, size_t, size_t, const size_t*, const E*, E*);                                       \
+        static constexpr Bin bin[4] = {&oracle_add_##S, &oracle_sub_##S, &oracle_mul_##S, &oracle_div_##S};              \
+        static constexpr Inp inplace[2] = {&oracle_add_inplace_##S, &oracle_sub_inplace_##S};                            \
+        static constexpr Un un[6] = {&oracle_neg_##S, &oracle_square_##S, &oracle_relu_##S, &oracle_tanh_##S, &oracle_gelu_##S, &oracle_exp_##S}; \
+        static constexpr Unc unc[4] = {&oracle_add_scalar_##S, &oracle_mul_scalar_##S, &oracle_div_scalar_##S, &oracle_pow_##S}; \
+        static constexpr Red red[2] = {&oracle_sum_##S, &oracle_mean_##S};                                               \
+        static constexpr auto gt_scalar = &oracle_gt_scalar_##S;                                                         \
+        static constexpr auto sum_to_shape = &oracle_sum_to_shape_##S;                                                   \
+        static constexpr auto matmul = &oracle_matmul_##S;                                                               \
+        static constexpr auto matmul_backward = &oracle_matmul_backward_##S;                                             \
+        /* The reference does these on the host as well. */                                                             \
+        static void fill(size_t n, E* p, E v) { for (size_t i = 0; i < n; ++i) p[i] = v; }                               \
+        static void cast_from_bool(size_t n, const uint8_t* in, E* out) { for (size_t i = 0; i < n; ++i) out[i] = in[i] ? orc_one<E>() : E(0); } \
+        /* crates/maidenx_tensor/src/f.rs:19-24: element by element through the logical index */                        \
+        static void copy_strided(size_t n, size_t nd, const size_t* md, const E* in, E* out) {                           \
+            const size_t *dims = md, *strides = md + nd;                                                                 \
+            const size_t off = md[2 * nd];                                                                               \
+            for (size_t i = 0; i < n; ++i) {                                                                             \
+                size_t rem = i, src = off;                                                                               \
+                for (size_t d = nd; d-- > 0;) {                                                                          \
+                    src += (rem % dims[d]) * strides[d];                                                                 \
+                    rem /= dims[d];                                                                                      \
+                }                                                                                                        \
+                out[i] = in[src];                                                                                        \
+            }                                                                                                            \
+        }                                                                                                                \
+        static void broadcast_scalar(size_t n, const E* src, E* dst) { fill(n, dst, *src); } /* transform.rs:328-331 */  \
+    };
+MXT_ORC_KERNELS(float, f32)
+MXT_ORC_KERNELS(uint16_t, bf16)
 using MxtBackend = OracleBackend;
 #include "../maidenx_amd/host/mx_capi.hpp"

@@ -8,11 +8,11 @@ import numpy as np
 TKAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_tensor_kat.json")))["cases"]
 
 
-def run_case(mx, case):
+def run_case(mx, case, dtype="f32"):
     """Returns {name: ndarray} for every named tensor and '<input>.grad'."""
     env = {}
     for name, spec in case["inputs"].items():
-        t = mx.tensor(np.array(spec["data"], np.float32).reshape(spec["shape"]))
+        t = mx.tensor(np.array(spec["data"], np.float32).reshape(spec["shape"]), dtype=dtype)
         if spec.get("grad"):
             t.with_grad()
         env[name] = t
@@ -38,8 +38,8 @@ def run_case(mx, case):
     return res
 
 
-def check_case(res, case):
-    tol = case["tol"]
+def check_case(res, case, tol=None):
+    tol = case["tol"] if tol is None else tol
     for key, exp in case["expect"].items():
         got = np.asarray(res[key], np.float64).ravel()
         exp = np.asarray(exp, np.float64)
@@ -137,3 +137,27 @@ def conv_numpy(x, w, b, stride, pad, target):
     gx = gxp[:, :, pad:pad + H, pad:pad + W]
     gw = (cols.T @ grad_flat).reshape(Cout, Cin, kh, kw)
     return {"out": out, "loss": loss, "grad_x": gx, "grad_w": gw, "grad_b": go.sum((0, 2, 3))}
+
+
+# ---- bf16 helpers and the elementwise forward + backward programs of configs[1] ------------------------
+def bf16_round(a):
+    """float32 values rounded to bf16 (nearest even), returned as float32."""
+    x = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((x + 0x7FFF + ((x >> 16) & 1)) >> 16) << 16
+    return r.astype(np.uint32).view(np.float32).reshape(np.shape(a))
+
+
+def elementwise_program(mx, op, case, dtype, R=12, C=20, seed=5):
+    """z = op(x[, y]); z.backward().  case: contig | bcast (rhs [1,C]) | transposed (x is a transposed view)."""
+    rng = np.random.default_rng(seed)
+    xs = rng.standard_normal((C, R) if case == "transposed" else (R, C)).astype(np.float32)
+    ys = (rng.standard_normal((1, C) if case == "bcast" else (R, C)) + 2.5).astype(np.float32)
+    base = mx.tensor(xs, dtype=dtype).with_grad()
+    x = base.transpose(0, 1) if case == "transposed" else base
+    y = mx.tensor(ys, dtype=dtype).with_grad()
+    z = getattr(x, op)(y) if op in ("add", "mul", "div") else getattr(x, op)()
+    z.backward()
+    out = {"z": z.numpy(), "gx": base.grad().numpy(), "z.dtype": z.dtype, "gx.dtype": base.grad().dtype, "xs": xs, "ys": ys}
+    if op in ("add", "mul", "div"):
+        out["gy"] = y.grad().numpy()
+    return out

@@ -3,7 +3,7 @@ CPU oracle and against the reference's own expectations."""
 import numpy as np
 import pytest
 
-from host_programs import TKAT, check_case, conv_inputs, conv_numpy, conv_step, mlp_numpy, mlp_run, run_case
+from host_programs import TKAT, check_case, conv_inputs, conv_numpy, conv_step, elementwise_program, mlp_numpy, mlp_run, run_case
 from maidenx_amd.tensor import MxError
 
 pytestmark = pytest.mark.gpu
@@ -124,3 +124,30 @@ def test_graph_replayed_training_equals_eager(mx_hip):
             np.testing.assert_array_equal(t.grad().numpy(), 2 * np.arange(12, dtype=np.float32).reshape(3, 4))
     finally:
         mx.set_graph_replay(True)
+
+
+@pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])
+def test_reference_tensor_cases_bf16(mx_hip, case):
+    check_case(run_case(mx_hip, case, dtype="bf16"), case, tol=0.1)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("op", ["add", "mul", "div", "exp", "relu", "gelu"])
+@pytest.mark.parametrize("case", ["contig", "bcast", "transposed"])
+def test_elementwise_forward_backward_matches_oracle(mx_hip, mx_oracle, op, case, dtype):
+    """configs[1] through the tensor API at a small size: forward value and every gradient, both dtypes (the bf16 gelu
+    closure runs mostly in f32 after the reference's promotions).  Elementwise kernels are bit-exact; the broadcast
+    gradient is a column sum (different order) and gets the reduction tolerance."""
+    if op in ("exp", "relu", "gelu") and case == "bcast":
+        pytest.skip("unary ops have no broadcast case")
+    got = elementwise_program(mx_hip, op, case, dtype, R=48, C=72)
+    ref = elementwise_program(mx_oracle, op, case, dtype, R=48, C=72)
+    assert got["z.dtype"] == ref["z.dtype"] and got["gx.dtype"] == ref["gx.dtype"]
+    np.testing.assert_array_equal(got["z"], ref["z"])
+    np.testing.assert_array_equal(got["gx"], ref["gx"])
+    if "gy" in ref:
+        if case == "bcast":
+            tol = 1e-5 if dtype == "f32" else 1e-2
+            assert np.max(np.abs(got["gy"] - ref["gy"])) <= tol * 48 * np.max(np.abs(ref["gy"]) + 1)
+        else:
+            np.testing.assert_array_equal(got["gy"], ref["gy"])

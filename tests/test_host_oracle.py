@@ -3,7 +3,8 @@ their gradients, error behaviour, and the two training workloads against closed 
 import numpy as np
 import pytest
 
-from host_programs import TKAT, check_case, conv_inputs, conv_numpy, conv_step, mlp_numpy, mlp_run, run_case
+from host_programs import (TKAT, bf16_round, check_case, conv_inputs, conv_numpy, conv_step, elementwise_program, mlp_numpy, mlp_run,
+                           run_case)
 from maidenx_amd.tensor import MxError
 
 
@@ -145,3 +146,78 @@ def test_bench_chain_is_the_host_layers_call_sequence(mx_oracle, op, case):
     z = getattr(x, op)(y) if op in ("add", "mul", "div") else getattr(x, op)()
     z.backward()
     assert mx.backend_calls() == want, (op, case, mx.backend_calls(), want)
+
+
+# ---- bf16 through the host layer --------------------------------------------------------------------------
+@pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])
+def test_reference_tensor_cases_bf16(mx_oracle, case):
+    # the reference runs the same tests for bf16 with |error| < 0.1 (e.g. tests/ops_binary.rs:28-45)
+    check_case(run_case(mx_oracle, case, dtype="bf16"), case, tol=0.1)
+
+
+def test_dtype_promotion_rules(mx_oracle):
+    mx = mx_oracle
+    x = mx.tensor([1.0, 2.0, 3.0], dtype="bf16")
+    assert x.dtype == "bf16" and x.mul_scalar(2.0).dtype == "bf16"          # integer-valued scalar keeps the dtype
+    assert x.mul_scalar(0.5).dtype == "f32" and x.add_scalar(0.25).dtype == "f32"   # ops/unary.rs:796-800, 872-876
+    assert x.add_scalar(1.0).dtype == "bf16" and x.div_scalar(3.0).dtype == "bf16"  # ops/unary.rs:911-915
+    assert x.pow(2.0).dtype == "bf16" and x.pow(0.5).dtype == "f32"         # ops/unary.rs:1044-1048
+    f = mx.tensor([1.0, 2.0, 3.0])
+    assert x.add(f).dtype == "f32" and f.mul(x).dtype == "f32"              # utils/promotion.rs:16-33
+    assert x.gt_scalar(1.5).dtype == "bool"
+    np.testing.assert_array_equal(x.gt_scalar(1.5).to_dtype("bf16").numpy(), [0.0, 1.0, 1.0])
+    np.testing.assert_array_equal(mx.tensor([1.00390625, 3.14159], dtype="bf16").numpy(), bf16_round([1.00390625, 3.14159]))
+    g = mx.tensor([0.5, -1.5], dtype="bf16").with_grad()
+    g.gelu().backward()
+    assert g.grad().dtype == "bf16"                                          # cast back when accumulated (ops/binary.rs:660-662)
+
+
+@pytest.mark.parametrize("op", ["add", "mul", "div", "exp", "relu", "gelu"])
+@pytest.mark.parametrize("case", ["contig", "bcast", "transposed"])
+def test_bench_chain_is_the_host_layers_call_sequence_bf16(mx_oracle, op, case):
+    """As above for bf16, where the gelu closure promotes to f32: kernel calls and whole-buffer casts both agree."""
+    import bench
+    if op in ("exp", "relu", "gelu") and case == "bcast":
+        pytest.skip("unary ops have no broadcast case")
+    mx = mx_oracle
+
+    class FakeLib:
+        def __getattr__(self, name):
+            return lambda *a: None
+    b = bench.ChainBuilder(FakeLib(), "x_", lambda count, dtag, init: (0, None), "bf16", 6, 8, seed=1)
+    getattr(b, op)(case)
+    want_casts = sum(1 for c in b.calls if c.tag.startswith("cast_"))
+    want_calls = len(b.calls) - want_casts
+    mx.reset_backend_calls()
+    elementwise_program(mx, op, case, "bf16", R=6, C=8)
+    assert (mx.backend_calls(), mx.cast_calls()) == (want_calls, want_casts), (op, case)
+
+
+@pytest.mark.parametrize("case", ["contig", "bcast", "transposed"])
+def test_bf16_forward_backward_values(mx_oracle, case):
+    """add / mul / div on bf16 tensors against per-operation bf16 rounding in numpy."""
+    for op in ("add", "mul", "div"):
+        r = elementwise_program(mx_oracle, op, case, "bf16")
+        x = bf16_round(r["xs"].T if case == "transposed" else r["xs"])
+        y = np.broadcast_to(bf16_round(r["ys"]), x.shape)
+        assert r["z.dtype"] == "bf16" and r["gx.dtype"] == "bf16"
+        fwd = {"add": x + y, "mul": x * y, "div": x / y}[op]
+        np.testing.assert_array_equal(r["z"], bf16_round(fwd), err_msg=op)
+        ones = np.ones_like(x)
+        if op == "add":
+            gx, gy_full = ones, ones
+        elif op == "mul":
+            gx, gy_full = bf16_round(ones * y), bf16_round(ones * x)
+        else:
+            gx = bf16_round(ones / y)
+            gy_full = -bf16_round(bf16_round(ones * x) / bf16_round(y * y))
+        if case == "transposed":
+            gx = gx.T                                           # gradient of the tensor the view was taken from
+        np.testing.assert_array_equal(r["gx"], gx, err_msg=op)
+        if case == "bcast":
+            # summed over rows in f32 and rounded once (crates/maidenx_cpu/src/ops/reduction.rs:568 accumulates in bf16;
+            # the column sums here are short enough for a loose bound)
+            ref = gy_full.astype(np.float64).sum(0, keepdims=True)
+            assert np.all(np.abs(r["gy"] - ref) <= np.abs(gy_full).sum(0, keepdims=True) * 2.0 ** -6), op
+        else:
+            np.testing.assert_array_equal(r["gy"], gy_full, err_msg=op)
