@@ -513,6 +513,31 @@ __global__ __launch_bounds__(GB) void gemm_wavedot_kernel(GemmArgs g) {
     if (live && lane == 0) ((T*)g.out)[idx] = Elem<T>::st(acc);
 }
 
+// One block per output element for a handful of outputs with a long reduction (the MLP's weight gradient:
+// 3 outputs of 10000 terms): threads stride over r, waves fold by shuffles, the block by LDS, in a fixed order.
+template <class T>
+__global__ __launch_bounds__(1024) void gemm_blockdot_kernel(GemmArgs g) {
+    __shared__ float part[1024 / WAVE];
+    const size_t idx = blockIdx.x;
+    const size_t per = (size_t)g.I * g.J;
+    const uint32_t b = (uint32_t)(idx / per), rem = (uint32_t)(idx % per);
+    const uint32_t i = rem / g.J, j = rem % g.J;
+    const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
+    const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
+    float acc = 0.0f;
+    for (uint32_t r = threadIdx.x; r < g.R; r += 1024) acc += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, WAVE);
+    if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 1024 / WAVE; ++w) sum += part[w];
+        ((T*)g.out)[idx] = Elem<T>::st(sum);
+    }
+}
+
 template <class T>
 void gemm_dispatch(GemmArgs g) {
     if (g.I == 0 || g.J == 0 || g.batch == 0) return;
@@ -520,6 +545,11 @@ void gemm_dispatch(GemmArgs g) {
     if (g.R <= 16 || (g.I < 16 && g.J < 16 && g.R < 256)) {
         hipLaunchKernelGGL(gemm_thread_kernel<T>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_thread");
+        return;
+    }
+    if (outputs <= 64 && g.R >= 4096) {
+        hipLaunchKernelGGL(gemm_blockdot_kernel<T>, dim3((unsigned)outputs), dim3(1024), 0, stream(), g);
+        MXH_LAUNCH_CHECK("gemm_blockdot");
         return;
     }
     if (outputs <= 4096 && (g.I < 32 || g.J < 32)) {
