@@ -715,15 +715,31 @@ def run_conv(args):
     result = base_result(args, round(args.steps / dt_s, 2), "steps/s", dt_s, "f32",
                          "configs[4]: Conv2d 64->64 3x3 s1 p1 + bias, MSE loss, forward + backward, input [32,64,56,56] f32",
                          {"backend_kernels_per_step": mx.backend_calls() / args.steps})
-    # dominant HBM kernel: im2col at this shape, timed on its own through the C ABI
+    # the data-movement kernels of this config, each timed on its own through the C ABI (HIP events); the dominant
+    # one, im2col, gives the roofline object
     Bn, Cc, H, W = 32, 64, 56, 56
-    n_in, n_col = Bn * Cc * H * W, Bn * H * W * Cc * 9
-    src, col = L.DeviceBuffer(n_in * 4), L.DeviceBuffer(n_col * 4)
+    n_in, n_col, n_pad = Bn * Cc * H * W, Bn * H * W * Cc * 9, Bn * Cc * (H + 2) * (W + 2)
+    src, col, pad = L.DeviceBuffer(n_in * 4), L.DeviceBuffer(n_col * 4), L.DeviceBuffer(n_pad * 4)
     lib.hip_fill_f32(n_in, src.ptr, 1.0)
+    lib.hip_fill_f32(n_col, col.ptr, 1.0)
     md = u64(Bn, Cc, H, W, 3, 3, H, W, 1, 1, 1, 1)
-    calls = [Call(lib.hip_conv2d_im2col_f32, (n_col, md.ctypes.data, src.ptr, col.ptr), (n_in + n_col) * 4, "im2col", md) for _ in range(4)]
-    _, durs = timed_run(L, lib, calls, argparse.Namespace(steps=5, warmup=1), "im2col")
-    result["roofline"] = hbm_roofline("im2col_kernel<float,4> (hip_conv2d_im2col_f32, [32,64,56,56] 3x3)", (n_in + n_col) * 4, durs)
+    mdp = u64([Bn, Cc, H, W], [Cc * H * W, H * W, W, 1], 0, [Bn, Cc, H + 2, W + 2], [0, 0, 0, 0, 1, 1, 1, 1])
+    solo = {
+        "im2col": (lib.hip_conv2d_im2col_f32, (n_col, md.ctypes.data, src.ptr, col.ptr), (n_in + n_col) * 4),
+        # the layer's call: num_els = B*C*H*W, so only the first 25.7 MB of the column matrix are read (nn/layers/conv.rs:393)
+        "col2im (layer call)": (lib.hip_conv2d_col2im_f32, (n_in, md.ctypes.data, col.ptr, src.ptr), 2 * n_in * 4),
+        "col2im (whole column matrix)": (lib.hip_conv2d_col2im_f32, (n_col, md.ctypes.data, col.ptr, src.ptr), (n_in + n_col) * 4),
+        "pad_with_constant": (lib.hip_pad_with_constant_f32, (n_in, n_pad, 4, mdp.ctypes.data, src.ptr, pad.ptr, 0.0), (n_in + n_pad) * 4),
+        "pad_with_constant_backward": (lib.hip_pad_with_constant_backward_f32, (n_in, n_pad, 4, mdp.ctypes.data, pad.ptr, src.ptr), (n_in + n_pad) * 4),
+    }
+    kernels = {}
+    for name, (fn, fargs, nbytes) in solo.items():
+        calls = [Call(fn, fargs, nbytes, name, (md, mdp)) for _ in range(4)]
+        _, durs = timed_run(L, lib, calls, argparse.Namespace(steps=5, warmup=1), name)
+        kernels[name] = {"us": round(float(np.mean(durs)) * 1e3, 1), "GB/s": round(nbytes / float(np.mean(durs)) / 1e6, 1)}
+        if name == "im2col":
+            result["roofline"] = hbm_roofline("im2col_kernel<float,4> (hip_conv2d_im2col_f32, [32,64,56,56] 3x3)", nbytes, durs)
+    result["config"]["kernels_alone"] = kernels
     result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_conv(args)
     return result
 

@@ -65,6 +65,10 @@ __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restr
     fd_divmod(r, m.d_W, r, w);
     fd_divmod(r, m.d_H, r, h);
     fd_divmod(r, m.d_Cc, b, c);
+    // every column index of this (b, c) plane is at least plane0; beyond num_els the reference skips them all
+    // (the layer passes num_els = B*C*H*W, so most planes end here)
+    const size_t plane0 = (size_t)(b * m.C + c) * m.kh * m.kw * m.oh * m.ow;
+    if (plane0 >= num_els) { out[idx] = T{}; return; }
     uint32_t h_pad = h + m.ph, w_pad = w + m.pw;
     uint32_t hs = h_pad > m.kh - 1 ? h_pad - (m.kh - 1) : 0, ws = w_pad > m.kw - 1 ? w_pad - (m.kw - 1) : 0;
     uint32_t h_start, w_start, h_last, w_last, rem;
