@@ -3,10 +3,12 @@
 // crates/maidenx_cpu/src/nn/conv.rs:13-149.
 // Metadata (12 slots, as the kernel reads them): B, C, H, W, kh, kw, oh, ow, pad_h, pad_w,
 // stride_h, stride_w.
-//   im2col : col[b][(c*kh+i)*kw+j][ho*ow+wo] = in[b,c,ho*sh-ph+i, wo*sw-pw+j] or 0.  Write-bound:
-//            each lane produces 4 consecutive wo of one column row and stores them as one
-//            128-bit vector (when ow % 4 == 0 and the buffer is aligned), the shifted input
-//            reads come from cache.
+//   im2col : col[b][(c*kh+i)*kw+j][ho*ow+wo] = in[b,c,ho*sh-ph+i, wo*sw-pw+j] or 0.  Write-bound.
+//            Whole column matrix with ow a multiple of the vector width: a block stages the input
+//            rows of one (b, c) plane (or a band of it) once in a zero-padded LDS tile and streams
+//            the kh*kw shifted copies out as 128-bit stores, so no global-load latency sits in
+//            front of a store.  Otherwise (truncated num_els, odd widths, tiles beyond LDS): one
+//            thread per vector or element with the shifted reads served by cache.
 //   col2im : gather form with the reference's fixed summation order (ho then wo ascending, at
 //            most kh*kw terms), so the result is bit-exact and deterministic; column indices at
 //            or beyond num_els are skipped exactly as the reference does.
@@ -50,6 +52,52 @@ __global__ __launch_bounds__(CB) void im2col_kernel(ConvMeta m, const T* __restr
     if (base + VEC <= num_els) *(CVec<T, VEC>*)(col + base) = o;
     else
         for (int e = 0; e < VEC; ++e) if (base + e < num_els) col[base + e] = o.v[e];
+}
+
+// im2col through LDS: one block owns a band of output rows of one (b, c) plane.  The input rows the
+// band needs are read once into a zero-padded LDS tile [HP][WP] (so the copy loop has no bounds
+// checks and no global-load latency), then the kh*kw shifted copies leave as 16-byte stores.
+struct BandMeta {
+    uint32_t nb, bands, HP, WP, nvec_seg;       // output rows per band, bands per plane, tile extent, vectors per (i, j) segment
+    FastDiv d_WP, d_bands, d_seg, d_owv, d_kw;
+};
+
+template <class T, int VEC>
+__global__ __launch_bounds__(CB) void im2col_band_kernel(ConvMeta m, BandMeta k, const T* __restrict__ in, T* __restrict__ col) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    T* tile = (T*)smem;
+    uint32_t plane, band;
+    fd_divmod(blockIdx.x, k.d_bands, plane, band);            // plane = b*C + c
+    const uint32_t ho0 = band * k.nb;
+    const uint32_t nrows = min(k.nb, m.oh - ho0);
+    const int hi0 = (int)(ho0 * m.sh) - (int)m.ph;             // input row of tile row 0
+    const uint32_t hp = (nrows - 1) * m.sh + m.kh;             // tile rows this band uses
+    const T* src = in + (size_t)plane * m.H * m.W;
+    for (uint32_t idx = threadIdx.x; idx < hp * k.WP; idx += CB) {
+        uint32_t r, cidx;
+        fd_divmod(idx, k.d_WP, r, cidx);
+        int hi = hi0 + (int)r, wi = (int)cidx - (int)m.pw;
+        bool ok = hi >= 0 && hi < (int)m.H && wi >= 0 && wi < (int)m.W;
+        tile[idx] = ok ? src[(size_t)hi * m.W + wi] : T{};
+    }
+    __syncthreads();
+    const uint32_t seg = nrows * (m.ow / VEC);                 // vectors of one (i, j) segment in this band
+    const uint32_t total = seg * m.kh * m.kw;
+    T* dst_plane = col + ((size_t)plane * m.kh * m.kw * m.oh + ho0) * m.ow;
+    // full bands: divide by the constant segment length; the last (short) band of a plane divides by its own
+    const bool full = nrows == k.nb;
+    for (uint32_t idx = threadIdx.x; idx < total; idx += CB) {
+        uint32_t ij, q, r, wov, i, j;
+        if (full) fd_divmod(idx, k.d_seg, ij, q);
+        else { ij = idx / seg; q = idx - ij * seg; }
+        fd_divmod(q, k.d_owv, r, wov);
+        fd_divmod(ij, k.d_kw, i, j);
+        const T* t = tile + (r * m.sh + i) * k.WP + wov * VEC * m.sw + j;
+        CVec<T, VEC> o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o.v[e] = t[e * m.sw];
+        *(CVec<T, VEC>*)(dst_plane + ((size_t)ij * m.oh + r) * m.ow + wov * VEC) = o;
+    }
 }
 
 template <class T> __device__ inline T acc_add(T a, T b);
@@ -112,6 +160,31 @@ void im2col(size_t num_els, const size_t* md, const T* in, T* col) {
     uint32_t owv = vec ? m.ow / VEC : m.ow;
     m.d_owv = make_fastdiv(owv); m.d_oh = make_fastdiv(m.oh); m.d_kw = make_fastdiv(m.kw);
     m.d_kh = make_fastdiv(m.kh); m.d_C = make_fastdiv(m.C);
+    if (vec && n == full && VEC > 1) {
+        // band kernel: whole column matrix, rows a multiple of the vector width
+        BandMeta k;
+        k.WP = (m.ow - 1) * m.sw + m.kw;
+        auto tile_bytes = [&](uint32_t nb) { return (size_t)((nb - 1) * m.sh + m.kh) * k.WP * sizeof(T); };
+        constexpr size_t LDS_MAX = 32 * 1024;
+        if (tile_bytes(1) <= LDS_MAX) {
+            uint32_t nb = m.oh;
+            while (nb > 1 && tile_bytes(nb) > LDS_MAX) nb = (nb + 1) / 2;
+            // enough blocks to fill the chip, as long as a segment stays a few KB long
+            while (nb > 1 && (size_t)m.B * m.C * cdiv(m.oh, nb) < 1024 && (size_t)(nb / 2) * m.ow * sizeof(T) >= 2048) nb = (nb + 1) / 2;
+            k.nb = nb;
+            k.bands = (uint32_t)cdiv(m.oh, nb);
+            k.HP = (nb - 1) * m.sh + m.kh;
+            k.nvec_seg = nb * (m.ow / VEC);
+            k.d_WP = make_fastdiv(k.WP); k.d_bands = make_fastdiv(k.bands); k.d_seg = make_fastdiv(k.nvec_seg);
+            k.d_owv = make_fastdiv(m.ow / VEC); k.d_kw = make_fastdiv(m.kw);
+            size_t blocks = (size_t)m.B * m.C * k.bands;
+            if (blocks < (1ull << 31)) {
+                hipLaunchKernelGGL((im2col_band_kernel<T, VEC>), dim3((unsigned)blocks), dim3(CB), tile_bytes(nb), stream(), m, k, in, col);
+                MXH_LAUNCH_CHECK("im2col");
+                return;
+            }
+        }
+    }
     size_t nvec = vec ? (n + VEC - 1) / VEC : n;
     if (vec) hipLaunchKernelGGL((im2col_kernel<T, VEC>), dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, in, col, nvec, n);
     else hipLaunchKernelGGL((im2col_kernel<T, 1>), dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, in, col, nvec, n);

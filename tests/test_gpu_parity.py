@@ -458,7 +458,9 @@ def test_pad_transposed_input(oracle, hip):
 
 
 CONV_CASES = [(2, 3, 8, 8, 3, 3, 1, 1), (1, 4, 12, 12, 3, 3, 1, 1), (2, 2, 9, 7, 2, 3, 1, 2), (1, 1, 5, 5, 1, 1, 0, 1), (2, 3, 10, 10, 5, 5, 2, 2),
-             (3, 8, 14, 14, 3, 3, 1, 1), (1, 2, 6, 6, 3, 3, 0, 1)]
+             (3, 8, 14, 14, 3, 3, 1, 1), (1, 2, 6, 6, 3, 3, 0, 1),
+             # several bands of output rows per plane: a short last band, stride 2, a tile limited by LDS
+             (1, 2, 37, 64, 3, 3, 1, 1), (1, 2, 80, 63, 3, 3, 1, 2), (1, 1, 24, 512, 3, 3, 1, 1), (2, 3, 16, 16, 3, 3, 1, 1)]
 
 
 @pytest.mark.parametrize("dt", DTS)
