@@ -137,6 +137,89 @@ __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restr
     out[idx] = sum;
 }
 
+// Unit stride along w: a thread owns VEC adjacent pixels of a row.  For a fixed tap (i, j) their column
+// entries are adjacent too, so the column matrix streams in as (element-aligned) vectors; each pixel
+// still adds its terms in the reference's order: ho ascending, then wo ascending, which is j descending.
+template <class T, int N> struct alignas(sizeof(T)) CUVec { T v[N]; };
+
+// KH, KW > 0: the kernel extent is known at compile time, so every tap's load is issued before the first
+// add (the sums are latency-bound otherwise: one round trip per tap).  KH = KW = 0: run-time extent.
+template <class T, int VEC, int KH, int KW>
+__global__ __launch_bounds__(CB) void col2im_row_kernel(ConvMeta m, const T* __restrict__ col, T* __restrict__ out, size_t nvec,
+                                                        size_t num_els) {
+    size_t idx = (size_t)blockIdx.x * CB + threadIdx.x;
+    if (idx >= nvec) return;
+    uint32_t r = (uint32_t)idx, wv, h, plane;
+    fd_divmod(r, m.d_W, r, wv);            // d_W divides by W / VEC here
+    fd_divmod(r, m.d_H, plane, h);
+    T* dst = out + idx * VEC;
+    CVec<T, VEC> acc;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc.v[e] = T{};
+    const size_t plane0 = (size_t)plane * m.kh * m.kw * m.oh * m.ow;
+    if (plane0 < num_els) {
+        const uint32_t h_pad = h + m.ph;
+        // one tap: fetch the VEC column entries of (i, j, ho) that exist, and say which do
+        auto fetch = [&](uint32_t i, int j, uint32_t ho, CUVec<T, VEC>& v) -> uint32_t {
+            const int wo0 = (int)(wv * VEC + m.pw) - j;
+            const int64_t ci0 = (int64_t)(plane0 + ((size_t)(i * m.kw + j) * m.oh + ho) * m.ow) + wo0;
+            if (wo0 >= 0 && wo0 + VEC <= (int)m.ow && (size_t)ci0 + VEC <= num_els) {
+                v = *(const CUVec<T, VEC>*)(col + ci0);
+                return (1u << VEC) - 1;
+            }
+            uint32_t mask = 0;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int wo = wo0 + e;
+                const bool ok = wo >= 0 && wo < (int)m.ow && (size_t)(ci0 + e) < num_els;
+                v.v[e] = ok ? col[ci0 + e] : T{};
+                mask |= (uint32_t)ok << e;
+            }
+            return mask;
+        };
+        if constexpr (KH > 0) {
+            CUVec<T, VEC> v[KH * KW];
+            uint32_t mask[KH * KW];
+            // ho ascending is i descending: ho = (h_pad - i) / sh where that division is exact
+#pragma unroll
+            for (int a = 0; a < KH; ++a) {
+                const int i = KH - 1 - a;
+                uint32_t ho = 0, rem = 1;
+                if (h_pad >= (uint32_t)i) fd_divmod(h_pad - i, m.d_sh, ho, rem);
+                const bool row_ok = rem == 0 && ho < m.oh;
+#pragma unroll
+                for (int c = 0; c < KW; ++c) {
+                    mask[a * KW + c] = 0;
+                    if (row_ok) mask[a * KW + c] = fetch(i, KW - 1 - c, ho, v[a * KW + c]);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < KH * KW; ++k)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    if (mask[k] >> e & 1) acc.v[e] = acc_add<T>(acc.v[e], v[k].v[e]);
+        } else {
+            const uint32_t hs = h_pad > m.kh - 1 ? h_pad - (m.kh - 1) : 0;
+            uint32_t h_start, h_last, rem;
+            fd_divmod(hs + m.sh - 1, m.d_sh, h_start, rem);
+            fd_divmod(h_pad, m.d_sh, h_last, rem);
+            const uint32_t h_end = min(h_last + 1, m.oh);
+            for (uint32_t ho = h_start; ho < h_end; ++ho) {
+                const uint32_t i = h_pad - ho * m.sh;
+                if (i >= m.kh) continue;
+                for (int j = (int)m.kw - 1; j >= 0; --j) {
+                    CUVec<T, VEC> v;
+                    const uint32_t mask = fetch(i, j, ho, v);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        if (mask >> e & 1) acc.v[e] = acc_add<T>(acc.v[e], v.v[e]);
+                }
+            }
+        }
+    }
+    *(CVec<T, VEC>*)dst = acc;
+}
+
 // need_stride: col2im divides by the stride slots (the reference panics on 0); im2col only multiplies by them
 static bool parse_conv(const size_t* md, ConvMeta& m, bool need_stride) {
     for (int k = 0; k < 12; ++k) if (md[k] >= (1ull << 31)) return false;
@@ -199,8 +282,21 @@ void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
     size_t n_out = (size_t)m.B * m.C * m.H * m.W;
     if (n_out == 0) return;
     if (n_out >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "col2im: 2^32 or more output elements"); return; }
-    m.d_W = make_fastdiv(m.W); m.d_H = make_fastdiv(m.H); m.d_Cc = make_fastdiv(m.C);
+    m.d_H = make_fastdiv(m.H); m.d_Cc = make_fastdiv(m.C);
     m.d_sh = make_fastdiv(m.sh); m.d_sw = make_fastdiv(m.sw);
+    constexpr int VEC = 16 / sizeof(T);
+    if (m.sw == 1 && m.W % VEC == 0 && ((uintptr_t)out % 16) == 0) {
+        m.d_W = make_fastdiv(m.W / VEC);
+        size_t nvec = n_out / VEC;
+        auto kern = col2im_row_kernel<T, VEC, 0, 0>;
+        if (m.kh == 3 && m.kw == 3) kern = col2im_row_kernel<T, VEC, 3, 3>;
+        else if (m.kh == 1 && m.kw == 1) kern = col2im_row_kernel<T, VEC, 1, 1>;
+        else if (m.kh == 5 && m.kw == 5 && sizeof(T) == 4) kern = col2im_row_kernel<T, VEC, 5, 5>;
+        hipLaunchKernelGGL(kern, dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, col, out, nvec, num_els);
+        MXH_LAUNCH_CHECK("col2im");
+        return;
+    }
+    m.d_W = make_fastdiv(m.W);
     hipLaunchKernelGGL(col2im_kernel<T>, dim3(cdiv(n_out, CB)), dim3(CB), 0, stream(), m, col, out, n_out, num_els);
     MXH_LAUNCH_CHECK("col2im");
 }

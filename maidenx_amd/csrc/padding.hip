@@ -16,25 +16,36 @@ struct PadSpace {
     uint32_t before[MAXD];
     FastDiv div[MAXD];
     int64_t in_strides[MAXD];
+    // the innermost dim, kept apart: a thread's elements mostly differ in this coordinate only
+    uint32_t out_last, in_last, before_last;
+    int64_t stride_last;
+    FastDiv div_last;
 };
+
 
 constexpr int PB = 256;
 
 // forward: out[i] = inside ? in[idx] : pad_value
 // backward (FWD = false): grad_in[idx] = 0 + grad_out[i] for every inside i
-// A thread owns Q consecutive output elements: one coordinate decomposition (multiply-high divisions), then
-// carries; the contiguous side (out for forward, grad_out for backward) moves as one Q-element vector.
+// A thread owns Q consecutive output elements: one coordinate decomposition (multiply-high divisions); the outer
+// coordinates ("the row") are located once and again only when the elements run past the end of a row, so an
+// element costs one compare and one add.  The contiguous side (out for forward, grad_out for backward) moves
+// as one Q-element vector.
 template <class T, bool FWD, int Q>
 __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __restrict__ src, T* __restrict__ dst,
                                                        size_t n_out, T pad_value) {
     size_t i0 = ((size_t)blockIdx.x * PB + threadIdx.x) * Q;
     if (i0 >= n_out) return;
+    // coordinates: x in the innermost dim, c[d] in the outer ones
     uint32_t c[MAXD];
+    uint32_t x;
     {
         uint32_t r = (uint32_t)i0;
+        if (sp.ndims > 1) fd_divmod(r, sp.div_last, r, x);
+        else { x = r; r = 0; }
 #pragma unroll
-        for (int d = MAXD - 1; d >= 0; --d) {
-            if (d >= sp.ndims) { c[d] = 0; continue; }
+        for (int d = MAXD - 2; d >= 0; --d) {
+            if (d >= sp.ndims - 1) { c[d] = 0; continue; }
             uint32_t q, m;
             if (d > 0) fd_divmod(r, sp.div[d], q, m);
             else { q = 0; m = r; }
@@ -42,6 +53,21 @@ __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __r
             r = q;
         }
     }
+    // the row (all outer coordinates): inside the input or not, and where it starts
+    bool row_in;
+    int64_t row_idx;
+    auto locate_row = [&]() {
+        row_in = true;
+        row_idx = 0;
+#pragma unroll
+        for (int d = 0; d < MAXD - 1; ++d) {
+            if (d >= sp.ndims - 1) break;
+            uint32_t ic = c[d] - sp.before[d];           // wraps when c < before → fails the test below
+            row_in = row_in && ic < sp.in_dims[d];
+            row_idx += (int64_t)ic * sp.in_strides[d];
+        }
+    };
+    locate_row();
     const bool full = i0 + Q <= n_out;
     AVec<T, Q> v;
     if constexpr (!FWD) {
@@ -51,34 +77,32 @@ __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __r
     }
 #pragma unroll
     for (int e = 0; e < Q; ++e) {
-        int64_t idx = 0;
-        bool inside = true;
-#pragma unroll
-        for (int d = 0; d < MAXD; ++d) {
-            if (d >= sp.ndims) break;
-            uint32_t ic = c[d] - sp.before[d];           // wraps when c < before → fails the test below
-            inside = inside && ic < sp.in_dims[d];
-            idx += (int64_t)ic * sp.in_strides[d];
-        }
+        const uint32_t ic = x - sp.before_last;
+        const bool inside = row_in && ic < sp.in_last && (full || i0 + e < n_out);
+        const int64_t idx = row_idx + (int64_t)ic * sp.stride_last;
         if constexpr (FWD) {
-            v.v[e] = inside && (full || i0 + e < n_out) ? src[idx] : pad_value;
+            v.v[e] = inside ? src[idx] : pad_value;
         } else {
-            if (inside && (full || i0 + e < n_out)) {
+            if (inside) {
                 T g = v.v[e];
                 if constexpr (sizeof(T) == 4) dst[idx] = 0.0f + g;        // −0 → +0 like the reference's sums from zero
                 else dst[idx] = f2bf(0.0f + bf2f(g));
             }
         }
-        // next output element: add one with carries
-        bool carry = true;
+        // next output element; at the end of a row, carry into the outer coordinates
+        if (++x == sp.out_last && e + 1 < Q) {
+            x = 0;
+            bool carry = true;
 #pragma unroll
-        for (int d = MAXD - 1; d >= 0; --d) {
-            if (d >= sp.ndims) continue;
-            if (carry) {
-                c[d] += 1;
-                carry = c[d] == sp.out_dims[d];
-                if (carry) c[d] = 0;
+            for (int d = MAXD - 2; d >= 0; --d) {
+                if (d >= sp.ndims - 1) continue;
+                if (carry) {
+                    c[d] += 1;
+                    carry = c[d] == sp.out_dims[d];
+                    if (carry) c[d] = 0;
+                }
             }
+            locate_row();
         }
     }
     if constexpr (FWD) {
@@ -124,6 +148,9 @@ static bool build_space(size_t nd, const size_t* md, PadSpace& sp, size_t* in_of
     if (n == 0) { od[0] = id[0] = 1; bf[0] = 0; is[0] = 1; n = 1; }
     if (n > MAXD) return false;
     sp.ndims = n;
+    sp.out_last = (uint32_t)od[n - 1]; sp.in_last = (uint32_t)id[n - 1]; sp.before_last = (uint32_t)bf[n - 1];
+    sp.stride_last = is[n - 1];
+    sp.div_last = make_fastdiv(sp.out_last);
     for (int d = 0; d < MAXD; ++d) {
         sp.out_dims[d] = d < n ? (uint32_t)od[d] : 1;
         sp.in_dims[d] = d < n ? (uint32_t)id[d] : 1;

@@ -460,7 +460,9 @@ def test_pad_transposed_input(oracle, hip):
 CONV_CASES = [(2, 3, 8, 8, 3, 3, 1, 1), (1, 4, 12, 12, 3, 3, 1, 1), (2, 2, 9, 7, 2, 3, 1, 2), (1, 1, 5, 5, 1, 1, 0, 1), (2, 3, 10, 10, 5, 5, 2, 2),
              (3, 8, 14, 14, 3, 3, 1, 1), (1, 2, 6, 6, 3, 3, 0, 1),
              # several bands of output rows per plane: a short last band, stride 2, a tile limited by LDS
-             (1, 2, 37, 64, 3, 3, 1, 1), (1, 2, 80, 63, 3, 3, 1, 2), (1, 1, 24, 512, 3, 3, 1, 1), (2, 3, 16, 16, 3, 3, 1, 1)]
+             (1, 2, 37, 64, 3, 3, 1, 1), (1, 2, 80, 63, 3, 3, 1, 2), (1, 1, 24, 512, 3, 3, 1, 1), (2, 3, 16, 16, 3, 3, 1, 1),
+             # unit stride with 5x5, 1x1 and 2x4 kernels (col2im's compile-time and run-time tap loops)
+             (1, 2, 16, 16, 5, 5, 2, 1), (1, 2, 8, 8, 1, 1, 0, 1), (2, 2, 9, 16, 2, 4, 1, 1)]
 
 
 @pytest.mark.parametrize("dt", DTS)
@@ -476,6 +478,19 @@ def test_im2col_col2im_bit_exact(oracle, hip, case, dt):
     assert same_bits(o, h)
     y = to_storage(r.standard_normal(n_col).astype(np.float32), dt)
     for num_els in (n_col, B * Cc * H * W):      # full, and the truncation the reference's Conv2d passes
+        (o,), (h,) = both(oracle, hip, f"conv2d_col2im_{dt}", lambda: (num_els, md, In(y), Out(B * Cc * H * W, dt)))
+        assert same_bits(o, h), num_els
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("k", [3, 4])
+def test_col2im_row_stride_two_column_stride_one(oracle, hip, k, dt):
+    B, Cc, H, W, p, sh, sw = 2, 3, 15, 16, 1, 2, 1
+    oh, ow = (H + 2 * p - k) // sh + 1, (W + 2 * p - k) // sw + 1
+    n_col = B * Cc * k * k * oh * ow
+    md = meta_conv(B, Cc, H, W, k, k, oh, ow, p, p, sh, sw)
+    y = to_storage(rng(68).standard_normal(n_col).astype(np.float32), dt)
+    for num_els in (n_col, n_col // 2 + 3):
         (o,), (h,) = both(oracle, hip, f"conv2d_col2im_{dt}", lambda: (num_els, md, In(y), Out(B * Cc * H * W, dt)))
         assert same_bits(o, h), num_els
 
