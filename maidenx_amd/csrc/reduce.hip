@@ -93,7 +93,19 @@ __global__ __launch_bounds__(RB) void row_reduce_kernel(const TIn* __restrict__ 
             float a[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) a[e] = R::init(src_bf16);
-            for (size_t i = beg + (size_t)t * VEC; i < end; i += (size_t)TPR * VEC) {
+            // four loads in flight per lane; the adds keep the order of the plain loop
+            constexpr size_t STEP = (size_t)TPR * VEC;
+            size_t i = beg + (size_t)t * VEC;
+            for (; i + 3 * STEP < end; i += 4 * STEP) {
+                AVec<TIn, VEC> v[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = *(const AVec<TIn, VEC>*)(src + i + k * STEP);
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v[k].v[e]));
+            }
+            for (; i < end; i += STEP) {
                 AVec<TIn, VEC> v = *(const AVec<TIn, VEC>*)(src + i);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v.v[e]));
@@ -143,6 +155,59 @@ __global__ __launch_bounds__(RB) void col_reduce_kernel(const TIn* __restrict__ 
 #pragma unroll
     for (int e = 0; e < VEC; ++e) r.v[e] = IO<TOut>::fin(a[e], div);
     *(AVec<TOut, VEC>*)(out + ((size_t)o * chunks + chunk) * S + (size_t)jv * VEC) = r;
+}
+
+// ---- plane reduce: [A, K, S] → [chunks, K], summing over a and s ------------------------------------
+// The gradient of a per-channel parameter ([B, C, H*W] → [1, C, 1]): every kept index k owns A
+// separate runs of S contiguous elements.  One block of PB threads per (k, chunk of rows a); the
+// threads sweep the runs as 16-byte vectors, four loads in flight each, then meet in a DPP
+// butterfly and LDS.  S % VEC == 0 and a 16-byte aligned base are required.
+constexpr int PLB = 1024;
+template <class TIn, class TOut, class R, int VEC>
+__global__ __launch_bounds__(PLB) void plane_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, uint32_t A,
+                                                           uint32_t K, uint32_t S, uint32_t a_chunk, FastDiv div_sv,
+                                                           bool src_bf16) {
+    const uint32_t k = blockIdx.x % K, chunk = blockIdx.x / K;
+    const uint32_t a0 = chunk * a_chunk, rows = min(a_chunk, A - a0);
+    const uint32_t sv = S / VEC, nvec = rows * sv;
+    const TIn* base = in + ((size_t)a0 * K + k) * S;
+    const size_t row_pitch = (size_t)K * S;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = R::init(src_bf16);
+    auto addr = [&](uint32_t f) {
+        uint32_t a, c;
+        fd_divmod(f, div_sv, a, c);
+        return base + a * row_pitch + (size_t)c * VEC;
+    };
+    uint32_t f = threadIdx.x;
+    for (; f + 3 * PLB < nvec; f += 4 * PLB) {
+        AVec<TIn, VEC> v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = *(const AVec<TIn, VEC>*)addr(f + q * PLB);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = R::op(acc[e], IO<TIn>::ld(v[q].v[e]));
+    }
+    for (; f < nvec; f += PLB) {
+        AVec<TIn, VEC> v = *(const AVec<TIn, VEC>*)addr(f);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = R::op(acc[e], IO<TIn>::ld(v.v[e]));
+    }
+    float r = acc[0];
+#pragma unroll
+    for (int e = 1; e < VEC; ++e) r = R::op(r, acc[e]);
+    r = wave_reduce<R>(r);
+    __shared__ float part[PLB / WAVE];
+    if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = r;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        r = part[0];
+#pragma unroll
+        for (int w = 1; w < PLB / WAVE; ++w) r = R::op(r, part[w]);
+        out[(size_t)chunk * K + k] = IO<TOut>::fin(r, 0.0f);
+    }
 }
 
 // ---- generic single-axis reduce over a strided input (the reference's non-contiguous branch) ----
@@ -285,6 +350,34 @@ void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, floa
     fold_partials<TOut, R>(part, out, outer, chunks, S, div, src_bf16);
 }
 
+// [A, K, S] (contiguous) → out[K], both outer axes summed.  False when the shape does not fit the kernel.
+template <class T>
+bool plane_reduce(const T* in, T* out, size_t A, size_t K, size_t S) {
+    constexpr int VEC = 16 / sizeof(T);
+    if (S % VEC != 0 || !aligned16(in) || A * (S / VEC) >= (1ull << 31) || K >= (1ull << 24) || A >= (1ull << 31) || S >= (1ull << 31)) return false;
+    if (A * (S / VEC) < 2 * PLB) return false;         // too little per block to be worth it
+    // one block per kept index when there are enough of them, else cut the rows into chunks
+    uint32_t chunks = 1;
+    if (K < 256) chunks = (uint32_t)std::min<size_t>(A, cdiv((size_t)512, K));
+    uint32_t a_chunk = (uint32_t)cdiv(A, (size_t)chunks);
+    chunks = (uint32_t)cdiv(A, (size_t)a_chunk);
+    FastDiv dsv = make_fastdiv((uint32_t)(S / VEC));
+    const bool bf = IO<T>::is_bf16;
+    if (chunks == 1) {
+        hipLaunchKernelGGL((plane_reduce_kernel<T, T, RSum, VEC>), dim3((unsigned)K), dim3(PLB), 0, stream(), in, out, (uint32_t)A,
+                           (uint32_t)K, (uint32_t)S, a_chunk, dsv, bf);
+        MXH_LAUNCH_CHECK("plane_reduce");
+        return true;
+    }
+    float* part = (float*)scratch(((size_t)chunks * K + 8 * K) * sizeof(float) + 1024);
+    if (!part) return true;      // status is set
+    hipLaunchKernelGGL((plane_reduce_kernel<T, float, RSum, VEC>), dim3((unsigned)(K * chunks)), dim3(PLB), 0, stream(), in, part,
+                       (uint32_t)A, (uint32_t)K, (uint32_t)S, a_chunk, dsv, bf);
+    MXH_LAUNCH_CHECK("plane_reduce");
+    fold_partials<T, RSum>(part, out, 1, chunks, K, 0.0f, bf);
+    return true;
+}
+
 // sum/mean/max/min metadata: dims[n] | strides[n] | red_len[r] | red_stride[r] | offset
 template <class T, class R>
 void reduce_axis(size_t num_els, size_t num_dims, size_t nred, const size_t* md, const T* in, T* out, bool mean) {
@@ -421,6 +514,8 @@ void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in
         const size_t* ins[1] = {&st1};
         const void* inp[1] = {src};
         ew_launch<OpZeroPlus<T>>(num_els, 1, &dims1, &st1, ins, out, inp, OpZeroPlus<T>{});
+    } else if (ng == 3 && g_red[0] && !g_red[1] && g_red[2] && plane_reduce<T>(src, out, g_len[0], g_len[1], g_len[2])) {
+        // [reduced, kept, reduced] in one pass
     } else {
         // fold reduced groups one at a time, innermost first
         const void* cur = src;

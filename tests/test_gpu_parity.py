@@ -276,7 +276,9 @@ def test_reduce_strided_input_follows_reference_quirk(oracle, hip):
 
 STS_CASES = [([64, 96], [64, 96]), ([64, 96], [1, 96]), ([64, 96], [64, 1]), ([8, 64, 128], [1, 64, 1]), ([8, 64, 128], [8, 1, 128]),
              ([2, 3, 4, 5], [1, 3, 1, 5]), ([2, 3, 4, 5], [2, 1, 4, 1]), ([10000, 1], [10000, 1]), ([10000, 1], [1, 1]), ([5], [1]),
-             ([300, 700], [1, 1]), ([2, 3, 4, 5, 6], [1, 3, 1, 5, 1])]
+             ([300, 700], [1, 1]), ([2, 3, 4, 5, 6], [1, 3, 1, 5, 1]),
+             # [reduced, kept, reduced] in one pass: rows cut into chunks (few kept), one block per kept index (many)
+             ([40, 3, 256], [1, 3, 1]), ([64, 300, 128], [1, 300, 1]), ([33, 7, 520], [1, 7, 1]), ([2, 4, 260, 2, 64], [1, 1, 260, 1, 1])]
 
 
 @pytest.mark.parametrize("dt", DTS)
