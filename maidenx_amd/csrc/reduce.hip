@@ -7,7 +7,11 @@
 //            read 128-bit vectors, partial sums meet in a wave64 DPP butterfly and then in LDS.
 //   S  > 1 : "column" reduce.  Lanes run along S (coalesced, 128-bit where alignment allows)
 //            and walk L; when outer*S alone cannot fill the chip, L is cut into chunks whose
-//            partial results go to library scratch and are folded by a second launch.
+//            partial results go to library scratch and are folded by a second launch.  Wide rows
+//            with a long axis use blocks of 16 waves that share 64 column vectors and split the
+//            axis among the waves (partials meet in LDS), so fewer chunks are needed.
+// sum_to_shape folds its reduced groups with these two, innermost first; the [reduced, kept, reduced]
+// shape of a per-channel gradient has a one-pass kernel of its own.
 // Accumulation is f32 in a fixed order (deterministic from run to run); bf16 is rounded once.
 // No atomics anywhere.
 #include <cfloat>
@@ -72,6 +76,7 @@ __device__ inline float wave_reduce(float v) {
 }
 
 constexpr int RB = 256;
+constexpr size_t COL_SPLIT_BLOCKS = 256;      // one 16-wave block per CU
 
 // ---- row reduce: [rows, L] → [rows, chunks] ---------------------------------------------------
 // TPR threads cooperate on one (row, chunk).  VEC > 1 requires L % VEC == 0, chunk_len % VEC == 0
@@ -155,6 +160,63 @@ __global__ __launch_bounds__(RB) void col_reduce_kernel(const TIn* __restrict__ 
 #pragma unroll
     for (int e = 0; e < VEC; ++e) r.v[e] = IO<TOut>::fin(a[e], div);
     *(AVec<TOut, VEC>*)(out + ((size_t)o * chunks + chunk) * S + (size_t)jv * VEC) = r;
+}
+
+// ---- column reduce with the reduced axis split inside the block -------------------------------------
+// A block is NW waves deep: wave w walks slice w of the chunk's rows for
+// the same 64 column vectors, COL_U loads in flight per lane, and the NW partial rows meet in LDS in wave
+// order.  Against one thread per column this multiplies the loads in flight without more partials to
+// write and fold.  Requires S % VEC == 0 and aligned bases.
+template <class TIn, class TOut, class R, int VEC, int NW>
+__global__ __launch_bounds__(WAVE * NW) void col_reduce_split_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t L,
+                                                                      size_t S, uint32_t sv, unsigned chunks, size_t chunk_len,
+                                                                      FastDiv div_jb, FastDiv div_chunks, float div, bool src_bf16) {
+    constexpr int U = 8;
+    const int lane = threadIdx.x % WAVE, w = threadIdx.x / WAVE;
+    uint32_t rest, jb, o, chunk;
+    fd_divmod(blockIdx.x, div_jb, rest, jb);
+    fd_divmod(rest, div_chunks, o, chunk);
+    const uint32_t jv = jb * WAVE + lane;
+    const bool live = jv < sv;
+    const size_t beg = (size_t)chunk * chunk_len, end = beg + chunk_len < L ? beg + chunk_len : L;
+    const size_t slice = (end - beg + NW - 1) / NW;
+    const size_t l0 = beg + (size_t)w * slice < end ? beg + (size_t)w * slice : end, l1 = l0 + slice < end ? l0 + slice : end;
+    float a[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) a[e] = R::init(src_bf16);
+    if (live) {
+        const TIn* src = in + ((size_t)o * L + l0) * S + (size_t)jv * VEC;
+        size_t l = l0;
+        for (; l + U <= l1; l += U, src += U * S) {
+            AVec<TIn, VEC> v[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) v[k] = *(const AVec<TIn, VEC>*)(src + k * S);
+#pragma unroll
+            for (int k = 0; k < U; ++k)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v[k].v[e]));
+        }
+        for (; l < l1; ++l, src += S) {
+            AVec<TIn, VEC> v = *(const AVec<TIn, VEC>*)src;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v.v[e]));
+        }
+    }
+    __shared__ float part[NW][VEC][WAVE];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[w][e][lane] = a[e];
+    __syncthreads();
+    if (w == 0 && live) {
+        AVec<TOut, VEC> r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float t = part[0][e][lane];
+#pragma unroll
+            for (int k = 1; k < NW; ++k) t = R::op(t, part[k][e][lane]);
+            r.v[e] = IO<TOut>::fin(t, div);
+        }
+        *(AVec<TOut, VEC>*)(out + ((size_t)o * chunks + chunk) * S + (size_t)jv * VEC) = r;
+    }
 }
 
 // ---- plane reduce: [A, K, S] → [chunks, K], summing over a and s ------------------------------------
@@ -329,9 +391,50 @@ void fold_partials(const float* part, TOut* out, size_t outer, unsigned chunks, 
     col_stage<float, TOut, R>(part, out, outer, chunks, S, 1, chunks, div, src_bf16);
 }
 
+// The split kernel: 16 waves deep.  False when the shape does not fit it.
+template <class TIn, class TOut, class R>
+bool col_split_stage(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, unsigned chunks, size_t chunk_len, float div,
+                     bool src_bf16) {
+    constexpr int VI = 16 / sizeof(TIn), VO = 16 / sizeof(TOut);
+    constexpr int VEC = VI < VO ? VI : VO;
+    constexpr int NW = 16;
+    if (S % VEC != 0 || ((uintptr_t)in % (VEC * sizeof(TIn))) != 0 || ((uintptr_t)out % (VEC * sizeof(TOut))) != 0) return false;
+    size_t sv = S / VEC, jblocks = cdiv(sv, (size_t)WAVE);
+    size_t blocks = outer * chunks * jblocks;
+    if (blocks >= (1ull << 31) || sv >= (1ull << 31)) return false;
+    hipLaunchKernelGGL((col_reduce_split_kernel<TIn, TOut, R, VEC, NW>), dim3((unsigned)blocks), dim3(WAVE * NW), 0, stream(), in, out,
+                       L, S, (uint32_t)sv, chunks, chunk_len, make_fastdiv((uint32_t)jblocks), make_fastdiv(chunks), div, src_bf16);
+    MXH_LAUNCH_CHECK("col_reduce_split");
+    return true;
+}
+
 // [outer, L, S] (contiguous) → out[outer, S]
 template <class TIn, class TOut, class R>
 void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, float div, bool src_bf16) {
+    {
+        // wide rows and a long axis: blocks of 16 waves that split the axis among their waves
+        constexpr int VI = 16 / sizeof(TIn), VO = 16 / sizeof(TOut);
+        constexpr int VEC = VI < VO ? VI : VO;
+        const size_t jblocks = cdiv(S / VEC, (size_t)WAVE);
+        if (S % VEC == 0 && S / VEC >= WAVE && L >= 256) {
+            size_t base = outer * jblocks;
+            unsigned chunks = 1;
+            if (base < COL_SPLIT_BLOCKS) chunks = (unsigned)std::min<size_t>(cdiv((size_t)COL_SPLIT_BLOCKS, base), L / 256);
+            if (chunks < 1) chunks = 1;
+            size_t chunk_len = cdiv(L, (size_t)chunks);
+            chunks = (unsigned)cdiv(L, chunk_len);
+            if (chunks == 1) {
+                if (col_split_stage<TIn, TOut, R>(in, out, outer, L, S, 1, L, div, src_bf16)) return;
+            } else {
+                float* part = (float*)scratch((outer * chunks * S + outer * 8 * S) * sizeof(float) + 1024);
+                if (!part) return;
+                if (col_split_stage<TIn, float, R>(in, part, outer, L, S, chunks, chunk_len, 0.0f, src_bf16)) {
+                    fold_partials<TOut, R>(part, out, outer, chunks, S, div, src_bf16);
+                    return;
+                }
+            }
+        }
+    }
     size_t base_blocks = (outer * (S / 4 + 1) + RB - 1) / RB;
     unsigned chunks = 1;
     size_t chunk_len = L;
