@@ -135,13 +135,17 @@ MX_DECL_UNARY(mx_bf16, bf16)
  * sum_to_shape metadata = in_dims[n] | in_strides[n] | out_dims[n] | offset; every output dim is 1
  * or the input dim.  Semantics: crates/maidenx_cpu/src/ops/reduction.rs:6-183, 185-272, 383-553
  * (mean divides once at the end; max starts from f32::MIN, min from f32::MAX; NaNs never win).
- * Accumulation is f32 in a fixed order; bf16 results are rounded once. */
+ * Accumulation is f32 in a fixed order; bf16 results are rounded once.
+ * fold metadata = dims[n] | strides[n] | fold_dim, window_dim, fold_size, step, window_size, offset: the
+ * adjoint of unfold, crates/maidenx_cpu/src/ops/reduction.rs:274-380 (output = the input shape without
+ * window_dim and with fold_dim resized to fold_size; num_els counts the input). */
 #define MX_DECL_REDUCE(T, S)                                                                                \
     void hip_sum_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out);  \
     void hip_mean_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out); \
     void hip_max_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out);  \
     void hip_min_##S(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const T* inp, T* out);  \
-    void hip_sum_to_shape_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* inp, T* out);
+    void hip_sum_to_shape_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* inp, T* out);  \
+    void hip_fold_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* inp, T* out);
 MX_DECL_REDUCE(float, f32)
 MX_DECL_REDUCE(mx_bf16, bf16)
 
@@ -168,6 +172,22 @@ MX_DECL_MATMUL(mx_bf16, bf16)
 MX_DECL_PAD(float, f32)
 MX_DECL_PAD(mx_bf16, bf16)
 
+/* reflection / replication modes of the same file (same metadata, no pad value).
+ * Semantics: crates/maidenx_cpu/src/ops/padding.rs:115-325 (forward, bit-exact) and :438-665 (backward:
+ * each input position receives the sum of the output gradients read from it, f32 accumulation in
+ * ascending output order).  Reflection of a padded dim of size 1 is refused (the reference never returns). */
+#define MX_DECL_PAD_EDGE(T, S)                                                                              \
+    void hip_pad_with_reflection_##S(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, \
+                                     const T* inp, T* out);                                                 \
+    void hip_pad_with_replication_##S(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, \
+                                      const T* inp, T* out);                                                \
+    void hip_pad_with_reflection_backward_##S(size_t num_els_in, size_t num_els_out, size_t num_dims,       \
+                                              const size_t* metadata, const T* grad_out, T* grad_in);       \
+    void hip_pad_with_replication_backward_##S(size_t num_els_in, size_t num_els_out, size_t num_dims,      \
+                                               const size_t* metadata, const T* grad_out, T* grad_in);
+MX_DECL_PAD_EDGE(float, f32)
+MX_DECL_PAD_EDGE(mx_bf16, bf16)
+
 /* ---- conv: replaces crates/maidenx_cuda/src/nn/conv.rs:12-24 --------------------------------------
  * metadata = 12 slots B, C, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w as the kernel
  * reads them (crates/maidenx_cpu/src/nn/conv.rs:20-34).  im2col writes [B][C*kh*kw][oh*ow];
@@ -177,6 +197,14 @@ MX_DECL_PAD(mx_bf16, bf16)
     void hip_conv2d_col2im_##S(size_t num_els, const size_t* metadata, const T* col, T* output);
 MX_DECL_CONV(float, f32)
 MX_DECL_CONV(mx_bf16, bf16)
+
+/* ---- softmax: replaces crates/maidenx_cuda/src/nn/activation/softmax.rs (cuda_softmax_<T>) ------------
+ * metadata = dims[n] | strides[n] | offset; dim >= num_dims means the last dim.
+ * Semantics: crates/maidenx_cpu/src/nn/activation/softmax.rs:62-207 (max from -inf, the sum seeded
+ * with exp(-inf - max), output contiguous; a strided input is indexed with the reference's own rule,
+ * which walks the leading dims from dim 0 upwards).  The sum is f32 in a fixed order. */
+void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const float* input, float* output);
+void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const mx_bf16* input, mx_bf16* output);
 
 /* ---- device-side fill / convert / strided copy --------------------------------------------------
  * No backend symbol exists for these in the reference: it builds host vectors

@@ -36,6 +36,11 @@ def signatures(dtypes=("f32", "bf16")):
         for op in REDUCE:
             sig[f"{op}_{dt}"] = [SZ, SZ, SZ, P, P, P]
         sig[f"sum_to_shape_{dt}"] = [SZ, SZ, P, P, P]
+        sig[f"fold_{dt}"] = [SZ, SZ, P, P, P]
+        sig[f"softmax_{dt}"] = [SZ, SZ, SZ, P, P, P]
+        for mode in ("reflection", "replication"):
+            sig[f"pad_with_{mode}_{dt}"] = [SZ, SZ, SZ, P, P, P]
+            sig[f"pad_with_{mode}_backward_{dt}"] = [SZ, SZ, SZ, P, P, P]
         sig[f"matmul_{dt}"] = [SZ, P, P, P, P]
         sig[f"matmul_backward_{dt}"] = [SZ, SZ, P, P, P, P, P, P]
         sig[f"pad_with_constant_{dt}"] = [SZ, SZ, SZ, P, P, P, c]

@@ -1,6 +1,6 @@
-// Constant padding, forward and backward.  Replaces cuda_pad_with_constant_<T> and
-// cuda_pad_with_constant_backward_<T> of crates/maidenx_cuda/src/ops/padding.rs:13-71 with the
-// CPU semantics of crates/maidenx_cpu/src/ops/padding.rs:7-113 and :327-436.
+// Padding, forward and backward.  Replaces cuda_pad_with_{constant,reflection,replication}_<T> and their
+// _backward_ partners of crates/maidenx_cuda/src/ops/padding.rs:13-71 with the CPU semantics of
+// crates/maidenx_cpu/src/ops/padding.rs (constant :7-113 and :327-436; the two edge modes further down).
 // Metadata: in_dims[n] | in_strides[n] | in_offset | out_dims[n] | (pad_before, pad_after)[n]
 // Pure data movement, bit-exact.  One lane per 16 bytes of output; the coordinate walk uses
 // multiply-high division on the collapsed shape (dims without padding whose input strides chain
@@ -198,6 +198,198 @@ void pad_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const 
     MXH_LAUNCH_CHECK("pad_const_backward");
 }
 
+// ---- reflection and replication -----------------------------------------------------------------------
+// Forward (padding.rs:115-325): every output coordinate maps to an input coordinate per dim — clamped
+// (replication) or mirrored at 0 and at dim-1 until inside (reflection) — and the element is copied.
+// Backward (:438-665): every input element receives the sum of the output gradients that were read
+// from it.  Gather form: per dim the output coordinates that map to an input coordinate p are
+// enumerated in ascending order (replication: a run; reflection: p + k*P and -p + k*P shifted by the
+// leading pad, P = 2*(dim-1)), and the dims are walked like an odometer, so a thread adds its terms in
+// ascending output index — the order the reference gets with one worker.  f32 accumulation.
+enum EdgeMode : int { EDGE_REFLECT = 0, EDGE_REPLICATE = 1 };
+
+__device__ inline uint32_t edge_pos(int mode, int64_t pos, int64_t dim) {
+    if (mode == EDGE_REPLICATE) return (uint32_t)(pos < 0 ? 0 : (pos > dim - 1 ? dim - 1 : pos));
+    if (pos < 0) pos = -pos;
+    else if (pos >= dim) pos = 2 * dim - pos - 2;
+    while (pos < 0 || pos >= dim) {
+        if (pos < 0) pos = -pos;
+        else pos = 2 * dim - pos - 2;
+    }
+    return (uint32_t)pos;
+}
+
+template <class T>
+__global__ __launch_bounds__(PB) void pad_edge_kernel(PadSpace sp, int mode, const T* __restrict__ src, T* __restrict__ dst, size_t n_out) {
+    size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
+    if (i >= n_out) return;
+    uint32_t r = (uint32_t)i;
+    int64_t idx = 0;
+#pragma unroll
+    for (int d = MAXD - 1; d >= 0; --d) {
+        if (d >= sp.ndims) continue;
+        uint32_t q, c;
+        if (d > 0) fd_divmod(r, sp.div[d], q, c);
+        else { q = 0; c = r; }
+        idx += (int64_t)edge_pos(mode, (int64_t)c - (int64_t)sp.before[d], (int64_t)sp.in_dims[d]) * sp.in_strides[d];
+        r = q;
+    }
+    dst[i] = src[idx];
+}
+
+// Ascending enumeration of the output coordinates of one dim that map to input coordinate p.
+struct EdgeIter {
+    int64_t a, b, hi, period;       // next candidates of the two progressions, last coordinate, step
+    __device__ void init(int mode, uint32_t p, uint32_t in_dim, uint32_t out_dim, uint32_t before) {
+        hi = (int64_t)out_dim - 1;
+        if (mode == EDGE_REPLICATE) {
+            // a run [first, last] walked with period 1; b never fires
+            a = p == 0 ? 0 : (int64_t)p + before;
+            int64_t last = p == in_dim - 1 ? hi : (int64_t)p + before;
+            hi = last < hi ? last : hi;
+            b = INT64_MAX;
+            period = 1;
+            return;
+        }
+        period = 2 * ((int64_t)in_dim - 1);
+        if (period == 0) { a = 0; b = INT64_MAX; period = 1; return; }     // in_dim == 1 (no padding allowed): everything maps to 0
+        // q = o - before must be congruent to p or -p modulo the period
+        auto first = [&](int64_t residue) {      // smallest o >= 0 with (o - before - residue) % period == 0
+            int64_t t = residue + (int64_t)before;     // o = t + k*period
+            int64_t k = t >= 0 ? -(t / period) : (-t + period - 1) / period;
+            return t + k * period;
+        };
+        a = first((int64_t)p);
+        b = first(-(int64_t)p);
+    }
+    __device__ bool done() const { return (a < b ? a : b) > hi; }
+    __device__ int64_t cur() const { return a < b ? a : b; }
+    __device__ void next() {
+        int64_t c = cur();
+        if (a == c) a += period;
+        if (b == c) b += period;
+    }
+};
+
+template <class T>
+__global__ __launch_bounds__(PB) void pad_edge_backward_kernel(PadSpace sp, int mode, const T* __restrict__ go, T* __restrict__ gi,
+                                                                size_t n_in, PadSpace in_walk) {
+    // in_walk.div / in_walk.out_dims describe the input's logical shape (for the coordinate split)
+    size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
+    if (i >= n_in) return;
+    uint32_t p[MAXD];
+    {
+        uint32_t r = (uint32_t)i;
+#pragma unroll
+        for (int d = MAXD - 1; d >= 0; --d) {
+            if (d >= sp.ndims) { p[d] = 0; continue; }
+            uint32_t q, c;
+            if (d > 0) fd_divmod(r, in_walk.div[d], q, c);
+            else { q = 0; c = r; }
+            p[d] = c;
+            r = q;
+        }
+    }
+    int64_t dst = 0;
+    for (int d = 0; d < sp.ndims; ++d) dst += (int64_t)p[d] * sp.in_strides[d];
+    // row-major strides of the output
+    int64_t ost[MAXD];
+    {
+        int64_t acc = 1;
+        for (int d = sp.ndims - 1; d >= 0; --d) { ost[d] = acc; acc *= sp.out_dims[d]; }
+    }
+    EdgeIter it[MAXD];
+    bool empty = false;
+    for (int d = 0; d < sp.ndims; ++d) {
+        it[d].init(mode, p[d], sp.in_dims[d], sp.out_dims[d], sp.before[d]);
+        empty = empty || it[d].done();
+    }
+    float acc = 0.0f;
+    if (!empty) {
+        while (true) {
+            int64_t o = 0;
+            for (int d = 0; d < sp.ndims; ++d) o += it[d].cur() * ost[d];
+            if constexpr (sizeof(T) == 4) acc += go[o];
+            else acc += bf2f(go[o]);
+            // odometer: advance the innermost dim, carry outwards
+            int d = sp.ndims - 1;
+            for (; d >= 0; --d) {
+                it[d].next();
+                if (!it[d].done()) break;
+                it[d].init(mode, p[d], sp.in_dims[d], sp.out_dims[d], sp.before[d]);
+            }
+            if (d < 0) break;
+        }
+    }
+    if constexpr (sizeof(T) == 4) gi[dst] = acc;
+    else gi[dst] = f2bf(acc);
+}
+
+static bool edge_space(size_t nd, const size_t* md, int mode, PadSpace& sp, PadSpace& in_walk, size_t* in_off, const char* who) {
+    // no collapsing: every dim keeps its own mapping
+    if (nd > (size_t)MAXD) { set_status(ERR_UNSUPPORTED, who); return false; }
+    const size_t* in_dims = md;
+    const size_t* in_strides = md + nd;
+    *in_off = md[2 * nd];
+    const size_t* out_dims = md + 2 * nd + 1;
+    const size_t* pads = md + 3 * nd + 1;
+    bool cont = ref_is_contiguous(nd, in_dims, in_strides);
+    size_t cs[MAXD];
+    contiguous_strides(nd, in_dims, cs);
+    const size_t* st = cont ? cs : in_strides;       // padding.rs:199-214: contiguous inputs are indexed row-major
+    sp.ndims = (int)(nd ? nd : 1);
+    in_walk.ndims = sp.ndims;
+    for (int d = 0; d < MAXD; ++d) {
+        bool real = d < (int)nd;
+        if (real && (in_dims[d] >= (1ull << 31) || out_dims[d] >= (1ull << 31) || pads[2 * d] >= (1ull << 31))) { set_status(ERR_TOO_LARGE, who); return false; }
+        if (real && in_dims[d] == 0 && out_dims[d] != 0) { set_status(ERR_INVALID, who); return false; }
+        // the reference's mirror loop never ends for a padded dim of size 1
+        if (real && mode == EDGE_REFLECT && in_dims[d] == 1 && out_dims[d] != 1) { set_status(ERR_INVALID, "pad_with_reflection: a dim of size 1 cannot be mirrored"); return false; }
+        sp.out_dims[d] = real ? (uint32_t)out_dims[d] : 1;
+        sp.in_dims[d] = real ? (uint32_t)in_dims[d] : 1;
+        sp.before[d] = real ? (uint32_t)pads[2 * d] : 0;
+        sp.in_strides[d] = real ? (int64_t)st[d] : 0;
+        sp.div[d] = make_fastdiv(sp.out_dims[d]);
+        in_walk.div[d] = make_fastdiv(sp.in_dims[d]);
+    }
+    sp.out_last = sp.in_last = 1; sp.before_last = 0; sp.stride_last = 0; sp.div_last = make_fastdiv(1);
+    in_walk.out_last = in_walk.in_last = 1; in_walk.before_last = 0; in_walk.stride_last = 0; in_walk.div_last = make_fastdiv(1);
+    return true;
+}
+
+template <class T>
+void pad_edge_forward(int mode, size_t n_in, size_t n_out, size_t nd, const size_t* md, const T* in, T* out) {
+    (void)n_in;
+    if (!md || !in || !out) { set_status(ERR_INVALID, "pad: null argument"); return; }
+    if (n_out == 0) return;
+    if (n_out >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad: output of 2^31 or more elements"); return; }
+    PadSpace sp, walk; size_t off;
+    if (!edge_space(nd, md, mode, sp, walk, &off, "pad_with_reflection/replication: bad shape or rank above 8")) return;
+    hipLaunchKernelGGL(pad_edge_kernel<T>, dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, mode, in + off, out, n_out);
+    MXH_LAUNCH_CHECK("pad_edge");
+}
+
+template <class T>
+void pad_edge_backward(int mode, size_t n_in, size_t n_out, size_t nd, const size_t* md, const T* go, T* gi) {
+    if (!md || !go || !gi) { set_status(ERR_INVALID, "pad_backward: null argument"); return; }
+    if (n_in == 0) return;
+    if (n_out >= (1ull << 31) || n_in >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad_backward: 2^31 or more elements"); return; }
+    PadSpace sp, walk; size_t off;
+    if (!edge_space(nd, md, mode, sp, walk, &off, "pad_with_reflection/replication backward: bad shape or rank above 8")) return;
+    // the reference writes num_els_in contiguous elements at grad_in + offset: positions a strided
+    // layout does not reach hold 0
+    bool cont = ref_is_contiguous(nd, md, md + nd);
+    if (!cont) {
+        hipLaunchKernelGGL(zero_kernel<T>, dim3(cdiv(n_in, PB)), dim3(PB), 0, stream(), gi + off, n_in);
+        MXH_LAUNCH_CHECK("pad_zero");
+    }
+    size_t logical = 1;
+    for (size_t d = 0; d < nd; ++d) logical *= md[d];
+    if (logical == 0) return;
+    hipLaunchKernelGGL(pad_edge_backward_kernel<T>, dim3(cdiv(logical, PB)), dim3(PB), 0, stream(), sp, mode, go, gi + off, logical, walk);
+    MXH_LAUNCH_CHECK("pad_edge_backward");
+}
+
 }  // namespace mxh
 
 using namespace mxh;
@@ -212,5 +404,25 @@ using namespace mxh;
         pad_backward<T>(n_in, n_out, nd, md, go, gi);                                                        \
     }
 
+#define MXH_PAD_EDGE_FOR(T, SUF)                                                                             \
+    extern "C" void hip_pad_with_reflection_##SUF(size_t n_in, size_t n_out, size_t nd, const size_t* md,    \
+                                                  const T* in, T* out) {                                     \
+        pad_edge_forward<T>(EDGE_REFLECT, n_in, n_out, nd, md, in, out);                                     \
+    }                                                                                                        \
+    extern "C" void hip_pad_with_replication_##SUF(size_t n_in, size_t n_out, size_t nd, const size_t* md,   \
+                                                   const T* in, T* out) {                                    \
+        pad_edge_forward<T>(EDGE_REPLICATE, n_in, n_out, nd, md, in, out);                                   \
+    }                                                                                                        \
+    extern "C" void hip_pad_with_reflection_backward_##SUF(size_t n_in, size_t n_out, size_t nd,             \
+                                                           const size_t* md, const T* go, T* gi) {           \
+        pad_edge_backward<T>(EDGE_REFLECT, n_in, n_out, nd, md, go, gi);                                     \
+    }                                                                                                        \
+    extern "C" void hip_pad_with_replication_backward_##SUF(size_t n_in, size_t n_out, size_t nd,            \
+                                                            const size_t* md, const T* go, T* gi) {          \
+        pad_edge_backward<T>(EDGE_REPLICATE, n_in, n_out, nd, md, go, gi);                                   \
+    }
+
+MXH_PAD_EDGE_FOR(float, f32)
+MXH_PAD_EDGE_FOR(bf16_t, bf16)
 MXH_PAD_FOR(float, f32)
 MXH_PAD_FOR(bf16_t, bf16)

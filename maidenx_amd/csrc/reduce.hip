@@ -657,6 +657,93 @@ void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in
     }
 }
 
+// ---- fold ---------------------------------------------------------------------------------------------
+// The adjoint of unfold (crates/maidenx_cpu/src/ops/reduction.rs:274-380): input element c adds to the
+// output at c without the window dim and with the fold dim set to c[fold]*step + c[window].  Gather
+// form: one thread per output element sums its windows in ascending order in f32 (the reference adds
+// in scheduling order in the storage dtype).  The source index is (sum c*stride) % num_els (:336-340).
+// metadata: dims[n] | strides[n] | fold_dim, window_dim, fold_size, step, window_size, offset
+struct FoldSpace {
+    int nd_out;                      // output rank (input rank - 1)
+    int fold_slot;                   // position of the folded dim among the output dims
+    uint32_t out_dims[MAXD];
+    FastDiv div[MAXD];
+    int64_t strides[MAXD];           // input stride of each output dim (the fold slot: unused)
+    int64_t fold_stride, window_stride;
+    uint32_t n_windows, window, step;
+};
+
+template <class T>
+__global__ __launch_bounds__(RB) void fold_kernel(FoldSpace sp, const T* __restrict__ in, T* __restrict__ out, size_t out_size,
+                                                  size_t num_els) {
+    size_t o = (size_t)blockIdx.x * RB + threadIdx.x;
+    if (o >= out_size) return;
+    uint32_t r = (uint32_t)o, p = 0;
+    int64_t base = 0;
+#pragma unroll
+    for (int d = MAXD - 1; d >= 0; --d) {
+        if (d >= sp.nd_out) continue;
+        uint32_t q, c;
+        if (d > 0) fd_divmod(r, sp.div[d], q, c);
+        else { q = 0; c = r; }
+        if (d == sp.fold_slot) p = c;
+        else base += (int64_t)c * sp.strides[d];
+        r = q;
+    }
+    float acc = 0.0f;
+    if (sp.step == 0) {
+        if (p < sp.window)
+            for (uint32_t w = 0; w < sp.n_windows; ++w)
+                acc += IO<T>::ld(in[(uint64_t)(base + (int64_t)w * sp.fold_stride + (int64_t)p * sp.window_stride) % num_els]);
+    } else {
+        uint32_t w0 = p >= sp.window ? (p - sp.window) / sp.step + 1 : 0;
+        uint32_t w1 = p / sp.step;
+        if (w1 >= sp.n_windows) w1 = sp.n_windows - 1;
+        for (uint32_t w = w0; w <= w1 && sp.n_windows > 0; ++w) {
+            uint32_t pos = p - w * sp.step;
+            acc += IO<T>::ld(in[(uint64_t)(base + (int64_t)w * sp.fold_stride + (int64_t)pos * sp.window_stride) % num_els]);
+        }
+    }
+    out[o] = IO<T>::fin(acc, 0.0f);
+}
+
+template <class T>
+void fold(size_t num_els, size_t nd, const size_t* md, const T* in, T* out) {
+    if (!md || !in || !out) { set_status(ERR_INVALID, "fold: null argument"); return; }
+    if (nd < 2 || nd > (size_t)MAXD + 1) { set_status(ERR_UNSUPPORTED, "fold: rank must be 2..9"); return; }
+    const size_t* dims = md;
+    const size_t* strides = md + nd;
+    const size_t fold_dim = md[2 * nd], window_dim = md[2 * nd + 1], fold_size = md[2 * nd + 2], step = md[2 * nd + 3];
+    const size_t offset = md[2 * nd + 5];
+    if (fold_dim >= nd || window_dim >= nd || fold_dim == window_dim) { set_status(ERR_INVALID, "fold: bad dims"); return; }
+    FoldSpace sp;
+    size_t out_size = 1;
+    int k = 0;
+    sp.fold_slot = 0;
+    for (size_t d = 0; d < nd; ++d) {
+        if (d == window_dim) continue;
+        size_t len = d == fold_dim ? fold_size : dims[d];
+        if (d == fold_dim) sp.fold_slot = k;
+        sp.out_dims[k] = (uint32_t)len;
+        sp.div[k] = make_fastdiv((uint32_t)len);
+        sp.strides[k] = (int64_t)strides[d];
+        out_size *= len;
+        ++k;
+    }
+    sp.nd_out = k;
+    for (; k < MAXD; ++k) { sp.out_dims[k] = 1; sp.div[k] = make_fastdiv(1); sp.strides[k] = 0; }
+    if (out_size == 0) return;
+    if (out_size >= (1ull << 31) || num_els >= (1ull << 31) || step >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "fold: 2^31 or more elements"); return; }
+    if (num_els == 0) { set_status(ERR_INVALID, "fold: empty input"); return; }
+    sp.fold_stride = (int64_t)strides[fold_dim];
+    sp.window_stride = (int64_t)strides[window_dim];
+    sp.n_windows = (uint32_t)dims[fold_dim];
+    sp.window = (uint32_t)dims[window_dim];
+    sp.step = (uint32_t)step;
+    hipLaunchKernelGGL(fold_kernel<T>, dim3(cdiv(out_size, RB)), dim3(RB), 0, stream(), sp, in + offset, out, out_size, num_els);
+    MXH_LAUNCH_CHECK("fold");
+}
+
 }  // namespace mxh
 
 using namespace mxh;
@@ -676,6 +763,9 @@ using namespace mxh;
     }                                                                                                           \
     extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {        \
         sum_to_shape<T>(n, nd, md, in, out);                                                                    \
+    }                                                                                                           \
+    extern "C" void hip_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {                \
+        fold<T>(n, nd, md, in, out);                                                                            \
     }
 
 MXH_REDUCE_FOR(float, f32)

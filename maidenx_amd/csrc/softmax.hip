@@ -1,0 +1,261 @@
+// Softmax along one dim.  Replaces cuda_softmax_<T> of crates/maidenx_cuda/src/nn/activation/softmax.rs
+// with the CPU semantics of crates/maidenx_cpu/src/nn/activation/softmax.rs:62-207.
+// Metadata: dims[n] | strides[n] | offset; `dim` out of range means the last dim (:74).
+// Per slice: m = max from -inf with `x > m` (NaNs never win), s = exp(-inf - m) + sum exp(x - m),
+// out = exp(x - m) / s, written contiguously.  The maximum is exact; the sum is taken in f32 in a fixed
+// tree order (the reference adds sequentially in the storage dtype), so results carry the tolerance of
+// a reduction.  bf16 rounds x - m, exp and the final quotient like the reference does and keeps only the
+// sum in f32.
+//   contiguous, dim last : a wave (rows up to 2048) or a block per row; 16-byte loads, the row is held in
+//                          registers between the three phases when it fits.
+//   contiguous, dim inner: lanes run along the trailing dims (coalesced), each walks its column 3 times.
+//   strided input        : one thread per slice with the reference's index rule (:120-136, the leading
+//                          dims are decomposed from dim 0 upwards).
+#include "elementwise.hpp"
+#include "mathfn.hpp"
+#include "mxh.hpp"
+
+namespace mxh {
+
+template <class T> struct SM;
+template <> struct SM<float> {
+    static __device__ float ld(float v) { return v; }
+    static __device__ float shifted(float x, float m) { return m_exp(x - m); }     // exp(x - m)
+    static __device__ float fin(float e, float s) { return e / s; }
+};
+template <> struct SM<bf16_t> {
+    static __device__ float ld(bf16_t v) { return bf2f(v); }
+    static __device__ float shifted(float x, float m) { return bf2f(f2bf(m_exp(bf2f(f2bf(x - m))))); }
+    static __device__ bf16_t fin(float e, float s) { return f2bf(e / bf2f(f2bf(s))); }
+};
+
+constexpr int SB = 256;
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float o = __shfl_xor(v, off, WAVE);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+// rows of length D, TPR threads per row (WAVE or SB); NREG vectors of the row live in registers, longer
+// rows are read again from cache in each phase
+template <class T, int TPR, int VEC, int NREG>
+__global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ in, T* __restrict__ out, size_t rows, size_t D) {
+    constexpr int RPB = SB / TPR;
+    const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / TPR;
+    const unsigned t = threadIdx.x % TPR;
+    const bool live = row < rows;
+    const T* src = in + (live ? row : 0) * D;
+    T* dst = out + (live ? row : 0) * D;
+    __shared__ float red[SB / WAVE];
+    AVec<T, VEC> keep[NREG];
+    const size_t step = (size_t)TPR * VEC;
+    const bool fits = D <= step * NREG;
+
+    float m = -INFINITY;
+    if (live) {
+        if (fits) {
+#pragma unroll
+            for (int k = 0; k < NREG; ++k) {
+                size_t i = (size_t)t * VEC + k * step;
+                if (i < D) {
+                    if constexpr (VEC > 1) keep[k] = *(const AVec<T, VEC>*)(src + i);
+                    else keep[k].v[0] = src[i];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(keep[k].v[e]); m = x > m ? x : m; }
+                }
+            }
+        } else {
+            for (size_t i = (size_t)t * VEC; i < D; i += step) {
+                AVec<T, VEC> v;
+                if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
+                else v.v[0] = src[i];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(v.v[e]); m = x > m ? x : m; }
+            }
+        }
+    }
+    m = wave_max(m);
+    if constexpr (TPR > WAVE) {
+        if (threadIdx.x % WAVE == 0) red[threadIdx.x / WAVE] = m;
+        __syncthreads();
+        m = red[0];
+#pragma unroll
+        for (int w = 1; w < SB / WAVE; ++w) m = red[w] > m ? red[w] : m;
+        __syncthreads();
+    }
+
+    float s = 0.0f;
+    if (live) {
+        if (fits) {
+#pragma unroll
+            for (int k = 0; k < NREG; ++k) {
+                size_t i = (size_t)t * VEC + k * step;
+                if (i < D) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) s += SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m);
+                }
+            }
+        } else {
+            for (size_t i = (size_t)t * VEC; i < D; i += step) {
+                AVec<T, VEC> v;
+                if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
+                else v.v[0] = src[i];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s += SM<T>::shifted(SM<T>::ld(v.v[e]), m);
+            }
+        }
+    }
+    s = wave_sum(s);
+    if constexpr (TPR > WAVE) {
+        if (threadIdx.x % WAVE == 0) red[threadIdx.x / WAVE] = s;
+        __syncthreads();
+        s = red[0];
+#pragma unroll
+        for (int w = 1; w < SB / WAVE; ++w) s += red[w];
+    }
+    s = m_exp(-INFINITY - m) + s;      // 0, or NaN when no element beat -inf
+
+    if (!live) return;
+    if (fits) {
+#pragma unroll
+        for (int k = 0; k < NREG; ++k) {
+            size_t i = (size_t)t * VEC + k * step;
+            if (i < D) {
+                AVec<T, VEC> o;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m), s);
+                if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
+                else dst[i] = o.v[0];
+            }
+        }
+    } else {
+        for (size_t i = (size_t)t * VEC; i < D; i += step) {
+            AVec<T, VEC> v, o;
+            if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
+            else v.v[0] = src[i];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(v.v[e]), m), s);
+            if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
+            else dst[i] = o.v[0];
+        }
+    }
+}
+
+// [pre, D, post] contiguous, post > 1: one thread per (pre, post) column
+template <class T>
+__global__ __launch_bounds__(SB) void softmax_col_kernel(const T* __restrict__ in, T* __restrict__ out, size_t slices, size_t D,
+                                                         size_t post) {
+    size_t s_id = (size_t)blockIdx.x * SB + threadIdx.x;
+    if (s_id >= slices) return;
+    size_t pre_idx = s_id / post, post_idx = s_id % post;
+    const T* src = in + pre_idx * D * post + post_idx;
+    T* dst = out + pre_idx * D * post + post_idx;
+    float m = -INFINITY;
+    for (size_t i = 0; i < D; ++i) { float x = SM<T>::ld(src[i * post]); m = x > m ? x : m; }
+    float s = 0.0f;
+    for (size_t i = 0; i < D; ++i) s += SM<T>::shifted(SM<T>::ld(src[i * post]), m);
+    s = m_exp(-INFINITY - m) + s;
+    for (size_t i = 0; i < D; ++i) dst[i * post] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(src[i * post]), m), s);
+}
+
+struct SoftmaxStrided {
+    int nd, dim;
+    uint32_t dims[MAXD];
+    int64_t strides[MAXD];
+};
+
+template <class T>
+__global__ __launch_bounds__(SB) void softmax_strided_kernel(SoftmaxStrided sp, const T* __restrict__ in, T* __restrict__ out,
+                                                             size_t slices, size_t D, size_t post) {
+    size_t s_id = (size_t)blockIdx.x * SB + threadIdx.x;
+    if (s_id >= slices) return;
+    size_t pre_idx = s_id / post, post_idx = s_id % post;
+    int64_t base = 0;
+    {
+        size_t rem = pre_idx;
+        for (int d = 0; d < sp.dim; ++d) { base += (int64_t)(rem % sp.dims[d]) * sp.strides[d]; rem /= sp.dims[d]; }
+        rem = post_idx;
+        for (int d = sp.nd - 1; d > sp.dim; --d) { base += (int64_t)(rem % sp.dims[d]) * sp.strides[d]; rem /= sp.dims[d]; }
+    }
+    const int64_t st = sp.strides[sp.dim];
+    T* dst = out + pre_idx * D * post + post_idx;
+    float m = -INFINITY;
+    for (size_t i = 0; i < D; ++i) { float x = SM<T>::ld(in[base + (int64_t)i * st]); m = x > m ? x : m; }
+    float s = 0.0f;
+    for (size_t i = 0; i < D; ++i) s += SM<T>::shifted(SM<T>::ld(in[base + (int64_t)i * st]), m);
+    s = m_exp(-INFINITY - m) + s;
+    for (size_t i = 0; i < D; ++i) dst[i * post] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(in[base + (int64_t)i * st]), m), s);
+}
+
+template <class T>
+void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const T* in, T* out) {
+    if (!md || !in || !out) return;       // the reference returns silently (:66-68)
+    if (nd == 0 || num_els == 0) return;
+    const size_t dim = dim_arg >= nd ? nd - 1 : dim_arg;
+    const size_t* dims = md;
+    const size_t* strides = md + nd;
+    const size_t offset = md[2 * nd];
+    size_t pre = 1, post = 1;
+    for (size_t d = 0; d < dim; ++d) pre *= dims[d];
+    for (size_t d = dim + 1; d < nd; ++d) post *= dims[d];
+    const size_t D = dims[dim], slices = pre * post;
+    if (D == 0 || slices == 0) return;
+    bool cont = true;       // the strict test of softmax.rs:88-100
+    {
+        size_t acc = 1;
+        for (size_t d = nd; d-- > 0;) {
+            if (strides[d] != acc) { cont = false; break; }
+            acc *= dims[d];
+        }
+    }
+    const T* src = in + offset;
+    if (cont && post == 1) {
+        constexpr int VEC = 16 / sizeof(T);
+        const bool vec = D % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)out % 16) == 0;
+        if (D <= 2048) {
+            unsigned blocks = cdiv(slices, SB / WAVE);
+            if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, VEC, 2048 / (WAVE * VEC)>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
+            else hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, 1, 8>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
+        } else {
+            if (slices >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "softmax: too many rows"); return; }
+            if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, SB, VEC, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
+            else hipLaunchKernelGGL((softmax_row_kernel<T, SB, 1, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
+        }
+        MXH_LAUNCH_CHECK("softmax_row");
+        return;
+    }
+    if (cont) {
+        hipLaunchKernelGGL(softmax_col_kernel<T>, dim3(cdiv(slices, SB)), dim3(SB), 0, stream(), src, out, slices, D, post);
+        MXH_LAUNCH_CHECK("softmax_col");
+        return;
+    }
+    if (nd > (size_t)MAXD) { set_status(ERR_UNSUPPORTED, "softmax: strided input of rank above 8"); return; }
+    SoftmaxStrided sp;
+    sp.nd = (int)nd; sp.dim = (int)dim;
+    for (int d = 0; d < MAXD; ++d) {
+        sp.dims[d] = d < (int)nd ? (uint32_t)dims[d] : 1;
+        sp.strides[d] = d < (int)nd ? (int64_t)strides[d] : 0;
+    }
+    hipLaunchKernelGGL(softmax_strided_kernel<T>, dim3(cdiv(slices, SB)), dim3(SB), 0, stream(), sp, src, out, slices, D, post);
+    MXH_LAUNCH_CHECK("softmax_strided");
+}
+
+}  // namespace mxh
+
+using namespace mxh;
+
+extern "C" void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const float* in, float* out) {
+    softmax<float>(num_els, num_dims, dim, md, in, out);
+}
+extern "C" void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const bf16_t* in, bf16_t* out) {
+    softmax<bf16_t>(num_els, num_dims, dim, md, in, out);
+}

@@ -2,6 +2,7 @@
 // Metadata layouts:
 //   sum/mean/max/min (reduction.rs:28-32): dims[n] | strides[n] | red_len[r] | red_stride[r] | offset
 //   sum_to_shape     (reduction.rs:111-114): in_dims[n] | in_strides[n] | out_dims[n] | offset
+//   fold             (reduction.rs:298-305): dims[n] | strides[n] | fold_dim, window_dim, fold_size, step, window_size, offset
 // The reference accumulates in the storage dtype, one locked `+=` per input element, in
 // whatever order rayon schedules.  With one thread this restatement visits input elements
 // in ascending logical order (the order a single-threaded rayon pool yields); with several
@@ -114,6 +115,47 @@ void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in
     for (size_t i = 0; i < out_size; ++i) out[i] = cells[i].val;
 }
 
+// fold_op! (reduction.rs:274-380): the adjoint of unfold.  Input element with coordinates c adds to the
+// output at c with the window dim dropped and the fold dim replaced by c[fold_dim]*step + c[window_dim]
+// (skipped when that is >= fold_size).  The source index is (sum c*stride) % num_els of the slice that
+// starts at `offset` (:336-340), contiguous or not.
+// metadata: dims[n] | strides[n] | fold_dim, window_dim, fold_size, step, window_size, offset
+template <typename T>
+void fold(size_t num_els, size_t nd, const size_t* md, const T* inp, T* out) {
+    const size_t* dims = md;
+    const size_t* strides = md + nd;
+    const size_t fold_dim = md[2 * nd], window_dim = md[2 * nd + 1], fold_size = md[2 * nd + 2], step = md[2 * nd + 3];
+    const size_t offset = md[2 * nd + 5];
+    const T* in = inp + offset;
+    size_t out_size = 1;
+    for (size_t d = 0; d < nd; ++d) {
+        if (d == window_dim) continue;
+        out_size *= d == fold_dim ? fold_size : dims[d];
+    }
+    std::vector<Cell<T>> cells(out_size);
+    for (auto& c : cells) c.val = zero_of<T>();
+    bool threaded = num_threads() > 1;
+    ORC_PAR_FOR
+    for (size_t i = 0; i < num_els; ++i) {
+        size_t coords[16] = {0};
+        size_t tmp = i;
+        for (size_t d = nd; d-- > 0;) { coords[d] = tmp % dims[d]; tmp /= dims[d]; }
+        size_t src = 0;
+        for (size_t d = 0; d < nd; ++d) src += coords[d] * strides[d];
+        src %= num_els;
+        size_t pos = coords[fold_dim] * step + coords[window_dim];
+        if (pos >= fold_size) continue;
+        size_t dst = 0;
+        for (size_t d = 0; d < nd; ++d) {
+            if (d == window_dim) continue;
+            dst = d == fold_dim ? dst * fold_size + pos : dst * dims[d] + coords[d];
+        }
+        T v = in[src];
+        locked(cells[dst], threaded, [&](T& o) { o += v; });
+    }
+    for (size_t i = 0; i < out_size; ++i) out[i] = cells[i].val;
+}
+
 }  // namespace
 
 #define ORC_REDUCE_FOR(T, SUF)                                                                                  \
@@ -137,6 +179,9 @@ void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in
     }                                                                                                           \
     extern "C" void oracle_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {     \
         sum_to_shape<T>(n, nd, md, in, out);                                                                    \
+    }                                                                                                           \
+    extern "C" void oracle_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {             \
+        fold<T>(n, nd, md, in, out);                                                                            \
     }
 
 ORC_REDUCE_FOR(float, f32)

@@ -7,7 +7,7 @@ import os
 import numpy as np
 
 from helpers import (In, InOut, Out, const_arg, contiguous_strides, meta_binary, meta_matmul, meta_pad, meta_reduce,
-                     meta_sum_to_shape, meta_unary, to_float, to_storage)
+                     meta_sum_to_shape, meta_unary, to_float, to_storage, u64)
 
 KAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kat.json")))
 
@@ -167,4 +167,42 @@ def run_pad(be, dt):
         check(gi[1:-1], c["grad"], dt, 0)
 
 
-ALL = [run_binary, run_compare, run_inplace, run_unary, run_unary_const, run_reduce, run_sum_to_shape, run_matmul, run_pad]
+def run_pad_edge(be, dt):
+    for c in KAT["pad_edge"]:
+        shape, pads = c["shape"], c["pads"]
+        out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+        n_in, n_out = int(np.prod(shape)), int(np.prod(out_shape))
+        md = meta_pad(shape, contiguous_strides(shape), 1, out_shape, pads)
+        (out,) = be.call(f"pad_with_{c['mode']}_{dt}", n_in, n_out, len(shape), md, In(padded(c["data"], dt)), Out(n_out, dt))
+        assert np.array_equal(to_float(out, dt), np.array(c["expect"], dtype=np.float32))
+        if "grad" in c:
+            go = to_storage(np.ones(n_out, dtype=np.float32), dt)
+            gi = padded(np.full(n_in, 7.0), dt)
+            (gi,) = be.call(f"pad_with_{c['mode']}_backward_{dt}", n_in, n_out, len(shape), md, In(go), InOut(gi))
+            check(gi[1:-1], c["grad"], dt, 0)
+
+
+def run_fold(be, dt):
+    for c in KAT["fold"]:
+        dims = c["dims"]
+        n = int(np.prod(dims))
+        md = u64(dims, c["strides"], c["fold_dim"], c["window_dim"], c["fold_size"], c["step"], dims[c["window_dim"]], 1)
+        # the unfolded view shares the 5- or 6-element buffer; the kernel may index up to num_els of it
+        data = np.concatenate([padded(c["data"], dt), to_storage(np.zeros(n, np.float32), dt)])
+        (out,) = be.call(f"fold_{dt}", n, len(dims), md, In(data), Out(len(c["expect"]), dt))
+        check(out, c["expect"], dt, 0)
+
+
+def run_softmax(be, dt):
+    for c in KAT["softmax"]:
+        shape = c["shape"]
+        n = int(np.prod(shape))
+        md = meta_unary(shape, contiguous_strides(shape), 1)
+        (out,) = be.call(f"softmax_{dt}", n, len(shape), c["dim"], md, In(padded(c["data"], dt)), Out(n, dt))
+        y = to_float(out, dt).astype(np.float64).reshape(shape)
+        tol = 1e-5 if dt != "bf16" else 2e-2
+        assert np.all(np.abs(y.sum(axis=c["dim"]) - 1.0) < tol), y
+        assert np.all(np.diff(y, axis=c["dim"]) > 0), y
+
+
+ALL = [run_pad_edge, run_fold, run_softmax, run_binary, run_compare, run_inplace, run_unary, run_unary_const, run_reduce, run_sum_to_shape, run_matmul, run_pad]

@@ -7,7 +7,7 @@ import pytest
 
 import layouts as LY
 from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
-                     meta_matmul, meta_pad, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
+                     meta_matmul, meta_pad, u64, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
                      ulp_diff_f32)
 
 pytestmark = pytest.mark.gpu
@@ -495,6 +495,135 @@ def test_col2im_row_stride_two_column_stride_one(oracle, hip, k, dt):
     for num_els in (n_col, n_col // 2 + 3):
         (o,), (h,) = both(oracle, hip, f"conv2d_col2im_{dt}", lambda: (num_els, md, In(y), Out(B * Cc * H * W, dt)))
         assert same_bits(o, h), num_els
+
+
+# ---------------------------------------------------------------------------------------------------
+# reflection / replication padding, fold, softmax
+# ---------------------------------------------------------------------------------------------------
+EDGE_CASES = [([7], [(3, 2)]), ([5, 6], [(1, 2), (0, 3)]), ([2, 3, 4], [(1, 0), (2, 2), (3, 1)]), ([4, 9], [(0, 0), (4, 8)]),
+              ([3], [(7, 5)]), ([2, 3, 20, 24], [(0, 0), (0, 0), (3, 3), (2, 5)]), ([1, 6], [(0, 0), (2, 2)])]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("mode", ["reflection", "replication"])
+@pytest.mark.parametrize("shape,pads", EDGE_CASES)
+def test_pad_edge_forward_backward(oracle, hip, shape, pads, mode, dt):
+    r = rng(103)
+    out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+    n_in, n_out = int(np.prod(shape)), int(np.prod(out_shape))
+    st = to_storage(np.concatenate([[9.0], r.standard_normal(n_in)]).astype(np.float32), dt)
+    md = meta_pad(shape, contiguous_strides(shape), 1, out_shape, pads)
+    (o,), (h,) = both(oracle, hip, f"pad_with_{mode}_{dt}", lambda: (n_in, n_out, len(shape), md, In(st), Out(n_out, dt)))
+    assert same_bits(o, h)
+    go = to_storage(r.standard_normal(n_out).astype(np.float32), dt)
+    (o,), (h,) = both(oracle, hip, f"pad_with_{mode}_backward_{dt}",
+                      lambda: (n_in, n_out, len(shape), md, In(go), InOut(to_storage(np.full(n_in + 2, 7.0, np.float32), dt))))
+    if dt == "f32":
+        assert same_bits(o, h)          # same terms in the same (ascending output) order
+    else:
+        # the reference rounds after every add, the kernel once: compare with the exact sums
+        assert same_bits(o[:1], h[:1]) and same_bits(o[n_in + 1:], h[n_in + 1:])
+        g64 = to_float(go, dt).astype(np.float64).reshape(out_shape)
+        np_mode = "reflect" if mode == "reflection" else "edge"
+        idx = np.pad(np.arange(n_in).reshape(shape), pads, mode=np_mode).ravel()
+        truth = np.bincount(idx, weights=g64.ravel(), minlength=n_in)
+        scale = np.bincount(idx, weights=np.abs(g64).ravel(), minlength=n_in)
+        assert np.max(np.abs(to_float(h, dt)[1:n_in + 1] - truth) / np.maximum(scale, 1e-30)) <= 1e-2
+
+
+@pytest.mark.parametrize("mode", ["reflection", "replication"])
+def test_pad_edge_transposed_input(oracle, hip, mode):
+    lay = LY.permuted([6, 9], [1, 0])
+    r = rng(107)
+    st = r.standard_normal(54).astype(np.float32)
+    pads = [(2, 1), (3, 4)]
+    md = meta_pad([6, 9], lay["strides"], 0, [9, 16], pads)
+    (o,), (h,) = both(oracle, hip, f"pad_with_{mode}_f32", lambda: (54, 144, 2, md, In(st), Out(144, "f32")))
+    assert same_bits(o, h)
+    go = r.standard_normal(144).astype(np.float32)
+    (o,), (h,) = both(oracle, hip, f"pad_with_{mode}_backward_f32", lambda: (54, 144, 2, md, In(go), InOut(np.full(54, 7.0, np.float32))))
+    assert same_bits(o, h)
+
+
+def test_pad_reflection_of_a_size_one_dim_is_refused(hip):
+    md = meta_pad([1, 4], [4, 1], 0, [3, 4], [(1, 1), (0, 0)])
+    with pytest.raises(Exception):
+        hip.call("pad_with_reflection_f32", 4, 12, 2, md, In(np.ones(4, np.float32)), Out(12, "f32"))
+
+
+FOLD_CASES = [([4, 2], [1, 1], 0, 1, 5, 1), ([2, 2, 2], [3, 1, 1], 1, 2, 3, 1), ([30, 7], [3, 1], 0, 1, 94, 3), ([5, 40, 6, 3], None, 1, 2, 84, 2),
+              ([6, 5, 9], None, 1, 0, 20, 3), ([50, 4], None, 0, 1, 4, 0)]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("dims,strides,fd,wd,fold_size,step", FOLD_CASES)
+def test_fold(oracle, hip, dims, strides, fd, wd, fold_size, step, dt):
+    r = rng(109)
+    n = int(np.prod(dims))
+    strides = strides or contiguous_strides(dims)
+    x = to_storage(r.standard_normal(n + 1).astype(np.float32), dt)
+    md = u64(dims, strides, fd, wd, fold_size, step, dims[wd], 1)
+    out_n = int(np.prod([fold_size if d == fd else v for d, v in enumerate(dims) if d != wd]))
+    (o,), (h,) = both(oracle, hip, f"fold_{dt}", lambda: (n, len(dims), md, In(x), Out(out_n, dt)))
+    if dt == "f32" and fd < wd:
+        assert same_bits(o, h)          # windows are added in ascending order by both
+    else:
+        a, b = to_float(o, dt).astype(np.float64), to_float(h, dt).astype(np.float64)
+        assert np.max(np.abs(a - b)) <= (1e-5 if dt == "f32" else 6e-2) * max(1.0, np.max(np.abs(a)))
+
+
+SOFTMAX_CASES = [([2, 3], 1), ([2, 2, 3], 2), ([2, 3], 0), ([64, 5], 1), ([33, 2048], 1), ([9, 2052], 1), ([3, 40000], 1), ([7, 300], 1),
+                 ([6, 50, 130], 1), ([4, 3, 5, 6], 0), ([5, 6], 7), ([10000], 0)]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,dim", SOFTMAX_CASES)
+def test_softmax(oracle, hip, shape, dim, dt):
+    from scipy.special import softmax as sp_softmax
+    r = rng(113)
+    n = int(np.prod(shape))
+    x = to_storage((r.standard_normal(n) * 3).astype(np.float32), dt)
+    md = meta_unary(shape, contiguous_strides(shape), 0)
+    (o,), (h,) = both(oracle, hip, f"softmax_{dt}", lambda: (n, len(shape), dim, md, In(x), Out(n, dt)))
+    axis = dim if dim < len(shape) else len(shape) - 1
+    truth = sp_softmax(to_float(x, dt).astype(np.float64).reshape(shape), axis=axis).ravel()
+    got = to_float(h, dt).astype(np.float64)
+    if dt == "f32":
+        assert np.all(np.abs(got - truth) <= 1e-5 * truth + 1e-30)
+        # the reference's own sequential f32 sum drifts from the exact value by about sqrt(D) roundings
+        ref_tol = max(1e-5, 4 * np.sqrt(shape[axis]) * 2.0 ** -24)
+        assert np.all(np.abs(got - to_float(o, dt)) <= ref_tol * truth + 1e-30)
+    else:
+        # bf16 rounds x - max and exp like the reference; only the sum differs: the reference's bf16 running sum
+        # stalls on long slices, the kernel sums in f32.  Compare with the exact sum of the same rounded terms.
+        xf = to_float(x, dt).reshape(shape)
+        t = bf16_to_f32(f32_to_bf16(xf - xf.max(axis=axis, keepdims=True)))
+        e = bf16_to_f32(f32_to_bf16(np.exp(t))).astype(np.float64)
+        truth = (e / e.sum(axis=axis, keepdims=True)).ravel()
+        assert np.all(np.abs(got - truth) <= 1e-2 * truth + 1e-30)
+        if shape[axis] <= 8:
+            assert np.max(np.abs(got - to_float(o, dt))) <= 2.0 ** -7
+
+
+def test_softmax_strided_and_special_values(oracle, hip):
+    r = rng(127)
+    lay = LY.permuted([6, 9], [1, 0], off=2)
+    st = np.concatenate([np.zeros(2), r.standard_normal(54)]).astype(np.float32)
+    for dim in (0, 1):
+        md = meta_unary([6, 9], lay["strides"], lay["off"])
+        (o,), (h,) = both(oracle, hip, "softmax_f32", lambda: (54, 2, dim, md, In(st), Out(54, "f32")))
+        assert np.allclose(o, h, rtol=1e-5, atol=0)
+    # three leading dims, permuted: the reference's own (dim 0 fastest) walk of the leading dims
+    lay = LY.permuted([3, 4, 5, 6], [2, 0, 3, 1])
+    st = r.standard_normal(360).astype(np.float32)
+    md = meta_unary([3, 4, 5, 6], lay["strides"], 0)
+    for dim in (1, 2, 3):
+        (o,), (h,) = both(oracle, hip, "softmax_f32", lambda: (360, 4, dim, md, In(st), Out(360, "f32")))
+        assert np.allclose(o, h, rtol=1e-5, atol=0)
+    v = np.array([[0.0, -np.inf, 1.0], [-np.inf, -np.inf, -np.inf], [np.nan, 1.0, 2.0], [np.inf, 1.0, 2.0]], dtype=np.float32)
+    (o,), (h,) = both(oracle, hip, "softmax_f32", lambda: (12, 2, 1, meta_unary([4, 3], [3, 1], 0), In(v.ravel()), Out(12, "f32")))
+    assert np.array_equal(np.isnan(o), np.isnan(h))
+    assert np.allclose(o[~np.isnan(o)], h[~np.isnan(o)], rtol=1e-6)
 
 
 # ---------------------------------------------------------------------------------------------------

@@ -259,3 +259,115 @@ def test_oracle_threaded_mode_agrees_with_sequential(oracle):
         oracle.set_threads(1)
     assert np.array_equal(seq, par)
     assert np.allclose(s1, s4, atol=1e-5)
+
+
+# ---- reflection / replication padding, fold, softmax -------------------------------------------------
+EDGE_CASES = [([7], [(3, 2)]), ([5, 6], [(1, 2), (0, 3)]), ([2, 3, 4], [(1, 0), (2, 2), (3, 1)]), ([4, 9], [(0, 0), (4, 8)])]
+
+
+@pytest.mark.parametrize("mode,np_mode", [("reflection", "reflect"), ("replication", "edge")])
+@pytest.mark.parametrize("shape,pads", EDGE_CASES)
+def test_oracle_edge_pad_vs_numpy_pad_and_adjoint(oracle, shape, pads, mode, np_mode):
+    r = rng(83)
+    x = r.standard_normal(shape)
+    out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+    n_in, n_out = x.size, int(np.prod(out_shape))
+    md = meta_pad(shape, contiguous_strides(shape), 0, out_shape, pads)
+    (y,) = oracle.call(f"pad_with_{mode}_f64", n_in, n_out, len(shape), md, In(x.ravel()), Out(n_out, "f64"))
+    assert np.array_equal(y.reshape(out_shape), np.pad(x, pads, mode=np_mode))      # numpy's own pad
+    # a transposed (strided) input reads the same logical tensor
+    if len(shape) == 2:
+        lay = LY.permuted(shape, [1, 0])
+        st = np.ascontiguousarray(x.T).ravel()
+        assert np.array_equal(LY.gather(st, lay), x)
+        mds = meta_pad(shape, lay["strides"], 0, out_shape, pads)
+        (ys,) = oracle.call(f"pad_with_{mode}_f64", n_in, n_out, 2, mds, In(st), Out(n_out, "f64"))
+        assert np.array_equal(ys, y)
+    # backward is the adjoint: <pad(x), g> = <x, pad_backward(g)>
+    g = r.standard_normal(n_out)
+    (gx,) = oracle.call(f"pad_with_{mode}_backward_f64", n_in, n_out, len(shape), md, In(g), InOut(np.full(n_in, 9.0)))
+    assert abs(np.dot(y, g) - np.dot(x.ravel(), gx)) <= 1e-9 * (np.abs(y * g).sum() + 1)
+
+
+def test_oracle_reflection_wraps_more_than_once(oracle):
+    # pads wider than the dim: the mirror loop of padding.rs:186-193 runs several times; numpy's reflect does the same
+    x = np.arange(1.0, 4.0)
+    md = meta_pad([3], [1], 0, [3 + 7 + 5], [(7, 5)])
+    (y,) = oracle.call("pad_with_reflection_f64", 3, 15, 1, md, In(x), Out(15, "f64"))
+    assert np.array_equal(y, np.pad(x, (7, 5), mode="reflect"))
+
+
+@pytest.mark.parametrize("shape,dim,size,step", [([9], 0, 3, 2), ([4, 10], 1, 4, 3), ([3, 8, 2], 1, 2, 1), ([6, 5], 0, 3, 3)])
+def test_oracle_fold_is_adjoint_of_unfold(oracle, shape, dim, size, step):
+    from numpy.lib.stride_tricks import sliding_window_view
+    r = rng(89)
+    x = r.standard_normal(shape)
+    # unfold as Layout::unfold builds it (layout.rs:193-250): windows at `dim`, the window dim right after
+    win = np.moveaxis(sliding_window_view(x, size, axis=dim), -1, dim + 1)
+    win = np.take(win, np.arange(0, win.shape[dim], step), axis=dim)
+    y = r.standard_normal(win.shape)
+    n_windows = win.shape[dim]
+    fold_size = (n_windows - 1) * step + size                  # tensor/ops/reduction.rs:257
+    md = u64_(list(win.shape), contiguous_strides(list(win.shape)), dim, dim + 1, fold_size, step, size, 0)
+    out_shape = list(shape)
+    out_shape[dim] = fold_size
+    (f,) = oracle.call("fold_f64", y.size, y.ndim, md, In(y.ravel()), Out(int(np.prod(out_shape)), "f64"))
+    xs = np.take(x, np.arange(fold_size), axis=dim)            # the part of x the windows cover
+    assert abs(np.sum(win * y) - np.sum(xs * f.reshape(out_shape))) <= 1e-9 * (np.abs(win * y).sum() + 1)
+    # and fold(unfold(x)) multiplies every position by the number of windows that contain it
+    (fx,) = oracle.call("fold_f64", win.size, win.ndim, md, In(np.ascontiguousarray(win).ravel()), Out(int(np.prod(out_shape)), "f64"))
+    (cnt,) = oracle.call("fold_f64", win.size, win.ndim, md, In(np.ones(win.size)), Out(int(np.prod(out_shape)), "f64"))
+    assert np.allclose(fx.reshape(out_shape), xs * cnt.reshape(out_shape), rtol=1e-12)
+
+
+def u64_(*parts):
+    from helpers import u64
+    return u64(*parts)
+
+
+@pytest.mark.parametrize("shape,dim", [([5, 7], 1), ([5, 7], 0), ([3, 4, 6], 1), ([2, 3, 4, 5], 3), ([2, 3, 4, 5], 0), ([6], 0), ([4, 3], 9)])
+def test_oracle_softmax_vs_scipy(oracle, shape, dim):
+    from scipy.special import softmax as sp_softmax
+    r = rng(97)
+    x = r.standard_normal(shape) * 3
+    n = x.size
+    md = meta_unary(shape, contiguous_strides(shape), 0)
+    (y,) = oracle.call("softmax_f64", n, len(shape), dim, md, In(x.ravel()), Out(n, "f64"))
+    axis = dim if dim < len(shape) else len(shape) - 1          # out of range means the last dim (softmax.rs:74)
+    assert np.allclose(y.reshape(shape), sp_softmax(x, axis=axis), rtol=1e-12, atol=0)
+    (y32,) = oracle.call("softmax_f32", n, len(shape), dim, md, In(x.astype(np.float32).ravel()), Out(n, "f32"))
+    assert np.allclose(y32.reshape(shape), sp_softmax(x.astype(np.float32).astype(np.float64), axis=axis), rtol=2e-6)
+
+
+def test_oracle_softmax_strided_two_dims_and_special_values(oracle):
+    from scipy.special import softmax as sp_softmax
+    r = rng(101)
+    x = r.standard_normal((6, 9))
+    lay = LY.permuted([6, 9], [1, 0], off=2)
+    st = np.concatenate([np.zeros(2), np.ascontiguousarray(x.T).ravel()])
+    assert np.array_equal(LY.gather(st, lay), x)
+    for dim in (0, 1):
+        md = meta_unary([6, 9], lay["strides"], lay["off"])
+        (y,) = oracle.call("softmax_f64", 54, 2, dim, md, In(st), Out(54, "f64"))
+        assert np.allclose(y.reshape(6, 9), sp_softmax(x, axis=dim), rtol=1e-12)
+    # -inf entries vanish, an all -inf slice is NaN (the sum starts from exp(-inf - -inf)), NaNs never become the maximum
+    v = np.array([[0.0, -np.inf, 1.0], [-np.inf, -np.inf, -np.inf], [np.nan, 1.0, 2.0]], dtype=np.float32)
+    (y,) = oracle.call("softmax_f32", 9, 2, 1, meta_unary([3, 3], [3, 1], 0), In(v.ravel()), Out(9, "f32"))
+    y = y.reshape(3, 3)
+    assert y[0, 1] == 0 and abs(y[0, 0] + y[0, 2] - 1) < 1e-6
+    assert np.all(np.isnan(y[1]))
+    assert np.isnan(y[2, 0]) and np.all(np.isnan(y[2]))        # exp(NaN - max) poisons the sum
+
+
+def test_oracle_softmax_bf16_rounds_every_step(oracle):
+    x = f32_to_bf16(np.array([0.1, 1.3, -0.7, 2.2], dtype=np.float32))
+    (y,) = oracle.call("softmax_bf16", 4, 1, 0, meta_unary([4], [1], 0), In(x), Out(4, "bf16"))
+    b = lambda v: bf16_to_f32(f32_to_bf16(np.float32(v)))
+    xf = bf16_to_f32(x)
+    m = xf.max()
+    e = [b(np.exp(np.float32(b(v - m)))) for v in xf]
+    s = np.float32(0)
+    for t in e:
+        s = b(s + t)
+    want = f32_to_bf16(np.array([t / s for t in e], dtype=np.float32)).ravel()
+    assert np.array_equal(y, want)
