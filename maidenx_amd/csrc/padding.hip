@@ -237,6 +237,12 @@ __global__ __launch_bounds__(PB) void pad_edge_kernel(PadSpace sp, int mode, con
     dst[i] = src[idx];
 }
 
+// what the backward walk needs besides the PadSpace: how to split an input index, where an output coordinate lands
+struct EdgeWalk {
+    FastDiv in_div[MAXD];
+    int64_t out_strides[MAXD];
+};
+
 // Ascending enumeration of the output coordinates of one dim that map to input coordinate p.
 struct EdgeIter {
     int64_t a, b, hi, period;       // next candidates of the two progressions, last coordinate, step
@@ -271,74 +277,82 @@ struct EdgeIter {
     }
 };
 
+// The dims are walked by compile-time recursion (coordinates and iterators stay in registers): dim D loops
+// over the output coordinates that map to p[D], the innermost level adds one gradient.
+template <class T, int D>
+__device__ __forceinline__ void edge_gather(const PadSpace& sp, const EdgeWalk& w, int mode, const uint32_t (&p)[MAXD], int64_t o,
+                                            const T* __restrict__ go, float& acc) {
+    if constexpr (D == MAXD) {
+        if constexpr (sizeof(T) == 4) acc += go[o];
+        else acc += bf2f(go[o]);
+    } else {
+        if (D >= sp.ndims) { edge_gather<T, MAXD>(sp, w, mode, p, o, go, acc); return; }
+        EdgeIter it;
+        for (it.init(mode, p[D], sp.in_dims[D], sp.out_dims[D], sp.before[D]); !it.done(); it.next())
+            edge_gather<T, D + 1>(sp, w, mode, p, o + it.cur() * w.out_strides[D], go, acc);
+    }
+}
+
 template <class T>
-__global__ __launch_bounds__(PB) void pad_edge_backward_kernel(PadSpace sp, int mode, const T* __restrict__ go, T* __restrict__ gi,
-                                                                size_t n_in, PadSpace in_walk) {
-    // in_walk.div / in_walk.out_dims describe the input's logical shape (for the coordinate split)
+__global__ __launch_bounds__(PB) void pad_edge_backward_kernel(PadSpace sp, EdgeWalk w, int mode, const T* __restrict__ go,
+                                                                T* __restrict__ gi, size_t n_in) {
     size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
     if (i >= n_in) return;
     uint32_t p[MAXD];
+    int64_t dst = 0;
     {
         uint32_t r = (uint32_t)i;
 #pragma unroll
         for (int d = MAXD - 1; d >= 0; --d) {
             if (d >= sp.ndims) { p[d] = 0; continue; }
             uint32_t q, c;
-            if (d > 0) fd_divmod(r, in_walk.div[d], q, c);
+            if (d > 0) fd_divmod(r, w.in_div[d], q, c);
             else { q = 0; c = r; }
             p[d] = c;
+            dst += (int64_t)c * sp.in_strides[d];
             r = q;
         }
     }
-    int64_t dst = 0;
-    for (int d = 0; d < sp.ndims; ++d) dst += (int64_t)p[d] * sp.in_strides[d];
-    // row-major strides of the output
-    int64_t ost[MAXD];
-    {
-        int64_t acc = 1;
-        for (int d = sp.ndims - 1; d >= 0; --d) { ost[d] = acc; acc *= sp.out_dims[d]; }
-    }
-    EdgeIter it[MAXD];
-    bool empty = false;
-    for (int d = 0; d < sp.ndims; ++d) {
-        it[d].init(mode, p[d], sp.in_dims[d], sp.out_dims[d], sp.before[d]);
-        empty = empty || it[d].done();
-    }
     float acc = 0.0f;
-    if (!empty) {
-        while (true) {
-            int64_t o = 0;
-            for (int d = 0; d < sp.ndims; ++d) o += it[d].cur() * ost[d];
-            if constexpr (sizeof(T) == 4) acc += go[o];
-            else acc += bf2f(go[o]);
-            // odometer: advance the innermost dim, carry outwards
-            int d = sp.ndims - 1;
-            for (; d >= 0; --d) {
-                it[d].next();
-                if (!it[d].done()) break;
-                it[d].init(mode, p[d], sp.in_dims[d], sp.out_dims[d], sp.before[d]);
-            }
-            if (d < 0) break;
-        }
-    }
+    edge_gather<T, 0>(sp, w, mode, p, 0, go, acc);
     if constexpr (sizeof(T) == 4) gi[dst] = acc;
     else gi[dst] = f2bf(acc);
 }
 
-static bool edge_space(size_t nd, const size_t* md, int mode, PadSpace& sp, PadSpace& in_walk, size_t* in_off, const char* who) {
-    // no collapsing: every dim keeps its own mapping
+static bool edge_space(size_t nd_full, const size_t* md_full, int mode, PadSpace& sp, EdgeWalk& in_walk, size_t* in_off, const char* who) {
+    if (nd_full > 64) { set_status(ERR_UNSUPPORTED, who); return false; }
+    *in_off = md_full[2 * nd_full];
+    // Merge runs of dims without padding whose input strides chain (they map to themselves), so that
+    // [B, C, H, W] padded on H and W walks three dims.
+    size_t in_dims[64], st_m[64], out_dims[64], pads[128];
+    size_t nd = 0;
+    {
+        const size_t* fin = md_full;
+        const size_t* fst = md_full + nd_full;
+        const size_t* fout = md_full + 2 * nd_full + 1;
+        const size_t* fp = md_full + 3 * nd_full + 1;
+        bool cont = ref_is_contiguous(nd_full, fin, fst);
+        size_t cs[64];
+        contiguous_strides(nd_full, fin, cs);
+        const size_t* st = cont ? cs : fst;       // padding.rs:199-214: contiguous inputs are indexed row-major
+        for (size_t d = 0; d < nd_full; ++d) {
+            bool plain = fp[2 * d] == 0 && fout[d] == fin[d];
+            if (plain && fin[d] == 1) continue;
+            if (nd > 0 && plain && pads[2 * (nd - 1)] == 0 && out_dims[nd - 1] == in_dims[nd - 1] && st_m[nd - 1] == st[d] * fin[d]) {
+                in_dims[nd - 1] *= fin[d]; out_dims[nd - 1] *= fout[d]; st_m[nd - 1] = st[d];
+            } else {
+                in_dims[nd] = fin[d]; out_dims[nd] = fout[d]; st_m[nd] = st[d]; pads[2 * nd] = fp[2 * d]; pads[2 * nd + 1] = fp[2 * d + 1]; ++nd;
+            }
+        }
+    }
     if (nd > (size_t)MAXD) { set_status(ERR_UNSUPPORTED, who); return false; }
-    const size_t* in_dims = md;
-    const size_t* in_strides = md + nd;
-    *in_off = md[2 * nd];
-    const size_t* out_dims = md + 2 * nd + 1;
-    const size_t* pads = md + 3 * nd + 1;
-    bool cont = ref_is_contiguous(nd, in_dims, in_strides);
-    size_t cs[MAXD];
-    contiguous_strides(nd, in_dims, cs);
-    const size_t* st = cont ? cs : in_strides;       // padding.rs:199-214: contiguous inputs are indexed row-major
+    const size_t* st = st_m;
     sp.ndims = (int)(nd ? nd : 1);
-    in_walk.ndims = sp.ndims;
+    int64_t ost = 1;
+    for (int d = MAXD - 1; d >= 0; --d) {
+        in_walk.out_strides[d] = d < (int)nd ? ost : 0;
+        if (d < (int)nd) ost *= (int64_t)out_dims[d];
+    }
     for (int d = 0; d < MAXD; ++d) {
         bool real = d < (int)nd;
         if (real && (in_dims[d] >= (1ull << 31) || out_dims[d] >= (1ull << 31) || pads[2 * d] >= (1ull << 31))) { set_status(ERR_TOO_LARGE, who); return false; }
@@ -350,10 +364,9 @@ static bool edge_space(size_t nd, const size_t* md, int mode, PadSpace& sp, PadS
         sp.before[d] = real ? (uint32_t)pads[2 * d] : 0;
         sp.in_strides[d] = real ? (int64_t)st[d] : 0;
         sp.div[d] = make_fastdiv(sp.out_dims[d]);
-        in_walk.div[d] = make_fastdiv(sp.in_dims[d]);
+        in_walk.in_div[d] = make_fastdiv(sp.in_dims[d]);
     }
     sp.out_last = sp.in_last = 1; sp.before_last = 0; sp.stride_last = 0; sp.div_last = make_fastdiv(1);
-    in_walk.out_last = in_walk.in_last = 1; in_walk.before_last = 0; in_walk.stride_last = 0; in_walk.div_last = make_fastdiv(1);
     return true;
 }
 
@@ -363,7 +376,7 @@ void pad_edge_forward(int mode, size_t n_in, size_t n_out, size_t nd, const size
     if (!md || !in || !out) { set_status(ERR_INVALID, "pad: null argument"); return; }
     if (n_out == 0) return;
     if (n_out >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad: output of 2^31 or more elements"); return; }
-    PadSpace sp, walk; size_t off;
+    PadSpace sp; EdgeWalk walk; size_t off;
     if (!edge_space(nd, md, mode, sp, walk, &off, "pad_with_reflection/replication: bad shape or rank above 8")) return;
     hipLaunchKernelGGL(pad_edge_kernel<T>, dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, mode, in + off, out, n_out);
     MXH_LAUNCH_CHECK("pad_edge");
@@ -374,7 +387,7 @@ void pad_edge_backward(int mode, size_t n_in, size_t n_out, size_t nd, const siz
     if (!md || !go || !gi) { set_status(ERR_INVALID, "pad_backward: null argument"); return; }
     if (n_in == 0) return;
     if (n_out >= (1ull << 31) || n_in >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad_backward: 2^31 or more elements"); return; }
-    PadSpace sp, walk; size_t off;
+    PadSpace sp; EdgeWalk walk; size_t off;
     if (!edge_space(nd, md, mode, sp, walk, &off, "pad_with_reflection/replication backward: bad shape or rank above 8")) return;
     // the reference writes num_els_in contiguous elements at grad_in + offset: positions a strided
     // layout does not reach hold 0
@@ -386,7 +399,7 @@ void pad_edge_backward(int mode, size_t n_in, size_t n_out, size_t nd, const siz
     size_t logical = 1;
     for (size_t d = 0; d < nd; ++d) logical *= md[d];
     if (logical == 0) return;
-    hipLaunchKernelGGL(pad_edge_backward_kernel<T>, dim3(cdiv(logical, PB)), dim3(PB), 0, stream(), sp, mode, go, gi + off, logical, walk);
+    hipLaunchKernelGGL(pad_edge_backward_kernel<T>, dim3(cdiv(logical, PB)), dim3(PB), 0, stream(), sp, walk, mode, go, gi + off, logical);
     MXH_LAUNCH_CHECK("pad_edge_backward");
 }
 

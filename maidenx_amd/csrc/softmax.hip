@@ -8,7 +8,8 @@
 // sum in f32.
 //   contiguous, dim last : a wave (rows up to 2048) or a block per row; 16-byte loads, the row is held in
 //                          registers between the three phases when it fits.
-//   contiguous, dim inner: lanes run along the trailing dims (coalesced), each walks its column 3 times.
+//   contiguous, dim inner: lanes run along the trailing dims (coalesced); short columns are walked by one
+//                          thread each, long ones are split among the 16 waves of a block.
 //   strided input        : one thread per slice with the reference's index rule (:120-136, the leading
 //                          dims are decomposed from dim 0 upwards).
 #include "elementwise.hpp"
@@ -94,6 +95,7 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
     }
 
     float s = 0.0f;
+    float ev[NREG][VEC];          // exp(x - m) of the held part of the row: computed once
     if (live) {
         if (fits) {
 #pragma unroll
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
                 size_t i = (size_t)t * VEC + k * step;
                 if (i < D) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) s += SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m);
+                    for (int e = 0; e < VEC; ++e) { ev[k][e] = SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m); s += ev[k][e]; }
                 }
             }
         } else {
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
             if (i < D) {
                 AVec<T, VEC> o;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m), s);
+                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(ev[k][e], s);
                 if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
                 else dst[i] = o.v[0];
             }
@@ -165,6 +167,69 @@ __global__ __launch_bounds__(SB) void softmax_col_kernel(const T* __restrict__ i
     for (size_t i = 0; i < D; ++i) s += SM<T>::shifted(SM<T>::ld(src[i * post]), m);
     s = m_exp(-INFINITY - m) + s;
     for (size_t i = 0; i < D; ++i) dst[i * post] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(src[i * post]), m), s);
+}
+
+// [pre, D, post] contiguous, long D: a block of NW waves shares 64*VEC columns and splits D among its
+// waves; the per-wave maxima and sums meet in LDS (in wave order).  Three passes over the block's slab.
+template <class T, int VEC, int NW>
+__global__ __launch_bounds__(WAVE * NW) void softmax_col_split_kernel(const T* __restrict__ in, T* __restrict__ out, size_t D,
+                                                                       size_t post, uint32_t cv, FastDiv div_jb) {
+    const int lane = threadIdx.x % WAVE, w = threadIdx.x / WAVE;
+    uint32_t pre_idx, jb;
+    fd_divmod(blockIdx.x, div_jb, pre_idx, jb);
+    const uint32_t j = jb * WAVE + lane;           // column vector inside the slab
+    const bool live = j < cv;
+    const size_t slice = (D + NW - 1) / NW;
+    const size_t l0 = (size_t)w * slice < D ? (size_t)w * slice : D, l1 = l0 + slice < D ? l0 + slice : D;
+    const T* src = in + (size_t)pre_idx * D * post + (size_t)j * VEC;
+    T* dst = out + (size_t)pre_idx * D * post + (size_t)j * VEC;
+    __shared__ float red[NW][VEC][WAVE];
+    auto load = [&](size_t l) {
+        AVec<T, VEC> v;
+        if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + l * post);
+        else v.v[0] = src[l * post];
+        return v;
+    };
+    auto combine = [&](float (&a)[VEC], bool is_max) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) red[w][e][lane] = a[e];
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float t = red[0][e][lane];
+#pragma unroll
+            for (int k = 1; k < NW; ++k) t = is_max ? (red[k][e][lane] > t ? red[k][e][lane] : t) : t + red[k][e][lane];
+            a[e] = t;
+        }
+        __syncthreads();
+    };
+    float m[VEC], s[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) { m[e] = -INFINITY; s[e] = 0.0f; }
+    if (live)
+        for (size_t l = l0; l < l1; ++l) {
+            AVec<T, VEC> v = load(l);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(v.v[e]); m[e] = x > m[e] ? x : m[e]; }
+        }
+    combine(m, true);
+    if (live)
+        for (size_t l = l0; l < l1; ++l) {
+            AVec<T, VEC> v = load(l);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s[e] += SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]);
+        }
+    combine(s, false);
+    if (!live) return;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) s[e] = m_exp(-INFINITY - m[e]) + s[e];
+    for (size_t l = l0; l < l1; ++l) {
+        AVec<T, VEC> v = load(l), o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]), s[e]);
+        if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + l * post) = o;
+        else dst[l * post] = o.v[0];
+    }
 }
 
 struct SoftmaxStrided {
@@ -231,6 +296,21 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
             else hipLaunchKernelGGL((softmax_row_kernel<T, SB, 1, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
         }
         MXH_LAUNCH_CHECK("softmax_row");
+        return;
+    }
+    if (cont && D >= 64 && pre < (1ull << 20) && post < (1ull << 31)) {
+        // long columns: blocks of 16 waves; narrow vectors when wide ones would leave CUs without a block
+        constexpr int VEC = 16 / sizeof(T), NW = 16;
+        const bool vec_ok = post % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)out % 16) == 0;
+        const size_t blocks_v = pre * cdiv(post / VEC, (size_t)WAVE);
+        if (vec_ok && blocks_v >= 256) {
+            uint32_t cv = (uint32_t)(post / VEC), jb = (uint32_t)cdiv(cv, (size_t)WAVE);
+            hipLaunchKernelGGL((softmax_col_split_kernel<T, VEC, NW>), dim3((unsigned)(pre * jb)), dim3(WAVE * NW), 0, stream(), src, out, D, post, cv, make_fastdiv(jb));
+        } else {
+            uint32_t cv = (uint32_t)post, jb = (uint32_t)cdiv(cv, (size_t)WAVE);
+            hipLaunchKernelGGL((softmax_col_split_kernel<T, 1, NW>), dim3((unsigned)(pre * jb)), dim3(WAVE * NW), 0, stream(), src, out, D, post, cv, make_fastdiv(jb));
+        }
+        MXH_LAUNCH_CHECK("softmax_col_split");
         return;
     }
     if (cont) {
