@@ -10,17 +10,25 @@
 // so the two transposed backward products need no materialised transpose: the operand whose
 // reduction index is strided is turned while it is staged into LDS.
 //
-// Large products run on MFMA (v_mfma_f32_32x32x16_bf16 / v_mfma_f32_32x32x2_f32), f32 accumulate, one
+// Large products run on MFMA (v_mfma_f32_16x16x32_bf16 / v_mfma_f32_32x32x2_f32), f32 accumulate, one
 // rounding at the end for bf16: 256x256 output tiles on 8-wave blocks (two waves per SIMD keep the matrix
 // pipe fed), 128x128 on 4-wave blocks for problems with few tiles, 256x64 for narrow outputs; products
 // with few tiles and a long reduction are split over the reduction and folded in a fixed order.
+// bf16 uses the 16x16x32 instruction: the kernel is power-limited on real data, and that shape does
+// about 15 % more work per joule than 32x32x16 (both measured in an MFMA-only loop on random operands).
 // Operands sit in LDS as [row][k] with the reduction index contiguous, so a lane fetches its whole
 // fragment with one 128-bit ds_read.
 // Small or skinny products (the MLP's [10000,3]x[3,1] and its [3,10000]x[10000,1] gradient) use
 // a thread-per-output kernel (bit-exact with the reference: k ascending, unfused f32) or a
 // wave-per-output dot kernel.
 
+#include <type_traits>
+
 #include "mxh.hpp"
+
+#ifndef MXH_GEMM_TS16
+#define MXH_GEMM_TS16 1
+#endif
 
 namespace mxh {
 
@@ -213,6 +221,10 @@ template <> struct Mma<bf16_t> {
     static __device__ void run(const u32x4& a, const u32x4& b, f32x16& c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
+    // 16x16 tiles, 32 reduction steps per instruction: lane (row l%16) holds k = 8*(l/16) .. +7
+    static __device__ void run(const u32x4& a, const u32x4& b, f32x4& c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
 };
 template <> struct Mma<float> {
     // one 16-byte fragment feeds four 32x32x2 steps; lane (row, h) holds k = 4h .. 4h+3 of an
@@ -225,7 +237,7 @@ template <> struct Mma<float> {
     }
 };
 
-// Block = WM x WN waves, each wave MI x MJ MFMA tiles of 32x32: block tile (32*MI*WM) x (32*MJ*WN).
+// Block = WM x WN waves, each wave MI x MJ MFMA tiles of TS x TS: block tile (TS*MI*WM) x (TS*MJ*WN).
 //   Big  : 4 x 2 waves of 2 x 4 tiles = 256 x 256, 512 threads.  One wave alone can issue a 32x32x16
 //          MFMA only every other slot of the matrix pipe, so the pipe needs two waves per SIMD: 8 waves
 //          per CU with 128 accumulator registers each (measured: 1.29 vs 1.81 PFLOP/s for an
@@ -233,30 +245,44 @@ template <> struct Mma<float> {
 //   Small: 2 x 2 waves of 2 x 2 tiles = 128 x 128, 256 threads, for problems with few tiles.
 // The MFMA is issued with the operands swapped (Y fragment as "A"), so the accumulator of a lane
 // holds 4 consecutive output columns of one output row and leaves as one packed store.
-template <int WM_, int WN_, int MI_, int MJ_> struct GemmCfg {
-    static constexpr int WM = WM_, WN = WN_, MI = MI_, MJ = MJ_;
-    static constexpr int NT = WAVE * WM * WN, TM = 32 * MI * WM, TN = 32 * MJ * WN;
+// TS = 16 (bf16 only): the same block and wave tiles built from 16x16x32 MFMAs.  On random data the
+// matrix pipe sustains about 15 % more under the power limit with these than with 32x32x16 (an
+// MFMA-only loop: 2.1 against 1.85 PFLOP/s; both reach 2.45 on constant data).
+template <int WM_, int WN_, int MI_, int MJ_, int TS_ = 32> struct GemmCfg {
+    static constexpr int WM = WM_, WN = WN_, MI = MI_, MJ = MJ_, TS = TS_;
+    static constexpr int NT = WAVE * WM * WN, TM = TS * MI * WM, TN = TS * MJ * WN;
+    using Acc = typename std::conditional<TS == 32, f32x16, f32x4>::type;
 };
-using CfgBig = GemmCfg<4, 2, 2, 4>;
-using CfgSmall = GemmCfg<2, 2, 2, 2>;
-using CfgTall = GemmCfg<4, 1, 2, 2>;     // 256 x 64: few output columns (the convolution GEMM has 64)
+template <class T> struct Cfgs {
+    using Big = GemmCfg<4, 2, 2, 4>;
+    using Small = GemmCfg<2, 2, 2, 2>;
+    using Tall = GemmCfg<4, 1, 2, 2>;     // 256 x 64: few output columns (the convolution GEMM has 64)
+};
+#if MXH_GEMM_TS16
+template <> struct Cfgs<bf16_t> {
+    using Big = GemmCfg<4, 2, 4, 8, 16>;
+    using Small = GemmCfg<2, 2, 4, 4, 16>;
+    using Tall = GemmCfg<4, 1, 4, 4, 16>;
+};
+#endif
 
 // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
 // column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
+// (16x16 tiles: one group of 4: column j0 + .. + 4*(lane/16) + e, row lane%16)
 template <class O, class Cfg, bool FAST>
-__device__ __forceinline__ void store_tile(O* out, const f32x16 (&acc)[Cfg::MI][Cfg::MJ], const GemmArgs& g, uint32_t i0, uint32_t j0,
+__device__ __forceinline__ void store_tile(O* out, const typename Cfg::Acc (&acc)[Cfg::MI][Cfg::MJ], const GemmArgs& g, uint32_t i0, uint32_t j0,
                                            int wm, int wn, int lane) {
-    constexpr int MI = Cfg::MI, MJ = Cfg::MJ;
-    const int lrow = lane % 32;
+    constexpr int MI = Cfg::MI, MJ = Cfg::MJ, TS = Cfg::TS;
+    const int lrow = lane % TS;
     const bool vec_store = FAST || ((g.J % 4 == 0) && ((uintptr_t)out % (4 * sizeof(O)) == 0));
 #pragma unroll
     for (int a = 0; a < MI; ++a) {
-        uint32_t row = i0 + wm * 32 * MI + a * 32 + lrow;
+        uint32_t row = i0 + wm * TS * MI + a * TS + lrow;
 #pragma unroll
         for (int c = 0; c < MJ; ++c) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t col = j0 + wn * 32 * MJ + c * 32 + 8 * q + 4 * (lane / 32);
+            for (int q = 0; q < (TS == 32 ? 4 : 1); ++q) {
+                uint32_t col = j0 + wn * TS * MJ + c * TS + (TS == 32 ? 8 * q + 4 * (lane / 32) : 4 * (lane / 16));
                 if (!FAST && (row >= g.I || col >= g.J)) continue;
                 O* dst = out + (int64_t)row * g.J + col;
                 if (vec_store && (FAST || col + 4 <= g.J)) {
@@ -312,15 +338,17 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
 
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-    const int lrow = lane % 32, lk = (lane / 32) * VEC;
+    constexpr int TS = Cfg::TS;
+    const int lrow = lane % TS, lk = (lane / TS) * VEC;
+    constexpr int KS = (WAVE / TS) * VEC;                   // reduction steps one MFMA (group) consumes
 
-    f32x16 acc[MI][MJ];
+    typename Cfg::Acc acc[MI][MJ];
 #pragma unroll
     for (int a = 0; a < MI; ++a)
 #pragma unroll
         for (int c = 0; c < MJ; ++c)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[a][c][e] = 0.0f;
+            for (int e = 0; e < (TS == 32 ? 16 : 4); ++e) acc[a][c][e] = 0.0f;
 
     // Software pipeline (all indices compile-time after unrolling, one barrier per k-tile).  While the
     // MFMAs work through LDS[cur] (tile kt), step s < S-1 of the tile
@@ -330,8 +358,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     // the last step starts with the barrier (LDS[cur^1] complete, LDS[cur] no longer read by anyone
     // once the fragments of step S-1 are in registers) and reads step 0 of the next tile under the cover
     // of its own MFMAs.  Loads past the last tile are redirected to it (harmless re-reads).
-    constexpr int S = TK / (2 * VEC);                       // k-steps per tile (4)
+    // Steps per tile.  32x32 tiles: one per KS reduction steps, every step reads MI + MJ fragments and
+    // issues MI*MJ MFMAs.  16x16 tiles: a k-step of 32 is cut in two halves of the column tiles, so a
+    // step reads MJ/2 Y fragments (and the MI X fragments at the first half) and issues MI*MJ/2 MFMAs.
+    constexpr int S = TS == 32 ? TK / KS : 2 * (TK / KS);
+    constexpr int MJH = TS == 32 ? MJ : MJ / 2;
     static_assert(S >= 2 && S % 2 == 0, "fragment double buffer assumes an even number of steps");
+    static_assert(TS == 32 || (sizeof(T) == 2 && MJ % 2 == 0), "16x16 tiles are for 16-bit operands");
     SX sx;
     SY sy;
     const uint32_t nk = (re - rb + TK - 1) / TK;
@@ -346,13 +379,41 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     }
     __syncthreads();
 
-    const int frag_x = (wm * 32 * MI + lrow) * PITCH + lk;   // + a*32*PITCH + s*2*VEC
-    const int frag_y = (wn * 32 * MJ + lrow) * PITCH + lk;
-    u32x4 fa[2][MI], fb[2][MJ];
+    const int frag_x = (wm * TS * MI + lrow) * PITCH + lk;   // + a*TS*PITCH + k-step*KS
+    const int frag_y = (wn * TS * MJ + lrow) * PITCH + lk;
+    u32x4 fa[2][MI], fb[2][MJH];
+    // fragments of step s from the tile at (bx, by)
+    auto read_frags = [&](int s, const T* bx, const T* by) {
+        if constexpr (TS == 32) {
 #pragma unroll
-    for (int a = 0; a < MI; ++a) fa[0][a] = *(const u32x4*)(lds_x + frag_x + a * 32 * PITCH);
+            for (int a = 0; a < MI; ++a) fa[s & 1][a] = *(const u32x4*)(bx + frag_x + a * TS * PITCH + s * KS);
 #pragma unroll
-    for (int c = 0; c < MJ; ++c) fb[0][c] = *(const u32x4*)(lds_y + frag_y + c * 32 * PITCH);
+            for (int c = 0; c < MJ; ++c) fb[s & 1][c] = *(const u32x4*)(by + frag_y + c * TS * PITCH + s * KS);
+        } else {
+            const int ks = s >> 1, h = s & 1;
+            if (h == 0) {
+#pragma unroll
+                for (int a = 0; a < MI; ++a) fa[ks & 1][a] = *(const u32x4*)(bx + frag_x + a * TS * PITCH + ks * KS);
+            }
+#pragma unroll
+            for (int c = 0; c < MJH; ++c) fb[s & 1][c] = *(const u32x4*)(by + frag_y + (h * MJH + c) * TS * PITCH + ks * KS);
+        }
+    };
+    auto mfmas = [&](int s) {
+        if constexpr (TS == 32) {
+#pragma unroll
+            for (int a = 0; a < MI; ++a)
+#pragma unroll
+                for (int c = 0; c < MJ; ++c) Mma<T>::run(fb[s & 1][c], fa[s & 1][a], acc[a][c]);
+        } else {
+            const int ks = s >> 1, h = s & 1;
+#pragma unroll
+            for (int a = 0; a < MI; ++a)
+#pragma unroll
+                for (int c = 0; c < MJH; ++c) Mma<T>::run(fb[s & 1][c], fa[ks & 1][a], acc[a][h * MJH + c]);
+        }
+    };
+    read_frags(0, lds_x, lds_y);
 
     for (uint32_t kt = 0; kt < nk; ++kt) {
         const int cur = kt & 1;
@@ -370,24 +431,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                 sy.store(ny, y0, y1);
                 sx.template load<FAST>(X, g.xi, g.xr, i0, nt, g.I, re, x0, x1);
                 sy.template load<FAST>(Y, g.yj, g.yr, j0, nt, g.J, re, y0, y1);
-#pragma unroll
-                for (int a = 0; a < MI; ++a) fa[(s + 1) & 1][a] = *(const u32x4*)(cx + frag_x + a * 32 * PITCH + (s + 1) * 2 * VEC);
-#pragma unroll
-                for (int c = 0; c < MJ; ++c) fb[(s + 1) & 1][c] = *(const u32x4*)(cy + frag_y + c * 32 * PITCH + (s + 1) * 2 * VEC);
+                read_frags(s + 1, cx, cy);
             } else {
                 __syncthreads();
-#pragma unroll
-                for (int a = 0; a < MI; ++a) fa[0][a] = *(const u32x4*)(nx + frag_x + a * 32 * PITCH);
-#pragma unroll
-                for (int c = 0; c < MJ; ++c) fb[0][c] = *(const u32x4*)(ny + frag_y + c * 32 * PITCH);
+                read_frags(0, nx, ny);
             }
             // keep the memory operations of the next stage ahead of this step's MFMAs: the matrix
             // pipe then works through them while LDS and the vector memory unit serve the next step
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int a = 0; a < MI; ++a)
-#pragma unroll
-                for (int c = 0; c < MJ; ++c) Mma<T>::run(fb[s & 1][c], fa[s & 1][a], acc[a][c]);
+            mfmas(s);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -430,10 +482,13 @@ void launch_mfma_impl(GemmArgs g) {
         if (!g.part) return;
     }
     auto kern = gemm_mfma_kernel<T, XR, YR, Cfg, FAST>;
-    static bool attr_done = false;     // per instantiation
-    if (!attr_done) {
+    // more than 64 KB of LDS has to be allowed once per kernel and device (setting it twice is harmless)
+    static bool attr_done[64] = {false};     // per instantiation, indexed by device
+    int dev = 0;
+    MXH_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64 || !attr_done[dev]) {
         MXH_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attr_done = true;
+        if (dev >= 0 && dev < 64) attr_done[dev] = true;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), lds_bytes, stream(), g);
     MXH_LAUNCH_CHECK("gemm_mfma");
@@ -563,7 +618,7 @@ void gemm_dispatch(GemmArgs g) {
     size_t big_blocks = (size_t)cdiv(g.I, 256) * cdiv(g.J, 256) * g.batch;
     bool big = g.I >= 256 && g.J >= 256 && big_blocks >= 192;
     const bool tall = !big && g.J <= 64 && g.I >= 1024;
-#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, CfgBig>(g) : tall ? launch_mfma<T, XR, YR, CfgTall>(g) : launch_mfma<T, XR, YR, CfgSmall>(g))
+#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, typename Cfgs<T>::Big>(g) : tall ? launch_mfma<T, XR, YR, typename Cfgs<T>::Tall>(g) : launch_mfma<T, XR, YR, typename Cfgs<T>::Small>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
     else if (xr && yj) MXH_GEMM_CASE(true, false);
     else if (xi && yr) MXH_GEMM_CASE(false, true);

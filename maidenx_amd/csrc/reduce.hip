@@ -464,6 +464,7 @@ bool plane_reduce(const T* in, T* out, size_t A, size_t K, size_t S) {
     if (K < 256) chunks = (uint32_t)std::min<size_t>(A, cdiv((size_t)512, K));
     uint32_t a_chunk = (uint32_t)cdiv(A, (size_t)chunks);
     chunks = (uint32_t)cdiv(A, (size_t)a_chunk);
+    if (K * chunks >= (1ull << 31)) return false;
     FastDiv dsv = make_fastdiv((uint32_t)(S / VEC));
     const bool bf = IO<T>::is_bf16;
     if (chunks == 1) {

@@ -286,19 +286,20 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
     if (cont && post == 1) {
         constexpr int VEC = 16 / sizeof(T);
         const bool vec = D % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)out % 16) == 0;
+        if (slices >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "softmax: 2^31 or more rows"); return; }
         if (D <= 2048) {
             unsigned blocks = cdiv(slices, SB / WAVE);
             if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, VEC, 2048 / (WAVE * VEC)>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
             else hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, 1, 8>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
         } else {
-            if (slices >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "softmax: too many rows"); return; }
             if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, SB, VEC, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
             else hipLaunchKernelGGL((softmax_row_kernel<T, SB, 1, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
         }
         MXH_LAUNCH_CHECK("softmax_row");
         return;
     }
-    if (cont && D >= 64 && pre < (1ull << 20) && post < (1ull << 31)) {
+    if (slices >= (1ull << 38)) { set_status(ERR_TOO_LARGE, "softmax: 2^38 or more slices"); return; }
+    if (cont && D >= 64 && pre * cdiv(post, (size_t)WAVE) < (1ull << 31) && post < (1ull << 31)) {
         // long columns: blocks of 16 waves; narrow vectors when wide ones would leave CUs without a block
         constexpr int VEC = 16 / sizeof(T), NW = 16;
         const bool vec_ok = post % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)out % 16) == 0;
