@@ -322,12 +322,18 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     T* lds_x = (T*)smem;                                  // [2][TM*PITCH]
     T* lds_y = lds_x + 2 * TM * PITCH;                    // [2][TN*PITCH]
 
-    // block → (batch, tile_i, tile_j); neighbouring blocks share the X panel (tile_j fastest)
-    uint32_t bid = blockIdx.x;
-    uint32_t tj = bid % g.tiles_j;
-    uint32_t rest = bid / g.tiles_j;
-    uint32_t ti = rest % g.tiles_i;
-    rest /= g.tiles_i;
+    // Blocks are handed to the 8 XCDs round robin, and each XCD has its own L2: give every XCD a compact
+    // patch of the tile grid (GM tile rows x as many columns as it gets), so that the operand panels its
+    // CUs stream are shared inside that L2 instead of being fetched by all eight.
+    const uint32_t per = g.tiles_i * g.tiles_j;
+    uint32_t rest = blockIdx.x / per;
+    uint32_t v = blockIdx.x - rest * per;
+    if (per % 8 == 0) v = (v % 8) * (per / 8) + v / 8;
+    constexpr uint32_t GM = 4;
+    const uint32_t group = v / (GM * g.tiles_j), in_group = v - group * (GM * g.tiles_j);
+    const uint32_t first_i = group * GM, rows = g.tiles_i - first_i < GM ? g.tiles_i - first_i : GM;
+    uint32_t ti = first_i + in_group % rows;
+    uint32_t tj = in_group / rows;
     uint32_t b = rest % g.batch;
     const uint32_t split = rest / g.batch;
     const uint32_t rb = split * g.r_chunk;                                  // this block reduces over [rb, re)
