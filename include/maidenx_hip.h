@@ -206,6 +206,34 @@ MX_DECL_CONV(mx_bf16, bf16)
 void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const float* input, float* output);
 void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const mx_bf16* input, mx_bf16* output);
 
+/* ---- index ops -----------------------------------------------------------------------------------
+ * No backend symbol exists for these in the reference: crates/maidenx_tensor/src/ops/indexing.rs runs them
+ * as host loops over get / set / add_at_index (index_select :93-124, index_add_ :15-91, gather :315-363,
+ * scatter_add_ :403-461, bincount :463-522; add_at_index utils/indexing.rs:96-140).  A layout is
+ * dims[n] | strides[n] | offset of one tensor; outputs of index_select / gather are contiguous; indices
+ * are read as i32 like the reference does; gather and scatter_add_ wrap negative indices; the in-place
+ * ops add in the storage dtype in the reference's order (bit-identical, deterministic).  An index
+ * outside its range is skipped and reported by hip_get_last_status() as an invalid argument
+ * (the reference returns IndexOutOfBounds); that call waits for the stream when index ops ran. */
+#define MX_DECL_INDEX(T, S, I, IS)                                                                                     \
+    void hip_index_select_##S##_##IS(size_t num_dims, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride, \
+                                     size_t idx_offset, const I* indices, const T* input, T* output);                  \
+    void hip_gather_##S##_##IS(size_t num_dims, size_t dim, const size_t* in_layout, const size_t* idx_layout,         \
+                               const I* index, const T* input, T* output);                                             \
+    void hip_index_add_##S##_##IS(size_t num_dims, size_t dim, const size_t* self_layout, const size_t* src_layout,    \
+                                  size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices, const T* src,  \
+                                  T* self);                                                                            \
+    void hip_scatter_add_##S##_##IS(size_t num_dims, size_t dim, const size_t* self_layout, const size_t* idx_layout,  \
+                                    const size_t* src_layout, const I* index, const T* src, T* self);                  \
+    void hip_bincount_weighted_##S##_##IS(size_t n, size_t stride, size_t offset, const I* input, size_t w_stride,     \
+                                          size_t w_offset, const T* weights, size_t out_size, T* output);
+MX_DECL_INDEX(float, f32, int32_t, i32)
+MX_DECL_INDEX(float, f32, int64_t, i64)
+MX_DECL_INDEX(mx_bf16, bf16, int32_t, i32)
+MX_DECL_INDEX(mx_bf16, bf16, int64_t, i64)
+void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output);
+void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output);
+
 /* ---- device-side fill / convert / strided copy --------------------------------------------------
  * No backend symbol exists for these in the reference: it builds host vectors
  * (crates/maidenx_tensor/src/creation.rs:144-164), converts dtypes on the host

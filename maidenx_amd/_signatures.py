@@ -50,9 +50,24 @@ def signatures(dtypes=("f32", "bf16")):
     return sig
 
 
+def index_signatures(dtypes=("f32", "bf16")):
+    """Index ops (host loops in the reference's tensor layer, device entry points here)."""
+    sig = {}
+    for dt in dtypes:
+        for it in ("i32", "i64"):
+            sig[f"index_select_{dt}_{it}"] = [SZ, SZ, P, SZ, SZ, SZ, P, P, P]
+            sig[f"gather_{dt}_{it}"] = [SZ, SZ, P, P, P, P, P]
+            sig[f"index_add_{dt}_{it}"] = [SZ, SZ, P, P, SZ, SZ, SZ, P, P, P]
+            sig[f"scatter_add_{dt}_{it}"] = [SZ, SZ, P, P, P, P, P, P]
+            sig[f"bincount_weighted_{dt}_{it}"] = [SZ, SZ, SZ, P, SZ, SZ, P, SZ, P]
+    for it in ("i32", "i64"):
+        sig[f"bincount_{it}"] = [SZ, SZ, SZ, P, SZ, P]
+    return sig
+
+
 def extension_signatures():
     """Entry points of the HIP library that have no counterpart symbol in the reference."""
-    sig = {}
+    sig = index_signatures()
     for dt in ("f32", "bf16", "bool"):
         sig[f"fill_{dt}"] = [SZ, P, CONST[dt]]
     for dt in ("f32", "bf16"):

@@ -1,0 +1,320 @@
+// Index ops on the device: index_select, index_add_, gather, scatter_add_, bincount.
+// The reference has no backend symbol for these: crates/maidenx_tensor/src/ops/indexing.rs runs them
+// as host loops over `get` / `set` / `add_at_index` (one buffer round trip per element).  The entry
+// points here take the tensors' layouts (dims[n] | strides[n] | offset, as the tensor layer holds
+// them) and do the same work in one launch, with the same results:
+//   index_select (:93-124)  out[.., i, ..] = in[.., idx[i], ..]            copy, bit-exact
+//   gather       (:315-363) out[p] = in[p with p[dim] = index[p]]         copy, bit-exact; negative wraps
+//   index_add_   (:15-91)   self[.., idx[i], ..] += src[.., i, ..]         i ascending
+//   scatter_add_ (:403-461) self[p with p[dim] = index[p]] += src[p]       p in row-major order
+//   bincount     (:463-522) counts, or sums of weights, per value
+// The adds are in the storage dtype (utils/indexing.rs:96-140) and their order matters for floats.
+// Updates of different "lines" (all coordinates but `dim` fixed) never meet, and inside a line the
+// reference's order is ascending position along `dim`: one thread owns a line and walks it in that
+// order, so results are bit-identical to the host loops and deterministic.  Counts are integers
+// (atomics are exact); weighted bincount lets one thread own a bin and scan the input in order.
+// An index outside its range is skipped and raises the device-side index flag, which
+// hip_get_last_status() reports as an invalid argument (the reference returns IndexOutOfBounds).
+#include "mxh.hpp"
+#include "ops.hpp"
+
+namespace mxh {
+
+constexpr int IB = 256;
+
+struct Lay {            // one tensor: shape walk + strides
+    int64_t strides[MAXD];
+    int64_t offset;
+};
+struct IdxSpace {
+    int nd, dim;
+    uint32_t dims[MAXD];        // iteration space
+    FastDiv div[MAXD];
+};
+
+// decompose a linear index over the iteration space into coordinates (row-major)
+__device__ inline void split(const IdxSpace& sp, uint32_t r, uint32_t (&c)[MAXD]) {
+#pragma unroll
+    for (int d = MAXD - 1; d >= 0; --d) {
+        if (d >= sp.nd) { c[d] = 0; continue; }
+        uint32_t q, m;
+        if (d > 0) fd_divmod(r, sp.div[d], q, m);
+        else { q = 0; m = r; }
+        c[d] = m;
+        r = q;
+    }
+}
+__device__ inline int64_t dot(const IdxSpace& sp, const uint32_t (&c)[MAXD], const Lay& l, int skip_dim) {
+    int64_t o = l.offset;
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d)
+        if (d < sp.nd && d != skip_dim) o += (int64_t)c[d] * l.strides[d];
+    return o;
+}
+
+// ---- index_select: iteration space = output dims ------------------------------------------------
+template <class T, class I>
+__global__ __launch_bounds__(IB) void index_select_kernel(IdxSpace sp, Lay in, const I* __restrict__ indices, int64_t idx_stride,
+                                                          int64_t idx_offset, uint32_t in_dim_size, const T* __restrict__ src,
+                                                          T* __restrict__ out, size_t n, int* flag) {
+    size_t o = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (o >= n) return;
+    uint32_t c[MAXD];
+    split(sp, (uint32_t)o, c);
+    // the reference reads the index `as_i32` (:113)
+    const int32_t idx = (int32_t)indices[idx_offset + (int64_t)c[sp.dim] * idx_stride];
+    if (idx < 0 || (uint32_t)idx >= in_dim_size) { *flag = 1; out[o] = T{}; return; }
+    out[o] = src[dot(sp, c, in, sp.dim) + (int64_t)idx * in.strides[sp.dim]];
+}
+
+// ---- gather: iteration space = index dims ---------------------------------------------------------
+template <class T, class I>
+__global__ __launch_bounds__(IB) void gather_kernel(IdxSpace sp, Lay in, Lay ix, uint32_t in_dim_size, const I* __restrict__ index,
+                                                    const T* __restrict__ src, T* __restrict__ out, size_t n, int* flag) {
+    size_t o = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (o >= n) return;
+    uint32_t c[MAXD];
+    split(sp, (uint32_t)o, c);
+    int32_t idx = (int32_t)index[dot(sp, c, ix, -1)];
+    if (idx < 0) idx += (int32_t)in_dim_size;              // :341-345
+    if (idx < 0 || (uint32_t)idx >= in_dim_size) { *flag = 1; out[o] = T{}; return; }
+    out[o] = src[dot(sp, c, in, sp.dim) + (int64_t)idx * in.strides[sp.dim]];
+}
+
+// ---- index_add_ / scatter_add_: iteration space = the lines (dims[dim] forced to 1) ----------------
+template <class T, class I>
+__global__ __launch_bounds__(IB) void index_add_kernel(IdxSpace sp, Lay self, Lay sr, const I* __restrict__ indices, int64_t idx_stride,
+                                                       int64_t idx_offset, uint32_t n_idx, uint32_t self_dim_size,
+                                                       const T* __restrict__ src, T* __restrict__ dst, size_t lines, int* flag) {
+    size_t l = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (l >= lines) return;
+    uint32_t c[MAXD];
+    split(sp, (uint32_t)l, c);
+    const int64_t s0 = dot(sp, c, sr, sp.dim), d0 = dot(sp, c, self, sp.dim);
+    for (uint32_t i = 0; i < n_idx; ++i) {
+        const int32_t idx = (int32_t)indices[idx_offset + (int64_t)i * idx_stride];
+        if (idx < 0 || (uint32_t)idx >= self_dim_size) { *flag = 1; continue; }
+        T* p = dst + d0 + (int64_t)idx * self.strides[sp.dim];
+        *p = Ar<T>::add(*p, src[s0 + (int64_t)i * sr.strides[sp.dim]]);
+    }
+}
+
+template <class T, class I>
+__global__ __launch_bounds__(IB) void scatter_add_kernel(IdxSpace sp, Lay self, Lay ix, Lay sr, uint32_t len, uint32_t self_dim_size,
+                                                         const I* __restrict__ index, const T* __restrict__ src, T* __restrict__ dst,
+                                                         size_t lines, int* flag) {
+    size_t l = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (l >= lines) return;
+    uint32_t c[MAXD];
+    split(sp, (uint32_t)l, c);
+    const int64_t s0 = dot(sp, c, sr, sp.dim), i0 = dot(sp, c, ix, sp.dim), d0 = dot(sp, c, self, sp.dim);
+    for (uint32_t k = 0; k < len; ++k) {
+        int32_t idx = (int32_t)index[i0 + (int64_t)k * ix.strides[sp.dim]];
+        if (idx < 0) idx += (int32_t)self_dim_size;          // :434-438
+        if (idx < 0 || (uint32_t)idx >= self_dim_size) { *flag = 1; continue; }
+        T* p = dst + d0 + (int64_t)idx * self.strides[sp.dim];
+        *p = Ar<T>::add(*p, src[s0 + (int64_t)k * sr.strides[sp.dim]]);
+    }
+}
+
+// ---- bincount ---------------------------------------------------------------------------------------
+template <class I>
+__global__ __launch_bounds__(IB) void zero_counts_kernel(I* out, size_t n) {
+    size_t i = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (i < n) out[i] = 0;
+}
+template <class I> __device__ inline void count_one(I* p);
+template <> __device__ inline void count_one<int32_t>(int32_t* p) { atomicAdd(p, 1); }
+template <> __device__ inline void count_one<int64_t>(int64_t* p) { atomicAdd((unsigned long long*)p, 1ull); }
+
+template <class I>
+__global__ __launch_bounds__(IB) void bincount_kernel(const I* __restrict__ in, int64_t stride, int64_t offset, size_t n, I* out,
+                                                      size_t out_size, int* flag) {
+    size_t i = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (i >= n) return;
+    const int32_t v = (int32_t)in[offset + (int64_t)i * stride];
+    if (v < 0 || (size_t)v >= out_size) { *flag = 1; return; }
+    count_one<I>(out + v);
+}
+// one thread per bin, input scanned in order: sum of the weights of the entries equal to the bin
+template <class T, class I>
+__global__ __launch_bounds__(IB) void bincount_weighted_kernel(const I* __restrict__ in, int64_t stride, int64_t offset,
+                                                               const T* __restrict__ w, int64_t w_stride, int64_t w_offset, size_t n,
+                                                               T* out, size_t out_size, int* flag) {
+    size_t b = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (b >= out_size) return;
+    T acc = Ar<T>::zero();
+    for (size_t i = 0; i < n; ++i) {
+        const int32_t v = (int32_t)in[offset + (int64_t)i * stride];
+        if (b == 0 && (v < 0 || (size_t)v >= out_size)) *flag = 1;
+        if (v >= 0 && (size_t)v == b) acc = Ar<T>::add(acc, w[w_offset + (int64_t)i * w_stride]);
+    }
+    out[b] = acc;
+}
+
+// ---- host side ----------------------------------------------------------------------------------------
+// layout = dims[n] | strides[n] | offset
+static bool read_layout(size_t nd, const size_t* layout, Lay& l) {
+    for (int d = 0; d < MAXD; ++d) l.strides[d] = d < (int)nd ? (int64_t)layout[nd + d] : 0;
+    l.offset = (int64_t)layout[2 * nd];
+    return true;
+}
+// iteration space over `dims` with dims[force_one] treated as 1 when force_one >= 0
+static bool make_space(size_t nd, const size_t* dims, size_t dim, int force_one, IdxSpace& sp, size_t* count, const char* who) {
+    if (nd == 0 || nd > (size_t)MAXD || dim >= nd) { set_status(ERR_INVALID, who); return false; }
+    sp.nd = (int)nd;
+    sp.dim = (int)dim;
+    size_t total = 1;
+    for (int d = 0; d < MAXD; ++d) {
+        size_t v = d < (int)nd ? dims[d] : 1;
+        if (d == force_one) v = 1;
+        if (v >= (1ull << 31)) { set_status(ERR_TOO_LARGE, who); return false; }
+        sp.dims[d] = (uint32_t)v;
+        sp.div[d] = make_fastdiv((uint32_t)v);
+        total *= v;
+    }
+    if (total >= (1ull << 31)) { set_status(ERR_TOO_LARGE, who); return false; }
+    *count = total;
+    return true;
+}
+
+template <class T, class I>
+void index_select(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices,
+                  const T* input, T* output) {
+    if (!in_layout || !indices || !input || !output) { set_status(ERR_INVALID, "index_select: null argument"); return; }
+    int* flag = index_flag();
+    if (!flag) return;
+    size_t out_dims[MAXD];
+    if (nd > (size_t)MAXD || dim >= nd) { set_status(ERR_INVALID, "index_select: rank above 8 or bad dim"); return; }
+    for (size_t d = 0; d < nd; ++d) out_dims[d] = d == dim ? n_idx : in_layout[d];
+    IdxSpace sp; size_t n; Lay in;
+    if (!make_space(nd, out_dims, dim, -1, sp, &n, "index_select: bad shape")) return;
+    read_layout(nd, in_layout, in);
+    if (n == 0) return;
+    hipLaunchKernelGGL((index_select_kernel<T, I>), dim3(cdiv(n, IB)), dim3(IB), 0, stream(), sp, in, indices, (int64_t)idx_stride,
+                       (int64_t)idx_offset, (uint32_t)in_layout[dim], input, output, n, flag);
+    MXH_LAUNCH_CHECK("index_select");
+}
+
+template <class T, class I>
+void gather(size_t nd, size_t dim, const size_t* in_layout, const size_t* idx_layout, const I* index, const T* input, T* output) {
+    if (!in_layout || !idx_layout || !index || !input || !output) { set_status(ERR_INVALID, "gather: null argument"); return; }
+    int* flag = index_flag();
+    if (!flag) return;
+    IdxSpace sp; size_t n; Lay in, ix;
+    if (!make_space(nd, idx_layout, dim, -1, sp, &n, "gather: bad shape, rank above 8 or bad dim")) return;
+    read_layout(nd, in_layout, in);
+    read_layout(nd, idx_layout, ix);
+    if (n == 0) return;
+    hipLaunchKernelGGL((gather_kernel<T, I>), dim3(cdiv(n, IB)), dim3(IB), 0, stream(), sp, in, ix, (uint32_t)in_layout[dim], index, input,
+                       output, n, flag);
+    MXH_LAUNCH_CHECK("gather");
+}
+
+template <class T, class I>
+void index_add(size_t nd, size_t dim, const size_t* self_layout, const size_t* src_layout, size_t n_idx, size_t idx_stride,
+               size_t idx_offset, const I* indices, const T* src, T* self) {
+    if (!self_layout || !src_layout || !indices || !src || !self) { set_status(ERR_INVALID, "index_add_: null argument"); return; }
+    int* flag = index_flag();
+    if (!flag) return;
+    IdxSpace sp; size_t lines; Lay sl, sr;
+    if (!make_space(nd, self_layout, dim, (int)dim, sp, &lines, "index_add_: bad shape, rank above 8 or bad dim")) return;
+    for (size_t d = 0; d < nd; ++d)
+        if (d != dim && src_layout[d] != self_layout[d]) { set_status(ERR_INVALID, "index_add_: source and self differ outside dim"); return; }
+    if (src_layout[dim] != n_idx) { set_status(ERR_INVALID, "index_add_: source extent along dim must equal the number of indices"); return; }
+    if (n_idx >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "index_add_: 2^31 or more indices"); return; }
+    read_layout(nd, self_layout, sl);
+    read_layout(nd, src_layout, sr);
+    if (lines == 0 || n_idx == 0) return;
+    hipLaunchKernelGGL((index_add_kernel<T, I>), dim3(cdiv(lines, IB)), dim3(IB), 0, stream(), sp, sl, sr, indices, (int64_t)idx_stride,
+                       (int64_t)idx_offset, (uint32_t)n_idx, (uint32_t)self_layout[dim], src, self, lines, flag);
+    MXH_LAUNCH_CHECK("index_add");
+}
+
+template <class T, class I>
+void scatter_add(size_t nd, size_t dim, const size_t* self_layout, const size_t* idx_layout, const size_t* src_layout, const I* index,
+                 const T* src, T* self) {
+    if (!self_layout || !idx_layout || !src_layout || !index || !src || !self) { set_status(ERR_INVALID, "scatter_add_: null argument"); return; }
+    int* flag = index_flag();
+    if (!flag) return;
+    IdxSpace sp; size_t lines; Lay sl, ix, sr;
+    if (!make_space(nd, src_layout, dim, (int)dim, sp, &lines, "scatter_add_: bad shape, rank above 8 or bad dim")) return;
+    for (size_t d = 0; d < nd; ++d) {
+        if (src_layout[d] != idx_layout[d]) { set_status(ERR_INVALID, "scatter_add_: source and index shapes differ"); return; }
+        // add_at_index (utils/indexing.rs:105-112) refuses coordinates beyond self
+        if (d != dim && src_layout[d] > self_layout[d]) { set_status(ERR_INVALID, "scatter_add_: source exceeds self outside dim"); return; }
+    }
+    if (src_layout[dim] >= (1ull << 31) || self_layout[dim] >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "scatter_add_: dim of 2^31 or more"); return; }
+    read_layout(nd, self_layout, sl);
+    read_layout(nd, idx_layout, ix);
+    read_layout(nd, src_layout, sr);
+    if (lines == 0 || src_layout[dim] == 0) return;
+    hipLaunchKernelGGL((scatter_add_kernel<T, I>), dim3(cdiv(lines, IB)), dim3(IB), 0, stream(), sp, sl, ix, sr, (uint32_t)src_layout[dim],
+                       (uint32_t)self_layout[dim], index, src, self, lines, flag);
+    MXH_LAUNCH_CHECK("scatter_add");
+}
+
+template <class I>
+void bincount(size_t n, size_t stride, size_t offset, const I* input, size_t out_size, I* output) {
+    if (!input || !output) { set_status(ERR_INVALID, "bincount: null argument"); return; }
+    int* flag = index_flag();
+    if (!flag) return;
+    if (n >= (1ull << 40) || out_size >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "bincount: too large"); return; }
+    if (out_size == 0) return;
+    hipLaunchKernelGGL(zero_counts_kernel<I>, dim3(cdiv(out_size, IB)), dim3(IB), 0, stream(), output, out_size);
+    if (n) hipLaunchKernelGGL(bincount_kernel<I>, dim3(cdiv(n, IB)), dim3(IB), 0, stream(), input, (int64_t)stride, (int64_t)offset, n, output, out_size, flag);
+    MXH_LAUNCH_CHECK("bincount");
+}
+
+template <class T, class I>
+void bincount_weighted(size_t n, size_t stride, size_t offset, const I* input, size_t w_stride, size_t w_offset, const T* weights,
+                       size_t out_size, T* output) {
+    if (!input || !weights || !output) { set_status(ERR_INVALID, "bincount: null argument"); return; }
+    int* flag = index_flag();
+    if (!flag) return;
+    // every bin's thread scans the whole input: fine for the label-count sizes this is used at
+    if (out_size >= (1ull << 31) || (double)n * (double)out_size > 1.0e12) { set_status(ERR_TOO_LARGE, "bincount with weights: input x bins above 1e12"); return; }
+    if (out_size == 0) return;
+    hipLaunchKernelGGL((bincount_weighted_kernel<T, I>), dim3(cdiv(out_size, IB)), dim3(IB), 0, stream(), input, (int64_t)stride,
+                       (int64_t)offset, weights, (int64_t)w_stride, (int64_t)w_offset, n, output, out_size, flag);
+    MXH_LAUNCH_CHECK("bincount_weighted");
+}
+
+}  // namespace mxh
+
+using namespace mxh;
+
+#define MXH_INDEX_FOR(T, TS, I, IS)                                                                                                  \
+    extern "C" void hip_index_select_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride,    \
+                                                 size_t idx_offset, const I* indices, const T* input, T* output) {                   \
+        index_select<T, I>(nd, dim, in_layout, n_idx, idx_stride, idx_offset, indices, input, output);                               \
+    }                                                                                                                                \
+    extern "C" void hip_gather_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, const size_t* idx_layout, const I* index, \
+                                           const T* input, T* output) {                                                             \
+        gather<T, I>(nd, dim, in_layout, idx_layout, index, input, output);                                                          \
+    }                                                                                                                                \
+    extern "C" void hip_index_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* src_layout,            \
+                                              size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices, const T* src,   \
+                                              T* self) {                                                                             \
+        index_add<T, I>(nd, dim, self_layout, src_layout, n_idx, idx_stride, idx_offset, indices, src, self);                        \
+    }                                                                                                                                \
+    extern "C" void hip_scatter_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* idx_layout,          \
+                                                const size_t* src_layout, const I* index, const T* src, T* self) {                  \
+        scatter_add<T, I>(nd, dim, self_layout, idx_layout, src_layout, index, src, self);                                           \
+    }                                                                                                                                \
+    extern "C" void hip_bincount_weighted_##TS##_##IS(size_t n, size_t stride, size_t offset, const I* input, size_t w_stride,       \
+                                                      size_t w_offset, const T* weights, size_t out_size, T* output) {              \
+        bincount_weighted<T, I>(n, stride, offset, input, w_stride, w_offset, weights, out_size, output);                            \
+    }
+
+MXH_INDEX_FOR(float, f32, int32_t, i32)
+MXH_INDEX_FOR(float, f32, int64_t, i64)
+MXH_INDEX_FOR(bf16_t, bf16, int32_t, i32)
+MXH_INDEX_FOR(bf16_t, bf16, int64_t, i64)
+
+extern "C" void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output) {
+    bincount<int32_t>(n, stride, offset, input, out_size, output);
+}
+extern "C" void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output) {
+    bincount<int64_t>(n, stride, offset, input, out_size, output);
+}

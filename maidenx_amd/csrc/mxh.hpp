@@ -25,6 +25,9 @@ hipStream_t stream();
 // Device scratch owned by the library (two independent slots per device), grown on demand and
 // reused by every call; safe because all work of the backend is ordered on one stream.
 void* scratch(size_t bytes, int slot = 0);
+// One int per device that kernels set to 1 when they meet an index outside its range; taking the
+// pointer marks it as possibly set, and hip_get_last_status() then reads and clears it.
+int* index_flag();
 
 #define MXH_HIP(expr)                                                                 \
     do {                                                                              \

@@ -62,6 +62,46 @@ void* scratch(size_t bytes, int slot) {
     return p;
 }
 
+static int* g_index_flag[16] = {nullptr};
+static bool g_index_flag_used[16] = {false};
+
+int* index_flag() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) { set_status(ERR_INVALID, "index flag: bad device"); return nullptr; }
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_index_flag[dev]) {
+        if (g_capturing) { set_status(ERR_INVALID, "the first index op of a device cannot run inside a graph capture"); return nullptr; }
+        int* p = nullptr;
+        hipError_t e = hipMalloc((void**)&p, 256);
+        if (e == hipSuccess) e = hipMemset(p, 0, 256);
+        if (e != hipSuccess) { set_status(ERR_OOM, "index flag: hipMalloc", (int)e); return nullptr; }
+        g_index_flag[dev] = p;
+    }
+    g_index_flag_used[dev] = true;
+    return g_index_flag[dev];
+}
+
+// Waits for the stream and folds a raised index flag of the current device into the status.
+static void collect_index_flag() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return;
+    int* p;
+    {
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        if (!g_index_flag_used[dev] || g_capturing) return;
+        g_index_flag_used[dev] = false;
+        p = g_index_flag[dev];
+    }
+    int v = 0;
+    if (hipStreamSynchronize(g_stream) != hipSuccess) return;
+    if (g_capture_stream) (void)hipStreamSynchronize(g_capture_stream);
+    if (hipMemcpy(&v, p, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) return;
+    if (v != 0) {
+        (void)hipMemset(p, 0, sizeof(int));
+        set_status(ERR_INVALID, "index out of bounds in index_select / index_add_ / gather / scatter_add_ / bincount");
+    }
+}
+
 }  // namespace mxh
 
 using namespace mxh;
@@ -116,6 +156,7 @@ int hip_event_elapsed_ms(void* start, void* stop, float* ms) { return (int)hipEv
 
 // First error recorded since the last call (0 = none); reading it clears it.
 int hip_get_last_status(void) {
+    collect_index_flag();
     hipError_t e = hipGetLastError();
     std::lock_guard<std::mutex> lk(g_mu);
     if (g_status == OK && e != hipSuccess) {

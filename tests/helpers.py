@@ -14,7 +14,7 @@ ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
 
 import maidenx_amd._signatures as S  # noqa: E402
 
-NP = {"f32": np.float32, "bf16": np.uint16, "bool": np.uint8, "f64": np.float64}
+NP = {"f32": np.float32, "bf16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64}
 
 
 # ---- bf16 <-> f32 on the host (round to nearest even, NaN quieted), as the `half` crate does ----
@@ -102,6 +102,11 @@ def meta_pad(in_dims, in_strides, in_off, out_dims, pads):   # tensor/ops/paddin
     return u64(in_dims, in_strides, in_off, out_dims, flat)
 
 
+def layout(dims, strides=None, off=0):
+    """dims[n] | strides[n] | offset of one tensor, as the index ops take it."""
+    return u64(dims, strides if strides is not None else contiguous_strides(dims), off)
+
+
 def meta_conv(B, Cc, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w):
     """12 slots in the order the kernels READ them (maidenx_cpu nn/conv.rs:20-34)."""
     return u64(B, Cc, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w)
@@ -154,10 +159,11 @@ class Runner:
         if kind == "oracle":
             self.lib = C.CDLL(ensure_oracle_built())
             self.prefix = "oracle_"
-            for name, args in S.signatures(("f32", "bf16", "f64")).items():
+            for name, args in {**S.signatures(("f32", "bf16", "f64")), **S.index_signatures(("f32", "bf16", "f64"))}.items():
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None
+            self.lib.oracle_index_error.restype = C.c_int
             self.lib.oracle_set_num_threads.argtypes = [C.c_int]
             self.lib.oracle_set_num_threads.restype = C.c_int
         else:

@@ -6,7 +6,7 @@ import os
 
 import numpy as np
 
-from helpers import (In, InOut, Out, const_arg, contiguous_strides, meta_binary, meta_matmul, meta_pad, meta_reduce,
+from helpers import (In, InOut, Out, const_arg, contiguous_strides, layout, meta_binary, meta_matmul, meta_pad, meta_reduce,
                      meta_sum_to_shape, meta_unary, to_float, to_storage, u64)
 
 KAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kat.json")))
@@ -205,4 +205,46 @@ def run_softmax(be, dt):
         assert np.all(np.diff(y, axis=c["dim"]) > 0), y
 
 
-ALL = [run_pad_edge, run_fold, run_softmax, run_binary, run_compare, run_inplace, run_unary, run_unary_const, run_reduce, run_sum_to_shape, run_matmul, run_pad]
+def run_index(be, dt):
+    # the reference's test tensors carry offset 1 (tests/utils/mod.rs:12-21); index tensors are i32
+    for it in ("i32", "i64"):
+        ity = np.int32 if it == "i32" else np.int64
+        for c in KAT["index"]:
+            op = c["op"]
+            if op == "index_select":
+                shape, dim = c["shape"], c["dim"]
+                idx = np.array([0] + c["indices"], dtype=ity)
+                n_out = len(c["expect"])
+                (out,) = be.call(f"index_select_{dt}_{it}", len(shape), dim, layout(shape, off=1), len(c["indices"]), 1, 1, In(idx),
+                                 In(padded(c["data"], dt)), Out(n_out, dt))
+                check(out, c["expect"], dt, 0)
+            elif op == "gather":
+                shape, ishape = c["shape"], c["index_shape"]
+                idx = np.array([0] + c["index"], dtype=ity)
+                (out,) = be.call(f"gather_{dt}_{it}", len(shape), c["dim"], layout(shape, off=1), layout(ishape, off=1), In(idx),
+                                 In(padded(c["data"], dt)), Out(len(c["expect"]), dt))
+                check(out, c["expect"], dt, 0)
+            elif op == "index_add":
+                shape, sshape = c["self_shape"], c["src_shape"]
+                idx = np.array([0] + c["indices"], dtype=ity)
+                (out,) = be.call(f"index_add_{dt}_{it}", len(shape), c["dim"], layout(shape, off=1), layout(sshape, off=1),
+                                 len(c["indices"]), 1, 1, In(idx), In(padded(c["src"], dt)), InOut(padded(c["self"], dt)))
+                check(out[1:-1], c["expect"], dt, 0)
+            elif op == "scatter_add":
+                shape, ishape = c["self_shape"], c["index_shape"]
+                idx = np.array([0] + c["index"], dtype=ity)
+                (out,) = be.call(f"scatter_add_{dt}_{it}", len(shape), c["dim"], layout(shape, off=1), layout(ishape, off=1),
+                                 layout(ishape, off=1), In(idx), In(padded(c["src"], dt)), InOut(padded(c["self"], dt)))
+                check(out[1:-1], c["expect"], dt, 0)
+            elif op == "bincount":
+                idx = np.array([0] + c["input"], dtype=ity)
+                (out,) = be.call(f"bincount_{it}", len(c["input"]), 1, 1, In(idx), c["out_size"], Out(c["out_size"], it))
+                assert out.tolist() == c["expect"]
+            elif op == "bincount_weighted":
+                idx = np.array([0] + c["input"], dtype=ity)
+                (out,) = be.call(f"bincount_weighted_{dt}_{it}", len(c["input"]), 1, 1, In(idx), 1, 1, In(padded(c["weights"], dt)),
+                                 c["out_size"], Out(c["out_size"], dt))
+                check(out, c["expect"], dt, 0)
+
+
+ALL = [run_index, run_pad_edge, run_fold, run_softmax, run_binary, run_compare, run_inplace, run_unary, run_unary_const, run_reduce, run_sum_to_shape, run_matmul, run_pad]

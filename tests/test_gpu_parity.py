@@ -7,7 +7,7 @@ import pytest
 
 import layouts as LY
 from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
-                     meta_matmul, meta_pad, u64, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
+                     layout, meta_matmul, meta_pad, u64, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
                      ulp_diff_f32)
 
 pytestmark = pytest.mark.gpu
@@ -626,6 +626,94 @@ def test_softmax_strided_and_special_values(oracle, hip):
     (o,), (h,) = both(oracle, hip, "softmax_f32", lambda: (12, 2, 1, meta_unary([4, 3], [3, 1], 0), In(v.ravel()), Out(12, "f32")))
     assert np.array_equal(np.isnan(o), np.isnan(h))
     assert np.allclose(o[~np.isnan(o)], h[~np.isnan(o)], rtol=1e-6)
+
+
+# ---------------------------------------------------------------------------------------------------
+# index ops: bit-exact, same order of the adds as the reference's host loops
+# ---------------------------------------------------------------------------------------------------
+INDEX_SHAPES = [([5, 7], 0), ([5, 7], 1), ([3, 4, 6], 1), ([2, 3, 4, 5], 2), ([300, 64], 0), ([64, 300], 1), ([17], 0)]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("it", ["i32", "i64"])
+@pytest.mark.parametrize("shape,dim", INDEX_SHAPES)
+def test_index_select_and_index_add(oracle, hip, shape, dim, it, dt):
+    r = rng(149)
+    ity = np.int32 if it == "i32" else np.int64
+    n = int(np.prod(shape))
+    x = to_storage(np.concatenate([[9.0], r.standard_normal(n)]).astype(np.float32), dt)
+    n_idx = 2 * shape[dim] + 3                                          # plenty of repeats
+    idx = np.concatenate([[0, 0], r.integers(0, shape[dim], n_idx)]).astype(ity)      # offset 2
+    out_shape = list(shape)
+    out_shape[dim] = n_idx
+    n_out = int(np.prod(out_shape))
+    (o,), (h,) = both(oracle, hip, f"index_select_{dt}_{it}",
+                      lambda: (len(shape), dim, layout(shape, off=1), n_idx, 1, 2, In(idx), In(x), Out(n_out, dt)))
+    assert same_bits(o, h)
+    src = to_storage(r.standard_normal(n_out + 1).astype(np.float32), dt)
+    (o,), (h,) = both(oracle, hip, f"index_add_{dt}_{it}",
+                      lambda: (len(shape), dim, layout(shape, off=1), layout(out_shape, off=1), n_idx, 1, 2, In(idx), In(src), InOut(x.copy())))
+    assert same_bits(o, h)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,dim,idx_len", [([5, 7], 1, 3), ([5, 7], 0, 8), ([3, 4, 6], 2, 6), ([2, 3, 4], 1, 1), ([128, 1000], 1, 1), ([200, 50], 0, 500)])
+def test_gather_and_scatter_add(oracle, hip, shape, dim, idx_len, dt):
+    r = rng(151)
+    n = int(np.prod(shape))
+    x = to_storage(r.standard_normal(n).astype(np.float32), dt)
+    ishape = list(shape)
+    ishape[dim] = idx_len
+    index = r.integers(-shape[dim], shape[dim], ishape).astype(np.int64).ravel()
+    m = index.size
+    (o,), (h,) = both(oracle, hip, f"gather_{dt}_i64", lambda: (len(shape), dim, layout(shape), layout(ishape), In(index), In(x), Out(m, dt)))
+    assert same_bits(o, h)
+    src = to_storage(r.standard_normal(m).astype(np.float32), dt)
+    (o,), (h,) = both(oracle, hip, f"scatter_add_{dt}_i64",
+                      lambda: (len(shape), dim, layout(shape), layout(ishape), layout(ishape), In(index), In(src), InOut(x.copy())))
+    assert same_bits(o, h)
+
+
+def test_index_ops_on_permuted_tensors(oracle, hip):
+    r = rng(157)
+    lay = LY.permuted([6, 9, 4], [2, 0, 1], off=3)
+    st = np.concatenate([np.zeros(3), r.standard_normal(216)]).astype(np.float32)
+    idx = r.integers(0, 9, 5).astype(np.int32)
+    L = layout([6, 9, 4], lay["strides"], lay["off"])
+    (o,), (h,) = both(oracle, hip, "index_select_f32_i32", lambda: (3, 1, L, 5, 1, 0, In(idx), In(st), Out(6 * 5 * 4, "f32")))
+    assert same_bits(o, h)
+    src = r.standard_normal(6 * 5 * 4).astype(np.float32)
+    (o,), (h,) = both(oracle, hip, "index_add_f32_i32", lambda: (3, 1, L, layout([6, 5, 4]), 5, 1, 0, In(idx), In(src), InOut(st.copy())))
+    assert same_bits(o, h)
+    index = r.integers(0, 4, (6, 9, 2)).astype(np.int32).ravel()
+    (o,), (h,) = both(oracle, hip, "gather_f32_i32", lambda: (3, 2, L, layout([6, 9, 2]), In(index), In(st), Out(index.size, "f32")))
+    assert same_bits(o, h)
+
+
+def test_bincount(oracle, hip):
+    r = rng(163)
+    for it, ity in (("i32", np.int32), ("i64", np.int64)):
+        v = r.integers(0, 1000, 200000).astype(ity)
+        (o,), (h,) = both(oracle, hip, f"bincount_{it}", lambda: (v.size, 1, 0, In(v), 1024, Out(1024, it)))
+        assert np.array_equal(o, h) and int(h.sum()) == v.size
+        for dt in DTS:
+            w = to_storage(r.standard_normal(5000).astype(np.float32), dt)
+            (o,), (h,) = both(oracle, hip, f"bincount_weighted_{dt}_{it}", lambda: (5000, 1, 0, In(v[:5000]), 1, 0, In(w), 1024, Out(1024, dt)))
+            assert same_bits(o, h)
+
+
+def test_index_out_of_bounds_is_reported(hip):
+    import maidenx_amd.lib as L
+    L.check()
+    bad = np.array([0, 3, 1], dtype=np.int32)
+    with pytest.raises(L.HipError, match="index out of bounds"):
+        hip.call("index_select_f32_i32", 1, 0, layout([3]), 3, 1, 0, In(bad), In(np.arange(3, dtype=np.float32)), Out(3, "f32"))
+    # the flag was cleared with the report: a valid call afterwards is clean
+    (h,) = hip.call("index_select_f32_i32", 1, 0, layout([3]), 3, 1, 0, In(np.array([2, 1, 0], dtype=np.int32)),
+                    In(np.arange(3, dtype=np.float32)), Out(3, "f32"))
+    assert h.tolist() == [2.0, 1.0, 0.0]
+    with pytest.raises(L.HipError, match="index out of bounds"):
+        hip.call("gather_f32_i32", 1, 0, layout([3]), layout([2]), In(np.array([-4, 0], dtype=np.int32)), In(np.arange(3, dtype=np.float32)), Out(2, "f32"))
 
 
 # ---------------------------------------------------------------------------------------------------

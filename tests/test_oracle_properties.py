@@ -371,3 +371,87 @@ def test_oracle_softmax_bf16_rounds_every_step(oracle):
         s = b(s + t)
     want = f32_to_bf16(np.array([t / s for t in e], dtype=np.float32)).ravel()
     assert np.array_equal(y, want)
+
+
+# ---- index ops: numpy's own take / take_along_axis / add.at / bincount -------------------------------------
+from helpers import layout  # noqa: E402
+
+
+@pytest.mark.parametrize("shape,dim", [([5, 7], 0), ([5, 7], 1), ([3, 4, 6], 1), ([2, 3, 4, 5], 2)])
+@pytest.mark.parametrize("it", ["i32", "i64"])
+def test_oracle_index_select_and_index_add_vs_numpy(oracle, shape, dim, it):
+    r = rng(131)
+    ity = np.int32 if it == "i32" else np.int64
+    x = r.standard_normal(shape)
+    n_idx = 9
+    idx = r.integers(0, shape[dim], n_idx).astype(ity)            # with repeats
+    out_shape = list(shape)
+    out_shape[dim] = n_idx
+    (y,) = oracle.call(f"index_select_f64_{it}", len(shape), dim, layout(shape), n_idx, 1, 0, In(idx), In(x.ravel()),
+                       Out(int(np.prod(out_shape)), "f64"))
+    assert np.array_equal(y.reshape(out_shape), np.take(x, idx, axis=dim))
+    # a permuted input reads the same logical tensor
+    perm = list(range(len(shape)))[::-1]
+    lay = LY.permuted(shape, perm)
+    st = np.ascontiguousarray(np.transpose(x, np.argsort(perm))).ravel()
+    assert np.array_equal(LY.gather(st, lay), x)
+    (y2,) = oracle.call(f"index_select_f64_{it}", len(shape), dim, layout(shape, lay["strides"]), n_idx, 1, 0, In(idx), In(st),
+                        Out(int(np.prod(out_shape)), "f64"))
+    assert np.array_equal(y2, y)
+    # index_add_ is the scatter that numpy's add.at does (unbuffered, in index order)
+    src = r.standard_normal(out_shape)
+    want = x.copy()
+    sl = [slice(None)] * len(shape)
+    for i, t in enumerate(idx):
+        a, b = list(sl), list(sl)
+        a[dim], b[dim] = int(t), i
+        want[tuple(a)] = want[tuple(a)] + src[tuple(b)]
+    (z,) = oracle.call(f"index_add_f64_{it}", len(shape), dim, layout(shape), layout(out_shape), n_idx, 1, 0, In(idx), In(src.ravel()),
+                       InOut(x.ravel().copy()))
+    assert np.array_equal(z.reshape(shape), want)
+    ref = x.copy()
+    index = [slice(None)] * len(shape)
+    index[dim] = idx
+    np.add.at(ref, tuple(index), src)
+    assert np.allclose(z.reshape(shape), ref, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("shape,dim,idx_len", [([5, 7], 1, 3), ([5, 7], 0, 8), ([3, 4, 6], 2, 6), ([2, 3, 4], 1, 1)])
+def test_oracle_gather_and_scatter_add_vs_numpy(oracle, shape, dim, idx_len):
+    r = rng(137)
+    x = r.standard_normal(shape)
+    ishape = list(shape)
+    ishape[dim] = idx_len
+    index = r.integers(-shape[dim], shape[dim], ishape).astype(np.int64)       # negative values wrap
+    (y,) = oracle.call("gather_f64_i64", len(shape), dim, layout(shape), layout(ishape), In(index.ravel()), In(x.ravel()),
+                       Out(index.size, "f64"))
+    assert np.array_equal(y.reshape(ishape), np.take_along_axis(x, np.where(index < 0, index + shape[dim], index), axis=dim))
+    src = r.standard_normal(ishape)
+    ref = x.copy()
+    pos = np.where(index < 0, index + shape[dim], index)
+    grids = list(np.meshgrid(*[np.arange(s) for s in ishape], indexing="ij"))
+    grids[dim] = pos
+    np.add.at(ref, tuple(grids), src)
+    (z,) = oracle.call("scatter_add_f64_i64", len(shape), dim, layout(shape), layout(ishape), layout(ishape), In(index.ravel()),
+                       In(src.ravel()), InOut(x.ravel().copy()))
+    assert np.allclose(z.reshape(shape), ref, rtol=1e-12, atol=1e-12)
+    # gather and scatter_add_ are adjoint: <gather(x), g> = <x, scatter_add(0, g)>
+    (s0,) = oracle.call("scatter_add_f64_i64", len(shape), dim, layout(shape), layout(ishape), layout(ishape), In(index.ravel()),
+                        In(src.ravel()), InOut(np.zeros(x.size)))
+    assert abs(np.dot(y, src.ravel()) - np.dot(x.ravel(), s0)) < 1e-9
+
+
+def test_oracle_bincount_vs_numpy_and_errors(oracle):
+    r = rng(139)
+    v = r.integers(0, 50, 1000).astype(np.int32)
+    (c,) = oracle.call("bincount_i32", 1000, 1, 0, In(v), 64, Out(64, "i32"))
+    assert np.array_equal(c, np.bincount(v, minlength=64))
+    w = r.standard_normal(1000)
+    (s,) = oracle.call("bincount_weighted_f64_i32", 1000, 1, 0, In(v), 1, 0, In(w), 64, Out(64, "f64"))
+    assert np.allclose(s, np.bincount(v, weights=w, minlength=64), rtol=1e-12, atol=1e-12)
+    assert oracle.lib.oracle_index_error() == 0
+    bad = np.array([0, 3, 1], dtype=np.int32)
+    oracle.call("index_select_f64_i32", 1, 0, layout([3]), 3, 1, 0, In(bad), In(np.arange(3.0)), Out(3, "f64"))
+    assert oracle.lib.oracle_index_error() == 1          # IndexOutOfBounds in the reference
+    oracle.call("gather_f64_i32", 1, 0, layout([3]), layout([2]), In(np.array([-4, 0], dtype=np.int32)), In(np.arange(3.0)), Out(2, "f64"))
+    assert oracle.lib.oracle_index_error() == 1
