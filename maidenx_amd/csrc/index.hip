@@ -13,8 +13,13 @@
 // reference's order is ascending position along `dim`: one thread owns a line and walks it in that
 // order, so results are bit-identical to the host loops and deterministic.  Counts are integers
 // (atomics are exact); weighted bincount lets one thread own a bin and scan the input in order.
+// index_add_ with many indices sorts them by destination first (stable), see below.
 // An index outside its range is skipped and raises the device-side index flag, which
 // hip_get_last_status() reports as an invalid argument (the reference returns IndexOutOfBounds).
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
 #include "mxh.hpp"
 #include "ops.hpp"
 
@@ -67,6 +72,30 @@ __global__ __launch_bounds__(IB) void index_select_kernel(IdxSpace sp, Lay in, c
     out[o] = src[dot(sp, c, in, sp.dim) + (int64_t)idx * in.strides[sp.dim]];
 }
 
+// contiguous input seen as [outer, D, inner] with inner a multiple of the 16-byte vector: rows move as vectors
+template <class T, class I, int VEC>
+__global__ __launch_bounds__(IB) void index_select_rows_kernel(const I* __restrict__ indices, int64_t idx_stride, int64_t idx_offset,
+                                                               uint32_t n_idx, uint32_t D, uint32_t inner_v, FastDiv div_inner,
+                                                               FastDiv div_nidx, const T* __restrict__ src, T* __restrict__ out,
+                                                               size_t nvec, int* flag) {
+    struct alignas(16) V { T v[VEC]; };
+    size_t o = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (o >= nvec) return;
+    uint32_t r, v, outer, i;
+    fd_divmod((uint32_t)o, div_inner, r, v);
+    fd_divmod(r, div_nidx, outer, i);
+    const int32_t idx = (int32_t)indices[idx_offset + (int64_t)i * idx_stride];
+    V val;
+    if (idx < 0 || (uint32_t)idx >= D) {
+        *flag = 1;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) val.v[e] = T{};
+    } else {
+        val = *(const V*)(src + (((size_t)outer * D + (uint32_t)idx) * inner_v + v) * VEC);
+    }
+    *(V*)(out + o * VEC) = val;
+}
+
 // ---- gather: iteration space = index dims ---------------------------------------------------------
 template <class T, class I>
 __global__ __launch_bounds__(IB) void gather_kernel(IdxSpace sp, Lay in, Lay ix, uint32_t in_dim_size, const I* __restrict__ index,
@@ -97,6 +126,77 @@ __global__ __launch_bounds__(IB) void index_add_kernel(IdxSpace sp, Lay self, La
         T* p = dst + d0 + (int64_t)idx * self.strides[sp.dim];
         *p = Ar<T>::add(*p, src[s0 + (int64_t)i * sr.strides[sp.dim]]);
     }
+}
+
+// Many indices, few lines (an embedding gradient): the indices are sorted by destination with a stable
+// radix sort (vendor primitive; equal destinations keep ascending i), and one thread per destination
+// element adds its sources in that order — the same order as the walk above, with parallelism over
+// the whole of self instead of over the lines.
+template <class I>
+__global__ __launch_bounds__(IB) void index_keys_kernel(const I* __restrict__ indices, int64_t idx_stride, int64_t idx_offset, uint32_t n_idx,
+                                                        uint32_t self_dim_size, uint32_t* keys, uint32_t* vals, int* flag) {
+    uint32_t i = blockIdx.x * IB + threadIdx.x;
+    if (i >= n_idx) return;
+    const int32_t idx = (int32_t)indices[idx_offset + (int64_t)i * idx_stride];
+    const bool ok = idx >= 0 && (uint32_t)idx < self_dim_size;
+    if (!ok) *flag = 1;
+    keys[i] = ok ? (uint32_t)idx : self_dim_size;       // out of range: sorted behind every real destination, never applied
+    vals[i] = i;
+}
+
+template <class T>
+__global__ __launch_bounds__(IB) void index_add_sorted_kernel(IdxSpace sp, Lay self, Lay sr, const uint32_t* __restrict__ keys,
+                                                              const uint32_t* __restrict__ vals, uint32_t n_idx, uint32_t lines,
+                                                              FastDiv div_lines, const T* __restrict__ src, T* __restrict__ dst,
+                                                              size_t work) {
+    size_t wi = (size_t)blockIdx.x * IB + threadIdx.x;
+    if (wi >= work) return;
+    uint32_t d, l;
+    fd_divmod((uint32_t)wi, div_lines, d, l);
+    // first entry with key >= d
+    uint32_t lo = 0, hi = n_idx;
+    while (lo < hi) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (keys[mid] < d) lo = mid + 1;
+        else hi = mid;
+    }
+    if (lo >= n_idx || keys[lo] != d) return;
+    uint32_t c[MAXD];
+    split(sp, l, c);
+    const int64_t s0 = dot(sp, c, sr, sp.dim);
+    T* p = dst + dot(sp, c, self, sp.dim) + (int64_t)d * self.strides[sp.dim];
+    T acc = *p;
+    for (uint32_t k = lo; k < n_idx && keys[k] == d; ++k) acc = Ar<T>::add(acc, src[s0 + (int64_t)vals[k] * sr.strides[sp.dim]]);
+    *p = acc;
+}
+
+// the same for contiguous self [outer, D, inner] and src [outer, n_idx, inner] with inner a multiple of the
+// 16-byte vector: a block owns (outer, destination row, 256 vectors of the row) and searches once
+template <class T, int VEC>
+__global__ __launch_bounds__(IB) void index_add_rows_kernel(const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals, uint32_t n_idx,
+                                                            uint32_t D, uint32_t inner_v, uint32_t chunks, FastDiv div_chunks, FastDiv div_D,
+                                                            const T* __restrict__ src, T* __restrict__ dst) {
+    struct alignas(16) V { T v[VEC]; };
+    uint32_t r, chunk, outer, d;
+    fd_divmod(blockIdx.x, div_chunks, r, chunk);
+    fd_divmod(r, div_D, outer, d);
+    uint32_t lo = 0, hi = n_idx;
+    while (lo < hi) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (keys[mid] < d) lo = mid + 1;
+        else hi = mid;
+    }
+    if (lo >= n_idx || keys[lo] != d) return;
+    const uint32_t v = chunk * IB + threadIdx.x;
+    if (v >= inner_v) return;
+    V* p = (V*)(dst + (((size_t)outer * D + d) * inner_v + v) * VEC);
+    V acc = *p;
+    for (uint32_t k = lo; k < n_idx && keys[k] == d; ++k) {
+        const V s = *(const V*)(src + (((size_t)outer * n_idx + vals[k]) * inner_v + v) * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc.v[e] = Ar<T>::add(acc.v[e], s.v[e]);
+    }
+    *p = acc;
 }
 
 template <class T, class I>
@@ -191,6 +291,21 @@ void index_select(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, 
     if (!make_space(nd, out_dims, dim, -1, sp, &n, "index_select: bad shape")) return;
     read_layout(nd, in_layout, in);
     if (n == 0) return;
+    {
+        constexpr int VEC = 16 / sizeof(T);
+        size_t inner = 1;
+        for (size_t d = dim + 1; d < nd; ++d) inner *= in_layout[d];
+        const T* base = input + in_layout[2 * nd];
+        if (ref_is_contiguous(nd, in_layout, in_layout + nd) && inner % VEC == 0 && ((uintptr_t)base % 16) == 0 && ((uintptr_t)output % 16) == 0 &&
+            n_idx < (1ull << 31) && inner / VEC < (1ull << 31)) {
+            size_t nvec = n / VEC;
+            hipLaunchKernelGGL((index_select_rows_kernel<T, I, VEC>), dim3(cdiv(nvec, IB)), dim3(IB), 0, stream(), indices, (int64_t)idx_stride,
+                               (int64_t)idx_offset, (uint32_t)n_idx, (uint32_t)in_layout[dim], (uint32_t)(inner / VEC),
+                               make_fastdiv((uint32_t)(inner / VEC)), make_fastdiv((uint32_t)n_idx), base, output, nvec, flag);
+            MXH_LAUNCH_CHECK("index_select");
+            return;
+        }
+    }
     hipLaunchKernelGGL((index_select_kernel<T, I>), dim3(cdiv(n, IB)), dim3(IB), 0, stream(), sp, in, indices, (int64_t)idx_stride,
                        (int64_t)idx_offset, (uint32_t)in_layout[dim], input, output, n, flag);
     MXH_LAUNCH_CHECK("index_select");
@@ -226,6 +341,47 @@ void index_add(size_t nd, size_t dim, const size_t* self_layout, const size_t* s
     read_layout(nd, self_layout, sl);
     read_layout(nd, src_layout, sr);
     if (lines == 0 || n_idx == 0) return;
+    const size_t D = self_layout[dim];
+    if (n_idx >= 256 && lines < (1ull << 31) && D * lines < (1ull << 31) && D < (1ull << 31) - 1) {
+        // [keys in | keys out | values in | values out | sort workspace] in scratch slot 1
+        size_t sort_bytes = 0;
+        uint32_t* nil = nullptr;
+        unsigned bits = 1;
+        while ((1ull << bits) <= D) ++bits;
+        if (rocprim::radix_sort_pairs(nullptr, sort_bytes, nil, nil, nil, nil, n_idx, 0u, bits, stream()) != hipSuccess) {
+            set_status(ERR_LAUNCH, "index_add_: sort workspace query failed");
+            return;
+        }
+        const size_t arr = (n_idx * sizeof(uint32_t) + 255) / 256 * 256;
+        char* ws = (char*)scratch(4 * arr + sort_bytes, 1);
+        if (!ws) return;
+        uint32_t *k_in = (uint32_t*)ws, *k_out = (uint32_t*)(ws + arr), *v_in = (uint32_t*)(ws + 2 * arr), *v_out = (uint32_t*)(ws + 3 * arr);
+        hipLaunchKernelGGL(index_keys_kernel<I>, dim3(cdiv(n_idx, IB)), dim3(IB), 0, stream(), indices, (int64_t)idx_stride, (int64_t)idx_offset,
+                           (uint32_t)n_idx, (uint32_t)D, k_in, v_in, flag);
+        MXH_HIP(rocprim::radix_sort_pairs(ws + 4 * arr, sort_bytes, k_in, k_out, v_in, v_out, n_idx, 0u, bits, stream()));
+        {
+            constexpr int VEC = 16 / sizeof(T);
+            size_t inner = 1, outer = 1;
+            for (size_t d = dim + 1; d < nd; ++d) inner *= self_layout[d];
+            for (size_t d = 0; d < dim; ++d) outer *= self_layout[d];
+            T* dbase = self + self_layout[2 * nd];
+            const T* sbase = src + src_layout[2 * nd];
+            const size_t inner_v = inner / VEC, chunks = cdiv(inner_v, (size_t)IB);
+            if (ref_is_contiguous(nd, self_layout, self_layout + nd) && ref_is_contiguous(nd, src_layout, src_layout + nd) && inner % VEC == 0 &&
+                ((uintptr_t)dbase % 16) == 0 && ((uintptr_t)sbase % 16) == 0 && outer * D * chunks < (1ull << 31)) {
+                hipLaunchKernelGGL((index_add_rows_kernel<T, VEC>), dim3((unsigned)(outer * D * chunks)), dim3(IB), 0, stream(), k_out, v_out,
+                                   (uint32_t)n_idx, (uint32_t)D, (uint32_t)inner_v, (uint32_t)chunks, make_fastdiv((uint32_t)chunks),
+                                   make_fastdiv((uint32_t)D), sbase, dbase);
+                MXH_LAUNCH_CHECK("index_add_rows");
+                return;
+            }
+        }
+        const size_t work = D * lines;
+        hipLaunchKernelGGL(index_add_sorted_kernel<T>, dim3(cdiv(work, IB)), dim3(IB), 0, stream(), sp, sl, sr, k_out, v_out, (uint32_t)n_idx,
+                           (uint32_t)lines, make_fastdiv((uint32_t)lines), src, self, work);
+        MXH_LAUNCH_CHECK("index_add_sorted");
+        return;
+    }
     hipLaunchKernelGGL((index_add_kernel<T, I>), dim3(cdiv(lines, IB)), dim3(IB), 0, stream(), sp, sl, sr, indices, (int64_t)idx_stride,
                        (int64_t)idx_offset, (uint32_t)n_idx, (uint32_t)self_layout[dim], src, self, lines, flag);
     MXH_LAUNCH_CHECK("index_add");

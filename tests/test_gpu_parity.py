@@ -674,6 +674,22 @@ def test_gather_and_scatter_add(oracle, hip, shape, dim, idx_len, dt):
     assert same_bits(o, h)
 
 
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,dim,n_idx", [([50, 64], 0, 3000), ([7, 40, 8], 1, 1000), ([33, 500], 1, 2048), ([3, 40, 2048], 1, 700), ([6, 50, 6], 1, 900)])
+def test_index_add_with_many_indices(oracle, hip, shape, dim, n_idx, dt):
+    # enough indices for the sorted path; some out of range, which both sides skip or stop at — so keep them valid here
+    r = rng(167)
+    n = int(np.prod(shape))
+    x = to_storage(r.standard_normal(n).astype(np.float32), dt)
+    idx = r.integers(0, shape[dim], n_idx).astype(np.int32)
+    src_shape = list(shape)
+    src_shape[dim] = n_idx
+    src = to_storage(r.standard_normal(int(np.prod(src_shape))).astype(np.float32), dt)
+    (o,), (h,) = both(oracle, hip, f"index_add_{dt}_i32",
+                      lambda: (len(shape), dim, layout(shape), layout(src_shape), n_idx, 1, 0, In(idx), In(src), InOut(x.copy())))
+    assert same_bits(o, h)
+
+
 def test_index_ops_on_permuted_tensors(oracle, hip):
     r = rng(157)
     lay = LY.permuted([6, 9, 4], [2, 0, 1], off=3)
