@@ -732,6 +732,37 @@ def test_index_out_of_bounds_is_reported(hip):
         hip.call("gather_f32_i32", 1, 0, layout([3]), layout([2]), In(np.array([-4, 0], dtype=np.int32)), In(np.arange(3, dtype=np.float32)), Out(2, "f32"))
 
 
+@pytest.mark.parametrize("dt", DTS)
+def test_empty_inputs_are_no_ops(hip, dt):
+    """Zero elements anywhere: nothing is launched, nothing is written, no error is recorded."""
+    import maidenx_amd.lib as L
+    L.check()
+    e = np.zeros(0, dtype=np.float32 if dt == "f32" else np.uint16)
+    poison = lambda n=4: Out(n, dt)
+    keep = poison().arr.copy()
+    for call in (
+        lambda: hip.call(f"add_{dt}", 0, 2, meta_binary([0, 5], [5, 1], [5, 1]), In(e), In(e), poison()),
+        lambda: hip.call(f"add_inplace_{dt}", 0, 1, meta_binary([0], [1], [1]), InOut(poison().arr), In(e)),
+        lambda: hip.call(f"exp_{dt}", 0, 1, meta_unary([0], [1]), In(e), poison()),
+        lambda: hip.call(f"mul_scalar_{dt}", 0, 1, meta_unary([0], [1]), In(e), const_arg(2.0, dt), poison()),
+        lambda: hip.call(f"sum_{dt}", 0, 2, 1, meta_reduce([0, 4], [4, 1], 1), In(e), poison()),
+        lambda: hip.call(f"sum_to_shape_{dt}", 0, 2, meta_sum_to_shape([0, 4], [4, 1], [0, 1]), In(e), poison()),
+        lambda: hip.call(f"matmul_{dt}", 0, meta_matmul([0, 3], [0, 2], [2, 3], [2, 1], [3, 1]), In(e), In(to_storage(np.ones(6, np.float32), dt)), poison()),
+        lambda: hip.call(f"pad_with_constant_{dt}", 0, 0, 2, meta_pad([0, 3], [3, 1], 0, [0, 5], [(0, 0), (1, 1)]), In(e), poison(), const_arg(1.0, dt)),
+        lambda: hip.call(f"pad_with_replication_{dt}", 0, 0, 2, meta_pad([0, 3], [3, 1], 0, [0, 5], [(0, 0), (1, 1)]), In(e), poison()),
+        lambda: hip.call(f"conv2d_im2col_{dt}", 0, meta_conv(0, 3, 4, 4, 3, 3, 4, 4, 1, 1, 1, 1), In(e), poison()),
+        lambda: hip.call(f"conv2d_col2im_{dt}", 0, meta_conv(0, 3, 4, 4, 3, 3, 4, 4, 1, 1, 1, 1), In(e), poison()),
+        lambda: hip.call(f"softmax_{dt}", 0, 2, 1, meta_unary([0, 4], [4, 1]), In(e), poison()),
+        lambda: hip.call(f"index_select_{dt}_i32", 2, 0, layout([3, 0]), 2, 1, 0, In(np.array([0, 1], dtype=np.int32)), In(e), poison()),
+        lambda: hip.call(f"gather_{dt}_i32", 1, 0, layout([3]), layout([0]), In(np.zeros(0, np.int32)), In(to_storage(np.ones(3, np.float32), dt)), poison()),
+        lambda: hip.call(f"fill_{dt}", 0, poison(), const_arg(1.0, dt)),
+        lambda: hip.call(f"copy_strided_{dt}", 0, 1, meta_unary([0], [1]), In(e), poison()),
+    ):
+        (out,) = call()[-1:]
+        assert same_bits(out[:4], keep), "an empty call wrote to its output"
+    L.check()
+
+
 # ---------------------------------------------------------------------------------------------------
 # fill / cast / strided copy (device-side helpers without a reference symbol)
 # ---------------------------------------------------------------------------------------------------
