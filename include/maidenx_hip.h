@@ -29,6 +29,7 @@ extern "C" {
 #endif
 
 typedef uint16_t mx_bf16;   /* bf16 bit pattern */
+typedef uint16_t mx_f16;    /* IEEE binary16 bit pattern (the `half` crate's f16) */
 typedef uint8_t mx_bool;    /* 0 or 1 */
 
 /* ---- status ------------------------------------------------------------------------------------ */
@@ -103,6 +104,7 @@ int hip_graph_destroy(void* graph_exec);
     void hip_div_inplace_##S(size_t num_els, size_t num_dims, const size_t* metadata, T* lhs, const T* rhs);
 MX_DECL_BINARY(float, f32)
 MX_DECL_BINARY(mx_bf16, bf16)
+MX_DECL_BINARY(mx_f16, f16)
 
 /* ---- unary: replaces crates/maidenx_cuda/src/ops/unary.rs:21-77 ------------------------------------
  * metadata = dims[n] | strides[n] | offset   (NULL: contiguous).  input == NULL means "in place on
@@ -128,6 +130,7 @@ MX_DECL_BINARY(mx_bf16, bf16)
     MX_DECL_UNARYC(gt_scalar, T, S, mx_bool) MX_DECL_UNARYC(ge_scalar, T, S, mx_bool)
 MX_DECL_UNARY(float, f32)
 MX_DECL_UNARY(mx_bf16, bf16)
+MX_DECL_UNARY(mx_f16, f16)
 
 /* ---- reduction: replaces crates/maidenx_cuda/src/ops/reduction.rs:19-35 ---------------------------
  * sum/mean/max/min metadata = dims[n] | strides[n] | red_len[r] | red_stride[r] | offset, r = 1
@@ -148,6 +151,7 @@ MX_DECL_UNARY(mx_bf16, bf16)
     void hip_fold_##S(size_t num_els, size_t num_dims, const size_t* metadata, const T* inp, T* out);
 MX_DECL_REDUCE(float, f32)
 MX_DECL_REDUCE(mx_bf16, bf16)
+MX_DECL_REDUCE(mx_f16, f16)
 
 /* ---- matmul: replaces crates/maidenx_cuda/src/ops/matmul.rs:12-29 ---------------------------------
  * metadata = out_ndim, a_ndim, b_ndim | out_shape | a_shape | b_shape | a_strides | b_strides | a_off | b_off
@@ -160,6 +164,7 @@ MX_DECL_REDUCE(mx_bf16, bf16)
                                  const T* a, const T* b, T* grad_a, T* grad_b);
 MX_DECL_MATMUL(float, f32)
 MX_DECL_MATMUL(mx_bf16, bf16)
+MX_DECL_MATMUL(mx_f16, f16)
 
 /* ---- padding: replaces crates/maidenx_cuda/src/ops/padding.rs:13-71 (constant mode) ---------------
  * metadata = in_dims[n] | in_strides[n] | in_offset | out_dims[n] | (pad_before, pad_after)[n]
@@ -171,6 +176,7 @@ MX_DECL_MATMUL(mx_bf16, bf16)
                                             const size_t* metadata, const T* grad_out, T* grad_in);
 MX_DECL_PAD(float, f32)
 MX_DECL_PAD(mx_bf16, bf16)
+MX_DECL_PAD(mx_f16, f16)
 
 /* reflection / replication modes of the same file (same metadata, no pad value).
  * Semantics: crates/maidenx_cpu/src/ops/padding.rs:115-325 (forward, bit-exact) and :438-665 (backward:
@@ -187,6 +193,7 @@ MX_DECL_PAD(mx_bf16, bf16)
                                                const size_t* metadata, const T* grad_out, T* grad_in);
 MX_DECL_PAD_EDGE(float, f32)
 MX_DECL_PAD_EDGE(mx_bf16, bf16)
+MX_DECL_PAD_EDGE(mx_f16, f16)
 
 /* ---- conv: replaces crates/maidenx_cuda/src/nn/conv.rs:12-24 --------------------------------------
  * metadata = 12 slots B, C, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w as the kernel
@@ -197,6 +204,7 @@ MX_DECL_PAD_EDGE(mx_bf16, bf16)
     void hip_conv2d_col2im_##S(size_t num_els, const size_t* metadata, const T* col, T* output);
 MX_DECL_CONV(float, f32)
 MX_DECL_CONV(mx_bf16, bf16)
+MX_DECL_CONV(mx_f16, f16)
 
 /* ---- softmax: replaces crates/maidenx_cuda/src/nn/activation/softmax.rs (cuda_softmax_<T>) ------------
  * metadata = dims[n] | strides[n] | offset; dim >= num_dims means the last dim.
@@ -205,6 +213,7 @@ MX_DECL_CONV(mx_bf16, bf16)
  * which walks the leading dims from dim 0 upwards).  The sum is f32 in a fixed order. */
 void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const float* input, float* output);
 void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const mx_bf16* input, mx_bf16* output);
+void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const mx_f16* input, mx_f16* output);
 
 /* ---- index ops -----------------------------------------------------------------------------------
  * No backend symbol exists for these in the reference: crates/maidenx_tensor/src/ops/indexing.rs runs them
@@ -231,6 +240,8 @@ MX_DECL_INDEX(float, f32, int32_t, i32)
 MX_DECL_INDEX(float, f32, int64_t, i64)
 MX_DECL_INDEX(mx_bf16, bf16, int32_t, i32)
 MX_DECL_INDEX(mx_bf16, bf16, int64_t, i64)
+MX_DECL_INDEX(mx_f16, f16, int32_t, i32)
+MX_DECL_INDEX(mx_f16, f16, int64_t, i64)
 void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output);
 void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output);
 
@@ -241,15 +252,21 @@ void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* inp
  * (crates/maidenx_tensor/src/f.rs:19-30).  hip_copy_strided takes the unary metadata layout. */
 void hip_fill_f32(size_t num_els, float* out, float value);
 void hip_fill_bf16(size_t num_els, mx_bf16* out, mx_bf16 value);
+void hip_fill_f16(size_t num_els, mx_f16* out, mx_f16 value);
 void hip_fill_bool(size_t num_els, mx_bool* out, mx_bool value);
 void hip_copy_strided_f32(size_t num_els, size_t num_dims, const size_t* metadata, const float* input, float* output);
 void hip_copy_strided_bf16(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bf16* input, mx_bf16* output);
+void hip_copy_strided_f16(size_t num_els, size_t num_dims, const size_t* metadata, const mx_f16* input, mx_f16* output);
 void hip_cast_bool_f32(size_t num_els, const mx_bool* input, float* output);
 void hip_cast_bool_bf16(size_t num_els, const mx_bool* input, mx_bf16* output);
 void hip_cast_f32_bf16(size_t num_els, const float* input, mx_bf16* output);
 void hip_cast_bf16_f32(size_t num_els, const mx_bf16* input, float* output);
 void hip_cast_f32_bool(size_t num_els, const float* input, mx_bool* output);
 void hip_cast_bf16_bool(size_t num_els, const mx_bf16* input, mx_bool* output);
+void hip_cast_bool_f16(size_t num_els, const mx_bool* input, mx_f16* output);
+void hip_cast_f32_f16(size_t num_els, const float* input, mx_f16* output);
+void hip_cast_f16_f32(size_t num_els, const mx_f16* input, float* output);
+void hip_cast_f16_bool(size_t num_els, const mx_f16* input, mx_bool* output);
 
 #ifdef __cplusplus
 }

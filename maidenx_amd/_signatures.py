@@ -6,7 +6,7 @@ identical argument lists, so a CPU restatement built with another prefix can be 
 import ctypes as C
 
 SZ, P = C.c_size_t, C.c_void_p
-CONST = {"f32": C.c_float, "f64": C.c_double, "bf16": C.c_uint16, "bool": C.c_uint8}
+CONST = {"f32": C.c_float, "f64": C.c_double, "bf16": C.c_uint16, "f16": C.c_uint16, "bool": C.c_uint8}
 
 BINARY = ["add", "sub", "mul", "div", "maximum", "minimum", "logical_and", "logical_or", "logical_xor",
           "eq", "ne", "lt", "le", "gt", "ge"]
@@ -20,7 +20,7 @@ BOOL_OUT = {"logical_and", "logical_or", "logical_xor", "eq", "ne", "lt", "le", 
             "eq_scalar", "ne_scalar", "lt_scalar", "le_scalar", "gt_scalar", "ge_scalar"}
 
 
-def signatures(dtypes=("f32", "bf16")):
+def signatures(dtypes=("f32", "bf16", "f16")):
     """name (without prefix) -> argtypes list."""
     sig = {}
     for dt in dtypes:
@@ -50,7 +50,7 @@ def signatures(dtypes=("f32", "bf16")):
     return sig
 
 
-def index_signatures(dtypes=("f32", "bf16")):
+def index_signatures(dtypes=("f32", "bf16", "f16")):
     """Index ops (host loops in the reference's tensor layer, device entry points here)."""
     sig = {}
     for dt in dtypes:
@@ -68,10 +68,11 @@ def index_signatures(dtypes=("f32", "bf16")):
 def extension_signatures():
     """Entry points of the HIP library that have no counterpart symbol in the reference."""
     sig = index_signatures()
-    for dt in ("f32", "bf16", "bool"):
+    for dt in ("f32", "bf16", "f16", "bool"):
         sig[f"fill_{dt}"] = [SZ, P, CONST[dt]]
-    for dt in ("f32", "bf16"):
+    for dt in ("f32", "bf16", "f16"):
         sig[f"copy_strided_{dt}"] = [SZ, SZ, P, P, P]
-    for a, b in (("bool", "f32"), ("bool", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "bool"), ("bf16", "bool")):
+    for a, b in (("bool", "f32"), ("bool", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "bool"), ("bf16", "bool"),
+                 ("bool", "f16"), ("f32", "f16"), ("f16", "f32"), ("f16", "bool")):
         sig[f"cast_{a}_{b}"] = [SZ, P, P]
     return sig

@@ -38,3 +38,4 @@ using namespace mxh;
 
 MXH_ALL_FOR(float, f32)
 MXH_ALL_FOR(bf16_t, bf16)
+MXH_ALL_FOR(f16_t, f16)

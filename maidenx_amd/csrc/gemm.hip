@@ -35,6 +35,7 @@ namespace mxh {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 struct GemmArgs {
     const void* X;
@@ -63,6 +64,12 @@ template <> struct Elem<bf16_t> {
     static __device__ bf16_t st(float v) { return f2bf(v); }
     static __device__ bf16_t zero() { return bf16_t{0}; }
 };
+template <> struct Elem<f16_t> {
+    static constexpr int VEC = 8;
+    static __device__ float ld(f16_t v) { return h2f(v); }
+    static __device__ f16_t st(float v) { return f2h(v); }
+    static __device__ f16_t zero() { return f16_t{0}; }
+};
 
 constexpr int GB = 256;          // threads per block of the small-shape kernels
 constexpr int TK_BYTES = 128;    // reduction extent of one staged tile, in bytes per row
@@ -73,6 +80,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <class T> __device__ inline uint32_t elem_bits(T v);
 template <> __device__ inline uint32_t elem_bits<float>(float v) { return __builtin_bit_cast(uint32_t, v); }
 template <> __device__ inline uint32_t elem_bits<bf16_t>(bf16_t v) { return v.bits; }
+template <> __device__ inline uint32_t elem_bits<f16_t>(f16_t v) { return v.bits; }
 // pack VEC elements (given one by one) into 16 bytes
 template <class T> struct Pack16;
 template <> struct Pack16<float> {
@@ -82,6 +90,10 @@ template <> struct Pack16<float> {
 template <> struct Pack16<bf16_t> {
     u32x4 r = {0u, 0u, 0u, 0u};
     __device__ void set(int e, bf16_t v) { r[e / 2] |= (uint32_t)v.bits << (16 * (e & 1)); }
+};
+template <> struct Pack16<f16_t> {
+    u32x4 r = {0u, 0u, 0u, 0u};
+    __device__ void set(int e, f16_t v) { r[e / 2] |= (uint32_t)v.bits << (16 * (e & 1)); }
 };
 
 // ---- staging one ROWS x TK operand tile into LDS as [row][TK + PAD] ---------------------------------
@@ -226,6 +238,14 @@ template <> struct Mma<bf16_t> {
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
 };
+template <> struct Mma<f16_t> {
+    static __device__ void run(const u32x4& a, const u32x4& b, f32x16& c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ void run(const u32x4& a, const u32x4& b, f32x4& c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
 template <> struct Mma<float> {
     // one 16-byte fragment feeds four 32x32x2 steps; lane (row, h) holds k = 4h .. 4h+3 of an
     // 8-wide slice, and step e pairs element e of both operands — any fixed pairing of k is valid.
@@ -264,6 +284,7 @@ template <> struct Cfgs<bf16_t> {
     using Small = GemmCfg<2, 2, 4, 4, 16>;
     using Tall = GemmCfg<4, 1, 4, 4, 16>;
 };
+template <> struct Cfgs<f16_t> : Cfgs<bf16_t> {};
 #endif
 
 // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
@@ -733,3 +754,4 @@ using namespace mxh;
 
 MXH_MATMUL_FOR(float, f32)
 MXH_MATMUL_FOR(bf16_t, bf16)
+MXH_MATMUL_FOR(f16_t, f16)

@@ -467,6 +467,8 @@ MXH_INDEX_FOR(float, f32, int32_t, i32)
 MXH_INDEX_FOR(float, f32, int64_t, i64)
 MXH_INDEX_FOR(bf16_t, bf16, int32_t, i32)
 MXH_INDEX_FOR(bf16_t, bf16, int64_t, i64)
+MXH_INDEX_FOR(f16_t, f16, int32_t, i32)
+MXH_INDEX_FOR(f16_t, f16, int64_t, i64)
 
 extern "C" void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output) {
     bincount<int32_t>(n, stride, offset, input, out_size, output);

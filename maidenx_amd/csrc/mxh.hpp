@@ -59,6 +59,19 @@ __host__ __device__ inline bf16_t f2bf(float f) {
     return r;
 }
 
+// ---- f16 storage type -------------------------------------------------------------------
+// IEEE binary16 as the `half` crate's f16 stores it; conversions are the hardware's
+// (round to nearest even; the crate's software path gives the same bits).
+struct f16_t {
+    uint16_t bits;
+};
+__host__ __device__ inline float h2f(f16_t h) { return (float)__builtin_bit_cast(_Float16, h.bits); }
+__host__ __device__ inline f16_t f2h(float f) {
+    f16_t r;
+    r.bits = __builtin_bit_cast(uint16_t, (_Float16)f);
+    return r;
+}
+
 // ---- division by an invariant 32-bit integer (numerators below 2^31) ---------------------
 struct FastDiv {
     uint32_t d, mul, shift;

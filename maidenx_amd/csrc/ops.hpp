@@ -40,6 +40,20 @@ template <> struct Ar<bf16_t> {
     static __device__ T max_(T a, T b) { return bf2f(a) > bf2f(b) ? a : b; }   // `if a > b { a } else { b }`
     static __device__ T min_(T a, T b) { return bf2f(a) < bf2f(b) ? a : b; }
 };
+template <> struct Ar<f16_t> {       // the `half` crate's f16: the same "f32 operation, round" scheme as bf16
+    using T = f16_t;
+    static __device__ T zero() { return T{0}; }
+    static __device__ T inf() { return T{0x7C00}; }
+    static __device__ T from_f32(float v) { return f2h(v); }
+    static __device__ float to_f32(T v) { return h2f(v); }
+    static __device__ T add(T a, T b) { return f2h(h2f(a) + h2f(b)); }
+    static __device__ T sub(T a, T b) { return f2h(h2f(a) - h2f(b)); }
+    static __device__ T mul(T a, T b) { return f2h(h2f(a) * h2f(b)); }
+    static __device__ T div(T a, T b) { return f2h(h2f(a) / h2f(b)); }
+    static __device__ T neg(T a) { return T{(uint16_t)(a.bits ^ 0x8000u)}; }
+    static __device__ T max_(T a, T b) { return h2f(a) > h2f(b) ? a : b; }
+    static __device__ T min_(T a, T b) { return h2f(a) < h2f(b) ? a : b; }
+};
 template <class T> __device__ inline float F(T v) { return Ar<T>::to_f32(v); }
 template <class T> __device__ inline bool is_zero(T v) { return F(v) == 0.0f; }
 

@@ -6,6 +6,7 @@
 // multiply-high division on the collapsed shape (dims without padding whose input strides chain
 // are merged, so [B,C,H,W] padded on H,W walks two divisions, not four).
 #include "elementwise.hpp"
+#include "ops.hpp"
 
 namespace mxh {
 
@@ -85,8 +86,7 @@ __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __r
         } else {
             if (inside) {
                 T g = v.v[e];
-                if constexpr (sizeof(T) == 4) dst[idx] = 0.0f + g;        // −0 → +0 like the reference's sums from zero
-                else dst[idx] = f2bf(0.0f + bf2f(g));
+                dst[idx] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(g));      // −0 → +0 like the reference's sums from zero
             }
         }
         // next output element; at the end of a row, carry into the outer coordinates
@@ -283,8 +283,7 @@ template <class T, int D>
 __device__ __forceinline__ void edge_gather(const PadSpace& sp, const EdgeWalk& w, int mode, const uint32_t (&p)[MAXD], int64_t o,
                                             const T* __restrict__ go, float& acc) {
     if constexpr (D == MAXD) {
-        if constexpr (sizeof(T) == 4) acc += go[o];
-        else acc += bf2f(go[o]);
+        acc += Ar<T>::to_f32(go[o]);
     } else {
         if (D >= sp.ndims) { edge_gather<T, MAXD>(sp, w, mode, p, o, go, acc); return; }
         EdgeIter it;
@@ -315,8 +314,7 @@ __global__ __launch_bounds__(PB) void pad_edge_backward_kernel(PadSpace sp, Edge
     }
     float acc = 0.0f;
     edge_gather<T, 0>(sp, w, mode, p, 0, go, acc);
-    if constexpr (sizeof(T) == 4) gi[dst] = acc;
-    else gi[dst] = f2bf(acc);
+    gi[dst] = Ar<T>::from_f32(acc);
 }
 
 static bool edge_space(size_t nd_full, const size_t* md_full, int mode, PadSpace& sp, EdgeWalk& in_walk, size_t* in_off, const char* who) {
@@ -437,5 +435,7 @@ using namespace mxh;
 
 MXH_PAD_EDGE_FOR(float, f32)
 MXH_PAD_EDGE_FOR(bf16_t, bf16)
+MXH_PAD_EDGE_FOR(f16_t, f16)
 MXH_PAD_FOR(float, f32)
 MXH_PAD_FOR(bf16_t, bf16)
+MXH_PAD_FOR(f16_t, f16)

@@ -51,6 +51,14 @@ template <> struct IO<bf16_t> {
         return div != 0.0f ? f2bf(bf2f(s) / bf2f(f2bf(div))) : s;
     }
 };
+template <> struct IO<f16_t> {
+    static constexpr bool is_bf16 = true;      // "16-bit": f16::from_f32(f32::MIN) is -inf as well (reduction.rs:602,615)
+    static __device__ float ld(f16_t v) { return h2f(v); }
+    static __device__ f16_t fin(float acc, float div) {
+        f16_t s = f2h(acc);
+        return div != 0.0f ? f2h(h2f(s) / h2f(f2h(div))) : s;
+    }
+};
 
 // ---- wave64 butterfly on DPP ------------------------------------------------------------------
 template <class R, int CTRL>
@@ -771,3 +779,4 @@ using namespace mxh;
 
 MXH_REDUCE_FOR(float, f32)
 MXH_REDUCE_FOR(bf16_t, bf16)
+MXH_REDUCE_FOR(f16_t, f16)

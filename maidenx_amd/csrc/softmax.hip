@@ -30,6 +30,12 @@ template <> struct SM<bf16_t> {
     static __device__ bf16_t fin(float e, float s) { return f2bf(e / bf2f(f2bf(s))); }
 };
 
+template <> struct SM<f16_t> {
+    static __device__ float ld(f16_t v) { return h2f(v); }
+    static __device__ float shifted(float x, float m) { return h2f(f2h(m_exp(h2f(f2h(x - m))))); }
+    static __device__ f16_t fin(float e, float s) { return f2h(e / h2f(f2h(s))); }
+};
+
 constexpr int SB = 256;
 
 __device__ inline float wave_max(float v) {
@@ -336,6 +342,9 @@ using namespace mxh;
 
 extern "C" void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const float* in, float* out) {
     softmax<float>(num_els, num_dims, dim, md, in, out);
+}
+extern "C" void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const f16_t* in, f16_t* out) {
+    softmax<f16_t>(num_els, num_dims, dim, md, in, out);
 }
 extern "C" void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const bf16_t* in, bf16_t* out) {
     softmax<bf16_t>(num_els, num_dims, dim, md, in, out);

@@ -27,6 +27,14 @@ template <> struct OpConvert<float, bf16_t> { using In = float; using Out = bf16
     __device__ bf16_t operator()(float x) const { return f2bf(x); } };
 template <> struct OpConvert<bf16_t, float> { using In = bf16_t; using Out = float; static constexpr int NIN = 1;
     __device__ float operator()(bf16_t x) const { return bf2f(x); } };
+template <> struct OpConvert<bool_t, f16_t> { using In = bool_t; using Out = f16_t; static constexpr int NIN = 1;
+    __device__ f16_t operator()(bool_t x) const { return f16_t{(uint16_t)(x ? 0x3C00 : 0)}; } };
+template <> struct OpConvert<float, f16_t> { using In = float; using Out = f16_t; static constexpr int NIN = 1;
+    __device__ f16_t operator()(float x) const { return f2h(x); } };
+template <> struct OpConvert<f16_t, float> { using In = f16_t; using Out = float; static constexpr int NIN = 1;
+    __device__ float operator()(f16_t x) const { return h2f(x); } };
+template <> struct OpConvert<f16_t, bool_t> { using In = f16_t; using Out = bool_t; static constexpr int NIN = 1;
+    __device__ bool_t operator()(f16_t x) const { return (bool_t)(h2f(x) != 0.0f); } };
 template <> struct OpConvert<float, bool_t> { using In = float; using Out = bool_t; static constexpr int NIN = 1;
     __device__ bool_t operator()(float x) const { return (bool_t)(x != 0.0f); } };
 template <> struct OpConvert<bf16_t, bool_t> { using In = bf16_t; using Out = bool_t; static constexpr int NIN = 1;
@@ -47,6 +55,7 @@ using namespace mxh;
     }
 MXH_UTIL_FOR(float, f32)
 MXH_UTIL_FOR(bf16_t, bf16)
+MXH_UTIL_FOR(f16_t, f16)
 extern "C" void hip_fill_bool(size_t n, bool_t* out, bool_t value) { ew_unary(n, 1, nullptr, nullptr, out, OpFill<bool_t>{value}); }
 
 #define MXH_CAST(TI, SI, TO, SO)                                                                           \
@@ -58,5 +67,9 @@ MXH_CAST(bool_t, bool, float, f32)
 MXH_CAST(bool_t, bool, bf16_t, bf16)
 MXH_CAST(float, f32, bf16_t, bf16)
 MXH_CAST(bf16_t, bf16, float, f32)
+MXH_CAST(bool_t, bool, f16_t, f16)
+MXH_CAST(float, f32, f16_t, f16)
+MXH_CAST(f16_t, f16, float, f32)
+MXH_CAST(f16_t, f16, bool_t, bool)
 MXH_CAST(float, f32, bool_t, bool)
 MXH_CAST(bf16_t, bf16, bool_t, bool)

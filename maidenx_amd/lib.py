@@ -76,7 +76,7 @@ def synchronize():
     check()
 
 
-NP_DTYPE = {"f32": np.float32, "bf16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64}
+NP_DTYPE = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64}
 
 
 class DeviceBuffer:

@@ -24,9 +24,9 @@ template <> struct F<double> {
     static double neg_inf() { return -std::numeric_limits<double>::infinity(); }
     static double exp(double x) { return std::exp(x); }
 };
-template <> struct F<bf16> {
-    static bf16 neg_inf() { return bf16::from_f32(-std::numeric_limits<float>::infinity()); }
-    static bf16 exp(bf16 x) { return bf16::from_f32(std::exp(x.to_f32())); }
+template <class C> struct F<half_t<C>> {
+    static half_t<C> neg_inf() { return half_t<C>::from_f32(-std::numeric_limits<float>::infinity()); }
+    static half_t<C> exp(half_t<C> x) { return half_t<C>::from_f32(std::exp(x.to_f32())); }
 };
 
 template <typename T>
@@ -84,3 +84,4 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
 ORC_SOFTMAX_FOR(float, f32)
 ORC_SOFTMAX_FOR(double, f64)
 ORC_SOFTMAX_FOR(bf16, bf16)
+ORC_SOFTMAX_FOR(f16, f16)

@@ -74,8 +74,10 @@ void binary_inplace(size_t num_els, size_t num_dims, const size_t* md, T* lhs, c
 // ---- element functions -----------------------------------------------------------------
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
+template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 template <typename T> inline T inf_of() { return std::numeric_limits<T>::infinity(); }
 template <> inline bf16 inf_of<bf16>() { return bf16::from_f32(std::numeric_limits<float>::infinity()); }
+template <> inline f16 inf_of<f16>() { return f16::from_f32(std::numeric_limits<float>::infinity()); }
 
 template <typename T> inline T op_add(T a, T b) { return a + b; }   // binary.rs:370-373
 template <typename T> inline T op_sub(T a, T b) { return a - b; }   // binary.rs:384-387
@@ -90,9 +92,11 @@ template <typename T> inline T op_div(T a, T b) {
 inline float op_maximum(float a, float b) { return std::fmax(a, b); }
 inline double op_maximum(double a, double b) { return std::fmax(a, b); }
 inline bf16 op_maximum(bf16 a, bf16 b) { return a > b ? a : b; }
+inline f16 op_maximum(f16 a, f16 b) { return a > b ? a : b; }
 inline float op_minimum(float a, float b) { return std::fmin(a, b); }   // binary.rs:594-597
 inline double op_minimum(double a, double b) { return std::fmin(a, b); }
 inline bf16 op_minimum(bf16 a, bf16 b) { return a < b ? a : b; }
+inline f16 op_minimum(f16 a, f16 b) { return a < b ? a : b; }
 
 }  // namespace
 
@@ -145,3 +149,4 @@ inline bf16 op_minimum(bf16 a, bf16 b) { return a < b ? a : b; }
 ORC_ALL_FOR(float, f32)
 ORC_ALL_FOR(double, f64)
 ORC_ALL_FOR(bf16, bf16)
+ORC_ALL_FOR(f16, f16)

@@ -21,34 +21,77 @@ namespace orc {
 // quiet bit.  Arithmetic is "convert both to f32, operate, convert back" per operation
 // (crates/maidenx_cpu/src/ops/binary.rs:372,400,416 use bf16 `+ - * /` directly).
 // ---------------------------------------------------------------------------------------
-struct bf16 {
+// One 16-bit storage float = a codec (f32 <-> 16 bits) plus "convert, operate in f32, convert back"
+// operators; bf16 and f16 differ only in the codec.
+template <class Codec> struct half_t {
     uint16_t bits;
-    bf16() = default;
-    static bf16 from_bits(uint16_t b) { bf16 r; r.bits = b; return r; }
-    static bf16 from_f32(float f) {
+    half_t() = default;
+    static half_t from_bits(uint16_t b) { half_t r; r.bits = b; return r; }
+    static half_t from_f32(float f) { return from_bits(Codec::encode(f)); }
+    float to_f32() const { return Codec::decode(bits); }
+};
+struct Bf16Codec {
+    static uint16_t encode(float f) {
         uint32_t x; std::memcpy(&x, &f, 4);
-        if ((x & 0x7FFFFFFFu) > 0x7F800000u) return from_bits((uint16_t)((x >> 16) | 0x0040u));
+        if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
         const uint32_t round_bit = 0x00008000u;
-        if ((x & round_bit) != 0 && (x & (3u * round_bit - 1u)) != 0)
-            return from_bits((uint16_t)((x >> 16) + 1u));
-        return from_bits((uint16_t)(x >> 16));
+        if ((x & round_bit) != 0 && (x & (3u * round_bit - 1u)) != 0) return (uint16_t)((x >> 16) + 1u);
+        return (uint16_t)(x >> 16);
     }
-    float to_f32() const {
-        uint32_t x = (uint32_t)bits << 16; float f; std::memcpy(&f, &x, 4); return f;
+    static float decode(uint16_t b) { uint32_t x = (uint32_t)b << 16; float f; std::memcpy(&f, &x, 4); return f; }
+};
+// IEEE binary16 (`half::f16`): 1 sign, 5 exponent (bias 15), 10 mantissa bits; round to nearest even,
+// overflow to infinity, gradual underflow, NaN kept NaN with the quiet bit forced.
+struct F16Codec {
+    static uint16_t encode(float f) {
+        uint32_t x; std::memcpy(&x, &f, 4);
+        const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+        const uint32_t e = (x >> 23) & 0xFFu, m = x & 0x007FFFFFu;
+        if (e == 0xFFu) return (uint16_t)(sign | 0x7C00u | (m ? 0x0200u : 0u) | (m >> 13));
+        const int he = (int)e - 127 + 15;                    // exponent field of the half
+        if (he >= 31) return (uint16_t)(sign | 0x7C00u);
+        if (he <= 0) {                                       // subnormal half (or zero): shift the 24-bit significand
+            if (he < -10) return sign;                       // below half of the smallest subnormal
+            const uint32_t sig = m | 0x00800000u;
+            const int shift = 14 - he;                       // 14 .. 24
+            uint32_t hm = sig >> shift;
+            const uint32_t rem = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
+            if (rem > half || (rem == half && (hm & 1u))) ++hm;
+            return (uint16_t)(sign | hm);                    // a carry into bit 10 is the smallest normal, as it should be
+        }
+        uint32_t h = ((uint32_t)he << 10) | (m >> 13);
+        const uint32_t rem = m & 0x1FFFu;
+        if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;      // a carry may reach the exponent: next binade or infinity
+        return (uint16_t)(sign | h);
+    }
+    static float decode(uint16_t b) {
+        const uint32_t sign = (uint32_t)(b & 0x8000u) << 16;
+        uint32_t e = (b >> 10) & 0x1Fu, m = b & 0x3FFu, x;
+        if (e == 0x1Fu) x = sign | 0x7F800000u | (m << 13);
+        else if (e != 0) x = sign | ((e + 112u) << 23) | (m << 13);
+        else if (m == 0) x = sign;
+        else {                                               // subnormal: normalise
+            int k = 0;
+            while (!(m & 0x400u)) { m <<= 1; ++k; }
+            x = sign | ((uint32_t)(113 - k) << 23) | ((m & 0x3FFu) << 13);
+        }
+        float f; std::memcpy(&f, &x, 4); return f;
     }
 };
-inline bf16 operator+(bf16 a, bf16 b) { return bf16::from_f32(a.to_f32() + b.to_f32()); }
-inline bf16 operator-(bf16 a, bf16 b) { return bf16::from_f32(a.to_f32() - b.to_f32()); }
-inline bf16 operator*(bf16 a, bf16 b) { return bf16::from_f32(a.to_f32() * b.to_f32()); }
-inline bf16 operator/(bf16 a, bf16 b) { return bf16::from_f32(a.to_f32() / b.to_f32()); }
-inline bf16 operator-(bf16 a) { return bf16::from_bits((uint16_t)(a.bits ^ 0x8000u)); }
-inline bf16& operator+=(bf16& a, bf16 b) { a = a + b; return a; }
-inline bool operator==(bf16 a, bf16 b) { return a.to_f32() == b.to_f32(); }
-inline bool operator!=(bf16 a, bf16 b) { return a.to_f32() != b.to_f32(); }
-inline bool operator<(bf16 a, bf16 b) { return a.to_f32() < b.to_f32(); }
-inline bool operator<=(bf16 a, bf16 b) { return a.to_f32() <= b.to_f32(); }
-inline bool operator>(bf16 a, bf16 b) { return a.to_f32() > b.to_f32(); }
-inline bool operator>=(bf16 a, bf16 b) { return a.to_f32() >= b.to_f32(); }
+using bf16 = half_t<Bf16Codec>;
+using f16 = half_t<F16Codec>;
+template <class C> inline half_t<C> operator+(half_t<C> a, half_t<C> b) { return half_t<C>::from_f32(a.to_f32() + b.to_f32()); }
+template <class C> inline half_t<C> operator-(half_t<C> a, half_t<C> b) { return half_t<C>::from_f32(a.to_f32() - b.to_f32()); }
+template <class C> inline half_t<C> operator*(half_t<C> a, half_t<C> b) { return half_t<C>::from_f32(a.to_f32() * b.to_f32()); }
+template <class C> inline half_t<C> operator/(half_t<C> a, half_t<C> b) { return half_t<C>::from_f32(a.to_f32() / b.to_f32()); }
+template <class C> inline half_t<C> operator-(half_t<C> a) { return half_t<C>::from_bits((uint16_t)(a.bits ^ 0x8000u)); }
+template <class C> inline half_t<C>& operator+=(half_t<C>& a, half_t<C> b) { a = a + b; return a; }
+template <class C> inline bool operator==(half_t<C> a, half_t<C> b) { return a.to_f32() == b.to_f32(); }
+template <class C> inline bool operator!=(half_t<C> a, half_t<C> b) { return a.to_f32() != b.to_f32(); }
+template <class C> inline bool operator<(half_t<C> a, half_t<C> b) { return a.to_f32() < b.to_f32(); }
+template <class C> inline bool operator<=(half_t<C> a, half_t<C> b) { return a.to_f32() <= b.to_f32(); }
+template <class C> inline bool operator>(half_t<C> a, half_t<C> b) { return a.to_f32() > b.to_f32(); }
+template <class C> inline bool operator>=(half_t<C> a, half_t<C> b) { return a.to_f32() >= b.to_f32(); }
 
 // ---------------------------------------------------------------------------------------
 // crates/maidenx_cpu/src/utils.rs:2-12  — contiguity test that ignores size-1 dims.

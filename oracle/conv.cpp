@@ -12,6 +12,7 @@ namespace {
 
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
+template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 
 struct CV { size_t B, C, H, W, kh, kw, oh, ow, ph, pw, sh, sw; };
 inline CV parse(const size_t* m) { return CV{m[0], m[1], m[2], m[3], m[4], m[5], m[6], m[7], m[8], m[9], m[10], m[11]}; }
@@ -91,3 +92,4 @@ void col2im(size_t num_els, const size_t* md, const T* col, T* output) {
 ORC_CONV_FOR(float, f32)
 ORC_CONV_FOR(double, f64)
 ORC_CONV_FOR(bf16, bf16)
+ORC_CONV_FOR(f16, f16)

@@ -15,6 +15,7 @@ int g_index_error = 0;
 
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
+template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 
 struct Layout {
     size_t nd;
@@ -177,7 +178,9 @@ ORC_INDEX_FOR(float, f32, int64_t, i64)
 ORC_INDEX_FOR(double, f64, int32_t, i32)
 ORC_INDEX_FOR(double, f64, int64_t, i64)
 ORC_INDEX_FOR(bf16, bf16, int32_t, i32)
+ORC_INDEX_FOR(f16, f16, int32_t, i32)
 ORC_INDEX_FOR(bf16, bf16, int64_t, i64)
+ORC_INDEX_FOR(f16, f16, int64_t, i64)
 
 extern "C" void oracle_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output) {
     bincount<int32_t>(n, stride, offset, input, out_size, output);

@@ -14,6 +14,7 @@ namespace {
 
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
+template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 
 struct MM {
     size_t out_ndim, a_ndim, b_ndim;
@@ -156,3 +157,4 @@ void matmul_backward(size_t num_els_a, size_t num_els_b, const size_t* md, const
 ORC_MATMUL_FOR(float, f32)
 ORC_MATMUL_FOR(double, f64)
 ORC_MATMUL_FOR(bf16, bf16)
+ORC_MATMUL_FOR(f16, f16)

@@ -10,6 +10,7 @@ namespace {
 
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
+template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 
 struct PadMeta {
     const size_t *in_dims, *in_strides, *out_dims, *pads;
@@ -157,3 +158,4 @@ void pad_edge_backward(Edge mode, size_t n_in, size_t n_out, size_t nd, const si
 ORC_PAD_FOR(float, f32)
 ORC_PAD_FOR(double, f64)
 ORC_PAD_FOR(bf16, bf16)
+ORC_PAD_FOR(f16, f16)

@@ -18,12 +18,16 @@ namespace {
 
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
+template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 template <typename T> inline T lowest_of() { return std::numeric_limits<T>::lowest(); }   // f32::MIN
 template <> inline bf16 lowest_of<bf16>() { return bf16::from_f32(std::numeric_limits<float>::lowest()); }
+template <> inline f16 lowest_of<f16>() { return f16::from_f32(std::numeric_limits<float>::lowest()); }
 template <typename T> inline T highest_of() { return std::numeric_limits<T>::max(); }     // f32::MAX
 template <> inline bf16 highest_of<bf16>() { return bf16::from_f32(std::numeric_limits<float>::max()); }
+template <> inline f16 highest_of<f16>() { return f16::from_f32(std::numeric_limits<float>::max()); }
 template <typename T> inline T from_count(size_t n) { return (T)n; }                      // `x as f32`
 template <> inline bf16 from_count<bf16>(size_t n) { return bf16::from_f32((float)n); }
+template <> inline f16 from_count<f16>(size_t n) { return f16::from_f32((float)n); }
 
 // One lock word + value per output element, like the reference's Vec<Mutex<T>>.
 template <typename T> struct Cell {
@@ -187,3 +191,4 @@ void fold(size_t num_els, size_t nd, const size_t* md, const T* inp, T* out) {
 ORC_REDUCE_FOR(float, f32)
 ORC_REDUCE_FOR(double, f64)
 ORC_REDUCE_FOR(bf16, bf16)
+ORC_REDUCE_FOR(f16, f16)

@@ -79,11 +79,11 @@ template <> struct Fx<double> : FloatFx<double> {};
 
 // bf16: "upcast, compute in f32, round once" for the transcendental forms, bf16 operators
 // (round per op) for the arithmetic forms — each as written in unary.rs.
-template <> struct Fx<bf16> {
-    using T = bf16;
+template <class C> struct Fx<half_t<C>> {
+    using T = half_t<C>;
     using F = FloatFx<float>;
-    static T r(float v) { return bf16::from_f32(v); }
-    static T z() { return bf16::from_f32(0.0f); }
+    static T r(float v) { return T::from_f32(v); }
+    static T z() { return T::from_f32(0.0f); }
     static T neg(T x) { return -x; }                                        // :132 sign-bit flip
     static T abs(T x) { return r(std::fabs(x.to_f32())); }                  // :142
     static T sign(T x) { return x > z() ? r(1.0f) : (x < z() ? r(-1.0f) : z()); }
@@ -158,3 +158,4 @@ template <> struct Fx<bf16> {
 ORC_ALL_FOR(float, f32)
 ORC_ALL_FOR(double, f64)
 ORC_ALL_FOR(bf16, bf16)
+ORC_ALL_FOR(f16, f16)

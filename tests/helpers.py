@@ -14,7 +14,7 @@ ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
 
 import maidenx_amd._signatures as S  # noqa: E402
 
-NP = {"f32": np.float32, "bf16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64}
+NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64}
 
 
 # ---- bf16 <-> f32 on the host (round to nearest even, NaN quieted), as the `half` crate does ----
@@ -36,12 +36,17 @@ def to_storage(a, dt):
     """float values -> storage array of dtype tag dt."""
     if dt == "bf16":
         return f32_to_bf16(np.asarray(a, dtype=np.float32))
+    if dt == "f16":      # numpy's float16 is IEEE binary16 with round-to-nearest-even conversions
+        with np.errstate(over="ignore"):
+            return np.ascontiguousarray(np.asarray(a, dtype=np.float32).astype(np.float16)).view(np.uint16)
     return np.ascontiguousarray(a, dtype=NP[dt])
 
 
 def to_float(a, dt):
     if dt == "bf16":
         return bf16_to_f32(a)
+    if dt == "f16":
+        return np.ascontiguousarray(a, dtype=np.uint16).view(np.float16).astype(np.float32)
     return np.asarray(a)
 
 
@@ -159,7 +164,7 @@ class Runner:
         if kind == "oracle":
             self.lib = C.CDLL(ensure_oracle_built())
             self.prefix = "oracle_"
-            for name, args in {**S.signatures(("f32", "bf16", "f64")), **S.index_signatures(("f32", "bf16", "f64"))}.items():
+            for name, args in {**S.signatures(("f32", "bf16", "f16", "f64")), **S.index_signatures(("f32", "bf16", "f16", "f64"))}.items():
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None
@@ -207,8 +212,8 @@ class Runner:
 
 def const_arg(v, dt):
     """A by-value constant of the input dtype."""
-    if dt == "bf16":
-        return int(f32_to_bf16(np.array([v], dtype=np.float32))[0])
+    if dt in ("bf16", "f16"):
+        return int(to_storage(np.array([v], dtype=np.float32), dt)[0])
     return float(v)
 
 

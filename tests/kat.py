@@ -21,13 +21,13 @@ def padded(values, dt):
 def tol_for(dt, tol):
     # the reference asserts |Δ| < 0.1 for bf16/f16 (e.g. ops_binary.rs:28); these cases are exact
     # or nearly so in bf16 as well, so a bf16 rounding step of the expected value is allowed.
-    return tol if dt != "bf16" else None
+    return tol if dt not in ("bf16", "f16") else None
 
 
 def check(actual_storage, expect, dt, tol):
     got = to_float(actual_storage, dt).astype(np.float64)
     exp = np.asarray(expect, dtype=np.float64)
-    if dt == "bf16":
+    if dt in ("bf16", "f16"):
         # value must be the bf16 rounding of something within 1 bf16 ulp of the expectation
         # (the reference itself only asserts |Δ| < 0.1 for bf16, e.g. ops_binary.rs:28)
         lim = np.abs(exp) * 2.0 ** -7 + tol
@@ -200,7 +200,7 @@ def run_softmax(be, dt):
         md = meta_unary(shape, contiguous_strides(shape), 1)
         (out,) = be.call(f"softmax_{dt}", n, len(shape), c["dim"], md, In(padded(c["data"], dt)), Out(n, dt))
         y = to_float(out, dt).astype(np.float64).reshape(shape)
-        tol = 1e-5 if dt != "bf16" else 2e-2
+        tol = 1e-5 if dt not in ("bf16", "f16") else 2e-2
         assert np.all(np.abs(y.sum(axis=c["dim"]) - 1.0) < tol), y
         assert np.all(np.diff(y, axis=c["dim"]) > 0), y
 

@@ -6,7 +6,7 @@ import kat
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("case", kat.ALL, ids=lambda f: f.__name__)
 def test_hip_matches_reference_vectors(hip, case, dt):
     case(hip, dt)

@@ -12,7 +12,7 @@ from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides,
 
 pytestmark = pytest.mark.gpu
 
-DTS = ["f32", "bf16"]
+DTS = ["f32", "bf16", "f16"]
 
 
 def both(oracle, hip, name, *args_builder):
@@ -202,13 +202,14 @@ def test_pow_f32_ulp(oracle, hip):
         assert np.max(ulp_diff_f32(o, h)) <= 1, c
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
 @pytest.mark.parametrize("op", ["exp", "tanh", "gelu", "sigmoid"])
-def test_unary_transcendental_bf16(oracle, hip, op):
-    # all 2^16 bf16 inputs: f32 evaluation (bit-identical) then the same single rounding
+def test_unary_transcendental_16bit(oracle, hip, op, dt):
+    # all 2^16 inputs: f32 evaluation (bit-identical) then the same single rounding
     bits = np.arange(1 << 16, dtype=np.uint16)
     md = meta_unary([bits.size], [1])
-    (o,), (h,) = both(oracle, hip, f"{op}_bf16", lambda: (bits.size, 1, md, In(bits), Out(bits.size, "bf16")))
-    fo, fh = bf16_to_f32(o), bf16_to_f32(h)
+    (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (bits.size, 1, md, In(bits), Out(bits.size, dt)))
+    fo, fh = to_float(o, dt), to_float(h, dt)
     assert np.array_equal(np.isnan(fo), np.isnan(fh))
     ok = ~np.isnan(fo)
     assert np.array_equal(o[ok], h[ok])
@@ -236,6 +237,10 @@ def test_reductions(oracle, hip, shape, dim, dt):
     for op in ["sum", "mean", "max", "min"]:
         (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(shape), 1, md, In(st), Out(n // shape[dim], dt)))
         fh = to_float(h, dt).astype(np.float64)
+        if op == "mean" and dt == "f16" and shape[dim] > 65504:
+            # the count itself overflows f16 (reduction.rs:584: f16::from_f32(x as f32) = inf), so the reference's mean is sum / inf = 0
+            assert np.array_equal(to_float(o, dt), to_float(h, dt)) and np.all(fh == 0), op
+            continue
         if op in ("max", "min"):
             assert np.array_equal(to_float(o, dt), to_float(h, dt)), op
             continue
@@ -414,7 +419,8 @@ def test_matmul_backward(oracle, hip, shape, dt):
     tb = np.einsum("bmk,bmn->bkn", av, gv)
     sa_ = np.einsum("bmn,bkn->bmk", np.abs(gv), np.abs(bv))
     sb_ = np.einsum("bmk,bmn->bkn", np.abs(av), np.abs(gv))
-    assert np.max(np.abs(to_float(ga, dt).reshape(ta.shape) - ta) / np.maximum(sa_, 1e-30)) <= tol
+    floor = 2.0 ** -24 if dt == "f16" else 0.0       # f16 results below 6.1e-5 are subnormal: absolute spacing 2^-24
+    assert np.max((np.abs(to_float(ga, dt).reshape(ta.shape) - ta) - floor) / np.maximum(sa_, 1e-30)) <= tol
     assert np.max(np.abs(to_float(gb, dt).reshape(tb.shape) - tb) / np.maximum(sb_, 1e-30)) <= tol
     # either gradient may be absent
     (ga2,) = hip.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), Out(batch * m * k, dt), None)
@@ -599,10 +605,11 @@ def test_softmax(oracle, hip, shape, dim, dt):
         # bf16 rounds x - max and exp like the reference; only the sum differs: the reference's bf16 running sum
         # stalls on long slices, the kernel sums in f32.  Compare with the exact sum of the same rounded terms.
         xf = to_float(x, dt).reshape(shape)
-        t = bf16_to_f32(f32_to_bf16(xf - xf.max(axis=axis, keepdims=True)))
-        e = bf16_to_f32(f32_to_bf16(np.exp(t))).astype(np.float64)
+        rnd = lambda v: to_float(to_storage(v, dt), dt)
+        t = rnd(xf - xf.max(axis=axis, keepdims=True))
+        e = rnd(np.exp(t)).astype(np.float64)
         truth = (e / e.sum(axis=axis, keepdims=True)).ravel()
-        assert np.all(np.abs(got - truth) <= 1e-2 * truth + 1e-30)
+        assert np.all(np.abs(got - truth) <= 1e-2 * truth + (2.0 ** -24 if dt == "f16" else 1e-30))      # f16 subnormal spacing
         if shape[axis] <= 8:
             assert np.max(np.abs(got - to_float(o, dt))) <= 2.0 ** -7
 
@@ -777,7 +784,22 @@ def test_fill_cast_copy(hip):
     assert np.array_equal(b, f32_to_bf16(x))
     (back,) = hip.call("cast_bf16_f32", 5000, In(b), Out(5000, "f32"))
     assert np.array_equal(back, bf16_to_f32(b))
+    # f16: every bit pattern to f32 and back, and f32 values across the f16 range (subnormals, overflow, ties) against numpy
+    hb = np.arange(1 << 16, dtype=np.uint16)
+    (hf,) = hip.call("cast_f16_f32", hb.size, In(hb), Out(hb.size, "f32"))
+    want = hb.view(np.float16).astype(np.float32)
+    assert np.array_equal(np.isnan(hf), np.isnan(want)) and np.array_equal(hf[~np.isnan(want)], want[~np.isnan(want)])
+    wide = (r.standard_normal(200000) * np.exp(r.uniform(-20, 12, 200000))).astype(np.float32)
+    (hh,) = hip.call("cast_f32_f16", wide.size, In(wide), Out(wide.size, "f16"))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(hh, wide.astype(np.float16).view(np.uint16))
+    (f,) = hip.call("fill_f16", 77, Out(77, "f16"), const_arg(1.0, "f16"))
+    assert np.all(f == 0x3C00)
     m = (x > 0).astype(np.uint8)
+    (mh,) = hip.call("cast_bool_f16", 5000, In(m), Out(5000, "f16"))
+    assert np.array_equal(mh, np.where(m, 0x3C00, 0).astype(np.uint16))
+    (mb,) = hip.call("cast_f16_bool", hb.size, In(hb), Out(hb.size, "bool"))
+    assert np.array_equal(mb, (np.nan_to_num(want, nan=1.0) != 0).astype(np.uint8))
     (mf,) = hip.call("cast_bool_f32", 5000, In(m), Out(5000, "f32"))
     assert np.array_equal(mf, m.astype(np.float32))
     lay = LY.permuted([70, 90], [1, 0], off=1)

@@ -4,7 +4,7 @@ import pytest
 import kat
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16", "f64"])
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16", "f64"])
 @pytest.mark.parametrize("case", kat.ALL, ids=lambda f: f.__name__)
 def test_oracle_matches_reference_vectors(oracle, case, dt):
     case(oracle, dt)

@@ -455,3 +455,28 @@ def test_oracle_bincount_vs_numpy_and_errors(oracle):
     assert oracle.lib.oracle_index_error() == 1          # IndexOutOfBounds in the reference
     oracle.call("gather_f64_i32", 1, 0, layout([3]), layout([2]), In(np.array([-4, 0], dtype=np.int32)), In(np.arange(3.0)), Out(2, "f64"))
     assert oracle.lib.oracle_index_error() == 1
+
+
+# ---- f16: the oracle's software codec against numpy's IEEE binary16 ---------------------------------------
+def test_oracle_f16_codec_matches_numpy_float16(oracle):
+    # decode: every bit pattern through a cast to f32 (cast_f16... is a HIP-only helper, so use neg twice + add 0 paths):
+    # add_f16(x, +0) returns encode(decode(x) + 0) — exact for every finite pattern and a NaN for NaNs
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    zero = np.zeros(1 << 16, dtype=np.uint16)
+    (out,) = oracle.call("add_f16", 1 << 16, 1, meta_binary([1 << 16], [1], [1]), In(bits), In(zero), Out(1 << 16, "f16"))
+    f = bits.view(np.float16)
+    nan = np.isnan(f)
+    keep = ~nan & (bits != 0x8000)                       # -0 + +0 = +0
+    assert np.array_equal(out[keep], bits[keep])
+    assert np.all(np.isnan(out[nan].view(np.float16)))
+    assert out[0x8000] == 0
+    # encode: products of random f16 pairs are exact in f32, so mul_f16 = encode(exact product); numpy rounds the same product
+    r = rng(171)
+    a = r.integers(0, 1 << 16, 1 << 20).astype(np.uint16)
+    b = r.integers(0, 1 << 16, 1 << 20).astype(np.uint16)
+    (m,) = oracle.call("mul_f16", a.size, 1, meta_binary([a.size], [1], [1]), In(a), In(b), Out(a.size, "f16"))
+    with np.errstate(all="ignore"):
+        want = (a.view(np.float16).astype(np.float32) * b.view(np.float16).astype(np.float32)).astype(np.float16)
+    ok = ~np.isnan(want)
+    assert np.array_equal(m[ok], want.view(np.uint16)[ok])           # overflow to inf, subnormals, ties to even
+    assert np.all(np.isnan(m[~ok].view(np.float16)))
