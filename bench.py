@@ -1,6 +1,6 @@
 """Benchmark of the maidenx_hip backend on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul|mlp|conv|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload elementwise|reduce|matmul|mlp|conv|copy|kernels]
 
 The default workload is the elementwise configuration (configs[1]): forward + backward of add, mul, div,
 exp, relu, gelu on [8192,8192] tensors, f32 and bf16, for contiguous operands, a [1,8192] broadcast
@@ -759,6 +759,24 @@ def cpu_baseline_conv(args):
             "sample": f"{n} steps at batch 2 in {el:.1f} s, divided by 16 for batch 32"}
 
 
+def run_kernels(args):
+    """Every kernel of the backend on its own, buffers rotated so that HBM serves them (maidenx_amd/kernel_bench.py).
+    The table goes to stderr as it is measured and into config.kernels; value = the contiguous f32 multiply."""
+    from maidenx_amd import kernel_bench
+    t0 = time.perf_counter()
+    rows = kernel_bench.run("", out=sys.stderr)
+    dt_s = time.perf_counter() - t0
+    mul = next(r for r in rows if r["kernel"] == "mul_f32/contig")
+    res = base_result(args, mul["GB/s"], "GB/s", dt_s, "f32", "every backend kernel alone on the configs' shapes, operands rotated among 4 allocations (not cache-warm)",
+                      {"kernels": rows})
+    res["steps"], res["warmup"], res["ms_per_step"] = 1, 0, round(dt_s * 1e3, 1)
+    res["roofline"] = {"bound": "hbm", "kernel": "ew_nd_kernel<OpMul<float>,4> (hip_mul_f32, contiguous [8192,8192])", "achieved": mul["GB/s"],
+                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(mul["GB/s"] / HBM_PEAK_GBS, 4), "avg_launch_us": mul["us"],
+                       "launches_timed": 20, "traffic": None}
+    res["cpu_baseline"] = None
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -769,7 +787,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X; nothing in this backend uses a second GPU (--gpus must be 1)")
-    runners = {"elementwise": run_elementwise, "reduce": run_reduce, "matmul": run_matmul, "copy": run_copy, "mlp": run_mlp, "conv": run_conv}
+    runners = {"elementwise": run_elementwise, "reduce": run_reduce, "matmul": run_matmul, "copy": run_copy, "mlp": run_mlp, "conv": run_conv, "kernels": run_kernels}
     if args.workload not in runners:
         sys.exit(f"unknown workload {args.workload}: choose from {sorted(runners)}")
     res = runners[args.workload](args)

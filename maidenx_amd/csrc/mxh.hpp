@@ -48,6 +48,12 @@ __host__ __device__ inline float bf2f(bf16_t h) {
     return c.f;
 }
 __host__ __device__ inline bf16_t f2bf(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // gfx950 converts in hardware (v_cvt_pk_bf16_f32): round to nearest even, NaN stays a quiet NaN
+    bf16_t h;
+    h.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
+    return h;
+#endif
     union { uint32_t u; float f; } c;
     c.f = f;
     uint32_t x = c.u;

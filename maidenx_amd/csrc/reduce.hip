@@ -373,6 +373,17 @@ void col_stage(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, unsig
     if (total >= (1ull << 32)) { set_status(ERR_TOO_LARGE, "column reduce: more than 2^32 work items"); return; }
     unsigned blocks = cdiv(total, RB);
     FastDiv dsv = make_fastdiv((uint32_t)sv), dch = make_fastdiv(chunks);
+    if constexpr (VEC == 8) {
+        // 16-bit elements and few threads (one wave per SIMD or less): 8-byte vectors double the waves, which
+        // hides the unpacking arithmetic behind the loads
+        if (vec && blocks <= 256) {
+            size_t sv4 = S / 4, total4 = outer * chunks * sv4;
+            hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, R, 4>), dim3(cdiv(total4, RB)), dim3(RB), 0, stream(), in, out, outer, L, S,
+                               chunks, chunk_len, make_fastdiv((uint32_t)sv4), dch, total4, div, src_bf16);
+            MXH_LAUNCH_CHECK("col_reduce");
+            return;
+        }
+    }
     if (vec)
         hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, R, VEC>), dim3(blocks), dim3(RB), 0, stream(), in, out, outer, L, S,
                            chunks, chunk_len, dsv, dch, total, div, src_bf16);

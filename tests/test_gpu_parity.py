@@ -784,6 +784,13 @@ def test_fill_cast_copy(hip):
     assert np.array_equal(b, f32_to_bf16(x))
     (back,) = hip.call("cast_bf16_f32", 5000, In(b), Out(5000, "f32"))
     assert np.array_equal(back, bf16_to_f32(b))
+    # bf16 from every kind of f32 (random bit patterns: all exponents, subnormals, infinities, NaNs) against the closed form
+    pat = r.integers(0, 1 << 32, 1 << 22, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    (pb,) = hip.call("cast_f32_bf16", pat.size, In(pat), Out(pat.size, "bf16"))
+    want_b = f32_to_bf16(pat)
+    isn = np.isnan(pat)
+    assert np.array_equal(pb[~isn], want_b[~isn])
+    assert np.all(np.isnan(bf16_to_f32(pb[isn])))
     # f16: every bit pattern to f32 and back, and f32 values across the f16 range (subnormals, overflow, ties) against numpy
     hb = np.arange(1 << 16, dtype=np.uint16)
     (hf,) = hip.call("cast_f16_f32", hb.size, In(hb), Out(hb.size, "f32"))
