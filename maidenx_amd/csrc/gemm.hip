@@ -26,6 +26,9 @@
 
 #include "mxh.hpp"
 
+#ifndef MXH_GEMM_INTERLEAVE
+#define MXH_GEMM_INTERLEAVE 1
+#endif
 #ifndef MXH_GEMM_TS16
 #define MXH_GEMM_TS16 1
 #endif
@@ -101,11 +104,26 @@ template <> struct Pack16<f16_t> {
 // in memory (natural); otherwise the row index has stride 1 and the tile is turned on the way in.
 // load() only issues global loads into registers; store() does any re-packing and writes LDS, so the
 // loads stay in flight across a whole k-tile of MFMAs.  NT = threads per block.
-template <class T, bool RCONT, int ROWS, int NT>
+// Bank conflicts of the fragment reads (ds_read_b128; LDS serves such a read in four passes, and timing
+// of access patterns says a pass takes lanes 0-7 with 24-31, 8-15 with 16-23, and the same in the upper
+// half):
+//   * 32x32 fragments (lane = row % 32, 16-byte chunk lane / 32): rows 16 bytes longer than the tile
+//     (PITCH = TK + VEC) are conflict free;
+//   * 16x16 fragments (lane = row % 16, chunk lane / 16): that padding leaves every read two-way
+//     conflicted (9 instead of 4.5 cycles).  SWZ stores unpadded rows of 8 chunks with the chunk index
+//     xor-ed by bits 1..3 of the row: both row sets of a pass then cover all 64 banks exactly once, and a
+//     pair of rows (2q, 2q+1) shares its key, which is what the turned 16-bit staging writes together.
+template <class T, bool RCONT, int ROWS, int NT, bool SWZ = false>
 struct Stager {
     static constexpr int VEC = Elem<T>::VEC;
     static constexpr int TK = TK_BYTES / sizeof(T);
-    static constexpr int PITCH = TK + VEC;                 // +16 bytes: keeps alignment, spreads banks
+    static constexpr int PITCH = SWZ ? TK : TK + VEC;      // +16 bytes: keeps alignment, spreads banks
+    static_assert(!SWZ || TK / VEC == 8, "the swizzle permutes 8 chunks per row");
+    // element offset of 16-byte chunk `chunk` of row `row` inside a staged tile
+    static __device__ __forceinline__ int at(int row, int chunk) {
+        if constexpr (SWZ) chunk ^= (row >> 1) & 7;
+        return row * PITCH + chunk * VEC;
+    }
     static constexpr int NV = ROWS * TK / VEC / NT;        // 16-byte units per thread
     static constexpr bool PAIRS = !RCONT && sizeof(T) == 2;
     static_assert(NV >= 1 && (!PAIRS || NV % 2 == 0), "tile too small for this block size");
@@ -203,7 +221,7 @@ struct Stager {
             for (int u = 0; u < NV / 2; ++u) {
                 if (u < u0 || u >= u1) continue;
                 int id = t + u * NT;
-                int row = (id % NP) * 2, kk = (id / NP) * VEC;
+                int row = (id % NP) * 2, ck = id / NP;
                 // d[e] = (row, k+e) | (row+1, k+e) << 16  →  [row][k..k+8) and [row+1][k..k+8)
                 u32x4 lo, hi;
 #pragma unroll
@@ -212,17 +230,17 @@ struct Stager {
                     lo[e] = (d0 & 0xffffu) | (d1 << 16);
                     hi[e] = (d0 >> 16) | (d1 & 0xffff0000u);
                 }
-                *(u32x4*)(lds + row * PITCH + kk) = lo;
-                *(u32x4*)(lds + (row + 1) * PITCH + kk) = hi;
+                *(u32x4*)(lds + at(row, ck)) = lo;
+                *(u32x4*)(lds + at(row + 1, ck)) = hi;
             }
         } else {
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
                 if (u < u0 || u >= u1) continue;
-                int id = t + u * NT, row, kk;
-                if constexpr (RCONT) { constexpr int KV = TK / VEC; row = id / KV; kk = (id % KV) * VEC; }
-                else { row = id % ROWS; kk = (id / ROWS) * VEC; }
-                *(u32x4*)(lds + row * PITCH + kk) = reg[u];
+                int id = t + u * NT, row, ck;
+                if constexpr (RCONT) { constexpr int KV = TK / VEC; row = id / KV; ck = id % KV; }
+                else { row = id % ROWS; ck = id / ROWS; }
+                *(u32x4*)(lds + at(row, ck)) = reg[u];
             }
         }
     }
@@ -334,8 +352,9 @@ __global__ __launch_bounds__(256) void gemm_fold_kernel(const float* __restrict_
 template <class T, bool XR, bool YR, class Cfg, bool FAST>
 __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
-    using SX = Stager<T, XR, TM, NT>;
-    using SY = Stager<T, YR, TN, NT>;
+    constexpr bool SWZ = Cfg::TS == 16;
+    using SX = Stager<T, XR, TM, NT, SWZ>;
+    using SY = Stager<T, YR, TN, NT, SWZ>;
     constexpr int VEC = Elem<T>::VEC;
     constexpr int TK = SX::TK;
     constexpr int PITCH = SX::PITCH;
@@ -408,6 +427,17 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
 
     const int frag_x = (wm * TS * MI + lrow) * PITCH + lk;   // + a*TS*PITCH + k-step*KS
     const int frag_y = (wn * TS * MJ + lrow) * PITCH + lk;
+    // 16x16 tiles: the swizzled chunk of a lane differs per k-step, so one offset per step (the tile
+    // offsets a * TS * PITCH keep bits 1..3 of the row and stay immediates)
+    int frag_xk[2] = {0, 0}, frag_yk[2] = {0, 0};
+    if constexpr (TS == 16) {
+        static_assert(TS != 16 || TK / KS == 2, "two k-steps per staged tile");
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            frag_xk[ks] = SX::at(wm * TS * MI + lrow, lane / TS + ks * (KS / VEC));
+            frag_yk[ks] = SY::at(wn * TS * MJ + lrow, lane / TS + ks * (KS / VEC));
+        }
+    }
     u32x4 fa[2][MI], fb[2][MJH];
     // fragments of step s from the tile at (bx, by)
     auto read_frags = [&](int s, const T* bx, const T* by) {
@@ -420,10 +450,10 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             const int ks = s >> 1, h = s & 1;
             if (h == 0) {
 #pragma unroll
-                for (int a = 0; a < MI; ++a) fa[ks & 1][a] = *(const u32x4*)(bx + frag_x + a * TS * PITCH + ks * KS);
+                for (int a = 0; a < MI; ++a) fa[ks & 1][a] = *(const u32x4*)(bx + frag_xk[ks] + a * TS * PITCH);
             }
 #pragma unroll
-            for (int c = 0; c < MJH; ++c) fb[s & 1][c] = *(const u32x4*)(by + frag_y + (h * MJH + c) * TS * PITCH + ks * KS);
+            for (int c = 0; c < MJH; ++c) fb[s & 1][c] = *(const u32x4*)(by + frag_yk[ks] + (h * MJH + c) * TS * PITCH);
         }
     };
     auto mfmas = [&](int s) {
@@ -465,9 +495,21 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             }
             // keep the memory operations of the next stage ahead of this step's MFMAs: the matrix
             // pipe then works through them while LDS and the vector memory unit serve the next step
+#if MXH_GEMM_INTERLEAVE
+            mfmas(s);
+#pragma unroll
+            for (int i = 0; i < MI * MJH; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global load
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#else
             __builtin_amdgcn_sched_barrier(0);
             mfmas(s);
             __builtin_amdgcn_sched_barrier(0);
+#endif
         }
     }
 
@@ -481,7 +523,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
 
 template <class T, bool XR, bool YR, class Cfg, bool FAST>
 void launch_mfma_impl(GemmArgs g) {
-    using SX = Stager<T, XR, Cfg::TM, Cfg::NT>;
+    using SX = Stager<T, XR, Cfg::TM, Cfg::NT, Cfg::TS == 16>;
     constexpr size_t lds_bytes = (size_t)2 * (Cfg::TM + Cfg::TN) * SX::PITCH * sizeof(T);
     constexpr uint32_t TK = TK_BYTES / sizeof(T);
     g.tiles_i = cdiv(g.I, Cfg::TM);
