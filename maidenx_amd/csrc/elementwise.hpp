@@ -11,7 +11,11 @@
 //           read along that dim in 64x64 tiles, turned through LDS, and consumed along the
 //           output's innermost dim, so both the read and the write stay coalesced.
 #pragma once
+#include <cstring>
+#include <type_traits>
+
 #include "mxh.hpp"
+#include "ew_registry.hpp"
 
 namespace mxh {
 
@@ -31,21 +35,24 @@ constexpr int EW_BLOCK = 256;
 #define MXH_EW_UNR 4
 #endif
 constexpr int EW_UNR = MXH_EW_UNR;
+constexpr unsigned EW_SMALL_BLOCKS = 256;      // fewer blocks than CUs: see ew_launch
 
 // ---- ew_nd -------------------------------------------------------------------------------
-template <class Op, int VEC>
-__global__ __launch_bounds__(EW_BLOCK) void ew_nd_kernel(NdSpace<Op::NIN + 1> sp, EwPtrs<Op::NIN> p, size_t nvec,
-                                                         Op op) {
+// The body takes its block and thread index as arguments: the kernel passes its own, the interpreter of
+// recorded programs virtual ones.
+template <class Op, int VEC, int UNR = EW_UNR, class Space>
+__device__ __forceinline__ void ew_nd_body(const Space& sp, const EwPtrs<Op::NIN>& p, size_t nvec, const Op& op,
+                                           unsigned bid, unsigned tid) {
     using In = typename Op::In;
     using Out = typename Op::Out;
     constexpr int NIN = Op::NIN;
     const int last = sp.ndims - 1;
-    size_t v0 = (size_t)blockIdx.x * (EW_BLOCK * EW_UNR) + threadIdx.x;
+    size_t v0 = (size_t)bid * (EW_BLOCK * UNR) + tid;
 
-    In vals[EW_UNR][NIN][VEC];
-    int64_t ooff[EW_UNR];
+    In vals[UNR][NIN][VEC];
+    int64_t ooff[UNR];
 #pragma unroll
-    for (int u = 0; u < EW_UNR; ++u) {
+    for (int u = 0; u < UNR; ++u) {
         size_t v = v0 + (size_t)u * EW_BLOCK;
         if (v >= nvec) break;
         int64_t off[NIN + 1];
@@ -59,7 +66,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_nd_kernel(NdSpace<Op::NIN + 1> sp
             for (int k = 0; k <= NIN; ++k) off[k] = 0;
             for (int d = last; d > 0; --d) {
                 uint32_t q, c;
-                fd_divmod(r, sp.div[d], q, c);
+                fd_divmod(r, FastDiv{sp.div[d].d, sp.div[d].mul, sp.div[d].shift}, q, c);   // member by member: `sp` may live in the constant address space
 #pragma unroll
                 for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)c * sp.strides[k][d];
                 r = q;
@@ -91,7 +98,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_nd_kernel(NdSpace<Op::NIN + 1> sp
         }
     }
 #pragma unroll
-    for (int u = 0; u < EW_UNR; ++u) {
+    for (int u = 0; u < UNR; ++u) {
         size_t v = v0 + (size_t)u * EW_BLOCK;
         if (v >= nvec) break;
         AVec<Out, VEC> r;
@@ -108,6 +115,19 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_nd_kernel(NdSpace<Op::NIN + 1> sp
         }
     }
 }
+template <class Op, int VEC, int UNR = EW_UNR>
+__global__ __launch_bounds__(EW_BLOCK) void ew_nd_kernel(NdSpace<Op::NIN + 1> sp, EwPtrs<Op::NIN> p, size_t nvec,
+                                                         Op op) {
+    ew_nd_body<Op, VEC, UNR>(sp, p, nvec, op, blockIdx.x, threadIdx.x);
+}
+// Argument block of one recorded ew_nd launch.
+template <class Op>
+struct EwProgArgs {
+    NdSpace<Op::NIN + 1> sp;
+    EwPtrs<Op::NIN> p;
+    size_t nvec;
+    Op op;
+};
 
 // ---- ew_tr -------------------------------------------------------------------------------
 constexpr int TR_TILE = 64;
@@ -310,6 +330,25 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_trv_kernel(NdSpace<Op::NIN + 1> s
     }
 }
 
+// While a capture is being recorded: the same launch as a command of a program (functors outside the list
+// and large grids are not recorded, which leaves the capture to the HIP graph).
+template <class Op>
+inline void ew_record(int vec, unsigned blocks, const NdSpace<Op::NIN + 1>& sp, const EwPtrs<Op::NIN>& p, size_t n,
+                      const Op& op) {
+    constexpr int idx = IndexOf<Op, EwProgOps>::value;
+    if constexpr (idx >= 0) {
+        static_assert(sizeof(EwProgArgs<Op>) <= PROG_ARG_BYTES, "argument block too large for a command");
+        if (!prog_recording() || blocks > PROG_MAX_GRID) return;
+        EwProgArgs<Op> a;
+        std::memset((void*)&a, 0, sizeof(a));
+        a.sp = sp;
+        a.p = p;
+        a.nvec = n;
+        a.op = op;
+        prog_record(prog_kid(PF_EW, (uint32_t)(idx * 2 + vec)), blocks, &a, sizeof(a));
+    }
+}
+
 // ---- host-side selection -------------------------------------------------------------------
 // in_strides[k] / out_strides are in elements, pointers already include the operand offsets.
 template <class Op>
@@ -411,13 +450,23 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
     if (vec_ok) vec_ok = aligned(out, sizeof(Out), 0);
     for (int k = 0; k < NIN && vec_ok; ++k)
         if (sp.strides[k + 1][last] == 1) vec_ok = aligned(in[k], sizeof(In), k + 1);
+    // A launch that cannot give every CU a block is latency bound: one vector per thread then spreads it over
+    // four times as many blocks (a 10000-element powf: 3 blocks of 16 elements per thread otherwise).
     if (vec_ok) {
         size_t nvec = num_els / VEC;
         unsigned blocks = cdiv(nvec, EW_BLOCK * EW_UNR);
-        hipLaunchKernelGGL((ew_nd_kernel<Op, VEC>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, nvec, op);
+        ew_record<Op>(1, blocks, sp, p, nvec, op);
+        if (blocks < EW_SMALL_BLOCKS)
+            hipLaunchKernelGGL((ew_nd_kernel<Op, VEC, 1>), dim3(cdiv(nvec, EW_BLOCK)), dim3(EW_BLOCK), 0, stream(), sp, p, nvec, op);
+        else
+            hipLaunchKernelGGL((ew_nd_kernel<Op, VEC>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, nvec, op);
     } else {
         unsigned blocks = cdiv(num_els, EW_BLOCK * EW_UNR);
-        hipLaunchKernelGGL((ew_nd_kernel<Op, 1>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, num_els, op);
+        ew_record<Op>(0, blocks, sp, p, num_els, op);
+        if (blocks < EW_SMALL_BLOCKS)
+            hipLaunchKernelGGL((ew_nd_kernel<Op, 1, 1>), dim3(cdiv(num_els, EW_BLOCK)), dim3(EW_BLOCK), 0, stream(), sp, p, num_els, op);
+        else
+            hipLaunchKernelGGL((ew_nd_kernel<Op, 1>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, num_els, op);
     }
     MXH_LAUNCH_CHECK("ew_nd");
 }

@@ -24,6 +24,7 @@
 
 #include <type_traits>
 
+#include "gemm_small.hpp"
 #include "mxh.hpp"
 
 #ifndef MXH_GEMM_INTERLEAVE
@@ -40,41 +41,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-struct GemmArgs {
-    const void* X;
-    const void* Y;
-    void* out;
-    int64_t xb, xi, xr;   // element strides of X: batch, output row, reduction
-    int64_t yb, yr, yj;   // element strides of Y: batch, reduction, output column
-    uint32_t I, J, R, batch;
-    uint32_t tiles_i, tiles_j;
-    // split-K: the reduction is cut into `splits` chunks of r_chunk (a multiple of the k-tile); with splits > 1
-    // every block writes its f32 partial tile to part[split][batch*I*J] and a second kernel folds them
-    uint32_t splits, r_chunk;
-    float* part;
-};
-
-template <class T> struct Elem;
-template <> struct Elem<float> {
-    static constexpr int VEC = 4;      // elements per 16-byte LDS fragment read
-    static __device__ float ld(float v) { return v; }
-    static __device__ float st(float v) { return v; }
-    static __device__ float zero() { return 0.0f; }
-};
-template <> struct Elem<bf16_t> {
-    static constexpr int VEC = 8;
-    static __device__ float ld(bf16_t v) { return bf2f(v); }
-    static __device__ bf16_t st(float v) { return f2bf(v); }
-    static __device__ bf16_t zero() { return bf16_t{0}; }
-};
-template <> struct Elem<f16_t> {
-    static constexpr int VEC = 8;
-    static __device__ float ld(f16_t v) { return h2f(v); }
-    static __device__ f16_t st(float v) { return f2h(v); }
-    static __device__ f16_t zero() { return f16_t{0}; }
-};
-
-constexpr int GB = 256;          // threads per block of the small-shape kernels
 constexpr int TK_BYTES = 128;    // reduction extent of one staged tile, in bytes per row
 
 template <class T, int N> struct alignas(sizeof(T) * N) GVec { T v[N]; };
@@ -388,13 +354,6 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     const int lrow = lane % TS, lk = (lane / TS) * VEC;
     constexpr int KS = (WAVE / TS) * VEC;                   // reduction steps one MFMA (group) consumes
 
-    typename Cfg::Acc acc[MI][MJ];
-#pragma unroll
-    for (int a = 0; a < MI; ++a)
-#pragma unroll
-        for (int c = 0; c < MJ; ++c)
-#pragma unroll
-            for (int e = 0; e < (TS == 32 ? 16 : 4); ++e) acc[a][c][e] = 0.0f;
 
     // Software pipeline (all indices compile-time after unrolling, one barrier per k-tile).  While the
     // MFMAs work through LDS[cur] (tile kt), step s < S-1 of the tile
@@ -414,16 +373,27 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     SX sx;
     SY sy;
     const uint32_t nk = (re - rb + TK - 1) / TK;
-    sx.template load<FAST>(X, g.xi, g.xr, i0, rb, g.I, re);
-    sy.template load<FAST>(Y, g.yj, g.yr, j0, rb, g.J, re);
-    sx.store(lds_x);
-    sy.store(lds_y);
     {
+        // tiles 0 and 1 are requested together (one memory latency instead of two); the accumulators are
+        // not live yet, so the second set of staging registers costs nothing
+        SX sx0;
+        SY sy0;
+        sx0.template load<FAST>(X, g.xi, g.xr, i0, rb, g.I, re);
+        sy0.template load<FAST>(Y, g.yj, g.yr, j0, rb, g.J, re);
         uint32_t r1 = rb + (nk > 1 ? 1u : 0u) * TK;
         sx.template load<FAST>(X, g.xi, g.xr, i0, r1, g.I, re);
         sy.template load<FAST>(Y, g.yj, g.yr, j0, r1, g.J, re);
+        sx0.store(lds_x);
+        sy0.store(lds_y);
     }
     __syncthreads();
+    typename Cfg::Acc acc[MI][MJ];
+#pragma unroll
+    for (int a = 0; a < MI; ++a)
+#pragma unroll
+        for (int c = 0; c < MJ; ++c)
+#pragma unroll
+            for (int e = 0; e < (TS == 32 ? 16 : 4); ++e) acc[a][c][e] = 0.0f;
 
     const int frag_x = (wm * TS * MI + lrow) * PITCH + lk;   // + a*TS*PITCH + k-step*KS
     const int frag_y = (wn * TS * MJ + lrow) * PITCH + lk;
@@ -588,24 +558,7 @@ void launch_mfma(GemmArgs g) {
     else launch_mfma_impl<T, XR, YR, Cfg, false>(g);
 }
 
-// ---- small shapes -----------------------------------------------------------------------------------
-// One thread per output element, r ascending, multiply and add unfused: the reference's own
-// order, so f32 results are bit-identical to it.
-template <class T>
-__global__ __launch_bounds__(GB) void gemm_thread_kernel(GemmArgs g) {
-    size_t idx = (size_t)blockIdx.x * GB + threadIdx.x;
-    size_t per = (size_t)g.I * g.J;
-    if (idx >= per * g.batch) return;
-    uint32_t b = (uint32_t)(idx / per);
-    uint32_t rem = (uint32_t)(idx % per);
-    uint32_t i = rem / g.J, j = rem % g.J;
-    const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
-    const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
-    float acc = 0.0f;
-    for (uint32_t r = 0; r < g.R; ++r) acc = acc + Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
-    ((T*)g.out)[idx] = Elem<T>::st(acc);
-}
-
+// ---- small shapes (the per-thread and per-block dot kernels are in gemm_small.hpp) -------------------
 // One wave per output element: lanes stride over r, 4 independent partial sums per lane, then a
 // fixed shuffle tree.  For few outputs with a long reduction.
 template <class T>
@@ -637,41 +590,22 @@ __global__ __launch_bounds__(GB) void gemm_wavedot_kernel(GemmArgs g) {
     if (live && lane == 0) ((T*)g.out)[idx] = Elem<T>::st(acc);
 }
 
-// One block per output element for a handful of outputs with a long reduction (the MLP's weight gradient:
-// 3 outputs of 10000 terms): threads stride over r, waves fold by shuffles, the block by LDS, in a fixed order.
-template <class T>
-__global__ __launch_bounds__(1024) void gemm_blockdot_kernel(GemmArgs g) {
-    __shared__ float part[1024 / WAVE];
-    const size_t idx = blockIdx.x;
-    const size_t per = (size_t)g.I * g.J;
-    const uint32_t b = (uint32_t)(idx / per), rem = (uint32_t)(idx % per);
-    const uint32_t i = rem / g.J, j = rem % g.J;
-    const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
-    const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
-    float acc = 0.0f;
-    for (uint32_t r = threadIdx.x; r < g.R; r += 1024) acc += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, WAVE);
-    if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float sum = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 1024 / WAVE; ++w) sum += part[w];
-        ((T*)g.out)[idx] = Elem<T>::st(sum);
-    }
-}
-
 template <class T>
 void gemm_dispatch(GemmArgs g) {
     if (g.I == 0 || g.J == 0 || g.batch == 0) return;
     size_t outputs = (size_t)g.I * g.J * g.batch;
     if (g.R <= 16 || (g.I < 16 && g.J < 16 && g.R < 256)) {
+        if constexpr (std::is_same<T, float>::value)
+            if (prog_recording() && cdiv(outputs, GB) <= PROG_MAX_GRID && (size_t)g.R * outputs <= PROG_MAX_ELEMS)
+                prog_record(prog_kid(PF_GEMM_THREAD, 0), (unsigned)cdiv(outputs, GB), &g, sizeof(g));
         hipLaunchKernelGGL(gemm_thread_kernel<T>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_thread");
         return;
     }
     if (outputs <= 64 && g.R >= 4096) {
+        if constexpr (std::is_same<T, float>::value)
+            if (prog_recording() && (size_t)g.R * outputs <= PROG_MAX_ELEMS)
+                prog_record(prog_kid(PF_GEMM_BLOCKDOT, 0), (unsigned)outputs, &g, sizeof(g));
         hipLaunchKernelGGL(gemm_blockdot_kernel<T>, dim3((unsigned)outputs), dim3(1024), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_blockdot");
         return;
@@ -694,6 +628,9 @@ void gemm_dispatch(GemmArgs g) {
     else if (xi && yj) MXH_GEMM_CASE(false, false);
     else {
         // no unit stride on one operand: correct but slow
+        if constexpr (std::is_same<T, float>::value)
+            if (prog_recording() && cdiv(outputs, GB) <= PROG_MAX_GRID && (size_t)g.R * outputs <= PROG_MAX_ELEMS)
+                prog_record(prog_kid(PF_GEMM_THREAD, 0), (unsigned)cdiv(outputs, GB), &g, sizeof(g));
         hipLaunchKernelGGL(gemm_thread_kernel<T>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_thread");
     }

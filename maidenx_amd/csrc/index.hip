@@ -358,6 +358,8 @@ void index_add(size_t nd, size_t dim, const size_t* self_layout, const size_t* s
         uint32_t *k_in = (uint32_t*)ws, *k_out = (uint32_t*)(ws + arr), *v_in = (uint32_t*)(ws + 2 * arr), *v_out = (uint32_t*)(ws + 3 * arr);
         hipLaunchKernelGGL(index_keys_kernel<I>, dim3(cdiv(n_idx, IB)), dim3(IB), 0, stream(), indices, (int64_t)idx_stride, (int64_t)idx_offset,
                            (uint32_t)n_idx, (uint32_t)D, k_in, v_in, flag);
+        MXH_LAUNCH_CHECK("index_keys");
+        prog_launch_seen();      // the sort's own launches
         MXH_HIP(rocprim::radix_sort_pairs(ws + 4 * arr, sort_bytes, k_in, k_out, v_in, v_out, n_idx, 0u, bits, stream()));
         {
             constexpr int VEC = 16 / sizeof(T);

@@ -5,6 +5,8 @@
 #include <cstddef>
 #include <cstdint>
 
+#include "program.hpp"
+
 namespace mxh {
 
 // ---- status codes returned by hip_get_last_status() ------------------------------------
@@ -34,7 +36,11 @@ int* index_flag();
         hipError_t e__ = (expr);                                                      \
         if (e__ != hipSuccess) ::mxh::set_status(::mxh::ERR_LAUNCH, #expr, (int)e__); \
     } while (0)
-#define MXH_LAUNCH_CHECK(name) MXH_HIP(hipGetLastError())
+#define MXH_LAUNCH_CHECK(name)            \
+    do {                                  \
+        MXH_HIP(hipGetLastError());       \
+        ::mxh::prog_launch_seen();        \
+    } while (0)
 
 // ---- bf16 storage type -----------------------------------------------------------------
 // Same bits as the `half` crate's bf16 the reference stores: upper half of a binary32,

@@ -148,4 +148,22 @@ MXH_UNC(OpLeScalar, bool_t, (bool_t)(F(x) <= F(c)))
 MXH_UNC(OpGtScalar, bool_t, (bool_t)(F(x) > F(c)))
 MXH_UNC(OpGeScalar, bool_t, (bool_t)(F(x) >= F(c)))
 
+// ---- functors without an arithmetic of their own ---------------------------------------------
+template <class T> struct OpFill {     // output-only "unary": the input value is ignored
+    using In = T; using Out = T; static constexpr int NIN = 1;
+    T c;
+    __device__ T operator()(T) const { return c; }
+};
+template <class T> struct OpIdentity {
+    using In = T; using Out = T; static constexpr int NIN = 1;
+    __device__ T operator()(T x) const { return x; }
+};
+// `0 + x`: what a sum_to_shape that keeps every dim does through its zero-initialised cells (-0 -> +0).
+// The 16-bit forms live with the reductions, whose rounding helpers they use.
+template <class T> struct OpZeroPlus;
+template <> struct OpZeroPlus<float> {
+    using In = float; using Out = float; static constexpr int NIN = 1;
+    __device__ float operator()(float x) const { return 0.0f + x; }
+};
+
 }  // namespace mxh

@@ -2,8 +2,10 @@
 // cuda_malloc / cuda_free / cuda_memcpy_* / cuda_set_device / cuda_get_device family of
 // crates/maidenx_cuda/src/lib.rs:39-117.
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "mxh.hpp"
 
@@ -18,6 +20,16 @@ static hipStream_t g_stream = nullptr;      // null = the device's default strea
 static hipStream_t g_capture_stream = nullptr;   // created on first use, default priority
 static hipStream_t g_saved_stream = nullptr;
 static bool g_capturing = false;
+// recording of a capture as a program (see program.hpp)
+static bool g_prog_enabled = true;
+static bool g_prog_ok = false;            // every launch of the open capture so far has a command
+static bool g_prog_pending = false;       // a command was recorded and its launch not yet seen
+static std::vector<ProgCmd> g_prog_cmds;
+struct GraphExec {                        // what hip_graph_end_capture hands out
+    hipGraphExec_t graph = nullptr;
+    ProgCmd* cmds = nullptr;              // device copy of the program, when the capture is one
+    uint32_t n = 0;
+};
 static void* g_scratch[16][2] = {{nullptr}};
 static size_t g_scratch_bytes[16][2] = {{0}};
 
@@ -33,6 +45,24 @@ void set_status(int code, const char* what, int hip_err) {
 }
 
 hipStream_t stream() { return g_stream; }
+
+bool prog_recording() { return g_capturing && g_prog_ok; }
+void prog_record(uint32_t kid, unsigned grid, const void* args, size_t bytes) {
+    if (!prog_recording()) return;
+    if (bytes > PROG_ARG_BYTES || grid > PROG_MAX_GRID || g_prog_pending || g_prog_cmds.size() >= 65536) { g_prog_ok = false; return; }
+    ProgCmd c;
+    std::memset((void*)&c, 0, sizeof(c));
+    c.kid = kid;
+    c.grid = grid;
+    std::memcpy(c.args, args, bytes);
+    g_prog_cmds.push_back(c);
+    g_prog_pending = true;
+}
+void prog_launch_seen() {
+    if (!g_capturing) return;
+    if (g_prog_pending) g_prog_pending = false;
+    else g_prog_ok = false;               // a launch without a command: only the HIP graph can replay this capture
+}
 
 void* scratch(size_t bytes, int slot) {
     int dev = 0;
@@ -132,6 +162,7 @@ int hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
     return (int)e;
 }
 int hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    prog_launch_seen();
     return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream());
 }
 
@@ -185,6 +216,9 @@ int hip_graph_begin_capture(void) {
     g_saved_stream = g_stream;
     g_stream = g_capture_stream;
     g_capturing = true;
+    g_prog_ok = g_prog_enabled;
+    g_prog_pending = false;
+    g_prog_cmds.clear();
     return 0;
 }
 int hip_graph_end_capture(void** graph_exec) {
@@ -193,23 +227,54 @@ int hip_graph_end_capture(void** graph_exec) {
     hipError_t e = hipStreamEndCapture(g_capture_stream, &graph);
     g_stream = g_saved_stream;
     g_capturing = false;
+    const bool as_program = g_prog_ok && !g_prog_pending && !g_prog_cmds.empty();
+    if (getenv("MXH_DEBUG_PROGRAM")) fprintf(stderr, "[maidenx_hip] capture closed: %zu commands recorded, %s\n", g_prog_cmds.size(), as_program ? "program" : "HIP graph");
     if (e != hipSuccess) return (int)e;
-    hipGraphExec_t exec = nullptr;
-    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) return (int)e;
-    *graph_exec = (void*)exec;
+    GraphExec* ge = new GraphExec();
+    if (as_program) {
+        // every launch of the capture has a command: replays are one launch of the interpreter
+        (void)hipGraphDestroy(graph);
+        const size_t bytes = g_prog_cmds.size() * sizeof(ProgCmd);
+        e = hipMalloc((void**)&ge->cmds, bytes);
+        if (e == hipSuccess) e = hipMemcpy(ge->cmds, g_prog_cmds.data(), bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) { if (ge->cmds) (void)hipFree(ge->cmds); delete ge; return (int)e; }
+        ge->n = (uint32_t)g_prog_cmds.size();
+    } else {
+        e = hipGraphInstantiate(&ge->graph, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        if (e != hipSuccess) { delete ge; return (int)e; }
+    }
+    g_prog_cmds.clear();
+    *graph_exec = (void*)ge;
     return 0;
+}
+// 1 when the capture behind `graph_exec` replays as one interpreter launch, 0 when it is a HIP graph.
+int hip_graph_is_program(void* graph_exec) { return graph_exec && ((GraphExec*)graph_exec)->cmds ? 1 : 0; }
+// Whether later captures may become programs (default 1); returns the previous setting.
+int hip_graph_set_programs(int enabled) {
+    int was = g_prog_enabled ? 1 : 0;
+    g_prog_enabled = enabled != 0;
+    return was;
 }
 // Replays run on the capture stream, a blocking stream: work on the default stream orders with it.
 int hip_graph_launch(void* graph_exec) {
     if (!graph_exec || !g_capture_stream || g_capturing) return (int)hipErrorInvalidValue;
-    return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, g_capture_stream);
+    GraphExec* ge = (GraphExec*)graph_exec;
+    if (ge->cmds) {
+        prog_launch(ge->cmds, ge->n, (void*)g_capture_stream);
+        return (int)hipGetLastError();
+    }
+    return (int)hipGraphLaunch(ge->graph, g_capture_stream);
 }
 int hip_graph_destroy(void* graph_exec) {
     if (!graph_exec) return 0;
     (void)hipStreamSynchronize(g_capture_stream);
-    return (int)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+    GraphExec* ge = (GraphExec*)graph_exec;
+    hipError_t e = hipSuccess;
+    if (ge->cmds) e = hipFree(ge->cmds);
+    if (ge->graph) e = hipGraphExecDestroy(ge->graph);
+    delete ge;
+    return (int)e;
 }
 
 }  // extern "C"

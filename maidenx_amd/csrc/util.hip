@@ -9,15 +9,6 @@
 
 namespace mxh {
 
-template <class T> struct OpFill {     // output-only "unary": the input value is ignored
-    using In = T; using Out = T; static constexpr int NIN = 1;
-    T c;
-    __device__ T operator()(T) const { return c; }
-};
-template <class T> struct OpIdentity {
-    using In = T; using Out = T; static constexpr int NIN = 1;
-    __device__ T operator()(T x) const { return x; }
-};
 template <class TI, class TO> struct OpConvert;
 template <> struct OpConvert<bool_t, float> { using In = bool_t; using Out = float; static constexpr int NIN = 1;
     __device__ float operator()(bool_t x) const { return x ? 1.0f : 0.0f; } };

@@ -47,6 +47,7 @@ def load():
         ("hip_event_elapsed_ms", [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)], C.c_int),
         ("hip_graph_begin_capture", [], C.c_int), ("hip_graph_end_capture", [C.POINTER(C.c_void_p)], C.c_int),
         ("hip_graph_launch", [C.c_void_p], C.c_int), ("hip_graph_destroy", [C.c_void_p], C.c_int),
+        ("hip_graph_is_program", [C.c_void_p], C.c_int), ("hip_graph_set_programs", [C.c_int], C.c_int),
     ]:
         fn = getattr(lib, name)
         fn.argtypes = args

@@ -1,0 +1,190 @@
+"""Recorded programs: a capture of small kernels replays as one interpreter launch (hip_graph_is_program == 1)
+and must leave exactly the bytes the eager calls leave; anything larger or without an interpreter body must
+fall back to a HIP graph and still replay correctly."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import maidenx_amd._signatures as S
+import maidenx_amd.lib as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if L.device_count() < 1:
+        pytest.skip("no GPU")
+    return L.load()
+
+
+def u64(*parts):
+    out = []
+    for x in parts:
+        out += list(x) if isinstance(x, (list, tuple)) else [x]
+    return np.array(out, dtype=np.uint64)
+
+
+class Seq:
+    """A list of backend calls on device buffers that can be run eagerly or inside a capture."""
+
+    def __init__(self, lib):
+        self.lib, self.calls, self.outs, self.keep = lib, [], [], []
+
+    def dev(self, a):
+        b = L.DeviceBuffer.from_numpy(np.ascontiguousarray(a))
+        self.keep.append(b)
+        return b
+
+    def out(self, nbytes, dtype):
+        b = L.DeviceBuffer(nbytes)
+        self.keep.append(b)
+        self.outs.append((b, nbytes, dtype))
+        return b
+
+    def add(self, name, *args):
+        self.keep.append(args)
+        self.calls.append((getattr(self.lib, "hip_" + name), args))
+
+    def run(self):
+        for fn, args in self.calls:
+            fn(*[a.ctypes.data if isinstance(a, np.ndarray) else a for a in args])
+
+    def clear_outputs(self):
+        for b, n, dt in self.outs:
+            if dt == "f4":
+                self.lib.hip_fill_f32(n // 4, b.ptr, C.c_float(-7.0))
+            elif dt == "u2":
+                self.lib.hip_fill_bf16(n // 2, b.ptr, C.c_uint16(0x7FC0))
+            else:
+                self.lib.hip_fill_bool(n, b.ptr, C.c_uint8(9))
+        assert self.lib.hip_synchronize() == 0
+
+    def read(self):
+        assert self.lib.hip_synchronize() == 0
+        return [b.to_numpy(np.dtype(dt), n // np.dtype(dt).itemsize).copy() for b, n, dt in self.outs]
+
+
+def replay_equals_eager(lib, seq, expect_program, replays=3):
+    seq.run()
+    eager = seq.read()
+    assert lib.hip_get_last_status() == 0, lib.hip_status_string()
+    seq.clear_outputs()
+    assert lib.hip_graph_begin_capture() == 0
+    seq.run()
+    h = C.c_void_p()
+    assert lib.hip_graph_end_capture(C.byref(h)) == 0
+    try:
+        assert lib.hip_graph_is_program(h) == (1 if expect_program else 0)
+        for _ in range(replays):
+            seq.clear_outputs()          # eager work and a synchronisation between the replays
+            assert lib.hip_graph_launch(h) == 0
+            got = seq.read()
+            for g, e in zip(got, eager):
+                assert g.tobytes() == e.tobytes()
+    finally:
+        assert lib.hip_graph_destroy(h) == 0
+    assert lib.hip_get_last_status() == 0, lib.hip_status_string()
+
+
+def elementwise_sequence(lib, shape, rhs_strides, seed):
+    """Every f32 elementwise entry point once, on the same operands (rhs optionally broadcast)."""
+    r = np.random.default_rng(seed)
+    n = int(np.prod(shape))
+    a = r.standard_normal(n).astype(np.float32)
+    a[::7] = 0.0
+    b_full = r.standard_normal(n).astype(np.float32)
+    b_full[::5] = 0.0
+    seq = Seq(lib)
+    da = seq.dev(a)
+    cont = [int(np.prod(shape[i + 1:])) for i in range(len(shape))]
+    if rhs_strides is None:
+        rhs_strides, db = cont, seq.dev(b_full)
+    else:
+        extent = 1 + sum((d - 1) * s for d, s in zip(shape, rhs_strides))
+        db = seq.dev(b_full[:extent])
+    md2 = u64(list(shape), cont, list(rhs_strides), 0, 0)
+    md1 = u64(list(shape), cont, 0)
+    nd = len(shape)
+    for op in S.BINARY:
+        o = seq.out(n * (1 if op in S.BOOL_OUT else 4), "u1" if op in S.BOOL_OUT else "f4")
+        seq.add(f"{op}_f32", n, nd, md2, da.ptr, db.ptr, o.ptr)
+    for op in S.UNARY:
+        o = seq.out(n * (1 if op in S.BOOL_OUT else 4), "u1" if op in S.BOOL_OUT else "f4")
+        seq.add(f"{op}_f32", n, nd, md1, da.ptr, o.ptr)
+    for op in S.UNARY_CONST:
+        o = seq.out(n * (1 if op in S.BOOL_OUT else 4), "u1" if op in S.BOOL_OUT else "f4")
+        seq.add(f"{op}_f32", n, nd, md1, da.ptr, C.c_float(0.5 if op != "pow" else 2.0), o.ptr)
+    return seq
+
+
+@pytest.mark.parametrize("shape,rhs_strides", [((1000,), None), ((37, 21), None), ((8, 128), (0, 1)), ((16, 64), (1, 0)), ((5, 3, 7), (0, 7, 1))],
+                         ids=["vector", "odd", "row-bcast", "col-bcast", "3d-bcast"])
+def test_every_f32_elementwise_op_replays_bit_exact(lib, shape, rhs_strides):
+    replay_equals_eager(lib, elementwise_sequence(lib, shape, rhs_strides, 1), expect_program=True)
+
+
+def test_dependent_chain_with_reductions_and_small_matmul(lib):
+    """A training-step-like chain: matmul -> bias add -> loss -> reductions -> in-place update, every call reading what
+    an earlier call of the same replay wrote."""
+    r = np.random.default_rng(3)
+    n, k = 200, 3
+    seq = Seq(lib)
+    x, w = seq.dev(r.standard_normal((n, k)).astype(np.float32)), seq.dev(r.standard_normal((k, 1)).astype(np.float32))
+    bias, y = seq.dev(np.array([0.25], np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    pred, pb, diff, sq = (seq.out(n * 4, "f4") for _ in range(4))
+    loss, mx, mn, rows = seq.out(4, "f4"), seq.out(4, "f4"), seq.out(4, "f4"), seq.out(10 * 4, "f4")
+    gw, wnew = seq.out(k * 4, "f4"), seq.out(k * 4, "f4")
+    mm = u64(2, 2, 2, [n, 1], [n, k], [k, 1], [k, 1], [1, 1], 0, 0)
+    seq.add("matmul_f32", n, mm, x.ptr, w.ptr, pred.ptr)
+    seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), pred.ptr, bias.ptr, pb.ptr)
+    seq.add("sub_f32", n, 1, u64([n], [1], [1], 0, 0), pb.ptr, y.ptr, diff.ptr)
+    seq.add("pow_f32", n, 1, u64([n], [1], 0), diff.ptr, C.c_float(2.0), sq.ptr)
+    for name, o in (("mean", loss), ("max", mx), ("min", mn)):
+        seq.add(f"{name}_f32", n, 1, 1, u64([n], [1], [n], [1], 0), sq.ptr, o.ptr)
+    seq.add("sum_f32", n, 2, 1, u64([10, 20], [20, 1], [20], [1], 0), sq.ptr, rows.ptr)          # 10 rows of 20
+    # gw[k,1] = x^T[k,n] . diff[n,1]  (a long reduction for few outputs when n is large; the per-thread kernel here)
+    mt = u64(2, 2, 2, [k, 1], [k, n], [n, 1], [1, k], [1, 1], 0, 0)
+    seq.add("matmul_f32", k, mt, x.ptr, diff.ptr, gw.ptr)
+    seq.add("mul_scalar_f32", k, 1, u64([k], [1], 0), gw.ptr, C.c_float(0.01), wnew.ptr)
+    seq.add("sub_inplace_f32", k, 1, u64([k], [1], [1], 0, 0), wnew.ptr, gw.ptr)
+    replay_equals_eager(lib, seq, expect_program=True)
+
+
+def test_block_dot_matmul_in_a_program(lib):
+    r = np.random.default_rng(4)
+    n = 8192
+    seq = Seq(lib)
+    x, g = seq.dev(r.standard_normal((n, 2)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    gw = seq.out(2 * 4, "f4")
+    seq.add("matmul_f32", 2, u64(2, 2, 2, [2, 1], [2, n], [n, 1], [1, 2], [1, 1], 0, 0), x.ptr, g.ptr, gw.ptr)
+    replay_equals_eager(lib, seq, expect_program=True)
+
+
+def test_large_or_unsupported_captures_stay_hip_graphs(lib):
+    r = np.random.default_rng(5)
+    # a tensor beyond one pass of the interpreter's work-group
+    n = 1 << 16
+    seq = Seq(lib)
+    a, o = seq.dev(r.standard_normal(n).astype(np.float32)), seq.out(n * 4, "f4")
+    seq.add("neg_f32", n, 1, u64([n], [1], 0), a.ptr, o.ptr)
+    replay_equals_eager(lib, seq, expect_program=False)
+    # a small one next to a kernel without an interpreter body (column reduction), and a bf16 op
+    seq = Seq(lib)
+    a = seq.dev(r.standard_normal((32, 48)).astype(np.float32))
+    o1, o2 = seq.out(32 * 48 * 4, "f4"), seq.out(48 * 4, "f4")
+    seq.add("neg_f32", 32 * 48, 2, u64([32, 48], [48, 1], 0), a.ptr, o1.ptr)
+    seq.add("sum_f32", 32 * 48, 2, 1, u64([32, 48], [48, 1], [32], [48], 0), o1.ptr, o2.ptr)
+    replay_equals_eager(lib, seq, expect_program=False)
+    seq = Seq(lib)
+    h = seq.dev((r.standard_normal(512).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    o = seq.out(512 * 2, "u2")
+    seq.add("neg_bf16", 512, 1, u64([512], [1], 0), h.ptr, o.ptr)
+    replay_equals_eager(lib, seq, expect_program=False)
+    # programs switched off
+    was = lib.hip_graph_set_programs(0)
+    try:
+        replay_equals_eager(lib, elementwise_sequence(lib, (1000,), None, 2), expect_program=False, replays=1)
+    finally:
+        lib.hip_graph_set_programs(was)
