@@ -25,6 +25,7 @@ struct PadSpace {
 
 
 constexpr int PB = 256;
+enum EdgeMode : int { EDGE_REFLECT = 0, EDGE_REPLICATE = 1, EDGE_NONE = 2 };     // NONE: constant padding, whose border feeds nothing back
 
 // forward: out[i] = inside ? in[idx] : pad_value
 // backward (FWD = false): grad_in[idx] = 0 + grad_out[i] for every inside i
@@ -113,6 +114,80 @@ __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __r
     }
 }
 
+// ---- at most three dims after merging (the usual [N*C, H, W] of a padded image batch) -------------------
+// The same walks with 32-bit coordinates and two divisions per thread.  Dims are right-aligned: slot 2 is the
+// innermost one, missing outer dims have size 1.
+struct Pad3 {
+    uint32_t out[3], in[3], before[3];
+    FastDiv out_div[3], in_div[3];
+    int64_t in_stride[3];
+    uint32_t out_stride[3];
+};
+static bool make_pad3(const PadSpace& sp, Pad3& p3) {
+    if (sp.ndims > 3) return false;
+    const int shift = 3 - sp.ndims;
+    uint64_t ost = 1;
+    for (int k = 2; k >= 0; --k) {
+        const int d = k - shift;
+        const bool real = d >= 0;
+        p3.out[k] = real ? sp.out_dims[d] : 1;
+        p3.in[k] = real ? sp.in_dims[d] : 1;
+        p3.before[k] = real ? sp.before[d] : 0;
+        p3.in_stride[k] = real ? sp.in_strides[d] : 0;
+        p3.out_div[k] = make_fastdiv(p3.out[k]);
+        p3.in_div[k] = make_fastdiv(p3.in[k]);
+        p3.out_stride[k] = (uint32_t)ost;
+        ost *= p3.out[k];
+    }
+    return ost < (1ull << 31);
+}
+
+template <class T, bool FWD, int Q>
+__global__ __launch_bounds__(PB) void pad_const3_kernel(Pad3 sp, const T* __restrict__ src, T* __restrict__ dst, uint32_t n_out, T pad_value) {
+    const uint32_t i0 = (blockIdx.x * PB + threadIdx.x) * Q;
+    if (i0 >= n_out) return;
+    uint32_t q, c2, c1, c0;
+    fd_divmod(i0, sp.out_div[2], q, c2);
+    fd_divmod(q, sp.out_div[1], c0, c1);
+    const bool full = i0 + Q <= n_out;
+    AVec<T, Q> v;
+    if constexpr (!FWD) {
+        if (full) v = *(const AVec<T, Q>*)(src + i0);
+        else
+            for (int e = 0; e < Q; ++e) v.v[e] = i0 + e < n_out ? src[i0 + e] : T{};
+    }
+    int64_t row = 0;
+    bool row_in = false, fresh = true;
+#pragma unroll
+    for (int e = 0; e < Q; ++e) {
+        if (fresh) {
+            const uint32_t i0c = c0 - sp.before[0], i1c = c1 - sp.before[1];      // wrap when outside: fail the test
+            row_in = i0c < sp.in[0] && i1c < sp.in[1];
+            row = (int64_t)i0c * sp.in_stride[0] + (int64_t)i1c * sp.in_stride[1];
+            fresh = false;
+        }
+        const uint32_t ic = c2 - sp.before[2];
+        const bool inside = row_in && ic < sp.in[2] && (full || i0 + e < n_out);
+        const int64_t idx = row + (int64_t)ic * sp.in_stride[2];
+        if constexpr (FWD) {
+            v.v[e] = inside ? src[idx] : pad_value;
+        } else {
+            if (inside) dst[idx] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(v.v[e]));      // -0 -> +0 like the reference's sums from zero
+        }
+        if (++c2 == sp.out[2]) {
+            c2 = 0;
+            fresh = true;
+            if (++c1 == sp.out[1]) { c1 = 0; ++c0; }
+        }
+    }
+    if constexpr (FWD) {
+        if (full) *(AVec<T, Q>*)(dst + i0) = v;
+        else
+            for (int e = 0; e < Q; ++e)
+                if (i0 + e < n_out) dst[i0 + e] = v.v[e];
+    }
+}
+
 template <class T>
 __global__ __launch_bounds__(PB) void zero_kernel(T* p, size_t n) {
     size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
@@ -170,11 +245,50 @@ void pad_forward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const T
     PadSpace sp; size_t off; bool cont, exact;
     if (!build_space(nd, md, sp, &off, &cont, &exact)) { set_status(ERR_UNSUPPORTED, "pad: rank above 8 after collapse"); return; }
     constexpr int Q = 16 / sizeof(T);
-    if ((uintptr_t)out % 16 == 0)
+    Pad3 p3;
+    if ((uintptr_t)out % 16 == 0 && make_pad3(sp, p3))
+        hipLaunchKernelGGL((pad_const3_kernel<T, true, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), p3, in + off, out, (uint32_t)n_out, pad_value);
+    else if ((uintptr_t)out % 16 == 0)
         hipLaunchKernelGGL((pad_const_kernel<T, true, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
     else
         hipLaunchKernelGGL((pad_const_kernel<T, true, 1>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
     MXH_LAUNCH_CHECK("pad_const");
+}
+
+// Backward of a constant pad onto a contiguous input that every output position of the interior maps to: a
+// crop.  A thread owns four consecutive input elements (one vector store); `0 + g` as in the scatter form.
+template <class T>
+__global__ __launch_bounds__(PB) void pad_crop3_kernel(Pad3 sp, const T* __restrict__ go, T* __restrict__ gi, uint32_t n_in, bool vec_store) {
+    constexpr uint32_t PER = 4;
+    const uint32_t i0 = (blockIdx.x * PB + threadIdx.x) * PER;
+    if (i0 >= n_in) return;
+    uint32_t p0, p1, p2, q;
+    fd_divmod(i0, sp.in_div[2], q, p2);
+    fd_divmod(q, sp.in_div[1], p0, p1);
+    uint32_t row = 0;
+    bool fresh = true;
+    AVec<T, PER> v;
+#pragma unroll
+    for (uint32_t e = 0; e < PER; ++e) {
+        if (i0 + e >= n_in) break;
+        if (fresh) {
+            row = (p0 + sp.before[0]) * sp.out_stride[0] + (p1 + sp.before[1]) * sp.out_stride[1] + sp.before[2];
+            fresh = false;
+        }
+        v.v[e] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(go[row + p2]));
+        if (++p2 == sp.in[2]) {
+            p2 = 0;
+            fresh = true;
+            if (++p1 == sp.in[1]) { p1 = 0; ++p0; }
+        }
+    }
+    if (vec_store && i0 + PER <= n_in) {
+        *(AVec<T, PER>*)(gi + i0) = v;
+    } else {
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e)
+            if (i0 + e < n_in) gi[i0 + e] = v.v[e];
+    }
 }
 
 template <class T>
@@ -191,7 +305,20 @@ void pad_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const 
     }
     if (n_out == 0) return;
     constexpr int Q = 16 / sizeof(T);
-    if ((uintptr_t)go % 16 == 0)
+    Pad3 p3;
+    size_t logical = 1;
+    for (size_t d = 0; d < nd; ++d) logical *= md[d];
+    if (cont && exact && logical == n_in && logical < (1ull << 31) && make_pad3(sp, p3)) {
+        // every input position is read back from exactly one output position: gather by input element, which
+        // keeps the stores whole vectors
+        hipLaunchKernelGGL(pad_crop3_kernel<T>, dim3(cdiv(logical, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, go, gi + off, (uint32_t)logical,
+                           (uintptr_t)(gi + off) % (4 * sizeof(T)) == 0);
+        MXH_LAUNCH_CHECK("pad_const_backward");
+        return;
+    }
+    if ((uintptr_t)go % 16 == 0 && make_pad3(sp, p3))
+        hipLaunchKernelGGL((pad_const3_kernel<T, false, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), p3, go, gi + off, (uint32_t)n_out, T{});
+    else if ((uintptr_t)go % 16 == 0)
         hipLaunchKernelGGL((pad_const_kernel<T, false, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
     else
         hipLaunchKernelGGL((pad_const_kernel<T, false, 1>), dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
@@ -206,7 +333,6 @@ void pad_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const 
 // enumerated in ascending order (replication: a run; reflection: p + k*P and -p + k*P shifted by the
 // leading pad, P = 2*(dim-1)), and the dims are walked like an odometer, so a thread adds its terms in
 // ascending output index — the order the reference gets with one worker.  f32 accumulation.
-enum EdgeMode : int { EDGE_REFLECT = 0, EDGE_REPLICATE = 1 };
 
 __device__ inline uint32_t edge_pos(int mode, int64_t pos, int64_t dim) {
     if (mode == EDGE_REPLICATE) return (uint32_t)(pos < 0 ? 0 : (pos > dim - 1 ? dim - 1 : pos));
@@ -235,6 +361,58 @@ __global__ __launch_bounds__(PB) void pad_edge_kernel(PadSpace sp, int mode, con
         r = q;
     }
     dst[i] = src[idx];
+}
+
+// The same copy for at most three dims and one reflection per side (see `simple_edge_shape`): two divisions and
+// 32-bit coordinates per element, four consecutive outputs of a row per thread.
+__device__ __forceinline__ uint32_t edge_pos_once(int mode, uint32_t o, uint32_t before, uint32_t dim) {
+    const int32_t q = (int32_t)o - (int32_t)before;
+    if (mode == EDGE_REPLICATE) return (uint32_t)(q < 0 ? 0 : (q > (int32_t)dim - 1 ? (int32_t)dim - 1 : q));
+    return (uint32_t)(q < 0 ? -q : (q >= (int32_t)dim ? 2 * (int32_t)dim - q - 2 : q));
+}
+template <class T>
+__global__ __launch_bounds__(PB) void pad_edge3_kernel(Pad3 sp, int mode, const T* __restrict__ src, T* __restrict__ dst, uint32_t n_out,
+                                                       bool vec_store) {
+    constexpr uint32_t PER = 4;
+    const uint32_t i0 = (blockIdx.x * PB + threadIdx.x) * PER;
+    if (i0 >= n_out) return;
+    uint32_t q, c2, c1, c0;
+    fd_divmod(i0, sp.out_div[2], q, c2);
+    fd_divmod(q, sp.out_div[1], c0, c1);
+    int64_t row = 0;
+    bool fresh = true;
+    AVec<T, PER> v;
+#pragma unroll
+    for (uint32_t e = 0; e < PER; ++e) {
+        if (i0 + e >= n_out) break;
+        if (fresh) {
+            row = (int64_t)edge_pos_once(mode, c0, sp.before[0], sp.in[0]) * sp.in_stride[0] +
+                  (int64_t)edge_pos_once(mode, c1, sp.before[1], sp.in[1]) * sp.in_stride[1];
+            fresh = false;
+        }
+        v.v[e] = src[row + (int64_t)edge_pos_once(mode, c2, sp.before[2], sp.in[2]) * sp.in_stride[2]];
+        if (++c2 == sp.out[2]) {          // carry into the outer coordinates
+            c2 = 0;
+            fresh = true;
+            if (++c1 == sp.out[1]) { c1 = 0; ++c0; }
+        }
+    }
+    if (vec_store && i0 + PER <= n_out) {
+        *(AVec<T, PER>*)(dst + i0) = v;
+    } else {
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e)
+            if (i0 + e < n_out) dst[i0 + e] = v.v[e];
+    }
+}
+static bool simple_edge_shape(const PadSpace& sp, int mode) {
+    if (sp.ndims > 3) return false;
+    for (int d = 0; d < sp.ndims; ++d) {
+        if ((uint64_t)sp.in_dims[d] + sp.before[d] > sp.out_dims[d] || sp.in_dims[d] == 0) return false;
+        const uint32_t after = sp.out_dims[d] - sp.in_dims[d] - sp.before[d];
+        if (mode == EDGE_REFLECT && (sp.before[d] > sp.in_dims[d] - 1 || after > sp.in_dims[d] - 1)) return false;
+    }
+    return true;
 }
 
 // what the backward walk needs besides the PadSpace: how to split an input index, where an output coordinate lands
@@ -317,6 +495,85 @@ __global__ __launch_bounds__(PB) void pad_edge_backward_kernel(PadSpace sp, Edge
     gi[dst] = Ar<T>::from_f32(acc);
 }
 
+// The common shape of the backward walk: at most three dims after merging and at most one reflection per side
+// (pads no larger than dim - 1).  The output coordinates that map to input coordinate p of one dim are then an
+// optional mirror image on the left, the run around p + before (longer than one only for a replicated border) and an
+// optional mirror image on the right - ascending, so the sums keep the reference's order.  All 32-bit, no division.
+struct EdgeSrc {
+    uint32_t cl, a0, a1, cr, has_l, n;
+    __device__ void init(int mode, uint32_t p, uint32_t in_dim, uint32_t out_dim, uint32_t before) {
+        const uint32_t after = out_dim - in_dim - before;
+        a0 = a1 = p + before;
+        cl = cr = 0;
+        has_l = 0;
+        uint32_t has_r = 0;
+        if (mode == EDGE_REPLICATE) {
+            if (p == 0) a0 = 0;
+            if (p == in_dim - 1) a1 = out_dim - 1;
+        } else if (mode == EDGE_REFLECT) {
+            if (p >= 1 && p <= before) { has_l = 1; cl = before - p; }
+            if (p + 1 < in_dim && p + after + 1 >= in_dim) { has_r = 1; cr = before + 2 * (in_dim - 1) - p; }
+        }
+        n = has_l + (a1 - a0 + 1) + has_r;
+    }
+    __device__ uint32_t at(uint32_t k) const {
+        if (k < has_l) return cl;
+        k -= has_l;
+        return k <= a1 - a0 ? a0 + k : cr;
+    }
+};
+
+// A thread owns four consecutive input elements; with a contiguous input they leave as one vector.
+template <class T>
+__global__ __launch_bounds__(PB) void pad_edge_backward3_kernel(Pad3 sp, int mode, const T* __restrict__ go, T* __restrict__ gi, uint32_t n_in,
+                                                                 bool vec_store) {
+    constexpr uint32_t PER = 4;
+    const uint32_t i0 = (blockIdx.x * PB + threadIdx.x) * PER;
+    if (i0 >= n_in) return;
+    uint32_t p0, p1, p2, q;
+    fd_divmod(i0, sp.in_div[2], q, p2);
+    fd_divmod(q, sp.in_div[1], p0, p1);
+    EdgeSrc s0, s1;
+    int64_t row = 0;
+    bool fresh = true;
+    AVec<T, PER> v;
+    int64_t dst[PER];
+#pragma unroll
+    for (uint32_t e = 0; e < PER; ++e) {
+        if (i0 + e >= n_in) break;
+        if (fresh) {
+            s0.init(mode, p0, sp.in[0], sp.out[0], sp.before[0]);
+            s1.init(mode, p1, sp.in[1], sp.out[1], sp.before[1]);
+            row = (int64_t)p0 * sp.in_stride[0] + (int64_t)p1 * sp.in_stride[1];
+            fresh = false;
+        }
+        EdgeSrc s2;
+        s2.init(mode, p2, sp.in[2], sp.out[2], sp.before[2]);
+        float acc = 0.0f;
+        for (uint32_t k0 = 0; k0 < s0.n; ++k0) {
+            const uint32_t o0 = s0.at(k0) * sp.out_stride[0];
+            for (uint32_t k1 = 0; k1 < s1.n; ++k1) {
+                const uint32_t o1 = o0 + s1.at(k1) * sp.out_stride[1];
+                for (uint32_t k2 = 0; k2 < s2.n; ++k2) acc += Ar<T>::to_f32(go[o1 + s2.at(k2)]);
+            }
+        }
+        v.v[e] = Ar<T>::from_f32(acc);
+        dst[e] = row + (int64_t)p2 * sp.in_stride[2];
+        if (++p2 == sp.in[2]) {
+            p2 = 0;
+            fresh = true;
+            if (++p1 == sp.in[1]) { p1 = 0; ++p0; }
+        }
+    }
+    if (vec_store && i0 + PER <= n_in) {
+        *(AVec<T, PER>*)(gi + i0) = v;
+    } else {
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e)
+            if (i0 + e < n_in) gi[dst[e]] = v.v[e];
+    }
+}
+
 static bool edge_space(size_t nd_full, const size_t* md_full, int mode, PadSpace& sp, EdgeWalk& in_walk, size_t* in_off, const char* who) {
     if (nd_full > 64) { set_status(ERR_UNSUPPORTED, who); return false; }
     *in_off = md_full[2 * nd_full];
@@ -376,7 +633,12 @@ void pad_edge_forward(int mode, size_t n_in, size_t n_out, size_t nd, const size
     if (n_out >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "pad: output of 2^31 or more elements"); return; }
     PadSpace sp; EdgeWalk walk; size_t off;
     if (!edge_space(nd, md, mode, sp, walk, &off, "pad_with_reflection/replication: bad shape or rank above 8")) return;
-    hipLaunchKernelGGL(pad_edge_kernel<T>, dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, mode, in + off, out, n_out);
+    Pad3 p3;
+    if (simple_edge_shape(sp, mode) && make_pad3(sp, p3))
+        hipLaunchKernelGGL(pad_edge3_kernel<T>, dim3(cdiv(n_out, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, mode, in + off, out, (uint32_t)n_out,
+                           (uintptr_t)out % (4 * sizeof(T)) == 0);
+    else
+        hipLaunchKernelGGL(pad_edge_kernel<T>, dim3(cdiv(n_out, PB)), dim3(PB), 0, stream(), sp, mode, in + off, out, n_out);
     MXH_LAUNCH_CHECK("pad_edge");
 }
 
@@ -397,7 +659,12 @@ void pad_edge_backward(int mode, size_t n_in, size_t n_out, size_t nd, const siz
     size_t logical = 1;
     for (size_t d = 0; d < nd; ++d) logical *= md[d];
     if (logical == 0) return;
-    hipLaunchKernelGGL(pad_edge_backward_kernel<T>, dim3(cdiv(logical, PB)), dim3(PB), 0, stream(), sp, walk, mode, go, gi + off, logical);
+    Pad3 p3;
+    if (simple_edge_shape(sp, mode) && make_pad3(sp, p3))
+        hipLaunchKernelGGL(pad_edge_backward3_kernel<T>, dim3(cdiv(logical, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, mode, go, gi + off, (uint32_t)logical,
+                           cont && (uintptr_t)(gi + off) % (4 * sizeof(T)) == 0);
+    else
+        hipLaunchKernelGGL(pad_edge_backward_kernel<T>, dim3(cdiv(logical, PB)), dim3(PB), 0, stream(), sp, walk, mode, go, gi + off, logical);
     MXH_LAUNCH_CHECK("pad_edge_backward");
 }
 

@@ -168,6 +168,8 @@ def run(flt="", sets=4, random_grad=False, out=sys.stdout):
     timeit("col2im_f32/num_els = B*C*H*W (the layer's call)", lambda: lib.hip_conv2d_col2im_f32(n_in, md.ctypes.data, col, xin), 2 * n_in * 4)
     timeit("col2im_f32/whole column matrix", lambda: lib.hip_conv2d_col2im_f32(ncol, md.ctypes.data, col, xin), (n_in + ncol) * 4)
     mdp = u64([B, Ci, H, W], [Ci * H * W, H * W, W, 1], 0, [B, Ci, 58, 58], [0, 0, 0, 0, 1, 1, 1, 1])
+    # calibration: a plain copy that moves as many bytes as a pad at this size (launch and ramp included)
+    timeit("memcpy_d2d 26.6MB (as much as one pad)", lambda: lib.hip_memcpy_d2d(col, xin, (n_in + n_pad) * 2), (n_in + n_pad) * 4)
     timeit("pad_with_constant_f32/[32,64,56,56]+1", lambda: lib.hip_pad_with_constant_f32(n_in, n_pad, 4, mdp.ctypes.data, xin, col, 0.0), (n_in + n_pad) * 4)
     timeit("pad_with_constant_backward_f32/[32,64,56,56]+1", lambda: lib.hip_pad_with_constant_backward_f32(n_in, n_pad, 4, mdp.ctypes.data, col, xin), (n_in + n_pad) * 4)
     for mode in ("reflection", "replication"):
