@@ -2,7 +2,6 @@
 // cuda_malloc / cuda_free / cuda_memcpy_* / cuda_set_device / cuda_get_device family of
 // crates/maidenx_cuda/src/lib.rs:39-117.
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -228,7 +227,6 @@ int hip_graph_end_capture(void** graph_exec) {
     g_stream = g_saved_stream;
     g_capturing = false;
     const bool as_program = g_prog_ok && !g_prog_pending && !g_prog_cmds.empty();
-    if (getenv("MXH_DEBUG_PROGRAM")) fprintf(stderr, "[maidenx_hip] capture closed: %zu commands recorded, %s\n", g_prog_cmds.size(), as_program ? "program" : "HIP graph");
     if (e != hipSuccess) return (int)e;
     GraphExec* ge = new GraphExec();
     if (as_program) {
