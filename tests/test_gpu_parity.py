@@ -202,6 +202,31 @@ def test_pow_f32_ulp(oracle, hip):
         assert np.max(ulp_diff_f32(o, h)) <= 1, c
 
 
+def test_pow_square_is_the_correctly_rounded_product(oracle, hip):
+    """pow(x, 2) takes the product path: the correctly rounded square (what a double pow rounded once gives),
+    special values included; the oracle's powf may differ from it by one ulp at most."""
+    r = rng(23)
+    x = np.concatenate([r.standard_normal(4096).astype(np.float32) * np.float32(10.0) ** r.integers(-25, 20, 4096).astype(np.float32),
+                        np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-30, -1e-30, 1e-23, 3e19, -3e19, 1.8446744e19, 1e-45], np.float32)])
+    n = x.size
+    md = meta_unary([n], [1])
+    (o,), (h,) = both(oracle, hip, "pow_f32", lambda: (n, 1, md, In(x), const_arg(2.0, "f32"), Out(n, "f32")))
+    with np.errstate(all="ignore"):
+        want = x * x
+    assert np.array_equal(np.isnan(want), np.isnan(h))
+    ok = ~np.isnan(want)
+    assert np.array_equal(want[ok].view(np.uint32), h[ok].view(np.uint32))
+    fin = ok & np.isfinite(o)
+    assert np.max(ulp_diff_f32(o[fin], h[fin])) <= 1
+    for dt in ("bf16", "f16"):
+        bits = np.arange(1 << 16, dtype=np.uint16)
+        mdb = meta_unary([bits.size], [1])
+        (ob,), (hb,) = both(oracle, hip, f"pow_{dt}", lambda: (bits.size, 1, mdb, In(bits), const_arg(2.0, dt), Out(bits.size, dt)))
+        fo = to_float(ob, dt)
+        okb = ~np.isnan(fo)
+        assert np.array_equal(ob[okb], hb[okb]), dt
+
+
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
 @pytest.mark.parametrize("op", ["exp", "tanh", "gelu", "sigmoid"])
 def test_unary_transcendental_16bit(oracle, hip, op, dt):
