@@ -260,13 +260,13 @@ template <int WM_, int WN_, int MI_, int MJ_, int TS_ = 32> struct GemmCfg {
 template <class T> struct Cfgs {
     using Big = GemmCfg<4, 2, 2, 4>;
     using Small = GemmCfg<2, 2, 2, 2>;
-    using Tall = GemmCfg<4, 1, 2, 2>;     // 256 x 64: few output columns (the convolution GEMM has 64)
+    using Tall = GemmCfg<2, 2, 1, 1>;     // 64 x 64, four blocks per CU: few output columns or a short reduction (see gemm_dispatch)
 };
 #if MXH_GEMM_TS16
 template <> struct Cfgs<bf16_t> {
     using Big = GemmCfg<4, 2, 4, 8, 16>;
     using Small = GemmCfg<2, 2, 4, 4, 16>;
-    using Tall = GemmCfg<4, 1, 4, 4, 16>;
+    using Tall = GemmCfg<2, 2, 2, 2, 16>;     // 64 x 64 (the conv-shaped bf16 weight gradient: 49 us, 205 us with 256 x 64 tiles)
 };
 template <> struct Cfgs<f16_t> : Cfgs<bf16_t> {};
 #endif
@@ -315,19 +315,11 @@ __global__ __launch_bounds__(256) void gemm_fold_kernel(const float* __restrict_
     out[i] = Elem<T>::st(acc);
 }
 
-template <class T, bool XR, bool YR, class Cfg, bool FAST>
-__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
-    constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
-    constexpr bool SWZ = Cfg::TS == 16;
-    using SX = Stager<T, XR, TM, NT, SWZ>;
-    using SY = Stager<T, YR, TN, NT, SWZ>;
-    constexpr int VEC = Elem<T>::VEC;
-    constexpr int TK = SX::TK;
-    constexpr int PITCH = SX::PITCH;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    T* lds_x = (T*)smem;                                  // [2][TM*PITCH]
-    T* lds_y = lds_x + 2 * TM * PITCH;                    // [2][TN*PITCH]
-
+// Which tile, batch and reduction chunk a block works on.
+struct TilePos {
+    uint32_t ti, tj, b, split;
+};
+__device__ __forceinline__ TilePos tile_of_block(const GemmArgs& g) {
     // Blocks are handed to the 8 XCDs round robin, and each XCD has its own L2: give every XCD a compact
     // patch of the tile grid (GM tile rows x as many columns as it gets), so that the operand panels its
     // CUs stream are shared inside that L2 instead of being fetched by all eight.
@@ -338,10 +330,28 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     constexpr uint32_t GM = 4;
     const uint32_t group = v / (GM * g.tiles_j), in_group = v - group * (GM * g.tiles_j);
     const uint32_t first_i = group * GM, rows = g.tiles_i - first_i < GM ? g.tiles_i - first_i : GM;
-    uint32_t ti = first_i + in_group % rows;
-    uint32_t tj = in_group / rows;
-    uint32_t b = rest % g.batch;
-    const uint32_t split = rest / g.batch;
+    TilePos t;
+    t.ti = first_i + in_group % rows;
+    t.tj = in_group / rows;
+    t.b = rest % g.batch;
+    t.split = rest / g.batch;
+    return t;
+}
+
+// FAST: the tile lies inside the operands in all three extents and the wide accesses are aligned (no checks).
+template <class T, bool XR, bool YR, class Cfg, bool FAST>
+__device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem) {
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
+    constexpr bool SWZ = Cfg::TS == 16;
+    using SX = Stager<T, XR, TM, NT, SWZ>;
+    using SY = Stager<T, YR, TN, NT, SWZ>;
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int TK = SX::TK;
+    constexpr int PITCH = SX::PITCH;
+    T* lds_x = (T*)smem;                                  // [2][TM*PITCH]
+    T* lds_y = lds_x + 2 * TM * PITCH;                    // [2][TN*PITCH]
+
+    const uint32_t ti = pos.ti, tj = pos.tj, b = pos.b, split = pos.split;
     const uint32_t rb = split * g.r_chunk;                                  // this block reduces over [rb, re)
     const uint32_t re = g.R - rb < g.r_chunk ? g.R : rb + g.r_chunk;
     const uint32_t i0 = ti * TM, j0 = tj * TN;
@@ -491,6 +501,22 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     }
 }
 
+// ALIGNED: the operands allow the unchecked body wherever a whole tile lies inside them (the host has checked
+// alignment, strides and that the reduction is a whole number of k-tiles); blocks on a ragged edge, and every block
+// of an unaligned problem, take the checked body.
+template <class T, bool XR, bool YR, class Cfg, bool ALIGNED>
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const TilePos pos = tile_of_block(g);
+    if constexpr (ALIGNED) {
+        if ((pos.ti + 1) * Cfg::TM <= g.I && (pos.tj + 1) * Cfg::TN <= g.J) {
+            gemm_mfma_body<T, XR, YR, Cfg, true>(g, pos, smem);
+            return;
+        }
+    }
+    gemm_mfma_body<T, XR, YR, Cfg, false>(g, pos, smem);
+}
+
 template <class T, bool XR, bool YR, class Cfg, bool FAST>
 void launch_mfma_impl(GemmArgs g) {
     using SX = Stager<T, XR, Cfg::TM, Cfg::NT, Cfg::TS == 16>;
@@ -543,6 +569,7 @@ template <class T, bool XR, bool YR, class Cfg>
 void launch_mfma(GemmArgs g) {
     constexpr int VEC = Elem<T>::VEC, TK = TK_BYTES / sizeof(T);
     auto op_ok = [&](const void* p, int64_t s_batch, int64_t s_row, int64_t s_red, bool rcont) {
+        if (g.batch == 1) s_batch = 0;      // never applied
         if (rcont) return (uintptr_t)p % 16 == 0 && s_row % VEC == 0 && s_batch % VEC == 0;
         if (sizeof(T) == 2) return (uintptr_t)p % 4 == 0 && s_red % 2 == 0 && s_batch % 2 == 0;
         return true;
@@ -551,9 +578,9 @@ void launch_mfma(GemmArgs g) {
     auto span_ok = [&](int64_t s_row, int64_t s_red, int rows) {
         return s_row >= 0 && s_red >= 0 && ((int64_t)rows * s_row + (int64_t)TK * s_red) * (int64_t)sizeof(T) < (1ll << 31);
     };
-    bool fast = span_ok(g.xi, g.xr, Cfg::TM) && span_ok(g.yj, g.yr, Cfg::TN) &&
-                g.I % Cfg::TM == 0 && g.J % Cfg::TN == 0 && g.R % TK == 0 && op_ok(g.X, g.xb, g.xi, g.xr, XR) &&
-                op_ok(g.Y, g.yb, g.yj, g.yr, YR) && (uintptr_t)g.out % 16 == 0;
+    // (ragged tiles are decided per block inside the kernel)
+    bool fast = span_ok(g.xi, g.xr, Cfg::TM) && span_ok(g.yj, g.yr, Cfg::TN) && g.R % TK == 0 && g.J % 4 == 0 &&
+                op_ok(g.X, g.xb, g.xi, g.xr, XR) && op_ok(g.Y, g.yb, g.yj, g.yr, YR) && (uintptr_t)g.out % 16 == 0;
     if (fast) launch_mfma_impl<T, XR, YR, Cfg, true>(g);
     else launch_mfma_impl<T, XR, YR, Cfg, false>(g);
 }
@@ -619,8 +646,14 @@ void gemm_dispatch(GemmArgs g) {
     bool xi = g.xi == 1, yj = g.yj == 1;
     // 256x256 tiles when they fill the chip about as well as 128x128 ones would
     size_t big_blocks = (size_t)cdiv(g.I, 256) * cdiv(g.J, 256) * g.batch;
-    bool big = g.I >= 256 && g.J >= 256 && big_blocks >= 192;
-    const bool tall = !big && g.J <= 64 && g.I >= 1024;
+    // Few output columns, or a reduction of a few k-tiles (prologue and epilogue are then most of a block's life, and
+    // many small blocks overlap them): the 64-column tiles.  Measured on the convolution layer's f32 products
+    // [100352,576]x[576,64], [100352,64]x[64,576], [576,100352]x[100352,64]: 76 / 112 / 106 us with 64x64 tiles
+    // (four blocks per CU), 86 / 116 / 144 us with 128x64, 196 / 124 / 196 us with 128x128, 340 / 137 / 339 us with
+    // 256x256.
+    constexpr uint32_t TKE = TK_BYTES / sizeof(T);
+    bool tall = g.I >= 128 && (g.J <= 64 || g.R <= 4 * TKE);
+    bool big = !tall && g.I >= 256 && g.J >= 256 && big_blocks >= 192;
 #define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, typename Cfgs<T>::Big>(g) : tall ? launch_mfma<T, XR, YR, typename Cfgs<T>::Tall>(g) : launch_mfma<T, XR, YR, typename Cfgs<T>::Small>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
     else if (xr && yj) MXH_GEMM_CASE(true, false);
