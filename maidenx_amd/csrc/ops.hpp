@@ -138,9 +138,7 @@ MXH_UNC(OpMulScalar, T, A::mul(x, c))
 MXH_UNC(OpDivScalar, T, is_zero(c) ? (is_zero(x) ? A::zero() : A::inf()) : A::div(x, c))
 MXH_UNC(OpMaximumScalar, T, A::max_(x, c))
 MXH_UNC(OpMinimumScalar, T, A::min_(x, c))
-// x^2 (the square of MSE and variance): the product of two floats is exact in double, so rounding it once is
-// bit for bit what the double pow() path returns - without the 200-instruction pow.  The branch is uniform.
-MXH_UNC(OpPow, T, A::from_f32(F(c) == 2.0f ? F(x) * F(x) : m_pow(F(x), F(c))))
+MXH_UNC(OpPow, T, A::from_f32(m_pow(F(x), F(c))))                      // (the entry point sends an exponent of 2 to OpSquare)
 MXH_UNC(OpLeakyRelu, T, F(x) > 0.0f ? x : A::mul(c, x))
 MXH_UNC(OpElu, T, F(x) > 0.0f ? x : A::from_f32(F(c) * (m_exp(F(x)) - 1.0f)))
 MXH_UNC(OpEqScalar, bool_t, (bool_t)(F(x) == F(c)))

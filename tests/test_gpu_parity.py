@@ -218,13 +218,16 @@ def test_pow_square_is_the_correctly_rounded_product(oracle, hip):
     assert np.array_equal(want[ok].view(np.uint32), h[ok].view(np.uint32))
     fin = ok & np.isfinite(o)
     assert np.max(ulp_diff_f32(o[fin], h[fin])) <= 1
+    (h1,) = hip.call("pow_f32", n, 1, md, In(x), const_arg(1.0, "f32"), Out(n, "f32"))          # x^1 is x
+    assert np.array_equal(x[ok].view(np.uint32), h1[ok].view(np.uint32)) and np.array_equal(np.isnan(x), np.isnan(h1))
     for dt in ("bf16", "f16"):
         bits = np.arange(1 << 16, dtype=np.uint16)
         mdb = meta_unary([bits.size], [1])
-        (ob,), (hb,) = both(oracle, hip, f"pow_{dt}", lambda: (bits.size, 1, mdb, In(bits), const_arg(2.0, dt), Out(bits.size, dt)))
-        fo = to_float(ob, dt)
-        okb = ~np.isnan(fo)
-        assert np.array_equal(ob[okb], hb[okb]), dt
+        for c in (2.0, 1.0):
+            (ob,), (hb,) = both(oracle, hip, f"pow_{dt}", lambda: (bits.size, 1, mdb, In(bits), const_arg(c, dt), Out(bits.size, dt)))
+            fo = to_float(ob, dt)
+            okb = ~np.isnan(fo)
+            assert np.array_equal(ob[okb], hb[okb]), (dt, c)
 
 
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
