@@ -244,6 +244,16 @@ void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* 
                                     const size_t* src_layout, const I* index, const T* src, T* self);                  \
     void hip_bincount_weighted_##S##_##IS(size_t n, size_t stride, size_t offset, const I* input, size_t w_stride,     \
                                           size_t w_offset, const T* weights, size_t out_size, T* output);
+/* index_put_ (indexing.rs:182-311): `indices` (host array) fixes the leading dims of self, src is copied into the
+ * sub-tensor that remains (its shape must equal those dims); with every dim fixed a 0-d src is one element and any
+ * other src goes element by element behind indices[0] of a 1-d self.  A shape mismatch, an index out of bounds or a
+ * source that does not fit is an error status and nothing is written. */
+#define MX_DECL_INDEX_PUT(T, S)                                                                                            \
+    void hip_index_put_##S(size_t self_num_dims, const size_t* self_layout, size_t num_indices, const size_t* indices,     \
+                           size_t src_num_dims, const size_t* src_layout, const T* src, T* self);
+MX_DECL_INDEX_PUT(float, f32)
+MX_DECL_INDEX_PUT(mx_bf16, bf16)
+MX_DECL_INDEX_PUT(mx_f16, f16)
 MX_DECL_INDEX(float, f32, int32_t, i32)
 MX_DECL_INDEX(float, f32, int64_t, i64)
 MX_DECL_INDEX(mx_bf16, bf16, int32_t, i32)

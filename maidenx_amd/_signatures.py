@@ -60,6 +60,7 @@ def index_signatures(dtypes=("f32", "bf16", "f16")):
             sig[f"index_add_{dt}_{it}"] = [SZ, SZ, P, P, SZ, SZ, SZ, P, P, P]
             sig[f"scatter_add_{dt}_{it}"] = [SZ, SZ, P, P, P, P, P, P]
             sig[f"bincount_weighted_{dt}_{it}"] = [SZ, SZ, SZ, P, SZ, SZ, P, SZ, P]
+        sig[f"index_put_{dt}"] = [SZ, P, SZ, P, SZ, P, P, P]
     for it in ("i32", "i64"):
         sig[f"bincount_{it}"] = [SZ, SZ, SZ, P, SZ, P]
     return sig

@@ -20,6 +20,7 @@
 
 #include <rocprim/rocprim.hpp>
 
+#include "elementwise.hpp"
 #include "mxh.hpp"
 #include "ops.hpp"
 
@@ -438,9 +439,68 @@ void bincount_weighted(size_t n, size_t stride, size_t offset, const I* input, s
     MXH_LAUNCH_CHECK("bincount_weighted");
 }
 
+// ---- index_put_ (tensor/ops/indexing.rs:182-311) ---------------------------------------------------------
+// `indices` fixes the leading dims of self; src (whose shape must equal self's remaining dims) is copied into that
+// sub-tensor through the strides of both.  With every dim fixed, a 0-d src is one element written at that
+// position, and any other src is written element by element (read with its stride 0 only, as the reference does)
+// to positions indices[0], indices[0] + 1, ... of a 1-d self.  The copy is the in-place elementwise path with an
+// "assign" functor.  Positions of self that alias each other (stride 0) are written in no particular order.
+template <class T>
+void index_put(size_t self_nd, const size_t* self_layout, size_t n_indices, const size_t* indices, size_t src_nd,
+               const size_t* src_layout, const T* src, T* self) {
+    if (!self_layout || !src_layout || !src || !self || (n_indices && !indices)) { set_status(ERR_INVALID, "index_put_: null argument"); return; }
+    if (self_nd > 64 || src_nd > 64) { set_status(ERR_INVALID, "index_put_: rank above 64"); return; }
+    if (n_indices > self_nd) { set_status(ERR_INVALID, "index_put_: more indices than dims"); return; }
+    const size_t *sd = self_layout, *ss = self_layout + self_nd, *rd = src_layout, *rs = src_layout + src_nd;
+    const size_t self_off = self_layout[2 * self_nd], src_off = src_layout[2 * src_nd];
+    const size_t remaining = self_nd - n_indices;
+    size_t md[3 * 64 + 2];
+    size_t nd = 0, num_els = 1, base = self_off;
+    if (remaining > 0) {
+        if (src_nd != remaining) { set_status(ERR_INVALID, "index_put_: source rank differs from the remaining dims"); return; }
+        for (size_t i = 0; i < remaining; ++i)
+            if (rd[i] != sd[n_indices + i]) { set_status(ERR_INVALID, "index_put_: source shape differs from the remaining dims"); return; }
+        for (size_t d = 0; d < n_indices; ++d) {
+            if (indices[d] >= sd[d]) { set_status(ERR_INVALID, "index_put_: index out of bounds"); return; }
+            base += indices[d] * ss[d];
+        }
+        nd = remaining;
+        for (size_t i = 0; i < nd; ++i) { md[i] = rd[i]; md[nd + i] = ss[n_indices + i]; md[2 * nd + i] = rs[i]; num_els *= rd[i]; }
+    } else if (src_nd == 0) {
+        for (size_t d = 0; d < n_indices; ++d) {
+            if (indices[d] >= sd[d]) { set_status(ERR_INVALID, "index_put_: index out of bounds"); return; }
+            base += indices[d] * ss[d];
+        }
+        nd = 1; md[0] = 1; md[1] = 1; md[2] = 1;
+    } else {
+        size_t src_size = 1, self_size = 1;
+        for (size_t i = 0; i < src_nd; ++i) src_size *= rd[i];
+        for (size_t i = 0; i < self_nd; ++i) self_size *= sd[i];
+        if (src_size == 0) return;
+        if (self_nd == 0) { set_status(ERR_INVALID, "index_put_: no index for a non-scalar source"); return; }
+        if (indices[0] + src_size > self_size) { set_status(ERR_INVALID, "index_put_: source does not fit behind the index"); return; }
+        if (self_nd != 1) { set_status(ERR_INVALID, "index_put_: a flat copy needs a 1-d destination"); return; }
+        base += indices[0] * ss[0];
+        nd = 1; md[0] = src_size; md[1] = ss[0]; md[2] = rs[0]; num_els = src_size;
+    }
+    if (num_els == 0) return;
+    md[3 * nd] = base;
+    md[3 * nd + 1] = src_off;
+    ew_binary(num_els, nd, md, self, src, nullptr, OpAssign<T>{}, true);
+}
+
 }  // namespace mxh
 
 using namespace mxh;
+
+#define MXH_INDEX_PUT_FOR(T, TS)                                                                                                    \
+    extern "C" void hip_index_put_##TS(size_t self_nd, const size_t* self_layout, size_t n_indices, const size_t* indices,          \
+                                       size_t src_nd, const size_t* src_layout, const T* src, T* self) {                            \
+        index_put<T>(self_nd, self_layout, n_indices, indices, src_nd, src_layout, src, self);                                      \
+    }
+MXH_INDEX_PUT_FOR(float, f32)
+MXH_INDEX_PUT_FOR(bf16_t, bf16)
+MXH_INDEX_PUT_FOR(f16_t, f16)
 
 #define MXH_INDEX_FOR(T, TS, I, IS)                                                                                                  \
     extern "C" void hip_index_select_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride,    \

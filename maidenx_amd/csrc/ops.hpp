@@ -158,6 +158,11 @@ template <class T> struct OpIdentity {
     using In = T; using Out = T; static constexpr int NIN = 1;
     __device__ T operator()(T x) const { return x; }
 };
+// lhs = rhs through the in-place path (index_put_): the old value is not used
+template <class T> struct OpAssign {
+    using In = T; using Out = T; static constexpr int NIN = 2;
+    __device__ T operator()(T, T b) const { return b; }
+};
 // `0 + x`: what a sum_to_shape that keeps every dim does through its zero-initialised cells (-0 -> +0).
 // The 16-bit forms live with the reductions, whose rounding helpers they use.
 template <class T> struct OpZeroPlus;

@@ -1,5 +1,5 @@
 // TEST INFRASTRUCTURE ONLY — CPU restatement of the host loops of crates/maidenx_tensor/src/ops/indexing.rs
-// (index_select :93-124, index_add_ :15-91, gather :315-363, scatter_add_ :403-461, bincount :463-522) and
+// (index_select :93-124, index_add_ :15-91, index_put_ :182-311, gather :315-363, scatter_add_ :403-461, bincount :463-522) and
 // of add_at_index (crates/maidenx_tensor/src/utils/indexing.rs:96-140): indices are read `as_i32`, the
 // adds are in the storage dtype, elements are visited in the order the reference's loops visit them.
 // A layout is dims[n] | strides[n] | offset.  On an index outside its range the reference returns an
@@ -148,6 +148,56 @@ void bincount_weighted(size_t n, size_t stride, size_t offset, const I* input, s
 
 }  // namespace
 
+// indexing.rs:182-311 with set_index (utils/indexing.rs:67-94).  The checks come in the reference's order; the copy of
+// a sub-tensor is its recursion over the source dims (row-major), every dim fixed means one element (0-d source) or
+// the element-by-element writes behind indices[0] that only a 1-d self accepts.
+template <typename T>
+void index_put(size_t self_nd, const size_t* self_layout, size_t n_indices, const size_t* indices, size_t src_nd, const size_t* src_layout,
+               const T* src, T* self) {
+    Layout sl(self_nd, self_layout), rl(src_nd, src_layout);
+    if (n_indices > self_nd) { g_index_error = 1; return; }
+    const size_t remaining = self_nd - n_indices;
+    if (remaining > 0) {
+        if (src_nd != remaining) { g_index_error = 1; return; }
+        for (size_t i = 0; i < remaining; ++i)
+            if (rl.dims[i] != sl.dims[n_indices + i]) { g_index_error = 1; return; }
+        size_t base = 0;
+        for (size_t d = 0; d < n_indices; ++d) {
+            if (indices[d] >= sl.dims[d]) { g_index_error = 1; return; }
+            base += indices[d] * sl.strides[d];
+        }
+        base += sl.offset;
+        walk(src_nd, rl.dims, [&](const size_t* c) {
+            size_t dst = base, from = rl.offset;
+            for (size_t d = 0; d < src_nd; ++d) { dst += c[d] * sl.strides[n_indices + d]; from += c[d] * rl.strides[d]; }
+            self[dst] = src[from];
+            return true;
+        });
+        return;
+    }
+    auto set_index = [&](const size_t* idx, size_t n, T v) {
+        if (n != self_nd) { g_index_error = 1; return false; }
+        for (size_t d = 0; d < n; ++d)
+            if (idx[d] >= sl.dims[d]) { g_index_error = 1; return false; }
+        size_t flat = sl.offset;
+        for (size_t d = 0; d < n; ++d) flat += idx[d] * sl.strides[d];
+        self[flat] = v;
+        return true;
+    };
+    if (src_nd == 0) { set_index(indices, n_indices, src[rl.offset]); return; }
+    size_t src_size = 1, self_size = 1;
+    for (size_t i = 0; i < src_nd; ++i) src_size *= rl.dims[i];
+    for (size_t i = 0; i < self_nd; ++i) self_size *= sl.dims[i];
+    if (src_size == 0) return;
+    if (n_indices == 0) { g_index_error = 1; return; }          // indices[0] of an empty slice: a panic in the reference
+    const size_t self_dim = indices[0];
+    if (self_dim + src_size > self_size) { g_index_error = 1; return; }
+    for (size_t i = 0; i < src_size; ++i) {
+        size_t one = self_dim + i;
+        if (!set_index(&one, 1, src[rl.offset + i * rl.strides[0]])) return;
+    }
+}
+
 extern "C" int oracle_index_error() { int e = g_index_error; g_index_error = 0; return e; }
 
 #define ORC_INDEX_FOR(T, TS, I, IS)                                                                                                  \
@@ -181,6 +231,16 @@ ORC_INDEX_FOR(bf16, bf16, int32_t, i32)
 ORC_INDEX_FOR(f16, f16, int32_t, i32)
 ORC_INDEX_FOR(bf16, bf16, int64_t, i64)
 ORC_INDEX_FOR(f16, f16, int64_t, i64)
+
+#define ORC_INDEX_PUT_FOR(T, TS)                                                                                                     \
+    extern "C" void oracle_index_put_##TS(size_t self_nd, const size_t* self_layout, size_t n_indices, const size_t* indices,        \
+                                          size_t src_nd, const size_t* src_layout, const T* src, T* self) {                         \
+        index_put<T>(self_nd, self_layout, n_indices, indices, src_nd, src_layout, src, self);                                       \
+    }
+ORC_INDEX_PUT_FOR(float, f32)
+ORC_INDEX_PUT_FOR(double, f64)
+ORC_INDEX_PUT_FOR(bf16, bf16)
+ORC_INDEX_PUT_FOR(f16, f16)
 
 extern "C" void oracle_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output) {
     bincount<int32_t>(n, stride, offset, input, out_size, output);

@@ -236,6 +236,13 @@ def run_index(be, dt):
                 (out,) = be.call(f"scatter_add_{dt}_{it}", len(shape), c["dim"], layout(shape, off=1), layout(ishape, off=1),
                                  layout(ishape, off=1), In(idx), In(padded(c["src"], dt)), InOut(padded(c["self"], dt)))
                 check(out[1:-1], c["expect"], dt, 0)
+            elif op == "index_put":
+                if it == "i64":
+                    continue                      # no index tensor: once is enough
+                shape, sshape = c["self_shape"], c["src_shape"]
+                (out,) = be.call(f"index_put_{dt}", len(shape), layout(shape, off=1), len(c["indices"]), np.array(c["indices"], dtype=np.uint64),
+                                 len(sshape), layout(sshape, off=1), In(padded(c["src"], dt)), InOut(padded(c["self"], dt)))
+                check(out[1:-1], c["expect"], dt, 0)
             elif op == "bincount":
                 idx = np.array([0] + c["input"], dtype=ity)
                 (out,) = be.call(f"bincount_{it}", len(c["input"]), 1, 1, In(idx), c["out_size"], Out(c["out_size"], it))

@@ -753,6 +753,55 @@ def test_bincount(oracle, hip):
             assert same_bits(o, h)
 
 
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape,n_fixed", [([6], 0), ([40, 50], 1), ([3, 40, 50], 1), ([3, 4, 5], 2), ([2, 3, 4, 5], 3), ([64, 1024], 1), ([8, 256, 256], 1)])
+def test_index_put(oracle, hip, shape, n_fixed, dt):
+    """Sub-tensor assignment, contiguous and through permuted views of both tensors, and the single-element and flat-copy
+    forms; every byte of self equals the oracle's, written or not."""
+    r = rng(163)
+    n = int(np.prod(shape))
+    x = to_storage(r.standard_normal(n + 2).astype(np.float32), dt)
+    fixed = [int(r.integers(0, shape[d])) for d in range(n_fixed)]
+    rest = shape[n_fixed:]
+    m = int(np.prod(rest))
+    src = to_storage(r.standard_normal(m + 3).astype(np.float32), dt)
+    idx = np.array(fixed + [0], dtype=np.uint64)
+    (o,), (h,) = both(oracle, hip, f"index_put_{dt}", lambda: (len(shape), layout(shape, off=2), n_fixed, idx, len(rest), layout(rest, off=3), In(src), InOut(x.copy())))
+    assert same_bits(o, h) and not same_bits(h, x)
+    if len(rest) >= 2:
+        st = contiguous_strides(shape[:-2] + [shape[-1], shape[-2]])
+        st[-1], st[-2] = st[-2], st[-1]
+        sst = contiguous_strides(rest[:-2] + [rest[-1], rest[-2]])
+        sst[-1], sst[-2] = sst[-2], sst[-1]
+        (o,), (h,) = both(oracle, hip, f"index_put_{dt}", lambda: (len(shape), layout(shape, st, off=2), n_fixed, idx, len(rest), layout(rest, sst, off=3), In(src), InOut(x.copy())))
+        assert same_bits(o, h) and not same_bits(h, x)
+    full = np.array([int(r.integers(0, s)) for s in shape], dtype=np.uint64)
+    (o,), (h,) = both(oracle, hip, f"index_put_{dt}", lambda: (len(shape), layout(shape, off=2), len(shape), full, 0, np.array([1], dtype=np.uint64), In(src), InOut(x.copy())))
+    assert same_bits(o, h)
+    if len(shape) == 1:
+        (o,), (h,) = both(oracle, hip, f"index_put_{dt}", lambda: (1, layout(shape, off=2), 1, np.array([2], dtype=np.uint64), 1, layout([2], [2], off=1), In(src), InOut(x.copy())))
+        assert same_bits(o, h) and not same_bits(h, x)
+
+
+def test_index_put_errors_write_nothing(hip):
+    import maidenx_amd.lib as L
+    L.check()
+    x = np.arange(10, dtype=np.float32)
+    cases = [
+        ("does not fit", (1, layout([10]), 1, np.array([8], dtype=np.uint64), 1, layout([3]))),
+        ("more indices than dims", (1, layout([10]), 2, np.array([1, 1], dtype=np.uint64), 0, layout([]))),
+        ("out of bounds", (2, layout([2, 5]), 1, np.array([2], dtype=np.uint64), 1, layout([5]))),
+        ("shape differs", (2, layout([2, 5]), 1, np.array([1], dtype=np.uint64), 1, layout([4]))),
+        ("1-d destination", (2, layout([2, 5]), 2, np.array([1, 1], dtype=np.uint64), 1, layout([2]))),
+    ]
+    for what, args in cases:
+        buf = InOut(x.copy())
+        with pytest.raises(L.HipError, match=what):
+            hip.call("index_put_f32", *args, In(np.ones(5, np.float32)), buf)
+    (h,) = hip.call("index_put_f32", 1, layout([10]), 1, np.array([7], dtype=np.uint64), 1, layout([3]), In(np.ones(5, np.float32)), InOut(x.copy()))
+    assert h.tolist() == [0, 1, 2, 3, 4, 5, 6, 1, 1, 1]
+
+
 def test_index_out_of_bounds_is_reported(hip):
     import maidenx_amd.lib as L
     L.check()

@@ -373,6 +373,63 @@ def test_oracle_softmax_bf16_rounds_every_step(oracle):
     assert np.array_equal(y, want)
 
 
+# ---- index_put_: numpy's sub-tensor assignment ------------------------------------------------------------------
+@pytest.mark.parametrize("shape,n_fixed", [([6], 0), ([4, 5], 1), ([3, 4, 5], 1), ([3, 4, 5], 2), ([2, 3, 4, 5], 3)])
+def test_oracle_index_put_vs_numpy(oracle, shape, n_fixed):
+    r = rng(401)
+    x = r.standard_normal(shape)
+    fixed = [int(r.integers(0, shape[d])) for d in range(n_fixed)]
+    rest = shape[n_fixed:]
+    src = r.standard_normal(rest)
+    # contiguous
+    (y,) = oracle.call("index_put_f64", len(shape), layout(shape), n_fixed, np.array(fixed + [0], dtype=np.uint64), len(rest), layout(rest),
+                       In(src.ravel()), InOut(x.ravel().copy()))
+    want = x.copy()
+    want[tuple(fixed)] = src
+    assert np.array_equal(y.reshape(shape), want) and oracle.lib.oracle_index_error() == 0
+    # permuted self and source, offsets
+    if len(shape) >= 2 and len(rest) >= 2:
+        xt = np.ascontiguousarray(np.moveaxis(x, -1, -2))                 # memory of a tensor whose last two dims are swapped
+        st = contiguous_strides(list(xt.shape))
+        st[-1], st[-2] = st[-2], st[-1]
+        srct = np.ascontiguousarray(np.moveaxis(src, -1, -2))
+        sst = contiguous_strides(list(srct.shape))
+        sst[-1], sst[-2] = sst[-2], sst[-1]
+        (y2,) = oracle.call("index_put_f64", len(shape), layout(shape, st, off=2), n_fixed, np.array(fixed + [0], dtype=np.uint64), len(rest),
+                            layout(rest, sst, off=3), In(np.concatenate([[7.0] * 3, srct.ravel()])), InOut(np.concatenate([[5.0] * 2, xt.ravel()])))
+        assert np.array_equal(np.moveaxis(y2[2:].reshape(xt.shape), -1, -2), want) and y2[0] == 5.0
+    # every dim fixed: one element from a 0-d source
+    full = [int(r.integers(0, s)) for s in shape]
+    (y3,) = oracle.call("index_put_f64", len(shape), layout(shape), len(shape), np.array(full, dtype=np.uint64), 0, np.array([4], dtype=np.uint64),
+                        In(np.arange(6.0)), InOut(x.ravel().copy()))
+    want3 = x.copy()
+    want3[tuple(full)] = 4.0
+    assert np.array_equal(y3.reshape(shape), want3)
+
+
+def test_oracle_index_put_flat_copy_and_errors(oracle):
+    x = np.arange(10.0)
+    # 1-d self, every dim fixed, 1-d source: copied behind the index, the source read with its stride
+    (y,) = oracle.call("index_put_f64", 1, layout([10], [1]), 1, np.array([4], dtype=np.uint64), 1, layout([3], [2]), In(np.arange(100.0, 106.0)),
+                       InOut(x.copy()))
+    assert y.tolist() == [0, 1, 2, 3, 100, 102, 104, 7, 8, 9]
+    def err(*args):
+        (out,) = oracle.call("index_put_f64", *args)
+        e = oracle.lib.oracle_index_error()
+        return e, out
+    same = lambda out: np.array_equal(out, x)
+    e, out = err(1, layout([10]), 1, np.array([8], dtype=np.uint64), 1, layout([3]), In(np.ones(3)), InOut(x.copy()))       # does not fit
+    assert e == 1 and same(out)
+    e, out = err(1, layout([10]), 2, np.array([1, 1], dtype=np.uint64), 0, layout([]), In(np.ones(1)), InOut(x.copy()))     # more indices than dims
+    assert e == 1 and same(out)
+    e, out = err(2, layout([2, 5]), 1, np.array([2], dtype=np.uint64), 1, layout([5]), In(np.ones(5)), InOut(x.copy()))     # index out of bounds
+    assert e == 1 and same(out)
+    e, out = err(2, layout([2, 5]), 1, np.array([1], dtype=np.uint64), 1, layout([4]), In(np.ones(4)), InOut(x.copy()))     # shape mismatch
+    assert e == 1 and same(out)
+    e, out = err(2, layout([2, 5]), 2, np.array([1, 1], dtype=np.uint64), 1, layout([2]), In(np.ones(2)), InOut(x.copy()))  # flat copy into a 2-d self
+    assert e == 1 and same(out)
+
+
 # ---- index ops: numpy's own take / take_along_axis / add.at / bincount -------------------------------------
 from helpers import layout  # noqa: E402
 
