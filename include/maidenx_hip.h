@@ -244,6 +244,20 @@ void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* 
                                     const size_t* src_layout, const I* index, const T* src, T* self);                  \
     void hip_bincount_weighted_##S##_##IS(size_t n, size_t stride, size_t offset, const I* input, size_t w_stride,     \
                                           size_t w_offset, const T* weights, size_t out_size, T* output);
+/* ---- fused Adam step --------------------------------------------------------------------------------
+ * No backend symbol exists for this in the reference: crates/maidenx_nn/src/optimizers/adam.rs:46-86 updates a
+ * parameter with fourteen tensor ops (mul_scalar, add, square, div_scalar, sqrt, add_scalar, div, sub_).  One call
+ * here applies the same element functions in the same order to contiguous param / grad / m / v of n elements and
+ * leaves exactly the bits that sequence leaves in param, m and v.  The scalars are the ones the reference passes to
+ * its *_scalar ops, in the tensor's dtype: beta1, 1-beta1, beta2, 1-beta2, the two bias terms 1-beta^(t+1) that m
+ * and v are divided by, epsilon, and lr_t = lr*sqrt(bias2)/bias1. */
+#define MX_DECL_ADAM(T, S)                                                                                                 \
+    void hip_adam_step_##S(size_t n, T* param, const T* grad, T* m, T* v, T beta1, T one_minus_beta1, T beta2,              \
+                           T one_minus_beta2, T bias1, T bias2, T epsilon, T lr_t);
+MX_DECL_ADAM(float, f32)
+MX_DECL_ADAM(mx_bf16, bf16)
+MX_DECL_ADAM(mx_f16, f16)
+
 /* index_put_ (indexing.rs:182-311): `indices` (host array) fixes the leading dims of self, src is copied into the
  * sub-tensor that remains (its shape must equal those dims); with every dim fixed a 0-d src is one element and any
  * other src goes element by element behind indices[0] of a 1-d self.  A shape mismatch, an index out of bounds or a

@@ -97,6 +97,13 @@ void mxt_module_release(mxt_module m);
 mxt_tensor mxt_mse_loss(mxt_tensor pred, mxt_tensor target);
 int mxt_sgd_step(mxt_module m, float lr);
 int mxt_sgd_zero_grad(mxt_module m);
+/* optimizers/adam.rs:16-99 with f64 hyper-parameters; the moments live in the optimizer object, one pair per
+ * parameter of the module it is first stepped with.  On the HIP build a contiguous f32 parameter is updated by one
+ * hip_adam_step_f32 call instead of the reference's fourteen ops (same bits); mxt_adam_set_fused(opt, 0) keeps the ops. */
+void* mxt_adam_new(double lr, double beta1, double beta2, double epsilon);
+void mxt_adam_release(void* opt);
+void mxt_adam_set_fused(void* opt, int enabled);
+int mxt_adam_step(void* opt, mxt_module m);
 
 /* The loop of examples/device/cpu.rs:32-38 (forward, MSE, backward, SGD step, zero_grad), `epochs` times,
  * without leaving native code.  losses (may be NULL) receives the loss of every epoch; reading it costs one

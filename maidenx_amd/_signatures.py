@@ -73,6 +73,7 @@ def extension_signatures():
         sig[f"fill_{dt}"] = [SZ, P, CONST[dt]]
     for dt in ("f32", "bf16", "f16"):
         sig[f"copy_strided_{dt}"] = [SZ, SZ, P, P, P]
+        sig[f"adam_step_{dt}"] = [SZ, P, P, P, P] + [CONST[dt]] * 8
     for a, b in (("bool", "f32"), ("bool", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "bool"), ("bf16", "bool"),
                  ("bool", "f16"), ("f32", "f16"), ("f16", "f32"), ("f16", "bool")):
         sig[f"cast_{a}_{b}"] = [SZ, P, P]

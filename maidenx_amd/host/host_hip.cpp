@@ -20,6 +20,7 @@ struct HipBackend {
                                               std::string("HIP backend: ") + hip_status_string());
     }
     static constexpr bool has_graphs = true;
+    static constexpr bool has_fused_adam = true;
     static void graph_begin() { if (hip_graph_begin_capture() != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_begin_capture failed"); }
     static void graph_end(void** exec) { if (hip_graph_end_capture(exec) != 0) { *exec = nullptr; throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_end_capture failed"); } }
     static void graph_launch(void* exec) { if (hip_graph_launch(exec) != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_launch failed"); }
@@ -41,13 +42,14 @@ struct HipBackend {
         using Red = void (*)(size_t, size_t, size_t, const size_t*, const E*, E*);                                       \
         static constexpr Bin bin[4] = {&hip_add_##S, &hip_sub_##S, &hip_mul_##S, &hip_div_##S};                          \
         static constexpr Inp inplace[2] = {&hip_add_inplace_##S, &hip_sub_inplace_##S};                                  \
-        static constexpr Un un[6] = {&hip_neg_##S, &hip_square_##S, &hip_relu_##S, &hip_tanh_##S, &hip_gelu_##S, &hip_exp_##S}; \
+        static constexpr Un un[7] = {&hip_neg_##S, &hip_square_##S, &hip_relu_##S, &hip_tanh_##S, &hip_gelu_##S, &hip_exp_##S, &hip_sqrt_##S}; \
         static constexpr Unc unc[4] = {&hip_add_scalar_##S, &hip_mul_scalar_##S, &hip_div_scalar_##S, &hip_pow_##S};      \
         static constexpr Red red[2] = {&hip_sum_##S, &hip_mean_##S};                                                     \
         static constexpr auto gt_scalar = &hip_gt_scalar_##S;                                                            \
         static constexpr auto sum_to_shape = &hip_sum_to_shape_##S;                                                      \
         static constexpr auto matmul = &hip_matmul_##S;                                                                  \
         static constexpr auto matmul_backward = &hip_matmul_backward_##S;                                                \
+        static constexpr auto adam_step = &hip_adam_step_##S;                                                            \
         /* host-side steps of the reference, done on the device */                                                       \
         static void fill(size_t n, E* p, E v) { if (n) hip_fill_##S(n, p, v); }                                          \
         static void cast_from_bool(size_t n, const uint8_t* in, E* out) { if (n) hip_cast_bool_##S(n, in, out); }        \

@@ -142,6 +142,7 @@ mxt_tensor mxt_unary(const char* op, mxt_tensor a) {
     return guard_t([&]() -> T {
         T& x = ref(a);
         if (is(op, "neg")) return x.neg();
+        if (is(op, "sqrt")) return x.sqrt();
         if (is(op, "square")) return x.square();
         if (is(op, "relu")) return x.relu();
         if (is(op, "tanh")) return x.tanh();
@@ -244,6 +245,11 @@ mxt_tensor mxt_mse_loss(mxt_tensor pred, mxt_tensor target) {
 }
 int mxt_sgd_step(mxt_module m, float lr) { return guard_i([&] { mxt::SGD<B>(lr).step(((Module*)m)->parameters()); }); }
 int mxt_sgd_zero_grad(mxt_module m) { return guard_i([&] { mxt::SGD<B>(0.0f).zero_grad(((Module*)m)->parameters()); }); }
+
+void* mxt_adam_new(double lr, double beta1, double beta2, double epsilon) { return new mxt::Adam<B>(lr, beta1, beta2, epsilon); }
+void mxt_adam_release(void* opt) { delete (mxt::Adam<B>*)opt; }
+void mxt_adam_set_fused(void* opt, int enabled) { ((mxt::Adam<B>*)opt)->fused = enabled != 0; }
+int mxt_adam_step(void* opt, mxt_module m) { return guard_i([&] { ((mxt::Adam<B>*)opt)->step(((Module*)m)->parameters()); }); }
 
 int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_t epochs, float* losses) {
     return guard_i([&] { g_replayed = mxt::train_loop<B>(*(Module*)m, ref(input), ref(target), lr, epochs, losses, g_graphs); });

@@ -141,7 +141,7 @@ void by_dtype(DType dt, const char* what, F&& f) {
 }
 enum BinOp { ADD, SUB, MUL, DIV };
 enum InplaceOp { ADD_INPLACE, SUB_INPLACE };
-enum UnOp { NEG, SQUARE, RELU, TANH, GELU, EXP };
+enum UnOp { NEG, SQUARE, RELU, TANH, GELU, EXP, SQRT };
 enum UncOp { ADD_SCALAR, MUL_SCALAR, DIV_SCALAR, POW };
 enum RedOp { SUM, MEAN };
 // a float scalar with an integer value keeps the tensor's dtype, any other promotes it to f32
@@ -576,6 +576,18 @@ struct Tensor {
             T input = *this;
             result.set_node("square", {*this}, [input](const std::vector<T>&, const T& go) {
                 return std::vector<T>{go.mul_scalar(2.0f).mul(input)};
+            });
+        }
+        return result;
+    }
+    T sqrt() const {                                                                // ops/unary.rs:149-184
+        if (!is_float(dtype)) throw Error(ErrKind::UnsupportedDType, "sqrt: needs a float tensor");
+        T result = unary_forward(SQRT);
+        if (requires_grad) {
+            result.with_grad();
+            T output = result;
+            result.set_node("sqrt", {*this}, [output](const std::vector<T>&, const T& go) {
+                return std::vector<T>{go.div(output.mul_scalar(2.0f))};
             });
         }
         return result;
@@ -1171,6 +1183,58 @@ struct SGD {                                                                    
     void step(const std::vector<Tensor<B>*>& params) const {
         for (Tensor<B>* p : params)
             if (p->has_grad()) p->sub_(p->grad().mul_scalar(lr));
+    }
+    void zero_grad(const std::vector<Tensor<B>*>& params) const {
+        for (Tensor<B>* p : params) p->zero_grad();
+    }
+};
+
+// nn/optimizers/adam.rs:6-99.  The hyper-parameters are f64 scalars (what the reference's `Adam::new(0.001, 0.9,
+// 0.999, 1e-8)` builds from literals), so the step's scalar arithmetic is f64 and every tensor op receives the
+// value rounded to the tensor's dtype.  The bias terms use beta^(t+1): the reference's loop multiplies t times
+// starting from beta (:56-61).  With a backend that has the fused kernel, a contiguous f32 parameter takes one
+// call instead of the fourteen ops; the results are the same bits (the moments are then updated in place).
+template <class B>
+struct Adam {
+    double lr, beta1, beta2, eps;
+    size_t t = 0;
+    bool fused = true;
+    std::vector<Tensor<B>> m, v;
+    Adam(double lr_, double b1, double b2, double eps_) : lr(lr_), beta1(b1), beta2(b2), eps(eps_) {}
+    void step(const std::vector<Tensor<B>*>& params) {
+        using T = Tensor<B>;
+        if (m.empty() || v.empty()) {
+            m.clear();
+            v.clear();
+            for (T* p : params) { m.push_back(T::zeros_like(*p)); v.push_back(T::zeros_like(*p)); }
+        }
+        if (m.size() != params.size()) throw Error(ErrKind::InvalidArgument, "Adam: the parameter list changed");
+        ++t;
+        for (size_t i = 0; i < params.size(); ++i) {
+            T* p = params[i];
+            if (!p->has_grad()) continue;
+            T grad = p->grad();
+            double b1t = beta1, b2t = beta2;
+            for (size_t k = 0; k < t; ++k) { b1t = b1t * beta1; b2t = b2t * beta2; }
+            const double c1 = 1.0 - b1t, c2 = 1.0 - b2t, lr_t = lr * std::sqrt(c2) / c1;
+            const double omb1 = 1.0 - beta1, omb2 = 1.0 - beta2;
+            if constexpr (B::has_fused_adam) {
+                auto plain = [](const T& x) { return x.dtype == DType::F32 && x.is_contiguous(); };
+                if (fused && plain(*p) && plain(grad) && plain(m[i]) && plain(v[i]) && grad.size() == p->size()) {
+                    B::template K<float>::adam_step(p->size(), p->template p<float>(), grad.template p<float>(), m[i].template p<float>(),
+                                                    v[i].template p<float>(), (float)beta1, (float)omb1, (float)beta2, (float)omb2, (float)c1,
+                                                    (float)c2, (float)eps, (float)lr_t);
+                    ++backend_calls();
+                    B::check();
+                    continue;
+                }
+            }
+            m[i] = m[i].mul_scalar((float)beta1).add(grad.mul_scalar((float)omb1));
+            v[i] = v[i].mul_scalar((float)beta2).add(grad.square().mul_scalar((float)omb2));
+            T m_hat = m[i].div_scalar((float)c1), v_hat = v[i].div_scalar((float)c2);
+            T step = m_hat.div(v_hat.sqrt().add_scalar((float)eps));
+            p->sub_(step.mul_scalar((float)lr_t));
+        }
     }
     void zero_grad(const std::vector<Tensor<B>*>& params) const {
         for (Tensor<B>* p : params) p->zero_grad();

@@ -159,6 +159,15 @@ def run(flt="", sets=4, random_grad=False, out=sys.stdout):
             timeit(f"matmul_{dt}/{b}x{m_}x{k}x{n} dA", lambda: g(b * m_ * k, b * k * n, md.ctypes.data, c, a, bb, ga, None), nb, reps=5, flops=fl)
             timeit(f"matmul_{dt}/{b}x{m_}x{k}x{n} dB", lambda: g(b * m_ * k, b * k * n, md.ctypes.data, c, a, bb, None, gb), nb, reps=5, flops=fl)
 
+    # ---- fused Adam step: 4 tensors read, 3 written (the reference's fourteen ops move about 40) -------------------
+    for dt, e in (("f32", 4), ("bf16", 2)):
+        n = N if dt == "f32" else 2 * N
+        pa, g, mm, vv = buf("x", N * 4), buf("y", N * 4), buf("z", N * 4), buf("ga", N * 4)
+        c = (lambda v: C.c_float(v)) if dt == "f32" else (lambda v: C.c_uint16(int(np.array([v], np.float32).view(np.uint32)[0] >> 16)))
+        sc = [c(v) for v in (0.9, 0.1, 0.999, 0.001, 0.19, 0.002, 1e-8, 2.4e-4)]
+        f = getattr(lib, f"hip_adam_step_{dt}")
+        timeit(f"adam_step_{dt}/{n} elements (one call for adam.rs:46-86)", lambda: f(n, pa, g, mm, vv, *sc), 7 * n * e)
+
     # ---- the pieces of Conv2d(64 -> 64, 3x3, s1, p1) on [32,64,56,56] and the pad kernels at that size -------------
     B, Ci, H, W = 32, 64, 56, 56
     md = u64(B, Ci, H, W, 3, 3, 56, 56, 1, 1, 1, 1)

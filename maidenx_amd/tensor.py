@@ -44,6 +44,7 @@ def _bind(lib):
         "mxt_module_bias": ([P], P), "mxt_module_release": ([P], None), "mxt_mse_loss": ([P, P], P), "mxt_sgd_step": ([P, F], I),
         "mxt_sgd_zero_grad": ([P], I), "mxt_train": ([P, P, P, F, SZ, P], I), "mxt_set_graph_replay": ([I], None),
         "mxt_last_train_replayed": ([], SZ),
+        "mxt_adam_new": ([C.c_double] * 4, P), "mxt_adam_release": ([P], None), "mxt_adam_set_fused": ([P, I], None), "mxt_adam_step": ([P, P], I),
         "mxt_backend_calls": ([], SZ), "mxt_reset_backend_calls": ([], None), "mxt_device_allocations": ([], SZ), "mxt_synchronize": ([], I),
     }
     for name, (args, res) in sig.items():
@@ -114,6 +115,9 @@ class Host:
         if not h:
             self._raise()
         return Module(self, h)
+
+    def Adam(self, lr=0.001, beta1=0.9, beta2=0.999, epsilon=1e-8):
+        return Adam(self, lr, beta1, beta2, epsilon)
 
     def mse_loss(self, pred, target):
         return self._t(self.lib.mxt_mse_loss(pred.h, target.h))
@@ -242,6 +246,7 @@ class Tensor:
     def tanh(self): return self._un(b"tanh")
     def gelu(self): return self._un(b"gelu")
     def exp(self): return self._un(b"exp")
+    def sqrt(self): return self._un(b"sqrt")
     def sum_all(self): return self._un(b"sum_all")
     def mean_all(self): return self._un(b"mean_all")
     def contiguous(self): return self._un(b"contiguous")
@@ -289,6 +294,25 @@ class Module:
 
     def zero_grad(self):
         self.m._rc(self.m.lib.mxt_sgd_zero_grad(self.h))
+
+
+class Adam:
+    """crates/maidenx_nn/src/optimizers/adam.rs; the moments belong to this object."""
+
+    def __init__(self, m, lr, beta1, beta2, epsilon):
+        self.m = m
+        self.h = m.lib.mxt_adam_new(lr, beta1, beta2, epsilon)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.m.lib.mxt_adam_release(self.h)
+            self.h = None
+
+    def set_fused(self, enabled):
+        self.m.lib.mxt_adam_set_fused(self.h, int(enabled))
+
+    def step(self, module):
+        self.m._rc(self.m.lib.mxt_adam_step(self.h, module.h))
 
 
 _host = None

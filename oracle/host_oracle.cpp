@@ -15,6 +15,7 @@ extern "C" {
     void oracle_add_inplace_##S(size_t, size_t, const size_t*, E*, const E*);                                       \
     void oracle_sub_inplace_##S(size_t, size_t, const size_t*, E*, const E*);                                       \
     void oracle_neg_##S(size_t, size_t, const size_t*, const E*, E*);                                               \
+    void oracle_sqrt_##S(size_t, size_t, const size_t*, const E*, E*);                                              \
     void oracle_square_##S(size_t, size_t, const size_t*, const E*, E*);                                            \
     void oracle_relu_##S(size_t, size_t, const size_t*, const E*, E*);                                              \
     void oracle_tanh_##S(size_t, size_t, const size_t*, const E*, E*);                                              \
@@ -45,6 +46,7 @@ struct OracleBackend {
     static void d2h(void* d, const void* s, size_t n) { std::memcpy(d, s, n); }
     static void check() {}
     static constexpr bool has_graphs = false;
+    static constexpr bool has_fused_adam = false;
     static constexpr auto im2col = &oracle_conv2d_im2col_f32;
     static constexpr auto col2im = &oracle_conv2d_col2im_f32;
     // with_dtype on the host, element by element, as the reference does (crates/maidenx_core/src/buffer/mod.rs:155-196)
@@ -64,7 +66,7 @@ template <> inline uint16_t orc_one<uint16_t>() { return 0x3F80; }
         using Red = void (*)(size_t, size_t, size_t, const size_t*, const E*, E*);                                       \
         static constexpr Bin bin[4] = {&oracle_add_##S, &oracle_sub_##S, &oracle_mul_##S, &oracle_div_##S};              \
         static constexpr Inp inplace[2] = {&oracle_add_inplace_##S, &oracle_sub_inplace_##S};                            \
-        static constexpr Un un[6] = {&oracle_neg_##S, &oracle_square_##S, &oracle_relu_##S, &oracle_tanh_##S, &oracle_gelu_##S, &oracle_exp_##S}; \
+        static constexpr Un un[7] = {&oracle_neg_##S, &oracle_square_##S, &oracle_relu_##S, &oracle_tanh_##S, &oracle_gelu_##S, &oracle_exp_##S, &oracle_sqrt_##S}; \
         static constexpr Unc unc[4] = {&oracle_add_scalar_##S, &oracle_mul_scalar_##S, &oracle_div_scalar_##S, &oracle_pow_##S}; \
         static constexpr Red red[2] = {&oracle_sum_##S, &oracle_mean_##S};                                               \
         static constexpr auto gt_scalar = &oracle_gt_scalar_##S;                                                         \

@@ -84,6 +84,45 @@ def mlp_numpy(epochs, n=10000, w0=(0.3, -0.2, 0.5), b0=0.1, lr=0.01):
     return np.array(losses), w, b
 
 
+def mlp_adam_run(mx, epochs, n=2000, w0=(0.3, -0.2, 0.5), b0=0.1, hyper=(0.01, 0.9, 0.999, 1e-8), fused=True):
+    """The README model trained with Adam through the tensor API (forward, MSE, backward, step, zero_grad)."""
+    x, y = mlp_data(n)
+    lin = mx.Linear(mx.tensor(np.array([w0], np.float32)), mx.tensor(np.array(b0, np.float32), shape=()))
+    xin, yt = mx.tensor(x), mx.tensor(y)
+    opt = mx.Adam(*hyper)
+    opt.set_fused(fused)
+    losses = []
+    for _ in range(epochs):
+        loss = mx.mse_loss(lin.forward(xin), yt)
+        losses.append(float(loss.numpy()))
+        loss.backward()
+        opt.step(lin)
+        lin.zero_grad()
+    return {"losses": np.array(losses), "weight": lin.weight.numpy(), "bias": lin.bias.numpy()}
+
+
+def mlp_adam_numpy(epochs, n=2000, w0=(0.3, -0.2, 0.5), b0=0.1, hyper=(0.01, 0.9, 0.999, 1e-8)):
+    """adam.rs:34-88 in float64 arithmetic on float64 gradients, with the reference's beta^(t+1) bias terms."""
+    lr, b1, b2, eps = hyper
+    x, y = mlp_data(n)
+    x, y = x.astype(np.float64), y.astype(np.float64)
+    p = [np.array([w0], np.float64), np.array(float(b0))]
+    m, v = [np.zeros_like(q) for q in p], [np.zeros_like(q) for q in p]
+    losses = []
+    for t in range(1, epochs + 1):
+        d = x @ p[0].T + p[1] - y
+        losses.append(float(np.mean(d * d)))
+        g = 2.0 * d / d.size
+        grads = [g.T @ x, np.array(float(g.sum()))]
+        c1, c2 = 1.0 - b1 ** (t + 1), 1.0 - b2 ** (t + 1)
+        lr_t = lr * np.sqrt(c2) / c1
+        for i in range(2):
+            m[i] = m[i] * b1 + grads[i] * (1.0 - b1)
+            v[i] = v[i] * b2 + grads[i] ** 2 * (1.0 - b2)
+            p[i] = p[i] - (m[i] / c1) / (np.sqrt(v[i] / c2) + eps) * lr_t
+    return np.array(losses), p[0], float(p[1])
+
+
 # ---- configs[4]: Conv2d + MSE forward/backward ---------------------------------------------------------
 def conv_inputs(B, Cin, H, W, Cout, k, seed):
     rng = np.random.default_rng(seed)

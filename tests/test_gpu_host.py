@@ -9,6 +9,24 @@ from maidenx_amd.tensor import MxError
 pytestmark = pytest.mark.gpu
 
 
+def test_adam_fused_step_equals_the_op_sequence(mx_hip, mx_oracle):
+    """The HIP host layer's Adam updates a contiguous f32 parameter with one fused call; weights and bias must be the
+    bits the fourteen-op form leaves, and both must agree with the CPU oracle's op-by-op run."""
+    from host_programs import mlp_adam_run
+    fused = mlp_adam_run(mx_hip, 30, fused=True)
+    calls_fused = mx_hip.backend_calls()
+    plain = mlp_adam_run(mx_hip, 30, fused=False)
+    calls_plain = mx_hip.backend_calls() - calls_fused
+    assert np.array_equal(fused["weight"], plain["weight"]) and np.array_equal(fused["bias"], plain["bias"])
+    assert np.array_equal(fused["losses"], plain["losses"])
+    ref = mlp_adam_run(mx_oracle, 30)
+    np.testing.assert_allclose(fused["losses"], ref["losses"], rtol=2e-5)
+    np.testing.assert_allclose(fused["weight"], ref["weight"], rtol=2e-4, atol=1e-6)
+    np.testing.assert_allclose(fused["bias"], ref["bias"], rtol=2e-4, atol=1e-6)
+    assert fused["losses"][-1] < 0.8 * fused["losses"][0]
+    assert calls_plain > calls_fused + 30 * 2 * 10          # thirteen fewer backend calls per parameter and step
+
+
 @pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])
 def test_reference_tensor_cases(mx_hip, case):
     check_case(run_case(mx_hip, case), case)

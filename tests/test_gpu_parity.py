@@ -817,6 +817,47 @@ def test_index_out_of_bounds_is_reported(hip):
 
 
 @pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("n", [1, 7, 1000, 4099, 1 << 16])
+def test_fused_adam_step_equals_the_fourteen_ops(oracle, hip, n, dt):
+    """adam.rs:46-86 as the op sequence it is, on the oracle and on the GPU, against one hip_adam_step call: the same
+    bits in param, m and v, over several steps with the reference's beta^(t+1) bias terms."""
+    r = rng(173)
+    st = lambda a: to_storage(np.asarray(a, dtype=np.float32), dt)
+    p0 = st(r.standard_normal(n))
+    m0, v0 = st(np.zeros(n)), st(np.zeros(n))
+    lr, b1, b2, eps = 0.001, 0.9, 0.999, 1e-8
+    md1 = meta_unary([n], [1])
+    md2 = meta_binary([n], [1], [1])
+
+    def chain(be, p, g, m, v, sc):
+        un = lambda op, x: be.call(f"{op}_{dt}", n, 1, md1, In(x), Out(n, dt))[0]
+        unc = lambda op, x, c: be.call(f"{op}_{dt}", n, 1, md1, In(x), const_arg(c, dt), Out(n, dt))[0]
+        bi = lambda op, a, b: be.call(f"{op}_{dt}", n, 1, md2, In(a), In(b), Out(n, dt))[0]
+        m = bi("add", unc("mul_scalar", m, sc[0]), unc("mul_scalar", g, sc[1]))
+        v = bi("add", unc("mul_scalar", v, sc[2]), unc("mul_scalar", un("square", g), sc[3]))
+        step = bi("div", unc("div_scalar", m, sc[4]), unc("add_scalar", un("sqrt", unc("div_scalar", v, sc[5])), sc[6]))
+        (p,) = be.call(f"sub_inplace_{dt}", n, 1, md2, InOut(p), In(unc("mul_scalar", step, sc[7])))
+        return p, m, v
+
+    po, mo, vo = p0.copy(), m0.copy(), v0.copy()
+    ph, mh, vh = p0.copy(), m0.copy(), v0.copy()
+    pf, mf, vf = p0.copy(), m0.copy(), v0.copy()
+    for t in range(1, 4):
+        g = st(r.standard_normal(n) * (0.0 if t == 2 and n == 7 else 1.0))          # a zero gradient: 0 / (0 + eps)
+        b1t, b2t = b1 ** (t + 1), b2 ** (t + 1)                                        # adam.rs:56-61 multiplies t times from beta
+        sc = [b1, 1 - b1, b2, 1 - b2, 1 - b1t, 1 - b2t, eps, lr * np.sqrt(1 - b2t) / (1 - b1t)]
+        po, mo, vo = chain(oracle, po, g, mo, vo, sc)
+        ph, mh, vh = chain(hip, ph, g, mh, vh, sc)
+        pf, mf, vf = hip.call(f"adam_step_{dt}", n, InOut(pf), In(g), InOut(mf), InOut(vf), *[const_arg(c, dt) for c in sc])
+        for a, b, c, what in ((po, ph, pf, "param"), (mo, mh, mf, "m"), (vo, vh, vf, "v")):
+            assert same_bits(a, b), (what, t, "op by op: oracle vs GPU")
+            assert same_bits(b, c), (what, t, "fused vs op by op")
+    assert not same_bits(mf, m0) and not same_bits(vf, v0)
+    if dt == "f32":
+        assert not same_bits(pf, p0)          # (a 16-bit parameter near 1 does not move by 0.001)
+
+
+@pytest.mark.parametrize("dt", DTS)
 def test_empty_inputs_are_no_ops(hip, dt):
     """Zero elements anywhere: nothing is launched, nothing is written, no error is recorded."""
     import maidenx_amd.lib as L

@@ -85,6 +85,26 @@ def test_mlp_training_matches_gradient_descent(mx_oracle):
     assert mx_oracle.device_allocations() > 0
 
 
+def test_adam_training_matches_the_update_rule(mx_oracle):
+    """adam.rs through the tensor API on the CPU oracle (op by op) against the update rule in float64."""
+    from host_programs import mlp_adam_numpy, mlp_adam_run
+    got = mlp_adam_run(mx_oracle, 25)
+    losses, w, b = mlp_adam_numpy(25)
+    assert losses[-1] < 0.8 * losses[0]
+    np.testing.assert_allclose(got["losses"], losses, rtol=2e-4)
+    np.testing.assert_allclose(got["weight"], w, rtol=2e-4, atol=1e-6)
+    np.testing.assert_allclose(got["bias"], b, rtol=2e-4, atol=1e-6)
+
+
+def test_sqrt_forward_and_backward(mx_oracle):
+    x = np.array([0.25, 1.0, 4.0, 9.0], np.float32)
+    t = mx_oracle.tensor(x).with_grad()
+    y = t.sqrt()
+    np.testing.assert_array_equal(y.numpy(), np.sqrt(x))
+    y.sum_all().backward()
+    np.testing.assert_allclose(t.grad().numpy(), 0.5 / np.sqrt(x), rtol=1e-6)          # unary.rs:176-178: go / (2 * sqrt(x))
+
+
 def test_mlp_call_count_is_stable(mx_oracle):
     mx = mx_oracle
     mlp_run(mx, 2, n=100)
