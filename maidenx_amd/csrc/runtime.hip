@@ -29,6 +29,11 @@ struct GraphExec {                        // what hip_graph_end_capture hands ou
     ProgCmd* cmds = nullptr;              // device copy of the program, when the capture is one
     uint32_t n = 0;
 };
+// A capture that called scratch() has the block's address baked into its graph or program: while such a capture is
+// alive the block must not be freed, so a later growth retires it instead (freed with the last live capture).
+static bool g_scratch_captured[16][2] = {{false}};
+static int g_live_captures = 0;
+static std::vector<void*> g_retired_scratch;
 static void* g_scratch[16][2] = {{nullptr}};
 static size_t g_scratch_bytes[16][2] = {{0}};
 
@@ -70,7 +75,10 @@ void* scratch(size_t bytes, int slot) {
         return nullptr;
     }
     std::lock_guard<std::mutex> lk(g_scratch_mu);
-    if (g_scratch_bytes[dev][slot] >= bytes) return g_scratch[dev][slot];
+    if (g_scratch_bytes[dev][slot] >= bytes) {
+        if (g_capturing) g_scratch_captured[dev][slot] = true;
+        return g_scratch[dev][slot];
+    }
     if (g_capturing) {      // growing means a synchronise and a free, neither of which a capture allows
         set_status(ERR_INVALID, "scratch would have to grow during graph capture: run the sequence eagerly once first");
         return nullptr;
@@ -78,7 +86,9 @@ void* scratch(size_t bytes, int slot) {
     // grow: work already queued on the stream may still use the old block, so drain first
     if (g_scratch[dev][slot]) {
         (void)hipStreamSynchronize(g_stream);
-        (void)hipFree(g_scratch[dev][slot]);
+        if (g_scratch_captured[dev][slot] && g_live_captures > 0) g_retired_scratch.push_back(g_scratch[dev][slot]);
+        else (void)hipFree(g_scratch[dev][slot]);
+        g_scratch_captured[dev][slot] = false;
         g_scratch[dev][slot] = nullptr;
         g_scratch_bytes[dev][slot] = 0;
     }
@@ -243,6 +253,10 @@ int hip_graph_end_capture(void** graph_exec) {
         if (e != hipSuccess) { delete ge; return (int)e; }
     }
     g_prog_cmds.clear();
+    {
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        ++g_live_captures;
+    }
     *graph_exec = (void*)ge;
     return 0;
 }
@@ -272,6 +286,16 @@ int hip_graph_destroy(void* graph_exec) {
     if (ge->cmds) e = hipFree(ge->cmds);
     if (ge->graph) e = hipGraphExecDestroy(ge->graph);
     delete ge;
+    {
+        // the last live capture is gone: nothing refers to retired scratch blocks, or to the current ones, any more
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        if (--g_live_captures <= 0) {
+            g_live_captures = 0;
+            for (void* p : g_retired_scratch) (void)hipFree(p);
+            g_retired_scratch.clear();
+            for (auto& dev : g_scratch_captured) dev[0] = dev[1] = false;
+        }
+    }
     return (int)e;
 }
 

@@ -188,3 +188,45 @@ def test_large_or_unsupported_captures_stay_hip_graphs(lib):
         replay_equals_eager(lib, elementwise_sequence(lib, (1000,), None, 2), expect_program=False, replays=1)
     finally:
         lib.hip_graph_set_programs(was)
+
+
+def test_scratch_used_by_a_capture_survives_later_growth(lib):
+    """A captured call that stages through the library's scratch block has that address in its graph.  A later eager
+    call that needs a larger block must not free the old one while the capture is alive: replays still write there."""
+    r = np.random.default_rng(7)
+    small = r.standard_normal((64, 48)).astype(np.float32)
+    seq = Seq(lib)
+    a, o = seq.dev(small), seq.out(48 * 4, "f4")
+    # sum over dim 0 of the transposed view of a [48, 64] buffer: gathered into scratch first
+    seq.add("sum_to_shape_f32", 64 * 48, 2, u64([64, 48], [1, 64], [1, 48], 0), a.ptr, o.ptr)
+    seq.run()
+    (want,) = seq.read()
+    assert lib.hip_graph_begin_capture() == 0
+    seq.run()
+    h = C.c_void_p()
+    assert lib.hip_graph_end_capture(C.byref(h)) == 0
+    try:
+        # an eager call whose staging copy needs more than the 32 MB block
+        n = 12 << 20
+        big = L.DeviceBuffer.from_numpy(np.ones(n, np.float32))
+        out = L.DeviceBuffer(3 * 4)
+        lib.hip_sum_to_shape_f32(n, 2, u64([n // 3, 3], [1, n // 3], [1, 3], 0).ctypes.data, big.ptr, out.ptr)
+        assert lib.hip_synchronize() == 0 and lib.hip_get_last_status() == 0
+        assert out.to_numpy(np.float32).tolist() == [n // 3] * 3
+        # allocations that would land in a freed block, filled with something else
+        junk = [L.DeviceBuffer(8 << 20) for _ in range(6)]
+        for j in junk:
+            lib.hip_fill_f32((8 << 20) // 4, j.ptr, C.c_float(3.0))
+        for _ in range(2):
+            seq.clear_outputs()
+            assert lib.hip_graph_launch(h) == 0
+            (got,) = seq.read()
+            assert got.tobytes() == want.tobytes()
+        for j in junk:
+            assert float(j.to_numpy(np.float32, 4)[0]) == 3.0
+    finally:
+        assert lib.hip_graph_destroy(h) == 0
+    seq.clear_outputs()
+    seq.run()
+    (again,) = seq.read()
+    assert again.tobytes() == want.tobytes() and lib.hip_get_last_status() == 0
