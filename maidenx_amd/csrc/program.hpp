@@ -17,11 +17,12 @@ namespace mxh {
 
 constexpr int PROG_ARG_BYTES = 496;
 constexpr unsigned PROG_THREADS = 1024;       // threads of the interpreter's work-group
-// One work-group has one CU's bandwidth (about 150 GB/s): a command that moves more than a few tens of KB
-// is faster as a graph node that spreads over the chip.  Measured per command, mul_f32: 1.0 / 1.7 / 1.9 / 4.6 us
-// in a program against 1.7 / 2.3 / 2.3 / 2.4 us in a HIP graph for 256 / 4096 / 10000 / 40000 elements.
-constexpr unsigned PROG_MAX_GRID = 4;         // virtual 256-thread blocks one command may have (one pass of the work-group)
-constexpr size_t PROG_MAX_ELEMS = 16384;      // elements a reduction or small matmul command may read
+// One work-group has one CU's bandwidth (about 150 GB/s) and one CU's ALUs: only very small commands are cheaper here
+// than as graph nodes.  Measured per command, mul_f32: 1.0 / 1.8 / 1.9 us in a program against 1.6 / 1.75 / 1.8 us
+// as a HIP graph node for 256 / 4096 / 10000 elements - so a command may have one virtual block (4096 elements in
+// vector form) and a capture is a program only if all of its launches are that small.
+constexpr unsigned PROG_MAX_GRID = 1;         // virtual 256-thread blocks one command may have
+constexpr size_t PROG_MAX_ELEMS = 4096;       // elements a reduction or small matmul command may read
 struct alignas(16) ProgCmd {
     uint32_t kid;                             // family << 16 | instantiation
     uint32_t grid;                            // virtual blocks

@@ -154,11 +154,11 @@ def test_dependent_chain_with_reductions_and_small_matmul(lib):
 
 def test_block_dot_matmul_in_a_program(lib):
     r = np.random.default_rng(4)
-    n = 8192
+    n = 4096
     seq = Seq(lib)
-    x, g = seq.dev(r.standard_normal((n, 2)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
-    gw = seq.out(2 * 4, "f4")
-    seq.add("matmul_f32", 2, u64(2, 2, 2, [2, 1], [2, n], [n, 1], [1, 2], [1, 1], 0, 0), x.ptr, g.ptr, gw.ptr)
+    x, g = seq.dev(r.standard_normal((n, 1)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    gw = seq.out(1 * 4, "f4")
+    seq.add("matmul_f32", 1, u64(2, 2, 2, [1, 1], [1, n], [n, 1], [1, 1], [1, 1], 0, 0), x.ptr, g.ptr, gw.ptr)
     replay_equals_eager(lib, seq, expect_program=True)
 
 
