@@ -176,3 +176,65 @@ def test_conv_kernels_config_size(hip):
     assert same_bits(p, xp.ravel())
     (gi,) = hip.call("pad_with_constant_backward_f32", x.size, xp.size, 4, mdp, In(xp.ravel()), Out(x.size, "f32"))
     assert same_bits(gi, (x + np.float32(0)).ravel())
+
+
+@pytest.mark.parametrize("mode,np_mode", [("reflection", "reflect"), ("replication", "edge")])
+def test_edge_pads_config_size(hip, mode, np_mode):
+    """[32,64,56,56] padded by (1,2) x (2,1) on H and W: forward against numpy.pad bit for bit, backward against the
+    transpose of that map accumulated in float64 (at most 9 terms per element) and through the adjoint identity."""
+    Bn, Cc, H, W = 32, 64, 56, 56
+    pads = [(0, 0), (0, 0), (1, 2), (2, 1)]
+    r = np.random.default_rng(0x5EED0006)
+    x = r.standard_normal((Bn, Cc, H, W), dtype=np.float32)
+    xp = np.pad(x, pads, mode=np_mode)
+    md = meta_pad([Bn, Cc, H, W], [Cc * H * W, H * W, W, 1], 0, list(xp.shape), pads)
+    (p,) = hip.call(f"pad_with_{mode}_f32", x.size, xp.size, 4, md, In(x.ravel()), Out(xp.size, "f32"))
+    assert same_bits(p, xp.ravel())
+    go = r.standard_normal(xp.shape, dtype=np.float32)
+    (gi,) = hip.call(f"pad_with_{mode}_backward_f32", x.size, xp.size, 4, md, In(go.ravel()), Out(x.size, "f32"))
+    # the index map of the forward, from padding an index tensor
+    idx = np.pad(np.arange(H * W, dtype=np.int64).reshape(H, W), pads[2:], mode=np_mode).ravel()
+    ref = np.zeros((Bn * Cc, H * W))
+    np.add.at(ref, (slice(None), idx), go.reshape(Bn * Cc, -1).astype(np.float64))
+    np.testing.assert_allclose(gi.reshape(Bn * Cc, H * W), ref, rtol=2e-6, atol=2e-6)
+    assert abs(float(np.vdot(xp.astype(np.float64), go)) - float(np.vdot(x.astype(np.float64), gi.reshape(x.shape)))) < 1e-6 * x.size ** 0.5 * 10
+
+
+def test_conv_layer_products_config_size(hip):
+    """The three f32 products of the Conv2d(64->64, 3x3) step at [32,64,56,56] (64x64 tiles, the unchecked body,
+    split-K for the weight gradient): sampled rows and columns against float64."""
+    M, K, N = 32 * 56 * 56, 576, 64
+    r = np.random.default_rng(0x5EED0007)
+    cols = r.standard_normal((M, K), dtype=np.float32)
+    w = (r.standard_normal((N, K), dtype=np.float32) * np.float32(0.05))
+    g = r.standard_normal((M, N), dtype=np.float32)
+    rows = r.integers(0, M, 64)
+    (out,) = hip.call("matmul_f32", M * N, meta_matmul([M, N], [M, K], [K, N], [K, 1], [1, K]), In(cols.ravel()), In(w.ravel()), Out(M * N, "f32"))
+    np.testing.assert_allclose(out.reshape(M, N)[rows], cols[rows].astype(np.float64) @ w.T.astype(np.float64), rtol=2e-5, atol=2e-5)
+    (gin,) = hip.call("matmul_f32", M * K, meta_matmul([M, K], [M, N], [N, K], [N, 1], [K, 1]), In(g.ravel()), In(w.ravel()), Out(M * K, "f32"))
+    np.testing.assert_allclose(gin.reshape(M, K)[rows], g[rows].astype(np.float64) @ w.astype(np.float64), rtol=2e-5, atol=2e-5)
+    (gw,) = hip.call("matmul_f32", K * N, meta_matmul([K, N], [K, M], [M, N], [1, K], [N, 1]), In(cols.ravel()), In(g.ravel()), Out(K * N, "f32"))
+    ks = r.integers(0, K, 16)
+    np.testing.assert_allclose(gw.reshape(K, N)[ks], cols[:, ks].T.astype(np.float64) @ g.astype(np.float64), rtol=1e-4, atol=2e-3)
+
+
+def test_fused_adam_16m_elements_bit_exact(hip):
+    """Every step of adam.rs:46-86 is one correctly rounded IEEE operation, so numpy's float32 arithmetic gives the
+    reference's bits; three steps on 2^24 elements."""
+    n = 1 << 24
+    r = np.random.default_rng(0x5EED0008)
+    p = r.standard_normal(n, dtype=np.float32)
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    hp, hm, hv = p.copy(), m.copy(), v.copy()
+    f = np.float32
+    lr, b1, b2, eps = 0.001, 0.9, 0.999, 1e-8
+    from helpers import InOut
+    for t in range(1, 4):
+        g = r.standard_normal(n, dtype=np.float32)
+        c1, c2 = 1 - b1 ** (t + 1), 1 - b2 ** (t + 1)
+        sc = [f(b1), f(1 - b1), f(b2), f(1 - b2), f(c1), f(c2), f(eps), f(lr * np.sqrt(c2) / c1)]
+        m = m * sc[0] + g * sc[1]
+        v = v * sc[2] + (g * g) * sc[3]
+        p = p - ((m / sc[4]) / (np.sqrt(v / sc[5]) + sc[6])) * sc[7]
+        hp, hm, hv = hip.call("adam_step_f32", n, InOut(hp), In(g), InOut(hm), InOut(hv), *[float(c) for c in sc])
+        assert same_bits(hm, m) and same_bits(hv, v) and same_bits(hp, p), t
