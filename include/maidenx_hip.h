@@ -84,6 +84,14 @@ int hip_graph_destroy(void* graph_exec);
  * hip_graph_set_programs: allow (1, default) or forbid (0) programs for later captures, returns the old value. */
 int hip_graph_is_program(void* graph_exec);
 int hip_graph_set_programs(int enabled);
+/* Inside a capture that is not a program, consecutive f32 elementwise launches over one index space (at most two
+ * collapsed dims, fewer than 2^20 elements) that meet each other's data only element for element are recorded as ONE
+ * kernel node that applies them in order per element (each output is still written; same bytes as separate launches).
+ * hip_graph_fused_launches: how many launches of the capture were fused, and into how many nodes;
+ * hip_graph_set_fusion: allow (1, default) or forbid (0) this for later captures, returns the old value.
+ * No counterpart in the reference. */
+int hip_graph_fused_launches(void* graph_exec, int* nodes);
+int hip_graph_set_fusion(int enabled);
 
 /* ---- binary: replaces crates/maidenx_cuda/src/ops/binary.rs:12-161 --------------------------------
  * metadata = dims[n] | lhs_strides[n] | rhs_strides[n] | lhs_offset | rhs_offset   (NULL: contiguous)

@@ -16,6 +16,7 @@
 
 #include "mxh.hpp"
 #include "ew_registry.hpp"
+#include "fuse.hpp"
 
 namespace mxh {
 
@@ -349,6 +350,30 @@ inline void ew_record(int vec, unsigned blocks, const NdSpace<Op::NIN + 1>& sp, 
     }
 }
 
+// While a capture is open: offers an f32 -> f32 launch of ew_nd to the open fused group (true: do not launch).
+template <class Op>
+inline bool ew_fuse(bool vec, const NdSpace<Op::NIN + 1>& sp, const EwPtrs<Op::NIN>& p, size_t n, const Op& op) {
+    constexpr int idx = IndexOf<Op, EwProgOps>::value;
+    if constexpr (idx >= 0 && std::is_same<typename Op::In, float>::value && std::is_same<typename Op::Out, float>::value && sizeof(Op) <= 8) {
+        // launch-bound sizes only: a large tensor is better off with four vectors per thread
+        if (sp.ndims < 1 || sp.ndims > 2 || n >= (size_t)EW_SMALL_BLOCKS * EW_BLOCK * EW_UNR) return false;
+        FuseCmd c;
+        std::memset((void*)&c, 0, sizeof(c));
+        c.out = p.out;
+        c.op = (uint32_t)idx;
+        c.nin = Op::NIN;
+        std::memcpy(c.payload, (const void*)&op, sizeof(Op));
+        for (int d = 0; d < sp.ndims; ++d) {
+            c.os[d] = sp.strides[0][d];
+            for (int k = 0; k < Op::NIN; ++k) c.is[k][d] = sp.strides[k + 1][d];
+        }
+        for (int k = 0; k < Op::NIN; ++k) c.in[k] = p.in[k];
+        if (vec && c.os[sp.ndims - 1] != 1) return false;
+        return fuse_record(c, (uint32_t)sp.ndims, sp.dims, vec, n, sizeof(float));
+    }
+    return false;
+}
+
 // ---- host-side selection -------------------------------------------------------------------
 // in_strides[k] / out_strides are in elements, pointers already include the operand offsets.
 template <class Op>
@@ -455,6 +480,7 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
     if (vec_ok) {
         size_t nvec = num_els / VEC;
         unsigned blocks = cdiv(nvec, EW_BLOCK * EW_UNR);
+        if (ew_fuse<Op>(true, sp, p, nvec, op)) return;
         ew_record<Op>(1, blocks, sp, p, nvec, op);
         if (blocks < EW_SMALL_BLOCKS)
             hipLaunchKernelGGL((ew_nd_kernel<Op, VEC, 1>), dim3(cdiv(nvec, EW_BLOCK)), dim3(EW_BLOCK), 0, stream(), sp, p, nvec, op);
@@ -462,6 +488,7 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
             hipLaunchKernelGGL((ew_nd_kernel<Op, VEC>), dim3(blocks), dim3(EW_BLOCK), 0, stream(), sp, p, nvec, op);
     } else {
         unsigned blocks = cdiv(num_els, EW_BLOCK * EW_UNR);
+        if (ew_fuse<Op>(false, sp, p, num_els, op)) return;
         ew_record<Op>(0, blocks, sp, p, num_els, op);
         if (blocks < EW_SMALL_BLOCKS)
             hipLaunchKernelGGL((ew_nd_kernel<Op, 1, 1>), dim3(cdiv(num_els, EW_BLOCK)), dim3(EW_BLOCK), 0, stream(), sp, p, num_els, op);

@@ -6,6 +6,7 @@
 #include <mutex>
 #include <vector>
 
+#include "fuse.hpp"
 #include "mxh.hpp"
 
 namespace mxh {
@@ -24,10 +25,16 @@ static bool g_prog_enabled = true;
 static bool g_prog_ok = false;            // every launch of the open capture so far has a command
 static bool g_prog_pending = false;       // a command was recorded and its launch not yet seen
 static std::vector<ProgCmd> g_prog_cmds;
+// fused runs of elementwise launches inside a capture (see fuse.hpp)
+static bool g_fuse_enabled = true;
+static FuseGroup g_fuse;                  // the open group (n == 0: none)
+static size_t g_fuse_elem_bytes = 4;
+static uint32_t g_fused_launches = 0, g_fuse_nodes = 0;     // of the open capture
 struct GraphExec {                        // what hip_graph_end_capture hands out
     hipGraphExec_t graph = nullptr;
     ProgCmd* cmds = nullptr;              // device copy of the program, when the capture is one
     uint32_t n = 0;
+    uint32_t fused_launches = 0, fuse_nodes = 0;
 };
 // A capture that called scratch() has the block's address baked into its graph or program: while such a capture is
 // alive the block must not be freed, so a later growth retires it instead (freed with the last live capture).
@@ -48,7 +55,87 @@ void set_status(int code, const char* what, int hip_err) {
         snprintf(g_what, sizeof(g_what), "%s", what);
 }
 
-hipStream_t stream() { return g_stream; }
+static void fuse_flush() {
+    if (g_fuse.n == 0) return;
+    fuse_launch(g_fuse, (void*)g_capture_stream);
+    ++g_fuse_nodes;
+    g_fuse.n = 0;
+}
+
+// Every launch and copy of the library asks for the stream right before it queues something: an open group of fused
+// launches has to run before that.
+hipStream_t stream() {
+    if (g_capturing && g_fuse.n) fuse_flush();
+    return g_stream;
+}
+
+// byte range an operand touches
+static void operand_range(const void* base, const int64_t* strides, uint32_t ndims, const uint32_t* dims, size_t esz, uintptr_t& lo, uintptr_t& hi) {
+    size_t span = 0;
+    for (uint32_t d = 0; d < ndims; ++d) span += (size_t)(dims[d] - 1) * (size_t)strides[d];
+    lo = (uintptr_t)base;
+    hi = lo + (span + 1) * esz;
+}
+static bool same_mapping(const void* a, const int64_t* sa, const void* b, const int64_t* sb, uint32_t ndims) {
+    if (a != b) return false;
+    for (uint32_t d = 0; d < ndims; ++d)
+        if (sa[d] != sb[d]) return false;
+    return true;
+}
+
+bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
+    // only once the capture cannot be a whole-capture program any more (that path launches for real)
+    if (!g_capturing || !g_fuse_enabled || g_prog_ok || ndims < 1 || ndims > 2) return false;
+    for (uint32_t d = 0; d < ndims; ++d)
+        if (c.os[d] < 0 || c.is[0][d] < 0 || (c.nin > 1 && c.is[1][d] < 0)) return false;
+    const bool fits = g_fuse.n > 0 && g_fuse.n < (uint32_t)FUSE_MAX_CMDS && g_fuse.ndims == ndims && g_fuse.vec == (vec ? 1u : 0u) &&
+                      g_fuse.nvec == nvec && g_fuse.dims[0] == dims[0] && (ndims == 1 || g_fuse.dims[1] == dims[1]) && g_fuse_elem_bytes == elem_bytes;
+    bool join = fits;
+    if (join) {
+        // every overlap with an earlier member must be element for element, so that a thread only meets its own data
+        uintptr_t olo, ohi;
+        operand_range(c.out, c.os, ndims, dims, elem_bytes, olo, ohi);
+        for (uint32_t k = 0; k < g_fuse.n && join; ++k) {
+            const FuseCmd& e = g_fuse.cmd[k];
+            uintptr_t lo, hi;
+            operand_range(e.out, e.os, ndims, dims, elem_bytes, lo, hi);
+            // read after write, and write after write
+            for (uint32_t j = 0; j < c.nin && join; ++j) {
+                uintptr_t ilo, ihi;
+                operand_range(c.in[j], c.is[j], ndims, dims, elem_bytes, ilo, ihi);
+                if (ilo < hi && lo < ihi && !same_mapping(c.in[j], c.is[j], e.out, e.os, ndims)) join = false;
+            }
+            if (olo < hi && lo < ohi && !same_mapping(c.out, c.os, e.out, e.os, ndims)) join = false;
+            // write after read
+            for (uint32_t j = 0; j < e.nin && join; ++j) {
+                uintptr_t ilo, ihi;
+                operand_range(e.in[j], e.is[j], ndims, dims, elem_bytes, ilo, ihi);
+                if (olo < ihi && ilo < ohi && !same_mapping(c.out, c.os, e.in[j], e.is[j], ndims)) join = false;
+            }
+        }
+    }
+    if (!join) {
+        fuse_flush();
+        g_fuse.ndims = ndims;
+        g_fuse.vec = vec ? 1u : 0u;
+        g_fuse.nvec = nvec;
+        g_fuse.dims[0] = dims[0];
+        g_fuse.dims[1] = ndims == 2 ? dims[1] : 1;
+        g_fuse.div_inner = make_fastdiv(g_fuse.dims[ndims - 1]);
+        g_fuse_elem_bytes = elem_bytes;
+    }
+    FuseCmd& slot = g_fuse.cmd[g_fuse.n];
+    slot = c;
+    slot.fwd = 0;
+    if (g_fuse.n > 0) {
+        const FuseCmd& prev = g_fuse.cmd[g_fuse.n - 1];
+        for (uint32_t j = 0; j < c.nin; ++j)
+            if (same_mapping(c.in[j], c.is[j], prev.out, prev.os, ndims)) slot.fwd |= 1u << j;
+    }
+    ++g_fuse.n;
+    ++g_fused_launches;
+    return true;
+}
 
 bool prog_recording() { return g_capturing && g_prog_ok; }
 void prog_record(uint32_t kid, unsigned grid, const void* args, size_t bytes) {
@@ -228,10 +315,13 @@ int hip_graph_begin_capture(void) {
     g_prog_ok = g_prog_enabled;
     g_prog_pending = false;
     g_prog_cmds.clear();
+    g_fuse.n = 0;
+    g_fused_launches = g_fuse_nodes = 0;
     return 0;
 }
 int hip_graph_end_capture(void** graph_exec) {
     if (!g_capturing || !graph_exec) return (int)hipErrorInvalidValue;
+    fuse_flush();
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamEndCapture(g_capture_stream, &graph);
     g_stream = g_saved_stream;
@@ -253,6 +343,8 @@ int hip_graph_end_capture(void** graph_exec) {
         if (e != hipSuccess) { delete ge; return (int)e; }
     }
     g_prog_cmds.clear();
+    ge->fused_launches = g_fused_launches;
+    ge->fuse_nodes = g_fuse_nodes;
     {
         std::lock_guard<std::mutex> lk(g_scratch_mu);
         ++g_live_captures;
@@ -262,6 +354,18 @@ int hip_graph_end_capture(void** graph_exec) {
 }
 // 1 when the capture behind `graph_exec` replays as one interpreter launch, 0 when it is a HIP graph.
 int hip_graph_is_program(void* graph_exec) { return graph_exec && ((GraphExec*)graph_exec)->cmds ? 1 : 0; }
+// Elementwise launches of the capture that were fused into groups, and (nodes != NULL) the kernel nodes they became.
+int hip_graph_fused_launches(void* graph_exec, int* nodes) {
+    if (!graph_exec) return 0;
+    if (nodes) *nodes = (int)((GraphExec*)graph_exec)->fuse_nodes;
+    return (int)((GraphExec*)graph_exec)->fused_launches;
+}
+// Whether later captures may fuse runs of elementwise launches (default 1); returns the previous setting.
+int hip_graph_set_fusion(int enabled) {
+    int was = g_fuse_enabled ? 1 : 0;
+    g_fuse_enabled = enabled != 0;
+    return was;
+}
 // Whether later captures may become programs (default 1); returns the previous setting.
 int hip_graph_set_programs(int enabled) {
     int was = g_prog_enabled ? 1 : 0;

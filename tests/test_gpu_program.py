@@ -230,3 +230,109 @@ def test_scratch_used_by_a_capture_survives_later_growth(lib):
     seq.run()
     (again,) = seq.read()
     assert again.tobytes() == want.tobytes() and lib.hip_get_last_status() == 0
+
+
+# ---- fused runs of elementwise launches inside a capture ----------------------------------------------------------
+def fused(lib, seq, want_launches=None, want_nodes=None, replays=2):
+    """Captures `seq` (after a first launch that cannot be part of a program, so that fusion is active), checks the
+    replays against the eager bytes and returns (fused launches, nodes)."""
+    seq.run()
+    eager = seq.read()
+    assert lib.hip_get_last_status() == 0, lib.hip_status_string()
+    big = L.DeviceBuffer(1 << 20)
+    assert lib.hip_graph_begin_capture() == 0
+    lib.hip_fill_f32((1 << 20) // 4, big.ptr, C.c_float(0.0))        # too large for a program command
+    seq.run()
+    h = C.c_void_p()
+    assert lib.hip_graph_end_capture(C.byref(h)) == 0
+    try:
+        nodes = C.c_int()
+        launches = lib.hip_graph_fused_launches(h, C.byref(nodes))
+        assert lib.hip_graph_is_program(h) == 0
+        for _ in range(replays):
+            seq.clear_outputs()
+            assert lib.hip_graph_launch(h) == 0
+            got = seq.read()
+            for k, (g, e) in enumerate(zip(got, eager)):
+                assert g.tobytes() == e.tobytes(), k
+    finally:
+        assert lib.hip_graph_destroy(h) == 0
+    assert lib.hip_get_last_status() == 0, lib.hip_status_string()
+    if want_launches is not None:
+        assert launches == want_launches, (launches, nodes.value)
+    if want_nodes is not None:
+        assert nodes.value == want_nodes, (launches, nodes.value)
+    return launches, nodes.value
+
+
+@pytest.mark.parametrize("n", [1, 3, 1000, 10000, 40004])
+def test_fused_chain_of_dependent_ops(lib, n):
+    """A chain in which every op reads what the one before wrote, element for element: one node."""
+    r = np.random.default_rng(11)
+    seq = Seq(lib)
+    x, y = seq.dev(r.standard_normal(n).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    outs = [seq.out(n * 4, "f4") for _ in range(7)]
+    md1, md2 = u64([n], [1], 0), u64([n], [1], [1], 0, 0)
+    seq.add("mul_f32", n, 1, md2, x.ptr, y.ptr, outs[0].ptr)
+    seq.add("add_scalar_f32", n, 1, md1, outs[0].ptr, C.c_float(0.5), outs[1].ptr)
+    seq.add("tanh_f32", n, 1, md1, outs[1].ptr, outs[2].ptr)
+    seq.add("sub_f32", n, 1, md2, outs[2].ptr, x.ptr, outs[3].ptr)
+    seq.add("pow_f32", n, 1, md1, outs[3].ptr, C.c_float(2.0), outs[4].ptr)
+    seq.add("div_f32", n, 1, md2, outs[4].ptr, outs[1].ptr, outs[5].ptr)          # also reads an older member's output
+    seq.add("add_inplace_f32", n, 1, md2, outs[5].ptr, y.ptr)                      # in place on the previous output
+    seq.add("neg_f32", n, 1, md1, outs[5].ptr, outs[6].ptr)
+    fused(lib, seq, want_launches=8, want_nodes=1)
+
+
+def test_fused_groups_split_where_threads_would_meet(lib):
+    """Overlaps that are not element for element must close the group: a broadcast of something the group wrote, a
+    shifted view, a transposed read of a buffer the group then overwrites."""
+    r = np.random.default_rng(12)
+    n = 4096
+    seq = Seq(lib)
+    x = seq.dev(r.standard_normal(n).astype(np.float32))
+    a, b, c, d, e = seq.out(n * 4, "f4"), seq.out(n * 4, "f4"), seq.out((n - 1) * 4, "f4"), seq.out(n * 4, "f4"), seq.out(n * 4, "f4")
+    md1, md2 = u64([n], [1], 0), u64([n], [1], [1], 0, 0)
+    seq.add("exp_f32", n, 1, md1, x.ptr, a.ptr)
+    # element 0 of `a` broadcast to every element: written by another thread of the same group -> new group
+    seq.add("mul_f32", n, 1, u64([n], [1], [0], 0, 0), x.ptr, a.ptr, b.ptr)
+    # `b` shifted by one element (read after write across threads) -> new group
+    seq.add("add_f32", n - 1, 1, u64([n - 1], [1], [1], 0, 1), x.ptr, b.ptr, c.ptr)
+    # [64,64] transposed read of `c`'s buffer, then an overwrite of that buffer (write after read across threads)
+    seq.add("mul_scalar_f32", n, 2, u64([64, 64], [64, 1], 0), b.ptr, C.c_float(2.0), d.ptr)        # same space as the next two
+    seq.add("add_f32", n, 1, md2, d.ptr, x.ptr, e.ptr)
+    seq.add("sub_f32", n, 1, md2, e.ptr, d.ptr, b.ptr)                                                # overwrites b: b was read element for element only
+    launches, nodes = fused(lib, seq)
+    assert launches == 6 and nodes == 4
+
+
+def test_fused_two_dim_broadcast_and_a_reduction_in_between(lib):
+    r = np.random.default_rng(13)
+    rows, cols = 48, 200
+    n = rows * cols
+    seq = Seq(lib)
+    x, row, col = seq.dev(r.standard_normal(n).astype(np.float32)), seq.dev(r.standard_normal(cols).astype(np.float32)), seq.dev(r.standard_normal(rows).astype(np.float32))
+    a, b, s, c, d = seq.out(n * 4, "f4"), seq.out(n * 4, "f4"), seq.out(rows * 4, "f4"), seq.out(n * 4, "f4"), seq.out(n * 4, "f4")
+    seq.add("add_f32", n, 2, u64([rows, cols], [cols, 1], [0, 1], 0, 0), x.ptr, row.ptr, a.ptr)       # + [1, cols]
+    seq.add("mul_f32", n, 2, u64([rows, cols], [cols, 1], [1, 0], 0, 0), a.ptr, col.ptr, b.ptr)       # * [rows, 1]
+    seq.add("sum_f32", n, 2, 1, u64([rows, cols], [cols, 1], [cols], [1], 0), b.ptr, s.ptr)            # a kernel node: the group before it runs first
+    seq.add("sub_f32", n, 2, u64([rows, cols], [cols, 1], [1, 0], 0, 0), b.ptr, s.ptr, c.ptr)         # reads the reduction's result
+    seq.add("relu_f32", n, 2, u64([rows, cols], [cols, 1], 0), c.ptr, d.ptr)
+    launches, nodes = fused(lib, seq)
+    assert launches == 4 and nodes == 3          # [add, mul], the reduction's kernel node, [sub], [relu: collapses to one dim]
+
+
+def test_fusion_can_be_switched_off(lib):
+    r = np.random.default_rng(14)
+    n = 1000
+    seq = Seq(lib)
+    x = seq.dev(r.standard_normal(n).astype(np.float32))
+    a, b = seq.out(n * 4, "f4"), seq.out(n * 4, "f4")
+    seq.add("exp_f32", n, 1, u64([n], [1], 0), x.ptr, a.ptr)
+    seq.add("neg_f32", n, 1, u64([n], [1], 0), a.ptr, b.ptr)
+    was = lib.hip_graph_set_fusion(0)
+    try:
+        fused(lib, seq, want_launches=0, want_nodes=0, replays=1)
+    finally:
+        lib.hip_graph_set_fusion(was)
+    fused(lib, seq, want_launches=2, want_nodes=1, replays=1)
