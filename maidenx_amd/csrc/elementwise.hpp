@@ -369,7 +369,7 @@ inline bool ew_fuse(bool vec, const NdSpace<Op::NIN + 1>& sp, const EwPtrs<Op::N
         }
         for (int k = 0; k < Op::NIN; ++k) c.in[k] = p.in[k];
         if (vec && c.os[sp.ndims - 1] != 1) return false;
-        return fuse_record(c, (uint32_t)sp.ndims, sp.dims, vec, n, sizeof(float));
+        return fuse_record(c, (uint32_t)sp.ndims, sp.dims, vec, n, sizeof(float));      // (a tiny member is taken element by element whatever `vec` says)
     }
     return false;
 }

@@ -44,16 +44,26 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
     }
     __syncthreads();
     const size_t v = (size_t)blockIdx.x * EW_BLOCK + threadIdx.x;
-    if (v >= g.nvec) return;
+    const bool tiny = g.tiny != 0;               // one block; every thread stays for the barriers
+    if (!tiny && v >= g.nvec) return;
     // coordinates of this thread's first element over (outer, inner); one dim: everything is "inner"
     uint32_t c0 = 0, c1 = (uint32_t)v * VEC;
-    if (g.ndims == 2) fd_divmod((uint32_t)v * VEC, g.div_inner, c0, c1);
-    const int inner = g.ndims == 2 ? 1 : 0;
+    uint32_t ndims = g.ndims;
+    if (!tiny && ndims == 2) fd_divmod((uint32_t)v * VEC, g.div_inner, c0, c1);
     AVec<float, VEC> r;          // what the previous member wrote at this thread's elements
 #pragma unroll
     for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f;
     for (uint32_t k = 0; k < g.n; ++k) {
         const FuseCmd& c = sg.cmd[k];
+        if (tiny) {
+            if (k) __syncthreads();              // the member before may have written what this one reads, anywhere
+            if (v >= c.nel) continue;
+            ndims = c.ndims;
+            c0 = 0;
+            c1 = (uint32_t)v;
+            if (ndims == 2) { c0 = (uint32_t)v / c.dims[1]; c1 = (uint32_t)v - c0 * c.dims[1]; }
+        }
+        const int inner = ndims == 2 ? 1 : 0;
         float val[2][VEC];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -68,7 +78,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
                 continue;
             }
             const int64_t s = c.is[j][inner];
-            const float* src = (const float*)c.in[j] + (g.ndims == 2 ? (int64_t)c0 * c.is[j][0] : 0) + (int64_t)c1 * s;
+            const float* src = (const float*)c.in[j] + (ndims == 2 ? (int64_t)c0 * c.is[j][0] : 0) + (int64_t)c1 * s;
             if (VEC > 1 && s == 1) {
                 const AVec<float, VEC> t = *(const AVec<float, VEC>*)src;
 #pragma unroll
@@ -86,7 +96,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
             MXH_FC8(0) MXH_FC8(8) MXH_FC8(16) MXH_FC8(24) MXH_FC8(32) MXH_FC8(40) MXH_FC8(48) MXH_FC8(56)
             default: break;
         }
-        float* dst = (float*)c.out + (g.ndims == 2 ? (int64_t)c0 * c.os[0] : 0) + (int64_t)c1 * c.os[inner];
+        float* dst = (float*)c.out + (ndims == 2 ? (int64_t)c0 * c.os[0] : 0) + (int64_t)c1 * c.os[inner];
         if (VEC > 1) {
             *(AVec<float, VEC>*)dst = r;
         } else {
@@ -96,7 +106,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
 }
 
 void fuse_launch(const FuseGroup& g, void* stream_) {
-    const unsigned blocks = cdiv(g.nvec, (size_t)EW_BLOCK);
+    const unsigned blocks = g.tiny ? 1u : cdiv(g.nvec, (size_t)EW_BLOCK);
     if (g.vec) hipLaunchKernelGGL(ew_group_kernel<4>, dim3(blocks), dim3(EW_BLOCK), 0, (hipStream_t)stream_, g);
     else hipLaunchKernelGGL(ew_group_kernel<1>, dim3(blocks), dim3(EW_BLOCK), 0, (hipStream_t)stream_, g);
     MXH_HIP(hipGetLastError());

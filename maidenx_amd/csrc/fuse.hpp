@@ -9,6 +9,8 @@
 // next thing queued on the stream, by a launch that does not fit, or by the end of the capture, and becomes ONE
 // kernel node that applies the members in order per element.  Every output is still written; results are the bytes
 // of the separate launches.
+// Members of at most 256 elements (a bias, a 3-element weight, a loss) need none of this care: a group of those is
+// run by a single work-group with a barrier between members, whatever their shapes and however they overlap.
 #pragma once
 #include <cstddef>
 #include <cstdint>
@@ -26,11 +28,15 @@ struct FuseCmd {
     uint32_t op;              // position of the functor in EwProgOps
     uint32_t nin;
     uint32_t fwd;             // bit j: input j is, element for element, what the previous member wrote (taken from registers)
+    uint32_t ndims;           // the member's own space: only read in a tiny group
+    uint32_t dims[2];
+    uint32_t nel;
     uint32_t reserved;
     uint32_t payload[2];      // the functor's state (a scalar constant), bit for bit
 };
 struct alignas(16) FuseGroup {
     uint32_t n, ndims, vec;   // vec: every member moves 16-byte vectors along the inner dim
+    uint32_t tiny;            // 1: members of at most one block's worth of elements each, any shapes, run by ONE block with a barrier between them
     uint32_t dims[2];
     FastDiv div_inner;
     size_t nvec;              // vectors (vec) or elements per member

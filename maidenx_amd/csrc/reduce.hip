@@ -234,9 +234,26 @@ void row_stage(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks,
     else launch_row<TIn, TOut, R, RB>(in, out, rows, L, chunks, chunk_len, div, src_bf16);
 }
 
+// `0 + x` per element: what an all-kept sum_to_shape does through its zero-initialised cells (−0 → +0), and what a
+// sum over an axis of length 1 is.
+template <class T> struct OpZeroPlus {
+    using In = T; using Out = T; static constexpr int NIN = 1;
+    __device__ T operator()(T x) const { return IO<T>::fin(0.0f + IO<T>::ld(x), 0.0f); }
+};
+
 // rows of length L (contiguous) → out[rows]
 template <class TIn, class TOut, class R>
 void row_reduce(const TIn* in, TOut* out, size_t rows, size_t L, float div, bool src_bf16) {
+    if constexpr (std::is_same<TIn, TOut>::value && std::is_same<R, RSum>::value) {
+        if (L == 1 && div == 0.0f) {
+            // one term per row: the sum is `0 + x`, an elementwise launch (which a capture can fuse with its neighbours)
+            size_t dims = rows, unit = 1;
+            const size_t* ins[1] = {&unit};
+            const void* inp[1] = {in};
+            ew_launch<OpZeroPlus<TIn>>(rows, 1, &dims, &unit, ins, out, inp, OpZeroPlus<TIn>{});
+            return;
+        }
+    }
     unsigned chunks = 1;
     size_t chunk_len = L;
     if (rows < TARGET_BLOCKS / 4 && L >= 16384) {
@@ -429,11 +446,6 @@ void reduce_axis(size_t num_els, size_t num_dims, size_t nred, const size_t* md,
 }
 
 // ---- sum_to_shape -----------------------------------------------------------------------------------
-// `0 + x` per element: what an all-kept sum_to_shape does through its zero-initialised cells (−0 → +0).
-template <class T> struct OpZeroPlus {
-    using In = T; using Out = T; static constexpr int NIN = 1;
-    __device__ T operator()(T x) const { return IO<T>::fin(0.0f + IO<T>::ld(x), 0.0f); }
-};
 
 // Non-contiguous input: gather into a contiguous copy with the reference's index rule
 // (reduction.rs:162-167): element (Σ coords·strides + offset) mod num_els of the already-offset slice.

@@ -88,6 +88,34 @@ bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool ve
     if (!g_capturing || !g_fuse_enabled || g_prog_ok || ndims < 1 || ndims > 2) return false;
     for (uint32_t d = 0; d < ndims; ++d)
         if (c.os[d] < 0 || c.is[0][d] < 0 || (c.nin > 1 && c.is[1][d] < 0)) return false;
+    // at most one block's worth of elements, one per thread: such members form groups of their own, in which a barrier
+    // between members orders everything (any shapes, any overlaps)
+    size_t nel = 1;
+    for (uint32_t d = 0; d < ndims; ++d) nel *= dims[d];
+    const bool tiny = nel <= 256;
+    if (tiny) {
+        if (!(g_fuse.n > 0 && g_fuse.tiny && g_fuse.n < (uint32_t)FUSE_MAX_CMDS)) {
+            fuse_flush();
+            g_fuse.tiny = 1;
+            g_fuse.vec = 0;
+            g_fuse.ndims = 1;
+            g_fuse.nvec = 256;
+            g_fuse.dims[0] = 256;
+            g_fuse.dims[1] = 1;
+            g_fuse.div_inner = make_fastdiv(1);
+            g_fuse_elem_bytes = elem_bytes;
+        }
+        FuseCmd& slot = g_fuse.cmd[g_fuse.n++];
+        slot = c;
+        slot.fwd = 0;            // the forwarded registers belong to another member's thread layout
+        slot.ndims = ndims;
+        slot.dims[0] = dims[0];
+        slot.dims[1] = ndims == 2 ? dims[1] : 1;
+        slot.nel = (uint32_t)nel;
+        ++g_fused_launches;
+        return true;
+    }
+    if (g_fuse.n > 0 && g_fuse.tiny) fuse_flush();
     const bool fits = g_fuse.n > 0 && g_fuse.n < (uint32_t)FUSE_MAX_CMDS && g_fuse.ndims == ndims && g_fuse.vec == (vec ? 1u : 0u) &&
                       g_fuse.nvec == nvec && g_fuse.dims[0] == dims[0] && (ndims == 1 || g_fuse.dims[1] == dims[1]) && g_fuse_elem_bytes == elem_bytes;
     bool join = fits;
@@ -116,6 +144,7 @@ bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool ve
     }
     if (!join) {
         fuse_flush();
+        g_fuse.tiny = 0;
         g_fuse.ndims = ndims;
         g_fuse.vec = vec ? 1u : 0u;
         g_fuse.nvec = nvec;

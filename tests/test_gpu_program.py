@@ -322,6 +322,24 @@ def test_fused_two_dim_broadcast_and_a_reduction_in_between(lib):
     assert launches == 4 and nodes == 3          # [add, mul], the reduction's kernel node, [sub], [relu: collapses to one dim]
 
 
+def test_fused_tiny_members_of_any_shape_share_one_block(lib):
+    """Members of at most 256 elements are run by one work-group with a barrier between them: different shapes, a
+    broadcast of what the member before wrote, a shifted view and an in-place update all stay in one node."""
+    r = np.random.default_rng(15)
+    seq = Seq(lib)
+    w, b = seq.dev(r.standard_normal(3).astype(np.float32)), seq.dev(r.standard_normal(1).astype(np.float32))
+    x = seq.dev(r.standard_normal(200).astype(np.float32))
+    gw, gb, t1, t2, t3, t4 = seq.out(3 * 4, "f4"), seq.out(4, "f4"), seq.out(200 * 4, "f4"), seq.out(199 * 4, "f4"), seq.out(12 * 16 * 4, "f4"), seq.out(3 * 4, "f4")
+    seq.add("mul_scalar_f32", 3, 1, u64([3], [1], 0), w.ptr, C.c_float(0.01), gw.ptr)
+    seq.add("mul_scalar_f32", 1, 1, u64([1], [1], 0), b.ptr, C.c_float(0.01), gb.ptr)
+    seq.add("add_f32", 200, 1, u64([200], [1], [0], 0, 0), x.ptr, gb.ptr, t1.ptr)                  # broadcast of the member before
+    seq.add("sub_f32", 199, 1, u64([199], [1], [1], 0, 1), x.ptr, t1.ptr, t2.ptr)                  # shifted view of it
+    seq.add("mul_f32", 192, 2, u64([12, 16], [16, 1], [1, 12], 0, 0), t1.ptr, t2.ptr, t3.ptr)      # transposed read
+    seq.add("sub_inplace_f32", 3, 1, u64([3], [1], [1], 0, 0), gw.ptr, w.ptr)
+    seq.add("add_f32", 3, 1, u64([3], [1], [0], 0, 0), gw.ptr, gb.ptr, t4.ptr)
+    fused(lib, seq, want_launches=7, want_nodes=1)
+
+
 def test_fusion_can_be_switched_off(lib):
     r = np.random.default_rng(14)
     n = 1000
