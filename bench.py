@@ -637,7 +637,7 @@ def run_mlp(args):
     from maidenx_amd.tensor import host
     mx = host()
     lin, x, y = _mlp_setup(mx)
-    steps = max(args.steps, 200)
+    steps = max(args.steps, 1000)          # the example's own 1000 epochs: the eager epochs and the capture inside the call are part of the job
     mx.train(lin, x, y, 0.01, max(args.warmup, 20))
     mx.synchronize()
     mx.reset_backend_calls()
@@ -648,7 +648,7 @@ def run_mlp(args):
     calls = mx.backend_calls() / steps
     a = argparse.Namespace(steps=steps, warmup=max(args.warmup, 20))
     result = base_result(a, round(steps / dt_s, 1), "steps/s", dt_s, "f32",
-                         "configs[0]: README Linear(3->1, bias) + MSE + SGD(lr=0.01), f32, full batch 10000x3",
+                         "configs[0]: README Linear(3->1, bias) + MSE + SGD(lr=0.01), f32, full batch 10000x3, 1000 epochs as in examples/device/cpu.rs",
                          {"backend_kernels_per_step": calls, "us_per_step": round(dt_s / steps * 1e6, 1)})
     result["roofline"] = None
     result["note"] = "launch-latency bound (about 200 KB touched per step): no roofline fraction applies"
