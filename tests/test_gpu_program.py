@@ -354,3 +354,93 @@ def test_fusion_can_be_switched_off(lib):
     finally:
         lib.hip_graph_set_fusion(was)
     fused(lib, seq, want_launches=2, want_nodes=1, replays=1)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_random_sequences_with_aliasing(lib, seed):
+    """Random chains over a small pool of buffers, with views that overlap in every way (same elements, shifted,
+    broadcast, transposed, in place): whatever the grouping decides, a replay must leave the bytes of the eager run
+    in every buffer."""
+    r = np.random.default_rng(1000 + seed)
+    n = int(r.choice([1, 3, 64, 200, 1024, 4096, 10000]))
+    rows = int(r.choice([d for d in (1, 2, 4, 8, 16, 64) if n % d == 0]))
+    cols = n // rows
+    pool = [L.DeviceBuffer.from_numpy(r.standard_normal(n + 8).astype(np.float32)) for _ in range(5)]
+    start = [p.to_numpy(np.float32).copy() for p in pool]
+    esz = 4
+
+    def view(kind, avoid=None):
+        """(pointer, dims, strides) of a view into a random pool buffer, (buffer index) appended; `avoid`: a buffer the
+        view must not touch unless it is the plain view of it (an op whose output overlaps its own input in any other
+        way races with itself even as a single launch)"""
+        bi = int(r.integers(0, len(pool)))
+        if avoid is not None and bi == avoid and kind != "flat":
+            bi = (bi + 1) % len(pool)
+        b = pool[bi]
+        if kind == "flat":
+            return b.ptr, [n], [1]
+        if kind == "shift":
+            return b.ptr + esz * int(r.integers(1, 8)), [n], [1]
+        if kind == "bcast":
+            return b.ptr + esz * int(r.integers(0, 8)), [n], [0]
+        if kind == "rowb":
+            return b.ptr, [rows, cols], [0, 1]
+        if kind == "colb":
+            return b.ptr, [rows, cols], [1, 0]
+        return b.ptr, [rows, cols], [1, rows]                      # transposed read of the same n elements
+
+    calls = []
+    for _ in range(int(r.integers(4, 14))):
+        two_d = r.random() < 0.3
+        out_i = int(r.integers(0, len(pool)))
+        out_shift = 0 if r.random() < 0.8 else int(r.integers(1, 8))
+        out_ptr = pool[out_i].ptr + esz * out_shift
+        kinds = ["flat", "flat", "flat", "shift", "bcast"] + (["rowb", "colb", "tr"] if two_d else [])
+        # inputs from other buffers, or exactly the output's own elements
+        def operand():
+            k = str(r.choice(kinds))
+            v = view(k, avoid=out_i)
+            if v[0] == pool[out_i].ptr and out_shift:          # the plain view of the output's buffer under a shifted output
+                return (out_ptr, v[1], v[2])
+            return v
+        a, b = operand(), operand()
+        dims = [rows, cols] if two_d else [n]
+        full = lambda v: (v[2] if len(v[1]) == len(dims) else ([cols * v[2][0], v[2][0]] if two_d else v[2]))
+        sa, sb = full(a), full(b)
+        op = str(r.choice(["add", "mul", "sub", "neg", "relu", "mul_scalar", "add_inplace", "square"]))
+        nd = len(dims)
+        if op in ("add", "mul", "sub"):
+            calls.append((f"{op}_f32", (n, nd, u64(dims, sa, sb, 0, 0), a[0], b[0], out_ptr)))
+        elif op == "add_inplace":
+            calls.append(("add_inplace_f32", (n, nd, u64(dims, [cols, 1] if two_d else [1], sb, 0, 0), out_ptr, b[0])))
+        elif op == "mul_scalar":
+            calls.append(("mul_scalar_f32", (n, nd, u64(dims, sa, 0), a[0], C.c_float(0.5), out_ptr)))
+        else:
+            calls.append((f"{op}_f32", (n, nd, u64(dims, sa, 0), a[0], out_ptr)))
+
+    def run():
+        for name, args in calls:
+            getattr(lib, "hip_" + name)(*[x.ctypes.data if isinstance(x, np.ndarray) else x for x in args])
+
+    def reset():
+        for p, s in zip(pool, start):
+            assert lib.hip_memcpy_h2d(p.ptr, s.ctypes.data, s.nbytes) == 0
+
+    run()
+    assert lib.hip_synchronize() == 0 and lib.hip_get_last_status() == 0, lib.hip_status_string()
+    want = [p.to_numpy(np.float32).copy() for p in pool]
+    big = L.DeviceBuffer(1 << 20)
+    assert lib.hip_graph_begin_capture() == 0
+    lib.hip_fill_f32((1 << 20) // 4, big.ptr, C.c_float(0.0))
+    run()
+    h = C.c_void_p()
+    assert lib.hip_graph_end_capture(C.byref(h)) == 0
+    try:
+        for _ in range(2):
+            reset()
+            assert lib.hip_graph_launch(h) == 0 and lib.hip_synchronize() == 0
+            for k, (p, w) in enumerate(zip(pool, want)):
+                got = p.to_numpy(np.float32)
+                assert got.tobytes() == w.tobytes(), (seed, k, n, [c[0] for c in calls])
+    finally:
+        assert lib.hip_graph_destroy(h) == 0
