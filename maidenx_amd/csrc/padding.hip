@@ -142,49 +142,92 @@ static bool make_pad3(const PadSpace& sp, Pad3& p3) {
     return ost < (1ull << 31);
 }
 
-template <class T, bool FWD, int Q>
+// A thread owns U vectors of Q consecutive output elements, PB*Q apart, and issues the loads of all of them before the
+// first store: one vector per thread leaves too few bytes in flight per CU to cover the memory latency.  Forward loads
+// are unconditional (position 0 stands in for an element outside the input), so none of them waits on a branch.
+template <class T, bool FWD, int Q, int U>
 __global__ __launch_bounds__(PB) void pad_const3_kernel(Pad3 sp, const T* __restrict__ src, T* __restrict__ dst, uint32_t n_out, T pad_value) {
-    const uint32_t i0 = (blockIdx.x * PB + threadIdx.x) * Q;
-    if (i0 >= n_out) return;
-    uint32_t q, c2, c1, c0;
-    fd_divmod(i0, sp.out_div[2], q, c2);
-    fd_divmod(q, sp.out_div[1], c0, c1);
-    const bool full = i0 + Q <= n_out;
-    AVec<T, Q> v;
-    if constexpr (!FWD) {
-        if (full) v = *(const AVec<T, Q>*)(src + i0);
-        else
-            for (int e = 0; e < Q; ++e) v.v[e] = i0 + e < n_out ? src[i0 + e] : T{};
-    }
-    int64_t row = 0;
-    bool row_in = false, fresh = true;
-#pragma unroll
-    for (int e = 0; e < Q; ++e) {
-        if (fresh) {
-            const uint32_t i0c = c0 - sp.before[0], i1c = c1 - sp.before[1];      // wrap when outside: fail the test
-            row_in = i0c < sp.in[0] && i1c < sp.in[1];
-            row = (int64_t)i0c * sp.in_stride[0] + (int64_t)i1c * sp.in_stride[1];
-            fresh = false;
-        }
-        const uint32_t ic = c2 - sp.before[2];
-        const bool inside = row_in && ic < sp.in[2] && (full || i0 + e < n_out);
-        const int64_t idx = row + (int64_t)ic * sp.in_stride[2];
-        if constexpr (FWD) {
-            v.v[e] = inside ? src[idx] : pad_value;
-        } else {
-            if (inside) dst[idx] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(v.v[e]));      // -0 -> +0 like the reference's sums from zero
-        }
-        if (++c2 == sp.out[2]) {
-            c2 = 0;
-            fresh = true;
-            if (++c1 == sp.out[1]) { c1 = 0; ++c0; }
-        }
-    }
+    const uint32_t base = (blockIdx.x * (uint32_t)(U * PB) + threadIdx.x) * Q;
+    AVec<T, Q> v[U];
     if constexpr (FWD) {
-        if (full) *(AVec<T, Q>*)(dst + i0) = v;
-        else
+        bool in_mask[U][Q];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t i0 = base + (uint32_t)u * (PB * Q);
+            const bool live = i0 < n_out;
+            uint32_t q, c2, c1, c0;
+            fd_divmod(live ? i0 : 0u, sp.out_div[2], q, c2);
+            fd_divmod(q, sp.out_div[1], c0, c1);
+            int64_t row = 0;
+            bool row_in = false, fresh = true;
+#pragma unroll
+            for (int e = 0; e < Q; ++e) {
+                if (fresh) {
+                    const uint32_t i0c = c0 - sp.before[0], i1c = c1 - sp.before[1];      // wrap when outside: fail the test
+                    row_in = i0c < sp.in[0] && i1c < sp.in[1];
+                    row = (int64_t)i0c * sp.in_stride[0] + (int64_t)i1c * sp.in_stride[1];
+                    fresh = false;
+                }
+                const uint32_t ic = c2 - sp.before[2];
+                const bool inside = live && row_in && ic < sp.in[2] && i0 + e < n_out;
+                const int64_t idx = row + (int64_t)ic * sp.in_stride[2];
+                in_mask[u][e] = inside;
+                v[u].v[e] = src[inside ? idx : 0];
+                if (++c2 == sp.out[2]) {
+                    c2 = 0;
+                    fresh = true;
+                    if (++c1 == sp.out[1]) { c1 = 0; ++c0; }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t i0 = base + (uint32_t)u * (PB * Q);
+            if (i0 >= n_out) continue;
+#pragma unroll
             for (int e = 0; e < Q; ++e)
-                if (i0 + e < n_out) dst[i0 + e] = v.v[e];
+                if (!in_mask[u][e]) v[u].v[e] = pad_value;
+            if (i0 + Q <= n_out) *(AVec<T, Q>*)(dst + i0) = v[u];
+            else
+                for (int e = 0; e < Q; ++e)
+                    if (i0 + e < n_out) dst[i0 + e] = v[u].v[e];
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t i0 = base + (uint32_t)u * (PB * Q);
+            if (i0 + Q <= n_out) v[u] = *(const AVec<T, Q>*)(src + i0);
+            else
+                for (int e = 0; e < Q; ++e) v[u].v[e] = i0 + e < n_out ? src[i0 + e] : T{};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t i0 = base + (uint32_t)u * (PB * Q);
+            if (i0 >= n_out) continue;
+            uint32_t q, c2, c1, c0;
+            fd_divmod(i0, sp.out_div[2], q, c2);
+            fd_divmod(q, sp.out_div[1], c0, c1);
+            int64_t row = 0;
+            bool row_in = false, fresh = true;
+#pragma unroll
+            for (int e = 0; e < Q; ++e) {
+                if (fresh) {
+                    const uint32_t i0c = c0 - sp.before[0], i1c = c1 - sp.before[1];
+                    row_in = i0c < sp.in[0] && i1c < sp.in[1];
+                    row = (int64_t)i0c * sp.in_stride[0] + (int64_t)i1c * sp.in_stride[1];
+                    fresh = false;
+                }
+                const uint32_t ic = c2 - sp.before[2];
+                const bool inside = row_in && ic < sp.in[2] && i0 + e < n_out;
+                const int64_t idx = row + (int64_t)ic * sp.in_stride[2];
+                if (inside) dst[idx] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(v[u].v[e]));      // -0 -> +0 like the reference's sums from zero
+                if (++c2 == sp.out[2]) {
+                    c2 = 0;
+                    fresh = true;
+                    if (++c1 == sp.out[1]) { c1 = 0; ++c0; }
+                }
+            }
+        }
     }
 }
 
@@ -192,6 +235,17 @@ template <class T>
 __global__ __launch_bounds__(PB) void zero_kernel(T* p, size_t n) {
     size_t i = (size_t)blockIdx.x * PB + threadIdx.x;
     if (i < n) p[i] = T{};
+}
+
+// Four vectors per thread once that still leaves every CU several blocks; one otherwise.
+template <class T, bool FWD>
+static void pad_const3_launch(const Pad3& p3, const T* src, T* dst, size_t n_out, T pad_value) {
+    constexpr int Q = 16 / sizeof(T);
+    const size_t vecs = cdiv(n_out, (size_t)Q);
+    if (vecs >= (size_t)PB * 4 * 1024)
+        hipLaunchKernelGGL((pad_const3_kernel<T, FWD, Q, 4>), dim3(cdiv(vecs, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, src, dst, (uint32_t)n_out, pad_value);
+    else
+        hipLaunchKernelGGL((pad_const3_kernel<T, FWD, Q, 1>), dim3(cdiv(vecs, (size_t)PB)), dim3(PB), 0, stream(), p3, src, dst, (uint32_t)n_out, pad_value);
 }
 
 static bool build_space(size_t nd, const size_t* md, PadSpace& sp, size_t* in_off, bool* cont, bool* exact) {
@@ -246,8 +300,11 @@ void pad_forward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const T
     if (!build_space(nd, md, sp, &off, &cont, &exact)) { set_status(ERR_UNSUPPORTED, "pad: rank above 8 after collapse"); return; }
     constexpr int Q = 16 / sizeof(T);
     Pad3 p3;
-    if ((uintptr_t)out % 16 == 0 && make_pad3(sp, p3))
-        hipLaunchKernelGGL((pad_const3_kernel<T, true, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), p3, in + off, out, (uint32_t)n_out, pad_value);
+    size_t logical = 1;
+    for (size_t d = 0; d < nd; ++d) logical *= md[d];
+    // (the three-dim kernel reads the input's first element in place of one outside it: not for an empty input)
+    if ((uintptr_t)out % 16 == 0 && logical > 0 && make_pad3(sp, p3))
+        pad_const3_launch<T, true>(p3, in + off, out, n_out, pad_value);
     else if ((uintptr_t)out % 16 == 0)
         hipLaunchKernelGGL((pad_const_kernel<T, true, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), sp, in + off, out, n_out, pad_value);
     else
@@ -257,37 +314,48 @@ void pad_forward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const T
 
 // Backward of a constant pad onto a contiguous input that every output position of the interior maps to: a
 // crop.  A thread owns four consecutive input elements (one vector store); `0 + g` as in the scatter form.
-template <class T>
+template <class T, int U>
 __global__ __launch_bounds__(PB) void pad_crop3_kernel(Pad3 sp, const T* __restrict__ go, T* __restrict__ gi, uint32_t n_in, bool vec_store) {
     constexpr uint32_t PER = 4;
-    const uint32_t i0 = (blockIdx.x * PB + threadIdx.x) * PER;
-    if (i0 >= n_in) return;
-    uint32_t p0, p1, p2, q;
-    fd_divmod(i0, sp.in_div[2], q, p2);
-    fd_divmod(q, sp.in_div[1], p0, p1);
-    uint32_t row = 0;
-    bool fresh = true;
-    AVec<T, PER> v;
+    const uint32_t base = (blockIdx.x * (uint32_t)(U * PB) + threadIdx.x) * PER;
+    AVec<T, PER> v[U];
 #pragma unroll
-    for (uint32_t e = 0; e < PER; ++e) {
-        if (i0 + e >= n_in) break;
-        if (fresh) {
-            row = (p0 + sp.before[0]) * sp.out_stride[0] + (p1 + sp.before[1]) * sp.out_stride[1] + sp.before[2];
-            fresh = false;
-        }
-        v.v[e] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(go[row + p2]));
-        if (++p2 == sp.in[2]) {
-            p2 = 0;
-            fresh = true;
-            if (++p1 == sp.in[1]) { p1 = 0; ++p0; }
+    for (int u = 0; u < U; ++u) {
+        const uint32_t i0 = base + (uint32_t)u * (PB * PER);
+        const bool live = i0 < n_in;
+        uint32_t p0, p1, p2, q;
+        fd_divmod(live ? i0 : 0u, sp.in_div[2], q, p2);
+        fd_divmod(q, sp.in_div[1], p0, p1);
+        uint32_t row = 0;
+        bool fresh = true;
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e) {
+            if (fresh) {
+                row = (p0 + sp.before[0]) * sp.out_stride[0] + (p1 + sp.before[1]) * sp.out_stride[1] + sp.before[2];
+                fresh = false;
+            }
+            const bool ok = live && i0 + e < n_in;           // every load is issued; position 0 of the first row stands in past the end
+            v[u].v[e] = go[ok ? row + p2 : sp.before[0] * sp.out_stride[0] + sp.before[1] * sp.out_stride[1] + sp.before[2]];
+            if (++p2 == sp.in[2]) {
+                p2 = 0;
+                fresh = true;
+                if (++p1 == sp.in[1]) { p1 = 0; ++p0; }
+            }
         }
     }
-    if (vec_store && i0 + PER <= n_in) {
-        *(AVec<T, PER>*)(gi + i0) = v;
-    } else {
 #pragma unroll
-        for (uint32_t e = 0; e < PER; ++e)
-            if (i0 + e < n_in) gi[i0 + e] = v.v[e];
+    for (int u = 0; u < U; ++u) {
+        const uint32_t i0 = base + (uint32_t)u * (PB * PER);
+        if (i0 >= n_in) continue;
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e) v[u].v[e] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(v[u].v[e]));
+        if (vec_store && i0 + PER <= n_in) {
+            *(AVec<T, PER>*)(gi + i0) = v[u];
+        } else {
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e)
+                if (i0 + e < n_in) gi[i0 + e] = v[u].v[e];
+        }
     }
 }
 
@@ -308,16 +376,19 @@ void pad_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, const 
     Pad3 p3;
     size_t logical = 1;
     for (size_t d = 0; d < nd; ++d) logical *= md[d];
-    if (cont && exact && logical == n_in && logical < (1ull << 31) && make_pad3(sp, p3)) {
+    if (cont && exact && logical == n_in && logical > 0 && logical < (1ull << 31) && make_pad3(sp, p3)) {
         // every input position is read back from exactly one output position: gather by input element, which
         // keeps the stores whole vectors
-        hipLaunchKernelGGL(pad_crop3_kernel<T>, dim3(cdiv(logical, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, go, gi + off, (uint32_t)logical,
-                           (uintptr_t)(gi + off) % (4 * sizeof(T)) == 0);
+        const bool vec_store = (uintptr_t)(gi + off) % (4 * sizeof(T)) == 0;
+        if (logical >= (size_t)PB * 16 * 1024)
+            hipLaunchKernelGGL((pad_crop3_kernel<T, 4>), dim3(cdiv(logical, (size_t)PB * 16)), dim3(PB), 0, stream(), p3, go, gi + off, (uint32_t)logical, vec_store);
+        else
+            hipLaunchKernelGGL((pad_crop3_kernel<T, 1>), dim3(cdiv(logical, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, go, gi + off, (uint32_t)logical, vec_store);
         MXH_LAUNCH_CHECK("pad_const_backward");
         return;
     }
     if ((uintptr_t)go % 16 == 0 && make_pad3(sp, p3))
-        hipLaunchKernelGGL((pad_const3_kernel<T, false, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), p3, go, gi + off, (uint32_t)n_out, T{});
+        pad_const3_launch<T, false>(p3, go, gi + off, n_out, T{});
     else if ((uintptr_t)go % 16 == 0)
         hipLaunchKernelGGL((pad_const_kernel<T, false, Q>), dim3(cdiv(cdiv(n_out, Q), PB)), dim3(PB), 0, stream(), sp, go, gi + off, n_out, T{});
     else
