@@ -121,6 +121,20 @@ int hip_graph_set_fusion(int enabled);
 MX_DECL_BINARY(float, f32)
 MX_DECL_BINARY(mx_bf16, bf16)
 MX_DECL_BINARY(mx_f16, f16)
+/* The rest of the family's dtypes (crates/maidenx_cuda/src/ops/binary.rs:172-181).  Integers saturate on add / sub /
+ * mul; a zero divisor gives 0 for 0/0 and otherwise the largest (negative dividend: the smallest) value, MIN / -1
+ * gives MAX; bool: add = maximum = or, sub = div = minimum = and, mul = xor
+ * (crates/maidenx_cpu/src/ops/binary.rs:374-410, 457-578, 584-606). */
+MX_DECL_BINARY(double, f64)
+MX_DECL_BINARY(mx_bool, bool)
+MX_DECL_BINARY(uint8_t, u8)
+MX_DECL_BINARY(uint16_t, u16)
+MX_DECL_BINARY(uint32_t, u32)
+MX_DECL_BINARY(uint64_t, u64)
+MX_DECL_BINARY(int8_t, i8)
+MX_DECL_BINARY(int16_t, i16)
+MX_DECL_BINARY(int32_t, i32)
+MX_DECL_BINARY(int64_t, i64)
 
 /* ---- unary: replaces crates/maidenx_cuda/src/ops/unary.rs:21-77 ------------------------------------
  * metadata = dims[n] | strides[n] | offset   (NULL: contiguous).  input == NULL means "in place on

@@ -50,6 +50,20 @@ def signatures(dtypes=("f32", "bf16", "f16")):
     return sig
 
 
+WIDE_DTYPES = ("f64", "bool", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64")
+
+
+def binary_signatures(dtypes=WIDE_DTYPES):
+    """The binary / comparison / logical / in-place families for the dtypes that only they cover so far."""
+    sig = {}
+    for dt in dtypes:
+        for op in BINARY:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, P, P]
+        for op in INPLACE:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, P]
+    return sig
+
+
 def index_signatures(dtypes=("f32", "bf16", "f16")):
     """Index ops (host loops in the reference's tensor layer, device entry points here)."""
     sig = {}

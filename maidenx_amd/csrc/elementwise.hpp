@@ -435,7 +435,7 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
                 }
             }
             pl.super = 0;
-            if (trv) {
+            if constexpr (sizeof(In) == 2 || sizeof(In) == 4) if (trv) {      // (the vector tiles are laid out for 16- and 32-bit elements)
                 pl.tiles_p = cdiv(sp.dims[pd], TrvCfg<In>::TP);
                 pl.tiles_l = cdiv(sp.dims[last], TrvCfg<In>::TL);
                 pl.super = (pl.tiles_p % 8 == 0 && pl.tiles_l % 8 == 0) ? 1u : 0u;

@@ -4,6 +4,8 @@
 // `half` crate: arithmetic forms round after every operation, transcendental forms upcast,
 // evaluate in f32 and round once.
 #pragma once
+#include <limits>
+#include <type_traits>
 #include "mathfn.hpp"
 #include "mxh.hpp"
 
@@ -14,6 +16,7 @@ using bool_t = uint8_t;   // the reference's `bool` output buffers: one byte, 0 
 template <class T> struct Ar;
 template <> struct Ar<float> {
     using T = float;
+    static constexpr bool kFloat = true;
     static __device__ T zero() { return 0.0f; }
     static __device__ T inf() { return INFINITY; }
     static __device__ T from_f32(float v) { return v; }
@@ -28,6 +31,7 @@ template <> struct Ar<float> {
 };
 template <> struct Ar<bf16_t> {
     using T = bf16_t;
+    static constexpr bool kFloat = true;
     static __device__ T zero() { return T{0}; }
     static __device__ T inf() { return T{0x7F80}; }
     static __device__ T from_f32(float v) { return f2bf(v); }
@@ -42,6 +46,7 @@ template <> struct Ar<bf16_t> {
 };
 template <> struct Ar<f16_t> {       // the `half` crate's f16: the same "f32 operation, round" scheme as bf16
     using T = f16_t;
+    static constexpr bool kFloat = true;
     static __device__ T zero() { return T{0}; }
     static __device__ T inf() { return T{0x7C00}; }
     static __device__ T from_f32(float v) { return f2h(v); }
@@ -54,8 +59,84 @@ template <> struct Ar<f16_t> {       // the `half` crate's f16: the same "f32 op
     static __device__ T max_(T a, T b) { return h2f(a) > h2f(b) ? a : b; }
     static __device__ T min_(T a, T b) { return h2f(a) < h2f(b) ? a : b; }
 };
+template <> struct Ar<double> {      // binary.rs:373,387,401,445-456,583,597
+    using T = double;
+    static constexpr bool kFloat = true;
+    static __device__ T zero() { return 0.0; }
+    static __device__ T inf() { return (double)INFINITY; }
+    static __device__ T from_f32(float v) { return (double)v; }
+    static __device__ float to_f32(T v) { return (float)v; }
+    static __device__ T add(T a, T b) { return a + b; }
+    static __device__ T sub(T a, T b) { return a - b; }
+    static __device__ T mul(T a, T b) { return a * b; }
+    static __device__ T div(T a, T b) { return a / b; }
+    static __device__ T neg(T a) { return -a; }
+    static __device__ T max_(T a, T b) { return fmax(a, b); }
+    static __device__ T min_(T a, T b) { return fmin(a, b); }
+};
+// The reference's `bool` as an operand dtype: one byte holding 0 or 1 (binary.rs:374,388,402,457,584,598:
+// add = or, sub = and, mul = xor, div = and, maximum = or, minimum = and).
+struct b8_t { uint8_t bits; };
+template <> struct Ar<b8_t> {
+    using T = b8_t;
+    static constexpr bool kFloat = false;
+    static __device__ T add(T a, T b) { return T{(uint8_t)(a.bits | b.bits)}; }
+    static __device__ T sub(T a, T b) { return T{(uint8_t)(a.bits & b.bits)}; }
+    static __device__ T mul(T a, T b) { return T{(uint8_t)(a.bits ^ b.bits)}; }
+    static __device__ T divq(T a, T b) { return T{(uint8_t)(a.bits & b.bits)}; }
+    static __device__ T max_(T a, T b) { return T{(uint8_t)(a.bits | b.bits)}; }
+    static __device__ T min_(T a, T b) { return T{(uint8_t)(a.bits & b.bits)}; }
+};
+// Integers saturate (binary.rs:375-382, 389-396, 403-410); a zero divisor gives 0 for 0/0 and otherwise the
+// extreme value with the sign of the dividend, and MIN / -1 saturates to MAX (:458-578).
+template <class I> struct IntAr {
+    using T = I;
+    static constexpr bool kFloat = false;
+    static constexpr bool kSigned = std::is_signed<I>::value;
+    static constexpr I kMax = std::numeric_limits<I>::max(), kMin = std::numeric_limits<I>::min();
+    static __device__ T add(T a, T b) {
+        T r;
+        if (__builtin_add_overflow(a, b, &r)) return kSigned && b < 0 ? kMin : kMax;
+        return r;
+    }
+    static __device__ T sub(T a, T b) {
+        T r;
+        if (__builtin_sub_overflow(a, b, &r)) return !kSigned || b > 0 ? kMin : kMax;
+        return r;
+    }
+    static __device__ T mul(T a, T b) {
+        T r;
+        if (__builtin_mul_overflow(a, b, &r)) return kSigned && ((a < 0) != (b < 0)) ? kMin : kMax;
+        return r;
+    }
+    static __device__ T divq(T a, T b) {
+        if (b == 0) return a == 0 ? (T)0 : (kSigned && a < 0 ? kMin : kMax);
+        if constexpr (kSigned) {
+            if (a == kMin && b == (T)-1) return kMax;
+        }
+        return (T)(a / b);
+    }
+    static __device__ T max_(T a, T b) { return a > b ? a : b; }
+    static __device__ T min_(T a, T b) { return a < b ? a : b; }
+};
+template <> struct Ar<uint8_t> : IntAr<uint8_t> {};
+template <> struct Ar<uint16_t> : IntAr<uint16_t> {};
+template <> struct Ar<uint32_t> : IntAr<uint32_t> {};
+template <> struct Ar<uint64_t> : IntAr<uint64_t> {};
+template <> struct Ar<int8_t> : IntAr<int8_t> {};
+template <> struct Ar<int16_t> : IntAr<int16_t> {};
+template <> struct Ar<int32_t> : IntAr<int32_t> {};
+template <> struct Ar<int64_t> : IntAr<int64_t> {};
+
 template <class T> __device__ inline float F(T v) { return Ar<T>::to_f32(v); }
-template <class T> __device__ inline bool is_zero(T v) { return F(v) == 0.0f; }
+// the value comparisons and zero tests are made on: f32 for the three float formats stored in 32 or 16 bits (as the
+// reference's `half` types compare), the value itself for f64 and the integers, 0 / 1 for bool
+template <class T> __device__ inline auto V(T v) {
+    if constexpr (std::is_same<T, b8_t>::value) return (int)v.bits;
+    else if constexpr (std::is_same<T, double>::value || std::is_integral<T>::value) return v;
+    else return F(v);
+}
+template <class T> __device__ inline bool is_zero(T v) { return V(v) == 0; }
 
 // ---- binary --------------------------------------------------------------------------------
 #define MXH_BIN(NAME, OUT, EXPR)                                          \
@@ -67,18 +148,25 @@ MXH_BIN(OpAdd, T, A::add(a, b))
 MXH_BIN(OpSub, T, A::sub(a, b))
 MXH_BIN(OpMul, T, A::mul(a, b))
 // b == 0 ⇒ (a == 0 ? 0 : +INF) — the sign of a is ignored and a NaN a gives +INF
-MXH_BIN(OpDiv, T, is_zero(b) ? (is_zero(a) ? A::zero() : A::inf()) : A::div(a, b))
+template <class T> struct OpDiv {
+    using In = T; using Out = T; static constexpr int NIN = 2;
+    __device__ T operator()(T a, T b) const {
+        using A = Ar<T>;
+        if constexpr (A::kFloat) return is_zero(b) ? (is_zero(a) ? A::zero() : A::inf()) : A::div(a, b);
+        else return A::divq(a, b);
+    }
+};
 MXH_BIN(OpMaximum, T, A::max_(a, b))
 MXH_BIN(OpMinimum, T, A::min_(a, b))
 MXH_BIN(OpLogicalAnd, bool_t, (bool_t)(!is_zero(a) && !is_zero(b)))
 MXH_BIN(OpLogicalOr, bool_t, (bool_t)(!is_zero(a) || !is_zero(b)))
 MXH_BIN(OpLogicalXor, bool_t, (bool_t)(!is_zero(a) != !is_zero(b)))
-MXH_BIN(OpEq, bool_t, (bool_t)(F(a) == F(b)))
-MXH_BIN(OpNe, bool_t, (bool_t)(F(a) != F(b)))
-MXH_BIN(OpLt, bool_t, (bool_t)(F(a) < F(b)))
-MXH_BIN(OpLe, bool_t, (bool_t)(F(a) <= F(b)))
-MXH_BIN(OpGt, bool_t, (bool_t)(F(a) > F(b)))
-MXH_BIN(OpGe, bool_t, (bool_t)(F(a) >= F(b)))
+MXH_BIN(OpEq, bool_t, (bool_t)(V(a) == V(b)))
+MXH_BIN(OpNe, bool_t, (bool_t)(V(a) != V(b)))
+MXH_BIN(OpLt, bool_t, (bool_t)(V(a) < V(b)))
+MXH_BIN(OpLe, bool_t, (bool_t)(V(a) <= V(b)))
+MXH_BIN(OpGt, bool_t, (bool_t)(V(a) > V(b)))
+MXH_BIN(OpGe, bool_t, (bool_t)(V(a) >= V(b)))
 
 // ---- unary ---------------------------------------------------------------------------------
 // EXPR_F sees `x` as f32 and yields f32 (rounded once for bf16); EXPR_T, when given, works on

@@ -140,6 +140,19 @@ def run(flt="", sets=4, random_grad=False, out=sys.stdout):
         timeit(f"softmax_{dt}/[8192,8192] dim1", lambda: f(N, 2, 1, md.ctypes.data, x, z), 2 * N * e)
         timeit(f"softmax_{dt}/[8192,8192] dim0", lambda: f(N, 2, 0, md.ctypes.data, x, z), 2 * N * e, reps=5)
 
+    # ---- the binary family on the other dtypes: the 64 M-element buffers read as 1-, 4- and 8-byte elements ----------
+    for dt, e in (("u8", 1), ("i32", 4), ("i64", 8), ("f64", 8)):
+        x, y, z = buf("x", N * 4), buf("y", N * 4), buf("z", N * 4)
+        rows = R * 4 // e                                   # the same 256 MB per operand
+        n = rows * Cc
+        for op, out_e in (("add", e), ("lt", 1)):
+            f = getattr(lib, f"hip_{op}_{dt}")
+            md = u64([rows, Cc], cont, cont, 0, 0)
+            timeit(f"{op}_{dt}/contig", lambda: f(n, 2, md.ctypes.data, x, y, z), n * (2 * e + out_e))
+        md = u64([rows, Cc], cont, row, 0, 0)
+        f = getattr(lib, f"hip_mul_{dt}")
+        timeit(f"mul_{dt}/bcast_row", lambda: f(n, 2, md.ctypes.data, x, y, z), n * 2 * e)
+
     # ---- what the memory system gives a plain stream -------------------------------------------------------
     zf = buf("z", N * 4)
     timeit("fill_f32/268MB (write only)", lambda: lib.hip_fill_f32(N, zf, 1.0), N * 4)

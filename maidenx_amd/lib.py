@@ -27,7 +27,7 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise HipError(f"{LIB_PATH} is missing: build it with `python -m maidenx_amd.build` (needs hipcc)")
     lib = C.CDLL(LIB_PATH)
-    for name, args in {**S.signatures(), **S.extension_signatures()}.items():
+    for name, args in {**S.signatures(), **S.binary_signatures(), **S.extension_signatures()}.items():
         fn = getattr(lib, "hip_" + name)
         fn.argtypes = args
         fn.restype = None

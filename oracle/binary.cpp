@@ -79,13 +79,48 @@ template <typename T> inline T inf_of() { return std::numeric_limits<T>::infinit
 template <> inline bf16 inf_of<bf16>() { return bf16::from_f32(std::numeric_limits<float>::infinity()); }
 template <> inline f16 inf_of<f16>() { return f16::from_f32(std::numeric_limits<float>::infinity()); }
 
-template <typename T> inline T op_add(T a, T b) { return a + b; }   // binary.rs:370-373
-template <typename T> inline T op_sub(T a, T b) { return a - b; }   // binary.rs:384-387
-template <typename T> inline T op_mul(T a, T b) { return a * b; }   // binary.rs:398-401
+// Integers: Rust's saturating_add / _sub / _mul / _div (binary.rs:375-382, 389-396, 403-410, 458-578), restated as
+// "compute exactly in 128 bits, clamp to the type".  bool (:374, 388, 402, 457): or, and, xor, and.
+template <typename T> struct is_int : std::integral_constant<bool, std::is_integral<T>::value && !std::is_same<T, bool>::value> {};
+template <typename T> using wide_t = typename std::conditional<std::is_signed<T>::value, __int128, unsigned __int128>::type;
+template <typename T> inline T clamp_to(wide_t<T> v) {
+    const wide_t<T> lo = std::numeric_limits<T>::min(), hi = std::numeric_limits<T>::max();
+    return (T)(v < lo ? lo : (v > hi ? hi : v));
+}
+
+template <typename T> inline T op_add(T a, T b) {   // binary.rs:370-382
+    if constexpr (std::is_same<T, bool>::value) return a | b;
+    else if constexpr (is_int<T>::value) return clamp_to<T>((wide_t<T>)a + (wide_t<T>)b);
+    else return a + b;
+}
+template <typename T> inline T op_sub(T a, T b) {   // binary.rs:384-396
+    if constexpr (std::is_same<T, bool>::value) return a & b;
+    else if constexpr (is_int<T>::value) {
+        if (!std::is_signed<T>::value && b > a) return 0;           // (an unsigned difference below zero)
+        return clamp_to<T>((wide_t<T>)a - (wide_t<T>)b);
+    } else return a - b;
+}
+template <typename T> inline T op_mul(T a, T b) {   // binary.rs:398-410
+    if constexpr (std::is_same<T, bool>::value) return a ^ b;
+    else if constexpr (is_int<T>::value) {
+        if (!std::is_signed<T>::value && sizeof(T) == 8) {          // the exact product of two u64 can exceed 128 signed bits but not 128 unsigned
+            unsigned __int128 p = (unsigned __int128)a * (unsigned __int128)b;
+            return p > (unsigned __int128)std::numeric_limits<T>::max() ? std::numeric_limits<T>::max() : (T)p;
+        }
+        return clamp_to<T>((wide_t<T>)a * (wide_t<T>)b);
+    } else return a * b;
+}
 // binary.rs:412-465: b == 0 ⇒ (a == 0 ? 0 : +INF), sign of a ignored, NaN a ⇒ +INF.
+// Integers (:458-578): b == 0 ⇒ 0 for a == 0, else MAX (MIN for a negative a); otherwise the quotient, clamped (MIN / -1).
 template <typename T> inline T op_div(T a, T b) {
-    if (b == zero_of<T>()) return a == zero_of<T>() ? zero_of<T>() : inf_of<T>();
-    return a / b;
+    if constexpr (std::is_same<T, bool>::value) return a & b;
+    else if constexpr (is_int<T>::value) {
+        if (b == 0) return a == 0 ? (T)0 : (a < 0 ? std::numeric_limits<T>::min() : std::numeric_limits<T>::max());
+        return clamp_to<T>((wide_t<T>)a / (wide_t<T>)b);
+    } else {
+        if (b == zero_of<T>()) return a == zero_of<T>() ? zero_of<T>() : inf_of<T>();
+        return a / b;
+    }
 }
 // binary.rs:580-583: f32/f64 use `f32::max` (a NaN operand is ignored; fmax has that rule),
 // bf16/f16 use `if a > b { a } else { b }`.
@@ -97,6 +132,15 @@ inline float op_minimum(float a, float b) { return std::fmin(a, b); }   // binar
 inline double op_minimum(double a, double b) { return std::fmin(a, b); }
 inline bf16 op_minimum(bf16 a, bf16 b) { return a < b ? a : b; }
 inline f16 op_minimum(f16 a, f16 b) { return a < b ? a : b; }
+// binary.rs:584-592, 598-606: bool or / and, integers Ord::max / Ord::min
+template <typename T, typename = typename std::enable_if<std::is_integral<T>::value>::type> inline T op_maximum(T a, T b) {
+    if constexpr (std::is_same<T, bool>::value) return a | b;
+    else return a > b ? a : b;
+}
+template <typename T, typename = typename std::enable_if<std::is_integral<T>::value>::type> inline T op_minimum(T a, T b) {
+    if constexpr (std::is_same<T, bool>::value) return a & b;
+    else return a < b ? a : b;
+}
 
 }  // namespace
 
@@ -150,3 +194,12 @@ ORC_ALL_FOR(float, f32)
 ORC_ALL_FOR(double, f64)
 ORC_ALL_FOR(bf16, bf16)
 ORC_ALL_FOR(f16, f16)
+ORC_ALL_FOR(bool, bool)
+ORC_ALL_FOR(uint8_t, u8)
+ORC_ALL_FOR(uint16_t, u16)
+ORC_ALL_FOR(uint32_t, u32)
+ORC_ALL_FOR(uint64_t, u64)
+ORC_ALL_FOR(int8_t, i8)
+ORC_ALL_FOR(int16_t, i16)
+ORC_ALL_FOR(int32_t, i32)
+ORC_ALL_FOR(int64_t, i64)

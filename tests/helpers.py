@@ -14,7 +14,8 @@ ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
 
 import maidenx_amd._signatures as S  # noqa: E402
 
-NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64}
+NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16, "bool": np.uint8, "f64": np.float64, "i32": np.int32, "i64": np.int64,
+      "u8": np.uint8, "u16": np.uint16, "u32": np.uint32, "u64": np.uint64, "i8": np.int8, "i16": np.int16}
 
 
 # ---- bf16 <-> f32 on the host (round to nearest even, NaN quieted), as the `half` crate does ----
@@ -164,7 +165,7 @@ class Runner:
         if kind == "oracle":
             self.lib = C.CDLL(ensure_oracle_built())
             self.prefix = "oracle_"
-            for name, args in {**S.signatures(("f32", "bf16", "f16", "f64")), **S.index_signatures(("f32", "bf16", "f16", "f64"))}.items():
+            for name, args in {**S.signatures(("f32", "bf16", "f16", "f64")), **S.binary_signatures(), **S.index_signatures(("f32", "bf16", "f16", "f64"))}.items():
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None

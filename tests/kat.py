@@ -7,7 +7,7 @@ import os
 import numpy as np
 
 from helpers import (In, InOut, Out, const_arg, contiguous_strides, layout, meta_binary, meta_matmul, meta_pad, meta_reduce,
-                     meta_sum_to_shape, meta_unary, to_float, to_storage, u64)
+                     meta_sum_to_shape, meta_unary, to_float, to_storage, u64, NP)
 
 KAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kat.json")))
 
@@ -61,6 +61,36 @@ def run_inplace(be, dt):
         (lhs,) = be.call(f"{c['op']}_{dt}", n, 1, md, InOut(padded(c["lhs"], dt)), In(padded(c["rhs"], dt)))
         check(lhs[1:-1], c["expect"], dt, 0)
         assert to_float(lhs, dt)[0] == 0 and to_float(lhs, dt)[-1] == 0     # neighbours untouched
+
+
+INT_DTYPES = ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
+
+
+def padded_int(values, dt):
+    return np.concatenate([[0], np.asarray(values), [0]]).astype(NP[dt])
+
+
+def run_binary_wide(be, dt):
+    """The integer and bool branches of the reference's binary tests (sections *_int, compare_bool)."""
+    md_of = lambda n: meta_binary([n], [1], [1], 1, 1)
+    if dt == "bool":
+        for c in KAT["compare_bool"]:
+            n = len(c["lhs"])
+            (out,) = be.call(f"{c['op']}_bool", n, 1, md_of(n), In(padded_int(c["lhs"], dt)), In(padded_int(c["rhs"], dt)), Out(n, "bool"))
+            assert out.tolist() == c["expect"], (c["op"], out)
+        return
+    for c in KAT["binary_int"]:
+        n = len(c["lhs"])
+        (out,) = be.call(f"{c['op']}_{dt}", n, 1, md_of(n), In(padded_int(c["lhs"], dt)), In(padded_int(c["rhs"], dt)), Out(n, dt))
+        assert out.tolist() == c["expect"], (c["op"], dt, out)
+    for c in KAT["compare_int"]:
+        n = len(c["lhs"])
+        (out,) = be.call(f"{c['op']}_{dt}", n, 1, md_of(n), In(padded_int(c["lhs"], dt)), In(padded_int(c["rhs"], dt)), Out(n, "bool"))
+        assert out.tolist() == c["expect"], (c["op"], dt, out)
+    for c in KAT["inplace_int"]:
+        n = len(c["lhs"])
+        (lhs,) = be.call(f"{c['op']}_{dt}", n, 1, md_of(n), InOut(padded_int(c["lhs"], dt)), In(padded_int(c["rhs"], dt)))
+        assert lhs.tolist() == [0] + c["expect"] + [0], (c["op"], dt, lhs)
 
 
 def run_unary(be, dt):

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_python_binding_covers_the_header():
     import maidenx_amd._signatures as S
-    bound = {"hip_" + n for n in {**S.signatures(), **S.extension_signatures()}}
+    bound = {"hip_" + n for n in {**S.signatures(), **S.binary_signatures(), **S.extension_signatures()}}
     runtime = {"hip_get_last_status", "hip_status_string", "hip_set_device", "hip_get_device", "hip_device_count", "hip_malloc",
                "hip_free", "hip_memcpy_h2d", "hip_memcpy_d2h", "hip_memcpy_d2d", "hip_stream_create", "hip_stream_destroy",
                "hip_stream_synchronize", "hip_set_stream", "hip_get_stream", "hip_synchronize", "hip_event_create",

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import layouts as LY
-from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
+from helpers import (NP, In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
                      layout, meta_matmul, meta_pad, u64, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
                      ulp_diff_f32)
 
@@ -943,3 +943,65 @@ def test_error_reporting(hip):
     with pytest.raises(L.HipError):
         L.check()
     L.check()                                            # reading the status cleared it
+
+
+# ---- the binary families for f64, bool and the integers ---------------------------------------------------------
+WIDE_DTS = ["f64", "bool", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
+
+
+def wide_values(r, n, dt):
+    if dt == "f64":
+        x = r.standard_normal(n)
+        k = min(n, 8)
+        x[:k] = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 1e308])[:k]
+        return x
+    if dt == "bool":
+        return r.integers(0, 2, n, dtype=np.uint8)
+    info = np.iinfo(NP[dt])
+    x = r.integers(info.min, info.max, n, dtype=NP[dt], endpoint=True)
+    sel = r.random(n)
+    x[sel < 0.35] = r.integers(max(info.min, -9), 9, int((sel < 0.35).sum()), dtype=NP[dt])      # zeros, small factors and divisors
+    x[(sel > 0.9)] = info.max
+    x[(sel > 0.95)] = info.min
+    if info.min < 0:
+        x[(sel > 0.85) & (sel <= 0.9)] = -1
+    return x
+
+
+@pytest.mark.parametrize("dt", WIDE_DTS)
+@pytest.mark.parametrize("lname", list(BIN_LAYOUTS))
+def test_binary_ops_wide_dtypes_bit_exact(oracle, hip, lname, dt):
+    ll, rl = BIN_LAYOUTS[lname]()
+    r = rng(hash(lname) % 1000 + 7)
+    ls, rs = wide_values(r, ll["size"], dt), wide_values(r, rl["size"], dt)
+    n = int(np.prod(ll["dims"]))
+    md = meta_binary(ll["dims"], ll["strides"], rl["strides"], ll["off"], rl["off"])
+    for op in ["add", "sub", "mul", "div", "maximum", "minimum"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(ll["dims"]), md, In(ls), In(rs), Out(n, dt)))
+        if dt == "f64":
+            assert np.array_equal(np.isnan(o), np.isnan(h)), op
+            if op in ("maximum", "minimum"):
+                assert np.array_equal(o, h, equal_nan=True), op                  # (either zero may come back for (+0, -0))
+            else:
+                assert same_bits(np.where(np.isnan(o), 0, o), np.where(np.isnan(h), 0, h)), op
+        else:
+            assert same_bits(o, h), op
+    for op in ["eq", "ne", "lt", "le", "gt", "ge", "logical_and", "logical_or", "logical_xor"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(ll["dims"]), md, In(ls), In(rs), Out(n, "bool")))
+        assert np.array_equal(o, h), op
+
+
+@pytest.mark.parametrize("dt", WIDE_DTS)
+@pytest.mark.parametrize("lname", ["contig", "offset_misaligned", "rhs_row_bcast", "scalar_bcast", "nhwc_view_plus_bias"])
+def test_inplace_ops_wide_dtypes_bit_exact(oracle, hip, lname, dt):
+    ll, rl = BIN_LAYOUTS[lname]()
+    lc = LY.contiguous(ll["dims"], off=ll["off"])
+    r = rng(11)
+    ls, rs = wide_values(r, lc["size"], dt), wide_values(r, rl["size"], dt)
+    if dt == "f64":
+        ls[:8], rs[:8] = r.standard_normal(min(8, ls.size)), r.standard_normal(min(8, rs.size))      # (NaN payloads are not compared here)
+    n = int(np.prod(lc["dims"]))
+    md = meta_binary(lc["dims"], lc["strides"], rl["strides"], lc["off"], rl["off"])
+    for op in ["add_inplace", "sub_inplace", "mul_inplace", "div_inplace"]:
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lc["dims"]), md, InOut(ls.copy()), In(rs)))
+        assert same_bits(o, h), op

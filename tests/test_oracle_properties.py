@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import layouts as LY
-from helpers import (In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
+from helpers import (NP, In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
                      meta_matmul, meta_pad, meta_reduce, meta_sum_to_shape, meta_unary, rng, ulp_diff_f32)
 
 
@@ -537,3 +537,77 @@ def test_oracle_f16_codec_matches_numpy_float16(oracle):
     ok = ~np.isnan(want)
     assert np.array_equal(m[ok], want.view(np.uint16)[ok])           # overflow to inf, subnormals, ties to even
     assert np.all(np.isnan(m[~ok].view(np.float16)))
+
+
+# ---- integers and bool: the oracle against exact (unbounded) integer arithmetic -------------------------------
+def int_operands(dt, n=4096, seed=3):
+    """Values that make every saturation and division case meet: the extremes, 0, +-1 and random fill."""
+    info = np.iinfo(NP[dt])
+    r = rng(seed)
+    edge = [info.min, info.max, 0, 1, info.max - 1, info.min + 1, 2, 3] + ([-1, -2] if info.min < 0 else [])
+    a = r.integers(info.min, info.max, n, dtype=NP[dt], endpoint=True)
+    b = r.integers(info.min, info.max, n, dtype=NP[dt], endpoint=True)
+    small = r.integers(max(info.min, -12), 12, n // 2, dtype=NP[dt])          # products and quotients that do not saturate
+    a[: n // 2: 2] = small[: n // 4]
+    b[1: n // 2: 2] = small[n // 4: n // 2]
+    k = len(edge)
+    grid_a, grid_b = np.repeat(np.array(edge, dtype=object), k), np.tile(np.array(edge, dtype=object), k)                     # every edge value against every edge value
+    a[-k * k:], b[-k * k:] = grid_a.astype(NP[dt]), grid_b.astype(NP[dt])
+    return a, b
+
+
+@pytest.mark.parametrize("dt", ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"])
+def test_oracle_integer_binary_ops_vs_exact_arithmetic(oracle, dt):
+    info = np.iinfo(NP[dt])
+    a, b = int_operands(dt)
+    n = a.size
+    A, B = [int(v) for v in a], [int(v) for v in b]                           # Python integers: exact
+    clip = lambda v: min(max(v, info.min), info.max)
+
+    def quotient(x, y):                                                      # truncation toward zero, then the clamp
+        if y == 0:
+            return 0 if x == 0 else (info.min if x < 0 else info.max)
+        q = abs(x) // abs(y)
+        return clip(q if (x < 0) == (y < 0) else -q)
+    want = {"add": [clip(x + y) for x, y in zip(A, B)], "sub": [clip(x - y) for x, y in zip(A, B)],
+            "mul": [clip(x * y) for x, y in zip(A, B)], "div": [quotient(x, y) for x, y in zip(A, B)],
+            "maximum": [max(x, y) for x, y in zip(A, B)], "minimum": [min(x, y) for x, y in zip(A, B)]}
+    md = meta_binary([n], [1], [1])
+    for op, exp in want.items():
+        (out,) = oracle.call(f"{op}_{dt}", n, 1, md, In(a), In(b), Out(n, dt))
+        assert [int(v) for v in out] == exp, op
+        if op in ("add", "sub", "mul", "div"):
+            (acc,) = oracle.call(f"{op}_inplace_{dt}", n, 1, md, InOut(a.copy()), In(b))
+            assert np.array_equal(acc, out), op
+    cmp = {"eq": a == b, "ne": a != b, "lt": a < b, "le": a <= b, "gt": a > b, "ge": a >= b,
+           "logical_and": (a != 0) & (b != 0), "logical_or": (a != 0) | (b != 0), "logical_xor": (a != 0) ^ (b != 0)}
+    for op, exp in cmp.items():
+        (out,) = oracle.call(f"{op}_{dt}", n, 1, md, In(a), In(b), Out(n, "bool"))
+        assert np.array_equal(out.astype(bool), exp), op
+
+
+def test_oracle_bool_binary_ops_truth_tables(oracle):
+    a = np.array([0, 0, 1, 1], dtype=np.uint8)
+    b = np.array([0, 1, 0, 1], dtype=np.uint8)
+    md = meta_binary([4], [1], [1])
+    # binary.rs:374 (add = or), :388 (sub = and), :402 (mul = xor), :457 (div = and), :584 (maximum = or), :598 (minimum = and)
+    tables = {"add": a | b, "sub": a & b, "mul": a ^ b, "div": a & b, "maximum": a | b, "minimum": a & b,
+              "eq": a == b, "ne": a != b, "lt": a < b, "le": a <= b, "gt": a > b, "ge": a >= b,
+              "logical_and": a & b, "logical_or": a | b, "logical_xor": a ^ b}
+    for op, exp in tables.items():
+        (out,) = oracle.call(f"{op}_bool", 4, 1, md, In(a), In(b), Out(4, "bool"))
+        assert out.tolist() == exp.astype(np.uint8).tolist(), op
+
+
+def test_oracle_f64_binary_vs_numpy(oracle):
+    r = rng(9)
+    a, b = r.standard_normal(1000), r.standard_normal(1000)
+    a[:6] = [0.0, 1.0, -2.0, np.nan, 0.0, 1e308]
+    b[:6] = [0.0, 0.0, 0.0, 0.0, 3.0, 1e308]
+    md = meta_binary([1000], [1], [1])
+    with np.errstate(all="ignore"):
+        want = {"add": a + b, "sub": a - b, "mul": a * b, "maximum": np.fmax(a, b), "minimum": np.fmin(a, b),
+                "div": np.where(b == 0, np.where(a == 0, 0.0, np.inf), a / np.where(b == 0, 1.0, b))}
+    for op, exp in want.items():
+        (out,) = oracle.call(f"{op}_f64", 1000, 1, md, In(a), In(b), Out(1000, "f64"))
+        assert np.array_equal(out, exp, equal_nan=True), op
