@@ -321,6 +321,138 @@ void hip_cast_bool_f16(size_t num_els, const mx_bool* input, mx_f16* output);
 void hip_cast_f32_f16(size_t num_els, const float* input, mx_f16* output);
 void hip_cast_f16_f32(size_t num_els, const mx_f16* input, float* output);
 void hip_cast_f16_bool(size_t num_els, const mx_f16* input, mx_bool* output);
+/* The same three for f64, the integers and bool, and conversions between every pair of the plain-number dtypes
+ * (f32, f64, bool, u8 … i64) with the results of the reference's host conversion
+ * (crates/maidenx_core/src/buffer/mod.rs:155-196, pair table :414-560): Rust's `as` — float to integer drops the
+ * fraction, saturates and sends NaN to 0; integer to float rounds to nearest even; integer to integer keeps the low
+ * bits; to bool is `!= 0`. */
+void hip_fill_f64(size_t num_els, double* out, double value);
+void hip_fill_u8(size_t num_els, uint8_t* out, uint8_t value);
+void hip_fill_u16(size_t num_els, uint16_t* out, uint16_t value);
+void hip_fill_u32(size_t num_els, uint32_t* out, uint32_t value);
+void hip_fill_u64(size_t num_els, uint64_t* out, uint64_t value);
+void hip_fill_i8(size_t num_els, int8_t* out, int8_t value);
+void hip_fill_i16(size_t num_els, int16_t* out, int16_t value);
+void hip_fill_i32(size_t num_els, int32_t* out, int32_t value);
+void hip_fill_i64(size_t num_els, int64_t* out, int64_t value);
+void hip_copy_strided_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_copy_strided_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_copy_strided_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_copy_strided_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_copy_strided_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_copy_strided_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_copy_strided_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_copy_strided_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_copy_strided_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_copy_strided_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_cast_f32_f64(size_t num_els, const float* input, double* output);
+void hip_cast_f32_u8(size_t num_els, const float* input, uint8_t* output);
+void hip_cast_f32_u16(size_t num_els, const float* input, uint16_t* output);
+void hip_cast_f32_u32(size_t num_els, const float* input, uint32_t* output);
+void hip_cast_f32_u64(size_t num_els, const float* input, uint64_t* output);
+void hip_cast_f32_i8(size_t num_els, const float* input, int8_t* output);
+void hip_cast_f32_i16(size_t num_els, const float* input, int16_t* output);
+void hip_cast_f32_i32(size_t num_els, const float* input, int32_t* output);
+void hip_cast_f32_i64(size_t num_els, const float* input, int64_t* output);
+void hip_cast_f64_f32(size_t num_els, const double* input, float* output);
+void hip_cast_f64_bool(size_t num_els, const double* input, mx_bool* output);
+void hip_cast_f64_u8(size_t num_els, const double* input, uint8_t* output);
+void hip_cast_f64_u16(size_t num_els, const double* input, uint16_t* output);
+void hip_cast_f64_u32(size_t num_els, const double* input, uint32_t* output);
+void hip_cast_f64_u64(size_t num_els, const double* input, uint64_t* output);
+void hip_cast_f64_i8(size_t num_els, const double* input, int8_t* output);
+void hip_cast_f64_i16(size_t num_els, const double* input, int16_t* output);
+void hip_cast_f64_i32(size_t num_els, const double* input, int32_t* output);
+void hip_cast_f64_i64(size_t num_els, const double* input, int64_t* output);
+void hip_cast_bool_f64(size_t num_els, const mx_bool* input, double* output);
+void hip_cast_bool_u8(size_t num_els, const mx_bool* input, uint8_t* output);
+void hip_cast_bool_u16(size_t num_els, const mx_bool* input, uint16_t* output);
+void hip_cast_bool_u32(size_t num_els, const mx_bool* input, uint32_t* output);
+void hip_cast_bool_u64(size_t num_els, const mx_bool* input, uint64_t* output);
+void hip_cast_bool_i8(size_t num_els, const mx_bool* input, int8_t* output);
+void hip_cast_bool_i16(size_t num_els, const mx_bool* input, int16_t* output);
+void hip_cast_bool_i32(size_t num_els, const mx_bool* input, int32_t* output);
+void hip_cast_bool_i64(size_t num_els, const mx_bool* input, int64_t* output);
+void hip_cast_u8_f32(size_t num_els, const uint8_t* input, float* output);
+void hip_cast_u8_f64(size_t num_els, const uint8_t* input, double* output);
+void hip_cast_u8_bool(size_t num_els, const uint8_t* input, mx_bool* output);
+void hip_cast_u8_u16(size_t num_els, const uint8_t* input, uint16_t* output);
+void hip_cast_u8_u32(size_t num_els, const uint8_t* input, uint32_t* output);
+void hip_cast_u8_u64(size_t num_els, const uint8_t* input, uint64_t* output);
+void hip_cast_u8_i8(size_t num_els, const uint8_t* input, int8_t* output);
+void hip_cast_u8_i16(size_t num_els, const uint8_t* input, int16_t* output);
+void hip_cast_u8_i32(size_t num_els, const uint8_t* input, int32_t* output);
+void hip_cast_u8_i64(size_t num_els, const uint8_t* input, int64_t* output);
+void hip_cast_u16_f32(size_t num_els, const uint16_t* input, float* output);
+void hip_cast_u16_f64(size_t num_els, const uint16_t* input, double* output);
+void hip_cast_u16_bool(size_t num_els, const uint16_t* input, mx_bool* output);
+void hip_cast_u16_u8(size_t num_els, const uint16_t* input, uint8_t* output);
+void hip_cast_u16_u32(size_t num_els, const uint16_t* input, uint32_t* output);
+void hip_cast_u16_u64(size_t num_els, const uint16_t* input, uint64_t* output);
+void hip_cast_u16_i8(size_t num_els, const uint16_t* input, int8_t* output);
+void hip_cast_u16_i16(size_t num_els, const uint16_t* input, int16_t* output);
+void hip_cast_u16_i32(size_t num_els, const uint16_t* input, int32_t* output);
+void hip_cast_u16_i64(size_t num_els, const uint16_t* input, int64_t* output);
+void hip_cast_u32_f32(size_t num_els, const uint32_t* input, float* output);
+void hip_cast_u32_f64(size_t num_els, const uint32_t* input, double* output);
+void hip_cast_u32_bool(size_t num_els, const uint32_t* input, mx_bool* output);
+void hip_cast_u32_u8(size_t num_els, const uint32_t* input, uint8_t* output);
+void hip_cast_u32_u16(size_t num_els, const uint32_t* input, uint16_t* output);
+void hip_cast_u32_u64(size_t num_els, const uint32_t* input, uint64_t* output);
+void hip_cast_u32_i8(size_t num_els, const uint32_t* input, int8_t* output);
+void hip_cast_u32_i16(size_t num_els, const uint32_t* input, int16_t* output);
+void hip_cast_u32_i32(size_t num_els, const uint32_t* input, int32_t* output);
+void hip_cast_u32_i64(size_t num_els, const uint32_t* input, int64_t* output);
+void hip_cast_u64_f32(size_t num_els, const uint64_t* input, float* output);
+void hip_cast_u64_f64(size_t num_els, const uint64_t* input, double* output);
+void hip_cast_u64_bool(size_t num_els, const uint64_t* input, mx_bool* output);
+void hip_cast_u64_u8(size_t num_els, const uint64_t* input, uint8_t* output);
+void hip_cast_u64_u16(size_t num_els, const uint64_t* input, uint16_t* output);
+void hip_cast_u64_u32(size_t num_els, const uint64_t* input, uint32_t* output);
+void hip_cast_u64_i8(size_t num_els, const uint64_t* input, int8_t* output);
+void hip_cast_u64_i16(size_t num_els, const uint64_t* input, int16_t* output);
+void hip_cast_u64_i32(size_t num_els, const uint64_t* input, int32_t* output);
+void hip_cast_u64_i64(size_t num_els, const uint64_t* input, int64_t* output);
+void hip_cast_i8_f32(size_t num_els, const int8_t* input, float* output);
+void hip_cast_i8_f64(size_t num_els, const int8_t* input, double* output);
+void hip_cast_i8_bool(size_t num_els, const int8_t* input, mx_bool* output);
+void hip_cast_i8_u8(size_t num_els, const int8_t* input, uint8_t* output);
+void hip_cast_i8_u16(size_t num_els, const int8_t* input, uint16_t* output);
+void hip_cast_i8_u32(size_t num_els, const int8_t* input, uint32_t* output);
+void hip_cast_i8_u64(size_t num_els, const int8_t* input, uint64_t* output);
+void hip_cast_i8_i16(size_t num_els, const int8_t* input, int16_t* output);
+void hip_cast_i8_i32(size_t num_els, const int8_t* input, int32_t* output);
+void hip_cast_i8_i64(size_t num_els, const int8_t* input, int64_t* output);
+void hip_cast_i16_f32(size_t num_els, const int16_t* input, float* output);
+void hip_cast_i16_f64(size_t num_els, const int16_t* input, double* output);
+void hip_cast_i16_bool(size_t num_els, const int16_t* input, mx_bool* output);
+void hip_cast_i16_u8(size_t num_els, const int16_t* input, uint8_t* output);
+void hip_cast_i16_u16(size_t num_els, const int16_t* input, uint16_t* output);
+void hip_cast_i16_u32(size_t num_els, const int16_t* input, uint32_t* output);
+void hip_cast_i16_u64(size_t num_els, const int16_t* input, uint64_t* output);
+void hip_cast_i16_i8(size_t num_els, const int16_t* input, int8_t* output);
+void hip_cast_i16_i32(size_t num_els, const int16_t* input, int32_t* output);
+void hip_cast_i16_i64(size_t num_els, const int16_t* input, int64_t* output);
+void hip_cast_i32_f32(size_t num_els, const int32_t* input, float* output);
+void hip_cast_i32_f64(size_t num_els, const int32_t* input, double* output);
+void hip_cast_i32_bool(size_t num_els, const int32_t* input, mx_bool* output);
+void hip_cast_i32_u8(size_t num_els, const int32_t* input, uint8_t* output);
+void hip_cast_i32_u16(size_t num_els, const int32_t* input, uint16_t* output);
+void hip_cast_i32_u32(size_t num_els, const int32_t* input, uint32_t* output);
+void hip_cast_i32_u64(size_t num_els, const int32_t* input, uint64_t* output);
+void hip_cast_i32_i8(size_t num_els, const int32_t* input, int8_t* output);
+void hip_cast_i32_i16(size_t num_els, const int32_t* input, int16_t* output);
+void hip_cast_i32_i64(size_t num_els, const int32_t* input, int64_t* output);
+void hip_cast_i64_f32(size_t num_els, const int64_t* input, float* output);
+void hip_cast_i64_f64(size_t num_els, const int64_t* input, double* output);
+void hip_cast_i64_bool(size_t num_els, const int64_t* input, mx_bool* output);
+void hip_cast_i64_u8(size_t num_els, const int64_t* input, uint8_t* output);
+void hip_cast_i64_u16(size_t num_els, const int64_t* input, uint16_t* output);
+void hip_cast_i64_u32(size_t num_els, const int64_t* input, uint32_t* output);
+void hip_cast_i64_u64(size_t num_els, const int64_t* input, uint64_t* output);
+void hip_cast_i64_i8(size_t num_els, const int64_t* input, int8_t* output);
+void hip_cast_i64_i16(size_t num_els, const int64_t* input, int16_t* output);
+void hip_cast_i64_i32(size_t num_els, const int64_t* input, int32_t* output);
 
 #ifdef __cplusplus
 }

@@ -6,7 +6,9 @@ identical argument lists, so a CPU restatement built with another prefix can be 
 import ctypes as C
 
 SZ, P = C.c_size_t, C.c_void_p
-CONST = {"f32": C.c_float, "f64": C.c_double, "bf16": C.c_uint16, "f16": C.c_uint16, "bool": C.c_uint8}
+CONST = {"f32": C.c_float, "f64": C.c_double, "bf16": C.c_uint16, "f16": C.c_uint16, "bool": C.c_uint8,
+         "u8": C.c_uint8, "u16": C.c_uint16, "u32": C.c_uint32, "u64": C.c_uint64,
+         "i8": C.c_int8, "i16": C.c_int16, "i32": C.c_int32, "i64": C.c_int64}
 
 BINARY = ["add", "sub", "mul", "div", "maximum", "minimum", "logical_and", "logical_or", "logical_xor",
           "eq", "ne", "lt", "le", "gt", "ge"]
@@ -64,6 +66,24 @@ def binary_signatures(dtypes=WIDE_DTYPES):
     return sig
 
 
+PLAIN_DTYPES = ("f32", "f64", "bool", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64")
+
+
+def cast_signatures():
+    """Conversions between every pair of the plain-number dtypes."""
+    return {f"cast_{a}_{b}": [SZ, P, P] for a in PLAIN_DTYPES for b in PLAIN_DTYPES if a != b}
+
+
+def wide_util_signatures():
+    """fill / copy_strided for the dtypes beyond f32, bf16, f16 (fill_bool is with those)."""
+    sig = {}
+    for dt in WIDE_DTYPES:
+        if dt != "bool":
+            sig[f"fill_{dt}"] = [SZ, P, CONST[dt]]
+        sig[f"copy_strided_{dt}"] = [SZ, SZ, P, P, P]
+    return sig
+
+
 def index_signatures(dtypes=("f32", "bf16", "f16")):
     """Index ops (host loops in the reference's tensor layer, device entry points here)."""
     sig = {}
@@ -91,4 +111,6 @@ def extension_signatures():
     for a, b in (("bool", "f32"), ("bool", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "bool"), ("bf16", "bool"),
                  ("bool", "f16"), ("f32", "f16"), ("f16", "f32"), ("f16", "bool")):
         sig[f"cast_{a}_{b}"] = [SZ, P, P]
+    sig.update(cast_signatures())
+    sig.update(wide_util_signatures())
     return sig

@@ -169,6 +169,10 @@ class Runner:
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None
+            for name, args in S.cast_signatures().items():
+                fn = getattr(self.lib, self.prefix + name)
+                fn.argtypes = args
+                fn.restype = None
             self.lib.oracle_index_error.restype = C.c_int
             self.lib.oracle_set_num_threads.argtypes = [C.c_int]
             self.lib.oracle_set_num_threads.restype = C.c_int
@@ -215,8 +219,45 @@ def const_arg(v, dt):
     """A by-value constant of the input dtype."""
     if dt in ("bf16", "f16"):
         return int(to_storage(np.array([v], dtype=np.float32), dt)[0])
-    return float(v)
+    if dt in ("f32", "f64"):
+        return float(v)
+    return int(v)
 
 
 def rng(seed):
     return np.random.default_rng(seed)
+
+
+PLAIN = ["f32", "f64", "bool", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
+
+
+def cast_inputs(dt, n=3000, seed=21):
+    """Source values for the dtype conversions: every boundary of every integer target, just inside and just outside,
+    fractions either side of zero, NaN and infinities for the floats; extremes and random fill for the integers."""
+    r = rng(seed)
+    if dt in ("f32", "f64"):
+        ft = NP[dt]
+        edges = []
+        for bits in (8, 16, 32, 64):
+            for v in (2.0 ** bits, 2.0 ** (bits - 1), -(2.0 ** (bits - 1))):
+                x = ft(v)
+                edges += [x, np.nextafter(x, ft(np.inf)), np.nextafter(x, ft(-np.inf)), x + ft(0.5), x - ft(0.5), x - ft(1), x + ft(1)]
+        edges += [0.0, -0.0, 0.5, -0.5, 0.999, -0.999, 1.5, -1.5, 255.5, -128.5, np.nan, np.inf, -np.inf, 1e30, -1e30, 3e38]
+        scale = r.choice([1.0, 1e2, 1e5, 1e10, 1e19], n - len(edges))
+        with np.errstate(over="ignore"):
+            x = np.concatenate([np.array(edges, dtype=ft), (r.standard_normal(n - len(edges)) * scale).astype(ft)])
+        return x
+    if dt == "bool":
+        return r.integers(0, 2, n, dtype=np.uint8)
+    info = np.iinfo(NP[dt])
+    x = r.integers(info.min, info.max, n, dtype=NP[dt], endpoint=True)
+    x[: n // 3] = r.integers(max(info.min, -300), min(info.max, 300), n // 3, dtype=NP[dt], endpoint=True)
+    edge = [info.min, info.max, 0, 1, info.max - 1, info.min + 1, info.max // 2, info.max // 2 + 1]
+    for bits in (8, 16, 24, 25, 32, 53, 54, 63):           # where narrower integers wrap and floats start to round
+        for v in (2 ** bits - 1, 2 ** bits, 2 ** bits + 1, 2 ** bits + 3):
+            if v <= info.max:
+                edge.append(v)
+            if -v >= info.min:
+                edge.append(-v)
+    x[-len(edge):] = np.array(edge, dtype=object).astype(NP[dt])
+    return x

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import layouts as LY
-from helpers import (NP, In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
+from helpers import (NP, PLAIN, cast_inputs, In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
                      layout, meta_matmul, meta_pad, u64, meta_reduce, meta_sum_to_shape, meta_unary, rng, to_float, to_storage,
                      ulp_diff_f32)
 
@@ -1005,3 +1005,33 @@ def test_inplace_ops_wide_dtypes_bit_exact(oracle, hip, lname, dt):
     for op in ["add_inplace", "sub_inplace", "mul_inplace", "div_inplace"]:
         (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lc["dims"]), md, InOut(ls.copy()), In(rs)))
         assert same_bits(o, h), op
+
+
+# ---- conversions between the plain-number dtypes; fill and strided copy for the wide dtypes -------------------------
+@pytest.mark.parametrize("src", PLAIN)
+def test_casts_bit_exact(oracle, hip, src):
+    x = cast_inputs(src, n=70001)
+    for dst in PLAIN:
+        if dst == src:
+            continue
+        (o,), (h,) = both(oracle, hip, f"cast_{src}_{dst}", lambda: (x.size, In(x), Out(x.size, dst)))
+        if dst in ("f32", "f64"):
+            assert np.array_equal(np.isnan(o), np.isnan(h)), (src, dst)
+            assert same_bits(np.where(np.isnan(o), 0, o), np.where(np.isnan(h), 0, h)), (src, dst)
+        else:
+            assert same_bits(o, h), (src, dst)
+
+
+@pytest.mark.parametrize("dt", WIDE_DTS)
+def test_fill_and_strided_copy_wide_dtypes(hip, dt):
+    r = rng(31)
+    if dt != "bool":
+        value = {"f64": -2.5}.get(dt, 7)
+        (f,) = hip.call(f"fill_{dt}", 5001, Out(5001, dt), const_arg(value, dt))
+        assert np.array_equal(f, np.full(5001, value, dtype=NP[dt]))
+    for lay in (LY.permuted([150, 200], [1, 0]), LY.broadcast([40, 50], [1, 50]), LY.contiguous([77, 13], off=1), LY.permuted([2, 5, 6, 7], [3, 1, 0, 2])):
+        src = wide_values(r, lay["size"], dt)
+        n = int(np.prod(lay["dims"]))
+        (c,) = hip.call(f"copy_strided_{dt}", n, len(lay["dims"]), meta_unary(lay["dims"], lay["strides"], lay["off"]), In(src), Out(n, dt))
+        want = np.lib.stride_tricks.as_strided(src[lay["off"]:], lay["dims"], [st * src.itemsize for st in lay["strides"]]).ravel()
+        assert same_bits(c, want), dt

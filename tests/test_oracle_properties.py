@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import layouts as LY
-from helpers import (NP, In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
+from helpers import (NP, PLAIN, cast_inputs, In, InOut, Out, bf16_to_f32, const_arg, contiguous_strides, f32_to_bf16, meta_binary, meta_conv,
                      meta_matmul, meta_pad, meta_reduce, meta_sum_to_shape, meta_unary, rng, ulp_diff_f32)
 
 
@@ -611,3 +611,65 @@ def test_oracle_f64_binary_vs_numpy(oracle):
     for op, exp in want.items():
         (out,) = oracle.call(f"{op}_f64", 1000, 1, md, In(a), In(b), Out(1000, "f64"))
         assert np.array_equal(out, exp, equal_nan=True), op
+
+
+# ---- dtype conversions: the oracle against exact arithmetic on Python numbers ----------------------------------------
+def exact_cast(values, src, dst):
+    """What Rust's `as` (towards bool: `!= 0`) gives, worked out with Python integers and numpy's IEEE conversions."""
+    if dst == "bool":
+        return [int(v != 0) for v in values.tolist()] if src not in ("f32", "f64") else [int(not (v == 0)) for v in values.tolist()]
+    if dst in ("f32", "f64"):
+        if src in ("f32", "f64"):
+            with np.errstate(over="ignore"):
+                return values.astype(NP[dst])                              # IEEE narrowing / widening
+        # integer -> float: round to nearest even, from the exact integer (via the fractions module, independent of any C cast)
+        from fractions import Fraction
+        out = []
+        for v in values.tolist():
+            f = float(Fraction(int(v)))                                   # correctly rounded to binary64
+            out.append(np.float32(f) if dst == "f32" else f)
+        # (binary64 -> binary32 of an integer below 2^64 cannot double-round wrongly only if the first step was exact;
+        #  integers above 2^53 are checked against the single rounding below instead)
+        if dst == "f32":
+            out = [np.float32(nearest_f32(int(v))) for v in values.tolist()]
+        return np.array(out, dtype=NP[dst])
+    info = np.iinfo(NP[dst])
+    out = []
+    for v in values.tolist():
+        if src in ("f32", "f64"):
+            if v != v:
+                out.append(0)
+            elif v in (float("inf"), float("-inf")):
+                out.append(info.max if v > 0 else info.min)
+            else:
+                out.append(min(max(int(v), info.min), info.max))          # int() drops the fraction; then saturate
+        else:
+            out.append((int(v) - info.min) % (info.max - info.min + 1) + info.min)      # keep the low bits (two's complement)
+    return out
+
+
+def nearest_f32(i):
+    """The binary32 nearest to the integer i, ties to even, by integer arithmetic alone."""
+    if i == 0:
+        return 0.0
+    sign, m = (-1.0 if i < 0 else 1.0), abs(i)
+    shift = max(m.bit_length() - 24, 0)
+    q, rem = m >> shift, m & ((1 << shift) - 1)
+    half = 1 << (shift - 1) if shift else 0
+    if shift and (rem > half or (rem == half and (q & 1))):
+        q += 1
+    return sign * float(q) * 2.0 ** shift
+
+
+@pytest.mark.parametrize("src", PLAIN)
+def test_oracle_casts_vs_exact_arithmetic(oracle, src):
+    x = cast_inputs(src)
+    for dst in PLAIN:
+        if dst == src:
+            continue
+        (out,) = oracle.call(f"cast_{src}_{dst}", x.size, In(x), Out(x.size, dst))
+        want = exact_cast(x, src, dst)
+        if dst in ("f32", "f64"):
+            assert np.array_equal(out, np.asarray(want, dtype=NP[dst]), equal_nan=True), (src, dst)
+        else:
+            assert [int(v) for v in out] == list(want), (src, dst)
