@@ -162,6 +162,192 @@ MX_DECL_UNARY(float, f32)
 MX_DECL_UNARY(mx_bf16, bf16)
 MX_DECL_UNARY(mx_f16, f16)
 
+/* ---- unary for f64, bool and the integers: crates/maidenx_cuda/src/ops/unary.rs:97-136, 152-191 ---------------------
+ * The forms that are exact everywhere (semantics: crates/maidenx_cpu/src/ops/unary.rs:124-230, 234-236, 354-369,
+ * 374-560, 564, 585-589, 650-740): integer neg / abs / square wrap on overflow as the reference's release build does,
+ * integer sqrt is `(x as f32).sqrt() as T` of |x| (i64 through f64), the scalar add / sub / mul saturate; bool: neg = not,
+ * add_scalar = or, sub_scalar = xor, mul_scalar = div_scalar = and, the rest identity.  Not built: the f64
+ * transcendentals, gelu, pow and elu, and the integer pow (a float powf and a cast in the reference). */
+void hip_logical_not_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, mx_bool* output);
+void hip_sign_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_square_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_sqrt_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_neg_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_abs_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_relu_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_recip_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_add_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_sub_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_mul_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_div_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_maximum_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_minimum_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_eq_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
+void hip_ne_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
+void hip_lt_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
+void hip_le_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
+void hip_gt_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
+void hip_ge_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
+void hip_leaky_relu_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_logical_not_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_neg_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_abs_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_sign_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_square_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_sqrt_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_relu_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_sigmoid_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_tanh_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
+void hip_add_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_sub_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_mul_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_div_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_maximum_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_minimum_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_eq_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_ne_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_lt_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_le_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_gt_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_ge_scalar_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_pow_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool constant, mx_bool* output);
+void hip_logical_not_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, mx_bool* output);
+void hip_sign_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_square_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_sqrt_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_add_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_sub_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_mul_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_div_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_maximum_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_minimum_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_eq_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, mx_bool* output);
+void hip_ne_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, mx_bool* output);
+void hip_lt_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, mx_bool* output);
+void hip_le_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, mx_bool* output);
+void hip_gt_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, mx_bool* output);
+void hip_ge_scalar_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, mx_bool* output);
+void hip_logical_not_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, mx_bool* output);
+void hip_sign_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_square_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_sqrt_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_add_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_sub_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_mul_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_div_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_maximum_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_minimum_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_eq_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, mx_bool* output);
+void hip_ne_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, mx_bool* output);
+void hip_lt_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, mx_bool* output);
+void hip_le_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, mx_bool* output);
+void hip_gt_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, mx_bool* output);
+void hip_ge_scalar_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, mx_bool* output);
+void hip_logical_not_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, mx_bool* output);
+void hip_sign_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_square_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_sqrt_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_add_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_sub_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_mul_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_div_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_maximum_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_minimum_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_eq_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, mx_bool* output);
+void hip_ne_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, mx_bool* output);
+void hip_lt_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, mx_bool* output);
+void hip_le_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, mx_bool* output);
+void hip_gt_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, mx_bool* output);
+void hip_ge_scalar_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, mx_bool* output);
+void hip_logical_not_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, mx_bool* output);
+void hip_sign_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_square_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_sqrt_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_add_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_sub_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_mul_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_div_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_maximum_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_minimum_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_eq_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, mx_bool* output);
+void hip_ne_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, mx_bool* output);
+void hip_lt_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, mx_bool* output);
+void hip_le_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, mx_bool* output);
+void hip_gt_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, mx_bool* output);
+void hip_ge_scalar_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, mx_bool* output);
+void hip_logical_not_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, mx_bool* output);
+void hip_sign_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_square_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_sqrt_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_neg_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_abs_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_add_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_sub_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_mul_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_div_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_maximum_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_minimum_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_eq_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, mx_bool* output);
+void hip_ne_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, mx_bool* output);
+void hip_lt_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, mx_bool* output);
+void hip_le_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, mx_bool* output);
+void hip_gt_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, mx_bool* output);
+void hip_ge_scalar_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, mx_bool* output);
+void hip_logical_not_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, mx_bool* output);
+void hip_sign_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_square_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_sqrt_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_neg_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_abs_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_add_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_sub_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_mul_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_div_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_maximum_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_minimum_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_eq_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, mx_bool* output);
+void hip_ne_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, mx_bool* output);
+void hip_lt_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, mx_bool* output);
+void hip_le_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, mx_bool* output);
+void hip_gt_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, mx_bool* output);
+void hip_ge_scalar_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, mx_bool* output);
+void hip_logical_not_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, mx_bool* output);
+void hip_sign_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_square_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_sqrt_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_neg_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_abs_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_add_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_sub_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_mul_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_div_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_maximum_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_minimum_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_eq_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, mx_bool* output);
+void hip_ne_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, mx_bool* output);
+void hip_lt_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, mx_bool* output);
+void hip_le_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, mx_bool* output);
+void hip_gt_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, mx_bool* output);
+void hip_ge_scalar_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, mx_bool* output);
+void hip_logical_not_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, mx_bool* output);
+void hip_sign_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_square_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_sqrt_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_neg_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_abs_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_add_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+void hip_sub_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+void hip_mul_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+void hip_div_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+void hip_maximum_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+void hip_minimum_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+void hip_eq_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
+void hip_ne_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
+void hip_lt_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
+void hip_le_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
+void hip_gt_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
+void hip_ge_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
+
 /* ---- reduction: replaces crates/maidenx_cuda/src/ops/reduction.rs:19-35 ---------------------------
  * sum/mean/max/min metadata = dims[n] | strides[n] | red_len[r] | red_stride[r] | offset, r = 1
  * (the only value the tensor layer produces, crates/maidenx_tensor/src/ops/reduction.rs:38).

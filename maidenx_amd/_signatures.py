@@ -84,6 +84,37 @@ def wide_util_signatures():
     return sig
 
 
+WIDE_CONST_OPS = ["add_scalar", "sub_scalar", "mul_scalar", "div_scalar", "maximum_scalar", "minimum_scalar",
+                  "eq_scalar", "ne_scalar", "lt_scalar", "le_scalar", "gt_scalar", "ge_scalar"]
+
+
+def wide_unary_ops(dt):
+    """(plain ops, ops with a constant) built for a dtype beyond f32 / bf16 / f16."""
+    plain, const = ["logical_not"], list(WIDE_CONST_OPS)
+    if dt == "bool":
+        plain += ["neg", "abs", "sign", "square", "sqrt", "relu", "sigmoid", "tanh"]
+        const += ["pow"]
+    else:
+        plain += ["sign", "square", "sqrt"]
+        if dt[0] in "if":
+            plain += ["neg", "abs"]
+        if dt == "f64":
+            plain += ["relu", "recip"]
+            const += ["leaky_relu"]
+    return plain, const
+
+
+def wide_unary_signatures(dtypes=WIDE_DTYPES):
+    sig = {}
+    for dt in dtypes:
+        plain, const = wide_unary_ops(dt)
+        for op in plain:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, P]
+        for op in const:
+            sig[f"{op}_{dt}"] = [SZ, SZ, P, P, CONST[dt], P]
+    return sig
+
+
 def index_signatures(dtypes=("f32", "bf16", "f16")):
     """Index ops (host loops in the reference's tensor layer, device entry points here)."""
     sig = {}
@@ -113,4 +144,5 @@ def extension_signatures():
         sig[f"cast_{a}_{b}"] = [SZ, P, P]
     sig.update(cast_signatures())
     sig.update(wide_util_signatures())
+    sig.update(wide_unary_signatures())
     return sig

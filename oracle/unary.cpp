@@ -128,6 +128,94 @@ template <class C> struct Fx<half_t<C>> {
     static bool ge_scalar(T x, T c) { return x >= c; }
 };
 
+// Integers (unary.rs:127-130, 137-140, 159-198, 209-216, 223-230, 362-369 and the scalar forms :377-384, 391-398,
+// 405-412, 453-533, 539-560, 664-740).  Negation, absolute value and square overflow in the reference (a panic in a
+// debug build, two's-complement wrap in a release build); the wrap is what is restated, through 128-bit arithmetic
+// reduced modulo 2^bits.  The scalar add / sub / mul saturate.
+template <typename I> struct IntFx {
+    using T = I;
+    using L = std::numeric_limits<I>;
+    static T wrap(__int128 v) {                                   // v modulo 2^bits, as a T
+        const __int128 span = (__int128)1 << (8 * sizeof(T));
+        __int128 r = ((v % span) + span) % span;                  // 0 .. span-1
+        if (std::is_signed<T>::value && r > (__int128)L::max()) r -= span;
+        return (T)r;
+    }
+    static T sat(__int128 v) { return v < (__int128)L::min() ? L::min() : (v > (__int128)L::max() ? L::max() : (T)v); }
+    static T neg(T x) { return wrap(-(__int128)x); }
+    static T abs(T x) { return wrap(x < 0 ? -(__int128)x : (__int128)x); }
+    static T sign(T x) { return x > 0 ? T(1) : (x < 0 ? T(-1) : T(0)); }
+    static T square(T x) {
+        if (!std::is_signed<T>::value && sizeof(T) == 8) return (T)((unsigned long long)x * (unsigned long long)x);   // (x^2 can pass 2^127: unsigned 64-bit product wraps as required)
+        return wrap((__int128)x * (__int128)x);
+    }
+    static T sqrt(T x) {                                          // `(x as f32).sqrt() as T`; i64: f64; of |x| for signed types
+        T a = std::is_signed<T>::value ? abs(x) : x;
+        long double r = std::is_same<T, int64_t>::value ? (long double)std::sqrt((double)a) : (long double)std::sqrt((float)a);
+        if (std::isnan(r)) return 0;
+        r = std::trunc(r);
+        return r > (long double)L::max() ? L::max() : (T)r;
+    }
+    static bool logical_not(T x) { return x == 0; }
+    static T add_scalar(T x, T c) { return std::is_signed<T>::value || sizeof(T) < 8 ? sat((__int128)x + c) : (T)((unsigned __int128)x + c > L::max() ? L::max() : x + c); }
+    static T sub_scalar(T x, T c) { return sat((__int128)x - (__int128)c); }
+    static T mul_scalar(T x, T c) {
+        if (!std::is_signed<T>::value && sizeof(T) == 8) {
+            unsigned __int128 p = (unsigned __int128)x * (unsigned __int128)c;
+            return p > (unsigned __int128)L::max() ? L::max() : (T)p;
+        }
+        return sat((__int128)x * (__int128)c);
+    }
+    static T div_scalar(T x, T c) {
+        if (c == 0) return x == 0 ? T(0) : (x < 0 ? L::min() : L::max());
+        if (!std::is_signed<T>::value) return x / c;
+        return sat((__int128)x / (__int128)c);
+    }
+    static T maximum_scalar(T x, T c) { return x > c ? x : c; }
+    static T minimum_scalar(T x, T c) { return x < c ? x : c; }
+    static bool eq_scalar(T x, T c) { return x == c; }
+    static bool ne_scalar(T x, T c) { return x != c; }
+    static bool lt_scalar(T x, T c) { return x < c; }
+    static bool le_scalar(T x, T c) { return x <= c; }
+    static bool gt_scalar(T x, T c) { return x > c; }
+    static bool ge_scalar(T x, T c) { return x >= c; }
+};
+template <> struct Fx<uint8_t> : IntFx<uint8_t> {};
+template <> struct Fx<uint16_t> : IntFx<uint16_t> {};
+template <> struct Fx<uint32_t> : IntFx<uint32_t> {};
+template <> struct Fx<uint64_t> : IntFx<uint64_t> {};
+template <> struct Fx<int8_t> : IntFx<int8_t> {};
+template <> struct Fx<int16_t> : IntFx<int16_t> {};
+template <> struct Fx<int32_t> : IntFx<int32_t> {};
+template <> struct Fx<int64_t> : IntFx<int64_t> {};
+
+// bool (unary.rs:126, 136, 158, 208, 222, 236, 254, 264, 361, 376, 390, 404, 452, 538, 552, 564, 656-661)
+template <> struct Fx<bool> {
+    using T = bool;
+    static T neg(T x) { return !x; }
+    static T abs(T x) { return x; }
+    static T sign(T x) { return x; }
+    static T square(T x) { return x; }
+    static T sqrt(T x) { return x; }
+    static T relu(T x) { return x; }
+    static T sigmoid(T x) { return x; }
+    static T tanh(T x) { return x; }
+    static bool logical_not(T x) { return !x; }
+    static T add_scalar(T x, T c) { return x || c; }
+    static T sub_scalar(T x, T c) { return x ^ c; }
+    static T mul_scalar(T x, T c) { return x && c; }
+    static T div_scalar(T x, T c) { return x && c; }
+    static T maximum_scalar(T x, T c) { return x | c; }
+    static T minimum_scalar(T x, T c) { return x & c; }
+    static T pow(T x, T) { return x; }
+    static bool eq_scalar(T x, T c) { return x == c; }
+    static bool ne_scalar(T x, T c) { return x != c; }
+    static bool lt_scalar(T x, T c) { return (!x) && c; }
+    static bool le_scalar(T x, T c) { return (!x) || c; }
+    static bool gt_scalar(T x, T c) { return x && (!c); }
+    static bool ge_scalar(T x, T c) { return x || (!c); }
+};
+
 }  // namespace
 
 #define ORC_UNARY(NAME, T, SUF, O)                                                                    \
@@ -159,3 +247,28 @@ ORC_ALL_FOR(float, f32)
 ORC_ALL_FOR(double, f64)
 ORC_ALL_FOR(bf16, bf16)
 ORC_ALL_FOR(f16, f16)
+
+#define ORC_COMMON_FOR(T, SUF)                                                                         \
+    ORC_UNARY(logical_not, T, SUF, bool)                                                               \
+    ORC_UNARY_C(add_scalar, T, SUF, T) ORC_UNARY_C(sub_scalar, T, SUF, T)                              \
+    ORC_UNARY_C(mul_scalar, T, SUF, T) ORC_UNARY_C(div_scalar, T, SUF, T)                              \
+    ORC_UNARY_C(maximum_scalar, T, SUF, T) ORC_UNARY_C(minimum_scalar, T, SUF, T)                      \
+    ORC_UNARY_C(eq_scalar, T, SUF, bool) ORC_UNARY_C(ne_scalar, T, SUF, bool)                          \
+    ORC_UNARY_C(lt_scalar, T, SUF, bool) ORC_UNARY_C(le_scalar, T, SUF, bool)                          \
+    ORC_UNARY_C(gt_scalar, T, SUF, bool) ORC_UNARY_C(ge_scalar, T, SUF, bool)
+#define ORC_UNSIGNED_FOR(T, SUF)                                                                       \
+    ORC_COMMON_FOR(T, SUF) ORC_UNARY(sign, T, SUF, T) ORC_UNARY(square, T, SUF, T) ORC_UNARY(sqrt, T, SUF, T)
+#define ORC_SIGNED_FOR(T, SUF) ORC_UNSIGNED_FOR(T, SUF) ORC_UNARY(neg, T, SUF, T) ORC_UNARY(abs, T, SUF, T)
+
+ORC_UNSIGNED_FOR(uint8_t, u8)
+ORC_UNSIGNED_FOR(uint16_t, u16)
+ORC_UNSIGNED_FOR(uint32_t, u32)
+ORC_UNSIGNED_FOR(uint64_t, u64)
+ORC_SIGNED_FOR(int8_t, i8)
+ORC_SIGNED_FOR(int16_t, i16)
+ORC_SIGNED_FOR(int32_t, i32)
+ORC_SIGNED_FOR(int64_t, i64)
+ORC_COMMON_FOR(bool, bool)
+ORC_UNARY(neg, bool, bool, bool) ORC_UNARY(abs, bool, bool, bool) ORC_UNARY(sign, bool, bool, bool)
+ORC_UNARY(square, bool, bool, bool) ORC_UNARY(sqrt, bool, bool, bool) ORC_UNARY(relu, bool, bool, bool)
+ORC_UNARY(sigmoid, bool, bool, bool) ORC_UNARY(tanh, bool, bool, bool) ORC_UNARY_C(pow, bool, bool, bool)

@@ -1035,3 +1035,42 @@ def test_fill_and_strided_copy_wide_dtypes(hip, dt):
         (c,) = hip.call(f"copy_strided_{dt}", n, len(lay["dims"]), meta_unary(lay["dims"], lay["strides"], lay["off"]), In(src), Out(n, dt))
         want = np.lib.stride_tricks.as_strided(src[lay["off"]:], lay["dims"], [st * src.itemsize for st in lay["strides"]]).ravel()
         assert same_bits(c, want), dt
+
+
+# ---- unary forms for f64, bool and the integers ------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", WIDE_DTS)
+@pytest.mark.parametrize("lname", list(UN_LAYOUTS))
+def test_unary_wide_dtypes_bit_exact(oracle, hip, lname, dt):
+    import maidenx_amd._signatures as S
+    lay = UN_LAYOUTS[lname]()
+    r = rng(hash(lname) % 1000 + 13)
+    x = wide_values(r, lay["size"], dt)
+    n = int(np.prod(lay["dims"]))
+    md = meta_unary(lay["dims"], lay["strides"], lay["off"])
+    plain, const = S.wide_unary_ops(dt)
+
+    def check(o, h, what):
+        if dt == "f64" and o.dtype == np.float64:
+            assert np.array_equal(np.isnan(o), np.isnan(h)), what
+            assert same_bits(np.where(np.isnan(o), 0, o), np.where(np.isnan(h), 0, h)), what
+        else:
+            assert same_bits(o, h), what
+    for op in plain:
+        odt = "bool" if op == "logical_not" else dt
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lay["dims"]), md, In(x), Out(n, odt)))
+        check(o, h, op)
+    if dt == "f64":
+        consts = [0.0, -1.5, 3.25]
+    elif dt == "bool":
+        consts = [0, 1]
+    else:
+        info = np.iinfo(NP[dt])
+        consts = [0, 3, info.max, info.min] + ([-1] if info.min < 0 else [])
+    for c in consts:
+        for op in const:
+            odt = "bool" if op in S.BOOL_OUT else dt
+            (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(lay["dims"]), md, In(x), const_arg(c, dt), Out(n, odt)))
+            if dt == "f64" and op in ("maximum_scalar", "minimum_scalar"):
+                assert np.array_equal(o, h, equal_nan=True), (op, c)
+            else:
+                check(o, h, (op, c))

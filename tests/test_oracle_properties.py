@@ -673,3 +673,81 @@ def test_oracle_casts_vs_exact_arithmetic(oracle, src):
             assert np.array_equal(out, np.asarray(want, dtype=NP[dst]), equal_nan=True), (src, dst)
         else:
             assert [int(v) for v in out] == list(want), (src, dst)
+
+
+# ---- unary forms of the integers and bool: the oracle against exact arithmetic / numpy ------------------------------
+@pytest.mark.parametrize("dt", ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"])
+def test_oracle_integer_unary_vs_exact_arithmetic(oracle, dt):
+    info = np.iinfo(NP[dt])
+    x, _ = int_operands(dt)
+    n, md = x.size, meta_unary([x.size], [1], 0)
+    X = [int(v) for v in x]
+    span = info.max - info.min + 1
+    wrap = lambda v: (v - info.min) % span + info.min
+    clip = lambda v: min(max(v, info.min), info.max)
+    plain = {"sign": [(v > 0) - (v < 0) for v in X], "square": [wrap(v * v) for v in X]}
+    if info.min < 0:
+        plain["neg"] = [wrap(-v) for v in X]
+        plain["abs"] = [wrap(abs(v)) for v in X]
+    for op, exp in plain.items():
+        (out,) = oracle.call(f"{op}_{dt}", n, 1, md, In(x), Out(n, dt))
+        assert [int(v) for v in out] == exp, op
+    # sqrt: numpy's correctly rounded float32 (int64: float64) square root of |x| (wrapped, so MIN stays negative -> NaN -> 0), then truncation
+    ft = np.float64 if dt == "i64" else np.float32
+    a = np.array([wrap(abs(v)) for v in X], dtype=object).astype(NP[dt])
+    with np.errstate(invalid="ignore"):
+        r = np.sqrt(a.astype(ft))
+    want = [0 if v != v else min(int(v), info.max) for v in r.tolist()]
+    (out,) = oracle.call(f"sqrt_{dt}", n, 1, md, In(x), Out(n, dt))
+    assert [int(v) for v in out] == want
+    (out,) = oracle.call(f"logical_not_{dt}", n, 1, md, In(x), Out(n, "bool"))
+    assert np.array_equal(out.astype(bool), x == 0)
+    for c in [0, 1, 3, info.max, info.min, info.max // 3] + ([-1, -7] if info.min < 0 else []):
+
+        def quotient(v):
+            if c == 0:
+                return 0 if v == 0 else (info.min if v < 0 else info.max)
+            q = abs(v) // abs(c)
+            return clip(q if (v < 0) == (c < 0) else -q)
+        const = {"add_scalar": [clip(v + c) for v in X], "sub_scalar": [clip(v - c) for v in X], "mul_scalar": [clip(v * c) for v in X],
+                 "div_scalar": [quotient(v) for v in X], "maximum_scalar": [max(v, c) for v in X], "minimum_scalar": [min(v, c) for v in X]}
+        for op, exp in const.items():
+            (out,) = oracle.call(f"{op}_{dt}", n, 1, md, In(x), const_arg(c, dt), Out(n, dt))
+            assert [int(v) for v in out] == exp, (op, c)
+        cv = NP[dt](c)
+        cmp = {"eq_scalar": x == cv, "ne_scalar": x != cv, "lt_scalar": x < cv, "le_scalar": x <= cv, "gt_scalar": x > cv, "ge_scalar": x >= cv}
+        for op, exp in cmp.items():
+            (out,) = oracle.call(f"{op}_{dt}", n, 1, md, In(x), const_arg(c, dt), Out(n, "bool"))
+            assert np.array_equal(out.astype(bool), exp), (op, c)
+
+
+def test_oracle_bool_unary_truth_tables(oracle):
+    x = np.array([1, 0, 0, 1], dtype=np.uint8)                    # the reference's TEST_DATA_BOOL (ops_unary.rs)
+    md = meta_unary([4], [1], 0)
+    for op in ["abs", "sign", "square", "sqrt", "relu", "sigmoid", "tanh"]:
+        (out,) = oracle.call(f"{op}_bool", 4, 1, md, In(x), Out(4, "bool"))
+        assert out.tolist() == x.tolist(), op
+    (out,) = oracle.call("neg_bool", 4, 1, md, In(x), Out(4, "bool"))
+    assert out.tolist() == [0, 1, 1, 0]
+    (out,) = oracle.call("logical_not_bool", 4, 1, md, In(x), Out(4, "bool"))
+    assert out.tolist() == [0, 1, 1, 0]                           # ops_unary.rs:1036-1040
+    for c in (0, 1):
+        tables = {"add_scalar": x | c, "sub_scalar": x ^ c, "mul_scalar": x & c, "div_scalar": x & c, "maximum_scalar": x | c,
+                  "minimum_scalar": x & c, "pow": x, "eq_scalar": x == c, "ne_scalar": x != c, "lt_scalar": x < c, "le_scalar": x <= c,
+                  "gt_scalar": x > c, "ge_scalar": x >= c}
+        for op, exp in tables.items():
+            (out,) = oracle.call(f"{op}_bool", 4, 1, md, In(x), const_arg(c, "bool"), Out(4, "bool"))
+            assert out.tolist() == np.asarray(exp).astype(np.uint8).tolist(), (op, c)
+
+
+def test_oracle_integer_scalar_comparisons_match_reference_vectors(oracle):
+    # ops_unary.rs: TEST_DATA_U32 = [1, 0, 2, 3]; eq/ne/lt/le_scalar(2), gt_scalar(1), logical_not (:1041-1046, 1472-1560)
+    for dt in ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]:
+        x = np.array([1, 0, 2, 3], dtype=NP[dt])
+        md = meta_unary([4], [1], 0)
+        for op, c, exp in (("eq_scalar", 2, [0, 0, 1, 0]), ("ne_scalar", 2, [1, 1, 0, 1]), ("lt_scalar", 2, [1, 1, 0, 0]),
+                           ("le_scalar", 2, [1, 1, 1, 0]), ("gt_scalar", 1, [0, 0, 1, 1])):
+            (out,) = oracle.call(f"{op}_{dt}", 4, 1, md, In(x), const_arg(c, dt), Out(4, "bool"))
+            assert out.tolist() == exp, (op, dt)
+        (out,) = oracle.call(f"logical_not_{dt}", 4, 1, md, In(x), Out(4, "bool"))
+        assert out.tolist() == [0, 1, 0, 0]
