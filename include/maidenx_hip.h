@@ -166,8 +166,9 @@ MX_DECL_UNARY(mx_f16, f16)
  * The forms that are exact everywhere (semantics: crates/maidenx_cpu/src/ops/unary.rs:124-230, 234-236, 354-369,
  * 374-560, 564, 585-589, 650-740): integer neg / abs / square wrap on overflow as the reference's release build does,
  * integer sqrt is `(x as f32).sqrt() as T` of |x| (i64 through f64), the scalar add / sub / mul saturate; bool: neg = not,
- * add_scalar = or, sub_scalar = xor, mul_scalar = div_scalar = and, the rest identity.  Not built: the f64
- * transcendentals, gelu, pow and elu, and the integer pow (a float powf and a cast in the reference). */
+ * add_scalar = or, sub_scalar = xor, mul_scalar = div_scalar = and, the rest identity.  The f64 transcendental forms
+ * use the device math library (within 2 ulp of the host libm).  Not built: the integer pow (a float powf and a cast
+ * in the reference). */
 void hip_logical_not_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, mx_bool* output);
 void hip_sign_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
 void hip_square_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
@@ -189,6 +190,21 @@ void hip_le_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, 
 void hip_gt_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
 void hip_ge_scalar_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, mx_bool* output);
 void hip_leaky_relu_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_sigmoid_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_tanh_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_gelu_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_sin_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_cos_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_tan_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_ln_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_log10_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_log2_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_exp_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_exp10_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_exp2_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_softplus_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_pow_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
+void hip_elu_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double constant, double* output);
 void hip_logical_not_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
 void hip_neg_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);
 void hip_abs_bool(size_t num_els, size_t num_dims, const size_t* metadata, const mx_bool* input, mx_bool* output);

@@ -99,8 +99,8 @@ def wide_unary_ops(dt):
         if dt[0] in "if":
             plain += ["neg", "abs"]
         if dt == "f64":
-            plain += ["relu", "recip"]
-            const += ["leaky_relu"]
+            plain += ["relu", "recip", "sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln", "log10", "log2", "exp", "exp10", "exp2", "softplus"]
+            const += ["leaky_relu", "pow", "elu"]
     return plain, const
 
 

@@ -6,6 +6,14 @@ MXH_WIDE_SIGNED(double, f64)
 MXH_WU(relu, WRelu, double, double, f64, double)
 MXH_WU(recip, WRecip, double, double, f64, double)
 MXH_WUC(leaky_relu, WLeakyRelu, double, double, f64, double)
+MXH_WU(sigmoid, WSigmoid, double, double, f64, double) MXH_WU(tanh, WTanh, double, double, f64, double)
+MXH_WU(gelu, WGelu, double, double, f64, double) MXH_WU(sin, WSin, double, double, f64, double)
+MXH_WU(cos, WCos, double, double, f64, double) MXH_WU(tan, WTan, double, double, f64, double)
+MXH_WU(ln, WLn, double, double, f64, double) MXH_WU(log10, WLog10, double, double, f64, double)
+MXH_WU(log2, WLog2, double, double, f64, double) MXH_WU(exp, WExp, double, double, f64, double)
+MXH_WU(exp10, WExp10, double, double, f64, double) MXH_WU(exp2, WExp2, double, double, f64, double)
+MXH_WU(softplus, WSoftplus, double, double, f64, double)
+MXH_WUC(pow, WPow, double, double, f64, double) MXH_WUC(elu, WElu, double, double, f64, double)
 
 MXH_WIDE_COMMON(mxh::b8_t, uint8_t, bool)
 MXH_WU(neg, WNeg, mxh::b8_t, uint8_t, bool, uint8_t)

@@ -1,7 +1,7 @@
 // Unary element functions for f64, bool and the integers, after crates/maidenx_cpu/src/ops/unary.rs (line numbers at
-// each group).  Only the forms that are exact in every implementation are here: negation, absolute value, sign,
-// square, square root, the scalar arithmetic and comparisons (f64 also relu, reciprocal, leaky relu); the f64
-// transcendentals and the integer `pow` (a float `powf` and a cast in the reference) are not built.
+// each group).  f64 has every form of the family (the transcendental ones through the device math library); bool and
+// the integers have the forms the reference gives them, except the integer `pow` (a float `powf` and a cast in the
+// reference), which is not built.
 // Integer negation, absolute value and square wrap on overflow, as the reference's release build does (its debug
 // build panics there); the scalar add / sub / mul saturate like the binary forms.
 #pragma once
@@ -29,6 +29,27 @@ template <> struct Wide<double> {
     static __device__ T maximum_scalar(T x, T c) { return fmax(x, c); }               // :537
     static __device__ T minimum_scalar(T x, T c) { return fmin(x, c); }
     static __device__ T leaky_relu(T x, T a) { return x > 0.0 ? x : a * x; }          // :585-589
+    // transcendental forms (unary.rs:253, 263, 274-279, 295-355, 563, 611-617): the device math library's double
+    // routines, each step a separate f64 operation as in the reference; results within 2 ulp of the host libm's
+    static __device__ T sigmoid(T x) { return 1.0 / (1.0 + ::exp(-x)); }
+    static __device__ T tanh(T x) { return ::tanh(x); }
+    static __device__ T gelu(T x) {
+        const T sqrt_2_over_pi = 0.7978845608028654, coeff = 0.044715;
+        const T tanh_arg = sqrt_2_over_pi * (x + coeff * x * x * x);
+        return 0.5 * x * (1.0 + ::tanh(tanh_arg));
+    }
+    static __device__ T sin(T x) { return ::sin(x); }
+    static __device__ T cos(T x) { return ::cos(x); }
+    static __device__ T tan(T x) { return ::tan(x); }
+    static __device__ T ln(T x) { return ::log(x); }
+    static __device__ T log10(T x) { return ::log10(x); }
+    static __device__ T log2(T x) { return ::log2(x); }
+    static __device__ T exp(T x) { return ::exp(x); }
+    static __device__ T exp10(T x) { return ::pow(10.0, x); }
+    static __device__ T exp2(T x) { return ::exp2(x); }
+    static __device__ T softplus(T x) { return ::log(1.0 + ::exp(x)); }
+    static __device__ T pow(T x, T c) { return ::pow(x, c); }
+    static __device__ T elu(T x, T a) { return x > 0.0 ? x : a * (::exp(x) - 1.0); }
 };
 
 template <class I> struct WideInt {                       // unary.rs:127-130, 137-140, 159-198, 209-216, 223-230, 362-369
@@ -93,6 +114,9 @@ template <> struct Wide<b8_t> {
     };
 MXH_W1(Neg, neg) MXH_W1(Abs, abs) MXH_W1(Sign, sign) MXH_W1(Square, square) MXH_W1(Sqrt, sqrt) MXH_W1(Relu, relu)
 MXH_W1(Recip, recip) MXH_W1(LogicalNot, logical_not) MXH_W1(Same, same)
+MXH_W1(Sigmoid, sigmoid) MXH_W1(Tanh, tanh) MXH_W1(Gelu, gelu) MXH_W1(Sin, sin) MXH_W1(Cos, cos) MXH_W1(Tan, tan) MXH_W1(Ln, ln)
+MXH_W1(Log10, log10) MXH_W1(Log2, log2) MXH_W1(Exp, exp) MXH_W1(Exp10, exp10) MXH_W1(Exp2, exp2) MXH_W1(Softplus, softplus)
+MXH_W1C(Elu, elu)
 MXH_W1C(AddScalar, add_scalar) MXH_W1C(SubScalar, sub_scalar) MXH_W1C(MulScalar, mul_scalar) MXH_W1C(DivScalar, div_scalar)
 MXH_W1C(MaximumScalar, maximum_scalar) MXH_W1C(MinimumScalar, minimum_scalar) MXH_W1C(LeakyRelu, leaky_relu) MXH_W1C(Pow, pow)
 // comparisons with a constant: on the value itself (bool: false < true), unary.rs:656-740
