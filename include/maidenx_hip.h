@@ -385,6 +385,48 @@ MX_DECL_REDUCE(float, f32)
 MX_DECL_REDUCE(mx_bf16, bf16)
 MX_DECL_REDUCE(mx_f16, f16)
 
+/* The same for f64 and the integers (crates/maidenx_cuda/src/ops/reduction.rs:59-113; mean for f64 only, as in
+ * crates/maidenx_cpu/src/ops/reduction.rs:581-586).  The accumulator is the storage type: integer sums wrap (the
+ * reference's release build), so they are bit-exact in any order; f64 sums differ from the sequential order by
+ * rounding.  sum_to_shape takes contiguous inputs only for these dtypes; fold is not built for them. */
+void hip_sum_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
+void hip_max_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
+void hip_min_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
+void hip_mean_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
+void hip_sum_to_shape_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_sum_u8(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_max_u8(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_min_u8(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_sum_to_shape_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_sum_u16(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_max_u16(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_min_u16(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_sum_to_shape_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_sum_u32(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_max_u32(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_min_u32(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_sum_to_shape_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_sum_u64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_max_u64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_min_u64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_sum_to_shape_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_sum_i8(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_max_i8(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_min_i8(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_sum_to_shape_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_sum_i16(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_max_i16(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_min_i16(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_sum_to_shape_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_sum_i32(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_max_i32(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_min_i32(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_sum_to_shape_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_sum_i64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_max_i64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_min_i64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+void hip_sum_to_shape_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
+
 /* ---- matmul: replaces crates/maidenx_cuda/src/ops/matmul.rs:12-29 ---------------------------------
  * metadata = out_ndim, a_ndim, b_ndim | out_shape | a_shape | b_shape | a_strides | b_strides | a_off | b_off
  * Semantics: crates/maidenx_cpu/src/ops/matmul.rs:5-122 (forward; strided operands use strides[0]

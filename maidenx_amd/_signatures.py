@@ -115,6 +115,19 @@ def wide_unary_signatures(dtypes=WIDE_DTYPES):
     return sig
 
 
+REDUCE_WIDE_DTYPES = ("f64", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64")
+
+
+def wide_reduce_signatures(dtypes=REDUCE_WIDE_DTYPES):
+    """sum / max / min / sum_to_shape for f64 and the integers, mean for f64."""
+    sig = {}
+    for dt in dtypes:
+        for op in ("sum", "max", "min") + (("mean",) if dt == "f64" else ()):
+            sig[f"{op}_{dt}"] = [SZ, SZ, SZ, P, P, P]
+        sig[f"sum_to_shape_{dt}"] = [SZ, SZ, P, P, P]
+    return sig
+
+
 def index_signatures(dtypes=("f32", "bf16", "f16")):
     """Index ops (host loops in the reference's tensor layer, device entry points here)."""
     sig = {}
@@ -145,4 +158,5 @@ def extension_signatures():
     sig.update(cast_signatures())
     sig.update(wide_util_signatures())
     sig.update(wide_unary_signatures())
+    sig.update(wide_reduce_signatures())
     return sig

@@ -153,6 +153,17 @@ def run(flt="", sets=4, random_grad=False, out=sys.stdout):
         f = getattr(lib, f"hip_mul_{dt}")
         timeit(f"mul_{dt}/bcast_row", lambda: f(n, 2, md.ctypes.data, x, y, z), n * 2 * e)
 
+    # ---- reductions on the other dtypes: 256 MB read as [rows, 8192] of 4- and 8-byte elements ---------------------------
+    for dt, e in (("i32", 4), ("i64", 8), ("f64", 8)):
+        x, z = buf("x", N * 4), buf("z", N * 4)
+        rows = R * 4 // e
+        n = rows * Cc
+        for op in ("sum", "max"):
+            f = getattr(lib, f"hip_{op}_{dt}")
+            for dim, red_stride in ((0, Cc), (1, 1)):
+                md = u64([rows, Cc], cont, [rows, Cc][dim], red_stride, 0)
+                timeit(f"{op}_{dt}/[{rows},{Cc}] dim {dim}", lambda: f(n, 2, 1, md.ctypes.data, x, z), n * e + (n // [rows, Cc][dim]) * e)
+
     # ---- what the memory system gives a plain stream -------------------------------------------------------
     zf = buf("z", N * 4)
     timeit("fill_f32/268MB (write only)", lambda: lib.hip_fill_f32(N, zf, 1.0), N * 4)

@@ -57,6 +57,15 @@ inline size_t dst_of(size_t i, size_t nred, const size_t* red_l, const size_t* r
     return dst;
 }
 
+// `+=` of the accumulating loops.  For the integer dtypes an overflow panics in the reference's debug build and wraps
+// in its release build; the wrap is restated (through the unsigned type, where C++ defines it).
+template <typename T> inline T add_wrap(T a, T b) {
+    if constexpr (std::is_integral<T>::value) {
+        using U = typename std::make_unsigned<T>::type;
+        return (T)(U)((U)a + (U)b);
+    } else return a + b;
+}
+
 // Shared skeleton of sum_op! (:6-89), mean_op! (:185-272), max_op! (:383-467), min_op! (:469-553).
 template <typename T, typename Acc, typename Fin>
 void reduce_axis(size_t num_els, size_t num_dims, size_t nred, const size_t* md, const T* inp, T* out, T init,
@@ -114,7 +123,7 @@ void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in
             src = (s + offset) % num_els;
         }
         T v = in[src];
-        locked(cells[dst], threaded, [&](T& o) { o += v; });
+        locked(cells[dst], threaded, [&](T& o) { o = add_wrap(o, v); });
     }
     for (size_t i = 0; i < out_size; ++i) out[i] = cells[i].val;
 }
@@ -164,7 +173,7 @@ void fold(size_t num_els, size_t nd, const size_t* md, const T* inp, T* out) {
 
 #define ORC_REDUCE_FOR(T, SUF)                                                                                  \
     extern "C" void oracle_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {   \
-        reduce_axis<T>(n, nd, nr, md, in, out, zero_of<T>(), [](T& o, T v) { o += v; }, [](T v) { return v; }); \
+        reduce_axis<T>(n, nd, nr, md, in, out, zero_of<T>(), [](T& o, T v) { o = add_wrap(o, v); }, [](T v) { return v; }); \
     }                                                                                                           \
     extern "C" void oracle_mean_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {  \
         size_t f = 1;                                                                                           \
@@ -192,3 +201,28 @@ ORC_REDUCE_FOR(float, f32)
 ORC_REDUCE_FOR(double, f64)
 ORC_REDUCE_FOR(bf16, bf16)
 ORC_REDUCE_FOR(f16, f16)
+
+// the integer dtypes have sum, max, min and sum_to_shape (reduction.rs:559-566, 572-579, 605-612, 618-625); no mean
+#define ORC_REDUCE_INT_FOR(T, SUF)                                                                              \
+    extern "C" void oracle_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {   \
+        reduce_axis<T>(n, nd, nr, md, in, out, T(0), [](T& o, T v) { o = add_wrap(o, v); }, [](T v) { return v; }); \
+    }                                                                                                           \
+    extern "C" void oracle_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {   \
+        reduce_axis<T>(n, nd, nr, md, in, out, std::numeric_limits<T>::min(), [](T& o, T v) { o = v > o ? v : o; }, \
+                       [](T v) { return v; });                                                                  \
+    }                                                                                                           \
+    extern "C" void oracle_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {   \
+        reduce_axis<T>(n, nd, nr, md, in, out, std::numeric_limits<T>::max(), [](T& o, T v) { o = v < o ? v : o; }, \
+                       [](T v) { return v; });                                                                  \
+    }                                                                                                           \
+    extern "C" void oracle_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {     \
+        sum_to_shape<T>(n, nd, md, in, out);                                                                    \
+    }
+ORC_REDUCE_INT_FOR(uint8_t, u8)
+ORC_REDUCE_INT_FOR(uint16_t, u16)
+ORC_REDUCE_INT_FOR(uint32_t, u32)
+ORC_REDUCE_INT_FOR(uint64_t, u64)
+ORC_REDUCE_INT_FOR(int8_t, i8)
+ORC_REDUCE_INT_FOR(int16_t, i16)
+ORC_REDUCE_INT_FOR(int32_t, i32)
+ORC_REDUCE_INT_FOR(int64_t, i64)

@@ -169,7 +169,8 @@ class Runner:
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None
-            for name, args in {**S.cast_signatures(), **S.wide_unary_signatures(tuple(d for d in S.WIDE_DTYPES if d != "f64"))}.items():
+            for name, args in {**S.cast_signatures(), **S.wide_unary_signatures(tuple(d for d in S.WIDE_DTYPES if d != "f64")),
+                               **S.wide_reduce_signatures(tuple(d for d in S.REDUCE_WIDE_DTYPES if d != "f64"))}.items():
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None

@@ -1097,3 +1097,59 @@ def test_unary_wide_dtypes_bit_exact(oracle, hip, lname, dt):
                 assert np.array_equal(o, h, equal_nan=True), (op, c)
             else:
                 check(o, h, (op, c))
+
+
+# ---- reductions for f64 and the integers ---------------------------------------------------------------------------------
+RED_WIDE = ["f64", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
+
+
+@pytest.mark.parametrize("dt", RED_WIDE)
+@pytest.mark.parametrize("shape,dim", RED_CASES)
+def test_reductions_wide_dtypes(oracle, hip, shape, dim, dt):
+    r = rng(43)
+    n = int(np.prod(shape))
+    off = 1 if n % 2 else 0
+    if dt == "f64":
+        x = np.concatenate([np.full(off, 5.0), r.uniform(-1, 1, n)])
+    else:
+        info = np.iinfo(NP[dt])
+        x = r.integers(info.min, info.max, n + off, dtype=NP[dt], endpoint=True)          # sums wrap many times over
+    md = meta_reduce(shape, contiguous_strides(shape), dim, off)
+    for op in ["sum", "max", "min"] + (["mean"] if dt == "f64" else []):
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(shape), 1, md, In(x), Out(n // shape[dim], dt)))
+        if dt != "f64" or op in ("max", "min"):
+            assert same_bits(o, h), op
+            continue
+        xs = x[off:].reshape(shape)
+        scale = np.abs(xs).sum(dim).ravel() / (shape[dim] if op == "mean" else 1)
+        assert np.max(np.abs(h - o) / np.maximum(scale, 1e-300)) <= 1e-13, op         # f64: the two summation orders agree to rounding
+
+
+@pytest.mark.parametrize("dt", RED_WIDE)
+@pytest.mark.parametrize("shape,out_shape", STS_CASES)
+def test_sum_to_shape_wide_dtypes(oracle, hip, shape, out_shape, dt):
+    r = rng(47)
+    n = int(np.prod(shape))
+    x = r.uniform(-1, 1, n) if dt == "f64" else r.integers(np.iinfo(NP[dt]).min, np.iinfo(NP[dt]).max, n, dtype=NP[dt], endpoint=True)
+    md = meta_sum_to_shape(shape, contiguous_strides(shape), out_shape, 0)
+    n_out = int(np.prod(out_shape))
+    (o,), (h,) = both(oracle, hip, f"sum_to_shape_{dt}", lambda: (n, len(shape), md, In(x), Out(n_out, dt)))
+    if dt != "f64":
+        assert same_bits(o, h)
+        return
+    axes = tuple(i for i, (a, b) in enumerate(zip(shape, out_shape)) if a != b)
+    scale = np.abs(x.reshape(shape)).sum(axis=axes).ravel() if axes else np.abs(x)
+    assert np.max(np.abs(h - o) / np.maximum(scale, 1e-300)) <= 1e-13
+
+
+def test_reduce_wide_strided_input_and_nan_rule(oracle, hip):
+    lay = LY.permuted([30, 50], [1, 0])
+    x = rng(53).integers(-1000, 1000, lay["size"], dtype=np.int64)
+    md = meta_reduce(lay["dims"], lay["strides"], 1, lay["off"])
+    (o,), (h,) = both(oracle, hip, "sum_i64", lambda: (30 * 50, 2, 1, md, In(x), Out(30, "i64")))
+    assert same_bits(o, h)
+    for data in ([-np.inf, np.nan, -np.inf, np.nan], [np.nan, 2.0, np.nan, -1.0]):
+        v = np.array(data, dtype=np.float64)
+        for op in ("max", "min"):
+            (o,), (h,) = both(oracle, hip, f"{op}_f64", lambda: (4, 1, 1, meta_reduce([4], [1], 0), In(v), Out(1, "f64")))
+            assert same_bits(o, h), (op, data)

@@ -751,3 +751,26 @@ def test_oracle_integer_scalar_comparisons_match_reference_vectors(oracle):
             assert out.tolist() == exp, (op, dt)
         (out,) = oracle.call(f"logical_not_{dt}", 4, 1, md, In(x), Out(4, "bool"))
         assert out.tolist() == [0, 1, 0, 0]
+
+
+# ---- integer reductions: the oracle against numpy's wrapping sums and exact extrema -----------------------------------
+@pytest.mark.parametrize("dt", ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"])
+@pytest.mark.parametrize("shape,dim", [([7, 9], 0), ([7, 9], 1), ([4, 5, 6], 1), ([300], 0)])
+def test_oracle_integer_reductions_vs_numpy(oracle, shape, dim, dt):
+    info = np.iinfo(NP[dt])
+    n = int(np.prod(shape))
+    x = rng(5).integers(info.min, info.max, n, dtype=NP[dt], endpoint=True)         # sums overflow: they must wrap
+    md = meta_reduce(shape, contiguous_strides(shape), dim, 0)
+    xs = x.reshape(shape)
+    with np.errstate(over="ignore"):
+        want = {"sum": xs.sum(axis=dim, dtype=NP[dt]), "max": xs.max(axis=dim), "min": xs.min(axis=dim)}      # numpy integer sums wrap
+    exact = np.asarray(np.array([int(v) for v in x], dtype=object).reshape(shape).sum(axis=dim), dtype=object).ravel()
+    span = info.max - info.min + 1
+    want = {k: np.asarray(v) for k, v in want.items()}
+    assert [int(v) for v in want["sum"].ravel()] == [(int(v) - info.min) % span + info.min for v in exact]      # ... and equal the exact sum modulo 2^bits
+    for op, exp in want.items():
+        (out,) = oracle.call(f"{op}_{dt}", n, len(shape), 1, md, In(x), Out(n // shape[dim], dt))
+        assert np.array_equal(out, exp.ravel()), op
+    out_shape = [1 if d == dim else v for d, v in enumerate(shape)]
+    (out,) = oracle.call(f"sum_to_shape_{dt}", n, len(shape), meta_sum_to_shape(shape, contiguous_strides(shape), out_shape, 0), In(x), Out(n // shape[dim], dt))
+    assert np.array_equal(out, want["sum"].ravel())
