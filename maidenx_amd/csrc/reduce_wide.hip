@@ -114,6 +114,61 @@ __global__ __launch_bounds__(WB) void wcol_kernel(const T* __restrict__ in, T* _
     *(AVec<T, VEC>*)(out + ((size_t)o * chunks + chunk) * S + (size_t)jv * VEC) = r;
 }
 
+// ---- [outer, L, S] -> [outer, chunks, S] with the axis split inside the block -------------------------------------------
+// A block is NW waves deep: wave w walks slice w of the chunk's rows for the same 64 column vectors with eight loads in
+// flight per lane, and the NW partial rows meet in LDS in wave order: the loads in flight of NW threads per column
+// without NW times the partials.  Needs S % VEC == 0 and aligned bases.
+template <class T, class R, int VEC, int NW>
+__global__ __launch_bounds__(WAVE * NW) void wcol_split_kernel(const T* __restrict__ in, T* __restrict__ out, size_t L, size_t S, uint32_t sv,
+                                                                unsigned chunks, size_t chunk_len, FastDiv div_jb, FastDiv div_chunks, double div) {
+    constexpr int U = 8;
+    const int lane = threadIdx.x % WAVE, w = threadIdx.x / WAVE;
+    uint32_t rest, jb, o, chunk;
+    fd_divmod(blockIdx.x, div_jb, rest, jb);
+    fd_divmod(rest, div_chunks, o, chunk);
+    const uint32_t jv = jb * WAVE + lane;
+    const bool live = jv < sv;
+    const size_t beg = (size_t)chunk * chunk_len, end = beg + chunk_len < L ? beg + chunk_len : L;
+    const size_t slice = (end - beg + NW - 1) / NW;
+    const size_t l0 = beg + (size_t)w * slice < end ? beg + (size_t)w * slice : end, l1 = l0 + slice < end ? l0 + slice : end;
+    T a[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) a[e] = R::template init<T>();
+    if (live) {
+        const T* src = in + ((size_t)o * L + l0) * S + (size_t)jv * VEC;
+        size_t l = l0;
+        for (; l + U <= l1; l += U, src += U * S) {
+            AVec<T, VEC> v[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) v[k] = *(const AVec<T, VEC>*)(src + k * S);
+#pragma unroll
+            for (int k = 0; k < U; ++k)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], v[k].v[e]);
+        }
+        for (; l < l1; ++l, src += S) {
+            AVec<T, VEC> v = *(const AVec<T, VEC>*)src;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], v.v[e]);
+        }
+    }
+    __shared__ T part[NW][VEC][WAVE];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[w][e][lane] = a[e];
+    __syncthreads();
+    if (w == 0 && live) {
+        AVec<T, VEC> r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            T t = part[0][e][lane];
+#pragma unroll
+            for (int k = 1; k < NW; ++k) t = R::op(t, part[k][e][lane]);
+            r.v[e] = wfin(t, div);
+        }
+        *(AVec<T, VEC>*)(out + ((size_t)o * chunks + chunk) * S + (size_t)jv * VEC) = r;
+    }
+}
+
 // ---- strided input: one thread per output element, indices as the reference's non-contiguous branch forms them -------
 template <class T, class R>
 __global__ __launch_bounds__(WB) void wgeneric_kernel(NdSpace<1> sp, const T* __restrict__ in, T* __restrict__ out, size_t num_els,
@@ -162,6 +217,19 @@ static bool wcol_stage(const T* in, T* out, size_t outer, size_t L, size_t S, un
     return true;
 }
 
+// The split kernel, 16 waves deep.  False when the shape does not fit it (nothing launched then).
+template <class T, class R>
+static bool wcol_split_stage(const T* in, T* out, size_t outer, size_t L, size_t S, unsigned chunks, size_t chunk_len, double div) {
+    constexpr int V = 16 / sizeof(T), NW = 16;
+    if (S % V != 0 || (uintptr_t)in % 16 != 0 || (uintptr_t)out % 16 != 0) return false;
+    const size_t sv = S / V, jblocks = cdiv(sv, (size_t)WAVE), blocks = outer * chunks * jblocks;
+    if (blocks >= (1ull << 31) || sv >= (1ull << 31)) return false;
+    hipLaunchKernelGGL((wcol_split_kernel<T, R, V, NW>), dim3((unsigned)blocks), dim3(WAVE * NW), 0, stream(), in, out, L, S, (uint32_t)sv, chunks,
+                       chunk_len, make_fastdiv((uint32_t)jblocks), make_fastdiv(chunks), div);
+    MXH_LAUNCH_CHECK("reduce_wide_col_split");
+    return true;
+}
+
 // [outer, L, S] (contiguous) -> [outer, S].  Few outputs: the axis is cut into chunks whose partial results (plain T,
 // in the library's scratch block) a second launch of the same kernels combines in chunk order.
 template <class T, class R>
@@ -183,6 +251,28 @@ static void wreduce(const T* in, T* out, size_t outer, size_t L, size_t S, doubl
         wrow_stage<T, R>(in, part, outer, L, (unsigned)chunks, chunk_len, 0.0);
         wrow_stage<T, R>(part, out, outer, chunks, 1, chunks, div);
         return;
+    }
+    {
+        // wide rows and a long axis: one 16-wave block per CU covers the memory latency, so few chunks (often none)
+        constexpr size_t V = 16 / sizeof(T);
+        if (S % V == 0 && S / V >= WAVE && L >= 256) {
+            const size_t base = outer * cdiv(S / V, (size_t)WAVE);
+            size_t nch = 1;
+            if (base < 256) nch = std::min<size_t>(cdiv((size_t)256, base), L / 256);
+            if (nch < 1) nch = 1;
+            const size_t clen = cdiv(L, nch);
+            nch = cdiv(L, clen);
+            if (nch == 1) {
+                if (wcol_split_stage<T, R>(in, out, outer, L, S, 1, L, div)) return;
+            } else {
+                T* part = (T*)scratch(outer * nch * S * sizeof(T) + 256);
+                if (!part) return;
+                if (wcol_split_stage<T, R>(in, part, outer, L, S, (unsigned)nch, clen, 0.0)) {
+                    wcol_stage<T, R>(part, out, outer, nch, S, 1, nch, div);
+                    return;
+                }
+            }
+        }
     }
     const size_t threads = outer * S / (S % (16 / sizeof(T)) == 0 ? 16 / sizeof(T) : 1);
     size_t chunks = 1;
