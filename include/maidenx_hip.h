@@ -440,6 +440,29 @@ MX_DECL_MATMUL(float, f32)
 MX_DECL_MATMUL(mx_bf16, bf16)
 MX_DECL_MATMUL(mx_f16, f16)
 
+/* The same for f64 and the integers (crates/maidenx_cuda/src/ops/matmul.rs:36-50): LDS-tiled products without a
+ * matrix instruction, each output accumulated in the storage type with the reduction index ascending and multiply and
+ * add unfused - the order of crates/maidenx_cpu/src/ops/matmul.rs:60-86 - so f64 results carry the reference's bits and
+ * integer results wrap as its release build does. */
+void hip_matmul_f64(size_t num_els, const size_t* metadata, const double* a, const double* b, double* c);
+void hip_matmul_backward_f64(size_t num_els_a, size_t num_els_b, const size_t* metadata, const double* grad_output, const double* a, const double* b, double* grad_a, double* grad_b);
+void hip_matmul_u8(size_t num_els, const size_t* metadata, const uint8_t* a, const uint8_t* b, uint8_t* c);
+void hip_matmul_backward_u8(size_t num_els_a, size_t num_els_b, const size_t* metadata, const uint8_t* grad_output, const uint8_t* a, const uint8_t* b, uint8_t* grad_a, uint8_t* grad_b);
+void hip_matmul_u16(size_t num_els, const size_t* metadata, const uint16_t* a, const uint16_t* b, uint16_t* c);
+void hip_matmul_backward_u16(size_t num_els_a, size_t num_els_b, const size_t* metadata, const uint16_t* grad_output, const uint16_t* a, const uint16_t* b, uint16_t* grad_a, uint16_t* grad_b);
+void hip_matmul_u32(size_t num_els, const size_t* metadata, const uint32_t* a, const uint32_t* b, uint32_t* c);
+void hip_matmul_backward_u32(size_t num_els_a, size_t num_els_b, const size_t* metadata, const uint32_t* grad_output, const uint32_t* a, const uint32_t* b, uint32_t* grad_a, uint32_t* grad_b);
+void hip_matmul_u64(size_t num_els, const size_t* metadata, const uint64_t* a, const uint64_t* b, uint64_t* c);
+void hip_matmul_backward_u64(size_t num_els_a, size_t num_els_b, const size_t* metadata, const uint64_t* grad_output, const uint64_t* a, const uint64_t* b, uint64_t* grad_a, uint64_t* grad_b);
+void hip_matmul_i8(size_t num_els, const size_t* metadata, const int8_t* a, const int8_t* b, int8_t* c);
+void hip_matmul_backward_i8(size_t num_els_a, size_t num_els_b, const size_t* metadata, const int8_t* grad_output, const int8_t* a, const int8_t* b, int8_t* grad_a, int8_t* grad_b);
+void hip_matmul_i16(size_t num_els, const size_t* metadata, const int16_t* a, const int16_t* b, int16_t* c);
+void hip_matmul_backward_i16(size_t num_els_a, size_t num_els_b, const size_t* metadata, const int16_t* grad_output, const int16_t* a, const int16_t* b, int16_t* grad_a, int16_t* grad_b);
+void hip_matmul_i32(size_t num_els, const size_t* metadata, const int32_t* a, const int32_t* b, int32_t* c);
+void hip_matmul_backward_i32(size_t num_els_a, size_t num_els_b, const size_t* metadata, const int32_t* grad_output, const int32_t* a, const int32_t* b, int32_t* grad_a, int32_t* grad_b);
+void hip_matmul_i64(size_t num_els, const size_t* metadata, const int64_t* a, const int64_t* b, int64_t* c);
+void hip_matmul_backward_i64(size_t num_els_a, size_t num_els_b, const size_t* metadata, const int64_t* grad_output, const int64_t* a, const int64_t* b, int64_t* grad_a, int64_t* grad_b);
+
 /* ---- padding: replaces crates/maidenx_cuda/src/ops/padding.rs:13-71 (constant mode) ---------------
  * metadata = in_dims[n] | in_strides[n] | in_offset | out_dims[n] | (pad_before, pad_after)[n]
  * Semantics: crates/maidenx_cpu/src/ops/padding.rs:7-113 and :327-436.  Bit-exact. */

@@ -119,12 +119,14 @@ REDUCE_WIDE_DTYPES = ("f64", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64
 
 
 def wide_reduce_signatures(dtypes=REDUCE_WIDE_DTYPES):
-    """sum / max / min / sum_to_shape for f64 and the integers, mean for f64."""
+    """sum / max / min / sum_to_shape and matmul / matmul_backward for f64 and the integers, mean for f64."""
     sig = {}
     for dt in dtypes:
         for op in ("sum", "max", "min") + (("mean",) if dt == "f64" else ()):
             sig[f"{op}_{dt}"] = [SZ, SZ, SZ, P, P, P]
         sig[f"sum_to_shape_{dt}"] = [SZ, SZ, P, P, P]
+        sig[f"matmul_{dt}"] = [SZ, P, P, P, P]
+        sig[f"matmul_backward_{dt}"] = [SZ, SZ, P, P, P, P, P, P]
     return sig
 
 

@@ -183,6 +183,14 @@ def run(flt="", sets=4, random_grad=False, out=sys.stdout):
             timeit(f"matmul_{dt}/{b}x{m_}x{k}x{n} dA", lambda: g(b * m_ * k, b * k * n, md.ctypes.data, c, a, bb, ga, None), nb, reps=5, flops=fl)
             timeit(f"matmul_{dt}/{b}x{m_}x{k}x{n} dB", lambda: g(b * m_ * k, b * k * n, md.ctypes.data, c, a, bb, None, gb), nb, reps=5, flops=fl)
 
+    # ---- matmul on f64 / i32: LDS-tiled products without a matrix instruction ------------------------------------------
+    for dt, e in (("f64", 8), ("i32", 4)):
+        b, m_, k, n = 1, 2048, 2048, 2048
+        a, bb, c = buf("x", N * 4), buf("y", N * 4), buf("z", N * 4)
+        md = u64(3, 3, 3, [b, m_, n], [b, m_, k], [b, k, n], [m_ * k, k, 1], [k * n, n, 1], 0, 0)
+        f = getattr(lib, f"hip_matmul_{dt}")
+        timeit(f"matmul_{dt}/{b}x{m_}x{k}x{n} fwd", lambda: f(b * m_ * n, md.ctypes.data, a, bb, c), 3 * m_ * k * e, reps=3, flops=2.0 * m_ * k * n)
+
     # ---- fused Adam step: 4 tensors read, 3 written (the reference's fourteen ops move about 40) -------------------
     for dt, e in (("f32", 4), ("bf16", 2)):
         n = N if dt == "f32" else 2 * N

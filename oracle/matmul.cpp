@@ -12,6 +12,19 @@ using namespace orc;
 
 namespace {
 
+// `acc += a * b`.  For the integer dtypes an overflow wraps (the reference's release build; a panic in its debug build):
+// done in the unsigned type, where C++ defines it.
+template <typename T> inline T mac(T acc, T a, T b) {
+    if constexpr (std::is_integral<T>::value) {
+        using U = typename std::make_unsigned<T>::type;
+        return (T)(U)((U)acc + (U)((U)a * (U)b));
+    } else {
+        acc += a * b;
+        return acc;
+    }
+}
+
+
 template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
 template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
@@ -62,7 +75,7 @@ void matmul(size_t num_els, const size_t* md, const T* a, const T* b, T* c) {
                 size_t b_base = batch_idx * (k * n);
                 for (size_t k_idx = 0; k_idx < k; ++k_idx) {
                     size_t ai = a_base + k_idx, bi = b_base + k_idx * n + n_idx;
-                    if (ai < a_size && bi < b_size) acc += as[ai] * bs[bi];
+                    if (ai < a_size && bi < b_size) acc = mac(acc, as[ai], bs[bi]);
                 }
             } else {
                 // :87-113 — the batch stride is strides[0] whatever the rank
@@ -73,7 +86,7 @@ void matmul(size_t num_els, const size_t* md, const T* a, const T* b, T* c) {
                     size_t bi = p.b_ndim >= 2 ? batch_idx * p.b_strides[0] + k_idx * p.b_strides[p.b_ndim - 2] +
                                                     n_idx * p.b_strides[p.b_ndim - 1]
                                               : n_idx * p.b_strides[0];
-                    if (ai < a_size && bi < b_size) acc += as[ai] * bs[bi];
+                    if (ai < a_size && bi < b_size) acc = mac(acc, as[ai], bs[bi]);
                 }
             }
             if (n_idx < row_len) c_row[n_idx] = acc;
@@ -112,7 +125,7 @@ void matmul_backward(size_t num_els_a, size_t num_els_b, const size_t* md, const
                     size_t g_base = batch_idx * (m * n) + m_idx * n, b_base = batch_idx * (k * n);
                     for (size_t n_idx = 0; n_idx < n; ++n_idx)
                         if (g_base + n_idx < go_size && b_base + k_idx * n + n_idx < num_els_b)
-                            acc += go[g_base + n_idx] * bs[b_base + k_idx * n + n_idx];
+                            acc = mac(acc, go[g_base + n_idx], bs[b_base + k_idx * n + n_idx]);
                 }
                 if (k_idx < row_len) g_row[k_idx] = acc;
             }
@@ -134,7 +147,7 @@ void matmul_backward(size_t num_els_a, size_t num_els_b, const size_t* md, const
                     size_t a_base = batch_idx * (m * k), g_base = batch_idx * (m * n);
                     for (size_t m_idx = 0; m_idx < m; ++m_idx) {
                         size_t ai = a_base + m_idx * k + k_idx, gi = g_base + m_idx * n + n_idx;
-                        if (ai < num_els_a && gi < go_size) acc += as[ai] * go[gi];
+                        if (ai < num_els_a && gi < go_size) acc = mac(acc, as[ai], go[gi]);
                     }
                 }
                 if (n_idx < row_len) g_row[n_idx] = acc;
@@ -158,3 +171,11 @@ ORC_MATMUL_FOR(float, f32)
 ORC_MATMUL_FOR(double, f64)
 ORC_MATMUL_FOR(bf16, bf16)
 ORC_MATMUL_FOR(f16, f16)
+ORC_MATMUL_FOR(uint8_t, u8)
+ORC_MATMUL_FOR(uint16_t, u16)
+ORC_MATMUL_FOR(uint32_t, u32)
+ORC_MATMUL_FOR(uint64_t, u64)
+ORC_MATMUL_FOR(int8_t, i8)
+ORC_MATMUL_FOR(int16_t, i16)
+ORC_MATMUL_FOR(int32_t, i32)
+ORC_MATMUL_FOR(int64_t, i64)

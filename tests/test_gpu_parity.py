@@ -1153,3 +1153,45 @@ def test_reduce_wide_strided_input_and_nan_rule(oracle, hip):
         for op in ("max", "min"):
             (o,), (h,) = both(oracle, hip, f"{op}_f64", lambda: (4, 1, 1, meta_reduce([4], [1], 0), In(v), Out(1, "f64")))
             assert same_bits(o, h), (op, data)
+
+
+# ---- matmul for f64 and the integers: the reference's accumulation order, so identical bits -----------------------------
+MM_WIDE_SHAPES = [(1, 128, 128, 128), (2, 130, 70, 97), (3, 64, 600, 64), (1, 1000, 3, 1), (1, 3, 1000, 1), (2, 37, 19, 53), (1, 100, 576, 64),
+                  (4, 16, 16, 16), (1, 1, 257, 1)]
+
+
+def wide_matrix(r, shape, dt):
+    if dt == "f64":
+        return r.standard_normal(shape)
+    info = np.iinfo(NP[dt])
+    return r.integers(info.min, info.max, shape, dtype=NP[dt], endpoint=True)      # products and sums wrap
+
+
+@pytest.mark.parametrize("dt", ["f64", "i32", "i64", "u8", "u64", "i16"])
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", MM_WIDE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_forward_wide_dtypes(oracle, hip, shape, a_perm, b_perm, dt):
+    batch, m, k, n = shape
+    r = rng(59)
+    a, b = wide_matrix(r, (batch, m, k), dt), wide_matrix(r, (batch, k, n), dt)
+    a_shape, b_shape = [batch, m, k], [batch, k, n]
+    a_st, b_st = contiguous_strides(a_shape), contiguous_strides(b_shape)
+    if a_perm:
+        a, a_st = np.ascontiguousarray(a.transpose(0, 2, 1)), [m * k, 1, m]
+    if b_perm:
+        b, b_st = np.ascontiguousarray(b.transpose(0, 2, 1)), [k * n, 1, k]
+    md = meta_matmul([batch, m, n], a_shape, b_shape, a_st, b_st)
+    (o,), (h,) = both(oracle, hip, f"matmul_{dt}", lambda: (batch * m * n, md, In(a.ravel()), In(b.ravel()), Out(batch * m * n, dt)))
+    assert same_bits(o, h)
+
+
+@pytest.mark.parametrize("dt", ["f64", "i32", "i64", "u16"])
+@pytest.mark.parametrize("shape", [(1, 128, 128, 128), (2, 130, 70, 97), (1, 10000, 3, 1), (3, 33, 65, 17)], ids=lambda s: "x".join(map(str, s)))
+def test_matmul_backward_wide_dtypes(oracle, hip, shape, dt):
+    batch, m, k, n = shape
+    r = rng(61)
+    a, b, go = wide_matrix(r, (batch, m, k), dt), wide_matrix(r, (batch, k, n), dt), wide_matrix(r, (batch, m, n), dt)
+    md = meta_matmul([batch, m, n], [batch, m, k], [batch, k, n], contiguous_strides([batch, m, k]), contiguous_strides([batch, k, n]))
+    build = lambda: (batch * m * k, batch * k * n, md, In(go.ravel()), In(a.ravel()), In(b.ravel()), Out(batch * m * k, dt), Out(batch * k * n, dt))
+    (oa, ob), (ha, hb) = both(oracle, hip, f"matmul_backward_{dt}", build)
+    assert same_bits(oa, ha) and same_bits(ob, hb)
