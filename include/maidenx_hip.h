@@ -503,6 +503,10 @@ MX_DECL_CONV(float, f32)
 MX_DECL_CONV(mx_bf16, bf16)
 MX_DECL_CONV(mx_f16, f16)
 
+/* f64 as well (crates/maidenx_cuda/src/nn/conv.rs:35): the same kernels, two elements per 16-byte vector. */
+void hip_conv2d_im2col_f64(size_t num_els, const size_t* metadata, const double* input, double* col);
+void hip_conv2d_col2im_f64(size_t num_els, const size_t* metadata, const double* col, double* output);
+
 /* ---- softmax: replaces crates/maidenx_cuda/src/nn/activation/softmax.rs (cuda_softmax_<T>) ------------
  * metadata = dims[n] | strides[n] | offset; dim >= num_dims means the last dim.
  * Semantics: crates/maidenx_cpu/src/nn/activation/softmax.rs:62-207 (max from -inf, the sum seeded

@@ -127,6 +127,9 @@ def wide_reduce_signatures(dtypes=REDUCE_WIDE_DTYPES):
         sig[f"sum_to_shape_{dt}"] = [SZ, SZ, P, P, P]
         sig[f"matmul_{dt}"] = [SZ, P, P, P, P]
         sig[f"matmul_backward_{dt}"] = [SZ, SZ, P, P, P, P, P, P]
+        if dt == "f64":
+            sig["conv2d_im2col_f64"] = [SZ, P, P, P]
+            sig["conv2d_col2im_f64"] = [SZ, P, P, P]
     return sig
 
 

@@ -102,6 +102,7 @@ __global__ __launch_bounds__(CB) void im2col_band_kernel(ConvMeta m, BandMeta k,
 
 template <class T> __device__ inline T acc_add(T a, T b);
 template <> __device__ inline float acc_add<float>(float a, float b) { return a + b; }
+template <> __device__ inline double acc_add<double>(double a, double b) { return a + b; }
 template <> __device__ inline bf16_t acc_add<bf16_t>(bf16_t a, bf16_t b) { return f2bf(bf2f(a) + bf2f(b)); }   // rounds per add
 template <> __device__ inline f16_t acc_add<f16_t>(f16_t a, f16_t b) { return f2h(h2f(a) + h2f(b)); }
 
@@ -317,3 +318,4 @@ using namespace mxh;
 MXH_CONV_FOR(float, f32)
 MXH_CONV_FOR(bf16_t, bf16)
 MXH_CONV_FOR(f16_t, f16)
+MXH_CONV_FOR(double, f64)      // (crates/maidenx_cuda/src/nn/conv.rs:35)

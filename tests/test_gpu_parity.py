@@ -501,7 +501,7 @@ CONV_CASES = [(2, 3, 8, 8, 3, 3, 1, 1), (1, 4, 12, 12, 3, 3, 1, 1), (2, 2, 9, 7,
              (1, 2, 16, 16, 5, 5, 2, 1), (1, 2, 8, 8, 1, 1, 0, 1), (2, 2, 9, 16, 2, 4, 1, 1)]
 
 
-@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("dt", DTS + ["f64"])
 @pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "_".join(map(str, c)))
 def test_im2col_col2im_bit_exact(oracle, hip, case, dt):
     B, Cc, H, W, kh, kw, p, s = case
@@ -518,7 +518,7 @@ def test_im2col_col2im_bit_exact(oracle, hip, case, dt):
         assert same_bits(o, h), num_els
 
 
-@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("dt", DTS + ["f64"])
 @pytest.mark.parametrize("k", [3, 4])
 def test_col2im_row_stride_two_column_stride_one(oracle, hip, k, dt):
     B, Cc, H, W, p, sh, sw = 2, 3, 15, 16, 1, 2, 1
