@@ -492,6 +492,14 @@ MX_DECL_PAD_EDGE(float, f32)
 MX_DECL_PAD_EDGE(mx_bf16, bf16)
 MX_DECL_PAD_EDGE(mx_f16, f16)
 
+/* The three pad modes for f64 as well (crates/maidenx_cuda/src/ops/padding.rs:82); backward sums are formed in f64. */
+void hip_pad_with_constant_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* input, double* output, double pad_value);
+void hip_pad_with_constant_backward_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* grad_out, double* grad_in);
+void hip_pad_with_reflection_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_pad_with_replication_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_pad_with_reflection_backward_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* grad_out, double* grad_in);
+void hip_pad_with_replication_backward_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* grad_out, double* grad_in);
+
 /* ---- conv: replaces crates/maidenx_cuda/src/nn/conv.rs:12-24 --------------------------------------
  * metadata = 12 slots B, C, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w as the kernel
  * reads them (crates/maidenx_cpu/src/nn/conv.rs:20-34).  im2col writes [B][C*kh*kw][oh*ow];

@@ -130,6 +130,11 @@ def wide_reduce_signatures(dtypes=REDUCE_WIDE_DTYPES):
         if dt == "f64":
             sig["conv2d_im2col_f64"] = [SZ, P, P, P]
             sig["conv2d_col2im_f64"] = [SZ, P, P, P]
+            sig["pad_with_constant_f64"] = [SZ, SZ, SZ, P, P, P, CONST["f64"]]
+            sig["pad_with_constant_backward_f64"] = [SZ, SZ, SZ, P, P, P]
+            for mode in ("reflection", "replication"):
+                sig[f"pad_with_{mode}_f64"] = [SZ, SZ, SZ, P, P, P]
+                sig[f"pad_with_{mode}_backward_f64"] = [SZ, SZ, SZ, P, P, P]
     return sig
 
 

@@ -25,6 +25,19 @@ struct PadSpace {
 
 
 constexpr int PB = 256;
+
+// The type the backward sums are formed in and its conversions: f32 for the three float formats of 32 or 16 bits (one
+// rounding at the end for the 16-bit ones), the storage type itself for f64.
+template <class T> struct PadAcc {
+    using A = float;
+    static __device__ A ld(T v) { return Ar<T>::to_f32(v); }
+    static __device__ T st(A a) { return Ar<T>::from_f32(a); }
+};
+template <> struct PadAcc<double> {
+    using A = double;
+    static __device__ A ld(double v) { return v; }
+    static __device__ double st(A a) { return a; }
+};
 enum EdgeMode : int { EDGE_REFLECT = 0, EDGE_REPLICATE = 1, EDGE_NONE = 2 };     // NONE: constant padding, whose border feeds nothing back
 
 // forward: out[i] = inside ? in[idx] : pad_value
@@ -87,7 +100,7 @@ __global__ __launch_bounds__(PB) void pad_const_kernel(PadSpace sp, const T* __r
         } else {
             if (inside) {
                 T g = v.v[e];
-                dst[idx] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(g));      // −0 → +0 like the reference's sums from zero
+                dst[idx] = PadAcc<T>::st((typename PadAcc<T>::A)0 + PadAcc<T>::ld(g));      // −0 → +0 like the reference's sums from zero
             }
         }
         // next output element; at the end of a row, carry into the outer coordinates
@@ -220,7 +233,7 @@ __global__ __launch_bounds__(PB) void pad_const3_kernel(Pad3 sp, const T* __rest
                 const uint32_t ic = c2 - sp.before[2];
                 const bool inside = row_in && ic < sp.in[2] && i0 + e < n_out;
                 const int64_t idx = row + (int64_t)ic * sp.in_stride[2];
-                if (inside) dst[idx] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(v[u].v[e]));      // -0 -> +0 like the reference's sums from zero
+                if (inside) dst[idx] = PadAcc<T>::st((typename PadAcc<T>::A)0 + PadAcc<T>::ld(v[u].v[e]));      // -0 -> +0 like the reference's sums from zero
                 if (++c2 == sp.out[2]) {
                     c2 = 0;
                     fresh = true;
@@ -348,7 +361,7 @@ __global__ __launch_bounds__(PB) void pad_crop3_kernel(Pad3 sp, const T* __restr
         const uint32_t i0 = base + (uint32_t)u * (PB * PER);
         if (i0 >= n_in) continue;
 #pragma unroll
-        for (uint32_t e = 0; e < PER; ++e) v[u].v[e] = Ar<T>::from_f32(0.0f + Ar<T>::to_f32(v[u].v[e]));
+        for (uint32_t e = 0; e < PER; ++e) v[u].v[e] = PadAcc<T>::st((typename PadAcc<T>::A)0 + PadAcc<T>::ld(v[u].v[e]));
         if (vec_store && i0 + PER <= n_in) {
             *(AVec<T, PER>*)(gi + i0) = v[u];
         } else {
@@ -530,9 +543,9 @@ struct EdgeIter {
 // over the output coordinates that map to p[D], the innermost level adds one gradient.
 template <class T, int D>
 __device__ __forceinline__ void edge_gather(const PadSpace& sp, const EdgeWalk& w, int mode, const uint32_t (&p)[MAXD], int64_t o,
-                                            const T* __restrict__ go, float& acc) {
+                                            const T* __restrict__ go, typename PadAcc<T>::A& acc) {
     if constexpr (D == MAXD) {
-        acc += Ar<T>::to_f32(go[o]);
+        acc = acc + PadAcc<T>::ld(go[o]);
     } else {
         if (D >= sp.ndims) { edge_gather<T, MAXD>(sp, w, mode, p, o, go, acc); return; }
         EdgeIter it;
@@ -561,9 +574,9 @@ __global__ __launch_bounds__(PB) void pad_edge_backward_kernel(PadSpace sp, Edge
             r = q;
         }
     }
-    float acc = 0.0f;
+    typename PadAcc<T>::A acc = 0;
     edge_gather<T, 0>(sp, w, mode, p, 0, go, acc);
-    gi[dst] = Ar<T>::from_f32(acc);
+    gi[dst] = PadAcc<T>::st(acc);
 }
 
 // The common shape of the backward walk: at most three dims after merging and at most one reflection per side
@@ -620,15 +633,15 @@ __global__ __launch_bounds__(PB) void pad_edge_backward3_kernel(Pad3 sp, int mod
         }
         EdgeSrc s2;
         s2.init(mode, p2, sp.in[2], sp.out[2], sp.before[2]);
-        float acc = 0.0f;
+        typename PadAcc<T>::A acc = 0;
         for (uint32_t k0 = 0; k0 < s0.n; ++k0) {
             const uint32_t o0 = s0.at(k0) * sp.out_stride[0];
             for (uint32_t k1 = 0; k1 < s1.n; ++k1) {
                 const uint32_t o1 = o0 + s1.at(k1) * sp.out_stride[1];
-                for (uint32_t k2 = 0; k2 < s2.n; ++k2) acc += Ar<T>::to_f32(go[o1 + s2.at(k2)]);
+                for (uint32_t k2 = 0; k2 < s2.n; ++k2) acc = acc + PadAcc<T>::ld(go[o1 + s2.at(k2)]);
             }
         }
-        v.v[e] = Ar<T>::from_f32(acc);
+        v.v[e] = PadAcc<T>::st(acc);
         dst[e] = row + (int64_t)p2 * sp.in_stride[2];
         if (++p2 == sp.in[2]) {
             p2 = 0;
@@ -777,3 +790,5 @@ MXH_PAD_EDGE_FOR(f16_t, f16)
 MXH_PAD_FOR(float, f32)
 MXH_PAD_FOR(bf16_t, bf16)
 MXH_PAD_FOR(f16_t, f16)
+MXH_PAD_EDGE_FOR(double, f64)      // (crates/maidenx_cuda/src/ops/padding.rs:82)
+MXH_PAD_FOR(double, f64)

@@ -463,7 +463,7 @@ PAD_CASES = [([2, 3, 8, 8], [(0, 0), (0, 0), (1, 1), (1, 1)]), ([7], [(3, 0)]), 
              ([4, 16, 14, 14], [(0, 0), (0, 0), (1, 1), (1, 1)]), ([3, 5], [(0, 0), (0, 0)])]
 
 
-@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("dt", DTS + ["f64"])
 @pytest.mark.parametrize("shape,pads", PAD_CASES)
 def test_pad_constant_forward_backward(oracle, hip, shape, pads, dt):
     r = rng(59)
@@ -538,7 +538,7 @@ EDGE_CASES = [([7], [(3, 2)]), ([5, 6], [(1, 2), (0, 3)]), ([2, 3, 4], [(1, 0), 
               ([3], [(7, 5)]), ([2, 3, 20, 24], [(0, 0), (0, 0), (3, 3), (2, 5)]), ([1, 6], [(0, 0), (2, 2)])]
 
 
-@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("dt", DTS + ["f64"])
 @pytest.mark.parametrize("mode", ["reflection", "replication"])
 @pytest.mark.parametrize("shape,pads", EDGE_CASES)
 def test_pad_edge_forward_backward(oracle, hip, shape, pads, mode, dt):
