@@ -774,3 +774,50 @@ def test_oracle_integer_reductions_vs_numpy(oracle, shape, dim, dt):
     out_shape = [1 if d == dim else v for d, v in enumerate(shape)]
     (out,) = oracle.call(f"sum_to_shape_{dt}", n, len(shape), meta_sum_to_shape(shape, contiguous_strides(shape), out_shape, 0), In(x), Out(n // shape[dim], dt))
     assert np.array_equal(out, want["sum"].ravel())
+
+
+# ---- matmul for the integers and f64: the oracle against exact integer products and a plain ascending loop ------------------
+@pytest.mark.parametrize("dt", ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64", "f64"])
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, True)])
+def test_oracle_wide_matmul_vs_exact_products(oracle, dt, a_perm, b_perm):
+    from helpers import meta_matmul
+    batch, m, k, n = 2, 5, 7, 4
+    r = rng(71)
+    if dt == "f64":
+        a, b = r.standard_normal((batch, m, k)), r.standard_normal((batch, k, n))
+    else:
+        info = np.iinfo(NP[dt])
+        a = r.integers(info.min, info.max, (batch, m, k), dtype=NP[dt], endpoint=True)
+        b = r.integers(info.min, info.max, (batch, k, n), dtype=NP[dt], endpoint=True)
+    a_st, b_st = contiguous_strides([batch, m, k]), contiguous_strides([batch, k, n])
+    sa, sb = a, b
+    if a_perm:
+        sa, a_st = np.ascontiguousarray(a.transpose(0, 2, 1)), [m * k, 1, m]
+    if b_perm:
+        sb, b_st = np.ascontiguousarray(b.transpose(0, 2, 1)), [k * n, 1, k]
+    md = meta_matmul([batch, m, n], [batch, m, k], [batch, k, n], a_st, b_st)
+    (out,) = oracle.call(f"matmul_{dt}", batch * m * n, md, In(sa.ravel()), In(sb.ravel()), Out(batch * m * n, dt))
+    if dt == "f64":
+        want = np.zeros((batch, m, n))
+        for bi in range(batch):
+            for i in range(m):
+                for j in range(n):
+                    acc = 0.0
+                    for t in range(k):                       # ascending, multiply and add as two roundings
+                        acc = acc + float(a[bi, i, t]) * float(b[bi, t, j])
+                    want[bi, i, j] = acc
+        assert np.array_equal(out.reshape(want.shape), want)
+        return
+    exact = np.einsum("bik,bkj->bij", a.astype(object), b.astype(object))           # Python integers: no overflow
+    span = info.max - info.min + 1
+    want = [(int(v) - info.min) % span + info.min for v in exact.ravel()]            # ... reduced modulo 2^bits
+    assert [int(v) for v in out] == want
+    # the two gradients are products of the same kind: dA = dC.B^T, dB = A^T.dC
+    go = r.integers(info.min, info.max, (batch, m, n), dtype=NP[dt], endpoint=True)
+    mdc = meta_matmul([batch, m, n], [batch, m, k], [batch, k, n], contiguous_strides([batch, m, k]), contiguous_strides([batch, k, n]))
+    ga, gb = oracle.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, mdc, In(go.ravel()), In(a.ravel()), In(b.ravel()),
+                         Out(batch * m * k, dt), Out(batch * k * n, dt))
+    ea = np.einsum("bij,bkj->bik", go.astype(object), b.astype(object))
+    eb = np.einsum("bik,bij->bkj", a.astype(object), go.astype(object))
+    assert [int(v) for v in ga] == [(int(v) - info.min) % span + info.min for v in ea.ravel()]
+    assert [int(v) for v in gb] == [(int(v) - info.min) % span + info.min for v in eb.ravel()]
