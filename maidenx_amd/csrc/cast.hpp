@@ -32,7 +32,7 @@ template <class TI, class TO> struct OpCast {
 }  // namespace mxh
 
 #define MXH_CAST_WIDE(TI, PI, SI, TO, PO, SO)                                                              \
-    extern "C" void hip_cast_##SI##_##SO(size_t n, const PI* in, PO* out) {                                \
+    extern "C" void hip_cast_##SI##_##SO(size_t n, const PI* in, PO* out) { MXH_API;                       \
         if (!in) { mxh::set_status(mxh::ERR_INVALID, "cast: null input"); return; }                        \
         mxh::ew_unary(n, 1, nullptr, (const TI*)in, (TO*)out, mxh::OpCast<TI, TO>{});                      \
     }

@@ -308,10 +308,10 @@ void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
 using namespace mxh;
 
 #define MXH_CONV_FOR(T, SUF)                                                                               \
-    extern "C" void hip_conv2d_im2col_##SUF(size_t num_els, const size_t* md, const T* in, T* col) {       \
+    extern "C" void hip_conv2d_im2col_##SUF(size_t num_els, const size_t* md, const T* in, T* col) { MXH_API; \
         im2col<T>(num_els, md, in, col);                                                                   \
     }                                                                                                      \
-    extern "C" void hip_conv2d_col2im_##SUF(size_t num_els, const size_t* md, const T* col, T* out) {      \
+    extern "C" void hip_conv2d_col2im_##SUF(size_t num_els, const size_t* md, const T* col, T* out) { MXH_API; \
         col2im<T>(num_els, md, col, out);                                                                  \
     }
 

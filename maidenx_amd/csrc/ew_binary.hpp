@@ -9,12 +9,12 @@ using namespace mxh;
 
 #define MXH_BINARY(NAME, OP, T, SUF, O)                                                                       \
     extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* lhs,       \
-                                       const T* rhs, O* out) {                                                \
+                                       const T* rhs, O* out) { MXH_API;                                       \
         ew_binary(num_els, num_dims, md, lhs, rhs, out, OP<T>{}, false);                                      \
     }
 #define MXH_INPLACE(NAME, OP, T, SUF)                                                                         \
     extern "C" void hip_##NAME##_inplace_##SUF(size_t num_els, size_t num_dims, const size_t* md, T* lhs,     \
-                                               const T* rhs) {                                                \
+                                               const T* rhs) { MXH_API;                                       \
         ew_binary(num_els, num_dims, md, lhs, rhs, nullptr, OP<T>{}, true);                                   \
     }
 

@@ -12,12 +12,12 @@ static inline float F_host(bf16_t v) { return bf2f(v); }
 static inline float F_host(f16_t v) { return h2f(v); }
 
 #define MXH_UNARY(NAME, OP, T, SUF, O)                                                                        \
-    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, O* out) { \
+    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, O* out) { MXH_API; \
         ew_unary(num_els, num_dims, md, in, out, OP<T>{});                                                    \
     }
 #define MXH_UNARY_C(NAME, OP, T, SUF, O)                                                                      \
     extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, T c,   \
-                                       O* out) {                                                              \
+                                       O* out) { MXH_API;                                                     \
         ew_unary(num_els, num_dims, md, in, out, OP<T>{c});                                                   \
     }
 
@@ -25,7 +25,7 @@ static inline float F_host(f16_t v) { return h2f(v); }
 // once is bit for bit what the double pow() path returns - without the 200 instructions of pow.  x^1 (the factor
 // x^(c-1) in the backward of that square) is x.
 #define MXH_POW(T, SUF)                                                                                       \
-    extern "C" void hip_pow_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, T c, T* out) { \
+    extern "C" void hip_pow_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, T c, T* out) { MXH_API; \
         if (F_host(c) == 2.0f) ew_unary(num_els, num_dims, md, in, out, OpSquare<T>{});                       \
         else if (F_host(c) == 1.0f) ew_unary(num_els, num_dims, md, in, out, OpIdentity<T>{});                \
         else ew_unary(num_els, num_dims, md, in, out, OpPow<T>{c});                                           \

@@ -86,11 +86,11 @@ static void gemm_wide_dispatch(GemmArgs g) {
 using namespace mxh;
 
 #define MXH_MATMUL_WIDE_FOR(T, SUF)                                                                         \
-    extern "C" void hip_matmul_##SUF(size_t num_els, const size_t* md, const T* a, const T* b, T* c) {      \
+    extern "C" void hip_matmul_##SUF(size_t num_els, const size_t* md, const T* a, const T* b, T* c) { MXH_API; \
         matmul_fwd<T>(num_els, md, a, b, c, [](GemmArgs g) { gemm_wide_dispatch<T>(g); });                  \
     }                                                                                                       \
     extern "C" void hip_matmul_backward_##SUF(size_t na, size_t nb, const size_t* md, const T* go,          \
-                                              const T* a, const T* b, T* ga, T* gb) {                       \
+                                              const T* a, const T* b, T* ga, T* gb) { MXH_API;              \
         matmul_bwd<T>(na, nb, md, go, a, b, ga, gb, [](GemmArgs g) { gemm_wide_dispatch<T>(g); });          \
     }
 MXH_MATMUL_WIDE_FOR(double, f64)

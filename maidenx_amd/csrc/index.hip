@@ -319,6 +319,10 @@ void gather(size_t nd, size_t dim, const size_t* in_layout, const size_t* idx_la
     if (!flag) return;
     IdxSpace sp; size_t n; Lay in, ix;
     if (!make_space(nd, idx_layout, dim, -1, sp, &n, "gather: bad shape, rank above 8 or bad dim")) return;
+    // the index tensor has the input's extent in every dim but `dim` (crates/maidenx_tensor/src/ops/indexing.rs:331-340):
+    // a larger one would send the kernel past the end of the input
+    for (size_t d = 0; d < nd; ++d)
+        if (d != dim && idx_layout[d] != in_layout[d]) { set_status(ERR_INVALID, "gather: index and input shapes differ outside dim"); return; }
     read_layout(nd, in_layout, in);
     read_layout(nd, idx_layout, ix);
     if (n == 0) return;
@@ -495,7 +499,7 @@ using namespace mxh;
 
 #define MXH_INDEX_PUT_FOR(T, TS)                                                                                                    \
     extern "C" void hip_index_put_##TS(size_t self_nd, const size_t* self_layout, size_t n_indices, const size_t* indices,          \
-                                       size_t src_nd, const size_t* src_layout, const T* src, T* self) {                            \
+                                       size_t src_nd, const size_t* src_layout, const T* src, T* self) { MXH_API;                   \
         index_put<T>(self_nd, self_layout, n_indices, indices, src_nd, src_layout, src, self);                                      \
     }
 MXH_INDEX_PUT_FOR(float, f32)
@@ -504,24 +508,24 @@ MXH_INDEX_PUT_FOR(f16_t, f16)
 
 #define MXH_INDEX_FOR(T, TS, I, IS)                                                                                                  \
     extern "C" void hip_index_select_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride,    \
-                                                 size_t idx_offset, const I* indices, const T* input, T* output) {                   \
+                                                 size_t idx_offset, const I* indices, const T* input, T* output) { MXH_API;          \
         index_select<T, I>(nd, dim, in_layout, n_idx, idx_stride, idx_offset, indices, input, output);                               \
     }                                                                                                                                \
     extern "C" void hip_gather_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, const size_t* idx_layout, const I* index, \
-                                           const T* input, T* output) {                                                             \
+                                           const T* input, T* output) { MXH_API;                                                    \
         gather<T, I>(nd, dim, in_layout, idx_layout, index, input, output);                                                          \
     }                                                                                                                                \
     extern "C" void hip_index_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* src_layout,            \
                                               size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices, const T* src,   \
-                                              T* self) {                                                                             \
+                                              T* self) { MXH_API;                                                                    \
         index_add<T, I>(nd, dim, self_layout, src_layout, n_idx, idx_stride, idx_offset, indices, src, self);                        \
     }                                                                                                                                \
     extern "C" void hip_scatter_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* idx_layout,          \
-                                                const size_t* src_layout, const I* index, const T* src, T* self) {                  \
+                                                const size_t* src_layout, const I* index, const T* src, T* self) { MXH_API;         \
         scatter_add<T, I>(nd, dim, self_layout, idx_layout, src_layout, index, src, self);                                           \
     }                                                                                                                                \
     extern "C" void hip_bincount_weighted_##TS##_##IS(size_t n, size_t stride, size_t offset, const I* input, size_t w_stride,       \
-                                                      size_t w_offset, const T* weights, size_t out_size, T* output) {              \
+                                                      size_t w_offset, const T* weights, size_t out_size, T* output) { MXH_API;     \
         bincount_weighted<T, I>(n, stride, offset, input, w_stride, w_offset, weights, out_size, output);                            \
     }
 
@@ -532,9 +536,9 @@ MXH_INDEX_FOR(bf16_t, bf16, int64_t, i64)
 MXH_INDEX_FOR(f16_t, f16, int32_t, i32)
 MXH_INDEX_FOR(f16_t, f16, int64_t, i64)
 
-extern "C" void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output) {
+extern "C" void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output) { MXH_API;
     bincount<int32_t>(n, stride, offset, input, out_size, output);
 }
-extern "C" void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output) {
+extern "C" void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output) { MXH_API;
     bincount<int64_t>(n, stride, offset, input, out_size, output);
 }

@@ -24,6 +24,26 @@ constexpr int WAVE = 64;
 
 void set_status(int code, const char* what, int hip_err = 0);
 hipStream_t stream();
+
+// Every extern "C" entry point holds the library's one lock from its first line to its return, so host threads may call
+// in concurrently (the reference's buffers are Send + Sync, crates/maidenx_core/src/buffer/mod.rs:36): calls are
+// serialised, and everything a call queues lands on the stream in one piece.  The lock is recursive (entry points call
+// each other).  While a graph capture is open, the stream, the fusion group and the command list belong to the thread
+// that opened it: a call from another thread is refused (`ok` false, status ERR_INVALID) instead of being recorded into
+// that thread's graph.
+struct ApiGuard {
+    bool ok;
+    ApiGuard();
+    ~ApiGuard();
+    ApiGuard(const ApiGuard&) = delete;
+    ApiGuard& operator=(const ApiGuard&) = delete;
+};
+#define MXH_API                    \
+    ::mxh::ApiGuard api_guard__;   \
+    if (!api_guard__.ok) return
+#define MXH_API_INT                \
+    ::mxh::ApiGuard api_guard__;   \
+    if (!api_guard__.ok) return (int)hipErrorStreamCaptureWrongThread
 // Device scratch owned by the library (two independent slots per device), grown on demand and
 // reused by every call; safe because all work of the backend is ordered on one stream.
 void* scratch(size_t bytes, int slot = 0);

@@ -132,12 +132,12 @@ MXH_WCMP(EqScalar, ==) MXH_WCMP(NeScalar, !=) MXH_WCMP(LtScalar, <) MXH_WCMP(LeS
 
 // P = the pointer / by-value type of the C ABI (uint8_t for bool), T the element type of the kernels
 #define MXH_WU(NAME, OP, T, P, SUF, PO)                                                                        \
-    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const P* in, PO* out) { \
+    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const P* in, PO* out) { MXH_API; \
         using O = typename mxh::OP<T>::Out;                                                                    \
         mxh::ew_unary(num_els, num_dims, md, (const T*)in, (O*)out, mxh::OP<T>{});                             \
     }
 #define MXH_WUC(NAME, OP, T, P, SUF, PO)                                                                       \
-    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const P* in, P c, PO* out) { \
+    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const P* in, P c, PO* out) { MXH_API; \
         using O = typename mxh::OP<T>::Out;                                                                    \
         T ct;                                                                                                  \
         static_assert(sizeof(T) == sizeof(P), "ABI type and element type differ in size");                     \

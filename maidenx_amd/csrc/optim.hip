@@ -66,7 +66,7 @@ using namespace mxh;
 
 #define MXH_ADAM_FOR(T, SUF)                                                                                               \
     extern "C" void hip_adam_step_##SUF(size_t n, T* param, const T* grad, T* m, T* v, T beta1, T one_minus_beta1, T beta2,  \
-                                        T one_minus_beta2, T bias1, T bias2, T epsilon, T lr_t) {                          \
+                                        T one_minus_beta2, T bias1, T bias2, T epsilon, T lr_t) { MXH_API;                 \
         adam_step<T>(n, param, grad, m, v, AdamScalars<T>{beta1, one_minus_beta1, beta2, one_minus_beta2, bias1, bias2, epsilon, lr_t}); \
     }
 MXH_ADAM_FOR(float, f32)

@@ -758,29 +758,29 @@ using namespace mxh;
 
 #define MXH_PAD_FOR(T, SUF)                                                                                  \
     extern "C" void hip_pad_with_constant_##SUF(size_t n_in, size_t n_out, size_t nd, const size_t* md,      \
-                                                const T* in, T* out, T pad_value) {                          \
+                                                const T* in, T* out, T pad_value) { MXH_API;                 \
         pad_forward<T>(n_in, n_out, nd, md, in, out, pad_value);                                             \
     }                                                                                                        \
     extern "C" void hip_pad_with_constant_backward_##SUF(size_t n_in, size_t n_out, size_t nd,               \
-                                                         const size_t* md, const T* go, T* gi) {             \
+                                                         const size_t* md, const T* go, T* gi) { MXH_API;    \
         pad_backward<T>(n_in, n_out, nd, md, go, gi);                                                        \
     }
 
 #define MXH_PAD_EDGE_FOR(T, SUF)                                                                             \
     extern "C" void hip_pad_with_reflection_##SUF(size_t n_in, size_t n_out, size_t nd, const size_t* md,    \
-                                                  const T* in, T* out) {                                     \
+                                                  const T* in, T* out) { MXH_API;                            \
         pad_edge_forward<T>(EDGE_REFLECT, n_in, n_out, nd, md, in, out);                                     \
     }                                                                                                        \
     extern "C" void hip_pad_with_replication_##SUF(size_t n_in, size_t n_out, size_t nd, const size_t* md,   \
-                                                   const T* in, T* out) {                                    \
+                                                   const T* in, T* out) { MXH_API;                           \
         pad_edge_forward<T>(EDGE_REPLICATE, n_in, n_out, nd, md, in, out);                                   \
     }                                                                                                        \
     extern "C" void hip_pad_with_reflection_backward_##SUF(size_t n_in, size_t n_out, size_t nd,             \
-                                                           const size_t* md, const T* go, T* gi) {           \
+                                                           const size_t* md, const T* go, T* gi) { MXH_API;  \
         pad_edge_backward<T>(EDGE_REFLECT, n_in, n_out, nd, md, go, gi);                                     \
     }                                                                                                        \
     extern "C" void hip_pad_with_replication_backward_##SUF(size_t n_in, size_t n_out, size_t nd,            \
-                                                            const size_t* md, const T* go, T* gi) {          \
+                                                            const size_t* md, const T* go, T* gi) { MXH_API; \
         pad_edge_backward<T>(EDGE_REPLICATE, n_in, n_out, nd, md, go, gi);                                   \
     }
 

@@ -669,22 +669,22 @@ void fold(size_t num_els, size_t nd, const size_t* md, const T* in, T* out) {
 using namespace mxh;
 
 #define MXH_REDUCE_FOR(T, SUF)                                                                                  \
-    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
         reduce_axis<T, RSum>(n, nd, nr, md, in, out, false);                                                    \
     }                                                                                                           \
-    extern "C" void hip_mean_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {     \
+    extern "C" void hip_mean_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
         reduce_axis<T, RSum>(n, nd, nr, md, in, out, true);                                                     \
     }                                                                                                           \
-    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
         reduce_axis<T, RMax>(n, nd, nr, md, in, out, false);                                                    \
     }                                                                                                           \
-    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
         reduce_axis<T, RMin>(n, nd, nr, md, in, out, false);                                                    \
     }                                                                                                           \
-    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {        \
+    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API;\
         sum_to_shape<T>(n, nd, md, in, out);                                                                    \
     }                                                                                                           \
-    extern "C" void hip_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {                \
+    extern "C" void hip_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API;       \
         fold<T>(n, nd, md, in, out);                                                                            \
     }
 

@@ -375,16 +375,16 @@ static void wsum_to_shape(size_t num_els, size_t num_dims, const size_t* md, con
 using namespace mxh;
 
 #define MXH_WREDUCE_FOR(T, SUF)                                                                                 \
-    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         wreduce_axis<T, WSum>(n, nd, nr, md, in, out, false);                                                   \
     }                                                                                                           \
-    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         wreduce_axis<T, WMax>(n, nd, nr, md, in, out, false);                                                   \
     }                                                                                                           \
-    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) {      \
+    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         wreduce_axis<T, WMin>(n, nd, nr, md, in, out, false);                                                   \
     }                                                                                                           \
-    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {        \
+    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API; \
         wsum_to_shape<T>(n, nd, md, in, out);                                                                   \
     }
 MXH_WREDUCE_FOR(double, f64)
@@ -396,6 +396,6 @@ MXH_WREDUCE_FOR(int8_t, i8)
 MXH_WREDUCE_FOR(int16_t, i16)
 MXH_WREDUCE_FOR(int32_t, i32)
 MXH_WREDUCE_FOR(int64_t, i64)
-extern "C" void hip_mean_f64(size_t n, size_t nd, size_t nr, const size_t* md, const double* in, double* out) {
+extern "C" void hip_mean_f64(size_t n, size_t nd, size_t nr, const size_t* md, const double* in, double* out) { MXH_API;
     wreduce_axis<double, WSum>(n, nd, nr, md, in, out, true);
 }

@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <thread>
 #include <vector>
 
 #include "fuse.hpp"
@@ -13,6 +14,8 @@ namespace mxh {
 
 static std::mutex g_mu;
 static std::mutex g_scratch_mu;
+static std::recursive_mutex g_api_mu;       // held by every entry point for its whole duration (ApiGuard)
+static std::thread::id g_capture_owner;     // the thread that opened the capture, while g_capturing
 static int g_status = OK;
 static int g_hip_err = 0;
 static char g_what[256] = "ok";
@@ -54,6 +57,15 @@ void set_status(int code, const char* what, int hip_err) {
     else
         snprintf(g_what, sizeof(g_what), "%s", what);
 }
+
+ApiGuard::ApiGuard() : ok(true) {
+    g_api_mu.lock();
+    if (g_capturing && g_capture_owner != std::this_thread::get_id()) {
+        ok = false;
+        set_status(ERR_INVALID, "another host thread has a graph capture open: calls from this thread are refused until it ends");
+    }
+}
+ApiGuard::~ApiGuard() { g_api_mu.unlock(); }
 
 static void fuse_flush() {
     if (g_fuse.n == 0) return;
@@ -202,6 +214,7 @@ void* scratch(size_t bytes, int slot) {
     // grow: work already queued on the stream may still use the old block, so drain first
     if (g_scratch[dev][slot]) {
         (void)hipStreamSynchronize(g_stream);
+        if (g_capture_stream) (void)hipStreamSynchronize(g_capture_stream);     // replays queued there use the block as well
         if (g_scratch_captured[dev][slot] && g_live_captures > 0) g_retired_scratch.push_back(g_scratch[dev][slot]);
         else (void)hipFree(g_scratch[dev][slot]);
         g_scratch_captured[dev][slot] = false;
@@ -263,30 +276,34 @@ using namespace mxh;
 
 extern "C" {
 
-int hip_set_device(int id) { return (int)hipSetDevice(id); }
-int hip_get_device(int* id) { return (int)hipGetDevice(id); }
+int hip_set_device(int id) { MXH_API_INT; return (int)hipSetDevice(id); }
+int hip_get_device(int* id) { MXH_API_INT; return (int)hipGetDevice(id); }
 int hip_device_count(int* n) { return (int)hipGetDeviceCount(n); }
 
 int hip_malloc(void** ptr, size_t bytes) {
+    MXH_API_INT;
     if (!ptr) return (int)hipErrorInvalidValue;
     if (bytes == 0) bytes = 1;
     hipError_t e = hipMalloc(ptr, bytes);
     return e == hipSuccess ? 0 : (e == hipErrorOutOfMemory ? ERR_OOM : (int)e);
 }
-int hip_free(void* ptr) { return (int)hipFree(ptr); }
+int hip_free(void* ptr) { MXH_API_INT; return (int)hipFree(ptr); }
 
 // The copies are ordered after everything queued on the backend's stream and return when done.
 int hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    MXH_API_INT;
     hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream());
     if (e == hipSuccess) e = hipStreamSynchronize(stream());
     return (int)e;
 }
 int hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    MXH_API_INT;
     hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream());
     if (e == hipSuccess) e = hipStreamSynchronize(stream());
     return (int)e;
 }
 int hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    MXH_API_INT;
     prog_launch_seen();
     return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream());
 }
@@ -295,9 +312,16 @@ int hip_stream_create(void** s) { return (int)hipStreamCreateWithFlags((hipStrea
 int hip_stream_destroy(void* s) { return (int)hipStreamDestroy((hipStream_t)s); }
 int hip_stream_synchronize(void* s) { return (int)hipStreamSynchronize((hipStream_t)s); }
 // Stream every later kernel and copy of the backend is queued on (null = default stream).
-int hip_set_stream(void* s) { g_stream = (hipStream_t)s; return 0; }
-void* hip_get_stream(void) { return (void*)g_stream; }
+int hip_set_stream(void* s) {
+    MXH_API_INT;
+    // replays queued on the capture stream were ordered with the old stream only
+    if (g_capture_stream && (hipStream_t)s != g_stream) (void)hipStreamSynchronize(g_capture_stream);
+    g_stream = (hipStream_t)s;
+    return 0;
+}
+void* hip_get_stream(void) { std::lock_guard<std::recursive_mutex> lk(g_api_mu); return (void*)g_stream; }
 int hip_synchronize(void) {
+    MXH_API_INT;
     hipError_t e = hipStreamSynchronize(stream());
     if (e == hipSuccess && g_capture_stream && !g_capturing) e = hipStreamSynchronize(g_capture_stream);   // graph replays
     return (int)e;
@@ -306,12 +330,13 @@ int hip_synchronize(void) {
 // Events on the backend's stream, for timing kernels where they run.
 int hip_event_create(void** ev) { return (int)hipEventCreate((hipEvent_t*)ev); }
 int hip_event_destroy(void* ev) { return (int)hipEventDestroy((hipEvent_t)ev); }
-int hip_event_record(void* ev) { return (int)hipEventRecord((hipEvent_t)ev, stream()); }
+int hip_event_record(void* ev) { MXH_API_INT; return (int)hipEventRecord((hipEvent_t)ev, stream()); }
 int hip_event_synchronize(void* ev) { return (int)hipEventSynchronize((hipEvent_t)ev); }
 int hip_event_elapsed_ms(void* start, void* stop, float* ms) { return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop); }
 
 // First error recorded since the last call (0 = none); reading it clears it.
 int hip_get_last_status(void) {
+    std::lock_guard<std::recursive_mutex> api(g_api_mu);     // not refused during another thread's capture: it queues nothing
     collect_index_flag();
     hipError_t e = hipGetLastError();
     std::lock_guard<std::mutex> lk(g_mu);
@@ -329,6 +354,7 @@ const char* hip_status_string(void) { return g_what; }
 
 
 int hip_graph_begin_capture(void) {
+    MXH_API_INT;
     if (g_capturing) return (int)hipErrorInvalidValue;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
@@ -341,6 +367,7 @@ int hip_graph_begin_capture(void) {
     g_saved_stream = g_stream;
     g_stream = g_capture_stream;
     g_capturing = true;
+    g_capture_owner = std::this_thread::get_id();
     g_prog_ok = g_prog_enabled;
     g_prog_pending = false;
     g_prog_cmds.clear();
@@ -349,6 +376,7 @@ int hip_graph_begin_capture(void) {
     return 0;
 }
 int hip_graph_end_capture(void** graph_exec) {
+    MXH_API_INT;
     if (!g_capturing || !graph_exec) return (int)hipErrorInvalidValue;
     fuse_flush();
     hipGraph_t graph = nullptr;
@@ -391,29 +419,38 @@ int hip_graph_fused_launches(void* graph_exec, int* nodes) {
 }
 // Whether later captures may fuse runs of elementwise launches (default 1); returns the previous setting.
 int hip_graph_set_fusion(int enabled) {
+    std::lock_guard<std::recursive_mutex> api(g_api_mu);
     int was = g_fuse_enabled ? 1 : 0;
     g_fuse_enabled = enabled != 0;
     return was;
 }
 // Whether later captures may become programs (default 1); returns the previous setting.
 int hip_graph_set_programs(int enabled) {
+    std::lock_guard<std::recursive_mutex> api(g_api_mu);
     int was = g_prog_enabled ? 1 : 0;
     g_prog_enabled = enabled != 0;
     return was;
 }
-// Replays run on the capture stream, a blocking stream: work on the default stream orders with it.
+// A replay is ordered with the library's eager work, which shares its tensors and both scratch slots.  With the default
+// (null) stream it runs on the capture stream: that one is a blocking stream, and the null stream orders with blocking
+// streams in both directions.  Once the caller has set a stream of its own (hip_stream_create gives non-blocking
+// ones, which order with nothing) the replay is queued on that stream, behind the eager work and ahead of what follows.
 int hip_graph_launch(void* graph_exec) {
+    MXH_API_INT;
     if (!graph_exec || !g_capture_stream || g_capturing) return (int)hipErrorInvalidValue;
     GraphExec* ge = (GraphExec*)graph_exec;
+    hipStream_t s = g_stream ? g_stream : g_capture_stream;
     if (ge->cmds) {
-        prog_launch(ge->cmds, ge->n, (void*)g_capture_stream);
+        prog_launch(ge->cmds, ge->n, (void*)s);
         return (int)hipGetLastError();
     }
-    return (int)hipGraphLaunch(ge->graph, g_capture_stream);
+    return (int)hipGraphLaunch(ge->graph, s);
 }
 int hip_graph_destroy(void* graph_exec) {
+    MXH_API_INT;
     if (!graph_exec) return 0;
     (void)hipStreamSynchronize(g_capture_stream);
+    if (g_stream) (void)hipStreamSynchronize(g_stream);      // replays run there once the caller has set a stream
     GraphExec* ge = (GraphExec*)graph_exec;
     hipError_t e = hipSuccess;
     if (ge->cmds) e = hipFree(ge->cmds);

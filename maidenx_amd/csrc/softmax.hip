@@ -340,12 +340,12 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
 
 using namespace mxh;
 
-extern "C" void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const float* in, float* out) {
+extern "C" void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const float* in, float* out) { MXH_API;
     softmax<float>(num_els, num_dims, dim, md, in, out);
 }
-extern "C" void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const f16_t* in, f16_t* out) {
+extern "C" void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const f16_t* in, f16_t* out) { MXH_API;
     softmax<f16_t>(num_els, num_dims, dim, md, in, out);
 }
-extern "C" void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const bf16_t* in, bf16_t* out) {
+extern "C" void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* md, const bf16_t* in, bf16_t* out) { MXH_API;
     softmax<bf16_t>(num_els, num_dims, dim, md, in, out);
 }

@@ -37,20 +37,20 @@ using namespace mxh;
 
 #define MXH_UTIL_FOR(T, SUF)                                                                               \
     /* out[0..n) = value */                                                                                \
-    extern "C" void hip_fill_##SUF(size_t n, T* out, T value) {                                            \
+    extern "C" void hip_fill_##SUF(size_t n, T* out, T value) { MXH_API;                                   \
         ew_unary(n, 1, nullptr, nullptr, out, OpFill<T>{value});                                           \
     }                                                                                                      \
     /* contiguous copy of a strided view; metadata as for the unary ops: dims | strides | offset */        \
-    extern "C" void hip_copy_strided_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {   \
+    extern "C" void hip_copy_strided_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API; \
         ew_unary(n, nd, md, in, out, OpIdentity<T>{});                                                     \
     }
 MXH_UTIL_FOR(float, f32)
 MXH_UTIL_FOR(bf16_t, bf16)
 MXH_UTIL_FOR(f16_t, f16)
-extern "C" void hip_fill_bool(size_t n, bool_t* out, bool_t value) { ew_unary(n, 1, nullptr, nullptr, out, OpFill<bool_t>{value}); }
+extern "C" void hip_fill_bool(size_t n, bool_t* out, bool_t value) { MXH_API; ew_unary(n, 1, nullptr, nullptr, out, OpFill<bool_t>{value}); }
 
 #define MXH_CAST(TI, SI, TO, SO)                                                                           \
-    extern "C" void hip_cast_##SI##_##SO(size_t n, const TI* in, TO* out) {                                \
+    extern "C" void hip_cast_##SI##_##SO(size_t n, const TI* in, TO* out) { MXH_API;                       \
         if (!in) { set_status(ERR_INVALID, "cast: null input"); return; }                                  \
         ew_unary(n, 1, nullptr, in, out, OpConvert<TI, TO>{});                                             \
     }

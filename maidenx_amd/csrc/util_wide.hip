@@ -6,10 +6,10 @@
 using namespace mxh;
 
 #define MXH_UTIL_WIDE(T, SUF)                                                                              \
-    extern "C" void hip_fill_##SUF(size_t n, T* out, T value) {                                            \
+    extern "C" void hip_fill_##SUF(size_t n, T* out, T value) { MXH_API;                                   \
         ew_unary(n, 1, nullptr, nullptr, out, OpFill<T>{value});                                           \
     }                                                                                                      \
-    extern "C" void hip_copy_strided_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {   \
+    extern "C" void hip_copy_strided_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API; \
         ew_unary(n, nd, md, in, out, OpIdentity<T>{});                                                     \
     }
 MXH_UTIL_WIDE(double, f64)
@@ -21,6 +21,6 @@ MXH_UTIL_WIDE(int8_t, i8)
 MXH_UTIL_WIDE(int16_t, i16)
 MXH_UTIL_WIDE(int32_t, i32)
 MXH_UTIL_WIDE(int64_t, i64)
-extern "C" void hip_copy_strided_bool(size_t n, size_t nd, const size_t* md, const bool_t* in, bool_t* out) {
+extern "C" void hip_copy_strided_bool(size_t n, size_t nd, const size_t* md, const bool_t* in, bool_t* out) { MXH_API;
     ew_unary(n, nd, md, in, out, OpIdentity<bool_t>{});
 }

@@ -816,6 +816,22 @@ def test_index_out_of_bounds_is_reported(hip):
         hip.call("gather_f32_i32", 1, 0, layout([3]), layout([2]), In(np.array([-4, 0], dtype=np.int32)), In(np.arange(3, dtype=np.float32)), Out(2, "f32"))
 
 
+def test_gather_refuses_an_index_larger_than_the_input_off_dim(hip):
+    """indexing.rs:331-340: the index tensor must have the input's extent in every dim but `dim`.  The host refuses the
+    call before anything is queued, so nothing is launched and the output keeps its poison."""
+    import maidenx_amd.lib as L
+    L.check()
+    x = np.arange(12, dtype=np.float32)
+    index = np.zeros(5 * 2, dtype=np.int32)
+    out = Out(10, "f32")
+    with pytest.raises(L.HipError, match="index and input shapes differ"):
+        hip.call("gather_f32_i32", 2, 1, layout([3, 4]), layout([5, 2]), In(index), In(x), out)
+    assert (out.arr.view(np.uint8) == 0xCD).all()
+    # the same extent off `dim` is accepted, whatever the extent along `dim`
+    (h,) = hip.call("gather_f32_i32", 2, 1, layout([3, 4]), layout([3, 6]), In(np.tile(np.array([3, 0, 1, 2, 3, 0], np.int32), 3)), In(x), Out(18, "f32"))
+    assert h.reshape(3, 6)[1].tolist() == [7.0, 4.0, 5.0, 6.0, 7.0, 4.0]
+
+
 @pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("n", [1, 7, 1000, 4099, 1 << 16])
 def test_fused_adam_step_equals_the_fourteen_ops(oracle, hip, n, dt):
