@@ -385,6 +385,18 @@ MX_DECL_REDUCE(float, f32)
 MX_DECL_REDUCE(mx_bf16, bf16)
 MX_DECL_REDUCE(mx_f16, f16)
 
+/* hip_sum_f32 for callers that cannot allocate.  No counterpart in the reference: it is for code that runs under HIP
+ * graph capture, tight serving loops and harnesses that forbid allocation, where hip_sum_f32's grown-on-demand scratch
+ * (its chunk partials when the reduced axis is cut to fill the chip) is not acceptable.  Same arguments, kernels and
+ * result bits as hip_sum_f32; the partials live in a fixed 4 MiB array inside the library's code object (one copy per
+ * GPU, held until the process ends), so the call performs no hipMalloc / hipFree.  A shape whose partials would not fit
+ * is refused: hip_get_last_status() == 3 (too large) and nothing is queued — [8192,8192] and [64,512,1024] along any
+ * axis fit.  All calls on a GPU share that GPU's array: calls that overlap in time on one GPU race.
+ * hip_noalloc_prepare() resolves the array's device address on the current device ahead of time (optional; the first
+ * hip_sum_f32_noalloc on a device does it otherwise).  Returns 0 on success. */
+void hip_sum_f32_noalloc(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const float* inp, float* out);
+int hip_noalloc_prepare(void);
+
 /* The same for f64 and the integers (crates/maidenx_cuda/src/ops/reduction.rs:59-113; mean for f64 only, as in
  * crates/maidenx_cpu/src/ops/reduction.rs:581-586).  The accumulator is the storage type: integer sums wrap (the
  * reference's release build), so they are bit-exact in any order; f64 sums differ from the sequential order by

@@ -165,6 +165,7 @@ def extension_signatures():
     for a, b in (("bool", "f32"), ("bool", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "bool"), ("bf16", "bool"),
                  ("bool", "f16"), ("f32", "f16"), ("f16", "f32"), ("f16", "bool")):
         sig[f"cast_{a}_{b}"] = [SZ, P, P]
+    sig["sum_f32_noalloc"] = [SZ, SZ, SZ, P, P, P]
     sig.update(cast_signatures())
     sig.update(wide_util_signatures())
     sig.update(wide_unary_signatures())

@@ -15,6 +15,7 @@
 // Accumulation is f32 in a fixed order (deterministic from run to run); bf16 is rounded once.
 // No atomics anywhere.
 #include <cfloat>
+#include <mutex>
 
 #include "elementwise.hpp"
 #include "mxh.hpp"
@@ -24,6 +25,39 @@
 namespace mxh {
 
 constexpr size_t COL_SPLIT_BLOCKS = 256;      // one 16-wave block per CU
+
+// ---- where the chunk partials live ---------------------------------------------------------------------
+// Normally in the library's scratch slot 0, which is allocated and grown on demand.  The entry points that must not
+// allocate (hip_sum_f32_noalloc) keep them in a fixed array that is part of the code object instead: every device the
+// library runs on holds its own copy of it from the first use of the library to the end of the process.
+constexpr size_t FIXED_PARTIALS_BYTES = 4u << 20;
+static __device__ __align__(256) unsigned char g_fixed_partials[FIXED_PARTIALS_BYTES];
+static std::mutex g_fixed_mu;
+static void* g_fixed_ptr[16] = {nullptr};            // device address of the array, per device (the name above is a host-side stand-in)
+static thread_local void* t_fixed = nullptr;         // set while a no-alloc entry point runs on this thread
+
+// Device address of this device's copy of the array; resolved once per device, with that device current.
+static void* fixed_partials() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) { set_status(ERR_INVALID, "no-alloc reduce: bad device"); return nullptr; }
+    std::lock_guard<std::mutex> lk(g_fixed_mu);
+    if (!g_fixed_ptr[dev]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_fixed_partials));
+        if (e != hipSuccess || !p) { set_status(ERR_LAUNCH, "no-alloc reduce: hipGetSymbolAddress", (int)e); return nullptr; }
+        g_fixed_ptr[dev] = p;
+    }
+    return g_fixed_ptr[dev];
+}
+
+static float* partials(size_t bytes) {
+    if (!t_fixed) return (float*)scratch(bytes);
+    if (bytes > FIXED_PARTIALS_BYTES) {
+        set_status(ERR_TOO_LARGE, "no-alloc reduce: the chunk partials of this shape exceed the fixed 4 MiB array; use the allocating entry point");
+        return nullptr;
+    }
+    return (float*)t_fixed;
+}
 
 // ---- column reduce: [outer, L, S] → [outer, chunks, S] ------------------------------------------
 template <class TIn, class TOut, class R, int VEC>
@@ -265,7 +299,7 @@ void row_reduce(const TIn* in, TOut* out, size_t rows, size_t L, float div, bool
         chunks = (unsigned)((L + chunk_len - 1) / chunk_len);
     }
     if (chunks == 1) { row_stage<TIn, TOut, R>(in, out, rows, L, 1, L, div, src_bf16); return; }
-    float* part = (float*)scratch(rows * chunks * sizeof(float) + 256);
+    float* part = partials(rows * chunks * sizeof(float) + 256);
     if (!part) return;
     row_stage<TIn, float, R>(in, part, rows, L, chunks, chunk_len, 0.0f, src_bf16);
     row_stage<float, TOut, R>(part, out, rows, chunks, 1, chunks, div, src_bf16);
@@ -354,7 +388,7 @@ void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, floa
             if (chunks == 1) {
                 if (col_split_stage<TIn, TOut, R>(in, out, outer, L, S, 1, L, div, src_bf16)) return;
             } else {
-                float* part = (float*)scratch((outer * chunks * S + outer * 8 * S) * sizeof(float) + 1024);
+                float* part = partials((outer * chunks * S + outer * 8 * S) * sizeof(float) + 1024);
                 if (!part) return;
                 if (col_split_stage<TIn, float, R>(in, part, outer, L, S, chunks, chunk_len, 0.0f, src_bf16)) {
                     fold_partials<TOut, R>(part, out, outer, chunks, S, div, src_bf16);
@@ -375,7 +409,7 @@ void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, floa
         chunks = (unsigned)((L + chunk_len - 1) / chunk_len);
     }
     if (chunks == 1) { col_stage<TIn, TOut, R>(in, out, outer, L, S, 1, L, div, src_bf16); return; }
-    float* part = (float*)scratch((outer * chunks * S + outer * 8 * S) * sizeof(float) + 1024);
+    float* part = partials((outer * chunks * S + outer * 8 * S) * sizeof(float) + 1024);
     if (!part) return;
     col_stage<TIn, float, R>(in, part, outer, L, S, chunks, chunk_len, 0.0f, src_bf16);
     fold_partials<TOut, R>(part, out, outer, chunks, S, div, src_bf16);
@@ -401,7 +435,7 @@ bool plane_reduce(const T* in, T* out, size_t A, size_t K, size_t S) {
         MXH_LAUNCH_CHECK("plane_reduce");
         return true;
     }
-    float* part = (float*)scratch(((size_t)chunks * K + 8 * K) * sizeof(float) + 1024);
+    float* part = partials(((size_t)chunks * K + 8 * K) * sizeof(float) + 1024);
     if (!part) return true;      // status is set
     hipLaunchKernelGGL((plane_reduce_kernel<T, float, RSum, VEC>), dim3((unsigned)(K * chunks)), dim3(PLB), 0, stream(), in, part,
                        (uint32_t)A, (uint32_t)K, (uint32_t)S, a_chunk, dsv, bf);
@@ -669,19 +703,19 @@ void fold(size_t num_els, size_t nd, const size_t* md, const T* in, T* out) {
 using namespace mxh;
 
 #define MXH_REDUCE_FOR(T, SUF)                                                                                  \
-    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
+    extern "C" void hip_sum_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         reduce_axis<T, RSum>(n, nd, nr, md, in, out, false);                                                    \
     }                                                                                                           \
-    extern "C" void hip_mean_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
+    extern "C" void hip_mean_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         reduce_axis<T, RSum>(n, nd, nr, md, in, out, true);                                                     \
     }                                                                                                           \
-    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
+    extern "C" void hip_max_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         reduce_axis<T, RMax>(n, nd, nr, md, in, out, false);                                                    \
     }                                                                                                           \
-    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API;\
+    extern "C" void hip_min_##SUF(size_t n, size_t nd, size_t nr, const size_t* md, const T* in, T* out) { MXH_API; \
         reduce_axis<T, RMin>(n, nd, nr, md, in, out, false);                                                    \
     }                                                                                                           \
-    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API;\
+    extern "C" void hip_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API; \
         sum_to_shape<T>(n, nd, md, in, out);                                                                    \
     }                                                                                                           \
     extern "C" void hip_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API;       \
@@ -691,3 +725,19 @@ using namespace mxh;
 MXH_REDUCE_FOR(float, f32)
 MXH_REDUCE_FOR(bf16_t, bf16)
 MXH_REDUCE_FOR(f16_t, f16)
+
+// hip_sum_f32 for callers that cannot allocate (under graph capture, in a serving loop, in a harness that forbids it):
+// same arguments, same kernels, same bits, but the chunk partials go to the fixed array above instead of the library's
+// grown-on-demand scratch, so the call performs no hipMalloc / hipFree whatever ran before it.  A shape whose partials
+// exceed the array is refused (status ERR_TOO_LARGE) and nothing is queued.  Every partial a launch reads was written
+// by the launch before it, so nothing needs clearing between calls; all calls on a device share that device's array,
+// so calls that overlap on one device (two streams, two threads that switch streams) race.
+extern "C" void hip_sum_f32_noalloc(size_t n, size_t nd, size_t nr, const size_t* md, const float* in, float* out) { MXH_API;
+    void* p = fixed_partials();
+    if (!p) return;
+    t_fixed = p;
+    reduce_axis<float, RSum>(n, nd, nr, md, in, out, false);
+    t_fixed = nullptr;
+}
+// Resolves the array's address on the current device ahead of time (optional: the first hip_sum_f32_noalloc does it too).
+extern "C" int hip_noalloc_prepare(void) { MXH_API_INT; return fixed_partials() ? 0 : (int)hipErrorInvalidSymbol; }
