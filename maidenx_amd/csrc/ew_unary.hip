@@ -3,6 +3,7 @@
 // crates/maidenx_cuda/src/ops/unary.rs:21-77; a null input means "in place on the output"
 // (crates/maidenx_cuda/kernels/ops/unary.cu:20).
 #include "elementwise.hpp"
+#include "lut16.hpp"
 #include "ops.hpp"
 
 using namespace mxh;
@@ -13,6 +14,17 @@ static inline float F_host(f16_t v) { return h2f(v); }
 
 #define MXH_UNARY(NAME, OP, T, SUF, O)                                                                        \
     extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, O* out) { MXH_API; \
+        ew_unary(num_els, num_dims, md, in, out, OP<T>{});                                                    \
+    }
+// The long-running functions: for the 16-bit dtypes a large call is a table lookup (lut16.hpp), f32 always computes.
+template <class Op>
+static inline bool by_table(size_t num_els, size_t num_dims, const size_t* md, const void* in, void* out) {
+    if constexpr (sizeof(typename Op::In) == 2) return lut16_unary<Op>(num_els, num_dims, md, in, out);
+    else return false;
+}
+#define MXH_UNARY_L(NAME, OP, T, SUF, O)                                                                      \
+    extern "C" void hip_##NAME##_##SUF(size_t num_els, size_t num_dims, const size_t* md, const T* in, O* out) { MXH_API; \
+        if (by_table<OP<T>>(num_els, num_dims, md, in, out)) return;                                          \
         ew_unary(num_els, num_dims, md, in, out, OP<T>{});                                                    \
     }
 #define MXH_UNARY_C(NAME, OP, T, SUF, O)                                                                      \
@@ -34,12 +46,12 @@ static inline float F_host(f16_t v) { return h2f(v); }
 #define MXH_ALL_FOR(T, SUF)                                                                                   \
     MXH_UNARY(neg, OpNeg, T, SUF, T) MXH_UNARY(abs, OpAbs, T, SUF, T) MXH_UNARY(sign, OpSign, T, SUF, T)      \
     MXH_UNARY(square, OpSquare, T, SUF, T) MXH_UNARY(sqrt, OpSqrt, T, SUF, T)                                 \
-    MXH_UNARY(relu, OpRelu, T, SUF, T) MXH_UNARY(sigmoid, OpSigmoid, T, SUF, T)                               \
-    MXH_UNARY(tanh, OpTanh, T, SUF, T) MXH_UNARY(gelu, OpGelu, T, SUF, T)                                     \
-    MXH_UNARY(sin, OpSin, T, SUF, T) MXH_UNARY(cos, OpCos, T, SUF, T) MXH_UNARY(tan, OpTan, T, SUF, T)        \
-    MXH_UNARY(ln, OpLn, T, SUF, T) MXH_UNARY(log10, OpLog10, T, SUF, T) MXH_UNARY(log2, OpLog2, T, SUF, T)    \
-    MXH_UNARY(exp, OpExp, T, SUF, T) MXH_UNARY(exp10, OpExp10, T, SUF, T) MXH_UNARY(exp2, OpExp2, T, SUF, T)  \
-    MXH_UNARY(softplus, OpSoftplus, T, SUF, T) MXH_UNARY(recip, OpRecip, T, SUF, T)                           \
+    MXH_UNARY(relu, OpRelu, T, SUF, T) MXH_UNARY_L(sigmoid, OpSigmoid, T, SUF, T)                             \
+    MXH_UNARY_L(tanh, OpTanh, T, SUF, T) MXH_UNARY_L(gelu, OpGelu, T, SUF, T)                                 \
+    MXH_UNARY_L(sin, OpSin, T, SUF, T) MXH_UNARY_L(cos, OpCos, T, SUF, T) MXH_UNARY_L(tan, OpTan, T, SUF, T)  \
+    MXH_UNARY_L(ln, OpLn, T, SUF, T) MXH_UNARY_L(log10, OpLog10, T, SUF, T) MXH_UNARY_L(log2, OpLog2, T, SUF, T) \
+    MXH_UNARY_L(exp, OpExp, T, SUF, T) MXH_UNARY_L(exp10, OpExp10, T, SUF, T) MXH_UNARY_L(exp2, OpExp2, T, SUF, T) \
+    MXH_UNARY_L(softplus, OpSoftplus, T, SUF, T) MXH_UNARY(recip, OpRecip, T, SUF, T)                         \
     MXH_UNARY(logical_not, OpLogicalNot, T, SUF, bool_t)                                                      \
     MXH_UNARY_C(add_scalar, OpAddScalar, T, SUF, T) MXH_UNARY_C(sub_scalar, OpSubScalar, T, SUF, T)           \
     MXH_UNARY_C(mul_scalar, OpMulScalar, T, SUF, T) MXH_UNARY_C(div_scalar, OpDivScalar, T, SUF, T)           \

@@ -60,7 +60,7 @@ static float* partials(size_t bytes) {
 }
 
 // ---- column reduce: [outer, L, S] → [outer, chunks, S] ------------------------------------------
-template <class TIn, class TOut, class R, int VEC>
+template <class TIn, class TOut, class R, int VEC, bool STREAM = false>
 __global__ __launch_bounds__(RB) void col_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t outer,
                                                         size_t L, size_t S, unsigned chunks, size_t chunk_len,
                                                         FastDiv div_sv, FastDiv div_chunks, size_t total, float div,
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(RB) void col_reduce_kernel(const TIn* __restrict__ 
     for (int e = 0; e < VEC; ++e) a[e] = R::init(src_bf16);
 #pragma unroll 8
     for (size_t l = beg; l < end; ++l, src += S) {
-        AVec<TIn, VEC> v = *(const AVec<TIn, VEC>*)src;
+        AVec<TIn, VEC> v = ld_vec<STREAM>((const AVec<TIn, VEC>*)src);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v.v[e]));
     }
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(RB) void col_reduce_kernel(const TIn* __restrict__ 
 // the same 64 column vectors, COL_U loads in flight per lane, and the NW partial rows meet in LDS in wave
 // order.  Against one thread per column this multiplies the loads in flight without more partials to
 // write and fold.  Requires S % VEC == 0 and aligned bases.
-template <class TIn, class TOut, class R, int VEC, int NW>
+template <class TIn, class TOut, class R, int VEC, int NW, bool STREAM = false>
 __global__ __launch_bounds__(WAVE * NW) void col_reduce_split_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t L,
                                                                       size_t S, uint32_t sv, unsigned chunks, size_t chunk_len,
                                                                       FastDiv div_jb, FastDiv div_chunks, float div, bool src_bf16) {
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(WAVE * NW) void col_reduce_split_kernel(const TIn* 
         for (; l + U <= l1; l += U, src += U * S) {
             AVec<TIn, VEC> v[U];
 #pragma unroll
-            for (int k = 0; k < U; ++k) v[k] = *(const AVec<TIn, VEC>*)(src + k * S);
+            for (int k = 0; k < U; ++k) v[k] = ld_vec<STREAM>((const AVec<TIn, VEC>*)(src + k * S));
 #pragma unroll
             for (int k = 0; k < U; ++k)
 #pragma unroll
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(WAVE * NW) void col_reduce_split_kernel(const TIn* 
 // threads sweep the runs as 16-byte vectors, four loads in flight each, then meet in a DPP
 // butterfly and LDS.  S % VEC == 0 and a 16-byte aligned base are required.
 constexpr int PLB = 1024;
-template <class TIn, class TOut, class R, int VEC>
+template <class TIn, class TOut, class R, int VEC, bool STREAM = false>
 __global__ __launch_bounds__(PLB) void plane_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, uint32_t A,
                                                            uint32_t K, uint32_t S, uint32_t a_chunk, FastDiv div_sv,
                                                            bool src_bf16) {
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(PLB) void plane_reduce_kernel(const TIn* __restrict
     for (; f + 3 * PLB < nvec; f += 4 * PLB) {
         AVec<TIn, VEC> v[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = *(const AVec<TIn, VEC>*)addr(f + q * PLB);
+        for (int q = 0; q < 4; ++q) v[q] = ld_vec<STREAM>((const AVec<TIn, VEC>*)addr(f + q * PLB));
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -235,6 +235,10 @@ constexpr size_t COL_MIN_ROWS = 128;
 
 template <class T> inline bool aligned16(const T* p) { return ((uintptr_t)p & 15u) == 0; }
 
+// An input of this many bytes is read once and cannot be in any cache when it is next needed: its loads then carry the
+// non-temporal hint (a read-only sweep of 268 MB: 44 -> 40 us).  Same threshold as the elementwise kernels.
+inline bool streams(size_t input_bytes) { return ew_stream_bytes() != 0 && input_bytes >= ew_stream_bytes() / 2; }
+
 template <class TIn, class TOut, class R, int TPR>
 void launch_row(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks, size_t chunk_len, float div,
                 bool src_bf16) {
@@ -250,7 +254,10 @@ void launch_row(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks
             prog_record(prog_kid(PF_ROW_REDUCE, row_prog_sub<R, TPR>(vec ? 1 : 0)), blocks, &a, sizeof(a));
         }
     }
-    if (vec)
+    if (vec && streams(rows * L * sizeof(TIn)))
+        hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, TPR, VEC, true>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows,
+                           L, chunks, chunk_len, div, src_bf16);
+    else if (vec)
         hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, TPR, VEC>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows,
                            L, chunks, chunk_len, div, src_bf16);
     else
@@ -327,7 +334,10 @@ void col_stage(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, unsig
             return;
         }
     }
-    if (vec)
+    if (vec && streams(outer * L * S * sizeof(TIn)))
+        hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, R, VEC, true>), dim3(blocks), dim3(RB), 0, stream(), in, out, outer, L, S,
+                           chunks, chunk_len, dsv, dch, total, div, src_bf16);
+    else if (vec)
         hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, R, VEC>), dim3(blocks), dim3(RB), 0, stream(), in, out, outer, L, S,
                            chunks, chunk_len, dsv, dch, total, div, src_bf16);
     else
@@ -364,8 +374,12 @@ bool col_split_stage(const TIn* in, TOut* out, size_t outer, size_t L, size_t S,
     size_t sv = S / VEC, jblocks = cdiv(sv, (size_t)WAVE);
     size_t blocks = outer * chunks * jblocks;
     if (blocks >= (1ull << 31) || sv >= (1ull << 31)) return false;
-    hipLaunchKernelGGL((col_reduce_split_kernel<TIn, TOut, R, VEC, NW>), dim3((unsigned)blocks), dim3(WAVE * NW), 0, stream(), in, out,
-                       L, S, (uint32_t)sv, chunks, chunk_len, make_fastdiv((uint32_t)jblocks), make_fastdiv(chunks), div, src_bf16);
+    if (streams(outer * L * S * sizeof(TIn)))
+        hipLaunchKernelGGL((col_reduce_split_kernel<TIn, TOut, R, VEC, NW, true>), dim3((unsigned)blocks), dim3(WAVE * NW), 0, stream(), in, out,
+                           L, S, (uint32_t)sv, chunks, chunk_len, make_fastdiv((uint32_t)jblocks), make_fastdiv(chunks), div, src_bf16);
+    else
+        hipLaunchKernelGGL((col_reduce_split_kernel<TIn, TOut, R, VEC, NW>), dim3((unsigned)blocks), dim3(WAVE * NW), 0, stream(), in, out,
+                           L, S, (uint32_t)sv, chunks, chunk_len, make_fastdiv((uint32_t)jblocks), make_fastdiv(chunks), div, src_bf16);
     MXH_LAUNCH_CHECK("col_reduce_split");
     return true;
 }
@@ -430,14 +444,14 @@ bool plane_reduce(const T* in, T* out, size_t A, size_t K, size_t S) {
     FastDiv dsv = make_fastdiv((uint32_t)(S / VEC));
     const bool bf = IO<T>::is_bf16;
     if (chunks == 1) {
-        hipLaunchKernelGGL((plane_reduce_kernel<T, T, RSum, VEC>), dim3((unsigned)K), dim3(PLB), 0, stream(), in, out, (uint32_t)A,
+        hipLaunchKernelGGL((plane_reduce_kernel<T, T, RSum, VEC, true>), dim3((unsigned)K), dim3(PLB), 0, stream(), in, out, (uint32_t)A,
                            (uint32_t)K, (uint32_t)S, a_chunk, dsv, bf);
         MXH_LAUNCH_CHECK("plane_reduce");
         return true;
     }
     float* part = partials(((size_t)chunks * K + 8 * K) * sizeof(float) + 1024);
     if (!part) return true;      // status is set
-    hipLaunchKernelGGL((plane_reduce_kernel<T, float, RSum, VEC>), dim3((unsigned)(K * chunks)), dim3(PLB), 0, stream(), in, part,
+    hipLaunchKernelGGL((plane_reduce_kernel<T, float, RSum, VEC, true>), dim3((unsigned)(K * chunks)), dim3(PLB), 0, stream(), in, part,
                        (uint32_t)A, (uint32_t)K, (uint32_t)S, a_chunk, dsv, bf);
     MXH_LAUNCH_CHECK("plane_reduce");
     fold_partials<T, RSum>(part, out, 1, chunks, K, 0.0f, bf);

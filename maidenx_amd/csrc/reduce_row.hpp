@@ -77,7 +77,7 @@ constexpr int RB = 256;
 // and a 16-byte aligned base.
 // Block and thread index are arguments (the interpreter of recorded programs passes virtual ones); `part`
 // is RB / WAVE floats of LDS owned by this (virtual) block.  Every thread reaches the barrier.
-template <class TIn, class TOut, class R, int TPR, int VEC>
+template <class TIn, class TOut, class R, int TPR, int VEC, bool STREAM = false>
 __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut* __restrict__ out, size_t rows, size_t L,
                                                 unsigned chunks, size_t chunk_len, float div, bool src_bf16, unsigned bid,
                                                 unsigned tid, float* part) {
@@ -100,7 +100,7 @@ __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut
             for (; i + 3 * STEP < end; i += 4 * STEP) {
                 AVec<TIn, VEC> v[4];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) v[k] = *(const AVec<TIn, VEC>*)(src + i + k * STEP);
+                for (int k = 0; k < 4; ++k) v[k] = ld_vec<STREAM>((const AVec<TIn, VEC>*)(src + i + k * STEP));
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -127,12 +127,12 @@ __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut
     }
     if (t == 0 && unit < total) out[unit] = IO<TOut>::fin(acc, div);
 }
-template <class TIn, class TOut, class R, int TPR, int VEC>
+template <class TIn, class TOut, class R, int TPR, int VEC, bool STREAM = false>
 __global__ __launch_bounds__(RB) void row_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t rows,
                                                         size_t L, unsigned chunks, size_t chunk_len, float div,
                                                         bool src_bf16) {
     __shared__ float part[RB / WAVE];
-    row_reduce_body<TIn, TOut, R, TPR, VEC>(in, out, rows, L, chunks, chunk_len, div, src_bf16, blockIdx.x, threadIdx.x, part);
+    row_reduce_body<TIn, TOut, R, TPR, VEC, STREAM>(in, out, rows, L, chunks, chunk_len, div, src_bf16, blockIdx.x, threadIdx.x, part);
 }
 // Argument block of one recorded row_reduce launch; instantiation number of (reducer, threads per row, vector form).
 struct RowProgArgs {

@@ -178,6 +178,7 @@ bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool ve
     return true;
 }
 
+bool capture_open() { return g_capturing; }
 bool prog_recording() { return g_capturing && g_prog_ok; }
 void prog_record(uint32_t kid, unsigned grid, const void* args, size_t bytes) {
     if (!prog_recording()) return;

@@ -243,6 +243,38 @@ def test_unary_transcendental_16bit(oracle, hip, op, dt):
     assert np.array_equal(o[ok], h[ok])
 
 
+TABLE_OPS = ["sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln", "log10", "log2", "exp", "exp10", "exp2", "softplus"]
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("op", TABLE_OPS)
+def test_large_16bit_unary_calls_go_through_the_table_and_keep_the_bits(oracle, hip, op, dt):
+    """A call of 2^20 elements or more on a 16-bit dtype is a table lookup (the table is the op's own kernel run over all
+    65536 codes).  Every code, in a shuffled 1.1 M-element input with a ragged tail, must give the bits of the small call
+    that computes - contiguous, in place, at an element offset that breaks the 16-byte alignment, and through a
+    transposed view - and for the functions the oracle restates bit for bit, the oracle's bits."""
+    codes = np.arange(1 << 16, dtype=np.uint16)
+    (small,) = hip.call(f"{op}_{dt}", codes.size, 1, meta_unary([codes.size], [1]), In(codes), Out(codes.size, dt))
+    n = (1 << 20) + (1 << 16) + 5
+    x = np.tile(codes, 18)[:n].copy()
+    rng(29).shuffle(x)
+    want = small[x]
+    (h,) = hip.call(f"{op}_{dt}", n, 1, meta_unary([n], [1]), In(x), Out(n, dt))
+    assert np.array_equal(h, want)
+    (hi,) = hip.call(f"{op}_{dt}", n, 1, meta_unary([n], [1]), None, InOut(x.copy()))            # null input: in place
+    assert np.array_equal(hi, want)
+    (ho,) = hip.call(f"{op}_{dt}", n - 3, 1, meta_unary([n - 3], [1], 3), In(x), Out(n - 3, dt))    # odd offset: misaligned
+    assert np.array_equal(ho, want[3:])
+    rows, cols = 1040, 1024                                                                       # [1040,1024] view of a [1024,1040] buffer
+    (ht,) = hip.call(f"{op}_{dt}", rows * cols, 2, meta_unary([rows, cols], [1, rows]), In(x[: rows * cols]), Out(rows * cols, dt))
+    assert np.array_equal(ht.reshape(rows, cols), want[: rows * cols].reshape(cols, rows).T)
+    if op in ("exp", "tanh", "gelu", "sigmoid"):
+        (o,) = oracle.call(f"{op}_{dt}", n, 1, meta_unary([n], [1]), In(x), Out(n, dt))
+        ok = ~np.isnan(to_float(o, dt))
+        assert np.array_equal(np.isnan(to_float(o, dt)), np.isnan(to_float(h, dt)))
+        assert np.array_equal(o[ok], h[ok])
+
+
 # ---------------------------------------------------------------------------------------------------
 # reductions
 # ---------------------------------------------------------------------------------------------------
