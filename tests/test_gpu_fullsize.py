@@ -238,3 +238,130 @@ def test_fused_adam_16m_elements_bit_exact(hip):
         p = p - ((m / sc[4]) / (np.sqrt(v / sc[5]) + sc[6])) * sc[7]
         hp, hm, hv = hip.call("adam_step_f32", n, InOut(hp), In(g), InOut(hm), InOut(hv), *[float(c) for c in sc])
         assert same_bits(hm, m) and same_bits(hv, v) and same_bits(hp, p), t
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_matmul_batched_config_forward_and_backward(hip, dt):
+    """[32,512,1024] x [32,1024,1024]: forward, dA = dC.B^T and dB = A^T.dC of sampled batches against float64, and
+    checksums over every batch (so that no batch or tile is skipped)."""
+    Bt, M, K, N = 32, 512, 1024, 1024
+    r = np.random.default_rng(0x5EED0014)
+    a = r.standard_normal((Bt, M, K), dtype=np.float32)
+    b = r.standard_normal((Bt, K, N), dtype=np.float32) * np.float32(0.02)
+    go = r.standard_normal((Bt, M, N), dtype=np.float32)
+    st = (lambda v: f32_to_bf16(v.ravel())) if dt == "bf16" else (lambda v: v.ravel())
+    val = lambda s, shape: to_float(s, dt).astype(np.float64).reshape(shape)
+    sa, sb, sg = st(a), st(b), st(go)
+    av, bv, gv = val(sa, a.shape), val(sb, b.shape), val(sg, go.shape)
+    md = meta_matmul([Bt, M, N], [Bt, M, K], [Bt, K, N], [M * K, K, 1], [K * N, N, 1])
+    tol = 1e-5 if dt == "f32" else 1e-2
+    (c,) = hip.call(f"matmul_{dt}", Bt * M * N, md, In(sa), In(sb), Out(Bt * M * N, dt))
+    ga, gb = hip.call(f"matmul_backward_{dt}", Bt * M * K, Bt * K * N, md, In(sg), In(sa), In(sb), Out(Bt * M * K, dt), Out(Bt * K * N, dt))
+    cv, gav, gbv = val(c, go.shape), val(ga, a.shape), val(gb, b.shape)
+    for bi in (0, 7, 18, 31):
+        assert np.max(np.abs(cv[bi] - av[bi] @ bv[bi]) / (np.abs(av[bi]) @ np.abs(bv[bi]))) <= tol, ("fwd", bi)
+        assert np.max(np.abs(gav[bi] - gv[bi] @ bv[bi].T) / (np.abs(gv[bi]) @ np.abs(bv[bi].T))) <= tol, ("dA", bi)
+        assert np.max(np.abs(gbv[bi] - av[bi].T @ gv[bi]) / (np.abs(av[bi].T) @ np.abs(gv[bi]))) <= tol, ("dB", bi)
+    # row sums of every batch: C 1 = A (B 1), dA 1 = dC (B^T 1), dB 1 = A^T (dC 1)
+    ones_n, ones_k = np.ones(N), np.ones(K)
+    assert np.max(np.abs(cv @ ones_n - np.einsum("bmk,bk->bm", av, bv @ ones_n)) / np.einsum("bmk,bk->bm", np.abs(av), np.abs(bv) @ ones_n)) <= tol
+    assert np.max(np.abs(gav @ ones_k - np.einsum("bmn,bn->bm", gv, np.einsum("bkn->bn", bv))) / np.einsum("bmn,bn->bm", np.abs(gv), np.einsum("bkn->bn", np.abs(bv)))) <= tol
+    assert np.max(np.abs(gbv @ ones_n - np.einsum("bmk,bm->bk", av, gv @ ones_n)) / np.einsum("bmk,bm->bk", np.abs(av), np.abs(gv) @ ones_n)) <= tol
+
+
+@pytest.mark.parametrize("case", ["rhs_row", "lhs_transposed"])
+def test_elementwise_8192_bf16_broadcast_and_transposed(hip, xy, case):
+    """bf16 add / div bit for bit against the f32-operation-then-round model, exp / gelu against the library's own results
+    on the 65536 codes (which test_unary_transcendental_16bit pins to the oracle), on a [1,8192] rhs and a transposed lhs."""
+    x, y = xy
+    xb, yb = f32_to_bf16(x.ravel()), f32_to_bf16(y.ravel())
+    xf, yf = to_float(xb, "bf16").reshape(R, C), to_float(yb, "bf16").reshape(R, C)
+    n = R * C
+    if case == "rhs_row":
+        md, rhs, a, b = meta_binary([R, C], [C, 1], [0, 1]), yb[:C], xf, yf[:1]
+        mdu, au = meta_unary([R, C], [C, 1]), xb.reshape(R, C)
+    else:
+        md, rhs, a, b = meta_binary([R, C], [1, R], [C, 1]), yb, xf.T, yf
+        mdu, au = meta_unary([R, C], [1, R]), xb.reshape(C, R).T
+    (out,) = hip.call("add_bf16", n, 2, md, In(xb), In(rhs), Out(n, "bf16"))
+    assert same_bits(out.reshape(R, C), f32_to_bf16(a + b).reshape(R, C))
+    (out,) = hip.call("div_bf16", n, 2, md, In(xb), In(rhs), Out(n, "bf16"))
+    with np.errstate(all="ignore"):
+        want = np.divide(a, b)
+    zero = np.broadcast_to(b == 0, want.shape)
+    want = np.where(zero, np.where(a == 0, np.float32(0), np.float32(np.inf)), want).astype(np.float32)
+    assert same_bits(out.reshape(R, C), f32_to_bf16(want).reshape(R, C))
+    codes = np.arange(1 << 16, dtype=np.uint16)
+    for op in ("exp", "gelu"):
+        (small,) = hip.call(f"{op}_bf16", codes.size, 1, meta_unary([codes.size], [1]), In(codes), Out(codes.size, "bf16"))
+        (out,) = hip.call(f"{op}_bf16", n, 2, mdu, In(xb), Out(n, "bf16"))
+        assert same_bits(out.reshape(R, C), small[au]), op
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_broadcast_gradient_chain_8192(hip, xy, dt):
+    """The backward of a [8192,8192] op [1,8192] pair at full size: sum_to_shape -> [1,8192] against float64, and the
+    transposed-back add_inplace (the accumulate of a transposed view's gradient into its base) bit for bit."""
+    x, y = xy
+    st = (lambda v: f32_to_bf16(v.ravel())) if dt == "bf16" else (lambda v: np.ascontiguousarray(v.ravel()))
+    sx, sy = st(x), st(y)
+    xv, yv = to_float(sx, dt).reshape(R, C), to_float(sy, dt).reshape(R, C)
+    n = R * C
+    (s,) = hip.call(f"sum_to_shape_{dt}", n, 2, meta_sum_to_shape([R, C], [C, 1], [1, C]), In(sx), Out(C, dt))
+    x64 = xv.astype(np.float64)
+    tol = 1e-5 if dt == "f32" else 1e-2
+    assert np.max(np.abs(to_float(s, dt) - x64.sum(0)) / np.abs(x64).sum(0)) <= tol
+    # base[C,R] += g[R,C]^T : lhs contiguous [C,R], rhs strides [1,R]... the rhs is g viewed transposed
+    from helpers import InOut
+    (acc,) = hip.call(f"add_inplace_{dt}", n, 2, meta_binary([C, R], [R, 1], [1, C]), InOut(sy.copy()), In(sx))
+    want = yv.reshape(C, R) + xv.T
+    want = f32_to_bf16(want.ravel()) if dt == "bf16" else want.ravel()
+    assert same_bits(acc, want)
+
+
+def test_conv2d_layer_step_config_size(mx_hip):
+    """One full Conv2d(64->64, 3x3, stride 1, pad 1, bias) + MSE step on [32,64,56,56] through the host layer against the
+    float64 restatement of the layer's data flow (host_programs.conv_numpy): output, loss and the three gradients."""
+    from host_programs import conv_inputs, conv_numpy, conv_step
+    x, w, b = conv_inputs(32, 64, 56, 56, 64, 3, seed=0x5EED0005)
+    target = np.random.default_rng(0x5EED0015).standard_normal((32, 64, 56, 56)).astype(np.float32)
+    got = conv_step(mx_hip, x, w, b, 1, 1, target)
+    num = conv_numpy(x, w, b, 1, 1, target)
+    for key, tol in (("out", 1e-5), ("loss", 1e-5), ("grad_b", 2e-5), ("grad_w", 1e-4), ("grad_x", 2e-5)):
+        scale = np.abs(num[key]).max() + 1e-30
+        assert np.abs(got[key] - num[key]).max() <= tol * scale, key
+    # the reference's truncation (col2im is handed num_els = B*C*H*W): only the first 227 planes and 5/9 of plane 227 get a gradient
+    gx = got["grad_x"].reshape(32 * 64, 56 * 56)
+    assert np.abs(gx[:227]).max() > 0 and not gx[228:].any()
+
+
+def test_bf16_accumulation_gpu_is_closer_to_exact_than_the_reference(hip, oracle):
+    """4096-term bf16 dot products and sums: the reference accumulates in bf16 (crates/maidenx_cpu/src/ops/matmul.rs:74-86,
+    reduction.rs:58), the GPU in f32 with one rounding.  Both are measured against float64, normalised by the sum of
+    |terms|; the GPU must be within the bf16 tolerance and no further from exact than the reference's own arithmetic, and
+    the GPU-to-reference distance is bounded by the sum of the two."""
+    r = np.random.default_rng(0x5EED0044)
+    M = N = 64
+    K = 4096
+    a16 = f32_to_bf16(r.standard_normal((M, K), dtype=np.float32).ravel())
+    b16 = f32_to_bf16((r.standard_normal((K, N), dtype=np.float32) * np.float32(0.02)).ravel())
+    av, bv = to_float(a16, "bf16").astype(np.float64).reshape(M, K), to_float(b16, "bf16").astype(np.float64).reshape(K, N)
+    md = meta_matmul([M, N], [M, K], [K, N], [K, 1], [N, 1])
+    oracle.set_threads(1)
+    (g,) = hip.call("matmul_bf16", M * N, md, In(a16), In(b16), Out(M * N, "bf16"))
+    (o,) = oracle.call("matmul_bf16", M * N, md, In(a16), In(b16), Out(M * N, "bf16"))
+    exact, scale = av @ bv, (np.abs(av) @ np.abs(bv)).max()
+    eg = np.abs(to_float(g, "bf16").reshape(M, N) - exact).max() / scale
+    eo = np.abs(to_float(o, "bf16").reshape(M, N) - exact).max() / scale
+    ego = np.abs(to_float(g, "bf16").astype(np.float64) - to_float(o, "bf16")).max() / scale
+    print(f"matmul bf16 K=4096: gpu-f64 {eg:.2e}  cpu-f64 {eo:.2e}  gpu-cpu {ego:.2e}")
+    assert eg <= 1e-2 and eg <= eo and ego <= eg + eo
+    mdr = meta_reduce([M, K], [K, 1], 1)
+    (g,) = hip.call("sum_bf16", M * K, 2, 1, mdr, In(a16), Out(M, "bf16"))
+    (o,) = oracle.call("sum_bf16", M * K, 2, 1, mdr, In(a16), Out(M, "bf16"))
+    exact, scale = av.sum(1), np.abs(av).sum(1).max()
+    eg = np.abs(to_float(g, "bf16") - exact).max() / scale
+    eo = np.abs(to_float(o, "bf16") - exact).max() / scale
+    ego = np.abs(to_float(g, "bf16").astype(np.float64) - to_float(o, "bf16")).max() / scale
+    print(f"sum bf16 L=4096: gpu-f64 {eg:.2e}  cpu-f64 {eo:.2e}  gpu-cpu {ego:.2e}")
+    assert eg <= 1e-2 and eg <= eo and ego <= eg + eo
