@@ -364,6 +364,18 @@ void hip_le_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, 
 void hip_gt_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
 void hip_ge_scalar_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, mx_bool* output);
 
+/* Integer pow: `(x as f64).powf(c as f64) as T`, u8 through f32 (crates/maidenx_cpu/src/ops/unary.rs:565-572; the CUDA
+ * crate lists it at crates/maidenx_cuda/src/ops/unary.rs:105-136).  Evaluated in exact integer arithmetic: the result is
+ * what a correctly rounded pow followed by Rust's saturating, truncating `as` gives. */
+void hip_pow_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t constant, uint8_t* output);
+void hip_pow_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t constant, uint16_t* output);
+void hip_pow_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t constant, uint32_t* output);
+void hip_pow_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t constant, uint64_t* output);
+void hip_pow_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t constant, int8_t* output);
+void hip_pow_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t constant, int16_t* output);
+void hip_pow_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t constant, int32_t* output);
+void hip_pow_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t constant, int64_t* output);
+
 /* ---- reduction: replaces crates/maidenx_cuda/src/ops/reduction.rs:19-35 ---------------------------
  * sum/mean/max/min metadata = dims[n] | strides[n] | red_len[r] | red_stride[r] | offset, r = 1
  * (the only value the tensor layer produces, crates/maidenx_tensor/src/ops/reduction.rs:38).
@@ -400,7 +412,17 @@ int hip_noalloc_prepare(void);
 /* The same for f64 and the integers (crates/maidenx_cuda/src/ops/reduction.rs:59-113; mean for f64 only, as in
  * crates/maidenx_cpu/src/ops/reduction.rs:581-586).  The accumulator is the storage type: integer sums wrap (the
  * reference's release build), so they are bit-exact in any order; f64 sums differ from the sequential order by
- * rounding.  sum_to_shape takes contiguous inputs only for these dtypes; fold is not built for them. */
+ * rounding.  sum_to_shape takes contiguous inputs only for these dtypes.  fold (crates/maidenx_cpu/src/ops/reduction.rs:
+ * 591-599): f64 adds its windows in ascending order in f64, the integers wrap. */
+void hip_fold_f64(size_t num_els, size_t num_dims, const size_t* metadata, const double* input, double* output);
+void hip_fold_u8(size_t num_els, size_t num_dims, const size_t* metadata, const uint8_t* input, uint8_t* output);
+void hip_fold_u16(size_t num_els, size_t num_dims, const size_t* metadata, const uint16_t* input, uint16_t* output);
+void hip_fold_u32(size_t num_els, size_t num_dims, const size_t* metadata, const uint32_t* input, uint32_t* output);
+void hip_fold_u64(size_t num_els, size_t num_dims, const size_t* metadata, const uint64_t* input, uint64_t* output);
+void hip_fold_i8(size_t num_els, size_t num_dims, const size_t* metadata, const int8_t* input, int8_t* output);
+void hip_fold_i16(size_t num_els, size_t num_dims, const size_t* metadata, const int16_t* input, int16_t* output);
+void hip_fold_i32(size_t num_els, size_t num_dims, const size_t* metadata, const int32_t* input, int32_t* output);
+void hip_fold_i64(size_t num_els, size_t num_dims, const size_t* metadata, const int64_t* input, int64_t* output);
 void hip_sum_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
 void hip_max_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
 void hip_min_f64(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const double* input, double* output);
@@ -512,6 +534,18 @@ void hip_pad_with_replication_f64(size_t num_els_in, size_t num_els_out, size_t 
 void hip_pad_with_reflection_backward_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* grad_out, double* grad_in);
 void hip_pad_with_replication_backward_f64(size_t num_els_in, size_t num_els_out, size_t num_dims, const size_t* metadata, const double* grad_out, double* grad_in);
 
+/* ... and for the integers (crates/maidenx_cuda/src/ops/padding.rs:83-90; CPU instantiations at
+ * crates/maidenx_cpu/src/ops/padding.rs:670-677, 683-690, 696-703, 710-717, 723-730, 736-743): the forward modes copy,
+ * the backward sums are formed in the storage type and wrap, as the reference's release build does. */
+MX_DECL_PAD(uint8_t, u8)   MX_DECL_PAD_EDGE(uint8_t, u8)
+MX_DECL_PAD(uint16_t, u16) MX_DECL_PAD_EDGE(uint16_t, u16)
+MX_DECL_PAD(uint32_t, u32) MX_DECL_PAD_EDGE(uint32_t, u32)
+MX_DECL_PAD(uint64_t, u64) MX_DECL_PAD_EDGE(uint64_t, u64)
+MX_DECL_PAD(int8_t, i8)    MX_DECL_PAD_EDGE(int8_t, i8)
+MX_DECL_PAD(int16_t, i16)  MX_DECL_PAD_EDGE(int16_t, i16)
+MX_DECL_PAD(int32_t, i32)  MX_DECL_PAD_EDGE(int32_t, i32)
+MX_DECL_PAD(int64_t, i64)  MX_DECL_PAD_EDGE(int64_t, i64)
+
 /* ---- conv: replaces crates/maidenx_cuda/src/nn/conv.rs:12-24 --------------------------------------
  * metadata = 12 slots B, C, H, W, kh, kw, oh, ow, pad_h, pad_w, stride_h, stride_w as the kernel
  * reads them (crates/maidenx_cpu/src/nn/conv.rs:20-34).  im2col writes [B][C*kh*kw][oh*ow];
@@ -535,6 +569,8 @@ void hip_conv2d_col2im_f64(size_t num_els, const size_t* metadata, const double*
 void hip_softmax_f32(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const float* input, float* output);
 void hip_softmax_bf16(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const mx_bf16* input, mx_bf16* output);
 void hip_softmax_f16(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const mx_f16* input, mx_f16* output);
+/* f64 (crates/maidenx_cuda/src/nn/activation/softmax.rs:26-31): formed in f64 throughout. */
+void hip_softmax_f64(size_t num_els, size_t num_dims, size_t dim, const size_t* metadata, const double* input, double* output);
 
 /* ---- index ops -----------------------------------------------------------------------------------
  * No backend symbol exists for these in the reference: crates/maidenx_tensor/src/ops/indexing.rs runs them
@@ -587,6 +623,34 @@ MX_DECL_INDEX(mx_bf16, bf16, int32_t, i32)
 MX_DECL_INDEX(mx_bf16, bf16, int64_t, i64)
 MX_DECL_INDEX(mx_f16, f16, int32_t, i32)
 MX_DECL_INDEX(mx_f16, f16, int64_t, i64)
+/* f64, bool and the integers: the reference's index ops are dtype-generic (they move Scalars, indexing.rs:15, 93, 182,
+ * 315, 403), so every storage dtype has them.  The in-place adds follow add_at_index (utils/indexing.rs:121-135): f64
+ * adds in f64, bool is `||`, the integers wrap.  The weighted bincount takes float weights: f64 besides the three above. */
+#define MX_DECL_INDEX_WIDE(T, S, I, IS)                                                                                \
+    void hip_index_select_##S##_##IS(size_t num_dims, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride, \
+                                     size_t idx_offset, const I* indices, const T* input, T* output);                  \
+    void hip_gather_##S##_##IS(size_t num_dims, size_t dim, const size_t* in_layout, const size_t* idx_layout,         \
+                               const I* index, const T* input, T* output);                                             \
+    void hip_index_add_##S##_##IS(size_t num_dims, size_t dim, const size_t* self_layout, const size_t* src_layout,    \
+                                  size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices, const T* src,  \
+                                  T* self);                                                                            \
+    void hip_scatter_add_##S##_##IS(size_t num_dims, size_t dim, const size_t* self_layout, const size_t* idx_layout,  \
+                                    const size_t* src_layout, const I* index, const T* src, T* self);
+#define MX_DECL_INDEX_WIDE_ALL(T, S) MX_DECL_INDEX_WIDE(T, S, int32_t, i32) MX_DECL_INDEX_WIDE(T, S, int64_t, i64) MX_DECL_INDEX_PUT(T, S)
+MX_DECL_INDEX_WIDE_ALL(double, f64)
+MX_DECL_INDEX_WIDE(mx_bool, bool, int32_t, i32)      /* (spelled out: `bool` is a macro in C and must reach ## unexpanded) */
+MX_DECL_INDEX_WIDE(mx_bool, bool, int64_t, i64)
+MX_DECL_INDEX_PUT(mx_bool, bool)
+MX_DECL_INDEX_WIDE_ALL(uint8_t, u8)
+MX_DECL_INDEX_WIDE_ALL(uint16_t, u16)
+MX_DECL_INDEX_WIDE_ALL(uint32_t, u32)
+MX_DECL_INDEX_WIDE_ALL(uint64_t, u64)
+MX_DECL_INDEX_WIDE_ALL(int8_t, i8)
+MX_DECL_INDEX_WIDE_ALL(int16_t, i16)
+MX_DECL_INDEX_WIDE_ALL(int32_t, i32)
+MX_DECL_INDEX_WIDE_ALL(int64_t, i64)
+void hip_bincount_weighted_f64_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t w_stride, size_t w_offset, const double* weights, size_t out_size, double* output);
+void hip_bincount_weighted_f64_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t w_stride, size_t w_offset, const double* weights, size_t out_size, double* output);
 void hip_bincount_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t out_size, int32_t* output);
 void hip_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output);
 

@@ -96,6 +96,8 @@ def wide_unary_ops(dt):
         const += ["pow"]
     else:
         plain += ["sign", "square", "sqrt"]
+        if dt != "f64":
+            const += ["pow"]
         if dt[0] in "if":
             plain += ["neg", "abs"]
         if dt == "f64":
@@ -127,27 +129,34 @@ def wide_reduce_signatures(dtypes=REDUCE_WIDE_DTYPES):
         sig[f"sum_to_shape_{dt}"] = [SZ, SZ, P, P, P]
         sig[f"matmul_{dt}"] = [SZ, P, P, P, P]
         sig[f"matmul_backward_{dt}"] = [SZ, SZ, P, P, P, P, P, P]
+        sig[f"fold_{dt}"] = [SZ, SZ, P, P, P]
+        sig[f"pad_with_constant_{dt}"] = [SZ, SZ, SZ, P, P, P, CONST[dt]]
+        sig[f"pad_with_constant_backward_{dt}"] = [SZ, SZ, SZ, P, P, P]
+        for mode in ("reflection", "replication"):
+            sig[f"pad_with_{mode}_{dt}"] = [SZ, SZ, SZ, P, P, P]
+            sig[f"pad_with_{mode}_backward_{dt}"] = [SZ, SZ, SZ, P, P, P]
         if dt == "f64":
+            sig["softmax_f64"] = [SZ, SZ, SZ, P, P, P]
             sig["conv2d_im2col_f64"] = [SZ, P, P, P]
             sig["conv2d_col2im_f64"] = [SZ, P, P, P]
-            sig["pad_with_constant_f64"] = [SZ, SZ, SZ, P, P, P, CONST["f64"]]
-            sig["pad_with_constant_backward_f64"] = [SZ, SZ, SZ, P, P, P]
-            for mode in ("reflection", "replication"):
-                sig[f"pad_with_{mode}_f64"] = [SZ, SZ, SZ, P, P, P]
-                sig[f"pad_with_{mode}_backward_f64"] = [SZ, SZ, SZ, P, P, P]
     return sig
 
 
-def index_signatures(dtypes=("f32", "bf16", "f16")):
-    """Index ops (host loops in the reference's tensor layer, device entry points here)."""
+INDEX_WIDE_DTYPES = ("bool", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64")
+
+
+def index_signatures(dtypes=("f32", "bf16", "f16", "f64"), wide=INDEX_WIDE_DTYPES):
+    """Index ops (host loops in the reference's tensor layer, device entry points here).  `wide`: the dtypes that have
+    everything but the weighted bincount (whose weights are floats)."""
     sig = {}
-    for dt in dtypes:
+    for dt in tuple(dtypes) + tuple(wide):
         for it in ("i32", "i64"):
             sig[f"index_select_{dt}_{it}"] = [SZ, SZ, P, SZ, SZ, SZ, P, P, P]
             sig[f"gather_{dt}_{it}"] = [SZ, SZ, P, P, P, P, P]
             sig[f"index_add_{dt}_{it}"] = [SZ, SZ, P, P, SZ, SZ, SZ, P, P, P]
             sig[f"scatter_add_{dt}_{it}"] = [SZ, SZ, P, P, P, P, P, P]
-            sig[f"bincount_weighted_{dt}_{it}"] = [SZ, SZ, SZ, P, SZ, SZ, P, SZ, P]
+            if dt in dtypes:
+                sig[f"bincount_weighted_{dt}_{it}"] = [SZ, SZ, SZ, P, SZ, SZ, P, SZ, P]
         sig[f"index_put_{dt}"] = [SZ, P, SZ, P, SZ, P, P, P]
     for it in ("i32", "i64"):
         sig[f"bincount_{it}"] = [SZ, SZ, SZ, P, SZ, P]

@@ -13,7 +13,7 @@ MXH_WU(ln, WLn, double, double, f64, double) MXH_WU(log10, WLog10, double, doubl
 MXH_WU(log2, WLog2, double, double, f64, double) MXH_WU(exp, WExp, double, double, f64, double)
 MXH_WU(exp10, WExp10, double, double, f64, double) MXH_WU(exp2, WExp2, double, double, f64, double)
 MXH_WU(softplus, WSoftplus, double, double, f64, double)
-MXH_WUC(pow, WPow, double, double, f64, double) MXH_WUC(elu, WElu, double, double, f64, double)
+MXH_WUC(elu, WElu, double, double, f64, double)      // (pow comes with MXH_WIDE_SIGNED)
 
 MXH_WIDE_COMMON(mxh::b8_t, uint8_t, bool)
 MXH_WU(neg, WNeg, mxh::b8_t, uint8_t, bool, uint8_t)

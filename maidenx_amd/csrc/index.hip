@@ -28,6 +28,16 @@ namespace mxh {
 
 constexpr int IB = 256;
 
+// add_at_index (crates/maidenx_tensor/src/utils/indexing.rs:121-135): `+` in the storage dtype.  The floats round per
+// add (Ar<T>::add), bool is `||` (its Ar<T>::add), the integers wrap (the reference's release build; the saturating add
+// of the binary op family is a different function).
+template <class T> __device__ inline T idx_add(T a, T b) {
+    if constexpr (std::is_integral<T>::value) {
+        using U = typename std::make_unsigned<T>::type;
+        return (T)(U)((U)a + (U)b);
+    } else return Ar<T>::add(a, b);
+}
+
 struct Lay {            // one tensor: shape walk + strides
     int64_t strides[MAXD];
     int64_t offset;
@@ -125,7 +135,7 @@ __global__ __launch_bounds__(IB) void index_add_kernel(IdxSpace sp, Lay self, La
         const int32_t idx = (int32_t)indices[idx_offset + (int64_t)i * idx_stride];
         if (idx < 0 || (uint32_t)idx >= self_dim_size) { *flag = 1; continue; }
         T* p = dst + d0 + (int64_t)idx * self.strides[sp.dim];
-        *p = Ar<T>::add(*p, src[s0 + (int64_t)i * sr.strides[sp.dim]]);
+        *p = idx_add<T>(*p, src[s0 + (int64_t)i * sr.strides[sp.dim]]);
     }
 }
 
@@ -167,7 +177,7 @@ __global__ __launch_bounds__(IB) void index_add_sorted_kernel(IdxSpace sp, Lay s
     const int64_t s0 = dot(sp, c, sr, sp.dim);
     T* p = dst + dot(sp, c, self, sp.dim) + (int64_t)d * self.strides[sp.dim];
     T acc = *p;
-    for (uint32_t k = lo; k < n_idx && keys[k] == d; ++k) acc = Ar<T>::add(acc, src[s0 + (int64_t)vals[k] * sr.strides[sp.dim]]);
+    for (uint32_t k = lo; k < n_idx && keys[k] == d; ++k) acc = idx_add<T>(acc, src[s0 + (int64_t)vals[k] * sr.strides[sp.dim]]);
     *p = acc;
 }
 
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(IB) void index_add_rows_kernel(const uint32_t* __re
     for (uint32_t k = lo; k < n_idx && keys[k] == d; ++k) {
         const V s = *(const V*)(src + (((size_t)outer * n_idx + vals[k]) * inner_v + v) * VEC);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc.v[e] = Ar<T>::add(acc.v[e], s.v[e]);
+        for (int e = 0; e < VEC; ++e) acc.v[e] = idx_add<T>(acc.v[e], s.v[e]);
     }
     *p = acc;
 }
@@ -214,7 +224,7 @@ __global__ __launch_bounds__(IB) void scatter_add_kernel(IdxSpace sp, Lay self, 
         if (idx < 0) idx += (int32_t)self_dim_size;          // :434-438
         if (idx < 0 || (uint32_t)idx >= self_dim_size) { *flag = 1; continue; }
         T* p = dst + d0 + (int64_t)idx * self.strides[sp.dim];
-        *p = Ar<T>::add(*p, src[s0 + (int64_t)k * sr.strides[sp.dim]]);
+        *p = idx_add<T>(*p, src[s0 + (int64_t)k * sr.strides[sp.dim]]);
     }
 }
 
@@ -248,7 +258,7 @@ __global__ __launch_bounds__(IB) void bincount_weighted_kernel(const I* __restri
     for (size_t i = 0; i < n; ++i) {
         const int32_t v = (int32_t)in[offset + (int64_t)i * stride];
         if (b == 0 && (v < 0 || (size_t)v >= out_size)) *flag = 1;
-        if (v >= 0 && (size_t)v == b) acc = Ar<T>::add(acc, w[w_offset + (int64_t)i * w_stride]);
+        if (v >= 0 && (size_t)v == b) acc = idx_add<T>(acc, w[w_offset + (int64_t)i * w_stride]);
     }
     out[b] = acc;
 }
@@ -528,6 +538,51 @@ MXH_INDEX_PUT_FOR(f16_t, f16)
                                                       size_t w_offset, const T* weights, size_t out_size, T* output) { MXH_API;     \
         bincount_weighted<T, I>(n, stride, offset, input, w_stride, w_offset, weights, out_size, output);                            \
     }
+
+// f64, bool and the integers: the tensor layer's index ops are dtype-generic (indexing.rs:15, 93, 182, 315, 403 go through
+// Scalar), so every storage dtype has them; the weighted bincount is for float weights (f64 here besides the three above)
+#define MXH_INDEX_WIDE_FOR(T, P, TS, I, IS)                                                                                          \
+    extern "C" void hip_index_select_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride,    \
+                                                 size_t idx_offset, const I* indices, const P* input, P* output) { MXH_API;          \
+        index_select<T, I>(nd, dim, in_layout, n_idx, idx_stride, idx_offset, indices, (const T*)input, (T*)output);                 \
+    }                                                                                                                                \
+    extern "C" void hip_gather_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, const size_t* idx_layout, const I* index, \
+                                           const P* input, P* output) { MXH_API;                                                    \
+        gather<T, I>(nd, dim, in_layout, idx_layout, index, (const T*)input, (T*)output);                                            \
+    }                                                                                                                                \
+    extern "C" void hip_index_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* src_layout,            \
+                                              size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices, const P* src,   \
+                                              P* self) { MXH_API;                                                                    \
+        index_add<T, I>(nd, dim, self_layout, src_layout, n_idx, idx_stride, idx_offset, indices, (const T*)src, (T*)self);          \
+    }                                                                                                                                \
+    extern "C" void hip_scatter_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* idx_layout,          \
+                                                const size_t* src_layout, const I* index, const P* src, P* self) { MXH_API;         \
+        scatter_add<T, I>(nd, dim, self_layout, idx_layout, src_layout, index, (const T*)src, (T*)self);                             \
+    }
+#define MXH_INDEX_WIDE(T, P, TS)                                                                                                     \
+    MXH_INDEX_WIDE_FOR(T, P, TS, int32_t, i32) MXH_INDEX_WIDE_FOR(T, P, TS, int64_t, i64)                                            \
+    extern "C" void hip_index_put_##TS(size_t self_nd, const size_t* self_layout, size_t n_indices, const size_t* indices,          \
+                                       size_t src_nd, const size_t* src_layout, const P* src, P* self) { MXH_API;                   \
+        index_put<T>(self_nd, self_layout, n_indices, indices, src_nd, src_layout, (const T*)src, (T*)self);                        \
+    }
+MXH_INDEX_WIDE(double, double, f64)
+MXH_INDEX_WIDE(b8_t, uint8_t, bool)
+MXH_INDEX_WIDE(uint8_t, uint8_t, u8)
+MXH_INDEX_WIDE(uint16_t, uint16_t, u16)
+MXH_INDEX_WIDE(uint32_t, uint32_t, u32)
+MXH_INDEX_WIDE(uint64_t, uint64_t, u64)
+MXH_INDEX_WIDE(int8_t, int8_t, i8)
+MXH_INDEX_WIDE(int16_t, int16_t, i16)
+MXH_INDEX_WIDE(int32_t, int32_t, i32)
+MXH_INDEX_WIDE(int64_t, int64_t, i64)
+extern "C" void hip_bincount_weighted_f64_i32(size_t n, size_t stride, size_t offset, const int32_t* input, size_t w_stride, size_t w_offset,
+                                              const double* weights, size_t out_size, double* output) { MXH_API;
+    bincount_weighted<double, int32_t>(n, stride, offset, input, w_stride, w_offset, weights, out_size, output);
+}
+extern "C" void hip_bincount_weighted_f64_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t w_stride, size_t w_offset,
+                                              const double* weights, size_t out_size, double* output) { MXH_API;
+    bincount_weighted<double, int64_t>(n, stride, offset, input, w_stride, w_offset, weights, out_size, output);
+}
 
 MXH_INDEX_FOR(float, f32, int32_t, i32)
 MXH_INDEX_FOR(float, f32, int64_t, i64)

@@ -1,7 +1,7 @@
 // Unary element functions for f64, bool and the integers, after crates/maidenx_cpu/src/ops/unary.rs (line numbers at
 // each group).  f64 has every form of the family (the transcendental ones through the device math library); bool and
-// the integers have the forms the reference gives them, except the integer `pow` (a float `powf` and a cast in the
-// reference), which is not built.
+// the integers have the forms the reference gives them; the integer `pow` (a float `powf` and a cast in the reference)
+// is evaluated in exact integer arithmetic and rounded the way a correctly rounded `powf` and the cast would.
 // Integer negation, absolute value and square wrap on overflow, as the reference's release build does (its debug
 // build panics there); the scalar add / sub / mul saturate like the binary forms.
 #pragma once
@@ -67,6 +67,45 @@ template <class I> struct WideInt {                       // unary.rs:127-130, 1
         const T a = std::is_signed<T>::value ? abs(x) : x;
         if constexpr (std::is_same<T, int64_t>::value) return float_to_int<T>(::sqrt((double)a));
         else return float_to_int<T>(sqrtf((float)a));
+    }
+    // `(x as f64).powf(c as f64) as T` (u8 through f32), unary.rs:565-572.  Base and exponent are integers, so the power
+    // is an integer, or for c < 0 a fraction that the cast truncates; no floating-point pow is evaluated.  The exact
+    // power is formed in 128 bits and abandoned once it passes 2^64 (the cast saturates there anyway), rounded to f64 as
+    // a correctly rounded pow returns it (exact below 2^53, which covers every non-saturating result of the types
+    // narrower than 64 bits), and cast with Rust's `as` (toward zero, saturating).  A 64-bit base or exponent is first
+    // rounded to f64 like the reference's `as f64`.
+    static __device__ T pow(T x, T c) {
+        using L = std::numeric_limits<T>;
+        const bool xneg = x < 0, cneg = c < 0;
+        uint64_t ax = xneg ? (uint64_t)(U)((U)0 - (U)x) : (uint64_t)(U)x;        // (back to U before widening: the subtraction is done in int)
+        uint64_t ac = cneg ? (uint64_t)(U)((U)0 - (U)c) : (uint64_t)(U)c;
+        unsigned __int128 base = ax;
+        bool odd = (ac & 1) != 0;
+        if constexpr (sizeof(T) == 8) {
+            // the operands as f64: above 2^53 they are rounded to even multiples of a power of two
+            const double bd = (double)ax;
+            base = bd >= 18446744073709551616.0 ? ((unsigned __int128)1 << 64) : (unsigned __int128)(uint64_t)bd;
+            if (ac > (1ull << 53)) { odd = false; }
+        }
+        if (ac == 0) return (T)1;                                    // pow(x, 0) = 1 for every x
+        const bool neg = xneg && odd;
+        if (cneg) {                                                  // 1 / |x|^|c|
+            if (base == 0) return L::max();                          // pow(0, negative) = +inf
+            if (base == 1) return neg ? (T)-1 : (T)1;
+            return (T)0;
+        }
+        if (base == 0) return (T)0;
+        if (base == 1) return neg ? (T)-1 : (T)1;
+        unsigned __int128 p = 1, b = base;
+        bool over = ac >= 64 || (base >> 64) != 0;                   // base >= 2: the 64th power is already 2^64 or more
+        for (uint64_t e = ac; e != 0 && !over; e >>= 1) {
+            if ((b >> 64) != 0) { over = true; break; }              // b enters the product at the top bit of e at the latest
+            if (e & 1) { p *= b; if ((p >> 64) != 0) over = true; }
+            b *= b;
+        }
+        double d = over ? 1.0e300 : (double)(uint64_t)p;             // (the integer to f64 conversion rounds to nearest even)
+        if (neg) d = -d;
+        return float_to_int<T>(d);
     }
     static __device__ bool_t logical_not(T x) { return (bool_t)(x == 0); }
     static __device__ T add_scalar(T x, T c) { return Ar<T>::add(x, c); }             // :377-384: saturating, like the binary forms
@@ -155,6 +194,7 @@ MXH_WCMP(EqScalar, ==) MXH_WCMP(NeScalar, !=) MXH_WCMP(LtScalar, <) MXH_WCMP(LeS
     MXH_WUC(gt_scalar, WGtScalar, T, P, SUF, uint8_t) MXH_WUC(ge_scalar, WGeScalar, T, P, SUF, uint8_t)
 #define MXH_WIDE_UNSIGNED(T, SUF)                                                                              \
     MXH_WIDE_COMMON(T, T, SUF)                                                                                 \
-    MXH_WU(sign, WSign, T, T, SUF, T) MXH_WU(square, WSquare, T, T, SUF, T) MXH_WU(sqrt, WSqrt, T, T, SUF, T)
+    MXH_WU(sign, WSign, T, T, SUF, T) MXH_WU(square, WSquare, T, T, SUF, T) MXH_WU(sqrt, WSqrt, T, T, SUF, T)              \
+    MXH_WUC(pow, WPow, T, T, SUF, T)
 #define MXH_WIDE_SIGNED(T, SUF)                                                                                \
     MXH_WIDE_UNSIGNED(T, SUF) MXH_WU(neg, WNeg, T, T, SUF, T) MXH_WU(abs, WAbs, T, T, SUF, T)

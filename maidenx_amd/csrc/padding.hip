@@ -38,6 +38,21 @@ template <> struct PadAcc<double> {
     static __device__ A ld(double v) { return v; }
     static __device__ double st(A a) { return a; }
 };
+// The integers sum in the storage type and wrap (the reference's release build; its debug build panics on overflow):
+// formed in the unsigned type, where wrapping is defined, which also makes the sums independent of their order.
+template <class T> struct PadAccInt {
+    using A = typename std::make_unsigned<T>::type;
+    static __device__ A ld(T v) { return (A)v; }
+    static __device__ T st(A a) { return (T)a; }
+};
+template <> struct PadAcc<uint8_t> : PadAccInt<uint8_t> {};
+template <> struct PadAcc<uint16_t> : PadAccInt<uint16_t> {};
+template <> struct PadAcc<uint32_t> : PadAccInt<uint32_t> {};
+template <> struct PadAcc<uint64_t> : PadAccInt<uint64_t> {};
+template <> struct PadAcc<int8_t> : PadAccInt<int8_t> {};
+template <> struct PadAcc<int16_t> : PadAccInt<int16_t> {};
+template <> struct PadAcc<int32_t> : PadAccInt<int32_t> {};
+template <> struct PadAcc<int64_t> : PadAccInt<int64_t> {};
 enum EdgeMode : int { EDGE_REFLECT = 0, EDGE_REPLICATE = 1, EDGE_NONE = 2 };     // NONE: constant padding, whose border feeds nothing back
 
 // forward: out[i] = inside ? in[idx] : pad_value
@@ -792,3 +807,13 @@ MXH_PAD_FOR(bf16_t, bf16)
 MXH_PAD_FOR(f16_t, f16)
 MXH_PAD_EDGE_FOR(double, f64)      // (crates/maidenx_cuda/src/ops/padding.rs:82)
 MXH_PAD_FOR(double, f64)
+// the integers (crates/maidenx_cuda/src/ops/padding.rs:83-90)
+#define MXH_PAD_INT(T, SUF) MXH_PAD_EDGE_FOR(T, SUF) MXH_PAD_FOR(T, SUF)
+MXH_PAD_INT(uint8_t, u8)
+MXH_PAD_INT(uint16_t, u16)
+MXH_PAD_INT(uint32_t, u32)
+MXH_PAD_INT(uint64_t, u64)
+MXH_PAD_INT(int8_t, i8)
+MXH_PAD_INT(int16_t, i16)
+MXH_PAD_INT(int32_t, i32)
+MXH_PAD_INT(int64_t, i64)

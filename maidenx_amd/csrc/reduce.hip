@@ -641,6 +641,24 @@ struct FoldSpace {
     uint32_t n_windows, window, step;
 };
 
+// The type a fold's sums are formed in: f32 for the 32- and 16-bit floats (one rounding at the end), f64 for f64, the
+// unsigned counterpart for the integers (wrapping, as the reference's release build; its debug build panics).
+template <class T, class = void> struct FoldAcc {
+    using A = float;
+    static __device__ A ld(T v) { return IO<T>::ld(v); }
+    static __device__ T st(A a) { return IO<T>::fin(a, 0.0f); }
+};
+template <> struct FoldAcc<double, void> {
+    using A = double;
+    static __device__ A ld(double v) { return v; }
+    static __device__ double st(A a) { return a; }
+};
+template <class T> struct FoldAcc<T, typename std::enable_if<std::is_integral<T>::value>::type> {
+    using A = typename std::make_unsigned<T>::type;
+    static __device__ A ld(T v) { return (A)v; }
+    static __device__ T st(A a) { return (T)a; }
+};
+
 template <class T>
 __global__ __launch_bounds__(RB) void fold_kernel(FoldSpace sp, const T* __restrict__ in, T* __restrict__ out, size_t out_size,
                                                   size_t num_els) {
@@ -658,21 +676,22 @@ __global__ __launch_bounds__(RB) void fold_kernel(FoldSpace sp, const T* __restr
         else base += (int64_t)c * sp.strides[d];
         r = q;
     }
-    float acc = 0.0f;
+    using FA = FoldAcc<T>;
+    typename FA::A acc = 0;
     if (sp.step == 0) {
         if (p < sp.window)
             for (uint32_t w = 0; w < sp.n_windows; ++w)
-                acc += IO<T>::ld(in[(uint64_t)(base + (int64_t)w * sp.fold_stride + (int64_t)p * sp.window_stride) % num_els]);
+                acc = acc + FA::ld(in[(uint64_t)(base + (int64_t)w * sp.fold_stride + (int64_t)p * sp.window_stride) % num_els]);
     } else {
         uint32_t w0 = p >= sp.window ? (p - sp.window) / sp.step + 1 : 0;
         uint32_t w1 = p / sp.step;
         if (w1 >= sp.n_windows) w1 = sp.n_windows - 1;
         for (uint32_t w = w0; w <= w1 && sp.n_windows > 0; ++w) {
             uint32_t pos = p - w * sp.step;
-            acc += IO<T>::ld(in[(uint64_t)(base + (int64_t)w * sp.fold_stride + (int64_t)pos * sp.window_stride) % num_els]);
+            acc = acc + FA::ld(in[(uint64_t)(base + (int64_t)w * sp.fold_stride + (int64_t)pos * sp.window_stride) % num_els]);
         }
     }
-    out[o] = IO<T>::fin(acc, 0.0f);
+    out[o] = FA::st(acc);
 }
 
 template <class T>
@@ -739,6 +758,22 @@ using namespace mxh;
 MXH_REDUCE_FOR(float, f32)
 MXH_REDUCE_FOR(bf16_t, bf16)
 MXH_REDUCE_FOR(f16_t, f16)
+
+// fold for f64 and the integers (crates/maidenx_cuda/src/ops/reduction.rs:44-93 lists `fold` for every dtype; CPU
+// instantiations at crates/maidenx_cpu/src/ops/reduction.rs:632-643).  Their other reductions are in reduce_wide.hip.
+#define MXH_FOLD_FOR(T, SUF)                                                                                    \
+    extern "C" void hip_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) { MXH_API;       \
+        fold<T>(n, nd, md, in, out);                                                                            \
+    }
+MXH_FOLD_FOR(double, f64)
+MXH_FOLD_FOR(uint8_t, u8)
+MXH_FOLD_FOR(uint16_t, u16)
+MXH_FOLD_FOR(uint32_t, u32)
+MXH_FOLD_FOR(uint64_t, u64)
+MXH_FOLD_FOR(int8_t, i8)
+MXH_FOLD_FOR(int16_t, i16)
+MXH_FOLD_FOR(int32_t, i32)
+MXH_FOLD_FOR(int64_t, i64)
 
 // hip_sum_f32 for callers that cannot allocate (under graph capture, in a serving loop, in a harness that forbids it):
 // same arguments, same kernels, same bits, but the chunk partials go to the fixed array above instead of the library's

@@ -6,6 +6,7 @@
 // dependency of the reference that is not vendored), the stride helpers of
 // crates/maidenx_cpu/src/utils.rs, and the sequential / threaded execution switch.
 #pragma once
+#include <type_traits>
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
@@ -120,6 +121,15 @@ inline size_t get_strided_index(size_t idx, size_t num_dims, const size_t* dims,
 // Number of worker threads: 1 = sequential, deterministic order (used for parity);
 // >1 = the reference's rayon decomposition replayed with OpenMP (used for timing only).
 int num_threads();
+
+// `+=` of the reference's accumulating loops.  For the integer dtypes an overflow panics in the reference's debug build
+// and wraps in its release build; the wrap is restated (through the unsigned type, where C++ defines it).
+template <typename T> inline T add_wrap(T a, T b) {
+    if constexpr (std::is_integral<T>::value) {
+        using U = typename std::make_unsigned<T>::type;
+        return (T)(U)((U)a + (U)b);
+    } else return a + b;
+}
 
 }  // namespace orc
 

@@ -17,6 +17,13 @@ template <typename T> inline T zero_of() { return T(0); }
 template <> inline bf16 zero_of<bf16>() { return bf16::from_f32(0.0f); }
 template <> inline f16 zero_of<f16>() { return f16::from_f32(0.0f); }
 
+// add_at_index (utils/indexing.rs:121-135): `+` in the storage dtype - wrapping for the integers (the reference's
+// release build), `||` for bool.
+template <typename T> inline T idx_add(T a, T b) {
+    if constexpr (std::is_same<T, bool>::value) return a || b;
+    else return add_wrap(a, b);
+}
+
 struct Layout {
     size_t nd;
     const size_t *dims, *strides;
@@ -99,7 +106,7 @@ void index_add(size_t nd, size_t dim, const size_t* self_layout, const size_t* s
                 s += (d == dim ? i : c[d]) * sr.strides[d];
                 d0 += (d == dim ? (size_t)idx : c[d]) * sl.strides[d];
             }
-            self[d0] = self[d0] + src[s];
+            self[d0] = idx_add(self[d0], src[s]);
             return true;
         });
     }
@@ -120,7 +127,7 @@ void scatter_add(size_t nd, size_t dim, const size_t* self_layout, const size_t*
             if (cd >= sl.dims[d]) { g_index_error = 1; return false; }      // add_at_index bounds check
             d0 += cd * sl.strides[d];
         }
-        self[d0] = self[d0] + src[sr.at(c)];
+        self[d0] = idx_add(self[d0], src[sr.at(c)]);
         return true;
     });
 }
@@ -223,6 +230,28 @@ extern "C" int oracle_index_error() { int e = g_index_error; g_index_error = 0; 
         bincount_weighted<T, I>(n, stride, offset, input, w_stride, w_offset, weights, out_size, output);                            \
     }
 
+// bool and the integers (the tensor layer's index ops are dtype-generic through Scalar, indexing.rs:15,93,182,315,403):
+// everything but the weighted bincount, whose weights are floats
+#define ORC_INDEX_WIDE_FOR(T, TS, I, IS)                                                                                             \
+    extern "C" void oracle_index_select_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, size_t n_idx, size_t idx_stride, \
+                                                    size_t idx_offset, const I* indices, const T* input, T* output) {                \
+        index_select<T, I>(nd, dim, in_layout, n_idx, idx_stride, idx_offset, indices, input, output);                               \
+    }                                                                                                                                \
+    extern "C" void oracle_gather_##TS##_##IS(size_t nd, size_t dim, const size_t* in_layout, const size_t* idx_layout,              \
+                                              const I* index, const T* input, T* output) {                                          \
+        gather<T, I>(nd, dim, in_layout, idx_layout, index, input, output);                                                          \
+    }                                                                                                                                \
+    extern "C" void oracle_index_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* src_layout,         \
+                                                 size_t n_idx, size_t idx_stride, size_t idx_offset, const I* indices,              \
+                                                 const T* src, T* self) {                                                           \
+        index_add<T, I>(nd, dim, self_layout, src_layout, n_idx, idx_stride, idx_offset, indices, src, self);                        \
+    }                                                                                                                                \
+    extern "C" void oracle_scatter_add_##TS##_##IS(size_t nd, size_t dim, const size_t* self_layout, const size_t* idx_layout,       \
+                                                   const size_t* src_layout, const I* index, const T* src, T* self) {               \
+        scatter_add<T, I>(nd, dim, self_layout, idx_layout, src_layout, index, src, self);                                           \
+    }
+#define ORC_INDEX_WIDE(T, TS) ORC_INDEX_WIDE_FOR(T, TS, int32_t, i32) ORC_INDEX_WIDE_FOR(T, TS, int64_t, i64) ORC_INDEX_PUT_FOR(T, TS)
+
 ORC_INDEX_FOR(float, f32, int32_t, i32)
 ORC_INDEX_FOR(float, f32, int64_t, i64)
 ORC_INDEX_FOR(double, f64, int32_t, i32)
@@ -248,3 +277,13 @@ extern "C" void oracle_bincount_i32(size_t n, size_t stride, size_t offset, cons
 extern "C" void oracle_bincount_i64(size_t n, size_t stride, size_t offset, const int64_t* input, size_t out_size, int64_t* output) {
     bincount<int64_t>(n, stride, offset, input, out_size, output);
 }
+
+ORC_INDEX_WIDE(bool, bool)
+ORC_INDEX_WIDE(uint8_t, u8)
+ORC_INDEX_WIDE(uint16_t, u16)
+ORC_INDEX_WIDE(uint32_t, u32)
+ORC_INDEX_WIDE(uint64_t, u64)
+ORC_INDEX_WIDE(int8_t, i8)
+ORC_INDEX_WIDE(int16_t, i16)
+ORC_INDEX_WIDE(int32_t, i32)
+ORC_INDEX_WIDE(int64_t, i64)

@@ -68,9 +68,9 @@ void pad_const_backward(size_t n_in, size_t n_out, size_t nd, const size_t* md, 
     std::vector<T> g(n_in, zero_of<T>());
     for (size_t i = 0; i < n_out; ++i) {
         size_t dst;
-        if (map_index(p, nd, i, &dst)) g[dst] += grad_out[i];
+        if (map_index(p, nd, i, &dst)) g[dst] = add_wrap(g[dst], grad_out[i]);
     }
-    for (size_t i = 0; i < n_in; ++i) { T z = zero_of<T>(); z += g[i]; grad_in[p.in_off + i] = z; }
+    for (size_t i = 0; i < n_in; ++i) { grad_in[p.in_off + i] = add_wrap(zero_of<T>(), g[i]); }
 }
 
 // Reflection (padding.rs:177-195, :497-516) and replication (:289-295, :617-622): output coordinate →
@@ -123,8 +123,8 @@ template <typename T>
 void pad_edge_backward(Edge mode, size_t n_in, size_t n_out, size_t nd, const size_t* md, const T* grad_out, T* grad_in) {
     PadMeta p = parse(nd, md);
     std::vector<T> g(n_in, zero_of<T>());
-    for (size_t i = 0; i < n_out; ++i) g[edge_index(p, mode, nd, i)] += grad_out[i];
-    for (size_t i = 0; i < n_in; ++i) { T z = zero_of<T>(); z += g[i]; grad_in[p.in_off + i] = z; }
+    for (size_t i = 0; i < n_out; ++i) { T& c = g[edge_index(p, mode, nd, i)]; c = add_wrap(c, grad_out[i]); }
+    for (size_t i = 0; i < n_in; ++i) { grad_in[p.in_off + i] = add_wrap(zero_of<T>(), g[i]); }
 }
 
 }  // namespace
@@ -159,3 +159,12 @@ ORC_PAD_FOR(float, f32)
 ORC_PAD_FOR(double, f64)
 ORC_PAD_FOR(bf16, bf16)
 ORC_PAD_FOR(f16, f16)
+// the integers (padding.rs:670-677, 683-690, 696-703, 710-717, 723-730, 736-743): copies forward, wrapping sums backward
+ORC_PAD_FOR(uint8_t, u8)
+ORC_PAD_FOR(uint16_t, u16)
+ORC_PAD_FOR(uint32_t, u32)
+ORC_PAD_FOR(uint64_t, u64)
+ORC_PAD_FOR(int8_t, i8)
+ORC_PAD_FOR(int16_t, i16)
+ORC_PAD_FOR(int32_t, i32)
+ORC_PAD_FOR(int64_t, i64)

@@ -57,15 +57,6 @@ inline size_t dst_of(size_t i, size_t nred, const size_t* red_l, const size_t* r
     return dst;
 }
 
-// `+=` of the accumulating loops.  For the integer dtypes an overflow panics in the reference's debug build and wraps
-// in its release build; the wrap is restated (through the unsigned type, where C++ defines it).
-template <typename T> inline T add_wrap(T a, T b) {
-    if constexpr (std::is_integral<T>::value) {
-        using U = typename std::make_unsigned<T>::type;
-        return (T)(U)((U)a + (U)b);
-    } else return a + b;
-}
-
 // Shared skeleton of sum_op! (:6-89), mean_op! (:185-272), max_op! (:383-467), min_op! (:469-553).
 template <typename T, typename Acc, typename Fin>
 void reduce_axis(size_t num_els, size_t num_dims, size_t nred, const size_t* md, const T* inp, T* out, T init,
@@ -164,7 +155,7 @@ void fold(size_t num_els, size_t nd, const size_t* md, const T* inp, T* out) {
             dst = d == fold_dim ? dst * fold_size + pos : dst * dims[d] + coords[d];
         }
         T v = in[src];
-        locked(cells[dst], threaded, [&](T& o) { o += v; });
+        locked(cells[dst], threaded, [&](T& o) { o = add_wrap(o, v); });
     }
     for (size_t i = 0; i < out_size; ++i) out[i] = cells[i].val;
 }
@@ -217,6 +208,9 @@ ORC_REDUCE_FOR(f16, f16)
     }                                                                                                           \
     extern "C" void oracle_sum_to_shape_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {     \
         sum_to_shape<T>(n, nd, md, in, out);                                                                    \
+    }                                                                                                           \
+    extern "C" void oracle_fold_##SUF(size_t n, size_t nd, const size_t* md, const T* in, T* out) {             \
+        fold<T>(n, nd, md, in, out);                                                                            \
     }
 ORC_REDUCE_INT_FOR(uint8_t, u8)
 ORC_REDUCE_INT_FOR(uint16_t, u16)

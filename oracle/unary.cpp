@@ -156,6 +156,15 @@ template <typename I> struct IntFx {
         r = std::trunc(r);
         return r > (long double)L::max() ? L::max() : (T)r;
     }
+    // unary.rs:565-572: `(x as f64).powf(c as f64) as T` (u8 through f32), Rust's `as`: toward zero, saturating, NaN -> 0
+    static T pow(T x, T c) {
+        long double r = std::is_same<T, uint8_t>::value ? (long double)std::pow((float)x, (float)c) : (long double)std::pow((double)x, (double)c);
+        if (std::isnan(r)) return 0;
+        r = std::trunc(r);
+        if (r >= (long double)L::max()) return L::max();
+        if (r <= (long double)L::min()) return L::min();
+        return (T)r;
+    }
     static bool logical_not(T x) { return x == 0; }
     static T add_scalar(T x, T c) { return std::is_signed<T>::value || sizeof(T) < 8 ? sat((__int128)x + c) : (T)((unsigned __int128)x + c > L::max() ? L::max() : x + c); }
     static T sub_scalar(T x, T c) { return sat((__int128)x - (__int128)c); }
@@ -257,7 +266,7 @@ ORC_ALL_FOR(f16, f16)
     ORC_UNARY_C(lt_scalar, T, SUF, bool) ORC_UNARY_C(le_scalar, T, SUF, bool)                          \
     ORC_UNARY_C(gt_scalar, T, SUF, bool) ORC_UNARY_C(ge_scalar, T, SUF, bool)
 #define ORC_UNSIGNED_FOR(T, SUF)                                                                       \
-    ORC_COMMON_FOR(T, SUF) ORC_UNARY(sign, T, SUF, T) ORC_UNARY(square, T, SUF, T) ORC_UNARY(sqrt, T, SUF, T)
+    ORC_COMMON_FOR(T, SUF) ORC_UNARY(sign, T, SUF, T) ORC_UNARY(square, T, SUF, T) ORC_UNARY(sqrt, T, SUF, T) ORC_UNARY_C(pow, T, SUF, T)
 #define ORC_SIGNED_FOR(T, SUF) ORC_UNSIGNED_FOR(T, SUF) ORC_UNARY(neg, T, SUF, T) ORC_UNARY(abs, T, SUF, T)
 
 ORC_UNSIGNED_FOR(uint8_t, u8)

@@ -165,7 +165,7 @@ class Runner:
         if kind == "oracle":
             self.lib = C.CDLL(ensure_oracle_built())
             self.prefix = "oracle_"
-            for name, args in {**S.signatures(("f32", "bf16", "f16", "f64")), **S.binary_signatures(), **S.index_signatures(("f32", "bf16", "f16", "f64"))}.items():
+            for name, args in {**S.signatures(("f32", "bf16", "f16", "f64")), **S.binary_signatures(), **S.index_signatures()}.items():
                 fn = getattr(self.lib, self.prefix + name)
                 fn.argtypes = args
                 fn.restype = None

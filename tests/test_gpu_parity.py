@@ -13,6 +13,7 @@ from helpers import (NP, PLAIN, cast_inputs, In, InOut, Out, bf16_to_f32, const_
 pytestmark = pytest.mark.gpu
 
 DTS = ["f32", "bf16", "f16"]
+INT_DTS = ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
 
 
 def both(oracle, hip, name, *args_builder):
@@ -241,6 +242,25 @@ def test_unary_transcendental_16bit(oracle, hip, op, dt):
     assert np.array_equal(np.isnan(fo), np.isnan(fh))
     ok = ~np.isnan(fo)
     assert np.array_equal(o[ok], h[ok])
+
+
+@pytest.mark.parametrize("dt", INT_DTS)
+def test_integer_pow_bit_exact(oracle, hip, dt):
+    """`(x as f64).powf(c as f64) as T` (unary.rs:565-572): the GPU's exact-integer evaluation against the oracle's libm
+    pow and cast - every (x, c) pair of the 8-bit types, boundary sets for the wider ones (the roots of the type's bounds,
+    powers of two, 2^53 and its neighbours, negative and huge exponents)."""
+    from test_oracle_properties import int_pow_cases
+    info = np.iinfo(NP[dt])
+    if info.bits == 8:
+        xs = np.arange(info.min, info.max + 1).astype(NP[dt])
+        cs = range(info.min, info.max + 1)
+    else:
+        xs, cs = int_pow_cases(dt, rng(97))
+    # one call per exponent on a 2-d strided view, so that the strided kernel is exercised as well
+    md = meta_unary([xs.size], [1])
+    for c in cs:
+        (o,), (h,) = both(oracle, hip, f"pow_{dt}", lambda: (xs.size, 1, md, In(xs), int(c), Out(xs.size, dt)))
+        assert np.array_equal(o, h), (dt, c, xs[np.nonzero(o != h)[0][:5]], o[o != h][:5], h[o != h][:5])
 
 
 TABLE_OPS = ["sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln", "log10", "log2", "exp", "exp10", "exp2", "softplus"]
@@ -513,6 +533,45 @@ def test_pad_constant_forward_backward(oracle, hip, shape, pads, dt):
     assert same_bits(o, h)
 
 
+def int_values(r, n, dt):
+    """Integers over the whole range of the dtype, so that the backward sums wrap."""
+    info = np.iinfo(NP[dt])
+    return r.integers(info.min, info.max, n, dtype=NP[dt], endpoint=True)
+
+
+@pytest.mark.parametrize("dt", INT_DTS)
+@pytest.mark.parametrize("shape,pads", PAD_CASES[:4] + [([3, 20, 24], [(0, 0), (3, 3), (2, 5)])])
+def test_pad_three_modes_integer_dtypes(oracle, hip, shape, pads, dt):
+    """Forward modes copy, backward modes add in the storage type with wrap-around: bit-exact whatever the order."""
+    r = rng(241)
+    out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+    n_in, n_out = int(np.prod(shape)), int(np.prod(out_shape))
+    x = np.concatenate([int_values(r, 1, dt), int_values(r, n_in, dt)])
+    go = int_values(r, n_out, dt)
+    md = meta_pad(shape, contiguous_strides(shape), 1, out_shape, pads)
+    (o,), (h,) = both(oracle, hip, f"pad_with_constant_{dt}", lambda: (n_in, n_out, len(shape), md, In(x), Out(n_out, dt), const_arg(5, dt)))
+    assert same_bits(o, h)
+    assert np.array_equal(h.reshape(out_shape), np.pad(x[1:].reshape(shape), pads, constant_values=5))
+    (o,), (h,) = both(oracle, hip, f"pad_with_constant_backward_{dt}",
+                      lambda: (n_in, n_out, len(shape), md, In(go), InOut(np.full(n_in + 2, 7, NP[dt]))))
+    assert same_bits(o, h)
+    for mode, np_mode in (("reflection", "reflect"), ("replication", "edge")):
+        if mode == "reflection" and any(s == 1 and (p[0] or p[1]) for s, p in zip(shape, pads)):
+            continue
+        (o,), (h,) = both(oracle, hip, f"pad_with_{mode}_{dt}", lambda: (n_in, n_out, len(shape), md, In(x), Out(n_out, dt)))
+        assert same_bits(o, h)
+        assert np.array_equal(h.reshape(out_shape), np.pad(x[1:].reshape(shape), pads, mode=np_mode))
+        (o,), (h,) = both(oracle, hip, f"pad_with_{mode}_backward_{dt}",
+                          lambda: (n_in, n_out, len(shape), md, In(go), InOut(np.full(n_in + 2, 7, NP[dt]))))
+        assert same_bits(o, h)
+        # each input position receives the wrapped sum of the output gradients that were read from it
+        idx = np.pad(np.arange(n_in).reshape(shape), pads, mode=np_mode).ravel()
+        want = np.zeros(n_in, dtype=NP[dt])
+        with np.errstate(over="ignore"):
+            np.add.at(want, idx, go)
+        assert np.array_equal(h[1:n_in + 1], want) and h[0] == 7 and h[-1] == 7
+
+
 def test_pad_transposed_input(oracle, hip):
     lay = LY.permuted([6, 9], [1, 0])
     r = rng(61)
@@ -638,6 +697,24 @@ def test_fold(oracle, hip, dims, strides, fd, wd, fold_size, step, dt):
         assert np.max(np.abs(a - b)) <= (1e-5 if dt == "f32" else 6e-2) * max(1.0, np.max(np.abs(a)))
 
 
+@pytest.mark.parametrize("dt", ["f64"] + INT_DTS)
+@pytest.mark.parametrize("dims,strides,fd,wd,fold_size,step", FOLD_CASES)
+def test_fold_f64_and_integers(oracle, hip, dims, strides, fd, wd, fold_size, step, dt):
+    """Integers add with wrap-around (order-free, so bit-exact); f64 adds its windows in ascending order, which is the
+    sequential reference's order when the window dim follows the fold dim (as the tensor layer builds it)."""
+    r = rng(113)
+    n = int(np.prod(dims))
+    strides = strides or contiguous_strides(dims)
+    x = r.standard_normal(n + 1) if dt == "f64" else int_values(r, n + 1, dt)
+    md = u64(dims, strides, fd, wd, fold_size, step, dims[wd], 1)
+    out_n = int(np.prod([fold_size if d == fd else v for d, v in enumerate(dims) if d != wd]))
+    (o,), (h,) = both(oracle, hip, f"fold_{dt}", lambda: (n, len(dims), md, In(x), Out(out_n, dt)))
+    if dt != "f64" or fd < wd:
+        assert same_bits(o, h)
+    else:
+        assert np.max(np.abs(o - h)) <= 1e-13 * max(1.0, np.max(np.abs(o)))
+
+
 SOFTMAX_CASES = [([2, 3], 1), ([2, 2, 3], 2), ([2, 3], 0), ([64, 5], 1), ([33, 2048], 1), ([9, 2052], 1), ([3, 40000], 1), ([7, 300], 1),
                  ([6, 50, 130], 1), ([4, 3, 5, 6], 0), ([5, 6], 7), ([10000], 0),
                  # long inner columns: the block-split kernel with narrow and with 16-byte column vectors
@@ -693,6 +770,36 @@ def test_softmax_strided_and_special_values(oracle, hip):
     (o,), (h,) = both(oracle, hip, "softmax_f32", lambda: (12, 2, 1, meta_unary([4, 3], [3, 1], 0), In(v.ravel()), Out(12, "f32")))
     assert np.array_equal(np.isnan(o), np.isnan(h))
     assert np.allclose(o[~np.isnan(o)], h[~np.isnan(o)], rtol=1e-6)
+
+
+@pytest.mark.parametrize("shape,dim", SOFTMAX_CASES)
+def test_softmax_f64(oracle, hip, shape, dim):
+    """f64 (softmax.rs:26-31 of the CUDA crate lists it): against scipy's softmax in float64 and against the oracle;
+    the only differences are the device library's exp (within 1 ulp of the host's) and the tree order of a long row's sum."""
+    from scipy.special import softmax as sp_softmax
+    r = rng(131)
+    n = int(np.prod(shape))
+    x = r.standard_normal(n) * 3
+    md = meta_unary(shape, contiguous_strides(shape), 0)
+    (o,), (h,) = both(oracle, hip, "softmax_f64", lambda: (n, len(shape), dim, md, In(x), Out(n, "f64")))
+    axis = dim if dim < len(shape) else len(shape) - 1
+    truth = sp_softmax(x.reshape(shape), axis=axis).ravel()
+    assert np.all(np.abs(h - truth) <= 1e-13 * truth + 1e-300)
+    assert np.all(np.abs(h - o) <= 1e-13 * truth + 1e-300)
+
+
+def test_softmax_f64_strided_and_special_values(oracle, hip):
+    r = rng(137)
+    lay = LY.permuted([3, 4, 5, 6], [2, 0, 3, 1], off=3)
+    st = np.concatenate([np.zeros(3), r.standard_normal(360)])
+    md = meta_unary([3, 4, 5, 6], lay["strides"], lay["off"])
+    for dim in (0, 1, 2, 3):
+        (o,), (h,) = both(oracle, hip, "softmax_f64", lambda: (360, 4, dim, md, In(st), Out(360, "f64")))
+        assert np.allclose(o, h, rtol=1e-13, atol=0)
+    v = np.array([[0.0, -np.inf, 1.0], [-np.inf, -np.inf, -np.inf], [np.nan, 1.0, 2.0], [np.inf, 1.0, 2.0]])
+    (o,), (h,) = both(oracle, hip, "softmax_f64", lambda: (12, 2, 1, meta_unary([4, 3], [3, 1], 0), In(v.ravel()), Out(12, "f64")))
+    assert np.array_equal(np.isnan(o), np.isnan(h))
+    assert np.allclose(o[~np.isnan(o)], h[~np.isnan(o)], rtol=1e-13)
 
 
 # ---------------------------------------------------------------------------------------------------
@@ -755,6 +862,44 @@ def test_index_add_with_many_indices(oracle, hip, shape, dim, n_idx, dt):
     (o,), (h,) = both(oracle, hip, f"index_add_{dt}_i32",
                       lambda: (len(shape), dim, layout(shape), layout(src_shape), n_idx, 1, 0, In(idx), In(src), InOut(x.copy())))
     assert same_bits(o, h)
+
+
+@pytest.mark.parametrize("dt", ["f64", "bool"] + INT_DTS)
+@pytest.mark.parametrize("it", ["i32", "i64"])
+def test_index_ops_wide_dtypes(oracle, hip, dt, it):
+    """Every storage dtype has the index ops (the reference moves Scalars).  Copies are bit-exact; the in-place adds are
+    add_at_index's: f64 in order, `||` for bool, wrap-around for the integers (full-range values, so they do wrap)."""
+    r = rng(179)
+    IT = NP[it]
+    shape, dim = [6, 40, 9], 1
+    n = int(np.prod(shape))
+    x = wide_values(r, n + 2, dt)
+    L = layout(shape, off=2)
+    # index_select with few and with many indices; gather with negative indices
+    for n_idx in (5, 700):
+        idx = r.integers(0, shape[dim], n_idx).astype(IT)
+        out_shape = [6, n_idx, 9]
+        (o,), (h,) = both(oracle, hip, f"index_select_{dt}_{it}", lambda: (3, dim, L, n_idx, 1, 0, In(idx), In(x), Out(int(np.prod(out_shape)), dt)))
+        assert same_bits(o, h)
+        assert same_bits(h.reshape(out_shape), np.take(x[2:].reshape(shape), idx, axis=dim))
+        src = wide_values(r, int(np.prod(out_shape)), dt)
+        (o,), (h,) = both(oracle, hip, f"index_add_{dt}_{it}", lambda: (3, dim, L, layout(out_shape), n_idx, 1, 0, In(idx), In(src), InOut(x.copy())))
+        assert same_bits(o, h), ("index_add", n_idx)
+    ishape = [6, 17, 9]
+    index = r.integers(-shape[dim], shape[dim], ishape).astype(IT).ravel()
+    (o,), (h,) = both(oracle, hip, f"gather_{dt}_{it}", lambda: (3, dim, L, layout(ishape), In(index), In(x), Out(index.size, dt)))
+    assert same_bits(o, h)
+    assert same_bits(h.reshape(ishape), np.take_along_axis(x[2:].reshape(shape), index.reshape(ishape).astype(np.int64) % shape[dim], axis=dim))
+    src = wide_values(r, index.size, dt)
+    (o,), (h,) = both(oracle, hip, f"scatter_add_{dt}_{it}", lambda: (3, dim, L, layout(ishape), layout(ishape), In(index), In(src), InOut(x.copy())))
+    assert same_bits(o, h)
+    # index_put_: a [40, 9] source into self[4]
+    srcp = wide_values(r, 40 * 9, dt)
+    (o,), (h,) = both(oracle, hip, f"index_put_{dt}", lambda: (3, L, 1, u64(4), 2, layout([40, 9]), In(srcp), InOut(x.copy())))
+    assert same_bits(o, h)
+    want = x.copy()
+    want[2:].reshape(shape)[4] = srcp.reshape(40, 9)
+    assert same_bits(h, want)
 
 
 def test_index_ops_on_permuted_tensors(oracle, hip):

@@ -289,6 +289,35 @@ def test_oracle_edge_pad_vs_numpy_pad_and_adjoint(oracle, shape, pads, mode, np_
     assert abs(np.dot(y, g) - np.dot(x.ravel(), gx)) <= 1e-9 * (np.abs(y * g).sum() + 1)
 
 
+@pytest.mark.parametrize("dt", ["u8", "i16", "u32", "i64"])
+def test_oracle_integer_pads_vs_numpy_and_wrapping_sums(oracle, dt):
+    """The integer instantiations (padding.rs:670-743): forward against numpy.pad, backward against numpy's wrapping
+    add.at over the index map that numpy.pad of an index tensor gives (an independent statement of which output reads
+    which input)."""
+    from helpers import NP
+    r = rng(89)
+    info = np.iinfo(NP[dt])
+    shape, pads = [4, 9], [(2, 1), (4, 8)]
+    out_shape = [s + p[0] + p[1] for s, p in zip(shape, pads)]
+    n_in, n_out = int(np.prod(shape)), int(np.prod(out_shape))
+    x = r.integers(info.min, info.max, shape, dtype=NP[dt], endpoint=True)
+    g = r.integers(info.min, info.max, n_out, dtype=NP[dt], endpoint=True)
+    md = meta_pad(shape, contiguous_strides(shape), 0, out_shape, pads)
+    (y,) = oracle.call(f"pad_with_constant_{dt}", n_in, n_out, 2, md, In(x.ravel()), Out(n_out, dt), 3)
+    assert np.array_equal(y.reshape(out_shape), np.pad(x, pads, constant_values=3))
+    (gx,) = oracle.call(f"pad_with_constant_backward_{dt}", n_in, n_out, 2, md, In(g), InOut(np.full(n_in, 9, NP[dt])))
+    assert np.array_equal(gx.reshape(shape), g.reshape(out_shape)[2:2 + 4, 4:4 + 9])
+    for mode, np_mode in (("reflection", "reflect"), ("replication", "edge")):
+        (y,) = oracle.call(f"pad_with_{mode}_{dt}", n_in, n_out, 2, md, In(x.ravel()), Out(n_out, dt))
+        assert np.array_equal(y.reshape(out_shape), np.pad(x, pads, mode=np_mode))
+        (gx,) = oracle.call(f"pad_with_{mode}_backward_{dt}", n_in, n_out, 2, md, In(g), InOut(np.full(n_in, 9, NP[dt])))
+        idx = np.pad(np.arange(n_in).reshape(shape), pads, mode=np_mode).ravel()
+        want = np.zeros(n_in, dtype=NP[dt])
+        with np.errstate(over="ignore"):
+            np.add.at(want, idx, g)
+        assert np.array_equal(gx, want)
+
+
 def test_oracle_reflection_wraps_more_than_once(oracle):
     # pads wider than the dim: the mirror loop of padding.rs:186-193 runs several times; numpy's reflect does the same
     x = np.arange(1.0, 4.0)
@@ -323,6 +352,30 @@ def test_oracle_fold_is_adjoint_of_unfold(oracle, shape, dim, size, step):
 def u64_(*parts):
     from helpers import u64
     return u64(*parts)
+
+
+@pytest.mark.parametrize("dt", ["u8", "i32", "u64"])
+def test_oracle_integer_fold_counts_windows_and_wraps(oracle, dt):
+    """fold of all-ones windows counts the windows that cover each position (a closed form); fold of full-range values
+    is numpy's wrapping add.at over the positions c[fold]*step + c[window]."""
+    from helpers import NP
+    n_windows, size, step, inner = 7, 4, 3, 5
+    fold_size = (n_windows - 1) * step + size
+    dims = [n_windows, size, inner]
+    md = u64_(dims, contiguous_strides(dims), 0, 1, fold_size, step, size, 0)
+    (cnt,) = oracle.call(f"fold_{dt}", n_windows * size * inner, 3, md, In(np.ones(n_windows * size * inner, NP[dt])), Out(fold_size * inner, dt))
+    pos = np.arange(fold_size)
+    want = np.array([sum(1 for w in range(n_windows) if 0 <= p - w * step < size) for p in pos])
+    assert np.array_equal(cnt.reshape(fold_size, inner), np.repeat(want[:, None], inner, 1).astype(NP[dt]))
+    r = rng(91)
+    info = np.iinfo(NP[dt])
+    y = r.integers(info.min, info.max, dims, dtype=NP[dt], endpoint=True)
+    (f,) = oracle.call(f"fold_{dt}", y.size, 3, md, In(y.ravel()), Out(fold_size * inner, dt))
+    acc = np.zeros((fold_size, inner), NP[dt])
+    w, k = np.meshgrid(np.arange(n_windows), np.arange(size), indexing="ij")
+    with np.errstate(over="ignore"):
+        np.add.at(acc, (w * step + k).ravel(), y.reshape(-1, inner))
+    assert np.array_equal(f.reshape(fold_size, inner), acc)
 
 
 @pytest.mark.parametrize("shape,dim", [([5, 7], 1), ([5, 7], 0), ([3, 4, 6], 1), ([2, 3, 4, 5], 3), ([2, 3, 4, 5], 0), ([6], 0), ([4, 3], 9)])
@@ -821,3 +874,104 @@ def test_oracle_wide_matmul_vs_exact_products(oracle, dt, a_perm, b_perm):
     eb = np.einsum("bik,bij->bkj", a.astype(object), go.astype(object))
     assert [int(v) for v in ga] == [(int(v) - info.min) % span + info.min for v in ea.ravel()]
     assert [int(v) for v in gb] == [(int(v) - info.min) % span + info.min for v in eb.ravel()]
+
+
+# ---- integer pow -------------------------------------------------------------------------------------
+def int_pow_model(x, c, dt):
+    """`(x as f64).powf(c as f64) as T` from first principles, in Python's unbounded integers: the exact power (a
+    fraction for c < 0), rounded to f64 as a correctly rounded pow returns it, truncated toward zero and clamped to the
+    type like Rust's `as`.  64-bit operands are first rounded to f64 like the reference's own conversion."""
+    from fractions import Fraction
+    from helpers import NP
+    info = np.iinfo(NP[dt])
+    x, c = int(x), int(c)
+    if info.bits == 64:
+        x, c = int(float(x)), int(float(c))
+    if c == 0:
+        v = 1.0
+    elif x == 0:
+        v = float("inf") if c < 0 else 0.0
+    elif abs(x) == 1:
+        v = float(x) if c % 2 else 1.0
+    elif c < 0:
+        v = 0.0                                              # |x| >= 2: a fraction below 1 in magnitude
+    elif c * (abs(x).bit_length() - 1) > 70:
+        v = float("inf") if x > 0 or c % 2 == 0 else float("-inf")      # beyond 2^70: saturates whatever it is exactly
+    else:
+        v = float(Fraction(x) ** c)                          # Python rounds int -> float to nearest even
+    if v != v:
+        return 0
+    if v >= float(info.max):
+        return info.max
+    if v <= float(info.min):
+        return info.min
+    return int(v)
+
+
+@pytest.mark.parametrize("dt", ["u8", "i8"])
+def test_oracle_integer_pow_exhaustive_8bit(oracle, dt):
+    from helpers import NP
+    info = np.iinfo(NP[dt])
+    xs = np.arange(info.min, info.max + 1).astype(NP[dt])
+    for c in range(info.min, info.max + 1):
+        (o,) = oracle.call(f"pow_{dt}", xs.size, 1, meta_unary([xs.size], [1]), In(xs), int(c), Out(xs.size, dt))
+        want = np.array([int_pow_model(x, c, dt) for x in xs], dtype=NP[dt])
+        assert np.array_equal(o, want), c
+
+
+def int_pow_cases(dt, r, n=400):
+    """Bases and exponents around every place the result changes character: 0, +-1, +-2, the square, cube and higher
+    roots of the type's bounds (one below, at, one above), powers of two, the bounds themselves, and random fill."""
+    from helpers import NP
+    info = np.iinfo(NP[dt])
+    xs = {0, 1, 2, 3, info.max, info.max - 1, info.min, info.min + 1 if info.min < 0 else 1}
+    for k in range(2, 64):
+        root = int(round(info.max ** (1.0 / k)))
+        for d in (-2, -1, 0, 1, 2):
+            xs.add(max(0, root + d))
+        xs.add(1 << min(k, info.bits - 2))
+    if info.min < 0:
+        xs |= {-v for v in xs if -v >= info.min}
+    if info.bits == 64:
+        xs |= {2 ** 53 - 1, 2 ** 53, 2 ** 53 + 1, 2 ** 53 + 3, 3037000499, 3037000500, 2642245, 2642246, 2 ** 32 - 1, 2 ** 32 + 1}
+    xs = sorted(v for v in xs if info.min <= v <= info.max)
+    xs = np.array(xs + list(r.integers(info.min, info.max, n, endpoint=True, dtype=NP[dt])), dtype=NP[dt])
+    cs = sorted({0, 1, 2, 3, 4, 5, 7, 8, 15, 16, 31, 32, 33, 52, 53, 62, 63, 64, 65, 100, info.max} | ({-1, -2, -3, info.min} if info.min < 0 else set()))
+    return xs, [c for c in cs if info.min <= c <= info.max]
+
+
+@pytest.mark.parametrize("dt", ["u16", "i16", "u32", "i32", "u64", "i64"])
+def test_oracle_integer_pow_on_boundary_sets(oracle, dt):
+    from helpers import NP
+    xs, cs = int_pow_cases(dt, rng(95))
+    for c in cs:
+        (o,) = oracle.call(f"pow_{dt}", xs.size, 1, meta_unary([xs.size], [1]), In(xs), int(c), Out(xs.size, dt))
+        want = np.array([int_pow_model(x, c, dt) for x in xs], dtype=NP[dt])
+        assert np.array_equal(o, want), c
+
+
+@pytest.mark.parametrize("dt", ["u8", "i32", "u64", "bool"])
+def test_oracle_integer_index_adds_wrap_and_bool_ors(oracle, dt):
+    """index_add_ / scatter_add_ on the integer dtypes against numpy's wrapping add.at, on bool against logical_or.at
+    (add_at_index, utils/indexing.rs:121-135)."""
+    from helpers import NP, layout
+    r = rng(99)
+    vals = (lambda n: r.integers(0, 2, n).astype(np.uint8)) if dt == "bool" else (lambda n: r.integers(np.iinfo(NP[dt]).min, np.iinfo(NP[dt]).max, n, dtype=NP[dt], endpoint=True))
+    shape, dim, n_idx = [5, 12, 4], 1, 30
+    x = vals(int(np.prod(shape)))
+    idx = r.integers(0, shape[dim], n_idx).astype(np.int32)
+    src_shape = [5, n_idx, 4]
+    src = vals(int(np.prod(src_shape)))
+    (got,) = oracle.call(f"index_add_{dt}_i32", 3, dim, layout(shape), layout(src_shape), n_idx, 1, 0, In(idx), In(src), InOut(x.copy()))
+    want = x.reshape(shape).copy()
+    moved = np.moveaxis(want, dim, 0)
+    with np.errstate(over="ignore"):
+        (np.logical_or if dt == "bool" else np.add).at(moved, idx, np.moveaxis(src.reshape(src_shape), dim, 0))
+    assert np.array_equal(got.reshape(shape), want)
+    index = r.integers(0, shape[dim], src_shape).astype(np.int32)
+    (got,) = oracle.call(f"scatter_add_{dt}_i32", 3, dim, layout(shape), layout(src_shape), layout(src_shape), In(index.ravel()), In(src), InOut(x.copy()))
+    want = x.reshape(shape).copy()
+    i0, _, i2 = np.meshgrid(np.arange(5), np.arange(n_idx), np.arange(4), indexing="ij")
+    with np.errstate(over="ignore"):
+        (np.logical_or if dt == "bool" else np.add).at(want, (i0.ravel(), index.ravel(), i2.ravel()), src)
+    assert np.array_equal(got.reshape(shape), want)
