@@ -142,24 +142,72 @@ MXH_HD float m_expm1(float x) {
     return y;
 }
 
+// a / b for operands whose quotient, reciprocal and remainders are all normal numbers: the correctly rounded IEEE
+// quotient.  On the device this is the compiler's own division sequence (reciprocal, one Newton step, three fused
+// residual corrections) without the operand scaling and the special-case fix-up that out-of-range operands need -
+// 8 instructions instead of 12; on the host it is the division itself.
+MXH_HD float div_in_range(float a, float b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    float y = __builtin_amdgcn_rcpf(b);
+    const float e0 = __builtin_fmaf(-b, y, 1.0f);
+    y = __builtin_fmaf(e0, y, y);
+    float q = a * y;
+    float r = __builtin_fmaf(-b, q, a);
+    q = __builtin_fmaf(r, y, q);
+    r = __builtin_fmaf(-b, q, a);
+    return __builtin_fmaf(r, y, q);
+#else
+    return a / b;
+#endif
+}
+
+// tanhf of FDLIBM, operation for operation, without a branch: every lane runs the same instructions and selects.
+//   |x| >= 1 : z = 1 - 2 / (t + 2),  t = expm1f(2|x|)         (reduction index k >= 3)
+//   |x| <  1 : z = -t / (t + 2),     t = expm1f(-2|x|)        (k in {0, -1, -2, -3})
+// expm1f is restated inline for exactly those arguments: the reduction a = hi - lo with its correction c, the
+// rational approximation, and the reconstruction by k: k = 0, k = -1, k <= -2 (y = 1 - (e - x), scaled, minus 1) and
+// 2 <= k < 23 (y = (1 - 2^-k) - (e - x), scaled).  For k >= 23 (|x| >= 7.8) FDLIBM forms y another way; there
+// t > 6e6 and z = 1 - 2/(t + 2) no longer depends on the last bits of t, and the k < 23 form gives the same z on every
+// input.  |x| >= 22 is 1 by FDLIBM's own shortcut; the tiny-|x| shortcut x * (1 + x) equals what the general path
+// returns; a NaN propagates through the arithmetic.  Each of these simplifications was kept only after the host build
+// of this function agreed with the library's tanhf on all 2^32 inputs (tests/test_mathfn.py, MATHFN_EXHAUSTIVE=1).
+// The two divisions have operands in [1, 2^64], far from any special case.
 MXH_HD float m_tanh(float x) {
-    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
-    const int32_t jx = (int32_t)f2u(x);
-    const int32_t ix = jx & 0x7fffffff;
-    if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;   // inf, NaN
-    // FDLIBM evaluates  1 - 2/(expm1(2|x|) + 2)  for |x| >= 1  and  -t/(t + 2), t = expm1(-2|x|)  below;
-    // both are one expm1 and one division, so each lane runs the same instructions with its own
-    // operands selected (the values, and therefore the bits, are those of the branchy original).
-    const bool big = ix >= 0x3f800000;
-    const float a2 = two * fabsf(x);
-    const float t = m_expm1(big ? a2 : -a2);
-    const float q = (big ? two : -t) / (t + two);
-    float z = big ? one - q : q;
-    if (ix >= 0x41b00000) z = one - tiny;         // |x| >= 22
-    float r = jx >= 0 ? z : -z;
-    if (ix < 0x24000000) r = x * (one + x);       // |x| < 2^-55
-    if (ix == 0) r = x;                           // +-0
-    return r;
+    const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f,
+                Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f,
+                Q5 = -2.0109921195e-07f;
+    const uint32_t ux = f2u(x), ix = ux & 0x7fffffffu;
+    const float ax = u2f(ix);
+    const bool big = ix >= 0x3f800000u;
+    const float a2 = ax + ax;
+    const float a = big ? a2 : -a2;                           // the argument of expm1
+    // k = (int)(invln2 * a +- 0.5).  FDLIBM sets k = -1 for 0.5 ln2 < |a| < 1.5 ln2 and skips the reduction below that;
+    // the formula gives the same k (and with k = 0 a reduction that changes nothing) for every one of these arguments.
+    const float tk = truncf(invln2 * a + (big ? 0.5f : -0.5f));
+    const int k = (int)tk;
+    const float hi = a - tk * ln2_hi;
+    const float lo = tk * ln2_lo;
+    const float xr = hi - lo;
+    const float c = (hi - xr) - lo;
+    const float hfx = 0.5f * xr;
+    const float hxs = xr * hfx;
+    const float r1 = 1.0f + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    const float t3 = 3.0f - r1 * hfx;
+    const float e = hxs * div_in_range(r1 - t3, 6.0f - xr * t3);
+    const float res0 = xr - (xr * e - hxs);                   // k = 0
+    float e2 = xr * (e - c) - c;
+    e2 -= hxs;
+    const float resm1 = 0.5f * (xr - e2) - 0.5f;              // k = -1
+    const float twomk = u2f((uint32_t)(0x7f - k) << 23);      // 2^-k
+    const float top = big ? 1.0f - twomk : 1.0f;              // 1 - 2^-k is exact for k < 25
+    float y = top - (e2 - xr);
+    y = u2f(f2u(y) + ((uint32_t)k << 23));                    // times 2^k
+    const float resg = big ? y : y - 1.0f;
+    const float t = k == 0 ? res0 : (k == -1 ? resm1 : resg);
+    const float q = div_in_range(big ? 2.0f : -t, t + 2.0f);
+    float z = big ? 1.0f - q : q;
+    if (ax >= 22.0f) z = 1.0f;                                // |x| >= 22 and +-inf; a NaN fails the test and has made z a NaN
+    return u2f((f2u(z) & 0x7fffffffu) | (ux & 0x80000000u));  // (|x| < 2^-55, FDLIBM's x * (1 + x) = x, comes out as x by itself)
 }
 
 MXH_HD float m_pow(float x, float c) { return (float)pow((double)x, (double)c); }

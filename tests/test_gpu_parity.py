@@ -263,6 +263,30 @@ def test_integer_pow_bit_exact(oracle, hip, dt):
         assert np.array_equal(o, h), (dt, c, xs[np.nonzero(o != h)[0][:5]], o[o != h][:5], h[o != h][:5])
 
 
+@pytest.mark.parametrize("op", ["tanh", "gelu"])
+def test_tanh_and_gelu_f32_bit_exact_on_16m_inputs(oracle, hip, op):
+    """The branch-free tanhf restatement (its two divisions use the reciprocal instruction and fused corrections) against the
+    oracle's libm on 2^24 inputs: every exponent from 2^-60 to 2^6 in both signs, dense around the switch points of the
+    algorithm (|x| = 0.5 ln 2 / 2, 1.5 ln 2 / 2, 1, 9, 19.6, 22), zeros, infinities, NaN."""
+    r = rng(31)
+    n = 1 << 24
+    x = (r.standard_normal(n) * np.exp2(r.integers(-60, 7, n))).astype(np.float32)
+    k = n // 16
+    for i, centre in enumerate((0.17328679, 0.51986039, 1.0, 9.0, 19.6, 22.0)):
+        x[i * k:(i + 1) * k] = (centre * (1.0 + r.uniform(-2e-3, 2e-3, k))).astype(np.float32) * r.choice(np.array([-1.0, 1.0], np.float32), k)
+    x[-8:] = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-39, -1e-39, 88.0], np.float32)
+    oracle.set_threads(0)
+    try:
+        (o,) = oracle.call(f"{op}_f32", n, 1, meta_unary([n], [1]), In(x), Out(n, "f32"))
+    finally:
+        oracle.set_threads(1)
+    (h,) = hip.call(f"{op}_f32", n, 1, meta_unary([n], [1]), In(x), Out(n, "f32"))
+    assert np.array_equal(np.isnan(o), np.isnan(h))
+    ok = ~np.isnan(o)
+    bad = np.nonzero(o[ok].view(np.uint32) != h[ok].view(np.uint32))[0]
+    assert bad.size == 0, (bad.size, x[ok][bad[:5]], o[ok][bad[:5]], h[ok][bad[:5]])
+
+
 TABLE_OPS = ["sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln", "log10", "log2", "exp", "exp10", "exp2", "softplus"]
 
 
