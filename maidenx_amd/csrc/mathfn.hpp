@@ -48,29 +48,29 @@ const uint64_t EXP2F_TAB[32] = {
     0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL
 };
 
+// Without a branch: the core runs for every input and the out-of-range results are selected afterwards, so the table
+// reads of the elements a thread owns are all in flight together (behind per-element branches each element waited
+// for its own read: [8192,8192] f32 took 110 us).
 MXH_HD float m_exp(float x) {
     const double InvLn2N = 0x1.71547652b82fep+0 * 32, Shift = 0x1.8p+52;
     const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32, C2 = 0x1.62e42ff0c52d6p-1 / 32;
-    uint32_t abstop = (f2u(x) >> 20) & 0x7ff;
-    if (abstop >= (f2u(88.0f) >> 20)) {
-        if (f2u(x) == f2u(-INFINITY)) return 0.0f;
-        if (abstop >= (f2u(INFINITY) >> 20)) return x + x;
-        if (x > 0x1.62e42ep6f) return INFINITY;      // overflow
-        if (x < -0x1.9fe368p6f) return 0.0f;         // underflow to zero
-    }
-    double xd = (double)x;
+    const double xd = (double)x;
     double kd = fma(InvLn2N, xd, Shift);
-    uint64_t ki = d2u(kd);
+    const uint64_t ki = d2u(kd);
     kd -= Shift;
-    double r = fma(InvLn2N, xd, -kd);
-    uint64_t t = EXP2F_TAB[ki % 32] + (ki << 47);
-    double s = u2d(t);
-    double z = fma(C0, r, C1);
-    double r2 = r * r;
+    const double r = fma(InvLn2N, xd, -kd);
+    const uint64_t t = EXP2F_TAB[ki % 32] + (ki << 47);
+    const double s = u2d(t);
+    const double z = fma(C0, r, C1);
+    const double r2 = r * r;
     double y = fma(C2, r, 1.0);
     y = fma(z, r2, y);
     y = y * s;
-    return (float)y;
+    float res = (float)y;                                   // (subnormal results round here, as in the library)
+    if (x > 0x1.62e42ep6f) res = INFINITY;                  // overflow, +inf
+    if (x < -0x1.9fe368p6f) res = 0.0f;                     // underflow to zero, -inf
+    if (x != x) res = x + x;                                // NaN
+    return res;
 }
 
 MXH_HD float m_expm1(float x) {
