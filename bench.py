@@ -601,6 +601,9 @@ def run_matmul(args):
         c, k = matmul_calls(lib, "hip_", new, dt, shapes, rng)
         chains += c; keep += k
     # the headline figure is the bf16 4096^3 forward + backward; f32 and the batched shape are reported beside it
+    # A pass of the headline chain is 0.37 ms: the K timed passes are over before the card has left its idle clocks
+    # unless the untimed part is long enough to raise them, so the warm-up is at least 200 passes (75 ms) here.
+    args = argparse.Namespace(**{**vars(args), "warmup": max(args.warmup, 200)})
     def rate(tags):
         sel = [c for c in chains if c.tag in tags]
         a = argparse.Namespace(steps=args.steps, warmup=args.warmup)
