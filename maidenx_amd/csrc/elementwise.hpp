@@ -388,6 +388,8 @@ inline bool ew_fuse(bool vec, const NdSpace<Op::NIN + 1>& sp, const EwPtrs<Op::N
     if constexpr (idx >= 0 && std::is_same<typename Op::In, float>::value && std::is_same<typename Op::Out, float>::value && sizeof(Op) <= 8) {
         // launch-bound sizes only: a large tensor is better off with four vectors per thread
         if (sp.ndims < 1 || sp.ndims > 2 || n >= (size_t)EW_SMALL_BLOCKS * EW_BLOCK * EW_UNR) return false;
+        // more than one block: the interpreter of recorded programs has no command for it, so the capture is a HIP graph
+        if (prog_recording() && cdiv(n, (size_t)EW_BLOCK * EW_UNR) > PROG_MAX_GRID) prog_abandon();
         FuseCmd c;
         std::memset((void*)&c, 0, sizeof(c));
         c.out = p.out;

@@ -1,16 +1,27 @@
-// Fused runs of elementwise launches inside a capture.
+// Fused chains of small launches inside a capture.
 //
-// A captured training step is mostly runs of elementwise kernels over one index space, each reading what the one
-// before wrote.  Replayed as graph nodes they cost 1.6-1.8 us apiece however small.  While a capture is open (and
-// cannot be a whole-capture program, see program.hpp), an f32 elementwise launch over a collapsed space of at most
-// two dims is not launched: it joins the open group when it iterates over the same space in the same form and every
-// overlap with the group's earlier members is element for element (same base, same strides) - then each thread
-// only ever re-reads what it wrote itself, and no ordering between threads is needed.  The group is closed by the
-// next thing queued on the stream, by a launch that does not fit, or by the end of the capture, and becomes ONE
-// kernel node that applies the members in order per element.  Every output is still written; results are the bytes
-// of the separate launches.
-// Members of at most 256 elements (a bias, a 3-element weight, a loss) need none of this care: a group of those is
-// run by a single work-group with a barrier between members, whatever their shapes and however they overlap.
+// A captured training step on small tensors is a few dozen dependent launches that each compute for well under a
+// microsecond; replayed as graph nodes they cost 2 to 4 us apiece however small, because each node waits for the one
+// before.  While a capture is open (and cannot be a whole-capture program, see program.hpp) such launches are not
+// launched: they join the open CHAIN, which becomes ONE kernel node with two phases.
+//
+// Parallel phase - members over one shared index space, every thread owning one vector (or element) of it:
+//   * an f32 elementwise launch over a collapsed space of at most two dims joins when it iterates over the same space in
+//     the same form and every overlap with the earlier members is element for element (same base, same strides): each
+//     thread then only ever re-reads what it wrote itself, and no ordering between threads is needed;
+//   * a small matmul of the one-thread-per-output kind (a reduction of at most 16 terms) joins as a producer over the
+//     flat space of its outputs; its operands are read across threads, so they may not overlap anything the chain's
+//     earlier members write, nor may a later member write them.
+// Serial phase ("tail") - stages run in order by the work-group that finishes the parallel phase last (every group
+// publishes its writes, then draws a ticket; the last ticket continues, the others exit, nobody waits):
+//   * elementwise launches of at most 256 elements (a bias, a 3-element weight, a loss), any shapes, any overlaps;
+//   * a row reduction that one work-group does in the eager path as well ([10000] -> [] sums);
+//   * a matmul with a handful of outputs and a long reduction (the weight gradient of a 3-feature layer).
+//   A stage is the same device code as its eager kernel, so results are the bytes of the separate launches.  A tail
+//   stage may depend on anything before it in stream order.  A parallel member that arrives after tail stages were
+//   queued is hoisted over them when it neither reads what they write nor writes what they read or write.
+// The chain is closed by the next thing queued on the stream, by a launch that does not fit, or by the end of the
+// capture.  Every output is still written.
 #pragma once
 #include <cstddef>
 #include <cstdint>
@@ -19,33 +30,80 @@
 
 namespace mxh {
 
-constexpr int FUSE_MAX_CMDS = 16;
+constexpr int FUSE_MAX_CMDS = 16;          // members of the parallel phase
+constexpr int FUSE_MAX_TAIL = 12;          // stages of the serial phase
+constexpr uint32_t FUSE_OP_DOT = 0xD07u;   // FuseCmd::op of a matmul producer (the other values index EwProgOps)
+constexpr int FUSE_TAIL_ARG_BYTES = 112;
+constexpr uint32_t FUSE_TICKETS = 1024;    // ticket slots per device
+
 struct FuseCmd {
     void* out;
     const void* in[2];
     int64_t os[2];            // element strides of the output over the (at most two) collapsed dims
-    int64_t is[2][2];         // the same for each input
-    uint32_t op;              // position of the functor in EwProgOps
+    int64_t is[2][2];         // the same for each input; FUSE_OP_DOT: {output row, reduction} of X, {reduction, output column} of Y
+    uint32_t op;              // position of the functor in EwProgOps, or FUSE_OP_DOT
     uint32_t nin;
     uint32_t fwd;             // bit j: input j is, element for element, what the previous member wrote (taken from registers)
-    uint32_t ndims;           // the member's own space: only read in a tiny group
-    uint32_t dims[2];
+    uint32_t ndims;           // the member's own space: only read in the tail
+    uint32_t dims[2];         // FUSE_OP_DOT: {output columns, reduction length}
     uint32_t nel;
-    uint32_t reserved;
+    // Byte j: where input j comes from when it is not forwarded.  Parallel phase: the number of the earlier member
+    // whose output it is element for element (read from that member's staged output), or FUSE_SRC_MEMORY.  Tail: the
+    // number of the earlier stage whose mirrored output holds it, FUSE_SRC_MEMORY (nothing in the tail writes it: it is
+    // fetched when the tail starts) or FUSE_SRC_MEMORY_LATE (read from memory when the stage runs).
+    uint32_t src;
     uint32_t payload[2];      // the functor's state (a scalar constant), bit for bit
 };
+constexpr uint32_t FUSE_SRC_MEMORY = 0xFFu, FUSE_SRC_MEMORY_LATE = 0xFEu;
+enum TailKind : uint32_t { TAIL_EW = 0, TAIL_ROW_REDUCE = 1, TAIL_DOT = 2 };
+struct TailCmd {
+    uint32_t kind;
+    uint32_t sub;             // TAIL_ROW_REDUCE: the instantiation number of row_prog_sub(); TAIL_DOT: 1 = the rows form
+    uint32_t sync;            // before this stage: 0 nothing, 1 a barrier that orders LDS, 2 one that also waits for memory
+    uint32_t fwd;             // TAIL_EW: as FuseCmd::fwd, against the stage before
+    int32_t moff[2];          // TAIL_EW, input from a mirror: element offset of the input's base from that stage's output
+    uint32_t mirrored;        // the stage's outputs (at most 256, contiguous) are also kept in LDS for later stages
+    uint32_t pad;
+    alignas(8) unsigned char arg[FUSE_TAIL_ARG_BYTES];      // FuseCmd, RowProgArgs or GemmArgs
+};
+static_assert(sizeof(FuseCmd) <= FUSE_TAIL_ARG_BYTES, "a tail stage holds an elementwise member");
 struct alignas(16) FuseGroup {
     uint32_t n, ndims, vec;   // vec: every member moves 16-byte vectors along the inner dim
-    uint32_t tiny;            // 1: members of at most one block's worth of elements each, any shapes, run by ONE block with a barrier between them
+    uint32_t ntail;
     uint32_t dims[2];
     FastDiv div_inner;
     size_t nvec;              // vectors (vec) or elements per member
-    FuseCmd cmd[FUSE_MAX_CMDS];
+    uint32_t* ticket;         // zero between launches: counts the work-groups that have finished the parallel phase
+    uint32_t prefetch;        // bit 2k+j: input j of tail stage k is fetched from memory when the tail starts
+    uint32_t blocks;          // work-groups of the launch
+    uint32_t pad[2];
+    alignas(16) FuseCmd cmd[FUSE_MAX_CMDS];
+    alignas(16) TailCmd tail[FUSE_MAX_TAIL];
+};
+static_assert(sizeof(FuseCmd) % 16 == 0 && sizeof(TailCmd) % 16 == 0, "the kernel copies whole 16-byte pieces of the members in use");
+static_assert(sizeof(FuseGroup) <= 4096, "the chain travels as kernel arguments");
+
+// byte range an operand of a recorded launch touches
+struct Extent {
+    uintptr_t lo, hi;
+    bool overlaps(const Extent& o) const { return lo < o.hi && o.lo < hi; }
 };
 
-// fuse.hip: one launch of the group on `stream`.
+// fuse.hip: one launch of the chain on `stream`.
 void fuse_launch(const FuseGroup& g, void* stream);
-// runtime.hip: offers a launch to the open group; true = taken (the caller must not launch).
+// fuse.hip: the current device's FUSE_TICKETS ticket slots (device memory, all zero); null when they cannot be located
+uint32_t* fuse_tickets();
+// runtime.hip: a graph capture is being recorded
+bool capture_open();
+// runtime.hip: offer a launch to the open chain; true = taken (the caller must not launch).
 bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes);
+// a one-thread-per-output f32 matmul: x, y are the extents of its operands
+bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y);
+// a tail stage with its argument block; in[0..nin) / out: the byte ranges it reads and writes (out: `outputs` contiguous
+// f32 values)
+bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs);
+// a capture that holds a launch the interpreter has no command for can only be a HIP graph: say so before offering that
+// launch to the chain (which only takes launches once the capture cannot be a program)
+void prog_abandon();
 
 }  // namespace mxh

@@ -22,8 +22,10 @@
 // a thread-per-output kernel (bit-exact with the reference: k ascending, unfused f32) or a
 // wave-per-output dot kernel.
 
+#include <cstring>
 #include <type_traits>
 
+#include "fuse.hpp"
 #include "gemm_host.hpp"
 #include "gemm_small.hpp"
 #include "mxh.hpp"
@@ -618,23 +620,78 @@ __global__ __launch_bounds__(GB) void gemm_wavedot_kernel(GemmArgs g) {
     if (live && lane == 0) ((T*)g.out)[idx] = Elem<T>::st(acc);
 }
 
+// byte range of a strided matmul operand: `rows` by `cols` elements at the given element strides
+static Extent operand_extent(const void* base, size_t rows, int64_t row_stride, size_t cols, int64_t col_stride, size_t batch, int64_t batch_stride, size_t esz) {
+    size_t span = (rows ? (rows - 1) * (size_t)row_stride : 0) + (cols ? (cols - 1) * (size_t)col_stride : 0) + (batch ? (batch - 1) * (size_t)batch_stride : 0);
+    return Extent{(uintptr_t)base, (uintptr_t)base + (span + 1) * esz};
+}
+static bool positive_strides(const GemmArgs& g) { return g.xb >= 0 && g.xi >= 0 && g.xr >= 0 && g.yb >= 0 && g.yr >= 0 && g.yj >= 0; }
+
+// While a capture is open: a one-thread-per-output f32 product offered to the open chain as a producer over the flat
+// space of its outputs (true: do not launch).
+static bool fuse_thread_dot(const GemmArgs& g, size_t outputs) {
+    if (!capture_open() || g.batch != 1 || g.R > 16 || outputs >= (1u << 24) || !positive_strides(g)) return false;
+    FuseCmd c;
+    std::memset((void*)&c, 0, sizeof(c));
+    c.out = g.out;
+    c.in[0] = g.X;
+    c.in[1] = g.Y;
+    c.os[0] = 1;
+    c.is[0][0] = g.xi; c.is[0][1] = g.xr;
+    c.is[1][0] = g.yr; c.is[1][1] = g.yj;
+    c.op = FUSE_OP_DOT;
+    c.nin = 2;
+    c.dims[0] = g.J; c.dims[1] = g.R;
+    return fuse_record_dot(c, outputs, operand_extent(g.X, g.I, g.xi, g.R, g.xr, 1, 0, sizeof(float)),
+                           operand_extent(g.Y, g.R, g.yr, g.J, g.yj, 1, 0, sizeof(float)));
+}
+// The same for a product of a handful of outputs with a long reduction: a stage of the chain's tail.
+static bool fuse_block_dot(const GemmArgs& g, size_t outputs, bool rows) {
+    if (!capture_open() || outputs > 8 || g.R > 65536 || !positive_strides(g)) return false;
+    static_assert(sizeof(GemmArgs) <= FUSE_TAIL_ARG_BYTES, "a tail stage holds a matmul's arguments");
+    const Extent in[2] = {operand_extent(g.X, g.I, g.xi, g.R, g.xr, g.batch, g.xb, sizeof(float)),
+                          operand_extent(g.Y, g.R, g.yr, g.J, g.yj, g.batch, g.yb, sizeof(float))};
+    const Extent out{(uintptr_t)g.out, (uintptr_t)g.out + outputs * sizeof(float)};
+    return fuse_record_tail(TAIL_DOT, rows ? 1 : 0, &g, sizeof(g), in, 2, out, outputs);
+}
+
+__global__ __launch_bounds__(256) void gemm_rowsdot_kernel(GemmArgs g) {
+    __shared__ float part[4 * 256 / WAVE];
+    gemm_rowsdot_any<256>(g, threadIdx.x, part);
+}
+
 template <class T>
 void gemm_dispatch(GemmArgs g) {
     if (g.I == 0 || g.J == 0 || g.batch == 0) return;
     size_t outputs = (size_t)g.I * g.J * g.batch;
     if (g.R <= 16 || (g.I < 16 && g.J < 16 && g.R < 256)) {
-        if constexpr (std::is_same<T, float>::value)
-            if (prog_recording() && cdiv(outputs, GB) <= PROG_MAX_GRID && (size_t)g.R * outputs <= PROG_MAX_ELEMS)
-                prog_record(prog_kid(PF_GEMM_THREAD, 0), (unsigned)cdiv(outputs, GB), &g, sizeof(g));
+        if constexpr (std::is_same<T, float>::value) {
+            const bool small = cdiv(outputs, GB) <= PROG_MAX_GRID && (size_t)g.R * outputs <= PROG_MAX_ELEMS;
+            if (prog_recording() && !small) prog_abandon();
+            if (fuse_thread_dot(g, outputs)) return;
+            if (prog_recording()) prog_record(prog_kid(PF_GEMM_THREAD, 0), (unsigned)cdiv(outputs, GB), &g, sizeof(g));
+        }
         hipLaunchKernelGGL(gemm_thread_kernel<T>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_thread");
         return;
     }
     if (outputs <= 64 && g.R >= 4096) {
-        if constexpr (std::is_same<T, float>::value)
-            if (prog_recording() && (size_t)g.R * outputs <= PROG_MAX_ELEMS)
-                prog_record(prog_kid(PF_GEMM_BLOCKDOT, 0), (unsigned)outputs, &g, sizeof(g));
-        hipLaunchKernelGGL(gemm_blockdot_kernel<T>, dim3((unsigned)outputs), dim3(1024), 0, stream(), g);
+        const bool wide = blockdot_threads(g.R) == 1024;
+        if constexpr (std::is_same<T, float>::value) {
+            const bool small = (size_t)g.R * outputs <= PROG_MAX_ELEMS;
+            if (prog_recording() && !small) prog_abandon();
+            const bool rows = rowsdot_applies(g);        // [1,R] x [R,J]: one block, vector loads
+            if (!wide && fuse_block_dot(g, outputs, rows)) return;
+            if (rows) {
+                if (prog_recording()) prog_record(prog_kid(PF_GEMM_ROWSDOT, 0), 1, &g, sizeof(g));
+                hipLaunchKernelGGL(gemm_rowsdot_kernel, dim3(1), dim3(256), 0, stream(), g);
+                MXH_LAUNCH_CHECK("gemm_rowsdot");
+                return;
+            }
+            if (prog_recording()) prog_record(prog_kid(PF_GEMM_BLOCKDOT, 0), (unsigned)outputs, &g, sizeof(g));
+        }
+        if (wide) hipLaunchKernelGGL((gemm_blockdot_kernel<T, 1024>), dim3((unsigned)outputs), dim3(1024), 0, stream(), g);
+        else hipLaunchKernelGGL((gemm_blockdot_kernel<T, 256>), dim3((unsigned)outputs), dim3(256), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_blockdot");
         return;
     }

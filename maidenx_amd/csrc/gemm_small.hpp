@@ -2,6 +2,7 @@
 // the GEMM dispatch and by the interpreter of recorded programs.
 #pragma once
 #include "mxh.hpp"
+#include "reduce_row.hpp"
 
 namespace mxh {
 
@@ -62,33 +63,162 @@ template <class T>
 __global__ __launch_bounds__(GB) void gemm_thread_kernel(GemmArgs g) { gemm_thread_body<T>(g, blockIdx.x, threadIdx.x); }
 
 // One block per output element for a handful of outputs with a long reduction (the MLP's weight gradient:
-// 3 outputs of 10000 terms): threads stride over r, waves fold by shuffles, the block by LDS, in a fixed order.
-// `part`: 1024 / WAVE floats of LDS; every thread reaches the barrier.
-template <class T>
-__device__ __forceinline__ void gemm_blockdot_body(const GemmArgs& g, unsigned bid, unsigned tid, float* part) {
-    const size_t idx = bid;
+// 3 outputs of 10000 terms): NT threads stride over r, waves fold by a DPP butterfly, the block by LDS, in a fixed order.
+// `part`: NT / WAVE floats of LDS per output reduced side by side; every thread of the block reaches the barrier (threads at and beyond NT, which a
+// larger work-group may have, contribute nothing).  NT is a function of the reduction length alone, so that every path
+// that runs this body for a given product - the kernel below, a recorded program, the tail of a fused chain - adds in
+// the same order.
+constexpr uint32_t BLOCKDOT_WIDE_R = 32768;      // reductions from this length on use 1024 threads, shorter ones 256
+inline unsigned blockdot_threads(uint32_t R) { return R >= BLOCKDOT_WIDE_R ? 1024u : 256u; }
+// NO outputs (bid .. bid + NO - 1, those below `outputs`) are reduced side by side, and the loads of 8 terms of each
+// are in flight together: the terms of an output are still added in ascending r per thread.
+template <class T, int NT, int NO = 1>
+__device__ __forceinline__ void gemm_blockdot_body(const GemmArgs& g, unsigned bid, unsigned outputs, unsigned tid, float* part, float* mirror = nullptr) {
+    constexpr int U = 8;
     const size_t per = (size_t)g.I * g.J;
-    const uint32_t b = (uint32_t)(idx / per), rem = (uint32_t)(idx % per);
-    const uint32_t i = rem / g.J, j = rem % g.J;
-    const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
-    const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
-    float acc = 0.0f;
-    for (uint32_t r = tid; r < g.R; r += 1024) acc += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
+    const uint32_t R = g.R;
+    const int64_t xstep = (int64_t)NT * g.xr, ystep = (int64_t)NT * g.yr;      // pointers advance by additions only
+    const T* x[NO];
+    const T* y[NO];
+    float acc[NO];
+    bool live[NO];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, WAVE);
-    if (tid % WAVE == 0) part[tid / WAVE] = acc;
+    for (int o = 0; o < NO; ++o) {
+        live[o] = bid + o < outputs;
+        const size_t idx = live[o] ? bid + o : bid;
+        const uint32_t b = (uint32_t)(idx / per), rem = (uint32_t)(idx % per);
+        const uint32_t i = rem / g.J, j = rem % g.J;
+        x[o] = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi + (int64_t)tid * g.xr;
+        y[o] = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj + (int64_t)tid * g.yr;
+        acc[o] = 0.0f;
+    }
+    if (tid < (unsigned)NT) {
+        for (uint32_t r0 = tid; r0 < R; r0 += U * NT) {
+            float p[NO][U];
+#pragma unroll
+            for (int o = 0; o < NO; ++o) {
+                if (!live[o]) continue;                      // uniform over the work-group
+                const T* xp = x[o];
+                const T* yp = y[o];
+#pragma unroll
+                for (int k = 0; k < U; ++k) {
+                    // steps past the end re-read the step before (an unconditional load; its product is not added)
+                    p[o][k] = Elem<T>::ld(*xp) * Elem<T>::ld(*yp);
+                    if (r0 + (k + 1) * NT < R) { xp += xstep; yp += ystep; }
+                }
+                x[o] += U * xstep;
+                y[o] += U * ystep;
+            }
+#pragma unroll
+            for (int o = 0; o < NO; ++o) {
+                if (!live[o]) continue;
+#pragma unroll
+                for (int k = 0; k < U; ++k)
+                    if (r0 + k * NT < R) acc[o] += p[o][k];
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < NO; ++o) {
+            acc[o] = wave_reduce<RSum>(acc[o]);      // the butterfly on DPP: a dozen instructions, no trips through LDS
+            if (tid % WAVE == 0) part[o * (NT / WAVE) + tid / WAVE] = acc[o];
+        }
+    }
     __syncthreads();
-    if (tid == 0) {
+    if (tid < (unsigned)NO && bid + tid < outputs) {
         float sum = 0.0f;
 #pragma unroll
-        for (int w = 0; w < 1024 / WAVE; ++w) sum += part[w];
-        ((T*)g.out)[idx] = Elem<T>::st(sum);
+        for (int w = 0; w < NT / WAVE; ++w) sum += part[tid * (NT / WAVE) + w];
+        ((T*)g.out)[bid + tid] = Elem<T>::st(sum);
+        if (mirror) mirror[bid + tid] = sum;      // LDS copy of the results for the caller's later stages
     }
 }
-template <class T>
-__global__ __launch_bounds__(1024) void gemm_blockdot_kernel(GemmArgs g) {
-    __shared__ float part[1024 / WAVE];
-    gemm_blockdot_body<T>(g, blockIdx.x, threadIdx.x, part);
+// out[j] = sum over r of X[r] * Y[r, j] for a contiguous f32 X and a row-major Y of J <= 4 columns: the weight gradient of a
+// layer with one output feature ([1,R] x [R,J]).  One block does all J outputs.  Thread t owns rows 4t .. 4t+3 of every
+// 4 * NT rows, so one 16-byte load brings four terms of X and J of them the 4 * J matching terms of Y (the strided form
+// above needs 4 + 4 * J scalar loads for the same terms); the loads of ten such groups are in flight together.  A thread
+// adds the terms of an output in ascending r; waves fold by a DPP butterfly, the block by LDS, in a fixed order.
+// `part`: J * NT / WAVE floats of LDS.
+// The same with the operands' roles exchanged ([J,R] x [R,1] with a column-major left operand: what matmul_backward asks
+// for as A^T . dC) is the same sum, a product of two floats not depending on their order: rowsdot_normalise() turns it
+// into the first form.
+__host__ __device__ inline bool rowsdot_normalise(GemmArgs& g) {
+    if (g.batch != 1 || g.R % 4 != 0 || g.R < 4096 || g.R >= BLOCKDOT_WIDE_R) return false;
+    if (g.J == 1 && g.I >= 1 && g.I <= 4 && g.xi == 1 && g.xr == (int64_t)g.I && g.yr == 1) {
+        // out[i] = sum_r X[r, i] * Y[r]: X is the row-major matrix, Y the vector
+        const void* m = g.X;
+        g.X = g.Y;
+        g.Y = m;
+        g.J = g.I;
+        g.I = 1;
+        g.xr = 1;
+        g.yr = (int64_t)g.J;
+        g.yj = 1;
+    }
+    return g.I == 1 && g.J >= 1 && g.J <= 4 && g.yj == 1 && g.yr == (int64_t)g.J && g.xr == 1 && ((uintptr_t)g.X % 16) == 0 &&
+           ((uintptr_t)g.Y % 16) == 0;
+}
+inline bool rowsdot_applies(const GemmArgs& g) {
+    GemmArgs n = g;
+    return rowsdot_normalise(n);
+}
+template <int NT, int J>
+__device__ __forceinline__ void gemm_rowsdot_body(const GemmArgs& g, unsigned tid, float* part, float* mirror = nullptr) {
+    constexpr int G = 10;     // 10 * (1 + J) 16-byte loads in flight per thread: a 10240-row product in one round trip
+    typedef float F4 __attribute__((ext_vector_type(4)));
+    const F4* X4 = (const F4*)g.X;
+    const F4* Y4 = (const F4*)g.Y;
+    const uint32_t groups = g.R / 4;
+    float acc[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) acc[j] = 0.0f;
+    if (tid < (unsigned)NT) {
+        for (uint32_t q0 = tid; q0 < groups; q0 += G * NT) {
+            F4 xv[G];
+            F4 yv[G][J];
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const uint32_t q = q0 + i * NT < groups ? q0 + i * NT : q0;      // past the end: re-read the first (not added)
+                xv[i] = X4[q];
+#pragma unroll
+                for (int jj = 0; jj < J; ++jj) yv[i][jj] = Y4[(size_t)q * J + jj];
+            }
+#pragma unroll
+            for (int i = 0; i < G; ++i)
+                if (q0 + i * NT < groups) {
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+                        for (int j = 0; j < J; ++j) acc[j] += xv[i][rr] * yv[i][(rr * J + j) / 4][(rr * J + j) % 4];
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            acc[j] = wave_reduce<RSum>(acc[j]);
+            if (tid % WAVE == 0) part[j * (NT / WAVE) + tid / WAVE] = acc[j];
+        }
+    }
+    __syncthreads();
+    if (tid < (unsigned)J) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NT / WAVE; ++w) sum += part[tid * (NT / WAVE) + w];
+        ((float*)g.out)[tid] = sum;
+        if (mirror) mirror[tid] = sum;
+    }
+}
+template <int NT>
+__device__ __forceinline__ void gemm_rowsdot_any(const GemmArgs& args, unsigned tid, float* part, float* mirror = nullptr) {
+    GemmArgs g = args;
+    rowsdot_normalise(g);
+    if (g.J == 1) gemm_rowsdot_body<NT, 1>(g, tid, part, mirror);
+    else if (g.J == 2) gemm_rowsdot_body<NT, 2>(g, tid, part, mirror);
+    else if (g.J == 3) gemm_rowsdot_body<NT, 3>(g, tid, part, mirror);
+    else gemm_rowsdot_body<NT, 4>(g, tid, part, mirror);
+}
+template <class T, int NT>
+__global__ __launch_bounds__(NT) void gemm_blockdot_kernel(GemmArgs g) {
+    __shared__ float part[NT / WAVE];
+    gemm_blockdot_body<T, NT>(g, blockIdx.x, gridDim.x, threadIdx.x, part);
 }
 
 }  // namespace mxh

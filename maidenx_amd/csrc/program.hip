@@ -99,11 +99,14 @@ __global__ __launch_bounds__(PROG_THREADS) void program_kernel(const ProgCmd* cm
             const GemmArgs g = load_args<GemmArgs>(c);
             const unsigned grid = c->grid;
             for (unsigned b0 = 0; b0 < grid; b0 += PROG_THREADS / GB) gemm_thread_body<float>(g, b0 + tid / GB, tid % GB);
+        } else if (family == PF_GEMM_ROWSDOT) {
+            const GemmArgs g = load_args<GemmArgs>(c);
+            gemm_rowsdot_any<256>(g, tid, lds);
         } else if (family == PF_GEMM_BLOCKDOT) {
             const GemmArgs g = load_args<GemmArgs>(c);
             const unsigned grid = c->grid;
             for (unsigned b = 0; b < grid; ++b) {
-                gemm_blockdot_body<float>(g, b, tid, lds);
+                gemm_blockdot_body<float, 256>(g, b, grid, tid, lds);      // a program command reads at most PROG_MAX_ELEMS: the short form
                 __syncthreads();
             }
         }

@@ -31,7 +31,7 @@ struct alignas(16) ProgCmd {
 };
 static_assert(sizeof(ProgCmd) == 512, "one command is 512 bytes");
 
-enum ProgFamily : uint32_t { PF_EW = 1, PF_ROW_REDUCE = 2, PF_GEMM_THREAD = 3, PF_GEMM_BLOCKDOT = 4 };
+enum ProgFamily : uint32_t { PF_EW = 1, PF_ROW_REDUCE = 2, PF_GEMM_THREAD = 3, PF_GEMM_BLOCKDOT = 4, PF_GEMM_ROWSDOT = 5 };
 inline uint32_t prog_kid(uint32_t family, uint32_t sub) { return (family << 16) | sub; }
 
 // Host side (runtime.hip).  prog_recording(): a capture is open and still replayable by the interpreter.

@@ -247,12 +247,21 @@ void launch_row(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks
     unsigned blocks = cdiv(rows * chunks, RPB);
     bool vec = aligned16(in) && L % VEC == 0 && chunk_len % VEC == 0;
     if constexpr (std::is_same<TIn, float>::value && std::is_same<TOut, float>::value) {
-        if (prog_recording() && blocks <= PROG_MAX_GRID && rows * L <= PROG_MAX_ELEMS) {
-            RowProgArgs a;
-            std::memset((void*)&a, 0, sizeof(a));
-            a.in = in; a.out = out; a.rows = rows; a.L = L; a.chunks = chunks; a.chunk_len = chunk_len; a.div = div; a.src_bf16 = src_bf16;
-            prog_record(prog_kid(PF_ROW_REDUCE, row_prog_sub<R, TPR>(vec ? 1 : 0)), blocks, &a, sizeof(a));
+        RowProgArgs a;
+        std::memset((void*)&a, 0, sizeof(a));
+        a.in = in; a.out = out; a.rows = rows; a.L = L; a.chunks = chunks; a.chunk_len = chunk_len; a.div = div; a.src_bf16 = src_bf16;
+        const bool small = blocks <= PROG_MAX_GRID && rows * L <= PROG_MAX_ELEMS;
+        if (prog_recording() && !small) prog_abandon();
+        if constexpr (std::is_same<R, RSum>::value) {
+            // a sum that one work-group does anyway: a stage in the tail of the open chain of fused launches
+            static_assert(sizeof(RowProgArgs) <= FUSE_TAIL_ARG_BYTES, "a tail stage holds a row reduction's arguments");
+            if (capture_open() && blocks == 1 && rows * L <= 65536) {
+                const Extent src{(uintptr_t)in, (uintptr_t)in + rows * L * sizeof(float)};
+                const Extent dst{(uintptr_t)out, (uintptr_t)out + rows * chunks * sizeof(float)};
+                if (fuse_record_tail(TAIL_ROW_REDUCE, row_prog_sub<R, TPR>(vec ? 1 : 0), &a, sizeof(a), &src, 1, dst, rows * chunks)) return;
+            }
         }
+        if (prog_recording() && small) prog_record(prog_kid(PF_ROW_REDUCE, row_prog_sub<R, TPR>(vec ? 1 : 0)), blocks, &a, sizeof(a));
     }
     if (vec && streams(rows * L * sizeof(TIn)))
         hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, TPR, VEC, true>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows,

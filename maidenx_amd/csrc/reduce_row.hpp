@@ -77,10 +77,12 @@ constexpr int RB = 256;
 // and a 16-byte aligned base.
 // Block and thread index are arguments (the interpreter of recorded programs passes virtual ones); `part`
 // is RB / WAVE floats of LDS owned by this (virtual) block.  Every thread reaches the barrier.
-template <class TIn, class TOut, class R, int TPR, int VEC, bool STREAM = false>
+// BATCH > 0: the loads of BATCH steps are in flight together whatever the row length (steps past the end are skipped),
+// for callers that run a single work-group and pay every memory latency in full; the adds keep the order.
+template <class TIn, class TOut, class R, int TPR, int VEC, bool STREAM = false, int BATCH = 0>
 __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut* __restrict__ out, size_t rows, size_t L,
                                                 unsigned chunks, size_t chunk_len, float div, bool src_bf16, unsigned bid,
-                                                unsigned tid, float* part) {
+                                                unsigned tid, float* part, float* mirror = nullptr) {
     constexpr int RPB = RB / TPR;
     size_t unit = (size_t)bid * RPB + tid / TPR;   // (row, chunk) pair
     const unsigned t = tid % TPR;
@@ -97,6 +99,19 @@ __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut
             // four loads in flight per lane; the adds keep the order of the plain loop
             constexpr size_t STEP = (size_t)TPR * VEC;
             size_t i = beg + (size_t)t * VEC;
+            if constexpr (BATCH > 0) {
+                for (; i < end; i += BATCH * STEP) {
+                    AVec<TIn, VEC> v[BATCH];
+#pragma unroll
+                    for (int k = 0; k < BATCH; ++k)      // steps past the end re-read the first (an unconditional load, not added)
+                        v[k] = *(const AVec<TIn, VEC>*)(src + (i + k * STEP < end ? i + k * STEP : i));
+#pragma unroll
+                    for (int k = 0; k < BATCH; ++k)
+                        if (i + k * STEP < end)
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) a[e] = R::op(a[e], IO<TIn>::ld(v[k].v[e]));
+                }
+            }
             for (; i + 3 * STEP < end; i += 4 * STEP) {
                 AVec<TIn, VEC> v[4];
 #pragma unroll
@@ -113,6 +128,15 @@ __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut
             }
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc = R::op(acc, a[e]);
+        } else if constexpr (BATCH > 0) {
+            for (size_t i = beg + t; i < end; i += (size_t)BATCH * TPR) {
+                TIn v[BATCH];
+#pragma unroll
+                for (int k = 0; k < BATCH; ++k) v[k] = src[i + (size_t)k * TPR < end ? i + (size_t)k * TPR : i];
+#pragma unroll
+                for (int k = 0; k < BATCH; ++k)
+                    if (i + (size_t)k * TPR < end) acc = R::op(acc, IO<TIn>::ld(v[k]));
+            }
         } else {
             for (size_t i = beg + t; i < end; i += TPR) acc = R::op(acc, IO<TIn>::ld(src[i]));
         }
@@ -125,7 +149,12 @@ __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut
 #pragma unroll
         for (int w = 1; w < RB / WAVE; ++w) acc = R::op(acc, part[w]);
     }
-    if (t == 0 && unit < total) out[unit] = IO<TOut>::fin(acc, div);
+    if (t == 0 && unit < total) {
+        const TOut res = IO<TOut>::fin(acc, div);
+        out[unit] = res;
+        if constexpr (std::is_same<TOut, float>::value)
+            if (mirror) mirror[unit] = res;      // LDS copy of the results for the caller's later stages
+    }
 }
 template <class TIn, class TOut, class R, int TPR, int VEC, bool STREAM = false>
 __global__ __launch_bounds__(RB) void row_reduce_kernel(const TIn* __restrict__ in, TOut* __restrict__ out, size_t rows,

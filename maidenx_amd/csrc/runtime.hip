@@ -67,26 +67,51 @@ ApiGuard::ApiGuard() : ok(true) {
 }
 ApiGuard::~ApiGuard() { g_api_mu.unlock(); }
 
+// ---- the open chain of fused launches (see fuse.hpp) ----------------------------------------------------------
+// What the recorded members read and write, for the checks a newcomer has to pass.
+struct ParMember {
+    Extent out, in[2];
+    bool across[2];           // input j is read across threads (a matmul operand): it can never be "the same mapping"
+};
+struct TailStage {
+    Extent out, in[2];
+    int nin;
+    bool late[2];             // input j is read from memory when the stage runs (not fetched when the tail starts, not from a mirror)
+    bool mirrored;            // the outputs are also kept in LDS
+};
+static ParMember g_par[FUSE_MAX_CMDS];
+static TailStage g_tail[FUSE_MAX_TAIL];
+static uint32_t g_lds_from = 0, g_mem_from = 0;      // first tail stage not yet ordered by a barrier (of LDS / that waits for memory)
+static uint32_t* g_tickets[16] = {nullptr};       // per device: the ticket slots of fuse.hip
+static bool g_tickets_ready = false;              // ... known for the device of the open capture
+static uint32_t g_next_ticket = 0;
+
 static void fuse_flush() {
-    if (g_fuse.n == 0) return;
+    if (g_fuse.n == 0 && g_fuse.ntail == 0) return;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    // Chains queued on one stream run one after the other, and each leaves its ticket at zero, so sharing would do;
+    // rotating over the slots keeps two captures that a caller replays on two streams at once apart as well.
+    g_fuse.ticket = g_tickets[dev] + (g_next_ticket++ % FUSE_TICKETS);
     fuse_launch(g_fuse, (void*)g_capture_stream);
     ++g_fuse_nodes;
     g_fuse.n = 0;
+    g_fuse.ntail = 0;
+    g_lds_from = g_mem_from = 0;
 }
 
-// Every launch and copy of the library asks for the stream right before it queues something: an open group of fused
+// Every launch and copy of the library asks for the stream right before it queues something: an open chain of fused
 // launches has to run before that.
 hipStream_t stream() {
-    if (g_capturing && g_fuse.n) fuse_flush();
+    if (g_capturing && (g_fuse.n || g_fuse.ntail)) fuse_flush();
     return g_stream;
 }
 
 // byte range an operand touches
-static void operand_range(const void* base, const int64_t* strides, uint32_t ndims, const uint32_t* dims, size_t esz, uintptr_t& lo, uintptr_t& hi) {
+static Extent operand_range(const void* base, const int64_t* strides, uint32_t ndims, const uint32_t* dims, size_t esz) {
     size_t span = 0;
     for (uint32_t d = 0; d < ndims; ++d) span += (size_t)(dims[d] - 1) * (size_t)strides[d];
-    lo = (uintptr_t)base;
-    hi = lo + (span + 1) * esz;
+    return Extent{(uintptr_t)base, (uintptr_t)base + (span + 1) * esz};
 }
 static bool same_mapping(const void* a, const int64_t* sa, const void* b, const int64_t* sb, uint32_t ndims) {
     if (a != b) return false;
@@ -94,88 +119,202 @@ static bool same_mapping(const void* a, const int64_t* sa, const void* b, const 
         if (sa[d] != sb[d]) return false;
     return true;
 }
+static bool fuse_accepting() { return g_capturing && g_fuse_enabled && !g_prog_ok && g_tickets_ready; }
 
-bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
-    // only once the capture cannot be a whole-capture program any more (that path launches for real)
-    if (!g_capturing || !g_fuse_enabled || g_prog_ok || ndims < 1 || ndims > 2) return false;
-    for (uint32_t d = 0; d < ndims; ++d)
-        if (c.os[d] < 0 || c.is[0][d] < 0 || (c.nin > 1 && c.is[1][d] < 0)) return false;
-    // at most one block's worth of elements, one per thread: such members form groups of their own, in which a barrier
-    // between members orders everything (any shapes, any overlaps)
-    size_t nel = 1;
-    for (uint32_t d = 0; d < ndims; ++d) nel *= dims[d];
-    const bool tiny = nel <= 256;
-    if (tiny) {
-        if (!(g_fuse.n > 0 && g_fuse.tiny && g_fuse.n < (uint32_t)FUSE_MAX_CMDS)) {
-            fuse_flush();
-            g_fuse.tiny = 1;
-            g_fuse.vec = 0;
-            g_fuse.ndims = 1;
-            g_fuse.nvec = 256;
-            g_fuse.dims[0] = 256;
-            g_fuse.dims[1] = 1;
-            g_fuse.div_inner = make_fastdiv(1);
-            g_fuse_elem_bytes = elem_bytes;
-        }
-        FuseCmd& slot = g_fuse.cmd[g_fuse.n++];
-        slot = c;
-        slot.fwd = 0;            // the forwarded registers belong to another member's thread layout
-        slot.ndims = ndims;
-        slot.dims[0] = dims[0];
-        slot.dims[1] = ndims == 2 ? dims[1] : 1;
-        slot.nel = (uint32_t)nel;
-        ++g_fused_launches;
-        return true;
+// A newcomer to the parallel phase against the tail stages already queued: it runs before them, so it may not read
+// what they write nor write what they read or write.
+static bool clear_of_tail(const ParMember& m, uint32_t nin) {
+    for (uint32_t k = 0; k < g_fuse.ntail; ++k) {
+        const TailStage& t = g_tail[k];
+        if (m.out.overlaps(t.out)) return false;
+        for (int j = 0; j < t.nin; ++j)
+            if (m.out.overlaps(t.in[j])) return false;
+        for (uint32_t j = 0; j < nin; ++j)
+            if (m.in[j].overlaps(t.out)) return false;
     }
-    if (g_fuse.n > 0 && g_fuse.tiny) fuse_flush();
-    const bool fits = g_fuse.n > 0 && g_fuse.n < (uint32_t)FUSE_MAX_CMDS && g_fuse.ndims == ndims && g_fuse.vec == (vec ? 1u : 0u) &&
-                      g_fuse.nvec == nvec && g_fuse.dims[0] == dims[0] && (ndims == 1 || g_fuse.dims[1] == dims[1]) && g_fuse_elem_bytes == elem_bytes;
-    bool join = fits;
-    if (join) {
-        // every overlap with an earlier member must be element for element, so that a thread only meets its own data
-        uintptr_t olo, ohi;
-        operand_range(c.out, c.os, ndims, dims, elem_bytes, olo, ohi);
-        for (uint32_t k = 0; k < g_fuse.n && join; ++k) {
-            const FuseCmd& e = g_fuse.cmd[k];
-            uintptr_t lo, hi;
-            operand_range(e.out, e.os, ndims, dims, elem_bytes, lo, hi);
-            // read after write, and write after write
-            for (uint32_t j = 0; j < c.nin && join; ++j) {
-                uintptr_t ilo, ihi;
-                operand_range(c.in[j], c.is[j], ndims, dims, elem_bytes, ilo, ihi);
-                if (ilo < hi && lo < ihi && !same_mapping(c.in[j], c.is[j], e.out, e.os, ndims)) join = false;
-            }
-            if (olo < hi && lo < ohi && !same_mapping(c.out, c.os, e.out, e.os, ndims)) join = false;
-            // write after read
-            for (uint32_t j = 0; j < e.nin && join; ++j) {
-                uintptr_t ilo, ihi;
-                operand_range(e.in[j], e.is[j], ndims, dims, elem_bytes, ilo, ihi);
-                if (olo < ihi && ilo < ohi && !same_mapping(c.out, c.os, e.in[j], e.is[j], ndims)) join = false;
-            }
-        }
+    return true;
+}
+// ... and against the earlier members of the parallel phase: every overlap must be element for element, so that a
+// thread only meets its own data.
+static bool clear_of_members(const FuseCmd& c, const ParMember& m, uint32_t ndims) {
+    for (uint32_t k = 0; k < g_fuse.n; ++k) {
+        const FuseCmd& e = g_fuse.cmd[k];
+        const ParMember& pe = g_par[k];
+        // read after write
+        for (uint32_t j = 0; j < c.nin; ++j)
+            if (m.in[j].overlaps(pe.out) && (m.across[j] || !same_mapping(c.in[j], c.is[j], e.out, e.os, ndims))) return false;
+        // write after write
+        if (m.out.overlaps(pe.out) && !same_mapping(c.out, c.os, e.out, e.os, ndims)) return false;
+        // write after read
+        for (uint32_t j = 0; j < e.nin; ++j)
+            if (m.out.overlaps(pe.in[j]) && (pe.across[j] || !same_mapping(c.out, c.os, e.in[j], e.is[j], ndims))) return false;
     }
-    if (!join) {
-        fuse_flush();
-        g_fuse.tiny = 0;
-        g_fuse.ndims = ndims;
-        g_fuse.vec = vec ? 1u : 0u;
-        g_fuse.nvec = nvec;
-        g_fuse.dims[0] = dims[0];
-        g_fuse.dims[1] = ndims == 2 ? dims[1] : 1;
-        g_fuse.div_inner = make_fastdiv(g_fuse.dims[ndims - 1]);
-        g_fuse_elem_bytes = elem_bytes;
-    }
+    return true;
+}
+static void open_space(uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
+    g_fuse.ndims = ndims;
+    g_fuse.vec = vec ? 1u : 0u;
+    g_fuse.nvec = nvec;
+    g_fuse.dims[0] = dims[0];
+    g_fuse.dims[1] = ndims == 2 ? dims[1] : 1;
+    g_fuse.div_inner = make_fastdiv(g_fuse.dims[ndims - 1]);
+    g_fuse_elem_bytes = elem_bytes;
+}
+// Adds a member to the parallel phase (joining the open chain when it may, closing it and opening a new one otherwise).
+static void add_member(const FuseCmd& c, const ParMember& m, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
+    bool join = (g_fuse.n > 0 || g_fuse.ntail > 0) && g_fuse.n < (uint32_t)FUSE_MAX_CMDS;
+    if (join && g_fuse.n > 0)
+        join = g_fuse.ndims == ndims && g_fuse.vec == (vec ? 1u : 0u) && g_fuse.nvec == nvec && g_fuse.dims[0] == dims[0] &&
+               (ndims == 1 || g_fuse.dims[1] == dims[1]) && g_fuse_elem_bytes == elem_bytes;
+    if (join) join = clear_of_members(c, m, ndims) && clear_of_tail(m, c.nin);
+    if (!join) fuse_flush();
+    if (g_fuse.n == 0) open_space(ndims, dims, vec, nvec, elem_bytes);
     FuseCmd& slot = g_fuse.cmd[g_fuse.n];
     slot = c;
     slot.fwd = 0;
-    if (g_fuse.n > 0) {
-        const FuseCmd& prev = g_fuse.cmd[g_fuse.n - 1];
+    slot.src = FUSE_SRC_MEMORY | (FUSE_SRC_MEMORY << 8);
+    if (c.op != FUSE_OP_DOT) {
+        // An input that is an earlier member's output (element for element: nothing else was let in) is not in memory yet:
+        // the members' stores wait until all of them are done.  It comes from the latest such member's staged output,
+        // or straight from registers when that is the member before.
         for (uint32_t j = 0; j < c.nin; ++j)
-            if (same_mapping(c.in[j], c.is[j], prev.out, prev.os, ndims)) slot.fwd |= 1u << j;
+            for (int k = (int)g_fuse.n - 1; k >= 0; --k) {
+                const FuseCmd& e = g_fuse.cmd[k];
+                if (!m.in[j].overlaps(g_par[k].out)) continue;
+                if ((uint32_t)k + 1 == g_fuse.n) slot.fwd |= 1u << j;
+                slot.src = (slot.src & ~(0xFFu << (8 * j))) | ((uint32_t)k << (8 * j));
+                (void)e;
+                break;
+            }
     }
+    g_par[g_fuse.n] = m;
     ++g_fuse.n;
     ++g_fused_launches;
+}
+
+static bool tail_same_thread(const FuseCmd* a, const void* pa, const int64_t* sa, const FuseCmd* b, const void* pb, const int64_t* sb) {
+    // thread v owns element v of a stage's own space: two operands are one thread's when the spaces and the mappings agree
+    return a && b && a->ndims == b->ndims && a->dims[0] == b->dims[0] && a->dims[1] == b->dims[1] && same_mapping(pa, sa, pb, sb, a->ndims);
+}
+
+bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs) {
+    if (!fuse_accepting() || arg_bytes > (size_t)FUSE_TAIL_ARG_BYTES || nin > 2) return false;
+    if (g_fuse.ntail >= (uint32_t)FUSE_MAX_TAIL) fuse_flush();
+    const uint32_t at = g_fuse.ntail;
+    if (at == 0) g_fuse.prefetch = 0;
+    TailCmd& t = g_fuse.tail[at];
+    std::memset((void*)&t, 0, sizeof(t));
+    t.kind = kind;
+    t.sub = sub;
+    std::memcpy(t.arg, arg, arg_bytes);
+    TailStage& st = g_tail[at];
+    st.out = out;
+    st.nin = nin;
+    for (int j = 0; j < 2; ++j) {
+        st.in[j] = j < nin ? in[j] : Extent{0, 0};
+        st.late[j] = false;
+    }
+    FuseCmd* c = kind == TAIL_EW ? (FuseCmd*)t.arg : nullptr;
+    auto stage_cmd = [&](uint32_t k) { return g_fuse.tail[k].kind == TAIL_EW ? (const FuseCmd*)g_fuse.tail[k].arg : (const FuseCmd*)nullptr; };
+    // Stages run in order, but by 256 threads that only meet at barriers.  Work out where each input comes from and
+    // which barrier, if any, the stage needs first.
+    uint32_t sync = 0;
+    if (c) {
+        c->src = 0;
+        st.mirrored = c->os[c->ndims - 1] == 1 && (c->ndims == 1 || c->os[0] == (int64_t)c->dims[1]);
+        for (int j = 0; j < nin; ++j) {
+            int writer = -1;                            // the latest earlier stage that writes some of this input
+            for (int k = (int)at - 1; k >= 0 && writer < 0; --k)
+                if (st.in[j].overlaps(g_tail[k].out)) writer = k;
+            uint32_t from = FUSE_SRC_MEMORY;
+            if (writer >= 0) {
+                const TailStage& w = g_tail[writer];
+                const FuseCmd* wc = stage_cmd((uint32_t)writer);
+                const bool own = tail_same_thread(c, c->in[j], c->is[j], wc, wc ? wc->out : nullptr, wc ? wc->os : nullptr);
+                if (w.mirrored && st.in[j].lo >= w.out.lo && st.in[j].hi <= w.out.hi) {
+                    from = (uint32_t)writer;
+                    t.moff[j] = (int32_t)((st.in[j].lo - w.out.lo) / sizeof(float));
+                    if (own && (uint32_t)writer + 1 == at) t.fwd |= 1u << j;
+                    if (!own && (uint32_t)writer >= g_lds_from && sync < 1) sync = 1;
+                } else {
+                    from = FUSE_SRC_MEMORY_LATE;
+                    st.late[j] = true;
+                    if (!own && (uint32_t)writer >= g_mem_from) sync = 2;
+                }
+            }
+            c->src |= from << (8 * j);
+            if (from == FUSE_SRC_MEMORY) g_fuse.prefetch |= 1u << (2 * at + j);
+        }
+    } else {
+        st.mirrored = outputs <= 256;
+        for (int j = 0; j < nin; ++j) {
+            st.late[j] = true;
+            for (uint32_t k = g_mem_from; k < at; ++k)
+                if (st.in[j].overlaps(g_tail[k].out)) sync = 2;
+        }
+        if (at > 0 && sync < 1) sync = 1;               // the fold's LDS is reused from stage to stage
+    }
+    // what the stage writes against what unordered earlier stages wrote, or read late, through other threads
+    for (uint32_t k = g_mem_from; k < at && sync < 2; ++k) {
+        const TailStage& e = g_tail[k];
+        const FuseCmd* ec = stage_cmd(k);
+        if (st.out.overlaps(e.out) && !tail_same_thread(c, c ? c->out : nullptr, c ? c->os : nullptr, ec, ec ? ec->out : nullptr, ec ? ec->os : nullptr)) sync = 2;
+        for (int j = 0; j < e.nin && sync < 2; ++j)
+            if (e.late[j] && st.out.overlaps(e.in[j]) &&
+                !tail_same_thread(c, c ? c->out : nullptr, c ? c->os : nullptr, ec, ec ? ec->in[j] : nullptr, ec ? ec->is[j] : nullptr)) sync = 2;
+    }
+    t.sync = sync;
+    t.mirrored = st.mirrored ? 1u : 0u;
+    if (sync >= 1) g_lds_from = at;
+    if (sync == 2) g_mem_from = at;
+    ++g_fuse.ntail;
+    ++g_fused_launches;
     return true;
+}
+
+bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
+    // only once the capture cannot be a whole-capture program any more (that path launches for real)
+    if (!fuse_accepting() || ndims < 1 || ndims > 2) return false;
+    for (uint32_t d = 0; d < ndims; ++d)
+        if (c.os[d] < 0 || c.is[0][d] < 0 || (c.nin > 1 && c.is[1][d] < 0)) return false;
+    ParMember m;
+    m.out = operand_range(c.out, c.os, ndims, dims, elem_bytes);
+    for (uint32_t j = 0; j < 2; ++j) {
+        m.in[j] = j < c.nin ? operand_range(c.in[j], c.is[j], ndims, dims, elem_bytes) : Extent{0, 0};
+        m.across[j] = false;
+    }
+    // at most one block's worth of elements, one per thread: a stage of the tail, where a barrier between stages
+    // orders everything (any shapes, any overlaps)
+    size_t nel = 1;
+    for (uint32_t d = 0; d < ndims; ++d) nel *= dims[d];
+    if (nel <= 256) {
+        FuseCmd t = c;
+        t.fwd = 0;
+        t.ndims = ndims;
+        t.dims[0] = dims[0];
+        t.dims[1] = ndims == 2 ? dims[1] : 1;
+        t.nel = (uint32_t)nel;
+        return fuse_record_tail(TAIL_EW, 0, &t, sizeof(t), m.in, (int)c.nin, m.out, nel);
+    }
+    add_member(c, m, ndims, dims, vec, nvec, elem_bytes);
+    return true;
+}
+
+bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y) {
+    if (!fuse_accepting() || outputs <= 256) return false;
+    ParMember m;
+    m.out = Extent{(uintptr_t)c.out, (uintptr_t)c.out + outputs * sizeof(float)};
+    m.in[0] = x;
+    m.in[1] = y;
+    m.across[0] = m.across[1] = true;
+    const bool vec = outputs % 4 == 0 && (uintptr_t)c.out % 16 == 0;
+    const uint32_t dims[1] = {(uint32_t)outputs};
+    add_member(c, m, 1, dims, vec, vec ? outputs / 4 : outputs, sizeof(float));
+    return true;
+}
+
+void prog_abandon() {
+    if (g_capturing) g_prog_ok = false;
 }
 
 bool capture_open() { return g_capturing; }
@@ -363,6 +502,13 @@ int hip_graph_begin_capture(void) {
         e = hipStreamCreate(&g_capture_stream);
         if (e != hipSuccess) return (int)e;
     }
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    g_tickets_ready = false;
+    if (dev >= 0 && dev < 16) {
+        if (!g_tickets[dev]) g_tickets[dev] = fuse_tickets();
+        g_tickets_ready = g_tickets[dev] != nullptr;
+    }
     e = hipStreamBeginCapture(g_capture_stream, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return (int)e;
     g_saved_stream = g_stream;
@@ -373,6 +519,8 @@ int hip_graph_begin_capture(void) {
     g_prog_pending = false;
     g_prog_cmds.clear();
     g_fuse.n = 0;
+    g_fuse.ntail = 0;
+    g_lds_from = g_mem_from = 0;
     g_fused_launches = g_fuse_nodes = 0;
     return 0;
 }

@@ -239,9 +239,9 @@ def fused(lib, seq, want_launches=None, want_nodes=None, replays=2):
     seq.run()
     eager = seq.read()
     assert lib.hip_get_last_status() == 0, lib.hip_status_string()
-    big = L.DeviceBuffer(1 << 20)
+    big = L.DeviceBuffer(1 << 23)
     assert lib.hip_graph_begin_capture() == 0
-    lib.hip_fill_f32((1 << 20) // 4, big.ptr, C.c_float(0.0))        # too large for a program command
+    lib.hip_fill_f32((1 << 23) // 4, big.ptr, C.c_float(0.0))        # too large for a program command, and for a fused chain
     seq.run()
     h = C.c_void_p()
     assert lib.hip_graph_end_capture(C.byref(h)) == 0
@@ -338,6 +338,94 @@ def test_fused_tiny_members_of_any_shape_share_one_block(lib):
     seq.add("sub_inplace_f32", 3, 1, u64([3], [1], [1], 0, 0), gw.ptr, w.ptr)
     seq.add("add_f32", 3, 1, u64([3], [1], [0], 0, 0), gw.ptr, gb.ptr, t4.ptr)
     fused(lib, seq, want_launches=7, want_nodes=1)
+
+
+def linear_step(lib, seq, n, feats, r):
+    """One training step of Linear(feats -> 1) + MSE + SGD spelled out in backend calls: a one-thread-per-output matmul,
+    elementwise members over [n], a row reduction to a scalar, scalar stages, the weight gradient as a long-reduction
+    matmul ([feats, n] x [n, 1], the left operand a transposed view) and the parameter updates."""
+    x, y = seq.dev(r.standard_normal((n, feats)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    w, b = seq.dev(r.standard_normal(feats).astype(np.float32)), seq.dev(r.standard_normal(1).astype(np.float32))
+    pred, pb, diff, sq = (seq.out(n * 4, "f4") for _ in range(4))
+    loss, lossn, scale = seq.out(4, "f4"), seq.out(4, "f4"), seq.out(4, "f4")
+    gpred, gx = seq.out(n * 4, "f4"), seq.out(n * feats * 4, "f4")
+    gw, gb, wstep, bstep, wnew, bnew = (seq.out(k * 4, "f4") for k in (feats, 1, feats, 1, feats, 1))
+    md1, md2 = u64([n], [1], 0), u64([n], [1], [1], 0, 0)
+    # forward: x [n, feats] . w^T [feats, 1]
+    seq.add("matmul_f32", n, u64(2, 2, 2, [n, 1], [n, feats], [feats, 1], [feats, 1], [1, feats], 0, 0), x.ptr, w.ptr, pred.ptr)
+    seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), pred.ptr, b.ptr, pb.ptr)
+    seq.add("sub_f32", n, 1, md2, pb.ptr, y.ptr, diff.ptr)
+    seq.add("square_f32", n, 1, md1, diff.ptr, sq.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), sq.ptr, loss.ptr)
+    seq.add("div_scalar_f32", 1, 1, u64([1], [1], 0), loss.ptr, C.c_float(n), lossn.ptr)
+    seq.add("fill_f32", 1, scale.ptr, C.c_float(2.0 / n))
+    # backward: d loss / d pred, then the input gradient [n, 1] x [1, feats] (one term per output) ...
+    seq.add("mul_f32", n, 1, u64([n], [1], [0], 0, 0), diff.ptr, scale.ptr, gpred.ptr)
+    seq.add("matmul_f32", n * feats, u64(2, 2, 2, [n, feats], [n, 1], [1, feats], [1, 1], [feats, 1], 0, 0), gpred.ptr, w.ptr, gx.ptr)
+    # ... the weight gradient x^T [feats, n] . gpred [n, 1], the bias gradient, and the updated parameters
+    seq.add("matmul_f32", feats, u64(2, 2, 2, [feats, 1], [feats, n], [n, 1], [1, feats], [1, 1], 0, 0), x.ptr, gpred.ptr, gw.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), gpred.ptr, gb.ptr)
+    seq.add("mul_scalar_f32", feats, 1, u64([feats], [1], 0), gw.ptr, C.c_float(0.01), wstep.ptr)
+    seq.add("sub_f32", feats, 1, u64([feats], [1], [1], 0, 0), w.ptr, wstep.ptr, wnew.ptr)
+    seq.add("mul_scalar_f32", 1, 1, u64([1], [1], 0), gb.ptr, C.c_float(0.01), bstep.ptr)
+    seq.add("sub_f32", 1, 1, u64([1], [1], [1], 0, 0), b.ptr, bstep.ptr, bnew.ptr)
+
+
+@pytest.mark.parametrize("n,feats", [(10000, 3), (4096, 4), (5000, 1), (12288, 2), (300, 3)])
+def test_chain_with_matmuls_reductions_and_a_serial_tail(lib, n, feats):
+    """A whole step becomes a few chains: matmul producers and elementwise members in the parallel phase, the sums, the
+    long-reduction matmul and the scalar work in the tail of the group that finishes last.  Replays are the eager bytes."""
+    r = np.random.default_rng(100 + n + feats)
+    seq = Seq(lib)
+    linear_step(lib, seq, n, feats, r)
+    launches, nodes = fused(lib, seq, replays=3)
+    if n >= 4096:
+        assert launches == 15 and nodes <= 3, (launches, nodes)
+
+
+def test_chain_member_is_hoisted_over_tail_stages_only_when_independent(lib):
+    """A member of the parallel phase that arrives after tail stages runs before them in the kernel: it is let in when it
+    touches nothing they write and writes nothing they read, and opens a new chain otherwise."""
+    r = np.random.default_rng(77)
+    n = 6000
+    seq = Seq(lib)
+    x = seq.dev(r.standard_normal(n).astype(np.float32))
+    a, s, t, b, c = seq.out(n * 4, "f4"), seq.out(4, "f4"), seq.out(4, "f4"), seq.out(n * 4, "f4"), seq.out(n * 4, "f4")
+    md1, md2 = u64([n], [1], 0), u64([n], [1], [1], 0, 0)
+    seq.add("tanh_f32", n, 1, md1, x.ptr, a.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), a.ptr, s.ptr)                   # tail
+    seq.add("mul_scalar_f32", 1, 1, u64([1], [1], 0), s.ptr, C.c_float(0.5), t.ptr)        # tail
+    seq.add("mul_f32", n, 1, md2, a.ptr, x.ptr, b.ptr)                                      # independent of the tail: hoisted
+    seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), b.ptr, t.ptr, c.ptr)                 # reads the tail's result: a new chain
+    launches, nodes = fused(lib, seq)
+    assert launches == 5 and nodes == 2, (launches, nodes)
+    # ... and one that would overwrite what the reduction reads must not be hoisted either
+    seq = Seq(lib)
+    x = seq.dev(r.standard_normal(n).astype(np.float32))
+    a, s = seq.out(n * 4, "f4"), seq.out(4, "f4")
+    seq.add("exp_f32", n, 1, md1, x.ptr, a.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), a.ptr, s.ptr)
+    seq.add("neg_f32", n, 1, md1, x.ptr, a.ptr)                                             # overwrites the sum's input
+    launches, nodes = fused(lib, seq)
+    assert launches == 3 and nodes == 2, (launches, nodes)
+
+
+def test_chain_tail_reads_memory_late_when_no_mirror_holds_the_value(lib):
+    """A tail stage whose input was written by two earlier stages (no single LDS mirror holds it), and one that writes
+    across what two earlier stages wrote, wait for memory instead."""
+    r = np.random.default_rng(78)
+    seq = Seq(lib)
+    x = seq.dev(r.standard_normal(64).astype(np.float32))
+    xs = seq.dev(r.standard_normal(5000).astype(np.float32))
+    big, halves, whole, across = seq.out(5000 * 4, "f4"), seq.out(64 * 4, "f4"), seq.out(64 * 4, "f4"), seq.out(32 * 4, "f4")
+    seq.add("exp_f32", 5000, 1, u64([5000], [1], 0), xs.ptr, big.ptr)                                  # the parallel phase
+    seq.add("mul_scalar_f32", 32, 1, u64([32], [1], 0), x.ptr, C.c_float(3.0), halves.ptr)             # halves[0:32]
+    seq.add("mul_scalar_f32", 32, 1, u64([32], [1], 32), x.ptr, C.c_float(5.0), halves.ptr + 128)      # halves[32:64]
+    seq.add("neg_f32", 64, 1, u64([64], [1], 0), halves.ptr, whole.ptr)                                # reads both
+    seq.add("add_f32", 32, 1, u64([32], [1], [1], 16, 0), whole.ptr, x.ptr, halves.ptr + 64)           # writes halves[16:48]
+    seq.add("sub_f32", 32, 1, u64([32], [1], [1], 0, 32), halves.ptr, halves.ptr, across.ptr)          # halves[0:32] - halves[32:64]
+    launches, nodes = fused(lib, seq)
+    assert launches == 6 and nodes == 1, (launches, nodes)
 
 
 def test_fusion_can_be_switched_off(lib):
