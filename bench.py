@@ -764,6 +764,37 @@ def _mlp_setup(mx):
     return lin, mx.tensor(x).with_grad(), mx.tensor(y)
 
 
+def empty_graph_floor(nodes_list=(3, 6, 13), replays=300):
+    """Replay time of a captured sequence of N launches that compute nothing (a one-element fill each, fusion and
+    programs switched off so that every launch stays a kernel node): what N dependent kernel nodes cost on this card
+    before any work is done.  Microseconds per replay, by N."""
+    import maidenx_amd.lib as L
+    lib = L.load()
+    buf = L.DeviceBuffer(256)
+    was_f, was_p = lib.hip_graph_set_fusion(0), lib.hip_graph_set_programs(0)
+    out = {}
+    try:
+        for n in nodes_list:
+            assert lib.hip_graph_begin_capture() == 0
+            for _ in range(n):
+                lib.hip_fill_f32(1, buf.ptr, C.c_float(1.0))
+            h = C.c_void_p()
+            assert lib.hip_graph_end_capture(C.byref(h)) == 0
+            for _ in range(20):
+                lib.hip_graph_launch(h)
+            L.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(replays):
+                lib.hip_graph_launch(h)
+            L.synchronize()
+            out[str(n)] = round((time.perf_counter() - t0) / replays * 1e6, 2)
+            lib.hip_graph_destroy(h)
+    finally:
+        lib.hip_graph_set_fusion(was_f)
+        lib.hip_graph_set_programs(was_p)
+    return out
+
+
 def run_mlp(args):
     """configs[0]: the loop of examples/device/cpu.rs (Linear(3->1) + MSELoss + SGD(0.01), 10000x3 input, full batch)
     through the host layer; a step is one epoch (forward, loss, backward, SGD step, zero_grad)."""
@@ -786,6 +817,7 @@ def run_mlp(args):
                          {"backend_kernels_per_step": calls, "us_per_step": round(dt_s / steps * 1e6, 1)})
     result["roofline"] = None
     result["note"] = "launch-latency bound (about 200 KB touched per step): no roofline fraction applies"
+    result["config"]["empty_graph_replay_us_by_nodes"] = empty_graph_floor()
     result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_mlp(args)
     return result
 

@@ -673,6 +673,118 @@ __global__ __launch_bounds__(PB) void pad_edge_backward3_kernel(Pad3 sp, int mod
     }
 }
 
+// The input coordinates of one dim that receive more than one output gradient ("special"): for a reflection those a
+// mirror image lands on (1 .. before on the left, in-1-after .. in-2 on the right), for a replication the two ends when
+// their side is padded.  Everything else receives exactly the gradient at p + before.
+struct SpecialSet {
+    uint32_t nl, l0, nr, r0;
+    __host__ __device__ uint32_t size() const { return nl + nr; }
+    __host__ __device__ uint32_t at(uint32_t k) const { return k < nl ? l0 + k : r0 + (k - nl); }
+};
+static SpecialSet special_set(int mode, uint32_t in_dim, uint32_t out_dim, uint32_t before) {
+    const uint32_t after = out_dim - in_dim - before;
+    SpecialSet s{0, 0, 0, 0};
+    if (mode == EDGE_REPLICATE) {
+        if (before) { s.nl = 1; s.l0 = 0; }
+        if (after) { s.nr = 1; s.r0 = in_dim - 1; }
+    } else {
+        s.nl = before; s.l0 = 1;
+        s.nr = after; s.r0 = in_dim - 1 - after;
+    }
+    return s;
+}
+struct SpecialSets {
+    SpecialSet d[3];
+    uint32_t count[3];        // elements of the box in which dim k runs over its special coordinates
+    __host__ __device__ static bool has(const SpecialSet& s, uint32_t p) { return p - s.l0 < s.nl || p - s.r0 < s.nr; }
+};
+// One launch, two classes of blocks, so that no wave meets both kinds of work.
+// The first `walk_blocks` blocks (first, so that their longer work starts early and the copy fills in around it): one
+// thread per element of the rows whose coordinate in dim 0 or in dim 1 is special (whole rows, so their stores are
+// contiguous), the full sum in the reference's order; a row special in both dims is written twice, with the same values.
+// The other blocks: a thread owns four consecutive input elements of the other rows and gives each its one gradient, the
+// one at p + before (vector loads of whole rows, vector stores); an element special in the last dim only - two or so per
+// row - gets the few gradients of its own output row instead.
+template <class T>
+__global__ __launch_bounds__(PB) void pad_edge_backward_split_kernel(Pad3 sp, int mode, SpecialSets sets, uint32_t walk_blocks, const T* __restrict__ go,
+                                                                     T* __restrict__ gi, uint32_t n_in, bool vec_store) {
+    constexpr uint32_t PER = 4;
+    if (blockIdx.x >= walk_blocks) {
+        const uint32_t i0 = ((blockIdx.x - walk_blocks) * PB + threadIdx.x) * PER;
+        if (i0 >= n_in) return;
+        uint32_t p0, p1, p2, q;
+        fd_divmod(i0, sp.in_div[2], q, p2);
+        fd_divmod(q, sp.in_div[1], p0, p1);
+        uint32_t row = 0;
+        bool fresh = true, row_special = false;
+        AVec<T, PER> v;
+        uint32_t skip = 0, walk = 0;
+        uint32_t rows[PER], cols[PER];
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e) {
+            if (fresh) {
+                row = (p0 + sp.before[0]) * sp.out_stride[0] + (p1 + sp.before[1]) * sp.out_stride[1];
+                row_special = SpecialSets::has(sets.d[0], p0) || SpecialSets::has(sets.d[1], p1);
+                fresh = false;
+            }
+            const bool ok = i0 + e < n_in;
+            if (!ok || row_special) skip |= 1u << e;
+            else if (SpecialSets::has(sets.d[2], p2)) walk |= 1u << e;
+            rows[e] = row;
+            cols[e] = p2;
+            v.v[e] = go[ok ? row + sp.before[2] + p2 : sp.before[0] * sp.out_stride[0] + sp.before[1] * sp.out_stride[1] + sp.before[2]];
+            if (++p2 == sp.in[2]) {
+                p2 = 0;
+                fresh = true;
+                if (++p1 == sp.in[1]) { p1 = 0; ++p0; }
+            }
+        }
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e) {
+            typename PadAcc<T>::A acc = 0;
+            if (walk & (1u << e)) {
+                // special in the last dim only: the few gradients of its own output row, in ascending order
+                EdgeSrc s2;
+                s2.init(mode, cols[e], sp.in[2], sp.out[2], sp.before[2]);
+                for (uint32_t k2 = 0; k2 < s2.n; ++k2) acc = acc + PadAcc<T>::ld(go[rows[e] + s2.at(k2)]);
+            } else {
+                acc = acc + PadAcc<T>::ld(v.v[e]);
+            }
+            v.v[e] = PadAcc<T>::st(acc);
+        }
+        if (vec_store && skip == 0) {
+            *(AVec<T, PER>*)(gi + i0) = v;
+        } else {
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e)
+                if (!(skip & (1u << e))) gi[i0 + e] = v.v[e];
+        }
+        return;
+    }
+    uint32_t t = blockIdx.x * PB + threadIdx.x;
+    int D = 0;
+    if (t >= sets.count[0]) { t -= sets.count[0]; D = 1; if (t >= sets.count[1]) return; }
+    // the box: dim D runs over the special coordinates, the others over the whole input; the last dim moves fastest
+    const uint32_t e1 = D == 1 ? sets.d[1].size() : sp.in[1], e2 = sp.in[2];
+    uint32_t p2 = t % e2, q = t / e2;
+    uint32_t p1 = q % e1, p0 = q / e1;
+    if (D == 0) p0 = sets.d[0].at(p0);
+    else p1 = sets.d[1].at(p1);
+    EdgeSrc s0, s1, s2;
+    s0.init(mode, p0, sp.in[0], sp.out[0], sp.before[0]);
+    s1.init(mode, p1, sp.in[1], sp.out[1], sp.before[1]);
+    s2.init(mode, p2, sp.in[2], sp.out[2], sp.before[2]);
+    typename PadAcc<T>::A acc = 0;
+    for (uint32_t k0 = 0; k0 < s0.n; ++k0) {
+        const uint32_t o0 = s0.at(k0) * sp.out_stride[0];
+        for (uint32_t k1 = 0; k1 < s1.n; ++k1) {
+            const uint32_t o1 = o0 + s1.at(k1) * sp.out_stride[1];
+            for (uint32_t k2 = 0; k2 < s2.n; ++k2) acc = acc + PadAcc<T>::ld(go[o1 + s2.at(k2)]);
+        }
+    }
+    gi[(int64_t)p0 * sp.in_stride[0] + (int64_t)p1 * sp.in_stride[1] + (int64_t)p2 * sp.in_stride[2]] = PadAcc<T>::st(acc);
+}
+
 static bool edge_space(size_t nd_full, const size_t* md_full, int mode, PadSpace& sp, EdgeWalk& in_walk, size_t* in_off, const char* who) {
     if (nd_full > 64) { set_status(ERR_UNSUPPORTED, who); return false; }
     *in_off = md_full[2 * nd_full];
@@ -759,7 +871,29 @@ void pad_edge_backward(int mode, size_t n_in, size_t n_out, size_t nd, const siz
     for (size_t d = 0; d < nd; ++d) logical *= md[d];
     if (logical == 0) return;
     Pad3 p3;
-    if (simple_edge_shape(sp, mode) && make_pad3(sp, p3))
+    const bool simple = simple_edge_shape(sp, mode) && make_pad3(sp, p3);
+    if (simple && cont && logical == n_in && logical >= (size_t)PB * 64 && logical < (1ull << 31)) {
+        // Large and contiguous: all but a thin border of the input receives exactly one gradient, the one at p + before.
+        // A kernel that tests per element spends a whole wave's time on the walk wherever one lane meets the border,
+        // which is in every wave once rows are shorter than a wave's 256 elements; here the copy and the walk are done by
+        // different blocks of one launch.
+        SpecialSets sets;
+        size_t border = 0;
+        for (int d = 0; d < 3; ++d) {
+            sets.d[d] = special_set(mode, p3.in[d], p3.out[d], p3.before[d]);
+            size_t count = sets.d[d].size();
+            for (int k = 0; k < 3; ++k)
+                if (k != d) count *= p3.in[k];
+            sets.count[d] = (uint32_t)count;
+            if (d < 2) border += count;
+        }
+        const uint32_t copy_blocks = (uint32_t)cdiv(logical, (size_t)PB * 4), walk_blocks = (uint32_t)cdiv(border, (size_t)PB);
+        hipLaunchKernelGGL(pad_edge_backward_split_kernel<T>, dim3(copy_blocks + walk_blocks), dim3(PB), 0, stream(), p3, mode, sets,
+                           walk_blocks, go, gi + off, (uint32_t)logical, (uintptr_t)(gi + off) % (4 * sizeof(T)) == 0);
+        MXH_LAUNCH_CHECK("pad_edge_backward_split");
+        return;
+    }
+    if (simple)
         hipLaunchKernelGGL(pad_edge_backward3_kernel<T>, dim3(cdiv(logical, (size_t)PB * 4)), dim3(PB), 0, stream(), p3, mode, go, gi + off, (uint32_t)logical,
                            cont && (uintptr_t)(gi + off) % (4 * sizeof(T)) == 0);
     else
