@@ -463,7 +463,8 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
             pl.staged = staged;
             // vector form: every access of 16 bytes must be aligned and never straddle a tile edge
             constexpr int TV = TrvCfg<In>::VEC;
-            bool trv = sizeof(Out) == sizeof(In) && sp.dims[pd] % TV == 0 && sp.dims[last] % TV == 0 &&
+            // (a narrower output - the bool of a comparison - leaves as vectors of the same element count)
+            bool trv = sizeof(Out) <= sizeof(In) && sp.dims[pd] % TV == 0 && sp.dims[last] % TV == 0 &&
                        (uintptr_t)out % 16 == 0;
             for (int d = 0; d < last && trv; ++d) trv = sp.strides[0][d] % TV == 0;
             for (int k = 0; k < NIN && trv; ++k) {

@@ -209,33 +209,47 @@ __global__ __launch_bounds__(WAVE * NW) void softmax_col_split_kernel(const T* _
         }
         __syncthreads();
     };
+    // 8 KB of loads in flight per wave (a wave's row is one or a few cache lines: taken one at a time, every row costs
+    // a memory latency, and with few bytes per row the 2048 waves of a [8192,8192] launch cannot cover the latency
+    // between them); the rows are still folded in ascending order
+    constexpr int ROW_BYTES = WAVE * VEC * (int)sizeof(T);
+    constexpr int U = 8192 / ROW_BYTES < 8 ? 8 : (8192 / ROW_BYTES > 32 ? 32 : 8192 / ROW_BYTES);
+    auto sweep = [&](auto&& each) {
+        size_t l = l0;
+        for (; l + U <= l1; l += U) {
+            AVec<T, VEC> v[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) v[k] = load(l + k);
+#pragma unroll
+            for (int k = 0; k < U; ++k) each(l + k, v[k]);
+        }
+        for (; l < l1; ++l) each(l, load(l));
+    };
     float m[VEC], s[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) { m[e] = -INFINITY; s[e] = 0.0f; }
     if (live)
-        for (size_t l = l0; l < l1; ++l) {
-            AVec<T, VEC> v = load(l);
+        sweep([&](size_t, const AVec<T, VEC>& v) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(v.v[e]); m[e] = x > m[e] ? x : m[e]; }
-        }
+        });
     combine(m, true);
     if (live)
-        for (size_t l = l0; l < l1; ++l) {
-            AVec<T, VEC> v = load(l);
+        sweep([&](size_t, const AVec<T, VEC>& v) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) s[e] += SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]);
-        }
+        });
     combine(s, false);
     if (!live) return;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) s[e] = m_exp(-INFINITY - m[e]) + s[e];
-    for (size_t l = l0; l < l1; ++l) {
-        AVec<T, VEC> v = load(l), o;
+    sweep([&](size_t l, const AVec<T, VEC>& v) {
+        AVec<T, VEC> o;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]), s[e]);
         if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + l * post) = o;
         else dst[l * post] = o.v[0];
-    }
+    });
 }
 
 struct SoftmaxStrided {

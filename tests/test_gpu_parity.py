@@ -108,6 +108,7 @@ UN_LAYOUTS = {
     "contig": lambda: LY.contiguous([5000]),
     "offset": lambda: LY.contiguous([77, 13], off=1),
     "transposed": lambda: LY.permuted([150, 200], [1, 0]),
+    "transposed_whole_tiles": lambda: LY.permuted([160, 256], [1, 0]),      # the vector form of the tile kernel, also for bool outputs
     "bcast": lambda: LY.broadcast([40, 50], [1, 50]),
     "perm4d": lambda: LY.permuted([2, 5, 6, 7], [3, 1, 0, 2]),
 }
