@@ -313,8 +313,18 @@ template <class T>
 __global__ __launch_bounds__(256) void gemm_fold_kernel(const float* __restrict__ part, T* __restrict__ out, size_t n, uint32_t splits) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
+    // sixteen partials in flight per thread (the launch is a few hundred blocks: taken one at a time, every partial
+    // costs a memory latency); added in split order
     float acc = part[i];
-    for (uint32_t s = 1; s < splits; ++s) acc += part[(size_t)s * n + i];
+    uint32_t s = 1;
+    for (; s + 16 <= splits; s += 16) {
+        float v[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) v[k] = part[(size_t)(s + k) * n + i];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) acc += v[k];
+    }
+    for (; s < splits; ++s) acc += part[(size_t)s * n + i];
     out[i] = Elem<T>::st(acc);
 }
 
@@ -342,7 +352,13 @@ __device__ __forceinline__ TilePos tile_of_block(const GemmArgs& g) {
 }
 
 // FAST: the tile lies inside the operands in all three extents and the wide accesses are aligned (no checks).
-template <class T, bool XR, bool YR, class Cfg, bool FAST>
+// PANEL: the block works through a run of consecutive output tiles (row-major over the tile grid: pos.ti is the first
+// tile, pos.tj the number of tiles), one after the other, in the same pipeline: the k-tiles of the next output tile are
+// requested while this one is being multiplied, and its stores leave while the next one works.  For products with a
+// reduction of a few k-tiles only (a convolution's input gradient, [100352,64]x[64,576]): as one block per output tile
+// such a product is 14112 short blocks, each of which pays the full memory latency for two k-tiles of work, and the four
+// blocks a CU holds do not cover it.  The launch has as many blocks as the chip holds at once, with equal shares.
+template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false>
 __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
     constexpr bool SWZ = Cfg::TS == 16;
@@ -385,17 +401,22 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
     static_assert(TS == 32 || (sizeof(T) == 2 && MJ % 2 == 0), "16x16 tiles are for 16-bit operands");
     SX sx;
     SY sy;
-    const uint32_t nk = (re - rb + TK - 1) / TK;
+    const uint32_t nk1 = (re - rb + TK - 1) / TK;                 // k-tiles of one output tile
+    const uint32_t nk = PANEL ? nk1 * pos.tj : nk1;               // steps of the pipeline
+    // where step q of the pipeline reads: its reduction offset and (PANEL) the first row and column of its output tile
+    auto red_of = [&](uint32_t q) { return rb + (PANEL ? q % nk1 : q) * TK; };
+    auto row_of = [&](uint32_t q) { return PANEL ? ((pos.ti + q / nk1) / g.tiles_j) * (uint32_t)TM : i0; };
+    auto col_of = [&](uint32_t q) { return PANEL ? ((pos.ti + q / nk1) % g.tiles_j) * (uint32_t)TN : j0; };
     {
         // tiles 0 and 1 are requested together (one memory latency instead of two); the accumulators are
         // not live yet, so the second set of staging registers costs nothing
         SX sx0;
         SY sy0;
-        sx0.template load<FAST>(X, g.xi, g.xr, i0, rb, g.I, re);
-        sy0.template load<FAST>(Y, g.yj, g.yr, j0, rb, g.J, re);
-        uint32_t r1 = rb + (nk > 1 ? 1u : 0u) * TK;
-        sx.template load<FAST>(X, g.xi, g.xr, i0, r1, g.I, re);
-        sy.template load<FAST>(Y, g.yj, g.yr, j0, r1, g.J, re);
+        sx0.template load<FAST>(X, g.xi, g.xr, row_of(0), rb, g.I, re);
+        sy0.template load<FAST>(Y, g.yj, g.yr, col_of(0), rb, g.J, re);
+        const uint32_t q1 = nk > 1 ? 1u : 0u;
+        sx.template load<FAST>(X, g.xi, g.xr, row_of(q1), red_of(q1), g.I, re);
+        sy.template load<FAST>(Y, g.yj, g.yr, col_of(q1), red_of(q1), g.J, re);
         sx0.store(lds_x);
         sy0.store(lds_y);
     }
@@ -461,7 +482,8 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
         const T* cy = lds_y + cur * TN * PITCH;
         T* nx = lds_x + (cur ^ 1) * TM * PITCH;
         T* ny = lds_y + (cur ^ 1) * TN * PITCH;
-        const uint32_t nt = rb + (kt + 2 < nk ? kt + 2 : nk - 1) * TK;
+        const uint32_t qn = kt + 2 < nk ? kt + 2 : nk - 1;
+        const uint32_t nt = red_of(qn), ni = row_of(qn), nj = col_of(qn);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             if (s + 1 < S) {
@@ -469,8 +491,8 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
                 const int y0 = SY::NU * s / (S - 1), y1 = SY::NU * (s + 1) / (S - 1);
                 sx.store(nx, x0, x1);
                 sy.store(ny, y0, y1);
-                sx.template load<FAST>(X, g.xi, g.xr, i0, nt, g.I, re, x0, x1);
-                sy.template load<FAST>(Y, g.yj, g.yr, j0, nt, g.J, re, y0, y1);
+                sx.template load<FAST>(X, g.xi, g.xr, ni, nt, g.I, re, x0, x1);
+                sy.template load<FAST>(Y, g.yj, g.yr, nj, nt, g.J, re, y0, y1);
                 read_frags(s + 1, cx, cy);
             } else {
                 __syncthreads();
@@ -494,7 +516,19 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
             __builtin_amdgcn_sched_barrier(0);
 #endif
         }
+        if constexpr (PANEL) {
+            if ((kt + 1) % nk1 == 0) {       // the last k-tile of an output tile: out it goes, and the accumulators start over
+                store_tile<T, Cfg, FAST>((T*)g.out, acc, g, row_of(kt), col_of(kt), wm, wn, lane);
+#pragma unroll
+                for (int a = 0; a < MI; ++a)
+#pragma unroll
+                    for (int c = 0; c < MJ; ++c)
+#pragma unroll
+                        for (int e = 0; e < (TS == 32 ? 16 : 4); ++e) acc[a][c][e] = 0.0f;
+            }
+        }
     }
+    if constexpr (PANEL) return;
 
     if (g.splits > 1) {
         float* part = g.part + ((int64_t)split * g.batch + b) * g.I * g.J;
@@ -507,6 +541,20 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
 // ALIGNED: the operands allow the unchecked body wherever a whole tile lies inside them (the host has checked
 // alignment, strides and that the reduction is a whole number of k-tiles); blocks on a ragged edge, and every block
 // of an unaligned problem, take the checked body.
+// whole tiles everywhere, one batch, no split: block b takes the tiles [b * per, (b + 1) * per) of the row-major tile grid
+template <class T, bool XR, bool YR, class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_panel_kernel(GemmArgs g, uint32_t per) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t tiles = g.tiles_i * g.tiles_j, first = blockIdx.x * per;
+    if (first >= tiles) return;
+    TilePos pos;
+    pos.ti = first;
+    pos.tj = tiles - first < per ? tiles - first : per;
+    pos.b = 0;
+    pos.split = 0;
+    gemm_mfma_body<T, XR, YR, Cfg, true, true>(g, pos, smem);
+}
+
 template <class T, bool XR, bool YR, class Cfg, bool ALIGNED>
 __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -548,6 +596,17 @@ void launch_mfma_impl(GemmArgs g) {
     if (g.splits > 1) {
         g.part = (float*)scratch(n_out * g.splits * sizeof(float));
         if (!g.part) return;
+    }
+    if constexpr (FAST && std::is_same<Cfg, typename Cfgs<T>::Tall>::value) {
+        // a reduction of a few k-tiles, many whole tiles: as many blocks as the chip holds, each with a run of tiles (see PANEL)
+        constexpr size_t slots = 256 * 4;       // four blocks of this configuration fit a CU's LDS
+        if (g.splits == 1 && g.batch == 1 && g.R <= 4 * TK && g.I % Cfg::TM == 0 && g.J % Cfg::TN == 0 && tiles >= 4 * slots && tiles < (1ull << 31)) {
+            auto pk = gemm_mfma_panel_kernel<T, XR, YR, Cfg>;
+            const uint32_t per = (uint32_t)cdiv(tiles, slots);
+            hipLaunchKernelGGL(pk, dim3((unsigned)cdiv(tiles, (size_t)per)), dim3(Cfg::NT), lds_bytes, stream(), g, per);
+            MXH_LAUNCH_CHECK("gemm_mfma_panel");
+            return;
+        }
     }
     auto kern = gemm_mfma_kernel<T, XR, YR, Cfg, FAST>;
     // more than 64 KB of LDS has to be allowed once per kernel and device (setting it twice is harmless)

@@ -499,6 +499,27 @@ def test_matmul_whole_256_tiles(hip, shape, a_perm, b_perm, dt):
     assert np.max(err) <= tol, float(np.max(err))
 
 
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", [(1, 32768, 64, 192), (1, 100352, 96, 128), (1, 40960, 128, 64 * 9), (1, 65600 * 64 // 64, 32, 64)], ids=lambda s: "x".join(map(str, s)))
+def test_matmul_short_reduction_row_panels(hip, shape, a_perm, b_perm, dt):
+    """Whole 64-wide tiles and a reduction of a few k-tiles: as many blocks as the chip holds, each walking a run of
+    output tiles (the convolution's input gradient is such a product), for every operand layout; tile counts that do and
+    do not divide evenly among the blocks, runs that cross from one tile row to the next."""
+    batch, m, k, n = shape
+    r = rng(61)
+    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt)
+    (h,) = hip.call(f"matmul_{dt}", batch * m * n, md, In(sa), In(sb), Out(batch * m * n, dt))
+    got = to_float(h, dt).reshape(batch, m, n)
+    rows = np.unique(np.concatenate([np.arange(0, 130), r.integers(0, m, 600), np.arange(m - 130, m)]))
+    truth = np.einsum("bmk,bkn->bmn", av[:, rows], bv)
+    scale = np.einsum("bmk,bkn->bmn", np.abs(av[:, rows]), np.abs(bv))
+    tol = 1e-5 if dt == "f32" else 1e-2
+    err = np.abs(got[:, rows] - truth) / np.maximum(scale, 1e-30)
+    assert np.max(err) <= tol, float(np.max(err))
+    assert np.isfinite(got).all()
+
+
 def test_matmul_broadcast_batch_uses_stride0(oracle, hip):
     r = rng(47)
     sa, sb, md, av, bv = matmul_inputs(r, 3, 40, 50, 60, False, False, "f32", b_bcast=True)
