@@ -938,6 +938,9 @@ def run_conv(args):
             result["roofline"] = hbm_roofline("im2col_band_kernel<float> (hip_conv2d_im2col_f32, [32,64,56,56] 3x3), operands rotated", nbytes, durs)
             result["roofline"]["launches_timed"] = 3 * SETS
             result["roofline"]["algorithmic_bytes"] = nbytes
+            src = "profiles/conv2d_32x64x56x56_kernel_trace.txt"
+            result["roofline"]["traffic"], when = profile_traffic(src, "im2col_f32/32x64x56x56/3x3")
+            result["roofline"]["traffic_source"] = f"{src} (rocprofv3 --pmc, measured {when})" if when else None
     result["config"]["kernels_alone"] = kernels
     worst = min(kernels, key=lambda k: kernels[k]["hbm_frac"])
     result["roofline"]["worst_of_chain"] = dict(kernel=worst, **kernels[worst])
