@@ -1291,22 +1291,35 @@ size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr
                 const size_t one = period;
                 period = one * std::max<size_t>(1, 12 / one);
                 while (period > one && 2 * period > epochs - done) period -= one;
+                // The recorded steps must follow the allocation pattern the warm-up settled into: a replay runs on the
+                // addresses recorded, and is only the next step's work if that step would have used the same ones.
+                const size_t warm = traces.size();
+                std::vector<std::vector<void*>> recorded(period);
                 B::graph_begin();
                 try {
-                    for (size_t k = 0; k < period; ++k) step(done + k);
+                    for (size_t k = 0; k < period; ++k) {
+                        pool.trace = &recorded[k];
+                        step(done + k);
+                        pool.trace = nullptr;
+                    }
                 } catch (...) {
+                    pool.trace = nullptr;
                     try { B::graph_end(&exec); } catch (...) { exec = nullptr; }
                     if (exec) B::graph_destroy(exec);
                     throw;
                 }
                 B::graph_end(&exec);
+                bool periodic = true;
+                for (size_t k = 0; k < period && periodic; ++k) periodic = recorded[k] == traces[warm - one + k % one];
                 if (pool.device_allocs != allocs_before) {
                     B::graph_destroy(exec);
                     throw Error(ErrKind::Backend, "training loop allocated device memory while it was being recorded");
                 }
                 // the recorded steps did not run yet: replay them, then as many more whole periods as fit
                 const size_t calls_per_period = backend_calls() - calls_before;
-                size_t periods = (epochs - done) / period;
+                // (a recording that left the pattern is still exactly the steps it recorded: it runs once, and the loop
+                // goes on eagerly)
+                size_t periods = periodic ? (epochs - done) / period : 1;
                 for (size_t r = 0; r < periods; ++r) B::graph_launch(exec);
                 backend_calls() += calls_per_period * (periods - 1);
                 done += periods * period;

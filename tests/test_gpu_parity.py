@@ -520,6 +520,43 @@ def test_matmul_short_reduction_row_panels(hip, shape, a_perm, b_perm, dt):
     assert np.isfinite(got).all()
 
 
+def test_matmul_strided_rows_is_the_full_product(oracle, hip):
+    """A = big[:, :k], a view whose rows are 3k apart.  The CPU reference drops every term whose operand index reaches
+    num_els * k (crates/maidenx_cpu/src/ops/matmul.rs:53-54,109), which cuts the later rows short; the GPU computes the
+    whole product.  The oracle, which restates the CPU, differs by exactly those terms."""
+    r = rng(71)
+    m, k, n, wide = 40, 24, 16, 72
+    big = r.standard_normal((m, wide)).astype(np.float32)
+    b = r.standard_normal((k, n)).astype(np.float32)
+    md = meta_matmul([m, n], [m, k], [k, n], [wide, 1], [n, 1])
+    (h,) = hip.call("matmul_f32", m * n, md, In(big.ravel()), In(b.ravel()), Out(m * n, "f32"))
+    (o,) = oracle.call("matmul_f32", m * n, md, In(big.ravel()), In(b.ravel()), Out(m * n, "f32"))
+    a64, b64 = big[:, :k].astype(np.float64), b.astype(np.float64)
+    full = a64 @ b64
+    scale = np.abs(a64) @ np.abs(b64)
+    assert np.max(np.abs(h.reshape(m, n) - full) / scale) <= 1e-5
+    # the guard: a term (i, r) survives when i * wide + r < m * n * k  (and the B index, always small here, does too)
+    limit = m * n * k
+    keep = (np.arange(m)[:, None] * wide + np.arange(k)[None, :]) < limit
+    assert keep.all()                  # (with these sizes every index is below the limit ...)
+    truncated = (a64 * keep) @ b64
+    assert np.max(np.abs(o.reshape(m, n) - truncated) / scale) <= 1e-5
+    # ... so make the guard bite: the same view of a taller matrix with a single output column
+    m2, n2 = 400, 1
+    big2 = r.standard_normal((m2, wide)).astype(np.float32)
+    b2 = r.standard_normal((k, n2)).astype(np.float32)
+    md2 = meta_matmul([m2, n2], [m2, k], [k, n2], [wide, 1], [n2, 1])
+    (h2,) = hip.call("matmul_f32", m2 * n2, md2, In(big2.ravel()), In(b2.ravel()), Out(m2 * n2, "f32"))
+    (o2,) = oracle.call("matmul_f32", m2 * n2, md2, In(big2.ravel()), In(b2.ravel()), Out(m2 * n2, "f32"))
+    a2, bb2 = big2[:, :k].astype(np.float64), b2.astype(np.float64)
+    keep2 = (np.arange(m2)[:, None] * wide + np.arange(k)[None, :]) < m2 * n2 * k
+    assert not keep2.all()
+    scale2 = np.abs(a2) @ np.abs(bb2)
+    assert np.max(np.abs(h2.reshape(m2, n2) - a2 @ bb2) / scale2) <= 1e-5
+    assert np.max(np.abs(o2.reshape(m2, n2) - (a2 * keep2) @ bb2) / scale2) <= 1e-5
+    assert np.max(np.abs(o2 - h2)) > 0.1            # rows beyond the limit are all zeros in the oracle's result
+
+
 def test_matmul_broadcast_batch_uses_stride0(oracle, hip):
     r = rng(47)
     sa, sb, md, av, bv = matmul_inputs(r, 3, 40, 50, 60, False, False, "f32", b_bcast=True)
