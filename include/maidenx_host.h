@@ -115,6 +115,11 @@ int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_
  * epoch eager; mxt_last_train_replayed() tells how many epochs of the last mxt_train call were replays. */
 void mxt_set_graph_replay(int enabled);
 size_t mxt_last_train_replayed(void);
+/* Conv2d backward (nn/layers/conv.rs:253-268): col2im is handed num_els = B*C*H*W and reads no entry of grad_cols at
+ * or beyond that flat index (crates/maidenx_cpu/src/nn/conv.rs:135), so by default only the leading
+ * ceil(B*C*H*W / (C*kh*kw)) rows of grad_cols are computed; the input gradient is the same bytes either way.
+ * enabled = 0 computes the whole product as the reference does. */
+void mxt_set_conv_skip_unread_grad_cols(int enabled);
 
 /* bookkeeping */
 size_t mxt_backend_calls(void);                  /* kernels dispatched since the last reset */

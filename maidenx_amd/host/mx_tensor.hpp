@@ -228,6 +228,8 @@ template <class B> struct GradCell {
 
 // Count of backend kernel calls (what `be::*` would dispatch), for reporting.
 inline size_t& backend_calls() { static size_t n = 0; return n; }
+// Conv2d backward: make only the rows of grad_cols that col2im reads (see Conv2d); false = the whole product.
+inline bool& conv_skip_unread_grad_cols() { static bool on = true; return on; }
 // Count of whole-buffer dtype conversions (with_dtype: a host loop in the reference, a kernel here).
 inline size_t& cast_calls() { static size_t n = 0; return n; }
 
@@ -1126,19 +1128,32 @@ struct Conv2d {                                                                 
             out.set_node("conv2d", inputs, [=](const std::vector<T>& in, const T& go) {              // conv.rs:236-306
                 const T &x = in[0], &w = in[1];
                 std::vector<T> grads;
-                auto flat_grad = [&]() {
+                // conv.rs:249-251 and :276-278 build the same [B*oh*ow, Cout] copy of the gradient twice; it is made once
+                T grad_flat;
+                if (x.requires_grad || w.requires_grad) {
                     T gr = go.transpose(2, 3).transpose(1, 3);
-                    return gr.reshape(Shape{go.shape()[0] * oh * ow, go.shape()[1]});
-                };
+                    grad_flat = gr.reshape(Shape{go.shape()[0] * oh * ow, go.shape()[1]});
+                }
                 if (x.requires_grad) {
                     const Shape& ws = w.shape();
                     T wm = w.reshape(Shape{ws[0], ws[1] * ws[2] * ws[3]});
-                    T grad_cols = flat_grad().matmul(wm);
                     // col2im divides by what it reads as the stride, i.e. by the padding the caller stored in
                     // slots 10, 11: with padding 0 the reference panics (division by zero)
                     if (ph_ == 0 || pw_ == 0)
                         throw Error(ErrKind::InvalidOperation, "col2im: division by zero (padding 0 is read as stride 0)");
                     T gi = T::empty({Bn, C, H, W});                                                  // col2im, conv.rs:378-418
+                    // col2im is handed num_els = B*C*H*W (conv.rs:391) and reads no column entry at or beyond that flat
+                    // index (crates/maidenx_cpu/src/nn/conv.rs:135), i.e. only the first ceil(B*C*H*W / (C*kh*kw)) rows of
+                    // grad_cols; the rows below are never read, so the product is made for those leading rows only (each of
+                    // them the same arithmetic as in the whole product).
+                    T lead = grad_flat;
+                    const size_t row_len = ws[1] * ws[2] * ws[3];
+                    const size_t used = row_len ? (gi.size() + row_len - 1) / row_len : 0;
+                    if (conv_skip_unread_grad_cols() && grad_flat.is_contiguous() && used < grad_flat.shape()[0]) {
+                        lead = T::share_buffer(grad_flat);
+                        lead.layout.shape[0] = used;
+                    }
+                    T grad_cols = lead.matmul(wm);
                     auto md = conv_meta(Bn, C, H, W, kh_, kw_, oh, ow, sh_, sw_, ph_, pw_);
                     B::col2im(gi.size(), md.data(), grad_cols.f32(), gi.f32());
                     ++backend_calls();
@@ -1148,7 +1163,7 @@ struct Conv2d {                                                                 
                     grads.push_back(T::zeros_like(x));
                 }
                 if (w.requires_grad) {
-                    T gw = cols.transpose(-1, -2).matmul(flat_grad());
+                    T gw = cols.transpose(-1, -2).matmul(grad_flat);
                     grads.push_back(gw.reshape(Shape{w.shape()[0], w.shape()[1], kh_, kw_}));
                 } else {
                     grads.push_back(T::zeros_like(w));

@@ -114,6 +114,25 @@ def test_conv2d_forward_backward(mx_hip, mx_oracle, B, Cin, H, W, Cout, k, strid
         assert np.abs(got[key] - num[key]).max() <= 1e-4 * scale, key
 
 
+@pytest.mark.parametrize("B,Cin,H,W,Cout,k,stride,pad", [(2, 3, 6, 5, 4, 3, 1, 1), (3, 4, 5, 5, 2, 1, 1, 1), (4, 16, 14, 14, 32, 3, 1, 1),
+                                                         (8, 64, 28, 28, 64, 3, 1, 1)])
+def test_conv2d_backward_makes_only_the_rows_of_grad_cols_that_col2im_reads(mx_hip, B, Cin, H, W, Cout, k, stride, pad):
+    """The product behind the input gradient is made for the leading rows that col2im reads (conv.rs:391,
+    crates/maidenx_cpu/src/nn/conv.rs:135); every gradient is the bytes that the whole product gives."""
+    x, w, b = conv_inputs(B, Cin, H, W, Cout, k, seed=B * 10 + W)
+    oh, ow = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    target = np.random.default_rng(6).standard_normal((B, Cout, oh, ow)).astype(np.float32)
+    try:
+        mx_hip.set_conv_skip_unread_grad_cols(False)
+        whole = conv_step(mx_hip, x, w, b, stride, pad, target)
+        mx_hip.set_conv_skip_unread_grad_cols(True)
+        lead = conv_step(mx_hip, x, w, b, stride, pad, target)
+    finally:
+        mx_hip.set_conv_skip_unread_grad_cols(True)
+    for key in ("out", "loss", "grad_b", "grad_w", "grad_x"):
+        np.testing.assert_array_equal(lead[key].view(np.uint32), whole[key].view(np.uint32), err_msg=key)
+
+
 def test_graph_replayed_training_equals_eager(mx_hip):
     """mxt_train records the step as a HIP graph and replays it; every run is compared with the eager loop, with
     eager work and synchronisations in between (the same graph machinery is set up and torn down each time)."""

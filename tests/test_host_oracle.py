@@ -127,6 +127,30 @@ def test_conv2d_forward_backward(mx_oracle, B, Cin, H, W, Cout, k, stride, pad):
         np.testing.assert_allclose(got[key], ref[key], rtol=1e-4, atol=1e-6, err_msg=key)
 
 
+@pytest.mark.parametrize("B,Cin,H,W,Cout,k,stride,pad", [(2, 3, 6, 5, 4, 3, 1, 1), (1, 2, 7, 7, 3, 3, 2, 2), (3, 4, 5, 5, 2, 1, 1, 1)])
+def test_conv2d_backward_makes_only_the_rows_of_grad_cols_that_col2im_reads(mx_oracle, B, Cin, H, W, Cout, k, stride, pad):
+    # col2im gets num_els = B*C*H*W and reads nothing at or beyond that flat index (conv.rs:391, cpu/nn/conv.rs:135): the
+    # product restricted to the leading rows must give the bytes of the whole product, with one matmul call either way
+    x, w, b = conv_inputs(B, Cin, H, W, Cout, k, seed=B * 10 + W)
+    oh, ow = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    target = np.random.default_rng(6).standard_normal((B, Cout, oh, ow)).astype(np.float32)
+    mx = mx_oracle
+    try:
+        mx.set_conv_skip_unread_grad_cols(False)
+        mx.reset_backend_calls()
+        whole = conv_step(mx, x, w, b, stride, pad, target)
+        calls_whole = mx.backend_calls()
+        mx.set_conv_skip_unread_grad_cols(True)
+        mx.reset_backend_calls()
+        lead = conv_step(mx, x, w, b, stride, pad, target)
+        calls_lead = mx.backend_calls()
+    finally:
+        mx.set_conv_skip_unread_grad_cols(True)
+    assert calls_lead == calls_whole
+    for key in ("out", "loss", "grad_b", "grad_w", "grad_x"):
+        np.testing.assert_array_equal(lead[key].view(np.uint32), whole[key].view(np.uint32), err_msg=key)
+
+
 def test_conv2d_backward_with_zero_padding_is_an_error(mx_oracle):
     # padding 0 lands in the slots col2im reads as its stride: the reference panics on the division
     x, w, b = conv_inputs(1, 2, 5, 5, 2, 3, seed=3)
