@@ -561,6 +561,21 @@ MX_DECL_CONV(mx_f16, f16)
 void hip_conv2d_im2col_f64(size_t num_els, const size_t* metadata, const double* input, double* col);
 void hip_conv2d_col2im_f64(size_t num_els, const size_t* metadata, const double* col, double* output);
 
+/* ---- the Conv2d layer's products with the column matrix, the matrix never stored --------------------------------
+ * No backend symbol exists for this in the reference: crates/maidenx_nn/src/layers/conv.rs:206-222 writes the column
+ * matrix with conv2d_im2col and multiplies it, reading the buffer [B][C*kh*kw][oh*ow] as a row-major matrix
+ * cols[M = B*oh*ow, K = C*kh*kw]; :279 multiplies its transpose with the output gradient.  One call here is that
+ * product with the entries of the matrix gathered from `input` while the tiles are staged (a ninth of the memory
+ * traffic for a 3x3 kernel, and no buffer of M*K elements):
+ *   transposed == 0:  out[M, n] = cols x rhs,     rhs [K, n]
+ *   transposed != 0:  out[K, n] = cols^T x rhs,   rhs [M, n]
+ * metadata: the 12 slots of hip_conv2d_im2col_f32; rhs_strides: element strides of rhs's two dims (one of them must
+ * be 1), rhs already points at its first element; out is contiguous.  Same tiles, same order of additions as
+ * hip_conv2d_im2col_f32 followed by hip_matmul_f32 on products that the latter runs on the matrix cores, so the
+ * same bits there.  M*K and B*C*H*W must be below 2^31. */
+void hip_conv2d_cols_matmul_f32(const size_t* metadata, int transposed, const float* input, const float* rhs, size_t n,
+                                const size_t* rhs_strides, float* out);
+
 /* ---- softmax: replaces crates/maidenx_cuda/src/nn/activation/softmax.rs (cuda_softmax_<T>) ------------
  * metadata = dims[n] | strides[n] | offset; dim >= num_dims means the last dim.
  * Semantics: crates/maidenx_cpu/src/nn/activation/softmax.rs:62-207 (max from -inf, the sum seeded

@@ -120,6 +120,14 @@ size_t mxt_last_train_replayed(void);
  * ceil(B*C*H*W / (C*kh*kw)) rows of grad_cols are computed; the input gradient is the same bytes either way.
  * enabled = 0 computes the whole product as the reference does. */
 void mxt_set_conv_skip_unread_grad_cols(int enabled);
+/* Conv2d forward (conv.rs:206-222) and its weight gradient (:279) multiply the column matrix.  The HIP build can
+ * gather the entries of that matrix from the input inside the product (hip_conv2d_cols_matmul_f32) instead of storing
+ * it with conv2d_im2col first.  mode 0: always store, as the reference does; 1 (default): gather when the input does
+ * not require a gradient, i.e. when no backward is recorded (the forward alone is faster that way; a training step is
+ * faster with the one stored matrix that serves both products); 2: gather in forward and backward (about 6 % slower
+ * per step on a 64-channel 3x3 layer, and no buffer of B*oh*ow x C*kh*kw elements is held for the backward).  The
+ * products are the same bits wherever the stored product runs on the matrix cores. */
+void mxt_set_conv_gathered_products(int mode);
 
 /* bookkeeping */
 size_t mxt_backend_calls(void);                  /* kernels dispatched since the last reset */

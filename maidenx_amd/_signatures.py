@@ -175,6 +175,7 @@ def extension_signatures():
                  ("bool", "f16"), ("f32", "f16"), ("f16", "f32"), ("f16", "bool")):
         sig[f"cast_{a}_{b}"] = [SZ, P, P]
     sig["sum_f32_noalloc"] = [SZ, SZ, SZ, P, P, P]
+    sig["conv2d_cols_matmul_f32"] = [P, C.c_int, P, P, SZ, P, P]
     sig.update(cast_signatures())
     sig.update(wide_util_signatures())
     sig.update(wide_unary_signatures())

@@ -215,6 +215,110 @@ struct Stager {
     }
 };
 
+// ---- the column matrix of a convolution as a left operand that is never stored -----------------------
+// What conv2d_im2col writes for an input [B,C,H,W] is the buffer col[b][(c*kh+i)*kw+j][ho*ow+wo]; the Conv2d layer
+// reads that buffer as a row-major matrix [B*oh*ow, C*kh*kw] (nn/layers/conv.rs:222, :279), i.e. entry (m, k) is flat
+// index f = m*K + k of the buffer, whatever plane and pixel that happens to be.  Rows [b*P, (b+1)*P) of the matrix are
+// batch b's part of the buffer (P = oh*ow), so within a batch the entry sits in plane (m - b*P)*K + k) / P at pixel
+// (...) % P.  A staged tile of the matrix is gathered straight from the input (which the caches hold: it is a ninth of
+// the matrix for a 3x3 kernel) instead of from a stored copy.
+struct ColsView {
+    const float* in;
+    uint32_t K, P;                 // columns of the matrix (C*kh*kw), pixels of a plane (oh*ow)
+    uint32_t H, W, HW, CHW, sh, sw;
+    int32_t ph, pw;
+    FastDiv d_P, d_khkw, d_kw, d_ow;
+};
+// The unit of the gather: matrix row m, columns k4 .. k4+3 (k4 a multiple of four).  VEC4: the four are neighbours in
+// one output row (K and ow multiples of four), located once; otherwise one by one.  `live`: bit e = entry e is wanted.
+template <bool VEC4>
+__device__ __forceinline__ f32x4 cols_gather4(const ColsView& v, uint32_t m, uint32_t k4, uint32_t live) {
+    f32x4 val = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t b = fd_div(m, v.d_P);
+    const uint32_t f0 = (m - b * v.P) * v.K + k4;           // flat index inside batch b
+    const float* plane0 = v.in + (size_t)b * v.CHW;
+    auto locate = [&](uint32_t f, const float*& row, int32_t& wi) -> bool {      // the input row and column of flat index f
+        uint32_t ckk, pix, ho, wo, c, t, i, j;
+        fd_divmod(f, v.d_P, ckk, pix);
+        fd_divmod(pix, v.d_ow, ho, wo);
+        fd_divmod(ckk, v.d_khkw, c, t);
+        fd_divmod(t, v.d_kw, i, j);
+        const int32_t hi = (int32_t)(ho * v.sh + i) - v.ph;
+        wi = (int32_t)(wo * v.sw + j) - v.pw;
+        const bool ok = (uint32_t)hi < v.H;
+        row = plane0 + c * v.HW + (ok ? (uint32_t)hi * v.W : 0u);
+        return ok;
+    };
+    if constexpr (VEC4) {
+        const float* row;
+        int32_t wi;
+        const bool hok = locate(f0, row, wi);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int32_t w = wi + e * (int32_t)v.sw;
+            const bool ok = hok && (uint32_t)w < v.W && ((live >> e) & 1u);
+            const float x = row[ok ? w : 0];
+            val[e] = ok ? x : 0.0f;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (!((live >> e) & 1u)) continue;
+            const float* row;
+            int32_t wi;
+            const bool ok = locate(f0 + e, row, wi) && (uint32_t)wi < v.W;
+            const float x = row[ok ? wi : 0];
+            val[e] = ok ? x : 0.0f;
+        }
+    }
+    return val;
+}
+
+// Stages a ROWS x TK tile of the matrix (TURNED: of its transpose, so the tile's rows are columns k of the matrix and
+// its reduction runs over the rows m) into the LDS layout [row][TK + pad] of Stager<float, ...>.  Either way a thread
+// gathers units of four consecutive k at one m (consecutive lanes take consecutive units along k: neighbouring
+// pixels); TURNED then writes the four to four LDS rows instead of one 16-byte vector to one.
+template <bool TURNED, bool VEC4, int ROWS, int NT>
+struct ColsStager {
+    static constexpr int TK = TK_BYTES / 4, PITCH = TK + 4;
+    static constexpr int NV = ROWS * TK / 4 / NT, NU = NV;
+    static constexpr int KV = (TURNED ? ROWS : TK) / 4;        // units along k
+    static_assert(NV >= 1 && NT % KV == 0, "tile too small for this block size");
+    f32x4 reg[NV];
+    template <bool FAST>
+    __device__ void load_cols(const ColsView& v, uint32_t row0, uint32_t red0, uint32_t nrows, uint32_t nred, int u0 = 0, int u1 = NU) {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            if (u < u0 || u >= u1) continue;
+            const int id = t + u * NT;
+            const uint32_t m = (TURNED ? red0 : row0) + id / KV, k4 = (TURNED ? row0 : red0) + (id % KV) * 4;
+            uint32_t live = 0xFu;
+            if constexpr (!FAST) {
+                const uint32_t nm = TURNED ? nred : nrows, nk = TURNED ? nrows : nred;
+                live = m >= nm || k4 >= nk ? 0u : nk - k4 >= 4 ? 0xFu : (1u << (nk - k4)) - 1u;
+            }
+            if (FAST || live) reg[u] = cols_gather4<VEC4>(v, m, k4, live);
+            else reg[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    __device__ void store(float* lds, int u0 = 0, int u1 = NU) const {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            if (u < u0 || u >= u1) continue;
+            const int id = t + u * NT;
+            if constexpr (!TURNED) {
+                *(f32x4*)(lds + (id / KV) * PITCH + (id % KV) * 4) = reg[u];
+            } else {
+                float* dst = lds + (id % KV) * 4 * PITCH + id / KV;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e * PITCH] = reg[u][e];
+            }
+        }
+    }
+};
+
 template <class T> struct Mma;
 template <> struct Mma<bf16_t> {
     static __device__ void run(const u32x4& a, const u32x4& b, f32x16& c) {
@@ -358,11 +462,14 @@ __device__ __forceinline__ TilePos tile_of_block(const GemmArgs& g) {
 // reduction of a few k-tiles only (a convolution's input gradient, [100352,64]x[64,576]): as one block per output tile
 // such a product is 14112 short blocks, each of which pays the full memory latency for two k-tiles of work, and the four
 // blocks a CU holds do not cover it.  The launch has as many blocks as the chip holds at once, with equal shares.
-template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false>
-__device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem) {
+// XCOLS (f32): X is the column matrix of a convolution (XR) or its transpose (!XR), gathered from the input (ColsView);
+// 2: four at a time (see cols_gather4), 1: one by one.
+template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false, int XCOLS = 0>
+__device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem, const ColsView* cv = nullptr) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
     constexpr bool SWZ = Cfg::TS == 16;
-    using SX = Stager<T, XR, TM, NT, SWZ>;
+    static_assert(!XCOLS || (std::is_same<T, float>::value && !PANEL), "the gathered operand is f32, one tile per block");
+    using SX = typename std::conditional<XCOLS != 0, ColsStager<!XR, XCOLS == 2, TM, NT>, Stager<T, XR, TM, NT, SWZ>>::type;
     using SY = Stager<T, YR, TN, NT, SWZ>;
     constexpr int VEC = Elem<T>::VEC;
     constexpr int TK = SX::TK;
@@ -407,15 +514,20 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
     auto red_of = [&](uint32_t q) { return rb + (PANEL ? q % nk1 : q) * TK; };
     auto row_of = [&](uint32_t q) { return PANEL ? ((pos.ti + q / nk1) / g.tiles_j) * (uint32_t)TM : i0; };
     auto col_of = [&](uint32_t q) { return PANEL ? ((pos.ti + q / nk1) % g.tiles_j) * (uint32_t)TN : j0; };
+    // units [u0, u1) of the X tile at (row, red) into the registers of stager st
+    auto load_x = [&](SX& st, uint32_t row, uint32_t red, int u0, int u1) {
+        if constexpr (XCOLS) st.template load_cols<FAST>(*cv, row, red, g.I, re, u0, u1);
+        else st.template load<FAST>(X, g.xi, g.xr, row, red, g.I, re, u0, u1);
+    };
     {
         // tiles 0 and 1 are requested together (one memory latency instead of two); the accumulators are
         // not live yet, so the second set of staging registers costs nothing
         SX sx0;
         SY sy0;
-        sx0.template load<FAST>(X, g.xi, g.xr, row_of(0), rb, g.I, re);
+        load_x(sx0, row_of(0), rb, 0, SX::NU);
         sy0.template load<FAST>(Y, g.yj, g.yr, col_of(0), rb, g.J, re);
         const uint32_t q1 = nk > 1 ? 1u : 0u;
-        sx.template load<FAST>(X, g.xi, g.xr, row_of(q1), red_of(q1), g.I, re);
+        load_x(sx, row_of(q1), red_of(q1), 0, SX::NU);
         sy.template load<FAST>(Y, g.yj, g.yr, col_of(q1), red_of(q1), g.J, re);
         sx0.store(lds_x);
         sy0.store(lds_y);
@@ -491,7 +603,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
                 const int y0 = SY::NU * s / (S - 1), y1 = SY::NU * (s + 1) / (S - 1);
                 sx.store(nx, x0, x1);
                 sy.store(ny, y0, y1);
-                sx.template load<FAST>(X, g.xi, g.xr, ni, nt, g.I, re, x0, x1);
+                load_x(sx, ni, nt, x0, x1);
                 sy.template load<FAST>(Y, g.yj, g.yr, nj, nt, g.J, re, y0, y1);
                 read_frags(s + 1, cx, cy);
             } else {
@@ -568,8 +680,22 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     gemm_mfma_body<T, XR, YR, Cfg, false>(g, pos, smem);
 }
 
-template <class T, bool XR, bool YR, class Cfg, bool FAST>
-void launch_mfma_impl(GemmArgs g) {
+template <bool XR, bool YR, class Cfg, bool ALIGNED, bool VEC4>
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_cols_kernel(GemmArgs g, ColsView v) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const TilePos pos = tile_of_block(g);
+    if constexpr (ALIGNED) {
+        if ((pos.ti + 1) * Cfg::TM <= g.I && (pos.tj + 1) * Cfg::TN <= g.J) {
+            gemm_mfma_body<float, XR, YR, Cfg, true, false, VEC4 ? 2 : 1>(g, pos, smem, &v);
+            return;
+        }
+    }
+    gemm_mfma_body<float, XR, YR, Cfg, false, false, VEC4 ? 2 : 1>(g, pos, smem, &v);
+}
+
+// cv: X is the gathered column matrix of a convolution (f32), see ColsView
+template <class T, bool XR, bool YR, class Cfg, bool FAST, int XCOLS = 0>
+void launch_mfma_impl(GemmArgs g, const ColsView* cv = nullptr) {
     using SX = Stager<T, XR, Cfg::TM, Cfg::NT, Cfg::TS == 16>;
     constexpr size_t lds_bytes = (size_t)2 * (Cfg::TM + Cfg::TN) * SX::PITCH * sizeof(T);
     constexpr uint32_t TK = TK_BYTES / sizeof(T);
@@ -596,6 +722,27 @@ void launch_mfma_impl(GemmArgs g) {
     if (g.splits > 1) {
         g.part = (float*)scratch(n_out * g.splits * sizeof(float));
         if (!g.part) return;
+    }
+    if constexpr (XCOLS != 0) {
+        {
+            auto ck = gemm_mfma_cols_kernel<XR, YR, Cfg, FAST, XCOLS == 2>;
+            if (lds_bytes > (64u << 10)) {
+                static bool allowed[64] = {false};     // per instantiation, indexed by device
+                int dev = 0;
+                MXH_HIP(hipGetDevice(&dev));
+                if (dev < 0 || dev >= 64 || !allowed[dev]) {
+                    MXH_HIP(hipFuncSetAttribute((const void*)ck, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+                    if (dev >= 0 && dev < 64) allowed[dev] = true;
+                }
+            }
+            hipLaunchKernelGGL(ck, dim3((unsigned)blocks), dim3(Cfg::NT), lds_bytes, stream(), g, *cv);
+            MXH_LAUNCH_CHECK("gemm_mfma_cols");
+            if (g.splits > 1) {
+                hipLaunchKernelGGL(gemm_fold_kernel<T>, dim3((unsigned)cdiv(n_out, 256)), dim3(256), 0, stream(), g.part, (T*)g.out, n_out, g.splits);
+                MXH_LAUNCH_CHECK("gemm_fold");
+            }
+            return;
+        }
     }
     if constexpr (FAST && std::is_same<Cfg, typename Cfgs<T>::Tall>::value) {
         // a reduction of a few k-tiles, many whole tiles: as many blocks as the chip holds, each with a run of tiles (see PANEL)
@@ -787,9 +934,73 @@ void gemm_dispatch(GemmArgs g) {
 #undef MXH_GEMM_CASE
 }
 
+// The Conv2d layer's two products with the column matrix, the matrix gathered from the input instead of stored.
+//   transposed == 0: out[M, n] = cols x rhs,    rhs [K, n]      (forward: nn/layers/conv.rs:222)
+//   transposed != 0: out[K, n] = cols^T x rhs,  rhs [M, n]      (weight gradient: conv.rs:279)
+// with M = B*oh*ow, K = C*kh*kw; md as conv2d_im2col reads it; rs: element strides of rhs (one of them 1).
+static void cols_matmul(const size_t* md, int transposed, const float* in, const float* rhs, size_t n, const size_t* rs, float* out) {
+    if (!md || !rs) { set_status(ERR_INVALID, "conv2d_cols_matmul: null metadata"); return; }
+    const size_t B = md[0], C = md[1], H = md[2], W = md[3], kh = md[4], kw = md[5], oh = md[6], ow = md[7];
+    const size_t ph = md[8], pw = md[9], sh = md[10], sw = md[11];
+    const size_t M = B * oh * ow, K = C * kh * kw;
+    if (M == 0 || K == 0 || n == 0) return;
+    if (!in || !rhs || !out) { set_status(ERR_INVALID, "conv2d_cols_matmul: null buffer"); return; }
+    if (H == 0 || W == 0) { set_status(ERR_INVALID, "conv2d_cols_matmul: empty input plane"); return; }
+    const size_t lim = (size_t)1 << 31;
+    if (M * K >= lim || B * C * H * W >= lim || n >= lim || ph >= lim || pw >= lim || sh * oh >= lim || sw * ow >= lim) {
+        set_status(ERR_TOO_LARGE, "conv2d_cols_matmul: 2^31 or more entries");
+        return;
+    }
+    if (rs[0] != 1 && rs[1] != 1) { set_status(ERR_UNSUPPORTED, "conv2d_cols_matmul: rhs needs a unit stride"); return; }
+    if (prog_recording()) prog_abandon();
+    ColsView v;
+    v.in = in;
+    v.K = (uint32_t)K; v.P = (uint32_t)(oh * ow);
+    v.H = (uint32_t)H; v.W = (uint32_t)W; v.HW = (uint32_t)(H * W); v.CHW = (uint32_t)(C * H * W);
+    v.sh = (uint32_t)sh; v.sw = (uint32_t)sw; v.ph = (int32_t)ph; v.pw = (int32_t)pw;
+    v.d_P = make_fastdiv(v.P); v.d_khkw = make_fastdiv((uint32_t)(kh * kw));
+    v.d_kw = make_fastdiv((uint32_t)kw); v.d_ow = make_fastdiv((uint32_t)ow);
+    const bool vec4 = K % 4 == 0 && ow % 4 == 0;            // (then P % 4 == 0 as well)
+    GemmArgs g;
+    std::memset((void*)&g, 0, sizeof(g));
+    g.X = in;                      // not addressed through the strides below: the tiles are gathered
+    g.Y = rhs;
+    g.out = out;
+    g.batch = 1;
+    g.J = (uint32_t)n;
+    g.yr = (int64_t)rs[0]; g.yj = (int64_t)rs[1];
+    if (!transposed) { g.I = (uint32_t)M; g.R = (uint32_t)K; g.xi = (int64_t)K; g.xr = 1; }
+    else { g.I = (uint32_t)K; g.R = (uint32_t)M; g.xi = 1; g.xr = (int64_t)K; }
+    // the choices gemm_dispatch makes for a stored matrix of this shape, so that both ways are the same arithmetic
+    constexpr uint32_t TK = TK_BYTES / sizeof(float);
+    const bool tall = g.I >= 128 && (g.J <= 64 || g.R <= 4 * TK);
+    const bool yr = g.yr == 1;
+    auto fast_of = [&](int rows_y) {
+        const bool span = g.yj >= 0 && g.yr >= 0 && ((int64_t)rows_y * g.yj + (int64_t)TK * g.yr) * 4 < (1ll << 31);
+        const bool y_ok = yr ? ((uintptr_t)g.Y % 16 == 0 && g.yj % 4 == 0) : true;
+        return span && y_ok && g.R % TK == 0 && g.J % 4 == 0 && (uintptr_t)g.out % 16 == 0;
+    };
+    // (one by one only with the checked body: odd widths are not the shapes to tune for)
+#define MXH_COLS_CASE(XR, YR, CFG)                                                                  \
+    (!vec4 ? launch_mfma_impl<float, XR, YR, CFG, false, 1>(g, &v)                                  \
+           : fast_of(CFG::TN) ? launch_mfma_impl<float, XR, YR, CFG, true, 2>(g, &v) : launch_mfma_impl<float, XR, YR, CFG, false, 2>(g, &v))
+    using TallCfg = Cfgs<float>::Tall;
+    using SmallCfg = Cfgs<float>::Small;
+#define MXH_COLS_CFG(XR, YR) (tall ? MXH_COLS_CASE(XR, YR, TallCfg) : MXH_COLS_CASE(XR, YR, SmallCfg))
+    if (!transposed) { if (yr) MXH_COLS_CFG(true, true); else MXH_COLS_CFG(true, false); }
+    else { if (yr) MXH_COLS_CFG(false, true); else MXH_COLS_CFG(false, false); }
+#undef MXH_COLS_CFG
+#undef MXH_COLS_CASE
+}
+
 }  // namespace mxh
 
 using namespace mxh;
+
+extern "C" void hip_conv2d_cols_matmul_f32(const size_t* metadata, int transposed, const float* input, const float* rhs, size_t n,
+                                           const size_t* rhs_strides, float* out) { MXH_API;
+    cols_matmul(metadata, transposed, input, rhs, n, rhs_strides, out);
+}
 
 #define MXH_MATMUL_FOR(T, SUF)                                                                              \
     extern "C" void hip_matmul_##SUF(size_t num_els, const size_t* md, const T* a, const T* b, T* c) { MXH_API; \

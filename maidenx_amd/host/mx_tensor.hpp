@@ -230,6 +230,11 @@ template <class B> struct GradCell {
 inline size_t& backend_calls() { static size_t n = 0; return n; }
 // Conv2d backward: make only the rows of grad_cols that col2im reads (see Conv2d); false = the whole product.
 inline bool& conv_skip_unread_grad_cols() { static bool on = true; return on; }
+// Conv2d on a backend that has the product with the gathered column matrix (the matrix is never stored): 0 = store
+// the matrix with im2col and multiply that, as the reference does; 1 = gather when no backward is recorded (the
+// forward alone is faster gathered, a training step is faster with the one stored matrix serving both products);
+// 2 = gather in forward and backward (no buffer of B*oh*ow x C*kh*kw elements lives between the two).
+inline int& conv_gathered_products() { static int mode = 1; return mode; }
 // Count of whole-buffer dtype conversions (with_dtype: a host loop in the reference, a kernel here).
 inline size_t& cast_calls() { static size_t n = 0; return n; }
 
@@ -1108,17 +1113,34 @@ struct Conv2d {                                                                 
         const size_t Bn = input.shape()[0], C = input.shape()[1], H = input.shape()[2], W = input.shape()[3];
         const size_t oh = (H + 2 * ph - kh) / sh + 1, ow = (W + 2 * pw - kw) / sw + 1;
         const size_t kh_ = kh, kw_ = kw, sh_ = sh, sw_ = sw, ph_ = ph, pw_ = pw;
-        // im2col (conv.rs:333-376); the input buffer is passed from its start, as the reference passes it
-        T cols = T::empty({Bn * oh * ow, C * kh * kw});
-        {
-            auto md = conv_meta(Bn, C, H, W, kh, kw, oh, ow, sh, sw, ph, pw);
+        const Shape& ws = weight.shape();
+        T wm = weight.reshape(Shape{ws[0], ws[1] * ws[2] * ws[3]});
+        const auto md = conv_meta(Bn, C, H, W, kh, kw, oh, ow, sh, sw, ph, pw);
+        const size_t M = Bn * oh * ow, K = C * kh * kw;
+        // Whether the two products with the column matrix gather its entries from the input instead of reading a stored
+        // copy (the same tiles and the same order of additions): the backend has the call, the index space fits it, and
+        // the weight matrix is the [Cout, K] it is multiplied with.
+        bool gathered = false;
+        if constexpr (B::has_cols_matmul)
+            gathered = (conv_gathered_products() == 2 || (conv_gathered_products() == 1 && !input.requires_grad)) && M && K && ws[0] && M * K < ((size_t)1 << 31) && input.size() < ((size_t)1 << 31) &&
+                       ws[1] == C && ws[2] == kh && ws[3] == kw && (wm.strides()[0] == 1 || wm.strides()[1] == 1);
+        T cols, out;
+        if (gathered) {
+            if constexpr (B::has_cols_matmul) {
+                out = T::empty({M, ws[0]});
+                const size_t rs[2] = {wm.strides()[1], wm.strides()[0]};                  // of wm^T: [K, Cout]
+                B::cols_matmul(md.data(), 0, input.f32(), wm.f32() + wm.offset(), ws[0], rs, out.f32());
+                ++backend_calls();
+                B::check();
+            }
+        } else {
+            // im2col (conv.rs:333-376); the input buffer is passed from its start, as the reference passes it
+            cols = T::empty({M, K});
             B::im2col(cols.size(), md.data(), input.f32(), cols.f32());
             ++backend_calls();
             B::check();
+            out = cols.matmul(wm.transpose(-1, -2));
         }
-        const Shape& ws = weight.shape();
-        T wm = weight.reshape(Shape{ws[0], ws[1] * ws[2] * ws[3]});
-        T out = cols.matmul(wm.transpose(-1, -2));
         out = out.reshape(std::vector<long>{(long)Bn, (long)oh, (long)ow, -1});
         out = out.transpose(1, 3).transpose(2, 3);
         if (has_bias) out = out.add(bias.reshape(Shape{1, bias.shape()[0], 1, 1}));
@@ -1163,7 +1185,25 @@ struct Conv2d {                                                                 
                     grads.push_back(T::zeros_like(x));
                 }
                 if (w.requires_grad) {
-                    T gw = cols.transpose(-1, -2).matmul(grad_flat);
+                    T gw;
+                    if (gathered && (grad_flat.strides()[0] == 1 || grad_flat.strides()[1] == 1)) {
+                        if constexpr (B::has_cols_matmul) {
+                            gw = T::empty({K, grad_flat.shape()[1]});
+                            const size_t rs[2] = {grad_flat.strides()[0], grad_flat.strides()[1]};
+                            B::cols_matmul(md.data(), 1, x.f32(), grad_flat.f32() + grad_flat.offset(), grad_flat.shape()[1], rs, gw.f32());
+                            ++backend_calls();
+                            B::check();
+                        }
+                    } else {
+                        T stored = cols;
+                        if (gathered) {                      // (a gradient the call cannot take: store the matrix after all)
+                            stored = T::empty({M, K});
+                            B::im2col(stored.size(), md.data(), x.f32(), stored.f32());
+                            ++backend_calls();
+                            B::check();
+                        }
+                        gw = stored.transpose(-1, -2).matmul(grad_flat);
+                    }
                     grads.push_back(gw.reshape(Shape{w.shape()[0], w.shape()[1], kh_, kw_}));
                 } else {
                     grads.push_back(T::zeros_like(w));

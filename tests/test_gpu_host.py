@@ -133,6 +133,46 @@ def test_conv2d_backward_makes_only_the_rows_of_grad_cols_that_col2im_reads(mx_h
         np.testing.assert_array_equal(lead[key].view(np.uint32), whole[key].view(np.uint32), err_msg=key)
 
 
+@pytest.mark.parametrize("B,Cin,H,W,Cout,k,stride,pad", [(2, 3, 6, 5, 4, 3, 1, 1), (1, 2, 7, 7, 3, 3, 2, 2), (4, 16, 14, 14, 32, 3, 1, 1),
+                                                         (8, 64, 28, 28, 64, 3, 1, 1)])
+def test_conv2d_with_the_column_matrix_stored_or_gathered(mx_hip, B, Cin, H, W, Cout, k, stride, pad):
+    """The layer multiplies the column matrix without storing it (hip_conv2d_cols_matmul_f32, mode 2) or stores it with
+    im2col first as the reference does (mode 0): the same numbers within the f32 matmul tolerance everywhere, and the same
+    bits where both products run on the matrix cores (the two larger cases).  By default (mode 1) a forward without a
+    recorded backward gathers, a recorded one stores."""
+    x, w, b = conv_inputs(B, Cin, H, W, Cout, k, seed=B * 7 + W)
+    oh, ow = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    target = np.random.default_rng(8).standard_normal((B, Cout, oh, ow)).astype(np.float32)
+    try:
+        mx_hip.set_conv_gathered_products(0)
+        mx_hip.reset_backend_calls()
+        stored = conv_step(mx_hip, x, w, b, stride, pad, target)
+        calls_stored = mx_hip.backend_calls()
+        mx_hip.set_conv_gathered_products(2)
+        mx_hip.reset_backend_calls()
+        gathered = conv_step(mx_hip, x, w, b, stride, pad, target)
+        calls_gathered = mx_hip.backend_calls()
+        # the default: gathered exactly when no backward is recorded
+        mx_hip.set_conv_gathered_products(1)
+        conv = mx_hip.Conv2d(mx_hip.tensor(w), mx_hip.tensor(b), stride=(stride, stride), padding=(pad, pad))
+        mx_hip.reset_backend_calls()
+        plain = conv.forward(mx_hip.tensor(x)).numpy()
+        calls_plain = mx_hip.backend_calls()
+        mx_hip.reset_backend_calls()
+        conv.forward(mx_hip.tensor(x).with_grad())
+        calls_recorded = mx_hip.backend_calls()
+    finally:
+        mx_hip.set_conv_gathered_products(1)
+    assert calls_recorded == calls_plain + 1            # im2col, then the product
+    np.testing.assert_array_equal(plain.view(np.uint32), gathered["out"].view(np.uint32))
+    assert calls_gathered == calls_stored - 1           # no im2col
+    for key in ("out", "loss", "grad_b", "grad_w", "grad_x"):
+        scale = np.abs(stored[key]).max() + 1e-30
+        assert np.abs(gathered[key] - stored[key]).max() <= 2e-5 * scale, key
+        if B * oh * ow >= 128 and Cout >= 32:
+            np.testing.assert_array_equal(gathered[key].view(np.uint32), stored[key].view(np.uint32), err_msg=key)
+
+
 def test_graph_replayed_training_equals_eager(mx_hip):
     """mxt_train records the step as a HIP graph and replays it; every run is compared with the eager loop, with
     eager work and synchronisations in between (the same graph machinery is set up and torn down each time)."""

@@ -692,6 +692,63 @@ def test_im2col_col2im_bit_exact(oracle, hip, case, dt):
         assert same_bits(o, h), num_els
 
 
+# (B, C, H, W, kh, kw, pad, stride): ragged tiles, odd widths (element-by-element gather), planes shorter than a tile's
+# run of rows, stride 2, whole 64-wide tiles with a 576-term reduction, a reduction long enough for the split
+COLS_CASES = CONV_CASES[:7] + [(2, 3, 16, 16, 3, 3, 1, 1), (1, 2, 9, 16, 2, 4, 1, 1), (4, 16, 14, 14, 3, 3, 1, 1), (2, 8, 16, 20, 3, 3, 1, 1),
+                               (2, 5, 12, 13, 3, 3, 1, 1), (3, 4, 23, 23, 3, 3, 2, 2), (8, 64, 28, 28, 3, 3, 1, 1), (2, 64, 56, 56, 3, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("rhs_turned", [False, True])
+@pytest.mark.parametrize("transposed", [0, 1])
+@pytest.mark.parametrize("n", [64, 24])
+@pytest.mark.parametrize("case", COLS_CASES, ids=lambda c: "_".join(map(str, c)))
+def test_conv2d_cols_matmul(oracle, hip, case, n, transposed, rhs_turned):
+    """The product of the (never stored) column matrix, or of its transpose, with a matrix: against the oracle's im2col
+    followed by its matmul, against float64, and bit for bit against the stored way (hip im2col, then hip matmul)
+    wherever that runs on the matrix cores too."""
+    B, Cc, H, W, kh, kw, p, s = case
+    oh, ow = (H + 2 * p - kh) // s + 1, (W + 2 * p - kw) // s + 1
+    M, K = B * oh * ow, Cc * kh * kw
+    r = rng(73)
+    x = r.standard_normal(B * Cc * H * W).astype(np.float32)
+    md = meta_conv(B, Cc, H, W, kh, kw, oh, ow, p, p, s, s)
+    rows = M if transposed else K                      # of rhs; out is [K, n] or [M, n]
+    I = K if transposed else M
+    rhs = r.standard_normal((rows, n)).astype(np.float32)
+    st = np.ascontiguousarray(rhs.T) if rhs_turned else rhs          # storage; rhs[i, j] at i*rs[0] + j*rs[1]
+    rs = u64(1, rows) if rhs_turned else u64(n, 1)
+    (h,) = hip.call("conv2d_cols_matmul_f32", md, transposed, In(x), In(st.ravel()), n, rs, Out(I * n, "f32"))
+    (cols,) = oracle.call("conv2d_im2col_f32", M * K, md, In(x), Out(M * K, "f32"))
+    a = cols.reshape(M, K).T if transposed else cols.reshape(M, K)
+    truth = a.astype(np.float64) @ rhs.astype(np.float64)
+    scale = np.abs(a).astype(np.float64) @ np.abs(rhs).astype(np.float64)
+    err = np.abs(h.reshape(I, n) - truth) / np.maximum(scale, 1e-30)
+    assert np.max(err) <= 1e-5, float(np.max(err))
+    a_str, b_str = ([1, K] if transposed else [K, 1]), [int(rs[0]), int(rs[1])]
+    mm = meta_matmul([I, n], [I, rows], [rows, n], a_str, b_str)
+    if I * n * rows <= 5_000_000:
+        (o,) = oracle.call("matmul_f32", I * n, mm, In(cols), In(st.ravel()), Out(I * n, "f32"))
+        assert np.max(np.abs(o - h).reshape(I, n) / np.maximum(scale, 1e-30)) <= 2e-5
+    (hc,) = hip.call("conv2d_im2col_f32", M * K, md, In(x), Out(M * K, "f32"))
+    assert same_bits(hc, cols)
+    (hs,) = hip.call("matmul_f32", I * n, mm, In(hc), In(st.ravel()), Out(I * n, "f32"))
+    outputs = I * n
+    on_matrix_cores = rows > 16 and not (I < 16 and n < 16 and rows < 256) and not (outputs <= 64 and rows >= 4096) and \
+        not (outputs <= 4096 and (I < 32 or n < 32))
+    if on_matrix_cores:
+        assert same_bits(hs, h)
+
+
+def test_conv2d_cols_matmul_rejects_what_it_cannot_index(hip):
+    x = np.zeros(16, np.float32)
+    md = meta_conv(1, 1, 4, 4, 3, 3, 4, 4, 1, 1, 1, 1)
+    with pytest.raises(hip.L.HipError, match="unit stride"):
+        hip.call("conv2d_cols_matmul_f32", md, 0, In(x), In(np.zeros(64, np.float32)), 2, u64(4, 2), Out(32, "f32"))
+    big = meta_conv(1 << 12, 64, 64, 64, 3, 3, 64, 64, 1, 1, 1, 1)       # a column matrix of 2^31 entries and more
+    with pytest.raises(hip.L.HipError, match="2\\^31"):
+        hip.call("conv2d_cols_matmul_f32", big, 0, In(x), In(np.zeros(64, np.float32)), 2, u64(2, 1), Out(32, "f32"))
+
+
 @pytest.mark.parametrize("dt", DTS + ["f64"])
 @pytest.mark.parametrize("k", [3, 4])
 def test_col2im_row_stride_two_column_stride_one(oracle, hip, k, dt):
