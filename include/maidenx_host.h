@@ -115,6 +115,11 @@ int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_
  * epoch eager; mxt_last_train_replayed() tells how many epochs of the last mxt_train call were replays. */
 void mxt_set_graph_replay(int enabled);
 size_t mxt_last_train_replayed(void);
+/* backward() leaves out three things that cannot change a bit of any gradient (enabled = 0: does them all, as the
+ * reference does): the gradient of a binary op's operand that requires none (computed and dropped in the reference,
+ * crates/maidenx_tensor/src/lib.rs:93-111), x.pow(1) in the backward of pow(2), and the zero fill in front of the first
+ * accumulation when the gradient is a broadcast view. */
+void mxt_set_autograd_shortcuts(int enabled);
 /* Conv2d backward (nn/layers/conv.rs:253-268): col2im is handed num_els = B*C*H*W and reads no entry of grad_cols at
  * or beyond that flat index (crates/maidenx_cpu/src/nn/conv.rs:135), so by default only the leading
  * ceil(B*C*H*W / (C*kh*kw)) rows of grad_cols are computed; the input gradient is the same bytes either way.

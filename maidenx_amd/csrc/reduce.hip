@@ -554,6 +554,21 @@ void sum_to_shape(size_t num_els, size_t num_dims, const size_t* md, const T* in
     bool any_red = false;
     int nred_groups = 0;
     for (int g = 0; g < ng; ++g) { any_red |= g_red[g]; nred_groups += g_red[g]; }
+    if (!cont && !any_red) {
+        // identity on a strided view (a broadcast gradient being accumulated for the first time): when no source index
+        // reaches num_els the reference's wrap-around (see sts_gather_kernel) never applies, and out = 0 + view is one
+        // elementwise pass over the view's own strides instead of a gathered copy followed by that pass
+        size_t last = offset;
+        for (size_t d = 0; d < num_dims; ++d) last += (in_dims[d] - 1) * in_strides[d];
+        if (last < num_els) {
+            size_t cs[64];
+            contiguous_strides(num_dims, in_dims, cs);
+            const size_t* ins[1] = {in_strides};
+            const void* inp[1] = {src + offset};
+            ew_launch<OpZeroPlus<T>>(num_els, num_dims, in_dims, cs, ins, out, inp, OpZeroPlus<T>{});
+            return;
+        }
+    }
     // Temporaries (slot 1 of the library scratch; the stage drivers' partials use slot 0):
     // [gathered contiguous copy | ping | pong]
     T* gathered = nullptr;

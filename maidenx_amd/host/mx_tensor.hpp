@@ -235,6 +235,12 @@ inline bool& conv_skip_unread_grad_cols() { static bool on = true; return on; }
 // forward alone is faster gathered, a training step is faster with the one stored matrix serving both products);
 // 2 = gather in forward and backward (no buffer of B*oh*ow x C*kh*kw elements lives between the two).
 inline int& conv_gathered_products() { static int mode = 1; return mode; }
+// Three things backward() leaves out without changing a bit of any gradient (false: do all of them, as the reference
+// does): the gradient of a binary op's operand that does not require one (the reference computes it and drops it,
+// lib.rs:93-111), x.pow(1) in the backward of pow(2) (x itself), and the zero-filled buffer that the first gradient
+// of a tensor is added into when that gradient is a broadcast view (0 + g is written straight away, as for a contiguous
+// gradient).
+inline bool& autograd_shortcuts() { static bool on = true; return on; }
 // Count of whole-buffer dtype conversions (with_dtype: a host loop in the reference, a kernel here).
 inline size_t& cast_calls() { static size_t n = 0; return n; }
 
@@ -358,7 +364,15 @@ struct Tensor {
     }
     void accumulate_grad(const T& g) const {                                        // lib.rs:221-241
         if (!has_grad()) return;
-        if (!grad_cell->g && g.dtype == grad_cell->dtype && g.is_contiguous() && g.shape() == grad_cell->shape) {
+        // (a view qualifies when every element it addresses lies inside the first size() elements of its buffer: the
+        // strided sum_to_shape kernel wraps source indices at num_els, reduction.rs:112-140, and must not get to)
+        auto inside = [](const T& v) {
+            size_t last = v.offset();
+            for (size_t i = 0; i < v.ndim(); ++i) last += (v.shape()[i] ? v.shape()[i] - 1 : 0) * v.strides()[i];
+            return last < v.size();
+        };
+        if (!grad_cell->g && g.dtype == grad_cell->dtype && g.shape() == grad_cell->shape &&
+            (g.is_contiguous() || (autograd_shortcuts() && g.size() && inside(g)))) {
             T fresh = empty(grad_cell->shape, g.dtype);
             auto md = meta_to_shape(g, g.shape());
             by_dtype(g.dtype, "accumulate_grad", [&](auto tag) {
@@ -479,14 +493,16 @@ struct Tensor {
         B::check();
         return result;
     }
+    // backward_tracking only looks at the gradient of an input that requires one
+    static bool wanted(const std::vector<T>& inputs, size_t i) { return !autograd_shortcuts() || inputs[i].requires_grad; }
     T add(const T& rhs) const {                                                     // ops/binary.rs:11-60
         T l, r;
         T result = binary_forward(rhs, ADD, l, r);
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
-            result.set_node("add", {*this, rhs}, [ls, rs](const std::vector<T>&, const T& go) {
-                return std::vector<T>{go.sum_to_shape(ls), go.sum_to_shape(rs)};
+            result.set_node("add", {*this, rhs}, [ls, rs](const std::vector<T>& in, const T& go) {
+                return std::vector<T>{wanted(in, 0) ? go.sum_to_shape(ls) : T(), wanted(in, 1) ? go.sum_to_shape(rs) : T()};
             });
         }
         return result;
@@ -497,8 +513,8 @@ struct Tensor {
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
-            result.set_node("sub", {*this, rhs}, [ls, rs](const std::vector<T>&, const T& go) {
-                return std::vector<T>{go.sum_to_shape(ls), go.neg().sum_to_shape(rs)};
+            result.set_node("sub", {*this, rhs}, [ls, rs](const std::vector<T>& in, const T& go) {
+                return std::vector<T>{wanted(in, 0) ? go.sum_to_shape(ls) : T(), wanted(in, 1) ? go.neg().sum_to_shape(rs) : T()};
             });
         }
         return result;
@@ -509,8 +525,8 @@ struct Tensor {
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
-            result.set_node("mul", {*this, rhs}, [ls, rs, l, r](const std::vector<T>&, const T& go) {
-                return std::vector<T>{go.mul(r).sum_to_shape(ls), go.mul(l).sum_to_shape(rs)};
+            result.set_node("mul", {*this, rhs}, [ls, rs, l, r](const std::vector<T>& in, const T& go) {
+                return std::vector<T>{wanted(in, 0) ? go.mul(r).sum_to_shape(ls) : T(), wanted(in, 1) ? go.mul(l).sum_to_shape(rs) : T()};
             });
         }
         return result;
@@ -521,8 +537,9 @@ struct Tensor {
         if (requires_grad || r.requires_grad) {
             result.with_grad();
             Shape ls = shape(), rs = rhs.shape();
-            result.set_node("div", {*this, rhs}, [ls, rs, l, r](const std::vector<T>&, const T& go) {
-                return std::vector<T>{go.div(r).sum_to_shape(ls), go.mul(l).div(r.square()).neg().sum_to_shape(rs)};
+            result.set_node("div", {*this, rhs}, [ls, rs, l, r](const std::vector<T>& in, const T& go) {
+                return std::vector<T>{wanted(in, 0) ? go.div(r).sum_to_shape(ls) : T(),
+                                      wanted(in, 1) ? go.mul(l).div(r.square()).neg().sum_to_shape(rs) : T()};
             });
         }
         return result;
@@ -680,7 +697,8 @@ struct Tensor {
             result.with_grad();
             T input = *this;
             result.set_node("pow", {*this}, [input, e](const std::vector<T>&, const T& go) {
-                return std::vector<T>{go.mul_scalar(e).mul(input.pow(e - 1.0f))};
+                // (powf(x, 1) is x)
+                return std::vector<T>{go.mul_scalar(e).mul(autograd_shortcuts() && e - 1.0f == 1.0f ? input : input.pow(e - 1.0f))};
             });
         }
         return result;

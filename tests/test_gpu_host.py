@@ -114,6 +114,56 @@ def test_conv2d_forward_backward(mx_hip, mx_oracle, B, Cin, H, W, Cout, k, strid
         assert np.abs(got[key] - num[key]).max() <= 1e-4 * scale, key
 
 
+def _shortcut_programs(mx):
+    """Programs whose backward passes contain what the shortcuts leave out: operands without a gradient, pow(2),
+    gradients that arrive as broadcast views (sum over dims, a broadcast operand, the MSE loss)."""
+    out = {}
+    rng = np.random.default_rng(12)
+    a = rng.standard_normal((6, 5, 4)).astype(np.float32)
+    b = (rng.standard_normal((1, 5, 1)) + 3.0).astype(np.float32)
+    for op in ("add", "sub", "mul", "div"):
+        for ga, gb in ((True, False), (False, True), (True, True)):
+            ta, tb = mx.tensor(a), mx.tensor(b)
+            if ga:
+                ta = ta.with_grad()
+            if gb:
+                tb = tb.with_grad()
+            z = getattr(ta, op)(tb).pow(2.0).sum_all()
+            z.backward()
+            key = f"{op}_{int(ga)}{int(gb)}"
+            out[key + "_z"] = z.numpy()
+            if ga:
+                out[key + "_ga"] = ta.grad().numpy()
+            if gb:
+                out[key + "_gb"] = tb.grad().numpy()
+    x, w, bias = conv_inputs(2, 3, 6, 5, 4, 3, seed=21)
+    target = rng.standard_normal((2, 4, 6, 5)).astype(np.float32)
+    for k, v in conv_step(mx, x, w, bias, 1, 1, target).items():
+        out["conv_" + k] = v
+    for k, v in mlp_run(mx, 3, n=200).items():
+        out["mlp_" + k] = v
+    return out
+
+
+def test_backward_shortcuts_change_no_bit(mx_hip):
+    mx = mx_hip
+    try:
+        mx.set_autograd_shortcuts(False)
+        mx.reset_backend_calls()
+        whole = _shortcut_programs(mx)
+        calls_whole = mx.backend_calls()
+        mx.set_autograd_shortcuts(True)
+        mx.reset_backend_calls()
+        short = _shortcut_programs(mx)
+        calls_short = mx.backend_calls()
+    finally:
+        mx.set_autograd_shortcuts(True)
+    assert calls_short < calls_whole
+    assert whole.keys() == short.keys()
+    for key in whole:
+        np.testing.assert_array_equal(np.asarray(short[key]).view(np.uint32), np.asarray(whole[key]).view(np.uint32), err_msg=key)
+
+
 @pytest.mark.parametrize("B,Cin,H,W,Cout,k,stride,pad", [(2, 3, 6, 5, 4, 3, 1, 1), (3, 4, 5, 5, 2, 1, 1, 1), (4, 16, 14, 14, 32, 3, 1, 1),
                                                          (8, 64, 28, 28, 64, 3, 1, 1)])
 def test_conv2d_backward_makes_only_the_rows_of_grad_cols_that_col2im_reads(mx_hip, B, Cin, H, W, Cout, k, stride, pad):

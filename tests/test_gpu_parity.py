@@ -430,6 +430,24 @@ def test_sum_to_shape_strided_input(oracle, hip):
         assert np.allclose(o, h, rtol=1e-5, atol=1e-5), out_shape
 
 
+@pytest.mark.parametrize("dt", DTS)
+def test_sum_to_shape_identity_on_strided_views(oracle, hip, dt):
+    """out = 0 + view for views that stay below num_els (one elementwise pass over the view's strides) and for one whose
+    indices pass num_els, where the reference's modulo applies (reduction.rs:162-167): the same bits as the oracle."""
+    r = rng(83)
+    cases = [([40, 30], [0, 1], 0, 40 * 30), ([40, 30], [1, 0], 0, 40 * 30), ([6, 40, 30], [0, 30, 1], 0, 6 * 40 * 30),
+             ([30, 40], [1, 30], 0, 30 * 40),                      # a transposed view: its last index is num_els - 1
+             ([30, 40], [1, 32], 0, 30 * 40 + 64),                 # rows 32 apart: indices reach 1277 >= 1200, wrapped
+             ([8192, 512], [0, 1], 0, 8192 * 512)]                 # a broadcast row as large as a gradient
+    for dims, strides, off, size in cases:
+        n = int(np.prod(dims))
+        st = to_storage(r.standard_normal(size).astype(np.float32), dt)
+        st[::7] = to_storage(np.array([-0.0], np.float32), dt)[0]
+        md = meta_sum_to_shape(dims, strides, dims, off)
+        (o,), (h,) = both(oracle, hip, f"sum_to_shape_{dt}", lambda: (n, len(dims), md, In(st), Out(n, dt)))
+        assert same_bits(o, h), (dims, strides)
+
+
 # ---------------------------------------------------------------------------------------------------
 # matmul
 # ---------------------------------------------------------------------------------------------------
