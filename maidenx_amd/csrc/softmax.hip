@@ -12,6 +12,8 @@
 //                          thread each, long ones are split among the 16 waves of a block.
 //   strided input        : one thread per slice with the reference's index rule (:120-136, the leading
 //                          dims are decomposed from dim 0 upwards).
+#include <algorithm>
+
 #include "elementwise.hpp"
 #include "mathfn.hpp"
 #include "mxh.hpp"
@@ -252,6 +254,122 @@ __global__ __launch_bounds__(WAVE * NW) void softmax_col_split_kernel(const T* _
     });
 }
 
+// [pre, D, post] contiguous, long D and few columns per CU (a [8192,8192] matrix along dim 0: one block per 64 column
+// vectors would be 32 blocks): the rows are cut into `groups` groups and a thread owns one column vector for one group's
+// rows, consecutive threads on consecutive vectors (a block reads 4 KB of a row at a time), eight rows in flight; three
+// launches that each read the rows once -
+//   PHASE 0: the maximum of every column over the group's rows                      -> part[pre][group][post]
+//   PHASE 1: the group's sum of exp(x - m), m = the column's maximum                 -> part[pre][group][post]
+//   PHASE 2: out = exp(x - m) / s
+// with softmax_col_fold_kernel between them, which folds the groups' values of a column in group order into
+// m[pre][post] (exact) and s[pre][post] = exp(-inf - m) + sum.
+template <class T, int VEC, int PHASE, bool STREAM>
+__global__ __launch_bounds__(256) void softmax_col_groups_kernel(const T* __restrict__ in, T* __restrict__ out, float* __restrict__ part,
+                                                                 const float* __restrict__ cmax, const float* __restrict__ csum, size_t D,
+                                                                 size_t post, uint32_t cv, uint32_t slabs, uint32_t groups,
+                                                                 uint32_t rows_per_group) {
+    constexpr int U = 8;
+    const uint32_t slab = blockIdx.x % slabs, group = (blockIdx.x / slabs) % groups, pre_idx = blockIdx.x / (slabs * groups);
+    const uint32_t j = slab * 256 + threadIdx.x;           // column vector
+    if (j >= cv) return;
+    const size_t l0 = (size_t)group * rows_per_group < D ? (size_t)group * rows_per_group : D;
+    const size_t l1 = l0 + rows_per_group < D ? l0 + rows_per_group : D;
+    const T* src = in + (size_t)pre_idx * D * post + (size_t)j * VEC;
+    T* dst = out + (size_t)pre_idx * D * post + (size_t)j * VEC;
+    float* mine = part + ((size_t)pre_idx * groups + group) * post + (size_t)j * VEC;
+    const size_t col = (size_t)pre_idx * post + (size_t)j * VEC;
+    auto sweep = [&](auto&& each) {
+        size_t l = l0;
+        for (; l + U <= l1; l += U) {
+            AVec<T, VEC> v[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) v[k] = ld_vec<STREAM>((const AVec<T, VEC>*)(src + (l + k) * post));
+#pragma unroll
+            for (int k = 0; k < U; ++k) each(l + k, v[k]);
+        }
+        for (; l < l1; ++l) each(l, ld_vec<STREAM>((const AVec<T, VEC>*)(src + l * post)));
+    };
+    float m[VEC], s[VEC];
+    if constexpr (PHASE == 0) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) m[e] = -INFINITY;
+        sweep([&](size_t, const AVec<T, VEC>& v) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(v.v[e]); m[e] = x > m[e] ? x : m[e]; }
+        });
+        AVec<float, VEC> r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = m[e];
+        *(AVec<float, VEC>*)mine = r;
+    } else {
+        const AVec<float, VEC> mv = *(const AVec<float, VEC>*)(cmax + col);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) m[e] = mv.v[e];
+        if constexpr (PHASE == 1) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s[e] = 0.0f;
+            sweep([&](size_t, const AVec<T, VEC>& v) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s[e] += SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]);
+            });
+            AVec<float, VEC> r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r.v[e] = s[e];
+            *(AVec<float, VEC>*)mine = r;
+        } else {
+            const AVec<float, VEC> sv = *(const AVec<float, VEC>*)(csum + col);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s[e] = sv.v[e];
+            sweep([&](size_t l, const AVec<T, VEC>& v) {
+                AVec<T, VEC> o;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]), s[e]);
+                st_vec<STREAM>((AVec<T, VEC>*)(dst + l * post), o);
+            });
+        }
+    }
+}
+
+// SUM ? s = exp(-inf - m) + part[0] + part[1] + ... : m = max(part[0], part[1], ...) for every column.  A block is 64
+// columns (the lanes) by 16 waves; wave w folds the w-th sixteenth of the groups in ascending order, eight loads in
+// flight, and the sixteen results meet in LDS in wave order.
+template <bool SUM>
+__global__ __launch_bounds__(1024) void softmax_col_fold_kernel(const float* __restrict__ part, const float* __restrict__ cmax, float* __restrict__ res,
+                                                                size_t post, size_t cols, uint32_t groups) {
+    constexpr int NW = 16;
+    const int lane = threadIdx.x % WAVE, w = threadIdx.x / WAVE;
+    const size_t c = (size_t)blockIdx.x * WAVE + lane;
+    const bool live = c < cols;
+    __shared__ float red[NW][WAVE];
+    const uint32_t per = (groups + NW - 1) / NW;
+    const uint32_t g0 = w * per < groups ? w * per : groups, g1 = g0 + per < groups ? g0 + per : groups;
+    float t = SUM ? 0.0f : -INFINITY;
+    if (live && g0 < g1) {
+        const size_t pre_idx = c / post, j = c - pre_idx * post;
+        const float* p = part + pre_idx * groups * post + j;
+        t = p[(size_t)g0 * post];
+        uint32_t g = g0 + 1;
+        for (; g + 8 <= g1; g += 8) {
+            float v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = p[(size_t)(g + k) * post];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) t = SUM ? t + v[k] : (v[k] > t ? v[k] : t);
+        }
+        for (; g < g1; ++g) { const float v = p[(size_t)g * post]; t = SUM ? t + v : (v > t ? v : t); }
+    }
+    red[w][lane] = t;
+    __syncthreads();
+    if (w != 0 || !live) return;
+    t = red[0][lane];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) {
+        if (k * per >= groups) break;            // (waves without groups hold the neutral value, but 0 + (-0) would lose a sign)
+        t = SUM ? t + red[k][lane] : (red[k][lane] > t ? red[k][lane] : t);
+    }
+    res[c] = SUM ? m_exp(-INFINITY - cmax[c]) + t : t;
+}
+
 struct SoftmaxStrided {
     int nd, dim;
     uint32_t dims[MAXD];
@@ -324,6 +442,30 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
         constexpr int VEC = 16 / sizeof(T), NW = 16;
         const bool vec_ok = post % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)out % 16) == 0;
         const size_t blocks_v = pre * cdiv(post / VEC, (size_t)WAVE);
+        // few columns per CU and long ones: the rows in groups, three launches (see softmax_col_groups_kernel)
+        if (vec_ok && blocks_v < 1024 && D >= 1024 && pre * post < (1ull << 31)) {
+            const uint32_t cv = (uint32_t)(post / VEC), slabs = (uint32_t)cdiv(cv, (size_t)256);
+            uint32_t groups = (uint32_t)std::min<size_t>(std::min<size_t>(cdiv((size_t)2048, pre * slabs), D / 16), 256);
+            const uint32_t rpg = (uint32_t)cdiv(D, (size_t)groups);
+            groups = (uint32_t)cdiv(D, (size_t)rpg);
+            const size_t part_n = pre * groups * post, cols = pre * post;
+            float* part = (float*)scratch((part_n + 2 * cols) * sizeof(float));
+            if (!part) return;
+            float *cm = part + part_n, *cs = cm + cols;
+            const dim3 grid((unsigned)(pre * slabs * groups)), block(256), fold((unsigned)cdiv(cols, (size_t)WAVE)), fold_block(1024);
+            const bool big = ew_stream_bytes() != 0 && num_els * sizeof(T) >= ew_stream_bytes();
+#define MXH_SM_PHASE(P)                                                                                                                   \
+    if (big) hipLaunchKernelGGL((softmax_col_groups_kernel<T, VEC, P, true>), grid, block, 0, stream(), src, out, part, cm, cs, D, post, cv, slabs, groups, rpg); \
+    else hipLaunchKernelGGL((softmax_col_groups_kernel<T, VEC, P, false>), grid, block, 0, stream(), src, out, part, cm, cs, D, post, cv, slabs, groups, rpg)
+            MXH_SM_PHASE(0);
+            hipLaunchKernelGGL((softmax_col_fold_kernel<false>), fold, fold_block, 0, stream(), part, (const float*)nullptr, cm, post, cols, groups);
+            MXH_SM_PHASE(1);
+            hipLaunchKernelGGL((softmax_col_fold_kernel<true>), fold, fold_block, 0, stream(), part, cm, cs, post, cols, groups);
+            MXH_SM_PHASE(2);
+#undef MXH_SM_PHASE
+            MXH_LAUNCH_CHECK("softmax_col_groups");
+            return;
+        }
         if (vec_ok && blocks_v >= 256) {
             uint32_t cv = (uint32_t)(post / VEC), jb = (uint32_t)cdiv(cv, (size_t)WAVE);
             hipLaunchKernelGGL((softmax_col_split_kernel<T, VEC, NW>), dim3((unsigned)(pre * jb)), dim3(WAVE * NW), 0, stream(), src, out, D, post, cv, make_fastdiv(jb));

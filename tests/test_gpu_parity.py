@@ -876,7 +876,9 @@ def test_fold_f64_and_integers(oracle, hip, dims, strides, fd, wd, fold_size, st
 SOFTMAX_CASES = [([2, 3], 1), ([2, 2, 3], 2), ([2, 3], 0), ([64, 5], 1), ([33, 2048], 1), ([9, 2052], 1), ([3, 40000], 1), ([7, 300], 1),
                  ([6, 50, 130], 1), ([4, 3, 5, 6], 0), ([5, 6], 7), ([10000], 0),
                  # long inner columns: the block-split kernel with narrow and with 16-byte column vectors
-                 ([3, 200, 132], 1), ([300, 64, 128], 1), ([1000, 70], 0)]
+                 ([3, 200, 132], 1), ([300, 64, 128], 1), ([1000, 70], 0),
+                 # few slabs of long columns: the rows in groups, three launches (a ragged last group, dead lanes, pre > 1)
+                 ([2048, 264], 0), ([1100, 520], 0), ([3, 1500, 136], 1), ([4096, 1024], 0)]
 
 
 @pytest.mark.parametrize("dt", DTS)
