@@ -196,8 +196,10 @@ struct Stager {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     uint32_t d0 = reg[2 * u + (2 * e) / 4][(2 * e) % 4], d1 = reg[2 * u + (2 * e + 1) / 4][(2 * e + 1) % 4];
-                    lo[e] = (d0 & 0xffffu) | (d1 << 16);
-                    hi[e] = (d0 >> 16) | (d1 & 0xffff0000u);
+                    // one byte permute each (as shifts and masks this is four vector-ALU instructions per pair, and on this
+                    // chip vector-ALU time is not hidden behind the MFMAs)
+                    lo[e] = __builtin_amdgcn_perm(d1, d0, 0x05040100u);      // d0.lo16 | d1.lo16 << 16
+                    hi[e] = __builtin_amdgcn_perm(d1, d0, 0x07060302u);      // d0.hi16 | d1.hi16 << 16
                 }
                 *(u32x4*)(lds + at(row, ck)) = lo;
                 *(u32x4*)(lds + at(row + 1, ck)) = hi;
