@@ -115,6 +115,10 @@ int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_
  * epoch eager; mxt_last_train_replayed() tells how many epochs of the last mxt_train call were replays. */
 void mxt_set_graph_replay(int enabled);
 size_t mxt_last_train_replayed(void);
+/* sum_all() (crates/maidenx_tensor/src/ops/reduction.rs:76-83) sums one dim after the other.  By default a contiguous f32
+ * tensor is summed by one sum_to_shape call to [1, .., 1] instead: the gradients are the same bytes, the sum is added
+ * up in another order (both within the f32 tolerance of a reduction).  enabled = 0: dim by dim. */
+void mxt_set_sum_all_in_one_pass(int enabled);
 /* backward() leaves out three things that cannot change a bit of any gradient (enabled = 0: does them all, as the
  * reference does): the gradient of a binary op's operand that requires none (computed and dropped in the reference,
  * crates/maidenx_tensor/src/lib.rs:93-111), x.pow(1) in the backward of pow(2), and the zero fill in front of the first

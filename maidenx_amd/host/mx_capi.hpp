@@ -256,6 +256,7 @@ int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_
 }
 void mxt_set_graph_replay(int enabled) { g_graphs = enabled != 0; }
 size_t mxt_last_train_replayed(void) { return g_replayed; }
+void mxt_set_sum_all_in_one_pass(int enabled) { mxt::sum_all_in_one_pass() = enabled != 0; }
 void mxt_set_autograd_shortcuts(int enabled) { mxt::autograd_shortcuts() = enabled != 0; }
 void mxt_set_conv_skip_unread_grad_cols(int enabled) { mxt::conv_skip_unread_grad_cols() = enabled != 0; }
 void mxt_set_conv_gathered_products(int mode) { mxt::conv_gathered_products() = mode < 0 ? 0 : mode > 2 ? 2 : mode; }

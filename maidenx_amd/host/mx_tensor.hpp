@@ -230,6 +230,8 @@ template <class B> struct GradCell {
 inline size_t& backend_calls() { static size_t n = 0; return n; }
 // Conv2d backward: make only the rows of grad_cols that col2im reads (see Conv2d); false = the whole product.
 inline bool& conv_skip_unread_grad_cols() { static bool on = true; return on; }
+// sum_all() of a contiguous f32 tensor as one reduction (true) or dim by dim as the reference does (false).
+inline bool& sum_all_in_one_pass() { static bool on = true; return on; }
 // Conv2d on a backend that has the product with the gathered column matrix (the matrix is never stored): 0 = store
 // the matrix with im2col and multiply that, as the reference does; 1 = gather when no backward is recorded (the
 // forward alone is faster gathered, a training step is faster with the one stored matrix serving both products);
@@ -773,6 +775,28 @@ struct Tensor {
         return result;
     }
     T sum_all() const {                                                             // ops/reduction.rs:76-83
+        // The reference sums one dim after the other, innermost first: n kernels forward and n small broadcasts and
+        // accumulations backward.  A contiguous f32 tensor is summed in one sum_to_shape call to [1, .., 1] instead (the
+        // MLP's own `[10000,1] -> []` is such a call); every gradient is the same bytes, the sum itself is added up in
+        // another order (within the f32 tolerance of a reduction either way).
+        if (sum_all_in_one_pass() && dtype == DType::F32 && ndim() >= 2 && size() > 0 && is_contiguous() && offset() == 0) {
+            // (a node of its own: a view of a [1, .., 1] result would share that result's buffer, and backward() takes
+            // tensors that share a buffer for one tensor, lib.rs:308-323)
+            const Shape ones(ndim(), 1);
+            T result = empty(Shape{}, dtype);
+            auto md = meta_to_shape(*this, ones);
+            K<float>::sum_to_shape(size(), ndim(), md.data(), this->template p<float>(), result.template p<float>());
+            ++backend_calls();
+            B::check();
+            if (requires_grad) {
+                result.with_grad();
+                Shape in_shape = shape();
+                result.set_node("sum_all", {*this}, [in_shape, ones](const std::vector<T>&, const T& go) {
+                    return std::vector<T>{go.reshape(ones).broadcast(in_shape)};
+                });
+            }
+            return result;
+        }
         T result = *this;
         for (size_t d = ndim(); d-- > 0;) result = result.sum((int)d, false);
         return result;

@@ -114,6 +114,34 @@ def test_conv2d_forward_backward(mx_hip, mx_oracle, B, Cin, H, W, Cout, k, strid
         assert np.abs(got[key] - num[key]).max() <= 1e-4 * scale, key
 
 
+def test_sum_all_in_one_pass_or_dim_by_dim(mx_hip):
+    """sum_all() of a contiguous f32 tensor as one reduction, or dim by dim as reduction.rs:76-83 does it: the same
+    gradients bit for bit, the sums within the f32 tolerance of a reduction of each other and of float64."""
+    mx = mx_hip
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal((5, 7, 9, 11)).astype(np.float32)
+    x, w, bias = conv_inputs(2, 3, 6, 5, 4, 3, seed=22)
+    target = rng.standard_normal((2, 4, 6, 5)).astype(np.float32)
+    res = {}
+    try:
+        for one_pass in (False, True):
+            mx.set_sum_all_in_one_pass(one_pass)
+            t = mx.tensor(a).with_grad()
+            mx.reset_backend_calls()
+            z = t.mul(t).sum_all()
+            z.backward()
+            res[one_pass] = dict(z=z.numpy(), g=t.grad().numpy(), calls=mx.backend_calls(), **conv_step(mx, x, w, bias, 1, 1, target))
+    finally:
+        mx.set_sum_all_in_one_pass(True)
+    assert res[True]["calls"] < res[False]["calls"]
+    for key in ("g", "grad_x", "grad_w", "grad_b", "out"):
+        np.testing.assert_array_equal(res[True][key].view(np.uint32), res[False][key].view(np.uint32), err_msg=key)
+    exact = float(np.sum(a.astype(np.float64) ** 2))
+    for one_pass in (False, True):
+        assert abs(float(res[one_pass]["z"]) - exact) <= 1e-5 * exact
+    assert abs(float(res[True]["loss"]) - float(res[False]["loss"])) <= 1e-5 * abs(float(res[False]["loss"]))
+
+
 def _shortcut_programs(mx):
     """Programs whose backward passes contain what the shortcuts leave out: operands without a gradient, pow(2),
     gradients that arrive as broadcast views (sum over dims, a broadcast operand, the MSE loss)."""
