@@ -279,6 +279,22 @@ template <class TIn, class TOut, class R>
 void row_stage(const TIn* in, TOut* out, size_t rows, size_t L, unsigned chunks, size_t chunk_len, float div,
                bool src_bf16) {
     size_t len = chunks > 1 ? chunk_len : L;
+    // many rows of a few dozen elements (the sums over the last dim of an image batch, rows of 56): a wave per row would
+    // leave three lanes in four without an element; 16 lanes per row, four rows per wave
+    constexpr int V16 = 16 / sizeof(TIn);
+    if (len > 32 && len <= 64 * V16 && rows * chunks >= 65536 && aligned16(in) && L % V16 == 0 && chunk_len % V16 == 0) {
+        if constexpr (std::is_same<TIn, float>::value && std::is_same<TOut, float>::value)
+            if (prog_recording()) prog_abandon();          // (far beyond what a recorded program holds)
+        const unsigned blocks = cdiv(rows * chunks, (size_t)(RB / 16));
+        if (streams(rows * L * sizeof(TIn)))
+            hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, 16, V16, true>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows, L, chunks,
+                               chunk_len, div, src_bf16);
+        else
+            hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, R, 16, V16>), dim3(blocks), dim3(RB), 0, stream(), in, out, rows, L, chunks,
+                               chunk_len, div, src_bf16);
+        MXH_LAUNCH_CHECK("row_reduce");
+        return;
+    }
     if (len <= 32) launch_row<TIn, TOut, R, 1>(in, out, rows, L, chunks, chunk_len, div, src_bf16);
     else if (len <= 2048) launch_row<TIn, TOut, R, WAVE>(in, out, rows, L, chunks, chunk_len, div, src_bf16);
     else launch_row<TIn, TOut, R, RB>(in, out, rows, L, chunks, chunk_len, div, src_bf16);

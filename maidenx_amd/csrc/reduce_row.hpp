@@ -70,10 +70,20 @@ __device__ inline float wave_reduce(float v) {
     return R::op(R::op(r0, r1), R::op(r2, r3));
 }
 
+// The same butterfly inside each 16-lane row of the wave (four rows, four results).
+template <class R>
+__device__ inline float row16_reduce(float v) {
+    v = dpp_combine<R, 0xB1>(v);
+    v = dpp_combine<R, 0x4E>(v);
+    v = dpp_combine<R, 0x141>(v);
+    v = dpp_combine<R, 0x140>(v);
+    return v;
+}
+
 constexpr int RB = 256;
 
 // ---- row reduce: [rows, L] → [rows, chunks] ---------------------------------------------------
-// TPR threads cooperate on one (row, chunk).  VEC > 1 requires L % VEC == 0, chunk_len % VEC == 0
+// TPR threads cooperate on one (row, chunk): one, a 16-lane row of a wave, a wave, or the block.  VEC > 1 requires L % VEC == 0, chunk_len % VEC == 0
 // and a 16-byte aligned base.
 // Block and thread index are arguments (the interpreter of recorded programs passes virtual ones); `part`
 // is RB / WAVE floats of LDS owned by this (virtual) block.  Every thread reaches the barrier.
@@ -142,6 +152,7 @@ __device__ __forceinline__ void row_reduce_body(const TIn* __restrict__ in, TOut
         }
     }
     if constexpr (TPR >= WAVE) acc = wave_reduce<R>(acc);
+    else if constexpr (TPR == 16) acc = row16_reduce<R>(acc);
     if constexpr (TPR > WAVE) {
         if (tid % WAVE == 0) part[tid / WAVE] = acc;
         __syncthreads();

@@ -325,7 +325,9 @@ def test_large_16bit_unary_calls_go_through_the_table_and_keep_the_bits(oracle, 
 # ---------------------------------------------------------------------------------------------------
 RED_CASES = [([64, 96], 0), ([64, 96], 1), ([257, 130], 0), ([257, 130], 1), ([8, 16, 32], 0), ([8, 16, 32], 1), ([8, 16, 32], 2),
              ([5000], 0), ([3, 70000], 1), ([70000, 3], 0), ([1, 40000], 0), ([10000, 1], 1), ([2, 3, 5, 7], 2), ([40000], 0),
-             ([300, 2048], 1), ([4, 300000], 1)]
+             ([300, 2048], 1), ([4, 300000], 1),
+             # at least 65536 rows of a few dozen elements: 16 lanes per row (rows of 56, 40, 256 and 64 elements)
+             ([1200, 56, 56], 2), ([70000, 40], 1), ([66000, 256], 1), ([65536, 64], 1)]
 
 
 @pytest.mark.parametrize("dt", DTS)
