@@ -119,10 +119,11 @@ size_t mxt_last_train_replayed(void);
  * tensor is summed by one sum_to_shape call to [1, .., 1] instead: the gradients are the same bytes, the sum is added
  * up in another order (both within the f32 tolerance of a reduction).  enabled = 0: dim by dim. */
 void mxt_set_sum_all_in_one_pass(int enabled);
-/* backward() leaves out three things that cannot change a bit of any gradient (enabled = 0: does them all, as the
- * reference does): the gradient of a binary op's operand that requires none (computed and dropped in the reference,
- * crates/maidenx_tensor/src/lib.rs:93-111), x.pow(1) in the backward of pow(2), and the zero fill in front of the first
- * accumulation when the gradient is a broadcast view. */
+/* backward() leaves out what cannot change a bit of any gradient (enabled = 0: does it all, as the reference does): the
+ * gradient of a binary op's operand that requires none (computed and dropped in the reference,
+ * crates/maidenx_tensor/src/lib.rs:93-111), x.pow(1) in the backward of pow(2), the zero fill in front of the first
+ * accumulation when the gradient is a broadcast view, and the first accumulation itself (0 + g) when g is a fresh
+ * sum_to_shape result, whose buffer then becomes the gradient. */
 void mxt_set_autograd_shortcuts(int enabled);
 /* Conv2d backward (nn/layers/conv.rs:253-268): col2im is handed num_els = B*C*H*W and reads no entry of grad_cols at
  * or beyond that flat index (crates/maidenx_cpu/src/nn/conv.rs:135), so by default only the leading

@@ -237,11 +237,11 @@ inline bool& sum_all_in_one_pass() { static bool on = true; return on; }
 // forward alone is faster gathered, a training step is faster with the one stored matrix serving both products);
 // 2 = gather in forward and backward (no buffer of B*oh*ow x C*kh*kw elements lives between the two).
 inline int& conv_gathered_products() { static int mode = 1; return mode; }
-// Three things backward() leaves out without changing a bit of any gradient (false: do all of them, as the reference
-// does): the gradient of a binary op's operand that does not require one (the reference computes it and drops it,
-// lib.rs:93-111), x.pow(1) in the backward of pow(2) (x itself), and the zero-filled buffer that the first gradient
-// of a tensor is added into when that gradient is a broadcast view (0 + g is written straight away, as for a contiguous
-// gradient).
+// What backward() leaves out without changing a bit of any gradient (false: do all of it, as the reference does): the
+// gradient of a binary op's operand that does not require one (the reference computes it and drops it, lib.rs:93-111),
+// x.pow(1) in the backward of pow(2) (x itself), the zero-filled buffer that the first gradient of a tensor is added
+// into when that gradient is a broadcast view (0 + g is written straight away, as for a contiguous gradient), and that
+// `0 + g` altogether when g is a fresh sum_to_shape result (sums that started from +0: it becomes the gradient as it is).
 inline bool& autograd_shortcuts() { static bool on = true; return on; }
 // Count of whole-buffer dtype conversions (with_dtype: a host loop in the reference, a kernel here).
 inline size_t& cast_calls() { static size_t n = 0; return n; }
@@ -254,6 +254,9 @@ struct Tensor {
     Layout layout;
     DType dtype = DType::F32;
     bool requires_grad = false;
+    // This tensor's elements are sums that started from +0 (what sum_to_shape writes), so `0 + x` would copy it bit for
+    // bit.  Not kept by views or copies of the tensor.
+    bool sums_from_zero = false;
     std::shared_ptr<Node<B>> node;
 
     using T = Tensor<B>;
@@ -366,6 +369,15 @@ struct Tensor {
     }
     void accumulate_grad(const T& g) const {                                        // lib.rs:221-241
         if (!has_grad()) return;
+        // The first gradient of a tensor is added into zeros.  When it is itself a fresh buffer of sums that started
+        // from +0 (an identity sum_to_shape in a binary op's backward), `0 + g` would be a copy of it bit for bit: the
+        // buffer becomes the gradient as it is.  (Nobody else holds it: the caller's vector of gradients does, and
+        // only reads it.)
+        if (autograd_shortcuts() && !grad_cell->g && g.sums_from_zero && g.buf.use_count() == 1 && g.dtype == grad_cell->dtype &&
+            g.is_contiguous() && g.offset() == 0 && g.shape() == grad_cell->shape) {
+            grad_cell->g = std::make_shared<T>(share_buffer(g));
+            return;
+        }
         // (a view qualifies when every element it addresses lies inside the first size() elements of its buffer: the
         // strided sum_to_shape kernel wraps source indices at num_els, reduction.rs:112-140, and must not get to)
         auto inside = [](const T& v) {
@@ -822,6 +834,7 @@ struct Tensor {
         });
         ++backend_calls();
         B::check();
+        result.sums_from_zero = true;
         if (requires_grad) {
             result.with_grad();
             Shape in_shape = shape();

@@ -242,8 +242,9 @@ def test_conv2d_backward_with_zero_padding_is_an_error(mx_oracle):
 @pytest.mark.parametrize("case", ["contig", "bcast", "transposed"])
 def test_bench_chain_is_the_host_layers_call_sequence(mx_oracle, op, case):
     """bench.py's ChainBuilder spells out, call by call, what forward + backward of each op dispatches to the
-    backend.  The host layer derives the same thing from the reference's backward closures; the number of backend
-    calls must agree (device-side casts are not backend calls in the reference and are not counted)."""
+    backend.  The host layer derives the same thing from the reference's backward closures (with none of its own
+    shortcuts); the number of backend calls must agree (device-side casts are not backend calls in the reference and are
+    not counted)."""
     import bench
     if op in ("exp", "relu", "gelu") and case == "bcast":
         pytest.skip("unary ops have no broadcast case")
@@ -264,10 +265,15 @@ def test_bench_chain_is_the_host_layers_call_sequence(mx_oracle, op, case):
     else:
         x = mx.tensor(rng.standard_normal((R, C)).astype(np.float32)).with_grad()
     y = mx.tensor(rng.standard_normal((1, C) if case == "bcast" else (R, C)).astype(np.float32) + 3.0).with_grad()
-    mx.reset_backend_calls()
-    z = getattr(x, op)(y) if op in ("add", "mul", "div") else getattr(x, op)()
-    z.backward()
-    assert mx.backend_calls() == want, (op, case, mx.backend_calls(), want)
+    # (the chain is the reference's own sequence: backward() with nothing left out)
+    try:
+        mx.set_autograd_shortcuts(False)
+        mx.reset_backend_calls()
+        z = getattr(x, op)(y) if op in ("add", "mul", "div") else getattr(x, op)()
+        z.backward()
+        assert mx.backend_calls() == want, (op, case, mx.backend_calls(), want)
+    finally:
+        mx.set_autograd_shortcuts(True)
 
 
 # ---- bf16 through the host layer --------------------------------------------------------------------------
@@ -310,9 +316,13 @@ def test_bench_chain_is_the_host_layers_call_sequence_bf16(mx_oracle, op, case):
     getattr(b, op)(case)
     want_casts = sum(1 for c in b.calls if c.tag.startswith("cast_"))
     want_calls = len(b.calls) - want_casts
-    mx.reset_backend_calls()
-    elementwise_program(mx, op, case, "bf16", R=6, C=8)
-    assert (mx.backend_calls(), mx.cast_calls()) == (want_calls, want_casts), (op, case)
+    try:
+        mx.set_autograd_shortcuts(False)
+        mx.reset_backend_calls()
+        elementwise_program(mx, op, case, "bf16", R=6, C=8)
+        assert (mx.backend_calls(), mx.cast_calls()) == (want_calls, want_casts), (op, case)
+    finally:
+        mx.set_autograd_shortcuts(True)
 
 
 @pytest.mark.parametrize("case", ["contig", "bcast", "transposed"])
