@@ -335,6 +335,42 @@ def test_conv2d_layer_step_config_size(mx_hip):
     assert np.abs(gx[:227]).max() > 0 and not gx[228:].any()
 
 
+def test_conv2d_layer_step_config_size_every_way_gives_the_same_gradients(mx_hip):
+    """The same full-size step with the switches of the host layer turned the reference's way: the column matrix stored
+    (im2col) or gathered inside the products, grad_cols whole or only the rows col2im reads, backward() with and without
+    its shortcuts.  Outputs and all gradients are the same bits; with sum_all dim by dim only the loss may differ, within
+    the reduction tolerance."""
+    from host_programs import conv_inputs, conv_step
+    x, w, b = conv_inputs(32, 64, 56, 56, 64, 3, seed=0x5EED0006)
+    target = np.random.default_rng(0x5EED0016).standard_normal((32, 64, 56, 56)).astype(np.float32)
+    mx = mx_hip
+    try:
+        base = conv_step(mx, x, w, b, 1, 1, target)
+        variants = {}
+        mx.set_conv_gathered_products(2)
+        variants["gathered"] = conv_step(mx, x, w, b, 1, 1, target)
+        mx.set_conv_gathered_products(1)
+        mx.set_conv_skip_unread_grad_cols(False)
+        variants["whole grad_cols"] = conv_step(mx, x, w, b, 1, 1, target)
+        mx.set_conv_skip_unread_grad_cols(True)
+        mx.set_autograd_shortcuts(False)
+        variants["no shortcuts"] = conv_step(mx, x, w, b, 1, 1, target)
+        mx.set_autograd_shortcuts(True)
+        mx.set_sum_all_in_one_pass(False)
+        dim_by_dim = conv_step(mx, x, w, b, 1, 1, target)
+    finally:
+        mx.set_conv_gathered_products(1)
+        mx.set_conv_skip_unread_grad_cols(True)
+        mx.set_autograd_shortcuts(True)
+        mx.set_sum_all_in_one_pass(True)
+    for name, got in variants.items():
+        for key in ("out", "loss", "grad_b", "grad_w", "grad_x"):
+            assert np.array_equal(got[key].view(np.uint32), base[key].view(np.uint32)), (name, key)
+    for key in ("out", "grad_b", "grad_w", "grad_x"):
+        assert np.array_equal(dim_by_dim[key].view(np.uint32), base[key].view(np.uint32)), ("sum_all dim by dim", key)
+    assert abs(float(dim_by_dim["loss"]) - float(base["loss"])) <= 1e-5 * abs(float(base["loss"]))
+
+
 def test_bf16_accumulation_gpu_is_closer_to_exact_than_the_reference(hip, oracle):
     """4096-term bf16 dot products and sums: the reference accumulates in bf16 (crates/maidenx_cpu/src/ops/matmul.rs:74-86,
     reduction.rs:58), the GPU in f32 with one rounding.  Both are measured against float64, normalised by the sum of
