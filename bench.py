@@ -827,7 +827,13 @@ def _oracle_host(threads):
     lib = C.CDLL(ensure_oracle_built(), mode=C.RTLD_GLOBAL)
     lib.oracle_set_num_threads.restype = C.c_int
     cores = lib.oracle_set_num_threads(threads)
-    return oracle_host(), cores
+    mo = oracle_host()
+    # the baseline is the reference's own sequence of backend calls: none of the host layer's shortcuts
+    mo.set_autograd_shortcuts(False)
+    mo.set_sum_all_in_one_pass(False)
+    mo.set_conv_skip_unread_grad_cols(False)
+    mo.set_conv_gathered_products(0)
+    return mo, cores
 
 
 def cpu_baseline_mlp(args):

@@ -73,8 +73,11 @@ def build_host(force=False):
     srcs = [os.path.join(hdir, f) for f in os.listdir(hdir)] + [os.path.join(HERE, "..", "include", "maidenx_host.h"), LIB]
     if not force and os.path.exists(HOST_LIB) and os.path.getmtime(HOST_LIB) > max(os.path.getmtime(f) for f in srcs):
         return HOST_LIB
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", os.path.join(hdir, "host_hip.cpp"), "-o", HOST_LIB,
-           "-L" + HERE, "-lmaidenx_hip", "-Wl,-rpath,$ORIGIN"]
+    # -fno-gnu-unique, -Bsymbolic: the layer's switches and counters are function-local statics of inline functions; as
+    # GNU-unique symbols they would be ONE object for every build of the layer loaded into a process (this one and the
+    # CPU oracle's), so that a switch set on one would set it on the other
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-fno-gnu-unique", os.path.join(hdir, "host_hip.cpp"), "-o", HOST_LIB,
+           "-L" + HERE, "-lmaidenx_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-Bsymbolic"]
     p = subprocess.run(cmd, capture_output=True, text=True)
     if p.returncode != 0:
         raise RuntimeError("host layer build failed:\n" + p.stdout + p.stderr)

@@ -105,6 +105,23 @@ def test_sqrt_forward_and_backward(mx_oracle):
     np.testing.assert_allclose(t.grad().numpy(), 0.5 / np.sqrt(x), rtol=1e-6)          # unary.rs:176-178: go / (2 * sqrt(x))
 
 
+def test_the_two_builds_of_the_host_layer_keep_their_own_state(mx_oracle):
+    """libmaidenx_host.so (over the HIP backend) and the oracle's build of the same headers live in one process in the
+    GPU tests and in bench.py: counters and switches of one must not be those of the other (as GNU-unique symbols the
+    function-local statics of the layer's inline functions would be shared)."""
+    import ctypes as C
+    from maidenx_amd.tensor import HOST_LIB_PATH
+    hip_host = C.CDLL(HOST_LIB_PATH)                 # loading needs no GPU; nothing below touches the device
+    hip_host.mxt_backend_calls.restype = C.c_size_t
+    hip_host.mxt_reset_backend_calls()
+    mx = mx_oracle
+    mx.reset_backend_calls()
+    t = mx.tensor(np.arange(6, dtype=np.float32).reshape(2, 3))
+    t.mul(t).add(t)
+    assert mx.backend_calls() == 2
+    assert hip_host.mxt_backend_calls() == 0
+
+
 def test_mlp_call_count_is_stable(mx_oracle):
     mx = mx_oracle
     mlp_run(mx, 2, n=100)
