@@ -62,6 +62,11 @@ static inline bool by_table(size_t num_els, size_t num_dims, const size_t* md, c
     MXH_UNARY_C(lt_scalar, OpLtScalar, T, SUF, bool_t) MXH_UNARY_C(le_scalar, OpLeScalar, T, SUF, bool_t)     \
     MXH_UNARY_C(gt_scalar, OpGtScalar, T, SUF, bool_t) MXH_UNARY_C(ge_scalar, OpGeScalar, T, SUF, bool_t)
 
+namespace mxh {
+const uint16_t* lut16_exp_bf16() { return lut16_table<OpExp<bf16_t>>(); }
+const uint16_t* lut16_exp_f16() { return lut16_table<OpExp<f16_t>>(); }
+}  // namespace mxh
+
 MXH_ALL_FOR(float, f32)
 MXH_ALL_FOR(bf16_t, bf16)
 MXH_ALL_FOR(f16_t, f16)

@@ -13,6 +13,7 @@
 //   strided input        : one thread per slice with the reference's index rule (:120-136, the leading
 //                          dims are decomposed from dim 0 upwards).
 #include <algorithm>
+#include <type_traits>
 
 #include "elementwise.hpp"
 #include "mathfn.hpp"
@@ -40,21 +41,25 @@ template <> struct SM<f16_t> {
 
 constexpr int SB = 256;
 
+// Butterflies over groups of W consecutive lanes (W = 64: the wave).  A narrower group's sum is, bit for bit, what the
+// wave-wide one gives when the other lanes hold 0: those steps add 0 to a sum of non-negative terms.
+template <int W = WAVE>
 __device__ inline float wave_max(float v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
+    for (int off = W / 2; off > 0; off >>= 1) {
         float o = __shfl_xor(v, off, WAVE);
         v = o > v ? o : v;
     }
     return v;
 }
+template <int W = WAVE>
 __device__ inline float wave_sum(float v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    for (int off = W / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
     return v;
 }
 
-// rows of length D, TPR threads per row (WAVE or SB); NREG vectors of the row live in registers, longer
+// rows of length D, TPR threads per row (8, 16, 32, WAVE or SB); NREG vectors of the row live in registers, longer
 // rows are read again from cache in each phase
 template <class T, int TPR, int VEC, int NREG>
 __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ in, T* __restrict__ out, size_t rows, size_t D) {
@@ -92,7 +97,7 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
             }
         }
     }
-    m = wave_max(m);
+    m = wave_max<(TPR < WAVE ? TPR : WAVE)>(m);
     if constexpr (TPR > WAVE) {
         if (threadIdx.x % WAVE == 0) red[threadIdx.x / WAVE] = m;
         __syncthreads();
@@ -124,7 +129,7 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
             }
         }
     }
-    s = wave_sum(s);
+    s = wave_sum<(TPR < WAVE ? TPR : WAVE)>(s);
     if constexpr (TPR > WAVE) {
         if (threadIdx.x % WAVE == 0) red[threadIdx.x / WAVE] = s;
         __syncthreads();
@@ -157,6 +162,102 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
             if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
             else dst[i] = o.v[0];
         }
+    }
+}
+
+// The same for bf16 / f16 with exp(x - m) taken from the dtype's table of exp (lut16.hpp): the term the kernel above
+// computes is round(exp(round(x - m))), a function of one 16-bit value, i.e. an entry of the table that hip_exp_<T> is
+// served from - the same bits.  The arithmetic form is bound by the bit-exact expf (28 % of HBM peak on [8192,8192]).
+// Here one 1024-thread block per CU copies the 128 KB table into LDS once, and then every WAVE works through rows of its
+// own, with no barrier: lane l stands for threads l, 64 + l, ... of the kernel above (VW of them: that kernel's block of
+// 64 * VW threads), holds their elements, adds their terms in their order into VW separate sums, folds each across the
+// wave as that kernel's waves do and adds the VW results in wave order - the same additions, the same bits.  The maximum
+// takes no part in this: no NaN ever enters it, and max over numbers does not depend on the order.  The 16 waves of a CU
+// drift apart, so loads, lookups and stores of different rows overlap; PF also fetches a wave's next row before it works
+// on the current one.  The row must fit the registers (D <= 64 * VW * VEC * NREG).
+template <class T> struct SMCode;
+template <> struct SMCode<bf16_t> { static __device__ uint32_t of(float v) { return f2bf(v).bits; } };
+template <> struct SMCode<f16_t> { static __device__ uint32_t of(float v) { return f2h(v).bits; } };
+template <class T, int TPR, int VW, int VEC, int NREG>
+struct LutRow {
+    AVec<T, VEC> v[VW][NREG];
+    static __device__ size_t at(int w, int k, unsigned t) { return (size_t)(w * TPR + t) * VEC + (size_t)k * (VW * TPR * VEC); }
+    __device__ void load(const T* __restrict__ src, unsigned t, size_t D) {
+#pragma unroll
+        for (int w = 0; w < VW; ++w)
+#pragma unroll
+            for (int k = 0; k < NREG; ++k)
+                if (at(w, k, t) < D) v[w][k] = *(const AVec<T, VEC>*)(src + at(w, k, t));
+    }
+};
+// TPR < 64 (short rows, VW = 1): 64 / TPR rows per wave, a group of TPR lanes each, as in the kernel above.
+template <class T, int TPR, int VW, int VEC, int NREG, bool PF, int BLK>
+__global__ __launch_bounds__(BLK) void softmax_row_lut_kernel(const uint16_t* __restrict__ table, const T* __restrict__ in, T* __restrict__ out,
+                                                              size_t rows, size_t D) {
+    static_assert(TPR == WAVE || VW == 1, "several waves' worth of threads only for whole-wave rows");
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    for (int i = threadIdx.x; i < 65536 * 2 / 16; i += BLK) ((u4*)lut)[i] = ((const u4*)table)[i];
+    __syncthreads();
+    constexpr int RPW = WAVE / TPR;
+    const unsigned lane = threadIdx.x % WAVE, t = lane % TPR;
+    const size_t stride = (size_t)gridDim.x * (BLK / WAVE) * RPW;
+    size_t row = ((size_t)blockIdx.x * (BLK / WAVE) + threadIdx.x / WAVE) * RPW + lane / TPR;
+    typedef LutRow<T, TPR, VW, VEC, NREG> Row;
+    Row cur, nxt;
+    if (row < rows) cur.load(in + row * D, t, D);
+    // a wave leaves the loop when its first row is past the end; the groups behind it are then past it too
+    for (; row - lane / TPR < rows; row += stride) {
+        const bool live = row < rows;
+        if (PF && row + stride < rows) nxt.load(in + (row + stride) * D, t, D);
+        float m = -INFINITY;
+        if (live) {
+#pragma unroll
+            for (int w = 0; w < VW; ++w)
+#pragma unroll
+                for (int k = 0; k < NREG; ++k)
+                    if (Row::at(w, k, t) < D) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(cur.v[w][k].v[e]); m = x > m ? x : m; }
+                    }
+        }
+        m = wave_max<TPR>(m);
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < VW; ++w) {
+            float sw = 0.0f;
+            if (live) {
+#pragma unroll
+                for (int k = 0; k < NREG; ++k)
+                    if (Row::at(w, k, t) < D) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) {
+                            T en;
+                            en.bits = lut[SMCode<T>::of(SM<T>::ld(cur.v[w][k].v[e]) - m)];
+                            cur.v[w][k].v[e] = en;          // the term is a 16-bit value: it stays where x was
+                            sw += SM<T>::ld(en);
+                        }
+                    }
+            }
+            sw = wave_sum<TPR>(sw);
+            s = w == 0 ? sw : s + sw;
+        }
+        s = m_exp(-INFINITY - m) + s;
+        if (live) {
+            T* dst = out + row * D;
+#pragma unroll
+            for (int w = 0; w < VW; ++w)
+#pragma unroll
+                for (int k = 0; k < NREG; ++k)
+                    if (Row::at(w, k, t) < D) {
+                        AVec<T, VEC> o;
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::ld(cur.v[w][k].v[e]), s);
+                        *(AVec<T, VEC>*)(dst + Row::at(w, k, t)) = o;
+                    }
+        }
+        if (PF) cur = nxt;
+        else if (row + stride < rows) cur.load(in + (row + stride) * D, t, D);
     }
 }
 
@@ -425,9 +526,50 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
         constexpr int VEC = 16 / sizeof(T);
         const bool vec = D % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)out % 16) == 0;
         if (slices >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "softmax: 2^31 or more rows"); return; }
+        if constexpr (sizeof(T) == 2) {
+            // a large 16-bit call whose rows fit the registers: exp from the table, one persistent block per CU (filling
+            // the tables costs every block about 3 us: below 2^22 elements the arithmetic kernel is as fast)
+            if (vec && slices * D >= (1u << 22) && D <= (size_t)SB * VEC * 4) {
+                const uint16_t* table = std::is_same<T, bf16_t>::value ? lut16_exp_bf16() : lut16_exp_f16();
+                static int cus[16] = {0};
+                int dev = 0;
+                if (table && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 16) {
+                    if (!cus[dev]) {
+                        hipDeviceProp_t prop;
+                        cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+                    }
+                    constexpr int LUT_LDS = 65536 * 2;
+                    auto launch = [&](auto kern, int blk, int tpr) {
+                        static bool allowed[16] = {false};
+                        if (!allowed[dev]) {
+                            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LUT_LDS) != hipSuccess) { (void)hipGetLastError(); return false; }
+                            allowed[dev] = true;
+                        }
+                        const unsigned blocks = (unsigned)std::min<size_t>((size_t)cus[dev], cdiv(slices, (size_t)(blk / tpr)));
+                        hipLaunchKernelGGL(kern, dim3(blocks), dim3(blk), LUT_LDS, stream(), table, src, out, slices, D);
+                        MXH_LAUNCH_CHECK("softmax_row_lut");
+                        return true;
+                    };
+                    // lanes per row, vectors per lane and waves' worth of lanes follow the arithmetic kernels below
+                    constexpr int WV = SB / WAVE, NW = 2048 / (WAVE * VEC);
+                    if (D <= 8 * VEC    ? launch(softmax_row_lut_kernel<T, 8, 1, VEC, 1, true, 1024>, 1024, 8)
+                        : D <= 16 * VEC ? launch(softmax_row_lut_kernel<T, 16, 1, VEC, 1, true, 1024>, 1024, 16)
+                        : D <= 32 * VEC ? launch(softmax_row_lut_kernel<T, 32, 1, VEC, 1, true, 1024>, 1024, 32)
+                        : D <= 2048     ? launch(softmax_row_lut_kernel<T, WAVE, 1, VEC, NW, true, 1024>, 1024, WAVE)
+                        : D <= (size_t)SB * VEC * 2 ? launch(softmax_row_lut_kernel<T, WAVE, WV, VEC, 2, false, 1024>, 1024, WAVE)
+                                                    : launch(softmax_row_lut_kernel<T, WAVE, WV, VEC, 4, false, 512>, 512, WAVE))
+                        return;
+                }
+            }
+        }
         if (D <= 2048) {
             unsigned blocks = cdiv(slices, SB / WAVE);
-            if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, VEC, 2048 / (WAVE * VEC)>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
+            // short rows: 8, 16 or 32 lanes each, so that a wave holds several
+            auto narrow = [&](auto kern, int tpr) { hipLaunchKernelGGL(kern, dim3((unsigned)cdiv(slices, (size_t)(SB / tpr))), dim3(SB), 0, stream(), src, out, slices, D); };
+            if (vec && D <= 8 * VEC) narrow(softmax_row_kernel<T, 8, VEC, 1>, 8);
+            else if (vec && D <= 16 * VEC) narrow(softmax_row_kernel<T, 16, VEC, 1>, 16);
+            else if (vec && D <= 32 * VEC) narrow(softmax_row_kernel<T, 32, VEC, 1>, 32);
+            else if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, VEC, 2048 / (WAVE * VEC)>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
             else hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, 1, 8>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
         } else {
             if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, SB, VEC, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);

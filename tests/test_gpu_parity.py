@@ -880,7 +880,9 @@ SOFTMAX_CASES = [([2, 3], 1), ([2, 2, 3], 2), ([2, 3], 0), ([64, 5], 1), ([33, 2
                  # long inner columns: the block-split kernel with narrow and with 16-byte column vectors
                  ([3, 200, 132], 1), ([300, 64, 128], 1), ([1000, 70], 0),
                  # few slabs of long columns: the rows in groups, three launches (a ragged last group, dead lanes, pre > 1)
-                 ([2048, 264], 0), ([1100, 520], 0), ([3, 1500, 136], 1), ([4096, 1024], 0)]
+                 ([2048, 264], 0), ([1100, 520], 0), ([3, 1500, 136], 1), ([4096, 1024], 0),
+                 # short rows: 8, 16 or 32 lanes each (a ragged last block, rows that fill a group exactly or in part)
+                 ([3001, 32], 1), ([70, 9, 64], 2), ([333, 128], 1), ([101, 256], 1), ([1000, 16], 1), ([517, 8], 1), ([259, 200], 1)]
 
 
 @pytest.mark.parametrize("dt", DTS)
@@ -910,7 +912,31 @@ def test_softmax(oracle, hip, shape, dim, dt):
         truth = (e / e.sum(axis=axis, keepdims=True)).ravel()
         assert np.all(np.abs(got - truth) <= 1e-2 * truth + (2.0 ** -24 if dt == "f16" else 1e-30))      # f16 subnormal spacing
         if shape[axis] <= 8:
-            assert np.max(np.abs(got - to_float(o, dt))) <= 2.0 ** -7
+            # the reference's running sum of D terms in the 16-bit type: at most D - 1 roundings of half a unit in its last place
+            ref = to_float(o, dt).astype(np.float64)
+            assert np.all(np.abs(got - ref) <= shape[axis] * 2.0 ** -8 * np.maximum(got, ref) + 2.0 ** -24)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("rows,D", [(2100, 2048), (8100, 520), (520, 8192), (515, 8200), (1030, 4096), (1400, 3000),
+                                    (131101, 32), (65603, 64), (32801, 128), (16401, 256), (262201, 16), (524301, 8)])
+def test_softmax_16bit_rows_by_table_are_the_arithmetic_kernels_bits(hip, rows, D, dt):
+    """A large 16-bit softmax along the last dim takes exp(x - m) from the dtype's table of exp; a call of fewer than 2^22
+    elements computes it.  Same rows, same bits - and the known sum of every row."""
+    r = rng(127)
+    x = to_storage((r.standard_normal(rows * D) * 3).astype(np.float32), dt)
+    x[:7] = to_storage(np.array([-np.inf, np.inf, np.nan, 0.0, -0.0, 88.0, -104.0], np.float32), dt)    # row 0: special values
+    md = meta_unary([rows, D], [D, 1], 0)
+    (big,) = hip.call(f"softmax_{dt}", rows * D, 2, 1, md, In(x), Out(rows * D, dt))
+    assert rows * D >= 1 << 22
+    part = max(1, ((1 << 22) - 1) // D)
+    for r0 in list(range(0, rows, part))[:3] + [rows - min(part, rows)]:
+        n = min(part, rows - r0)
+        mdp = meta_unary([n, D], [D, 1], 0)
+        (small,) = hip.call(f"softmax_{dt}", n * D, 2, 1, mdp, In(x[r0 * D:(r0 + n) * D]), Out(n * D, dt))
+        assert same_bits(small, big[r0 * D:(r0 + n) * D]), r0
+    sums = to_float(big, dt).reshape(rows, D)[1:].astype(np.float64).sum(1)
+    assert np.all(np.abs(sums - 1.0) <= 2e-2)
 
 
 def test_softmax_strided_and_special_values(oracle, hip):
