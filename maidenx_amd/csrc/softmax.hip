@@ -364,15 +364,26 @@ __global__ __launch_bounds__(WAVE * NW) void softmax_col_split_kernel(const T* _
 //   PHASE 2: out = exp(x - m) / s
 // with softmax_col_fold_kernel between them, which folds the groups' values of a column in group order into
 // m[pre][post] (exact) and s[pre][post] = exp(-inf - m) + sum.
-template <class T, int VEC, int PHASE, bool STREAM>
-__global__ __launch_bounds__(256) void softmax_col_groups_kernel(const T* __restrict__ in, T* __restrict__ out, float* __restrict__ part,
-                                                                 const float* __restrict__ cmax, const float* __restrict__ csum, size_t D,
-                                                                 size_t post, uint32_t cv, uint32_t slabs, uint32_t groups,
-                                                                 uint32_t rows_per_group) {
+// LUT (bf16 / f16): exp(x - m) is the entry of the dtype's table of exp, held in LDS, for the code of the rounded
+// difference - the bits SM<T>::shifted computes (see softmax_row_lut_kernel).
+template <class T, int VEC, int PHASE, bool STREAM, bool LUT>
+__device__ __forceinline__ void softmax_col_groups_body(uint32_t vblock, uint32_t tid, const uint16_t* lut, const T* __restrict__ in,
+                                                        T* __restrict__ out, float* __restrict__ part, const float* __restrict__ cmax,
+                                                        const float* __restrict__ csum, size_t D, size_t post, uint32_t cv, uint32_t slabs,
+                                                        uint32_t groups, uint32_t rows_per_group) {
     constexpr int U = 8;
-    const uint32_t slab = blockIdx.x % slabs, group = (blockIdx.x / slabs) % groups, pre_idx = blockIdx.x / (slabs * groups);
-    const uint32_t j = slab * 256 + threadIdx.x;           // column vector
+    const uint32_t slab = vblock % slabs, group = (vblock / slabs) % groups, pre_idx = vblock / (slabs * groups);
+    const uint32_t j = slab * 256 + tid;                   // column vector
     if (j >= cv) return;
+    auto term = [&](T x, float mx) -> float {
+        if constexpr (LUT) {
+            T en;
+            en.bits = lut[SMCode<T>::of(SM<T>::ld(x) - mx)];
+            return SM<T>::ld(en);
+        } else {
+            return SM<T>::shifted(SM<T>::ld(x), mx);
+        }
+    };
     const size_t l0 = (size_t)group * rows_per_group < D ? (size_t)group * rows_per_group : D;
     const size_t l1 = l0 + rows_per_group < D ? l0 + rows_per_group : D;
     const T* src = in + (size_t)pre_idx * D * post + (size_t)j * VEC;
@@ -411,7 +422,7 @@ __global__ __launch_bounds__(256) void softmax_col_groups_kernel(const T* __rest
             for (int e = 0; e < VEC; ++e) s[e] = 0.0f;
             sweep([&](size_t, const AVec<T, VEC>& v) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) s[e] += SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]);
+                for (int e = 0; e < VEC; ++e) s[e] += term(v.v[e], m[e]);
             });
             AVec<float, VEC> r;
 #pragma unroll
@@ -424,11 +435,34 @@ __global__ __launch_bounds__(256) void softmax_col_groups_kernel(const T* __rest
             sweep([&](size_t l, const AVec<T, VEC>& v) {
                 AVec<T, VEC> o;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(v.v[e]), m[e]), s[e]);
+                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(term(v.v[e], m[e]), s[e]);
                 st_vec<STREAM>((AVec<T, VEC>*)(dst + l * post), o);
             });
         }
     }
+}
+template <class T, int VEC, int PHASE, bool STREAM>
+__global__ __launch_bounds__(256) void softmax_col_groups_kernel(const T* __restrict__ in, T* __restrict__ out, float* __restrict__ part,
+                                                                 const float* __restrict__ cmax, const float* __restrict__ csum, size_t D,
+                                                                 size_t post, uint32_t cv, uint32_t slabs, uint32_t groups,
+                                                                 uint32_t rows_per_group) {
+    softmax_col_groups_body<T, VEC, PHASE, STREAM, false>(blockIdx.x, threadIdx.x, nullptr, in, out, part, cmax, csum, D, post, cv, slabs, groups,
+                                                          rows_per_group);
+}
+// The same work by one persistent 1024-thread block per CU that holds the table: every quarter of the block is one block
+// of the kernel above after the other (no barrier between them: a thread's columns are its own).
+template <class T, int VEC, int PHASE, bool STREAM>
+__global__ __launch_bounds__(1024) void softmax_col_groups_lut_kernel(const uint16_t* __restrict__ table, uint32_t vblocks, const T* __restrict__ in,
+                                                                      T* __restrict__ out, float* __restrict__ part, const float* __restrict__ cmax,
+                                                                      const float* __restrict__ csum, size_t D, size_t post, uint32_t cv,
+                                                                      uint32_t slabs, uint32_t groups, uint32_t rows_per_group) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    for (int i = threadIdx.x; i < 65536 * 2 / 16; i += 1024) ((u4*)lut)[i] = ((const u4*)table)[i];
+    __syncthreads();
+    for (uint32_t vb = blockIdx.x * 4 + threadIdx.x / 256; vb < vblocks; vb += gridDim.x * 4)
+        softmax_col_groups_body<T, VEC, PHASE, STREAM, true>(vb, threadIdx.x % 256, lut, in, out, part, cmax, csum, D, post, cv, slabs, groups,
+                                                             rows_per_group);
 }
 
 // SUM ? s = exp(-inf - m) + part[0] + part[1] + ... : m = max(part[0], part[1], ...) for every column.  A block is 64
@@ -599,11 +633,41 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
 #define MXH_SM_PHASE(P)                                                                                                                   \
     if (big) hipLaunchKernelGGL((softmax_col_groups_kernel<T, VEC, P, true>), grid, block, 0, stream(), src, out, part, cm, cs, D, post, cv, slabs, groups, rpg); \
     else hipLaunchKernelGGL((softmax_col_groups_kernel<T, VEC, P, false>), grid, block, 0, stream(), src, out, part, cm, cs, D, post, cv, slabs, groups, rpg)
+            // 16-bit, 2^22 elements or more: the two phases with exp in them by table, one persistent block per CU
+            const uint16_t* table = nullptr;
+            int dev = 0, cus = 0;
+            if constexpr (sizeof(T) == 2) {
+                if (num_els >= (1u << 22) && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 16) {
+                    table = std::is_same<T, bf16_t>::value ? lut16_exp_bf16() : lut16_exp_f16();
+                    static int cu_count[16] = {0};
+                    if (!cu_count[dev]) {
+                        hipDeviceProp_t prop;
+                        cu_count[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+                    }
+                    cus = cu_count[dev];
+                }
+            }
+            auto by_table = [&](auto kern) {
+                static bool allowed[16] = {false};
+                if (!table) return false;
+                if (!allowed[dev]) {
+                    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 65536 * 2) != hipSuccess) { (void)hipGetLastError(); return false; }
+                    allowed[dev] = true;
+                }
+                const uint32_t vblocks = grid.x;
+                hipLaunchKernelGGL(kern, dim3(std::min<unsigned>((unsigned)cus, (unsigned)cdiv((size_t)vblocks, (size_t)4))), dim3(1024), 65536 * 2, stream(), table,
+                                   vblocks, src, out, part, (const float*)cm, (const float*)cs, D, post, cv, slabs, groups, rpg);
+                return true;
+            };
+            bool done = false;
             MXH_SM_PHASE(0);
             hipLaunchKernelGGL((softmax_col_fold_kernel<false>), fold, fold_block, 0, stream(), part, (const float*)nullptr, cm, post, cols, groups);
-            MXH_SM_PHASE(1);
+            if constexpr (sizeof(T) == 2) done = big ? by_table(softmax_col_groups_lut_kernel<T, VEC, 1, true>) : by_table(softmax_col_groups_lut_kernel<T, VEC, 1, false>);
+            if (!done) { MXH_SM_PHASE(1); }
             hipLaunchKernelGGL((softmax_col_fold_kernel<true>), fold, fold_block, 0, stream(), part, cm, cs, post, cols, groups);
-            MXH_SM_PHASE(2);
+            done = false;
+            if constexpr (sizeof(T) == 2) done = big ? by_table(softmax_col_groups_lut_kernel<T, VEC, 2, true>) : by_table(softmax_col_groups_lut_kernel<T, VEC, 2, false>);
+            if (!done) { MXH_SM_PHASE(2); }
 #undef MXH_SM_PHASE
             MXH_LAUNCH_CHECK("softmax_col_groups");
             return;

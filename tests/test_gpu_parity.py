@@ -939,6 +939,27 @@ def test_softmax_16bit_rows_by_table_are_the_arithmetic_kernels_bits(hip, rows, 
     assert np.all(np.abs(sums - 1.0) <= 2e-2)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("pre,D,post,sub", [(1, 4096, 2048, 512), (2, 1500, 2048, 512), (1, 8190, 1024, 256)])
+def test_softmax_16bit_columns_by_table_are_the_arithmetic_kernels_bits(hip, pre, D, post, sub, dt):
+    """Long columns in groups of rows: a 16-bit call of 2^22 elements or more takes exp(x - m) from the table.  The same
+    columns as a call of fewer elements (same D and as many groups, so the same order of additions) are computed: same bits."""
+    r = rng(139)
+    n = pre * D * post
+    x = to_storage((r.standard_normal(n) * 3).astype(np.float32), dt).reshape(pre, D, post)
+    x[0, :7, 3] = to_storage(np.array([-np.inf, np.inf, np.nan, 0.0, -0.0, 88.0, -104.0], np.float32), dt)
+    x[0, :, 5] = to_storage(np.full(D, -np.inf, np.float32), dt)
+    assert n >= 1 << 22 and pre * D * sub < 1 << 22
+    (big,) = hip.call(f"softmax_{dt}", n, 3, 1, meta_unary([pre, D, post], contiguous_strides([pre, D, post]), 0), In(x.ravel()), Out(n, dt))
+    big = big.reshape(pre, D, post)
+    for c0 in (0, post - sub):
+        part = np.ascontiguousarray(x[:, :, c0:c0 + sub])
+        (small,) = hip.call(f"softmax_{dt}", part.size, 3, 1, meta_unary([pre, D, sub], contiguous_strides([pre, D, sub]), 0), In(part.ravel()), Out(part.size, dt))
+        assert same_bits(small, np.ascontiguousarray(big[:, :, c0:c0 + sub]).ravel()), c0
+    sums = to_float(big.ravel(), dt).reshape(pre, D, post).astype(np.float64).sum(1)[:, 8:]
+    assert np.all(np.abs(sums - 1.0) <= 2e-2)
+
+
 def test_softmax_strided_and_special_values(oracle, hip):
     r = rng(127)
     lay = LY.permuted([6, 9], [1, 0], off=2)
