@@ -26,17 +26,20 @@ template <> struct SM<float> {
     static __device__ float ld(float v) { return v; }
     static __device__ float shifted(float x, float m) { return m_exp(x - m); }     // exp(x - m)
     static __device__ float fin(float e, float s) { return e / s; }
+    static __device__ void keep(float& slot, float e) { slot = e; }
 };
 template <> struct SM<bf16_t> {
     static __device__ float ld(bf16_t v) { return bf2f(v); }
     static __device__ float shifted(float x, float m) { return bf2f(f2bf(m_exp(bf2f(f2bf(x - m))))); }
     static __device__ bf16_t fin(float e, float s) { return f2bf(e / bf2f(f2bf(s))); }
+    static __device__ void keep(bf16_t& slot, float e) { slot = f2bf(e); }         // e is a bf16 value: exact
 };
 
 template <> struct SM<f16_t> {
     static __device__ float ld(f16_t v) { return h2f(v); }
     static __device__ float shifted(float x, float m) { return h2f(f2h(m_exp(h2f(f2h(x - m))))); }
     static __device__ f16_t fin(float e, float s) { return f2h(e / h2f(f2h(s))); }
+    static __device__ void keep(f16_t& slot, float e) { slot = f2h(e); }
 };
 
 constexpr int SB = 256;
@@ -59,9 +62,10 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
-// rows of length D, TPR threads per row (8, 16, 32, WAVE or SB); NREG vectors of the row live in registers, longer
-// rows are read again from cache in each phase
-template <class T, int TPR, int VEC, int NREG>
+// rows of length D, TPR threads per row (8, 16, 32, WAVE or SB).  FITS: the row is held in registers, NREG vectors a
+// thread (the host has checked D <= TPR * VEC * NREG), and exp(x - m) - a value of T - replaces x there, computed once;
+// otherwise the row is read again from cache in each phase.
+template <class T, int TPR, int VEC, int NREG, bool FITS>
 __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ in, T* __restrict__ out, size_t rows, size_t D) {
     constexpr int RPB = SB / TPR;
     const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / TPR;
@@ -70,28 +74,34 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
     const T* src = in + (live ? row : 0) * D;
     T* dst = out + (live ? row : 0) * D;
     __shared__ float red[SB / WAVE];
-    AVec<T, VEC> keep[NREG];
+    AVec<T, VEC> keep[FITS ? NREG : 1];
     const size_t step = (size_t)TPR * VEC;
-    const bool fits = D <= step * NREG;
+    auto load = [&](size_t i) {
+        AVec<T, VEC> v;
+        if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
+        else v.v[0] = src[i];
+        return v;
+    };
+    auto store = [&](size_t i, const AVec<T, VEC>& o) {
+        if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
+        else dst[i] = o.v[0];
+    };
 
     float m = -INFINITY;
     if (live) {
-        if (fits) {
+        if constexpr (FITS) {
 #pragma unroll
             for (int k = 0; k < NREG; ++k) {
-                size_t i = (size_t)t * VEC + k * step;
+                const size_t i = (size_t)t * VEC + k * step;
                 if (i < D) {
-                    if constexpr (VEC > 1) keep[k] = *(const AVec<T, VEC>*)(src + i);
-                    else keep[k].v[0] = src[i];
+                    keep[k] = load(i);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(keep[k].v[e]); m = x > m ? x : m; }
                 }
             }
         } else {
             for (size_t i = (size_t)t * VEC; i < D; i += step) {
-                AVec<T, VEC> v;
-                if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
-                else v.v[0] = src[i];
+                const AVec<T, VEC> v = load(i);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) { float x = SM<T>::ld(v.v[e]); m = x > m ? x : m; }
             }
@@ -108,22 +118,23 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
     }
 
     float s = 0.0f;
-    float ev[NREG][VEC];          // exp(x - m) of the held part of the row: computed once
     if (live) {
-        if (fits) {
+        if constexpr (FITS) {
 #pragma unroll
             for (int k = 0; k < NREG; ++k) {
-                size_t i = (size_t)t * VEC + k * step;
+                const size_t i = (size_t)t * VEC + k * step;
                 if (i < D) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) { ev[k][e] = SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m); s += ev[k][e]; }
+                    for (int e = 0; e < VEC; ++e) {
+                        const float ev = SM<T>::shifted(SM<T>::ld(keep[k].v[e]), m);
+                        SM<T>::keep(keep[k].v[e], ev);
+                        s += ev;
+                    }
                 }
             }
         } else {
             for (size_t i = (size_t)t * VEC; i < D; i += step) {
-                AVec<T, VEC> v;
-                if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
-                else v.v[0] = src[i];
+                const AVec<T, VEC> v = load(i);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) s += SM<T>::shifted(SM<T>::ld(v.v[e]), m);
             }
@@ -140,27 +151,24 @@ __global__ __launch_bounds__(SB) void softmax_row_kernel(const T* __restrict__ i
     s = m_exp(-INFINITY - m) + s;      // 0, or NaN when no element beat -inf
 
     if (!live) return;
-    if (fits) {
+    if constexpr (FITS) {
 #pragma unroll
         for (int k = 0; k < NREG; ++k) {
-            size_t i = (size_t)t * VEC + k * step;
+            const size_t i = (size_t)t * VEC + k * step;
             if (i < D) {
                 AVec<T, VEC> o;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(ev[k][e], s);
-                if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
-                else dst[i] = o.v[0];
+                for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::ld(keep[k].v[e]), s);
+                store(i, o);
             }
         }
     } else {
         for (size_t i = (size_t)t * VEC; i < D; i += step) {
-            AVec<T, VEC> v, o;
-            if constexpr (VEC > 1) v = *(const AVec<T, VEC>*)(src + i);
-            else v.v[0] = src[i];
+            const AVec<T, VEC> v = load(i);
+            AVec<T, VEC> o;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) o.v[e] = SM<T>::fin(SM<T>::shifted(SM<T>::ld(v.v[e]), m), s);
-            if constexpr (VEC > 1) *(AVec<T, VEC>*)(dst + i) = o;
-            else dst[i] = o.v[0];
+            store(i, o);
         }
     }
 }
@@ -600,14 +608,16 @@ void softmax(size_t num_els, size_t nd, size_t dim_arg, const size_t* md, const 
             unsigned blocks = cdiv(slices, SB / WAVE);
             // short rows: 8, 16 or 32 lanes each, so that a wave holds several
             auto narrow = [&](auto kern, int tpr) { hipLaunchKernelGGL(kern, dim3((unsigned)cdiv(slices, (size_t)(SB / tpr))), dim3(SB), 0, stream(), src, out, slices, D); };
-            if (vec && D <= 8 * VEC) narrow(softmax_row_kernel<T, 8, VEC, 1>, 8);
-            else if (vec && D <= 16 * VEC) narrow(softmax_row_kernel<T, 16, VEC, 1>, 16);
-            else if (vec && D <= 32 * VEC) narrow(softmax_row_kernel<T, 32, VEC, 1>, 32);
-            else if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, VEC, 2048 / (WAVE * VEC)>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
-            else hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, 1, 8>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
+            if (vec && D <= 8 * VEC) narrow(softmax_row_kernel<T, 8, VEC, 1, true>, 8);
+            else if (vec && D <= 16 * VEC) narrow(softmax_row_kernel<T, 16, VEC, 1, true>, 16);
+            else if (vec && D <= 32 * VEC) narrow(softmax_row_kernel<T, 32, VEC, 1, true>, 32);
+            else if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, VEC, 2048 / (WAVE * VEC), true>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
+            else if (D <= WAVE * 8) hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, 1, 8, true>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
+            else hipLaunchKernelGGL((softmax_row_kernel<T, WAVE, 1, 8, false>), dim3(blocks), dim3(SB), 0, stream(), src, out, slices, D);
         } else {
-            if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, SB, VEC, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
-            else hipLaunchKernelGGL((softmax_row_kernel<T, SB, 1, 8>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
+            if (vec && D <= (size_t)SB * VEC * 8) hipLaunchKernelGGL((softmax_row_kernel<T, SB, VEC, 8, true>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
+            else if (vec) hipLaunchKernelGGL((softmax_row_kernel<T, SB, VEC, 8, false>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
+            else hipLaunchKernelGGL((softmax_row_kernel<T, SB, 1, 8, false>), dim3((unsigned)slices), dim3(SB), 0, stream(), src, out, slices, D);
         }
         MXH_LAUNCH_CHECK("softmax_row");
         return;
