@@ -416,6 +416,13 @@ inline size_t ew_stream_bytes() {
     return v;
 }
 
+// A functor may bring a kernel of its own for the vector form of the transposed-view path (lut16.hpp does, for the table
+// functor): launch(...) returns false to leave the launch to ew_trv_kernel.
+template <class Op>
+struct TrvOverride {
+    static bool launch(const NdSpace<Op::NIN + 1>&, const EwPtrs<Op::NIN>&, const TrPlan<Op::NIN>&, size_t, bool, const Op&) { return false; }
+};
+
 // ---- host-side selection -------------------------------------------------------------------
 // in_strides[k] / out_strides are in elements, pointers already include the operand offsets.
 template <class Op>
@@ -489,6 +496,7 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
                 for (int d = 0; d < last; ++d)
                     if (d != pd) outer *= sp.dims[d];
                 size_t blocks = outer * pl.tiles_p * pl.tiles_l;
+                if (TrvOverride<Op>::launch(sp, p, pl, blocks, streams, op)) return;
                 if (streams) hipLaunchKernelGGL((ew_trv_kernel<Op, true>), dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream(), sp, p, pl, op);
                 else hipLaunchKernelGGL((ew_trv_kernel<Op, false>), dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream(), sp, p, pl, op);
                 MXH_LAUNCH_CHECK("ew_trv");

@@ -313,6 +313,10 @@ def test_large_16bit_unary_calls_go_through_the_table_and_keep_the_bits(oracle, 
     rows, cols = 1040, 1024                                                                       # [1040,1024] view of a [1024,1040] buffer
     (ht,) = hip.call(f"{op}_{dt}", rows * cols, 2, meta_unary([rows, cols], [1, rows]), In(x[: rows * cols]), Out(rows * cols, dt))
     assert np.array_equal(ht.reshape(rows, cols), want[: rows * cols].reshape(cols, rows).T)
+    # [2,1024,512] view of a [2,512,1024] buffer: an outer dim, and tile counts that take the 8x8 block order
+    xb = np.tile(x, 1)[: 2 * 512 * 1024]
+    (hb,) = hip.call(f"{op}_{dt}", xb.size, 3, meta_unary([2, 1024, 512], [512 * 1024, 1, 1024]), In(xb), Out(xb.size, dt))
+    assert np.array_equal(hb.reshape(2, 1024, 512), want[: xb.size].reshape(2, 512, 1024).transpose(0, 2, 1))
     if op in ("exp", "tanh", "gelu", "sigmoid"):
         (o,) = oracle.call(f"{op}_{dt}", n, 1, meta_unary([n], [1]), In(x), Out(n, dt))
         ok = ~np.isnan(to_float(o, dt))
