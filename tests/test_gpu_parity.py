@@ -288,6 +288,22 @@ def test_tanh_and_gelu_f32_bit_exact_on_16m_inputs(oracle, hip, op):
     assert bad.size == 0, (bad.size, x[ok][bad[:5]], o[ok][bad[:5]], h[ok][bad[:5]])
 
 
+@pytest.mark.parametrize("dt,shape,perm", [("f32", [2056, 2120], [1, 0]), ("f32", [5, 1032, 1024], [0, 2, 1]), ("f32", [3, 1032, 1024], [2, 1, 0]),
+                                           ("bf16", [4104, 2120], [1, 0]), ("f16", [3, 2056, 2048], [0, 2, 1])])
+def test_unary_on_transposed_views_of_a_thousand_tiles_and_more(oracle, hip, dt, shape, perm):
+    """Transposed views of a thousand tiles and more: ragged edge tiles, an outer dim, the 8x8 tile order - bit for bit
+    the oracle (exp on the 16-bit dtypes is the table functor's standing grid, the others one block a tile)."""
+    r = rng(173)
+    n = int(np.prod(shape))
+    x = to_storage(r.standard_normal(n).astype(np.float32) * 2, dt)
+    base = [shape[perm.index(d)] for d in range(len(shape))]            # the buffer's own shape
+    bs = contiguous_strides(base)
+    md = meta_unary(shape, [bs[p] for p in perm], 0)
+    for op in ("neg", "relu", "exp"):
+        (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(shape), md, In(x), Out(n, dt)))
+        assert same_bits(o, h), op
+
+
 TABLE_OPS = ["sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln", "log10", "log2", "exp", "exp10", "exp2", "softplus"]
 
 
