@@ -81,7 +81,12 @@ __device__ __forceinline__ void ew_nd_body(const Space& sp, const EwPtrs<Op::NIN
     const int last = sp.ndims - 1;
     size_t v0 = (size_t)bid * (EW_BLOCK * UNR) + tid;
 
-    In vals[UNR][NIN][VEC];
+    // The operands stay packed, as the words they arrived in, until the arithmetic: a narrow dtype unpacked where it is
+    // loaded makes every load wait for its data before the next one is issued (add_u8: one 16-byte load in flight).
+    using InVec = AVec<In, VEC>;
+    using InRaw = typename RawVec<sizeof(InVec)>::type;
+    using Held = std::conditional_t<std::is_void<InRaw>::value, InVec, InRaw>;
+    Held vals[UNR][NIN];
     int64_t ooff[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
@@ -111,20 +116,24 @@ __device__ __forceinline__ void ew_nd_body(const Space& sp, const EwPtrs<Op::NIN
         for (int k = 0; k < NIN; ++k) {
             const In* src = (const In*)p.in[k] + off[k + 1];
             if constexpr (VEC == 1) {
-                vals[u][k][0] = src[0];
+                InVec t;
+                t.v[0] = src[0];
+                vals[u][k] = __builtin_bit_cast(Held, t);
             } else {
                 const int64_t s = sp.strides[k + 1][last];
                 if (s == 1) {
-                    AVec<In, VEC> t = k == 0 ? ld_vec<(STREAM & 2) != 0>((const AVec<In, VEC>*)src) : ld_vec<(STREAM & 4) != 0>((const AVec<In, VEC>*)src);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) vals[u][k][e] = t.v[e];
+                    vals[u][k] = k == 0 ? ld_vec<(STREAM & 2) != 0>((const Held*)src) : ld_vec<(STREAM & 4) != 0>((const Held*)src);
                 } else if (s == 0) {
-                    In t = src[0];
+                    InVec t;
+                    t.v[0] = src[0];
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) vals[u][k][e] = t;
+                    for (int e = 1; e < VEC; ++e) t.v[e] = t.v[0];
+                    vals[u][k] = __builtin_bit_cast(Held, t);
                 } else {
+                    InVec t;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) vals[u][k][e] = src[(int64_t)e * s];
+                    for (int e = 0; e < VEC; ++e) t.v[e] = src[(int64_t)e * s];
+                    vals[u][k] = __builtin_bit_cast(Held, t);
                 }
             }
         }
@@ -134,10 +143,13 @@ __device__ __forceinline__ void ew_nd_body(const Space& sp, const EwPtrs<Op::NIN
         size_t v = v0 + (size_t)u * EW_BLOCK;
         if (v >= nvec) break;
         AVec<Out, VEC> r;
+        InVec x[NIN];
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) x[k] = __builtin_bit_cast(InVec, vals[u][k]);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            if constexpr (NIN == 1) r.v[e] = op(vals[u][0][e]);
-            else r.v[e] = op(vals[u][0][e], vals[u][1][e]);
+            if constexpr (NIN == 1) r.v[e] = op(x[0].v[e]);
+            else r.v[e] = op(x[0].v[e], x[1].v[e]);
         }
         Out* dst = (Out*)p.out + ooff[u];
         if constexpr (VEC == 1) {
