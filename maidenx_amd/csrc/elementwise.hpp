@@ -183,6 +183,7 @@ struct TrPlan {
     uint32_t tiles_p, tiles_l;
     FastDiv div_tiles_l, div_tiles_p;
     uint32_t super;        // 8x8 super-tile block order (both tile counts are multiples of 8)
+    uint32_t same;         // two inputs, one and the same view (x * x): staged once, read twice from the tile
 };
 
 template <class Op>
@@ -309,7 +310,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_trv_kernel(NdSpace<Op::NIN + 1> s
     constexpr int N1 = TL * VPR / EW_BLOCK;             // 4 vectors per thread
 #pragma unroll
     for (int k = 0; k < NIN; ++k) {
-        if (!((pl.staged >> k) & 1u)) continue;
+        if (!((pl.staged >> k) & 1u) || (k == 1 && pl.same)) continue;
         const In* src = (const In*)p.in[k] + base[k + 1];
         const int64_t sl = sp.strides[k + 1][last];
         AVec<In, VEC> v[N1];
@@ -345,8 +346,13 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_trv_kernel(NdSpace<Op::NIN + 1> s
 #pragma unroll
         for (int k = 0; k < NIN; ++k) {
             if ((pl.staged >> k) & 1u) {
+                if (k == 1 && pl.same) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) x[k][e] = tile[k][(jl + e) * PITCH + il];
+                    for (int e = 0; e < VEC; ++e) x[1][e] = x[0][e];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) x[k][e] = tile[k][(jl + e) * PITCH + il];
+                }
             } else {
                 const In* src = (const In*)p.in[k] + base[k + 1] + (int64_t)i * sp.strides[k + 1][pd] + (int64_t)j * sp.strides[k + 1][last];
                 const int64_t s = sp.strides[k + 1][last];
@@ -625,6 +631,12 @@ void ew_launch(size_t num_els, size_t num_dims, const size_t* dims, const size_t
                 }
             }
             pl.super = 0;
+            pl.same = 0;
+            if constexpr (NIN == 2) {
+                bool same = staged == 3u && in[0] == in[1];
+                for (int d = 0; d <= last && same; ++d) same = sp.strides[1][d] == sp.strides[2][d];
+                pl.same = same ? 1u : 0u;
+            }
             if constexpr (sizeof(In) == 2 || sizeof(In) == 4) if (trv) {      // (the vector tiles are laid out for 16- and 32-bit elements)
                 pl.tiles_p = cdiv(sp.dims[pd], TrvCfg<In>::TP);
                 pl.tiles_l = cdiv(sp.dims[last], TrvCfg<In>::TL);

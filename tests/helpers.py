@@ -191,14 +191,18 @@ class Runner:
         fn = getattr(self.lib, self.prefix + name)
         cargs, post = [], []
         keep = []
+        seen = {}
         for a in args:
             if isinstance(a, Null) or a is None:
                 cargs.append(None)
             elif isinstance(a, (In, Out)):
                 if self.kind == "oracle":
                     cargs.append(a.arr.ctypes.data)
+                elif id(a) in seen:                      # the same In object given twice: one buffer, the same pointer
+                    cargs.append(seen[id(a)].ptr)
                 else:
                     buf = self.L.DeviceBuffer.from_numpy(a.arr)
+                    seen[id(a)] = buf
                     keep.append(buf)
                     cargs.append(buf.ptr)
                     if isinstance(a, (Out, InOut)):

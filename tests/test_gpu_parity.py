@@ -304,6 +304,24 @@ def test_unary_on_transposed_views_of_a_thousand_tiles_and_more(oracle, hip, dt,
         assert same_bits(o, h), op
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape", [[264, 328], [3, 136, 200]])
+def test_binary_of_one_transposed_view_given_twice(oracle, hip, dt, shape):
+    """x * x, x + x, x - y with x one and the same transposed view (same pointer, same strides): the tile of x is staged
+    once and read for both operands; a second view of ANOTHER buffer with the same strides must not be taken for it."""
+    r = rng(179)
+    n = int(np.prod(shape))
+    x, y = In(to_storage(r.standard_normal(n).astype(np.float32), dt)), In(to_storage(r.standard_normal(n).astype(np.float32), dt))
+    base = shape[:-2] + [shape[-1], shape[-2]]
+    st = contiguous_strides(base)
+    st = st[:-2] + [st[-1], st[-2]]
+    md = meta_binary(shape, st, st)
+    for op in ("mul", "add", "sub"):
+        for a, b in ((x, x), (x, y)):
+            (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(shape), md, a, b, Out(n, dt)))
+            assert same_bits(o, h), (op, a is b)
+
+
 TABLE_OPS = ["sigmoid", "tanh", "gelu", "sin", "cos", "tan", "ln", "log10", "log2", "exp", "exp10", "exp2", "softplus"]
 
 
