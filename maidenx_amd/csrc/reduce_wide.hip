@@ -8,9 +8,13 @@
 #include <cfloat>
 
 #include "elementwise.hpp"
+#include "ops.hpp"
 #include "mxh.hpp"
 
 namespace mxh {
+
+bool capture_open();      // runtime.hip: a graph capture is being recorded
+
 
 constexpr int WB = 256;
 
@@ -305,6 +309,23 @@ static void wreduce_axis(size_t num_els, size_t num_dims, size_t nred, const siz
         return;
     }
     if (num_els >= (1ull << 31)) { set_status(ERR_TOO_LARGE, "reduce: strided input with 2^31 or more elements"); return; }
+    // A large strided input whose logical index space divides into whole slices is copied into logical order (the
+    // elementwise identity walks the view by the reference's index rule) and reduced as the contiguous layout
+    // [outer, L, s] the reference's formula describes - see reduce_axis in reduce.hip.
+    {
+        const size_t se = s != 0 ? s : 1;
+        if (num_els >= (1u << 18) && num_dims <= 64 && num_els % (L * se) == 0 && !capture_open()) {
+            T* tmp = (T*)scratch(num_els * sizeof(T), 1);
+            if (!tmp) return;
+            size_t cs[64];
+            contiguous_strides(num_dims, dims, cs);
+            const size_t* ins[1] = {strides};
+            const void* inp[1] = {src};
+            ew_launch<OpIdentity<T>>(num_els, num_dims, dims, cs, ins, tmp, inp, OpIdentity<T>{});
+            wreduce<T, R>(tmp, out, num_els / (L * se), L, se, div);
+            return;
+        }
+    }
     if (num_dims > (size_t)MAXD) { set_status(ERR_UNSUPPORTED, "reduce: strided input of rank above 8"); return; }
     NdSpace<1> sp;            // not collapsed: the walk must visit the dims exactly as the reference's index function does
     sp.ndims = (int)(num_dims ? num_dims : 1);

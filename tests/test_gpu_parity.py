@@ -424,6 +424,31 @@ def test_reduce_strided_input_follows_reference_quirk(oracle, hip):
         assert np.allclose(o, h, atol=1e-6)
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dims,perm", [([520, 640], [1, 0]), ([40, 72, 128], [2, 0, 1]), ([6, 300, 200], [0, 2, 1])])
+def test_reduce_large_strided_input_is_the_reduction_of_its_logical_copy(oracle, hip, dims, perm, dt):
+    """From 2^18 elements a strided input is copied into logical order and reduced as a contiguous tensor: the same
+    elements per output as the reference's walk (max and min are order-independent: bit for bit), sums to rounding."""
+    lay = LY.permuted(dims, perm)
+    r = rng(181)
+    st = to_storage(r.uniform(-1, 1, lay["size"]).astype(np.float32), dt)
+    n = int(np.prod(lay["dims"]))
+    assert n >= 1 << 18
+    for dim in range(len(dims)):
+        md = meta_reduce(lay["dims"], lay["strides"], dim, 0)
+        out_n = n // lay["dims"][dim]
+        for op in ("max", "min"):
+            (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(dims), 1, md, In(st), Out(out_n, dt)))
+            assert same_bits(o, h), (op, dim)
+        for op in ("sum", "mean"):
+            (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(dims), 1, md, In(st), Out(out_n, dt)))
+            if dt == "f32":
+                assert np.allclose(o, h, rtol=1e-5, atol=2e-4), (op, dim)
+            else:
+                # the reference's bf16 running sum against an f32 sum rounded once: loose, the index sets are pinned by max / min
+                assert np.allclose(to_float(o, dt), to_float(h, dt), rtol=0.1, atol=1.0), (op, dim)
+
+
 STS_CASES = [([64, 96], [64, 96]), ([64, 96], [1, 96]), ([64, 96], [64, 1]), ([8, 64, 128], [1, 64, 1]), ([8, 64, 128], [8, 1, 128]),
              ([2, 3, 4, 5], [1, 3, 1, 5]), ([2, 3, 4, 5], [2, 1, 4, 1]), ([10000, 1], [10000, 1]), ([10000, 1], [1, 1]), ([5], [1]),
              ([300, 700], [1, 1]), ([2, 3, 4, 5, 6], [1, 3, 1, 5, 1]),
@@ -1580,6 +1605,26 @@ def test_sum_to_shape_wide_dtypes(oracle, hip, shape, out_shape, dt):
     axes = tuple(i for i, (a, b) in enumerate(zip(shape, out_shape)) if a != b)
     scale = np.abs(x.reshape(shape)).sum(axis=axes).ravel() if axes else np.abs(x)
     assert np.max(np.abs(h - o) / np.maximum(scale, 1e-300)) <= 1e-13
+
+
+@pytest.mark.parametrize("dt", ["i32", "u8", "i64", "f64"])
+def test_reduce_wide_large_strided_input_is_the_reduction_of_its_logical_copy(oracle, hip, dt):
+    """As for f32: from 2^18 elements a strided input is reduced through its logical-order copy.  Integer sums wrap, so
+    any order gives the reference's bits; f64 sums agree to rounding; max / min bit for bit."""
+    r = rng(191)
+    for dims, perm in (([520, 640], [1, 0]), ([6, 300, 200], [0, 2, 1])):
+        lay = LY.permuted(dims, perm)
+        n = int(np.prod(dims))
+        st = r.standard_normal(lay["size"]) if dt == "f64" else r.integers(0 if dt == "u8" else -100, 100, lay["size"]).astype(NP[dt])
+        for dim in range(len(dims)):
+            md = meta_reduce(lay["dims"], lay["strides"], dim, 0)
+            out_n = n // lay["dims"][dim]
+            for op in ("sum", "max", "min"):
+                (o,), (h,) = both(oracle, hip, f"{op}_{dt}", lambda: (n, len(dims), 1, md, In(st), Out(out_n, dt)))
+                if dt == "f64" and op == "sum":
+                    assert np.allclose(o, h, rtol=1e-12, atol=1e-11), (op, dim)
+                else:
+                    assert same_bits(o, h), (op, dim)
 
 
 def test_reduce_wide_strided_input_and_nan_rule(oracle, hip):
