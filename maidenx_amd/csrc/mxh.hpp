@@ -47,6 +47,8 @@ struct ApiGuard {
 // Device scratch owned by the library (two independent slots per device), grown on demand and
 // reused by every call; safe because all work of the backend is ordered on one stream.
 void* scratch(size_t bytes, int slot = 0);
+// runtime.hip: a graph capture is being recorded (nothing may be allocated or grown)
+bool capture_open();
 // The 65536-entry tables of exp for bf16 / f16 on the current device (lut16.hpp; defined next to the unary entry points);
 // null while they cannot be built (a graph capture is open and the table does not exist yet).
 const uint16_t* lut16_exp_bf16();

@@ -7,7 +7,9 @@
 // the reference's own order, strided inputs with its index rule (leading dims decomposed from dim 0 upwards).
 #include <cmath>
 
+#include "elementwise.hpp"
 #include "mxh.hpp"
+#include "ops.hpp"
 
 namespace mxh {
 
@@ -172,6 +174,25 @@ static void softmax_f64(size_t num_els, size_t nd, size_t dim_arg, const size_t*
         hipLaunchKernelGGL(softmax_col_f64_kernel, dim3((unsigned)(pre * jblocks)), dim3(64 * SCW), 0, stream(), src, out, D, post, jblocks);
         MXH_LAUNCH_CHECK("softmax_col_f64");
         return;
+    }
+    // a large strided input with at most one leading dim of more than one element: the contiguous softmax of its
+    // logical-order copy (as for f32, softmax.hip)
+    if (!cont) {
+        size_t leading = 0;
+        for (size_t d = 0; d < dim; ++d) leading += dims[d] > 1;
+        if (leading <= 1 && num_els >= (1u << 18) && num_els < (1ull << 31) && nd <= 64 && !capture_open()) {
+            double* tmp = (double*)scratch(num_els * sizeof(double), 1);
+            if (!tmp) return;
+            size_t cmd[2 * 64 + 1];
+            for (size_t d = 0; d < nd; ++d) cmd[d] = dims[d];
+            contiguous_strides(nd, dims, cmd + nd);
+            cmd[2 * nd] = 0;
+            const size_t* ins[1] = {strides};
+            const void* inp[1] = {src};
+            ew_launch<OpIdentity<double>>(num_els, nd, dims, cmd + nd, ins, tmp, inp, OpIdentity<double>{});
+            softmax_f64(num_els, nd, dim, cmd, tmp, out);
+            return;
+        }
     }
     if (!cont && nd > (size_t)MAXD) { set_status(ERR_UNSUPPORTED, "softmax: strided input of rank above 8"); return; }
     SoftmaxStridedF64 sp;
