@@ -495,6 +495,32 @@ def test_sum_to_shape_strided_input(oracle, hip):
         assert np.allclose(o, h, rtol=1e-5, atol=1e-5), out_shape
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_sum_to_shape_of_permuted_views_with_a_reduction(oracle, hip, dt):
+    """Permuted views (every index below num_els, so the reference's modulo never applies) are copied into logical order
+    by the elementwise identity and reduced; a view whose indices pass num_els keeps the gather with the modulo."""
+    r = rng(199)
+    cases = [(LY.permuted([72, 200], [1, 0]), [[1, 200], [72, 1], [1, 1]]), (LY.permuted([6, 40, 56], [2, 0, 1]), [[1, 40, 1], [6, 1, 56], [1, 1, 56]]),
+             (dict(dims=[30, 40], strides=[1, 32], off=0, size=30 * 40 + 64), [[1, 40], [30, 1]])]
+    for lay, outs in cases:
+        n = int(np.prod(lay["dims"]))
+        st = to_storage(r.uniform(-1, 1, max(lay["size"], n)).astype(np.float32), dt)
+        for out_shape in outs:
+            md = meta_sum_to_shape(lay["dims"], lay["strides"], out_shape, 0)
+            n_out = int(np.prod(out_shape))
+            (o,), (h,) = both(oracle, hip, f"sum_to_shape_{dt}", lambda: (n, len(lay["dims"]), md, In(st), Out(n_out, dt)))
+            a, b = to_float(o, dt).astype(np.float64), to_float(h, dt).astype(np.float64)
+            if dt == "f32":
+                assert np.allclose(a, b, rtol=1e-5, atol=1e-5), (lay["dims"], out_shape)
+            elif lay["size"] <= n:
+                # bf16: the reference's running sum in bf16 drifts by several units; the kernel's f32 sum rounded once is
+                # held to the exact sum of the same elements
+                logical = to_float(LY.gather(st, lay), dt).astype(np.float64)
+                axes = tuple(d for d, (i, k) in enumerate(zip(lay["dims"], out_shape)) if k == 1 and i != 1)
+                exact = logical.sum(axis=axes).ravel()
+                assert np.all(np.abs(b - exact) <= 2.0 ** -8 * np.abs(exact) + 1e-3), (lay["dims"], out_shape)
+
+
 @pytest.mark.parametrize("dt", DTS)
 def test_sum_to_shape_identity_on_strided_views(oracle, hip, dt):
     """out = 0 + view for views that stay below num_els (one elementwise pass over the view's strides) and for one whose
