@@ -41,11 +41,11 @@ struct GraphExec {                        // what hip_graph_end_capture hands ou
 };
 // A capture that called scratch() has the block's address baked into its graph or program: while such a capture is
 // alive the block must not be freed, so a later growth retires it instead (freed with the last live capture).
-static bool g_scratch_captured[16][2] = {{false}};
+static bool g_scratch_captured[16][3] = {{false}};
 static int g_live_captures = 0;
 static std::vector<void*> g_retired_scratch;
-static void* g_scratch[16][2] = {{nullptr}};
-static size_t g_scratch_bytes[16][2] = {{0}};
+static void* g_scratch[16][3] = {{nullptr}};
+static size_t g_scratch_bytes[16][3] = {{0}};
 
 void set_status(int code, const char* what, int hip_err) {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -338,7 +338,7 @@ void prog_launch_seen() {
 
 void* scratch(size_t bytes, int slot) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16 || slot < 0 || slot > 1) {
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16 || slot < 0 || slot > 2) {
         set_status(ERR_INVALID, "scratch: bad device or slot");
         return nullptr;
     }
@@ -612,7 +612,7 @@ int hip_graph_destroy(void* graph_exec) {
             g_live_captures = 0;
             for (void* p : g_retired_scratch) (void)hipFree(p);
             g_retired_scratch.clear();
-            for (auto& dev : g_scratch_captured) dev[0] = dev[1] = false;
+            for (auto& dev : g_scratch_captured) dev[0] = dev[1] = dev[2] = false;
         }
     }
     return (int)e;

@@ -365,7 +365,10 @@ RED_CASES = [([64, 96], 0), ([64, 96], 1), ([257, 130], 0), ([257, 130], 1), ([8
              ([5000], 0), ([3, 70000], 1), ([70000, 3], 0), ([1, 40000], 0), ([10000, 1], 1), ([2, 3, 5, 7], 2), ([40000], 0),
              ([300, 2048], 1), ([4, 300000], 1),
              # at least 65536 rows of a few dozen elements: 16 lanes per row (rows of 56, 40, 256 and 64 elements)
-             ([1200, 56, 56], 2), ([70000, 40], 1), ([66000, 256], 1), ([65536, 64], 1)]
+             ([1200, 56, 56], 2), ([70000, 40], 1), ([66000, 256], 1), ([65536, 64], 1),
+             # narrow rows under a long axis: 256 rows at a time as one wide row, the partial rows folded by a second call
+             # (left-over rows, an outer dim whose slices must stay whole, an axis too ragged to regroup)
+             ([300000, 5], 0), ([40001, 7], 0), ([2, 16384, 3], 1), ([3, 8200, 6], 1), ([1, 9000, 33], 1), ([5, 8192, 1], 1)]
 
 
 @pytest.mark.parametrize("dt", DTS)
