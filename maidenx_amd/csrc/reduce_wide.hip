@@ -256,6 +256,21 @@ static void wreduce(const T* in, T* out, size_t outer, size_t L, size_t S, doubl
         wrow_stage<T, R>(part, out, outer, chunks, 1, chunks, div);
         return;
     }
+    // narrow rows under a long axis: G rows at a time as one wide row, the G partial rows (and the one of the left-over
+    // rows, when there is one slice) folded by a second call - see col_reduce in reduce.hip
+    if (S < 64 && L >= 8192 && !capture_open()) {
+        size_t G = 256;
+        if (outer > 1) while (G > 1 && L % G != 0) G /= 2;
+        const size_t L0 = L / G * G, rem = L - L0;
+        if (G >= 16 && G * S >= 256) {
+            T* P = (T*)scratch(outer * (G + 1) * S * sizeof(T) + 256, 2);
+            if (!P) return;
+            wreduce<T, R>(in, P, outer, L0 / G, G * S, 0.0);
+            if (rem) wreduce<T, R>(in + L0 * S, P + G * S, 1, rem, S, 0.0);
+            wreduce<T, R>(P, out, outer, G + (rem ? 1 : 0), S, div);
+            return;
+        }
+    }
     {
         // wide rows and a long axis: one 16-wave block per CU covers the memory latency, so few chunks (often none)
         constexpr size_t V = 16 / sizeof(T);
