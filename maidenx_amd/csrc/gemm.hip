@@ -868,6 +868,85 @@ __global__ __launch_bounds__(256) void gemm_rowsdot_kernel(GemmArgs g) {
     gemm_rowsdot_any<256>(g, threadIdx.x, part);
 }
 
+// A few output rows against a row-major Y ([1..8, R] x [R, J]: a batch of one to eight through a weight matrix).  The
+// product is Y read once, so the kernel is a stream over Y's rows: a lane owns one 16-byte vector of columns, a wave 64
+// of them (1 KB of every row) over its own run of r_chunk rows, eight rows in flight; X's elements are the same for the
+// whole wave.  Every wave writes its f32 partial rows to part[chunk][I * J], and gemm_fold_kernel adds the chunks in order.
+// (One wave per output, lanes striding down a column of Y, reads 4 bytes of every cache line it touches: [1,4096] x
+// [4096,4096] in f32 took 100 us, 8 % of what the 64 MB of Y allow.)
+template <class T, int MI>
+__global__ __launch_bounds__(256) void gemm_fewrows_kernel(GemmArgs g) {
+    constexpr int VEC = 16 / sizeof(T), U = 8;
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t j = (blockIdx.x * WAVE + lane) * VEC;
+    const uint32_t chunk = blockIdx.y * (256 / WAVE) + w;
+    if (chunk >= g.splits) return;
+    const bool live = j < g.J;
+    const uint32_t r0 = chunk * g.r_chunk, r1 = r0 + g.r_chunk < g.R ? r0 + g.r_chunk : g.R;
+    float acc[MI][VEC];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[i][e] = 0.0f;
+    const T* y = (const T*)g.Y + (live ? j : 0);
+    const T* x = (const T*)g.X;
+    auto rows = [&](uint32_t r, auto count) {
+        constexpr int N = decltype(count)::value;
+        AVec<T, VEC> v[N];
+#pragma unroll
+        for (int u = 0; u < N; ++u) v[u] = *(const AVec<T, VEC>*)(y + (int64_t)(r + u) * g.yr);
+#pragma unroll
+        for (int u = 0; u < N; ++u)
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const float a = (uint32_t)i < g.I ? Elem<T>::ld(x[(int64_t)i * g.xi + (int64_t)(r + u) * g.xr]) : 0.0f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[i][e] += a * Elem<T>::ld(v[u].v[e]);
+            }
+    };
+    uint32_t r = r0;
+    for (; r + U <= r1; r += U) rows(r, std::integral_constant<int, U>{});
+    for (; r < r1; ++r) rows(r, std::integral_constant<int, 1>{});
+    if (!live) return;
+    float* dst = g.part + (size_t)chunk * g.I * g.J + j;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+        if ((uint32_t)i < g.I) {
+            AVec<float, VEC> o;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o.v[e] = acc[i][e];
+            *(AVec<float, VEC>*)(dst + (size_t)i * g.J) = o;
+        }
+}
+
+// false: the shape is not this kernel's
+template <class T>
+bool launch_fewrows(GemmArgs g) {
+    constexpr int VEC = 16 / sizeof(T);
+    if (g.batch != 1 || g.I > 8 || g.yj != 1 || g.J < 256 || g.R < 256 || g.J % VEC != 0 || g.yr % VEC != 0 || g.yr < 0 ||
+        (uintptr_t)g.Y % 16 != 0 || capture_open() || prog_recording())
+        return false;
+    const uint32_t colgroups = (uint32_t)cdiv((size_t)g.J / VEC, (size_t)WAVE);
+    // about four waves per CU, at least 32 rows each
+    uint32_t chunks = (uint32_t)std::min<size_t>(std::max<size_t>(cdiv((size_t)1024, (size_t)colgroups), 1), g.R / 32);
+    g.r_chunk = (uint32_t)cdiv((size_t)g.R, (size_t)chunks);
+    chunks = (uint32_t)cdiv((size_t)g.R, (size_t)g.r_chunk);
+    g.splits = chunks;
+    const size_t n_out = (size_t)g.I * g.J;
+    g.part = (float*)scratch(chunks * n_out * sizeof(float) + 256);
+    if (!g.part) return true;          // status is set
+    const dim3 grid(colgroups, (unsigned)cdiv((size_t)chunks, (size_t)(256 / WAVE)));
+    if (g.I == 1) hipLaunchKernelGGL((gemm_fewrows_kernel<T, 1>), grid, dim3(256), 0, stream(), g);
+    else if (g.I == 2) hipLaunchKernelGGL((gemm_fewrows_kernel<T, 2>), grid, dim3(256), 0, stream(), g);
+    else if (g.I <= 4) hipLaunchKernelGGL((gemm_fewrows_kernel<T, 4>), grid, dim3(256), 0, stream(), g);
+    else hipLaunchKernelGGL((gemm_fewrows_kernel<T, 8>), grid, dim3(256), 0, stream(), g);
+    MXH_LAUNCH_CHECK("gemm_fewrows");
+    hipLaunchKernelGGL(gemm_fold_kernel<T>, dim3((unsigned)cdiv(n_out, (size_t)256)), dim3(256), 0, stream(), g.part, (T*)g.out, n_out, chunks);
+    MXH_LAUNCH_CHECK("gemm_fold");
+    return true;
+}
+
 template <class T>
 void gemm_dispatch(GemmArgs g) {
     if (g.I == 0 || g.J == 0 || g.batch == 0) return;
@@ -903,6 +982,7 @@ void gemm_dispatch(GemmArgs g) {
         MXH_LAUNCH_CHECK("gemm_blockdot");
         return;
     }
+    if (launch_fewrows<T>(g)) return;
     if (outputs <= 4096 && (g.I < 32 || g.J < 32)) {
         hipLaunchKernelGGL(gemm_wavedot_kernel<T>, dim3(cdiv(outputs, GB / WAVE)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_wavedot");

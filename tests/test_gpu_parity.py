@@ -632,6 +632,35 @@ def test_matmul_short_reduction_row_panels(hip, shape, a_perm, b_perm, dt):
     assert np.isfinite(got).all()
 
 
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("a_perm", [False, True])
+@pytest.mark.parametrize("shape", [(1, 1, 300, 256), (1, 2, 4096, 264), (1, 3, 1000, 520), (1, 5, 257, 1024), (1, 8, 2050, 512), (1, 1, 4099, 4096)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_matmul_few_rows_against_a_row_major_matrix(oracle, hip, shape, a_perm, dt):
+    """One to eight output rows: the kernel that streams the right operand's rows (a lane per 16-byte vector of columns,
+    a wave per run of rows, partial rows folded in chunk order) - ragged reductions, column counts that leave lanes of
+    the last wave idle, a left operand given transposed, and the right operand as a column slice of a wider matrix."""
+    batch, m, k, n = shape
+    r = rng(67)
+    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, a_perm, False, dt)
+    (h,) = hip.call(f"matmul_{dt}", m * n, md, In(sa), In(sb), Out(m * n, dt))
+    truth = np.einsum("bmk,bkn->bmn", av, bv)
+    scale = np.einsum("bmk,bkn->bmn", np.abs(av), np.abs(bv))
+    tol = 1e-5 if dt == "f32" else 1e-2
+    err = np.abs(to_float(h, dt).reshape(truth.shape) - truth) / np.maximum(scale, 1e-30)
+    assert np.max(err) <= tol, float(np.max(err))
+    if dt == "f32" and m * n * k <= 5_000_000:
+        (o,) = oracle.call("matmul_f32", m * n, md, In(sa), In(sb), Out(m * n, "f32"))
+        assert np.max(np.abs(o - h).reshape(truth.shape) / np.maximum(scale, 1e-30)) <= 2e-5
+    # the right operand as the first n columns of a matrix twice as wide (row stride 2n)
+    wide = np.zeros((k, 2 * n), np.float32)
+    wide[:, :n] = bv[0]
+    wide[:, n:] = 7.0
+    mdw = meta_matmul([m, n], [m, k], [k, n], [1, m] if a_perm else [k, 1], [2 * n, 1])
+    (hw,) = hip.call(f"matmul_{dt}", m * n, mdw, In(sa), In(to_storage(wide.ravel(), dt)), Out(m * n, dt))
+    assert same_bits(h, hw)
+
+
 def test_matmul_strided_rows_is_the_full_product(oracle, hip):
     """A = big[:, :k], a view whose rows are 3k apart.  The CPU reference drops every term whose operand index reaches
     num_els * k (crates/maidenx_cpu/src/ops/matmul.rs:53-54,109), which cuts the later rows short; the GPU computes the
