@@ -633,16 +633,18 @@ def test_matmul_short_reduction_row_panels(hip, shape, a_perm, b_perm, dt):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("a_perm", [False, True])
-@pytest.mark.parametrize("shape", [(1, 1, 300, 256), (1, 2, 4096, 264), (1, 3, 1000, 520), (1, 5, 257, 1024), (1, 8, 2050, 512), (1, 1, 4099, 4096)],
+@pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True)])
+@pytest.mark.parametrize("shape", [(1, 1, 300, 256), (1, 2, 4096, 264), (1, 3, 1000, 520), (1, 5, 257, 1024), (1, 8, 2050, 512), (1, 1, 4099, 4096),
+                                   (1, 8, 2048, 515), (1, 5, 512, 1000), (1, 4, 8200, 70)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_matmul_few_rows_against_a_row_major_matrix(oracle, hip, shape, a_perm, dt):
-    """One to eight output rows: the kernel that streams the right operand's rows (a lane per 16-byte vector of columns,
-    a wave per run of rows, partial rows folded in chunk order) - ragged reductions, column counts that leave lanes of
-    the last wave idle, a left operand given transposed, and the right operand as a column slice of a wider matrix."""
+def test_matmul_few_rows(oracle, hip, shape, a_perm, b_perm, dt):
+    """One to eight output rows.  Against a row-major right operand: the kernel that streams its rows (a lane per 16-byte
+    vector of columns, a wave per run of rows, partial rows folded in chunk order) - ragged reductions, column counts
+    that leave lanes of the last wave idle, a left operand given transposed, the right operand as a column slice of a
+    wider matrix.  Against a right operand given transposed (a linear layer's x W^T): a wave per output column."""
     batch, m, k, n = shape
     r = rng(67)
-    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, a_perm, False, dt)
+    sa, sb, md, av, bv = matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt)
     (h,) = hip.call(f"matmul_{dt}", m * n, md, In(sa), In(sb), Out(m * n, dt))
     truth = np.einsum("bmk,bkn->bmn", av, bv)
     scale = np.einsum("bmk,bkn->bmn", np.abs(av), np.abs(bv))
@@ -652,6 +654,8 @@ def test_matmul_few_rows_against_a_row_major_matrix(oracle, hip, shape, a_perm, 
     if dt == "f32" and m * n * k <= 5_000_000:
         (o,) = oracle.call("matmul_f32", m * n, md, In(sa), In(sb), Out(m * n, "f32"))
         assert np.max(np.abs(o - h).reshape(truth.shape) / np.maximum(scale, 1e-30)) <= 2e-5
+    if b_perm:
+        return
     # the right operand as the first n columns of a matrix twice as wide (row stride 2n)
     wide = np.zeros((k, 2 * n), np.float32)
     wide[:, :n] = bv[0]
