@@ -1063,7 +1063,9 @@ void gemm_dispatch(GemmArgs g) {
     // (four blocks per CU), 86 / 116 / 144 us with 128x64, 196 / 124 / 196 us with 128x128, 340 / 137 / 339 us with
     // 256x256.
     constexpr uint32_t TKE = TK_BYTES / sizeof(T);
-    bool tall = g.I >= 128 && (g.J <= 64 || g.R <= 4 * TKE);
+    // At most 64 output rows (a small batch through a weight matrix): a 128-row tile would compute mostly rows that do
+    // not exist - [16,4096] x [4096,4096] in f32 took 49 us, the time of 128 rows.
+    bool tall = (g.I >= 128 && (g.J <= 64 || g.R <= 4 * TKE)) || g.I <= 64;
     bool big = !tall && g.I >= 256 && g.J >= 256 && big_blocks >= 192;
 #define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, typename Cfgs<T>::Big>(g) : tall ? launch_mfma<T, XR, YR, typename Cfgs<T>::Tall>(g) : launch_mfma<T, XR, YR, typename Cfgs<T>::Small>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
@@ -1120,7 +1122,7 @@ static void cols_matmul(const size_t* md, int transposed, const float* in, const
     else { g.I = (uint32_t)K; g.R = (uint32_t)M; g.xi = 1; g.xr = (int64_t)K; }
     // the choices gemm_dispatch makes for a stored matrix of this shape, so that both ways are the same arithmetic
     constexpr uint32_t TK = TK_BYTES / sizeof(float);
-    const bool tall = g.I >= 128 && (g.J <= 64 || g.R <= 4 * TK);
+    const bool tall = (g.I >= 128 && (g.J <= 64 || g.R <= 4 * TK)) || g.I <= 64;
     const bool yr = g.yr == 1;
     auto fast_of = [&](int rows_y) {
         const bool span = g.yj >= 0 && g.yr >= 0 && ((int64_t)rows_y * g.yj + (int64_t)TK * g.yr) * 4 < (1ll << 31);
