@@ -100,20 +100,30 @@ struct Stager {
 
     // Buffer descriptor of one tile: the (uniform) tile origin is the base, so every lane addresses with
     // one loop-invariant 32-bit offset plus a scalar offset per load instead of a 64-bit pointer each.
-    static __device__ __amdgpu_buffer_rsrc_t tile_rsrc(const T* base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0) {
+    static __device__ __amdgpu_buffer_rsrc_t tile_rsrc(const T* base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0,
+                                                       int records = 0x7fffffff) {
         const T* origin = base + (int64_t)row0 * s_row + (int64_t)red0 * s_red;
-        return __builtin_amdgcn_make_buffer_rsrc((void*)origin, 0, 0x7fffffff, 0x00020000);
+        return __builtin_amdgcn_make_buffer_rsrc((void*)origin, 0, records, 0x00020000);
     }
     // FAST: the tile lies fully inside the operand, wide accesses are aligned and offsets inside a tile
     // fit 31 bits (no checks at all)
     // A "unit" is what one pass of all threads loads: NU of them make the tile.  load()/store() take a
     // unit range so that a tile's traffic can be spread over the k-steps of the previous tile.
     static constexpr int NU = PAIRS ? NV / 2 : NV;
-    template <bool FAST>
+    // BOUND (with FAST, RCONT): the tile's last rows may lie past the operand's nrows rows while its reduction range is
+    // whole.  The descriptor then ends with row nrows - 1, and the hardware returns zeros for every load past it (rows
+    // are contiguous and at least a reduction range long, so "past the last row" is "past that byte").
+    template <bool FAST, bool BOUND = false>
     __device__ void load(const T* __restrict__ base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0,
                          uint32_t nrows, uint32_t nred, int u0 = 0, int u1 = NU) {
         constexpr bool fast = FAST;
+        static_assert(!BOUND || (FAST && RCONT), "bounded loads: the unchecked form of a row-contiguous operand");
         const int t = threadIdx.x;
+        int records = 0x7fffffff;
+        if constexpr (BOUND) {
+            const int64_t left = ((int64_t)(nrows - row0) * s_row - (int64_t)red0) * (int64_t)sizeof(T);
+            records = nrows > row0 ? (int)(left < 0x7fffffff ? left : 0x7fffffff) : 0;
+        }
         if constexpr (RCONT) {
             constexpr int KV = TK / VEC;   // vectors per row
 #pragma unroll
@@ -125,7 +135,9 @@ struct Stager {
                 if constexpr (fast) {
                     uint32_t voff = (uint32_t)(((t / KV) * s_row + (t % KV) * VEC) * (int64_t)sizeof(T));
                     uint32_t soff = (uint32_t)((int64_t)u * (NT / KV) * s_row * (int64_t)sizeof(T));
-                    reg[u] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base, s_row, s_red, row0, red0), voff, soff, 0);
+                    // (bounded: the whole offset in the vector operand, which is what the range check is sure to see)
+                    if constexpr (BOUND) reg[u] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base, s_row, s_red, row0, red0, records), voff + soff, 0, 0);
+                    else reg[u] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base, s_row, s_red, row0, red0), voff, soff, 0);
                 } else {
                     Pack16<T> pk;
 #pragma unroll
@@ -370,12 +382,14 @@ template <class T> struct Cfgs {
     using Big = GemmCfg<4, 2, 2, 4>;
     using Small = GemmCfg<2, 2, 2, 2>;
     using Tall = GemmCfg<2, 2, 1, 1>;     // 64 x 64, four blocks per CU: few output columns or a short reduction (see gemm_dispatch)
+    using Flat = GemmCfg<1, 4, 1, 1>;     // 32 x 128: at most 32 output rows
 };
 #if MXH_GEMM_TS16
 template <> struct Cfgs<bf16_t> {
     using Big = GemmCfg<4, 2, 4, 8, 16>;
     using Small = GemmCfg<2, 2, 4, 4, 16>;
     using Tall = GemmCfg<2, 2, 2, 2, 16>;     // 64 x 64 (the conv-shaped bf16 weight gradient: 49 us, 205 us with 256 x 64 tiles)
+    using Flat = Tall;                        // (a 32-row tile is too small for the turned 16-bit stager's row pairs)
 };
 template <> struct Cfgs<f16_t> : Cfgs<bf16_t> {};
 #endif
@@ -383,7 +397,7 @@ template <> struct Cfgs<f16_t> : Cfgs<bf16_t> {};
 // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
 // column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
 // (16x16 tiles: one group of 4: column j0 + .. + 4*(lane/16) + e, row lane%16)
-template <class O, class Cfg, bool FAST>
+template <class O, class Cfg, bool FAST, bool ROWS = false>      // ROWS: FAST, but rows from g.I on do not exist
 __device__ __forceinline__ void store_tile(O* out, const typename Cfg::Acc (&acc)[Cfg::MI][Cfg::MJ], const GemmArgs& g, uint32_t i0, uint32_t j0,
                                            int wm, int wn, int lane) {
     constexpr int MI = Cfg::MI, MJ = Cfg::MJ, TS = Cfg::TS;
@@ -398,6 +412,7 @@ __device__ __forceinline__ void store_tile(O* out, const typename Cfg::Acc (&acc
             for (int q = 0; q < (TS == 32 ? 4 : 1); ++q) {
                 uint32_t col = j0 + wn * TS * MJ + c * TS + (TS == 32 ? 8 * q + 4 * (lane / 32) : 4 * (lane / 16));
                 if (!FAST && (row >= g.I || col >= g.J)) continue;
+                if (ROWS && row >= g.I) continue;
                 O* dst = out + (int64_t)row * g.J + col;
                 if (vec_store && (FAST || col + 4 <= g.J)) {
                     GVec<O, 4> v;
@@ -466,8 +481,11 @@ __device__ __forceinline__ TilePos tile_of_block(const GemmArgs& g) {
 // blocks a CU holds do not cover it.  The launch has as many blocks as the chip holds at once, with equal shares.
 // XCOLS (f32): X is the column matrix of a convolution (XR) or its transpose (!XR), gathered from the input (ColsView);
 // 2: four at a time (see cols_gather4), 1: one by one.
-template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false, int XCOLS = 0>
+// RB: FAST for a tile whose last rows lie past g.I (X row-contiguous, every other extent whole): X is loaded through a
+// descriptor that ends with its last row, and the rows that do not exist are not stored.
+template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false, int XCOLS = 0, bool RB = false>
 __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem, const ColsView* cv = nullptr) {
+    static_assert(!RB || (FAST && XR && !PANEL && XCOLS == 0), "bounded rows: the unchecked body, X row-contiguous and stored");
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
     constexpr bool SWZ = Cfg::TS == 16;
     static_assert(!XCOLS || (std::is_same<T, float>::value && !PANEL), "the gathered operand is f32, one tile per block");
@@ -519,7 +537,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
     // units [u0, u1) of the X tile at (row, red) into the registers of stager st
     auto load_x = [&](SX& st, uint32_t row, uint32_t red, int u0, int u1) {
         if constexpr (XCOLS) st.template load_cols<FAST>(*cv, row, red, g.I, re, u0, u1);
-        else st.template load<FAST>(X, g.xi, g.xr, row, red, g.I, re, u0, u1);
+        else st.template load<FAST, RB>(X, g.xi, g.xr, row, red, g.I, re, u0, u1);
     };
     {
         // tiles 0 and 1 are requested together (one memory latency instead of two); the accumulators are
@@ -632,7 +650,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
         }
         if constexpr (PANEL) {
             if ((kt + 1) % nk1 == 0) {       // the last k-tile of an output tile: out it goes, and the accumulators start over
-                store_tile<T, Cfg, FAST>((T*)g.out, acc, g, row_of(kt), col_of(kt), wm, wn, lane);
+                store_tile<T, Cfg, FAST, RB>((T*)g.out, acc, g, row_of(kt), col_of(kt), wm, wn, lane);
 #pragma unroll
                 for (int a = 0; a < MI; ++a)
 #pragma unroll
@@ -646,9 +664,9 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
 
     if (g.splits > 1) {
         float* part = g.part + ((int64_t)split * g.batch + b) * g.I * g.J;
-        store_tile<float, Cfg, FAST>(part, acc, g, i0, j0, wm, wn, lane);
+        store_tile<float, Cfg, FAST, RB>(part, acc, g, i0, j0, wm, wn, lane);
     } else {
-        store_tile<T, Cfg, FAST>((T*)g.out + (int64_t)b * g.I * g.J, acc, g, i0, j0, wm, wn, lane);
+        store_tile<T, Cfg, FAST, RB>((T*)g.out + (int64_t)b * g.I * g.J, acc, g, i0, j0, wm, wn, lane);
     }
 }
 
@@ -677,6 +695,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         if ((pos.ti + 1) * Cfg::TM <= g.I && (pos.tj + 1) * Cfg::TN <= g.J) {
             gemm_mfma_body<T, XR, YR, Cfg, true>(g, pos, smem);
             return;
+        }
+        // the configurations of few output rows: a tile whose columns are whole and whose rows run past g.I
+        if constexpr (XR && Cfg::TM <= 64) {
+            if ((pos.tj + 1) * Cfg::TN <= g.J) {
+                gemm_mfma_body<T, XR, YR, Cfg, true, false, 0, true>(g, pos, smem);
+                return;
+            }
         }
     }
     gemm_mfma_body<T, XR, YR, Cfg, false>(g, pos, smem);
@@ -924,7 +949,9 @@ __global__ __launch_bounds__(256) void gemm_fewrows_kernel(GemmArgs g) {
 template <class T>
 bool launch_fewrows(GemmArgs g) {
     constexpr int VEC = 16 / sizeof(T);
-    if (g.batch != 1 || g.I > 8 || g.yj != 1 || g.J < 256 || g.R < 256 || g.J % VEC != 0 || g.yr % VEC != 0 || g.yr < 0 ||
+    // (f32, one or two rows: from three rows, and for the 16-bit dtypes from the first, the MFMA tiles with bounded
+    // rows are faster - bf16 one row 21 us here, 14 us there)
+    if (sizeof(T) != 4 || g.batch != 1 || g.I > 2 || g.yj != 1 || g.J < 256 || g.R < 256 || g.J % VEC != 0 || g.yr % VEC != 0 || g.yr < 0 ||
         (uintptr_t)g.Y % 16 != 0 || capture_open() || prog_recording())
         return false;
     const uint32_t colgroups = (uint32_t)cdiv((size_t)g.J / VEC, (size_t)WAVE);
@@ -999,7 +1026,8 @@ __global__ __launch_bounds__(256) void gemm_fewrows_t_kernel(GemmArgs g) {
 template <class T>
 bool launch_fewrows_t(const GemmArgs& g) {
     constexpr int VEC = 16 / sizeof(T);
-    if (g.batch != 1 || g.I < 2 || g.I > 8 || g.yr != 1 || g.xr != 1 || g.R < 512 || g.R % VEC != 0 || g.yj % VEC != 0 || g.xi % VEC != 0 ||
+    // (two rows: from three the MFMA tiles with bounded rows are faster - f32 four rows 24 us here, 21 us there)
+    if (g.batch != 1 || g.I != 2 || g.yr != 1 || g.xr != 1 || g.R < 512 || g.R % VEC != 0 || g.yj % VEC != 0 || g.xi % VEC != 0 ||
         g.yj < 0 || g.xi < 0 || (uintptr_t)g.Y % 16 != 0 || (uintptr_t)g.X % 16 != 0 || prog_recording())
         return false;
     // one column a wave: with two or four (X loaded once for several rows of W) the fewer waves cost more than the
@@ -1048,7 +1076,8 @@ void gemm_dispatch(GemmArgs g) {
         return;
     }
     if (launch_fewrows<T>(g) || launch_fewrows_t<T>(g)) return;
-    if (outputs <= 4096 && (g.I < 32 || g.J < 32)) {
+    // (a few rows against a large row-major Y are not for the kernel below, whose lanes would stride down Y's columns)
+    if (outputs <= 4096 && (g.I < 32 || g.J < 32) && !(g.yj == 1 && g.J >= 256 && g.R >= 256)) {
         hipLaunchKernelGGL(gemm_wavedot_kernel<T>, dim3(cdiv(outputs, GB / WAVE)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_wavedot");
         return;
@@ -1067,7 +1096,8 @@ void gemm_dispatch(GemmArgs g) {
     // not exist - [16,4096] x [4096,4096] in f32 took 49 us, the time of 128 rows.
     bool tall = (g.I >= 128 && (g.J <= 64 || g.R <= 4 * TKE)) || g.I <= 64;
     bool big = !tall && g.I >= 256 && g.J >= 256 && big_blocks >= 192;
-#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, typename Cfgs<T>::Big>(g) : tall ? launch_mfma<T, XR, YR, typename Cfgs<T>::Tall>(g) : launch_mfma<T, XR, YR, typename Cfgs<T>::Small>(g))
+    const bool flat = g.I <= 32 && g.J >= 128;
+#define MXH_GEMM_CASE(XR, YR) (big ? launch_mfma<T, XR, YR, typename Cfgs<T>::Big>(g) : flat ? launch_mfma<T, XR, YR, typename Cfgs<T>::Flat>(g) : tall ? launch_mfma<T, XR, YR, typename Cfgs<T>::Tall>(g) : launch_mfma<T, XR, YR, typename Cfgs<T>::Small>(g))
     if (xr && yr) MXH_GEMM_CASE(true, true);
     else if (xr && yj) MXH_GEMM_CASE(true, false);
     else if (xi && yr) MXH_GEMM_CASE(false, true);
