@@ -1044,12 +1044,20 @@ template <class T>
 void gemm_dispatch(GemmArgs g) {
     if (g.I == 0 || g.J == 0 || g.batch == 0) return;
     size_t outputs = (size_t)g.I * g.J * g.batch;
-    if (g.R <= 16 || (g.I < 16 && g.J < 16 && g.R < 256)) {
+    // (16-bit dtypes: a reduction shorter than a k-tile would be a ragged tile for the MFMA kernel, i.e. its checked body)
+    const bool short_r16 = sizeof(T) == 2 && g.R < 64 && !prog_recording() && gemm_thread_vec_ok<T>(g);
+    if (g.R <= 16 || short_r16 || (g.I < 16 && g.J < 16 && g.R < 256)) {
         if constexpr (std::is_same<T, float>::value) {
             const bool small = cdiv(outputs, GB) <= PROG_MAX_GRID && (size_t)g.R * outputs <= PROG_MAX_ELEMS;
             if (prog_recording() && !small) prog_abandon();
             if (fuse_thread_dot(g, outputs)) return;
             if (prog_recording()) prog_record(prog_kid(PF_GEMM_THREAD, 0), (unsigned)cdiv(outputs, GB), &g, sizeof(g));
+        }
+        if (!prog_recording() && gemm_thread_vec_ok<T>(g)) {
+            constexpr int VEC = 16 / sizeof(T);
+            hipLaunchKernelGGL(gemm_thread_vec_kernel<T>, dim3((unsigned)cdiv((size_t)g.I * (g.J / VEC), (size_t)GB), g.batch), dim3(GB), 0, stream(), g);
+            MXH_LAUNCH_CHECK("gemm_thread_vec");
+            return;
         }
         hipLaunchKernelGGL(gemm_thread_kernel<T>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_thread");

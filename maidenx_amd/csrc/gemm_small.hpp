@@ -62,6 +62,41 @@ __device__ __forceinline__ void gemm_thread_body(const GemmArgs& g, unsigned bid
 template <class T>
 __global__ __launch_bounds__(GB) void gemm_thread_kernel(GemmArgs g) { gemm_thread_body<T>(g, blockIdx.x, threadIdx.x); }
 
+// The same sums for Y with unit column stride and J a multiple of the 16-byte vector: a thread owns VEC neighbouring
+// outputs of one row (one vector load of Y per term, one vector store), blockIdx.y is the batch, and nothing is divided
+// in 64 bits - with a short reduction the kernel above spends its time on its index arithmetic ([4096,8] x [8,4096]:
+// 90 us for 64 MB of output).  Every output is still its terms in ascending r, multiply and add unfused.
+template <class T>
+__global__ __launch_bounds__(GB) void gemm_thread_vec_kernel(GemmArgs g) {
+    constexpr int VEC = 16 / sizeof(T);
+    const uint32_t jv = g.J / VEC;                        // vectors per output row
+    const uint32_t v = blockIdx.x * GB + threadIdx.x;
+    if (v >= g.I * jv) return;
+    const uint32_t i = v / jv, j = (v % jv) * VEC, b = blockIdx.y;
+    const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
+    const T* y = (const T*)g.Y + (int64_t)b * g.yb + j;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+    for (uint32_t r = 0; r < g.R; ++r) {
+        const float a = Elem<T>::ld(x[(int64_t)r * g.xr]);
+        const AVec<T, VEC> yv = *(const AVec<T, VEC>*)(y + (int64_t)r * g.yr);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = acc[e] + a * Elem<T>::ld(yv.v[e]);
+    }
+    AVec<T, VEC> o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.v[e] = Elem<T>::st(acc[e]);
+    *(AVec<T, VEC>*)((T*)g.out + ((size_t)b * g.I + i) * g.J + j) = o;
+}
+// whether the vector form applies
+template <class T>
+inline bool gemm_thread_vec_ok(const GemmArgs& g) {
+    constexpr int VEC = 16 / sizeof(T);
+    return g.yj == 1 && g.J % VEC == 0 && g.yr % VEC == 0 && g.yb % VEC == 0 && (uintptr_t)g.Y % 16 == 0 && (uintptr_t)g.out % 16 == 0 &&
+           g.batch <= 65535 && (size_t)g.I * (g.J / VEC) < (1ull << 32) && (size_t)g.I * g.J >= 65536;
+}
+
 // One block per output element for a handful of outputs with a long reduction (the MLP's weight gradient:
 // 3 outputs of 10000 terms): NT threads stride over r, waves fold by a DPP butterfly, the block by LDS, in a fixed order.
 // `part`: NT / WAVE floats of LDS per output reduced side by side; every thread of the block reaches the barrier (threads at and beyond NT, which a
