@@ -110,19 +110,23 @@ struct Stager {
     // A "unit" is what one pass of all threads loads: NU of them make the tile.  load()/store() take a
     // unit range so that a tile's traffic can be spread over the k-steps of the previous tile.
     static constexpr int NU = PAIRS ? NV / 2 : NV;
-    // BOUND (with FAST, RCONT): the tile's last rows may lie past the operand's nrows rows while its reduction range is
-    // whole.  The descriptor then ends with row nrows - 1, and the hardware returns zeros for every load past it (rows
-    // are contiguous and at least a reduction range long, so "past the last row" is "past that byte").
+    // BOUND (with FAST): the tile's last rows may lie past the operand's nrows rows while its reduction range is whole.
+    // The descriptor then ends with the operand's last element (row nrows - 1, reduction step nred - 1), and the
+    // hardware returns zeros for every load past it.  A load of a row that does not exist either lies past that end or
+    // reads other entries of the operand; what it brings only reaches outputs that are not stored.
     template <bool FAST, bool BOUND = false>
     __device__ void load(const T* __restrict__ base, int64_t s_row, int64_t s_red, uint32_t row0, uint32_t red0,
                          uint32_t nrows, uint32_t nred, int u0 = 0, int u1 = NU) {
         constexpr bool fast = FAST;
-        static_assert(!BOUND || (FAST && RCONT), "bounded loads: the unchecked form of a row-contiguous operand");
+        static_assert(!BOUND || FAST, "bounded loads: the unchecked form");
         const int t = threadIdx.x;
         int records = 0x7fffffff;
         if constexpr (BOUND) {
-            const int64_t left = ((int64_t)(nrows - row0) * s_row - (int64_t)red0) * (int64_t)sizeof(T);
-            records = nrows > row0 ? (int)(left < 0x7fffffff ? left : 0x7fffffff) : 0;
+            // bytes from the tile's origin to the end of the operand, to a whole dword (the 16-bit row pairs are loaded as
+            // dwords; the operand starts on a dword and its strides are even, so its last dword is its own memory)
+            const int64_t last = (int64_t)(nrows - 1 - row0) * (RCONT ? s_row : 1) + (int64_t)(nred - 1 - red0) * (RCONT ? 1 : s_red);
+            const int64_t left = ((last + 1) * (int64_t)sizeof(T) + 3) & ~(int64_t)3;
+            records = nrows > row0 && nred > red0 ? (int)(left < 0x7fffffff ? left : 0x7fffffff) : 0;
         }
         if constexpr (RCONT) {
             constexpr int KV = TK / VEC;   // vectors per row
@@ -161,7 +165,8 @@ struct Stager {
                     if constexpr (fast) {
                         uint32_t voff = (uint32_t)(((t % NP) * 2 + (t / NP) * VEC * s_red) * (int64_t)sizeof(T));
                         uint32_t soff = (uint32_t)(((int64_t)u * (NT / NP) * VEC + e) * s_red * (int64_t)sizeof(T));
-                        d = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0), voff, soff, 0);
+                        if constexpr (BOUND) d = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0, records), voff + soff, 0, 0);
+                        else d = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0), voff, soff, 0);
                     } else {
                         uint32_t lo = (row < nrows && red + e < nred) ? p[(int64_t)e * s_red].bits : 0u;
                         uint32_t hi = (row + 1 < nrows && red + e < nred) ? p[(int64_t)e * s_red + 1].bits : 0u;
@@ -185,7 +190,8 @@ struct Stager {
                     if constexpr (fast) {
                         uint32_t voff = (uint32_t)(((t % ROWS) + (t / ROWS) * VEC * s_red) * (int64_t)sizeof(T));
                         uint32_t soff = (uint32_t)(((int64_t)u * (NT / ROWS) * VEC + e) * s_red * (int64_t)sizeof(T));
-                        pk.r[e] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0), voff, soff, 0);
+                        if constexpr (BOUND) pk.r[e] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0, records), voff + soff, 0, 0);
+                        else pk.r[e] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(base, 1, s_red, row0, red0), voff, soff, 0);
                     } else {
                         pk.set(e, (row < nrows && red + e < nred) ? p[(int64_t)e * s_red] : Elem<T>::zero());
                     }
@@ -397,7 +403,7 @@ template <> struct Cfgs<f16_t> : Cfgs<bf16_t> {};
 // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
 // column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
 // (16x16 tiles: one group of 4: column j0 + .. + 4*(lane/16) + e, row lane%16)
-template <class O, class Cfg, bool FAST, bool ROWS = false>      // ROWS: FAST, but rows from g.I on do not exist
+template <class O, class Cfg, bool FAST, bool EDGE = false>      // EDGE: FAST, but rows from g.I and columns from g.J on do not exist
 __device__ __forceinline__ void store_tile(O* out, const typename Cfg::Acc (&acc)[Cfg::MI][Cfg::MJ], const GemmArgs& g, uint32_t i0, uint32_t j0,
                                            int wm, int wn, int lane) {
     constexpr int MI = Cfg::MI, MJ = Cfg::MJ, TS = Cfg::TS;
@@ -412,7 +418,7 @@ __device__ __forceinline__ void store_tile(O* out, const typename Cfg::Acc (&acc
             for (int q = 0; q < (TS == 32 ? 4 : 1); ++q) {
                 uint32_t col = j0 + wn * TS * MJ + c * TS + (TS == 32 ? 8 * q + 4 * (lane / 32) : 4 * (lane / 16));
                 if (!FAST && (row >= g.I || col >= g.J)) continue;
-                if (ROWS && row >= g.I) continue;
+                if (EDGE && (row >= g.I || col >= g.J)) continue;      // (g.J is whole groups of four columns)
                 O* dst = out + (int64_t)row * g.J + col;
                 if (vec_store && (FAST || col + 4 <= g.J)) {
                     GVec<O, 4> v;
@@ -481,11 +487,11 @@ __device__ __forceinline__ TilePos tile_of_block(const GemmArgs& g) {
 // blocks a CU holds do not cover it.  The launch has as many blocks as the chip holds at once, with equal shares.
 // XCOLS (f32): X is the column matrix of a convolution (XR) or its transpose (!XR), gathered from the input (ColsView);
 // 2: four at a time (see cols_gather4), 1: one by one.
-// RB: FAST for a tile whose last rows lie past g.I (X row-contiguous, every other extent whole): X is loaded through a
-// descriptor that ends with its last row, and the rows that do not exist are not stored.
+// RB: FAST for a tile whose last rows lie past g.I or whose last columns lie past g.J (the reduction whole k-tiles): X and Y
+// are loaded through descriptors that end with their last entries, and the outputs that do not exist are not stored.
 template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false, int XCOLS = 0, bool RB = false>
 __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem, const ColsView* cv = nullptr) {
-    static_assert(!RB || (FAST && XR && !PANEL && XCOLS == 0), "bounded rows: the unchecked body, X row-contiguous and stored");
+    static_assert(!RB || (FAST && !PANEL && XCOLS == 0), "bounded rows: the unchecked body of stored operands");
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
     constexpr bool SWZ = Cfg::TS == 16;
     static_assert(!XCOLS || (std::is_same<T, float>::value && !PANEL), "the gathered operand is f32, one tile per block");
@@ -545,10 +551,10 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
         SX sx0;
         SY sy0;
         load_x(sx0, row_of(0), rb, 0, SX::NU);
-        sy0.template load<FAST>(Y, g.yj, g.yr, col_of(0), rb, g.J, re);
+        sy0.template load<FAST, RB>(Y, g.yj, g.yr, col_of(0), rb, g.J, re);
         const uint32_t q1 = nk > 1 ? 1u : 0u;
         load_x(sx, row_of(q1), red_of(q1), 0, SX::NU);
-        sy.template load<FAST>(Y, g.yj, g.yr, col_of(q1), red_of(q1), g.J, re);
+        sy.template load<FAST, RB>(Y, g.yj, g.yr, col_of(q1), red_of(q1), g.J, re);
         sx0.store(lds_x);
         sy0.store(lds_y);
     }
@@ -624,7 +630,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
                 sx.store(nx, x0, x1);
                 sy.store(ny, y0, y1);
                 load_x(sx, ni, nt, x0, x1);
-                sy.template load<FAST>(Y, g.yj, g.yr, nj, nt, g.J, re, y0, y1);
+                sy.template load<FAST, RB>(Y, g.yj, g.yr, nj, nt, g.J, re, y0, y1);
                 read_frags(s + 1, cx, cy);
             } else {
                 __syncthreads();
@@ -696,13 +702,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             gemm_mfma_body<T, XR, YR, Cfg, true>(g, pos, smem);
             return;
         }
-        // the configurations of few output rows: a tile whose columns are whole and whose rows run past g.I
-        if constexpr (XR && Cfg::TM <= 64) {
-            if ((pos.tj + 1) * Cfg::TN <= g.J) {
-                gemm_mfma_body<T, XR, YR, Cfg, true, false, 0, true>(g, pos, smem);
-                return;
-            }
-        }
+        // a tile that runs past g.I or g.J
+        gemm_mfma_body<T, XR, YR, Cfg, true, false, 0, true>(g, pos, smem);
+        return;
     }
     gemm_mfma_body<T, XR, YR, Cfg, false>(g, pos, smem);
 }

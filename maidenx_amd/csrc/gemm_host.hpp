@@ -38,6 +38,9 @@ void matmul_fwd(size_t num_els, const size_t* md, const T* a, const T* b, T* c, 
         set_status(ERR_INVALID, "matmul: num_els is not batch*m*n or an extent is 2^31 or more");
         return;
     }
+    // (the reference indexes b with a's reduction length whatever b's shape says; a caller whose shapes disagree would have
+    // the kernels read past b)
+    if (p.b_ndim >= 2 && p.b_shape[p.b_ndim - 2] != k) { set_status(ERR_INVALID, "matmul: a's last extent is not b's second to last"); return; }
     GemmArgs g{};
     g.X = a + p.a_off; g.Y = b + p.b_off; g.out = c;
     g.I = (uint32_t)m; g.J = (uint32_t)n; g.R = (uint32_t)k; g.batch = (uint32_t)(num_els / (m * n));

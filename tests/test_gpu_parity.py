@@ -565,7 +565,9 @@ def matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt, b_bcast=False):
     return sa, sb, md, av, np.broadcast_to(bv, (batch, k, n))
 
 
-MM_SHAPES = [(1, 300, 8, 256), (3, 128, 5, 264), (1, 4096, 16, 64),      # short reductions, many outputs: a thread per 16-byte vector of them
+MM_SHAPES = [# whole k-tiles, last tiles running past the rows and the columns (loaded through bounded descriptors); ragged in all three
+             (1, 1000, 1024, 1000), (2, 130, 256, 200), (1, 250, 192, 260), (1, 129, 128, 4), (1, 33, 640, 132), (1, 1000, 1000, 1000),
+             (1, 300, 8, 256), (3, 128, 5, 264), (1, 4096, 16, 64),      # short reductions, many outputs: a thread per 16-byte vector of them
              (1, 128, 128, 128), (1, 256, 192, 320), (2, 130, 70, 97), (3, 64, 600, 64), (1, 1000, 3, 1), (1, 3, 1000, 1),
              (1, 10000, 3, 1), (1, 1, 257, 1), (2, 37, 19, 53), (1, 512, 64, 64), (1, 100, 576, 64), (4, 16, 16, 16),
              # long reductions with few output tiles (split over the reduction), tall outputs with few columns
