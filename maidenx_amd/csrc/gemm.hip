@@ -723,8 +723,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_cols_kernel(GemmArgs g, Col
 }
 
 // cv: X is the gathered column matrix of a convolution (f32), see ColsView
+// r_split: the reduction length that decides how the reduction is cut (g.R is that length padded to whole k-tiles), 0: g.R
 template <class T, bool XR, bool YR, class Cfg, bool FAST, int XCOLS = 0>
-void launch_mfma_impl(GemmArgs g, const ColsView* cv = nullptr) {
+void launch_mfma_impl(GemmArgs g, const ColsView* cv = nullptr, uint32_t r_split = 0) {
     using SX = Stager<T, XR, Cfg::TM, Cfg::NT, Cfg::TS == 16>;
     constexpr size_t lds_bytes = (size_t)2 * (Cfg::TM + Cfg::TN) * SX::PITCH * sizeof(T);
     constexpr uint32_t TK = TK_BYTES / sizeof(T);
@@ -738,11 +739,12 @@ void launch_mfma_impl(GemmArgs g, const ColsView* cv = nullptr) {
     g.r_chunk = g.R;
     g.part = nullptr;
     const size_t want_blocks = Cfg::NT >= 512 ? 256 : 512;       // one or two resident blocks per CU
-    if (tiles <= 128 && g.R >= 16 * TK) {
-        uint32_t want = (uint32_t)std::min<size_t>(cdiv(want_blocks, tiles), g.R / (8 * TK));
+    const uint32_t Rs = r_split ? r_split : g.R;
+    if (tiles <= 128 && Rs >= 16 * TK) {
+        uint32_t want = (uint32_t)std::min<size_t>(cdiv(want_blocks, tiles), Rs / (8 * TK));
         if (want > 1) {
-            g.r_chunk = (uint32_t)(cdiv(cdiv(g.R, want), TK) * TK);
-            g.splits = (uint32_t)cdiv(g.R, g.r_chunk);
+            g.r_chunk = (uint32_t)(cdiv(cdiv(Rs, want), TK) * TK);
+            g.splits = (uint32_t)cdiv(Rs, g.r_chunk);
         }
     }
     size_t blocks = tiles * g.splits;
@@ -801,6 +803,22 @@ void launch_mfma_impl(GemmArgs g, const ColsView* cv = nullptr) {
     }
 }
 
+// One operand (nrows rows of R reduction steps, any strides) copied into the layout the unchecked body wants, in its own
+// orientation: rows of Rp >= R steps each when the reduction index is the contiguous one (RCONT), else Rp rows of
+// `pitch` entries.  Steps from R on and the entries past nrows are zeros.  One thread per entry of the copy.
+template <class T, bool RCONT>
+__global__ __launch_bounds__(256) void gemm_repack_kernel(const T* __restrict__ src, T* __restrict__ dst, uint32_t nrows, uint32_t R,
+                                                          uint32_t Rp, uint32_t pitch, int64_t s_batch, int64_t s_row, int64_t s_red) {
+    const uint32_t per = RCONT ? nrows * Rp : Rp * pitch;
+    const uint32_t id = blockIdx.x * 256 + threadIdx.x;
+    if (id >= per) return;
+    const uint32_t b = blockIdx.y;
+    const uint32_t row = RCONT ? id / Rp : id % pitch, red = RCONT ? id % Rp : id / pitch;
+    T v = Elem<T>::zero();
+    if (row < nrows && red < R) v = src[(int64_t)b * s_batch + (int64_t)row * s_row + (int64_t)red * s_red];
+    dst[(size_t)b * per + id] = v;
+}
+
 // The unchecked kernel needs whole tiles in all three extents, 16-byte aligned rows for naturally laid
 // out operands (4-byte aligned row pairs for turned 16-bit ones) and an output it can store 4 wide.
 template <class T, bool XR, bool YR, class Cfg>
@@ -817,10 +835,42 @@ void launch_mfma(GemmArgs g) {
         return s_row >= 0 && s_red >= 0 && ((int64_t)rows * s_row + (int64_t)TK * s_red) * (int64_t)sizeof(T) < (1ll << 31);
     };
     // (ragged tiles are decided per block inside the kernel)
-    bool fast = span_ok(g.xi, g.xr, Cfg::TM) && span_ok(g.yj, g.yr, Cfg::TN) && g.R % TK == 0 && g.J % 4 == 0 &&
-                op_ok(g.X, g.xb, g.xi, g.xr, XR) && op_ok(g.Y, g.yb, g.yj, g.yr, YR) && (uintptr_t)g.out % 16 == 0;
-    if (fast) launch_mfma_impl<T, XR, YR, Cfg, true>(g);
-    else launch_mfma_impl<T, XR, YR, Cfg, false>(g);
+    const bool x_fast = span_ok(g.xi, g.xr, Cfg::TM) && g.R % TK == 0 && op_ok(g.X, g.xb, g.xi, g.xr, XR);
+    const bool y_fast = span_ok(g.yj, g.yr, Cfg::TN) && g.R % TK == 0 && op_ok(g.Y, g.yb, g.yj, g.yr, YR);
+    const bool out_fast = g.J % 4 == 0 && (uintptr_t)g.out % 16 == 0;
+    if (x_fast && y_fast && out_fast) { launch_mfma_impl<T, XR, YR, Cfg, true>(g); return; }
+    // A reduction that is not whole k-tiles, or operands that are not aligned: the checked body loads element by element
+    // (bf16 [1000,1000]x[1000,1000] ran at 23 TFLOP/s).  A product of some size copies such an operand first - a few
+    // microseconds - with its reduction padded with zeros to whole k-tiles, which changes no bit of the result: the checked
+    // body multiplies the same zeros, and the reduction is cut into chunks as it would be without the copy.
+    const uint32_t Rp = (uint32_t)(cdiv(g.R, TK) * TK);
+    const uint32_t pitch_x = (uint32_t)(cdiv(g.I, 8) * 8), pitch_y = (uint32_t)(cdiv(g.J, 8) * 8);
+    const size_t per_x = x_fast ? 0 : (XR ? (size_t)g.I * Rp : (size_t)Rp * pitch_x);
+    const size_t per_y = y_fast ? 0 : (YR ? (size_t)g.J * Rp : (size_t)Rp * pitch_y);
+    const size_t bytes_x = (per_x * g.batch * sizeof(T) + 255) & ~(size_t)255, bytes_y = per_y * g.batch * sizeof(T);
+    const bool repack = out_fast && !capture_open() && !prog_recording() && g.batch <= 65535 &&
+                        (double)g.I * g.J * g.R * g.batch >= (double)(1 << 24) && per_x < (1ull << 31) && per_y < (1ull << 31) &&
+                        bytes_x + bytes_y <= ((size_t)1 << 30);
+    if (!repack) { launch_mfma_impl<T, XR, YR, Cfg, false>(g); return; }
+    unsigned char* buf = (unsigned char*)scratch(bytes_x + bytes_y, 1);
+    if (!buf) return;
+    GemmArgs p = g;
+    if (!x_fast) {
+        hipLaunchKernelGGL((gemm_repack_kernel<T, XR>), dim3((unsigned)cdiv(per_x, 256), g.batch), dim3(256), 0, stream(), (const T*)g.X, (T*)buf,
+                           g.I, g.R, Rp, pitch_x, g.xb, g.xi, g.xr);
+        MXH_LAUNCH_CHECK("gemm_repack");
+        p.X = buf; p.xb = (int64_t)per_x;
+        if (XR) { p.xi = Rp; p.xr = 1; } else { p.xi = 1; p.xr = pitch_x; }
+    }
+    if (!y_fast) {
+        hipLaunchKernelGGL((gemm_repack_kernel<T, YR>), dim3((unsigned)cdiv(per_y, 256), g.batch), dim3(256), 0, stream(), (const T*)g.Y,
+                           (T*)(buf + bytes_x), g.J, g.R, Rp, pitch_y, g.yb, g.yj, g.yr);
+        MXH_LAUNCH_CHECK("gemm_repack");
+        p.Y = buf + bytes_x; p.yb = (int64_t)per_y;
+        if (YR) { p.yj = Rp; p.yr = 1; } else { p.yj = 1; p.yr = pitch_y; }
+    }
+    p.R = Rp;
+    launch_mfma_impl<T, XR, YR, Cfg, true>(p, nullptr, g.R);
 }
 
 // ---- small shapes (the per-thread and per-block dot kernels are in gemm_small.hpp) -------------------

@@ -44,7 +44,7 @@ struct ApiGuard {
 #define MXH_API_INT                \
     ::mxh::ApiGuard api_guard__;   \
     if (!api_guard__.ok) return (int)hipErrorStreamCaptureWrongThread
-// Device scratch owned by the library (two independent slots per device), grown on demand and
+// Device scratch owned by the library (three independent slots per device), grown on demand and
 // reused by every call; safe because all work of the backend is ordered on one stream.
 void* scratch(size_t bytes, int slot = 0);
 // runtime.hip: a graph capture is being recorded (nothing may be allocated or grown)
