@@ -596,6 +596,37 @@ def test_matmul_forward(oracle, hip, shape, a_perm, b_perm, dt):
             assert same_bits(o, h)
 
 
+def test_matmul_refuses_operands_whose_inner_extents_disagree(hip):
+    """The kernels index b with a's reduction length: a b that says it has fewer rows would be read past its end."""
+    md = meta_matmul([8, 16], [8, 16], [4, 16], [16, 1], [16, 1])
+    with pytest.raises(Exception):
+        hip.call("matmul_f32", 8 * 16, md, In(np.ones(8 * 16, np.float32)), In(np.ones(4 * 16, np.float32)), Out(8 * 16, "f32"))
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("layout", ["row-major operands", "a turned", "b turned"])
+def test_matmul_of_unaligned_views_matches_the_aligned_product(hip, layout, dt):
+    """Operands that start one element into their buffers (no 16-byte alignment) with a reduction of whole k-tiles plus a
+    tail: the product copies them, zero-padded, and runs the unchecked kernels.  Same values as the float64 product."""
+    m, k, n = 300, 1000, 256
+    r = rng(67)
+    a = r.standard_normal((m, k)).astype(np.float32)
+    b = r.standard_normal((k, n)).astype(np.float32)
+    a_store, a_st = (a.T.copy(), [1, m]) if layout == "a turned" else (a, [k, 1])
+    b_store, b_st = (b.T.copy(), [1, k]) if layout == "b turned" else (b, [n, 1])
+    sa = to_storage(np.concatenate([[0.0], a_store.ravel()]).astype(np.float32), dt)
+    sb = to_storage(np.concatenate([[0.0], b_store.ravel()]).astype(np.float32), dt)
+    md = meta_matmul([m, n], [m, k], [k, n], a_st, b_st, 1, 1)
+    (h,) = hip.call(f"matmul_{dt}", m * n, md, In(sa), In(sb), Out(m * n, dt))
+    av = to_float(sa, dt)[1:].reshape(a_store.shape).astype(np.float64)
+    bv = to_float(sb, dt)[1:].reshape(b_store.shape).astype(np.float64)
+    av = av.T if layout == "a turned" else av
+    bv = bv.T if layout == "b turned" else bv
+    truth, scale = av @ bv, np.abs(av) @ np.abs(bv)
+    tol = 1e-5 if dt == "f32" else 1e-2
+    assert np.max(np.abs(to_float(h, dt).reshape(m, n) - truth) / scale) <= tol
+
+
 @pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("a_perm,b_perm", [(False, False), (True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("shape", [(1, 4096, 64, 3072), (1, 4096, 128, 3072), (1, 3072, 320, 4096), (3, 2048, 192, 2048)],
