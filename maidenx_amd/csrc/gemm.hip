@@ -702,9 +702,12 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             gemm_mfma_body<T, XR, YR, Cfg, true>(g, pos, smem);
             return;
         }
-        // a tile that runs past g.I or g.J
-        gemm_mfma_body<T, XR, YR, Cfg, true, false, 0, true>(g, pos, smem);
-        return;
+        // A tile that runs past g.I or g.J.  (Not in the 256 x 256 configuration with both operands turned: it has no
+        // register to spare, and with this body beside the other the compiler spills in it.)
+        if constexpr (!(Cfg::TM >= 256 && !XR && !YR)) {
+            gemm_mfma_body<T, XR, YR, Cfg, true, false, 0, true>(g, pos, smem);
+            return;
+        }
     }
     gemm_mfma_body<T, XR, YR, Cfg, false>(g, pos, smem);
 }
