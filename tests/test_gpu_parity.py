@@ -567,6 +567,8 @@ def matmul_inputs(r, batch, m, k, n, a_perm, b_perm, dt, b_bcast=False):
 
 MM_SHAPES = [# whole k-tiles, last tiles running past the rows and the columns (loaded through bounded descriptors); ragged in all three
              (1, 1000, 1024, 1000), (2, 130, 256, 200), (1, 250, 192, 260), (1, 129, 128, 4), (1, 33, 640, 132), (1, 1000, 1000, 1000),
+             # a reduction that is not whole k-tiles, in batches: the operands are copied with the reduction zero-padded
+             (2, 130, 1000, 200), (3, 256, 100, 256),
              (1, 300, 8, 256), (3, 128, 5, 264), (1, 4096, 16, 64),      # short reductions, many outputs: a thread per 16-byte vector of them
              (1, 128, 128, 128), (1, 256, 192, 320), (2, 130, 70, 97), (3, 64, 600, 64), (1, 1000, 3, 1), (1, 3, 1000, 1),
              (1, 10000, 3, 1), (1, 1, 257, 1), (2, 37, 19, 53), (1, 512, 64, 64), (1, 100, 576, 64), (4, 16, 16, 16),
