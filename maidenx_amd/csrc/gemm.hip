@@ -1140,7 +1140,10 @@ void gemm_dispatch(GemmArgs g) {
     }
     if (launch_fewrows<T>(g) || launch_fewrows_t<T>(g)) return;
     // (a few rows against a large row-major Y are not for the kernel below, whose lanes would stride down Y's columns)
-    if (outputs <= 4096 && (g.I < 32 || g.J < 32) && !(g.yj == 1 && g.J >= 256 && g.R >= 256)) {
+    // (nor is a long reduction along which both operands are strided, a weight gradient [128,10000]^T x [10000,10]: every
+    // lane of a wave would read a cache line of its own, 74 us; the tiles below cut the reduction over the chip)
+    const bool both_strided = g.xr != 1 && g.yr != 1 && g.R >= 2048 && g.I >= 32;
+    if (outputs <= 4096 && (g.I < 32 || g.J < 32) && !(g.yj == 1 && g.J >= 256 && g.R >= 256) && !both_strided) {
         hipLaunchKernelGGL(gemm_wavedot_kernel<T>, dim3(cdiv(outputs, GB / WAVE)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_wavedot");
         return;

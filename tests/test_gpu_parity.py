@@ -574,6 +574,8 @@ MM_SHAPES = [# whole k-tiles, last tiles running past the rows and the columns (
              (1, 10000, 3, 1), (1, 1, 257, 1), (2, 37, 19, 53), (1, 512, 64, 64), (1, 100, 576, 64), (4, 16, 16, 16),
              # long reductions with few output tiles (split over the reduction), tall outputs with few columns
              (1, 96, 5000, 64), (1, 130, 4100, 70), (2, 64, 2048, 64), (1, 2048, 576, 64), (1, 1100, 100, 33),
+             # few output columns and a long reduction along which both operands are strided (a_perm): tiles, not a wave per output
+             (1, 128, 5000, 10), (1, 40, 2100, 12),
              # a handful of outputs, each a long dot product (one block per output)
              (1, 2, 5000, 3), (2, 1, 4096, 1)]
 
