@@ -97,8 +97,11 @@ class ChainBuilder:
         e = ESZ[dt]
         md = u64([self.R, self.C], self.lay[la][0], self.lay[lb][0], 0, 0)
         # an operand given twice (x * x) is read from HBM once
-        nb = (self.lay[la][1] + (0 if (b == a and lb == la) else self.lay[lb][1])) * e + self.N * ESZ[out_dt or dt]
-        self.calls.append(Call(self._fn(f"{op}_{dt}"), (self.N, 2, md.ctypes.data, a, b, out), nb, tag or f"{op}_{dt}/{la}+{lb}", md))
+        same = b == a and lb == la
+        nb = (self.lay[la][1] + (0 if same else self.lay[lb][1])) * e + self.N * ESZ[out_dt or dt]
+        # ... and is a launch class of its own: fewer bytes, a shorter launch than one with two distinct operands
+        self.calls.append(Call(self._fn(f"{op}_{dt}"), (self.N, 2, md.ctypes.data, a, b, out), nb,
+                               tag or (f"{op}_{dt}/{la}+same" if same else f"{op}_{dt}/{la}+{lb}"), md))
 
     def inplace(self, op, acc, b, lb, dims=None):
         dims = dims or [self.R, self.C]

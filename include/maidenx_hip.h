@@ -57,7 +57,9 @@ int hip_memcpy_d2d(void* dst, const void* src, size_t size);
 int hip_stream_create(void** stream);
 int hip_stream_destroy(void* stream);
 int hip_stream_synchronize(void* stream);
-int hip_set_stream(void* stream);       /* stream used by every later kernel/copy (NULL = default) */
+int hip_set_stream(void* stream);       /* stream used by every later kernel/copy (NULL = default); waits for the work
+                                           queued on the previous stream first (the scratch buffers are one per device),
+                                           unless that stream is being captured */
 void* hip_get_stream(void);
 int hip_synchronize(void);              /* wait for everything queued on the backend's stream */
 /* events recorded on the backend's stream (no counterpart in the reference; used for timing) */
@@ -399,15 +401,21 @@ MX_DECL_REDUCE(mx_f16, f16)
 
 /* hip_sum_f32 for callers that cannot allocate.  No counterpart in the reference: it is for code that runs under HIP
  * graph capture, tight serving loops and harnesses that forbid allocation, where hip_sum_f32's grown-on-demand scratch
- * (its chunk partials when the reduced axis is cut to fill the chip) is not acceptable.  Same arguments, kernels and
- * result bits as hip_sum_f32; the partials live in a fixed 4 MiB array inside the library's code object (one copy per
- * GPU, held until the process ends), so the call performs no hipMalloc / hipFree.  A shape whose partials would not fit
- * is refused: hip_get_last_status() == 3 (too large) and nothing is queued — [8192,8192] and [64,512,1024] along any
- * axis fit.  All calls on a GPU share that GPU's array: calls that overlap in time on one GPU race.
+ * (its chunk partials when the reduced axis is cut to fill the chip) is not acceptable.  Same arguments and kernels as
+ * hip_sum_f32, and for a contiguous input the same result bits; the partials live in a fixed 4 MiB array inside the
+ * library's code object (one copy per GPU, held until the process ends: 3 MiB for chunk partials, 1 MiB for the partial
+ * rows of a narrow-row reduction), so the call performs no hipMalloc, hipFree or stream synchronisation.  A strided
+ * (e.g. transposed) input is summed one thread per output in ascending order - the reference's sequential order -
+ * because hip_sum_f32's logical-order copy of such an input lives in grown scratch: equal to hip_sum_f32 to rounding,
+ * not bit for bit.  A shape whose partials would not fit is refused: hip_get_last_status() == 3 (too large) and nothing
+ * is queued — [8192,8192] and [64,512,1024] along any axis fit.  All calls on a GPU share that GPU's array: calls that overlap in time on one GPU race.
  * hip_noalloc_prepare() resolves the array's device address on the current device ahead of time (optional; the first
  * hip_sum_f32_noalloc on a device does it otherwise).  Returns 0 on success. */
 void hip_sum_f32_noalloc(size_t num_els, size_t num_dims, size_t num_red_dims, const size_t* metadata, const float* inp, float* out);
 int hip_noalloc_prepare(void);
+/* How many times the library's scratch buffers were allocated or grown (hipMalloc) since the process began; a caller
+ * that must not allocate can watch it.  No counterpart in the reference. */
+size_t hip_scratch_allocations(void);
 
 /* The same for f64 and the integers (crates/maidenx_cuda/src/ops/reduction.rs:59-113; mean for f64 only, as in
  * crates/maidenx_cpu/src/ops/reduction.rs:581-586).  The accumulator is the storage type: integer sums wrap (the

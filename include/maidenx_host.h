@@ -76,7 +76,7 @@ mxt_tensor mxt_detach(mxt_tensor t);
  *   unary          : neg square relu tanh gelu exp sum_all mean_all contiguous squeeze_all
  *   unary_scalar   : add_scalar mul_scalar div_scalar pow gt_scalar
  *   reduce         : sum mean                      (dim may be negative)
- *   shape_op       : view reshape (-1 allowed) broadcast sum_to_shape transpose (2 args) squeeze unsqueeze (1 arg) */
+ *   shape_op       : view reshape (-1 allowed) broadcast broadcast_left sum_to_shape transpose (2 args) squeeze unsqueeze (1 arg) */
 mxt_tensor mxt_binary(const char* op, mxt_tensor a, mxt_tensor b);
 int mxt_binary_inplace(const char* op, mxt_tensor a, mxt_tensor b);
 mxt_tensor mxt_unary(const char* op, mxt_tensor a);

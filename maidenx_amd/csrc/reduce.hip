@@ -50,13 +50,28 @@ static void* fixed_partials() {
     return g_fixed_ptr[dev];
 }
 
+// The array is cut in two: chunk partials in the first 3 MiB, the partial rows of a regrouped narrow-row reduction
+// (col_reduce below) in the last one.
+constexpr size_t FIXED_CHUNK_BYTES = 3u << 20;
+constexpr size_t FIXED_REGROUP_BYTES = FIXED_PARTIALS_BYTES - FIXED_CHUNK_BYTES;
+
 static float* partials(size_t bytes) {
     if (!t_fixed) return (float*)scratch(bytes);
-    if (bytes > FIXED_PARTIALS_BYTES) {
-        set_status(ERR_TOO_LARGE, "no-alloc reduce: the chunk partials of this shape exceed the fixed 4 MiB array; use the allocating entry point");
+    if (bytes > FIXED_CHUNK_BYTES) {
+        set_status(ERR_TOO_LARGE, "no-alloc reduce: the chunk partials of this shape exceed their 3 MiB of the fixed array; use the allocating entry point");
         return nullptr;
     }
     return (float*)t_fixed;
+}
+
+// Partial rows of a regrouped reduction: scratch slot 2, or the last MiB of the fixed array.
+static float* regroup_rows(size_t bytes) {
+    if (!t_fixed) return (float*)scratch(bytes, 2);
+    if (bytes > FIXED_REGROUP_BYTES) {
+        set_status(ERR_TOO_LARGE, "no-alloc reduce: the regrouped partial rows of this shape exceed their 1 MiB of the fixed array; use the allocating entry point");
+        return nullptr;
+    }
+    return (float*)((unsigned char*)t_fixed + FIXED_CHUNK_BYTES);
 }
 
 // ---- column reduce: [outer, L, S] → [outer, chunks, S] ------------------------------------------
@@ -416,12 +431,12 @@ void col_reduce(const TIn* in, TOut* out, size_t outer, size_t L, size_t S, floa
     // threads.  G rows at a time are one wide row: [L, S] is read as [L / G, G * S], reduced to G * S partial columns by
     // the wide-row kernels below, and those G partial rows (plus one for the L % G rows left over, when there is one
     // slice) are folded by a second, small call.  [16777216, 5]: 2600 -> about 60 us.
-    if (S < 64 && L >= 8192 && !t_fixed && !capture_open()) {
+    if (S < 64 && L >= 8192 && (t_fixed || !capture_open())) {
         size_t G = 256;
         if (outer > 1) while (G > 1 && L % G != 0) G /= 2;         // slices must stay whole
         const size_t L0 = L / G * G, rem = L - L0;
         if (G >= 8 && G * S >= 256) {
-            float* P = (float*)scratch(outer * (G + 1) * S * sizeof(float) + 256, 2);
+            float* P = regroup_rows(outer * (G + 1) * S * sizeof(float) + 256);
             if (!P) return;
             col_reduce<TIn, float, R>(in, P, outer, L0 / G, G * S, 0.0f, src_bf16);
             if (rem) col_reduce<TIn, float, R>(in + L0 * S, P + G * S, 1, rem, S, 0.0f, src_bf16);      // (outer == 1)
@@ -529,7 +544,7 @@ void reduce_axis(size_t num_els, size_t num_dims, size_t nred, const size_t* md,
     // capture is open, where the scratch block cannot grow; small inputs keep the one-thread-per-output kernel.)
     {
         const size_t se = s != 0 ? s : 1;          // s = 0: logical index d * L + l, the layout [out_size, L]
-        if (num_els >= (1u << 18) && num_dims <= 64 && num_els % (L * se) == 0 && !capture_open()) {
+        if (num_els >= (1u << 18) && num_dims <= 64 && num_els % (L * se) == 0 && !capture_open() && !t_fixed) {
             T* tmp = (T*)scratch(num_els * sizeof(T), 1);
             if (!tmp) return;                      // status is set
             size_t cs[64];
@@ -867,9 +882,12 @@ MXH_FOLD_FOR(int32_t, i32)
 MXH_FOLD_FOR(int64_t, i64)
 
 // hip_sum_f32 for callers that cannot allocate (under graph capture, in a serving loop, in a harness that forbids it):
-// same arguments, same kernels, same bits, but the chunk partials go to the fixed array above instead of the library's
-// grown-on-demand scratch, so the call performs no hipMalloc / hipFree whatever ran before it.  A shape whose partials
-// exceed the array is refused (status ERR_TOO_LARGE) and nothing is queued.  Every partial a launch reads was written
+// same arguments and kernels, but chunk partials and regrouped partial rows go to the fixed array above instead of the
+// library's grown-on-demand scratch, so the call performs no hipMalloc / hipFree / stream synchronisation whatever ran
+// before it.  For a contiguous input the result has the bits of hip_sum_f32 (outside a capture).  A strided input is
+// never copied into logical order here (that copy lives in grown scratch): it is summed one thread per output in
+// ascending order, the reference's sequential order, which agrees with hip_sum_f32's tree to rounding only.  A shape
+// whose partials exceed their part of the array is refused (status ERR_TOO_LARGE) and nothing is queued.  Every partial a launch reads was written
 // by the launch before it, so nothing needs clearing between calls; all calls on a device share that device's array,
 // so calls that overlap on one device (two streams, two threads that switch streams) race.
 extern "C" void hip_sum_f32_noalloc(size_t n, size_t nd, size_t nr, const size_t* md, const float* in, float* out) { MXH_API;

@@ -336,6 +336,8 @@ void prog_launch_seen() {
     else g_prog_ok = false;               // a launch without a command: only the HIP graph can replay this capture
 }
 
+static size_t g_scratch_allocs = 0;       // hipMallocs made by scratch() (under g_scratch_mu)
+
 void* scratch(size_t bytes, int slot) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16 || slot < 0 || slot > 2) {
@@ -367,6 +369,7 @@ void* scratch(size_t bytes, int slot) {
     if (e != hipSuccess) { set_status(ERR_OOM, "scratch: hipMalloc", (int)e); return nullptr; }
     g_scratch[dev][slot] = p;
     g_scratch_bytes[dev][slot] = want;
+    ++g_scratch_allocs;
     return p;
 }
 
@@ -456,6 +459,14 @@ int hip_set_stream(void* s) {
     MXH_API_INT;
     // replays queued on the capture stream were ordered with the old stream only
     if (g_capture_stream && (hipStream_t)s != g_stream) (void)hipStreamSynchronize(g_capture_stream);
+    // Work still queued on the old stream may use the scratch slots and the fixed no-alloc array, which are one per
+    // device and which the first call on the new stream may overwrite: drain the old stream.  (Not when it is being
+    // captured - by the library or by the caller: nothing is running on it then, and a capture forbids the wait.)
+    if ((hipStream_t)s != g_stream && !g_capturing) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(g_stream, &st) == hipSuccess && st == hipStreamCaptureStatusNone) (void)hipStreamSynchronize(g_stream);
+        else (void)hipGetLastError();
+    }
     g_stream = (hipStream_t)s;
     return 0;
 }
@@ -474,6 +485,8 @@ int hip_event_record(void* ev) { MXH_API_INT; return (int)hipEventRecord((hipEve
 int hip_event_synchronize(void* ev) { return (int)hipEventSynchronize((hipEvent_t)ev); }
 int hip_event_elapsed_ms(void* start, void* stop, float* ms) { return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop); }
 
+// hipMallocs the scratch buffers have cost so far (for callers and tests that must see none).
+size_t hip_scratch_allocations(void) { std::lock_guard<std::mutex> lk(g_scratch_mu); return g_scratch_allocs; }
 // First error recorded since the last call (0 = none); reading it clears it.
 int hip_get_last_status(void) {
     std::lock_guard<std::recursive_mutex> api(g_api_mu);     // not refused during another thread's capture: it queues nothing

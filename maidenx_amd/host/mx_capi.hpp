@@ -189,6 +189,7 @@ mxt_tensor mxt_shape_op(const char* op, mxt_tensor a, const int64_t* args, size_
         if (is(op, "view")) return x.view(v);
         if (is(op, "reshape")) return x.reshape(v);
         if (is(op, "broadcast")) return x.broadcast(as_shape());
+        if (is(op, "broadcast_left")) return x.broadcast_left(as_shape());
         if (is(op, "sum_to_shape")) return x.sum_to_shape(as_shape());
         if (is(op, "transpose") && nargs == 2) return x.transpose((int)v[0], (int)v[1]);
         if (is(op, "squeeze") && nargs == 1) return x.squeeze((int)v[0]);

@@ -278,6 +278,7 @@ class Tensor:
     def view(self, shape): return self._shp(b"view", shape)
     def reshape(self, shape): return self._shp(b"reshape", shape)
     def broadcast(self, shape): return self._shp(b"broadcast", shape)
+    def broadcast_left(self, batch_dims): return self._shp(b"broadcast_left", batch_dims)
     def sum_to_shape(self, shape): return self._shp(b"sum_to_shape", shape)
     def transpose(self, d0, d1): return self._shp(b"transpose", (d0, d1))
     def squeeze(self, d): return self._shp(b"squeeze", (d,))

@@ -772,6 +772,13 @@ def test_matmul_backward(oracle, hip, shape, dt):
     (ga2,) = hip.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), Out(batch * m * k, dt), None)
     (gb2,) = hip.call(f"matmul_backward_{dt}", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), None, Out(batch * k * n, dt))
     assert same_bits(ga, ga2) and same_bits(gb, gb2)
+    # and, in f32, against the CPU restatement of matmul_backward (matmul.rs:124-268) itself where it finishes in a moment
+    # (its 16-bit forms accumulate in the storage type, matmul.rs:281-282: their own rounding is the larger error)
+    if dt == "f32" and batch * m * k * n <= 5_000_000:
+        oa, ob = oracle.call("matmul_backward_f32", batch * m * k, batch * k * n, md, In(sg), In(sa), In(sb), Out(batch * m * k, dt),
+                             Out(batch * k * n, dt))
+        assert np.max(np.abs(ga.astype(np.float64) - oa).reshape(ta.shape) / np.maximum(sa_, 1e-30)) <= 2e-5
+        assert np.max(np.abs(gb.astype(np.float64) - ob).reshape(tb.shape) / np.maximum(sb_, 1e-30)) <= 2e-5
 
 
 # ---------------------------------------------------------------------------------------------------

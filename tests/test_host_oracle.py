@@ -293,6 +293,28 @@ def test_bench_chain_is_the_host_layers_call_sequence(mx_oracle, op, case):
         mx.set_autograd_shortcuts(True)
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_bench_chain_tags_name_one_launch_class(dt):
+    """bench.py averages the launch times of a tag and divides ONE byte count by that average, so launches that share a
+    tag must move the same bytes (x * x reads one operand, x * y two: two tags)."""
+    import bench
+
+    class FakeLib:
+        def __getattr__(self, name):
+            return lambda *a: None
+    ptr = iter(range(1, 1000))
+    b = bench.ChainBuilder(FakeLib(), "x_", lambda count, dtag, init: (next(ptr) << 20, None), dt, 16, 32, seed=1)
+    seen = {}
+    for c in b.build():
+        assert seen.setdefault(c.tag, c.bytes) == c.bytes, c.tag
+    e = 4 if dt == "f32" else 2
+    assert seen[f"mul_{dt}/contig+contig"] == 3 * 16 * 32 * e
+    assert any(t.endswith("+same") and v == 2 * 16 * 32 * ESZ_OF[t.split("/")[0].rsplit("_", 1)[1]] for t, v in seen.items())
+
+
+ESZ_OF = {"f32": 4, "bf16": 2}
+
+
 # ---- bf16 through the host layer --------------------------------------------------------------------------
 @pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])
 def test_reference_tensor_cases_bf16(mx_oracle, case):

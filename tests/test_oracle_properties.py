@@ -412,6 +412,33 @@ def test_oracle_softmax_strided_two_dims_and_special_values(oracle):
     assert np.isnan(y[2, 0]) and np.all(np.isnan(y[2]))        # exp(NaN - max) poisons the sum
 
 
+@pytest.mark.parametrize("shape,perm,dim", [([3, 4, 5], (0, 2, 1), 2), ([2, 3, 4, 5], (3, 1, 0, 2), 2), ([2, 3, 4, 5], (1, 0, 3, 2), 3),
+                                            ([4, 3, 5], (2, 1, 0), 2), ([2, 5, 3, 2], (0, 1, 3, 2), 2)])
+def test_oracle_softmax_strided_with_several_leading_dims(oracle, shape, perm, dim):
+    """The non-contiguous branch with two or more dims in front of `dim` (softmax.rs:120-126) decomposes the slice number
+    with dim 0 FASTEST, and writes slice number `pre_idx` to the pre_idx-th block of the contiguous output
+    (softmax.rs:176-178).  So the output, read as [prod(leading), D, post], holds at block p the softmax of the logical
+    slice whose leading coordinates are the Fortran-order decomposition of p: scipy's softmax of the logical tensor with
+    its leading dims reversed (transpose, then flatten in C order).  A C-order decomposition gives another tensor whenever
+    two leading dims differ in size, as they do in every case here."""
+    from scipy.special import softmax as sp_softmax
+    r = rng(103)
+    base = r.standard_normal([shape[p] for p in np.argsort(perm)]) * 2          # storage, contiguous
+    x = base.transpose(perm)                                                      # the logical tensor, a permuted view
+    assert list(x.shape) == shape and not x.flags["C_CONTIGUOUS"]
+    strides = [st // 8 for st in x.strides]
+    n = x.size
+    (y,) = oracle.call("softmax_f64", n, len(shape), dim, meta_unary(shape, strides, 0), In(base.ravel()), Out(n, "f64"))
+    sm = sp_softmax(x, axis=dim)
+    lead = list(range(dim))
+    want = sm.transpose(lead[::-1] + list(range(dim, len(shape))))               # leading dims reversed: C flatten = F decomposition
+    assert np.allclose(y, want.ravel(), rtol=1e-12, atol=0)
+    c_order = sm.ravel()
+    assert not np.allclose(y, c_order, rtol=1e-6), "the case cannot tell the two decompositions apart"
+    (y32,) = oracle.call("softmax_f32", n, len(shape), dim, meta_unary(shape, strides, 0), In(base.astype(np.float32).ravel()), Out(n, "f32"))
+    assert np.allclose(y32, sp_softmax(x.astype(np.float32).astype(np.float64), axis=dim).transpose(lead[::-1] + list(range(dim, len(shape)))).ravel(), rtol=2e-6)
+
+
 def test_oracle_softmax_bf16_rounds_every_step(oracle):
     x = f32_to_bf16(np.array([0.1, 1.3, -0.7, 2.2], dtype=np.float32))
     (y,) = oracle.call("softmax_bf16", 4, 1, 0, meta_unary([4], [1], 0), In(x), Out(4, "bf16"))
