@@ -25,6 +25,7 @@
 #pragma once
 #include <cstddef>
 #include <cstdint>
+#include <functional>
 
 #include "mxh.hpp"
 
@@ -98,7 +99,9 @@ bool capture_open();
 // runtime.hip: offer a launch to the open chain; true = taken (the caller must not launch).
 bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes);
 // a one-thread-per-output f32 matmul: x, y are the extents of its operands
-bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y);
+// `relaunch`: launches the product for real; needed for products a chain refuses (at most 256 outputs, or - chain_ok
+// false - a reduction of more than 16 terms) and a resident step program takes
+bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y, std::function<void()> relaunch = {}, bool chain_ok = true);
 // a tail stage with its argument block; in[0..nin) / out: the byte ranges it reads and writes (out: `outputs` contiguous
 // f32 values)
 bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs);

@@ -918,7 +918,8 @@ static bool positive_strides(const GemmArgs& g) { return g.xb >= 0 && g.xi >= 0 
 // While a capture is open: a one-thread-per-output f32 product offered to the open chain as a producer over the flat
 // space of its outputs (true: do not launch).
 static bool fuse_thread_dot(const GemmArgs& g, size_t outputs) {
-    if (!capture_open() || g.batch != 1 || g.R > 16 || outputs >= (1u << 24) || !positive_strides(g)) return false;
+    // (a chain takes reductions of at most 16 terms; a resident step program any this dispatch sends here)
+    if (!capture_open() || g.batch != 1 || g.R > 256 || outputs >= (1u << 24) || !positive_strides(g)) return false;
     FuseCmd c;
     std::memset((void*)&c, 0, sizeof(c));
     c.out = g.out;
@@ -931,7 +932,10 @@ static bool fuse_thread_dot(const GemmArgs& g, size_t outputs) {
     c.nin = 2;
     c.dims[0] = g.J; c.dims[1] = g.R;
     return fuse_record_dot(c, outputs, operand_extent(g.X, g.I, g.xi, g.R, g.xr, 1, 0, sizeof(float)),
-                           operand_extent(g.Y, g.R, g.yr, g.J, g.yj, 1, 0, sizeof(float)));
+                           operand_extent(g.Y, g.R, g.yr, g.J, g.yj, 1, 0, sizeof(float)), [g, outputs] {
+                               hipLaunchKernelGGL(gemm_thread_kernel<float>, dim3(cdiv(outputs, GB)), dim3(GB), 0, stream(), g);
+                               MXH_LAUNCH_CHECK("gemm_thread");
+                           }, g.R <= 16);
 }
 // The same for a product of a handful of outputs with a long reduction: a stage of the chain's tail.
 static bool fuse_block_dot(const GemmArgs& g, size_t outputs, bool rows) {

@@ -196,9 +196,10 @@ inline bool rowsdot_applies(const GemmArgs& g) {
     GemmArgs n = g;
     return rowsdot_normalise(n);
 }
-template <int NT, int J>
+// G: groups whose loads are in flight together (it does not change the order of the additions).
+template <int NT, int J, int G = 10>
 __device__ __forceinline__ void gemm_rowsdot_body(const GemmArgs& g, unsigned tid, float* part, float* mirror = nullptr) {
-    constexpr int G = 10;     // 10 * (1 + J) 16-byte loads in flight per thread: a 10240-row product in one round trip
+    // G = 10: 10 * (1 + J) 16-byte loads in flight per thread, a 10240-row product in one round trip
     typedef float F4 __attribute__((ext_vector_type(4)));
     const F4* X4 = (const F4*)g.X;
     const F4* Y4 = (const F4*)g.Y;
@@ -241,14 +242,14 @@ __device__ __forceinline__ void gemm_rowsdot_body(const GemmArgs& g, unsigned ti
         if (mirror) mirror[tid] = sum;
     }
 }
-template <int NT>
+template <int NT, int G = 10>
 __device__ __forceinline__ void gemm_rowsdot_any(const GemmArgs& args, unsigned tid, float* part, float* mirror = nullptr) {
     GemmArgs g = args;
     rowsdot_normalise(g);
-    if (g.J == 1) gemm_rowsdot_body<NT, 1>(g, tid, part, mirror);
-    else if (g.J == 2) gemm_rowsdot_body<NT, 2>(g, tid, part, mirror);
-    else if (g.J == 3) gemm_rowsdot_body<NT, 3>(g, tid, part, mirror);
-    else gemm_rowsdot_body<NT, 4>(g, tid, part, mirror);
+    if (g.J == 1) gemm_rowsdot_body<NT, 1, G>(g, tid, part, mirror);
+    else if (g.J == 2) gemm_rowsdot_body<NT, 2, G>(g, tid, part, mirror);
+    else if (g.J == 3) gemm_rowsdot_body<NT, 3, G>(g, tid, part, mirror);
+    else gemm_rowsdot_body<NT, 4, G>(g, tid, part, mirror);
 }
 template <class T, int NT>
 __global__ __launch_bounds__(NT) void gemm_blockdot_kernel(GemmArgs g) {

@@ -2,13 +2,17 @@
 // cuda_malloc / cuda_free / cuda_memcpy_* / cuda_set_device / cuda_get_device family of
 // crates/maidenx_cuda/src/lib.rs:39-117.
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <algorithm>
+#include <functional>
 #include <mutex>
 #include <thread>
 #include <vector>
 
 #include "fuse.hpp"
 #include "mxh.hpp"
+#include "resident.hpp"
 
 namespace mxh {
 
@@ -33,8 +37,14 @@ static bool g_fuse_enabled = true;
 static FuseGroup g_fuse;                  // the open group (n == 0: none)
 static size_t g_fuse_elem_bytes = 4;
 static uint32_t g_fused_launches = 0, g_fuse_nodes = 0;     // of the open capture
+// a capture as a resident step program (see resident.hpp): launches are kept here instead of being launched
+static size_t g_res_elems = RES_DEFAULT_ELEMS;       // elements a kept launch may span; 0: no resident programs
+static bool g_res_ok = false;             // every launch of the open capture so far is one the program can hold
+static bool g_res_spilling = false;       // the kept launches are being handed on to the fused chains
+static std::vector<ResRecord> g_res;
 struct GraphExec {                        // what hip_graph_end_capture hands out
     hipGraphExec_t graph = nullptr;
+    ResProgram res;                       // the capture as a resident step program (res.device_cmds != null)
     ProgCmd* cmds = nullptr;              // device copy of the program, when the capture is one
     uint32_t n = 0;
     uint32_t fused_launches = 0, fuse_nodes = 0;
@@ -102,7 +112,9 @@ static void fuse_flush() {
 
 // Every launch and copy of the library asks for the stream right before it queues something: an open chain of fused
 // launches has to run before that.
+static void res_spill();
 hipStream_t stream() {
+    if (g_capturing && g_res_ok && !g_res_spilling) res_spill();      // something is about to be launched for real
     if (g_capturing && (g_fuse.n || g_fuse.ntail)) fuse_flush();
     return g_stream;
 }
@@ -197,7 +209,7 @@ static bool tail_same_thread(const FuseCmd* a, const void* pa, const int64_t* sa
     return a && b && a->ndims == b->ndims && a->dims[0] == b->dims[0] && a->dims[1] == b->dims[1] && same_mapping(pa, sa, pb, sb, a->ndims);
 }
 
-bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs) {
+static bool chain_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs) {
     if (!fuse_accepting() || arg_bytes > (size_t)FUSE_TAIL_ARG_BYTES || nin > 2) return false;
     if (g_fuse.ntail >= (uint32_t)FUSE_MAX_TAIL) fuse_flush();
     const uint32_t at = g_fuse.ntail;
@@ -272,7 +284,7 @@ bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_b
     return true;
 }
 
-bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
+static bool chain_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
     // only once the capture cannot be a whole-capture program any more (that path launches for real)
     if (!fuse_accepting() || ndims < 1 || ndims > 2) return false;
     for (uint32_t d = 0; d < ndims; ++d)
@@ -294,13 +306,13 @@ bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool ve
         t.dims[0] = dims[0];
         t.dims[1] = ndims == 2 ? dims[1] : 1;
         t.nel = (uint32_t)nel;
-        return fuse_record_tail(TAIL_EW, 0, &t, sizeof(t), m.in, (int)c.nin, m.out, nel);
+        return chain_record_tail(TAIL_EW, 0, &t, sizeof(t), m.in, (int)c.nin, m.out, nel);
     }
     add_member(c, m, ndims, dims, vec, nvec, elem_bytes);
     return true;
 }
 
-bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y) {
+static bool chain_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y) {
     if (!fuse_accepting() || outputs <= 256) return false;
     ParMember m;
     m.out = Extent{(uintptr_t)c.out, (uintptr_t)c.out + outputs * sizeof(float)};
@@ -311,6 +323,112 @@ bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Ex
     const uint32_t dims[1] = {(uint32_t)outputs};
     add_member(c, m, 1, dims, vec, vec ? outputs / 4 : outputs, sizeof(float));
     return true;
+}
+
+// ---- the capture as a resident step program: the launch sites' offers are kept, not launched ---------------------
+static bool res_accepting() { return g_res_ok && !g_res_spilling && fuse_accepting(); }
+
+// The capture is not going to be a resident program: what was kept goes to the fused chains in order (which take
+// exactly these offers) or is launched, and later offers go there directly.
+static void res_spill() {
+    if (!g_res_ok) return;
+    if (getenv("MXH_RESIDENT_DEBUG")) fprintf(stderr, "[resident] handing %zu kept records to the chains\n", g_res.size());
+    g_res_ok = false;
+    g_res_spilling = true;
+    std::vector<ResRecord> recs;
+    recs.swap(g_res);
+    for (const ResRecord& r : recs)
+        if (r.kind != RES_DISCARD) --g_fused_launches;      // counted again by whoever takes them now
+    for (ResRecord& r : recs) {
+        bool taken = true;
+        if (r.kind == RES_DISCARD) continue;
+        if (r.kind == RES_EW) taken = chain_record(*(const FuseCmd*)r.arg, r.ndims, r.dims, r.vec, r.units, sizeof(float));
+        else if (r.kind == RES_DOT) taken = r.chain_ok && chain_record_dot(*(const FuseCmd*)r.arg, r.outputs, r.in[0], r.in[1]);
+        else taken = chain_record_tail(r.tail_kind, r.sub, r.arg, r.arg_bytes, r.in, r.nin, r.out, r.outputs);
+        if (!taken) {
+            if (r.relaunch) r.relaunch();
+            else set_status(ERR_LAUNCH, "a launch kept for a resident step program could be neither fused nor launched");
+        }
+    }
+    g_res_spilling = false;
+}
+
+bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
+    if (res_accepting()) {
+        bool fits = ndims >= 1 && ndims <= 2 && elem_bytes == sizeof(float) && nvec * (vec ? 4 : 1) <= g_res_elems;
+        for (uint32_t d = 0; d < ndims && fits; ++d) fits = c.os[d] >= 0 && c.is[0][d] >= 0 && (c.nin < 2 || c.is[1][d] >= 0);
+        if (fits) {
+            ResRecord r;
+            r.kind = RES_EW;
+            r.vec = vec;
+            r.ndims = ndims;
+            r.dims[0] = dims[0];
+            r.dims[1] = ndims == 2 ? dims[1] : 1;
+            r.units = nvec;
+            std::memset(r.arg, 0, sizeof(r.arg));
+            std::memcpy(r.arg, &c, sizeof(c));
+            r.arg_bytes = sizeof(c);
+            r.nin = (int)c.nin;
+            r.out = operand_range(c.out, c.os, ndims, dims, elem_bytes);
+            for (uint32_t j = 0; j < c.nin; ++j) r.in[j] = operand_range(c.in[j], c.is[j], ndims, dims, elem_bytes);
+            g_res.push_back(std::move(r));
+            ++g_fused_launches;
+            return true;
+        }
+        res_spill();
+    }
+    return chain_record(c, ndims, dims, vec, nvec, elem_bytes);
+}
+
+bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y, std::function<void()> relaunch, bool chain_ok) {
+    if (res_accepting()) {
+        if (outputs <= g_res_elems && (x.hi - x.lo) / sizeof(float) <= g_res_elems && ((outputs > 256 && chain_ok) || relaunch)) {
+            ResRecord r;
+            r.kind = RES_DOT;
+            r.vec = outputs % 4 == 0 && (uintptr_t)c.out % 16 == 0;
+            r.units = r.vec ? outputs / 4 : outputs;
+            r.outputs = outputs;
+            std::memset(r.arg, 0, sizeof(r.arg));
+            std::memcpy(r.arg, &c, sizeof(c));
+            r.arg_bytes = sizeof(c);
+            r.nin = 2;
+            r.out = Extent{(uintptr_t)c.out, (uintptr_t)c.out + outputs * sizeof(float)};
+            r.in[0] = x;
+            r.in[1] = y;
+            r.relaunch = std::move(relaunch);
+            r.chain_ok = chain_ok;
+            g_res.push_back(std::move(r));
+            ++g_fused_launches;
+            return true;
+        }
+        res_spill();
+    }
+    return chain_ok && chain_record_dot(c, outputs, x, y);
+}
+
+bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs) {
+    if (res_accepting()) {
+        bool fits = arg_bytes <= (size_t)FUSE_TAIL_ARG_BYTES && nin >= 1 && nin <= 2 && (kind == TAIL_ROW_REDUCE || kind == TAIL_DOT);
+        for (int j = 0; j < nin && fits; ++j) fits = (in[j].hi - in[j].lo) / sizeof(float) <= g_res_elems;
+        if (fits) {
+            ResRecord r;
+            r.kind = kind == TAIL_ROW_REDUCE ? RES_ROW : RES_TAILDOT;
+            r.tail_kind = kind;
+            r.sub = sub;
+            r.outputs = outputs;
+            std::memset(r.arg, 0, sizeof(r.arg));
+            std::memcpy(r.arg, arg, arg_bytes);
+            r.arg_bytes = arg_bytes;
+            r.nin = nin;
+            r.out = out;
+            for (int j = 0; j < nin; ++j) r.in[j] = in[j];
+            g_res.push_back(std::move(r));
+            ++g_fused_launches;
+            return true;
+        }
+        res_spill();
+    }
+    return chain_record_tail(kind, sub, arg, arg_bytes, in, nin, out, outputs);
 }
 
 void prog_abandon() {
@@ -528,7 +646,11 @@ int hip_graph_begin_capture(void) {
     g_stream = g_capture_stream;
     g_capturing = true;
     g_capture_owner = std::this_thread::get_id();
-    g_prog_ok = g_prog_enabled;
+    // a resident step program holds what a whole-capture program holds and more: it takes that one's place
+    g_res_ok = g_res_elems > 0 && g_fuse_enabled && g_tickets_ready;
+    g_res_spilling = false;
+    g_res.clear();
+    g_prog_ok = g_prog_enabled && !g_res_ok;
     g_prog_pending = false;
     g_prog_cmds.clear();
     g_fuse.n = 0;
@@ -540,6 +662,18 @@ int hip_graph_begin_capture(void) {
 int hip_graph_end_capture(void** graph_exec) {
     MXH_API_INT;
     if (!g_capturing || !graph_exec) return (int)hipErrorInvalidValue;
+    ResProgram res;
+    bool as_res = false;
+    static const bool res_debug = getenv("MXH_RESIDENT_DEBUG") != nullptr;
+    if (res_debug) fprintf(stderr, "[resident] end of capture: candidate %d, %zu records kept\n", (int)g_res_ok, g_res.size());
+    if (g_res_ok) {
+        as_res = !g_res.empty() && res_build(g_res, res);
+        if (res_debug)
+            fprintf(stderr, "[resident] program %d: %u + %u + %u commands, %u LDS operands, %u barriers a pass, %u bytes of arena\n", (int)as_res,
+                    res.n_pro, res.n_body, res.n_epi, res.in_lds, res.barriers, res.lds_bytes);
+        if (as_res) { g_res.clear(); g_res_ok = false; }
+        else res_spill();
+    }
     fuse_flush();
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamEndCapture(g_capture_stream, &graph);
@@ -548,7 +682,12 @@ int hip_graph_end_capture(void** graph_exec) {
     const bool as_program = g_prog_ok && !g_prog_pending && !g_prog_cmds.empty();
     if (e != hipSuccess) return (int)e;
     GraphExec* ge = new GraphExec();
-    if (as_program) {
+    if (as_res) {
+        // nothing was launched into the capture: replays are one launch of the resident interpreter
+        (void)hipGraphDestroy(graph);
+        if (!res_upload(res)) { delete ge; return (int)hipErrorOutOfMemory; }
+        ge->res = res;
+    } else if (as_program) {
         // every launch of the capture has a command: replays are one launch of the interpreter
         (void)hipGraphDestroy(graph);
         const size_t bytes = g_prog_cmds.size() * sizeof(ProgCmd);
@@ -602,11 +741,65 @@ int hip_graph_launch(void* graph_exec) {
     if (!graph_exec || !g_capture_stream || g_capturing) return (int)hipErrorInvalidValue;
     GraphExec* ge = (GraphExec*)graph_exec;
     hipStream_t s = g_stream ? g_stream : g_capture_stream;
+    if (ge->res.device_cmds) {
+        res_launch(ge->res, 1, (void*)s);
+        return (int)hipGetLastError();
+    }
     if (ge->cmds) {
         prog_launch(ge->cmds, ge->n, (void*)s);
         return (int)hipGetLastError();
     }
     return (int)hipGraphLaunch(ge->graph, s);
+}
+// `times` replays in a row.  A resident step program makes them in ONE launch: its tensors stay in LDS from the first
+// replay to the last, and memory sees the final state (the same bytes as `times` separate replays leave).
+int hip_graph_launch_n(void* graph_exec, size_t times) {
+    MXH_API_INT;
+    if (!graph_exec || !g_capture_stream || g_capturing) return (int)hipErrorInvalidValue;
+    GraphExec* ge = (GraphExec*)graph_exec;
+    hipStream_t s = g_stream ? g_stream : g_capture_stream;
+    if (ge->res.device_cmds) {
+        while (times > 0) {
+            const uint32_t chunk = (uint32_t)std::min<size_t>(times, 4096);      // bounds one kernel's running time
+            res_launch(ge->res, chunk, (void*)s);
+            times -= chunk;
+        }
+        return (int)hipGetLastError();
+    }
+    for (size_t i = 0; i < times; ++i) {
+        hipError_t e = hipSuccess;
+        if (ge->cmds) { prog_launch(ge->cmds, ge->n, (void*)s); e = hipGetLastError(); }
+        else e = hipGraphLaunch(ge->graph, s);
+        if (e != hipSuccess) return (int)e;
+    }
+    return 0;
+}
+// Body commands of the resident step program behind `graph_exec` (0: the capture is not one); optionally how many
+// operand references it serves from LDS and how many work-group barriers one replay makes.
+int hip_graph_is_resident(void* graph_exec, int* lds_operands, int* barriers) {
+    if (!graph_exec || !((GraphExec*)graph_exec)->res.device_cmds) return 0;
+    const ResProgram& r = ((GraphExec*)graph_exec)->res;
+    if (lds_operands) *lds_operands = (int)r.in_lds;
+    if (barriers) *barriers = (int)r.barriers;
+    return (int)r.n_body;
+}
+// The largest tensor, in elements, a launch may touch for later captures to stay resident step programs (0: never; at
+// most 65536; default 4096); returns the previous setting.
+int hip_graph_set_resident(int max_elements) {
+    std::lock_guard<std::recursive_mutex> api(g_api_mu);
+    const int was = (int)g_res_elems;
+    g_res_elems = max_elements <= 0 ? 0 : std::min<size_t>((size_t)max_elements, RES_MAX_ELEMS);
+    return was;
+}
+// The caller no longer needs what [ptr, ptr + bytes) holds (a pooled buffer went back to its pool).  Outside a capture
+// nothing happens.  Inside one it lets a resident step program skip the write-back of tensors that nobody will read.
+void hip_buffer_discard(void* ptr, size_t bytes) {
+    MXH_API;
+    if (!g_capturing || !g_res_ok || g_res_spilling || !ptr || bytes == 0) return;
+    ResRecord r;
+    r.kind = RES_DISCARD;
+    r.out = Extent{(uintptr_t)ptr, (uintptr_t)ptr + bytes};
+    g_res.push_back(std::move(r));
 }
 int hip_graph_destroy(void* graph_exec) {
     MXH_API_INT;
@@ -617,6 +810,7 @@ int hip_graph_destroy(void* graph_exec) {
     hipError_t e = hipSuccess;
     if (ge->cmds) e = hipFree(ge->cmds);
     if (ge->graph) e = hipGraphExecDestroy(ge->graph);
+    res_destroy(ge->res);
     delete ge;
     {
         // the last live capture is gone: nothing refers to retired scratch blocks, or to the current ones, any more

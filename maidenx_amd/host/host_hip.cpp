@@ -26,7 +26,9 @@ struct HipBackend {
     static void graph_begin() { if (hip_graph_begin_capture() != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_begin_capture failed"); }
     static void graph_end(void** exec) { if (hip_graph_end_capture(exec) != 0) { *exec = nullptr; throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_end_capture failed"); } }
     static void graph_launch(void* exec) { if (hip_graph_launch(exec) != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_launch failed"); }
+    static void graph_launch_n(void* exec, size_t times) { if (hip_graph_launch_n(exec, times) != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_launch_n failed"); }
     static void graph_destroy(void* exec) { hip_graph_destroy(exec); }
+    static void discard(void* p, size_t bytes) { hip_buffer_discard(p, bytes); }
     // f32-only kernels (conv) and the float <-> float conversions
     static constexpr auto im2col = &hip_conv2d_im2col_f32;
     static constexpr auto col2im = &hip_conv2d_col2im_f32;

@@ -189,6 +189,7 @@ struct Pool {
     }
     void put(void* p, size_t cap) {
         live -= cap;
+        B::discard(p, cap);             // nobody needs the contents any more (a recorded step may then keep them out of memory)
         if (cached + cap > kMaxCached) { B::sync(); B::free(p); return; }
         free_blocks[cap].insert(p);
         cached += cap;
@@ -238,7 +239,8 @@ inline bool& sum_all_in_one_pass() { static bool on = true; return on; }
 // 2 = gather in forward and backward (no buffer of B*oh*ow x C*kh*kw elements lives between the two).
 inline int& conv_gathered_products() { static int mode = 1; return mode; }
 // What backward() leaves out without changing a bit of any gradient (false: do all of it, as the reference does): the
-// gradient of a binary op's operand that does not require one (the reference computes it and drops it, lib.rs:93-111),
+// gradient of a binary op's or a matmul's operand that does not require one (the reference computes it and drops it,
+// lib.rs:93-111),
 // x.pow(1) in the backward of pow(2) (x itself), the zero-filled buffer that the first gradient of a tensor is added
 // into when that gradient is a broadcast view (0 + g is written straight away, as for a contiguous gradient), and that
 // `0 + g` altogether when g is a fresh sum_to_shape result (sums that started from +0: it becomes the gradient as it is).
@@ -1062,16 +1064,19 @@ struct Tensor {
                 const DType dt = promoted(promoted(in[0].dtype, in[1].dtype), go_in.dtype);
                 const T l = in[0].to_dtype(dt), r = in[1].to_dtype(dt), go = go_in.to_dtype(dt);
                 auto mm = meta_matmul(l, r);
-                T gl = empty(l.shape(), dt), gr = empty(r.shape(), dt);     // zeros_like in the reference; both are fully written
+                // (zeros_like in the reference; both are fully written.  The backend leaves out a gradient whose buffer is
+                // null: the one of an input that requires none - the data a first layer multiplies - is not made)
+                const bool want_l = wanted(in, 0), want_r = wanted(in, 1);
+                T gl = want_l ? empty(l.shape(), dt) : T(), gr = want_r ? empty(r.shape(), dt) : T();
                 by_dtype(dt, "matmul backward", [&](auto tag) {
                     using E = typename decltype(tag)::type;
-                    K<E>::matmul_backward(gl.size(), gr.size(), mm.first.data(), go.template p<E>(), l.template p<E>(), r.template p<E>(),
-                                          gl.template p<E>(), gr.template p<E>());
+                    K<E>::matmul_backward(l.size(), r.size(), mm.first.data(), go.template p<E>(), l.template p<E>(), r.template p<E>(),
+                                          want_l ? gl.template p<E>() : nullptr, want_r ? gr.template p<E>() : nullptr);
                 });
                 ++backend_calls();
                 B::check();
                 // the gradients go back in the inputs' own dtypes (matmul.rs:137-143)
-                return std::vector<T>{gl.to_dtype(in[0].dtype), gr.to_dtype(in[1].dtype)};
+                return std::vector<T>{want_l ? gl.to_dtype(in[0].dtype) : T(), want_r ? gr.to_dtype(in[1].dtype) : T()};
             });
         }
         return result;
@@ -1395,46 +1400,51 @@ size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr
                 }
             }
             if (period) {
-                void* exec = nullptr;
-                const size_t allocs_before = pool.device_allocs, calls_before = backend_calls();
-                // several periods per graph: one graph launch costs a few microseconds however many nodes it holds
-                const size_t one = period;
-                period = one * std::max<size_t>(1, 12 / one);
-                while (period > one && 2 * period > epochs - done) period -= one;
-                // The recorded steps must follow the allocation pattern the warm-up settled into: a replay runs on the
-                // addresses recorded, and is only the next step's work if that step would have used the same ones.
-                const size_t warm = traces.size();
-                std::vector<std::vector<void*>> recorded(period);
-                B::graph_begin();
-                try {
-                    for (size_t k = 0; k < period; ++k) {
-                        pool.trace = &recorded[k];
-                        step(done + k);
+                const size_t one = period, warm = traces.size();
+                // Records `span` steps (a multiple of the period) and replays them as often as whole spans fit; false when
+                // the recording left the allocation pattern (it then ran once, and the loop goes on eagerly).  The recorded
+                // steps must follow the pattern the warm-up settled into: a replay runs on the addresses recorded, and is
+                // only the next step's work if that step would have used the same ones.
+                auto record_and_replay = [&](size_t span) {
+                    void* exec = nullptr;
+                    const size_t allocs_before = pool.device_allocs, calls_before = backend_calls();
+                    std::vector<std::vector<void*>> recorded(span);
+                    B::graph_begin();
+                    try {
+                        for (size_t k = 0; k < span; ++k) {
+                            pool.trace = &recorded[k];
+                            step(done + k);
+                            pool.trace = nullptr;
+                        }
+                    } catch (...) {
                         pool.trace = nullptr;
+                        try { B::graph_end(&exec); } catch (...) { exec = nullptr; }
+                        if (exec) B::graph_destroy(exec);
+                        throw;
                     }
-                } catch (...) {
-                    pool.trace = nullptr;
-                    try { B::graph_end(&exec); } catch (...) { exec = nullptr; }
-                    if (exec) B::graph_destroy(exec);
-                    throw;
-                }
-                B::graph_end(&exec);
-                bool periodic = true;
-                for (size_t k = 0; k < period && periodic; ++k) periodic = recorded[k] == traces[warm - one + k % one];
-                if (pool.device_allocs != allocs_before) {
+                    B::graph_end(&exec);
+                    bool periodic = true;
+                    for (size_t k = 0; k < span && periodic; ++k) periodic = recorded[k] == traces[warm - one + k % one];
+                    if (pool.device_allocs != allocs_before) {
+                        B::graph_destroy(exec);
+                        throw Error(ErrKind::Backend, "training loop allocated device memory while it was being recorded");
+                    }
+                    // the recorded steps did not run yet: replay them, then as many more whole spans as fit
+                    const size_t calls_per_span = backend_calls() - calls_before;
+                    // (one call for all the replays: a backend that keeps the recording as a resident step program makes
+                    // them in one launch)
+                    size_t spans = periodic ? (epochs - done) / span : 1;
+                    B::graph_launch_n(exec, spans);
+                    backend_calls() += calls_per_span * (spans - 1);
+                    done += spans * span;
+                    replayed += spans * span;
                     B::graph_destroy(exec);
-                    throw Error(ErrKind::Backend, "training loop allocated device memory while it was being recorded");
-                }
-                // the recorded steps did not run yet: replay them, then as many more whole periods as fit
-                const size_t calls_per_period = backend_calls() - calls_before;
-                // (a recording that left the pattern is still exactly the steps it recorded: it runs once, and the loop
-                // goes on eagerly)
-                size_t periods = periodic ? (epochs - done) / period : 1;
-                for (size_t r = 0; r < periods; ++r) B::graph_launch(exec);
-                backend_calls() += calls_per_period * (periods - 1);
-                done += periods * period;
-                replayed = periods * period;
-                B::graph_destroy(exec);
+                    return periodic;
+                };
+                // several periods per graph: a graph launch costs a few microseconds however many nodes it holds
+                size_t span = one * std::max<size_t>(1, 12 / one);
+                while (span > one && 2 * span > epochs - done) span -= one;
+                record_and_replay(span);
             }
         }
     }

@@ -50,6 +50,9 @@ def load():
         ("hip_graph_is_program", [C.c_void_p], C.c_int), ("hip_graph_set_programs", [C.c_int], C.c_int),
         ("hip_graph_fused_launches", [C.c_void_p, C.POINTER(C.c_int)], C.c_int), ("hip_graph_set_fusion", [C.c_int], C.c_int),
         ("hip_noalloc_prepare", [], C.c_int), ("hip_scratch_allocations", [], C.c_size_t),
+        ("hip_graph_launch_n", [C.c_void_p, C.c_size_t], C.c_int),
+        ("hip_graph_is_resident", [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
+        ("hip_graph_set_resident", [C.c_int], C.c_int), ("hip_buffer_discard", [C.c_void_p, C.c_size_t], None),
     ]:
         fn = getattr(lib, name)
         fn.argtypes = args

@@ -42,6 +42,7 @@ struct OracleBackend {
     static void* alloc(size_t bytes) { return std::malloc(bytes); }
     static void free(void* p) { std::free(p); }
     static void sync() {}
+    static void discard(void*, size_t) {}
     static void h2d(void* d, const void* s, size_t n) { std::memcpy(d, s, n); }
     static void d2h(void* d, const void* s, size_t n) { std::memcpy(d, s, n); }
     static void check() {}

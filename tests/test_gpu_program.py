@@ -19,6 +19,15 @@ def lib():
     return L.load()
 
 
+@pytest.fixture(autouse=True)
+def without_resident_programs(lib):
+    """These tests pin down whole-capture programs and fused chains; a capture they make would otherwise become a resident
+    step program (tests/test_gpu_resident.py runs the same sequences that way)."""
+    was = lib.hip_graph_set_resident(0)
+    yield
+    lib.hip_graph_set_resident(was)
+
+
 def u64(*parts):
     out = []
     for x in parts:
@@ -76,7 +85,9 @@ def replay_equals_eager(lib, seq, expect_program, replays=3):
     h = C.c_void_p()
     assert lib.hip_graph_end_capture(C.byref(h)) == 0
     try:
-        assert lib.hip_graph_is_program(h) == (1 if expect_program else 0)
+        # one launch of one work-group: a program, or (where those are allowed) the resident step program that replaces it
+        one_launch = lib.hip_graph_is_program(h) == 1 or lib.hip_graph_is_resident(h, None, None) > 0
+        assert one_launch == bool(expect_program)
         for _ in range(replays):
             seq.clear_outputs()          # eager work and a synchronisation between the replays
             assert lib.hip_graph_launch(h) == 0
@@ -446,9 +457,13 @@ def test_fusion_can_be_switched_off(lib):
 
 @pytest.mark.parametrize("seed", range(24))
 def test_fused_random_sequences_with_aliasing(lib, seed):
+    random_sequence_with_aliasing(lib, seed, resident=False)
+
+
+def random_sequence_with_aliasing(lib, seed, resident):
     """Random chains over a small pool of buffers, with views that overlap in every way (same elements, shifted,
     broadcast, transposed, in place): whatever the grouping decides, a replay must leave the bytes of the eager run
-    in every buffer."""
+    in every buffer.  resident: the capture holds nothing else and must become a resident step program."""
     r = np.random.default_rng(1000 + seed)
     n = int(r.choice([1, 3, 64, 200, 1024, 4096, 10000]))
     rows = int(r.choice([d for d in (1, 2, 4, 8, 16, 64) if n % d == 0]))
@@ -518,12 +533,15 @@ def test_fused_random_sequences_with_aliasing(lib, seed):
     assert lib.hip_synchronize() == 0 and lib.hip_get_last_status() == 0, lib.hip_status_string()
     want = [p.to_numpy(np.float32).copy() for p in pool]
     big = L.DeviceBuffer(1 << 20)
+    reset()
     assert lib.hip_graph_begin_capture() == 0
-    lib.hip_fill_f32((1 << 20) // 4, big.ptr, C.c_float(0.0))
+    if not resident:
+        lib.hip_fill_f32((1 << 20) // 4, big.ptr, C.c_float(0.0))
     run()
     h = C.c_void_p()
     assert lib.hip_graph_end_capture(C.byref(h)) == 0
     try:
+        assert (lib.hip_graph_is_resident(h, None, None) > 0) == resident
         for _ in range(2):
             reset()
             assert lib.hip_graph_launch(h) == 0 and lib.hip_synchronize() == 0
