@@ -12,6 +12,7 @@
 //   col2im : gather form with the reference's fixed summation order (ho then wo ascending, at
 //            most kh*kw terms), so the result is bit-exact and deterministic; column indices at
 //            or beyond num_els are skipped exactly as the reference does.
+#include "elementwise.hpp"
 #include "mxh.hpp"
 
 namespace mxh {
@@ -59,10 +60,12 @@ __global__ __launch_bounds__(CB) void im2col_kernel(ConvMeta m, const T* __restr
 // checks and no global-load latency), then the kh*kw shifted copies leave as 16-byte stores.
 struct BandMeta {
     uint32_t nb, bands, HP, WP, nvec_seg;       // output rows per band, bands per plane, tile extent, vectors per (i, j) segment
-    FastDiv d_WP, d_bands, d_seg, d_owv, d_kw;
+    uint32_t vec_in;                            // the input rows are whole aligned 16-byte vectors
+    FastDiv d_WP, d_bands, d_seg, d_owv, d_kw, d_wv;
 };
 
-template <class T, int VEC>
+// STREAM: the column matrix will not fit the last-level cache, so its stores carry the non-temporal hint.
+template <class T, int VEC, bool STREAM = false>
 __global__ __launch_bounds__(CB) void im2col_band_kernel(ConvMeta m, BandMeta k, const T* __restrict__ in, T* __restrict__ col) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* tile = (T*)smem;
@@ -73,12 +76,50 @@ __global__ __launch_bounds__(CB) void im2col_band_kernel(ConvMeta m, BandMeta k,
     const int hi0 = (int)(ho0 * m.sh) - (int)m.ph;             // input row of tile row 0
     const uint32_t hp = (nrows - 1) * m.sh + m.kh;             // tile rows this band uses
     const T* src = in + (size_t)plane * m.H * m.W;
-    for (uint32_t idx = threadIdx.x; idx < hp * k.WP; idx += CB) {
-        uint32_t r, cidx;
-        fd_divmod(idx, k.d_WP, r, cidx);
-        int hi = hi0 + (int)r, wi = (int)cidx - (int)m.pw;
-        bool ok = hi >= 0 && hi < (int)m.H && wi >= 0 && wi < (int)m.W;
-        tile[idx] = ok ? src[(size_t)hi * m.W + wi] : T{};
+    if (k.vec_in) {
+        // The band's input rows as 16-byte vectors, up to four a thread, all requested before anything else happens: one
+        // memory latency for the tile.  (Element by element, each behind its own bounds test, a thread waited for fourteen
+        // loads one after the other - and every block of the launch did so at the same time, the grid being one round of
+        // blocks: a fifth of the kernel passed before the first store.)  The tile is zeroed while the loads are in flight.
+        const uint32_t wv = m.W / VEC;
+        const int r_lo = hi0 < 0 ? -hi0 : 0, r_hi = min((int)hp, (int)m.H - hi0);       // tile rows that exist in the input
+        const uint32_t nload = r_hi > r_lo ? (uint32_t)(r_hi - r_lo) * wv : 0u;
+        const T* first = src + (size_t)(hi0 + r_lo) * m.W;
+        for (uint32_t base = 0; base < nload || base == 0; base += 4 * CB) {
+            CVec<T, VEC> v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t idx = base + q * CB + threadIdx.x;
+                if (idx < nload) v[q] = *(const CVec<T, VEC>*)(first + (size_t)idx * VEC);
+            }
+            if (base == 0) {
+                CVec<T, VEC> z;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) z.v[e] = T{};
+                const uint32_t nz = (hp * k.WP * (uint32_t)sizeof(T) + 15) / 16;      // (the tile's allocation is a whole number of vectors)
+                for (uint32_t i = threadIdx.x; i < nz; i += CB) ((CVec<T, VEC>*)tile)[i] = z;
+                __syncthreads();
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t idx = base + q * CB + threadIdx.x;
+                if (idx < nload) {
+                    uint32_t r, cv;
+                    fd_divmod(idx, k.d_wv, r, cv);
+                    T* t = tile + ((uint32_t)r_lo + r) * k.WP + m.pw + cv * VEC;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) t[e] = v[q].v[e];
+                }
+            }
+        }
+    } else {
+        for (uint32_t idx = threadIdx.x; idx < hp * k.WP; idx += CB) {
+            uint32_t r, cidx;
+            fd_divmod(idx, k.d_WP, r, cidx);
+            int hi = hi0 + (int)r, wi = (int)cidx - (int)m.pw;
+            bool ok = hi >= 0 && hi < (int)m.H && wi >= 0 && wi < (int)m.W;
+            tile[idx] = ok ? src[(size_t)hi * m.W + wi] : T{};
+        }
     }
     __syncthreads();
     const uint32_t seg = nrows * (m.ow / VEC);                 // vectors of one (i, j) segment in this band
@@ -96,7 +137,7 @@ __global__ __launch_bounds__(CB) void im2col_band_kernel(ConvMeta m, BandMeta k,
         CVec<T, VEC> o;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o.v[e] = t[e * m.sw];
-        *(CVec<T, VEC>*)(dst_plane + ((size_t)ij * m.oh + r) * m.ow + wov * VEC) = o;
+        st_vec<STREAM>((CVec<T, VEC>*)(dst_plane + ((size_t)ij * m.oh + r) * m.ow + wov * VEC), o);
     }
 }
 
@@ -249,22 +290,31 @@ void im2col(size_t num_els, const size_t* md, const T* in, T* col) {
         // band kernel: whole column matrix, rows a multiple of the vector width
         BandMeta k;
         k.WP = (m.ow - 1) * m.sw + m.kw;
-        auto tile_bytes = [&](uint32_t nb) { return (size_t)((nb - 1) * m.sh + m.kh) * k.WP * sizeof(T); };
+        auto tile_bytes = [&](uint32_t nb) { return ((size_t)((nb - 1) * m.sh + m.kh) * k.WP * sizeof(T) + 15) / 16 * 16; };
         constexpr size_t LDS_MAX = 32 * 1024;
         if (tile_bytes(1) <= LDS_MAX) {
             uint32_t nb = m.oh;
             while (nb > 1 && tile_bytes(nb) > LDS_MAX) nb = (nb + 1) / 2;
-            // enough blocks to fill the chip, as long as a segment stays a few KB long
-            while (nb > 1 && (size_t)m.B * m.C * cdiv(m.oh, nb) < 1024 && (size_t)(nb / 2) * m.ow * sizeof(T) >= 2048) nb = (nb + 1) / 2;
+            // Several rounds of blocks, as long as a segment stays a few KB long: a block first loads its tile and then only
+            // stores, and in a launch of one round every block is in the same phase at the same time.  [32,64,56,56] 3x3:
+            // whole planes (2048 blocks, one round) 48.8 us, bands of 28 / 14 / 7 rows 49.5 / 45.9 / 48.0 us.
+            while (nb > 1 && (size_t)m.B * m.C * cdiv(m.oh, nb) < 8192 && (size_t)(nb / 2) * m.ow * sizeof(T) >= 2048) nb = (nb + 1) / 2;
             k.nb = nb;
             k.bands = (uint32_t)cdiv(m.oh, nb);
             k.HP = (nb - 1) * m.sh + m.kh;
             k.nvec_seg = nb * (m.ow / VEC);
             k.d_WP = make_fastdiv(k.WP); k.d_bands = make_fastdiv(k.bands); k.d_seg = make_fastdiv(k.nvec_seg);
             k.d_owv = make_fastdiv(m.ow / VEC); k.d_kw = make_fastdiv(m.kw);
+            // whole input rows as vectors: the padded tile must hold every input column (a pad narrower than the kernel
+            // reaches always does, but the metadata is the caller's)
+            k.vec_in = m.W % VEC == 0 && ((uintptr_t)in % 16) == 0 && m.pw + m.W <= k.WP ? 1u : 0u;
+            k.d_wv = make_fastdiv(k.vec_in ? m.W / VEC : 1);
             size_t blocks = (size_t)m.B * m.C * k.bands;
             if (blocks < (1ull << 31)) {
-                hipLaunchKernelGGL((im2col_band_kernel<T, VEC>), dim3((unsigned)blocks), dim3(CB), tile_bytes(nb), stream(), m, k, in, col);
+                if (ew_stream_bytes() != 0 && full * sizeof(T) >= ew_stream_bytes())
+                    hipLaunchKernelGGL((im2col_band_kernel<T, VEC, true>), dim3((unsigned)blocks), dim3(CB), tile_bytes(nb), stream(), m, k, in, col);
+                else
+                    hipLaunchKernelGGL((im2col_band_kernel<T, VEC>), dim3((unsigned)blocks), dim3(CB), tile_bytes(nb), stream(), m, k, in, col);
                 MXH_LAUNCH_CHECK("im2col");
                 return;
             }
