@@ -422,6 +422,20 @@ MX_DECL_REDUCE(float, f32)
 MX_DECL_REDUCE(mx_bf16, bf16)
 MX_DECL_REDUCE(mx_f16, f16)
 
+/* Fused loss and optimizer steps (no counterpart in the reference's backend: its MSELoss is four tensor ops and six more
+ * backward, crates/maidenx_nn/src/losses/mse.rs:21-29, its SGD two per parameter, optimizers/sgd.rs:17-27).  The same
+ * element functions in the same order on values held in registers, contiguous f32 buffers:
+ *   hip_mse_loss_f32           loss[0] = (sum of square(pred[i] - target[i])) / n          (16-byte aligned operands)
+ *   hip_mse_loss_backward_f32  grad_pred[i] = 0 + (((grad_loss[0] / n) * 2) * (pred[i] - target[i])),
+ *                              grad_target[i] = 0 + (-(that product)); either output may be NULL
+ *   hip_sgd_step_f32           param[i] = param[i] - grad[i] * lr
+ * Gradients and parameters are bit for bit what sub / pow / sum_all / div_scalar and their backward, or mul_scalar and
+ * sub_inplace, give; the loss is a sum of n terms added in a fixed tree of its own (within the f32 tolerance of a
+ * reduction of the op sequence's, whose order the reference does not fix either). */
+void hip_mse_loss_f32(size_t n, const float* pred, const float* target, float* loss);
+void hip_mse_loss_backward_f32(size_t n, const float* pred, const float* target, const float* grad_loss, float* grad_pred, float* grad_target);
+void hip_sgd_step_f32(size_t n, float* param, const float* grad, float lr);
+
 /* hip_sum_f32 for callers that cannot allocate.  No counterpart in the reference: it is for code that runs under HIP
  * graph capture, tight serving loops and harnesses that forbid allocation, where hip_sum_f32's grown-on-demand scratch
  * (its chunk partials when the reduced axis is cut to fill the chip) is not acceptable.  Same arguments and kernels as

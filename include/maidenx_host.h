@@ -125,6 +125,12 @@ void mxt_set_sum_all_in_one_pass(int enabled);
  * accumulation when the gradient is a broadcast view, and the first accumulation itself (0 + g) when g is a fresh
  * sum_to_shape result, whose buffer then becomes the gradient. */
 void mxt_set_autograd_shortcuts(int enabled);
+/* MSELoss (crates/maidenx_nn/src/losses/mse.rs:21-29: sub, pow(2), sum_all, div_scalar) and SGD::step
+ * (optimizers/sgd.rs:17-27: mul_scalar, in-place sub) are one backend call each on the HIP build (hip_mse_loss_f32 and
+ * its backward, hip_sgd_step_f32) for contiguous f32 tensors: every gradient and every updated parameter is the same
+ * bytes as the op sequence gives, the loss is summed in another order (within the f32 tolerance of a reduction).
+ * enabled = 0: the op sequences. */
+void mxt_set_fused_nn_kernels(int enabled);
 /* Conv2d backward (nn/layers/conv.rs:253-268): col2im is handed num_els = B*C*H*W and reads no entry of grad_cols at
  * or beyond that flat index (crates/maidenx_cpu/src/nn/conv.rs:135), so by default only the leading
  * ceil(B*C*H*W / (C*kh*kw)) rows of grad_cols are computed; the input gradient is the same bytes either way.

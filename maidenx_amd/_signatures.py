@@ -175,6 +175,9 @@ def extension_signatures():
                  ("bool", "f16"), ("f32", "f16"), ("f16", "f32"), ("f16", "bool")):
         sig[f"cast_{a}_{b}"] = [SZ, P, P]
     sig["sum_f32_noalloc"] = [SZ, SZ, SZ, P, P, P]
+    sig["mse_loss_f32"] = [SZ, P, P, P]
+    sig["mse_loss_backward_f32"] = [SZ, P, P, P, P, P]
+    sig["sgd_step_f32"] = [SZ, P, P, C.c_float]
     sig["conv2d_cols_matmul_f32"] = [P, C.c_int, P, P, SZ, P, P]
     sig.update(cast_signatures())
     sig.update(wide_util_signatures())

@@ -21,6 +21,10 @@ struct HipBackend {
     }
     static constexpr bool has_graphs = true;
     static constexpr bool has_fused_adam = true;
+    static constexpr bool has_fused_nn = true;
+    static constexpr auto mse_loss = &hip_mse_loss_f32;
+    static constexpr auto mse_loss_backward = &hip_mse_loss_backward_f32;
+    static constexpr auto sgd_step = &hip_sgd_step_f32;
     static constexpr bool has_cols_matmul = true;
     static constexpr auto cols_matmul = &hip_conv2d_cols_matmul_f32;
     static void graph_begin() { if (hip_graph_begin_capture() != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_begin_capture failed"); }

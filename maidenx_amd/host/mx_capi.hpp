@@ -259,6 +259,7 @@ void mxt_set_graph_replay(int enabled) { g_graphs = enabled != 0; }
 size_t mxt_last_train_replayed(void) { return g_replayed; }
 void mxt_set_sum_all_in_one_pass(int enabled) { mxt::sum_all_in_one_pass() = enabled != 0; }
 void mxt_set_autograd_shortcuts(int enabled) { mxt::autograd_shortcuts() = enabled != 0; }
+void mxt_set_fused_nn_kernels(int enabled) { mxt::fused_nn_kernels() = enabled != 0; }
 void mxt_set_conv_skip_unread_grad_cols(int enabled) { mxt::conv_skip_unread_grad_cols() = enabled != 0; }
 void mxt_set_conv_gathered_products(int mode) { mxt::conv_gathered_products() = mode < 0 ? 0 : mode > 2 ? 2 : mode; }
 

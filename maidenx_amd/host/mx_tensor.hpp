@@ -245,6 +245,10 @@ inline int& conv_gathered_products() { static int mode = 1; return mode; }
 // into when that gradient is a broadcast view (0 + g is written straight away, as for a contiguous gradient), and that
 // `0 + g` altogether when g is a fresh sum_to_shape result (sums that started from +0: it becomes the gradient as it is).
 inline bool& autograd_shortcuts() { static bool on = true; return on; }
+// MSELoss and SGD::step as one backend call each where the backend has the fused kernels (the same element functions in
+// the same order: every gradient and parameter is the same bytes; the loss is summed in a tree of its own, within the f32
+// tolerance of a reduction).  false: the op sequences of the reference.
+inline bool& fused_nn_kernels() { static bool on = true; return on; }
 // Count of whole-buffer dtype conversions (with_dtype: a host loop in the reference, a kernel here).
 inline size_t& cast_calls() { static size_t n = 0; return n; }
 
@@ -1285,8 +1289,44 @@ struct Conv2d {                                                                 
     }
 };
 
+// whether a tensor is a plain f32 block a fused kernel can take: contiguous from the start of a 16-byte aligned buffer
+template <class B>
+inline bool plain_f32(const Tensor<B>& t) {
+    return t.dtype == DType::F32 && t.size() > 0 && t.is_contiguous() && t.offset() == 0 && ((uintptr_t)t.template p<float>() % 16) == 0;
+}
+
 template <class B>
 Tensor<B> mse_loss(const Tensor<B>& pred, const Tensor<B>& target) {                // nn/losses/mse.rs:21-29
+    using T = Tensor<B>;
+    if constexpr (B::has_fused_nn) {
+        // sub, pow(2), sum_all and div_scalar as one kernel, and their six backward ops as another: the difference is
+        // recomputed there instead of stored, every gradient is what the op sequence gives bit for bit
+        if (fused_nn_kernels() && plain_f32(pred) && plain_f32(target) && pred.shape() == target.shape()) {
+            T loss = T::empty(Shape{}, DType::F32);
+            B::mse_loss(pred.size(), pred.template p<float>(), target.template p<float>(), loss.template p<float>());
+            ++backend_calls();
+            B::check();
+            if (pred.requires_grad || target.requires_grad) {
+                loss.with_grad();
+                loss.set_node("mse_loss", {pred, target}, [](const std::vector<T>& in, const T& go_in) {
+                    const T go = go_in.to_dtype(DType::F32).contiguous();
+                    const bool want_p = T::wanted(in, 0), want_t = T::wanted(in, 1);
+                    T gp = want_p ? T::empty(in[0].shape(), DType::F32) : T(), gt = want_t ? T::empty(in[1].shape(), DType::F32) : T();
+                    if (want_p || want_t) {
+                        B::mse_loss_backward(in[0].size(), in[0].template p<float>(), in[1].template p<float>(),
+                                             go.template p<float>() + go.offset(), want_p ? gp.template p<float>() : nullptr,
+                                             want_t ? gt.template p<float>() : nullptr);
+                        ++backend_calls();
+                        B::check();
+                    }
+                    gp.sums_from_zero = want_p;      // `0 + g`, as sub's sum_to_shape leaves it
+                    gt.sums_from_zero = want_t;
+                    return std::vector<T>{gp, gt};
+                });
+            }
+            return loss;
+        }
+    }
     Tensor<B> squared = pred.sub(target).pow(2.0f);
     return squared.sum_all().div_scalar((float)squared.size());
 }
@@ -1296,8 +1336,20 @@ struct SGD {                                                                    
     float lr;
     explicit SGD(float lr_) : lr(lr_) {}
     void step(const std::vector<Tensor<B>*>& params) const {
-        for (Tensor<B>* p : params)
-            if (p->has_grad()) p->sub_(p->grad().mul_scalar(lr));
+        for (Tensor<B>* p : params) {
+            if (!p->has_grad()) continue;
+            if constexpr (B::has_fused_nn) {
+                // mul_scalar and the in-place sub as one pass: the same two roundings per element
+                const Tensor<B> g = p->grad();
+                if (fused_nn_kernels() && plain_f32(*p) && plain_f32(g) && g.shape() == p->shape()) {
+                    B::sgd_step(p->size(), p->template p<float>(), g.template p<float>(), lr);
+                    ++backend_calls();
+                    B::check();
+                    continue;
+                }
+            }
+            p->sub_(p->grad().mul_scalar(lr));
+        }
     }
     void zero_grad(const std::vector<Tensor<B>*>& params) const {
         for (Tensor<B>* p : params) p->zero_grad();

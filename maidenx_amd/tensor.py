@@ -43,7 +43,7 @@ def _bind(lib):
         "mxt_conv2d_new": ([P, P, SZ, SZ, SZ, SZ, SZ, SZ], P), "mxt_module_forward": ([P, P], P), "mxt_module_weight": ([P], P),
         "mxt_module_bias": ([P], P), "mxt_module_release": ([P], None), "mxt_mse_loss": ([P, P], P), "mxt_sgd_step": ([P, F], I),
         "mxt_sgd_zero_grad": ([P], I), "mxt_train": ([P, P, P, F, SZ, P], I), "mxt_set_graph_replay": ([I], None),
-        "mxt_last_train_replayed": ([], SZ), "mxt_set_conv_skip_unread_grad_cols": ([I], None), "mxt_set_autograd_shortcuts": ([I], None), "mxt_set_sum_all_in_one_pass": ([I], None), "mxt_set_conv_gathered_products": ([I], None),
+        "mxt_last_train_replayed": ([], SZ), "mxt_set_conv_skip_unread_grad_cols": ([I], None), "mxt_set_autograd_shortcuts": ([I], None), "mxt_set_fused_nn_kernels": ([I], None), "mxt_set_sum_all_in_one_pass": ([I], None), "mxt_set_conv_gathered_products": ([I], None),
         "mxt_adam_new": ([C.c_double] * 4, P), "mxt_adam_release": ([P], None), "mxt_adam_set_fused": ([P, I], None), "mxt_adam_step": ([P, P], I),
         "mxt_backend_calls": ([], SZ), "mxt_reset_backend_calls": ([], None), "mxt_device_allocations": ([], SZ), "mxt_synchronize": ([], I),
     }
@@ -145,6 +145,11 @@ class Host:
     def set_autograd_shortcuts(self, enabled):
         """backward() skips work that cannot change any gradient (default), or does everything the reference does."""
         self.lib.mxt_set_autograd_shortcuts(int(enabled))
+
+    def set_fused_nn_kernels(self, enabled):
+        """MSELoss and SGD.step as one backend call each (default; same gradients and parameters bit for bit), or the op
+        sequences of the reference."""
+        self.lib.mxt_set_fused_nn_kernels(int(enabled))
 
     def set_conv_gathered_products(self, mode):
         """Conv2d's products with the column matrix: 0 = store the matrix first (im2col), 1 = gather it inside the product

@@ -48,6 +48,7 @@ struct OracleBackend {
     static void check() {}
     static constexpr bool has_graphs = false;
     static constexpr bool has_fused_adam = false;
+    static constexpr bool has_fused_nn = false;
     static constexpr bool has_cols_matmul = false;
     static constexpr auto im2col = &oracle_conv2d_im2col_f32;
     static constexpr auto col2im = &oracle_conv2d_col2im_f32;

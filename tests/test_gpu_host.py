@@ -27,6 +27,30 @@ def test_adam_fused_step_equals_the_op_sequence(mx_hip, mx_oracle):
     assert calls_plain > calls_fused + 30 * 2 * 10          # thirteen fewer backend calls per parameter and step
 
 
+def test_fused_mse_and_sgd_leave_the_op_sequences_weights(mx_hip, mx_oracle):
+    """MSELoss and SGD.step as one backend call each (the default on the HIP build) against the op sequences: the same
+    weights, bias and input gradient bit for bit after 25 epochs, losses within the tolerance of a sum; fewer calls."""
+    from host_programs import mlp_run
+    try:
+        mx_hip.set_graph_replay(False)
+        mx_hip.reset_backend_calls()
+        fused = mlp_run(mx_hip, 25, n=3000)
+        calls_fused = mx_hip.backend_calls()
+        mx_hip.set_fused_nn_kernels(False)
+        plain = mlp_run(mx_hip, 25, n=3000)
+        calls_plain = mx_hip.backend_calls() - calls_fused
+    finally:
+        mx_hip.set_fused_nn_kernels(True)
+        mx_hip.set_graph_replay(True)
+    for key in ("weight", "bias", "input_grad"):
+        assert np.array_equal(fused[key], plain[key]), key
+    np.testing.assert_allclose(fused["losses"], plain["losses"], rtol=2e-6)
+    ref = mlp_run(mx_oracle, 25, n=3000)
+    np.testing.assert_allclose(fused["losses"], ref["losses"], rtol=2e-5)
+    np.testing.assert_allclose(fused["weight"], ref["weight"], rtol=2e-4, atol=1e-6)
+    assert calls_plain >= calls_fused + 25 * 8          # the loss: 10 calls -> 2; the two parameter updates: 4 -> 2
+
+
 @pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])
 def test_reference_tensor_cases(mx_hip, case):
     check_case(run_case(mx_hip, case), case)

@@ -1469,6 +1469,63 @@ def test_fused_adam_step_equals_the_fourteen_ops(oracle, hip, n, dt):
         assert not same_bits(pf, p0)          # (a 16-bit parameter near 1 does not move by 0.001)
 
 
+@pytest.mark.parametrize("n", [1, 3, 7, 1000, 10000, 65536, 65540, (1 << 20) + 5, 32 * 64 * 56 * 56])
+def test_fused_mse_loss_equals_the_op_sequence(oracle, hip, n):
+    """losses/mse.rs:21-29 as the ops it is - sub, pow(2), a sum of everything, div_scalar - and their backward
+    (div_scalar, the broadcast, mul_scalar(2), mul, sub's `0 + g` and neg) against hip_mse_loss_f32 and
+    hip_mse_loss_backward_f32: both gradients bit for bit (on the GPU's ops and, where it finishes in a moment, the
+    oracle's), the loss within 1e-5 of the sum of the terms' magnitudes divided by n (f64)."""
+    r = rng(181)
+    pred = r.standard_normal(n).astype(np.float32)
+    target = r.standard_normal(n).astype(np.float32)
+    target[::5] = pred[::5]                                   # exact zeros among the differences (+0 and, negated, -0)
+    g = np.array([0.37], np.float32)                          # the loss's incoming gradient (backward() seeds it with 1)
+    md1, md2 = meta_unary([n], [1]), meta_binary([n], [1], [1])
+    mdb = meta_binary([n], [0], [1])                          # the scalar broadcast over [n]
+
+    def chain(be):
+        diff = be.call("sub_f32", n, 1, md2, In(pred), In(target), Out(n, "f32"))[0]
+        g1 = be.call("div_scalar_f32", 1, 1, meta_unary([1], [1]), In(g), const_arg(float(n), "f32"), Out(1, "f32"))[0]
+        g2 = be.call("mul_scalar_f32", n, 1, meta_unary([n], [0]), In(g1), const_arg(2.0, "f32"), Out(n, "f32"))[0]
+        g3 = be.call("mul_f32", n, 1, md2, In(g2), In(diff), Out(n, "f32"))[0]
+        gp = be.call("sum_to_shape_f32", n, 1, meta_sum_to_shape([n], [1], [n]), In(g3), Out(n, "f32"))[0]
+        neg = be.call("neg_f32", n, 1, md1, In(g3), Out(n, "f32"))[0]
+        gt = be.call("sum_to_shape_f32", n, 1, meta_sum_to_shape([n], [1], [n]), In(neg), Out(n, "f32"))[0]
+        return diff, gp, gt
+    diff, gp, gt = chain(hip)
+    (loss,) = hip.call("mse_loss_f32", n, In(pred), In(target), Out(1, "f32"))
+    fp, ft = hip.call("mse_loss_backward_f32", n, In(pred), In(target), In(g), Out(n, "f32"), Out(n, "f32"))
+    assert same_bits(fp, gp) and same_bits(ft, gt)
+    (fp2,) = hip.call("mse_loss_backward_f32", n, In(pred), In(target), In(g), Out(n, "f32"), None)
+    (ft2,) = hip.call("mse_loss_backward_f32", n, In(pred), In(target), In(g), None, Out(n, "f32"))
+    assert same_bits(fp2, gp) and same_bits(ft2, gt)
+    if n <= (1 << 20) + 5:
+        _, op, ot = chain(oracle)
+        assert same_bits(fp, op) and same_bits(ft, ot)
+    d64 = pred.astype(np.float64) - target.astype(np.float64)
+    want = float((d64 * d64).sum() / n)
+    assert abs(float(loss[0]) - want) <= 1e-5 * want + 1e-30
+    # the unfused loss of the GPU's own ops, for comparison (another order of the same sum)
+    sq = hip.call("square_f32", n, 1, md1, In(diff), Out(n, "f32"))[0]
+    (s,) = hip.call("sum_f32", n, 1, 1, meta_reduce([n], [1], 0), In(sq), Out(1, "f32"))
+    assert abs(float(loss[0]) - float(s[0]) / n) <= 2e-5 * want + 1e-30
+
+
+@pytest.mark.parametrize("n", [1, 3, 1000, 4099, 1 << 16, 64 * 64 * 9])
+def test_fused_sgd_step_equals_mul_scalar_and_sub_inplace(oracle, hip, n):
+    """optimizers/sgd.rs:17-27: param.sub_(grad.mul_scalar(lr)), against one hip_sgd_step_f32 call."""
+    r = rng(182)
+    p0 = r.standard_normal(n).astype(np.float32)
+    g = (r.standard_normal(n) * 10).astype(np.float32)
+    md1, md2 = meta_unary([n], [1]), meta_binary([n], [1], [1])
+    outs = []
+    for be in (oracle, hip):
+        step = be.call("mul_scalar_f32", n, 1, md1, In(g), const_arg(0.01, "f32"), Out(n, "f32"))[0]
+        outs.append(be.call("sub_inplace_f32", n, 1, md2, InOut(p0.copy()), In(step))[0])
+    (fused,) = hip.call("sgd_step_f32", n, InOut(p0.copy()), In(g), const_arg(0.01, "f32"))
+    assert same_bits(outs[0], outs[1]) and same_bits(fused, outs[1]) and not same_bits(fused, p0)
+
+
 @pytest.mark.parametrize("dt", DTS)
 def test_empty_inputs_are_no_ops(hip, dt):
     """Zero elements anywhere: nothing is launched, nothing is written, no error is recorded."""
