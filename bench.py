@@ -820,7 +820,9 @@ def run_mlp(args):
                          {"backend_kernels_per_step": calls, "us_per_step": round(dt_s / steps * 1e6, 1)})
     result["roofline"] = None
     result["note"] = "launch-latency bound (about 200 KB touched per step): no roofline fraction applies"
-    result["config"]["empty_graph_replay_us_by_nodes"] = empty_graph_floor()
+    # (rocprofv3 has crashed inside hipGraphLaunch on this measurement's 900 replays when it follows the training graphs:
+    # the profiles' command skips it)
+    result["config"]["empty_graph_replay_us_by_nodes"] = None if args.no_graph_floor else empty_graph_floor()
     result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_mlp(args)
     return result
 
@@ -1045,6 +1047,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="all")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph-floor", action="store_true", help="mlp: leave out the empty-graph replay measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X; nothing in this backend uses a second GPU (--gpus must be 1)")

@@ -7,6 +7,7 @@
 #include "fuse.hpp"
 #include "fuse_ops.hpp"
 #include "gemm_small.hpp"
+#include "loss.hpp"
 #include "mxh.hpp"
 #include "ops.hpp"
 #include "reduce_row.hpp"
@@ -81,6 +82,7 @@ __device__ __forceinline__ int64_t tail_elem(const FuseCmd& c, int64_t s0, int64
 // the tail writes are fetched from memory all at once when the tail starts (`pre`), so that a stage costs LDS latencies
 // and not a round trip to memory.  Every output is still stored to memory, without anybody waiting for the store.
 constexpr int TAIL_SLOT = 256;
+static_assert(MSE_THREADS == EW_BLOCK, "the fused MSE sum is a stage of the tail with its own work-group's thread count");
 template <int TPR>
 __device__ __forceinline__ void tail_row(uint32_t vec, const RowProgArgs& a, unsigned tid, float* part, float* mirror) {
     if (vec) row_reduce_body<float, float, RSum, TPR, 4, false, 16>((const float*)a.in, (float*)a.out, a.rows, a.L, a.chunks, a.chunk_len, a.div, a.src_bf16, 0, tid, part, mirror);
@@ -137,6 +139,14 @@ __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, ui
             if (tpr == 0) tail_row<1>(vec, a, tid, part, mirror);
             else if (tpr == 1) tail_row<WAVE>(vec, a, tid, part, mirror);
             else tail_row<RB>(vec, a, tid, part, mirror);
+        } else if (t.kind == TAIL_MSE) {
+            const MseArgs a = lds_uniform<MseArgs>(sg.tail[k].arg);
+            const float sum = mse_block_sum(a.pred, a.target, (size_t)a.n, 0, 1, tid, part);
+            if (tid == 0) {
+                const float loss = OpDivScalar<float>{(float)(size_t)a.n}(sum);
+                gl((void*)a.loss)[0] = loss;
+                if (mirror) mirror[0] = loss;
+            }
         } else {
             const GemmArgs g = lds_uniform<GemmArgs>(sg.tail[k].arg);
             const unsigned outputs = g.I * g.J * g.batch;
@@ -236,7 +246,13 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
                         for (int e = 0; e < VEC; ++e) val[j][e] = src[(int64_t)e * s];
                     }
                 }
-                fuse_apply<VEC>(c.op, val[0], val[1], r.v, c.payload);
+                if (c.op == FUSE_OP_MSE_BACKWARD) {
+                    const float scale = mse_grad_scale(gl((const void*)(((uint64_t)c.payload[1] << 32) | c.payload[0]))[0], (float)c.nel);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) r.v[e] = mse_grad(scale, val[0][e], val[1][e]);
+                } else {
+                    fuse_apply<VEC>(c.op, val[0], val[1], r.v, c.payload);
+                }
             }
             staged[k * EW_BLOCK] = r;
             where[k * EW_BLOCK] = (float*)c.out + (ndims == 2 ? (int64_t)c0 * c.os[0] + (int64_t)c1 * c.os[1] : (int64_t)c1 * c.os[0]);

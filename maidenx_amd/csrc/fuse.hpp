@@ -11,12 +11,15 @@
 //     thread then only ever re-reads what it wrote itself, and no ordering between threads is needed;
 //   * a small matmul of the one-thread-per-output kind (a reduction of at most 16 terms) joins as a producer over the
 //     flat space of its outputs; its operands are read across threads, so they may not overlap anything the chain's
-//     earlier members write, nor may a later member write them.
+//     earlier members write, nor may a later member write them;
+//   * the backward pass of the fused MSE loss joins as an elementwise member of two inputs; the one value every thread
+//     reads besides (the gradient of the loss) is held to the rule of a matmul's operands.
 // Serial phase ("tail") - stages run in order by the work-group that finishes the parallel phase last (every group
 // publishes its writes, then draws a ticket; the last ticket continues, the others exit, nobody waits):
 //   * elementwise launches of at most 256 elements (a bias, a 3-element weight, a loss), any shapes, any overlaps;
 //   * a row reduction that one work-group does in the eager path as well ([10000] -> [] sums);
-//   * a matmul with a handful of outputs and a long reduction (the weight gradient of a 3-feature layer).
+//   * a matmul with a handful of outputs and a long reduction (the weight gradient of a 3-feature layer);
+//   * the fused MSE loss of at most 65536 elements (one work-group in the eager path as well).
 //   A stage is the same device code as its eager kernel, so results are the bytes of the separate launches.  A tail
 //   stage may depend on anything before it in stream order.  A parallel member that arrives after tail stages were
 //   queued is hoisted over them when it neither reads what they write nor writes what they read or write.
@@ -34,6 +37,9 @@ namespace mxh {
 constexpr int FUSE_MAX_CMDS = 16;          // members of the parallel phase
 constexpr int FUSE_MAX_TAIL = 12;          // stages of the serial phase
 constexpr uint32_t FUSE_OP_DOT = 0xD07u;   // FuseCmd::op of a matmul producer (the other values index EwProgOps)
+// FuseCmd::op of the fused MSE loss's backward pass (loss.hpp): out = 0 + ((g / nel) * 2) * (in0 - in1), where g is the
+// f32 the payload's 8 bytes point to (read by every thread) and nel the element count
+constexpr uint32_t FUSE_OP_MSE_BACKWARD = 0xB5Eu;
 constexpr int FUSE_TAIL_ARG_BYTES = 112;
 constexpr uint32_t FUSE_TICKETS = 1024;    // ticket slots per device
 
@@ -42,7 +48,7 @@ struct FuseCmd {
     const void* in[2];
     int64_t os[2];            // element strides of the output over the (at most two) collapsed dims
     int64_t is[2][2];         // the same for each input; FUSE_OP_DOT: {output row, reduction} of X, {reduction, output column} of Y
-    uint32_t op;              // position of the functor in EwProgOps, or FUSE_OP_DOT
+    uint32_t op;              // position of the functor in EwProgOps, FUSE_OP_DOT or FUSE_OP_MSE_BACKWARD
     uint32_t nin;
     uint32_t fwd;             // bit j: input j is, element for element, what the previous member wrote (taken from registers)
     uint32_t ndims;           // the member's own space: only read in the tail
@@ -56,7 +62,7 @@ struct FuseCmd {
     uint32_t payload[2];      // the functor's state (a scalar constant), bit for bit
 };
 constexpr uint32_t FUSE_SRC_MEMORY = 0xFFu, FUSE_SRC_MEMORY_LATE = 0xFEu;
-enum TailKind : uint32_t { TAIL_EW = 0, TAIL_ROW_REDUCE = 1, TAIL_DOT = 2 };
+enum TailKind : uint32_t { TAIL_EW = 0, TAIL_ROW_REDUCE = 1, TAIL_DOT = 2, TAIL_MSE = 3 };
 struct TailCmd {
     uint32_t kind;
     uint32_t sub;             // TAIL_ROW_REDUCE: the instantiation number of row_prog_sub(); TAIL_DOT: 1 = the rows form
@@ -65,7 +71,7 @@ struct TailCmd {
     int32_t moff[2];          // TAIL_EW, input from a mirror: element offset of the input's base from that stage's output
     uint32_t mirrored;        // the stage's outputs (at most 256, contiguous) are also kept in LDS for later stages
     uint32_t pad;
-    alignas(8) unsigned char arg[FUSE_TAIL_ARG_BYTES];      // FuseCmd, RowProgArgs or GemmArgs
+    alignas(8) unsigned char arg[FUSE_TAIL_ARG_BYTES];      // FuseCmd, RowProgArgs, GemmArgs or MseArgs
 };
 static_assert(sizeof(FuseCmd) <= FUSE_TAIL_ARG_BYTES, "a tail stage holds an elementwise member");
 struct alignas(16) FuseGroup {
@@ -102,6 +108,9 @@ bool fuse_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims, bool ve
 // `relaunch`: launches the product for real; needed for products a chain refuses (at most 256 outputs, or - chain_ok
 // false - a reduction of more than 16 terms) and a resident step program takes
 bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Extent& y, std::function<void()> relaunch = {}, bool chain_ok = true);
+// the backward pass of the fused MSE loss (c.op = FUSE_OP_MSE_BACKWARD, contiguous operands of c.nel elements):
+// grad_loss is the one f32 every thread reads
+bool fuse_record_mse_backward(const FuseCmd& c, bool vec, size_t nvec, const Extent& grad_loss);
 // a tail stage with its argument block; in[0..nin) / out: the byte ranges it reads and writes (out: `outputs` contiguous
 // f32 values)
 bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs);

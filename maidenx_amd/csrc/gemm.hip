@@ -30,13 +30,6 @@
 #include "gemm_small.hpp"
 #include "mxh.hpp"
 
-#ifndef MXH_GEMM_INTERLEAVE
-#define MXH_GEMM_INTERLEAVE 1
-#endif
-#ifndef MXH_GEMM_TS16
-#define MXH_GEMM_TS16 1
-#endif
-
 namespace mxh {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -390,7 +383,6 @@ template <class T> struct Cfgs {
     using Tall = GemmCfg<2, 2, 1, 1>;     // 64 x 64, four blocks per CU: few output columns or a short reduction (see gemm_dispatch)
     using Flat = GemmCfg<1, 4, 1, 1>;     // 32 x 128: at most 32 output rows
 };
-#if MXH_GEMM_TS16
 template <> struct Cfgs<bf16_t> {
     using Big = GemmCfg<4, 2, 4, 8, 16>;
     using Small = GemmCfg<2, 2, 4, 4, 16>;
@@ -398,7 +390,6 @@ template <> struct Cfgs<bf16_t> {
     using Flat = Tall;                        // (a 32-row tile is too small for the turned 16-bit stager's row pairs)
 };
 template <> struct Cfgs<f16_t> : Cfgs<bf16_t> {};
-#endif
 
 // swapped operands: accumulator element e of tile (a, c) is output row i0 + .. + lane%32 and output
 // column j0 + .. + 8*(e/4) + 4*(lane/32) + e%4  → four consecutive columns per group of 4 elements
@@ -638,7 +629,6 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
             }
             // keep the memory operations of the next stage ahead of this step's MFMAs: the matrix
             // pipe then works through them while LDS and the vector memory unit serve the next step
-#if MXH_GEMM_INTERLEAVE
             mfmas(s);
 #pragma unroll
             for (int i = 0; i < MI * MJH; ++i) {
@@ -648,11 +638,6 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
             }
             __builtin_amdgcn_sched_barrier(0);
-#else
-            __builtin_amdgcn_sched_barrier(0);
-            mfmas(s);
-            __builtin_amdgcn_sched_barrier(0);
-#endif
         }
         if constexpr (PANEL) {
             if ((kt + 1) % nk1 == 0) {       // the last k-tile of an output tile: out it goes, and the accumulators start over

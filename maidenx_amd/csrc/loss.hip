@@ -14,62 +14,26 @@
 // of n terms: like every sum of this library it is added in a fixed tree of its own, within the f32 tolerance of a
 // reduction of the op sequence's sum (which the reference adds in an order that changes from run to run).
 // Contiguous f32 tensors of one shape; anything else stays with the separate ops.
+// Inside a capture, at launch-bound sizes, the three join the fused chains (fuse.hpp): the step as an elementwise
+// launch (OpSgdStep), the one-block loss as a stage of the serial phase, the backward pass as a member of the parallel one.
 #include "elementwise.hpp"
+#include "fuse.hpp"
+#include "loss.hpp"
 #include "mxh.hpp"
 #include "ops.hpp"
 #include "reduce_row.hpp"
 
 namespace mxh {
 
-constexpr int LB = 256;
+constexpr int LB = MSE_THREADS;
 static inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 constexpr unsigned MSE_MAX_BLOCKS = 1024;
 
-// one block's share of the squared differences, folded to one value in thread 0
-__device__ __forceinline__ float mse_block_sum(const float* __restrict__ pred, const float* __restrict__ target, size_t n, unsigned blocks, float* part) {
-    typedef float F4 __attribute__((ext_vector_type(4)));
-    const size_t nvec = n / 4;
-    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const size_t stride = (size_t)blocks * LB;
-    size_t v = (size_t)blockIdx.x * LB + threadIdx.x;
-    for (; v + 3 * stride < nvec; v += 4 * stride) {      // four pairs of loads in flight
-        F4 p[4], t[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            p[k] = ((const F4*)pred)[v + k * stride];
-            t[k] = ((const F4*)target)[v + k * stride];
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) a[e] = a[e] + OpSquare<float>{}(OpSub<float>{}(p[k][e], t[k][e]));
-    }
-    for (; v < nvec; v += stride) {
-        const F4 p = ((const F4*)pred)[v], t = ((const F4*)target)[v];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) a[e] = a[e] + OpSquare<float>{}(OpSub<float>{}(p[e], t[e]));
-    }
-    float acc = (a[0] + a[1]) + (a[2] + a[3]);
-    if (blockIdx.x == 0 && threadIdx.x < n % 4) {          // the last n % 4 elements
-        const size_t i = nvec * 4 + threadIdx.x;
-        acc = acc + OpSquare<float>{}(OpSub<float>{}(pred[i], target[i]));
-    }
-    acc = wave_reduce<RSum>(acc);
-    if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = acc;
-    __syncthreads();
-    float sum = 0.0f;
-    if (threadIdx.x == 0) {
-        sum = part[0];
-#pragma unroll
-        for (int w = 1; w < LB / WAVE; ++w) sum = sum + part[w];
-    }
-    return sum;
-}
 // blocks == 1: the loss itself; more: one partial per block
 __global__ __launch_bounds__(LB) void mse_sum_kernel(const float* __restrict__ pred, const float* __restrict__ target, size_t n, unsigned blocks,
                                                      float* __restrict__ out, float count) {
     __shared__ float part[LB / WAVE];
-    const float sum = mse_block_sum(pred, target, n, blocks, part);
+    const float sum = mse_block_sum(pred, target, n, blockIdx.x, blocks, threadIdx.x, part);
     if (threadIdx.x == 0) out[blockIdx.x] = blocks == 1 ? OpDivScalar<float>{count}(sum) : sum;
 }
 // the blocks' partials in block order, then the division
@@ -95,28 +59,16 @@ __global__ __launch_bounds__(LB) void mse_backward_kernel(size_t nunits, const f
     const size_t i = (size_t)blockIdx.x * LB + threadIdx.x;
     if (i >= nunits) return;
     // the scalar chain of the op sequence: div_scalar's backward, then pow's mul_scalar(2)
-    const float scale = OpMulScalar<float>{2.0f}(OpDivScalar<float>{count}(grad_loss[0]));
+    const float scale = mse_grad_scale(grad_loss[0], count);
     const AVec<float, VEC> p = ((const AVec<float, VEC>*)pred)[i], t = ((const AVec<float, VEC>*)target)[i];
     AVec<float, VEC> gp, gt;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-        const float u = OpMul<float>{}(scale, OpSub<float>{}(p.v[e], t.v[e]));
-        gp.v[e] = 0.0f + u;
-        if (WITH_TARGET) gt.v[e] = 0.0f + OpNeg<float>{}(u);
+        gp.v[e] = mse_grad(scale, p.v[e], t.v[e]);
+        if (WITH_TARGET) gt.v[e] = 0.0f + OpNeg<float>{}(OpMul<float>{}(scale, OpSub<float>{}(p.v[e], t.v[e])));
     }
     if (grad_pred) ((AVec<float, VEC>*)grad_pred)[i] = gp;
     if (WITH_TARGET) ((AVec<float, VEC>*)grad_target)[i] = gt;
-}
-
-template <int VEC>
-__global__ __launch_bounds__(LB) void sgd_step_kernel(size_t nunits, float* __restrict__ param, const float* __restrict__ grad, float lr) {
-    const size_t i = (size_t)blockIdx.x * LB + threadIdx.x;
-    if (i >= nunits) return;
-    AVec<float, VEC> p = ((const AVec<float, VEC>*)param)[i];
-    const AVec<float, VEC> g = ((const AVec<float, VEC>*)grad)[i];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) p.v[e] = OpSub<float>{}(p.v[e], OpMulScalar<float>{lr}(g.v[e]));
-    ((AVec<float, VEC>*)param)[i] = p;
 }
 
 }  // namespace mxh
@@ -132,6 +84,12 @@ extern "C" void hip_mse_loss_f32(size_t n, const float* pred, const float* targe
     unsigned blocks = 1;
     if (n > 65536) blocks = (unsigned)std::min<size_t>(MSE_MAX_BLOCKS, cdiv(n, (size_t)4096));
     if (blocks == 1) {
+        if (capture_open()) {       // a stage of the open chain's serial phase: the same device function, run by one work-group of 256
+            const MseArgs a{pred, target, loss, (uint64_t)n};
+            const Extent in[2] = {{(uintptr_t)pred, (uintptr_t)(pred + n)}, {(uintptr_t)target, (uintptr_t)(target + n)}};
+            const Extent out{(uintptr_t)loss, (uintptr_t)(loss + 1)};
+            if (fuse_record_tail(TAIL_MSE, 0, &a, sizeof(a), in, 2, out, 1)) return;
+        }
         hipLaunchKernelGGL(mse_sum_kernel, dim3(1), dim3(LB), 0, stream(), pred, target, n, 1u, loss, (float)n);
         MXH_LAUNCH_CHECK("mse_sum");
         return;
@@ -152,6 +110,21 @@ extern "C" void hip_mse_loss_backward_f32(size_t n, const float* pred, const flo
     const size_t units = vec ? n / 4 : n;
     const dim3 grid((unsigned)cdiv(units, (size_t)LB));
     if (units >= (1ull << 31) * LB) { set_status(ERR_TOO_LARGE, "mse_loss_backward: too many elements"); return; }
+    if (capture_open() && grad_pred && !grad_target && n > 256 && units < (size_t)EW_SMALL_BLOCKS * EW_BLOCK * EW_UNR) {
+        // launch-bound sizes inside a capture: a member of the open chain's parallel phase (two inputs walked element for
+        // element like any elementwise member, and the loss's gradient read by every thread)
+        FuseCmd c;
+        std::memset((void*)&c, 0, sizeof(c));
+        c.out = grad_pred;
+        c.in[0] = pred;
+        c.in[1] = target;
+        c.os[0] = c.is[0][0] = c.is[1][0] = 1;
+        c.op = FUSE_OP_MSE_BACKWARD;
+        c.nin = 2;
+        c.nel = (uint32_t)n;
+        std::memcpy(c.payload, (const void*)&grad_loss, sizeof(grad_loss));
+        if (fuse_record_mse_backward(c, vec, units, Extent{(uintptr_t)grad_loss, (uintptr_t)(grad_loss + 1)})) return;
+    }
     if (vec) {
         if (grad_target) hipLaunchKernelGGL((mse_backward_kernel<4, true>), grid, dim3(LB), 0, stream(), units, pred, target, grad_loss, grad_pred, grad_target, (float)n);
         else hipLaunchKernelGGL((mse_backward_kernel<4, false>), grid, dim3(LB), 0, stream(), units, pred, target, grad_loss, grad_pred, grad_target, (float)n);
@@ -165,11 +138,9 @@ extern "C" void hip_mse_loss_backward_f32(size_t n, const float* pred, const flo
 extern "C" void hip_sgd_step_f32(size_t n, float* param, const float* grad, float lr) { MXH_API;
     if (!param || !grad) { set_status(ERR_INVALID, "sgd_step: null buffer"); return; }
     if (n == 0) return;
-    const bool vec = n % 4 == 0 && aligned16(param) && aligned16(grad);
-    const size_t units = vec ? n / 4 : n;
-    if (units >= (1ull << 31) * LB) { set_status(ERR_TOO_LARGE, "sgd_step: too many elements"); return; }
-    const dim3 grid((unsigned)cdiv(units, (size_t)LB));
-    if (vec) hipLaunchKernelGGL(sgd_step_kernel<4>, grid, dim3(LB), 0, stream(), units, param, grad, lr);
-    else hipLaunchKernelGGL(sgd_step_kernel<1>, grid, dim3(LB), 0, stream(), units, param, grad, lr);
-    MXH_LAUNCH_CHECK("sgd_step");
+    // an elementwise launch of two inputs, written over the first: inside a capture it joins the fused chains like any other
+    const size_t dims = n, unit = 1;
+    const size_t* ins[2] = {&unit, &unit};
+    const void* inp[2] = {param, grad};
+    ew_launch<OpSgdStep<float>>(n, 1, &dims, &unit, ins, param, inp, OpSgdStep<float>{lr});
 }

@@ -213,6 +213,14 @@ template <class T> struct OpLogicalNot {
     __device__ bool_t operator()(T x) const { return (bool_t)is_zero(x); }
 };
 
+// SGD's update as one function of (parameter, gradient): p - g * lr, the product rounded before the difference is
+// taken - mul_scalar, then sub (crates/maidenx_nn/src/optimizers/sgd.rs:17-27)
+template <class T> struct OpSgdStep {
+    using In = T; using Out = T; static constexpr int NIN = 2;
+    T lr;
+    __device__ T operator()(T p, T g) const { using A = Ar<T>; return A::sub(p, A::mul(g, lr)); }
+};
+
 // ---- unary with a constant of the input dtype --------------------------------------------------
 #define MXH_UNC(NAME, OUT, EXPR)                                          \
     template <class T> struct NAME {                                      \

@@ -82,6 +82,7 @@ ApiGuard::~ApiGuard() { g_api_mu.unlock(); }
 struct ParMember {
     Extent out, in[2];
     bool across[2];           // input j is read across threads (a matmul operand): it can never be "the same mapping"
+    Extent extra{0, 0};       // one more range read across threads (the scalar of FUSE_OP_MSE_BACKWARD); empty: none
 };
 struct TailStage {
     Extent out, in[2];
@@ -143,6 +144,7 @@ static bool clear_of_tail(const ParMember& m, uint32_t nin) {
             if (m.out.overlaps(t.in[j])) return false;
         for (uint32_t j = 0; j < nin; ++j)
             if (m.in[j].overlaps(t.out)) return false;
+        if (m.extra.overlaps(t.out)) return false;
     }
     return true;
 }
@@ -160,6 +162,8 @@ static bool clear_of_members(const FuseCmd& c, const ParMember& m, uint32_t ndim
         // write after read
         for (uint32_t j = 0; j < e.nin; ++j)
             if (m.out.overlaps(pe.in[j]) && (pe.across[j] || !same_mapping(c.out, c.os, e.in[j], e.is[j], ndims))) return false;
+        // the range every thread reads: nothing of the chain may write it, before or after
+        if (m.extra.overlaps(pe.out) || m.out.overlaps(pe.extra)) return false;
     }
     return true;
 }
@@ -186,6 +190,7 @@ static void add_member(const FuseCmd& c, const ParMember& m, uint32_t ndims, con
     slot.fwd = 0;
     slot.src = FUSE_SRC_MEMORY | (FUSE_SRC_MEMORY << 8);
     if (c.op != FUSE_OP_DOT) {
+        // (FUSE_OP_MSE_BACKWARD included: its two inputs are an elementwise member's)
         // An input that is an earlier member's output (element for element: nothing else was let in) is not in memory yet:
         // the members' stores wait until all of them are done.  It comes from the latest such member's staged output,
         // or straight from registers when that is the member before.
@@ -325,6 +330,21 @@ static bool chain_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, 
     return true;
 }
 
+static bool chain_record_mse_backward(const FuseCmd& c, bool vec, size_t nvec, const Extent& grad_loss) {
+    if (!fuse_accepting() || c.nel <= 256) return false;
+    ParMember m;
+    const uint32_t dims[1] = {c.nel};
+    m.out = operand_range(c.out, c.os, 1, dims, sizeof(float));
+    for (uint32_t j = 0; j < 2; ++j) {
+        m.in[j] = operand_range(c.in[j], c.is[j], 1, dims, sizeof(float));
+        m.across[j] = false;
+    }
+    m.extra = grad_loss;
+    if (m.extra.overlaps(m.out)) return false;
+    add_member(c, m, 1, dims, vec, nvec, sizeof(float));
+    return true;
+}
+
 // ---- the capture as a resident step program: the launch sites' offers are kept, not launched ---------------------
 static bool res_accepting() { return g_res_ok && !g_res_spilling && fuse_accepting(); }
 
@@ -429,6 +449,11 @@ bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_b
         res_spill();
     }
     return chain_record_tail(kind, sub, arg, arg_bytes, in, nin, out, outputs);
+}
+
+bool fuse_record_mse_backward(const FuseCmd& c, bool vec, size_t nvec, const Extent& grad_loss) {
+    if (res_accepting()) res_spill();      // (a resident step program has no command for it)
+    return chain_record_mse_backward(c, vec, nvec, grad_loss);
 }
 
 void prog_abandon() {

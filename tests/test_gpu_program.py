@@ -394,6 +394,58 @@ def test_chain_with_matmuls_reductions_and_a_serial_tail(lib, n, feats):
         assert launches == 15 and nodes <= 3, (launches, nodes)
 
 
+def fused_nn_step(lib, seq, n, feats, r):
+    """The step of linear_step() with the loss, its backward pass and the parameter updates as the fused calls."""
+    x, y = seq.dev(r.standard_normal((n, feats)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    w0, b0 = r.standard_normal(feats).astype(np.float32), r.standard_normal(1).astype(np.float32)
+    w, b = seq.out(feats * 4, "f4"), seq.out(4, "f4")          # updated in place: restored at the start of every run
+    w_init, b_init = seq.dev(w0), seq.dev(b0)
+    pred, pb, gpred = (seq.out(n * 4, "f4") for _ in range(3))
+    loss, gloss, gw, gb = seq.out(4, "f4"), seq.out(4, "f4"), seq.out(feats * 4, "f4"), seq.out(4, "f4")
+    seq.add("add_scalar_f32", feats, 1, u64([feats], [1], 0), w_init.ptr, C.c_float(0.0), w.ptr)
+    seq.add("add_scalar_f32", 1, 1, u64([1], [1], 0), b_init.ptr, C.c_float(0.0), b.ptr)
+    seq.add("matmul_f32", n, u64(2, 2, 2, [n, 1], [n, feats], [feats, 1], [feats, 1], [1, feats], 0, 0), x.ptr, w.ptr, pred.ptr)
+    seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), pred.ptr, b.ptr, pb.ptr)
+    seq.add("mse_loss_f32", n, pb.ptr, y.ptr, loss.ptr)
+    seq.add("fill_f32", 1, gloss.ptr, C.c_float(1.0))
+    seq.add("mse_loss_backward_f32", n, pb.ptr, y.ptr, gloss.ptr, gpred.ptr, None)
+    seq.add("matmul_f32", feats, u64(2, 2, 2, [feats, 1], [feats, n], [n, 1], [1, feats], [1, 1], 0, 0), x.ptr, gpred.ptr, gw.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), gpred.ptr, gb.ptr)
+    seq.add("sgd_step_f32", feats, w.ptr, gw.ptr, C.c_float(0.01))
+    seq.add("sgd_step_f32", 1, b.ptr, gb.ptr, C.c_float(0.01))
+
+
+@pytest.mark.parametrize("n,feats", [(10000, 3), (4096, 4), (5001, 1), (65536, 2), (300, 3), (7, 2)])
+def test_fused_loss_and_sgd_calls_join_the_chains(lib, n, feats):
+    """hip_mse_loss_f32 (a stage of the serial phase), hip_mse_loss_backward_f32 (a member of the parallel phase whose
+    scalar operand the stage before wrote: a new chain) and hip_sgd_step_f32 (an elementwise launch in place) inside a
+    capture: every launch is taken by a chain and the replays are the eager bytes."""
+    r = np.random.default_rng(300 + n + feats)
+    seq = Seq(lib)
+    fused_nn_step(lib, seq, n, feats, r)
+    launches, nodes = fused(lib, seq, replays=3)
+    if 4096 <= n <= 16384:           # (beyond that the weight gradient is a launch of its own: 1024 threads)
+        assert launches == 11 and nodes <= 3, (launches, nodes)
+
+
+def test_fused_loss_backward_waits_for_a_gradient_written_in_the_same_chain(lib):
+    """The loss's gradient is read by every thread of the backward member: when an earlier member of the same space
+    writes it (here: the buffer is a slice of a tensor the chain fills), the member must open a new chain; and a member
+    that would overwrite it afterwards must not join either."""
+    n = 4096
+    r = np.random.default_rng(8)
+    seq = Seq(lib)
+    p, t = seq.dev(r.standard_normal(n).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    g, gp, gp2 = seq.out(n * 4, "f4"), seq.out(n * 4, "f4"), seq.out(n * 4, "f4")
+    md1 = u64([n], [1], 0)
+    seq.add("add_scalar_f32", n, 1, md1, p.ptr, C.c_float(1.5), g.ptr)                     # writes g[0..n): g[5] is the "loss gradient"
+    seq.add("mse_loss_backward_f32", n, p.ptr, t.ptr, g.ptr + 20, gp.ptr, None)
+    seq.add("mul_scalar_f32", n, 1, md1, t.ptr, C.c_float(3.0), g.ptr)                     # overwrites it
+    seq.add("mse_loss_backward_f32", n, p.ptr, t.ptr, g.ptr + 20, gp2.ptr, None)
+    launches, nodes = fused(lib, seq, replays=3)
+    assert launches == 4 and nodes == 4, (launches, nodes)
+
+
 def test_chain_member_is_hoisted_over_tail_stages_only_when_independent(lib):
     """A member of the parallel phase that arrives after tail stages runs before them in the kernel: it is let in when it
     touches nothing they write and writes nothing they read, and opens a new chain otherwise."""
