@@ -886,6 +886,8 @@ def run_conv(args):
     from maidenx_amd.tensor import host
     mx = host()
     conv, x, target = _conv_setup(mx, 32)
+    # (50 steps at least: the figure settles after about 20)
+    args = argparse.Namespace(**{**vars(args), "steps": max(args.steps, 50)})
     for _ in range(max(args.warmup, 2)):
         _conv_step(mx, conv, x, target)
     mx.synchronize()

@@ -115,6 +115,14 @@ int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_
  * epoch eager; mxt_last_train_replayed() tells how many epochs of the last mxt_train call were replays. */
 void mxt_set_graph_replay(int enabled);
 size_t mxt_last_train_replayed(void);
+/* The same for any step: calls fn(user, e) for e = 0 .. steps-1 (a non-zero return ends the loop with an error), or - on
+ * the HIP build, from 32 steps on - runs it eagerly until the buffer addresses of a step repeat, records some more steps as
+ * a graph and replays that for the rest; mxt_last_train_replayed() counts the replays.  The step must issue the same
+ * tensor calls every time, must not read values back from the device, and hands results on only through tensors it
+ * updates (parameters, gradients): tensors it creates are gone when it returns.  No counterpart in the reference, whose
+ * loops are written in the caller's Rust. */
+typedef int (*mxt_step_fn)(void* user, size_t step);
+int mxt_run_steps(mxt_step_fn fn, void* user, size_t steps);
 /* sum_all() (crates/maidenx_tensor/src/ops/reduction.rs:76-83) sums one dim after the other.  By default a contiguous f32
  * tensor is summed by one sum_to_shape call to [1, .., 1] instead: the gradients are the same bytes, the sum is added
  * up in another order (both within the f32 tolerance of a reduction).  enabled = 0: dim by dim. */

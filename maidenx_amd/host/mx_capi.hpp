@@ -255,6 +255,14 @@ int mxt_adam_step(void* opt, mxt_module m) { return guard_i([&] { ((mxt::Adam<B>
 int mxt_train(mxt_module m, mxt_tensor input, mxt_tensor target, float lr, size_t epochs, float* losses) {
     return guard_i([&] { g_replayed = mxt::train_loop<B>(*(Module*)m, ref(input), ref(target), lr, epochs, losses, g_graphs); });
 }
+int mxt_run_steps(mxt_step_fn fn, void* user, size_t steps) {
+    return guard_i([&] {
+        if (!fn) throw mxt::Error(mxt::ErrKind::InvalidArgument, "run_steps: no step function");
+        g_replayed = mxt::run_steps<B>([&](size_t e) {
+            if (fn(user, e) != 0) throw mxt::Error(mxt::ErrKind::InvalidOperation, "run_steps: the step function reported a failure");
+        }, steps, g_graphs);
+    });
+}
 void mxt_set_graph_replay(int enabled) { g_graphs = enabled != 0; }
 size_t mxt_last_train_replayed(void) { return g_replayed; }
 void mxt_set_sum_all_in_one_pass(int enabled) { mxt::sum_all_in_one_pass() = enabled != 0; }

@@ -231,7 +231,8 @@ template <class B> struct GradCell {
 inline size_t& backend_calls() { static size_t n = 0; return n; }
 // Conv2d backward: make only the rows of grad_cols that col2im reads (see Conv2d); false = the whole product.
 inline bool& conv_skip_unread_grad_cols() { static bool on = true; return on; }
-// sum_all() of a contiguous f32 tensor as one reduction (true) or dim by dim as the reference does (false).
+// sum_all() of a contiguous f32 tensor, and the bias gradient of Conv2d (sums over W, H and the batch), as one reduction
+// (true) or dim by dim as the reference does (false).
 inline bool& sum_all_in_one_pass() { static bool on = true; return on; }
 // Conv2d on a backend that has the product with the gathered column matrix (the matrix is never stored): 0 = store
 // the matrix with im2col and multiply that, as the reference does; 1 = gather when no backward is recorded (the
@@ -1274,8 +1275,13 @@ struct Conv2d {                                                                 
                 }
                 if (in.size() > 2) {
                     const T& b = in[2];
-                    if (b.requires_grad) grads.push_back(go.sum(3, false).sum(2, false).sum(0, false));
-                    else grads.push_back(T::zeros_like(b));
+                    // conv.rs:287-291 sums the gradient over W, H and the batch, one launch and one intermediate each; a
+                    // contiguous f32 gradient is summed to [1, Cout, 1, 1] in one sum_to_shape call instead (the sums are
+                    // added up in another order, within the f32 tolerance of a reduction either way)
+                    if (!b.requires_grad) grads.push_back(T::zeros_like(b));
+                    else if (sum_all_in_one_pass() && go.dtype == DType::F32 && go.is_contiguous() && go.offset() == 0 && go.size() > 0)
+                        grads.push_back(go.sum_to_shape(Shape{1, go.shape()[1], 1, 1}).reshape(Shape{go.shape()[1]}));
+                    else grads.push_back(go.sum(3, false).sum(2, false).sum(0, false));
                 }
                 return grads;
             });
@@ -1408,30 +1414,22 @@ struct Adam {
     }
 };
 
-// ---- the training loop of examples/device/cpu.rs:32-38 -----------------------------------------------
-// forward, loss, backward, optimizer step, zero_grad.  `losses` (may be null) receives every epoch's loss, which
-// costs a device-to-host copy per epoch.
+// ---- a step, many times -------------------------------------------------------------------------------
+// Calls step(e) for e = 0 .. epochs-1, or does the same work by replaying a recording of it.
 //
-// When the backend can record graphs and no loss is read back, the loop is launch-bound (tens of small kernels per
-// step), so it is recorded once and replayed: the pool hands out the same blocks in the same order every `period`
-// steps once it is warm (a step's allocations and releases are a fixed sequence), which makes the recorded pointers
-// valid for every replay and leaves the host-side tensors pointing at the right blocks afterwards.  The period is
-// measured, not assumed; without one the loop stays eager.
-template <class B, class Model>
-size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr, size_t epochs, float* losses, bool allow_graph) {
-    SGD<B> opt(lr);
-    auto step = [&](size_t e) {
-        Tensor<B> pred = model.forward(x);
-        Tensor<B> loss = mse_loss<B>(pred, y);
-        loss.backward();
-        opt.step(model.parameters());
-        opt.zero_grad(model.parameters());
-        if (losses) losses[e] = loss.item();
-    };
+// A step on small tensors is launch-bound (tens of small kernels), so when the backend can record graphs it is recorded
+// once and replayed: the pool hands out the same blocks in the same order every `period` steps once it is warm (a
+// step's allocations and releases are a fixed sequence), which makes the recorded pointers valid for every replay and
+// leaves the host-side tensors pointing at the right blocks afterwards.  The period is measured, not assumed; without
+// one the loop stays eager.  The step must do the same backend work every time it is called (no value read back from
+// the device may steer it) and may not keep tensors it creates from one call to the next, other than through the
+// tensors it updates (parameters, gradients).  Returns the number of steps that were replays.
+template <class B, class Step>
+size_t run_steps(Step&& step, size_t epochs, bool allow_graph) {
     size_t done = 0, replayed = 0;
     if constexpr (B::has_graphs) {
         constexpr size_t kMinWarm = 8, kMaxWarm = 64, kMaxPeriod = 4;   // the README loop settles into period 3 after 5 steps
-        if (allow_graph && !losses && epochs >= 4 * kMinWarm) {
+        if (allow_graph && epochs >= 4 * kMinWarm) {
             Pool<B>& pool = Pool<B>::instance();
             std::vector<std::vector<void*>> traces;
             size_t period = 0;
@@ -1479,7 +1477,7 @@ size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr
                     for (size_t k = 0; k < span && periodic; ++k) periodic = recorded[k] == traces[warm - one + k % one];
                     if (pool.device_allocs != allocs_before) {
                         B::graph_destroy(exec);
-                        throw Error(ErrKind::Backend, "training loop allocated device memory while it was being recorded");
+                        throw Error(ErrKind::Backend, "the step allocated device memory while it was being recorded");
                     }
                     // the recorded steps did not run yet: replay them, then as many more whole spans as fit
                     const size_t calls_per_span = backend_calls() - calls_before;
@@ -1502,6 +1500,23 @@ size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr
     }
     for (; done < epochs; ++done) step(done);
     return replayed;
+}
+
+// ---- the training loop of examples/device/cpu.rs:32-38 -----------------------------------------------
+// forward, loss, backward, optimizer step, zero_grad.  `losses` (may be null) receives every epoch's loss, which
+// costs a device-to-host copy per epoch (and keeps the loop eager: see run_steps).
+template <class B, class Model>
+size_t train_loop(Model& model, const Tensor<B>& x, const Tensor<B>& y, float lr, size_t epochs, float* losses, bool allow_graph) {
+    SGD<B> opt(lr);
+    auto step = [&](size_t e) {
+        Tensor<B> pred = model.forward(x);
+        Tensor<B> loss = mse_loss<B>(pred, y);
+        loss.backward();
+        opt.step(model.parameters());
+        opt.zero_grad(model.parameters());
+        if (losses) losses[e] = loss.item();
+    };
+    return run_steps<B>(step, epochs, allow_graph && !losses);
 }
 
 }  // namespace mxt

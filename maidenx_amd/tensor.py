@@ -22,6 +22,9 @@ _KINDS = ["None", "InvalidShape", "ShapeMismatch", "DimensionOutOfBounds", "Inco
           "InvalidArgument", "UnsupportedDType", "OutOfMemory", "Backend"]
 
 
+STEP_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_size_t)      # mxt_step_fn
+
+
 class MxError(RuntimeError):
     def __init__(self, kind, text):
         super().__init__(f"{kind}: {text}")
@@ -43,7 +46,7 @@ def _bind(lib):
         "mxt_conv2d_new": ([P, P, SZ, SZ, SZ, SZ, SZ, SZ], P), "mxt_module_forward": ([P, P], P), "mxt_module_weight": ([P], P),
         "mxt_module_bias": ([P], P), "mxt_module_release": ([P], None), "mxt_mse_loss": ([P, P], P), "mxt_sgd_step": ([P, F], I),
         "mxt_sgd_zero_grad": ([P], I), "mxt_train": ([P, P, P, F, SZ, P], I), "mxt_set_graph_replay": ([I], None),
-        "mxt_last_train_replayed": ([], SZ), "mxt_set_conv_skip_unread_grad_cols": ([I], None), "mxt_set_autograd_shortcuts": ([I], None), "mxt_set_fused_nn_kernels": ([I], None), "mxt_set_sum_all_in_one_pass": ([I], None), "mxt_set_conv_gathered_products": ([I], None),
+        "mxt_last_train_replayed": ([], SZ), "mxt_run_steps": ([P, P, SZ], I), "mxt_set_conv_skip_unread_grad_cols": ([I], None), "mxt_set_autograd_shortcuts": ([I], None), "mxt_set_fused_nn_kernels": ([I], None), "mxt_set_sum_all_in_one_pass": ([I], None), "mxt_set_conv_gathered_products": ([I], None),
         "mxt_adam_new": ([C.c_double] * 4, P), "mxt_adam_release": ([P], None), "mxt_adam_set_fused": ([P, I], None), "mxt_adam_step": ([P, P], I),
         "mxt_backend_calls": ([], SZ), "mxt_reset_backend_calls": ([], None), "mxt_device_allocations": ([], SZ), "mxt_synchronize": ([], I),
     }
@@ -127,6 +130,26 @@ class Host:
         losses = np.zeros(epochs, np.float32) if record_losses else None
         self._rc(self.lib.mxt_train(module.h, x.h, y.h, lr, epochs, losses.ctypes.data if record_losses else None))
         return losses
+
+    def run_steps(self, step, n):
+        """Runs step() n times, or - on the HIP build, from 32 steps on, once the buffer addresses of a step repeat - records
+        it as a graph and replays that.  step() must issue the same tensor calls every time, read nothing back from the
+        device and keep none of the tensors it creates; what it updates (parameters, gradients) is as after n calls."""
+        failure = []
+
+        def call(_user, _e):
+            try:
+                step()
+                return 0
+            except BaseException as ex:      # (must not travel through the native frames)
+                failure.append(ex)
+                return 1
+
+        fn = STEP_FN(call)
+        rc = self.lib.mxt_run_steps(C.cast(fn, C.c_void_p), None, n)
+        if failure:
+            raise failure[0]
+        self._rc(rc)
 
     def set_graph_replay(self, enabled):
         self.lib.mxt_set_graph_replay(int(enabled))

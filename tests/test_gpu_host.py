@@ -158,8 +158,11 @@ def test_sum_all_in_one_pass_or_dim_by_dim(mx_hip):
     finally:
         mx.set_sum_all_in_one_pass(True)
     assert res[True]["calls"] < res[False]["calls"]
-    for key in ("g", "grad_x", "grad_w", "grad_b", "out"):
+    for key in ("g", "grad_x", "grad_w", "out"):
         np.testing.assert_array_equal(res[True][key].view(np.uint32), res[False][key].view(np.uint32), err_msg=key)
+    # the bias gradient of Conv2d is itself a sum over W, H and the batch (conv.rs:287-291): one pass or three
+    scale = np.abs(res[False]["grad_b"]).max()
+    assert np.abs(res[True]["grad_b"] - res[False]["grad_b"]).max() <= 1e-5 * scale
     exact = float(np.sum(a.astype(np.float64) ** 2))
     for one_pass in (False, True):
         assert abs(float(res[one_pass]["z"]) - exact) <= 1e-5 * exact
@@ -303,6 +306,64 @@ def test_graph_replayed_training_equals_eager(mx_hip):
             np.testing.assert_array_equal(t.grad().numpy(), 2 * np.arange(12, dtype=np.float32).reshape(3, 4))
     finally:
         mx.set_graph_replay(True)
+
+
+def test_run_steps_replays_a_conv_step_and_equals_the_eager_loop(mx_hip):
+    """mxt_run_steps with a step written by the caller (Conv2d forward, MSE, backward, zero_grad of the layer, the
+    input's gradient accumulating from step to step): eager until the addresses repeat, then replays of a recorded
+    graph; the accumulated input gradient is the eager loop's, bit for bit."""
+    mx = mx_hip
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((4, 8, 12, 12), dtype=np.float32)
+    w = rng.uniform(-0.2, 0.2, (6, 8, 3, 3)).astype(np.float32)
+    b = rng.uniform(-0.2, 0.2, (6,)).astype(np.float32)
+    t = rng.standard_normal((4, 6, 12, 12), dtype=np.float32)
+
+    def run(steps, graphs):
+        mx.set_graph_replay(graphs)
+        conv = mx.Conv2d(mx.tensor(w), mx.tensor(b), stride=(1, 1), padding=(1, 1))
+        xin, target = mx.tensor(x).with_grad(), mx.tensor(t)
+
+        def step():
+            loss = mx.mse_loss(conv.forward(xin), target)
+            loss.backward()
+            conv.zero_grad()
+        mx.run_steps(step, steps)
+        mx.synchronize()
+        return xin.grad().numpy(), mx.last_train_replayed()
+    try:
+        for steps in (40, 57):
+            g0, r0 = run(steps, False)
+            assert r0 == 0
+            g1, r1 = run(steps, True)
+            assert r1 >= steps // 2 - 4, "the loop fell back to eager launches"
+            np.testing.assert_array_equal(g0.view(np.uint32), g1.view(np.uint32))
+        # few steps: eager
+        g2, r2 = run(5, True)
+        assert r2 == 0
+    finally:
+        mx.set_graph_replay(True)
+
+
+def test_run_steps_hands_on_a_failure_of_the_step(mx_hip):
+    """An exception inside the step ends the loop (and an open recording) and reaches the caller as it was raised; the
+    library works on afterwards."""
+    mx = mx_hip
+    a = mx.tensor(np.ones((3, 4), np.float32)).with_grad()
+    calls = []
+
+    def step():
+        calls.append(1)
+        if len(calls) == 20:
+            raise KeyError("step 20")
+        a.mul(a).sum_all().backward()
+    with pytest.raises(KeyError):
+        mx.run_steps(step, 64)
+    assert len(calls) == 20
+    mx.synchronize()
+    a2 = mx.tensor(np.full((3, 4), 2.0, np.float32)).with_grad()
+    a2.mul(a2).sum_all().backward()
+    np.testing.assert_array_equal(a2.grad().numpy(), np.full((3, 4), 4.0, np.float32))
 
 
 @pytest.mark.parametrize("case", TKAT, ids=[f"{c['program'][0][1]}@{c['cite'].split('/')[-1]}" for c in TKAT])

@@ -85,6 +85,25 @@ def test_mlp_training_matches_gradient_descent(mx_oracle):
     assert mx_oracle.device_allocations() > 0
 
 
+def test_run_steps_on_the_cpu_build_is_the_plain_loop(mx_oracle):
+    """mxt_run_steps without a graph-capable backend: n calls of the step, failures handed on."""
+    mx = mx_oracle
+    a = mx.tensor(np.full((2, 3), 3.0, np.float32)).with_grad()
+    calls = []
+
+    def step():
+        calls.append(1)
+        a.mul(a).sum_all().backward()
+    mx.run_steps(step, 40)
+    assert len(calls) == 40 and mx.last_train_replayed() == 0
+    np.testing.assert_array_equal(a.grad().numpy(), np.full((2, 3), 40 * 6.0, np.float32))
+
+    def bad():
+        raise ValueError("no")
+    with pytest.raises(ValueError):
+        mx.run_steps(bad, 3)
+
+
 def test_adam_training_matches_the_update_rule(mx_oracle):
     """adam.rs through the tensor API on the CPU oracle (op by op) against the update rule in float64."""
     from host_programs import mlp_adam_numpy, mlp_adam_run
@@ -145,8 +164,9 @@ def test_conv2d_forward_backward(mx_oracle, B, Cin, H, W, Cout, k, stride, pad):
 
 
 def test_sum_all_in_one_pass_or_dim_by_dim(mx_oracle):
-    """sum_all() of a contiguous f32 tensor as one reduction, or dim by dim as reduction.rs:76-83 does it: the same
-    gradients bit for bit, the sums within the f32 tolerance of a reduction of each other and of float64."""
+    """sum_all() of a contiguous f32 tensor (and the bias gradient of Conv2d) as one reduction, or dim by dim as
+    reduction.rs:76-83 does it: the same gradients bit for bit, the sums within the f32 tolerance of a reduction of each
+    other and of float64."""
     mx = mx_oracle
     rng = np.random.default_rng(31)
     a = rng.standard_normal((5, 7, 9, 11)).astype(np.float32)
@@ -164,8 +184,11 @@ def test_sum_all_in_one_pass_or_dim_by_dim(mx_oracle):
     finally:
         mx.set_sum_all_in_one_pass(True)
     assert res[True]["calls"] < res[False]["calls"]
-    for key in ("g", "grad_x", "grad_w", "grad_b", "out"):
+    for key in ("g", "grad_x", "grad_w", "out"):
         np.testing.assert_array_equal(res[True][key].view(np.uint32), res[False][key].view(np.uint32), err_msg=key)
+    # the bias gradient of Conv2d is itself a sum over W, H and the batch (conv.rs:287-291): one pass or three
+    scale = np.abs(res[False]["grad_b"]).max()
+    assert np.abs(res[True]["grad_b"] - res[False]["grad_b"]).max() <= 1e-5 * scale
     exact = float(np.sum(a.astype(np.float64) ** 2))
     for one_pass in (False, True):
         assert abs(float(res[one_pass]["z"]) - exact) <= 1e-5 * exact
