@@ -431,7 +431,10 @@ MX_DECL_REDUCE(mx_f16, f16)
  *   hip_sgd_step_f32           param[i] = param[i] - grad[i] * lr
  * Gradients and parameters are bit for bit what sub / pow / sum_all / div_scalar and their backward, or mul_scalar and
  * sub_inplace, give; the loss is a sum of n terms added in a fixed tree of its own (within the f32 tolerance of a
- * reduction of the op sequence's, whose order the reference does not fix either). */
+ * reduction of the op sequence's, whose order the reference does not fix either).  Inside a graph capture, at sizes
+ * where a launch is latency bound, the three join the fused chains like the ops they replace (the step as an elementwise
+ * member, the loss of at most 65536 elements as a stage of the serial phase, the backward pass as a member of the
+ * parallel phase): the replayed bytes are those of the calls made one by one. */
 void hip_mse_loss_f32(size_t n, const float* pred, const float* target, float* loss);
 void hip_mse_loss_backward_f32(size_t n, const float* pred, const float* target, const float* grad_loss, float* grad_pred, float* grad_target);
 void hip_sgd_step_f32(size_t n, float* param, const float* grad, float lr);
