@@ -427,7 +427,8 @@ MX_DECL_REDUCE(mx_f16, f16)
  * element functions in the same order on values held in registers, contiguous f32 buffers:
  *   hip_mse_loss_f32           loss[0] = (sum of square(pred[i] - target[i])) / n          (16-byte aligned operands)
  *   hip_mse_loss_backward_f32  grad_pred[i] = 0 + (((grad_loss[0] / n) * 2) * (pred[i] - target[i])),
- *                              grad_target[i] = 0 + (-(that product)); either output may be NULL
+ *                              grad_target[i] = 0 + (-(that product)); either output may be NULL; grad_loss == NULL
+ *                              stands for a gradient of 1 (the seed of backward(), which then need not be written)
  *   hip_sgd_step_f32           param[i] = param[i] - grad[i] * lr
  * Gradients and parameters are bit for bit what sub / pow / sum_all / div_scalar and their backward, or mul_scalar and
  * sub_inplace, give; the loss is a sum of n terms added in a fixed tree of its own (within the f32 tolerance of a

@@ -247,7 +247,8 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
                     }
                 }
                 if (c.op == FUSE_OP_MSE_BACKWARD) {
-                    const float scale = mse_grad_scale(gl((const void*)(((uint64_t)c.payload[1] << 32) | c.payload[0]))[0], (float)c.nel);
+                    const uint64_t seed = ((uint64_t)c.payload[1] << 32) | c.payload[0];      // (0: the gradient of the loss is 1)
+                    const float scale = mse_grad_scale(seed ? gl((const void*)seed)[0] : 1.0f, (float)c.nel);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) r.v[e] = mse_grad(scale, val[0][e], val[1][e]);
                 } else {

@@ -38,7 +38,7 @@ constexpr int FUSE_MAX_CMDS = 16;          // members of the parallel phase
 constexpr int FUSE_MAX_TAIL = 12;          // stages of the serial phase
 constexpr uint32_t FUSE_OP_DOT = 0xD07u;   // FuseCmd::op of a matmul producer (the other values index EwProgOps)
 // FuseCmd::op of the fused MSE loss's backward pass (loss.hpp): out = 0 + ((g / nel) * 2) * (in0 - in1), where g is the
-// f32 the payload's 8 bytes point to (read by every thread) and nel the element count
+// f32 the payload's 8 bytes point to (read by every thread; a null pointer stands for 1) and nel the element count
 constexpr uint32_t FUSE_OP_MSE_BACKWARD = 0xB5Eu;
 constexpr int FUSE_TAIL_ARG_BYTES = 112;
 constexpr uint32_t FUSE_TICKETS = 1024;    // ticket slots per device

@@ -7,6 +7,7 @@
 // apply the same element functions in the same order to values held in registers:
 //   forward   loss = (sum over i of square(pred[i] - target[i])) / n              one read of pred and target
 //   backward  grad_pred[i]   = 0 + (((g / n) * 2) * (pred[i] - target[i]))         one read of pred and target, one write
+//             (g = grad_loss[0], or 1 when no grad_loss is given: the seed of backward(), never written anywhere)
 //             grad_target[i] = 0 + (-(((g / n) * 2) * (pred[i] - target[i])))      (when asked for)
 //   sgd       param[i] = param[i] - grad[i] * lr
 // Every gradient and every updated parameter is bit for bit what the op-by-op sequence gives (f32, no fused
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(LB) void mse_backward_kernel(size_t nunits, const f
     const size_t i = (size_t)blockIdx.x * LB + threadIdx.x;
     if (i >= nunits) return;
     // the scalar chain of the op sequence: div_scalar's backward, then pow's mul_scalar(2)
-    const float scale = mse_grad_scale(grad_loss[0], count);
+    const float scale = mse_grad_scale(grad_loss ? grad_loss[0] : 1.0f, count);
     const AVec<float, VEC> p = ((const AVec<float, VEC>*)pred)[i], t = ((const AVec<float, VEC>*)target)[i];
     AVec<float, VEC> gp, gt;
 #pragma unroll
@@ -104,7 +105,7 @@ extern "C" void hip_mse_loss_f32(size_t n, const float* pred, const float* targe
 
 extern "C" void hip_mse_loss_backward_f32(size_t n, const float* pred, const float* target, const float* grad_loss, float* grad_pred,
                                           float* grad_target) { MXH_API;
-    if (!pred || !target || !grad_loss) { set_status(ERR_INVALID, "mse_loss_backward: null buffer"); return; }
+    if (!pred || !target) { set_status(ERR_INVALID, "mse_loss_backward: null buffer"); return; }
     if (n == 0 || (!grad_pred && !grad_target)) return;
     const bool vec = n % 4 == 0 && aligned16(pred) && aligned16(target) && (!grad_pred || aligned16(grad_pred)) && (!grad_target || aligned16(grad_target));
     const size_t units = vec ? n / 4 : n;
@@ -123,7 +124,8 @@ extern "C" void hip_mse_loss_backward_f32(size_t n, const float* pred, const flo
         c.nin = 2;
         c.nel = (uint32_t)n;
         std::memcpy(c.payload, (const void*)&grad_loss, sizeof(grad_loss));
-        if (fuse_record_mse_backward(c, vec, units, Extent{(uintptr_t)grad_loss, (uintptr_t)(grad_loss + 1)})) return;
+        const Extent seed = grad_loss ? Extent{(uintptr_t)grad_loss, (uintptr_t)(grad_loss + 1)} : Extent{0, 0};
+        if (fuse_record_mse_backward(c, vec, units, seed)) return;
     }
     if (vec) {
         if (grad_target) hipLaunchKernelGGL((mse_backward_kernel<4, true>), grid, dim3(LB), 0, stream(), units, pred, target, grad_loss, grad_pred, grad_target, (float)n);

@@ -264,6 +264,9 @@ struct Tensor {
     // This tensor's elements are sums that started from +0 (what sum_to_shape writes), so `0 + x` would copy it bit for
     // bit.  Not kept by views or copies of the tensor.
     bool sums_from_zero = false;
+    // The seed of backward() - ones_like(loss), lib.rs:293-301 - not yet written anywhere: a tensor without a buffer that
+    // only a backward closure which asked for it (Node::takes_unit_seed) ever sees.
+    bool unit_seed = false;
     std::shared_ptr<Node<B>> node;
 
     using T = Tensor<B>;
@@ -427,7 +430,15 @@ struct Tensor {
     }
     void backward() const {                                                         // lib.rs:293-301
         if (!requires_grad) return;
-        T go = ones_like(*this);
+        // (a one-element loss whose node takes the seed as a constant: no fill, and nothing for its backward pass to wait for)
+        T go;
+        if (autograd_shortcuts() && node && node->takes_unit_seed && size() == 1) {
+            go.layout = layout;
+            go.dtype = dtype;
+            go.unit_seed = true;
+        } else {
+            go = ones_like(*this);
+        }
         std::unordered_set<const void*> visited;
         backward_tracking(go, visited);
     }
@@ -1093,6 +1104,7 @@ struct Node {
     std::string op;
     std::vector<Tensor<B>> inputs;
     typename Tensor<B>::BackwardFn backward;
+    bool takes_unit_seed = false;      // the closure handles a Tensor::unit_seed gradient (all ones, no buffer)
 };
 
 // ---- seeded normal values (the reference's randn draws from an unseeded thread_rng, creation.rs:318-331) ----
@@ -1315,12 +1327,14 @@ Tensor<B> mse_loss(const Tensor<B>& pred, const Tensor<B>& target) {            
             if (pred.requires_grad || target.requires_grad) {
                 loss.with_grad();
                 loss.set_node("mse_loss", {pred, target}, [](const std::vector<T>& in, const T& go_in) {
-                    const T go = go_in.to_dtype(DType::F32).contiguous();
+                    // (the seed of backward() arrives without a buffer: the kernel then takes the gradient of the loss as 1)
+                    const T go = go_in.unit_seed ? go_in : go_in.to_dtype(DType::F32).contiguous();
+                    const float* seed = go_in.unit_seed ? nullptr : go.template p<float>() + go.offset();
                     const bool want_p = T::wanted(in, 0), want_t = T::wanted(in, 1);
                     T gp = want_p ? T::empty(in[0].shape(), DType::F32) : T(), gt = want_t ? T::empty(in[1].shape(), DType::F32) : T();
                     if (want_p || want_t) {
                         B::mse_loss_backward(in[0].size(), in[0].template p<float>(), in[1].template p<float>(),
-                                             go.template p<float>() + go.offset(), want_p ? gp.template p<float>() : nullptr,
+                                             seed, want_p ? gp.template p<float>() : nullptr,
                                              want_t ? gt.template p<float>() : nullptr);
                         ++backend_calls();
                         B::check();
@@ -1329,6 +1343,7 @@ Tensor<B> mse_loss(const Tensor<B>& pred, const Tensor<B>& target) {            
                     gt.sums_from_zero = want_t;
                     return std::vector<T>{gp, gt};
                 });
+                loss.node->takes_unit_seed = true;
             }
             return loss;
         }

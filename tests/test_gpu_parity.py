@@ -1499,6 +1499,10 @@ def test_fused_mse_loss_equals_the_op_sequence(oracle, hip, n):
     (fp2,) = hip.call("mse_loss_backward_f32", n, In(pred), In(target), In(g), Out(n, "f32"), None)
     (ft2,) = hip.call("mse_loss_backward_f32", n, In(pred), In(target), In(g), None, Out(n, "f32"))
     assert same_bits(fp2, gp) and same_bits(ft2, gt)
+    # no grad_loss: the seed of backward(), a gradient of exactly 1
+    (fp1,) = hip.call("mse_loss_backward_f32", n, In(pred), In(target), None, Out(n, "f32"), None)
+    (fpo,) = hip.call("mse_loss_backward_f32", n, In(pred), In(target), In(np.array([1.0], np.float32)), Out(n, "f32"), None)
+    assert same_bits(fp1, fpo)
     if n <= (1 << 20) + 5:
         _, op, ot = chain(oracle)
         assert same_bits(fp, op) and same_bits(ft, ot)

@@ -394,8 +394,9 @@ def test_chain_with_matmuls_reductions_and_a_serial_tail(lib, n, feats):
         assert launches == 15 and nodes <= 3, (launches, nodes)
 
 
-def fused_nn_step(lib, seq, n, feats, r):
-    """The step of linear_step() with the loss, its backward pass and the parameter updates as the fused calls."""
+def fused_nn_step(lib, seq, n, feats, r, seeded=True):
+    """The step of linear_step() with the loss, its backward pass and the parameter updates as the fused calls; seeded:
+    the gradient of the loss is a tensor filled with 1, else it is left out of the backward call (which then takes 1)."""
     x, y = seq.dev(r.standard_normal((n, feats)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
     w0, b0 = r.standard_normal(feats).astype(np.float32), r.standard_normal(1).astype(np.float32)
     w, b = seq.out(feats * 4, "f4"), seq.out(4, "f4")          # updated in place: restored at the start of every run
@@ -408,7 +409,7 @@ def fused_nn_step(lib, seq, n, feats, r):
     seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), pred.ptr, b.ptr, pb.ptr)
     seq.add("mse_loss_f32", n, pb.ptr, y.ptr, loss.ptr)
     seq.add("fill_f32", 1, gloss.ptr, C.c_float(1.0))
-    seq.add("mse_loss_backward_f32", n, pb.ptr, y.ptr, gloss.ptr, gpred.ptr, None)
+    seq.add("mse_loss_backward_f32", n, pb.ptr, y.ptr, gloss.ptr if seeded else None, gpred.ptr, None)
     seq.add("matmul_f32", feats, u64(2, 2, 2, [feats, 1], [feats, n], [n, 1], [1, feats], [1, 1], 0, 0), x.ptr, gpred.ptr, gw.ptr)
     seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), gpred.ptr, gb.ptr)
     seq.add("sgd_step_f32", feats, w.ptr, gw.ptr, C.c_float(0.01))
@@ -426,6 +427,21 @@ def test_fused_loss_and_sgd_calls_join_the_chains(lib, n, feats):
     launches, nodes = fused(lib, seq, replays=3)
     if 4096 <= n <= 16384:           # (beyond that the weight gradient is a launch of its own: 1024 threads)
         assert launches == 11 and nodes <= 3, (launches, nodes)
+
+
+@pytest.mark.parametrize("n,feats", [(10000, 3), (4096, 4), (5001, 1)])
+def test_fused_loss_backward_without_a_seed_stays_in_the_forward_chain(lib, n, feats):
+    """With no gradient tensor to wait for, the backward member meets the prediction element for element and is hoisted
+    over the loss stage: the step is two chains (and the bytes of the seeded form)."""
+    seqs = []
+    for seeded in (True, False):
+        seq = Seq(lib)
+        fused_nn_step(lib, seq, n, feats, np.random.default_rng(300 + n + feats), seeded=seeded)
+        launches, nodes = fused(lib, seq, replays=3)
+        seqs.append((seq, nodes))
+    assert seqs[1][1] == seqs[0][1] - 1, (seqs[0][1], seqs[1][1])
+    for a, b in zip(seqs[0][0].read(), seqs[1][0].read()):
+        assert a.tobytes() == b.tobytes()
 
 
 def test_fused_loss_backward_waits_for_a_gradient_written_in_the_same_chain(lib):
