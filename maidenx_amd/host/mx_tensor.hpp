@@ -246,6 +246,14 @@ inline int& conv_gathered_products() { static int mode = 1; return mode; }
 // into when that gradient is a broadcast view (0 + g is written straight away, as for a contiguous gradient), and that
 // `0 + g` altogether when g is a fresh sum_to_shape result (sums that started from +0: it becomes the gradient as it is).
 inline bool& autograd_shortcuts() { static bool on = true; return on; }
+// Nesting depth of backward() on this thread.  Inside it tensors are temporaries of the walk - nobody writes into them in
+// place - so a result that would be a bit-for-bit copy of its input (`0 + x` of sums that started from +0) may be that
+// input, or a view of it.
+inline int& backward_depth() { static thread_local int depth = 0; return depth; }
+struct BackwardScope {
+    BackwardScope() { ++backward_depth(); }
+    ~BackwardScope() { --backward_depth(); }
+};
 // MSELoss and SGD::step as one backend call each where the backend has the fused kernels (the same element functions in
 // the same order: every gradient and parameter is the same bytes; the loss is summed in a tree of its own, within the f32
 // tolerance of a reduction).  false: the op sequences of the reference.
@@ -261,8 +269,8 @@ struct Tensor {
     Layout layout;
     DType dtype = DType::F32;
     bool requires_grad = false;
-    // This tensor's elements are sums that started from +0 (what sum_to_shape writes), so `0 + x` would copy it bit for
-    // bit.  Not kept by views or copies of the tensor.
+    // This tensor's elements are sums that started from +0 (what sum_to_shape, sum and matmul write: +0 plus anything is
+    // never -0), so `0 + x` would copy it bit for bit.  Kept by reshaping views of a tensor that records no gradient.
     bool sums_from_zero = false;
     // The seed of backward() - ones_like(loss), lib.rs:293-301 - not yet written anywhere: a tensor without a buffer that
     // only a backward closure which asked for it (Node::takes_unit_seed) ever sees.
@@ -439,6 +447,7 @@ struct Tensor {
         } else {
             go = ones_like(*this);
         }
+        BackwardScope scope;
         std::unordered_set<const void*> visited;
         backward_tracking(go, visited);
     }
@@ -506,7 +515,16 @@ struct Tensor {
             if (ad == 1 || bd == 1 || ad == bd) out[on - 1 - i] = std::max(ad, bd);
             else throw Error(ErrKind::InvalidShape, "Cannot broadcast shapes " + shape_str(a.shape()) + " and " + shape_str(b.shape()));
         }
-        return {a.broadcast(out), b.broadcast(out)};
+        // A 0-d operand is materialised by the reference (broadcast_scalar_to: item() and a host fill); the kernels read a
+        // view with zero strides just as well, and the result is the same bits.
+        auto spread = [&](const T& t) {
+            if (!autograd_shortcuts() || !t.shape().empty() || out.empty()) return t.broadcast(out);
+            T v = share_buffer(t);
+            v.layout = t.layout.broadcast_to(out);
+            if (t.requires_grad) v.with_grad();
+            return v;
+        };
+        return {spread(a), spread(b)};
     }
     // promote both sides to the common dtype, broadcast, run the kernel (ops/binary.rs:17-44)
     T binary_forward(const T& rhs_in, BinOp op, T& lhs_b, T& rhs_b) const {
@@ -782,6 +800,7 @@ struct Tensor {
         });
         ++backend_calls();
         B::check();
+        result.sums_from_zero = op == SUM;
         if (keep_dim) {
             Shape ks = shape();
             ks[dim] = 1;
@@ -791,6 +810,12 @@ struct Tensor {
     }
     T sum(int dim_in, bool keep_dim) const {                                        // ops/reduction.rs:9-74
         size_t dim = norm_dim(dim_in, ndim());
+        // (inside backward(): the sum over an axis of length 1 is `0 + x`; of sums that started from +0 that is x itself)
+        if (autograd_shortcuts() && backward_depth() > 0 && !requires_grad && sums_from_zero && shape()[dim] == 1 && is_contiguous()) {
+            Shape ns = shape();
+            if (!keep_dim) ns.erase(ns.begin() + dim);
+            return view_like("sum", ns);
+        }
         T result = reduce_forward(SUM, dim, keep_dim);
         if (requires_grad) {
             result.with_grad();
@@ -844,6 +869,8 @@ struct Tensor {
             if (target[i] == 0 || shape()[i] % target[i] != 0)
                 throw Error(ErrKind::ShapeMismatch, "Dimension " + std::to_string(i) + " is not divisible: " + std::to_string(shape()[i]) +
                                                         " -> " + std::to_string(target[i]));
+        // (inside backward(): `0 + x` of sums that started from +0 is x)
+        if (autograd_shortcuts() && backward_depth() > 0 && !requires_grad && sums_from_zero && shape() == target) return *this;
         T result = empty(target, dtype);    // zero-filled in the reference (reduction.rs:112); fully written by the kernel
         auto md = meta_to_shape(*this, target);
         by_dtype(dtype, "sum_to_shape", [&](auto tag) {
@@ -889,6 +916,7 @@ struct Tensor {
     T view_like(const char* op, const Shape& ns) const {
         T result = share_buffer(*this);
         result.layout.view(ns);
+        result.sums_from_zero = sums_from_zero && !requires_grad;
         if (requires_grad) {
             result.with_grad();
             Shape orig = shape();
@@ -1071,6 +1099,7 @@ struct Tensor {
         });
         ++backend_calls();
         B::check();
+        result.sums_from_zero = true;       // every output is +0 plus its products
         if (ln == 1 && rn == 1) result = result.squeeze_all();
         else if (ln == 1 && rn >= 2) { int d = (int)result.ndim() - 2; if (result.shape()[d] == 1) result = result.squeeze(d); }
         else if (ln >= 2 && rn == 1) { int d = (int)result.ndim() - 1; if (result.shape()[d] == 1) result = result.squeeze(d); }
@@ -1091,6 +1120,8 @@ struct Tensor {
                 });
                 ++backend_calls();
                 B::check();
+                gl.sums_from_zero = want_l;
+                gr.sums_from_zero = want_r;
                 // the gradients go back in the inputs' own dtypes (matmul.rs:137-143)
                 return std::vector<T>{want_l ? gl.to_dtype(in[0].dtype) : T(), want_r ? gr.to_dtype(in[1].dtype) : T()};
             });
@@ -1270,6 +1301,7 @@ struct Conv2d {                                                                 
                             B::cols_matmul(md.data(), 1, x.f32(), grad_flat.f32() + grad_flat.offset(), grad_flat.shape()[1], rs, gw.f32());
                             ++backend_calls();
                             B::check();
+                            gw.sums_from_zero = true;       // a matmul's outputs, like the stored way's
                         }
                     } else {
                         T stored = cols;

@@ -191,6 +191,25 @@ def _shortcut_programs(mx):
                 out[key + "_ga"] = ta.grad().numpy()
             if gb:
                 out[key + "_gb"] = tb.grad().numpy()
+    # a 0-d operand (materialised by the reference, read through zero strides with the shortcuts), zeros of both signs in
+    # the data, and a matmul whose gradients are sums of a single term
+    az = a.copy()
+    az[::2, 1, :] = 0.0
+    az[1::2, 2, :] = -0.0
+    for op in ("add", "sub", "mul", "div"):
+        for sval in (-2.5, 0.0):
+            if op == "div" and sval == 0.0:
+                continue
+            ta, ts = mx.tensor(az).with_grad(), mx.tensor(np.array(sval, np.float32), shape=()).with_grad()
+            y = getattr(ta, op)(ts)
+            z = y.mul(y).sum_all()
+            z.backward()
+            key = f"scalar_{op}_{sval}"
+            out[key + "_y"], out[key + "_ga"], out[key + "_gs"] = y.numpy(), ta.grad().numpy(), ts.grad().numpy()
+    m1, m2 = mx.tensor(az.reshape(30, 4)).with_grad(), mx.tensor(rng.standard_normal((4, 1)).astype(np.float32)).with_grad()
+    mm = m1.matmul(m2)
+    mm.sum_all().backward()
+    out["mm_y"], out["mm_g1"], out["mm_g2"] = mm.numpy(), m1.grad().numpy(), m2.grad().numpy()
     x, w, bias = conv_inputs(2, 3, 6, 5, 4, 3, seed=21)
     target = rng.standard_normal((2, 4, 6, 5)).astype(np.float32)
     for k, v in conv_step(mx, x, w, bias, 1, 1, target).items():
