@@ -625,6 +625,15 @@ void hip_conv2d_col2im_f64(size_t num_els, const size_t* metadata, const double*
 void hip_conv2d_cols_matmul_f32(const size_t* metadata, int transposed, const float* input, const float* rhs, size_t n,
                                 const size_t* rhs_strides, float* out);
 
+/* The forward product of the layer with what follows it in the store (no backend symbol in the reference:
+ * crates/maidenx_nn/src/layers/conv.rs:217-232 multiplies, reshapes to [B, oh, ow, Cout], transposes twice and adds the
+ * bias - a second pass over the output through a transposed view):
+ *   out[b][j][p] = (x[b*P + p][:] . w[j][:]) + bias[j]      x [M = B*P, K] and w [J, K] row-major, out [B, J, P]
+ * The product's tiles and order of additions are hip_matmul_f32's, the addition is hip_add_f32's: the same bits as the
+ * three calls.  Returns 1 when it ran, 0 when the shapes are not for it and nothing was queued (whole 64-row tiles,
+ * J = 64, K a multiple of 32, 16-byte aligned operands, more than 128 tiles): the caller then makes the separate calls. */
+int hip_conv2d_forward_product_f32(size_t M, size_t K, size_t J, size_t P, const float* x, const float* w, const float* bias, float* out);
+
 /* ---- softmax: replaces crates/maidenx_cuda/src/nn/activation/softmax.rs (cuda_softmax_<T>) ------------
  * metadata = dims[n] | strides[n] | offset; dim >= num_dims means the last dim.
  * Semantics: crates/maidenx_cpu/src/nn/activation/softmax.rs:62-207 (max from -inf, the sum seeded

@@ -426,6 +426,37 @@ __device__ __forceinline__ void store_tile(O* out, const typename Cfg::Acc (&acc
     }
 }
 
+// The store of a Conv2d forward product: output row m = b * P + p of the [B*P, J] product is pixel p of batch b, and the
+// layer wants out[b][j][p] = product[m][j] + bias[j] (nn/layers/conv.rs:222-232: reshape, two transposes, add).  A lane
+// holds one row and 16 columns of a 32x32 tile, so for a given column the 32 lanes of a half-wave write 32 consecutive
+// pixels: 128 contiguous bytes.  The addition is the elementwise kernel's f32 add on the same two values.
+struct GemmEpi {
+    const float* bias;
+    uint32_t P;
+    FastDiv d_P;
+};
+template <class Cfg>
+__device__ __forceinline__ void store_tile_planes(float* out, const typename Cfg::Acc (&acc)[Cfg::MI][Cfg::MJ], const GemmArgs& g, const GemmEpi& e,
+                                                  uint32_t i0, uint32_t j0, int wm, int wn, int lane) {
+    constexpr int MI = Cfg::MI, MJ = Cfg::MJ, TS = Cfg::TS;
+    static_assert(TS == 32, "f32 tiles");
+#pragma unroll
+    for (int a = 0; a < MI; ++a) {
+        const uint32_t row = i0 + wm * TS * MI + a * TS + lane % TS;
+        const uint32_t b = fd_div(row, e.d_P), p = row - b * e.P;
+        float* plane0 = out + ((int64_t)b * g.J) * e.P + p;
+#pragma unroll
+        for (int c = 0; c < MJ; ++c)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t col = j0 + wn * TS * MJ + c * TS + 8 * q + 4 * (lane / 32);
+                const f32x4 bias = *(const f32x4*)(e.bias + col);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) plane0[(int64_t)(col + k) * e.P] = acc[a][c][4 * q + k] + bias[k];      // (never contracted: -ffp-contract=off)
+            }
+    }
+}
+
 // Folds the split-K partials in split order (deterministic) and rounds once.
 template <class T>
 __global__ __launch_bounds__(256) void gemm_fold_kernel(const float* __restrict__ part, T* __restrict__ out, size_t n, uint32_t splits) {
@@ -480,9 +511,11 @@ __device__ __forceinline__ TilePos tile_of_block(const GemmArgs& g) {
 // 2: four at a time (see cols_gather4), 1: one by one.
 // RB: FAST for a tile whose last rows lie past g.I or whose last columns lie past g.J (the reduction whole k-tiles): X and Y
 // are loaded through descriptors that end with their last entries, and the outputs that do not exist are not stored.
-template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false, int XCOLS = 0, bool RB = false>
-__device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem, const ColsView* cv = nullptr) {
+template <class T, bool XR, bool YR, class Cfg, bool FAST, bool PANEL = false, int XCOLS = 0, bool RB = false, bool PLANES = false>
+__device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos& pos, unsigned char* smem, const ColsView* cv = nullptr,
+                                               const GemmEpi* epi = nullptr) {
     static_assert(!RB || (FAST && !PANEL && XCOLS == 0), "bounded rows: the unchecked body of stored operands");
+    static_assert(!PLANES || (std::is_same<T, float>::value && FAST && !PANEL && !RB), "the Conv2d store: f32, whole tiles, no split");
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, MJ = Cfg::MJ, NT = Cfg::NT;
     constexpr bool SWZ = Cfg::TS == 16;
     static_assert(!XCOLS || (std::is_same<T, float>::value && !PANEL), "the gathered operand is f32, one tile per block");
@@ -656,6 +689,8 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, const TilePos&
     if (g.splits > 1) {
         float* part = g.part + ((int64_t)split * g.batch + b) * g.I * g.J;
         store_tile<float, Cfg, FAST, RB>(part, acc, g, i0, j0, wm, wn, lane);
+    } else if constexpr (PLANES) {
+        store_tile_planes<Cfg>((float*)g.out, acc, g, *epi, i0, j0, wm, wn, lane);
     } else {
         store_tile<T, Cfg, FAST, RB>((T*)g.out + (int64_t)b * g.I * g.J, acc, g, i0, j0, wm, wn, lane);
     }
@@ -676,6 +711,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_panel_kernel(GemmArgs g, ui
     pos.b = 0;
     pos.split = 0;
     gemm_mfma_body<T, XR, YR, Cfg, true, true>(g, pos, smem);
+}
+
+// whole tiles everywhere, one batch, no split, both operands reduction-contiguous: the Conv2d forward product with its
+// bias add and layout change in the store (GemmEpi)
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_planes_kernel(GemmArgs g, GemmEpi e) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const TilePos pos = tile_of_block(g);
+    gemm_mfma_body<float, true, true, Cfg, true, false, 0, false, true>(g, pos, smem, nullptr, &e);
 }
 
 template <class T, bool XR, bool YR, class Cfg, bool ALIGNED>
@@ -1234,6 +1278,42 @@ using namespace mxh;
 extern "C" void hip_conv2d_cols_matmul_f32(const size_t* metadata, int transposed, const float* input, const float* rhs, size_t n,
                                            const size_t* rhs_strides, float* out) { MXH_API;
     cols_matmul(metadata, transposed, input, rhs, n, rhs_strides, out);
+}
+
+// out[b][j][p] = (X[b*P + p][:] . W[j][:]) + bias[j] for X [M, K] and W [J, K], both row-major: 1 when it ran, 0 when the
+// shapes are not for it (nothing queued)
+extern "C" int hip_conv2d_forward_product_f32(size_t M, size_t K, size_t J, size_t P, const float* x, const float* w, const float* bias,
+                                              float* out) {
+    MXH_API_INT;
+    using Cfg = Cfgs<float>::Tall;
+    constexpr size_t TK = TK_BYTES / sizeof(float);
+    if (!x || !w || !bias || !out || M == 0 || K == 0 || J == 0 || P == 0) return 0;
+    if (M % P != 0 || M % Cfg::TM != 0 || J % Cfg::TN != 0 || K % TK != 0 || M >= (1ull << 31) || K >= (1ull << 31) || J > 64) return 0;
+    if ((uintptr_t)x % 16 || (uintptr_t)w % 16 || (uintptr_t)bias % 16 || M * J >= (1ull << 31) || M * K >= (1ull << 62)) return 0;
+    if (((int64_t)Cfg::TM * (int64_t)K + (int64_t)TK) * 4 >= (1ll << 31)) return 0;      // per-thread offsets inside a tile are 32-bit
+    if (prog_recording()) prog_abandon();
+    GemmArgs g;
+    std::memset((void*)&g, 0, sizeof(g));
+    g.X = x; g.Y = w; g.out = out;
+    g.xb = 0; g.xi = (int64_t)K; g.xr = 1;
+    g.yb = 0; g.yr = 1; g.yj = (int64_t)K;
+    g.I = (uint32_t)M; g.J = (uint32_t)J; g.R = (uint32_t)K; g.batch = 1;
+    g.tiles_i = (uint32_t)(M / Cfg::TM);
+    g.tiles_j = (uint32_t)(J / Cfg::TN);
+    g.splits = 1;
+    g.r_chunk = g.R;
+    g.part = nullptr;
+    if ((size_t)g.tiles_i * g.tiles_j <= 128) return 0;        // (few tiles: the plain product cuts the reduction over the chip)
+    GemmEpi e;
+    e.bias = bias;
+    e.P = (uint32_t)P;
+    e.d_P = make_fastdiv((uint32_t)P);
+    using SX = Stager<float, true, Cfg::TM, Cfg::NT, false>;
+    constexpr size_t lds_bytes = (size_t)2 * (Cfg::TM + Cfg::TN) * SX::PITCH * sizeof(float);
+    static_assert(lds_bytes <= (64u << 10), "no attribute needed");
+    hipLaunchKernelGGL(gemm_mfma_planes_kernel<Cfg>, dim3(g.tiles_i * g.tiles_j), dim3(Cfg::NT), lds_bytes, stream(), g, e);
+    MXH_LAUNCH_CHECK("gemm_mfma_planes");
+    return 1;
 }
 
 #define MXH_MATMUL_FOR(T, SUF)                                                                              \

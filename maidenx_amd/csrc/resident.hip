@@ -681,15 +681,6 @@ bool res_build(const std::vector<ResRecord>& recs, ResProgram& out) {
         }
         for (int k = 0; k < p.nacc; ++k) pending.push_back(p.acc[k]);
     }
-    if (getenv("MXH_RESIDENT_DEBUG")) {
-        for (const Region& g : regions)
-            fprintf(stderr, "[resident] region %p + %6zu: written %d, inherited %d, candidate %d, pinned %d, in LDS at the end %d (offset %u)\n", (void*)g.lo,
-                    g.size(), (int)g.written, (int)g.live_in, (int)g.candidate, (int)g.pinned, (int)g.in_lds, g.lds_off);
-        for (size_t i = 0; i < all.size(); ++i) {
-            const ResCmd& c = all[i].cmd;
-            fprintf(stderr, "[resident] cmd %3zu kind %u op %4u units %6u flags %02x mode %06x\n", i, c.kind, c.sub, c.units, c.flags, c.mode);
-        }
-    }
     out.host_cmds.resize(all.size());
     for (size_t i = 0; i < all.size(); ++i) out.host_cmds[i] = all[i].cmd;
     out.device_cmds = nullptr;
@@ -703,11 +694,14 @@ bool res_build(const std::vector<ResRecord>& recs, ResProgram& out) {
 }
 
 bool res_upload(ResProgram& p) {
-    static bool attr_set = false;
-    if (!attr_set) {
+    // more than 64 KB of LDS has to be allowed once per device
+    static bool attr_set[64] = {false};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) { (void)hipGetLastError(); return false; }
+    if (device < 0 || device >= 64 || !attr_set[device]) {
         hipError_t e = hipFuncSetAttribute((const void*)resident_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RES_LDS_BYTES);
         if (e != hipSuccess) { (void)hipGetLastError(); return false; }
-        attr_set = true;
+        if (device >= 0 && device < 64) attr_set[device] = true;
     }
     ResCmd* dev = nullptr;
     const size_t bytes = p.host_cmds.size() * sizeof(ResCmd);

@@ -352,7 +352,6 @@ static bool res_accepting() { return g_res_ok && !g_res_spilling && fuse_accepti
 // exactly these offers) or is launched, and later offers go there directly.
 static void res_spill() {
     if (!g_res_ok) return;
-    if (getenv("MXH_RESIDENT_DEBUG")) fprintf(stderr, "[resident] handing %zu kept records to the chains\n", g_res.size());
     g_res_ok = false;
     g_res_spilling = true;
     std::vector<ResRecord> recs;
@@ -689,13 +688,8 @@ int hip_graph_end_capture(void** graph_exec) {
     if (!g_capturing || !graph_exec) return (int)hipErrorInvalidValue;
     ResProgram res;
     bool as_res = false;
-    static const bool res_debug = getenv("MXH_RESIDENT_DEBUG") != nullptr;
-    if (res_debug) fprintf(stderr, "[resident] end of capture: candidate %d, %zu records kept\n", (int)g_res_ok, g_res.size());
     if (g_res_ok) {
         as_res = !g_res.empty() && res_build(g_res, res);
-        if (res_debug)
-            fprintf(stderr, "[resident] program %d: %u + %u + %u commands, %u LDS operands, %u barriers a pass, %u bytes of arena\n", (int)as_res,
-                    res.n_pro, res.n_body, res.n_epi, res.in_lds, res.barriers, res.lds_bytes);
         if (as_res) { g_res.clear(); g_res_ok = false; }
         else res_spill();
     }

@@ -1233,6 +1233,7 @@ struct Conv2d {                                                                 
             gathered = (conv_gathered_products() == 2 || (conv_gathered_products() == 1 && !input.requires_grad)) && M && K && ws[0] && M * K < ((size_t)1 << 31) && input.size() < ((size_t)1 << 31) &&
                        ws[1] == C && ws[2] == kh && ws[3] == kw && (wm.strides()[0] == 1 || wm.strides()[1] == 1);
         T cols, out;
+        bool in_store = false;       // the product's store already made the layout change and the bias add
         if (gathered) {
             if constexpr (B::has_cols_matmul) {
                 out = T::empty({M, ws[0]});
@@ -1247,11 +1248,31 @@ struct Conv2d {                                                                 
             B::im2col(cols.size(), md.data(), input.f32(), cols.f32());
             ++backend_calls();
             B::check();
-            out = cols.matmul(wm.transpose(-1, -2));
+            // The product, the [B, oh, ow, Cout] -> [B, Cout, oh, ow] change of layout and the bias add as one call where the
+            // backend has it and takes the shapes (the same bits: the product's tiles, then the elementwise add).  Only when
+            // the layer's own node records the backward (or nothing does): the ops' nodes are not made this way.
+            if constexpr (B::has_conv_forward_product) {
+                const bool own_node = input.requires_grad || !(weight.requires_grad || (has_bias && bias.requires_grad));
+                if (fused_nn_kernels() && has_bias && own_node && wm.is_contiguous() && bias.is_contiguous() && bias.dtype == DType::F32 &&
+                    weight.dtype == DType::F32) {
+                    T planes = T::empty({Bn, ws[0], oh, ow});
+                    if (B::conv_forward_product(M, K, ws[0], oh * ow, cols.f32(), wm.f32() + wm.offset(), bias.f32() + bias.offset(), planes.f32())) {
+                        ++backend_calls();
+                        B::check();
+                        out = planes;
+                        // (what matmul and add would have left on the result)
+                        if (weight.requires_grad || bias.requires_grad) out.with_grad();
+                        in_store = true;
+                    }
+                }
+            }
+            if (!in_store) out = cols.matmul(wm.transpose(-1, -2));
         }
-        out = out.reshape(std::vector<long>{(long)Bn, (long)oh, (long)ow, -1});
-        out = out.transpose(1, 3).transpose(2, 3);
-        if (has_bias) out = out.add(bias.reshape(Shape{1, bias.shape()[0], 1, 1}));
+        if (!in_store) {
+            out = out.reshape(std::vector<long>{(long)Bn, (long)oh, (long)ow, -1});
+            out = out.transpose(1, 3).transpose(2, 3);
+            if (has_bias) out = out.add(bias.reshape(Shape{1, bias.shape()[0], 1, 1}));
+        }
         if (input.requires_grad) {
             std::vector<T> inputs{input, weight};
             if (has_bias) inputs.push_back(bias);

@@ -53,6 +53,7 @@ def load():
         ("hip_graph_launch_n", [C.c_void_p, C.c_size_t], C.c_int),
         ("hip_graph_is_resident", [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         ("hip_graph_set_resident", [C.c_int], C.c_int), ("hip_buffer_discard", [C.c_void_p, C.c_size_t], None),
+        ("hip_conv2d_forward_product_f32", [C.c_size_t] * 4 + [C.c_void_p] * 4, C.c_int),
     ]:
         fn = getattr(lib, name)
         fn.argtypes = args

@@ -212,7 +212,7 @@ class Runner:
                 cargs.append(a.ctypes.data)
             else:
                 cargs.append(a)
-        fn(*cargs)
+        self.last_return = fn(*cargs)        # (None for the void entry points)
         if self.kind == "hip":
             for a, buf in post:
                 a.arr[...] = buf.to_numpy(a.arr.dtype, a.arr.size)

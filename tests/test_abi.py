@@ -37,7 +37,7 @@ def test_python_binding_covers_the_header():
                "hip_graph_begin_capture", "hip_graph_end_capture", "hip_graph_launch", "hip_graph_destroy",
                "hip_graph_is_program", "hip_graph_set_programs", "hip_graph_fused_launches", "hip_graph_set_fusion",
                "hip_noalloc_prepare", "hip_scratch_allocations", "hip_graph_launch_n", "hip_graph_is_resident",
-               "hip_graph_set_resident", "hip_buffer_discard"}
+               "hip_graph_set_resident", "hip_buffer_discard", "hip_conv2d_forward_product_f32"}
     assert set(declared_symbols()) == bound | runtime
 
 

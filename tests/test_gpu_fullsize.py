@@ -356,9 +356,13 @@ def test_conv2d_layer_step_config_size_every_way_gives_the_same_gradients(mx_hip
         mx.set_autograd_shortcuts(False)
         variants["no shortcuts"] = conv_step(mx, x, w, b, 1, 1, target)
         mx.set_autograd_shortcuts(True)
+        mx.set_fused_nn_kernels(False)
+        op_by_op = conv_step(mx, x, w, b, 1, 1, target)
+        mx.set_fused_nn_kernels(True)
         mx.set_sum_all_in_one_pass(False)
         dim_by_dim = conv_step(mx, x, w, b, 1, 1, target)
     finally:
+        mx.set_fused_nn_kernels(True)
         mx.set_conv_gathered_products(1)
         mx.set_conv_skip_unread_grad_cols(True)
         mx.set_autograd_shortcuts(True)
@@ -366,6 +370,11 @@ def test_conv2d_layer_step_config_size_every_way_gives_the_same_gradients(mx_hip
     for name, got in variants.items():
         for key in ("out", "loss", "grad_b", "grad_w", "grad_x"):
             assert np.array_equal(got[key].view(np.uint32), base[key].view(np.uint32)), (name, key)
+    # the loss, its backward pass and the forward product's store as the separate ops of the reference: the loss is summed in
+    # another order, everything else is the same bits
+    for key in ("out", "grad_b", "grad_w", "grad_x"):
+        assert np.array_equal(op_by_op[key].view(np.uint32), base[key].view(np.uint32)), ("op by op", key)
+    assert abs(float(op_by_op["loss"]) - float(base["loss"])) <= 1e-5 * abs(float(base["loss"]))
     for key in ("out", "grad_w", "grad_x"):
         assert np.array_equal(dim_by_dim[key].view(np.uint32), base[key].view(np.uint32)), ("sum_all dim by dim", key)
     assert abs(float(dim_by_dim["loss"]) - float(base["loss"])) <= 1e-5 * abs(float(base["loss"]))

@@ -929,6 +929,37 @@ def test_conv2d_cols_matmul(oracle, hip, case, n, transposed, rhs_turned):
         assert same_bits(hs, h)
 
 
+@pytest.mark.parametrize("Bn,P,K,J", [(3, 3136, 576, 64), (192, 49, 64, 64), (16, 1000, 96, 64), (2, 4160, 32, 64)])
+def test_conv2d_forward_product_is_matmul_then_transposes_then_add(oracle, hip, Bn, P, K, J):
+    """hip_conv2d_forward_product_f32 against the three calls it stands for (conv.rs:217-232): the product [B*P, K] x [K, J]
+    (w^T as a strided operand), the [B, P, J] -> [B, J, P] view, the bias add through it - bit for bit; and against the
+    oracle's product to the GEMM tolerance.  Planes of 49 and 1000 pixels put batch boundaries inside the 64-row tiles."""
+    r = rng(900 + P)
+    M = Bn * P
+    x = r.standard_normal((M, K)).astype(np.float32)
+    w = (r.standard_normal((J, K)) * 0.1).astype(np.float32)
+    bias = r.standard_normal(J).astype(np.float32)
+    (got,) = hip.call("conv2d_forward_product_f32", M, K, J, P, In(x), In(w), In(bias), Out(M * J, "f32"))
+    assert hip.last_return == 1
+    (prod,) = hip.call("matmul_f32", M * J, meta_matmul([M, J], [M, K], [K, J], [K, 1], [1, K]), In(x), In(w), Out(M * J, "f32"))
+    md = meta_binary([Bn, J, P], [P * J, 1, J], [0, 1, 0])
+    (want,) = hip.call("add_f32", M * J, 3, md, In(prod), In(bias), Out(M * J, "f32"))
+    assert same_bits(got, want)
+    ref = (x.astype(np.float64) @ w.astype(np.float64).T).reshape(Bn, P, J).transpose(0, 2, 1) + bias[None, :, None]
+    scale = (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T).max() + np.abs(bias).max()
+    assert np.abs(got.reshape(Bn, J, P) - ref).max() <= 1e-5 * scale
+
+
+def test_conv2d_forward_product_declines_other_shapes(hip):
+    """Rows that are not whole tiles, another column count, a ragged reduction, few tiles: 0 and nothing written."""
+    x, w, bias = np.zeros(64 * 300 * 40, np.float32), np.zeros(64 * 40, np.float32), np.zeros(64, np.float32)
+    for M, K, J, P in ((64 * 300 + 8, 32, 64, 4), (64 * 300, 32, 128, 100), (64 * 300, 40, 64, 100), (64 * 100, 32, 64, 100), (64 * 300, 32, 64, 7)):
+        out = np.full(8, -3.0, np.float32)
+        (o,) = hip.call("conv2d_forward_product_f32", M, K, J, P, In(x), In(w), In(bias), InOut(out))
+        assert hip.last_return == 0, (M, K, J, P)
+        assert (o == -3.0).all()
+
+
 def test_conv2d_cols_matmul_rejects_what_it_cannot_index(hip):
     x = np.zeros(16, np.float32)
     md = meta_conv(1, 1, 4, 4, 3, 3, 4, 4, 1, 1, 1, 1)
