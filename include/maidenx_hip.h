@@ -606,6 +606,13 @@ MX_DECL_CONV(float, f32)
 MX_DECL_CONV(mx_bf16, bf16)
 MX_DECL_CONV(mx_f16, f16)
 
+/* col2im accumulated into a gradient that exists (no backend symbol in the reference: its backward() adds the input
+ * gradient that conv2d_col2im wrote with a separate add_, crates/maidenx_tensor/src/lib.rs:221-241):
+ *   grad[i] = grad[i] + (the value hip_conv2d_col2im_f32 writes to output[i])
+ * - the sum formed as there, then one f32 add: the bits of the two calls, without writing the intermediate and reading it
+ * back. */
+void hip_conv2d_col2im_add_f32(size_t num_els, const size_t* metadata, const float* col, float* grad);
+
 /* f64 as well (crates/maidenx_cuda/src/nn/conv.rs:35): the same kernels, two elements per 16-byte vector. */
 void hip_conv2d_im2col_f64(size_t num_els, const size_t* metadata, const double* input, double* col);
 void hip_conv2d_col2im_f64(size_t num_els, const size_t* metadata, const double* col, double* output);

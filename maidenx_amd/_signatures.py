@@ -179,6 +179,7 @@ def extension_signatures():
     sig["mse_loss_backward_f32"] = [SZ, P, P, P, P, P]
     sig["sgd_step_f32"] = [SZ, P, P, C.c_float]
     sig["conv2d_cols_matmul_f32"] = [P, C.c_int, P, P, SZ, P, P]
+    sig["conv2d_col2im_add_f32"] = [SZ, P, P, P]
     sig.update(cast_signatures())
     sig.update(wide_util_signatures())
     sig.update(wide_unary_signatures())

@@ -149,7 +149,8 @@ template <> __device__ inline f16_t acc_add<f16_t>(f16_t a, f16_t b) { return f2
 
 template <class T>
 __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restrict__ col, T* __restrict__ out, size_t n_out,
-                                                    size_t num_els) {
+                                                    size_t num_els, bool accumulate) {
+    // accumulate: out[idx] = out[idx] + (the sum), i.e. the in-place add of the result into a gradient that exists
     size_t idx = (size_t)blockIdx.x * CB + threadIdx.x;
     if (idx >= n_out) return;
     uint32_t r = (uint32_t)idx, w, h, c, b;
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restr
     // every column index of this (b, c) plane is at least plane0; beyond num_els the reference skips them all
     // (the layer passes num_els = B*C*H*W, so most planes end here)
     const size_t plane0 = (size_t)(b * m.C + c) * m.kh * m.kw * m.oh * m.ow;
-    if (plane0 >= num_els) { out[idx] = T{}; return; }
+    if (plane0 >= num_els) { out[idx] = accumulate ? acc_add<T>(out[idx], T{}) : T{}; return; }
     uint32_t h_pad = h + m.ph, w_pad = w + m.pw;
     uint32_t hs = h_pad > m.kh - 1 ? h_pad - (m.kh - 1) : 0, ws = w_pad > m.kw - 1 ? w_pad - (m.kw - 1) : 0;
     uint32_t h_start, w_start, h_last, w_last, rem;
@@ -177,7 +178,7 @@ __global__ __launch_bounds__(CB) void col2im_kernel(ConvMeta m, const T* __restr
                 if (ci < num_els) sum = acc_add<T>(sum, col[ci]);
             }
         }
-    out[idx] = sum;
+    out[idx] = accumulate ? acc_add<T>(out[idx], sum) : sum;
 }
 
 // Unit stride along w: a thread owns VEC adjacent pixels of a row.  For a fixed tap (i, j) their column
@@ -189,16 +190,17 @@ template <class T, int N> struct alignas(sizeof(T)) CUVec { T v[N]; };
 // add (the sums are latency-bound otherwise: one round trip per tap).  KH = KW = 0: run-time extent.
 template <class T, int VEC, int KH, int KW>
 __global__ __launch_bounds__(CB) void col2im_row_kernel(ConvMeta m, const T* __restrict__ col, T* __restrict__ out, size_t nvec,
-                                                        size_t num_els) {
+                                                        size_t num_els, bool accumulate) {
     size_t idx = (size_t)blockIdx.x * CB + threadIdx.x;
     if (idx >= nvec) return;
     uint32_t r = (uint32_t)idx, wv, h, plane;
     fd_divmod(r, m.d_W, r, wv);            // d_W divides by W / VEC here
     fd_divmod(r, m.d_H, plane, h);
     T* dst = out + idx * VEC;
-    CVec<T, VEC> acc;
+    CVec<T, VEC> acc, old;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc.v[e] = T{};
+    for (int e = 0; e < VEC; ++e) acc.v[e] = old.v[e] = T{};
+    if (accumulate) old = *(const CVec<T, VEC>*)dst;        // (requested before the taps: its latency passes with theirs)
     const size_t plane0 = (size_t)plane * m.kh * m.kw * m.oh * m.ow;
     if (plane0 < num_els) {
         const uint32_t h_pad = h + m.ph;
@@ -259,6 +261,10 @@ __global__ __launch_bounds__(CB) void col2im_row_kernel(ConvMeta m, const T* __r
                 }
             }
         }
+    }
+    if (accumulate) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc.v[e] = acc_add<T>(old.v[e], acc.v[e]);
     }
     *(CVec<T, VEC>*)dst = acc;
 }
@@ -327,7 +333,7 @@ void im2col(size_t num_els, const size_t* md, const T* in, T* col) {
 }
 
 template <class T>
-void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
+void col2im(size_t num_els, const size_t* md, const T* col, T* out, bool accumulate = false) {
     if (!md || !col || !out) return;
     ConvMeta m;
     if (!parse_conv(md, m, true)) { set_status(ERR_INVALID, "col2im: bad metadata (stride slot is 0)"); return; }
@@ -344,12 +350,12 @@ void col2im(size_t num_els, const size_t* md, const T* col, T* out) {
         if (m.kh == 3 && m.kw == 3) kern = col2im_row_kernel<T, VEC, 3, 3>;
         else if (m.kh == 1 && m.kw == 1) kern = col2im_row_kernel<T, VEC, 1, 1>;
         else if (m.kh == 5 && m.kw == 5 && sizeof(T) == 4) kern = col2im_row_kernel<T, VEC, 5, 5>;
-        hipLaunchKernelGGL(kern, dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, col, out, nvec, num_els);
+        hipLaunchKernelGGL(kern, dim3(cdiv(nvec, CB)), dim3(CB), 0, stream(), m, col, out, nvec, num_els, accumulate);
         MXH_LAUNCH_CHECK("col2im");
         return;
     }
     m.d_W = make_fastdiv(m.W);
-    hipLaunchKernelGGL(col2im_kernel<T>, dim3(cdiv(n_out, CB)), dim3(CB), 0, stream(), m, col, out, n_out, num_els);
+    hipLaunchKernelGGL(col2im_kernel<T>, dim3(cdiv(n_out, CB)), dim3(CB), 0, stream(), m, col, out, n_out, num_els, accumulate);
     MXH_LAUNCH_CHECK("col2im");
 }
 
@@ -366,6 +372,10 @@ using namespace mxh;
     }
 
 MXH_CONV_FOR(float, f32)
+// col2im added into a gradient that already exists: grad[i] = grad[i] + (what hip_conv2d_col2im_f32 would write to i)
+extern "C" void hip_conv2d_col2im_add_f32(size_t num_els, const size_t* md, const float* col, float* grad) { MXH_API;
+    col2im<float>(num_els, md, col, grad, true);
+}
 MXH_CONV_FOR(bf16_t, bf16)
 MXH_CONV_FOR(f16_t, f16)
 MXH_CONV_FOR(double, f64)      // (crates/maidenx_cuda/src/nn/conv.rs:35)

@@ -27,6 +27,8 @@ struct HipBackend {
     static constexpr auto sgd_step = &hip_sgd_step_f32;
     static constexpr bool has_cols_matmul = true;
     static constexpr auto cols_matmul = &hip_conv2d_cols_matmul_f32;
+    static constexpr bool has_col2im_add = true;
+    static constexpr auto col2im_add = &hip_conv2d_col2im_add_f32;
     static constexpr bool has_conv_forward_product = true;
     static constexpr auto conv_forward_product = &hip_conv2d_forward_product_f32;
     static void graph_begin() { if (hip_graph_begin_capture() != 0) throw mxt::Error(mxt::ErrKind::Backend, "hip_graph_begin_capture failed"); }

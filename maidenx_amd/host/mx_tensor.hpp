@@ -458,7 +458,8 @@ struct Tensor {
         std::vector<T> grads = node->backward(node->inputs, go);                    // lib.rs:93-111
         for (size_t i = 0; i < node->inputs.size(); ++i) {
             const T& in = node->inputs[i];
-            if (in.requires_grad && i < grads.size()) {
+            // (a closure that already added its gradient into the input's - a leaf's - hands back a tensor without a buffer)
+            if (in.requires_grad && i < grads.size() && grads[i].buf) {
                 in.accumulate_grad(grads[i]);
                 in.backward_tracking(grads[i], visited);
             }
@@ -1292,21 +1293,36 @@ struct Conv2d {                                                                 
                     // slots 10, 11: with padding 0 the reference panics (division by zero)
                     if (ph_ == 0 || pw_ == 0)
                         throw Error(ErrKind::InvalidOperation, "col2im: division by zero (padding 0 is read as stride 0)");
-                    T gi = T::empty({Bn, C, H, W});                                                  // col2im, conv.rs:378-418
+                    // When x is a leaf whose gradient already exists, backward() would only add the col2im result to it
+                    // (lib.rs:221-241): the backend's accumulating form writes grad + (that result) in one pass - the same
+                    // sum, then the same add - and nothing is handed back.
+                    T* into = nullptr;
+                    if constexpr (B::has_col2im_add) {
+                        if (fused_nn_kernels() && autograd_shortcuts() && !x.node && x.grad_cell && x.grad_cell->g) {
+                            T& g = *x.grad_cell->g;
+                            if (g.dtype == DType::F32 && g.is_contiguous() && g.offset() == 0 && g.shape() == x.shape() && ((uintptr_t)g.f32() % 16) == 0)
+                                into = &g;
+                        }
+                    }
+                    T gi = into ? T() : T::empty({Bn, C, H, W});                                     // col2im, conv.rs:378-418
                     // col2im is handed num_els = B*C*H*W (conv.rs:391) and reads no column entry at or beyond that flat
                     // index (crates/maidenx_cpu/src/nn/conv.rs:135), i.e. only the first ceil(B*C*H*W / (C*kh*kw)) rows of
                     // grad_cols; the rows below are never read, so the product is made for those leading rows only (each of
                     // them the same arithmetic as in the whole product).
                     T lead = grad_flat;
                     const size_t row_len = ws[1] * ws[2] * ws[3];
-                    const size_t used = row_len ? (gi.size() + row_len - 1) / row_len : 0;
+                    const size_t n_in = Bn * C * H * W;
+                    const size_t used = row_len ? (n_in + row_len - 1) / row_len : 0;
                     if (conv_skip_unread_grad_cols() && grad_flat.is_contiguous() && used < grad_flat.shape()[0]) {
                         lead = T::share_buffer(grad_flat);
                         lead.layout.shape[0] = used;
                     }
                     T grad_cols = lead.matmul(wm);
                     auto md = conv_meta(Bn, C, H, W, kh_, kw_, oh, ow, sh_, sw_, ph_, pw_);
-                    B::col2im(gi.size(), md.data(), grad_cols.f32(), gi.f32());
+                    if constexpr (B::has_col2im_add) {
+                        if (into) B::col2im_add(into->size(), md.data(), grad_cols.f32(), into->f32());
+                    }
+                    if (!into) B::col2im(n_in, md.data(), grad_cols.f32(), gi.f32());
                     ++backend_calls();
                     B::check();
                     grads.push_back(gi);

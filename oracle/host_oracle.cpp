@@ -51,6 +51,7 @@ struct OracleBackend {
     static constexpr bool has_fused_nn = false;
     static constexpr bool has_cols_matmul = false;
     static constexpr bool has_conv_forward_product = false;
+    static constexpr bool has_col2im_add = false;
     static constexpr auto im2col = &oracle_conv2d_im2col_f32;
     static constexpr auto col2im = &oracle_conv2d_col2im_f32;
     // with_dtype on the host, element by element, as the reference does (crates/maidenx_core/src/buffer/mod.rs:155-196)

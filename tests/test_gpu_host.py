@@ -364,6 +364,37 @@ def test_run_steps_replays_a_conv_step_and_equals_the_eager_loop(mx_hip):
         mx.set_graph_replay(True)
 
 
+def test_conv_input_gradient_accumulated_by_col2im_equals_the_separate_add(mx_hip):
+    """From the second backward() on, the input (a leaf) has a gradient and the layer's closure lets col2im add into it
+    (hip_conv2d_col2im_add_f32) instead of handing back a tensor for backward() to add: the accumulated gradient after
+    several steps is the bits of the op-by-op way, also when the input feeds a second consumer."""
+    mx = mx_hip
+    rng = np.random.default_rng(33)
+    x = rng.standard_normal((2, 4, 8, 8), dtype=np.float32)
+    w = rng.uniform(-0.3, 0.3, (4, 4, 3, 3)).astype(np.float32)
+    b = rng.uniform(-0.3, 0.3, (4,)).astype(np.float32)
+    t = rng.standard_normal((2, 4, 8, 8), dtype=np.float32)
+
+    def run(fused):
+        mx.set_fused_nn_kernels(fused)
+        conv = mx.Conv2d(mx.tensor(w), mx.tensor(b), stride=(1, 1), padding=(1, 1))
+        xin, target = mx.tensor(x).with_grad(), mx.tensor(t)
+        grads = []
+        for _ in range(4):
+            y = conv.forward(xin)
+            loss = mx.mse_loss(y.add(xin.mul(xin)), target)           # xin also reaches the loss directly
+            loss.backward()
+            conv.zero_grad()
+            grads.append(xin.grad().numpy().copy())
+        return grads
+    try:
+        a, c = run(True), run(False)
+    finally:
+        mx.set_fused_nn_kernels(True)
+    for step, (ga, gc) in enumerate(zip(a, c)):
+        np.testing.assert_array_equal(ga.view(np.uint32), gc.view(np.uint32), err_msg=str(step))
+
+
 def test_run_steps_hands_on_a_failure_of_the_step(mx_hip):
     """An exception inside the step ends the loop (and an open recording) and reaches the caller as it was raised; the
     library works on afterwards."""

@@ -983,6 +983,28 @@ def test_col2im_row_stride_two_column_stride_one(oracle, hip, k, dt):
         assert same_bits(o, h), num_els
 
 
+@pytest.mark.parametrize("B,Cc,H,W,k,p,sh,sw", [(2, 3, 16, 16, 3, 1, 1, 1), (2, 3, 15, 16, 3, 1, 2, 1), (1, 2, 9, 7, 3, 1, 1, 1), (3, 4, 12, 12, 5, 2, 1, 1),
+                                                 (2, 5, 8, 8, 1, 1, 1, 1), (2, 2, 10, 12, 4, 1, 2, 3)])
+def test_col2im_add_is_col2im_then_add_inplace(oracle, hip, B, Cc, H, W, k, p, sh, sw):
+    """hip_conv2d_col2im_add_f32 against the two calls it stands for - col2im into a fresh buffer, then add_inplace into
+    the gradient (lib.rs:221-241) - on the GPU and on the oracle: the same bits, for whole and truncated num_els (planes
+    beyond num_els add +0: a -0 in the gradient becomes +0 there), vector and scalar kernels."""
+    oh, ow = (H + 2 * p - k) // sh + 1, (W + 2 * p - k) // sw + 1
+    n_col, n_in = B * Cc * k * k * oh * ow, B * Cc * H * W
+    md = meta_conv(B, Cc, H, W, k, k, oh, ow, p, p, sh, sw)
+    r = rng(70 + k + H)
+    y = r.standard_normal(n_col).astype(np.float32)
+    grad0 = r.standard_normal(n_in).astype(np.float32)
+    grad0[::7] = -0.0
+    grad0[3::11] = 0.0
+    for num_els in (n_col, n_in, n_col // 2 + 3):
+        (got,) = hip.call("conv2d_col2im_add_f32", num_els, md, In(y), InOut(grad0.copy()))
+        for be in (hip, oracle):
+            (gi,) = be.call("conv2d_col2im_f32", num_els, md, In(y), Out(n_in, "f32"))
+            (want,) = be.call("add_inplace_f32", n_in, 1, meta_binary([n_in], [1], [1]), InOut(grad0.copy()), In(gi))
+            assert same_bits(got, want), (num_els, be.kind)
+
+
 # ---------------------------------------------------------------------------------------------------
 # reflection / replication padding, fold, softmax
 # ---------------------------------------------------------------------------------------------------
