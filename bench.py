@@ -820,11 +820,36 @@ def run_mlp(args):
                          {"backend_kernels_per_step": calls, "us_per_step": round(dt_s / steps * 1e6, 1)})
     result["roofline"] = None
     result["note"] = "launch-latency bound (about 200 KB touched per step): no roofline fraction applies"
+    # the same loop on 1000 rows, where the recorded step is a resident step program (one work-group, tensors in LDS) by
+    # default, against the same step as fused chains
+    result["config"]["rows_1000_us_per_step"] = _small_mlp(mx, 1000)
     # (rocprofv3 has crashed inside hipGraphLaunch on this measurement's 900 replays when it follows the training graphs:
     # the profiles' command skips it)
     result["config"]["empty_graph_replay_us_by_nodes"] = None if args.no_graph_floor else empty_graph_floor()
     result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_mlp(args)
     return result
+
+
+def _small_mlp(mx, rows, epochs=2000):
+    L, lib, _ = hip_backend()
+    rng = np.random.default_rng(0x5EED0007)
+    out = {}
+    for mode, limit in (("resident_step_program", None), ("fused_chains", 0)):
+        was = lib.hip_graph_set_resident(limit) if limit is not None else None
+        try:
+            x = mx.tensor(rng.standard_normal((rows, 3)).astype(np.float32)).with_grad()
+            y = mx.tensor(rng.standard_normal((rows, 1)).astype(np.float32))
+            lin = mx.Linear(in_features=3, out_features=1, with_bias=True, seed=3)
+            mx.train(lin, x, y, 0.01, 100)
+            mx.synchronize()
+            t0 = time.perf_counter()
+            mx.train(lin, x, y, 0.01, epochs)
+            mx.synchronize()
+            out[mode] = round((time.perf_counter() - t0) / epochs * 1e6, 1)
+        finally:
+            if was is not None:
+                lib.hip_graph_set_resident(was)
+    return out
 
 
 def _oracle_host(threads):

@@ -62,6 +62,7 @@ template <class T> struct OpFill;
 template <class T> struct OpIdentity;
 template <class T> struct OpZeroPlus;
 template <class T> struct OpSgdStep;
+template <class T> struct OpMseGradUnit;
 
 template <class... Ts> struct TypeList { static constexpr int size = (int)sizeof...(Ts); };
 template <class T, class L> struct IndexOf;
@@ -81,7 +82,7 @@ template <int I, class H, class... R> struct TypeAt<I, TypeList<H, R...>> { usin
         OpLog10<T>, OpLog2<T>, OpExp<T>, OpExp10<T>, OpExp2<T>, OpSoftplus<T>, OpRecip<T>, OpLogicalNot<T>,           \
         OpAddScalar<T>, OpSubScalar<T>, OpMulScalar<T>, OpDivScalar<T>, OpMaximumScalar<T>, OpMinimumScalar<T>,       \
         OpPow<T>, OpLeakyRelu<T>, OpElu<T>, OpEqScalar<T>, OpNeScalar<T>, OpLtScalar<T>, OpLeScalar<T>,               \
-        OpGtScalar<T>, OpGeScalar<T>, OpFill<T>, OpIdentity<T>, OpZeroPlus<T>, OpSgdStep<T>
+        OpGtScalar<T>, OpGeScalar<T>, OpFill<T>, OpIdentity<T>, OpZeroPlus<T>, OpSgdStep<T>, OpMseGradUnit<T>
 // f32: the dtype of the small training loops this is for
 using EwProgOps = TypeList<MXH_PROG_EW_OPS(float)>;
 

@@ -150,7 +150,9 @@ __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, ui
         } else {
             const GemmArgs g = lds_uniform<GemmArgs>(sg.tail[k].arg);
             const unsigned outputs = g.I * g.J * g.batch;
-            if (t.sub == 1) gemm_rowsdot_any<EW_BLOCK>(g, tid, part, mirror);        // the eager path's choice, made on the host
+            if (t.sub == 2) {            // one wave per output, the waves of the group taking the outputs in turn
+                for (unsigned o = tid / WAVE; o < outputs; o += EW_BLOCK / WAVE) gemm_wavedot_body<float>(g, o, (int)(tid % WAVE), mirror);
+            } else if (t.sub == 1) gemm_rowsdot_any<EW_BLOCK>(g, tid, part, mirror);        // the eager path's choice, made on the host
             else for (unsigned o = 0; o < outputs; o += 4) {
                 if (o) __syncthreads();              // the fold of the outputs before still reads `part`
                 gemm_blockdot_body<float, EW_BLOCK, 4>(g, o, outputs, tid, part, mirror);

@@ -65,7 +65,7 @@ constexpr uint32_t FUSE_SRC_MEMORY = 0xFFu, FUSE_SRC_MEMORY_LATE = 0xFEu;
 enum TailKind : uint32_t { TAIL_EW = 0, TAIL_ROW_REDUCE = 1, TAIL_DOT = 2, TAIL_MSE = 3 };
 struct TailCmd {
     uint32_t kind;
-    uint32_t sub;             // TAIL_ROW_REDUCE: the instantiation number of row_prog_sub(); TAIL_DOT: 1 = the rows form
+    uint32_t sub;             // TAIL_ROW_REDUCE: the instantiation number of row_prog_sub(); TAIL_DOT: 1 = the rows form, 2 = a wave per output
     uint32_t sync;            // before this stage: 0 nothing, 1 a barrier that orders LDS, 2 one that also waits for memory
     uint32_t fwd;             // TAIL_EW: as FuseCmd::fwd, against the stage before
     int32_t moff[2];          // TAIL_EW, input from a mirror: element offset of the input's base from that stage's output

@@ -906,35 +906,10 @@ void launch_mfma(GemmArgs g) {
 }
 
 // ---- small shapes (the per-thread and per-block dot kernels are in gemm_small.hpp) -------------------
-// One wave per output element: lanes stride over r, 4 independent partial sums per lane, then a
-// fixed shuffle tree.  For few outputs with a long reduction.
+// One wave per output element (gemm_wavedot_body in gemm_small.hpp).  For few outputs with a long reduction.
 template <class T>
 __global__ __launch_bounds__(GB) void gemm_wavedot_kernel(GemmArgs g) {
-    size_t idx = (size_t)blockIdx.x * (GB / WAVE) + threadIdx.x / WAVE;
-    size_t per = (size_t)g.I * g.J;
-    const int lane = threadIdx.x % WAVE;
-    float acc = 0.0f;
-    bool live = idx < per * g.batch;
-    if (live) {
-        uint32_t b = (uint32_t)(idx / per);
-        uint32_t rem = (uint32_t)(idx % per);
-        uint32_t i = rem / g.J, j = rem % g.J;
-        const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
-        const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
-        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-        uint32_t r = lane;
-        for (; r + 3 * WAVE < g.R; r += 4 * WAVE) {
-            a0 += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
-            a1 += Elem<T>::ld(x[(int64_t)(r + WAVE) * g.xr]) * Elem<T>::ld(y[(int64_t)(r + WAVE) * g.yr]);
-            a2 += Elem<T>::ld(x[(int64_t)(r + 2 * WAVE) * g.xr]) * Elem<T>::ld(y[(int64_t)(r + 2 * WAVE) * g.yr]);
-            a3 += Elem<T>::ld(x[(int64_t)(r + 3 * WAVE) * g.xr]) * Elem<T>::ld(y[(int64_t)(r + 3 * WAVE) * g.yr]);
-        }
-        for (; r < g.R; r += WAVE) a0 += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
-        acc = (a0 + a1) + (a2 + a3);
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, WAVE);
-    if (live && lane == 0) ((T*)g.out)[idx] = Elem<T>::st(acc);
+    gemm_wavedot_body<T>(g, (size_t)blockIdx.x * (GB / WAVE) + threadIdx.x / WAVE, threadIdx.x % WAVE, nullptr);
 }
 
 // byte range of a strided matmul operand: `rows` by `cols` elements at the given element strides
@@ -974,6 +949,14 @@ static bool fuse_block_dot(const GemmArgs& g, size_t outputs, bool rows) {
                           operand_extent(g.Y, g.R, g.yr, g.J, g.yj, g.batch, g.yb, sizeof(float))};
     const Extent out{(uintptr_t)g.out, (uintptr_t)g.out + outputs * sizeof(float)};
     return fuse_record_tail(TAIL_DOT, rows ? 1 : 0, &g, sizeof(g), in, 2, out, outputs);
+}
+
+// ... and for a handful of outputs that the dispatch gives a wave each (a reduction of a few hundred to a few thousand terms)
+static bool fuse_wave_dot(const GemmArgs& g, size_t outputs) {
+    if (!capture_open() || outputs > 16 || g.batch != 1 || !positive_strides(g)) return false;
+    const Extent in[2] = {operand_extent(g.X, g.I, g.xi, g.R, g.xr, 1, 0, sizeof(float)), operand_extent(g.Y, g.R, g.yr, g.J, g.yj, 1, 0, sizeof(float))};
+    const Extent out{(uintptr_t)g.out, (uintptr_t)g.out + outputs * sizeof(float)};
+    return fuse_record_tail(TAIL_DOT, 2, &g, sizeof(g), in, 2, out, outputs);
 }
 
 __global__ __launch_bounds__(256) void gemm_rowsdot_kernel(GemmArgs g) {
@@ -1151,7 +1134,9 @@ void gemm_dispatch(GemmArgs g) {
         MXH_LAUNCH_CHECK("gemm_thread");
         return;
     }
-    if (outputs <= 64 && g.R >= 4096) {
+    // (up to eight outputs from 1024 terms on: such a product is a stage of a captured chain's tail, where one wave per
+    // output would leave most of the work-group idle)
+    if (outputs <= 64 && (g.R >= 4096 || (outputs <= 8 && g.R >= 1024))) {
         const bool wide = blockdot_threads(g.R) == 1024;
         if constexpr (std::is_same<T, float>::value) {
             const bool small = (size_t)g.R * outputs <= PROG_MAX_ELEMS;
@@ -1177,6 +1162,10 @@ void gemm_dispatch(GemmArgs g) {
     // lane of a wave would read a cache line of its own, 74 us; the tiles below cut the reduction over the chip)
     const bool both_strided = g.xr != 1 && g.yr != 1 && g.R >= 2048 && g.I >= 32;
     if (outputs <= 4096 && (g.I < 32 || g.J < 32) && !(g.yj == 1 && g.J >= 256 && g.R >= 256) && !both_strided) {
+        if constexpr (std::is_same<T, float>::value) {
+            if (prog_recording()) prog_abandon();
+            if (fuse_wave_dot(g, outputs)) return;
+        }
         hipLaunchKernelGGL(gemm_wavedot_kernel<T>, dim3(cdiv(outputs, GB / WAVE)), dim3(GB), 0, stream(), g);
         MXH_LAUNCH_CHECK("gemm_wavedot");
         return;

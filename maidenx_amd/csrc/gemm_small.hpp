@@ -56,11 +56,56 @@ __device__ __forceinline__ void gemm_thread_body(const GemmArgs& g, unsigned bid
     const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
     const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
     float acc = 0.0f;
-    for (uint32_t r = 0; r < g.R; ++r) acc = acc + Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
+    // eight terms' operands requested together (one memory latency instead of eight), added in ascending r as before
+    constexpr int Q = 8;
+    uint32_t r = 0;
+    for (; r + Q <= g.R; r += Q) {
+        float xv[Q], yv[Q];
+#pragma unroll
+        for (int k = 0; k < Q; ++k) {
+            xv[k] = Elem<T>::ld(x[(int64_t)(r + k) * g.xr]);
+            yv[k] = Elem<T>::ld(y[(int64_t)(r + k) * g.yr]);
+        }
+#pragma unroll
+        for (int k = 0; k < Q; ++k) acc = acc + xv[k] * yv[k];
+    }
+    for (; r < g.R; ++r) acc = acc + Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
     ((T*)g.out)[idx] = Elem<T>::st(acc);
 }
 template <class T>
 __global__ __launch_bounds__(GB) void gemm_thread_kernel(GemmArgs g) { gemm_thread_body<T>(g, blockIdx.x, threadIdx.x); }
+
+// One wave per output element `idx`: lanes stride over r, 4 independent partial sums per lane, then a fixed shuffle tree.
+// Every lane of the wave calls it; `mirror` (may be null): LDS copy of the outputs, element idx.
+template <class T>
+__device__ __forceinline__ void gemm_wavedot_body(const GemmArgs& g, size_t idx, int lane, float* mirror) {
+    size_t per = (size_t)g.I * g.J;
+    float acc = 0.0f;
+    bool live = idx < per * g.batch;
+    if (live) {
+        uint32_t b = (uint32_t)(idx / per);
+        uint32_t rem = (uint32_t)(idx % per);
+        uint32_t i = rem / g.J, j = rem % g.J;
+        const T* x = (const T*)g.X + (int64_t)b * g.xb + (int64_t)i * g.xi;
+        const T* y = (const T*)g.Y + (int64_t)b * g.yb + (int64_t)j * g.yj;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        uint32_t r = lane;
+        for (; r + 3 * WAVE < g.R; r += 4 * WAVE) {
+            a0 += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
+            a1 += Elem<T>::ld(x[(int64_t)(r + WAVE) * g.xr]) * Elem<T>::ld(y[(int64_t)(r + WAVE) * g.yr]);
+            a2 += Elem<T>::ld(x[(int64_t)(r + 2 * WAVE) * g.xr]) * Elem<T>::ld(y[(int64_t)(r + 2 * WAVE) * g.yr]);
+            a3 += Elem<T>::ld(x[(int64_t)(r + 3 * WAVE) * g.xr]) * Elem<T>::ld(y[(int64_t)(r + 3 * WAVE) * g.yr]);
+        }
+        for (; r < g.R; r += WAVE) a0 += Elem<T>::ld(x[(int64_t)r * g.xr]) * Elem<T>::ld(y[(int64_t)r * g.yr]);
+        acc = (a0 + a1) + (a2 + a3);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, WAVE);
+    if (live && lane == 0) {
+        ((T*)g.out)[idx] = Elem<T>::st(acc);
+        if (mirror) mirror[idx] = acc;
+    }
+}
 
 // The same sums for Y with unit column stride and J a multiple of the 16-byte vector: a thread owns VEC neighbouring
 // outputs of one row (one vector load of Y per term, one vector store), blockIdx.y is the batch, and nothing is divided

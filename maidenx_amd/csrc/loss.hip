@@ -107,6 +107,15 @@ extern "C" void hip_mse_loss_backward_f32(size_t n, const float* pred, const flo
                                           float* grad_target) { MXH_API;
     if (!pred || !target) { set_status(ERR_INVALID, "mse_loss_backward: null buffer"); return; }
     if (n == 0 || (!grad_pred && !grad_target)) return;
+    if (!grad_loss && grad_pred && !grad_target) {
+        // the seed of backward(): an elementwise launch of two inputs with the constant folded into the functor - inside a
+        // capture it joins the fused chains, recorded and resident programs like any other
+        const size_t dims = n, unit = 1;
+        const size_t* ins[2] = {&unit, &unit};
+        const void* inp[2] = {pred, target};
+        ew_launch<OpMseGradUnit<float>>(n, 1, &dims, &unit, ins, grad_pred, inp, OpMseGradUnit<float>{(float)n});
+        return;
+    }
     const bool vec = n % 4 == 0 && aligned16(pred) && aligned16(target) && (!grad_pred || aligned16(grad_pred)) && (!grad_target || aligned16(grad_target));
     const size_t units = vec ? n / 4 : n;
     const dim3 grid((unsigned)cdiv(units, (size_t)LB));

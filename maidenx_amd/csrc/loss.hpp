@@ -21,11 +21,12 @@ struct MseArgs {
 };
 
 // One block's share (block `block` of `blocks`) of the squared differences, folded to one value in thread 0; the 256
-// threads of the block all call it.  `part`: MSE_THREADS / WAVE floats of LDS.
+// threads of the block all call it.  `part`: MSE_THREADS / WAVE floats of LDS.  `active` false: a thread of a larger
+// work-group that only takes part in the barrier (tid is then anything).
 __device__ __forceinline__ float mse_block_sum(const float* pred, const float* target, size_t n, unsigned block, unsigned blocks, unsigned tid,
-                                               float* part) {
+                                               float* part, bool active = true) {
     typedef float F4 __attribute__((ext_vector_type(4)));
-    const size_t nvec = n / 4;
+    const size_t nvec = active ? n / 4 : 0;
     float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const size_t stride = (size_t)blocks * MSE_THREADS;
     size_t v = (size_t)block * MSE_THREADS + tid;
@@ -47,15 +48,15 @@ __device__ __forceinline__ float mse_block_sum(const float* pred, const float* t
         for (int e = 0; e < 4; ++e) a[e] = a[e] + OpSquare<float>{}(OpSub<float>{}(p[e], t[e]));
     }
     float acc = (a[0] + a[1]) + (a[2] + a[3]);
-    if (block == 0 && tid < n % 4) {                       // the last n % 4 elements
+    if (active && block == 0 && tid < n % 4) {             // the last n % 4 elements
         const size_t i = nvec * 4 + tid;
         acc = acc + OpSquare<float>{}(OpSub<float>{}(pred[i], target[i]));
     }
     acc = wave_reduce<RSum>(acc);
-    if (tid % WAVE == 0) part[tid / WAVE] = acc;
+    if (active && tid % WAVE == 0) part[tid / WAVE] = acc;
     __syncthreads();
     float sum = 0.0f;
-    if (tid == 0) {
+    if (active && tid == 0) {
         sum = part[0];
 #pragma unroll
         for (int w = 1; w < MSE_THREADS / WAVE; ++w) sum = sum + part[w];

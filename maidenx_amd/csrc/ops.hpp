@@ -232,6 +232,18 @@ MXH_UNC(OpAddScalar, T, A::add(x, c))
 MXH_UNC(OpSubScalar, T, A::sub(x, c))
 MXH_UNC(OpMulScalar, T, A::mul(x, c))
 MXH_UNC(OpDivScalar, T, is_zero(c) ? (is_zero(x) ? A::zero() : A::inf()) : A::div(x, c))
+// The backward pass of the MSE loss when the gradient of the loss is the seed of backward(), 1: 0 + (((1 / n) * 2) * (p - t)),
+// every step the functor of the op sequence (crates/maidenx_nn/src/losses/mse.rs:21-29 backwards: div_scalar, mul_scalar(2),
+// mul, and the `0 + g` of sub's sum_to_shape)
+template <class T> struct OpMseGradUnit {
+    using In = T; using Out = T; static constexpr int NIN = 2;
+    T count;
+    __device__ T operator()(T p, T t) const {
+        using A = Ar<T>;
+        const T scale = OpMulScalar<T>{A::from_f32(2.0f)}(OpDivScalar<T>{count}(A::from_f32(1.0f)));
+        return A::add(A::zero(), OpMul<T>{}(scale, OpSub<T>{}(p, t)));
+    }
+};
 MXH_UNC(OpMaximumScalar, T, A::max_(x, c))
 MXH_UNC(OpMinimumScalar, T, A::min_(x, c))
 MXH_UNC(OpPow, T, A::from_f32(m_pow(F(x), F(c))))                      // (the entry point sends an exponent of 2 to OpSquare)

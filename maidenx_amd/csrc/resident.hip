@@ -9,6 +9,7 @@
 #include "fuse.hpp"
 #include "fuse_ops.hpp"
 #include "gemm_small.hpp"
+#include "loss.hpp"
 #include "mxh.hpp"
 #include "ops.hpp"
 #include "reduce_row.hpp"
@@ -171,9 +172,10 @@ __device__ __forceinline__ void res_ew(ResCmdPtr c, uint32_t flags, uint32_t uni
 // gemm_thread_body adds them.  A thread owns U units at a time and fetches Q terms of each before it adds any (terms past
 // the end re-read the first of the chunk and are not added): one memory latency per chunk instead of one per term.
 // Offsets are 32-bit element offsets (the planner checks that the operands allow it).
-template <int VEC, class PX, class PY>
+// U units a thread, Q terms of every one of them requested together
+template <int VEC, int U, int Q, class PX, class PY>
 __device__ __forceinline__ void res_dot_units(const FuseCmd& f, const FastDiv& dj, const ResOperand& out, PX X, PY Y, uint32_t units, unsigned tid, LdsByte* arena) {
-    constexpr int U = VEC == 4 ? 5 : 8, Q = 2, N = U * VEC;
+    constexpr int N = U * VEC;
     const uint32_t R = f.dims[1];
     const uint32_t xi = (uint32_t)f.is[0][0], xr = (uint32_t)f.is[0][1], yr = (uint32_t)f.is[1][0], yj = (uint32_t)f.is[1][1];
     for (uint32_t u0 = 0; u0 < units; u0 += U * RES_THREADS) {
@@ -226,10 +228,20 @@ __device__ __forceinline__ void res_dot(ResCmdPtr c, uint32_t flags, uint32_t un
     const LdsFloat* yl = (const LdsFloat*)(arena + (uint32_t)fy);
     const MemFloat* xm = (const MemFloat*)fx;
     const MemFloat* ym = (const MemFloat*)fy;
-    if (lx && ly) res_dot_units<VEC>(f, dj, out, xl, yl, units, tid, arena);
-    else if (lx) res_dot_units<VEC>(f, dj, out, xl, ym, units, tid, arena);
-    else if (ly) res_dot_units<VEC>(f, dj, out, xm, yl, units, tid, arena);
-    else res_dot_units<VEC>(f, dj, out, xm, ym, units, tid, arena);
+    // at most a unit a thread (a weight gradient's handful of outputs over a reduction of a few dozen terms): eight terms in
+    // flight, so that the reduction costs an eighth of its memory latencies; else several units a thread, two terms each
+    constexpr int UM = VEC == 4 ? 5 : 8;
+    if (units <= RES_THREADS) {
+        if (lx && ly) res_dot_units<VEC, 1, 8>(f, dj, out, xl, yl, units, tid, arena);
+        else if (lx) res_dot_units<VEC, 1, 8>(f, dj, out, xl, ym, units, tid, arena);
+        else if (ly) res_dot_units<VEC, 1, 8>(f, dj, out, xm, yl, units, tid, arena);
+        else res_dot_units<VEC, 1, 8>(f, dj, out, xm, ym, units, tid, arena);
+    } else {
+        if (lx && ly) res_dot_units<VEC, UM, 2>(f, dj, out, xl, yl, units, tid, arena);
+        else if (lx) res_dot_units<VEC, UM, 2>(f, dj, out, xl, ym, units, tid, arena);
+        else if (ly) res_dot_units<VEC, UM, 2>(f, dj, out, xm, yl, units, tid, arena);
+        else res_dot_units<VEC, UM, 2>(f, dj, out, xm, ym, units, tid, arena);
+    }
 }
 
 template <int TPR>
@@ -254,7 +266,9 @@ __device__ __forceinline__ void res_taildot_cmd(ResCmdPtr c, uint32_t flags, uns
     g.Y = res_ptr(c->p_in1, flags & RES_LDS_IN1, arena);
     g.out = res_ptr(c->p_out, flags & RES_LDS_OUT, arena);
     const unsigned outputs = g.I * g.J * g.batch;
-    if (c->sub == 1) {      // the eager path's choice, made on the host (fewer loads in flight than there: this kernel has half the registers)
+    if (c->sub == 2) {      // one wave per output, the eight waves taking the outputs in turn
+        for (unsigned o = tid / WAVE; o < outputs; o += RES_THREADS / WAVE) gemm_wavedot_body<float>(g, o, (int)(tid % WAVE), nullptr);
+    } else if (c->sub == 1) {      // the eager path's choice, made on the host (fewer loads in flight than there: this kernel has half the registers)
         if (g.I * g.J <= 3) gemm_rowsdot_any<EW_BLOCK, 8>(g, tid, part);
         else gemm_rowsdot_any<EW_BLOCK, 5>(g, tid, part);
     }
@@ -262,6 +276,17 @@ __device__ __forceinline__ void res_taildot_cmd(ResCmdPtr c, uint32_t flags, uns
         if (o) __syncthreads();              // the fold of the outputs before still reads `part`
         gemm_blockdot_body<float, EW_BLOCK, 4>(g, o, outputs, tid, part);
     }
+}
+
+// the fused MSE loss of at most 65536 elements: the eager kernel's one block, run by the first 256 threads
+__device__ __forceinline__ void res_mse_cmd(ResCmdPtr c, uint32_t flags, unsigned tid, LdsByte* arena, float* part) {
+    const MseArgs a = res_args<MseArgs>(c);
+    const float* pred = res_ptr(c->p_in0, flags & RES_LDS_IN0, arena);
+    const float* target = res_ptr(c->p_in1, flags & RES_LDS_IN1, arena);
+    float* loss = res_ptr(c->p_out, flags & RES_LDS_OUT, arena);
+    const bool active = tid < (unsigned)MSE_THREADS;
+    const float sum = mse_block_sum(pred, target, (size_t)a.n, 0, 1, tid, part, active);
+    if (tid == 0) loss[0] = OpDivScalar<float>{(float)(size_t)a.n}(sum);
 }
 
 // Dynamic LDS: the arena.
@@ -290,6 +315,8 @@ __global__ __launch_bounds__(RES_THREADS) void resident_kernel(const ResCmd* cmd
             else res_dot<1>(c, flags, units, tid, arena);
         } else if (kind == RES_ROW) {
             res_row_cmd(c, flags, tid, arena, part);
+        } else if (kind == RES_MSE) {
+            res_mse_cmd(c, flags, tid, arena, part);
         } else {
             res_taildot_cmd(c, flags, tid, arena, part);
         }
@@ -381,6 +408,10 @@ void** operand_field(ResCmd& c, int k) {
     if (c.kind == RES_ROW) {
         RowProgArgs* a = (RowProgArgs*)c.arg;
         return k == 0 ? &a->out : (void**)&a->in;
+    }
+    if (c.kind == RES_MSE) {
+        MseArgs* a = (MseArgs*)c.arg;
+        return k == 0 ? (void**)&a->loss : (k == 1 ? (void**)&a->pred : (void**)&a->target);
     }
     GemmArgs* g = (GemmArgs*)c.arg;
     return k == 0 ? &g->out : (k == 1 ? (void**)&g->X : (void**)&g->Y);
@@ -640,7 +671,7 @@ bool res_build(const std::vector<ResRecord>& recs, ResProgram& out) {
         if (ew)
             for (int k = 1; k <= nin; ++k)
                 if (p.acc[k].overlaps(p.acc[0]) && !p.acc[k].same_walk(p.acc[0])) return false;
-        if (r.kind == RES_ROW || r.kind == RES_TAILDOT) {      // the fold's own LDS is reused from command to command
+        if (r.kind == RES_ROW || r.kind == RES_TAILDOT || r.kind == RES_MSE) {      // the fold's own LDS is reused from command to command
             AccessKey& a = p.acc[p.nacc++];
             a.space = 2;
             a.lo = 0;

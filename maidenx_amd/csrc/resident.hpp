@@ -5,7 +5,7 @@
 // microseconds each - for dependencies, not for work: a result written by one kernel is read by the next through
 // memory, and a work-group that waits for another pays a device-scope release.  When every launch of a capture is one
 // the fused chains would take (f32 elementwise over at most two collapsed dims, the one-thread-per-output matmul, a row
-// sum that one work-group does, the few-output long-reduction matmul) and small, the capture is recorded as a list of
+// sum that one work-group does, the few-output long-reduction matmul, the fused MSE loss) and small, the capture is recorded as a list of
 // commands instead, and a replay is ONE launch of ONE 512-thread work-group that
 //   * keeps every tensor the commands write in LDS for as long as it is alive (a liveness plan made on the host from
 //     the commands' operand ranges and from the caller's hints that a buffer was released, hip_buffer_discard): a
@@ -29,7 +29,7 @@
 
 namespace mxh {
 
-enum ResKind : uint32_t { RES_EW = 0, RES_DOT = 1, RES_ROW = 2, RES_TAILDOT = 3 };
+enum ResKind : uint32_t { RES_EW = 0, RES_DOT = 1, RES_ROW = 2, RES_TAILDOT = 3, RES_MSE = 4 };
 constexpr uint32_t RES_BARRIER = 1u;          // ResCmd::flags: a work-group barrier before the command
 constexpr uint32_t RES_VEC = 2u;              // elementwise / matmul producer: a unit is a 16-byte vector
 constexpr uint32_t RES_FAST = 8u;             // elementwise: every operand is one scalar or walked linearly (step[] is valid)
@@ -43,10 +43,11 @@ constexpr size_t RES_LDS_BYTES = (160u << 10) - 256;  // dynamic LDS of the work
 constexpr size_t RES_MAX_REGION = 64u << 10;          // larger tensors stay in memory
 // Elements one command may span: the hard limit, and the default of hip_graph_set_resident().  One work-group's
 // instruction stream is what a command costs: about 0.7 us for up to 2048 elements (one vector a thread), 1.5 us for
-// 10000 - where the fused chains, which spread a launch over ten work-groups, are ahead again (the README step: 52 us a
-// pass here, 42 us as three chains).
+// 10000 - where the fused chains, which spread a launch over ten work-groups, are ahead again.  The README step
+// (Linear(3 -> 1) + MSE + SGD) on n rows, us per step here / as chains: n = 256 12.4 / 17.5, 1000 15.8 / 22.8, 2000 18.3 /
+// 24.3, 3000 23.6 / 26.7, 5000 26.3 / 24.0, 10000 34.6 / 26.6 - the default keeps tensors of up to 8192 elements here.
 constexpr size_t RES_MAX_ELEMS = 1u << 16;
-constexpr size_t RES_DEFAULT_ELEMS = 4096;
+constexpr size_t RES_DEFAULT_ELEMS = 8192;
 constexpr uint32_t RES_MODE_LINEAR = 0, RES_MODE_SCALAR = 1, RES_MODE_2D = 2;
 
 // The first 64 bytes are all an elementwise command in its fast form needs: one scalar load.
@@ -58,7 +59,7 @@ struct alignas(64) ResCmd {
     uint32_t mode;                            // byte k: how operand k is addressed in the general form (RES_MODE_*)
     FastDiv div_inner;                        // elementwise over two dims: the inner extent; matmul producer: J
     uint32_t pad;
-    alignas(16) unsigned char arg[FUSE_TAIL_ARG_BYTES];      // FuseCmd (RES_EW, RES_DOT), RowProgArgs, GemmArgs
+    alignas(16) unsigned char arg[FUSE_TAIL_ARG_BYTES];      // FuseCmd (RES_EW, RES_DOT), RowProgArgs, GemmArgs, MseArgs
 };
 static_assert(sizeof(ResCmd) == 192 && offsetof(ResCmd, mode) == 60, "the fast form is the first 64 bytes");
 

@@ -427,11 +427,11 @@ bool fuse_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, const Ex
 
 bool fuse_record_tail(uint32_t kind, uint32_t sub, const void* arg, size_t arg_bytes, const Extent* in, int nin, const Extent& out, size_t outputs) {
     if (res_accepting()) {
-        bool fits = arg_bytes <= (size_t)FUSE_TAIL_ARG_BYTES && nin >= 1 && nin <= 2 && (kind == TAIL_ROW_REDUCE || kind == TAIL_DOT);
+        bool fits = arg_bytes <= (size_t)FUSE_TAIL_ARG_BYTES && nin >= 1 && nin <= 2 && (kind == TAIL_ROW_REDUCE || kind == TAIL_DOT || kind == TAIL_MSE);
         for (int j = 0; j < nin && fits; ++j) fits = (in[j].hi - in[j].lo) / sizeof(float) <= g_res_elems;
         if (fits) {
             ResRecord r;
-            r.kind = kind == TAIL_ROW_REDUCE ? RES_ROW : RES_TAILDOT;
+            r.kind = kind == TAIL_ROW_REDUCE ? RES_ROW : kind == TAIL_DOT ? RES_TAILDOT : RES_MSE;
             r.tail_kind = kind;
             r.sub = sub;
             r.outputs = outputs;

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import maidenx_amd.lib as L
-from test_gpu_program import Seq, elementwise_sequence, linear_step, random_sequence_with_aliasing, u64
+from test_gpu_program import Seq, elementwise_sequence, fused_nn_step, linear_step, random_sequence_with_aliasing, u64
 
 pytestmark = pytest.mark.gpu
 
@@ -21,7 +21,7 @@ def lib():
 
 @pytest.fixture(autouse=True)
 def resident_programs_of_any_size(lib):
-    """By default a capture stays a resident step program only while its tensors have at most 4096 elements (beyond that
+    """By default a capture stays a resident step program only while its tensors have at most 8192 elements (beyond that
     the fused chains are faster); these tests take the mechanism to its limits."""
     was = lib.hip_graph_set_resident(1 << 16)
     yield
@@ -102,9 +102,30 @@ def test_whole_training_step(lib, n, feats):
     r = np.random.default_rng(100 + n + feats)
     seq = Seq(lib)
     linear_step(lib, seq, n, feats, r)
-    # (the weight gradient of 300 rows is a one-wave-per-output product, which has no resident command)
-    cmds, lds, bars = resident_replay_equals_eager(lib, seq, expect=n != 300)
-    assert cmds == (15 if n != 300 else 0)
+    # (the weight gradient of 300 rows is a one-wave-per-output product: a command as well)
+    cmds, lds, bars = resident_replay_equals_eager(lib, seq)
+    assert cmds == 15
+
+
+@pytest.mark.parametrize("n,feats", [(10000, 3), (4096, 4), (5001, 1), (64, 2), (7, 2)])
+def test_training_step_with_the_fused_loss_and_sgd_calls(lib, n, feats):
+    """The same step with hip_mse_loss_f32 (a command of its own: the eager kernel's one block run by the first 256
+    threads), hip_mse_loss_backward_f32 without a gradient tensor (the seed of backward(): an elementwise functor) and
+    hip_sgd_step_f32 (an elementwise functor in place): one resident program, the eager bytes."""
+    r = np.random.default_rng(500 + n + feats)
+    seq = Seq(lib)
+    fused_nn_step(lib, seq, n, feats, r, seeded=False)
+    cmds, lds, bars = resident_replay_equals_eager(lib, seq)
+    assert cmds == 11
+
+
+def test_a_seeded_loss_gradient_hands_the_capture_to_the_chains(lib):
+    """hip_mse_loss_backward_f32 with a gradient tensor has no resident command: the launches kept so far go to the fused
+    chains and the replay is still the eager bytes."""
+    r = np.random.default_rng(9)
+    seq = Seq(lib)
+    fused_nn_step(lib, seq, 4096, 4, r, seeded=True)
+    resident_replay_equals_eager(lib, seq, expect=False)
 
 
 def training_loop(lib, n, feats, seed, discard):
@@ -230,10 +251,10 @@ def test_switch_and_size_limit(lib):
     was = lib.hip_graph_set_resident(0)
     try:
         resident_replay_equals_eager(lib, one(100), expect=False, replays=1)
-        assert lib.hip_graph_set_resident(4096) == 0          # the default limit
-        resident_replay_equals_eager(lib, one(4096), expect=True, replays=1)
-        resident_replay_equals_eager(lib, one(4100), expect=False, replays=1)
-        assert lib.hip_graph_set_resident(1 << 20) == 4096 and lib.hip_graph_set_resident(5) == 1 << 16
+        assert lib.hip_graph_set_resident(8192) == 0          # the default limit
+        resident_replay_equals_eager(lib, one(8192), expect=True, replays=1)
+        resident_replay_equals_eager(lib, one(8196), expect=False, replays=1)
+        assert lib.hip_graph_set_resident(1 << 20) == 8192 and lib.hip_graph_set_resident(5) == 1 << 16
     finally:
         lib.hip_graph_set_resident(was)
     resident_replay_equals_eager(lib, one(100), expect=True, replays=1)
