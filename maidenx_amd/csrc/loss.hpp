@@ -30,15 +30,16 @@ __device__ __forceinline__ float mse_block_sum(const float* pred, const float* t
     float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const size_t stride = (size_t)blocks * MSE_THREADS;
     size_t v = (size_t)block * MSE_THREADS + tid;
-    for (; v + 3 * stride < nvec; v += 4 * stride) {      // four pairs of loads in flight
-        F4 p[4], t[4];
+    constexpr int U = 8;                                   // pairs of loads in flight (the terms are added in ascending v whatever U is)
+    for (; v + (U - 1) * stride < nvec; v += U * stride) {
+        F4 p[U], t[U];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < U; ++k) {
             p[k] = ((const F4*)pred)[v + k * stride];
             t[k] = ((const F4*)target)[v + k * stride];
         }
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
+        for (int k = 0; k < U; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) a[e] = a[e] + OpSquare<float>{}(OpSub<float>{}(p[k][e], t[k][e]));
     }
