@@ -52,10 +52,11 @@ struct FuseHead {
     FastDiv div_inner;
     size_t nvec;
     uint32_t* ticket;
-    uint32_t prefetch, blocks, pad[2];
+    uint32_t prefetch, blocks, nwide, wide_m, wide_nvec, pad[1];
 };
 static_assert(sizeof(FuseHead) <= offsetof(FuseGroup, cmd) && offsetof(FuseHead, ticket) == offsetof(FuseGroup, ticket) &&
-              offsetof(FuseHead, blocks) == offsetof(FuseGroup, blocks), "FuseHead mirrors FuseGroup");
+              offsetof(FuseHead, blocks) == offsetof(FuseGroup, blocks) && offsetof(FuseHead, wide_nvec) == offsetof(FuseGroup, wide_nvec),
+              "FuseHead mirrors FuseGroup");
 // the fields of a TailCmd ahead of its argument block
 struct TailHead {
     uint32_t kind, sub, sync, fwd;
@@ -90,26 +91,32 @@ __device__ __forceinline__ void tail_row(uint32_t vec, const RowProgArgs& a, uns
 }
 
 __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, uint32_t want, unsigned tid, float* part, float* mir, float* pre) {
-    // `want`: which (stage, input) pairs are fetched up front
+    // `want`: which (stage, input) pairs are fetched up front; they go to LDS when the first elementwise stage comes up,
+    // so that the stages before it overlap the fetch (volatile: the loads are issued here, not where their values are used)
+    float got[2 * FUSE_MAX_TAIL];
+#pragma unroll
+    for (int q = 0; q < 2 * FUSE_MAX_TAIL; ++q) got[q] = 0.0f;
     if (want) {
-        float got[2 * FUSE_MAX_TAIL];
 #pragma unroll
         for (int k = 0; k < FUSE_MAX_TAIL; ++k) {
-            got[2 * k] = got[2 * k + 1] = 0.0f;
             if ((want >> (2 * k)) & 3u) {
                 const FuseCmd c = lds_uniform<FuseCmd>(sg.tail[k].arg);
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    if (((want >> (2 * k + j)) & 1u) && tid < c.nel) got[2 * k + j] = gl(c.in[j])[tail_elem(c, c.is[j][0], c.is[j][1], tid)];
+                    if (((want >> (2 * k + j)) & 1u) && tid < c.nel) got[2 * k + j] = *(volatile GCFloat*)(gl(c.in[j]) + tail_elem(c, c.is[j][0], c.is[j][1], tid));
             }
         }
-#pragma unroll
-        for (int q = 0; q < 2 * FUSE_MAX_TAIL; ++q)
-            if (want & (1u << q)) pre[q * TAIL_SLOT + tid] = got[q];
     }
+    bool fetched = want == 0;
     float prev = 0.0f;            // what this thread wrote in the stage before (an elementwise stage of the same layout)
     for (uint32_t k = 0; k < ntail; ++k) {
         const TailHead t = lds_uniform<TailHead>(&sg.tail[k]);
+        if (t.kind == TAIL_EW && !fetched) {
+#pragma unroll
+            for (int q = 0; q < 2 * FUSE_MAX_TAIL; ++q)
+                if (want & (1u << q)) pre[q * TAIL_SLOT + tid] = got[q];        // (read back by this thread only)
+            fetched = true;
+        }
         if (t.sync == 2) __syncthreads();
         else if (t.sync == 1) lds_barrier();
         float* mirror = t.mirrored ? mir + k * TAIL_SLOT : nullptr;
@@ -161,6 +168,111 @@ __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, ui
     }
 }
 
+// ---- the members of the parallel phase --------------------------------------------------------------------------
+// A matmul producer at unit `u` of its flat output space: one output per element, r ascending, multiply and add
+// unfused (gemm_thread_body's order).  `own`: when the left operand is a first-space member's staged output (a wide
+// member of one term, c.src names the member), own[member * EW_BLOCK * VEC + row - row0] holds row `row` of it
+// (row0: the first row this work-group staged).
+template <int VEC>
+__device__ __forceinline__ void member_dot(const FuseCmd& c, uint32_t u, const float* own, uint32_t row0, AVec<float, VEC>& r) {
+    const uint32_t J = c.dims[0], R = c.dims[1];
+    const uint32_t from = c.src & 0xFFu;
+    uint32_t row[VEC], col[VEC];
+    row[0] = (u * VEC) / J;
+    col[0] = u * VEC - row[0] * J;
+#pragma unroll
+    for (int e = 1; e < VEC; ++e) {
+        col[e] = col[e - 1] + 1;
+        row[e] = row[e - 1];
+        if (col[e] == J) { col[e] = 0; ++row[e]; }
+    }
+    if (own && from != FUSE_SRC_MEMORY) {
+        float y[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y[e] = gl(c.in[1])[(int64_t)col[e] * c.is[1][1]];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f + own[from * (EW_BLOCK * VEC) + (row[e] - row0)] * y[e];
+        return;
+    }
+    // the terms of four steps of every element are requested together (steps past the end re-read the last term and
+    // are not added): a thread waits once per four terms, not once per term and element
+    constexpr int Q = 4;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+    for (uint32_t q0 = 0; q0 < R; q0 += Q) {
+        float xv[VEC][Q], yv[VEC][Q];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            GCFloat* x = gl(c.in[0]) + (int64_t)row[e] * c.is[0][0];
+            GCFloat* y = gl(c.in[1]) + (int64_t)col[e] * c.is[1][1];
+#pragma unroll
+            for (int t = 0; t < Q; ++t) {
+                const uint32_t qq = q0 + t < R ? q0 + t : R - 1;
+                xv[e][t] = x[(int64_t)qq * c.is[0][1]];
+                yv[e][t] = y[(int64_t)qq * c.is[1][0]];
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < Q; ++t)
+            if (q0 + t < R)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] = acc[e] + xv[e][t] * yv[e][t];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) r.v[e] = acc[e];
+}
+// An elementwise member (FUSE_OP_MSE_BACKWARD included) at the VEC elements that start at coordinates (c0, c1).  `r`
+// comes in as what the member before wrote at these elements and goes out as this member's values; an input that is
+// an earlier member's output is read from that member's staging slot, number `member * slot_mul + slot_add`.
+template <int VEC>
+__device__ __forceinline__ void member_ew(const FuseCmd& c, uint32_t ndims, uint32_t c0, uint32_t c1, const AVec<float, VEC>* staged,
+                                          uint32_t slot_mul, int slot_add, AVec<float, VEC>& r) {
+    float val[2][VEC];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (j >= (int)c.nin) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val[j][e] = 0.0f;
+            continue;
+        }
+        if (c.fwd & (1u << j)) {         // the value is still in registers
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val[j][e] = r.v[e];
+            continue;
+        }
+        const uint32_t from = (c.src >> (8 * j)) & 0xFFu;
+        if (from != FUSE_SRC_MEMORY) {   // an earlier member's output, element for element: still staged
+            const AVec<float, VEC> t = staged[(uint32_t)((int)(from * slot_mul) + slot_add) * EW_BLOCK];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val[j][e] = t.v[e];
+            continue;
+        }
+        const int64_t s = ndims == 2 ? c.is[j][1] : c.is[j][0];
+        GCFloat* src = gl(c.in[j]) + (ndims == 2 ? (int64_t)c0 * c.is[j][0] : 0) + (int64_t)c1 * s;
+        if (VEC > 1 && s == 1) {
+            const AVec<float, VEC> t = gload<VEC>(src);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val[j][e] = t.v[e];
+        } else if (s == 0) {
+            const float t = src[0];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val[j][e] = t;
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val[j][e] = src[(int64_t)e * s];
+        }
+    }
+    if (c.op == FUSE_OP_MSE_BACKWARD) {
+        const uint64_t seed = ((uint64_t)c.payload[1] << 32) | c.payload[0];      // (0: the gradient of the loss is 1)
+        const float scale = mse_grad_scale(seed ? gl((const void*)seed)[0] : 1.0f, (float)c.nel);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = mse_grad(scale, val[0][e], val[1][e]);
+    } else {
+        fuse_apply<VEC>(c.op, val[0], val[1], r.v, c.payload);
+    }
+}
+
 // ---- the chain kernel ----------------------------------------------------------------------------------------
 template <int VEC>
 __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
@@ -187,92 +299,75 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
     // that misses its cache, a microsecond each time.
     const FuseHead h = lds_uniform<FuseHead>(&sg);
     const size_t v = (size_t)blockIdx.x * EW_BLOCK + threadIdx.x;
-    if (v < h.nvec) {
-        // coordinates of this thread's first element over (outer, inner); one dim: everything is "inner"
-        uint32_t c0 = 0, c1 = (uint32_t)v * VEC;
-        const uint32_t ndims = h.ndims;
-        if (ndims == 2) fd_divmod((uint32_t)v * VEC, h.div_inner, c0, c1);
-        AVec<float, VEC>* staged = (AVec<float, VEC>*)pool + threadIdx.x;      // + member * EW_BLOCK
-        float** where = (float**)(pool + FUSE_MAX_CMDS * EW_BLOCK * VEC) + threadIdx.x;      // where each staged output goes
-        AVec<float, VEC> r;          // what the previous member wrote at this thread's elements
+    AVec<float, VEC>* staged = (AVec<float, VEC>*)pool + threadIdx.x;      // + slot * EW_BLOCK
+    float** where = (float**)(pool + FUSE_MAX_CMDS * EW_BLOCK * VEC) + threadIdx.x;      // where each staged output goes
+    // One loop over the members of the first space, then over the rounds of the wide space (round-major: a member
+    // then finds what the member before it wrote, same round, in registers) - one copy of the member code, so that
+    // what the first rounds bring into the instruction cache serves the later ones.
+    const uint32_t m = h.wide_m, items = h.n + h.nwide * m;
+    const uint32_t slots = items;
+    AVec<float, VEC> r;          // what the previous member wrote at this thread's elements
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f;
-        for (uint32_t k = 0; k < h.n; ++k) {
-            const FuseCmd c = lds_uniform<FuseCmd>(&sg.cmd[k]);
-            if (c.op == FUSE_OP_DOT) {
-                // one output per element, r ascending, multiply and add unfused: gemm_thread_body's order
-                const uint32_t J = c.dims[0], R = c.dims[1];
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const uint32_t idx = (uint32_t)v * VEC + e;
-                    const uint32_t i = idx / J, j = idx - i * J;
-                    GCFloat* x = gl(c.in[0]) + (int64_t)i * c.is[0][0];
-                    GCFloat* y = gl(c.in[1]) + (int64_t)j * c.is[1][1];
-                    float acc = 0.0f;
-                    for (uint32_t q = 0; q < R; ++q) acc = acc + x[(int64_t)q * c.is[0][1]] * y[(int64_t)q * c.is[1][0]];
-                    r.v[e] = acc;
-                }
-            } else {
-                float val[2][VEC];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if (j >= (int)c.nin) {
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) val[j][e] = 0.0f;
-                        continue;
-                    }
-                    if (c.fwd & (1u << j)) {         // the value is still in registers
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) val[j][e] = r.v[e];
-                        continue;
-                    }
-                    const uint32_t from = (c.src >> (8 * j)) & 0xFFu;
-                    if (from != FUSE_SRC_MEMORY) {   // an earlier member's output, element for element: still staged
-                        const AVec<float, VEC> t = staged[from * EW_BLOCK];
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) val[j][e] = t.v[e];
-                        continue;
-                    }
-                    const int64_t s = ndims == 2 ? c.is[j][1] : c.is[j][0];
-                    GCFloat* src = gl(c.in[j]) + (ndims == 2 ? (int64_t)c0 * c.is[j][0] : 0) + (int64_t)c1 * s;
-                    if (VEC > 1 && s == 1) {
-                        const AVec<float, VEC> t = gload<VEC>(src);
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) val[j][e] = t.v[e];
-                    } else if (s == 0) {
-                        const float t = src[0];
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) val[j][e] = t;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) val[j][e] = src[(int64_t)e * s];
-                    }
-                }
-                if (c.op == FUSE_OP_MSE_BACKWARD) {
-                    const uint64_t seed = ((uint64_t)c.payload[1] << 32) | c.payload[0];      // (0: the gradient of the loss is 1)
-                    const float scale = mse_grad_scale(seed ? gl((const void*)seed)[0] : 1.0f, (float)c.nel);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) r.v[e] = mse_grad(scale, val[0][e], val[1][e]);
-                } else {
-                    fuse_apply<VEC>(c.op, val[0], val[1], r.v, c.payload);
-                }
-            }
-            staged[k * EW_BLOCK] = r;
-            where[k * EW_BLOCK] = (float*)c.out + (ndims == 2 ? (int64_t)c0 * c.os[0] + (int64_t)c1 * c.os[1] : (int64_t)c1 * c.os[0]);
+    for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f;
+    uint32_t c0 = 0, c1 = (uint32_t)v * VEC;      // first space: coordinates over (outer, inner); one dim: everything is "inner"
+    if (h.ndims == 2) fd_divmod((uint32_t)v * VEC, h.div_inner, c0, c1);
+    const uint32_t row0 = (uint32_t)blockIdx.x * EW_BLOCK * VEC;       // the first element this work-group stages of every member
+    uint32_t k = 0, q = 0;
+    for (uint32_t it = 0; it < items; ++it) {
+        const bool first = it < h.n;
+        if (it == h.n) {
+            lds_barrier();      // the group's staged first-space outputs are readable by all its threads
+            k = h.n;
         }
+        // wide space: this work-group's threads take its units [EW_BLOCK m w, EW_BLOCK m (w + 1)), m rounds of one unit a thread
+        const uint32_t unit = first ? (uint32_t)v : ((uint32_t)blockIdx.x * m + q) * EW_BLOCK + threadIdx.x;
+        const uint32_t slot = first ? k : h.n + (k - h.n) * m + q;
+        const FuseCmd c = lds_uniform<FuseCmd>(&sg.cmd[k]);
+        float* dst = nullptr;
+        if (unit < (first ? h.nvec : (size_t)h.wide_nvec)) {
+            const uint32_t ndims = first ? h.ndims : 1u;
+            const uint32_t u0 = first ? c0 : 0u, u1 = first ? c1 : unit * VEC;
+            if (c.op == FUSE_OP_DOT) member_dot<VEC>(c, unit, first ? nullptr : pool, row0, r);
+            else member_ew<VEC>(c, ndims, u0, u1, staged, first ? 1u : m, first ? 0 : (int)(h.n + q) - (int)(h.n * m), r);
+            staged[slot * EW_BLOCK] = r;
+            dst = (float*)c.out + (ndims == 2 ? (int64_t)u0 * c.os[0] + (int64_t)u1 * c.os[1] : (int64_t)u1 * c.os[0]);
+        }
+        where[slot * EW_BLOCK] = dst;
+        if (c.fwd & FUSE_NEXT_IS_ZERO_PLUS) {
+            // the pass that accumulates a gradient for the first time, `0 + g`: made here from the registers, for the
+            // price of reading where it goes instead of a member's whole interpretation
+            struct OutOf { void* out; const void* in[2]; int64_t os[2]; };
+            const OutOf n = lds_uniform<OutOf>(&sg.cmd[k + 1]);
+            const uint32_t slot2 = first ? slot + 1 : slot + m;
+            float* dst2 = nullptr;
+            if (dst) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) r.v[e] = OpZeroPlus<float>{}(r.v[e]);
+                staged[slot2 * EW_BLOCK] = r;
+                const uint32_t u0 = first ? c0 : 0u, u1 = first ? c1 : unit * VEC;
+                dst2 = (float*)n.out + (first && h.ndims == 2 ? (int64_t)u0 * n.os[0] + (int64_t)u1 * n.os[1] : (int64_t)u1 * n.os[0]);
+            }
+            where[slot2 * EW_BLOCK] = dst2;
+            ++k;
+            ++it;
+        }
+        ++k;
+        if (!first && k == h.n + h.nwide) { k = h.n; ++q; }
+    }
+    {
         // every member's output to memory, in member order (a later member may write where an earlier one did)
-        for (uint32_t k0 = 0; k0 < h.n; k0 += 4) {
+        for (uint32_t k0 = 0; k0 < slots; k0 += 4) {
             AVec<float, VEC> o[4];
             float* dst[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const uint32_t k = k0 + i < h.n ? k0 + i : k0;
+                const uint32_t k = k0 + i < slots ? k0 + i : k0;
                 o[i] = staged[k * EW_BLOCK];
                 dst[i] = where[k * EW_BLOCK];
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                if (k0 + i < h.n) {
+                if (k0 + i < slots && dst[i]) {
                     gstore<VEC>(gl(dst[i]), o[i]);
                 }
             }

@@ -14,6 +14,14 @@
 //     earlier members write, nor may a later member write them;
 //   * the backward pass of the fused MSE loss joins as an elementwise member of two inputs; the one value every thread
 //     reads besides (the gradient of the loss) is held to the rule of a matmul's operands.
+//   A second, WIDE space of m times as many units (m = 2..4) may follow the first: work-group w, which owns units
+//   [256 w, 256 w + 256) of the first space, then owns units [256 m w, 256 m (w + 1)) of the wide one.  Its members run
+//   after a work-group barrier that follows all members of the first space, so a wide member may read what its OWN
+//   work-group's threads wrote there: the outer product [N,1] x [1,m] (a matmul producer of one term, the input
+//   gradient of a layer with one output feature) whose left operand is, row for row, a first-space member's output
+//   takes its rows i = idx / m - the work-group's own - from the staged outputs.  Apart from that a wide member
+//   touches nothing a first-space member writes and writes nothing one reads, and among themselves wide members keep
+//   the rule above.  Once a wide member has joined, the first space takes no more members.
 // Serial phase ("tail") - stages run in order by the work-group that finishes the parallel phase last (every group
 // publishes its writes, then draws a ticket; the last ticket continues, the others exit, nobody waits):
 //   * elementwise launches of at most 256 elements (a bias, a 3-element weight, a loss), any shapes, any overlaps;
@@ -34,7 +42,8 @@
 
 namespace mxh {
 
-constexpr int FUSE_MAX_CMDS = 16;          // members of the parallel phase
+constexpr int FUSE_MAX_CMDS = 16;          // members of the parallel phase (staging slots: a wide member takes wide_m)
+constexpr int FUSE_MAX_WIDE = 4;           // most units of the wide space per unit of the first
 constexpr int FUSE_MAX_TAIL = 12;          // stages of the serial phase
 constexpr uint32_t FUSE_OP_DOT = 0xD07u;   // FuseCmd::op of a matmul producer (the other values index EwProgOps)
 // FuseCmd::op of the fused MSE loss's backward pass (loss.hpp): out = 0 + ((g / nel) * 2) * (in0 - in1), where g is the
@@ -50,7 +59,8 @@ struct FuseCmd {
     int64_t is[2][2];         // the same for each input; FUSE_OP_DOT: {output row, reduction} of X, {reduction, output column} of Y
     uint32_t op;              // position of the functor in EwProgOps, FUSE_OP_DOT or FUSE_OP_MSE_BACKWARD
     uint32_t nin;
-    uint32_t fwd;             // bit j: input j is, element for element, what the previous member wrote (taken from registers)
+    uint32_t fwd;             // bit j: input j is, element for element, what the previous member wrote (taken from registers);
+                              // FUSE_NEXT_IS_ZERO_PLUS: the member after this one is `0 + this one's output`, made along with it
     uint32_t ndims;           // the member's own space: only read in the tail
     uint32_t dims[2];         // FUSE_OP_DOT: {output columns, reduction length}
     uint32_t nel;
@@ -61,6 +71,7 @@ struct FuseCmd {
     uint32_t src;
     uint32_t payload[2];      // the functor's state (a scalar constant), bit for bit
 };
+constexpr uint32_t FUSE_NEXT_IS_ZERO_PLUS = 1u << 8;
 constexpr uint32_t FUSE_SRC_MEMORY = 0xFFu, FUSE_SRC_MEMORY_LATE = 0xFEu;
 enum TailKind : uint32_t { TAIL_EW = 0, TAIL_ROW_REDUCE = 1, TAIL_DOT = 2, TAIL_MSE = 3 };
 struct TailCmd {
@@ -83,7 +94,10 @@ struct alignas(16) FuseGroup {
     uint32_t* ticket;         // zero between launches: counts the work-groups that have finished the parallel phase
     uint32_t prefetch;        // bit 2k+j: input j of tail stage k is fetched from memory when the tail starts
     uint32_t blocks;          // work-groups of the launch
-    uint32_t pad[2];
+    uint32_t nwide;           // members of the wide space: cmd[n .. n + nwide); n + nwide * wide_m staging slots in all
+    uint32_t wide_m;          // units of the wide space per unit of the first
+    uint32_t wide_nvec;       // units of the wide space (= wide_m * nvec)
+    uint32_t pad[1];
     alignas(16) FuseCmd cmd[FUSE_MAX_CMDS];
     alignas(16) TailCmd tail[FUSE_MAX_TAIL];
 };

@@ -10,6 +10,7 @@
 #include <thread>
 #include <vector>
 
+#include "ew_registry.hpp"
 #include "fuse.hpp"
 #include "mxh.hpp"
 #include "resident.hpp"
@@ -107,6 +108,7 @@ static void fuse_flush() {
     fuse_launch(g_fuse, (void*)g_capture_stream);
     ++g_fuse_nodes;
     g_fuse.n = 0;
+    g_fuse.nwide = g_fuse.wide_m = g_fuse.wide_nvec = 0;
     g_fuse.ntail = 0;
     g_lds_from = g_mem_from = 0;
 }
@@ -149,11 +151,22 @@ static bool clear_of_tail(const ParMember& m, uint32_t nin) {
     return true;
 }
 // ... and against the earlier members of the parallel phase: every overlap must be element for element, so that a
-// thread only meets its own data.
-static bool clear_of_members(const FuseCmd& c, const ParMember& m, uint32_t ndims) {
-    for (uint32_t k = 0; k < g_fuse.n; ++k) {
+// thread only meets its own data.  `wide`: the newcomer belongs to the wide space, where this holds against the wide
+// members; of the first space's members it may only read an output as the rows of a one-term product (`own_rows`: the
+// member it does that with, or -1), and otherwise shares no byte with what they write, nor writes what they read.
+static bool clear_of_members(const FuseCmd& c, const ParMember& m, uint32_t ndims, bool wide, int own_rows) {
+    const uint32_t members = g_fuse.n + g_fuse.nwide;
+    for (uint32_t k = 0; k < members; ++k) {
         const FuseCmd& e = g_fuse.cmd[k];
         const ParMember& pe = g_par[k];
+        if (wide && k < g_fuse.n) {
+            for (uint32_t j = 0; j < c.nin; ++j)
+                if (m.in[j].overlaps(pe.out) && !(j == 0 && (int)k == own_rows)) return false;
+            if (m.out.overlaps(pe.out) || m.out.overlaps(pe.extra) || m.extra.overlaps(pe.out)) return false;
+            for (uint32_t j = 0; j < e.nin; ++j)
+                if (m.out.overlaps(pe.in[j])) return false;
+            continue;
+        }
         // read after write
         for (uint32_t j = 0; j < c.nin; ++j)
             if (m.in[j].overlaps(pe.out) && (m.across[j] || !same_mapping(c.in[j], c.is[j], e.out, e.os, ndims))) return false;
@@ -174,18 +187,54 @@ static void open_space(uint32_t ndims, const uint32_t* dims, bool vec, size_t nv
     g_fuse.dims[0] = dims[0];
     g_fuse.dims[1] = ndims == 2 ? dims[1] : 1;
     g_fuse.div_inner = make_fastdiv(g_fuse.dims[ndims - 1]);
+    g_fuse.nwide = g_fuse.wide_m = g_fuse.wide_nvec = 0;
     g_fuse_elem_bytes = elem_bytes;
+}
+// The first-space member whose output is, row for row, the left operand of the one-term product `c` over `m` columns
+// (the latest that writes any of it), -1 when there is none, -2 when the operand meets such outputs in any other way.
+static int own_rows_member(const FuseCmd& c, const ParMember& m, uint32_t wide_m) {
+    for (int k = (int)g_fuse.n - 1; k >= 0; --k) {
+        if (!m.in[0].overlaps(g_par[k].out)) continue;
+        const FuseCmd& e = g_fuse.cmd[k];
+        const bool rows = c.op == FUSE_OP_DOT && c.dims[1] == 1 && c.dims[0] == wide_m && c.in[0] == (const void*)e.out && c.is[0][0] == 1 &&
+                          e.os[0] == 1 && m.in[0].lo == g_par[k].out.lo && m.in[0].hi == g_par[k].out.hi;
+        return rows ? k : -2;
+    }
+    return -1;
 }
 // Adds a member to the parallel phase (joining the open chain when it may, closing it and opening a new one otherwise).
 static void add_member(const FuseCmd& c, const ParMember& m, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
-    bool join = (g_fuse.n > 0 || g_fuse.ntail > 0) && g_fuse.n < (uint32_t)FUSE_MAX_CMDS;
-    if (join && g_fuse.n > 0)
-        join = g_fuse.ndims == ndims && g_fuse.vec == (vec ? 1u : 0u) && g_fuse.nvec == nvec && g_fuse.dims[0] == dims[0] &&
-               (ndims == 1 || g_fuse.dims[1] == dims[1]) && g_fuse_elem_bytes == elem_bytes;
-    if (join) join = clear_of_members(c, m, ndims) && clear_of_tail(m, c.nin);
-    if (!join) fuse_flush();
+    const uint32_t members = g_fuse.n + g_fuse.nwide;
+    bool join = (g_fuse.n > 0 || g_fuse.ntail > 0) && members < (uint32_t)FUSE_MAX_CMDS;
+    bool wide = false;
+    int own_rows = -1;
+    if (join && g_fuse.n > 0) {
+        const bool same_form = g_fuse.ndims == ndims && g_fuse.vec == (vec ? 1u : 0u) && g_fuse_elem_bytes == elem_bytes;
+        const bool first_space = same_form && g_fuse.nwide == 0 && g_fuse.nvec == nvec && g_fuse.dims[0] == dims[0] && (ndims == 1 || g_fuse.dims[1] == dims[1]);
+        if (!first_space) {
+            // the wide space: m times the units of a one-dim first space, and staging slots left for m rounds
+            const size_t mult = same_form && ndims == 1 && nvec % g_fuse.nvec == 0 ? nvec / g_fuse.nvec : 0;
+            wide = mult >= 2 && mult <= (size_t)FUSE_MAX_WIDE && nvec <= 0xFFFFFFFFull / 4 && (g_fuse.nwide == 0 || g_fuse.wide_m == mult) &&
+                   g_fuse.n + (g_fuse.nwide + 1) * mult <= (size_t)FUSE_MAX_CMDS;
+            if (wide) {
+                own_rows = own_rows_member(c, m, (uint32_t)mult);
+                wide = own_rows != -2;
+            }
+            join = wide;
+            if (wide && g_fuse.nwide == 0) {
+                g_fuse.wide_m = (uint32_t)mult;
+                g_fuse.wide_nvec = (uint32_t)nvec;
+            }
+        }
+    }
+    if (join) join = clear_of_members(c, m, ndims, wide, own_rows) && clear_of_tail(m, c.nin);
+    if (!join) {
+        fuse_flush();
+        wide = false;
+    }
     if (g_fuse.n == 0) open_space(ndims, dims, vec, nvec, elem_bytes);
-    FuseCmd& slot = g_fuse.cmd[g_fuse.n];
+    const uint32_t at = g_fuse.n + g_fuse.nwide;
+    FuseCmd& slot = g_fuse.cmd[at];
     slot = c;
     slot.fwd = 0;
     slot.src = FUSE_SRC_MEMORY | (FUSE_SRC_MEMORY << 8);
@@ -193,19 +242,26 @@ static void add_member(const FuseCmd& c, const ParMember& m, uint32_t ndims, con
         // (FUSE_OP_MSE_BACKWARD included: its two inputs are an elementwise member's)
         // An input that is an earlier member's output (element for element: nothing else was let in) is not in memory yet:
         // the members' stores wait until all of them are done.  It comes from the latest such member's staged output,
-        // or straight from registers when that is the member before.
+        // or straight from registers when that is the member before.  (A wide member only meets wide members so.)
+        const int lowest = wide ? (int)g_fuse.n : 0;
         for (uint32_t j = 0; j < c.nin; ++j)
-            for (int k = (int)g_fuse.n - 1; k >= 0; --k) {
-                const FuseCmd& e = g_fuse.cmd[k];
+            for (int k = (int)at - 1; k >= lowest; --k) {
                 if (!m.in[j].overlaps(g_par[k].out)) continue;
-                if ((uint32_t)k + 1 == g_fuse.n) slot.fwd |= 1u << j;
+                if ((uint32_t)k + 1 == at) slot.fwd |= 1u << j;
                 slot.src = (slot.src & ~(0xFFu << (8 * j))) | ((uint32_t)k << (8 * j));
-                (void)e;
                 break;
             }
+    } else if (wide && own_rows >= 0) {
+        slot.src = (slot.src & ~0xFFu) | (uint32_t)own_rows;
     }
-    g_par[g_fuse.n] = m;
-    ++g_fuse.n;
+    // `0 + the member before` (a gradient's first accumulation): that member makes it along with its own output
+    const bool after_one_of_its_space = at > (wide ? g_fuse.n : 0u);
+    if (after_one_of_its_space && c.op == (uint32_t)IndexOf<OpZeroPlus<float>, EwProgOps>::value && c.nin == 1 && slot.fwd == 1u &&
+        !(g_fuse.cmd[at - 1].fwd & FUSE_NEXT_IS_ZERO_PLUS) && (at < 2 || at - 1 == g_fuse.n || !(g_fuse.cmd[at - 2].fwd & FUSE_NEXT_IS_ZERO_PLUS)))
+        g_fuse.cmd[at - 1].fwd |= FUSE_NEXT_IS_ZERO_PLUS;
+    g_par[at] = m;
+    if (wide) ++g_fuse.nwide;
+    else ++g_fuse.n;
     ++g_fused_launches;
 }
 
@@ -678,6 +734,7 @@ int hip_graph_begin_capture(void) {
     g_prog_pending = false;
     g_prog_cmds.clear();
     g_fuse.n = 0;
+    g_fuse.nwide = g_fuse.wide_m = g_fuse.wide_nvec = 0;
     g_fuse.ntail = 0;
     g_lds_from = g_mem_from = 0;
     g_fused_launches = g_fuse_nodes = 0;

@@ -444,6 +444,157 @@ def test_fused_loss_backward_without_a_seed_stays_in_the_forward_chain(lib, n, f
         assert a.tobytes() == b.tobytes()
 
 
+def readme_step(lib, seq, n, feats, r):
+    """The training step of the README example as the host layer issues it: fused_nn_step() without a seed, with the
+    `0 + g` pass over the prediction's gradient, the input gradient [n,1] x [1,feats] and its accumulation."""
+    x, y = seq.dev(r.standard_normal((n, feats)).astype(np.float32)), seq.dev(r.standard_normal(n).astype(np.float32))
+    w0, b0 = r.standard_normal(feats).astype(np.float32), r.standard_normal(1).astype(np.float32)
+    w, b = seq.out(feats * 4, "f4"), seq.out(4, "f4")
+    w_init, b_init = seq.dev(w0), seq.dev(b0)
+    pred, pb, gp0, gpred = (seq.out(n * 4, "f4") for _ in range(4))
+    gx0, gx = seq.out(n * feats * 4, "f4"), seq.out(n * feats * 4, "f4")
+    loss, gw, gb = seq.out(4, "f4"), seq.out(feats * 4, "f4"), seq.out(4, "f4")
+    seq.add("add_scalar_f32", feats, 1, u64([feats], [1], 0), w_init.ptr, C.c_float(0.0), w.ptr)
+    seq.add("add_scalar_f32", 1, 1, u64([1], [1], 0), b_init.ptr, C.c_float(0.0), b.ptr)
+    seq.add("matmul_f32", n, u64(2, 2, 2, [n, 1], [n, feats], [feats, 1], [feats, 1], [1, feats], 0, 0), x.ptr, w.ptr, pred.ptr)
+    seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), pred.ptr, b.ptr, pb.ptr)
+    seq.add("mse_loss_f32", n, pb.ptr, y.ptr, loss.ptr)
+    seq.add("mse_loss_backward_f32", n, pb.ptr, y.ptr, None, gp0.ptr, None)
+    seq.add("sum_to_shape_f32", n, 1, u64([n], [1], [n], 0), gp0.ptr, gpred.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), gpred.ptr, gb.ptr)
+    seq.add("matmul_f32", n * feats, u64(2, 2, 2, [n, feats], [n, 1], [1, feats], [1, 1], [feats, 1], 0, 0), gpred.ptr, w.ptr, gx0.ptr)
+    seq.add("sum_to_shape_f32", n * feats, 1, u64([n * feats], [1], [n * feats], 0), gx0.ptr, gx.ptr)
+    seq.add("matmul_f32", feats, u64(2, 2, 2, [feats, 1], [feats, n], [n, 1], [1, feats], [1, 1], 0, 0), x.ptr, gpred.ptr, gw.ptr)
+    seq.add("sgd_step_f32", feats, w.ptr, gw.ptr, C.c_float(0.01))
+    seq.add("sgd_step_f32", 1, b.ptr, gb.ptr, C.c_float(0.01))
+
+
+@pytest.mark.parametrize("n,feats", [(10000, 3), (4096, 4), (12288, 2), (5001, 2), (5003, 3), (300, 3), (1028, 4), (10000, 1), (10000, 5), (5002, 2)])
+def test_input_gradient_of_a_one_output_layer_joins_the_step_as_a_wide_member(lib, n, feats):
+    """[n,1] x [1,feats] over the rows a chain's own members wrote, and the pass that accumulates it, run in the same
+    chain as the forward pass: work-group w, which staged rows [1024 w, 1024 w + 1024), also makes their feats-fold
+    products.  The whole step is then one chain (the node before it restores the parameters)."""
+    r = np.random.default_rng(500 + n + feats)
+    seq = Seq(lib)
+    readme_step(lib, seq, n, feats, r)
+    launches, nodes = fused(lib, seq, replays=3)
+    same_form = (n % 4 == 0) == (n * feats % 4 == 0)          # both spaces in 16-byte vectors, or both in elements
+    if 2 <= feats <= 4 and 4096 <= n <= 16384 and same_form:
+        assert launches == 13 and nodes == 2, (launches, nodes)
+    if feats in (1, 5) or not same_form:          # as wide as the first space, too wide, or of the other form: a chain of its own
+        assert nodes >= 3, (launches, nodes)
+
+
+def test_wide_members_split_where_work_groups_would_meet(lib):
+    """A member of the wide space runs with other work-groups' members of the first space still under way: apart from
+    the rows of a one-term product it may not read what they write, nor write what they read or write."""
+    n, m = 6000, 3
+    r = np.random.default_rng(91)
+    md1, mdw = u64([n], [1], 0), u64([n * m], [1], 0)
+    outer = lambda: u64(2, 2, 2, [n, m], [n, 1], [1, m], [1, 1], [m, 1], 0, 0)
+
+    def case(build, want_nodes):
+        seq = Seq(lib)
+        x, wide_in = seq.dev(r.standard_normal(n + 8).astype(np.float32)), seq.dev(r.standard_normal(n * m + 8).astype(np.float32))
+        y3 = seq.dev(r.standard_normal(m).astype(np.float32))
+        a, big, big2 = seq.out((n + 8) * 4, "f4"), seq.out((n * m + 8) * 4, "f4"), seq.out((n * m + 8) * 4, "f4")
+        build(seq, x, wide_in, y3, a, big, big2)
+        seq.clear_outputs()          # (no case writes every element of every buffer)
+        launches, nodes = fused(lib, seq)
+        assert nodes == want_nodes, (launches, nodes)
+
+    def rows_of_own_group(seq, x, wide_in, y3, a, big, big2):
+        seq.add("tanh_f32", n, 1, md1, x.ptr, a.ptr)
+        seq.add("matmul_f32", n * m, outer(), a.ptr, y3.ptr, big.ptr)
+        seq.add("mul_f32", n * m, 1, u64([n * m], [1], [1], 0, 0), big.ptr, wide_in.ptr, big2.ptr)
+    case(rows_of_own_group, 1)
+
+    def rows_from_memory(seq, x, wide_in, y3, a, big, big2):          # the left operand is nobody's output: read from memory
+        seq.add("tanh_f32", n, 1, md1, x.ptr, a.ptr)
+        seq.add("matmul_f32", n * m, outer(), x.ptr, y3.ptr, big.ptr)
+    case(rows_from_memory, 1)
+
+    def shifted_rows(seq, x, wide_in, y3, a, big, big2):              # rows 1 .. n of the output: another group's at the seams
+        seq.add("tanh_f32", n + 1, 1, u64([n + 1], [1], 0), x.ptr, a.ptr)
+        seq.add("matmul_f32", n * m, outer(), a.ptr + 4, y3.ptr, big.ptr)
+    case(shifted_rows, 2)
+
+    def elementwise_read_of_the_first_space(seq, x, wide_in, y3, a, big, big2):
+        seq.add("tanh_f32", n, 1, md1, x.ptr, big.ptr)                 # writes big[0 .. n)
+        seq.add("neg_f32", n * m, 1, mdw, big.ptr, big2.ptr)           # reads big[0 .. 3n)
+    case(elementwise_read_of_the_first_space, 2)
+
+    def write_over_what_the_first_space_reads(seq, x, wide_in, y3, a, big, big2):
+        seq.add("tanh_f32", n, 1, md1, big.ptr + 4 * n, a.ptr)         # reads big[n .. 2n)
+        seq.add("neg_f32", n * m, 1, mdw, wide_in.ptr, big.ptr)        # writes big[0 .. 3n)
+    case(write_over_what_the_first_space_reads, 2)
+
+    def write_over_what_the_first_space_writes(seq, x, wide_in, y3, a, big, big2):
+        seq.add("tanh_f32", n, 1, md1, x.ptr, big.ptr)
+        seq.add("neg_f32", n * m, 1, mdw, wide_in.ptr, big.ptr)
+    case(write_over_what_the_first_space_writes, 2)
+
+    def right_operand_written_by_the_first_space(seq, x, wide_in, y3, a, big, big2):
+        seq.add("tanh_f32", n, 1, md1, x.ptr, a.ptr)
+        seq.add("exp_f32", n, 1, md1, x.ptr, big2.ptr)
+        seq.add("matmul_f32", n * m, outer(), a.ptr, big2.ptr + 16, big.ptr)
+    case(right_operand_written_by_the_first_space, 2)
+
+    def first_space_member_after_the_wide_ones(seq, x, wide_in, y3, a, big, big2):
+        seq.add("tanh_f32", n, 1, md1, x.ptr, a.ptr)
+        seq.add("matmul_f32", n * m, outer(), a.ptr, y3.ptr, big.ptr)
+        seq.add("exp_f32", n, 1, md1, x.ptr, big2.ptr)                 # the first space is closed: a new chain
+    case(first_space_member_after_the_wide_ones, 2)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_fused_random_sequences_over_two_spaces(lib, seed):
+    """Random launches over [n] and over [m n] - elementwise, one-term products [n,1] x [1,m], sums - on a small pool of
+    buffers, so that operands overlap in every way: whatever the grouping decides, a replay leaves the eager bytes."""
+    r = np.random.default_rng(4000 + seed)
+    n = int(r.choice([300, 1024, 4096, 10000, 5001, 2052]))
+    m = int(r.choice([2, 3, 4]))
+    seq = Seq(lib)
+    pool = [seq.out((n * m + 8) * 4, "f4") for _ in range(4)]
+    src = [seq.dev(r.standard_normal(n * m + 8).astype(np.float32)) for _ in range(2)]
+    for k, p in enumerate(pool):
+        seq.add("add_scalar_f32", n * m + 8, 1, u64([n * m + 8], [1], 0), src[k % 2].ptr, C.c_float(0.25 * k), p.ptr)
+    small = seq.out(64 * 4, "f4")
+    seq.add("add_scalar_f32", 64, 1, u64([64], [1], 0), src[0].ptr, C.c_float(0.0), small.ptr)
+    for _ in range(int(r.integers(4, 12))):
+        kind = str(r.choice(["ew", "ew", "wide", "wide", "outer", "outer", "sum"]))
+        oi = int(r.integers(0, len(pool)))
+        others = [i for i in range(len(pool)) if i != oi]
+        if kind in ("ew", "sum"):
+            off = int(r.choice([0, 0, n, 1, 2 * n if m > 2 else n]))
+            a_i = int(r.choice(others + [oi]))
+            a_ptr = pool[a_i].ptr + 4 * (off if a_i == oi else int(r.choice([0, n, 3])))
+            if kind == "sum":
+                seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), a_ptr, small.ptr + 4 * int(r.integers(0, 64)))
+            elif r.random() < 0.5:
+                seq.add(str(r.choice(["tanh_f32", "neg_f32", "square_f32"])), n, 1, u64([n], [1], 0), a_ptr, pool[oi].ptr + 4 * off)
+            else:
+                b_ptr = pool[int(r.choice(others))].ptr + 4 * int(r.choice([0, n]))
+                seq.add(str(r.choice(["add_f32", "mul_f32"])), n, 1, u64([n], [1], [1], 0, 0), a_ptr, b_ptr, pool[oi].ptr + 4 * off)
+        elif kind == "wide":
+            a_i = int(r.choice(others + [oi]))
+            a_ptr = pool[a_i].ptr + (0 if a_i == oi else 4 * int(r.choice([0, 0, 2])))
+            if r.random() < 0.5:
+                seq.add(str(r.choice(["neg_f32", "relu_f32"])), n * m, 1, u64([n * m], [1], 0), a_ptr, pool[oi].ptr)
+            else:
+                b_ptr = pool[int(r.choice(others))].ptr
+                seq.add(str(r.choice(["add_f32", "sub_f32"])), n * m, 1, u64([n * m], [1], [1], 0, 0), a_ptr, b_ptr, pool[oi].ptr)
+        else:
+            xi = int(r.choice(others))
+            x_ptr = pool[xi].ptr + 4 * int(r.choice([0, 0, 0, n, 1]))
+            if r.random() < 0.5:
+                y_ptr = small.ptr + 4 * int(r.integers(0, 60))
+            else:
+                y_ptr = pool[int(r.choice(others))].ptr + 4 * int(r.integers(0, n))
+            seq.add("matmul_f32", n * m, u64(2, 2, 2, [n, m], [n, 1], [1, m], [1, 1], [m, 1], 0, 0), x_ptr, y_ptr, pool[oi].ptr)
+    fused(lib, seq, replays=2)
+
+
 def test_fused_loss_backward_waits_for_a_gradient_written_in_the_same_chain(lib):
     """The loss's gradient is read by every thread of the backward member: when an earlier member of the same space
     writes it (here: the buffer is a slice of a tensor the chain fills), the member must open a new chain; and a member
