@@ -105,6 +105,14 @@ static void fuse_flush() {
     // Chains queued on one stream run one after the other, and each leaves its ticket at zero, so sharing would do;
     // rotating over the slots keeps two captures that a caller replays on two streams at once apart as well.
     g_fuse.ticket = g_tickets[dev] + (g_next_ticket++ % FUSE_TICKETS);
+    // MXH_CHAIN_TRACE in the environment: the shape of every chain as it is queued
+    static const bool trace = getenv("MXH_CHAIN_TRACE") != nullptr;
+    if (trace) {
+        fprintf(stderr, "chain: %u members over %zu %s, %u wide x %u, tail stages of kind", g_fuse.n, g_fuse.nvec, g_fuse.vec ? "vectors" : "elements", g_fuse.nwide,
+                g_fuse.wide_m);
+        for (uint32_t k = 0; k < g_fuse.ntail; ++k) fprintf(stderr, " %u", g_fuse.tail[k].kind);
+        fprintf(stderr, "\n");
+    }
     fuse_launch(g_fuse, (void*)g_capture_stream);
     ++g_fuse_nodes;
     g_fuse.n = 0;
