@@ -92,7 +92,7 @@ __device__ __forceinline__ void tail_row(uint32_t vec, const RowProgArgs& a, uns
 
 __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, uint32_t want, unsigned tid, float* part, float* mir, float* pre) {
     // `want`: which (stage, input) pairs are fetched up front; they go to LDS when the first elementwise stage comes up,
-    // so that the stages before it overlap the fetch (volatile: the loads are issued here, not where their values are used)
+    // so that the stages before it can overlap the fetch
     float got[2 * FUSE_MAX_TAIL];
 #pragma unroll
     for (int q = 0; q < 2 * FUSE_MAX_TAIL; ++q) got[q] = 0.0f;
@@ -103,7 +103,7 @@ __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, ui
                 const FuseCmd c = lds_uniform<FuseCmd>(sg.tail[k].arg);
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    if (((want >> (2 * k + j)) & 1u) && tid < c.nel) got[2 * k + j] = *(volatile GCFloat*)(gl(c.in[j]) + tail_elem(c, c.is[j][0], c.is[j][1], tid));
+                    if (((want >> (2 * k + j)) & 1u) && tid < c.nel) got[2 * k + j] = gl(c.in[j])[tail_elem(c, c.is[j][0], c.is[j][1], tid)];
             }
         }
     }
@@ -169,6 +169,7 @@ __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, ui
 }
 
 // ---- the members of the parallel phase --------------------------------------------------------------------------
+// (Element offsets are computed in 32 bits: the host only lets operands in whose elements lie within 2^31 of their base.)
 // A matmul producer at unit `u` of its flat output space: one output per element, r ascending, multiply and add
 // unfused (gemm_thread_body's order).  `own`: when the left operand is a first-space member's staged output (a wide
 // member of one term, c.src names the member), own[member * EW_BLOCK * VEC + row - row0] holds row `row` of it
@@ -189,38 +190,21 @@ __device__ __forceinline__ void member_dot(const FuseCmd& c, uint32_t u, const f
     if (own && from != FUSE_SRC_MEMORY) {
         float y[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) y[e] = gl(c.in[1])[(int64_t)col[e] * c.is[1][1]];
+        for (int e = 0; e < VEC; ++e) y[e] = gl(c.in[1])[col[e] * (uint32_t)c.is[1][1]];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f + own[from * (EW_BLOCK * VEC) + (row[e] - row0)] * y[e];
         return;
     }
-    // the terms of four steps of every element are requested together (steps past the end re-read the last term and
-    // are not added): a thread waits once per four terms, not once per term and element
-    constexpr int Q = 4;
-    float acc[VEC];
+    // (term by term: requesting several terms of an element together costs more instructions than it saves latencies
+    // for the reductions of one to three terms this is for)
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
-    for (uint32_t q0 = 0; q0 < R; q0 += Q) {
-        float xv[VEC][Q], yv[VEC][Q];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            GCFloat* x = gl(c.in[0]) + (int64_t)row[e] * c.is[0][0];
-            GCFloat* y = gl(c.in[1]) + (int64_t)col[e] * c.is[1][1];
-#pragma unroll
-            for (int t = 0; t < Q; ++t) {
-                const uint32_t qq = q0 + t < R ? q0 + t : R - 1;
-                xv[e][t] = x[(int64_t)qq * c.is[0][1]];
-                yv[e][t] = y[(int64_t)qq * c.is[1][0]];
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < Q; ++t)
-            if (q0 + t < R)
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) acc[e] = acc[e] + xv[e][t] * yv[e][t];
+    for (int e = 0; e < VEC; ++e) {
+        GCFloat* x = gl(c.in[0]) + row[e] * (uint32_t)c.is[0][0];
+        GCFloat* y = gl(c.in[1]) + col[e] * (uint32_t)c.is[1][1];
+        float acc = 0.0f;
+        for (uint32_t q = 0; q < R; ++q) acc = acc + x[q * (uint32_t)c.is[0][1]] * y[q * (uint32_t)c.is[1][0]];
+        r.v[e] = acc;
     }
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) r.v[e] = acc[e];
 }
 // An elementwise member (FUSE_OP_MSE_BACKWARD included) at the VEC elements that start at coordinates (c0, c1).  `r`
 // comes in as what the member before wrote at these elements and goes out as this member's values; an input that is
@@ -248,8 +232,8 @@ __device__ __forceinline__ void member_ew(const FuseCmd& c, uint32_t ndims, uint
             for (int e = 0; e < VEC; ++e) val[j][e] = t.v[e];
             continue;
         }
-        const int64_t s = ndims == 2 ? c.is[j][1] : c.is[j][0];
-        GCFloat* src = gl(c.in[j]) + (ndims == 2 ? (int64_t)c0 * c.is[j][0] : 0) + (int64_t)c1 * s;
+        const uint32_t s = (uint32_t)(ndims == 2 ? c.is[j][1] : c.is[j][0]);
+        GCFloat* src = gl(c.in[j]) + ((ndims == 2 ? c0 * (uint32_t)c.is[j][0] : 0u) + c1 * s);
         if (VEC > 1 && s == 1) {
             const AVec<float, VEC> t = gload<VEC>(src);
 #pragma unroll
@@ -260,7 +244,7 @@ __device__ __forceinline__ void member_ew(const FuseCmd& c, uint32_t ndims, uint
             for (int e = 0; e < VEC; ++e) val[j][e] = t;
         } else {
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) val[j][e] = src[(int64_t)e * s];
+            for (int e = 0; e < VEC; ++e) val[j][e] = src[(uint32_t)e * s];
         }
     }
     if (c.op == FUSE_OP_MSE_BACKWARD) {
@@ -330,7 +314,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
             if (c.op == FUSE_OP_DOT) member_dot<VEC>(c, unit, first ? nullptr : pool, row0, r);
             else member_ew<VEC>(c, ndims, u0, u1, staged, first ? 1u : m, first ? 0 : (int)(h.n + q) - (int)(h.n * m), r);
             staged[slot * EW_BLOCK] = r;
-            dst = (float*)c.out + (ndims == 2 ? (int64_t)u0 * c.os[0] + (int64_t)u1 * c.os[1] : (int64_t)u1 * c.os[0]);
+            dst = (float*)c.out + (ndims == 2 ? u0 * (uint32_t)c.os[0] + u1 * (uint32_t)c.os[1] : u1 * (uint32_t)c.os[0]);
         }
         where[slot * EW_BLOCK] = dst;
         if (c.fwd & FUSE_NEXT_IS_ZERO_PLUS) {
@@ -345,7 +329,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
                 for (int e = 0; e < VEC; ++e) r.v[e] = OpZeroPlus<float>{}(r.v[e]);
                 staged[slot2 * EW_BLOCK] = r;
                 const uint32_t u0 = first ? c0 : 0u, u1 = first ? c1 : unit * VEC;
-                dst2 = (float*)n.out + (first && h.ndims == 2 ? (int64_t)u0 * n.os[0] + (int64_t)u1 * n.os[1] : (int64_t)u1 * n.os[0]);
+                dst2 = (float*)n.out + (first && h.ndims == 2 ? u0 * (uint32_t)n.os[0] + u1 * (uint32_t)n.os[1] : u1 * (uint32_t)n.os[0]);
             }
             where[slot2 * EW_BLOCK] = dst2;
             ++k;

@@ -210,6 +210,11 @@ static int own_rows_member(const FuseCmd& c, const ParMember& m, uint32_t wide_m
     }
     return -1;
 }
+// the kernel computes a member's element offsets in 32 bits
+static bool offsets_fit(const ParMember& m) {
+    const uint64_t limit = 1ull << 33;          // 2^31 elements of four bytes
+    return m.out.hi - m.out.lo < limit && m.in[0].hi - m.in[0].lo < limit && m.in[1].hi - m.in[1].lo < limit;
+}
 // Adds a member to the parallel phase (joining the open chain when it may, closing it and opening a new one otherwise).
 static void add_member(const FuseCmd& c, const ParMember& m, uint32_t ndims, const uint32_t* dims, bool vec, size_t nvec, size_t elem_bytes) {
     const uint32_t members = g_fuse.n + g_fuse.nwide;
@@ -377,6 +382,7 @@ static bool chain_record(const FuseCmd& c, uint32_t ndims, const uint32_t* dims,
         t.nel = (uint32_t)nel;
         return chain_record_tail(TAIL_EW, 0, &t, sizeof(t), m.in, (int)c.nin, m.out, nel);
     }
+    if (!offsets_fit(m)) return false;
     add_member(c, m, ndims, dims, vec, nvec, elem_bytes);
     return true;
 }
@@ -390,6 +396,7 @@ static bool chain_record_dot(const FuseCmd& c, size_t outputs, const Extent& x, 
     m.across[0] = m.across[1] = true;
     const bool vec = outputs % 4 == 0 && (uintptr_t)c.out % 16 == 0;
     const uint32_t dims[1] = {(uint32_t)outputs};
+    if (!offsets_fit(m)) return false;
     add_member(c, m, 1, dims, vec, vec ? outputs / 4 : outputs, sizeof(float));
     return true;
 }
@@ -405,6 +412,7 @@ static bool chain_record_mse_backward(const FuseCmd& c, bool vec, size_t nvec, c
     }
     m.extra = grad_loss;
     if (m.extra.overlaps(m.out)) return false;
+    if (!offsets_fit(m)) return false;
     add_member(c, m, 1, dims, vec, nvec, sizeof(float));
     return true;
 }
