@@ -109,7 +109,7 @@ int hip_graph_set_fusion(int enabled);
  * hip_graph_set_resident: the largest tensor, in elements, that a launch of a later capture may touch for the capture
  *   to be kept this way: 0 never, at most 65536, default 8192 (one work-group's instruction stream is what a recorded
  *   kernel costs - about 0.7 us up to 2048 elements, 1.5 us for 10000, where the fused chains are ahead again: a
- *   Linear(3 -> 1) + MSE + SGD step on 1000 rows replays in 15.8 us this way and 22.8 us as chains, on 10000 rows in 35 and 27);
+ *   Linear(3 -> 1) + MSE + SGD step on 1000 rows replays in 14.2 us this way and 19.0 us as chains, on 10000 rows in 34 and 23);
  *   returns the old value.
  * hip_buffer_discard: a hint that the contents of [ptr, ptr + bytes) are no longer needed (a caching allocator calls it
  *   when a buffer goes back to its pool, where the reference would call cuda_free, crates/maidenx_cuda/src/lib.rs:

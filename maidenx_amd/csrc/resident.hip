@@ -332,6 +332,7 @@ namespace {
 struct Region {
     uintptr_t lo = 0, hi = 0;
     bool written = false, live_in = false, candidate = false, pinned = false;
+    uint32_t readers = 0;              // commands of a pass that read it
     int state = 0;                     // 0 as the pass found it, 1 defined by a write of this pass, 2 released
     bool in_lds = false;
     uint32_t slot_off = 0, slot_size = 0, lds_off = 0;
@@ -520,6 +521,7 @@ bool res_build(const std::vector<ResRecord>& recs, ResProgram& out) {
         for (int j = 0; j < inputs_of(r); ++j) {
             Region& g = region_of(r.in[j]);
             if (g.state == 0) g.live_in = true;
+            if (j == 0 || &g != &region_of(r.in[0])) ++g.readers;
         }
         Region& g = region_of(r.out);
         g.written = true;
@@ -536,6 +538,22 @@ bool res_build(const std::vector<ResRecord>& recs, ResProgram& out) {
         if (g.candidate && g.live_in) pinned.push_back(&g);
     }
     std::sort(pinned.begin(), pinned.end(), [](const Region* a, const Region* b) { return a->size() < b->size(); });
+    // Inputs that nothing writes and two or more commands of a pass read (the samples and targets of a training step): a
+    // copy in the arena for the whole launch - one trip to memory per launch instead of one per reading command and
+    // pass - as long as they leave most of the arena to the tensors the commands write.
+    {
+        std::vector<Region*> inputs;
+        for (Region& g : regions)
+            if (!g.written && g.live_in && g.readers >= 2 && g.size() <= RES_MAX_REGION && g.size() % 4 == 0 && g.lo % 4 == 0) inputs.push_back(&g);
+        std::sort(inputs.begin(), inputs.end(), [](const Region* a, const Region* b) { return a->size() < b->size(); });
+        size_t taken = 0;
+        for (Region* g : inputs) {
+            if (taken + g->slot_size > RES_INPUT_BYTES) break;
+            taken += g->slot_size;
+            g->candidate = true;
+            pinned.push_back(g);
+        }
+    }
     for (Region* g : pinned) {
         if (!arena.get(g->slot_size, g->slot_off)) { g->candidate = false; continue; }
         g->pinned = g->in_lds = true;

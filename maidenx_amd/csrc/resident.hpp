@@ -41,11 +41,12 @@ constexpr unsigned RES_THREADS = 512;
 constexpr int RES_UNROLL = 5;                 // units a thread has in flight (10000 elements are 2500 vectors: one round)
 constexpr size_t RES_LDS_BYTES = (160u << 10) - 256;  // dynamic LDS of the work-group: the arena
 constexpr size_t RES_MAX_REGION = 64u << 10;          // larger tensors stay in memory
+constexpr size_t RES_INPUT_BYTES = 64u << 10;         // of the arena for copies of inputs that no command writes
 // Elements one command may span: the hard limit, and the default of hip_graph_set_resident().  One work-group's
 // instruction stream is what a command costs: about 0.7 us for up to 2048 elements (one vector a thread), 1.5 us for
 // 10000 - where the fused chains, which spread a launch over ten work-groups, are ahead again.  The README step
-// (Linear(3 -> 1) + MSE + SGD) on n rows, us per step here / as chains: n = 256 12.4 / 17.5, 1000 15.8 / 22.8, 2000 18.3 /
-// 24.3, 3000 23.6 / 26.7, 5000 26.3 / 24.0, 10000 34.6 / 26.6 - the default keeps tensors of up to 8192 elements here.
+// (Linear(3 -> 1) + MSE + SGD) on n rows, us per step here / as chains: n = 256 12.0 / 19.3, 1000 14.2 / 19.0, 2000 15.5 /
+// 21.8, 3000 20.4 / 23.9, 5000 25.5 / 21.6, 10000 34.0 / 22.6 - the default keeps tensors of up to 8192 elements here.
 constexpr size_t RES_MAX_ELEMS = 1u << 16;
 constexpr size_t RES_DEFAULT_ELEMS = 8192;
 constexpr uint32_t RES_MODE_LINEAR = 0, RES_MODE_SCALAR = 1, RES_MODE_2D = 2;
