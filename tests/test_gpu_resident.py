@@ -197,6 +197,67 @@ def test_many_replays_in_one_launch(lib, n, feats, discard):
     assert lib.hip_get_last_status() == 0, lib.hip_status_string()
 
 
+@pytest.mark.parametrize("n,feats", [(1000, 3), (5000, 3), (16000, 1), (12000, 3)])
+def test_inputs_nothing_writes_are_read_again_at_every_launch(lib, n, feats):
+    """The samples and the targets of a step - read by two or more commands, written by none - are copied into LDS when a
+    launch starts (as long as they fit 64 KB of it; beyond that they stay in memory): data the host writes between two
+    launches of the same program is what the second one computes on, and several passes of one launch see one copy."""
+    r = np.random.default_rng(40 + n)
+    seq = Seq(lib)
+    xs = [r.standard_normal((n, feats)).astype(np.float32) for _ in range(2)]
+    ys = [r.standard_normal(n).astype(np.float32) for _ in range(2)]
+    x, y = seq.dev(xs[0]), seq.dev(ys[0])
+    w, b = seq.out(feats * 4, "f4"), seq.out(4, "f4")
+    w0, b0 = (r.standard_normal(feats) * 0.1).astype(np.float32), np.array([0.3], np.float32)
+    pred, pb, gpred = (seq.out(n * 4, "f4") for _ in range(3))
+    loss, gw, gb = seq.out(4, "f4"), seq.out(feats * 4, "f4"), seq.out(4, "f4")
+    seq.add("matmul_f32", n, u64(2, 2, 2, [n, 1], [n, feats], [feats, 1], [feats, 1], [1, feats], 0, 0), x.ptr, w.ptr, pred.ptr)
+    seq.add("add_f32", n, 1, u64([n], [1], [0], 0, 0), pred.ptr, b.ptr, pb.ptr)
+    seq.add("mse_loss_f32", n, pb.ptr, y.ptr, loss.ptr)
+    seq.add("mse_loss_backward_f32", n, pb.ptr, y.ptr, None, gpred.ptr, None)
+    seq.add("matmul_f32", feats, u64(2, 2, 2, [feats, 1], [feats, n], [n, 1], [1, feats], [1, 1], 0, 0), x.ptr, gpred.ptr, gw.ptr)
+    seq.add("sum_f32", n, 1, 1, u64([n], [1], [n], [1], 0), gpred.ptr, gb.ptr)
+    seq.add("sgd_step_f32", feats, w.ptr, gw.ptr, C.c_float(0.05))
+    seq.add("sgd_step_f32", 1, b.ptr, gb.ptr, C.c_float(0.05))
+
+    def load(which):
+        assert lib.hip_memcpy_h2d(x.ptr, xs[which].ctypes.data, xs[which].nbytes) == 0
+        assert lib.hip_memcpy_h2d(y.ptr, ys[which].ctypes.data, ys[which].nbytes) == 0
+
+    def reset():
+        assert lib.hip_memcpy_h2d(w.ptr, w0.ctypes.data, w0.nbytes) == 0 and lib.hip_memcpy_h2d(b.ptr, b0.ctypes.data, 4) == 0
+
+    # eager: three steps on the first data set, then two on the second
+    seq.clear_outputs()
+    reset()
+    load(0)
+    for _ in range(3):
+        seq.run()
+    load(1)
+    for _ in range(2):
+        seq.run()
+    want = seq.read()
+    assert lib.hip_get_last_status() == 0, lib.hip_status_string()
+    seq.clear_outputs()
+    reset()
+    load(0)
+    assert lib.hip_graph_begin_capture() == 0
+    seq.run()
+    h = C.c_void_p()
+    assert lib.hip_graph_end_capture(C.byref(h)) == 0
+    try:
+        assert lib.hip_graph_is_resident(h, None, None) == len(seq.calls)
+        assert lib.hip_graph_launch_n(h, 3) == 0
+        load(1)
+        assert lib.hip_graph_launch(h) == 0 and lib.hip_graph_launch(h) == 0
+        got = seq.read()
+        for k, (g, e) in enumerate(zip(got, want)):
+            assert g.tobytes() == e.tobytes(), k
+    finally:
+        assert lib.hip_graph_destroy(h) == 0
+    assert lib.hip_get_last_status() == 0, lib.hip_status_string()
+
+
 def test_a_launch_of_another_kind_hands_the_capture_to_the_chains(lib):
     """A column reduction has no resident command: what was kept until then is fused or launched in order, the capture
     is a HIP graph, and the replay is the eager bytes."""
