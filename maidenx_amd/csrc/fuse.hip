@@ -171,13 +171,10 @@ __device__ __forceinline__ void run_tail(const FuseGroup& sg, uint32_t ntail, ui
 // ---- the members of the parallel phase --------------------------------------------------------------------------
 // (Element offsets are computed in 32 bits: the host only lets operands in whose elements lie within 2^31 of their base.)
 // A matmul producer at unit `u` of its flat output space: one output per element, r ascending, multiply and add
-// unfused (gemm_thread_body's order).  `own`: when the left operand is a first-space member's staged output (a wide
-// member of one term, c.src names the member), own[member * EW_BLOCK * VEC + row - row0] holds row `row` of it
-// (row0: the first row this work-group staged).
+// unfused (gemm_thread_body's order).
 template <int VEC>
-__device__ __forceinline__ void member_dot(const FuseCmd& c, uint32_t u, const float* own, uint32_t row0, AVec<float, VEC>& r) {
+__device__ __forceinline__ void member_dot(const FuseCmd& c, uint32_t u, AVec<float, VEC>& r) {
     const uint32_t J = c.dims[0], R = c.dims[1];
-    const uint32_t from = c.src & 0xFFu;
     uint32_t row[VEC], col[VEC];
     row[0] = (u * VEC) / J;
     col[0] = u * VEC - row[0] * J;
@@ -186,14 +183,6 @@ __device__ __forceinline__ void member_dot(const FuseCmd& c, uint32_t u, const f
         col[e] = col[e - 1] + 1;
         row[e] = row[e - 1];
         if (col[e] == J) { col[e] = 0; ++row[e]; }
-    }
-    if (own && from != FUSE_SRC_MEMORY) {
-        float y[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) y[e] = gl(c.in[1])[col[e] * (uint32_t)c.is[1][1]];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f + own[from * (EW_BLOCK * VEC) + (row[e] - row0)] * y[e];
-        return;
     }
     // (term by term: requesting several terms of an element together costs more instructions than it saves latencies
     // for the reductions of one to three terms this is for)
@@ -204,6 +193,23 @@ __device__ __forceinline__ void member_dot(const FuseCmd& c, uint32_t u, const f
         float acc = 0.0f;
         for (uint32_t q = 0; q < R; ++q) acc = acc + x[q * (uint32_t)c.is[0][1]] * y[q * (uint32_t)c.is[1][0]];
         r.v[e] = acc;
+    }
+}
+// The one-term product of the wide space whose left operand is a first-space member's output, row for row: round q of
+// this thread's m = J units.  Its VEC * J outputs are the thread's own VEC rows (`own`, that member's staged output) times
+// the J entries of the right operand, so which row and which entry meet at element e of the round is the same for every
+// thread.
+template <int VEC>
+__device__ __forceinline__ void member_dot_own(const FuseCmd& c, uint32_t q, const AVec<float, VEC>& own, AVec<float, VEC>& r) {
+    const uint32_t J = c.dims[0];
+    const uint32_t yj = (uint32_t)c.is[1][1];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        const uint32_t at = q * VEC + e, row = at / J, col = at - row * J;      // (uniform)
+        float x = own.v[0];
+#pragma unroll
+        for (int i = 1; i < VEC; ++i) x = row == (uint32_t)i ? own.v[i] : x;
+        r.v[e] = 0.0f + x * gl(c.in[1])[col * yj];
     }
 }
 // An elementwise member (FUSE_OP_MSE_BACKWARD included) at the VEC elements that start at coordinates (c0, c1).  `r`
@@ -287,7 +293,8 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
     float** where = (float**)(pool + FUSE_MAX_CMDS * EW_BLOCK * VEC) + threadIdx.x;      // where each staged output goes
     // One loop over the members of the first space, then over the rounds of the wide space (round-major: a member
     // then finds what the member before it wrote, same round, in registers) - one copy of the member code, so that
-    // what the first rounds bring into the instruction cache serves the later ones.
+    // what the first rounds bring into the instruction cache serves the later ones.  The thread that owns unit v of the
+    // first space owns units m v .. m v + m - 1 of the wide one, one per round.
     const uint32_t m = h.wide_m, items = h.n + h.nwide * m;
     const uint32_t slots = items;
     AVec<float, VEC> r;          // what the previous member wrote at this thread's elements
@@ -295,24 +302,25 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_group_kernel(FuseGroup g) {
     for (int e = 0; e < VEC; ++e) r.v[e] = 0.0f;
     uint32_t c0 = 0, c1 = (uint32_t)v * VEC;      // first space: coordinates over (outer, inner); one dim: everything is "inner"
     if (h.ndims == 2) fd_divmod((uint32_t)v * VEC, h.div_inner, c0, c1);
-    const uint32_t row0 = (uint32_t)blockIdx.x * EW_BLOCK * VEC;       // the first element this work-group stages of every member
+    const bool in_space = v < h.nvec;
     uint32_t k = 0, q = 0;
     for (uint32_t it = 0; it < items; ++it) {
         const bool first = it < h.n;
-        if (it == h.n) {
-            lds_barrier();      // the group's staged first-space outputs are readable by all its threads
-            k = h.n;
-        }
-        // wide space: this work-group's threads take its units [EW_BLOCK m w, EW_BLOCK m (w + 1)), m rounds of one unit a thread
-        const uint32_t unit = first ? (uint32_t)v : ((uint32_t)blockIdx.x * m + q) * EW_BLOCK + threadIdx.x;
+        if (it == h.n) k = h.n;
+        const uint32_t unit = first ? (uint32_t)v : (uint32_t)v * m + q;
         const uint32_t slot = first ? k : h.n + (k - h.n) * m + q;
         const FuseCmd c = lds_uniform<FuseCmd>(&sg.cmd[k]);
         float* dst = nullptr;
-        if (unit < (first ? h.nvec : (size_t)h.wide_nvec)) {
+        if (in_space) {
             const uint32_t ndims = first ? h.ndims : 1u;
             const uint32_t u0 = first ? c0 : 0u, u1 = first ? c1 : unit * VEC;
-            if (c.op == FUSE_OP_DOT) member_dot<VEC>(c, unit, first ? nullptr : pool, row0, r);
-            else member_ew<VEC>(c, ndims, u0, u1, staged, first ? 1u : m, first ? 0 : (int)(h.n + q) - (int)(h.n * m), r);
+            if (c.op == FUSE_OP_DOT) {
+                const uint32_t from = c.src & 0xFFu;
+                if (!first && from != FUSE_SRC_MEMORY) member_dot_own<VEC>(c, q, staged[from * EW_BLOCK], r);
+                else member_dot<VEC>(c, unit, r);
+            } else {
+                member_ew<VEC>(c, ndims, u0, u1, staged, first ? 1u : m, first ? 0 : (int)(h.n + q) - (int)(h.n * m), r);
+            }
             staged[slot * EW_BLOCK] = r;
             dst = (float*)c.out + (ndims == 2 ? u0 * (uint32_t)c.os[0] + u1 * (uint32_t)c.os[1] : u1 * (uint32_t)c.os[0]);
         }

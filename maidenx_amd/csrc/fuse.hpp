@@ -14,14 +14,13 @@
 //     earlier members write, nor may a later member write them;
 //   * the backward pass of the fused MSE loss joins as an elementwise member of two inputs; the one value every thread
 //     reads besides (the gradient of the loss) is held to the rule of a matmul's operands.
-//   A second, WIDE space of m times as many units (m = 2..4) may follow the first: work-group w, which owns units
-//   [256 w, 256 w + 256) of the first space, then owns units [256 m w, 256 m (w + 1)) of the wide one.  Its members run
-//   after a work-group barrier that follows all members of the first space, so a wide member may read what its OWN
-//   work-group's threads wrote there: the outer product [N,1] x [1,m] (a matmul producer of one term, the input
-//   gradient of a layer with one output feature) whose left operand is, row for row, a first-space member's output
-//   takes its rows i = idx / m - the work-group's own - from the staged outputs.  Apart from that a wide member
-//   touches nothing a first-space member writes and writes nothing one reads, and among themselves wide members keep
-//   the rule above.  Once a wide member has joined, the first space takes no more members.
+//   A second, WIDE space of m times as many units (m = 2..4) may follow the first: the thread that owns unit v of the
+//   first space owns units m v .. m v + m - 1 of the wide one, and takes them in m rounds after the members of the first
+//   space.  A wide member may therefore read what its OWN thread wrote there: the outer product [N,1] x [1,m] (a matmul
+//   producer of one term, the input gradient of a layer with one output feature) whose left operand is, row for row, a
+//   first-space member's output takes its rows idx / m - the thread's own - from that member's staged output.  Apart
+//   from that a wide member touches nothing a first-space member writes and writes nothing one reads, and among
+//   themselves wide members keep the rule above.  Once a wide member has joined, the first space takes no more members.
 // Serial phase ("tail") - stages run in order by the work-group that finishes the parallel phase last (every group
 // publishes its writes, then draws a ticket; the last ticket continues, the others exit, nobody waits):
 //   * elementwise launches of at most 256 elements (a bias, a 3-element weight, a loss), any shapes, any overlaps;
