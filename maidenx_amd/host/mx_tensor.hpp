@@ -29,6 +29,9 @@
 #pragma once
 #include <cmath>
 #include <cstdint>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <map>
@@ -1511,6 +1514,10 @@ struct Adam {
 template <class B, class Step>
 size_t run_steps(Step&& step, size_t epochs, bool allow_graph) {
     size_t done = 0, replayed = 0;
+    // MXT_TRACE_STEPS in the environment: where the wall-clock time of a call goes (warm-up, recording, replays, the rest)
+    static const bool trace_steps = std::getenv("MXT_TRACE_STEPS") != nullptr;
+    const auto clock0 = std::chrono::steady_clock::now();
+    auto since = [&] { return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - clock0).count(); };
     if constexpr (B::has_graphs) {
         constexpr size_t kMinWarm = 8, kMaxWarm = 64, kMaxPeriod = 4;   // the README loop settles into period 3 after 5 steps
         if (allow_graph && epochs >= 4 * kMinWarm) {
@@ -1533,6 +1540,7 @@ size_t run_steps(Step&& step, size_t epochs, bool allow_graph) {
                     if (same) period = p;
                 }
             }
+            if (trace_steps) std::fprintf(stderr, "run_steps: %zu eager steps until period %zu: %.3f ms\n", done, period, since());
             if (period) {
                 const size_t one = period, warm = traces.size();
                 // Records `span` steps (a multiple of the period) and replays them as often as whole spans fit; false when
@@ -1556,7 +1564,9 @@ size_t run_steps(Step&& step, size_t epochs, bool allow_graph) {
                         if (exec) B::graph_destroy(exec);
                         throw;
                     }
+                    if (trace_steps) std::fprintf(stderr, "run_steps: %zu steps recorded: %.3f ms\n", span, since());
                     B::graph_end(&exec);
+                    if (trace_steps) std::fprintf(stderr, "run_steps: recording closed: %.3f ms\n", since());
                     bool periodic = true;
                     for (size_t k = 0; k < span && periodic; ++k) periodic = recorded[k] == traces[warm - one + k % one];
                     if (pool.device_allocs != allocs_before) {
@@ -1569,10 +1579,12 @@ size_t run_steps(Step&& step, size_t epochs, bool allow_graph) {
                     // them in one launch)
                     size_t spans = periodic ? (epochs - done) / span : 1;
                     B::graph_launch_n(exec, spans);
+                    if (trace_steps) std::fprintf(stderr, "run_steps: %zu replays of %zu steps queued: %.3f ms\n", spans, span, since());
                     backend_calls() += calls_per_span * (spans - 1);
                     done += spans * span;
                     replayed += spans * span;
                     B::graph_destroy(exec);
+                    if (trace_steps) std::fprintf(stderr, "run_steps: recording released: %.3f ms\n", since());
                     return periodic;
                 };
                 // several periods per graph: a graph launch costs a few microseconds however many nodes it holds
@@ -1582,7 +1594,9 @@ size_t run_steps(Step&& step, size_t epochs, bool allow_graph) {
             }
         }
     }
+    const size_t rest = epochs - done;
     for (; done < epochs; ++done) step(done);
+    if (trace_steps) std::fprintf(stderr, "run_steps: %zu eager steps at the end, all queued: %.3f ms\n", rest, since());
     return replayed;
 }
 
