@@ -18,10 +18,10 @@
 // hip_get_last_status() reports as an invalid argument (the reference returns IndexOutOfBounds).
 #include <cstring>
 
-#include <rocprim/rocprim.hpp>
 
 #include "elementwise.hpp"
 #include "mxh.hpp"
+#include "radix_sort.hpp"
 #include "ops.hpp"
 
 namespace mxh {
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(IB) void index_add_kernel(IdxSpace sp, Lay self, La
 }
 
 // Many indices, few lines (an embedding gradient): the indices are sorted by destination with a stable
-// radix sort (vendor primitive; equal destinations keep ascending i), and one thread per destination
+// radix sort (radix_sort.hpp; equal destinations keep ascending i), and one thread per destination
 // element adds its sources in that order — the same order as the walk above, with parallelism over
 // the whole of self instead of over the lines.
 template <class I>
@@ -358,24 +358,20 @@ void index_add(size_t nd, size_t dim, const size_t* self_layout, const size_t* s
     if (lines == 0 || n_idx == 0) return;
     const size_t D = self_layout[dim];
     if (n_idx >= 256 && lines < (1ull << 31) && D * lines < (1ull << 31) && D < (1ull << 31) - 1) {
-        // [keys in | keys out | values in | values out | sort workspace] in scratch slot 1
-        size_t sort_bytes = 0;
-        uint32_t* nil = nullptr;
+        // [keys a | keys b | values a | values b | the sort's counts] in scratch slot 1
         unsigned bits = 1;
         while ((1ull << bits) <= D) ++bits;
-        if (rocprim::radix_sort_pairs(nullptr, sort_bytes, nil, nil, nil, nil, n_idx, 0u, bits, stream()) != hipSuccess) {
-            set_status(ERR_LAUNCH, "index_add_: sort workspace query failed");
-            return;
-        }
         const size_t arr = (n_idx * sizeof(uint32_t) + 255) / 256 * 256;
-        char* ws = (char*)scratch(4 * arr + sort_bytes, 1);
+        char* ws = (char*)scratch(4 * arr + rs_workspace_bytes(n_idx), 1);
         if (!ws) return;
-        uint32_t *k_in = (uint32_t*)ws, *k_out = (uint32_t*)(ws + arr), *v_in = (uint32_t*)(ws + 2 * arr), *v_out = (uint32_t*)(ws + 3 * arr);
+        uint32_t *k_a = (uint32_t*)ws, *k_b = (uint32_t*)(ws + arr), *v_a = (uint32_t*)(ws + 2 * arr), *v_b = (uint32_t*)(ws + 3 * arr);
         hipLaunchKernelGGL(index_keys_kernel<I>, dim3(cdiv(n_idx, IB)), dim3(IB), 0, stream(), indices, (int64_t)idx_stride, (int64_t)idx_offset,
-                           (uint32_t)n_idx, (uint32_t)D, k_in, v_in, flag);
+                           (uint32_t)n_idx, (uint32_t)D, k_a, v_a, flag);
         MXH_LAUNCH_CHECK("index_keys");
         prog_launch_seen();      // the sort's own launches
-        MXH_HIP(rocprim::radix_sort_pairs(ws + 4 * arr, sort_bytes, k_in, k_out, v_in, v_out, n_idx, 0u, bits, stream()));
+        const bool in_b = radix_sort_pairs_u32(k_a, v_a, k_b, v_b, n_idx, bits, (uint32_t*)(ws + 4 * arr), stream());
+        MXH_LAUNCH_CHECK("radix_sort");
+        const uint32_t *k_out = in_b ? k_b : k_a, *v_out = in_b ? v_b : v_a;
         {
             constexpr int VEC = 16 / sizeof(T);
             size_t inner = 1, outer = 1;

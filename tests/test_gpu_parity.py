@@ -1336,6 +1336,24 @@ def test_index_add_with_many_indices(oracle, hip, shape, dim, n_idx, dt):
     assert same_bits(o, h)
 
 
+@pytest.mark.parametrize("shape,dim,n_idx,spread", [([70000, 2], 0, 200000, 70000), ([300000], 0, 50000, 300000), ([2, 66000, 1], 1, 9000, 17),
+                                                    ([5000, 4], 0, 131072, 5000), ([1 << 17, 1], 0, 4097, 1 << 17)])
+def test_index_add_sorts_many_indices_over_many_destinations(oracle, hip, shape, dim, n_idx, spread):
+    """Destinations of up to 19 bits (three passes of the radix sort), index counts that make several blocks of it and
+    one that ends a block with a single element, many equal destinations (`spread` 17): the f32 sums are added in the
+    reference's order, so the bits are the oracle's."""
+    r = rng(171 + n_idx)
+    n = int(np.prod(shape))
+    x = r.standard_normal(n).astype(np.float32)
+    idx = r.integers(0, spread, n_idx).astype(np.int32)
+    src_shape = list(shape)
+    src_shape[dim] = n_idx
+    src = r.standard_normal(int(np.prod(src_shape))).astype(np.float32)
+    (o,), (h,) = both(oracle, hip, "index_add_f32_i32",
+                      lambda: (len(shape), dim, layout(shape), layout(src_shape), n_idx, 1, 0, In(idx), In(src), InOut(x.copy())))
+    assert same_bits(o, h)
+
+
 @pytest.mark.parametrize("dt", ["f64", "bool"] + INT_DTS)
 @pytest.mark.parametrize("it", ["i32", "i64"])
 def test_index_ops_wide_dtypes(oracle, hip, dt, it):
