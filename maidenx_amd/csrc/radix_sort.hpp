@@ -14,14 +14,16 @@ namespace mxh {
 
 constexpr int RS_THREADS = 256;
 constexpr int RS_BINS = 256;
-constexpr uint32_t RS_MAX_BLOCKS = 16384;
+constexpr uint32_t RS_MAX_BLOCKS = 2048;       // (the scan is one work-group over RS_BINS * blocks counts)
 
 struct RsPlan {
     uint32_t blocks, chunk;      // every block sorts `chunk` consecutive elements (a multiple of RS_THREADS)
 };
 inline RsPlan rs_plan(size_t n) {
     RsPlan p;
-    size_t chunk = 4096;
+    // (measured on an embedding gradient's sort: chunks of 2048-4096 are best for 65536 pairs, 8192-16384 for 2^20;
+    // smaller chunks scatter a block's elements over too many short runs)
+    size_t chunk = n >= (1u << 19) ? 8192 : 4096;
     while ((n + chunk - 1) / chunk > RS_MAX_BLOCKS) chunk *= 2;
     p.chunk = (uint32_t)chunk;
     p.blocks = (uint32_t)((n + chunk - 1) / chunk);
