@@ -1,7 +1,7 @@
 // A stable least-significant-digit radix sort of (32-bit key, 32-bit value) pairs, eight bits a pass: what index_add_
 // orders its sources with (equal destinations keep ascending source order, so the sums are added as the reference's
-// walk adds them).  A pass is three launches: per-block digit counts, one exclusive scan over (digit, block), and a
-// scatter in which every block walks its chunk again in 256-element groups - inside a group an element's place among
+// walk adds them).  A pass is three launches: per-block digit counts, one exclusive scan over (digit, block) - which
+// the scatter does itself when the blocks are few - and a scatter in which every block walks its chunk again in 256-element groups - inside a group an element's place among
 // the elements of its digit is a count of the lower lanes of its wave that hold the same digit (eight ballots) plus
 // the counts of the waves before it, and a running count per digit carries from group to group.
 #pragma once
@@ -14,6 +14,7 @@ namespace mxh {
 
 constexpr int RS_THREADS = 256;
 constexpr int RS_BINS = 256;
+constexpr uint32_t RS_SCAN_IN_SCATTER = 64;   // up to this many blocks the scatter scans the counts itself
 constexpr uint32_t RS_MAX_BLOCKS = 2048;       // (the scan is one work-group over RS_BINS * blocks counts)
 
 struct RsPlan {
@@ -21,9 +22,11 @@ struct RsPlan {
 };
 inline RsPlan rs_plan(size_t n) {
     RsPlan p;
-    // (measured on an embedding gradient's sort: chunks of 2048-4096 are best for 65536 pairs, 8192-16384 for 2^20;
-    // smaller chunks scatter a block's elements over too many short runs)
-    size_t chunk = n >= (1u << 19) ? 8192 : 4096;
+    // (measured on an embedding gradient's sort: for 65536 pairs chunks of 1024 are best - 64 blocks, which still scan
+    // the counts themselves -, 8192-16384 for 2^20; smaller chunks scatter a block's elements over too many short runs)
+    size_t chunk = 1024;
+    while (chunk < 4096 && (n + chunk - 1) / chunk > RS_SCAN_IN_SCATTER) chunk *= 2;
+    if (n >= (1u << 19)) chunk = 8192;
     while ((n + chunk - 1) / chunk > RS_MAX_BLOCKS) chunk *= 2;
     p.chunk = (uint32_t)chunk;
     p.blocks = (uint32_t)((n + chunk - 1) / chunk);
@@ -74,12 +77,34 @@ __global__ __launch_bounds__(RS_SCAN_THREADS) void rs_scan_kernel(uint32_t* __re
 __global__ __launch_bounds__(RS_THREADS) void rs_scatter_kernel(const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
                                                                 uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, uint32_t n,
                                                                 uint32_t shift, uint32_t chunk, uint32_t blocks,
-                                                                const uint32_t* __restrict__ offsets) {
+                                                                const uint32_t* __restrict__ offsets, bool scanned) {
     constexpr int WAVES = RS_THREADS / WAVE;
     __shared__ uint32_t next[RS_BINS];                 // where the block's next element of each digit goes
     __shared__ uint32_t wave_count[WAVES][RS_BINS];    // a group's elements per wave and digit, then their first places
     const unsigned tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-    next[tid] = offsets[(size_t)tid * blocks + blockIdx.x];
+    if (scanned) {
+        next[tid] = offsets[(size_t)tid * blocks + blockIdx.x];
+    } else {
+        // few blocks: `offsets` still holds the counts, and every block works out its own places from them (digit tid:
+        // the elements of lower digits anywhere, plus this digit's in the blocks before) - one launch less per pass
+        uint32_t before = 0, all = 0;
+        for (uint32_t b = 0; b < blocks; ++b) {
+            const uint32_t c = offsets[(size_t)tid * blocks + b];
+            before += b < blockIdx.x ? c : 0u;
+            all += c;
+        }
+        uint32_t* scan = &wave_count[0][0];            // (free until the first group)
+        scan[tid] = all;
+        __syncthreads();
+        for (int d = 1; d < RS_BINS; d *= 2) {          // inclusive prefix over the digits
+            const uint32_t add = tid >= (unsigned)d ? scan[tid - d] : 0u;
+            __syncthreads();
+            scan[tid] += add;
+            __syncthreads();
+        }
+        next[tid] = scan[tid] - all + before;
+        __syncthreads();
+    }
     const uint32_t beg = blockIdx.x * chunk, end = n - beg < chunk ? n : beg + chunk;
     for (uint32_t group = beg; group < end; group += RS_THREADS) {
 #pragma unroll
@@ -130,8 +155,10 @@ inline bool radix_sort_pairs_u32(uint32_t* keys_a, uint32_t* vals_a, uint32_t* k
         const uint32_t *ki = in_b ? keys_b : keys_a, *vi = in_b ? vals_b : vals_a;
         uint32_t *ko = in_b ? keys_a : keys_b, *vo = in_b ? vals_a : vals_b;
         hipLaunchKernelGGL(rs_count_kernel, dim3(p.blocks), dim3(RS_THREADS), 0, s, ki, (uint32_t)n, shift, p.chunk, p.blocks, counts);
-        hipLaunchKernelGGL(rs_scan_kernel, dim3(1), dim3(RS_SCAN_THREADS), 0, s, counts, (uint32_t)(RS_BINS * p.blocks));
-        hipLaunchKernelGGL(rs_scatter_kernel, dim3(p.blocks), dim3(RS_THREADS), 0, s, ki, vi, ko, vo, (uint32_t)n, shift, p.chunk, p.blocks, counts);
+        const bool scan_launch = p.blocks > RS_SCAN_IN_SCATTER;
+        if (scan_launch) hipLaunchKernelGGL(rs_scan_kernel, dim3(1), dim3(RS_SCAN_THREADS), 0, s, counts, (uint32_t)(RS_BINS * p.blocks));
+        hipLaunchKernelGGL(rs_scatter_kernel, dim3(p.blocks), dim3(RS_THREADS), 0, s, ki, vi, ko, vo, (uint32_t)n, shift, p.chunk, p.blocks, counts,
+                           scan_launch);
         in_b = !in_b;
     }
     return in_b;
